@@ -1,0 +1,214 @@
+#!/usr/bin/env python3
+"""Benchmark of the deformable-kernel hot path on one MI355X.
+
+A "step" is one forward + backward of a DeformKernel2d layer's operator
+(sample_depthwise: forward, grad-input, grad-rotation, grad-filter) over one
+batch of synthetic input resident in HBM, issued through the C ABI of
+libdk_hip.so on torch's current stream with preallocated outputs.
+
+Default workload: BASELINE config 2 -- N=64, C=144, 56x56, 3x3 taps, scope 4x4,
+stride 1, pad 1, fp32, rotation ~ N(0, 1).
+
+Prints ONE JSON line: the BASELINE metric (achieved HBM GB/s on the
+algorithmic bytes of the step), a `roofline` object for the dominant kernel
+(timed with events on the launch stream) and a `cpu_baseline` object (the CPU
+oracle, OpenMP, on a bounded slice of the same workload).
+"""
+import argparse
+import ctypes
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+for p in (ROOT, os.path.join(ROOT, "deformable-kernels_amd"), os.path.join(ROOT, "tests")):
+    if p not in sys.path:
+        sys.path.insert(0, p)
+
+HBM_PEAK_GBPS = 8000.0  # MI355X published HBM3E bandwidth
+
+WORKLOADS = {
+    # name: (N, C, H, W, k, S, stride, pad, dil, groups, rot_std)
+    "cfg2": (64, 144, 56, 56, 3, (4, 4), 1, 1, 1, 1, 1.0),
+    "cfg1": (2, 32, 28, 28, 3, (4, 4), 1, 1, 1, 1, 0.5),
+}
+DTYPES = {"fp32": "float32", "bf16": "bfloat16", "fp16": "float16"}
+
+
+def algorithmic_bytes(N, C, H, W, Ho, Wo, k, S, groups, esz):
+    """Compulsory traffic, every tensor touched once (bytes), per kernel and per step."""
+    x = N * C * H * W * esz
+    y = N * C * Ho * Wo * esz
+    rot = N * groups * k * k * 2 * Ho * Wo * esz
+    wt = C * S[0] * S[1] * esz
+    per_kernel = {
+        "forward": x + rot + wt + y,
+        "grad_input": y + rot + wt + x,
+        "grad_rotation": y + x + rot + wt + rot,
+        "grad_filter": y + x + rot + wt,
+    }
+    fwd = x + rot + wt + y
+    bwd = (y + x + rot + wt) + (x + rot + wt)  # read gout, x, rot, Wt; write gin, grot, gWt
+    return per_kernel, fwd, bwd
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--workload", default="cfg2", choices=sorted(WORKLOADS))
+    ap.add_argument("--dtype", default="fp32", choices=sorted(DTYPES))
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    a = ap.parse_args()
+    if a.gpus != 1:
+        sys.exit("bench.py measures one GPU only: every box of this build has one GPU and no "
+                 "multi-GPU path exists (the operator shards over the batch with no exchange); "
+                 "run with --gpus 1")
+
+    import torch
+    from _cases import make_local
+    from deformable_kernels.ops.deform_kernel import _lib
+
+    if not torch.cuda.is_available():
+        sys.exit("bench.py needs a GPU")
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    tdtype = getattr(torch, DTYPES[a.dtype])
+    N, C, H, W, k, S, stride, pad, dil, groups, rot_std = WORKLOADS[a.workload]
+    x, wt, rot, gout, cfg = make_local(N, C, H, W, k, S, stride, pad, dil, groups, rot_std, seed=0, dtype=tdtype)
+    Ho, Wo = gout.shape[2], gout.shape[3]
+    xg, wg, rg, gg = [t.to(dev) for t in (x, wt, rot, gout)]
+    out = torch.empty_like(gg)
+    gin = torch.empty_like(xg)
+    grot = torch.empty_like(rg)
+    gw = torch.empty_like(wg)
+    L = _lib.lib()
+    desc = _lib.conv_desc(xg, wg, cfg["kernel_size"], cfg["stride"], cfg["padding"], cfg["dilation"], groups)
+    ws, ws_bytes = _lib.workspace(L.dk_sample_depthwise_backward_filter_workspace(desc), dev)
+    stream = _lib.stream_ptr(xg)
+    P = _lib.ptr
+
+    def k_forward():
+        _lib.check(L.dk_sample_depthwise_forward(desc, P(xg), P(rg), P(wg), P(out), stream), "forward")
+
+    def k_grad_input():
+        _lib.check(L.dk_sample_depthwise_backward_data(desc, P(gg), P(rg), P(wg), P(gin), stream), "grad_input")
+
+    def k_grad_rotation():
+        _lib.check(L.dk_sample_depthwise_backward_rotation(desc, P(gg), P(xg), P(rg), P(wg), P(grot), stream),
+                   "grad_rotation")
+
+    def k_grad_filter():
+        _lib.check(L.dk_sample_depthwise_backward_filter(desc, P(gg), P(xg), P(rg), P(gw), P(ws), ws_bytes, stream),
+                   "grad_filter")
+
+    kernels = {"forward": k_forward, "grad_input": k_grad_input, "grad_rotation": k_grad_rotation,
+               "grad_filter": k_grad_filter}
+
+    def step():
+        k_forward()
+        k_grad_input()
+        k_grad_rotation()
+        k_grad_filter()
+
+    for _ in range(a.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(a.steps):
+        step()
+    torch.cuda.synchronize()
+    ms_per_step = (time.perf_counter() - t0) * 1e3 / a.steps
+
+    # per-entry-point launch duration: events on the stream the kernels are launched on
+    per_kernel_us = {}
+    reps = max(a.steps, 20)
+    for name, fn in kernels.items():
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        fn()
+        e0.record()
+        for _ in range(reps):
+            fn()
+        e1.record()
+        e1.synchronize()
+        per_kernel_us[name] = e0.elapsed_time(e1) * 1e3 / reps
+
+    esz = xg.element_size()
+    per_kernel_bytes, fwd_b, bwd_b = algorithmic_bytes(N, C, H, W, Ho, Wo, k, S, groups, esz)
+    step_bytes = fwd_b + bwd_b
+    gbps = step_bytes / (ms_per_step * 1e-3) / 1e9
+    dominant = max(per_kernel_us, key=per_kernel_us.get)
+    achieved = per_kernel_bytes[dominant] / (per_kernel_us[dominant] * 1e-6) / 1e9
+
+    result = {
+        "metric": "DK fwd+bwd achieved HBM GB/s",
+        "value": round(gbps, 2),
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": a.steps,
+        "warmup": a.warmup,
+        "ms_per_step": round(ms_per_step, 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": {"fp32": "f32", "bf16": "bf16", "fp16": "f16"}[a.dtype],
+        "data": "synthetic",
+        "config": {"workload": "%s: DeformKernel2d op fwd+bwd N=%d C=%d %dx%d k=%d scope=%dx%d stride=%d pad=%d %s"
+                               % (a.workload, N, C, H, W, k, S[0], S[1], stride, pad, a.dtype),
+                   "algorithmic_MB_per_step": round(step_bytes / 1e6, 2)},
+        "pct_of_hbm_peak": round(100.0 * gbps / HBM_PEAK_GBPS, 2),
+        "images_per_s": round(N / (ms_per_step * 1e-3), 1),
+        "layers_per_s": round(1.0 / (ms_per_step * 1e-3), 1),
+        "kernel_us": {n: round(v, 2) for n, v in per_kernel_us.items()},
+        "roofline": {
+            "kernel": dominant,
+            "bound": "hbm",
+            "achieved": round(achieved, 2),
+            "peak": HBM_PEAK_GBPS,
+            "unit": "GB/s",
+            "frac": round(achieved / HBM_PEAK_GBPS, 4),
+            "traffic": None,
+        },
+    }
+
+    if not a.no_cpu_baseline:
+        result["cpu_baseline"] = cpu_baseline(N, C, H, W, k, S, stride, pad, dil, groups, rot_std, esz)
+    print(json.dumps(result))
+
+
+def cpu_baseline(N, C, H, W, k, S, stride, pad, dil, groups, rot_std, esz):
+    """The CPU oracle (a port of the reference's arithmetic; the reference has no CPU path),
+    OpenMP over the host cores, fp32, on the first `n` images of the same seeded workload."""
+    from _cases import make_local
+    from oracle import dk_oracle as orc
+    n = min(N, 8)
+    x, wt, rot, gout, cfg = make_local(n, C, H, W, k, S, stride, pad, dil, groups, rot_std, seed=0)
+    xs, ws_, rs, gs = [t.numpy() for t in (x, wt, rot, gout)]
+    threads = min(orc.max_threads(), 16)
+    orc.set_threads(threads)
+    best = None
+    t_all = time.perf_counter()
+    for _ in range(5):
+        t0 = time.perf_counter()
+        orc.sample_depthwise_forward(xs, rs, ws_, **cfg)
+        orc.sample_depthwise_backward(gs, xs, rs, ws_, **cfg)
+        dt = time.perf_counter() - t0
+        best = dt if best is None else min(best, dt)
+        if time.perf_counter() - t_all > 25:
+            break
+    Ho, Wo = gout.shape[2], gout.shape[3]
+    _, fwd_b, bwd_b = algorithmic_bytes(n, C, H, W, Ho, Wo, k, S, groups, 4)
+    return {
+        "value": round((fwd_b + bwd_b) / best / 1e9, 3),
+        "unit": "GB/s",
+        "cores": threads,
+        "kind": "port",
+        "sample": "first %d of %d images of the same seeded workload, fwd + 3 grads, fp32, best of <=5 runs "
+                  "(%.3f s per run, %.1f images/s)" % (n, N, best, n / best),
+    }
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,342 @@
+// C ABI of libdk_hip.so (declared in include/dk_hip.h): argument validation,
+// geometry derivation and dispatch to the tuned or the generic kernels.
+// Each entry point names the reference pybind function it stands in for
+// (K.cpp = deformable_kernels/ops/deform_kernel/csrc/filter_sample_depthwise_cuda.cpp,
+//  ND.cpp = .../csrc/nd_linear_sample_cuda.cpp).
+#include "dk_kernels.h"
+#include "dk_nd.h"
+
+using namespace dk;
+
+namespace {
+
+constexpr long kMaxElems = 2147483647L;  // plane-relative indices are 32-bit
+
+int make_geo(const dk_conv_desc* d, Geo& g) {
+  if (!d) return DK_ERR_NULL_POINTER;
+  if (d->dtype < DK_F32 || d->dtype > DK_F64) return DK_ERR_BAD_DTYPE;
+  if (d->batch < 0 || d->channel <= 0 || d->in_h <= 0 || d->in_w <= 0 || d->k_h <= 0 ||
+      d->k_w <= 0 || d->stride_h <= 0 || d->stride_w <= 0 || d->pad_h < 0 || d->pad_w < 0 ||
+      d->dil_h <= 0 || d->dil_w <= 0 || d->scope_h <= 0 || d->scope_w <= 0 || d->groups <= 0)
+    return DK_ERR_BAD_SHAPE;
+  if (d->channel % d->groups != 0) return DK_ERR_BAD_SHAPE;
+  // K.cpp:42-43
+  const long oh = ((long)d->in_h + 2L * d->pad_h - ((long)d->dil_h * (d->k_h - 1) + 1)) / d->stride_h + 1;
+  const long ow = ((long)d->in_w + 2L * d->pad_w - ((long)d->dil_w * (d->k_w - 1) + 1)) / d->stride_w + 1;
+  if ((long)d->in_h + 2L * d->pad_h < (long)d->dil_h * (d->k_h - 1) + 1 ||
+      (long)d->in_w + 2L * d->pad_w < (long)d->dil_w * (d->k_w - 1) + 1 || oh <= 0 || ow <= 0)
+    return DK_ERR_BAD_SHAPE;
+  const long taps2 = 2L * d->k_h * d->k_w;
+  if ((long)d->batch * d->channel * d->in_h * d->in_w > kMaxElems ||
+      (long)d->batch * d->channel * oh * ow > kMaxElems ||
+      (long)d->batch * d->groups * taps2 * oh * ow > kMaxElems ||
+      (long)d->batch * d->channel * taps2 / 2 * oh * ow > 4 * kMaxElems ||
+      (long)d->channel * d->scope_h * d->scope_w > kMaxElems)
+    return DK_ERR_TOO_LARGE;
+  g.batch = d->batch;
+  g.channel = d->channel;
+  g.in_h = d->in_h;
+  g.in_w = d->in_w;
+  g.k_h = d->k_h;
+  g.k_w = d->k_w;
+  g.stride_h = d->stride_h;
+  g.stride_w = d->stride_w;
+  g.pad_h = d->pad_h;
+  g.pad_w = d->pad_w;
+  g.dil_h = d->dil_h;
+  g.dil_w = d->dil_w;
+  g.out_h = (int)oh;
+  g.out_w = (int)ow;
+  g.scope_h = d->scope_h;
+  g.scope_w = d->scope_w;
+  g.groups = d->groups;
+  g.centre_h = (d->scope_h - d->k_h) / 2.0;  // K.cu:338-341
+  g.centre_w = (d->scope_w - d->k_w) / 2.0;
+  return DK_OK;
+}
+
+int launch_status() { return hipGetLastError() == hipSuccess ? DK_OK : DK_ERR_LAUNCH; }
+
+// Calls f.template operator()<T>() with T the element type tagged by `dtype`.
+template <typename F>
+int by_dtype(int dtype, F&& f) {
+  switch (dtype) {
+    case DK_F32: f.template operator()<float>(); break;
+    case DK_F16: f.template operator()<__half>(); break;
+    case DK_BF16: f.template operator()<bf16_t>(); break;
+    case DK_F64: f.template operator()<double>(); break;
+    default: return DK_ERR_BAD_DTYPE;
+  }
+  return launch_status();
+}
+
+// The tuned kernels exist for the 16- and 32-bit types only.
+template <typename T> constexpr bool kHasFast = !std::is_same<T, double>::value;
+
+template <typename T> const T* in(const void* p) { return static_cast<const T*>(p); }
+template <typename T> T* out(void* p) { return static_cast<T*>(p); }
+
+size_t local_filter_ws(const Geo& g, int dtype) {
+  const size_t a = dtype == DK_F64 ? 0 : fast_local_grad_filter_workspace(g);
+  return a ? a : generic_grad_filter_workspace(g, dtype);
+}
+
+}  // namespace
+
+extern "C" {
+
+int dk_version(void) { return (0 << 16) | 1; }
+
+const char* dk_status_string(int status) {
+  switch (status) {
+    case DK_OK: return "ok";
+    case DK_ERR_NULL_POINTER: return "null pointer argument";
+    case DK_ERR_BAD_SHAPE: return "invalid shape (non-positive size, empty output, or channel % groups != 0)";
+    case DK_ERR_BAD_DTYPE: return "unknown dtype tag";
+    case DK_ERR_TOO_LARGE: return "tensor has 2^31 or more elements";
+    case DK_ERR_WORKSPACE: return "workspace missing or too small";
+    case DK_ERR_LAUNCH: return "HIP kernel launch failed";
+    case DK_ERR_UNSUPPORTED: return "unsupported configuration";
+    default: return "unknown status";
+  }
+}
+
+int dk_conv_out_size(const dk_conv_desc* desc, int32_t* out_h, int32_t* out_w) {
+  Geo g;
+  const int rc = make_geo(desc, g);
+  if (rc != DK_OK) return rc;
+  if (out_h) *out_h = g.out_h;
+  if (out_w) *out_w = g.out_w;
+  return DK_OK;
+}
+
+// ---- local ------------------------------------------------------------------------------
+
+int dk_sample_depthwise_forward(const dk_conv_desc* desc, const void* input, const void* rotation,
+                                const void* filter, void* output, void* stream) {
+  Geo g;
+  const int rc = make_geo(desc, g);
+  if (rc != DK_OK) return rc;
+  if (!input || !rotation || !filter || !output) return DK_ERR_NULL_POINTER;
+  if (g.batch == 0) return DK_OK;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  return by_dtype(desc->dtype, [&]<typename T>() {
+    if constexpr (kHasFast<T>)
+      if (fast_local_gather<T>(g, false, in<T>(input), in<T>(rotation), in<T>(filter), out<T>(output), s)) return;
+    generic_forward<T>(g, false, in<T>(input), (const T*)nullptr, in<T>(rotation), in<T>(filter), out<T>(output), s);
+  });
+}
+
+int dk_sample_depthwise_backward_data(const dk_conv_desc* desc, const void* out_grad,
+                                      const void* rotation, const void* filter, void* in_grad,
+                                      void* stream) {
+  Geo g;
+  const int rc = make_geo(desc, g);
+  if (rc != DK_OK) return rc;
+  if (!out_grad || !rotation || !filter || !in_grad) return DK_ERR_NULL_POINTER;
+  if (g.batch == 0) return DK_OK;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  return by_dtype(desc->dtype, [&]<typename T>() {
+    if constexpr (kHasFast<T>)
+      if (fast_local_gather<T>(g, true, in<T>(out_grad), in<T>(rotation), in<T>(filter), out<T>(in_grad), s)) return;
+    generic_local_grad_input<T>(g, in<T>(out_grad), in<T>(rotation), in<T>(filter), out<T>(in_grad), s);
+  });
+}
+
+size_t dk_sample_depthwise_backward_filter_workspace(const dk_conv_desc* desc) {
+  Geo g;
+  if (make_geo(desc, g) != DK_OK) return 0;
+  return local_filter_ws(g, desc->dtype);
+}
+
+int dk_sample_depthwise_backward_filter(const dk_conv_desc* desc, const void* out_grad,
+                                        const void* input, const void* rotation, void* filter_grad,
+                                        void* workspace, size_t workspace_bytes, void* stream) {
+  Geo g;
+  const int rc = make_geo(desc, g);
+  if (rc != DK_OK) return rc;
+  if (!out_grad || !input || !rotation || !filter_grad) return DK_ERR_NULL_POINTER;
+  const size_t need = local_filter_ws(g, desc->dtype);
+  if (need && (!workspace || workspace_bytes < need)) return DK_ERR_WORKSPACE;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  return by_dtype(desc->dtype, [&]<typename T>() {
+    if constexpr (kHasFast<T>)
+      if (fast_local_grad_filter<T>(g, in<T>(out_grad), in<T>(input), in<T>(rotation), out<T>(filter_grad), workspace, s)) return;
+    generic_grad_filter<T>(g, false, in<T>(out_grad), in<T>(input), (const T*)nullptr, in<T>(rotation),
+                           out<T>(filter_grad), workspace, s);
+  });
+}
+
+int dk_sample_depthwise_backward_rotation(const dk_conv_desc* desc, const void* out_grad,
+                                          const void* input, const void* rotation,
+                                          const void* filter, void* rotation_grad, void* stream) {
+  Geo g;
+  const int rc = make_geo(desc, g);
+  if (rc != DK_OK) return rc;
+  if (!out_grad || !input || !rotation || !filter || !rotation_grad) return DK_ERR_NULL_POINTER;
+  if (g.batch == 0) return DK_OK;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  return by_dtype(desc->dtype, [&]<typename T>() {
+    if constexpr (kHasFast<T>)
+      if (fast_local_grad_rotation<T>(g, in<T>(out_grad), in<T>(input), in<T>(rotation), in<T>(filter), out<T>(rotation_grad), s)) return;
+    generic_grad_rotation<T>(g, false, in<T>(out_grad), in<T>(input), (const T*)nullptr, in<T>(rotation),
+                             in<T>(filter), out<T>(rotation_grad), s);
+  });
+}
+
+// ---- deformable --------------------------------------------------------------------------
+
+int dk_deformable_sample_depthwise_forward(const dk_conv_desc* desc, const void* input,
+                                           const void* offset, const void* rotation,
+                                           const void* filter, void* output, void* stream) {
+  Geo g;
+  const int rc = make_geo(desc, g);
+  if (rc != DK_OK) return rc;
+  if (!input || !offset || !rotation || !filter || !output) return DK_ERR_NULL_POINTER;
+  if (g.batch == 0) return DK_OK;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  return by_dtype(desc->dtype, [&]<typename T>() {
+    generic_forward<T>(g, true, in<T>(input), in<T>(offset), in<T>(rotation), in<T>(filter), out<T>(output), s);
+  });
+}
+
+size_t dk_deformable_sample_depthwise_backward_data_workspace(const dk_conv_desc* desc) {
+  Geo g;
+  if (make_geo(desc, g) != DK_OK) return 0;
+  return generic_deform_grad_input_workspace(g, desc->dtype);
+}
+
+int dk_deformable_sample_depthwise_backward_data(const dk_conv_desc* desc, const void* out_grad,
+                                                 const void* offset, const void* rotation,
+                                                 const void* filter, void* in_grad, void* workspace,
+                                                 size_t workspace_bytes, void* stream) {
+  Geo g;
+  const int rc = make_geo(desc, g);
+  if (rc != DK_OK) return rc;
+  if (!out_grad || !offset || !rotation || !filter || !in_grad) return DK_ERR_NULL_POINTER;
+  const size_t need = generic_deform_grad_input_workspace(g, desc->dtype);
+  if (need && (!workspace || workspace_bytes < need)) return DK_ERR_WORKSPACE;
+  if (g.batch == 0) return DK_OK;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  return by_dtype(desc->dtype, [&]<typename T>() {
+    generic_deform_grad_input<T>(g, in<T>(out_grad), in<T>(offset), in<T>(rotation), in<T>(filter),
+                                 out<T>(in_grad), workspace, s);
+  });
+}
+
+size_t dk_deformable_sample_depthwise_backward_filter_workspace(const dk_conv_desc* desc) {
+  Geo g;
+  if (make_geo(desc, g) != DK_OK) return 0;
+  return generic_grad_filter_workspace(g, desc->dtype);
+}
+
+int dk_deformable_sample_depthwise_backward_filter(const dk_conv_desc* desc, const void* out_grad,
+                                                   const void* input, const void* offset,
+                                                   const void* rotation, void* filter_grad,
+                                                   void* workspace, size_t workspace_bytes,
+                                                   void* stream) {
+  Geo g;
+  const int rc = make_geo(desc, g);
+  if (rc != DK_OK) return rc;
+  if (!out_grad || !input || !offset || !rotation || !filter_grad) return DK_ERR_NULL_POINTER;
+  const size_t need = generic_grad_filter_workspace(g, desc->dtype);
+  if (need && (!workspace || workspace_bytes < need)) return DK_ERR_WORKSPACE;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  return by_dtype(desc->dtype, [&]<typename T>() {
+    generic_grad_filter<T>(g, true, in<T>(out_grad), in<T>(input), in<T>(offset), in<T>(rotation),
+                           out<T>(filter_grad), workspace, s);
+  });
+}
+
+int dk_deformable_sample_depthwise_backward_offset(const dk_conv_desc* desc, const void* out_grad,
+                                                   const void* input, const void* offset,
+                                                   const void* rotation, const void* filter,
+                                                   void* offset_grad, void* stream) {
+  Geo g;
+  const int rc = make_geo(desc, g);
+  if (rc != DK_OK) return rc;
+  if (!out_grad || !input || !offset || !rotation || !filter || !offset_grad) return DK_ERR_NULL_POINTER;
+  if (g.batch == 0) return DK_OK;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  return by_dtype(desc->dtype, [&]<typename T>() {
+    generic_grad_offset<T>(g, in<T>(out_grad), in<T>(input), in<T>(offset), in<T>(rotation), in<T>(filter),
+                           out<T>(offset_grad), s);
+  });
+}
+
+int dk_deformable_sample_depthwise_backward_rotation(const dk_conv_desc* desc, const void* out_grad,
+                                                     const void* input, const void* offset,
+                                                     const void* rotation, const void* filter,
+                                                     void* rotation_grad, void* stream) {
+  Geo g;
+  const int rc = make_geo(desc, g);
+  if (rc != DK_OK) return rc;
+  if (!out_grad || !input || !offset || !rotation || !filter || !rotation_grad) return DK_ERR_NULL_POINTER;
+  if (g.batch == 0) return DK_OK;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  return by_dtype(desc->dtype, [&]<typename T>() {
+    generic_grad_rotation<T>(g, true, in<T>(out_grad), in<T>(input), in<T>(offset), in<T>(rotation),
+                             in<T>(filter), out<T>(rotation_grad), s);
+  });
+}
+
+// ---- N-d linear sample --------------------------------------------------------------------
+
+static int check_nd(const dk_nd_desc* d) {
+  if (!d) return DK_ERR_NULL_POINTER;
+  if (d->dtype < DK_F32 || d->dtype > DK_F64) return DK_ERR_BAD_DTYPE;
+  if (d->dims < 1 || d->dims > DK_ND_MAX_DIMS) return DK_ERR_UNSUPPORTED;
+  if (d->batch < 0 || d->channel <= 0) return DK_ERR_BAD_SHAPE;
+  long prod = d->channel;
+  for (int i = 0; i < d->dims; ++i) {
+    if (d->shape[i] <= 0) return DK_ERR_BAD_SHAPE;
+    prod *= d->shape[i];
+    if (prod > kMaxElems) return DK_ERR_TOO_LARGE;
+  }
+  if (d->batch * d->channel > 16L * kMaxElems) return DK_ERR_TOO_LARGE;
+  return DK_OK;
+}
+
+int dk_nd_linear_sample_forward(const dk_nd_desc* desc, const void* data, const void* coord,
+                                void* output, void* stream) {
+  const int rc = check_nd(desc);
+  if (rc != DK_OK) return rc;
+  if (!data || !coord || !output) return DK_ERR_NULL_POINTER;
+  if (desc->batch == 0) return DK_OK;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  return by_dtype(desc->dtype, [&]<typename T>() { nd_forward<T>(*desc, in<T>(data), in<T>(coord), out<T>(output), s); });
+}
+
+size_t dk_nd_linear_sample_backward_data_workspace(const dk_nd_desc* desc) {
+  if (check_nd(desc) != DK_OK) return 0;
+  return nd_grad_data_workspace(*desc);
+}
+
+int dk_nd_linear_sample_backward_data(const dk_nd_desc* desc, const void* out_grad,
+                                      const void* coord, void* in_grad, void* workspace,
+                                      size_t workspace_bytes, void* stream) {
+  const int rc = check_nd(desc);
+  if (rc != DK_OK) return rc;
+  if (!in_grad || (desc->batch > 0 && (!out_grad || !coord))) return DK_ERR_NULL_POINTER;
+  const size_t need = nd_grad_data_workspace(*desc);
+  if (need && (!workspace || workspace_bytes < need)) return DK_ERR_WORKSPACE;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  return by_dtype(desc->dtype, [&]<typename T>() {
+    nd_grad_data<T>(*desc, in<T>(out_grad), in<T>(coord), out<T>(in_grad), workspace, s);
+  });
+}
+
+int dk_nd_linear_sample_backward_coord(const dk_nd_desc* desc, const void* out_grad,
+                                       const void* data, const void* coord, void* coord_grad,
+                                       void* stream) {
+  const int rc = check_nd(desc);
+  if (rc != DK_OK) return rc;
+  if (desc->batch == 0) return DK_OK;
+  if (!out_grad || !data || !coord || !coord_grad) return DK_ERR_NULL_POINTER;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  return by_dtype(desc->dtype, [&]<typename T>() {
+    nd_grad_coord<T>(*desc, in<T>(out_grad), in<T>(data), in<T>(coord), out<T>(coord_grad), s);
+  });
+}
+
+}  // extern "C"

@@ -1,0 +1,48 @@
+// Internal interface between the C-ABI layer (dk_api.hip) and the kernel
+// translation units.  Every `fast_*` function returns false, launching
+// nothing, when the geometry is outside what the tuned kernels cover; the
+// caller then uses the `generic_*` kernels, which take any geometry and dtype.
+#pragma once
+
+#include "dk_common.h"
+
+namespace dk {
+
+template <typename CT, typename T>
+void launch_reduce_partials(const CT* partial, int parts, int count, T* out, hipStream_t stream);
+
+// ---- tuned local path (dk_local_fast.hip): 3x3 taps, scope 3x3 / 4x4 / 5x5, fp32/fp16/bf16
+template <typename T>
+bool fast_local_gather(const Geo& g, bool transposed, const T* src, const T* rot, const T* filter,
+                       T* dst, hipStream_t stream);
+template <typename T>
+bool fast_local_grad_rotation(const Geo& g, const T* gout, const T* x, const T* rot,
+                              const T* filter, T* grot, hipStream_t stream);
+size_t fast_local_grad_filter_workspace(const Geo& g);
+template <typename T>
+bool fast_local_grad_filter(const Geo& g, const T* gout, const T* x, const T* rot, T* gfilter,
+                            void* ws, hipStream_t stream);
+
+// ---- generic path (dk_generic.hip): any geometry, all four dtypes, local and deformable
+template <typename T>
+void generic_forward(const Geo& g, bool deform, const T* x, const T* off, const T* rot,
+                     const T* filter, T* out, hipStream_t stream);
+template <typename T>
+void generic_local_grad_input(const Geo& g, const T* gout, const T* rot, const T* filter, T* gin,
+                              hipStream_t stream);
+size_t generic_deform_grad_input_workspace(const Geo& g, int dtype);
+template <typename T>
+void generic_deform_grad_input(const Geo& g, const T* gout, const T* off, const T* rot,
+                               const T* filter, T* gin, void* ws, hipStream_t stream);
+template <typename T>
+void generic_grad_rotation(const Geo& g, bool deform, const T* gout, const T* x, const T* off,
+                           const T* rot, const T* filter, T* grot, hipStream_t stream);
+template <typename T>
+void generic_grad_offset(const Geo& g, const T* gout, const T* x, const T* off, const T* rot,
+                         const T* filter, T* goff, hipStream_t stream);
+size_t generic_grad_filter_workspace(const Geo& g, int dtype);
+template <typename T>
+void generic_grad_filter(const Geo& g, bool deform, const T* gout, const T* x, const T* off,
+                         const T* rot, T* gfilter, void* ws, hipStream_t stream);
+
+}  // namespace dk

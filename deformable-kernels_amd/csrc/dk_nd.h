@@ -1,0 +1,18 @@
+// Internal interface of the N-d linear sample kernels (dk_nd.hip).
+#pragma once
+
+#include "dk_common.h"
+
+namespace dk {
+
+template <typename T>
+void nd_forward(const dk_nd_desc& d, const T* data, const T* coord, T* out, hipStream_t stream);
+size_t nd_grad_data_workspace(const dk_nd_desc& d);
+template <typename T>
+void nd_grad_data(const dk_nd_desc& d, const T* gout, const T* coord, T* gdata, void* ws,
+                  hipStream_t stream);
+template <typename T>
+void nd_grad_coord(const dk_nd_desc& d, const T* gout, const T* data, const T* coord, T* gcoord,
+                   hipStream_t stream);
+
+}  // namespace dk

@@ -1,0 +1,209 @@
+"""User-facing deformable-kernel layers.
+
+Counterparts of the reference's ``modules/deform_kernel.py``: same class names,
+constructor signatures, attribute names and state-dict keys
+(``weight`` / ``fc.*`` for the global variant, ``rotation_conv.*`` /
+``inner_conv.weight`` for the local one, ``offset_conv.*`` /
+``inner_conv.weight`` for the conv variant).  ``apex`` is not needed: the
+fp32-under-AMP behaviour of ``amp.float_function`` (``:76``) is provided by an
+autocast-aware cast.
+"""
+import torch
+from torch import nn
+
+from ..ops.deform_kernel.functions import nd_linear_sample
+from ..ops.deform_kernel.modules import (
+    SampleDepthwise,
+    DeformableSampleDepthwise,
+)
+
+__all__ = [
+    'GlobalDeformKernel2d',
+    'LocalDeformKernel2d',
+    'DeformKernel2d',
+    'DeformKernelConv2d',
+]
+
+
+def _centred_tap_grid(weight_shape, kernel_size, weight_dilate):
+    """Scope coordinates of the undeformed taps, (h, w[, extra dims]) per tap in
+    tap order: the ``fc_bias`` list of the reference (``:64-74``, ``:188-203``)."""
+    start_h = (weight_shape[0] - (kernel_size - 1) * weight_dilate - 1) / 2.0
+    start_w = (weight_shape[1] - (kernel_size - 1) * weight_dilate - 1) / 2.0
+    grid = []
+    for h in range(kernel_size):
+        for w in range(kernel_size):
+            grid += [start_h + h * weight_dilate, start_w + w * weight_dilate]
+            grid += [(extent - 1) / 2.0 for extent in weight_shape[2:]]
+    return grid
+
+
+class GlobalDeformKernel2d(nn.Module):
+    """One set of kernel-space offsets per image, predicted from the pooled
+    input; the per-image kernels are sampled with ``nd_linear_sample`` and
+    applied by one grouped convolution (reference ``:28-118``)."""
+
+    def __init__(self, weight_shape, in_planes, out_planes, kernel_size=1, stride=1, padding=0,
+                 dilation=1, groups=1, bias=False):
+        super().__init__()
+        assert not bias
+        assert len(weight_shape) >= 2
+        self.kernel_size = kernel_size
+        self.weight_shape = weight_shape
+        self.weight_dilate = 1
+        self.stride = stride
+        self.padding = padding
+        self.dilation = dilation
+        self.out_planes = out_planes
+        self.in_planes = in_planes
+        self.group = groups
+
+        self.weight = nn.Parameter(torch.empty(out_planes, in_planes // self.group, *self.weight_shape))
+        self.fc = nn.Linear(in_planes, kernel_size * kernel_size * len(self.weight_shape))
+        self.fc.zero_init = True
+        self.fc_bias = _centred_tap_grid(weight_shape, kernel_size, self.weight_dilate)
+        self.reset_parameters()
+
+    def reset_parameters(self):
+        # The reference leaves `weight` uninitialised (torch.Tensor(...), :52-54) for an external
+        # initialiser; give it a definite default so a fresh module is usable.
+        nn.init.kaiming_normal_(self.weight.view(self.weight.size(0), self.weight.size(1), -1))
+
+    def dynamic_weight(self, x, weight):
+        if torch.is_autocast_enabled():
+            with torch.autocast(device_type="cuda", enabled=False):
+                return self._dynamic_weight(x.float(), weight.float())
+        return self._dynamic_weight(x, weight)
+
+    def _dynamic_weight(self, x, weight):
+        n, c, h, w = x.shape
+        taps = self.kernel_size * self.kernel_size
+        kernels = self.out_planes * self.in_planes // self.group
+        avg_x = x.reshape(n, c, -1).mean(2)
+        centre = torch.tensor(self.fc_bias, dtype=x.dtype, device=x.device).unsqueeze(0)
+        coord = self.fc(avg_x) * self.weight_dilate + centre
+        # every dimension is clamped with the extent of dimension 0, as in the reference (:83)
+        coord = torch.clamp(coord, 0, self.weight_shape[0] - 1)
+        sampled = nd_linear_sample(
+            weight.reshape(kernels, *self.weight_shape),
+            coord.reshape(n * taps, len(self.weight_shape)),
+        ).view(n, taps, kernels)
+        return sampled.transpose(1, 2).reshape(
+            n * self.out_planes, self.in_planes // self.group, self.kernel_size, self.kernel_size)
+
+    def forward(self, x):
+        n, c, h, w = x.shape
+        weight = self.dynamic_weight(x, self.weight).to(x.dtype)
+        out = nn.functional.conv2d(
+            x.reshape(1, n * c, h, w), weight, stride=self.stride, padding=self.padding,
+            dilation=self.dilation, groups=n * self.group)
+        return out.view(n, self.out_planes, out.shape[2], out.shape[3])
+
+    def extra_repr(self):
+        s = '{}, {}, weight_shape={}, kernel_size={}, stride={}, weight_dilate={}'.format(
+            self.in_planes, self.out_planes, self.weight_shape, self.kernel_size, self.stride,
+            self.weight_dilate)
+        if self.padding != 0:
+            s += ', padding={}'.format(self.padding)
+        if self.dilation != 1:
+            s += ', dilation={}'.format(self.dilation)
+        if self.group != 1:
+            s += ', group={}'.format(self.group)
+        return s
+
+
+class LocalDeformKernel2d(nn.Module):
+    """Per-pixel kernel-space offsets predicted by ``rotation_conv`` and applied
+    by the fused sample + depthwise-convolution operator (reference ``:135-221``)."""
+
+    def __init__(self, weight_shape, in_planes, out_planes, kernel_size=1, stride=1, padding=0,
+                 dilation=1, groups=1, rotation_groups=1, bias=False, rotation_clip=None):
+        super().__init__()
+        assert not bias
+        assert len(weight_shape) >= 2
+        self.kernel_size = kernel_size
+        self.weight_shape = weight_shape
+        self.weight_dilate = 1
+        self.stride = stride
+        self.padding = padding
+        self.dilation = dilation
+        self.out_planes = out_planes
+        self.in_planes = in_planes
+        self.rotation_groups = rotation_groups
+        self.group = groups
+
+        self.rotation_conv = nn.Conv2d(
+            in_planes, rotation_groups * kernel_size * kernel_size * 2,
+            kernel_size, stride, padding, dilation, bias=True)
+        self.rotation_conv.zero_init = True
+        self.rotation_clip = rotation_clip
+
+        self.inner_conv = SampleDepthwise(
+            weight_shape, in_planes, out_planes, kernel_size=kernel_size, stride=stride,
+            padding=padding, dilation=dilation, groups=groups, rotation_groups=rotation_groups,
+            bias=bias)
+
+    def _clip_rotation(self, rotation):
+        clip = self.rotation_clip
+        if isinstance(clip, dict):
+            return rotation.clamp(**clip)
+        if isinstance(clip, (tuple, list)) and len(clip) == 2:
+            # the reference `**`-expands a tuple here (:186-187), which cannot work; read it as (min, max)
+            return rotation.clamp(clip[0], clip[1])
+        if clip == 'scope':
+            centre = rotation.new_tensor(
+                _centred_tap_grid(self.weight_shape, self.kernel_size, self.weight_dilate)
+            ).repeat(self.rotation_groups)[None, :, None, None]
+            coord = (rotation * self.weight_dilate + centre).clamp(0, self.weight_shape[0] - 1)
+            return (coord - centre) / self.weight_dilate
+        raise NotImplementedError(
+            'Expect rotation_clip to be a (min, max) pair, a clamp kwargs dict or "scope", '
+            'but get {}'.format(clip))
+
+    def forward(self, x):
+        rotation = self.rotation_conv(x)
+        if self.rotation_clip is not None:
+            rotation = self._clip_rotation(rotation)
+        if self.weight_dilate != 1:
+            rotation = rotation * self.weight_dilate
+        return self.inner_conv(x, rotation)
+
+
+# refer to local deformable kernel as the default.
+DeformKernel2d = LocalDeformKernel2d
+
+
+class DeformKernelConv2d(nn.Module):
+    """Image-space offsets predicted by ``offset_conv`` feeding the deformable
+    sample + depthwise operator; kernel-space offsets stay zero, as in the
+    reference (``:228-281``, ``rotation = None`` at ``:278``)."""
+
+    def __init__(self, weight_shape, in_planes, out_planes, kernel_size=1, stride=1, padding=0,
+                 dilation=1, groups=1, bias=False, offset_clip=None):
+        super().__init__()
+        assert not bias
+        self.kernel_size = kernel_size
+        self.stride = stride
+        self.padding = padding
+        self.dilation = dilation
+        self.out_planes = out_planes
+        self.in_planes = in_planes
+        self.group = groups
+
+        self.offset_conv = nn.Conv2d(
+            in_planes, kernel_size * kernel_size * 2,
+            kernel_size, stride, padding, dilation, bias=True)
+        self.offset_conv.zero_init = True
+        self.offset_clip = offset_clip
+
+        self.inner_conv = DeformableSampleDepthwise(
+            weight_shape, in_planes, out_planes, kernel_size=kernel_size, stride=stride,
+            padding=padding, dilation=dilation, groups=groups, bias=bias)
+
+    def forward(self, x):
+        offset = self.offset_conv(x)
+        if self.offset_clip is not None:
+            offset = offset.clamp(**self.offset_clip)
+        if self.dilation != 1:
+            offset = offset * self.dilation
+        return self.inner_conv(x, offset, None)

@@ -1,0 +1,138 @@
+"""ctypes binding of ``libdk_hip.so`` (C ABI in ``include/dk_hip.h``).
+
+Takes the place of the reference's two pybind11 extension modules
+(``from .. import filter_sample_depthwise_cuda`` --
+``functions/filter_sample_depthwise.py:14`` -- and ``nd_linear_sample_cuda`` --
+``functions/nd_linear_sample.py:13``).  The library is built in-tree by
+``make -C deformable-kernels_amd/csrc``; there is no fallback: if it is
+missing or an entry point reports an error, the caller gets an exception.
+"""
+import ctypes
+import os
+
+import torch
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libdk_hip.so")
+
+DK_F32, DK_F16, DK_BF16, DK_F64 = 0, 1, 2, 3
+_DTYPES = {torch.float32: DK_F32, torch.float16: DK_F16, torch.bfloat16: DK_BF16, torch.float64: DK_F64}
+
+ND_MAX_DIMS = 8
+
+
+class ConvDesc(ctypes.Structure):
+    _fields_ = [(n, ctypes.c_int32) for n in (
+        "batch", "channel", "in_h", "in_w", "k_h", "k_w", "stride_h", "stride_w",
+        "pad_h", "pad_w", "dil_h", "dil_w", "scope_h", "scope_w", "groups", "dtype")]
+
+
+class NdDesc(ctypes.Structure):
+    _fields_ = [("batch", ctypes.c_int64), ("channel", ctypes.c_int32), ("dims", ctypes.c_int32),
+                ("shape", ctypes.c_int32 * ND_MAX_DIMS), ("dtype", ctypes.c_int32)]
+
+
+class DkError(RuntimeError):
+    pass
+
+
+_P, _SZ = ctypes.c_void_p, ctypes.c_size_t
+_CD, _ND = ctypes.POINTER(ConvDesc), ctypes.POINTER(NdDesc)
+
+# name -> (restype, argtypes); must list every symbol include/dk_hip.h declares
+SIGNATURES = {
+    "dk_version": (ctypes.c_int, []),
+    "dk_status_string": (ctypes.c_char_p, [ctypes.c_int]),
+    "dk_conv_out_size": (ctypes.c_int, [_CD, ctypes.POINTER(ctypes.c_int32), ctypes.POINTER(ctypes.c_int32)]),
+    "dk_sample_depthwise_forward": (ctypes.c_int, [_CD, _P, _P, _P, _P, _P]),
+    "dk_sample_depthwise_backward_data": (ctypes.c_int, [_CD, _P, _P, _P, _P, _P]),
+    "dk_sample_depthwise_backward_filter_workspace": (_SZ, [_CD]),
+    "dk_sample_depthwise_backward_filter": (ctypes.c_int, [_CD, _P, _P, _P, _P, _P, _SZ, _P]),
+    "dk_sample_depthwise_backward_rotation": (ctypes.c_int, [_CD, _P, _P, _P, _P, _P, _P]),
+    "dk_deformable_sample_depthwise_forward": (ctypes.c_int, [_CD, _P, _P, _P, _P, _P, _P]),
+    "dk_deformable_sample_depthwise_backward_data_workspace": (_SZ, [_CD]),
+    "dk_deformable_sample_depthwise_backward_data": (ctypes.c_int, [_CD, _P, _P, _P, _P, _P, _P, _SZ, _P]),
+    "dk_deformable_sample_depthwise_backward_filter_workspace": (_SZ, [_CD]),
+    "dk_deformable_sample_depthwise_backward_filter": (ctypes.c_int, [_CD, _P, _P, _P, _P, _P, _P, _SZ, _P]),
+    "dk_deformable_sample_depthwise_backward_offset": (ctypes.c_int, [_CD, _P, _P, _P, _P, _P, _P, _P]),
+    "dk_deformable_sample_depthwise_backward_rotation": (ctypes.c_int, [_CD, _P, _P, _P, _P, _P, _P, _P]),
+    "dk_nd_linear_sample_forward": (ctypes.c_int, [_ND, _P, _P, _P, _P]),
+    "dk_nd_linear_sample_backward_data_workspace": (_SZ, [_ND]),
+    "dk_nd_linear_sample_backward_data": (ctypes.c_int, [_ND, _P, _P, _P, _P, _SZ, _P]),
+    "dk_nd_linear_sample_backward_coord": (ctypes.c_int, [_ND, _P, _P, _P, _P, _P]),
+}
+
+_lib = None
+
+
+def lib():
+    """The loaded library; raises if it has not been built."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise DkError(
+                "libdk_hip.so not found at %s -- build it with "
+                "`make -C deformable-kernels_amd/csrc` (there is no CPU or eager fallback)" % LIB_PATH)
+        handle = ctypes.CDLL(LIB_PATH)
+        for name, (res, args) in SIGNATURES.items():
+            fn = getattr(handle, name)
+            fn.restype, fn.argtypes = res, args
+        _lib = handle
+    return _lib
+
+
+def check(status, what):
+    if status != 0:
+        raise DkError("%s failed: %s (status %d)" % (what, lib().dk_status_string(status).decode(), status))
+
+
+def dtype_tag(t):
+    try:
+        return _DTYPES[t.dtype]
+    except KeyError:
+        raise TypeError("unsupported dtype %s (float32, float16, bfloat16, float64)" % t.dtype)
+
+
+def stream_ptr(t):
+    return ctypes.c_void_p(torch.cuda.current_stream(t.device).cuda_stream)
+
+
+def ptr(t):
+    return ctypes.c_void_p(t.data_ptr()) if t is not None else ctypes.c_void_p(0)
+
+
+def require_gpu(*tensors):
+    """The operators exist on the GPU only, as in the reference
+    (``functions/filter_sample_depthwise.py:43-44``)."""
+    for t in tensors:
+        if not t.is_cuda:
+            raise NotImplementedError("deformable-kernel operators are implemented for GPU tensors only")
+    dev, dt = tensors[0].device, tensors[0].dtype
+    for t in tensors[1:]:
+        if t.device != dev:
+            raise ValueError("all tensors must be on the same device")
+        if t.dtype != dt:
+            raise TypeError("all tensors must have the same dtype (got %s and %s)" % (dt, t.dtype))
+
+
+def workspace(nbytes, device):
+    if nbytes == 0:
+        return None, 0
+    buf = torch.empty(nbytes, dtype=torch.uint8, device=device)
+    return buf, nbytes
+
+
+def conv_desc(input, weight, kernel_size, stride, padding, dilation, rotation_groups):
+    return ConvDesc(
+        input.size(0), input.size(1), input.size(2), input.size(3),
+        int(kernel_size[0]), int(kernel_size[1]), int(stride[0]), int(stride[1]),
+        int(padding[0]), int(padding[1]), int(dilation[0]), int(dilation[1]),
+        weight.size(2), weight.size(3), int(rotation_groups), dtype_tag(input))
+
+
+def nd_desc(data, coord):
+    dims = data.dim() - 1
+    if dims < 1 or dims > ND_MAX_DIMS:
+        raise ValueError("nd_linear_sample supports 1..%d sampling dimensions, got %d" % (ND_MAX_DIMS, dims))
+    shape = (ctypes.c_int32 * ND_MAX_DIMS)(*(list(data.shape[1:]) + [1] * (ND_MAX_DIMS - dims)))
+    return NdDesc(coord.size(0), data.size(0), dims, shape, dtype_tag(data))

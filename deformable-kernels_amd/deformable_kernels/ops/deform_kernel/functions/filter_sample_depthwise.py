@@ -1,0 +1,211 @@
+"""Autograd Functions of the depthwise deformable-kernel operators.
+
+Same call signatures, tensor layouts and gradient set as the reference's
+``SampleDepthwiseFunction`` and ``DeformableSampleDepthwiseFunction``
+(``functions/filter_sample_depthwise.py:19-102`` and ``:105-206``); the bodies
+call the C ABI of ``libdk_hip.so`` instead of the CUDA extension.
+
+Differences a user can observe:
+  * ``backward`` returns one gradient slot per forward argument (the
+    reference returns one too few -- ``:87`` and ``:191`` -- which current
+    PyTorch rejects);
+  * tensors are validated (device, dtype, shape) and a failing native call
+    raises instead of printing;
+  * bfloat16 is accepted; fp16/bf16 accumulate in fp32;
+  * the ``apex.amp.float_function`` wrapper (``:209-211``) is replaced by an
+    autocast-aware cast to fp32, apex not being a dependency.
+"""
+import torch
+from torch.autograd import Function
+
+from .. import _lib
+
+__all__ = ['sample_depthwise', 'deform_sample_depthwise']
+
+
+def _output_size(input, kernel_size, stride, padding, dilation):
+    # reference functions/filter_sample_depthwise.py:90-102
+    output_size = (input.size(0), input.size(1))
+    for d in range(input.dim() - 2):
+        in_size = input.size(d + 2)
+        pad = padding[d]
+        kernel = dilation[d] * (kernel_size[d] - 1) + 1
+        stride_ = stride[d]
+        output_size += ((in_size + (2 * pad) - kernel) // stride_ + 1, )
+    if not all(map(lambda s: s > 0, output_size)):
+        raise ValueError(
+            "convolution input is too small (output would be {})".format(
+                'x'.join(map(str, output_size))))
+    return output_size
+
+
+def _check_shapes(input, rotation, weight, out_size, kernel_size, rotation_groups, offset=None):
+    if input.dim() != 4 or weight.dim() != 4:
+        raise ValueError("input must be [N, C, H, W] and weight [C, 1, S_h, S_w]")
+    c = input.size(1)
+    if weight.size(0) != c or weight.size(1) != 1:
+        raise ValueError("weight must be [C, 1, S_h, S_w] with C = %d, got %s" % (c, tuple(weight.shape)))
+    if rotation_groups < 1 or c % rotation_groups != 0:
+        raise ValueError("channels (%d) must be divisible by rotation_groups (%d)" % (c, rotation_groups))
+    taps2 = kernel_size[0] * kernel_size[1] * 2
+    want = (input.size(0), rotation_groups * taps2, out_size[2], out_size[3])
+    if tuple(rotation.shape) != want:
+        raise ValueError("rotation must be %s, got %s" % (want, tuple(rotation.shape)))
+    if offset is not None:
+        want = (input.size(0), taps2, out_size[2], out_size[3])
+        if tuple(offset.shape) != want:
+            raise ValueError("offset must be %s, got %s" % (want, tuple(offset.shape)))
+
+
+class SampleDepthwiseFunction(Function):
+    @staticmethod
+    def forward(
+        ctx,
+        input,
+        rotation,
+        weight,
+        kernel_size=(3, 3),
+        stride=(1, 1),
+        padding=(1, 1),
+        dilation=(1, 1),
+        rotation_groups=1,
+    ):
+        ctx.kernel_size = kernel_size
+        ctx.stride = stride
+        ctx.padding = padding
+        ctx.dilation = dilation
+        ctx.rotation_groups = rotation_groups
+
+        _lib.require_gpu(input, rotation, weight)
+        out_size = _output_size(input, kernel_size, stride, padding, dilation)
+        _check_shapes(input, rotation, weight, out_size, kernel_size, rotation_groups)
+        input, rotation, weight = input.contiguous(), rotation.contiguous(), weight.contiguous()
+        ctx.save_for_backward(input, rotation, weight)
+        output = input.new_empty(out_size)
+        desc = _lib.conv_desc(input, weight, kernel_size, stride, padding, dilation, rotation_groups)
+        with torch.cuda.device(input.device):
+            _lib.check(_lib.lib().dk_sample_depthwise_forward(
+                desc, _lib.ptr(input), _lib.ptr(rotation), _lib.ptr(weight), _lib.ptr(output),
+                _lib.stream_ptr(input)), "sample_depthwise forward")
+        return output
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        input, rotation, weight = ctx.saved_tensors
+        grad_input = grad_rotation = grad_weight = None
+        _lib.require_gpu(grad_output, input)
+        grad_output = grad_output.contiguous()
+        desc = _lib.conv_desc(input, weight, ctx.kernel_size, ctx.stride, ctx.padding, ctx.dilation,
+                              ctx.rotation_groups)
+        L = _lib.lib()
+        with torch.cuda.device(input.device):
+            s = _lib.stream_ptr(input)
+            if ctx.needs_input_grad[0]:
+                grad_input = torch.empty_like(input)
+                _lib.check(L.dk_sample_depthwise_backward_data(
+                    desc, _lib.ptr(grad_output), _lib.ptr(rotation), _lib.ptr(weight),
+                    _lib.ptr(grad_input), s), "sample_depthwise backward_data")
+            if ctx.needs_input_grad[1]:
+                grad_rotation = torch.empty_like(rotation)
+                _lib.check(L.dk_sample_depthwise_backward_rotation(
+                    desc, _lib.ptr(grad_output), _lib.ptr(input), _lib.ptr(rotation), _lib.ptr(weight),
+                    _lib.ptr(grad_rotation), s), "sample_depthwise backward_rotation")
+            if ctx.needs_input_grad[2]:
+                grad_weight = torch.empty_like(weight)
+                ws, nbytes = _lib.workspace(L.dk_sample_depthwise_backward_filter_workspace(desc), input.device)
+                _lib.check(L.dk_sample_depthwise_backward_filter(
+                    desc, _lib.ptr(grad_output), _lib.ptr(input), _lib.ptr(rotation),
+                    _lib.ptr(grad_weight), _lib.ptr(ws), nbytes, s), "sample_depthwise backward_filter")
+        return (grad_input, grad_rotation, grad_weight,) + (None,) * 5
+
+
+class DeformableSampleDepthwiseFunction(Function):
+    @staticmethod
+    def forward(
+        ctx,
+        input,
+        offset,
+        rotation,
+        weight,
+        kernel_size=(3, 3),
+        stride=(1, 1),
+        padding=(1, 1),
+        dilation=(1, 1),
+        rotation_groups=1,
+    ):
+        ctx.kernel_size = kernel_size
+        ctx.stride = stride
+        ctx.padding = padding
+        ctx.dilation = dilation
+        ctx.rotation_groups = rotation_groups
+
+        _lib.require_gpu(input, offset, rotation, weight)
+        out_size = _output_size(input, kernel_size, stride, padding, dilation)
+        _check_shapes(input, rotation, weight, out_size, kernel_size, rotation_groups, offset)
+        input, offset = input.contiguous(), offset.contiguous()
+        rotation, weight = rotation.contiguous(), weight.contiguous()
+        ctx.save_for_backward(input, offset, rotation, weight)
+        output = input.new_empty(out_size)
+        desc = _lib.conv_desc(input, weight, kernel_size, stride, padding, dilation, rotation_groups)
+        with torch.cuda.device(input.device):
+            _lib.check(_lib.lib().dk_deformable_sample_depthwise_forward(
+                desc, _lib.ptr(input), _lib.ptr(offset), _lib.ptr(rotation), _lib.ptr(weight),
+                _lib.ptr(output), _lib.stream_ptr(input)), "deform_sample_depthwise forward")
+        return output
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        input, offset, rotation, weight = ctx.saved_tensors
+        grad_input = grad_offset = grad_rotation = grad_weight = None
+        _lib.require_gpu(grad_output, input)
+        grad_output = grad_output.contiguous()
+        desc = _lib.conv_desc(input, weight, ctx.kernel_size, ctx.stride, ctx.padding, ctx.dilation,
+                              ctx.rotation_groups)
+        L = _lib.lib()
+        p = _lib.ptr
+        with torch.cuda.device(input.device):
+            s = _lib.stream_ptr(input)
+            if ctx.needs_input_grad[0]:
+                grad_input = torch.empty_like(input)
+                ws, nbytes = _lib.workspace(
+                    L.dk_deformable_sample_depthwise_backward_data_workspace(desc), input.device)
+                _lib.check(L.dk_deformable_sample_depthwise_backward_data(
+                    desc, p(grad_output), p(offset), p(rotation), p(weight), p(grad_input),
+                    p(ws), nbytes, s), "deform_sample_depthwise backward_data")
+            if ctx.needs_input_grad[1]:
+                grad_offset = torch.empty_like(offset)
+                _lib.check(L.dk_deformable_sample_depthwise_backward_offset(
+                    desc, p(grad_output), p(input), p(offset), p(rotation), p(weight),
+                    p(grad_offset), s), "deform_sample_depthwise backward_offset")
+            if ctx.needs_input_grad[2]:
+                grad_rotation = torch.empty_like(rotation)
+                _lib.check(L.dk_deformable_sample_depthwise_backward_rotation(
+                    desc, p(grad_output), p(input), p(offset), p(rotation), p(weight),
+                    p(grad_rotation), s), "deform_sample_depthwise backward_rotation")
+            if ctx.needs_input_grad[3]:
+                grad_weight = torch.empty_like(weight)
+                ws, nbytes = _lib.workspace(
+                    L.dk_deformable_sample_depthwise_backward_filter_workspace(desc), input.device)
+                _lib.check(L.dk_deformable_sample_depthwise_backward_filter(
+                    desc, p(grad_output), p(input), p(offset), p(rotation), p(grad_weight),
+                    p(ws), nbytes, s), "deform_sample_depthwise backward_filter")
+        return (grad_input, grad_offset, grad_rotation, grad_weight,) + (None,) * 5
+
+
+def _float_function(fn):
+    """Stand-in for ``apex.amp.float_function`` (reference ``:209-211``): inside an
+    autocast region the floating-point tensor arguments are cast to fp32 and the
+    op runs with autocast off; outside one it is the identity wrapper."""
+    def wrapper(*args):
+        if torch.is_autocast_enabled():
+            args = tuple(a.float() if torch.is_tensor(a) and a.is_floating_point() else a for a in args)
+            with torch.autocast(device_type="cuda", enabled=False):
+                return fn(*args)
+        return fn(*args)
+    wrapper.__wrapped__ = fn
+    return wrapper
+
+
+# register as fp32 functions.
+sample_depthwise = _float_function(SampleDepthwiseFunction.apply)
+deform_sample_depthwise = _float_function(DeformableSampleDepthwiseFunction.apply)

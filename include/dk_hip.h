@@ -1,0 +1,185 @@
+/*
+ * dk_hip.h -- C ABI of libdk_hip.so: the deformable-kernel operators as
+ * hand-written gfx950 (MI355X) HIP kernels.
+ *
+ * One entry point per function of the reference's two pybind11 extension
+ * modules (the Python -> native boundary of the operator path):
+ *
+ *   filter_sample_depthwise_cuda   csrc/filter_sample_depthwise_cuda.cpp:540-569
+ *   nd_linear_sample_cuda          csrc/nd_linear_sample_cuda.cpp:67-74
+ *
+ * Conventions shared by every entry point
+ *   - plain C: raw device pointers, sizes and a descriptor struct; no torch
+ *     or HIP types appear in a signature (`stream` is a hipStream_t passed
+ *     as void*, NULL = the default stream);
+ *   - all tensors are dense, contiguous, row-major (NCHW) and of the one
+ *     dtype named in the descriptor; the caller owns all memory, including
+ *     the optional workspace, whose size the matching *_workspace() query
+ *     returns; the library itself never allocates;
+ *   - every output buffer is OVERWRITTEN (no pre-zeroing is needed; the
+ *     reference's filter/data gradients accumulate atomically into buffers
+ *     its Python caller zero-fills -- functions/filter_sample_depthwise.py:64-80);
+ *   - calls are asynchronous on `stream`, thread-safe and hold no global
+ *     mutable state;
+ *   - the return value is DK_OK (0) or a negative dk_status; nothing is
+ *     launched when an argument is rejected.  (The reference validates
+ *     nothing and always returns 1 -- filter_sample_depthwise_cuda.cpp:61.)
+ *   - fp16 / bf16 tensors are computed in fp32 registers and accumulators.
+ */
+#ifndef DK_HIP_H
+#define DK_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef enum {
+  DK_OK = 0,
+  DK_ERR_NULL_POINTER = -1,   /* a required pointer (descriptor, tensor) is NULL        */
+  DK_ERR_BAD_SHAPE = -2,      /* non-positive size, output would be empty or negative,  */
+                              /* channel not divisible by rotation groups               */
+  DK_ERR_BAD_DTYPE = -3,      /* dtype tag not one of dk_dtype                          */
+  DK_ERR_TOO_LARGE = -4,      /* a tensor has >= 2^31 elements (32-bit plane indexing)  */
+  DK_ERR_WORKSPACE = -5,      /* workspace NULL or smaller than the *_workspace() query */
+  DK_ERR_LAUNCH = -6,         /* the HIP runtime refused the launch                     */
+  DK_ERR_UNSUPPORTED = -7     /* e.g. more than DK_ND_MAX_DIMS sampling dimensions      */
+} dk_status;
+
+typedef enum { DK_F32 = 0, DK_F16 = 1, DK_BF16 = 2, DK_F64 = 3 } dk_dtype;
+
+/* Geometry of one depthwise deformable-kernel layer: the fields the
+ * reference packs into SampleDepthwiseArgs (csrc/filter_sample_depthwise_cuda.h:1-28)
+ * from the tensor sizes and the eleven ints of each pybind call; out_h/out_w
+ * are derived inside the library by the rule of filter_sample_depthwise_cuda.cpp:42-43:
+ *   out = (in + 2*pad - (dil*(k-1)+1)) / stride + 1
+ *
+ * Tensor layouts
+ *   input     [batch, channel, in_h, in_w]
+ *   filter    [channel, 1, scope_h, scope_w]     the per-channel scope tile
+ *   rotation  [batch, groups*k_h*k_w*2, out_h, out_w]  kernel-space offsets, channel index
+ *             g*(k_h*k_w*2) + (f_h*k_w + f_w)*2 + dir, dir 0 = h, 1 = w; channel c uses g = c % groups
+ *   offset    [batch, k_h*k_w*2, out_h, out_w]   image-space offsets, same (tap, dir) order
+ *   output    [batch, channel, out_h, out_w]
+ */
+typedef struct dk_conv_desc {
+  int32_t batch, channel, in_h, in_w;
+  int32_t k_h, k_w;
+  int32_t stride_h, stride_w;
+  int32_t pad_h, pad_w;
+  int32_t dil_h, dil_w;
+  int32_t scope_h, scope_w;
+  int32_t groups;           /* rotation groups ("sampling_group") */
+  int32_t dtype;            /* dk_dtype of every tensor of the call */
+} dk_conv_desc;
+
+/* Output extent for the descriptor, or a negative dk_status. */
+int dk_conv_out_size(const dk_conv_desc *desc, int32_t *out_h, int32_t *out_w);
+
+/* ---- local deformable kernel: kernel-space offsets only ------------------- */
+
+/* sample_depthwise_forward_cuda (filter_sample_depthwise_cuda.cpp:8-62). */
+int dk_sample_depthwise_forward(const dk_conv_desc *desc, const void *input, const void *rotation,
+                                const void *filter, void *output, void *stream);
+
+/* sample_depthwise_backward_data_cuda (filter_sample_depthwise_cuda.cpp:64-119).
+ * `input` is not needed for this gradient and is not an argument. */
+int dk_sample_depthwise_backward_data(const dk_conv_desc *desc, const void *out_grad,
+                                      const void *rotation, const void *filter, void *in_grad,
+                                      void *stream);
+
+/* sample_depthwise_backward_filter_cuda (filter_sample_depthwise_cuda.cpp:121-176).
+ * Needs a workspace for per-workgroup partial sums (reduced without global atomics). */
+size_t dk_sample_depthwise_backward_filter_workspace(const dk_conv_desc *desc);
+int dk_sample_depthwise_backward_filter(const dk_conv_desc *desc, const void *out_grad,
+                                        const void *input, const void *rotation,
+                                        void *filter_grad, void *workspace,
+                                        size_t workspace_bytes, void *stream);
+
+/* sample_depthwise_backward_rotation_cuda (filter_sample_depthwise_cuda.cpp:178-235). */
+int dk_sample_depthwise_backward_rotation(const dk_conv_desc *desc, const void *out_grad,
+                                          const void *input, const void *rotation,
+                                          const void *filter, void *rotation_grad, void *stream);
+
+/* ---- deformable kernel with image-space offsets ---------------------------- */
+
+/* deformable_sample_depthwise_forward_cuda (filter_sample_depthwise_cuda.cpp:237-294). */
+int dk_deformable_sample_depthwise_forward(const dk_conv_desc *desc, const void *input,
+                                           const void *offset, const void *rotation,
+                                           const void *filter, void *output, void *stream);
+
+/* deformable_sample_depthwise_backward_data_cuda (filter_sample_depthwise_cuda.cpp:296-354). */
+size_t dk_deformable_sample_depthwise_backward_data_workspace(const dk_conv_desc *desc);
+int dk_deformable_sample_depthwise_backward_data(const dk_conv_desc *desc, const void *out_grad,
+                                                 const void *offset, const void *rotation,
+                                                 const void *filter, void *in_grad,
+                                                 void *workspace, size_t workspace_bytes,
+                                                 void *stream);
+
+/* deformable_sample_depthwise_backward_filter_cuda (filter_sample_depthwise_cuda.cpp:356-414). */
+size_t dk_deformable_sample_depthwise_backward_filter_workspace(const dk_conv_desc *desc);
+int dk_deformable_sample_depthwise_backward_filter(const dk_conv_desc *desc, const void *out_grad,
+                                                   const void *input, const void *offset,
+                                                   const void *rotation, void *filter_grad,
+                                                   void *workspace, size_t workspace_bytes,
+                                                   void *stream);
+
+/* deformable_sample_depthwise_backward_offset_cuda (filter_sample_depthwise_cuda.cpp:416-476). */
+int dk_deformable_sample_depthwise_backward_offset(const dk_conv_desc *desc, const void *out_grad,
+                                                   const void *input, const void *offset,
+                                                   const void *rotation, const void *filter,
+                                                   void *offset_grad, void *stream);
+
+/* deformable_sample_depthwise_backward_rotation_cuda (filter_sample_depthwise_cuda.cpp:478-538). */
+int dk_deformable_sample_depthwise_backward_rotation(const dk_conv_desc *desc,
+                                                     const void *out_grad, const void *input,
+                                                     const void *offset, const void *rotation,
+                                                     const void *filter, void *rotation_grad,
+                                                     void *stream);
+
+/* ---- N-d linear sample -------------------------------------------------------
+ * data [channel, shape[0..dims-1]], coord [batch, dims] in absolute index units,
+ * output [batch, channel].  The reference passes `shape` as a device tensor of the
+ * data's floating dtype (functions/nd_linear_sample.py:22); here it is host
+ * integers in the descriptor, which removes a host-to-device copy per call. */
+#define DK_ND_MAX_DIMS 8
+typedef struct dk_nd_desc {
+  int64_t batch;                    /* number of sample points              */
+  int32_t channel;
+  int32_t dims;                     /* 1..DK_ND_MAX_DIMS                    */
+  int32_t shape[DK_ND_MAX_DIMS];
+  int32_t dtype;
+} dk_nd_desc;
+
+/* nd_linear_sample_forward_cuda (nd_linear_sample_cuda.cpp:10-26). */
+int dk_nd_linear_sample_forward(const dk_nd_desc *desc, const void *data, const void *coord,
+                                void *output, void *stream);
+
+/* nd_linear_sample_backward_data_cuda (nd_linear_sample_cuda.cpp:29-45); in_grad is
+ * fully written (the reference zero-fills it in C++ and scatters atomically).  fp16 / bf16
+ * gradients are accumulated in an fp32 workspace of the data's element count. */
+size_t dk_nd_linear_sample_backward_data_workspace(const dk_nd_desc *desc);
+int dk_nd_linear_sample_backward_data(const dk_nd_desc *desc, const void *out_grad,
+                                      const void *coord, void *in_grad, void *workspace,
+                                      size_t workspace_bytes, void *stream);
+
+/* nd_linear_sample_backward_coord_cuda (nd_linear_sample_cuda.cpp:47-64) fused with the
+ * `.sum(2)` its Python caller applies (functions/nd_linear_sample.py:48-55):
+ * coord_grad is [batch, dims], already summed over channels. */
+int dk_nd_linear_sample_backward_coord(const dk_nd_desc *desc, const void *out_grad,
+                                       const void *data, const void *coord, void *coord_grad,
+                                       void *stream);
+
+/* ---- misc ------------------------------------------------------------------- */
+
+const char *dk_status_string(int status);
+
+/* Library version, (major << 16) | minor. */
+int dk_version(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* DK_HIP_H */

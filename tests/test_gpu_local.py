@@ -1,0 +1,173 @@
+"""GPU parity of the local deformable-kernel operator (forward, grad-input,
+grad-rotation, grad-filter) against the CPU oracle, through the Python
+Functions and therefore through the C ABI of libdk_hip.so.
+
+Tolerances (relative to the largest magnitude of the expected tensor):
+  fp32: forward and grad-input 1e-5 against the fp32 oracle; grad-rotation and
+        grad-filter 1e-4 against the fp64 oracle (summation order differs);
+  fp64: 1e-11 everywhere;
+  fp16 / bf16: 1e-2 against the fp32 oracle evaluated on the rounded inputs.
+"""
+import numpy as np
+import pytest
+import torch
+
+from _cases import make_local, rel_err
+from oracle import dk_oracle as orc
+
+pytestmark = pytest.mark.gpu
+
+# N, C, H, W, k, S, stride, pad, dil, groups, rot_std
+TUNED = [
+    (2, 32, 28, 28, 3, (4, 4), 1, 1, 1, 1, 0.5),    # BASELINE config 1
+    (3, 20, 17, 23, 3, (4, 4), 1, 1, 1, 1, 1.0),    # ragged sizes, partial tiles
+    (2, 24, 19, 19, 3, (4, 4), 2, 1, 1, 1, 1.0),    # stride 2
+    (2, 12, 15, 14, 3, (4, 4), 1, 2, 2, 3, 1.0),    # dilation 2, rotation groups 3
+    (2, 16, 13, 13, 3, (3, 3), 1, 1, 1, 1, 1.0),    # scope == kernel
+    (1, 16, 13, 12, 3, (5, 5), 1, 0, 1, 2, 1.5),    # scope 5, no padding
+    (1, 200, 9, 9, 3, (4, 4), 1, 1, 1, 1, 2.0),     # many channels, many samples outside the scope
+]
+GENERIC = [
+    (2, 6, 9, 8, (5, 3), (7, 4), (1, 2), (2, 0), 1, 3, 0.7),
+    (1, 4, 10, 11, 3, (5, 3), 1, 2, 2, 1, 1.5),
+    (2, 5, 6, 5, 1, (2, 2), 1, 0, 1, 1, 0.6),
+    (1, 4, 8, 8, 2, (4, 4), 2, 0, 1, 2, 0.5),
+]
+
+
+def _run(case, dtype, seed=0):
+    from deformable_kernels.ops.deform_kernel.functions import sample_depthwise
+    N, C, H, W, k, S, s, p, d, G, rs = case
+    x, wt, rot, gout, cfg = make_local(N, C, H, W, k, S, s, p, d, G, rs, seed=seed, dtype=dtype)
+    dev = torch.device("cuda:0")
+    xg, rg, wg = [t.to(dev).requires_grad_() for t in (x, rot, wt)]
+    out = sample_depthwise(xg, rg, wg, cfg["kernel_size"], cfg["stride"], cfg["padding"], cfg["dilation"],
+                           cfg["groups"])
+    out.backward(gout.to(dev))
+    torch.cuda.synchronize()
+    got = [t.detach().cpu() for t in (out, xg.grad, rg.grad, wg.grad)]
+    return (x, wt, rot, gout, cfg), got
+
+
+def _oracle(inputs, np_dtype):
+    x, wt, rot, gout, cfg = inputs
+    a = [t.to(torch.float64).numpy().astype(np_dtype) for t in (x, rot, wt, gout)]
+    out = orc.sample_depthwise_forward(a[0], a[1], a[2], **cfg)
+    gin, grot, gw = orc.sample_depthwise_backward(a[3], a[0], a[1], a[2], **cfg)
+    return out, gin, grot, gw
+
+
+@pytest.mark.parametrize("case", TUNED + GENERIC)
+def test_fp32_matches_oracle(case):
+    inputs, got = _run(case, torch.float32)
+    o32 = _oracle(inputs, np.float32)
+    o64 = _oracle(inputs, np.float64)
+    assert got[0].dtype == torch.float32
+    assert rel_err(got[0], o32[0]) < 1e-5, "forward"
+    assert rel_err(got[1], o32[1]) < 1e-5, "grad input"
+    assert rel_err(got[2], o64[2]) < 1e-4, "grad rotation"
+    assert rel_err(got[3], o64[3]) < 1e-4, "grad filter"
+
+
+@pytest.mark.parametrize("case", TUNED[:4] + GENERIC[:2])
+def test_fp64_matches_oracle(case):
+    inputs, got = _run(case, torch.float64)
+    want = _oracle(inputs, np.float64)
+    for g, w, name in zip(got, want, ("forward", "grad input", "grad rotation", "grad filter")):
+        assert g.dtype == torch.float64
+        assert rel_err(g, w) < 1e-11, name
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("case", TUNED[:5] + GENERIC[:2])
+def test_half_precisions_match_fp32_oracle(case, dtype):
+    inputs, got = _run(case, dtype)
+    want = _oracle(inputs, np.float32)  # the inputs are already rounded to `dtype`
+    for g, w, name in zip(got, want, ("forward", "grad input", "grad rotation", "grad filter")):
+        assert g.dtype == dtype
+        assert rel_err(g.float(), w) < 1e-2, name
+
+
+def test_taps_outside_the_scope_and_nan_free_borders():
+    # rotations that push every tap outside (-1, S): all four results are exact zeros
+    from deformable_kernels.ops.deform_kernel.functions import sample_depthwise
+    x, wt, rot, gout, cfg = make_local(2, 8, 10, 10, 3, (4, 4), 1, 1, 1, 1, 0.0, seed=3)
+    dev = torch.device("cuda:0")
+    for shift in (-10.0, 10.0, -3.5, 4.0):
+        xg, rg, wg = [t.to(dev).requires_grad_() for t in (x, rot + shift, wt)]
+        out = sample_depthwise(xg, rg, wg, (3, 3), (1, 1), (1, 1), (1, 1), 1)
+        out.backward(gout.to(dev))
+        for t in (out, xg.grad, rg.grad, wg.grad):
+            assert torch.count_nonzero(t).item() == 0
+
+
+def test_non_contiguous_inputs_and_needs_input_grad_gating():
+    from deformable_kernels.ops.deform_kernel.functions import sample_depthwise
+    x, wt, rot, gout, cfg = make_local(2, 8, 12, 10, 3, (4, 4), 1, 1, 1, 1, 0.8, seed=4)
+    dev = torch.device("cuda:0")
+    xt = x.transpose(2, 3).contiguous().transpose(2, 3).to(dev)  # same values, strided layout
+    assert not xt.is_contiguous()
+    rg = rot.to(dev).requires_grad_()
+    out = sample_depthwise(xt, rg, wt.to(dev), (3, 3), (1, 1), (1, 1), (1, 1), 1)
+    out.backward(gout.to(dev))
+    want = orc.sample_depthwise_forward(x.numpy(), rot.numpy(), wt.numpy(), **cfg)
+    _, grot, _ = orc.sample_depthwise_backward(gout.double().numpy(), x.double().numpy(), rot.double().numpy(),
+                                               wt.double().numpy(), **cfg)
+    assert rel_err(out.detach().cpu(), want) < 1e-5
+    assert rel_err(rg.grad.cpu(), grot) < 1e-4
+
+
+def test_runs_on_a_side_stream_and_empty_batch():
+    from deformable_kernels.ops.deform_kernel.functions import sample_depthwise
+    x, wt, rot, gout, cfg = make_local(2, 8, 12, 10, 3, (4, 4), 1, 1, 1, 1, 0.8, seed=5)
+    dev = torch.device("cuda:0")
+    xg, rg, wg = x.to(dev), rot.to(dev), wt.to(dev)
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    with torch.cuda.stream(side):
+        out = sample_depthwise(xg, rg, wg, (3, 3), (1, 1), (1, 1), (1, 1), 1)
+    side.synchronize()
+    want = orc.sample_depthwise_forward(x.numpy(), rot.numpy(), wt.numpy(), **cfg)
+    assert rel_err(out.cpu(), want) < 1e-5
+    # an empty batch is rejected by the output-size rule, as in the reference
+    # (functions/filter_sample_depthwise.py:98-101 tests every output extent, batch included)
+    with pytest.raises(ValueError):
+        sample_depthwise(xg[:0], rg[:0], wg, (3, 3), (1, 1), (1, 1), (1, 1), 1)
+
+
+def test_headline_shape_properties_at_full_size():
+    """BASELINE config 2 (N=64, C=144, 56x56, k=3, scope 4x4, fp32) at full size: the oracle is
+    run on a slice of images; the rest is covered by size-independent properties -- batch
+    independence, linearity in the input, and <gout, F(x)> = <grad_input, x>."""
+    from deformable_kernels.ops.deform_kernel.functions import sample_depthwise
+    N, C = 64, 144
+    x, wt, rot, gout, cfg = make_local(N, C, 56, 56, 3, (4, 4), 1, 1, 1, 1, 1.0, seed=0)
+    dev = torch.device("cuda:0")
+    xg, rg, wg = [t.to(dev).requires_grad_() for t in (x, rot, wt)]
+    args = ((3, 3), (1, 1), (1, 1), (1, 1), 1)
+    out = sample_depthwise(xg, rg, wg, *args)
+    out.backward(gout.to(dev))
+    torch.cuda.synchronize()
+    # oracle on images {0, 37, 63}
+    for n in (0, 37, 63):
+        sl = slice(n, n + 1)
+        want = orc.sample_depthwise_forward(x[sl].numpy(), rot[sl].numpy(), wt.numpy(), **cfg)
+        gin, grot, _ = orc.sample_depthwise_backward(
+            gout[sl].double().numpy(), x[sl].double().numpy(), rot[sl].double().numpy(), wt.double().numpy(), **cfg)
+        assert rel_err(out[sl].detach().cpu(), want) < 1e-5
+        assert rel_err(xg.grad[sl].cpu(), gin) < 1e-5
+        assert rel_err(rg.grad[sl].cpu(), grot) < 1e-4
+    # grad filter: full batch against the fp64 oracle (a few seconds of CPU)
+    _, _, gw = orc.sample_depthwise_backward(gout.double().numpy(), x.double().numpy(), rot.double().numpy(),
+                                             wt.double().numpy(), **cfg)
+    assert rel_err(wg.grad.cpu(), gw) < 1e-4
+    # linearity in the input
+    with torch.no_grad():
+        x2 = torch.randn_like(xg)
+        lhs = sample_depthwise(2 * xg + 3 * x2, rg, wg, *args)
+        rhs = 2 * out + 3 * sample_depthwise(x2, rg, wg, *args)
+        assert rel_err(lhs.cpu(), rhs.cpu()) < 1e-5
+        # adjoint identity in fp64 accumulation
+        a = (gout.to(dev).double() * out.double()).sum().item()
+        b = (xg.grad.double() * xg.double()).sum().item()
+        assert abs(a - b) < 1e-6 * max(abs(a), 1.0)
