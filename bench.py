@@ -61,6 +61,7 @@ def main():
     ap.add_argument("--workload", default="cfg2", choices=sorted(WORKLOADS))
     ap.add_argument("--dtype", default="fp32", choices=sorted(DTYPES))
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--kernels", default="", help="comma list restricting the per-kernel timing (tuning aid)")
     a = ap.parse_args()
     if a.gpus != 1:
         sys.exit("bench.py measures one GPU only: every box of this build has one GPU and no "
@@ -108,6 +109,10 @@ def main():
                "grad_filter": k_grad_filter}
 
     def step():
+        if a.kernels:  # tuning aid: time only the named entry points
+            for name in a.kernels.split(","):
+                kernels[name]()
+            return
         k_forward()
         k_grad_input()
         k_grad_rotation()
@@ -125,7 +130,10 @@ def main():
     # per-entry-point launch duration: events on the stream the kernels are launched on
     per_kernel_us = {}
     reps = max(a.steps, 20)
+    only = [k for k in a.kernels.split(",") if k]
     for name, fn in kernels.items():
+        if only and name not in only:
+            continue
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         fn()
         e0.record()

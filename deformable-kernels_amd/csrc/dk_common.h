@@ -86,7 +86,7 @@ struct ScopeTap {
 
 template <typename CT>
 __device__ __forceinline__ ScopeTap<CT> make_scope_tap(CT h, CT w, int scope_h, int scope_w,
-                                                       int row_stride) {
+                                                       int row_stride, int cell_scale = 1) {
   ScopeTap<CT> t;
   const bool inside = (h > CT(-1)) && (w > CT(-1)) && (h < CT(scope_h)) && (w < CT(scope_w));
   const CT hf = floor(h), wf = floor(w);
@@ -94,7 +94,7 @@ __device__ __forceinline__ ScopeTap<CT> make_scope_tap(CT h, CT w, int scope_h, 
   const CT hh = CT(1) - lh, hw = CT(1) - lw;
   const int hl = inside ? static_cast<int>(hf) : -1;
   const int wl = inside ? static_cast<int>(wf) : -1;
-  t.cell = (hl + 1) * row_stride + (wl + 1);
+  t.cell = ((hl + 1) * row_stride + (wl + 1)) * cell_scale;
   t.c00 = inside ? hh * hw : CT(0);
   t.c01 = inside ? hh * lw : CT(0);
   t.c10 = inside ? lh * hw : CT(0);
@@ -143,5 +143,48 @@ __device__ __forceinline__ ImageTap<CT> make_image_tap(CT h, CT w, int H, int W)
 }
 
 __host__ __device__ __forceinline__ int ceil_div(int a, int b) { return (a + b - 1) / b; }
+
+// ---------------------------------------------------------------------------
+// Buffer-addressed plane access.  A plane (one image channel) is described by a
+// 128-bit buffer resource whose num_records is the plane's size in bytes; every
+// access gives a 32-bit byte offset in a VGPR.  The hardware range-checks the
+// offset: a load beyond num_records returns 0 and a store is dropped.  Taps that
+// fall in the zero padding and lanes beyond the end of a plane are therefore
+// expressed as the offset kOutOfRange, with no branch, exec masking or select,
+// and no 64-bit address arithmetic is spent on the vector ALU.
+// ---------------------------------------------------------------------------
+constexpr unsigned kOutOfRange = 0x80000000u;
+constexpr int kRsrcFlags = 0x00020000;  // raw buffer, 32-bit data format (gfx9 family)
+
+using rsrc_t = __amdgpu_buffer_rsrc_t;
+
+template <typename T>
+__device__ __forceinline__ rsrc_t plane_rsrc(const T* base, int elems) {
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(base), 0, elems * (int)sizeof(T), kRsrcFlags);
+}
+
+__device__ __forceinline__ float buf_ld(rsrc_t r, unsigned byte_off, const float*) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(r, (int)byte_off, 0, 0));
+}
+__device__ __forceinline__ float buf_ld(rsrc_t r, unsigned byte_off, const __half*) {
+  const unsigned short b = __builtin_amdgcn_raw_buffer_load_b16(r, (int)byte_off, 0, 0);
+  return static_cast<float>(__builtin_bit_cast(_Float16, b));
+}
+__device__ __forceinline__ float buf_ld(rsrc_t r, unsigned byte_off, const bf16_t*) {
+  const unsigned short b = __builtin_amdgcn_raw_buffer_load_b16(r, (int)byte_off, 0, 0);
+  return __uint_as_float(static_cast<uint32_t>(b) << 16);
+}
+__device__ __forceinline__ void buf_st(rsrc_t r, unsigned byte_off, float v, float*) {
+  __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, v), r, (int)byte_off, 0, 0);
+}
+__device__ __forceinline__ void buf_st(rsrc_t r, unsigned byte_off, float v, __half*) {
+  const _Float16 h = static_cast<_Float16>(v);
+  __builtin_amdgcn_raw_buffer_store_b16(__builtin_bit_cast(unsigned short, h), r, (int)byte_off, 0, 0);
+}
+__device__ __forceinline__ void buf_st(rsrc_t r, unsigned byte_off, float v, bf16_t*) {
+  bf16_t t;
+  st(&t, v);
+  __builtin_amdgcn_raw_buffer_store_b16(t.bits, r, (int)byte_off, 0, 0);
+}
 
 }  // namespace dk

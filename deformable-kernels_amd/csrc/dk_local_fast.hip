@@ -13,6 +13,8 @@
 //   grad input     K.cu:577-669   -> local_gather_kernel<.., true>
 //   grad rotation  K.cu:1285-1370 -> local_grad_rotation_kernel
 //   grad filter    K.cu:836-955   -> local_grad_filter_kernel + reduce_partials_kernel
+#include <cstdlib>
+
 #include "dk_kernels.h"
 
 namespace dk {
@@ -27,6 +29,54 @@ struct Table {
   static constexpr int RS = SW + 2;
   static constexpr int SIZE = (SH + 2) * RS;
 };
+
+// Corner-expanded scope table of one channel: one float4 {tl, tr, bl, br} per 2x2 block of the
+// zero-padded tile, (SH + 1) x (SW + 1) blocks, so a tap needs a single 16-byte LDS read.
+//
+// gfx950 serves a ds_read_b128 at 256 B/clk from 64 banks, so two float4 blocks collide when
+// their block slots are congruent mod 16.  For the 5 x 5 blocks of a 4 x 4 scope the slots are
+// permuted so that colliding pairs are blocks at opposite borders of the tile (4 apart in a
+// coordinate, or a far corner against the opposite inner corner), which the lanes of one wave
+// rarely address together; a row-major order would pair blocks only (3, 1) apart.
+template <int SH, int SW>
+struct WideTable {
+  static constexpr int RS = SW + 1;
+  static constexpr int BLOCKS = (SH + 1) * RS;
+  static constexpr int SIZE = BLOCKS * 4;
+  __host__ __device__ static constexpr int slot(int block) { return block; }
+};
+
+template <>
+struct WideTable<4, 4> {
+  static constexpr int RS = 5;
+  static constexpr int BLOCKS = 25;
+  static constexpr int SIZE = BLOCKS * 4;
+  // block (r, c) = r * 5 + c  ->  slot; slots s and s + 16 share banks
+  __host__ __device__ static constexpr int slot(int block) {
+    constexpr signed char lut[25] = {
+        /* r=0 */ 24, 0, 1, 2, 3,
+        /* r=1 */ 4, 7, 9, 10, 20,
+        /* r=2 */ 5, 11, 12, 13, 21,
+        /* r=3 */ 6, 14, 15, 8, 22,
+        /* r=4 */ 16, 17, 18, 19, 23};
+    return lut[block];
+  }
+};
+
+template <typename T, int SH, int SW>
+__device__ __forceinline__ void stage_wide_tables(float* tbl, const T* filter, int c_first,
+                                                  int c_step, int nch) {
+  using Tb = WideTable<SH, SW>;
+  for (int e = threadIdx.x; e < nch * Tb::SIZE; e += blockDim.x) {
+    const int j = e / Tb::SIZE, r = e % Tb::SIZE;
+    const int blk = r / 4, corner = r % 4;
+    const int i = blk / Tb::RS - 1 + (corner >> 1), k = blk % Tb::RS - 1 + (corner & 1);
+    float v = 0.f;
+    if (i >= 0 && i < SH && k >= 0 && k < SW)
+      v = ld(filter + (size_t)(c_first + j * c_step) * (SH * SW) + i * SW + k);
+    tbl[j * Tb::SIZE + Tb::slot(blk) * 4 + corner] = v;
+  }
+}
 
 template <typename T, int SH, int SW>
 __device__ __forceinline__ void stage_tables(float* tbl, const T* filter, int c_first, int c_step,
@@ -83,21 +133,27 @@ __device__ __forceinline__ bool tap_geometry(const Geo& g, int ph, int pw, int f
 // ---------------------------------------------------------------------------
 // forward and grad-input: dst[n, c, p] = sum_t src[n, c, tap_t(p)] * B_t(p; Wt[c])
 // grid = (pixel tiles, channel splits, batch * groups)
+//
+// Channels are walked kUnroll at a time: the 9 * kUnroll input loads of a block are
+// issued first (buffer loads, offsets fixed per lane), then each channel's 9 taps take
+// two ds_read2_b32 each at immediate offsets from one per-tap LDS address.
 // ---------------------------------------------------------------------------
+constexpr int kUnroll = 2;
+
 template <typename T, int KH, int KW, int SH, int SW, bool TRANSPOSED>
-__global__ __launch_bounds__(kBlock) void local_gather_kernel(Geo g, const T* __restrict__ src,
-                                                              const T* __restrict__ rot,
-                                                              const T* __restrict__ filter,
-                                                              T* __restrict__ dst, int ch_per_block) {
-  using Tb = Table<SH, SW>;
+__global__ __launch_bounds__(kBlock, 2) void local_gather_kernel(Geo g, const T* __restrict__ src,
+                                                                 const T* __restrict__ rot,
+                                                                 const T* __restrict__ filter,
+                                                                 T* __restrict__ dst, int ch_per_block) {
+  using Tb = WideTable<SH, SW>;
   constexpr int K = KH * KW;
-  extern __shared__ float tbl[];
+  extern __shared__ __align__(16) float tbl[];
 
   const int n = blockIdx.z / g.groups, grp = blockIdx.z % g.groups;
   const int cpg = g.channel / g.groups;  // channels per rotation group
   const int j0 = blockIdx.y * ch_per_block;
   const int nch = min(ch_per_block, cpg - j0);
-  stage_tables<T, SH, SW>(tbl, filter, grp + g.groups * j0, g.groups, nch);
+  stage_wide_tables<T, SH, SW>(tbl, filter, grp + g.groups * j0, g.groups, nch);
 
   const int out_plane = g.out_h * g.out_w, in_plane = g.in_h * g.in_w;
   const int dst_plane = TRANSPOSED ? in_plane : out_plane;
@@ -109,45 +165,63 @@ __global__ __launch_bounds__(kBlock) void local_gather_kernel(Geo g, const T* __
   const int ph = pc / dst_w, pw = pc % dst_w;
 
   ScopeTap<float> tap[K];
-  int soff[K];
-  unsigned live = 0;
-  const T* rbase = rot + (size_t)(n * g.groups + grp) * (K * 2) * out_plane;
+  unsigned soff[K];  // byte offset of the tap's source element in a source plane
+  const rsrc_t rr = plane_rsrc(rot + (size_t)(n * g.groups + grp) * (K * 2) * out_plane, K * 2 * out_plane);
 #pragma unroll
   for (int t = 0; t < K; ++t) {
     const int f_h = t / KW, f_w = t % KW;
-    int rpix;
-    const bool ok = tap_geometry<TRANSPOSED>(g, ph, pw, f_h, f_w, soff[t], rpix) && active;
-    float r_h = 0.f, r_w = 0.f;
-    if (ok) {
-      r_h = ld(rbase + (size_t)(2 * t) * out_plane + rpix);
-      r_w = ld(rbase + (size_t)(2 * t + 1) * out_plane + rpix);
-    }
+    int s_el, rpix;
+    const bool ok = tap_geometry<TRANSPOSED>(g, ph, pw, f_h, f_w, s_el, rpix) && active;
+    soff[t] = ok ? (unsigned)s_el * (unsigned)sizeof(T) : kOutOfRange;
+    const unsigned ro = ok ? (unsigned)((2 * t) * out_plane + rpix) * (unsigned)sizeof(T) : kOutOfRange;
+    const float r_h = buf_ld(rr, ro, rot);
+    const float r_w = buf_ld(rr, ro + (unsigned)out_plane * (unsigned)sizeof(T), rot);
     tap[t] = make_scope_tap<float>(scope_coord<float>(f_h, r_h, g.centre_h),
                                    scope_coord<float>(f_w, r_w, g.centre_w), SH, SW, Tb::RS);
-    live |= ok ? (1u << t) : 0u;
+    tap[t].cell = Tb::slot(tap[t].cell) * 4;
   }
   __syncthreads();
-  if (!active) return;
 
   const size_t chan0 = (size_t)n * g.channel + grp + (size_t)g.groups * j0;
   const T* sp = src + chan0 * src_plane;
-  T* dp = dst + chan0 * dst_plane + p;
+  T* dp = dst + chan0 * dst_plane;
   const size_t s_step = (size_t)g.groups * src_plane, d_step = (size_t)g.groups * dst_plane;
-#pragma unroll 2
-  for (int j = 0; j < nch; ++j) {
-    const float* tb = tbl + j * Tb::SIZE;
-    float acc = 0.f;
+  const unsigned doff = active ? (unsigned)p * (unsigned)sizeof(T) : kOutOfRange;
+
+  // Two register stages of kUnroll channels each: the loads of the next stage are in flight
+  // while the current one is computed, so a wave always has input loads outstanding.
+  // Channels beyond nch load through a zero-length resource (hardware returns 0) and
+  // store to an out-of-range offset (dropped), which keeps the loop free of branches.
+  auto load_stage = [&](float (&xv)[kUnroll][K], int jb) {
 #pragma unroll
-    for (int t = 0; t < K; ++t) {
-      const float xv = (live >> t & 1u) ? ld(sp + soff[t]) : 0.f;
-      const float* q = tb + tap[t].cell;
-      const float b = tap[t].c00 * q[0] + tap[t].c01 * q[1] + tap[t].c10 * q[Tb::RS] +
-                      tap[t].c11 * q[Tb::RS + 1];
-      acc += xv * b;
+    for (int u = 0; u < kUnroll; ++u) {
+      const rsrc_t rs = plane_rsrc(sp + (size_t)(jb + u) * s_step, (jb + u) < nch ? src_plane : 0);
+#pragma unroll
+      for (int t = 0; t < K; ++t) xv[u][t] = buf_ld(rs, soff[t], src);
     }
-    st(dp, acc);
-    sp += s_step;
-    dp += d_step;
+  };
+  auto compute_stage = [&](const float (&xv)[kUnroll][K], int jb) {
+    const float* tb = tbl + jb * Tb::SIZE;
+#pragma unroll
+    for (int u = 0; u < kUnroll; ++u) {
+      float acc = 0.f;
+#pragma unroll
+      for (int t = 0; t < K; ++t) {
+        const float4 q = *reinterpret_cast<const float4*>(tb + tap[t].cell + u * Tb::SIZE);
+        const float b = tap[t].c00 * q.x + tap[t].c01 * q.y + tap[t].c10 * q.z + tap[t].c11 * q.w;
+        acc += xv[u][t] * b;
+      }
+      buf_st(plane_rsrc(dp + (size_t)(jb + u) * d_step, (jb + u) < nch ? dst_plane : 0), doff, acc, dst);
+    }
+  };
+
+  float xa[kUnroll][K], xb[kUnroll][K];
+  load_stage(xa, 0);
+  for (int j = 0; j < nch; j += 2 * kUnroll) {
+    load_stage(xb, j + kUnroll);
+    compute_stage(xa, j);
+    load_stage(xa, j + 2 * kUnroll);
+    compute_stage(xb, j + kUnroll);
   }
 }
 
@@ -165,7 +239,7 @@ __global__ __launch_bounds__(kBlock) void local_grad_rotation_kernel(
     const T* __restrict__ filter, T* __restrict__ grot, int ch_per_pass) {
   using Tb = Table<SH, SW>;
   constexpr int K = KH * KW;
-  extern __shared__ float tbl[];
+  extern __shared__ __align__(16) float tbl[];
 
   const int n = blockIdx.z / g.groups, grp = blockIdx.z % g.groups;
   const int cpg = g.channel / g.groups;
@@ -245,112 +319,177 @@ __global__ __launch_bounds__(kBlock) void local_grad_rotation_kernel(
 }
 
 // ---------------------------------------------------------------------------
-// grad filter: a workgroup owns CCH channels of one rotation group and walks
-// (image, pixel tile) work items.  Contributions x_t * gout * coef_k go into an
-// LDS accumulator of the padded table shape, replicated 32 times with the
-// replica chosen by lane id so that a wave's 64 adds fall on 32 distinct banks
-// whatever cells they address.  Each workgroup finally writes one partial
-// [CCH][SH*SW] to the workspace; reduce_partials_kernel sums the partials in a
-// fixed order.  No global atomics.
-// grid = (parts, channel chunks, groups)
+// grad filter: gW[c][i][j] = sum over (image, pixel, tap) of x_t * gout * hat(h_t - i) * hat(w_t - j).
+//
+// LDS float atomics serialise per lane on this hardware, and a scatter by cell is data
+// dependent, so the sum is kept DENSE and in registers: a lane owns a pixel, holds for each
+// tap the SH + SW hat-function weights (channel independent), and per channel adds
+// ps * a_i * b_j into SH*SW private accumulators -- static register indices, no atomics.
+// After each channel the 64 lanes' accumulators are folded through a per-wave LDS
+// transpose (write [lane][cell], read back [cell] over 16 lanes, two cross-row
+// exchanges) and lanes 0..CELLS-1 add the wave's sum into a per-wave LDS accumulator that
+// persists over all the (image, tile) items the workgroup walks.  One partial per
+// workgroup goes to the workspace; reduce_partials_kernel adds the partials in order.
+// grid = (parts, channel splits, groups)
 // ---------------------------------------------------------------------------
-constexpr int kRep = 32;
-
-template <typename T, int KH, int KW, int SH, int SW, int CCH>
-__global__ __launch_bounds__(kBlock) void local_grad_filter_kernel(
+template <typename T, int KH, int KW, int SH, int SW>
+__global__ __launch_bounds__(kBlock, 2) void local_grad_filter_kernel(
     Geo g, const T* __restrict__ gout, const T* __restrict__ x, const T* __restrict__ rot,
-    float* __restrict__ partial, int tiles) {
-  using Tb = Table<SH, SW>;
+    float* __restrict__ partial, int tiles, int ch_per_block) {
   constexpr int K = KH * KW;
-  __shared__ float acc[CCH * Tb::SIZE * kRep];
+  constexpr int CELLS = SH * SW;
+  static_assert(CELLS <= 16, "the fold below handles up to 16 cells per 16-lane row");
+  constexpr int kPitch = 20;  // floats per lane in the transpose scratch: 16-byte aligned, bank-skewed
+  constexpr int kWaves = kBlock / 64;
+  extern __shared__ __align__(16) float lds[];
+  float* wacc = lds;                                  // [kWaves][ch_per_block][16]
+  float* scratch = lds + kWaves * ch_per_block * 16;  // [kWaves][64][kPitch]
 
-  for (int e = threadIdx.x; e < CCH * Tb::SIZE * kRep; e += kBlock) acc[e] = 0.f;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  for (int e = threadIdx.x; e < kWaves * ch_per_block * 16; e += kBlock) wacc[e] = 0.f;
   __syncthreads();
 
   const int grp = blockIdx.z;
   const int cpg = g.channel / g.groups;
-  const int j0 = blockIdx.y * CCH;
-  const int nch = min(CCH, cpg - j0);
+  const int j0 = blockIdx.y * ch_per_block;
+  const int nch = min(ch_per_block, cpg - j0);
   const int out_plane = g.out_h * g.out_w, in_plane = g.in_h * g.in_w;
-  const int rep = threadIdx.x & (kRep - 1);
   const int items = g.batch * tiles;
+  float* my_acc = wacc + wave * ch_per_block * 16;
+  float* my_scr = scratch + wave * 64 * kPitch;
+  // read-back pattern of the fold: lane (row = lane / 16, m = lane % 16) sums cell m over the
+  // 16 lanes of its row, starting 4 * row lanes in so the four rows hit disjoint banks
+  const int row = lane >> 4, m = lane & 15;
 
   for (int item = blockIdx.x; item < items; item += gridDim.x) {
     const int n = item / tiles, tile = item % tiles;
     const int p = tile * kBlock + threadIdx.x;
-    if (p >= out_plane) continue;
-    const int ph = p / g.out_w, pw = p % g.out_w;
+    const bool active = p < out_plane;
+    const int pc = active ? p : 0;
+    const int ph = pc / g.out_w, pw = pc % g.out_w;
 
-    ScopeTap<float> tap[K];
-    int soff[K];
-    unsigned live = 0;
-    const T* rbase = rot + (size_t)(n * g.groups + grp) * (K * 2) * out_plane + p;
+    float ah[K][SH], bw[K][SW];
+    unsigned soff[K];
+    const rsrc_t rr = plane_rsrc(rot + (size_t)(n * g.groups + grp) * (K * 2) * out_plane, K * 2 * out_plane);
 #pragma unroll
     for (int t = 0; t < K; ++t) {
       const int f_h = t / KW, f_w = t % KW;
-      int rpix;
-      const bool ok = tap_geometry<false>(g, ph, pw, f_h, f_w, soff[t], rpix);
-      float r_h = 0.f, r_w = 0.f;
-      if (ok) {
-        r_h = ld(rbase + (size_t)(2 * t) * out_plane);
-        r_w = ld(rbase + (size_t)(2 * t + 1) * out_plane);
-      }
-      tap[t] = make_scope_tap<float>(scope_coord<float>(f_h, r_h, g.centre_h),
-                                     scope_coord<float>(f_w, r_w, g.centre_w), SH, SW, Tb::RS);
-      live |= ok ? (1u << t) : 0u;
+      int s_el, rpix;
+      const bool ok = tap_geometry<false>(g, ph, pw, f_h, f_w, s_el, rpix) && active;
+      soff[t] = ok ? (unsigned)s_el * (unsigned)sizeof(T) : kOutOfRange;
+      const unsigned ro = ok ? (unsigned)((2 * t) * out_plane + rpix) * (unsigned)sizeof(T) : kOutOfRange;
+      const float h = scope_coord<float>(f_h, buf_ld(rr, ro, rot), g.centre_h);
+      const float w = scope_coord<float>(f_w, buf_ld(rr, ro + (unsigned)out_plane * (unsigned)sizeof(T), rot),
+                                         g.centre_w);
+      // hat(h - i) = lh at i = floor(h) + 1, 1 - lh at i = floor(h), else 0: the same products
+      // (hh, lh) x (hw, lw) as K.cu:101-112, laid out densely; all zero outside (-1, S).
+      const bool in = (h > -1.f) && (w > -1.f) && (h < float(SH)) && (w < float(SW));
+      const float hf = floorf(h), wf = floorf(w);
+      const int hl = in ? (int)hf : -8, wl = in ? (int)wf : -8;
+      const float lh = h - hf, lw = w - wf;
+#pragma unroll
+      for (int i = 0; i < SH; ++i) ah[t][i] = (i == hl) ? 1.f - lh : (i == hl + 1) ? lh : 0.f;
+#pragma unroll
+      for (int i = 0; i < SW; ++i) bw[t][i] = (i == wl) ? 1.f - lw : (i == wl + 1) ? lw : 0.f;
     }
+    const unsigned goff = active ? (unsigned)p * (unsigned)sizeof(T) : kOutOfRange;
 
     const size_t chan0 = (size_t)n * g.channel + grp + (size_t)g.groups * j0;
     const T* xp = x + chan0 * in_plane;
-    const T* gp = gout + chan0 * out_plane + p;
-    for (int j = 0; j < nch; ++j) {
-      const float go = ld(gp);
-      float* a = acc + (j * Tb::SIZE) * kRep + rep;
+    const T* gp = gout + chan0 * out_plane;
+    const size_t x_step = (size_t)g.groups * in_plane, g_step = (size_t)g.groups * out_plane;
+
+    float xv[2][K], gv[2];
+    auto load = [&](int s, int j) {
+      const rsrc_t rx = plane_rsrc(xp + (size_t)j * x_step, j < nch ? in_plane : 0);
+      const rsrc_t rg = plane_rsrc(gp + (size_t)j * g_step, j < nch ? out_plane : 0);
+      gv[s] = buf_ld(rg, goff, gout);
+#pragma unroll
+      for (int t = 0; t < K; ++t) xv[s][t] = buf_ld(rx, soff[t], x);
+    };
+    auto accumulate = [&](int s, int j) {
+      float acc[SH][SW];
+#pragma unroll
+      for (int i = 0; i < SH; ++i)
+#pragma unroll
+        for (int k = 0; k < SW; ++k) acc[i][k] = 0.f;
 #pragma unroll
       for (int t = 0; t < K; ++t) {
-        if (live >> t & 1u) {
-          const float ps = ld(xp + soff[t]) * go;
-          float* q = a + tap[t].cell * kRep;
-          atomicAdd(q, ps * tap[t].c00);
-          atomicAdd(q + kRep, ps * tap[t].c01);
-          atomicAdd(q + Tb::RS * kRep, ps * tap[t].c10);
-          atomicAdd(q + (Tb::RS + 1) * kRep, ps * tap[t].c11);
-        }
+        const float ps = xv[s][t] * gv[s];
+        float u[SW];
+#pragma unroll
+        for (int k = 0; k < SW; ++k) u[k] = ps * bw[t][k];
+#pragma unroll
+        for (int i = 0; i < SH; ++i)
+#pragma unroll
+          for (int k = 0; k < SW; ++k) acc[i][k] += ah[t][i] * u[k];
       }
-      xp += (size_t)g.groups * in_plane;
-      gp += (size_t)g.groups * out_plane;
+      // fold the wave: transpose through the wave's scratch
+      float* mine = my_scr + lane * kPitch;
+#pragma unroll
+      for (int i = 0; i < SH; ++i)
+#pragma unroll
+        for (int k = 0; k < SW; ++k) mine[i * SW + k] = acc[i][k];
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+      __builtin_amdgcn_wave_barrier();
+      float sum = 0.f;
+      if (m < CELLS) {
+#pragma unroll
+        for (int q = 0; q < 16; ++q) sum += my_scr[(row * 16 + ((q + 4 * row) & 15)) * kPitch + m];
+      }
+      sum += __shfl_xor(sum, 16, 64);
+      sum += __shfl_xor(sum, 32, 64);
+      __builtin_amdgcn_wave_barrier();
+      if (lane < CELLS && j < nch) my_acc[j * 16 + lane] += sum;
+    };
+
+    load(0, 0);
+    for (int j = 0; j < nch; j += 2) {
+      load(1, j + 1);
+      accumulate(0, j);
+      load(0, j + 2);
+      accumulate(1, j + 1);
     }
   }
   __syncthreads();
 
-  // fold the replicas; lane-rotated start keeps the 32 reads of a step on 32 banks
-  for (int e = threadIdx.x; e < nch * SH * SW; e += kBlock) {
-    const int j = e / (SH * SW), r = e % (SH * SW);
-    const int i = r / SW, k = r % SW;
-    const float* a = acc + (j * Tb::SIZE + (i + 1) * Tb::RS + (k + 1)) * kRep;
-    float s = 0.f;
-    for (int q = 0; q < kRep; ++q) s += a[(q + threadIdx.x) & (kRep - 1)];
+  for (int e = threadIdx.x; e < nch * CELLS; e += kBlock) {
+    const int j = e / CELLS, r = e % CELLS;
+    float s_ = 0.f;
+#pragma unroll
+    for (int wv = 0; wv < kWaves; ++wv) s_ += wacc[(wv * ch_per_block + j) * 16 + r];
     const int c = grp + g.groups * (j0 + j);
-    partial[((size_t)blockIdx.x * g.channel + c) * (SH * SW) + r] = s;
+    partial[((size_t)blockIdx.x * g.channel + c) * CELLS + r] = s_;
   }
 }
 
 }  // namespace
 
-// out[e] = sum over parts of partial[part][e], in part order.
+// out[e] = sum over parts of partial[part][e].  32 elements per workgroup, 8 threads per
+// element each summing every 8th part, combined in a fixed order (run-to-run reproducible).
 template <typename CT, typename T>
-__global__ void reduce_partials_kernel(const CT* __restrict__ partial, int parts, int count,
-                                       T* __restrict__ out) {
-  const int e = blockIdx.x * blockDim.x + threadIdx.x;
-  if (e >= count) return;
+__global__ __launch_bounds__(256) void reduce_partials_kernel(const CT* __restrict__ partial,
+                                                              int parts, int count,
+                                                              T* __restrict__ out) {
+  __shared__ CT part_sum[8][32];
+  const int el = threadIdx.x & 31, slice = threadIdx.x >> 5;
+  const int e = blockIdx.x * 32 + el;
   CT s = 0;
-  for (int q = 0; q < parts; ++q) s += partial[(size_t)q * count + e];
-  st(out + e, s);
+  if (e < count)
+    for (int q = slice; q < parts; q += 8) s += partial[(size_t)q * count + e];
+  part_sum[slice][el] = s;
+  __syncthreads();
+  if (slice == 0 && e < count) {
+    CT t = 0;
+#pragma unroll
+    for (int k = 0; k < 8; ++k) t += part_sum[k][el];
+    st(out + e, t);
+  }
 }
 
 template <typename CT, typename T>
 void launch_reduce_partials(const CT* partial, int parts, int count, T* out, hipStream_t stream) {
-  reduce_partials_kernel<CT, T><<<ceil_div(count, 256), 256, 0, stream>>>(partial, parts, count, out);
+  reduce_partials_kernel<CT, T><<<ceil_div(count, 32), 256, 0, stream>>>(partial, parts, count, out);
 }
 template void launch_reduce_partials<float, float>(const float*, int, int, float*, hipStream_t);
 template void launch_reduce_partials<float, __half>(const float*, int, int, __half*, hipStream_t);
@@ -362,7 +501,6 @@ template void launch_reduce_partials<double, double>(const double*, int, int, do
 // ---------------------------------------------------------------------------
 namespace {
 
-constexpr int kFilterCch = 8;        // channels per grad-filter workgroup
 constexpr int kMaxLdsTables = 96 * 1024;  // bytes of LDS a workgroup may spend on scope tables
 
 template <int SH, int SW>
@@ -379,6 +517,8 @@ int pick_splits(const Geo& g, int planes_pixels) {
   const long waves = (long)ceil_div(planes_pixels, kBlock) * (kBlock / 64) * g.batch * g.groups;
   const int cpg = g.channel / g.groups;
   int splits = 1;
+  const char* env = getenv("DK_SPLITS");  // tuning aid
+  if (env) return atoi(env);
   while (waves * splits < 8192 && cpg / (splits * 2) >= 16) splits *= 2;
   return splits;
 }
@@ -390,7 +530,8 @@ bool run_gather(const Geo& g, bool transposed, const T* src, const T* rot, const
   const int pixels = transposed ? g.in_h * g.in_w : g.out_h * g.out_w;
   const int per = channels_per_block<SH, SW>(cpg, pick_splits(g, pixels));
   const dim3 grid(ceil_div(pixels, kBlock), ceil_div(cpg, per), g.batch * g.groups);
-  const size_t lds = (size_t)per * Table<SH, SW>::SIZE * sizeof(float);
+  // stages past the last channel still read (and discard) table entries: pad to whole stages
+  const size_t lds = (size_t)(per + 2 * kUnroll) * WideTable<SH, SW>::SIZE * sizeof(float);
   if (transposed)
     local_gather_kernel<T, 3, 3, SH, SW, true><<<grid, kBlock, lds, stream>>>(g, src, rot, filter, dst, per);
   else
@@ -409,29 +550,46 @@ bool run_grad_rotation(const Geo& g, const T* gout, const T* x, const T* rot, co
   return true;
 }
 
-int filter_parts(const Geo& g) {
-  const int tiles = ceil_div(g.out_h * g.out_w, kBlock);
-  const int items = g.batch * tiles;
-  const int chunks = ceil_div(g.channel / g.groups, kFilterCch) * g.groups;
-  int parts = ceil_div(2048, chunks);  // ~8 workgroups per CU in total
-  if (parts > items) parts = items;
-  if (parts < 1) parts = 1;
-  return parts;
+// grad-filter launch shape: channel splits of at most kFilterChPerBlock channels, and enough
+// (image, tile) parts that the grid has a few workgroups per CU.
+constexpr int kFilterChPerBlock = 72;
+
+struct FilterGrid {
+  int per, splits, parts, tiles;
+};
+
+FilterGrid filter_grid(const Geo& g) {
+  FilterGrid f;
+  const int cpg = g.channel / g.groups;
+  f.splits = ceil_div(cpg, kFilterChPerBlock);
+  f.per = ceil_div(cpg, f.splits);
+  f.tiles = ceil_div(g.out_h * g.out_w, kBlock);
+  const int items = g.batch * f.tiles;
+  f.parts = ceil_div(1024, f.splits * g.groups);
+  if (f.parts > items) f.parts = items;
+  if (f.parts < 1) f.parts = 1;
+  return f;
 }
 
 template <typename T, int SH, int SW>
 bool run_grad_filter(const Geo& g, const T* gout, const T* x, const T* rot, T* gfilter, float* ws,
                      hipStream_t stream) {
-  const int tiles = ceil_div(g.out_h * g.out_w, kBlock);
-  const int parts = filter_parts(g);
-  const dim3 grid(parts, ceil_div(g.channel / g.groups, kFilterCch), g.groups);
-  local_grad_filter_kernel<T, 3, 3, SH, SW, kFilterCch><<<grid, kBlock, 0, stream>>>(g, gout, x, rot, ws, tiles);
-  launch_reduce_partials<float, T>(ws, parts, g.channel * SH * SW, gfilter, stream);
-  return true;
+  if constexpr (SH * SW > 16) {
+    return false;
+  } else {
+    const FilterGrid f = filter_grid(g);
+    const dim3 grid(f.parts, f.splits, g.groups);
+    const size_t lds = ((size_t)(kBlock / 64) * f.per * 16 + (size_t)(kBlock / 64) * 64 * 20) * sizeof(float);
+    local_grad_filter_kernel<T, 3, 3, SH, SW><<<grid, kBlock, lds, stream>>>(g, gout, x, rot, ws, f.tiles, f.per);
+    launch_reduce_partials<float, T>(ws, f.parts, g.channel * SH * SW, gfilter, stream);
+    return true;
+  }
 }
 
 bool fast_shape(const Geo& g) {
+  const long plane_limit = (1L << 31) / 4 / 32;  // byte offsets inside a plane (x 18 for rotation) stay below 2^31
   return g.k_h == 3 && g.k_w == 3 && (long)g.batch * g.groups <= 65535 &&
+         (long)g.in_h * g.in_w < plane_limit && (long)g.out_h * g.out_w < plane_limit &&
          ((g.scope_h == 4 && g.scope_w == 4) || (g.scope_h == 3 && g.scope_w == 3) ||
           (g.scope_h == 5 && g.scope_w == 5));
 }
@@ -462,14 +620,14 @@ bool fast_local_grad_rotation(const Geo& g, const T* gout, const T* x, const T* 
 }
 
 size_t fast_local_grad_filter_workspace(const Geo& g) {
-  if (!fast_shape(g)) return 0;
-  return (size_t)filter_parts(g) * g.channel * g.scope_h * g.scope_w * sizeof(float);
+  if (!fast_shape(g) || g.scope_h * g.scope_w > 16) return 0;
+  return (size_t)filter_grid(g).parts * g.channel * g.scope_h * g.scope_w * sizeof(float);
 }
 
 template <typename T>
 bool fast_local_grad_filter(const Geo& g, const T* gout, const T* x, const T* rot, T* gfilter,
                             void* ws, hipStream_t stream) {
-  if (!fast_shape(g)) return false;
+  if (!fast_shape(g) || g.scope_h * g.scope_w > 16) return false;
 #define CALL(SH, SW) run_grad_filter<T, SH, SW>(g, gout, x, rot, gfilter, static_cast<float*>(ws), stream)
   DK_DISPATCH_SCOPE(g, CALL)
 #undef CALL
