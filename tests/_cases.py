@@ -45,8 +45,8 @@ def make_deform(N, C, H, W, k=3, S=(4, 4), stride=1, pad=1, dil=1, groups=1, rot
 
 def rel_err(a, b):
     """max |a-b| over max |b|: error relative to the scale of the expected tensor."""
-    a = torch.as_tensor(a, dtype=torch.float64)
-    b = torch.as_tensor(b, dtype=torch.float64)
+    a = torch.as_tensor(a).detach().to(torch.float64)
+    b = torch.as_tensor(b).detach().to(torch.float64)
     if b.numel() == 0:
         return 0.0
     scale = float(b.abs().max())

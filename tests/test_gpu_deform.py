@@ -1,0 +1,108 @@
+"""GPU parity of the deformable variant (kernel-space + image-space offsets):
+forward, grad-input, grad-offset, grad-rotation, grad-filter against the CPU
+oracle, through the Python Function and the C ABI.
+
+Tolerances relative to the largest expected magnitude: fp32 forward 1e-5
+against the fp32 oracle; the four gradients 1e-4 against the fp64 oracle
+(grad-input is an atomic scatter, the others are reductions, so summation order
+differs from the oracle's); fp64 1e-11; fp16 / bf16 1e-2 against the fp32
+oracle on the rounded inputs."""
+import numpy as np
+import pytest
+import torch
+
+from _cases import make_deform, rel_err
+from oracle import dk_oracle as orc
+
+pytestmark = pytest.mark.gpu
+
+# N, C, H, W, k, S, stride, pad, dil, groups, rot_std, off_std
+CASES = [
+    (2, 16, 14, 14, 3, (4, 4), 2, 1, 1, 1, 0.5, 2.0),     # BASELINE config 4 geometry, small
+    (2, 12, 13, 11, 3, (4, 4), 1, 1, 1, 1, 1.0, 2.0),
+    (2, 12, 9, 10, 3, (4, 4), 1, 2, 2, 3, 0.7, 3.0),      # dilation, rotation groups
+    (1, 8, 12, 12, 3, (3, 3), 1, 1, 1, 1, 0.0, 1.5),      # DeformConv2d: scope == kernel, zero rotation
+    (2, 6, 8, 8, (2, 3), (4, 5), (1, 2), (0, 1), 1, 3, 0.7, 1.0),
+    (1, 3, 6, 5, 1, (2, 2), 1, 0, 1, 1, 0.6, 3.0),
+]
+NAMES = ("forward", "grad input", "grad offset", "grad rotation", "grad filter")
+
+
+def _run(case, dtype, seed=0):
+    from deformable_kernels.ops.deform_kernel.functions import deform_sample_depthwise
+    N, C, H, W, k, S, s, p, d, G, rs, os_ = case
+    x, wt, rot, off, gout, cfg = make_deform(N, C, H, W, k, S, s, p, d, G, rs, os_, seed=seed, dtype=dtype)
+    dev = torch.device("cuda:0")
+    xg, og, rg, wg = [t.to(dev).requires_grad_() for t in (x, off, rot, wt)]
+    out = deform_sample_depthwise(xg, og, rg, wg, cfg["kernel_size"], cfg["stride"], cfg["padding"],
+                                  cfg["dilation"], cfg["groups"])
+    out.backward(gout.to(dev))
+    torch.cuda.synchronize()
+    return (x, wt, rot, off, gout, cfg), [t.detach().cpu() for t in (out, xg.grad, og.grad, rg.grad, wg.grad)]
+
+
+def _oracle(inputs, np_dtype):
+    x, wt, rot, off, gout, cfg = inputs
+    a = [t.to(torch.float64).numpy().astype(np_dtype) for t in (x, off, rot, wt, gout)]
+    out = orc.deform_sample_depthwise_forward(a[0], a[1], a[2], a[3], **cfg)
+    return (out,) + tuple(orc.deform_sample_depthwise_backward(a[4], a[0], a[1], a[2], a[3], **cfg))
+
+
+@pytest.mark.parametrize("case", CASES)
+def test_fp32_matches_oracle(case):
+    inputs, got = _run(case, torch.float32)
+    o32, o64 = _oracle(inputs, np.float32), _oracle(inputs, np.float64)
+    assert rel_err(got[0], o32[0]) < 1e-5, NAMES[0]
+    for i in range(1, 5):
+        assert rel_err(got[i], o64[i]) < 1e-4, NAMES[i]
+
+
+@pytest.mark.parametrize("case", CASES[:3])
+def test_fp64_matches_oracle(case):
+    inputs, got = _run(case, torch.float64)
+    want = _oracle(inputs, np.float64)
+    for g, w, name in zip(got, want, NAMES):
+        assert rel_err(g, w) < 1e-11, name
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("case", CASES[:3])
+def test_half_precisions_match_fp32_oracle(case, dtype):
+    inputs, got = _run(case, dtype)
+    want = _oracle(inputs, np.float32)
+    for g, w, name in zip(got, want, NAMES):
+        assert g.dtype == dtype
+        assert rel_err(g.float(), w) < 1e-2, name
+
+
+def test_zero_image_offsets_equal_the_local_operator_on_gpu():
+    from deformable_kernels.ops.deform_kernel.functions import deform_sample_depthwise, sample_depthwise
+    x, wt, rot, off, gout, cfg = make_deform(2, 16, 12, 12, 3, (4, 4), 1, 1, 1, 1, 1.0, 0.0, seed=3)
+    dev = torch.device("cuda:0")
+    args = (cfg["kernel_size"], cfg["stride"], cfg["padding"], cfg["dilation"], cfg["groups"])
+    a = deform_sample_depthwise(x.to(dev), off.to(dev), rot.to(dev), wt.to(dev), *args)
+    b = sample_depthwise(x.to(dev), rot.to(dev), wt.to(dev), *args)
+    assert rel_err(a.cpu(), b.cpu()) < 1e-6
+
+
+def test_samples_outside_the_image_give_exact_zeros():
+    from deformable_kernels.ops.deform_kernel.functions import deform_sample_depthwise
+    x, wt, rot, off, gout, cfg = make_deform(1, 4, 8, 8, 3, (4, 4), 1, 1, 1, 1, 0.3, 0.0, seed=4)
+    dev = torch.device("cuda:0")
+    for shift in (-30.0, 30.0):
+        ts = [t.to(dev).requires_grad_() for t in (x, off + shift, rot, wt)]
+        out = deform_sample_depthwise(*ts, (3, 3), (1, 1), (1, 1), (1, 1), 1)
+        out.backward(gout.to(dev))
+        for t in [out] + [t.grad for t in ts]:
+            assert torch.count_nonzero(t).item() == 0
+
+
+def test_config4_shape_on_a_batch_slice():
+    """BASELINE config 4 geometry at full channel count (C=512, 28x28 -> 14x14, stride 2) on 4
+    images: forward and all four gradients against the oracle."""
+    case = (4, 512, 28, 28, 3, (4, 4), 2, 1, 1, 1, 0.5, 2.0)
+    inputs, got = _run(case, torch.float32)
+    o32, o64 = _oracle(inputs, np.float32), _oracle(inputs, np.float64)
+    assert rel_err(got[0], o32[0]) < 1e-5
+    for i in range(1, 5):
+        assert rel_err(got[i], o64[i]) < 1e-4, NAMES[i]

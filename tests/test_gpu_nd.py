@@ -1,0 +1,92 @@
+"""GPU parity of the N-d linear sampler (forward, grad-data, grad-coord) against the CPU
+oracle.  fp32: forward 1e-5 against the fp32 oracle, gradients 1e-4 against the fp64 oracle;
+fp64 1e-11; fp16 / bf16 1e-2 against the fp32 oracle on the rounded inputs."""
+import numpy as np
+import pytest
+import torch
+
+from _cases import rel_err
+from oracle import dk_oracle as orc
+
+pytestmark = pytest.mark.gpu
+
+
+def _inputs(shape, C, B, seed, dtype, lo=-1.5, extra=1.5):
+    g = torch.Generator().manual_seed(seed)
+    data = torch.randn(C, *shape, generator=g)
+    hi = torch.tensor(shape, dtype=torch.float32)
+    coord = torch.rand(B, len(shape), generator=g) * (hi + extra - lo) + lo  # spills outside on both sides
+    gout = torch.randn(B, C, generator=g)
+    return data.to(dtype), coord.to(dtype), gout.to(dtype)
+
+
+def _run(data, coord, gout):
+    from deformable_kernels.ops.deform_kernel.functions import nd_linear_sample
+    dev = torch.device("cuda:0")
+    dg, cg = data.to(dev).requires_grad_(), coord.to(dev).requires_grad_()
+    out = nd_linear_sample(dg, cg)
+    out.backward(gout.to(dev))
+    torch.cuda.synchronize()
+    return out.detach().cpu(), dg.grad.cpu(), cg.grad.cpu()
+
+
+def _oracle(data, coord, gout, np_dtype):
+    a = [t.to(torch.float64).numpy().astype(np_dtype) for t in (data, coord, gout)]
+    out = orc.nd_linear_sample_forward(a[0], a[1])
+    gd, gc = orc.nd_linear_sample_backward(a[2], a[0], a[1])
+    return out, gd, gc
+
+
+@pytest.mark.parametrize("shape,C,B", [((9,), 5, 70), ((5, 5), 256, 1152), ((4, 5, 6), 7, 333),
+                                       ((3, 4, 2, 5), 3, 200), ((2, 2), 1, 1)])
+def test_fp32_matches_oracle(shape, C, B):
+    data, coord, gout = _inputs(shape, C, B, seed=41, dtype=torch.float32)
+    got = _run(data, coord, gout)
+    o32, o64 = _oracle(data, coord, gout, np.float32), _oracle(data, coord, gout, np.float64)
+    assert got[0].shape == (B, C)
+    assert rel_err(got[0], o32[0]) < 1e-5
+    assert rel_err(got[1], o64[1]) < 1e-4
+    assert rel_err(got[2], o64[2]) < 1e-4
+
+
+def test_fp64_matches_oracle():
+    data, coord, gout = _inputs((4, 5, 6), 9, 257, seed=42, dtype=torch.float64)
+    got = _run(data, coord, gout)
+    want = _oracle(data, coord, gout, np.float64)
+    for g, w in zip(got, want):
+        assert rel_err(g, w) < 1e-11
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_half_precisions_match_fp32_oracle(dtype):
+    data, coord, gout = _inputs((5, 5), 64, 300, seed=43, dtype=dtype)
+    got = _run(data, coord, gout)
+    want = _oracle(data, coord, gout, np.float32)
+    for g, w in zip(got, want):
+        assert g.dtype == dtype
+        assert rel_err(g.float(), w) < 1e-2
+
+
+def test_zero_rule_and_fade_bands_on_gpu():
+    data = torch.ones(1, 4, 4)
+    pts = torch.tensor([[-1.0, 1.0], [1.0, -1.0], [4.0, 1.0], [1.0, 4.0], [-0.5, 1.0], [3.5, 3.5], [3.0, 3.0]])
+    out, _, gc = _run(data, pts, torch.ones(7, 1))
+    assert out[:4, 0].tolist() == [0, 0, 0, 0]
+    assert torch.allclose(out[4:, 0], torch.tensor([0.5, 0.25, 1.0]))
+    assert torch.count_nonzero(gc[:4]).item() == 0
+
+
+def test_trilinear_volume_slice_of_config5():
+    """Config 5's standalone case at reduced point count: data [64, 32, 32, 32], coordinates
+    uniform in [-1, 1]^3 as written there (half the points in the fade band) and uniform over
+    the whole volume."""
+    g = torch.Generator().manual_seed(44)
+    data = torch.randn(64, 32, 32, 32, generator=g)
+    for lo, hi in ((-1.0, 1.0), (-1.0, 32.0)):
+        coord = torch.rand(4096, 3, generator=g) * (hi - lo) + lo
+        gout = torch.randn(4096, 64, generator=g)
+        got = _run(data, coord, gout)
+        o32, o64 = _oracle(data, coord, gout, np.float32), _oracle(data, coord, gout, np.float64)
+        assert rel_err(got[0], o32[0]) < 1e-5
+        assert rel_err(got[1], o64[1]) < 1e-4
+        assert rel_err(got[2], o64[2]) < 1e-4
