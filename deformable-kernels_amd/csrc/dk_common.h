@@ -144,6 +144,14 @@ __device__ __forceinline__ ImageTap<CT> make_image_tap(CT h, CT w, int H, int W)
 
 __host__ __device__ __forceinline__ int ceil_div(int a, int b) { return (a + b - 1) / b; }
 
+// Value held by the previous / next lane of the wave (0 at the wave's ends): one DPP move.
+__device__ __forceinline__ float from_lane_below(float v) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x138 /* wave_shr:1 */, 0xf, 0xf, true));
+}
+__device__ __forceinline__ float from_lane_above(float v) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x130 /* wave_shl:1 */, 0xf, 0xf, true));
+}
+
 // ---------------------------------------------------------------------------
 // Buffer-addressed plane access.  A plane (one image channel) is described by a
 // 128-bit buffer resource whose num_records is the plane's size in bytes; every

@@ -226,53 +226,182 @@ __global__ __launch_bounds__(kBlock, 2) void local_gather_kernel(Geo g, const T*
 }
 
 // ---------------------------------------------------------------------------
-// grad rotation: the lane owns output pixel p of (n, group) and sums over the
-// group's channels.  d/dh and d/dw of the bilinear read are linear in the four
-// corner weights with channel-independent coefficients, so the lane only
-// accumulates  S_k[t] = sum_c x_t[c] * gout[c] * corner_k[c]  and combines the
-// four sums per tap once at the end (K.cu:137-158 gives the combination).
+// forward and grad-input for "same" geometries (stride 1, 3 taps per row at unit spacing,
+// pad_w = 1, so input and output planes have the same width).
+//
+// In that case the nine taps of a pixel are three runs of three consecutive plane elements,
+// and lane l's left / right element is lane l -+ 1's centre element.  A wave therefore covers
+// 62 pixels with lanes 1..62 plus one halo lane at each end; every lane loads only the
+// centre element of each of the three tap rows (3 loads per channel instead of 9 -- the
+// vector-memory address unit was the busiest unit of the general kernel) and takes the
+// side elements from its neighbours with one DPP move each.  Rows above / below the plane
+// fall outside the buffer range and read 0; taps whose column wraps to the neighbouring row
+// get zero coefficients.
+// grid = (pixel tiles of kRowPix, channel splits, batch * groups)
+// ---------------------------------------------------------------------------
+constexpr int kRowLanes = 62;                          // pixels per wave
+constexpr int kRowPix = kRowLanes * (kBlock / 64);     // pixels per workgroup
+
+template <typename T, int KH, int SH, int SW, bool TRANSPOSED>
+__global__ __launch_bounds__(kBlock, 2) void local_gather_rows_kernel(Geo g, const T* __restrict__ src,
+                                                                      const T* __restrict__ rot,
+                                                                      const T* __restrict__ filter,
+                                                                      T* __restrict__ dst,
+                                                                      int ch_per_block) {
+  using Tb = WideTable<SH, SW>;
+  constexpr int KW = 3, K = KH * KW;
+  extern __shared__ __align__(16) float tbl[];
+
+  const int n = blockIdx.z / g.groups, grp = blockIdx.z % g.groups;
+  const int cpg = g.channel / g.groups;
+  const int j0 = blockIdx.y * ch_per_block;
+  const int nch = min(ch_per_block, cpg - j0);
+  stage_wide_tables<T, SH, SW>(tbl, filter, grp + g.groups * j0, g.groups, nch);
+
+  const int W = g.in_w;  // == out_w
+  const int out_plane = g.out_h * W, in_plane = g.in_h * W;
+  const int dst_plane = TRANSPOSED ? in_plane : out_plane;
+  const int src_plane = TRANSPOSED ? out_plane : in_plane;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int p = blockIdx.x * kRowPix + wave * kRowLanes + lane - 1;  // lanes 0 and 63 are halo
+  const bool owns = lane >= 1 && lane <= kRowLanes && p < dst_plane;  // p >= 0 whenever lane >= 1
+  const int pc = owns ? p : 0;
+  const int ph = pc / W, pw = pc % W;
+
+  // centre element of tap row f_h, as a byte offset into a source plane (out of range -> reads 0)
+  unsigned roff[KH];
+#pragma unroll
+  for (int r = 0; r < KH; ++r) {
+    const int dr = TRANSPOSED ? g.pad_h - r * g.dil_h : r * g.dil_h - g.pad_h;
+    const long e = (long)p + (long)dr * W;
+    roff[r] = (e >= 0 && e < src_plane) ? (unsigned)e * (unsigned)sizeof(T) : kOutOfRange;
+  }
+
+  ScopeTap<float> tap[K];
+  const rsrc_t rr = plane_rsrc(rot + (size_t)(n * g.groups + grp) * (K * 2) * out_plane, K * 2 * out_plane);
+#pragma unroll
+  for (int t = 0; t < K; ++t) {
+    const int f_h = t / KW, f_w = t % KW;
+    int s_el, rpix;
+    const bool ok = tap_geometry<TRANSPOSED>(g, ph, pw, f_h, f_w, s_el, rpix) && owns;
+    const unsigned ro = ok ? (unsigned)((2 * t) * out_plane + rpix) * (unsigned)sizeof(T) : kOutOfRange;
+    const float r_h = buf_ld(rr, ro, rot);
+    const float r_w = buf_ld(rr, ro + (unsigned)out_plane * (unsigned)sizeof(T), rot);
+    tap[t] = make_scope_tap<float>(scope_coord<float>(f_h, r_h, g.centre_h),
+                                   scope_coord<float>(f_w, r_w, g.centre_w), SH, SW, Tb::RS);
+    tap[t].cell = Tb::slot(tap[t].cell) * 4;
+    if (!ok) tap[t].c00 = tap[t].c01 = tap[t].c10 = tap[t].c11 = 0.f;  // tap in the padding
+  }
+  __syncthreads();
+
+  const size_t chan0 = (size_t)n * g.channel + grp + (size_t)g.groups * j0;
+  const T* sp = src + chan0 * src_plane;
+  T* dp = dst + chan0 * dst_plane;
+  const size_t s_step = (size_t)g.groups * src_plane, d_step = (size_t)g.groups * dst_plane;
+  const unsigned doff = owns ? (unsigned)p * (unsigned)sizeof(T) : kOutOfRange;
+
+  auto load_stage = [&](float (&xc)[kUnroll][KH], int jb) {
+#pragma unroll
+    for (int u = 0; u < kUnroll; ++u) {
+      const rsrc_t rs = plane_rsrc(sp + (size_t)(jb + u) * s_step, (jb + u) < nch ? src_plane : 0);
+#pragma unroll
+      for (int r = 0; r < KH; ++r) xc[u][r] = buf_ld(rs, roff[r], src);
+    }
+  };
+  auto compute_stage = [&](const float (&xc)[kUnroll][KH], int jb) {
+    const float* tb = tbl + jb * Tb::SIZE;
+#pragma unroll
+    for (int u = 0; u < kUnroll; ++u) {
+      float acc = 0.f;
+#pragma unroll
+      for (int r = 0; r < KH; ++r) {
+        // elements at columns -1, 0, +1 of this row; the tap that reads column dc is
+        // f_w = dc + 1 (forward) or f_w = 1 - dc (grad input)
+        const float xm = from_lane_below(xc[u][r]), x0 = xc[u][r], xp = from_lane_above(xc[u][r]);
+#pragma unroll
+        for (int f_w = 0; f_w < KW; ++f_w) {
+          const int t = r * KW + f_w;
+          const int dc = TRANSPOSED ? 1 - f_w : f_w - 1;
+          const float xv = dc < 0 ? xm : dc == 0 ? x0 : xp;
+          const float4 q = *reinterpret_cast<const float4*>(tb + tap[t].cell + u * Tb::SIZE);
+          const float b = tap[t].c00 * q.x + tap[t].c01 * q.y + tap[t].c10 * q.z + tap[t].c11 * q.w;
+          acc += xv * b;
+        }
+      }
+      buf_st(plane_rsrc(dp + (size_t)(jb + u) * d_step, (jb + u) < nch ? dst_plane : 0), doff, acc, dst);
+    }
+  };
+
+  float xa[kUnroll][KH], xb[kUnroll][KH];
+  load_stage(xa, 0);
+  for (int j = 0; j < nch; j += 2 * kUnroll) {
+    load_stage(xb, j + kUnroll);
+    compute_stage(xa, j);
+    load_stage(xa, j + 2 * kUnroll);
+    compute_stage(xb, j + kUnroll);
+  }
+}
+
+// ---------------------------------------------------------------------------
+// grad rotation: the lane owns output pixel p of (n, group) and sums over channels.
+// d/dh and d/dw of the bilinear read are linear in the four corner weights with
+// channel-independent coefficients, so the lane only accumulates
+//   S_k[t] = sum_c x_t[c] * gout[c] * corner_k[c]
+// and combines the four sums per tap once at the end (K.cu:137-158 gives the combination);
+// the fractional parts needed for that are recomputed from the rotation rather than kept
+// in registers across the channel loop.
+//
+// ROWS = true is the "same"-geometry form (see local_gather_rows_kernel): 62 pixels per
+// wave, centre-column loads and DPP neighbours; ROWS = false loads every tap.
+// The scope tables of the group's channels are staged in passes of ch_per_pass channels.
 // grid = (pixel tiles, 1, batch * groups)
 // ---------------------------------------------------------------------------
-template <typename T, int KH, int KW, int SH, int SW>
-__global__ __launch_bounds__(kBlock) void local_grad_rotation_kernel(
+template <typename T, int KH, int KW, int SH, int SW, bool ROWS>
+__global__ __launch_bounds__(kBlock, 2) void local_grad_rotation_kernel(
     Geo g, const T* __restrict__ gout, const T* __restrict__ x, const T* __restrict__ rot,
     const T* __restrict__ filter, T* __restrict__ grot, int ch_per_pass) {
-  using Tb = Table<SH, SW>;
+  using Tb = WideTable<SH, SW>;
   constexpr int K = KH * KW;
+  constexpr int NLOAD = ROWS ? KH : K;  // input loads per channel
   extern __shared__ __align__(16) float tbl[];
 
   const int n = blockIdx.z / g.groups, grp = blockIdx.z % g.groups;
   const int cpg = g.channel / g.groups;
   const int out_plane = g.out_h * g.out_w, in_plane = g.in_h * g.in_w;
-  const int p = blockIdx.x * kBlock + threadIdx.x;
-  const bool active = p < out_plane;
-  const int pc = active ? p : 0;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int p = ROWS ? blockIdx.x * kRowPix + wave * kRowLanes + lane - 1 : blockIdx.x * kBlock + threadIdx.x;
+  const bool owns = (ROWS ? (lane >= 1 && lane <= kRowLanes) : true) && p < out_plane;
+  const int pc = owns ? p : 0;
   const int ph = pc / g.out_w, pw = pc % g.out_w;
 
-  int cell[K], soff[K];
-  float lh[K], lw[K];
-  unsigned live = 0, inside = 0;
+  int cell[K];
+  unsigned soff[NLOAD];
+  unsigned inside = 0, live = 0;
   const size_t rplane0 = (size_t)(n * g.groups + grp) * (K * 2) * out_plane;
+  const rsrc_t rr = plane_rsrc(rot + rplane0, K * 2 * out_plane);
 #pragma unroll
   for (int t = 0; t < K; ++t) {
     const int f_h = t / KW, f_w = t % KW;
-    int rpix;
-    const bool ok = tap_geometry<false>(g, ph, pw, f_h, f_w, soff[t], rpix) && active;
-    float r_h = 0.f, r_w = 0.f;
-    if (active) {
-      r_h = ld(rot + rplane0 + (size_t)(2 * t) * out_plane + pc);
-      r_w = ld(rot + rplane0 + (size_t)(2 * t + 1) * out_plane + pc);
-    }
-    const float h = scope_coord<float>(f_h, r_h, g.centre_h);
-    const float w = scope_coord<float>(f_w, r_w, g.centre_w);
+    int s_el, rpix;
+    const bool ok = tap_geometry<false>(g, ph, pw, f_h, f_w, s_el, rpix) && owns;
+    if (!ROWS) soff[t] = ok ? (unsigned)s_el * (unsigned)sizeof(T) : kOutOfRange;
+    const unsigned ro = owns ? (unsigned)((2 * t) * out_plane + pc) * (unsigned)sizeof(T) : kOutOfRange;
+    const float h = scope_coord<float>(f_h, buf_ld(rr, ro, rot), g.centre_h);
+    const float w = scope_coord<float>(f_w, buf_ld(rr, ro + (unsigned)out_plane * (unsigned)sizeof(T), rot),
+                                       g.centre_w);
     const bool in = (h > -1.f) && (w > -1.f) && (h < float(SH)) && (w < float(SW));
-    const float hf = floorf(h), wf = floorf(w);
-    lh[t] = h - hf;
-    lw[t] = w - wf;
-    cell[t] = in ? (static_cast<int>(hf) + 1) * Tb::RS + static_cast<int>(wf) + 1 : 0;
-    live |= ok ? (1u << t) : 0u;
+    cell[t] = Tb::slot(in ? (static_cast<int>(floorf(h)) + 1) * Tb::RS + static_cast<int>(floorf(w)) + 1 : 0) * 4;
     inside |= (in && ok) ? (1u << t) : 0u;
+    live |= ok ? (1u << t) : 0u;
   }
+  if (ROWS) {
+#pragma unroll
+    for (int r = 0; r < KH; ++r) {
+      const long e = (long)p + (long)(r * g.dil_h - g.pad_h) * g.in_w;
+      soff[r] = (e >= 0 && e < in_plane) ? (unsigned)e * (unsigned)sizeof(T) : kOutOfRange;
+    }
+  }
+  const unsigned goff = owns ? (unsigned)p * (unsigned)sizeof(T) : kOutOfRange;
 
   float s00[K], s01[K], s10[K], s11[K];
 #pragma unroll
@@ -281,41 +410,67 @@ __global__ __launch_bounds__(kBlock) void local_grad_rotation_kernel(
   for (int j0 = 0; j0 < cpg; j0 += ch_per_pass) {
     const int nch = min(ch_per_pass, cpg - j0);
     __syncthreads();
-    stage_tables<T, SH, SW>(tbl, filter, grp + g.groups * j0, g.groups, nch);
+    stage_wide_tables<T, SH, SW>(tbl, filter, grp + g.groups * j0, g.groups, nch);
     __syncthreads();
-    if (active) {
-      const size_t chan0 = (size_t)n * g.channel + grp + (size_t)g.groups * j0;
-      const T* xp = x + chan0 * in_plane;
-      const T* gp = gout + chan0 * out_plane + p;
-#pragma unroll 2
-      for (int j = 0; j < nch; ++j) {
-        const float* tb = tbl + j * Tb::SIZE;
-        const float go = ld(gp);
+    const size_t chan0 = (size_t)n * g.channel + grp + (size_t)g.groups * j0;
+    const T* xp = x + chan0 * in_plane;
+    const T* gp = gout + chan0 * out_plane;
+    const size_t x_step = (size_t)g.groups * in_plane, g_step = (size_t)g.groups * out_plane;
+
+    float xv[2][NLOAD], gv[2];
+    auto load = [&](int s, int j) {
+      const rsrc_t rx = plane_rsrc(xp + (size_t)j * x_step, j < nch ? in_plane : 0);
+      const rsrc_t rg = plane_rsrc(gp + (size_t)j * g_step, j < nch ? out_plane : 0);
+      gv[s] = buf_ld(rg, goff, gout);
 #pragma unroll
-        for (int t = 0; t < K; ++t) {
-          const float xv = (live >> t & 1u) ? ld(xp + soff[t]) : 0.f;
-          const float ps = xv * go;
-          const float* q = tb + cell[t];
-          s00[t] += ps * q[0];
-          s01[t] += ps * q[1];
-          s10[t] += ps * q[Tb::RS];
-          s11[t] += ps * q[Tb::RS + 1];
+      for (int t = 0; t < NLOAD; ++t) xv[s][t] = buf_ld(rx, soff[t], x);
+    };
+    auto accumulate = [&](int s, int j) {
+      const float* tb = tbl + min(j, nch - 1) * Tb::SIZE;  // j >= nch only with zero inputs
+#pragma unroll
+      for (int t = 0; t < K; ++t) {
+        float xt;
+        if (ROWS) {
+          const int r = t / KW, f_w = t % KW;
+          xt = f_w == 0 ? from_lane_below(xv[s][r]) : f_w == 1 ? xv[s][r] : from_lane_above(xv[s][r]);
+        } else {
+          xt = xv[s][t];
         }
-        xp += (size_t)g.groups * in_plane;
-        gp += (size_t)g.groups * out_plane;
+        // gv is 0 on lanes that own no pixel, and taps in the padding are masked at the end
+        const float ps = xt * gv[s];
+        const float4 q = *reinterpret_cast<const float4*>(tb + cell[t]);
+        s00[t] += ps * q.x;
+        s01[t] += ps * q.y;
+        s10[t] += ps * q.z;
+        s11[t] += ps * q.w;
       }
+    };
+    load(0, 0);
+    for (int j = 0; j < nch; j += 2) {
+      load(1, j + 1);
+      accumulate(0, j);
+      load(0, j + 2);
+      accumulate(1, j + 1);
     }
   }
-  if (!active) return;
+
+  const rsrc_t ro_ = plane_rsrc(grot + rplane0, K * 2 * out_plane);
 #pragma unroll
   for (int t = 0; t < K; ++t) {
-    const float hh = 1.f - lh[t], hw = 1.f - lw[t];
-    float gh = hw * (s10[t] - s00[t]) + lw[t] * (s11[t] - s01[t]);
-    float gw = hh * (s01[t] - s00[t]) + lh[t] * (s11[t] - s10[t]);
+    const int f_h = t / KW, f_w = t % KW;
+    const unsigned ro = owns ? (unsigned)((2 * t) * out_plane + pc) * (unsigned)sizeof(T) : kOutOfRange;
+    const float h = scope_coord<float>(f_h, buf_ld(rr, ro, rot), g.centre_h);
+    const float w = scope_coord<float>(f_w, buf_ld(rr, ro + (unsigned)out_plane * (unsigned)sizeof(T), rot),
+                                       g.centre_w);
+    const float lh = h - floorf(h), lw = w - floorf(w);
+    const float hh = 1.f - lh, hw = 1.f - lw;
+    float gh = hw * (s10[t] - s00[t]) + lw * (s11[t] - s01[t]);
+    float gw = hh * (s01[t] - s00[t]) + lh * (s11[t] - s10[t]);
     if (!(inside >> t & 1u)) gh = gw = 0.f;
-    st(grot + rplane0 + (size_t)(2 * t) * out_plane + p, gh);
-    st(grot + rplane0 + (size_t)(2 * t + 1) * out_plane + p, gw);
+    buf_st(ro_, ro, gh, grot);
+    buf_st(ro_, ro + (unsigned)out_plane * (unsigned)sizeof(T), gw, grot);
   }
+  (void)live;
 }
 
 // ---------------------------------------------------------------------------
@@ -503,6 +658,13 @@ namespace {
 
 constexpr int kMaxLdsTables = 96 * 1024;  // bytes of LDS a workgroup may spend on scope tables
 
+// stride 1, unit column spacing and pad_w = 1: input and output planes share their width and a
+// pixel's taps are three runs of three consecutive elements
+bool same_width_geometry(const Geo& g) {
+  return g.stride_h == 1 && g.stride_w == 1 && g.dil_w == 1 && g.pad_w == 1 && g.k_w == 3 &&
+         g.in_w == g.out_w && !getenv("DK_NO_ROWS");
+}
+
 template <int SH, int SW>
 int channels_per_block(int cpg, int wanted_splits) {
   const int fit = kMaxLdsTables / (Table<SH, SW>::SIZE * 4);
@@ -528,6 +690,16 @@ bool run_gather(const Geo& g, bool transposed, const T* src, const T* rot, const
                 hipStream_t stream) {
   const int cpg = g.channel / g.groups;
   const int pixels = transposed ? g.in_h * g.in_w : g.out_h * g.out_w;
+  if (same_width_geometry(g)) {
+    const int per = channels_per_block<SH, SW>(cpg, pick_splits(g, pixels));
+    const dim3 grid(ceil_div(pixels, kRowPix), ceil_div(cpg, per), g.batch * g.groups);
+    const size_t lds = (size_t)(per + 2 * kUnroll) * WideTable<SH, SW>::SIZE * sizeof(float);
+    if (transposed)
+      local_gather_rows_kernel<T, 3, SH, SW, true><<<grid, kBlock, lds, stream>>>(g, src, rot, filter, dst, per);
+    else
+      local_gather_rows_kernel<T, 3, SH, SW, false><<<grid, kBlock, lds, stream>>>(g, src, rot, filter, dst, per);
+    return true;
+  }
   const int per = channels_per_block<SH, SW>(cpg, pick_splits(g, pixels));
   const dim3 grid(ceil_div(pixels, kBlock), ceil_div(cpg, per), g.batch * g.groups);
   // stages past the last channel still read (and discard) table entries: pad to whole stages
@@ -542,11 +714,17 @@ bool run_gather(const Geo& g, bool transposed, const T* src, const T* rot, const
 template <typename T, int SH, int SW>
 bool run_grad_rotation(const Geo& g, const T* gout, const T* x, const T* rot, const T* filter,
                        T* grot, hipStream_t stream) {
+  using Tb = WideTable<SH, SW>;
   const int cpg = g.channel / g.groups;
-  const int per = channels_per_block<SH, SW>(cpg, 1);
-  const dim3 grid(ceil_div(g.out_h * g.out_w, kBlock), 1, g.batch * g.groups);
-  const size_t lds = (size_t)per * Table<SH, SW>::SIZE * sizeof(float);
-  local_grad_rotation_kernel<T, 3, 3, SH, SW><<<grid, kBlock, lds, stream>>>(g, gout, x, rot, filter, grot, per);
+  const int per = cpg < 36 ? cpg : 36;  // channels staged per pass
+  const size_t lds = (size_t)per * Tb::SIZE * sizeof(float);
+  if (same_width_geometry(g)) {
+    const dim3 grid(ceil_div(g.out_h * g.out_w, kRowPix), 1, g.batch * g.groups);
+    local_grad_rotation_kernel<T, 3, 3, SH, SW, true><<<grid, kBlock, lds, stream>>>(g, gout, x, rot, filter, grot, per);
+  } else {
+    const dim3 grid(ceil_div(g.out_h * g.out_w, kBlock), 1, g.batch * g.groups);
+    local_grad_rotation_kernel<T, 3, 3, SH, SW, false><<<grid, kBlock, lds, stream>>>(g, gout, x, rot, filter, grot, per);
+  }
   return true;
 }
 
