@@ -487,12 +487,14 @@ __global__ __launch_bounds__(kBlock, 2) void local_grad_rotation_kernel(
 // workgroup goes to the workspace; reduce_partials_kernel adds the partials in order.
 // grid = (parts, channel splits, groups)
 // ---------------------------------------------------------------------------
-template <typename T, int KH, int KW, int SH, int SW>
+template <typename T, int KH, int KW, int SH, int SW, bool ROWS>
 __global__ __launch_bounds__(kBlock, 2) void local_grad_filter_kernel(
     Geo g, const T* __restrict__ gout, const T* __restrict__ x, const T* __restrict__ rot,
     float* __restrict__ partial, int tiles, int ch_per_block) {
   constexpr int K = KH * KW;
   constexpr int CELLS = SH * SW;
+  constexpr int NLOAD = ROWS ? KH : K;
+  constexpr int PIX = ROWS ? kRowPix : kBlock;  // pixels per (image, tile) item
   static_assert(CELLS <= 16, "the fold below handles up to 16 cells per 16-lane row");
   constexpr int kPitch = 20;  // floats per lane in the transpose scratch: 16-byte aligned, bank-skewed
   constexpr int kWaves = kBlock / 64;
@@ -518,27 +520,28 @@ __global__ __launch_bounds__(kBlock, 2) void local_grad_filter_kernel(
 
   for (int item = blockIdx.x; item < items; item += gridDim.x) {
     const int n = item / tiles, tile = item % tiles;
-    const int p = tile * kBlock + threadIdx.x;
-    const bool active = p < out_plane;
-    const int pc = active ? p : 0;
+    const int p = ROWS ? tile * PIX + wave * kRowLanes + lane - 1 : tile * PIX + (int)threadIdx.x;
+    const bool owns = (ROWS ? (lane >= 1 && lane <= kRowLanes) : true) && p < out_plane;
+    const int pc = owns ? p : 0;
     const int ph = pc / g.out_w, pw = pc % g.out_w;
 
     float ah[K][SH], bw[K][SW];
-    unsigned soff[K];
+    unsigned soff[NLOAD];
     const rsrc_t rr = plane_rsrc(rot + (size_t)(n * g.groups + grp) * (K * 2) * out_plane, K * 2 * out_plane);
 #pragma unroll
     for (int t = 0; t < K; ++t) {
       const int f_h = t / KW, f_w = t % KW;
       int s_el, rpix;
-      const bool ok = tap_geometry<false>(g, ph, pw, f_h, f_w, s_el, rpix) && active;
-      soff[t] = ok ? (unsigned)s_el * (unsigned)sizeof(T) : kOutOfRange;
+      const bool ok = tap_geometry<false>(g, ph, pw, f_h, f_w, s_el, rpix) && owns;
+      if (!ROWS) soff[t] = ok ? (unsigned)s_el * (unsigned)sizeof(T) : kOutOfRange;
       const unsigned ro = ok ? (unsigned)((2 * t) * out_plane + rpix) * (unsigned)sizeof(T) : kOutOfRange;
       const float h = scope_coord<float>(f_h, buf_ld(rr, ro, rot), g.centre_h);
       const float w = scope_coord<float>(f_w, buf_ld(rr, ro + (unsigned)out_plane * (unsigned)sizeof(T), rot),
                                          g.centre_w);
       // hat(h - i) = lh at i = floor(h) + 1, 1 - lh at i = floor(h), else 0: the same products
-      // (hh, lh) x (hw, lw) as K.cu:101-112, laid out densely; all zero outside (-1, S).
-      const bool in = (h > -1.f) && (w > -1.f) && (h < float(SH)) && (w < float(SW));
+      // (hh, lh) x (hw, lw) as K.cu:101-112, laid out densely; all zero outside (-1, S) and for
+      // taps in the padding.
+      const bool in = ok && (h > -1.f) && (w > -1.f) && (h < float(SH)) && (w < float(SW));
       const float hf = floorf(h), wf = floorf(w);
       const int hl = in ? (int)hf : -8, wl = in ? (int)wf : -8;
       const float lh = h - hf, lw = w - wf;
@@ -547,20 +550,27 @@ __global__ __launch_bounds__(kBlock, 2) void local_grad_filter_kernel(
 #pragma unroll
       for (int i = 0; i < SW; ++i) bw[t][i] = (i == wl) ? 1.f - lw : (i == wl + 1) ? lw : 0.f;
     }
-    const unsigned goff = active ? (unsigned)p * (unsigned)sizeof(T) : kOutOfRange;
+    if (ROWS) {
+#pragma unroll
+      for (int r = 0; r < KH; ++r) {
+        const long e = (long)p + (long)(r * g.dil_h - g.pad_h) * g.in_w;
+        soff[r] = (e >= 0 && e < in_plane) ? (unsigned)e * (unsigned)sizeof(T) : kOutOfRange;
+      }
+    }
+    const unsigned goff = owns ? (unsigned)p * (unsigned)sizeof(T) : kOutOfRange;
 
     const size_t chan0 = (size_t)n * g.channel + grp + (size_t)g.groups * j0;
     const T* xp = x + chan0 * in_plane;
     const T* gp = gout + chan0 * out_plane;
     const size_t x_step = (size_t)g.groups * in_plane, g_step = (size_t)g.groups * out_plane;
 
-    float xv[2][K], gv[2];
+    float xv[2][NLOAD], gv[2];
     auto load = [&](int s, int j) {
       const rsrc_t rx = plane_rsrc(xp + (size_t)j * x_step, j < nch ? in_plane : 0);
       const rsrc_t rg = plane_rsrc(gp + (size_t)j * g_step, j < nch ? out_plane : 0);
       gv[s] = buf_ld(rg, goff, gout);
 #pragma unroll
-      for (int t = 0; t < K; ++t) xv[s][t] = buf_ld(rx, soff[t], x);
+      for (int t = 0; t < NLOAD; ++t) xv[s][t] = buf_ld(rx, soff[t], x);
     };
     auto accumulate = [&](int s, int j) {
       float acc[SH][SW];
@@ -570,7 +580,14 @@ __global__ __launch_bounds__(kBlock, 2) void local_grad_filter_kernel(
         for (int k = 0; k < SW; ++k) acc[i][k] = 0.f;
 #pragma unroll
       for (int t = 0; t < K; ++t) {
-        const float ps = xv[s][t] * gv[s];
+        float xt;
+        if (ROWS) {
+          const int r = t / KW, f_w = t % KW;
+          xt = f_w == 0 ? from_lane_below(xv[s][r]) : f_w == 1 ? xv[s][r] : from_lane_above(xv[s][r]);
+        } else {
+          xt = xv[s][t];
+        }
+        const float ps = xt * gv[s];
         float u[SW];
 #pragma unroll
         for (int k = 0; k < SW; ++k) u[k] = ps * bw[t][k];
@@ -620,31 +637,34 @@ __global__ __launch_bounds__(kBlock, 2) void local_grad_filter_kernel(
 
 }  // namespace
 
-// out[e] = sum over parts of partial[part][e].  32 elements per workgroup, 8 threads per
-// element each summing every 8th part, combined in a fixed order (run-to-run reproducible).
+// out[e] = sum over parts of partial[part][e].  8 elements per workgroup, 32 threads per
+// element each summing every 32nd part, combined in a fixed order (run-to-run reproducible).
+constexpr int kRedEl = 8, kRedSlices = 32;
+
 template <typename CT, typename T>
-__global__ __launch_bounds__(256) void reduce_partials_kernel(const CT* __restrict__ partial,
-                                                              int parts, int count,
-                                                              T* __restrict__ out) {
-  __shared__ CT part_sum[8][32];
-  const int el = threadIdx.x & 31, slice = threadIdx.x >> 5;
-  const int e = blockIdx.x * 32 + el;
+__global__ __launch_bounds__(kRedEl * kRedSlices) void reduce_partials_kernel(
+    const CT* __restrict__ partial, int parts, int count, T* __restrict__ out) {
+  __shared__ CT part_sum[kRedSlices][kRedEl];
+  const int el = threadIdx.x % kRedEl, slice = threadIdx.x / kRedEl;
+  const int e = blockIdx.x * kRedEl + el;
   CT s = 0;
-  if (e < count)
-    for (int q = slice; q < parts; q += 8) s += partial[(size_t)q * count + e];
+  if (e < count) {
+#pragma unroll 4
+    for (int q = slice; q < parts; q += kRedSlices) s += partial[(size_t)q * count + e];
+  }
   part_sum[slice][el] = s;
   __syncthreads();
   if (slice == 0 && e < count) {
     CT t = 0;
 #pragma unroll
-    for (int k = 0; k < 8; ++k) t += part_sum[k][el];
+    for (int k = 0; k < kRedSlices; ++k) t += part_sum[k][el];
     st(out + e, t);
   }
 }
 
 template <typename CT, typename T>
 void launch_reduce_partials(const CT* partial, int parts, int count, T* out, hipStream_t stream) {
-  reduce_partials_kernel<CT, T><<<ceil_div(count, 32), 256, 0, stream>>>(partial, parts, count, out);
+  reduce_partials_kernel<CT, T><<<ceil_div(count, kRedEl), kRedEl * kRedSlices, 0, stream>>>(partial, parts, count, out);
 }
 template void launch_reduce_partials<float, float>(const float*, int, int, float*, hipStream_t);
 template void launch_reduce_partials<float, __half>(const float*, int, int, __half*, hipStream_t);
@@ -730,7 +750,7 @@ bool run_grad_rotation(const Geo& g, const T* gout, const T* x, const T* rot, co
 
 // grad-filter launch shape: channel splits of at most kFilterChPerBlock channels, and enough
 // (image, tile) parts that the grid has a few workgroups per CU.
-constexpr int kFilterChPerBlock = 72;
+constexpr int kFilterChPerBlock = 36;
 
 struct FilterGrid {
   int per, splits, parts, tiles;
@@ -741,10 +761,11 @@ FilterGrid filter_grid(const Geo& g) {
   const int cpg = g.channel / g.groups;
   f.splits = ceil_div(cpg, kFilterChPerBlock);
   f.per = ceil_div(cpg, f.splits);
-  f.tiles = ceil_div(g.out_h * g.out_w, kBlock);
+  f.tiles = ceil_div(g.out_h * g.out_w, same_width_geometry(g) ? kRowPix : kBlock);
   const int items = g.batch * f.tiles;
-  f.parts = ceil_div(1024, f.splits * g.groups);
-  if (f.parts > items) f.parts = items;
+  // one (image, tile) item per workgroup while that keeps the partial buffer small; many more
+  // workgroups than the GPU holds at once, so the dispatcher evens out the load
+  f.parts = items < 1024 ? items : 1024;
   if (f.parts < 1) f.parts = 1;
   return f;
 }
@@ -758,7 +779,10 @@ bool run_grad_filter(const Geo& g, const T* gout, const T* x, const T* rot, T* g
     const FilterGrid f = filter_grid(g);
     const dim3 grid(f.parts, f.splits, g.groups);
     const size_t lds = ((size_t)(kBlock / 64) * f.per * 16 + (size_t)(kBlock / 64) * 64 * 20) * sizeof(float);
-    local_grad_filter_kernel<T, 3, 3, SH, SW><<<grid, kBlock, lds, stream>>>(g, gout, x, rot, ws, f.tiles, f.per);
+    if (same_width_geometry(g))
+      local_grad_filter_kernel<T, 3, 3, SH, SW, true><<<grid, kBlock, lds, stream>>>(g, gout, x, rot, ws, f.tiles, f.per);
+    else
+      local_grad_filter_kernel<T, 3, 3, SH, SW, false><<<grid, kBlock, lds, stream>>>(g, gout, x, rot, ws, f.tiles, f.per);
     launch_reduce_partials<float, T>(ws, f.parts, g.channel * SH * SW, gfilter, stream);
     return true;
   }
