@@ -35,6 +35,15 @@ WORKLOADS = {
 }
 DTYPES = {"fp32": "float32", "bf16": "bfloat16", "fp16": "float16"}
 
+# Other rows of the operator path, timed per entry point with --workload (not the headline metric).
+OTHER_WORKLOADS = {
+    # deformable variant, BASELINE config 4: N, C, H, W, k, S, stride, pad, dil, groups, rot_std, off_std
+    "cfg4": ("deform", (64, 512, 28, 28, 3, (4, 4), 2, 1, 1, 1, 0.5, 2.0)),
+    # N-d sampler: data shape [C, s...], points, coordinate range
+    "nd_cfg3": ("nd", ((256, 5, 5), 1152, (0.0, 4.0))),             # GlobalDeformKernel2d, config 3
+    "nd_cfg5": ("nd", ((64, 32, 32, 32), 1 << 20, (-1.0, 32.0))),   # trilinear volume, config 5, full-volume coords
+}
+
 
 def algorithmic_bytes(N, C, H, W, Ho, Wo, k, S, groups, esz):
     """Compulsory traffic, every tensor touched once (bytes), per kernel and per step."""
@@ -58,7 +67,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--workload", default="cfg2", choices=sorted(WORKLOADS))
+    ap.add_argument("--workload", default="cfg2", choices=sorted(WORKLOADS) + sorted(OTHER_WORKLOADS))
     ap.add_argument("--dtype", default="fp32", choices=sorted(DTYPES))
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--kernels", default="", help="comma list restricting the per-kernel timing (tuning aid)")
@@ -74,6 +83,8 @@ def main():
 
     if not torch.cuda.is_available():
         sys.exit("bench.py needs a GPU")
+    if a.workload in OTHER_WORKLOADS:
+        return other_workload(a)
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
     tdtype = getattr(torch, DTYPES[a.dtype])
@@ -184,6 +195,93 @@ def main():
     if not a.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(N, C, H, W, k, S, stride, pad, dil, groups, rot_std, esz)
     print(json.dumps(result))
+
+
+def _time_us(fn, reps):
+    import torch
+    fn()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(reps):
+        fn()
+    e1.record()
+    e1.synchronize()
+    return e0.elapsed_time(e1) * 1e3 / reps
+
+
+def other_workload(a):
+    """Per-entry-point timing of the deformable variant or the N-d sampler (one JSON line,
+    `metric` says which; these are not the BASELINE headline)."""
+    import torch
+    from _cases import make_deform
+    from deformable_kernels.ops.deform_kernel import _lib
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    tdtype = getattr(torch, DTYPES[a.dtype])
+    kind, spec = OTHER_WORKLOADS[a.workload]
+    L, P = _lib.lib(), _lib.ptr
+    reps = max(a.steps, 10)
+    us, nbytes = {}, {}
+    if kind == "deform":
+        N, C, H, W, k, S, stride, pad, dil, groups, rot_std, off_std = spec
+        x, wt, rot, off, gout, cfg = make_deform(N, C, H, W, k, S, stride, pad, dil, groups, rot_std, off_std,
+                                                 seed=0, dtype=tdtype)
+        xg, wg, rg, og, gg = [t.to(dev) for t in (x, wt, rot, off, gout)]
+        out, gin, grot, goff, gw = [torch.empty_like(t) for t in (gg, xg, rg, og, wg)]
+        desc = _lib.conv_desc(xg, wg, cfg["kernel_size"], cfg["stride"], cfg["padding"], cfg["dilation"], groups)
+        ws1, n1 = _lib.workspace(L.dk_deformable_sample_depthwise_backward_data_workspace(desc), dev)
+        ws2, n2 = _lib.workspace(L.dk_deformable_sample_depthwise_backward_filter_workspace(desc), dev)
+        st = _lib.stream_ptr(xg)
+        e = xg.element_size()
+        bx, by, br, bo, bw = [t.numel() * e for t in (xg, gg, rg, og, wg)]
+        calls = {
+            "forward": (lambda: _lib.check(L.dk_deformable_sample_depthwise_forward(
+                desc, P(xg), P(og), P(rg), P(wg), P(out), st), "fwd"), bx + bo + br + bw + by),
+            "grad_input": (lambda: _lib.check(L.dk_deformable_sample_depthwise_backward_data(
+                desc, P(gg), P(og), P(rg), P(wg), P(gin), P(ws1), n1, st), "gin"), by + bo + br + bw + bx),
+            "grad_offset": (lambda: _lib.check(L.dk_deformable_sample_depthwise_backward_offset(
+                desc, P(gg), P(xg), P(og), P(rg), P(wg), P(goff), st), "goff"), by + bx + bo + br + bw + bo),
+            "grad_rotation": (lambda: _lib.check(L.dk_deformable_sample_depthwise_backward_rotation(
+                desc, P(gg), P(xg), P(og), P(rg), P(wg), P(grot), st), "grot"), by + bx + bo + br + bw + br),
+            "grad_filter": (lambda: _lib.check(L.dk_deformable_sample_depthwise_backward_filter(
+                desc, P(gg), P(xg), P(og), P(rg), P(gw), P(ws2), n2, st), "gw"), by + bx + bo + br + bw),
+        }
+        label = "cfg4: deform_sample_depthwise N=%d C=%d %dx%d->%dx%d k=%d scope=%dx%d stride=%d %s" % (
+            N, C, H, W, gg.shape[2], gg.shape[3], k, S[0], S[1], stride, a.dtype)
+    else:
+        shape, B, (lo, hi) = spec
+        g = torch.Generator().manual_seed(0)
+        data = torch.randn(*shape, generator=g).to(tdtype).to(dev)
+        coord = (torch.rand(B, len(shape) - 1, generator=g) * (hi - lo) + lo).to(tdtype).to(dev)
+        go = torch.randn(B, shape[0], generator=g).to(tdtype).to(dev)
+        out, gd, gc = torch.empty_like(go), torch.empty_like(data), torch.empty_like(coord)
+        desc = _lib.nd_desc(data, coord)
+        ws, nb = _lib.workspace(L.dk_nd_linear_sample_backward_data_workspace(desc), dev)
+        wf, nf = _lib.workspace(L.dk_nd_linear_sample_forward_workspace(desc), dev)
+        st = _lib.stream_ptr(data)
+        e = data.element_size()
+        bd, bc, bo = data.numel() * e, coord.numel() * e, go.numel() * e
+        calls = {
+            "forward": (lambda: _lib.check(L.dk_nd_linear_sample_forward(desc, P(data), P(coord), P(out), P(wf), nf, st), "fwd"),
+                        bd + bc + bo),
+            "grad_data": (lambda: _lib.check(L.dk_nd_linear_sample_backward_data(
+                desc, P(go), P(coord), P(gd), P(ws), nb, st), "gd"), bo + bc + bd),
+            "grad_coord": (lambda: _lib.check(L.dk_nd_linear_sample_backward_coord(
+                desc, P(go), P(data), P(coord), P(gc), P(wf), nf, st), "gc"), bo + bd + bc + bc),
+        }
+        label = "%s: nd_linear_sample data=%s points=%d %s" % (a.workload, list(shape), B, a.dtype)
+    for name, (fn, nb_) in calls.items():
+        us[name] = _time_us(fn, reps)
+        nbytes[name] = nb_
+    total_us = sum(us.values())
+    print(json.dumps({
+        "metric": "per-entry-point time (secondary workload, not the BASELINE headline)",
+        "config": {"workload": label},
+        "kernel_us": {k_: round(v, 2) for k_, v in us.items()},
+        "algorithmic_GBps": {k_: round(nbytes[k_] / (us[k_] * 1e-6) / 1e9, 1) for k_ in us},
+        "sum_us": round(total_us, 2),
+        "n_gpus": 1, "dtype": a.dtype, "data": "synthetic",
+    }))
 
 
 def cpu_baseline(N, C, H, W, k, S, stride, pad, dil, groups, rot_std, esz):

@@ -297,14 +297,24 @@ static int check_nd(const dk_nd_desc* d) {
   return DK_OK;
 }
 
+size_t dk_nd_linear_sample_forward_workspace(const dk_nd_desc* desc) {
+  if (check_nd(desc) != DK_OK) return 0;
+  return nd_data_cl_workspace(*desc);
+}
+
 int dk_nd_linear_sample_forward(const dk_nd_desc* desc, const void* data, const void* coord,
-                                void* output, void* stream) {
+                                void* output, void* workspace, size_t workspace_bytes,
+                                void* stream) {
   const int rc = check_nd(desc);
   if (rc != DK_OK) return rc;
   if (!data || !coord || !output) return DK_ERR_NULL_POINTER;
+  const size_t need = nd_data_cl_workspace(*desc);
+  if (need && (!workspace || workspace_bytes < need)) return DK_ERR_WORKSPACE;
   if (desc->batch == 0) return DK_OK;
   hipStream_t s = static_cast<hipStream_t>(stream);
-  return by_dtype(desc->dtype, [&]<typename T>() { nd_forward<T>(*desc, in<T>(data), in<T>(coord), out<T>(output), s); });
+  return by_dtype(desc->dtype, [&]<typename T>() {
+    nd_forward<T>(*desc, in<T>(data), in<T>(coord), out<T>(output), workspace, s);
+  });
 }
 
 size_t dk_nd_linear_sample_backward_data_workspace(const dk_nd_desc* desc) {
@@ -326,16 +336,23 @@ int dk_nd_linear_sample_backward_data(const dk_nd_desc* desc, const void* out_gr
   });
 }
 
+size_t dk_nd_linear_sample_backward_coord_workspace(const dk_nd_desc* desc) {
+  if (check_nd(desc) != DK_OK) return 0;
+  return nd_data_cl_workspace(*desc);
+}
+
 int dk_nd_linear_sample_backward_coord(const dk_nd_desc* desc, const void* out_grad,
                                        const void* data, const void* coord, void* coord_grad,
-                                       void* stream) {
+                                       void* workspace, size_t workspace_bytes, void* stream) {
   const int rc = check_nd(desc);
   if (rc != DK_OK) return rc;
   if (desc->batch == 0) return DK_OK;
   if (!out_grad || !data || !coord || !coord_grad) return DK_ERR_NULL_POINTER;
+  const size_t need = nd_data_cl_workspace(*desc);
+  if (need && (!workspace || workspace_bytes < need)) return DK_ERR_WORKSPACE;
   hipStream_t s = static_cast<hipStream_t>(stream);
   return by_dtype(desc->dtype, [&]<typename T>() {
-    nd_grad_coord<T>(*desc, in<T>(out_grad), in<T>(data), in<T>(coord), out<T>(coord_grad), s);
+    nd_grad_coord<T>(*desc, in<T>(out_grad), in<T>(data), in<T>(coord), out<T>(coord_grad), workspace, s);
   });
 }
 

@@ -144,6 +144,21 @@ __device__ __forceinline__ ImageTap<CT> make_image_tap(CT h, CT w, int H, int W)
 
 __host__ __device__ __forceinline__ int ceil_div(int a, int b) { return (a + b - 1) / b; }
 
+// Sum of v over the 64 lanes of the wave, returned in every lane: six DPP adds and one readlane
+// (no LDS crossbar traffic, unlike a shuffle-based butterfly).
+__device__ __forceinline__ float wave_sum(float v) {
+#define DK_DPP_ADD(ctrl, row_mask)                                                              \
+  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), ctrl, row_mask, 0xf, true))
+  DK_DPP_ADD(0xB1, 0xf);   // quad_perm [1,0,3,2]
+  DK_DPP_ADD(0x4E, 0xf);   // quad_perm [2,3,0,1]
+  DK_DPP_ADD(0x141, 0xf);  // row_half_mirror
+  DK_DPP_ADD(0x140, 0xf);  // row_mirror: every lane now holds its 16-lane row's sum
+  DK_DPP_ADD(0x142, 0xa);  // row_bcast15 into rows 1 and 3
+  DK_DPP_ADD(0x143, 0xc);  // row_bcast31 into rows 2 and 3: lane 63 holds the total
+#undef DK_DPP_ADD
+  return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 63));
+}
+
 // Value held by the previous / next lane of the wave (0 at the wave's ends): one DPP move.
 __device__ __forceinline__ float from_lane_below(float v) {
   return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x138 /* wave_shr:1 */, 0xf, 0xf, true));

@@ -4,11 +4,17 @@
 //   nd_linear ND.cu:45-88, nd_linear_backward_data ND.cu:90-131,
 //   nd_linear_backward_coord ND.cu:133-177; kernels ND.cu:183-287.
 //
-// The per-point work (which 2^n corners exist and with what weight) does not
-// depend on the channel, so each lane derives it once from its point and then
-// only multiplies and adds per corner.  The coordinate gradient is reduced over
-// channels inside the kernel (one wave per point, lanes over channels, shuffle
-// reduction) instead of materialising the reference's [B, n, C] intermediate.
+// Two paths.
+//  * Channel-last path (1..3 sampling dimensions, enough work to pay for a transpose):
+//    `data` [C, P] is first copied to [P, C] in the caller's workspace, so the C values of
+//    one corner are contiguous.  A wave takes 64 points: with lane <-> point it derives each
+//    point's 2^n corner offsets and weights once, then walks its points with lane <-> channel,
+//    broadcasting the point's corners by readlane; every corner read and every output row
+//    is one contiguous run.  The reference maps adjacent threads to adjacent channels whose
+//    data lie a whole volume apart (ND.cu:197-199).
+//  * Direct path (any dimension count, small problems): one lane per (point, channel).
+// The coordinate gradient is reduced over channels inside the kernel instead of
+// materialising the reference's [B, n, C] intermediate (ND.cu:281-286 and the caller's sum).
 #include "dk_nd.h"
 
 namespace dk {
@@ -16,6 +22,8 @@ namespace dk {
 namespace {
 
 constexpr int kBlock = 256;
+constexpr int kClMaxDims = 3;
+constexpr int kClCorners = 1 << kClMaxDims;
 
 struct NdGeo {
   long batch;
@@ -24,13 +32,14 @@ struct NdGeo {
   int shape[DK_ND_MAX_DIMS];
 };
 
-// Per-point corner bookkeeping: low index and fractional weight per dimension,
-// and whether the whole sample is void (any x <= -1 or x >= s, ND.cu:47-53).
+// ---------------------------------------------------------------------------
+// per-point corner bookkeeping shared by both paths
+// ---------------------------------------------------------------------------
 template <typename CT>
 struct NdPoint {
   int low[DK_ND_MAX_DIMS];
   CT frac[DK_ND_MAX_DIMS];
-  bool inside;
+  bool inside;  // false: some x <= -1 or x >= s, the whole sample is zero (ND.cu:47-53)
 };
 
 template <typename T, typename CT>
@@ -42,8 +51,9 @@ __device__ __forceinline__ NdPoint<CT> load_point(const NdGeo& g, const T* coord
     if (d < g.dims) {
       const CT x = ld(coord_b + d);
       const CT xf = floor(x);
-      if (!(x > CT(-1) && x < CT(g.shape[d]))) p.inside = false;
-      p.low[d] = (x > CT(-1) && x < CT(g.shape[d])) ? (int)xf : 0;
+      const bool in = x > CT(-1) && x < CT(g.shape[d]);
+      if (!in) p.inside = false;
+      p.low[d] = in ? (int)xf : 0;
       p.frac[d] = x - xf;
     } else {
       p.low[d] = 0;
@@ -53,9 +63,9 @@ __device__ __forceinline__ NdPoint<CT> load_point(const NdGeo& g, const T* coord
   return p;
 }
 
-// Offset and weight of corner `i` (bit d selects low/high in dimension d,
-// ND.cu:67); `skip_dim` >= 0 replaces that dimension's weight by -1 / +1
-// (ND.cu:161,165).  Returns false where the reference breaks out of the corner.
+// Offset and weight of corner `i` (bit d selects low/high in dimension d, ND.cu:67);
+// `skip_dim` >= 0 replaces that dimension's weight by -1 / +1 (ND.cu:161,165).
+// Returns false where the reference breaks out of the corner.
 template <typename CT>
 __device__ __forceinline__ bool corner(const NdGeo& g, const NdPoint<CT>& p, unsigned i,
                                        int skip_dim, long& offset, CT& weight) {
@@ -81,7 +91,9 @@ __device__ __forceinline__ bool corner(const NdGeo& g, const NdPoint<CT>& p, uns
   return true;
 }
 
-// forward, ND.cu:183-201: one thread per (b, c), c fastest.
+// ---------------------------------------------------------------------------
+// direct path
+// ---------------------------------------------------------------------------
 template <typename T>
 __global__ __launch_bounds__(kBlock) void nd_forward_kernel(NdGeo g, const T* __restrict__ data,
                                                             const T* __restrict__ coord,
@@ -104,8 +116,9 @@ __global__ __launch_bounds__(kBlock) void nd_forward_kernel(NdGeo g, const T* __
   }
 }
 
-// grad data, ND.cu:225-243: scatter with hardware float atomics into a zeroed buffer.
-template <typename T, typename CT>
+// scatter with hardware float atomics into a zeroed buffer laid out [C][P] (cl = false) or
+// [P][C] (cl = true)
+template <typename T, typename CT, bool CL>
 __global__ __launch_bounds__(kBlock) void nd_grad_data_kernel(NdGeo g, const T* __restrict__ gout,
                                                               const T* __restrict__ coord,
                                                               CT* __restrict__ gdata, long total) {
@@ -115,16 +128,16 @@ __global__ __launch_bounds__(kBlock) void nd_grad_data_kernel(NdGeo g, const T* 
     const NdPoint<CT> p = load_point<T, CT>(g, coord + b * g.dims);
     if (!p.inside) continue;
     const CT go = ld(gout + id);
-    CT* dc = gdata + (size_t)c * g.prod_shape;
     for (unsigned i = 0; i < (1u << g.dims); ++i) {
       long o;
       CT w;
-      if (corner<CT>(g, p, i, -1, o, w)) atomicAdd(dc + o, w * go);
+      if (corner<CT>(g, p, i, -1, o, w))
+        atomicAdd(CL ? gdata + (size_t)o * g.channel + c : gdata + (size_t)c * g.prod_shape + o, w * go);
     }
   }
 }
 
-// grad coord, ND.cu:267-287 + the caller's sum over channels: one wave per point.
+// one wave per point, lanes over channels, shuffle reduction
 template <typename T>
 __global__ __launch_bounds__(kBlock) void nd_grad_coord_kernel(NdGeo g, const T* __restrict__ gout,
                                                                const T* __restrict__ data,
@@ -143,7 +156,7 @@ __global__ __launch_bounds__(kBlock) void nd_grad_coord_kernel(NdGeo g, const T*
         const CT go = ld(gout + b * g.channel + c);
         const T* dc = data + (size_t)c * g.prod_shape;
         for (unsigned i = 0; i < (1u << g.dims); ++i) {
-          // the corner exists for every gdim or for none: its range tests do not depend on gdim
+          // a corner exists for every differentiated dimension or for none
           long o;
           CT w;
           if (!corner<CT>(g, p, i, -1, o, w)) continue;
@@ -167,6 +180,185 @@ __global__ __launch_bounds__(kBlock) void nd_grad_coord_kernel(NdGeo g, const T*
         for (int sft = 32; sft > 0; sft >>= 1) v += __shfl_xor(v, sft, 64);
         if (lane == 0) st(gcoord + b * g.dims + d, v);
       }
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------
+// channel-last path
+// ---------------------------------------------------------------------------
+
+// in [rows][cols] -> out [cols][rows], converting A -> B; 32 x 32 tiles through LDS
+template <typename A, typename B>
+__global__ __launch_bounds__(256) void nd_transpose_kernel(const A* __restrict__ in, B* __restrict__ out,
+                                                           long rows, long cols) {
+  __shared__ float tile[32][33];
+  const long r0 = (long)blockIdx.y * 32, c0 = (long)blockIdx.x * 32;
+  const int tx = threadIdx.x & 31, ty = threadIdx.x >> 5;
+#pragma unroll
+  for (int k = 0; k < 32; k += 8) {
+    const long r = r0 + ty + k, c = c0 + tx;
+    tile[ty + k][tx] = (r < rows && c < cols) ? static_cast<float>(ld(in + r * cols + c)) : 0.f;
+  }
+  __syncthreads();
+#pragma unroll
+  for (int k = 0; k < 32; k += 8) {
+    const long c = c0 + ty + k, r = r0 + tx;
+    if (r < rows && c < cols) st(out + c * rows + r, tile[tx][ty + k]);
+  }
+}
+
+// Corner offsets (in units of C elements of the channel-last copy) and weights of one
+// point, padded to kClCorners; absent corners get weight 0 at offset 0.
+struct ClCorners {
+  int off[kClCorners];
+  float w[kClCorners];
+};
+
+template <typename T>
+__device__ __forceinline__ ClCorners cl_corners(const NdGeo& g, const T* coord, long b, bool valid) {
+  ClCorners cc;
+  NdPoint<float> p;
+  p.inside = false;
+  if (valid) p = load_point<T, float>(g, coord + b * g.dims);
+#pragma unroll
+  for (int i = 0; i < kClCorners; ++i) {
+    long o = 0;
+    float w = 0.f;
+    const bool ok = valid && p.inside && i < (1 << g.dims) && corner<float>(g, p, (unsigned)i, -1, o, w);
+    cc.off[i] = ok ? (int)o : 0;
+    cc.w[i] = ok ? w : 0.f;
+  }
+  return cc;
+}
+
+// forward: a wave owns `ppw` (a power of two <= 64) consecutive points and walks them four at a
+// time so that the corner reads of four points are in flight together
+template <typename T>
+__global__ __launch_bounds__(kBlock) void nd_forward_cl_kernel(NdGeo g, const T* __restrict__ data_cl,
+                                                               const T* __restrict__ coord,
+                                                               T* __restrict__ out, int ppw) {
+  const int lane = threadIdx.x & 63;
+  const long wave0 = ((long)blockIdx.x * (kBlock / 64) + (threadIdx.x >> 6)) * ppw;
+  if (wave0 >= g.batch) return;
+  const int npts = (int)min((long)ppw, g.batch - wave0);
+  const ClCorners mine = cl_corners<T>(g, coord, wave0 + lane, lane < npts);
+  const int ncorner = 1 << g.dims;
+  constexpr int PU = 4;
+  for (int q0 = 0; q0 < npts; q0 += PU) {
+    int off[PU][kClCorners];
+    float w[PU][kClCorners];
+#pragma unroll
+    for (int u = 0; u < PU; ++u) {
+      const int q = min(q0 + u, npts - 1);
+#pragma unroll
+      for (int i = 0; i < kClCorners; ++i) {
+        off[u][i] = __builtin_amdgcn_readlane(mine.off[i], q);
+        w[u][i] = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, mine.w[i]), q));
+      }
+    }
+    for (int c = lane; c < g.channel; c += 64) {
+      float v[PU][kClCorners];
+#pragma unroll
+      for (int u = 0; u < PU; ++u)
+#pragma unroll
+        for (int i = 0; i < kClCorners; ++i)
+          v[u][i] = i < ncorner ? ld(data_cl + (size_t)off[u][i] * g.channel + c) : 0.f;
+#pragma unroll
+      for (int u = 0; u < PU; ++u) {
+        float acc = 0.f;
+#pragma unroll
+        for (int i = 0; i < kClCorners; ++i) acc += w[u][i] * v[u][i];
+        if (q0 + u < npts) st(out + (wave0 + q0 + u) * g.channel + c, acc);
+      }
+    }
+  }
+}
+
+// grad coord: same walk; per point the lanes' partial gradients are reduced by shuffles
+template <typename T>
+__global__ __launch_bounds__(kBlock) void nd_grad_coord_cl_kernel(NdGeo g, const T* __restrict__ gout,
+                                                                  const T* __restrict__ data_cl,
+                                                                  const T* __restrict__ coord,
+                                                                  T* __restrict__ gcoord, int ppw) {
+  const int lane = threadIdx.x & 63;
+  const long wave0 = ((long)blockIdx.x * (kBlock / 64) + (threadIdx.x >> 6)) * ppw;
+  if (wave0 >= g.batch) return;
+  const int npts = (int)min((long)ppw, g.batch - wave0);
+  const bool valid = lane < npts;
+  const ClCorners mine = cl_corners<T>(g, coord, wave0 + lane, valid);
+  const int ncorner = 1 << g.dims;
+  // s[i] of point q lands in lane q: sum over channels of gout * data at corner i
+  float s[kClCorners];
+#pragma unroll
+  for (int i = 0; i < kClCorners; ++i) s[i] = 0.f;
+  for (int q = 0; q < npts; ++q) {
+    int off[kClCorners];
+#pragma unroll
+    for (int i = 0; i < kClCorners; ++i) off[i] = __builtin_amdgcn_readlane(mine.off[i], q);
+    float part[kClCorners];
+#pragma unroll
+    for (int i = 0; i < kClCorners; ++i) part[i] = 0.f;
+    const T* grow = gout + (wave0 + q) * g.channel;
+    for (int c = lane; c < g.channel; c += 64) {
+      const float go = ld(grow + c);
+#pragma unroll
+      for (int i = 0; i < kClCorners; ++i)
+        if (i < ncorner) part[i] += go * ld(data_cl + (size_t)off[i] * g.channel + c);
+    }
+#pragma unroll
+    for (int i = 0; i < kClCorners; ++i) {
+      if (i < ncorner) {
+        const float v = wave_sum(part[i]);
+        if (lane == q) s[i] = v;
+      }
+    }
+  }
+  if (!valid) return;
+  // lane <-> point again: apply the derivative weights (ND.cu:161,165) to the corner sums
+  const NdPoint<float> p = load_point<T, float>(g, coord + (wave0 + lane) * g.dims);
+#pragma unroll
+  for (int d = 0; d < kClMaxDims; ++d) {
+    if (d < g.dims) {
+      float gd = 0.f;
+      if (p.inside) {
+#pragma unroll
+        for (int i = 0; i < kClCorners; ++i) {
+          long o;
+          float w;
+          if (i < ncorner && corner<float>(g, p, (unsigned)i, d, o, w)) gd += s[i] * w;
+        }
+      }
+      st(gcoord + (wave0 + lane) * g.dims + d, gd);
+    }
+  }
+}
+
+// grad data: scatter into the zeroed channel-last fp32 image; one 64-channel run per atomic
+template <typename T>
+__global__ __launch_bounds__(kBlock) void nd_grad_data_cl_kernel(NdGeo g, const T* __restrict__ gout,
+                                                                 const T* __restrict__ coord,
+                                                                 float* __restrict__ gdata_cl, int ppw) {
+  const int lane = threadIdx.x & 63;
+  const long wave0 = ((long)blockIdx.x * (kBlock / 64) + (threadIdx.x >> 6)) * ppw;
+  if (wave0 >= g.batch) return;
+  const int npts = (int)min((long)ppw, g.batch - wave0);
+  const ClCorners mine = cl_corners<T>(g, coord, wave0 + lane, lane < npts);
+  const int ncorner = 1 << g.dims;
+  for (int q = 0; q < npts; ++q) {
+    int off[kClCorners];
+    float w[kClCorners];
+#pragma unroll
+    for (int i = 0; i < kClCorners; ++i) {
+      off[i] = __builtin_amdgcn_readlane(mine.off[i], q);
+      w[i] = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, mine.w[i]), q));
+    }
+    const T* grow = gout + (wave0 + q) * g.channel;
+    for (int c = lane; c < g.channel; c += 64) {
+      const float go = ld(grow + c);
+#pragma unroll
+      for (int i = 0; i < kClCorners; ++i)
+        if (i < ncorner && w[i] != 0.f) atomicAdd(gdata_cl + (size_t)off[i] * g.channel + c, w[i] * go);
     }
   }
 }
@@ -202,20 +394,64 @@ NdGeo make_geo(const dk_nd_desc& d) {
   return g;
 }
 
+size_t elem_size(int dtype) { return dtype == DK_F64 ? 8 : dtype == DK_F32 ? 4 : 2; }
+
+// points per wave of the channel-last kernels: as many as keep at least ~8192 waves in the grid
+int points_per_wave(const NdGeo& g) {
+  int ppw = 64;
+  while (ppw > 1 && g.batch / ppw < 8192) ppw >>= 1;
+  return ppw;
+}
+
+template <typename A, typename B>
+void transpose(const A* in, B* out, long rows, long cols, hipStream_t stream) {
+  const dim3 grid((unsigned)((cols + 31) / 32), (unsigned)((rows + 31) / 32));
+  nd_transpose_kernel<A, B><<<grid, 256, 0, stream>>>(in, out, rows, cols);
+}
+
 }  // namespace
 
+// The channel-last path pays for a transpose of `data`; it is taken for 1..3 dimensions in
+// fp32 / fp16 / bf16 when there are enough (point, channel) pairs to amortise it.
+bool nd_use_channel_last(const dk_nd_desc& d) {
+  if (d.dtype == DK_F64 || d.dims > kClMaxDims) return false;
+  long prod = 1;
+  for (int i = 0; i < d.dims; ++i) prod *= d.shape[i];
+  if (prod > 2147483647L / 4) return false;  // corner offsets are kept as 32-bit element counts
+  return d.batch * d.channel >= 65536 && d.channel >= 16;
+}
+
+size_t nd_data_cl_workspace(const dk_nd_desc& d) {
+  if (!nd_use_channel_last(d)) return 0;
+  size_t n = (size_t)d.channel;
+  for (int i = 0; i < d.dims; ++i) n *= (size_t)d.shape[i];
+  return n * elem_size(d.dtype);
+}
+
 template <typename T>
-void nd_forward(const dk_nd_desc& d, const T* data, const T* coord, T* out, hipStream_t stream) {
+void nd_forward(const dk_nd_desc& d, const T* data, const T* coord, T* out, void* ws,
+                hipStream_t stream) {
   const NdGeo g = make_geo(d);
+  if constexpr (!std::is_same<T, double>::value) {
+    if (nd_use_channel_last(d)) {
+      T* data_cl = static_cast<T*>(ws);
+      transpose<T, T>(data, data_cl, g.channel, g.prod_shape, stream);
+      const int ppw = points_per_wave(g);
+      const long waves = (g.batch + ppw - 1) / ppw;
+      nd_forward_cl_kernel<T><<<(unsigned)((waves + 3) / 4), kBlock, 0, stream>>>(g, data_cl, coord, out, ppw);
+      return;
+    }
+  }
   const long total = g.batch * g.channel;
   nd_forward_kernel<T><<<grid_for(total), kBlock, 0, stream>>>(g, data, coord, out, total);
 }
 
 size_t nd_grad_data_workspace(const dk_nd_desc& d) {
-  if (d.dtype != DK_F16 && d.dtype != DK_BF16) return 0;
   size_t n = (size_t)d.channel;
   for (int i = 0; i < d.dims; ++i) n *= (size_t)d.shape[i];
-  return n * sizeof(float);
+  if (nd_use_channel_last(d)) return n * sizeof(float);  // fp32 channel-last accumulation image
+  if (d.dtype == DK_F16 || d.dtype == DK_BF16) return n * sizeof(float);
+  return 0;
 }
 
 template <typename T>
@@ -225,27 +461,48 @@ void nd_grad_data(const dk_nd_desc& d, const T* gout, const T* coord, T* gdata, 
   const NdGeo g = make_geo(d);
   const long n_data = (long)g.channel * g.prod_shape;
   const long total = g.batch * g.channel;
+  if constexpr (!std::is_same<T, double>::value) {
+    if (nd_use_channel_last(d)) {
+      float* acc = static_cast<float*>(ws);
+      nd_fill_zero_kernel<float><<<grid_for(n_data), kBlock, 0, stream>>>(acc, n_data);
+      const int ppw = points_per_wave(g);
+      const long waves = (g.batch + ppw - 1) / ppw;
+      nd_grad_data_cl_kernel<T><<<(unsigned)((waves + 3) / 4), kBlock, 0, stream>>>(g, gout, coord, acc, ppw);
+      transpose<float, T>(acc, gdata, g.prod_shape, g.channel, stream);
+      return;
+    }
+  }
   constexpr bool direct = sizeof(T) == sizeof(CT);
   CT* acc = direct ? reinterpret_cast<CT*>(gdata) : static_cast<CT*>(ws);
   nd_fill_zero_kernel<CT><<<grid_for(n_data), kBlock, 0, stream>>>(acc, n_data);
   if (total > 0)
-    nd_grad_data_kernel<T, CT><<<grid_for(total), kBlock, 0, stream>>>(g, gout, coord, acc, total);
+    nd_grad_data_kernel<T, CT, false><<<grid_for(total), kBlock, 0, stream>>>(g, gout, coord, acc, total);
   if (!direct) nd_convert_kernel<CT, T><<<grid_for(n_data), kBlock, 0, stream>>>(acc, gdata, n_data);
 }
 
 template <typename T>
 void nd_grad_coord(const dk_nd_desc& d, const T* gout, const T* data, const T* coord, T* gcoord,
-                   hipStream_t stream) {
+                   void* ws, hipStream_t stream) {
   const NdGeo g = make_geo(d);
+  if constexpr (!std::is_same<T, double>::value) {
+    if (nd_use_channel_last(d)) {
+      T* data_cl = static_cast<T*>(ws);
+      transpose<T, T>(data, data_cl, g.channel, g.prod_shape, stream);
+      const int ppw = points_per_wave(g);
+      const long waves = (g.batch + ppw - 1) / ppw;
+      nd_grad_coord_cl_kernel<T><<<(unsigned)((waves + 3) / 4), kBlock, 0, stream>>>(g, gout, data_cl, coord, gcoord, ppw);
+      return;
+    }
+  }
   long blocks = (g.batch + 3) / 4;
   if (blocks > 65536) blocks = 65536;
   nd_grad_coord_kernel<T><<<(int)blocks, kBlock, 0, stream>>>(g, gout, data, coord, gcoord);
 }
 
-#define DK_INSTANTIATE(T)                                                                      \
-  template void nd_forward<T>(const dk_nd_desc&, const T*, const T*, T*, hipStream_t);          \
-  template void nd_grad_data<T>(const dk_nd_desc&, const T*, const T*, T*, void*, hipStream_t); \
-  template void nd_grad_coord<T>(const dk_nd_desc&, const T*, const T*, const T*, T*, hipStream_t);
+#define DK_INSTANTIATE(T)                                                                             \
+  template void nd_forward<T>(const dk_nd_desc&, const T*, const T*, T*, void*, hipStream_t);          \
+  template void nd_grad_data<T>(const dk_nd_desc&, const T*, const T*, T*, void*, hipStream_t);        \
+  template void nd_grad_coord<T>(const dk_nd_desc&, const T*, const T*, const T*, T*, void*, hipStream_t);
 DK_INSTANTIATE(float)
 DK_INSTANTIATE(double)
 DK_INSTANTIATE(__half)

@@ -27,10 +27,12 @@ class NdLinearSampleFunction(Function):
         ctx.save_for_backward(input, coord)
         output = input.new_empty(NdLinearSampleFunction._output_size(input, coord))
         desc = _lib.nd_desc(input, coord)
+        L = _lib.lib()
         with torch.cuda.device(input.device):
-            _lib.check(_lib.lib().dk_nd_linear_sample_forward(
-                desc, _lib.ptr(input), _lib.ptr(coord), _lib.ptr(output), _lib.stream_ptr(input)),
-                "nd_linear_sample forward")
+            ws, nbytes = _lib.workspace(L.dk_nd_linear_sample_forward_workspace(desc), input.device)
+            _lib.check(L.dk_nd_linear_sample_forward(
+                desc, _lib.ptr(input), _lib.ptr(coord), _lib.ptr(output), _lib.ptr(ws), nbytes,
+                _lib.stream_ptr(input)), "nd_linear_sample forward")
         return output
 
     @staticmethod
@@ -51,9 +53,10 @@ class NdLinearSampleFunction(Function):
                     _lib.ptr(ws), nbytes, s), "nd_linear_sample backward_data")
             if ctx.needs_input_grad[1]:
                 grad_coord = torch.zeros_like(coord)
+                ws, nbytes = _lib.workspace(L.dk_nd_linear_sample_backward_coord_workspace(desc), input.device)
                 _lib.check(L.dk_nd_linear_sample_backward_coord(
                     desc, _lib.ptr(grad_output), _lib.ptr(input), _lib.ptr(coord),
-                    _lib.ptr(grad_coord), s), "nd_linear_sample backward_coord")
+                    _lib.ptr(grad_coord), _lib.ptr(ws), nbytes, s), "nd_linear_sample backward_coord")
         return (grad_input, grad_coord)
 
     @staticmethod

@@ -153,13 +153,19 @@ typedef struct dk_nd_desc {
   int32_t dtype;
 } dk_nd_desc;
 
-/* nd_linear_sample_forward_cuda (nd_linear_sample_cuda.cpp:10-26). */
+/* nd_linear_sample_forward_cuda (nd_linear_sample_cuda.cpp:10-26).  For large problems the
+ * library samples from a channel-last copy of `data` that it writes into the workspace (so
+ * the channels of one corner are one contiguous read); the query returns 0 when the direct
+ * path is used. */
+size_t dk_nd_linear_sample_forward_workspace(const dk_nd_desc *desc);
 int dk_nd_linear_sample_forward(const dk_nd_desc *desc, const void *data, const void *coord,
-                                void *output, void *stream);
+                                void *output, void *workspace, size_t workspace_bytes,
+                                void *stream);
 
 /* nd_linear_sample_backward_data_cuda (nd_linear_sample_cuda.cpp:29-45); in_grad is
- * fully written (the reference zero-fills it in C++ and scatters atomically).  fp16 / bf16
- * gradients are accumulated in an fp32 workspace of the data's element count. */
+ * fully written (the reference zero-fills it in C++ and scatters atomically).  The workspace
+ * holds an fp32 accumulation image of the data's element count when one is needed (fp16 / bf16
+ * gradients, and the channel-last path for large problems). */
 size_t dk_nd_linear_sample_backward_data_workspace(const dk_nd_desc *desc);
 int dk_nd_linear_sample_backward_data(const dk_nd_desc *desc, const void *out_grad,
                                       const void *coord, void *in_grad, void *workspace,
@@ -168,9 +174,10 @@ int dk_nd_linear_sample_backward_data(const dk_nd_desc *desc, const void *out_gr
 /* nd_linear_sample_backward_coord_cuda (nd_linear_sample_cuda.cpp:47-64) fused with the
  * `.sum(2)` its Python caller applies (functions/nd_linear_sample.py:48-55):
  * coord_grad is [batch, dims], already summed over channels. */
+size_t dk_nd_linear_sample_backward_coord_workspace(const dk_nd_desc *desc);
 int dk_nd_linear_sample_backward_coord(const dk_nd_desc *desc, const void *out_grad,
                                        const void *data, const void *coord, void *coord_grad,
-                                       void *stream);
+                                       void *workspace, size_t workspace_bytes, void *stream);
 
 /* ---- misc ------------------------------------------------------------------- */
 

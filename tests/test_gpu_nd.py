@@ -38,7 +38,8 @@ def _oracle(data, coord, gout, np_dtype):
 
 
 @pytest.mark.parametrize("shape,C,B", [((9,), 5, 70), ((5, 5), 256, 1152), ((4, 5, 6), 7, 333),
-                                       ((3, 4, 2, 5), 3, 200), ((2, 2), 1, 1)])
+                                       ((3, 4, 2, 5), 3, 200), ((2, 2), 1, 1),
+                                       ((9,), 40, 3000), ((6, 7, 5), 100, 1001), ((5, 4), 16, 4097)])
 def test_fp32_matches_oracle(shape, C, B):
     data, coord, gout = _inputs(shape, C, B, seed=41, dtype=torch.float32)
     got = _run(data, coord, gout)
@@ -57,9 +58,10 @@ def test_fp64_matches_oracle():
         assert rel_err(g, w) < 1e-11
 
 
+@pytest.mark.parametrize("points", [300, 4096])   # direct path / channel-last path
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
-def test_half_precisions_match_fp32_oracle(dtype):
-    data, coord, gout = _inputs((5, 5), 64, 300, seed=43, dtype=dtype)
+def test_half_precisions_match_fp32_oracle(dtype, points):
+    data, coord, gout = _inputs((5, 5), 64, points, seed=43, dtype=dtype)
     got = _run(data, coord, gout)
     want = _oracle(data, coord, gout, np.float32)
     for g, w in zip(got, want):
