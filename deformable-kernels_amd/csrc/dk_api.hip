@@ -184,6 +184,33 @@ int dk_sample_depthwise_backward_rotation(const dk_conv_desc* desc, const void* 
   });
 }
 
+size_t dk_sample_depthwise_backward_workspace(const dk_conv_desc* desc) {
+  return dk_sample_depthwise_backward_filter_workspace(desc);
+}
+
+int dk_sample_depthwise_backward(const dk_conv_desc* desc, const void* out_grad, const void* input,
+                                 const void* rotation, const void* filter, void* in_grad,
+                                 void* rotation_grad, void* filter_grad, void* workspace,
+                                 size_t workspace_bytes, void* stream) {
+  Geo g;
+  const int rc = make_geo(desc, g);
+  if (rc != DK_OK) return rc;
+  if (!out_grad || !input || !rotation || !filter) return DK_ERR_NULL_POINTER;
+  if (filter_grad) {
+    const size_t need = local_filter_ws(g, desc->dtype);
+    if (need && (!workspace || workspace_bytes < need)) return DK_ERR_WORKSPACE;
+  }
+  int st = DK_OK;
+  if (in_grad && st == DK_OK)
+    st = dk_sample_depthwise_backward_data(desc, out_grad, rotation, filter, in_grad, stream);
+  if (rotation_grad && st == DK_OK)
+    st = dk_sample_depthwise_backward_rotation(desc, out_grad, input, rotation, filter, rotation_grad, stream);
+  if (filter_grad && st == DK_OK)
+    st = dk_sample_depthwise_backward_filter(desc, out_grad, input, rotation, filter_grad, workspace,
+                                             workspace_bytes, stream);
+  return st;
+}
+
 // ---- deformable --------------------------------------------------------------------------
 
 int dk_deformable_sample_depthwise_forward(const dk_conv_desc* desc, const void* input,

@@ -100,22 +100,20 @@ class SampleDepthwiseFunction(Function):
         L = _lib.lib()
         with torch.cuda.device(input.device):
             s = _lib.stream_ptr(input)
+            # one native call for the whole backward pass: the gradients that are not needed
+            # are passed as NULL and skipped (the reference issues one call per gradient)
             if ctx.needs_input_grad[0]:
                 grad_input = torch.empty_like(input)
-                _lib.check(L.dk_sample_depthwise_backward_data(
-                    desc, _lib.ptr(grad_output), _lib.ptr(rotation), _lib.ptr(weight),
-                    _lib.ptr(grad_input), s), "sample_depthwise backward_data")
             if ctx.needs_input_grad[1]:
                 grad_rotation = torch.empty_like(rotation)
-                _lib.check(L.dk_sample_depthwise_backward_rotation(
-                    desc, _lib.ptr(grad_output), _lib.ptr(input), _lib.ptr(rotation), _lib.ptr(weight),
-                    _lib.ptr(grad_rotation), s), "sample_depthwise backward_rotation")
+            ws, nbytes = None, 0
             if ctx.needs_input_grad[2]:
                 grad_weight = torch.empty_like(weight)
-                ws, nbytes = _lib.workspace(L.dk_sample_depthwise_backward_filter_workspace(desc), input.device)
-                _lib.check(L.dk_sample_depthwise_backward_filter(
-                    desc, _lib.ptr(grad_output), _lib.ptr(input), _lib.ptr(rotation),
-                    _lib.ptr(grad_weight), _lib.ptr(ws), nbytes, s), "sample_depthwise backward_filter")
+                ws, nbytes = _lib.workspace(L.dk_sample_depthwise_backward_workspace(desc), input.device)
+            _lib.check(L.dk_sample_depthwise_backward(
+                desc, _lib.ptr(grad_output), _lib.ptr(input), _lib.ptr(rotation), _lib.ptr(weight),
+                _lib.ptr(grad_input), _lib.ptr(grad_rotation), _lib.ptr(grad_weight),
+                _lib.ptr(ws), nbytes, s), "sample_depthwise backward")
         return (grad_input, grad_rotation, grad_weight,) + (None,) * 5
 
 

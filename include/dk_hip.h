@@ -103,6 +103,17 @@ int dk_sample_depthwise_backward_rotation(const dk_conv_desc *desc, const void *
                                           const void *input, const void *rotation,
                                           const void *filter, void *rotation_grad, void *stream);
 
+/* The three gradients of one backward pass in one call; any of in_grad / rotation_grad /
+ * filter_grad may be NULL to skip it.  Stands in for the three consecutive pybind calls of
+ * SampleDepthwiseFunction.backward (functions/filter_sample_depthwise.py:63-85): one call that
+ * issues the launches of the three entry points above on `stream`.  Workspace as for
+ * *_backward_filter (only needed when filter_grad is requested). */
+size_t dk_sample_depthwise_backward_workspace(const dk_conv_desc *desc);
+int dk_sample_depthwise_backward(const dk_conv_desc *desc, const void *out_grad, const void *input,
+                                 const void *rotation, const void *filter, void *in_grad,
+                                 void *rotation_grad, void *filter_grad, void *workspace,
+                                 size_t workspace_bytes, void *stream);
+
 /* ---- deformable kernel with image-space offsets ---------------------------- */
 
 /* deformable_sample_depthwise_forward_cuda (filter_sample_depthwise_cuda.cpp:237-294). */
