@@ -134,6 +134,13 @@ def main():
         k_forward()
         k_backward()  # grad input + grad rotation + grad filter, one native call
 
+    # A plain streaming kernel of known size (|x| read, |x| written): the calibration kernel for
+    # the FETCH_SIZE / WRITE_SIZE counters when this script runs under rocprofv3 --pmc.  (An
+    # elementwise multiply rather than copy_(), which the runtime turns into its own blit.)
+    calib = torch.empty_like(xg)
+    torch.mul(xg, 1.0, out=calib)
+    del calib
+
     for _ in range(a.warmup):
         step()
     torch.cuda.synchronize()

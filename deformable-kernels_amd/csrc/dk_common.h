@@ -144,6 +144,23 @@ __device__ __forceinline__ ImageTap<CT> make_image_tap(CT h, CT w, int H, int W)
 
 __host__ __device__ __forceinline__ int ceil_div(int a, int b) { return (a + b - 1) / b; }
 
+// ---------------------------------------------------------------------------
+// XCD-aware block order.  MI355X has 8 XCDs with one L2 each, and the dispatcher hands
+// consecutive workgroups of a grid to consecutive XCDs (block b runs on XCD b % 8).  Work items
+// that share data (the tiles of one image, the channel splits of one tile) should therefore not
+// be consecutive blocks but blocks congruent mod 8.  Grids are launched 1-D with
+// xcd_grid_size(total) blocks; logical_block() gives block b the logical index
+//   (b % 8) * ceil(total / 8) + b / 8,
+// so each XCD walks one contiguous eighth of the logical order.  Indices >= total (at most 7)
+// are padding and must exit.
+// ---------------------------------------------------------------------------
+constexpr int kXcds = 8;
+__host__ __device__ __forceinline__ long xcd_grid_size(long total) { return (total + kXcds - 1) / kXcds * kXcds; }
+__device__ __forceinline__ long logical_block(long total) {
+  const long chunk = (total + kXcds - 1) / kXcds;
+  return (long)(blockIdx.x % kXcds) * chunk + blockIdx.x / kXcds;
+}
+
 // Sum of v over the 64 lanes of the wave, returned in every lane: six DPP adds and one readlane
 // (no LDS crossbar traffic, unlike a shuffle-based butterfly).
 __device__ __forceinline__ float wave_sum(float v) {

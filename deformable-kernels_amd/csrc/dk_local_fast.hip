@@ -149,17 +149,23 @@ __global__ __launch_bounds__(kBlock, 2) void local_gather_kernel(Geo g, const T*
   constexpr int K = KH * KW;
   extern __shared__ __align__(16) float tbl[];
 
-  const int n = blockIdx.z / g.groups, grp = blockIdx.z % g.groups;
   const int cpg = g.channel / g.groups;  // channels per rotation group
-  const int j0 = blockIdx.y * ch_per_block;
-  const int nch = min(ch_per_block, cpg - j0);
-  stage_wide_tables<T, SH, SW>(tbl, filter, grp + g.groups * j0, g.groups, nch);
-
   const int out_plane = g.out_h * g.out_w, in_plane = g.in_h * g.in_w;
   const int dst_plane = TRANSPOSED ? in_plane : out_plane;
   const int src_plane = TRANSPOSED ? out_plane : in_plane;
   const int dst_w = TRANSPOSED ? g.in_w : g.out_w;
-  const int p = blockIdx.x * kBlock + threadIdx.x;
+  // logical block = (tile, channel split, image * group), tile fastest: one XCD gets whole images
+  const int tiles = ceil_div(dst_plane, kBlock), splits = ceil_div(cpg, ch_per_block);
+  const long total = (long)tiles * splits * g.batch * g.groups;
+  const long lb = logical_block(total);
+  if (lb >= total) return;
+  const int bx = (int)(lb % tiles), by = (int)(lb / tiles % splits), bz = (int)(lb / tiles / splits);
+  const int n = bz / g.groups, grp = bz % g.groups;
+  const int j0 = by * ch_per_block;
+  const int nch = min(ch_per_block, cpg - j0);
+  stage_wide_tables<T, SH, SW>(tbl, filter, grp + g.groups * j0, g.groups, nch);
+
+  const int p = bx * kBlock + threadIdx.x;
   const bool active = p < dst_plane;
   const int pc = active ? p : 0;
   const int ph = pc / dst_w, pw = pc % dst_w;
@@ -252,18 +258,24 @@ __global__ __launch_bounds__(kBlock, 2) void local_gather_rows_kernel(Geo g, con
   constexpr int KW = 3, K = KH * KW;
   extern __shared__ __align__(16) float tbl[];
 
-  const int n = blockIdx.z / g.groups, grp = blockIdx.z % g.groups;
   const int cpg = g.channel / g.groups;
-  const int j0 = blockIdx.y * ch_per_block;
-  const int nch = min(ch_per_block, cpg - j0);
-  stage_wide_tables<T, SH, SW>(tbl, filter, grp + g.groups * j0, g.groups, nch);
-
   const int W = g.in_w;  // == out_w
   const int out_plane = g.out_h * W, in_plane = g.in_h * W;
   const int dst_plane = TRANSPOSED ? in_plane : out_plane;
   const int src_plane = TRANSPOSED ? out_plane : in_plane;
+  // logical block = (tile, channel split, image * group), tile fastest: one XCD gets whole images
+  const int tiles = ceil_div(dst_plane, kRowPix), splits = ceil_div(cpg, ch_per_block);
+  const long total = (long)tiles * splits * g.batch * g.groups;
+  const long lb = logical_block(total);
+  if (lb >= total) return;
+  const int bx = (int)(lb % tiles), by = (int)(lb / tiles % splits), bz = (int)(lb / tiles / splits);
+  const int n = bz / g.groups, grp = bz % g.groups;
+  const int j0 = by * ch_per_block;
+  const int nch = min(ch_per_block, cpg - j0);
+  stage_wide_tables<T, SH, SW>(tbl, filter, grp + g.groups * j0, g.groups, nch);
+
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int p = blockIdx.x * kRowPix + wave * kRowLanes + lane - 1;  // lanes 0 and 63 are halo
+  const int p = bx * kRowPix + wave * kRowLanes + lane - 1;  // lanes 0 and 63 are halo
   const bool owns = lane >= 1 && lane <= kRowLanes && p < dst_plane;  // p >= 0 whenever lane >= 1
   const int pc = owns ? p : 0;
   const int ph = pc / W, pw = pc % W;
@@ -365,11 +377,17 @@ __global__ __launch_bounds__(kBlock, 2) void local_grad_rotation_kernel(
   constexpr int NLOAD = ROWS ? KH : K;  // input loads per channel
   extern __shared__ __align__(16) float tbl[];
 
-  const int n = blockIdx.z / g.groups, grp = blockIdx.z % g.groups;
   const int cpg = g.channel / g.groups;
   const int out_plane = g.out_h * g.out_w, in_plane = g.in_h * g.in_w;
+  // logical block = (tile, image * group), tile fastest
+  const int tiles = ceil_div(out_plane, ROWS ? kRowPix : kBlock);
+  const long total = (long)tiles * g.batch * g.groups;
+  const long lb = logical_block(total);
+  if (lb >= total) return;
+  const int bx = (int)(lb % tiles), bz = (int)(lb / tiles);
+  const int n = bz / g.groups, grp = bz % g.groups;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int p = ROWS ? blockIdx.x * kRowPix + wave * kRowLanes + lane - 1 : blockIdx.x * kBlock + threadIdx.x;
+  const int p = ROWS ? bx * kRowPix + wave * kRowLanes + lane - 1 : bx * kBlock + threadIdx.x;
   const bool owns = (ROWS ? (lane >= 1 && lane <= kRowLanes) : true) && p < out_plane;
   const int pc = owns ? p : 0;
   const int ph = pc / g.out_w, pw = pc % g.out_w;
@@ -490,7 +508,7 @@ __global__ __launch_bounds__(kBlock, 2) void local_grad_rotation_kernel(
 template <typename T, int KH, int KW, int SH, int SW, bool ROWS>
 __global__ __launch_bounds__(kBlock, 2) void local_grad_filter_kernel(
     Geo g, const T* __restrict__ gout, const T* __restrict__ x, const T* __restrict__ rot,
-    float* __restrict__ partial, int tiles, int ch_per_block) {
+    float* __restrict__ partial, int tiles, int ch_per_block, int parts) {
   constexpr int K = KH * KW;
   constexpr int CELLS = SH * SW;
   constexpr int NLOAD = ROWS ? KH : K;
@@ -502,13 +520,20 @@ __global__ __launch_bounds__(kBlock, 2) void local_grad_filter_kernel(
   float* wacc = lds;                                  // [kWaves][ch_per_block][16]
   float* scratch = lds + kWaves * ch_per_block * 16;  // [kWaves][64][kPitch]
 
+  // logical block = (channel split, part, group), split fastest: the splits of one
+  // (image, tile) item and the items of one image share an XCD
+  const int cpg = g.channel / g.groups;
+  const int splits = ceil_div(cpg, ch_per_block);
+  const long total = (long)splits * parts * g.groups;
+  const long lb = logical_block(total);
+  if (lb >= total) return;
+  const int by = (int)(lb % splits), bx = (int)(lb / splits % parts), grp = (int)(lb / splits / parts);
+
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   for (int e = threadIdx.x; e < kWaves * ch_per_block * 16; e += kBlock) wacc[e] = 0.f;
   __syncthreads();
 
-  const int grp = blockIdx.z;
-  const int cpg = g.channel / g.groups;
-  const int j0 = blockIdx.y * ch_per_block;
+  const int j0 = by * ch_per_block;
   const int nch = min(ch_per_block, cpg - j0);
   const int out_plane = g.out_h * g.out_w, in_plane = g.in_h * g.in_w;
   const int items = g.batch * tiles;
@@ -518,7 +543,7 @@ __global__ __launch_bounds__(kBlock, 2) void local_grad_filter_kernel(
   // 16 lanes of its row, starting 4 * row lanes in so the four rows hit disjoint banks
   const int row = lane >> 4, m = lane & 15;
 
-  for (int item = blockIdx.x; item < items; item += gridDim.x) {
+  for (int item = bx; item < items; item += parts) {
     const int n = item / tiles, tile = item % tiles;
     const int p = ROWS ? tile * PIX + wave * kRowLanes + lane - 1 : tile * PIX + (int)threadIdx.x;
     const bool owns = (ROWS ? (lane >= 1 && lane <= kRowLanes) : true) && p < out_plane;
@@ -631,7 +656,7 @@ __global__ __launch_bounds__(kBlock, 2) void local_grad_filter_kernel(
 #pragma unroll
     for (int wv = 0; wv < kWaves; ++wv) s_ += wacc[(wv * ch_per_block + j) * 16 + r];
     const int c = grp + g.groups * (j0 + j);
-    partial[((size_t)blockIdx.x * g.channel + c) * CELLS + r] = s_;
+    partial[((size_t)bx * g.channel + c) * CELLS + r] = s_;
   }
 }
 
@@ -712,7 +737,7 @@ bool run_gather(const Geo& g, bool transposed, const T* src, const T* rot, const
   const int pixels = transposed ? g.in_h * g.in_w : g.out_h * g.out_w;
   if (same_width_geometry(g)) {
     const int per = channels_per_block<SH, SW>(cpg, pick_splits(g, pixels));
-    const dim3 grid(ceil_div(pixels, kRowPix), ceil_div(cpg, per), g.batch * g.groups);
+    const unsigned grid = (unsigned)xcd_grid_size((long)ceil_div(pixels, kRowPix) * ceil_div(cpg, per) * g.batch * g.groups);
     const size_t lds = (size_t)(per + 2 * kUnroll) * WideTable<SH, SW>::SIZE * sizeof(float);
     if (transposed)
       local_gather_rows_kernel<T, 3, SH, SW, true><<<grid, kBlock, lds, stream>>>(g, src, rot, filter, dst, per);
@@ -721,7 +746,7 @@ bool run_gather(const Geo& g, bool transposed, const T* src, const T* rot, const
     return true;
   }
   const int per = channels_per_block<SH, SW>(cpg, pick_splits(g, pixels));
-  const dim3 grid(ceil_div(pixels, kBlock), ceil_div(cpg, per), g.batch * g.groups);
+  const unsigned grid = (unsigned)xcd_grid_size((long)ceil_div(pixels, kBlock) * ceil_div(cpg, per) * g.batch * g.groups);
   // stages past the last channel still read (and discard) table entries: pad to whole stages
   const size_t lds = (size_t)(per + 2 * kUnroll) * WideTable<SH, SW>::SIZE * sizeof(float);
   if (transposed)
@@ -739,10 +764,10 @@ bool run_grad_rotation(const Geo& g, const T* gout, const T* x, const T* rot, co
   const int per = cpg < 36 ? cpg : 36;  // channels staged per pass
   const size_t lds = (size_t)per * Tb::SIZE * sizeof(float);
   if (same_width_geometry(g)) {
-    const dim3 grid(ceil_div(g.out_h * g.out_w, kRowPix), 1, g.batch * g.groups);
+    const unsigned grid = (unsigned)xcd_grid_size((long)ceil_div(g.out_h * g.out_w, kRowPix) * g.batch * g.groups);
     local_grad_rotation_kernel<T, 3, 3, SH, SW, true><<<grid, kBlock, lds, stream>>>(g, gout, x, rot, filter, grot, per);
   } else {
-    const dim3 grid(ceil_div(g.out_h * g.out_w, kBlock), 1, g.batch * g.groups);
+    const unsigned grid = (unsigned)xcd_grid_size((long)ceil_div(g.out_h * g.out_w, kBlock) * g.batch * g.groups);
     local_grad_rotation_kernel<T, 3, 3, SH, SW, false><<<grid, kBlock, lds, stream>>>(g, gout, x, rot, filter, grot, per);
   }
   return true;
@@ -777,12 +802,12 @@ bool run_grad_filter(const Geo& g, const T* gout, const T* x, const T* rot, T* g
     return false;
   } else {
     const FilterGrid f = filter_grid(g);
-    const dim3 grid(f.parts, f.splits, g.groups);
+    const unsigned grid = (unsigned)xcd_grid_size((long)f.parts * f.splits * g.groups);
     const size_t lds = ((size_t)(kBlock / 64) * f.per * 16 + (size_t)(kBlock / 64) * 64 * 20) * sizeof(float);
     if (same_width_geometry(g))
-      local_grad_filter_kernel<T, 3, 3, SH, SW, true><<<grid, kBlock, lds, stream>>>(g, gout, x, rot, ws, f.tiles, f.per);
+      local_grad_filter_kernel<T, 3, 3, SH, SW, true><<<grid, kBlock, lds, stream>>>(g, gout, x, rot, ws, f.tiles, f.per, f.parts);
     else
-      local_grad_filter_kernel<T, 3, 3, SH, SW, false><<<grid, kBlock, lds, stream>>>(g, gout, x, rot, ws, f.tiles, f.per);
+      local_grad_filter_kernel<T, 3, 3, SH, SW, false><<<grid, kBlock, lds, stream>>>(g, gout, x, rot, ws, f.tiles, f.per, f.parts);
     launch_reduce_partials<float, T>(ws, f.parts, g.channel * SH * SW, gfilter, stream);
     return true;
   }
@@ -790,7 +815,7 @@ bool run_grad_filter(const Geo& g, const T* gout, const T* x, const T* rot, T* g
 
 bool fast_shape(const Geo& g) {
   const long plane_limit = (1L << 31) / 4 / 32;  // byte offsets inside a plane (x 18 for rotation) stay below 2^31
-  return g.k_h == 3 && g.k_w == 3 && (long)g.batch * g.groups <= 65535 &&
+  return g.k_h == 3 && g.k_w == 3 && (long)g.batch * g.groups <= (1L << 20) &&
          (long)g.in_h * g.in_w < plane_limit && (long)g.out_h * g.out_w < plane_limit &&
          ((g.scope_h == 4 && g.scope_w == 4) || (g.scope_h == 3 && g.scope_w == 3) ||
           (g.scope_h == 5 && g.scope_w == 5));
