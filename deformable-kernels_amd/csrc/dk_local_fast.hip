@@ -30,8 +30,13 @@ struct Table {
   static constexpr int SIZE = (SH + 2) * RS;
 };
 
-// Corner-expanded scope table of one channel: one float4 {tl, tr, bl, br} per 2x2 block of the
+// Corner-expanded scope table of one channel: one float4 per 2x2 block {tl, tr, bl, br} of the
 // zero-padded tile, (SH + 1) x (SW + 1) blocks, so a tap needs a single 16-byte LDS read.
+// The float4 holds the block in difference form
+//   a = tl,  b = tr - tl,  c = bl - tl,  d = br - tr - bl + tl,
+// which turns the bilinear read at fractional position (lh, lw) into three fused multiply-adds,
+//   a + lw * b + lh * (c + lw * d),
+// with only (lh, lw) per tap in registers, and makes its derivatives c + lw * d and b + lh * d.
 //
 // gfx950 serves a ds_read_b128 at 256 B/clk from 64 banks, so two float4 blocks collide when
 // their block slots are congruent mod 16.  For the 5 x 5 blocks of a 4 x 4 scope the slots are
@@ -63,19 +68,81 @@ struct WideTable<4, 4> {
   }
 };
 
+// Stage the tables of channels c_first + j * c_step, j < nch.  A thread owns one block of the
+// tile for every (256 / 32)-th channel: which corners exist, their offsets in a channel's
+// filter and the destination slot are fixed per thread, so a channel costs four range-checked
+// loads (missing corners read 0), three subtractions and one 16-byte LDS write.
 template <typename T, int SH, int SW>
-__device__ __forceinline__ void stage_wide_tables(float* tbl, const T* filter, int c_first,
+__device__ __forceinline__ void stage_wide_tables(float* tbl, const T* filter, int channels, int c_first,
                                                   int c_step, int nch) {
   using Tb = WideTable<SH, SW>;
-  for (int e = threadIdx.x; e < nch * Tb::SIZE; e += blockDim.x) {
-    const int j = e / Tb::SIZE, r = e % Tb::SIZE;
-    const int blk = r / 4, corner = r % 4;
-    const int i = blk / Tb::RS - 1 + (corner >> 1), k = blk % Tb::RS - 1 + (corner & 1);
-    float v = 0.f;
-    if (i >= 0 && i < SH && k >= 0 && k < SW)
-      v = ld(filter + (size_t)(c_first + j * c_step) * (SH * SW) + i * SW + k);
-    tbl[j * Tb::SIZE + Tb::slot(blk) * 4 + corner] = v;
+  constexpr int CB = Tb::BLOCKS <= 32 ? 32 : 64;  // threads per channel
+  const int m = threadIdx.x % CB;
+  if (m >= Tb::BLOCKS) return;
+  const int i = m / Tb::RS - 1, k = m % Tb::RS - 1;
+  unsigned off[4];
+#pragma unroll
+  for (int q = 0; q < 4; ++q) {
+    const int ii = i + (q >> 1), kk = k + (q & 1);
+    off[q] = (ii >= 0 && ii < SH && kk >= 0 && kk < SW) ? (unsigned)(ii * SW + kk) * (unsigned)sizeof(T) : kOutOfRange;
   }
+  const rsrc_t rf = plane_rsrc(filter, channels * SH * SW);
+  float* dst = tbl + Tb::slot(m) * 4;
+  constexpr int CPP = kBlock / CB;  // channels per sweep of the workgroup
+  constexpr int kSweeps = 4;        // sweeps whose loads are issued together
+  for (int jb = threadIdx.x / CB; jb < nch; jb += kSweeps * CPP) {
+    float tl[kSweeps], tr[kSweeps], bl[kSweeps], br[kSweeps];
+#pragma unroll
+    for (int u = 0; u < kSweeps; ++u) {
+      const int j = jb + u * CPP;
+      const unsigned cb = j < nch ? (unsigned)(c_first + j * c_step) * (unsigned)(SH * SW * sizeof(T)) : kOutOfRange;
+      tl[u] = buf_ld(rf, off[0] + cb, filter);
+      tr[u] = buf_ld(rf, off[1] + cb, filter);
+      bl[u] = buf_ld(rf, off[2] + cb, filter);
+      br[u] = buf_ld(rf, off[3] + cb, filter);
+    }
+#pragma unroll
+    for (int u = 0; u < kSweeps; ++u) {
+      const int j = jb + u * CPP;
+      if (j < nch)
+        *reinterpret_cast<float4*>(dst + j * Tb::SIZE) =
+            make_float4(tl[u], tr[u] - tl[u], bl[u] - tl[u], (br[u] - tr[u]) - (bl[u] - tl[u]));
+    }
+  }
+}
+
+// One 16-byte LDS read for a caller that uses only some components: the empty asm counts as
+// a use of all four, so the compiler keeps the single wide read instead of two narrower ones
+// (two LDS issues).
+__device__ __forceinline__ float4 lds_read4(const float* p) {
+  const float4 q = *reinterpret_cast<const float4*>(p);
+  asm volatile("" ::"v"(q.x), "v"(q.y), "v"(q.z), "v"(q.w));
+  return q;
+}
+
+// (pixel, tap) descriptor for the difference-form table: the LDS float index of the tap's
+// block and the fractional position inside it.  A tap that contributes nothing (outside the
+// scope band, in the padding, or not owned) points at block (-1, -1) with lh = lw = 0, which
+// evaluates to that block's `a` entry: a padding zero.
+struct LiteTap {
+  int cell;
+  float lh, lw;
+};
+
+template <int SH, int SW>
+__device__ __forceinline__ LiteTap make_lite_tap(float h, float w, bool ok) {
+  using Tb = WideTable<SH, SW>;
+  const bool in = ok && (h > -1.f) && (w > -1.f) && (h < float(SH)) && (w < float(SW));
+  const float hf = floorf(h), wf = floorf(w);
+  LiteTap t;
+  t.lh = in ? h - hf : 0.f;
+  t.lw = in ? w - wf : 0.f;
+  t.cell = Tb::slot(in ? (static_cast<int>(hf) + 1) * Tb::RS + static_cast<int>(wf) + 1 : 0) * 4;
+  return t;
+}
+
+__device__ __forceinline__ float lite_weight(const LiteTap& t, const float4& q) {
+  return fmaf(t.lh, fmaf(t.lw, q.w, q.z), fmaf(t.lw, q.y, q.x));
 }
 
 template <typename T, int SH, int SW>
@@ -136,7 +203,7 @@ __device__ __forceinline__ bool tap_geometry(const Geo& g, int ph, int pw, int f
 //
 // Channels are walked kUnroll at a time: the 9 * kUnroll input loads of a block are
 // issued first (buffer loads, offsets fixed per lane), then each channel's 9 taps take
-// two ds_read2_b32 each at immediate offsets from one per-tap LDS address.
+// one ds_read_b128 each at an immediate offset from one per-tap LDS address.
 // ---------------------------------------------------------------------------
 constexpr int kUnroll = 2;
 
@@ -163,14 +230,14 @@ __global__ __launch_bounds__(kBlock, 2) void local_gather_kernel(Geo g, const T*
   const int n = bz / g.groups, grp = bz % g.groups;
   const int j0 = by * ch_per_block;
   const int nch = min(ch_per_block, cpg - j0);
-  stage_wide_tables<T, SH, SW>(tbl, filter, grp + g.groups * j0, g.groups, nch);
+  stage_wide_tables<T, SH, SW>(tbl, filter, g.channel, grp + g.groups * j0, g.groups, nch);
 
   const int p = bx * kBlock + threadIdx.x;
   const bool active = p < dst_plane;
   const int pc = active ? p : 0;
   const int ph = pc / dst_w, pw = pc % dst_w;
 
-  ScopeTap<float> tap[K];
+  LiteTap tap[K];
   unsigned soff[K];  // byte offset of the tap's source element in a source plane
   const rsrc_t rr = plane_rsrc(rot + (size_t)(n * g.groups + grp) * (K * 2) * out_plane, K * 2 * out_plane);
 #pragma unroll
@@ -182,9 +249,8 @@ __global__ __launch_bounds__(kBlock, 2) void local_gather_kernel(Geo g, const T*
     const unsigned ro = ok ? (unsigned)((2 * t) * out_plane + rpix) * (unsigned)sizeof(T) : kOutOfRange;
     const float r_h = buf_ld(rr, ro, rot);
     const float r_w = buf_ld(rr, ro + (unsigned)out_plane * (unsigned)sizeof(T), rot);
-    tap[t] = make_scope_tap<float>(scope_coord<float>(f_h, r_h, g.centre_h),
-                                   scope_coord<float>(f_w, r_w, g.centre_w), SH, SW, Tb::RS);
-    tap[t].cell = Tb::slot(tap[t].cell) * 4;
+    tap[t] = make_lite_tap<SH, SW>(scope_coord<float>(f_h, r_h, g.centre_h),
+                                   scope_coord<float>(f_w, r_w, g.centre_w), ok);
   }
   __syncthreads();
 
@@ -214,8 +280,7 @@ __global__ __launch_bounds__(kBlock, 2) void local_gather_kernel(Geo g, const T*
 #pragma unroll
       for (int t = 0; t < K; ++t) {
         const float4 q = *reinterpret_cast<const float4*>(tb + tap[t].cell + u * Tb::SIZE);
-        const float b = tap[t].c00 * q.x + tap[t].c01 * q.y + tap[t].c10 * q.z + tap[t].c11 * q.w;
-        acc += xv[u][t] * b;
+        acc = fmaf(xv[u][t], lite_weight(tap[t], q), acc);
       }
       buf_st(plane_rsrc(dp + (size_t)(jb + u) * d_step, (jb + u) < nch ? dst_plane : 0), doff, acc, dst);
     }
@@ -272,7 +337,7 @@ __global__ __launch_bounds__(kBlock, 2) void local_gather_rows_kernel(Geo g, con
   const int n = bz / g.groups, grp = bz % g.groups;
   const int j0 = by * ch_per_block;
   const int nch = min(ch_per_block, cpg - j0);
-  stage_wide_tables<T, SH, SW>(tbl, filter, grp + g.groups * j0, g.groups, nch);
+  stage_wide_tables<T, SH, SW>(tbl, filter, g.channel, grp + g.groups * j0, g.groups, nch);
 
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int p = bx * kRowPix + wave * kRowLanes + lane - 1;  // lanes 0 and 63 are halo
@@ -289,7 +354,7 @@ __global__ __launch_bounds__(kBlock, 2) void local_gather_rows_kernel(Geo g, con
     roff[r] = (e >= 0 && e < src_plane) ? (unsigned)e * (unsigned)sizeof(T) : kOutOfRange;
   }
 
-  ScopeTap<float> tap[K];
+  LiteTap tap[K];
   const rsrc_t rr = plane_rsrc(rot + (size_t)(n * g.groups + grp) * (K * 2) * out_plane, K * 2 * out_plane);
 #pragma unroll
   for (int t = 0; t < K; ++t) {
@@ -299,10 +364,8 @@ __global__ __launch_bounds__(kBlock, 2) void local_gather_rows_kernel(Geo g, con
     const unsigned ro = ok ? (unsigned)((2 * t) * out_plane + rpix) * (unsigned)sizeof(T) : kOutOfRange;
     const float r_h = buf_ld(rr, ro, rot);
     const float r_w = buf_ld(rr, ro + (unsigned)out_plane * (unsigned)sizeof(T), rot);
-    tap[t] = make_scope_tap<float>(scope_coord<float>(f_h, r_h, g.centre_h),
-                                   scope_coord<float>(f_w, r_w, g.centre_w), SH, SW, Tb::RS);
-    tap[t].cell = Tb::slot(tap[t].cell) * 4;
-    if (!ok) tap[t].c00 = tap[t].c01 = tap[t].c10 = tap[t].c11 = 0.f;  // tap in the padding
+    tap[t] = make_lite_tap<SH, SW>(scope_coord<float>(f_h, r_h, g.centre_h),
+                                   scope_coord<float>(f_w, r_w, g.centre_w), ok);  // !ok: tap in the padding
   }
   __syncthreads();
 
@@ -336,8 +399,7 @@ __global__ __launch_bounds__(kBlock, 2) void local_gather_rows_kernel(Geo g, con
           const int dc = TRANSPOSED ? 1 - f_w : f_w - 1;
           const float xv = dc < 0 ? xm : dc == 0 ? x0 : xp;
           const float4 q = *reinterpret_cast<const float4*>(tb + tap[t].cell + u * Tb::SIZE);
-          const float b = tap[t].c00 * q.x + tap[t].c01 * q.y + tap[t].c10 * q.z + tap[t].c11 * q.w;
-          acc += xv * b;
+          acc = fmaf(xv, lite_weight(tap[t], q), acc);
         }
       }
       buf_st(plane_rsrc(dp + (size_t)(jb + u) * d_step, (jb + u) < nch ? dst_plane : 0), doff, acc, dst);
@@ -356,10 +418,11 @@ __global__ __launch_bounds__(kBlock, 2) void local_gather_rows_kernel(Geo g, con
 
 // ---------------------------------------------------------------------------
 // grad rotation: the lane owns output pixel p of (n, group) and sums over channels.
-// d/dh and d/dw of the bilinear read are linear in the four corner weights with
-// channel-independent coefficients, so the lane only accumulates
-//   S_k[t] = sum_c x_t[c] * gout[c] * corner_k[c]
-// and combines the four sums per tap once at the end (K.cu:137-158 gives the combination);
+// With the block in difference form {a, b, c, d} the derivatives of the bilinear read are
+// d/dh = c + lw * d and d/dw = b + lh * d (K.cu:137-158 in corner form), with channel-independent
+// lh, lw, so the lane only accumulates
+//   S_b[t], S_c[t], S_d[t] = sum_c x_t[c] * gout[c] * {b, c, d}[c]
+// and combines the three sums per tap once at the end;
 // the fractional parts needed for that are recomputed from the rotation rather than kept
 // in registers across the channel loop.
 //
@@ -421,14 +484,14 @@ __global__ __launch_bounds__(kBlock, 2) void local_grad_rotation_kernel(
   }
   const unsigned goff = owns ? (unsigned)p * (unsigned)sizeof(T) : kOutOfRange;
 
-  float s00[K], s01[K], s10[K], s11[K];
+  float sb[K], sc[K], sd[K];
 #pragma unroll
-  for (int t = 0; t < K; ++t) s00[t] = s01[t] = s10[t] = s11[t] = 0.f;
+  for (int t = 0; t < K; ++t) sb[t] = sc[t] = sd[t] = 0.f;
 
   for (int j0 = 0; j0 < cpg; j0 += ch_per_pass) {
     const int nch = min(ch_per_pass, cpg - j0);
     __syncthreads();
-    stage_wide_tables<T, SH, SW>(tbl, filter, grp + g.groups * j0, g.groups, nch);
+    stage_wide_tables<T, SH, SW>(tbl, filter, g.channel, grp + g.groups * j0, g.groups, nch);
     __syncthreads();
     const size_t chan0 = (size_t)n * g.channel + grp + (size_t)g.groups * j0;
     const T* xp = x + chan0 * in_plane;
@@ -456,11 +519,10 @@ __global__ __launch_bounds__(kBlock, 2) void local_grad_rotation_kernel(
         }
         // gv is 0 on lanes that own no pixel, and taps in the padding are masked at the end
         const float ps = xt * gv[s];
-        const float4 q = *reinterpret_cast<const float4*>(tb + cell[t]);
-        s00[t] += ps * q.x;
-        s01[t] += ps * q.y;
-        s10[t] += ps * q.z;
-        s11[t] += ps * q.w;
+        const float4 q = lds_read4(tb + cell[t]);
+        sb[t] = fmaf(ps, q.y, sb[t]);
+        sc[t] = fmaf(ps, q.z, sc[t]);
+        sd[t] = fmaf(ps, q.w, sd[t]);
       }
     };
     load(0, 0);
@@ -481,9 +543,8 @@ __global__ __launch_bounds__(kBlock, 2) void local_grad_rotation_kernel(
     const float w = scope_coord<float>(f_w, buf_ld(rr, ro + (unsigned)out_plane * (unsigned)sizeof(T), rot),
                                        g.centre_w);
     const float lh = h - floorf(h), lw = w - floorf(w);
-    const float hh = 1.f - lh, hw = 1.f - lw;
-    float gh = hw * (s10[t] - s00[t]) + lw * (s11[t] - s01[t]);
-    float gw = hh * (s01[t] - s00[t]) + lh * (s11[t] - s10[t]);
+    float gh = fmaf(lw, sd[t], sc[t]);
+    float gw = fmaf(lh, sd[t], sb[t]);
     if (!(inside >> t & 1u)) gh = gw = 0.f;
     buf_st(ro_, ro, gh, grot);
     buf_st(ro_, ro + (unsigned)out_plane * (unsigned)sizeof(T), gw, grot);
