@@ -156,9 +156,9 @@ __host__ __device__ __forceinline__ int ceil_div(int a, int b) { return (a + b -
 // ---------------------------------------------------------------------------
 constexpr int kXcds = 8;
 __host__ __device__ __forceinline__ long xcd_grid_size(long total) { return (total + kXcds - 1) / kXcds * kXcds; }
-__device__ __forceinline__ long logical_block(long total) {
-  const long chunk = (total + kXcds - 1) / kXcds;
-  return (long)(blockIdx.x % kXcds) * chunk + blockIdx.x / kXcds;
+__device__ __forceinline__ int logical_block(int total) {
+  const int chunk = (total + kXcds - 1) / kXcds;
+  return (int)(blockIdx.x % kXcds) * chunk + (int)(blockIdx.x / kXcds);
 }
 
 // Sum of v over the 64 lanes of the wave, returned in every lane: six DPP adds and one readlane
@@ -182,6 +182,19 @@ __device__ __forceinline__ float from_lane_below(float v) {
 }
 __device__ __forceinline__ float from_lane_above(float v) {
   return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x130 /* wave_shl:1 */, 0xf, 0xf, true));
+}
+
+// acc + (value of x held by the previous / next lane) * w in one instruction: the multiply-add
+// takes its first operand through the DPP lane shift (0 at the wave's ends).  The s_nop covers
+// the two idle states a DPP read needs after a vector write of its operand, in case the
+// compiler schedules such a write directly in front.
+__device__ __forceinline__ float fma_lane_below(float x, float w, float acc) {
+  asm("s_nop 1\n\tv_fmac_f32_dpp %0, %1, %2 wave_shr:1 row_mask:0xf bank_mask:0xf bound_ctrl:1" : "+v"(acc) : "v"(x), "v"(w));
+  return acc;
+}
+__device__ __forceinline__ float fma_lane_above(float x, float w, float acc) {
+  asm("s_nop 1\n\tv_fmac_f32_dpp %0, %1, %2 wave_shl:1 row_mask:0xf bank_mask:0xf bound_ctrl:1" : "+v"(acc) : "v"(x), "v"(w));
+  return acc;
 }
 
 // ---------------------------------------------------------------------------

@@ -15,6 +15,8 @@
 //   grad filter    K.cu:836-955   -> local_grad_filter_kernel + reduce_partials_kernel
 #include <cstdlib>
 
+#include <algorithm>
+
 #include "dk_kernels.h"
 
 namespace dk {
@@ -223,10 +225,10 @@ __global__ __launch_bounds__(kBlock, 2) void local_gather_kernel(Geo g, const T*
   const int dst_w = TRANSPOSED ? g.in_w : g.out_w;
   // logical block = (tile, channel split, image * group), tile fastest: one XCD gets whole images
   const int tiles = ceil_div(dst_plane, kBlock), splits = ceil_div(cpg, ch_per_block);
-  const long total = (long)tiles * splits * g.batch * g.groups;
-  const long lb = logical_block(total);
+  const int total = tiles * splits * g.batch * g.groups;
+  const int lb = logical_block(total);
   if (lb >= total) return;
-  const int bx = (int)(lb % tiles), by = (int)(lb / tiles % splits), bz = (int)(lb / tiles / splits);
+  const int bx = lb % tiles, by = lb / tiles % splits, bz = lb / tiles / splits;
   const int n = bz / g.groups, grp = bz % g.groups;
   const int j0 = by * ch_per_block;
   const int nch = min(ch_per_block, cpg - j0);
@@ -330,10 +332,10 @@ __global__ __launch_bounds__(kBlock, 2) void local_gather_rows_kernel(Geo g, con
   const int src_plane = TRANSPOSED ? out_plane : in_plane;
   // logical block = (tile, channel split, image * group), tile fastest: one XCD gets whole images
   const int tiles = ceil_div(dst_plane, kRowPix), splits = ceil_div(cpg, ch_per_block);
-  const long total = (long)tiles * splits * g.batch * g.groups;
-  const long lb = logical_block(total);
+  const int total = tiles * splits * g.batch * g.groups;
+  const int lb = logical_block(total);
   if (lb >= total) return;
-  const int bx = (int)(lb % tiles), by = (int)(lb / tiles % splits), bz = (int)(lb / tiles / splits);
+  const int bx = lb % tiles, by = lb / tiles % splits, bz = lb / tiles / splits;
   const int n = bz / g.groups, grp = bz % g.groups;
   const int j0 = by * ch_per_block;
   const int nch = min(ch_per_block, cpg - j0);
@@ -392,14 +394,15 @@ __global__ __launch_bounds__(kBlock, 2) void local_gather_rows_kernel(Geo g, con
       for (int r = 0; r < KH; ++r) {
         // elements at columns -1, 0, +1 of this row; the tap that reads column dc is
         // f_w = dc + 1 (forward) or f_w = 1 - dc (grad input)
-        const float xm = from_lane_below(xc[u][r]), x0 = xc[u][r], xp = from_lane_above(xc[u][r]);
 #pragma unroll
         for (int f_w = 0; f_w < KW; ++f_w) {
           const int t = r * KW + f_w;
           const int dc = TRANSPOSED ? 1 - f_w : f_w - 1;
-          const float xv = dc < 0 ? xm : dc == 0 ? x0 : xp;
           const float4 q = *reinterpret_cast<const float4*>(tb + tap[t].cell + u * Tb::SIZE);
-          acc = fmaf(xv, lite_weight(tap[t], q), acc);
+          const float wt = lite_weight(tap[t], q);
+          // columns -1 / +1 of the row are the neighbouring lanes' centre elements
+          acc = dc < 0 ? fma_lane_below(xc[u][r], wt, acc) : dc == 0 ? fmaf(xc[u][r], wt, acc)
+                                                                     : fma_lane_above(xc[u][r], wt, acc);
         }
       }
       buf_st(plane_rsrc(dp + (size_t)(jb + u) * d_step, (jb + u) < nch ? dst_plane : 0), doff, acc, dst);
@@ -444,10 +447,10 @@ __global__ __launch_bounds__(kBlock, 2) void local_grad_rotation_kernel(
   const int out_plane = g.out_h * g.out_w, in_plane = g.in_h * g.in_w;
   // logical block = (tile, image * group), tile fastest
   const int tiles = ceil_div(out_plane, ROWS ? kRowPix : kBlock);
-  const long total = (long)tiles * g.batch * g.groups;
-  const long lb = logical_block(total);
+  const int total = tiles * g.batch * g.groups;
+  const int lb = logical_block(total);
   if (lb >= total) return;
-  const int bx = (int)(lb % tiles), bz = (int)(lb / tiles);
+  const int bx = lb % tiles, bz = lb / tiles;
   const int n = bz / g.groups, grp = bz % g.groups;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int p = ROWS ? bx * kRowPix + wave * kRowLanes + lane - 1 : bx * kBlock + threadIdx.x;
@@ -585,10 +588,10 @@ __global__ __launch_bounds__(kBlock, 2) void local_grad_filter_kernel(
   // (image, tile) item and the items of one image share an XCD
   const int cpg = g.channel / g.groups;
   const int splits = ceil_div(cpg, ch_per_block);
-  const long total = (long)splits * parts * g.groups;
-  const long lb = logical_block(total);
+  const int total = splits * parts * g.groups;
+  const int lb = logical_block(total);
   if (lb >= total) return;
-  const int by = (int)(lb % splits), bx = (int)(lb / splits % parts), grp = (int)(lb / splits / parts);
+  const int by = lb % splits, bx = lb / splits % parts, grp = lb / splits / parts;
 
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   for (int e = threadIdx.x; e < kWaves * ch_per_block * 16; e += kBlock) wacc[e] = 0.f;
@@ -876,7 +879,10 @@ bool run_grad_filter(const Geo& g, const T* gout, const T* x, const T* rot, T* g
 
 bool fast_shape(const Geo& g) {
   const long plane_limit = (1L << 31) / 4 / 32;  // byte offsets inside a plane (x 18 for rotation) stay below 2^31
-  return g.k_h == 3 && g.k_w == 3 && (long)g.batch * g.groups <= (1L << 20) &&
+  // every grid is 1-D with at most tiles * channels * batch blocks, indexed in 32 bits
+  const long max_plane = std::max((long)g.in_h * g.in_w, (long)g.out_h * g.out_w);
+  const long max_blocks = ((max_plane + kRowPix - 1) / kRowPix) * g.channel * g.batch;
+  return g.k_h == 3 && g.k_w == 3 && max_blocks < (1L << 31) - 8 &&
          (long)g.in_h * g.in_w < plane_limit && (long)g.out_h * g.out_w < plane_limit &&
          ((g.scope_h == 4 && g.scope_w == 4) || (g.scope_h == 3 && g.scope_w == 3) ||
           (g.scope_h == 5 && g.scope_w == 5));
