@@ -726,6 +726,276 @@ __global__ __launch_bounds__(kBlock, 2) void local_grad_filter_kernel(
 
 }  // namespace
 
+// ---------------------------------------------------------------------------
+// grad filter on the matrix cores, for "same" geometries (see local_gather_rows_kernel).
+//
+// With k = (pixel, tap) the reduction is a matrix product per block of 16 channels,
+//   gW[cell][c] = sum_k A[cell][k] * P[k][c],
+//   A[cell = (i, j)][k] = hat(h_k - i) * hat(w_k - j)      (channel independent),
+//   P[k][c] = x_k[c] * gout[c],
+// and v_mfma_f32_16x16x4_f32 adds a 16 (cells) x 16 (channels) block over four k per issue in
+// full fp32: lane l supplies A[l % 16][l / 16] and P[l / 16][l % 16].  So a lane stands for
+// cell l % 16 on the A side and for channel l % 16 on the P side, and for pixel quad l / 16.
+//
+// A unit of work is (image, 128-pixel tile, channel block); a workgroup of 8 waves walks a
+// contiguous range of units, channel block fastest, so that all workgroups (two per CU, all
+// resident) carry the same load.  Wave w owns pixels 16 w .. 16 w + 15 of the tile.
+//   * per tile: the scope coordinates (h, w) of every (pixel, tap) go to LDS (taps in the
+//     padding and coordinates outside the scope band as (-2, -2), where every hat is 0) and
+//     every lane derives its 36 A values (4 pixels x 9 taps), kept in registers for all the
+//     channel blocks of the tile;
+//   * per unit: the 16 channels' tiles of gout and of x with its halo rows are staged
+//     channel-major in LDS from loads coalesced along pixels; a lane reads its channel's
+//     4 gout and 3 x 6 input values and issues 36 MFMAs.  The loads of the next unit are
+//     issued before the MFMAs and land in registers while they run.
+//   * the 8 waves' 16 x 16 results of a unit are added into a per-channel-block accumulator in
+//     LDS (by a fixed owner thread, in wave order), piggybacked on the next unit's barriers.
+// One partial per workgroup goes to the workspace; reduce_partials_kernel adds them in order.
+// grid = (workgroups, channel splits, groups); a channel split is at most kMfMaxBlk blocks
+// ---------------------------------------------------------------------------
+constexpr int kMfPix = 128;            // output pixels per tile
+constexpr int kMfCh = 16;              // channels per unit
+constexpr int kMfBlock = 512;          // threads per workgroup
+constexpr int kMfPitchG = kMfPix + 4;  // floats per channel of the gout tile (16-byte reads, bank skew)
+constexpr int kMfX = 6;                // input elements per lane and channel: tile + halo rows <= 64 * kMfX
+constexpr int kMfMaxBlk = 16;          // channel blocks accumulated by one workgroup
+
+typedef float mf4 __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ float hat(float d) { return __builtin_amdgcn_fmed3f(1.f - fabsf(d), 0.f, 1.f); }
+
+template <typename T, int SH, int SW>
+__global__ __launch_bounds__(kMfBlock, 4) void local_grad_filter_mfma_kernel(
+    Geo g, const T* __restrict__ gout, const T* __restrict__ x, const T* __restrict__ rot,
+    float* __restrict__ partial, int tiles, int nwg, int csplits, int pitch_x) {
+  constexpr int K = 9, CELLS = SH * SW;
+  constexpr int kWaves = kMfBlock / 64;
+  static_assert(CELLS <= 16, "one 16-row MFMA block holds the cells");
+  static_assert(kMfPix == 16 * kWaves, "one 16-pixel group per wave");
+  extern __shared__ __align__(16) float lds[];
+  float* xs = lds;                                                  // [kMfCh][pitch_x]
+  float* gs = xs + kMfCh * pitch_x;                                 // [kMfCh][kMfPitchG]
+  float2* hw = reinterpret_cast<float2*>(gs + kMfCh * kMfPitchG);   // [K][kMfPix]
+  float* red = reinterpret_cast<float*>(hw + K * kMfPix);           // [kWaves][256]
+  float* accs = red + kWaves * 256;                                 // [blocks of this split][256]
+
+  const int cpg = g.channel / g.groups;
+  const int nblk_all = ceil_div(cpg, kMfCh);
+  const int total = nwg * csplits * g.groups;
+  const int lb = logical_block(total);
+  if (lb >= total) return;
+  const int wg = lb % nwg, cs = lb / nwg % csplits, grp = lb / nwg / csplits;
+  const int blk_per = ceil_div(nblk_all, csplits);
+  const int cb_lo = cs * blk_per, nblk = min(blk_per, nblk_all - cb_lo);
+
+  const int W = g.in_w;  // == out_w
+  const int out_plane = g.out_h * W, in_plane = g.in_h * W;
+  // the wave index picks channel planes (buffer resources): tell the compiler it is uniform
+  const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int q = lane & 15, kg = lane >> 4;
+  const int row_step = g.dil_h * W;               // elements between two tap rows
+  const int lo = -g.pad_h * W - 1;                // first staged input element, relative to the tile
+  const int xt = kMfPix + 2 + 2 * row_step;       // staged input elements per channel
+  const float ci = q < CELLS ? float(q / SW) : 64.f, cj = float(q % SW);  // rows 9..15 of a 3x3 scope stay 0
+
+  for (int e = threadIdx.x; e < nblk * 256; e += kMfBlock) accs[e] = 0.f;
+
+  // This workgroup's share of the (tile, channel block) units of its group and channel split, as
+  // segments (tile, first block, end block).  Whole tiles are dealt out round-robin, tile t to
+  // workgroup t % nwg, so that neighbouring workgroups (same XCD, same pace) hold neighbouring
+  // tiles of the same channel block at the same time and the halo rows they share are fetched
+  // from memory once; the channel blocks of the last items % nwg tiles are dealt out singly to
+  // keep the load even.
+  const int items = g.batch * tiles;
+  const int whole = items / nwg;                      // whole tiles per workgroup
+  const int rest_units = (items - whole * nwg) * nblk;
+  const int nseg = whole + (rest_units > wg ? (rest_units - wg + nwg - 1) / nwg : 0);
+  auto segment = [&](int k, int& item, int& cb_begin, int& cb_end) {
+    if (k < whole) {
+      item = wg + k * nwg;
+      cb_begin = 0;
+      cb_end = nblk;
+    } else {
+      const int r = wg + (k - whole) * nwg;
+      item = whole * nwg + r / nblk;
+      cb_begin = r % nblk;
+      cb_end = cb_begin + 1;
+    }
+  };
+
+  // Register stage of one unit: what this thread loads (the rotation values of its pixel for
+  // its share of the taps when the unit starts a tile; kMfX input and 2 gout values of each of
+  // its wave's 2 channels).
+  constexpr int kChW = kMfCh / kWaves;                                  // channels staged per wave
+  constexpr int kTapsT = (K + kMfBlock / kMfPix - 1) / (kMfBlock / kMfPix);  // taps staged per thread
+  const int pix = threadIdx.x % kMfPix;                                 // pixel whose coordinates this thread stages
+  const int tapq = __builtin_amdgcn_readfirstlane(threadIdx.x / kMfPix);  // ... for taps tapq + 4 k
+  float r_rot[2 * kTapsT], r_x[kChW][kMfX], r_g[kChW][kMfPix / 64];
+  auto issue_loads = [&](int item, int cbi, bool with_rot) {
+    const int cb = cb_lo + cbi;
+    const int n = item / tiles, p0 = (item % tiles) * kMfPix;
+    if (with_rot) {
+      const int p = p0 + pix;
+      const rsrc_t rr = plane_rsrc(rot + (size_t)(n * g.groups + grp) * (K * 2) * out_plane, K * 2 * out_plane);
+      const unsigned ro = p < out_plane ? (unsigned)p * (unsigned)sizeof(T) : kOutOfRange;
+#pragma unroll
+      for (int k = 0; k < kTapsT; ++k) {
+        const int t = tapq + (kMfBlock / kMfPix) * k;
+        const unsigned o = t < K ? ro + (unsigned)(2 * t * out_plane) * (unsigned)sizeof(T) : kOutOfRange;
+        r_rot[2 * k] = buf_ld(rr, o, rot);
+        r_rot[2 * k + 1] = buf_ld(rr, o + (unsigned)out_plane * (unsigned)sizeof(T), rot);
+      }
+    }
+#pragma unroll
+    for (int jj = 0; jj < kChW; ++jj) {
+      const int cj_ = cb * kMfCh + wave + jj * kWaves;
+      const bool chan = cj_ < cpg;
+      const size_t c = (size_t)n * g.channel + grp + (size_t)g.groups * (chan ? cj_ : 0);
+      const rsrc_t rx = plane_rsrc(x + c * in_plane, chan ? in_plane : 0);
+      const rsrc_t rg = plane_rsrc(gout + c * out_plane, chan ? out_plane : 0);
+#pragma unroll
+      for (int k = 0; k < kMfX; ++k) {
+        const int i = lane + 64 * k;
+        const long e = (long)p0 + lo + i;
+        r_x[jj][k] = buf_ld(rx, (i < xt && e >= 0 && e < in_plane) ? (unsigned)e * (unsigned)sizeof(T) : kOutOfRange, x);
+      }
+#pragma unroll
+      for (int k = 0; k < kMfPix / 64; ++k) {
+        const int e = p0 + lane + 64 * k;
+        r_g[jj][k] = buf_ld(rg, e < out_plane ? (unsigned)e * (unsigned)sizeof(T) : kOutOfRange, gout);
+      }
+    }
+  };
+  // Register stage -> LDS.  Scope coordinates: K.cu:338-341 and the band test of K.cu:59.
+  auto store_unit = [&](int item, bool with_rot) {
+    if (with_rot) {
+      const int p = (item % tiles) * kMfPix + pix;
+      const bool live = p < out_plane;
+      const int pc = live ? p : 0;
+      const int ph = pc / W, pw = pc % W;
+#pragma unroll
+      for (int k = 0; k < kTapsT; ++k) {
+        const int t = tapq + (kMfBlock / kMfPix) * k;
+        if (t < K) {
+          const int f_h = t / 3, f_w = t % 3;
+          const int ih = ph + f_h * g.dil_h - g.pad_h, iw = pw + f_w - 1;
+          const bool ok = live && ih >= 0 && ih < g.in_h && iw >= 0 && iw < W;
+          const float h = scope_coord<float>(f_h, r_rot[2 * k], g.centre_h);
+          const float w = scope_coord<float>(f_w, r_rot[2 * k + 1], g.centre_w);
+          const bool in = ok && (h > -1.f) && (w > -1.f) && (h < float(SH)) && (w < float(SW));
+          hw[t * kMfPix + pix] = in ? make_float2(h, w) : make_float2(-2.f, -2.f);
+        }
+      }
+    }
+#pragma unroll
+    for (int jj = 0; jj < kChW; ++jj) {
+      const int j = wave + jj * kWaves;
+#pragma unroll
+      for (int k = 0; k < kMfX; ++k)
+        if (lane + 64 * k < xt) xs[j * pitch_x + lane + 64 * k] = r_x[jj][k];
+#pragma unroll
+      for (int k = 0; k < kMfPix / 64; ++k) gs[j * kMfPitchG + lane + 64 * k] = r_g[jj][k];
+    }
+  };
+
+  const int px = wave * 16 + 4 * kg;  // first of this lane's four pixels in the tile
+  float A[4][K];
+  mf4 acc = {0.f, 0.f, 0.f, 0.f};
+  int done_cb = -1;  // channel block (within the split) whose result `acc` holds
+
+  // stage the unit whose loads are in flight, hand the previous unit's result to its owner
+  // threads, start the next unit's loads (n_item < 0: there is none)
+  auto begin_unit = [&](int item, bool new_tile, int n_item, int n_cbi, bool n_new_tile) {
+    __syncthreads();  // the previous unit's reads of the tiles (and of `red`) are done
+    store_unit(item, new_tile);
+    if (done_cb >= 0) *reinterpret_cast<mf4*>(red + (wave * 64 + lane) * 4) = acc;
+    __syncthreads();
+    if (n_item >= 0) issue_loads(n_item, n_cbi, n_new_tile);
+    if (done_cb >= 0 && threadIdx.x < 256) {
+      float s = 0.f;
+#pragma unroll
+      for (int w = 0; w < kWaves; ++w) s += red[w * 256 + threadIdx.x];
+      accs[done_cb * 256 + threadIdx.x] += s;
+    }
+  };
+  auto multiply_unit = [&](int cbi) {
+    mf4 acc0 = {0.f, 0.f, 0.f, 0.f}, acc1 = {0.f, 0.f, 0.f, 0.f};
+    const float4 gv = *reinterpret_cast<const float4*>(gs + q * kMfPitchG + px);
+    const float gq[4] = {gv.x, gv.y, gv.z, gv.w};
+#pragma unroll
+    for (int r = 0; r < 3; ++r) {
+      // columns -1 .. +4 of tap row r around the four pixels
+      const float* xr = xs + q * pitch_x + px + r * row_step;
+      float x6[6];
+#pragma unroll
+      for (int k = 0; k < 6; ++k) x6[k] = xr[k];
+#pragma unroll
+      for (int f_w = 0; f_w < 3; ++f_w) {
+        const int t = r * 3 + f_w;
+#pragma unroll
+        for (int ii = 0; ii < 4; ++ii) {
+          const float b = x6[ii + f_w] * gq[ii];
+          if ((ii + t) & 1)
+            acc1 = __builtin_amdgcn_mfma_f32_16x16x4f32(A[ii][t], b, acc1, 0, 0, 0);
+          else
+            acc0 = __builtin_amdgcn_mfma_f32_16x16x4f32(A[ii][t], b, acc0, 0, 0, 0);
+        }
+      }
+    }
+    acc = acc0 + acc1;
+    done_cb = cbi;
+  };
+
+  int item = 0, cb_begin = 0, cb_end = 0;
+  if (nseg > 0) {
+    segment(0, item, cb_begin, cb_end);
+    issue_loads(item, cb_begin, true);
+  }
+  for (int k = 0; k < nseg; ++k) {
+    int n_item = -1, n_begin = 0, n_end = 0;  // the next segment, whose first unit follows this one's last
+    if (k + 1 < nseg) segment(k + 1, n_item, n_begin, n_end);
+    const bool single = cb_begin + 1 == cb_end;
+    begin_unit(item, true, single ? n_item : item, single ? n_begin : cb_begin + 1, single);
+#pragma unroll
+    for (int t = 0; t < K; ++t) {
+      const float4 hw01 = *reinterpret_cast<const float4*>(hw + t * kMfPix + px);
+      const float4 hw23 = *reinterpret_cast<const float4*>(hw + t * kMfPix + px + 2);
+      A[0][t] = hat(hw01.x - ci) * hat(hw01.y - cj);
+      A[1][t] = hat(hw01.z - ci) * hat(hw01.w - cj);
+      A[2][t] = hat(hw23.x - ci) * hat(hw23.y - cj);
+      A[3][t] = hat(hw23.z - ci) * hat(hw23.w - cj);
+    }
+    multiply_unit(cb_begin);
+    for (int cbi = cb_begin + 1; cbi < cb_end; ++cbi) {
+      const bool last = cbi + 1 == cb_end;
+      begin_unit(item, false, last ? n_item : item, last ? n_begin : cbi + 1, last);
+      multiply_unit(cbi);
+    }
+    item = n_item;
+    cb_begin = n_begin;
+    cb_end = n_end;
+  }
+
+  // the last unit's result, then D[cell = 4 * (l / 16) + r][channel = l % 16] (register r of lane l,
+  // entry 4 l + r of a block's accumulator) goes out as this workgroup's partial
+  __syncthreads();
+  if (done_cb >= 0) *reinterpret_cast<mf4*>(red + (wave * 64 + lane) * 4) = acc;
+  __syncthreads();
+  if (done_cb >= 0 && threadIdx.x < 256) {
+    float s = 0.f;
+#pragma unroll
+    for (int w = 0; w < kWaves; ++w) s += red[w * 256 + threadIdx.x];
+    accs[done_cb * 256 + threadIdx.x] += s;
+  }
+  __syncthreads();
+  for (int e = threadIdx.x; e < nblk * 256; e += kMfBlock) {
+    const int b = e / 256, l = (e % 256) / 4, r = e % 4;
+    const int cell = 4 * (l / 16) + r, cj_ = (cb_lo + b) * kMfCh + l % 16;
+    if (cell < CELLS && cj_ < cpg)
+      partial[((size_t)wg * g.channel + grp + (size_t)g.groups * cj_) * CELLS + cell] = accs[e];
+  }
+}
+
 // out[e] = sum over parts of partial[part][e].  8 elements per workgroup, 32 threads per
 // element each summing every 32nd part, combined in a fixed order (run-to-run reproducible).
 constexpr int kRedEl = 8, kRedSlices = 32;
@@ -843,11 +1113,40 @@ constexpr int kFilterChPerBlock = 36;
 
 struct FilterGrid {
   int per, splits, parts, tiles;
+  bool mfma;       // matrix-core kernel: 16 channels per workgroup, 256-pixel tiles
+  int pitch_x;     // its floats per channel of the staged input tile
+  size_t lds;      // its LDS bytes
 };
 
 FilterGrid filter_grid(const Geo& g) {
   FilterGrid f;
   const int cpg = g.channel / g.groups;
+  f.mfma = false;
+  f.pitch_x = 0;
+  f.lds = 0;
+  if (same_width_geometry(g) && g.scope_h * g.scope_w <= 16 && !getenv("DK_NO_MFMA")) {
+    const long xt = kMfPix + 2 + 2L * g.dil_h * g.in_w;
+    long pitch = (xt + 3) / 4 * 4;
+    while (pitch % 64 != 4) pitch += 4;  // channel rows 4 banks apart: 16 channels read conflict-free
+    const int nblk = ceil_div(cpg, kMfCh);
+    const int csplits = ceil_div(nblk, kMfMaxBlk);
+    const long lds = ((long)kMfCh * pitch + (long)kMfCh * kMfPitchG) * 4 + 9L * kMfPix * 8 +
+                     (long)(kMfBlock / 64) * 256 * 4 + (long)ceil_div(nblk, csplits) * 256 * 4;
+    if (lds <= 64 * 1024 && xt <= 64 * kMfX) {
+      f.mfma = true;
+      f.pitch_x = (int)pitch;
+      f.lds = (size_t)lds;
+      f.per = kMfCh;
+      f.splits = csplits;
+      f.tiles = ceil_div(g.out_h * g.out_w, kMfPix);
+      // two workgroups of 8 waves fit a CU: launch at most that many, all resident at once,
+      // each walking an equal share of the (tile, channel block) units
+      const long units = (long)g.batch * f.tiles * ceil_div(nblk, csplits);
+      const long slots = std::max(1, 2 * 256 / (csplits * g.groups));
+      f.parts = (int)std::max(1L, std::min(units, slots));
+      return f;
+    }
+  }
   f.splits = ceil_div(cpg, kFilterChPerBlock);
   f.per = ceil_div(cpg, f.splits);
   f.tiles = ceil_div(g.out_h * g.out_w, same_width_geometry(g) ? kRowPix : kBlock);
@@ -867,6 +1166,11 @@ bool run_grad_filter(const Geo& g, const T* gout, const T* x, const T* rot, T* g
   } else {
     const FilterGrid f = filter_grid(g);
     const unsigned grid = (unsigned)xcd_grid_size((long)f.parts * f.splits * g.groups);
+    if (f.mfma) {
+      local_grad_filter_mfma_kernel<T, SH, SW><<<grid, kMfBlock, f.lds, stream>>>(g, gout, x, rot, ws, f.tiles, f.parts, f.splits, f.pitch_x);
+      launch_reduce_partials<float, T>(ws, f.parts, g.channel * SH * SW, gfilter, stream);
+      return true;
+    }
     const size_t lds = ((size_t)(kBlock / 64) * f.per * 16 + (size_t)(kBlock / 64) * 64 * 20) * sizeof(float);
     if (same_width_geometry(g))
       local_grad_filter_kernel<T, 3, 3, SH, SW, true><<<grid, kBlock, lds, stream>>>(g, gout, x, rot, ws, f.tiles, f.per, f.parts);
