@@ -762,6 +762,11 @@ constexpr int kMfMaxBlk = 16;          // channel blocks accumulated by one work
 
 typedef float mf4 __attribute__((ext_vector_type(4)));
 
+// First float of channel j's row in the staged input tile.  The rows are a multiple of 64 floats
+// apart plus a skew: in the MFMA phase lane (channel q, pixel quad kg) reads row q at
+// 4 * kg + const, and (q % 4) + 16 * (q / 4) + 4 * kg covers the 64 banks exactly once.
+__device__ __forceinline__ int mf_row(int j, int pitch_x) { return j * pitch_x + (j & 3) + 16 * (j >> 2); }
+
 __device__ __forceinline__ float hat(float d) { return __builtin_amdgcn_fmed3f(1.f - fabsf(d), 0.f, 1.f); }
 
 template <typename T, int SH, int SW>
@@ -892,7 +897,7 @@ __global__ __launch_bounds__(kMfBlock, 4) void local_grad_filter_mfma_kernel(
       const int j = wave + jj * kWaves;
 #pragma unroll
       for (int k = 0; k < kMfX; ++k)
-        if (lane + 64 * k < xt) xs[j * pitch_x + lane + 64 * k] = r_x[jj][k];
+        if (lane + 64 * k < xt) xs[mf_row(j, pitch_x) + lane + 64 * k] = r_x[jj][k];
 #pragma unroll
       for (int k = 0; k < kMfPix / 64; ++k) gs[j * kMfPitchG + lane + 64 * k] = r_g[jj][k];
     }
@@ -925,7 +930,7 @@ __global__ __launch_bounds__(kMfBlock, 4) void local_grad_filter_mfma_kernel(
 #pragma unroll
     for (int r = 0; r < 3; ++r) {
       // columns -1 .. +4 of tap row r around the four pixels
-      const float* xr = xs + q * pitch_x + px + r * row_step;
+      const float* xr = xs + mf_row(q, pitch_x) + px + r * row_step;
       float x6[6];
 #pragma unroll
       for (int k = 0; k < 6; ++k) x6[k] = xr[k];
@@ -1126,8 +1131,7 @@ FilterGrid filter_grid(const Geo& g) {
   f.lds = 0;
   if (same_width_geometry(g) && g.scope_h * g.scope_w <= 16 && !getenv("DK_NO_MFMA")) {
     const long xt = kMfPix + 2 + 2L * g.dil_h * g.in_w;
-    long pitch = (xt + 3) / 4 * 4;
-    while (pitch % 64 != 4) pitch += 4;  // channel rows 4 banks apart: 16 channels read conflict-free
+    const long pitch = (xt + 51 + 63) / 64 * 64;  // rows 64 floats apart plus the skew of mf_row() (at most 51)
     const int nblk = ceil_div(cpg, kMfCh);
     const int csplits = ceil_div(nblk, kMfMaxBlk);
     const long lds = ((long)kMfCh * pitch + (long)kMfCh * kMfPitchG) * 4 + 9L * kMfPix * 8 +
