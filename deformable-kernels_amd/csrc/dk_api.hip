@@ -223,6 +223,8 @@ int dk_deformable_sample_depthwise_forward(const dk_conv_desc* desc, const void*
   if (g.batch == 0) return DK_OK;
   hipStream_t s = static_cast<hipStream_t>(stream);
   return by_dtype(desc->dtype, [&]<typename T>() {
+    if constexpr (kHasFast<T>)
+      if (fast_deform_forward<T>(g, in<T>(input), in<T>(offset), in<T>(rotation), in<T>(filter), out<T>(output), s)) return;
     generic_forward<T>(g, true, in<T>(input), in<T>(offset), in<T>(rotation), in<T>(filter), out<T>(output), s);
   });
 }

@@ -23,6 +23,12 @@ template <typename T>
 bool fast_local_grad_filter(const Geo& g, const T* gout, const T* x, const T* rot, T* gfilter,
                             void* ws, hipStream_t stream);
 
+// ---- tuned deformable path (dk_deform_fast.hip): 3x3 taps, scope 3x3 / 4x4 / 5x5, fp32/fp16/bf16,
+//      input planes at most 64 columns wide that fit LDS
+template <typename T>
+bool fast_deform_forward(const Geo& g, const T* x, const T* off, const T* rot, const T* filter, T* out,
+                         hipStream_t stream);
+
 // ---- generic path (dk_generic.hip): any geometry, all four dtypes, local and deformable
 template <typename T>
 void generic_forward(const Geo& g, bool deform, const T* x, const T* off, const T* rot,
