@@ -268,6 +268,8 @@ def other_workload(a):
         desc = _lib.conv_desc(xg, wg, cfg["kernel_size"], cfg["stride"], cfg["padding"], cfg["dilation"], groups)
         ws1, n1 = _lib.workspace(L.dk_deformable_sample_depthwise_backward_data_workspace(desc), dev)
         ws2, n2 = _lib.workspace(L.dk_deformable_sample_depthwise_backward_filter_workspace(desc), dev)
+        ws3, n3 = _lib.workspace(L.dk_deformable_sample_depthwise_backward_offset_workspace(desc), dev)
+        ws4, n4 = _lib.workspace(L.dk_deformable_sample_depthwise_backward_rotation_workspace(desc), dev)
         st = _lib.stream_ptr(xg)
         e = xg.element_size()
         bx, by, br, bo, bw = [t.numel() * e for t in (xg, gg, rg, og, wg)]
@@ -277,9 +279,9 @@ def other_workload(a):
             "grad_input": (lambda: _lib.check(L.dk_deformable_sample_depthwise_backward_data(
                 desc, P(gg), P(og), P(rg), P(wg), P(gin), P(ws1), n1, st), "gin"), by + bo + br + bw + bx),
             "grad_offset": (lambda: _lib.check(L.dk_deformable_sample_depthwise_backward_offset(
-                desc, P(gg), P(xg), P(og), P(rg), P(wg), P(goff), st), "goff"), by + bx + bo + br + bw + bo),
+                desc, P(gg), P(xg), P(og), P(rg), P(wg), P(goff), P(ws3), n3, st), "goff"), by + bx + bo + br + bw + bo),
             "grad_rotation": (lambda: _lib.check(L.dk_deformable_sample_depthwise_backward_rotation(
-                desc, P(gg), P(xg), P(og), P(rg), P(wg), P(grot), st), "grot"), by + bx + bo + br + bw + br),
+                desc, P(gg), P(xg), P(og), P(rg), P(wg), P(grot), P(ws4), n4, st), "grot"), by + bx + bo + br + bw + br),
             "grad_filter": (lambda: _lib.check(L.dk_deformable_sample_depthwise_backward_filter(
                 desc, P(gg), P(xg), P(og), P(rg), P(gw), P(ws2), n2, st), "gw"), by + bx + bo + br + bw),
         }

@@ -3,6 +3,8 @@
 // Each entry point names the reference pybind function it stands in for
 // (K.cpp = deformable_kernels/ops/deform_kernel/csrc/filter_sample_depthwise_cuda.cpp,
 //  ND.cpp = .../csrc/nd_linear_sample_cuda.cpp).
+#include <algorithm>
+
 #include "dk_kernels.h"
 #include "dk_nd.h"
 
@@ -232,7 +234,7 @@ int dk_deformable_sample_depthwise_forward(const dk_conv_desc* desc, const void*
 size_t dk_deformable_sample_depthwise_backward_data_workspace(const dk_conv_desc* desc) {
   Geo g;
   if (make_geo(desc, g) != DK_OK) return 0;
-  return generic_deform_grad_input_workspace(g, desc->dtype);
+  return std::max(generic_deform_grad_input_workspace(g, desc->dtype), fast_deform_grad_input_workspace(g));
 }
 
 int dk_deformable_sample_depthwise_backward_data(const dk_conv_desc* desc, const void* out_grad,
@@ -243,11 +245,14 @@ int dk_deformable_sample_depthwise_backward_data(const dk_conv_desc* desc, const
   const int rc = make_geo(desc, g);
   if (rc != DK_OK) return rc;
   if (!out_grad || !offset || !rotation || !filter || !in_grad) return DK_ERR_NULL_POINTER;
-  const size_t need = generic_deform_grad_input_workspace(g, desc->dtype);
+  const size_t need = dk_deformable_sample_depthwise_backward_data_workspace(desc);
   if (need && (!workspace || workspace_bytes < need)) return DK_ERR_WORKSPACE;
   if (g.batch == 0) return DK_OK;
   hipStream_t s = static_cast<hipStream_t>(stream);
   return by_dtype(desc->dtype, [&]<typename T>() {
+    if constexpr (kHasFast<T>)
+      if (fast_deform_grad_input<T>(g, in<T>(out_grad), in<T>(offset), in<T>(rotation), in<T>(filter),
+                                    out<T>(in_grad), workspace, s)) return;
     generic_deform_grad_input<T>(g, in<T>(out_grad), in<T>(offset), in<T>(rotation), in<T>(filter),
                                  out<T>(in_grad), workspace, s);
   });
@@ -256,7 +261,7 @@ int dk_deformable_sample_depthwise_backward_data(const dk_conv_desc* desc, const
 size_t dk_deformable_sample_depthwise_backward_filter_workspace(const dk_conv_desc* desc) {
   Geo g;
   if (make_geo(desc, g) != DK_OK) return 0;
-  return generic_grad_filter_workspace(g, desc->dtype);
+  return std::max(generic_grad_filter_workspace(g, desc->dtype), fast_deform_grad_filter_workspace(g));
 }
 
 int dk_deformable_sample_depthwise_backward_filter(const dk_conv_desc* desc, const void* out_grad,
@@ -268,42 +273,70 @@ int dk_deformable_sample_depthwise_backward_filter(const dk_conv_desc* desc, con
   const int rc = make_geo(desc, g);
   if (rc != DK_OK) return rc;
   if (!out_grad || !input || !offset || !rotation || !filter_grad) return DK_ERR_NULL_POINTER;
-  const size_t need = generic_grad_filter_workspace(g, desc->dtype);
+  const size_t need = dk_deformable_sample_depthwise_backward_filter_workspace(desc);
   if (need && (!workspace || workspace_bytes < need)) return DK_ERR_WORKSPACE;
   hipStream_t s = static_cast<hipStream_t>(stream);
+  if (g.batch == 0) return DK_OK;
   return by_dtype(desc->dtype, [&]<typename T>() {
+    if constexpr (kHasFast<T>)
+      if (fast_deform_grad_filter<T>(g, in<T>(out_grad), in<T>(input), in<T>(offset), in<T>(rotation),
+                                     out<T>(filter_grad), workspace, s)) return;
     generic_grad_filter<T>(g, true, in<T>(out_grad), in<T>(input), in<T>(offset), in<T>(rotation),
                            out<T>(filter_grad), workspace, s);
   });
 }
 
+size_t dk_deformable_sample_depthwise_backward_offset_workspace(const dk_conv_desc* desc) {
+  Geo g;
+  if (make_geo(desc, g) != DK_OK) return 0;
+  return fast_deform_grad_coord_workspace(g, false);
+}
+
 int dk_deformable_sample_depthwise_backward_offset(const dk_conv_desc* desc, const void* out_grad,
                                                    const void* input, const void* offset,
                                                    const void* rotation, const void* filter,
-                                                   void* offset_grad, void* stream) {
+                                                   void* offset_grad, void* workspace,
+                                                   size_t workspace_bytes, void* stream) {
   Geo g;
   const int rc = make_geo(desc, g);
   if (rc != DK_OK) return rc;
   if (!out_grad || !input || !offset || !rotation || !filter || !offset_grad) return DK_ERR_NULL_POINTER;
+  const size_t need = fast_deform_grad_coord_workspace(g, false);
+  if (need && (!workspace || workspace_bytes < need)) return DK_ERR_WORKSPACE;
   if (g.batch == 0) return DK_OK;
   hipStream_t s = static_cast<hipStream_t>(stream);
   return by_dtype(desc->dtype, [&]<typename T>() {
+    if constexpr (kHasFast<T>)
+      if (need && fast_deform_grad_coord<T>(g, false, in<T>(out_grad), in<T>(input), in<T>(offset), in<T>(rotation),
+                                            in<T>(filter), out<T>(offset_grad), workspace, s)) return;
     generic_grad_offset<T>(g, in<T>(out_grad), in<T>(input), in<T>(offset), in<T>(rotation), in<T>(filter),
                            out<T>(offset_grad), s);
   });
 }
 
+size_t dk_deformable_sample_depthwise_backward_rotation_workspace(const dk_conv_desc* desc) {
+  Geo g;
+  if (make_geo(desc, g) != DK_OK) return 0;
+  return fast_deform_grad_coord_workspace(g, true);
+}
+
 int dk_deformable_sample_depthwise_backward_rotation(const dk_conv_desc* desc, const void* out_grad,
                                                      const void* input, const void* offset,
                                                      const void* rotation, const void* filter,
-                                                     void* rotation_grad, void* stream) {
+                                                     void* rotation_grad, void* workspace,
+                                                     size_t workspace_bytes, void* stream) {
   Geo g;
   const int rc = make_geo(desc, g);
   if (rc != DK_OK) return rc;
   if (!out_grad || !input || !offset || !rotation || !filter || !rotation_grad) return DK_ERR_NULL_POINTER;
+  const size_t need = fast_deform_grad_coord_workspace(g, true);
+  if (need && (!workspace || workspace_bytes < need)) return DK_ERR_WORKSPACE;
   if (g.batch == 0) return DK_OK;
   hipStream_t s = static_cast<hipStream_t>(stream);
   return by_dtype(desc->dtype, [&]<typename T>() {
+    if constexpr (kHasFast<T>)
+      if (need && fast_deform_grad_coord<T>(g, true, in<T>(out_grad), in<T>(input), in<T>(offset), in<T>(rotation),
+                                            in<T>(filter), out<T>(rotation_grad), workspace, s)) return;
     generic_grad_rotation<T>(g, true, in<T>(out_grad), in<T>(input), in<T>(offset), in<T>(rotation),
                              in<T>(filter), out<T>(rotation_grad), s);
   });

@@ -40,9 +40,14 @@ struct ImgTap {
   float lh, lw;
 };
 
-template <typename T, int SH, int SW>
+// Scope coordinates of tap t; (-2, -2), outside every scope band, where the tap samples nothing.
+struct ScopeCoord {
+  float h, w;
+};
+
+template <typename T>
 __device__ __forceinline__ void deform_taps(const Geo& g, const T* off, const T* rot, int n, int grp, int p,
-                                            bool live, int RS, ImgTap (&it)[K9], LiteTap (&st)[K9]) {
+                                            bool live, int RS, ImgTap (&it)[K9], ScopeCoord (&sc)[K9]) {
   const int out_plane = g.out_h * g.out_w;
   const int pc = live ? p : 0;
   const int oh = pc / g.out_w, ow = pc % g.out_w;
@@ -61,9 +66,20 @@ __device__ __forceinline__ void deform_taps(const Geo& g, const T* off, const T*
     it[t].pidx = hit ? (static_cast<int>(hf) + 1) * RS + static_cast<int>(wf) + 1 : 0;
     it[t].lh = hit ? h - hf : 0.f;
     it[t].lw = hit ? w - wf : 0.f;
-    st[t] = make_lite_tap<SH, SW>(scope_coord<float>(f_h, buf_ld(rr, o, rot), g.centre_h),
-                                  scope_coord<float>(f_w, buf_ld(rr, o + step, rot), g.centre_w), hit);
+    const float sh = scope_coord<float>(f_h, buf_ld(rr, o, rot), g.centre_h);
+    const float sw = scope_coord<float>(f_w, buf_ld(rr, o + step, rot), g.centre_w);
+    sc[t].h = hit ? sh : -2.f;
+    sc[t].w = hit ? sw : -2.f;
   }
+}
+
+template <typename T, int SH, int SW>
+__device__ __forceinline__ void deform_taps(const Geo& g, const T* off, const T* rot, int n, int grp, int p,
+                                            bool live, int RS, ImgTap (&it)[K9], LiteTap (&st)[K9]) {
+  ScopeCoord sc[K9];
+  deform_taps<T>(g, off, rot, n, grp, p, live, RS, it, sc);
+#pragma unroll
+  for (int t = 0; t < K9; ++t) st[t] = make_lite_tap<SH, SW>(sc[t].h, sc[t].w, true);
 }
 
 // The four corners of a sample in the padded plane, and their bilinear combination.
@@ -187,6 +203,343 @@ __global__ __launch_bounds__(kDBlock, 2) void deform_forward_kernel(
   }
 }
 
+
+// ---------------------------------------------------------------------------
+// grad offset / grad rotation: the lane owns output pixel p and sums over the channels of its
+// chunk; one fp32 partial per chunk goes to the workspace and reduce_partials_kernel adds the
+// chunks in order.
+//   rotation (K.cu:1410-1508): with the scope block in difference form the derivatives of the
+//     scope read are c + lw * d and b + lh * d, so the lane accumulates
+//     S_{b,c,d}[t] = sum_c sample_t[c] * gout[c] * {b, c, d}[c] and combines at the end;
+//   offset (K.cu:1147-1243, get_coordinate_weight K.cu:231-268): d sample / dh =
+//     (1 - lw) (bl - tl) + lw (br - tr), d sample / dw = (1 - lh) (tr - tl) + lh (br - bl), the
+//     zero padding standing for the reference's per-corner range tests; times gout * B(Wt[c]).
+// partial layout: [part][image (* group for rotation)][2 t + dir][pixel], part = chunk for
+// rotation and group * chunks + chunk for offset (which sums over the groups as well).
+// ---------------------------------------------------------------------------
+template <typename T, int SH, int SW, int NPASS, bool ROTATION>
+__global__ __launch_bounds__(kDBlock, 2) void deform_grad_coord_kernel(
+    Geo g, const T* __restrict__ gout, const T* __restrict__ x, const T* __restrict__ off,
+    const T* __restrict__ rot, const T* __restrict__ filter, float* __restrict__ partial,
+    int ch_per_block, int shift) {
+  using Tb = WideTable<SH, SW>;
+  extern __shared__ __align__(16) float lds[];
+  const int H = g.in_h, W = g.in_w, RS = W + 2;
+  const int PS = ((H + 2) * RS + 3) & ~3;
+  float* planes = lds;
+  float* tbl = lds + 2 * PS;
+
+  const int cpg = g.channel / g.groups;
+  const int out_plane = g.out_h * g.out_w, in_plane = H * W;
+  const int chunks = ceil_div(cpg, ch_per_block);
+  const BlockId b = decode_block(g, ceil_div(out_plane, kDBlock), chunks);
+  if (!b.valid) return;
+  const int j0 = b.chunk * ch_per_block;
+  const int nch = min(ch_per_block, cpg - j0);
+
+  for (int e = threadIdx.x; e < 2 * PS; e += kDBlock) planes[e] = 0.f;
+  stage_wide_tables<T, SH, SW>(tbl, filter, g.channel, b.grp + g.groups * j0, g.groups, nch);
+
+  const int p = b.tile * kDBlock + threadIdx.x;
+  const bool live = p < out_plane;
+  ImgTap it[K9];
+  LiteTap st[K9];
+  deform_taps<T, SH, SW>(g, off, rot, b.n, b.grp, p, live, RS, it, st);
+
+  const size_t chan0 = (size_t)b.n * g.channel + b.grp + (size_t)g.groups * j0;
+  const T* xp = x + chan0 * in_plane;
+  const T* gp = gout + chan0 * out_plane;
+  const size_t x_step = (size_t)g.groups * in_plane, g_step = (size_t)g.groups * out_plane;
+  const unsigned goff = live ? (unsigned)p * (unsigned)sizeof(T) : kOutOfRange;
+
+  float s0[K9], s1[K9], s2[K9];
+#pragma unroll
+  for (int t = 0; t < K9; ++t) s0[t] = s1[t] = s2[t] = 0.f;
+
+  PlaneStage<T, NPASS> stage;
+  stage.load(xp, true, H, W, shift);
+  float gv = buf_ld(plane_rsrc(gp, out_plane), goff, gout);
+  __syncthreads();
+  stage.store(planes, H, W, shift);
+  __syncthreads();
+  for (int j = 0; j < nch; ++j) {
+    float gv_next = 0.f;
+    if (j + 1 < nch) {
+      stage.load(xp + (size_t)(j + 1) * x_step, true, H, W, shift);
+      gv_next = buf_ld(plane_rsrc(gp + (size_t)(j + 1) * g_step, out_plane), goff, gout);
+    }
+    const float* pl = planes + (j & 1) * PS;
+    const float* tb = tbl + j * Tb::SIZE;
+#pragma unroll
+    for (int t = 0; t < K9; ++t) {
+      const Corners cq = read_corners(pl, it[t].pidx, RS);
+      if (ROTATION) {
+        const float ps = lerp2(cq, it[t].lh, it[t].lw) * gv;
+        const float4 q = lds_read4(tb + st[t].cell);
+        s0[t] = fmaf(ps, q.y, s0[t]);
+        s1[t] = fmaf(ps, q.z, s1[t]);
+        s2[t] = fmaf(ps, q.w, s2[t]);
+      } else {
+        const float4 q = *reinterpret_cast<const float4*>(tb + st[t].cell);
+        const float gw = gv * lite_weight(st[t], q);
+        const float ca = cq.c - cq.a, ba = cq.b - cq.a;
+        const float dh = fmaf(it[t].lw, (cq.d - cq.b) - ca, ca);
+        const float dw = fmaf(it[t].lh, (cq.d - cq.c) - ba, ba);
+        s0[t] = fmaf(dh, gw, s0[t]);
+        s1[t] = fmaf(dw, gw, s1[t]);
+      }
+    }
+    gv = gv_next;
+    if (j + 1 < nch) stage.store(planes + ((j + 1) & 1) * PS, H, W, shift);
+    __syncthreads();
+  }
+
+  if (live) {
+    const size_t part = ROTATION ? (size_t)b.chunk : (size_t)b.grp * chunks + b.chunk;
+    const size_t img = ROTATION ? (size_t)(b.n * g.groups + b.grp) : (size_t)b.n;
+    const size_t imgs = ROTATION ? (size_t)g.batch * g.groups : (size_t)g.batch;
+    float* dst = partial + ((part * imgs + img) * (K9 * 2)) * out_plane + p;
+#pragma unroll
+    for (int t = 0; t < K9; ++t) {
+      const float dh = ROTATION ? fmaf(st[t].lw, s2[t], s1[t]) : s0[t];
+      const float dw = ROTATION ? fmaf(st[t].lh, s2[t], s0[t]) : s1[t];
+      dst[(size_t)(2 * t) * out_plane] = dh;
+      dst[(size_t)(2 * t + 1) * out_plane] = dw;
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------
+// grad input (K.cu:704-795): every (pixel, tap, channel) adds gout * B(Wt[c]) * corner weight to
+// the four input elements around its sample -- a scatter with data-dependent targets, done by
+// the reference with global float atomics.  LDS float atomics are slow on gfx950 (about 190 clk
+// per wave instruction) but 64-bit integer ones are not (about 15 clk), so the workgroup, which
+// owns the whole output plane of its channels, accumulates each channel's input-gradient plane
+// in LDS in 64-bit FIXED POINT: a contribution v becomes round(v * 2^s) through the
+// "add 1.5 * 2^52 in double" trick and ds_add_u64 adds it.  s is chosen per channel from
+// max|gout| (over the tensor, computed by a small kernel into the workspace) times max|Wt[c]| so
+// that a term stays below 2^44 and the plane's sum below 2^62: the grid is 2^-44 of the largest
+// possible term, far below fp32 rounding, and the sum is exact on that grid and independent of
+// the order of the additions (run-to-run reproducible, which float atomics are not).
+// Corners outside the image fall on the plane's zero padding, which is never read back.
+// One block per (image, group, channel chunk); blockDim = output pixels rounded up to a wave.
+// ---------------------------------------------------------------------------
+template <typename T>
+__global__ void absmax_kernel(const T* __restrict__ p, long n, unsigned* __restrict__ out) {
+  float m = 0.f;
+  for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (long)gridDim.x * blockDim.x)
+    m = fmaxf(m, fabsf(ld(p + i)));
+  for (int s = 32; s > 0; s >>= 1) m = fmaxf(m, __shfl_xor(m, s));
+  if ((threadIdx.x & 63) == 0) atomicMax(out, __float_as_uint(m));  // non-negative floats order like their bits
+}
+__global__ void clear_word_kernel(unsigned* p) { *p = 0u; }
+
+template <typename T, int SH, int SW>
+__global__ __launch_bounds__(1024) void deform_grad_input_kernel(
+    Geo g, const T* __restrict__ gout, const T* __restrict__ off, const T* __restrict__ rot,
+    const T* __restrict__ filter, T* __restrict__ gin, const unsigned* __restrict__ gmax_bits,
+    int ch_per_block, int shift) {
+  using Tb = WideTable<SH, SW>;
+  extern __shared__ __align__(16) float lds[];
+  const int H = g.in_h, W = g.in_w, RS = W + 2;
+  const int PS = ((H + 2) * RS + 3) & ~3;
+  unsigned long long* planes = reinterpret_cast<unsigned long long*>(lds);  // [2][PS]
+  float* tbl = lds + 4 * PS;                                                // [ch_per_block][Tb::SIZE]
+  float* wmax = tbl + ch_per_block * Tb::SIZE;                              // [ch_per_block]
+
+  const int cpg = g.channel / g.groups;
+  const int out_plane = g.out_h * g.out_w, in_plane = H * W;
+  const BlockId b = decode_block(g, 1, ceil_div(cpg, ch_per_block));
+  if (!b.valid) return;
+  const int j0 = b.chunk * ch_per_block;
+  const int nch = min(ch_per_block, cpg - j0);
+
+  for (int e = threadIdx.x; e < 2 * PS; e += blockDim.x) planes[e] = 0ull;
+  stage_wide_tables<T, SH, SW>(tbl, filter, g.channel, b.grp + g.groups * j0, g.groups, nch);
+  for (int j = threadIdx.x; j < nch; j += blockDim.x) {
+    const T* f = filter + (size_t)(b.grp + g.groups * (j0 + j)) * (SH * SW);
+    float m = 0.f;
+    for (int e = 0; e < SH * SW; ++e) m = fmaxf(m, fabsf(ld(f + e)));
+    wmax[j] = m;
+  }
+
+  const int p = threadIdx.x;
+  const bool live = p < out_plane;
+  ImgTap it[K9];
+  LiteTap st[K9];
+  unsigned hits = 0;  // taps that sample the image inside the scope band: the others add nothing
+  {
+    ScopeCoord sc[K9];
+    deform_taps<T>(g, off, rot, b.n, b.grp, p, live, RS, it, sc);
+#pragma unroll
+    for (int t = 0; t < K9; ++t) {
+      st[t] = make_lite_tap<SH, SW>(sc[t].h, sc[t].w, true);
+      const bool in = (sc[t].h > -1.f) && (sc[t].w > -1.f) && (sc[t].h < float(SH)) && (sc[t].w < float(SW));
+      hits |= in ? (1u << t) : 0u;
+    }
+  }
+
+  const size_t chan0 = (size_t)b.n * g.channel + b.grp + (size_t)g.groups * j0;
+  const T* gp = gout + chan0 * out_plane;
+  T* ip = gin + chan0 * in_plane;
+  const size_t g_step = (size_t)g.groups * out_plane, i_step = (size_t)g.groups * in_plane;
+  const unsigned goff = live ? (unsigned)p * (unsigned)sizeof(T) : kOutOfRange;
+  const float gmax = __uint_as_float(*gmax_bits);
+  const int col = threadIdx.x & ((1 << shift) - 1), sub = threadIdx.x >> shift;
+  const int rpp = (int)blockDim.x >> shift;
+
+  float gv = buf_ld(plane_rsrc(gp, out_plane), goff, gout);
+  __syncthreads();
+  for (int j = 0; j < nch; ++j) {
+    float gv_next = 0.f;
+    if (j + 1 < nch) gv_next = buf_ld(plane_rsrc(gp + (size_t)(j + 1) * g_step, out_plane), goff, gout);
+    unsigned long long* pl = planes + (j & 1) * PS;
+    const float* tb = tbl + j * Tb::SIZE;
+    // a term is at most gmax * wmax < 2^e: scale 2^(44 - e)
+    int e;
+    (void)frexpf(gmax * wmax[j], &e);
+    const double scale = ldexp(1.0, 44 - e), unscale = ldexp(1.0, e - 44);
+    constexpr double kMagic = 6755399441055744.0;  // 1.5 * 2^52: the sum's low mantissa bits are the rounded integer
+#pragma unroll
+    for (int t = 0; t < K9; ++t) {
+      if (hits >> t & 1u) {
+        const float4 q = *reinterpret_cast<const float4*>(tb + st[t].cell);
+        const float gw = gv * lite_weight(st[t], q);
+        const float lh = it[t].lh, lw = it[t].lw, hh = 1.f - lh, hw = 1.f - lw;
+        const float term[4] = {hh * hw * gw, hh * lw * gw, lh * hw * gw, lh * lw * gw};  // K.cu:776-789
+        const int at[4] = {it[t].pidx, it[t].pidx + 1, it[t].pidx + RS, it[t].pidx + RS + 1};
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+          const double d = fma((double)term[k], scale, kMagic);
+          // bits(d) - bits(kMagic): the magic's low word is 0, so only the high word changes
+          const unsigned long long fixed = (unsigned long long)__double_as_longlong(d) - 0x4338000000000000ull;
+          atomicAdd(pl + at[k], fixed);
+        }
+      }
+    }
+    gv = gv_next;
+    __syncthreads();
+    // read the channel's plane back, clear it for the channel after next
+    T* dst = ip + (size_t)j * i_step;
+    for (int row = sub; row < H; row += rpp) {
+      if (col < W) {
+        unsigned long long* cell = pl + (row + 1) * RS + 1 + col;
+        const long long v = (long long)*cell;
+        *cell = 0ull;
+        dk::st(dst + row * W + col, (float)((double)v * unscale));
+      }
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------
+// grad filter (K.cu:1002-1097): gW[c][i][j] = sum over (image, pixel, tap) of
+// sample_t * gout * hat(sh_t - i) * hat(sw_t - j).  As in the local operator the sum is kept
+// dense and in registers (per tap the lane holds the SH + SW hat weights, per channel it adds
+// ps * a_i * b_j into SH * SW accumulators); after each channel the 64 lanes are summed with DPP
+// wave reductions and lane `cell` adds the wave's total to a per-wave LDS accumulator.  One
+// partial per (image, tile) workgroup; reduce_partials_kernel adds them in order.
+// ---------------------------------------------------------------------------
+template <typename T, int SH, int SW, int NPASS>
+__global__ __launch_bounds__(kDBlock, 2) void deform_grad_filter_kernel(
+    Geo g, const T* __restrict__ gout, const T* __restrict__ x, const T* __restrict__ off,
+    const T* __restrict__ rot, float* __restrict__ partial, int ch_per_block, int shift) {
+  constexpr int CELLS = SH * SW;
+  constexpr int kWaves = kDBlock / 64;
+  extern __shared__ __align__(16) float lds[];
+  const int H = g.in_h, W = g.in_w, RS = W + 2;
+  const int PS = ((H + 2) * RS + 3) & ~3;
+  float* planes = lds;
+  float* wacc = lds + 2 * PS;  // [kWaves][ch_per_block][CELLS]
+
+  const int cpg = g.channel / g.groups;
+  const int out_plane = g.out_h * g.out_w, in_plane = H * W;
+  const int tiles = ceil_div(out_plane, kDBlock);
+  const BlockId b = decode_block(g, tiles, ceil_div(cpg, ch_per_block));
+  if (!b.valid) return;
+  const int j0 = b.chunk * ch_per_block;
+  const int nch = min(ch_per_block, cpg - j0);
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+
+  for (int e = threadIdx.x; e < 2 * PS; e += kDBlock) planes[e] = 0.f;
+  for (int e = threadIdx.x; e < kWaves * ch_per_block * CELLS; e += kDBlock) wacc[e] = 0.f;
+
+  const int p = b.tile * kDBlock + threadIdx.x;
+  const bool live = p < out_plane;
+  ImgTap it[K9];
+  float ah[K9][SH], bw[K9][SW];
+  {
+    ScopeCoord sc[K9];
+    deform_taps<T>(g, off, rot, b.n, b.grp, p, live, RS, it, sc);
+#pragma unroll
+    for (int t = 0; t < K9; ++t) {
+      // outside the open box (-1, S) every hat below is 0 by itself, NaN coordinates excepted
+      const bool in = (sc[t].h > -1.f) && (sc[t].w > -1.f) && (sc[t].h < float(SH)) && (sc[t].w < float(SW));
+#pragma unroll
+      for (int i = 0; i < SH; ++i) ah[t][i] = in ? fmaxf(1.f - fabsf(sc[t].h - float(i)), 0.f) : 0.f;
+#pragma unroll
+      for (int i = 0; i < SW; ++i) bw[t][i] = in ? fmaxf(1.f - fabsf(sc[t].w - float(i)), 0.f) : 0.f;
+    }
+  }
+
+  const size_t chan0 = (size_t)b.n * g.channel + b.grp + (size_t)g.groups * j0;
+  const T* xp = x + chan0 * in_plane;
+  const T* gp = gout + chan0 * out_plane;
+  const size_t x_step = (size_t)g.groups * in_plane, g_step = (size_t)g.groups * out_plane;
+  const unsigned goff = live ? (unsigned)p * (unsigned)sizeof(T) : kOutOfRange;
+
+  PlaneStage<T, NPASS> stage;
+  stage.load(xp, true, H, W, shift);
+  float gv = buf_ld(plane_rsrc(gp, out_plane), goff, gout);
+  __syncthreads();
+  stage.store(planes, H, W, shift);
+  __syncthreads();
+  for (int j = 0; j < nch; ++j) {
+    float gv_next = 0.f;
+    if (j + 1 < nch) {
+      stage.load(xp + (size_t)(j + 1) * x_step, true, H, W, shift);
+      gv_next = buf_ld(plane_rsrc(gp + (size_t)(j + 1) * g_step, out_plane), goff, gout);
+    }
+    const float* pl = planes + (j & 1) * PS;
+    float acc[SH][SW];
+#pragma unroll
+    for (int i = 0; i < SH; ++i)
+#pragma unroll
+      for (int k = 0; k < SW; ++k) acc[i][k] = 0.f;
+#pragma unroll
+    for (int t = 0; t < K9; ++t) {
+      const float ps = lerp2(read_corners(pl, it[t].pidx, RS), it[t].lh, it[t].lw) * gv;
+#pragma unroll
+      for (int i = 0; i < SH; ++i) {
+        const float a = ah[t][i] * ps;
+#pragma unroll
+        for (int k = 0; k < SW; ++k) acc[i][k] = fmaf(a, bw[t][k], acc[i][k]);
+      }
+    }
+    float mine = 0.f;
+#pragma unroll
+    for (int i = 0; i < SH; ++i)
+#pragma unroll
+      for (int k = 0; k < SW; ++k) {
+        const float s = wave_sum(acc[i][k]);
+        if (lane == i * SW + k) mine = s;
+      }
+    if (lane < CELLS) wacc[(wave * ch_per_block + j) * CELLS + lane] += mine;
+    gv = gv_next;
+    if (j + 1 < nch) stage.store(planes + ((j + 1) & 1) * PS, H, W, shift);
+    __syncthreads();
+  }
+
+  const size_t part = (size_t)b.n * tiles + b.tile;
+  for (int e = threadIdx.x; e < nch * CELLS; e += kDBlock) {
+    float s = 0.f;
+#pragma unroll
+    for (int w = 0; w < kWaves; ++w) s += wacc[w * ch_per_block * CELLS + e];
+    const int c = b.grp + g.groups * (j0 + e / CELLS);
+    partial[(part * g.channel + c) * CELLS + e % CELLS] = s;
+  }
+}
+
 // ---------------------------------------------------------------------------
 // host side
 // ---------------------------------------------------------------------------
@@ -252,6 +605,81 @@ bool run_deform_forward(const Geo& g, const T* x, const T* off, const T* rot, co
   return true;
 }
 
+
+template <typename T, int SH, int SW>
+bool run_deform_grad_coord(const Geo& g, bool rotation, const T* gout, const T* x, const T* off, const T* rot,
+                           const T* filter, T* result, float* ws, hipStream_t stream) {
+  const DeformPlan d = deform_plan(g, WideTable<SH, SW>::SIZE, 2, kDBlock);
+  if (!d.ok) return false;
+  const unsigned grid = (unsigned)xcd_grid_size((long)d.tiles * d.chunks * g.batch * g.groups);
+#define DK_LAUNCH(NP, ROT)                                                                          \
+  deform_grad_coord_kernel<T, SH, SW, NP, ROT><<<grid, kDBlock, d.lds, stream>>>(g, gout, x, off, rot, filter, ws, \
+                                                                                 d.per, d.shift)
+  if (rotation) {
+    if (d.npass == 4) DK_LAUNCH(4, true);
+    else if (d.npass == 8) DK_LAUNCH(8, true);
+    else DK_LAUNCH(16, true);
+  } else {
+    if (d.npass == 4) DK_LAUNCH(4, false);
+    else if (d.npass == 8) DK_LAUNCH(8, false);
+    else DK_LAUNCH(16, false);
+  }
+#undef DK_LAUNCH
+  const int plane18 = 18 * g.out_h * g.out_w;
+  if (rotation)
+    launch_reduce_partials<float, T>(ws, d.chunks, g.batch * g.groups * plane18, result, stream);
+  else
+    launch_reduce_partials<float, T>(ws, d.chunks * g.groups, g.batch * plane18, result, stream);
+  return true;
+}
+
+// blockDim of the grad-input kernel: it owns a whole output plane
+int grad_input_block(const Geo& g) { return ceil_div(g.out_h * g.out_w, 64) * 64; }
+
+template <int SH, int SW>
+DeformPlan grad_input_plan(const Geo& g) {
+  DeformPlan d{};
+  d.ok = false;
+  if (g.out_h * g.out_w > 1024) return d;
+  // 4 floats of LDS per plane element (two 64-bit planes), one more float per channel for max|Wt[c]|
+  return deform_plan(g, WideTable<SH, SW>::SIZE + 1, 4, grad_input_block(g));
+}
+
+template <typename T, int SH, int SW>
+bool run_deform_grad_input(const Geo& g, const T* gout, const T* off, const T* rot, const T* filter, T* gin,
+                           void* ws, hipStream_t stream) {
+  const DeformPlan d = grad_input_plan<SH, SW>(g);
+  if (!d.ok) return false;
+  unsigned* gmax = static_cast<unsigned*>(ws);
+  clear_word_kernel<<<1, 1, 0, stream>>>(gmax);
+  const long n = (long)g.batch * g.channel * g.out_h * g.out_w;
+  absmax_kernel<T><<<(unsigned)std::min<long>(1024, (n + 255) / 256), 256, 0, stream>>>(gout, n, gmax);
+  const unsigned grid = (unsigned)xcd_grid_size((long)d.chunks * g.batch * g.groups);
+  deform_grad_input_kernel<T, SH, SW><<<grid, grad_input_block(g), d.lds, stream>>>(g, gout, off, rot, filter, gin, gmax,
+                                                                                   d.per, d.shift);
+  return true;
+}
+
+template <typename T, int SH, int SW>
+bool run_deform_grad_filter(const Geo& g, const T* gout, const T* x, const T* off, const T* rot, T* gfilter,
+                            float* ws, hipStream_t stream) {
+  if constexpr (SH * SW > 16) {
+    return false;  // 25 dense accumulators and 90 hat weights per lane do not fit the register budget
+  } else {
+    const DeformPlan d = deform_plan(g, (kDBlock / 64) * SH * SW, 2, kDBlock);
+    if (!d.ok) return false;
+    const unsigned grid = (unsigned)xcd_grid_size((long)d.tiles * d.chunks * g.batch * g.groups);
+#define DK_LAUNCH(NP) \
+  deform_grad_filter_kernel<T, SH, SW, NP><<<grid, kDBlock, d.lds, stream>>>(g, gout, x, off, rot, ws, d.per, d.shift)
+    if (d.npass == 4) DK_LAUNCH(4);
+    else if (d.npass == 8) DK_LAUNCH(8);
+    else DK_LAUNCH(16);
+#undef DK_LAUNCH
+    launch_reduce_partials<float, T>(ws, g.batch * d.tiles, g.channel * SH * SW, gfilter, stream);
+    return true;
+  }
+}
+
 }  // namespace
 
 #define DK_DISPATCH_SCOPE(g, CALL)    \
@@ -268,8 +696,57 @@ bool fast_deform_forward(const Geo& g, const T* x, const T* off, const T* rot, c
 #undef CALL
 }
 
+
+template <typename T>
+bool fast_deform_grad_coord(const Geo& g, bool rotation, const T* gout, const T* x, const T* off, const T* rot,
+                            const T* filter, T* result, void* ws, hipStream_t stream) {
+#define CALL(SH, SW) \
+  run_deform_grad_coord<T, SH, SW>(g, rotation, gout, x, off, rot, filter, result, static_cast<float*>(ws), stream)
+  DK_DISPATCH_SCOPE(g, CALL)
+#undef CALL
+}
+
+size_t fast_deform_grad_coord_workspace(const Geo& g, bool rotation) {
+  const int table = g.scope_h == 3 ? WideTable<3, 3>::SIZE : g.scope_h == 4 ? WideTable<4, 4>::SIZE : WideTable<5, 5>::SIZE;
+  const DeformPlan d = deform_plan(g, table, 2, kDBlock);
+  if (!d.ok) return 0;
+  (void)rotation;  // both lay out chunks * groups * batch planes of 18 * out pixels
+  return (size_t)d.chunks * g.groups * g.batch * 18 * g.out_h * g.out_w * sizeof(float);
+}
+
+template <typename T>
+bool fast_deform_grad_input(const Geo& g, const T* gout, const T* off, const T* rot, const T* filter, T* gin,
+                            void* ws, hipStream_t stream) {
+#define CALL(SH, SW) run_deform_grad_input<T, SH, SW>(g, gout, off, rot, filter, gin, ws, stream)
+  DK_DISPATCH_SCOPE(g, CALL)
+#undef CALL
+}
+
+size_t fast_deform_grad_input_workspace(const Geo& g) {
+  (void)g;
+  return 256;  // one word: max |gout|
+}
+
+template <typename T>
+bool fast_deform_grad_filter(const Geo& g, const T* gout, const T* x, const T* off, const T* rot, T* gfilter,
+                             void* ws, hipStream_t stream) {
+#define CALL(SH, SW) run_deform_grad_filter<T, SH, SW>(g, gout, x, off, rot, gfilter, static_cast<float*>(ws), stream)
+  DK_DISPATCH_SCOPE(g, CALL)
+#undef CALL
+}
+
+size_t fast_deform_grad_filter_workspace(const Geo& g) {
+  return (size_t)g.batch * ceil_div(g.out_h * g.out_w, kDBlock) * g.channel * g.scope_h * g.scope_w * sizeof(float);
+}
+
 #define DK_INSTANTIATE(T)                                                                              \
-  template bool fast_deform_forward<T>(const Geo&, const T*, const T*, const T*, const T*, T*, hipStream_t);
+  template bool fast_deform_forward<T>(const Geo&, const T*, const T*, const T*, const T*, T*, hipStream_t);      \
+  template bool fast_deform_grad_coord<T>(const Geo&, bool, const T*, const T*, const T*, const T*, const T*, T*,  \
+                                          void*, hipStream_t);                                                     \
+  template bool fast_deform_grad_input<T>(const Geo&, const T*, const T*, const T*, const T*, T*, void*,           \
+                                          hipStream_t);                                                            \
+  template bool fast_deform_grad_filter<T>(const Geo&, const T*, const T*, const T*, const T*, T*, void*,          \
+                                           hipStream_t);
 DK_INSTANTIATE(float)
 DK_INSTANTIATE(__half)
 DK_INSTANTIATE(bf16_t)

@@ -28,6 +28,19 @@ bool fast_local_grad_filter(const Geo& g, const T* gout, const T* x, const T* ro
 template <typename T>
 bool fast_deform_forward(const Geo& g, const T* x, const T* off, const T* rot, const T* filter, T* out,
                          hipStream_t stream);
+size_t fast_deform_grad_input_workspace(const Geo& g);
+template <typename T>
+bool fast_deform_grad_input(const Geo& g, const T* gout, const T* off, const T* rot, const T* filter, T* gin,
+                            void* ws, hipStream_t stream);
+// rotation = false: gradient w.r.t. the image-space offsets
+size_t fast_deform_grad_coord_workspace(const Geo& g, bool rotation);
+template <typename T>
+bool fast_deform_grad_coord(const Geo& g, bool rotation, const T* gout, const T* x, const T* off, const T* rot,
+                            const T* filter, T* result, void* ws, hipStream_t stream);
+size_t fast_deform_grad_filter_workspace(const Geo& g);
+template <typename T>
+bool fast_deform_grad_filter(const Geo& g, const T* gout, const T* x, const T* off, const T* rot, T* gfilter,
+                             void* ws, hipStream_t stream);
 
 // ---- generic path (dk_generic.hip): any geometry, all four dtypes, local and deformable
 template <typename T>

@@ -172,14 +172,18 @@ class DeformableSampleDepthwiseFunction(Function):
                     p(ws), nbytes, s), "deform_sample_depthwise backward_data")
             if ctx.needs_input_grad[1]:
                 grad_offset = torch.empty_like(offset)
+                ws, nbytes = _lib.workspace(
+                    L.dk_deformable_sample_depthwise_backward_offset_workspace(desc), input.device)
                 _lib.check(L.dk_deformable_sample_depthwise_backward_offset(
                     desc, p(grad_output), p(input), p(offset), p(rotation), p(weight),
-                    p(grad_offset), s), "deform_sample_depthwise backward_offset")
+                    p(grad_offset), p(ws), nbytes, s), "deform_sample_depthwise backward_offset")
             if ctx.needs_input_grad[2]:
                 grad_rotation = torch.empty_like(rotation)
+                ws, nbytes = _lib.workspace(
+                    L.dk_deformable_sample_depthwise_backward_rotation_workspace(desc), input.device)
                 _lib.check(L.dk_deformable_sample_depthwise_backward_rotation(
                     desc, p(grad_output), p(input), p(offset), p(rotation), p(weight),
-                    p(grad_rotation), s), "deform_sample_depthwise backward_rotation")
+                    p(grad_rotation), p(ws), nbytes, s), "deform_sample_depthwise backward_rotation")
             if ctx.needs_input_grad[3]:
                 grad_weight = torch.empty_like(weight)
                 ws, nbytes = _lib.workspace(

@@ -137,17 +137,23 @@ int dk_deformable_sample_depthwise_backward_filter(const dk_conv_desc *desc, con
                                                    void *workspace, size_t workspace_bytes,
                                                    void *stream);
 
-/* deformable_sample_depthwise_backward_offset_cuda (filter_sample_depthwise_cuda.cpp:416-476). */
+/* deformable_sample_depthwise_backward_offset_cuda (filter_sample_depthwise_cuda.cpp:416-476).
+ * The workspace holds per-channel-chunk partial sums that are added in a fixed order. */
+size_t dk_deformable_sample_depthwise_backward_offset_workspace(const dk_conv_desc *desc);
 int dk_deformable_sample_depthwise_backward_offset(const dk_conv_desc *desc, const void *out_grad,
                                                    const void *input, const void *offset,
                                                    const void *rotation, const void *filter,
-                                                   void *offset_grad, void *stream);
+                                                   void *offset_grad, void *workspace,
+                                                   size_t workspace_bytes, void *stream);
 
-/* deformable_sample_depthwise_backward_rotation_cuda (filter_sample_depthwise_cuda.cpp:478-538). */
+/* deformable_sample_depthwise_backward_rotation_cuda (filter_sample_depthwise_cuda.cpp:478-538).
+ * Workspace as for the offset gradient. */
+size_t dk_deformable_sample_depthwise_backward_rotation_workspace(const dk_conv_desc *desc);
 int dk_deformable_sample_depthwise_backward_rotation(const dk_conv_desc *desc,
                                                      const void *out_grad, const void *input,
                                                      const void *offset, const void *rotation,
                                                      const void *filter, void *rotation_grad,
+                                                     void *workspace, size_t workspace_bytes,
                                                      void *stream);
 
 /* ---- N-d linear sample -------------------------------------------------------

@@ -24,6 +24,10 @@ CASES = [
     (1, 8, 12, 12, 3, (3, 3), 1, 1, 1, 1, 0.0, 1.5),      # DeformConv2d: scope == kernel, zero rotation
     (2, 6, 8, 8, (2, 3), (4, 5), (1, 2), (0, 1), 1, 3, 0.7, 1.0),
     (1, 3, 6, 5, 1, (2, 2), 1, 0, 1, 1, 0.6, 3.0),
+    (1, 20, 24, 24, 3, (4, 4), 1, 1, 1, 2, 0.7, 2.0),     # 576 output pixels: three pixel tiles, two groups
+    (1, 6, 33, 60, 3, (5, 5), 1, 1, 1, 1, 1.0, 2.5),      # wide plane (16 staging passes), scope 5, > 1024 output pixels
+    (2, 80, 10, 10, 3, (3, 3), 1, 1, 1, 1, 0.8, 1.0),     # many channels: several channel chunks per image
+    (1, 8, 20, 18, 3, (4, 4), 2, 1, 1, 1, 0.5, 6.0),      # large offsets: many samples outside the image
 ]
 NAMES = ("forward", "grad input", "grad offset", "grad rotation", "grad filter")
 
