@@ -60,10 +60,17 @@ struct Geo {
 // `f + r + (scope - k) / 2.0`: int + scalar_t in scalar_t, then + double in
 // double, rounded to scalar_t on assignment.  Reproduced operation by
 // operation so the floor below lands on the same cell as the reference's.
+// For float the detour through double is a single correctly rounded float
+// addition: the centre is a multiple of 0.5, so float(t) + centre is exact in
+// double (or leaves t unchanged when t is huge) and its rounding to float is
+// what the float addition returns.
 template <typename CT>
 __device__ __forceinline__ CT scope_coord(int f, CT r, double centre) {
   CT t = static_cast<CT>(f) + r;
-  return static_cast<CT>(static_cast<double>(t) + centre);
+  if constexpr (sizeof(CT) == 4)
+    return t + static_cast<CT>(centre);
+  else
+    return static_cast<CT>(static_cast<double>(t) + centre);
 }
 
 // ---------------------------------------------------------------------------

@@ -377,6 +377,8 @@ __global__ __launch_bounds__(kBlock, 2) void local_grad_rotation_kernel(
 #pragma unroll
   for (int t = 0; t < K; ++t) sb[t] = sc[t] = sd[t] = 0.f;
 
+  // ch_per_pass + 1 tables: the spare one is read, times zero, by the odd channel out of a pair
+  for (int e = threadIdx.x; e < (ch_per_pass + 1) * Tb::SIZE; e += kBlock) tbl[e] = 0.f;
   for (int j0 = 0; j0 < cpg; j0 += ch_per_pass) {
     const int nch = min(ch_per_pass, cpg - j0);
     __syncthreads();
@@ -396,7 +398,8 @@ __global__ __launch_bounds__(kBlock, 2) void local_grad_rotation_kernel(
       for (int t = 0; t < NLOAD; ++t) xv[s][t] = buf_ld(rx, soff[t], x);
     };
     auto accumulate = [&](int s, int j) {
-      const float* tb = tbl + min(j, nch - 1) * Tb::SIZE;  // j >= nch only with zero inputs
+      // j == nch happens (odd nch) with zero inputs: that table is a stale or the zeroed spare one
+      const float* tb = tbl + j * Tb::SIZE;
 #pragma unroll
       for (int t = 0; t < K; ++t) {
         float xt;
@@ -987,7 +990,7 @@ bool run_grad_rotation(const Geo& g, const T* gout, const T* x, const T* rot, co
   using Tb = WideTable<SH, SW>;
   const int cpg = g.channel / g.groups;
   const int per = cpg < 36 ? cpg : 36;  // channels staged per pass
-  const size_t lds = (size_t)per * Tb::SIZE * sizeof(float);
+  const size_t lds = (size_t)(per + 1) * Tb::SIZE * sizeof(float);
   if (same_width_geometry(g)) {
     const unsigned grid = (unsigned)xcd_grid_size((long)ceil_div(g.out_h * g.out_w, kRowPix) * g.batch * g.groups);
     local_grad_rotation_kernel<T, 3, 3, SH, SW, true><<<grid, kBlock, lds, stream>>>(g, gout, x, rot, filter, grot, per);
