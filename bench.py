@@ -122,7 +122,7 @@ def main():
     gw = torch.empty_like(wg)
     L = _lib.lib()
     desc = _lib.conv_desc(xg, wg, cfg["kernel_size"], cfg["stride"], cfg["padding"], cfg["dilation"], groups)
-    ws, ws_bytes = _lib.workspace(L.dk_sample_depthwise_backward_filter_workspace(desc), dev)
+    ws, ws_bytes = _lib.workspace(L.dk_sample_depthwise_backward_workspace(desc), dev)
     P = _lib.ptr
 
     def cur():  # resolved at call time, so launches follow a graph capture's stream
@@ -135,7 +135,7 @@ def main():
         _lib.check(L.dk_sample_depthwise_backward_data(desc, P(gg), P(rg), P(wg), P(gin), cur()), "grad_input")
 
     def k_grad_rotation():
-        _lib.check(L.dk_sample_depthwise_backward_rotation(desc, P(gg), P(xg), P(rg), P(wg), P(grot), cur()),
+        _lib.check(L.dk_sample_depthwise_backward_rotation(desc, P(gg), P(xg), P(rg), P(wg), P(grot), P(ws), ws_bytes, cur()),
                    "grad_rotation")
 
     def k_grad_filter():

@@ -169,25 +169,37 @@ int dk_sample_depthwise_backward_filter(const dk_conv_desc* desc, const void* ou
   });
 }
 
+size_t dk_sample_depthwise_backward_rotation_workspace(const dk_conv_desc* desc) {
+  Geo g;
+  if (make_geo(desc, g) != DK_OK) return 0;
+  return desc->dtype == DK_F64 ? 0 : fast_local_grad_rotation_workspace(g);
+}
+
 int dk_sample_depthwise_backward_rotation(const dk_conv_desc* desc, const void* out_grad,
                                           const void* input, const void* rotation,
-                                          const void* filter, void* rotation_grad, void* stream) {
+                                          const void* filter, void* rotation_grad, void* workspace,
+                                          size_t workspace_bytes, void* stream) {
   Geo g;
   const int rc = make_geo(desc, g);
   if (rc != DK_OK) return rc;
   if (!out_grad || !input || !rotation || !filter || !rotation_grad) return DK_ERR_NULL_POINTER;
+  const size_t need = dk_sample_depthwise_backward_rotation_workspace(desc);
+  if (need && (!workspace || workspace_bytes < need)) return DK_ERR_WORKSPACE;
   if (g.batch == 0) return DK_OK;
   hipStream_t s = static_cast<hipStream_t>(stream);
   return by_dtype(desc->dtype, [&]<typename T>() {
     if constexpr (kHasFast<T>)
-      if (fast_local_grad_rotation<T>(g, in<T>(out_grad), in<T>(input), in<T>(rotation), in<T>(filter), out<T>(rotation_grad), s)) return;
+      if (fast_local_grad_rotation<T>(g, in<T>(out_grad), in<T>(input), in<T>(rotation), in<T>(filter),
+                                      out<T>(rotation_grad), workspace, s)) return;
     generic_grad_rotation<T>(g, false, in<T>(out_grad), in<T>(input), (const T*)nullptr, in<T>(rotation),
                              in<T>(filter), out<T>(rotation_grad), s);
   });
 }
 
+// The rotation and the filter gradient run one after the other on the stream and share the buffer.
 size_t dk_sample_depthwise_backward_workspace(const dk_conv_desc* desc) {
-  return dk_sample_depthwise_backward_filter_workspace(desc);
+  return std::max(dk_sample_depthwise_backward_filter_workspace(desc),
+                  dk_sample_depthwise_backward_rotation_workspace(desc));
 }
 
 int dk_sample_depthwise_backward(const dk_conv_desc* desc, const void* out_grad, const void* input,
@@ -198,15 +210,15 @@ int dk_sample_depthwise_backward(const dk_conv_desc* desc, const void* out_grad,
   const int rc = make_geo(desc, g);
   if (rc != DK_OK) return rc;
   if (!out_grad || !input || !rotation || !filter) return DK_ERR_NULL_POINTER;
-  if (filter_grad) {
-    const size_t need = local_filter_ws(g, desc->dtype);
-    if (need && (!workspace || workspace_bytes < need)) return DK_ERR_WORKSPACE;
-  }
+  const size_t need = std::max(filter_grad ? dk_sample_depthwise_backward_filter_workspace(desc) : 0,
+                               rotation_grad ? dk_sample_depthwise_backward_rotation_workspace(desc) : 0);
+  if (need && (!workspace || workspace_bytes < need)) return DK_ERR_WORKSPACE;
   int st = DK_OK;
   if (in_grad && st == DK_OK)
     st = dk_sample_depthwise_backward_data(desc, out_grad, rotation, filter, in_grad, stream);
   if (rotation_grad && st == DK_OK)
-    st = dk_sample_depthwise_backward_rotation(desc, out_grad, input, rotation, filter, rotation_grad, stream);
+    st = dk_sample_depthwise_backward_rotation(desc, out_grad, input, rotation, filter, rotation_grad, workspace,
+                                               workspace_bytes, stream);
   if (filter_grad && st == DK_OK)
     st = dk_sample_depthwise_backward_filter(desc, out_grad, input, rotation, filter_grad, workspace,
                                              workspace_bytes, stream);

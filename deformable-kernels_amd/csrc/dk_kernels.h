@@ -15,9 +15,10 @@ void launch_reduce_partials(const CT* partial, int parts, int count, T* out, hip
 template <typename T>
 bool fast_local_gather(const Geo& g, bool transposed, const T* src, const T* rot, const T* filter,
                        T* dst, hipStream_t stream);
+size_t fast_local_grad_rotation_workspace(const Geo& g);
 template <typename T>
 bool fast_local_grad_rotation(const Geo& g, const T* gout, const T* x, const T* rot,
-                              const T* filter, T* grot, hipStream_t stream);
+                              const T* filter, T* grot, void* ws, hipStream_t stream);
 size_t fast_local_grad_filter_workspace(const Geo& g);
 template <typename T>
 bool fast_local_grad_filter(const Geo& g, const T* gout, const T* x, const T* rot, T* gfilter,

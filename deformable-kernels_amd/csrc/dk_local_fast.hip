@@ -318,12 +318,17 @@ __global__ __launch_bounds__(kBlock, 2) void local_gather_rows_kernel(Geo g, con
 // ROWS = true is the "same"-geometry form (see local_gather_rows_kernel): 62 pixels per
 // wave, centre-column loads and DPP neighbours; ROWS = false loads every tap.
 // The scope tables of the group's channels are staged in passes of ch_per_pass channels.
-// grid = (pixel tiles, 1, batch * groups)
+// Small planes give too few (tile, image) blocks to fill the GPU: the channels of a group are
+// then split over `splits` blocks, each writing an fp32 partial [split][image * group][18][pixel]
+// to the workspace, and reduce_partials_kernel adds the splits in order.  splits == 1 writes the
+// result directly.
+// grid = (pixel tiles, splits, batch * groups)
 // ---------------------------------------------------------------------------
 template <typename T, int KH, int KW, int SH, int SW, bool ROWS>
 __global__ __launch_bounds__(kBlock, 2) void local_grad_rotation_kernel(
     Geo g, const T* __restrict__ gout, const T* __restrict__ x, const T* __restrict__ rot,
-    const T* __restrict__ filter, T* __restrict__ grot, int ch_per_pass) {
+    const T* __restrict__ filter, T* __restrict__ grot, float* __restrict__ partial, int splits,
+    int ch_per_pass) {
   using Tb = WideTable<SH, SW>;
   constexpr int K = KH * KW;
   constexpr int NLOAD = ROWS ? KH : K;  // input loads per channel
@@ -331,13 +336,15 @@ __global__ __launch_bounds__(kBlock, 2) void local_grad_rotation_kernel(
 
   const int cpg = g.channel / g.groups;
   const int out_plane = g.out_h * g.out_w, in_plane = g.in_h * g.in_w;
-  // logical block = (tile, image * group), tile fastest
+  // logical block = (tile, channel split, image * group), tile fastest
   const int tiles = ceil_div(out_plane, ROWS ? kRowPix : kBlock);
-  const int total = tiles * g.batch * g.groups;
+  const int total = tiles * splits * g.batch * g.groups;
   const int lb = logical_block(total);
   if (lb >= total) return;
-  const int bx = lb % tiles, bz = lb / tiles;
+  const int bx = lb % tiles, split = lb / tiles % splits, bz = lb / tiles / splits;
   const int n = bz / g.groups, grp = bz % g.groups;
+  const int per_split = ceil_div(cpg, splits);
+  const int c_begin = split * per_split, c_end = min(cpg, c_begin + per_split);
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int p = ROWS ? bx * kRowPix + wave * kRowLanes + lane - 1 : bx * kBlock + threadIdx.x;
   const bool owns = (ROWS ? (lane >= 1 && lane <= kRowLanes) : true) && p < out_plane;
@@ -379,8 +386,8 @@ __global__ __launch_bounds__(kBlock, 2) void local_grad_rotation_kernel(
 
   // ch_per_pass + 1 tables: the spare one is read, times zero, by the odd channel out of a pair
   for (int e = threadIdx.x; e < (ch_per_pass + 1) * Tb::SIZE; e += kBlock) tbl[e] = 0.f;
-  for (int j0 = 0; j0 < cpg; j0 += ch_per_pass) {
-    const int nch = min(ch_per_pass, cpg - j0);
+  for (int j0 = c_begin; j0 < c_end; j0 += ch_per_pass) {
+    const int nch = min(ch_per_pass, c_end - j0);
     __syncthreads();
     stage_wide_tables<T, SH, SW>(tbl, filter, g.channel, grp + g.groups * j0, g.groups, nch);
     __syncthreads();
@@ -438,8 +445,14 @@ __global__ __launch_bounds__(kBlock, 2) void local_grad_rotation_kernel(
     float gh = fmaf(lw, sd[t], sc[t]);
     float gw = fmaf(lh, sd[t], sb[t]);
     if (!(inside >> t & 1u)) gh = gw = 0.f;
-    buf_st(ro_, ro, gh, grot);
-    buf_st(ro_, ro + (unsigned)out_plane * (unsigned)sizeof(T), gw, grot);
+    if (splits == 1) {
+      buf_st(ro_, ro, gh, grot);
+      buf_st(ro_, ro + (unsigned)out_plane * (unsigned)sizeof(T), gw, grot);
+    } else if (owns) {
+      float* dst = partial + (((size_t)split * g.batch * g.groups + bz) * (K * 2) + 2 * t) * out_plane + pc;
+      dst[0] = gh;
+      dst[out_plane] = gw;
+    }
   }
   (void)live;
 }
@@ -984,20 +997,33 @@ bool run_gather(const Geo& g, bool transposed, const T* src, const T* rot, const
   return true;
 }
 
+// Channel splits of the grad-rotation grid: 1 when the (tile, image, group) blocks alone give a
+// block per CU, else enough for four per CU with at least 16 channels per split.
+int rotation_splits(const Geo& g) {
+  const int cpg = g.channel / g.groups;
+  const long base = (long)ceil_div(g.out_h * g.out_w, same_width_geometry(g) ? kRowPix : kBlock) * g.batch * g.groups;
+  if (base >= 256) return 1;  // measured: at one block per CU and more, splitting does not pay
+  const long want = (1024 + base - 1) / base;
+  return (int)std::max<long>(1, std::min<long>(want, cpg / 16));
+}
+
 template <typename T, int SH, int SW>
 bool run_grad_rotation(const Geo& g, const T* gout, const T* x, const T* rot, const T* filter,
-                       T* grot, hipStream_t stream) {
+                       T* grot, float* ws, hipStream_t stream) {
   using Tb = WideTable<SH, SW>;
   const int cpg = g.channel / g.groups;
-  const int per = cpg < 36 ? cpg : 36;  // channels staged per pass
+  const int splits = rotation_splits(g);
+  const int per = std::min(ceil_div(cpg, splits), 36);  // channels staged per pass
   const size_t lds = (size_t)(per + 1) * Tb::SIZE * sizeof(float);
   if (same_width_geometry(g)) {
-    const unsigned grid = (unsigned)xcd_grid_size((long)ceil_div(g.out_h * g.out_w, kRowPix) * g.batch * g.groups);
-    local_grad_rotation_kernel<T, 3, 3, SH, SW, true><<<grid, kBlock, lds, stream>>>(g, gout, x, rot, filter, grot, per);
+    const unsigned grid = (unsigned)xcd_grid_size((long)ceil_div(g.out_h * g.out_w, kRowPix) * splits * g.batch * g.groups);
+    local_grad_rotation_kernel<T, 3, 3, SH, SW, true><<<grid, kBlock, lds, stream>>>(g, gout, x, rot, filter, grot, ws, splits, per);
   } else {
-    const unsigned grid = (unsigned)xcd_grid_size((long)ceil_div(g.out_h * g.out_w, kBlock) * g.batch * g.groups);
-    local_grad_rotation_kernel<T, 3, 3, SH, SW, false><<<grid, kBlock, lds, stream>>>(g, gout, x, rot, filter, grot, per);
+    const unsigned grid = (unsigned)xcd_grid_size((long)ceil_div(g.out_h * g.out_w, kBlock) * splits * g.batch * g.groups);
+    local_grad_rotation_kernel<T, 3, 3, SH, SW, false><<<grid, kBlock, lds, stream>>>(g, gout, x, rot, filter, grot, ws, splits, per);
   }
+  if (splits > 1)
+    launch_reduce_partials<float, T>(ws, splits, g.batch * g.groups * 18 * g.out_h * g.out_w, grot, stream);
   return true;
 }
 
@@ -1103,11 +1129,17 @@ bool fast_local_gather(const Geo& g, bool transposed, const T* src, const T* rot
 
 template <typename T>
 bool fast_local_grad_rotation(const Geo& g, const T* gout, const T* x, const T* rot,
-                              const T* filter, T* grot, hipStream_t stream) {
+                              const T* filter, T* grot, void* ws, hipStream_t stream) {
   if (!fast_shape(g)) return false;
-#define CALL(SH, SW) run_grad_rotation<T, SH, SW>(g, gout, x, rot, filter, grot, stream)
+#define CALL(SH, SW) run_grad_rotation<T, SH, SW>(g, gout, x, rot, filter, grot, static_cast<float*>(ws), stream)
   DK_DISPATCH_SCOPE(g, CALL)
 #undef CALL
+}
+
+size_t fast_local_grad_rotation_workspace(const Geo& g) {
+  if (!fast_shape(g)) return 0;
+  const int splits = rotation_splits(g);
+  return splits > 1 ? (size_t)splits * g.batch * g.groups * 18 * g.out_h * g.out_w * sizeof(float) : 0;
 }
 
 size_t fast_local_grad_filter_workspace(const Geo& g) {
@@ -1126,7 +1158,7 @@ bool fast_local_grad_filter(const Geo& g, const T* gout, const T* x, const T* ro
 
 #define DK_INSTANTIATE(T)                                                                           \
   template bool fast_local_gather<T>(const Geo&, bool, const T*, const T*, const T*, T*, hipStream_t); \
-  template bool fast_local_grad_rotation<T>(const Geo&, const T*, const T*, const T*, const T*, T*,  \
+  template bool fast_local_grad_rotation<T>(const Geo&, const T*, const T*, const T*, const T*, T*, void*,  \
                                             hipStream_t);                                           \
   template bool fast_local_grad_filter<T>(const Geo&, const T*, const T*, const T*, T*, void*,      \
                                           hipStream_t);

@@ -109,6 +109,7 @@ class SampleDepthwiseFunction(Function):
             ws, nbytes = None, 0
             if ctx.needs_input_grad[2]:
                 grad_weight = torch.empty_like(weight)
+            if ctx.needs_input_grad[1] or ctx.needs_input_grad[2]:
                 ws, nbytes = _lib.workspace(L.dk_sample_depthwise_backward_workspace(desc), input.device)
             _lib.check(L.dk_sample_depthwise_backward(
                 desc, _lib.ptr(grad_output), _lib.ptr(input), _lib.ptr(rotation), _lib.ptr(weight),

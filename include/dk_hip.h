@@ -98,10 +98,14 @@ int dk_sample_depthwise_backward_filter(const dk_conv_desc *desc, const void *ou
                                         void *filter_grad, void *workspace,
                                         size_t workspace_bytes, void *stream);
 
-/* sample_depthwise_backward_rotation_cuda (filter_sample_depthwise_cuda.cpp:178-235). */
+/* sample_depthwise_backward_rotation_cuda (filter_sample_depthwise_cuda.cpp:178-235).
+ * Small planes split the channel sum over several workgroups whose partial sums go through the
+ * workspace and are added in a fixed order; the query returns 0 when no split is used. */
+size_t dk_sample_depthwise_backward_rotation_workspace(const dk_conv_desc *desc);
 int dk_sample_depthwise_backward_rotation(const dk_conv_desc *desc, const void *out_grad,
                                           const void *input, const void *rotation,
-                                          const void *filter, void *rotation_grad, void *stream);
+                                          const void *filter, void *rotation_grad, void *workspace,
+                                          size_t workspace_bytes, void *stream);
 
 /* The three gradients of one backward pass in one call; any of in_grad / rotation_grad /
  * filter_grad may be NULL to skip it.  Stands in for the three consecutive pybind calls of
