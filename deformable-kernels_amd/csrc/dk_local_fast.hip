@@ -95,7 +95,7 @@ __device__ __forceinline__ bool tap_geometry(const Geo& g, int ph, int pw, int f
 // ---------------------------------------------------------------------------
 constexpr int kUnroll = 2;
 
-template <typename T, int KH, int KW, int SH, int SW, bool TRANSPOSED>
+template <typename T, int KH, int KW, int SH, int SW, bool TRANSPOSED, int NT>
 __global__ __launch_bounds__(kBlock, 2) void local_gather_kernel(Geo g, const T* __restrict__ src,
                                                                  const T* __restrict__ rot,
                                                                  const T* __restrict__ filter,
@@ -125,19 +125,24 @@ __global__ __launch_bounds__(kBlock, 2) void local_gather_kernel(Geo g, const T*
   const int pc = active ? p : 0;
   const int ph = pc / dst_w, pw = pc % dst_w;
 
-  LiteTap tap[K];
-  unsigned soff[K];  // byte offset of the tap's source element in a source plane
+  static_assert(NT == K || (TRANSPOSED && NT == 4 && KH == 3 && KW == 3), "tap slots: all taps, or the stride-2 subset");
+  LiteTap tap[NT];
+  unsigned soff[NT];  // byte offset of the tap's source element in a source plane
   const rsrc_t rr = plane_rsrc(rot + (size_t)(n * g.groups + grp) * (K * 2) * out_plane, K * 2 * out_plane);
 #pragma unroll
-  for (int t = 0; t < K; ++t) {
-    const int f_h = t / KW, f_w = t % KW;
+  for (int slot = 0; slot < NT; ++slot) {
+    // NT == 4: stride 2 x 2, undilated.  An input pixel is fed only by the taps with
+    // f = (p + pad) mod 2 (+ 2), at most two per direction; the slots enumerate those.
+    const int f_h = NT == K ? slot / KW : ((ph + g.pad_h) & 1) + 2 * (slot >> 1);
+    const int f_w = NT == K ? slot % KW : ((pw + g.pad_w) & 1) + 2 * (slot & 1);
+    const int t = NT == K ? slot : min(f_h, KH - 1) * KW + min(f_w, KW - 1);
     int s_el, rpix;
-    const bool ok = tap_geometry<TRANSPOSED>(g, ph, pw, f_h, f_w, s_el, rpix) && active;
-    soff[t] = ok ? (unsigned)s_el * (unsigned)sizeof(T) : kOutOfRange;
+    const bool ok = f_h < KH && f_w < KW && tap_geometry<TRANSPOSED>(g, ph, pw, f_h, f_w, s_el, rpix) && active;
+    soff[slot] = ok ? (unsigned)s_el * (unsigned)sizeof(T) : kOutOfRange;
     const unsigned ro = ok ? (unsigned)((2 * t) * out_plane + rpix) * (unsigned)sizeof(T) : kOutOfRange;
     const float r_h = buf_ld(rr, ro, rot);
     const float r_w = buf_ld(rr, ro + (unsigned)out_plane * (unsigned)sizeof(T), rot);
-    tap[t] = make_lite_tap<SH, SW>(scope_coord<float>(f_h, r_h, g.centre_h),
+    tap[slot] = make_lite_tap<SH, SW>(scope_coord<float>(f_h, r_h, g.centre_h),
                                    scope_coord<float>(f_w, r_w, g.centre_w), ok);
   }
   __syncthreads();
@@ -152,21 +157,21 @@ __global__ __launch_bounds__(kBlock, 2) void local_gather_kernel(Geo g, const T*
   // while the current one is computed, so a wave always has input loads outstanding.
   // Channels beyond nch load through a zero-length resource (hardware returns 0) and
   // store to an out-of-range offset (dropped), which keeps the loop free of branches.
-  auto load_stage = [&](float (&xv)[kUnroll][K], int jb) {
+  auto load_stage = [&](float (&xv)[kUnroll][NT], int jb) {
 #pragma unroll
     for (int u = 0; u < kUnroll; ++u) {
       const rsrc_t rs = plane_rsrc(sp + (size_t)(jb + u) * s_step, (jb + u) < nch ? src_plane : 0);
 #pragma unroll
-      for (int t = 0; t < K; ++t) xv[u][t] = buf_ld(rs, soff[t], src);
+      for (int t = 0; t < NT; ++t) xv[u][t] = buf_ld(rs, soff[t], src);
     }
   };
-  auto compute_stage = [&](const float (&xv)[kUnroll][K], int jb) {
+  auto compute_stage = [&](const float (&xv)[kUnroll][NT], int jb) {
     const float* tb = tbl + jb * Tb::SIZE;
 #pragma unroll
     for (int u = 0; u < kUnroll; ++u) {
       float acc = 0.f;
 #pragma unroll
-      for (int t = 0; t < K; ++t) {
+      for (int t = 0; t < NT; ++t) {
         const float4 q = *reinterpret_cast<const float4*>(tb + tap[t].cell + u * Tb::SIZE);
         acc = fmaf(xv[u][t], lite_weight(tap[t], q), acc);
       }
@@ -174,7 +179,7 @@ __global__ __launch_bounds__(kBlock, 2) void local_gather_kernel(Geo g, const T*
     }
   };
 
-  float xa[kUnroll][K], xb[kUnroll][K];
+  float xa[kUnroll][NT], xb[kUnroll][NT];
   load_stage(xa, 0);
   for (int j = 0; j < nch; j += 2 * kUnroll) {
     load_stage(xb, j + kUnroll);
@@ -990,10 +995,12 @@ bool run_gather(const Geo& g, bool transposed, const T* src, const T* rot, const
   const unsigned grid = (unsigned)xcd_grid_size((long)ceil_div(pixels, kBlock) * ceil_div(cpg, per) * g.batch * g.groups);
   // stages past the last channel still read (and discard) table entries: pad to whole stages
   const size_t lds = (size_t)(per + 2 * kUnroll) * WideTable<SH, SW>::SIZE * sizeof(float);
-  if (transposed)
-    local_gather_kernel<T, 3, 3, SH, SW, true><<<grid, kBlock, lds, stream>>>(g, src, rot, filter, dst, per);
+  if (transposed && g.stride_h == 2 && g.stride_w == 2 && g.dil_h == 1 && g.dil_w == 1)
+    local_gather_kernel<T, 3, 3, SH, SW, true, 4><<<grid, kBlock, lds, stream>>>(g, src, rot, filter, dst, per);
+  else if (transposed)
+    local_gather_kernel<T, 3, 3, SH, SW, true, 9><<<grid, kBlock, lds, stream>>>(g, src, rot, filter, dst, per);
   else
-    local_gather_kernel<T, 3, 3, SH, SW, false><<<grid, kBlock, lds, stream>>>(g, src, rot, filter, dst, per);
+    local_gather_kernel<T, 3, 3, SH, SW, false, 9><<<grid, kBlock, lds, stream>>>(g, src, rot, filter, dst, per);
   return true;
 }
 
