@@ -325,12 +325,17 @@ __global__ __launch_bounds__(kDBlock, 2) void deform_grad_coord_kernel(
 // One block per (image, group, channel chunk); blockDim = output pixels rounded up to a wave.
 // ---------------------------------------------------------------------------
 template <typename T>
-__global__ void absmax_kernel(const T* __restrict__ p, long n, unsigned* __restrict__ out) {
+__global__ __launch_bounds__(256) void absmax_kernel(const T* __restrict__ p, long n, unsigned* __restrict__ out) {
+  __shared__ float wave_max[4];
   float m = 0.f;
   for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (long)gridDim.x * blockDim.x)
     m = fmaxf(m, fabsf(ld(p + i)));
   for (int s = 32; s > 0; s >>= 1) m = fmaxf(m, __shfl_xor(m, s));
-  if ((threadIdx.x & 63) == 0) atomicMax(out, __float_as_uint(m));  // non-negative floats order like their bits
+  if ((threadIdx.x & 63) == 0) wave_max[threadIdx.x >> 6] = m;
+  __syncthreads();
+  // one atomic per block (atomics on one address serialise): non-negative floats order like their bits
+  if (threadIdx.x == 0)
+    atomicMax(out, __float_as_uint(fmaxf(fmaxf(wave_max[0], wave_max[1]), fmaxf(wave_max[2], wave_max[3]))));
 }
 __global__ void clear_word_kernel(unsigned* p) { *p = 0u; }
 
