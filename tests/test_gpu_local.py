@@ -26,6 +26,10 @@ TUNED = [
     (2, 16, 13, 13, 3, (3, 3), 1, 1, 1, 1, 1.0),    # scope == kernel
     (1, 16, 13, 12, 3, (5, 5), 1, 0, 1, 2, 1.5),    # scope 5, no padding
     (1, 200, 9, 9, 3, (4, 4), 1, 1, 1, 1, 2.0),     # many channels, many samples outside the scope
+    (3, 40, 21, 17, 3, (4, 4), 1, 1, 1, 2, 1.0),    # same-width geometry, 2 groups, 20 channels per group (1.25 MFMA blocks)
+    (1, 272, 12, 12, 3, (3, 3), 1, 1, 1, 1, 1.0),   # more than 256 channels: two channel splits of the matrix-core grad filter
+    (2, 10, 16, 18, 3, (4, 4), 2, 0, 1, 1, 1.0),    # stride 2 without padding, even sizes (tap parity of grad input)
+    (2, 8, 70, 40, 3, (4, 4), 1, 1, 1, 1, 0.7),     # 2800-pixel planes: many tiles per image, partial last tile
 ]
 GENERIC = [
     (2, 6, 9, 8, (5, 3), (7, 4), (1, 2), (2, 0), 1, 3, 0.7),
