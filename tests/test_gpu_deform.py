@@ -110,3 +110,35 @@ def test_config4_shape_on_a_batch_slice():
     assert rel_err(got[0], o32[0]) < 1e-5
     for i in range(1, 5):
         assert rel_err(got[i], o64[i]) < 1e-4, NAMES[i]
+
+
+def test_config4_properties_at_full_size():
+    """BASELINE config 4 (N=64, C=512, 28x28 -> 14x14, stride 2, fp32) at full size: the oracle on
+    two images; the whole batch through properties that need no oracle -- the operator is linear
+    in the input and in the filter, so <gout, F> = <grad_input, x> = <grad_filter, Wt>, and it is
+    independent per image."""
+    from deformable_kernels.ops.deform_kernel.functions import deform_sample_depthwise
+    case = (64, 512, 28, 28, 3, (4, 4), 2, 1, 1, 1, 0.5, 2.0)
+    (x, wt, rot, off, gout, cfg), got = _run(case, torch.float32)
+    out, gin, goff, grot, gw = got
+    for n in (0, 63):
+        sl = slice(n, n + 1)
+        a = [t[sl].double().numpy() for t in (x, off, rot)] + [wt.double().numpy(), gout[sl].double().numpy()]
+        want = orc.deform_sample_depthwise_forward(a[0], a[1], a[2], a[3], **cfg)
+        w_gin, w_goff, w_grot, _ = orc.deform_sample_depthwise_backward(a[4], a[0], a[1], a[2], a[3], **cfg)
+        assert rel_err(out[sl], want) < 1e-5
+        assert rel_err(gin[sl], w_gin) < 1e-4
+        assert rel_err(goff[sl], w_goff) < 1e-4
+        assert rel_err(grot[sl], w_grot) < 1e-4
+    lhs = (gout.double() * out.double()).sum().item()
+    via_x = (gin.double() * x.double()).sum().item()
+    via_w = (gw.double() * wt.double()).sum().item()
+    assert abs(lhs - via_x) < 1e-5 * max(abs(lhs), 1.0)
+    assert abs(lhs - via_w) < 1e-5 * max(abs(lhs), 1.0)
+    # batch independence: images 10..13 alone give the same rows
+    dev = torch.device("cuda:0")
+    sl = slice(10, 14)
+    with torch.no_grad():
+        part = deform_sample_depthwise(x[sl].to(dev), off[sl].to(dev), rot[sl].to(dev), wt.to(dev), cfg["kernel_size"],
+                                       cfg["stride"], cfg["padding"], cfg["dilation"], cfg["groups"])
+    assert torch.equal(part.cpu(), out[sl])
