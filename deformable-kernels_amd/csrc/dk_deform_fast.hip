@@ -563,7 +563,7 @@ struct DeformPlan {
 DeformPlan deform_plan(const Geo& g, int table_floats, int planes, int block) {
   DeformPlan d{};
   d.ok = false;
-  if (getenv("DK_NO_DEFORM_FAST")) return d;
+  if (path_disabled("DK_NO_DEFORM_FAST")) return d;
   if (g.k_h != 3 || g.k_w != 3 || g.in_w > 64) return d;
   if (!((g.scope_h == 3 && g.scope_w == 3) || (g.scope_h == 4 && g.scope_w == 4) ||
         (g.scope_h == 5 && g.scope_w == 5)))

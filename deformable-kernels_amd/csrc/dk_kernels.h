@@ -6,7 +6,18 @@
 
 #include "dk_common.h"
 
+#include <cstdlib>
+
 namespace dk {
+
+// Test switches.  Setting one of these environment variables (to anything) makes the dispatch
+// skip a specialised kernel family and take the next more general one, so that every kernel can
+// be reached for the same shape:
+//   DK_NO_ROWS         the "same-width" row kernels (and with them the matrix-core grad filter)
+//   DK_NO_MFMA         the matrix-core grad filter (the dense register form runs instead)
+//   DK_NO_DEFORM_FAST  the tuned deformable kernels (the generic ones run instead)
+// Read at every call, so a test can toggle them inside one process.
+inline bool path_disabled(const char* name) { return std::getenv(name) != nullptr; }
 
 template <typename CT, typename T>
 void launch_reduce_partials(const CT* partial, int parts, int count, T* out, hipStream_t stream);

@@ -953,7 +953,7 @@ constexpr int kMaxLdsTables = 96 * 1024;  // bytes of LDS a workgroup may spend 
 // pixel's taps are three runs of three consecutive elements
 bool same_width_geometry(const Geo& g) {
   return g.stride_h == 1 && g.stride_w == 1 && g.dil_w == 1 && g.pad_w == 1 && g.k_w == 3 &&
-         g.in_w == g.out_w && !getenv("DK_NO_ROWS");
+         g.in_w == g.out_w && !path_disabled("DK_NO_ROWS");
 }
 
 template <int SH, int SW>
@@ -970,8 +970,6 @@ int pick_splits(const Geo& g, int planes_pixels) {
   const long waves = (long)ceil_div(planes_pixels, kBlock) * (kBlock / 64) * g.batch * g.groups;
   const int cpg = g.channel / g.groups;
   int splits = 1;
-  const char* env = getenv("DK_SPLITS");  // tuning aid
-  if (env) return atoi(env);
   while (waves * splits < 8192 && cpg / (splits * 2) >= 16) splits *= 2;
   return splits;
 }
@@ -1051,7 +1049,7 @@ FilterGrid filter_grid(const Geo& g) {
   f.mfma = false;
   f.pitch_x = 0;
   f.lds = 0;
-  if (same_width_geometry(g) && g.scope_h * g.scope_w <= 16 && !getenv("DK_NO_MFMA")) {
+  if (same_width_geometry(g) && g.scope_h * g.scope_w <= 16 && !path_disabled("DK_NO_MFMA")) {
     const long xt = kMfPix + 2 + 2L * g.dil_h * g.in_w;
     const long pitch = (xt + 51 + 63) / 64 * 64;  // rows 64 floats apart plus the skew of mf_row() (at most 51)
     const int nblk = ceil_div(cpg, kMfCh);

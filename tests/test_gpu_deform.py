@@ -142,3 +142,13 @@ def test_config4_properties_at_full_size():
         part = deform_sample_depthwise(x[sl].to(dev), off[sl].to(dev), rot[sl].to(dev), wt.to(dev), cfg["kernel_size"],
                                        cfg["stride"], cfg["padding"], cfg["dilation"], cfg["groups"])
     assert torch.equal(part.cpu(), out[sl])
+
+
+def test_generic_kernels_on_a_shape_the_tuned_ones_cover(monkeypatch):
+    """With the tuned deformable kernels switched off the generic ones serve the same shape."""
+    monkeypatch.setenv("DK_NO_DEFORM_FAST", "1")
+    inputs, got = _run(CASES[0], torch.float32)
+    o32, o64 = _oracle(inputs, np.float32), _oracle(inputs, np.float64)
+    assert rel_err(got[0], o32[0]) < 1e-5
+    for i in range(1, 5):
+        assert rel_err(got[i], o64[i]) < 1e-4, NAMES[i]

@@ -175,3 +175,18 @@ def test_headline_shape_properties_at_full_size():
         a = (gout.to(dev).double() * out.double()).sum().item()
         b = (xg.grad.double() * xg.double()).sum().item()
         assert abs(a - b) < 1e-6 * max(abs(a), 1.0)
+
+
+@pytest.mark.parametrize("switch", ["DK_NO_MFMA", "DK_NO_ROWS"])
+def test_more_general_kernels_on_a_same_width_shape(switch, monkeypatch):
+    """The dispatch prefers the most specialised kernel; the library's test switches make it take
+    the next more general family for the same shape (dense grad filter instead of the
+    matrix-core one; per-tap loads instead of the row kernels), which must give the same results."""
+    monkeypatch.setenv(switch, "1")
+    case = (2, 40, 20, 24, 3, (4, 4), 1, 1, 1, 2, 1.0)
+    inputs, got = _run(case, torch.float32)
+    o32, o64 = _oracle(inputs, np.float32), _oracle(inputs, np.float64)
+    assert rel_err(got[0], o32[0]) < 1e-5
+    assert rel_err(got[1], o32[1]) < 1e-5
+    assert rel_err(got[2], o64[2]) < 1e-4
+    assert rel_err(got[3], o64[3]) < 1e-4
