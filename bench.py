@@ -91,7 +91,8 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--workload", default="cfg2", choices=sorted(WORKLOADS) + sorted(OTHER_WORKLOADS))
+    ap.add_argument("--workload", default="cfg2", choices=sorted(WORKLOADS) + sorted(OTHER_WORKLOADS) + ["mbv2_dk"])
+    ap.add_argument("--batch", type=int, default=64, help="batch size of the mbv2_dk workload")
     ap.add_argument("--dtype", default="fp32", choices=sorted(DTYPES))
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--kernels", default="", help="comma list restricting the per-kernel timing (tuning aid)")
@@ -107,6 +108,8 @@ def main():
 
     if not torch.cuda.is_available():
         sys.exit("bench.py needs a GPU")
+    if a.workload == "mbv2_dk":
+        return mobilenet_workload(a)
     if a.workload in OTHER_WORKLOADS:
         return other_workload(a)
     dev = torch.device("cuda:0")
@@ -163,7 +166,6 @@ def main():
     calib = torch.empty_like(xg)
     torch.mul(xg, 1.0, out=calib)
     del calib
-
     for _ in range(a.warmup):
         step()
     torch.cuda.synchronize()
@@ -188,6 +190,15 @@ def main():
         e1.record()
         e1.synchronize()
         per_kernel_us[name] = e0.elapsed_time(e1) * 1e3 / reps
+
+    # measured streaming bandwidth of this GPU: an elementwise pass over 2 x 1 GiB (far beyond the
+    # 256 MB memory-side cache)
+    big_a = torch.empty(1 << 28, dtype=torch.float32, device=dev).fill_(1.0)
+    big_b = torch.empty_like(big_a)
+    copy_us = _time_us(lambda: torch.mul(big_a, 1.0, out=big_b), 10)
+    copy_gbps = 2 * big_a.numel() * 4 / copy_us / 1e3
+    del big_a, big_b
+
 
     esz = xg.element_size()
     per_kernel_bytes, fwd_b, bwd_b = algorithmic_bytes(N, C, H, W, Ho, Wo, k, S, groups, esz)
@@ -214,6 +225,8 @@ def main():
                                % (a.workload, N, C, H, W, k, S[0], S[1], stride, pad, a.dtype),
                    "algorithmic_MB_per_step": round(step_bytes / 1e6, 2)},
         "pct_of_hbm_peak": round(100.0 * gbps / HBM_PEAK_GBPS, 2),
+        "device_copy_GBps": round(copy_gbps, 1),
+        "pct_of_device_copy": round(100.0 * gbps / copy_gbps, 2),
         "images_per_s": round(N / (ms_per_step * 1e-3), 1),
         "layers_per_s": round(1.0 / (ms_per_step * 1e-3), 1),
         "kernel_us": {n: round(v, 2) for n, v in per_kernel_us.items()},
@@ -323,6 +336,58 @@ def other_workload(a):
     }))
 
 
+# The 17 depthwise 3x3 layers of MobileNetV2 at 224 x 224 (channels, input size, stride), each
+# replaced by DeformKernel2d with a 4 x 4 scope (BASELINE config 5, operator calls only).
+MBV2_DW_LAYERS = [(32, 112, 1), (96, 112, 2), (144, 56, 1), (144, 56, 2), (192, 28, 1), (192, 28, 1), (192, 28, 2),
+                  (384, 14, 1), (384, 14, 1), (384, 14, 1), (384, 14, 1), (576, 14, 1), (576, 14, 1), (576, 14, 2),
+                  (960, 7, 1), (960, 7, 1), (960, 7, 1)]
+
+
+def mobilenet_workload(a):
+    """Forward + backward of the 17 deformable-kernel depthwise layers of MobileNetV2-DK, operator
+    calls only (one JSON line; secondary to the BASELINE headline)."""
+    import collections
+    import torch
+    from _cases import make_local
+    from deformable_kernels.ops.deform_kernel import _lib
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    tdtype = getattr(torch, DTYPES[a.dtype])
+    L, P = _lib.lib(), _lib.ptr
+    reps = max(a.steps // 10, 10)
+    per_layer, total_us, total_bytes = [], 0.0, 0
+    for (C, H, stride), count in collections.Counter(MBV2_DW_LAYERS).items():
+        x, wt, rot, gout, cfg = make_local(a.batch, C, H, H, 3, (4, 4), stride, 1, 1, 1, 0.5, seed=0, dtype=tdtype)
+        xg, wg, rg, gg = [t.to(dev) for t in (x, wt, rot, gout)]
+        out, gin, grot, gw = [torch.empty_like(t) for t in (gg, xg, rg, wg)]
+        desc = _lib.conv_desc(xg, wg, cfg["kernel_size"], cfg["stride"], cfg["padding"], cfg["dilation"], 1)
+        ws, nb = _lib.workspace(L.dk_sample_depthwise_backward_workspace(desc), dev)
+        st = _lib.stream_ptr(xg)
+
+        def step():
+            _lib.check(L.dk_sample_depthwise_forward(desc, P(xg), P(rg), P(wg), P(out), st), "forward")
+            _lib.check(L.dk_sample_depthwise_backward(desc, P(gg), P(xg), P(rg), P(wg), P(gin), P(grot), P(gw),
+                                                      P(ws), nb, st), "backward")
+        us = _time_us(step, reps)
+        e = xg.element_size()
+        _, fwd_b, bwd_b = algorithmic_bytes(a.batch, C, H, H, gg.shape[2], gg.shape[3], 3, (4, 4), 1, e)
+        per_layer.append({"C": C, "HW": H, "stride": stride, "count": count, "us": round(us, 1),
+                          "GBps": round((fwd_b + bwd_b) / us / 1e3, 1)})
+        total_us += us * count
+        total_bytes += (fwd_b + bwd_b) * count
+        del xg, wg, rg, gg, out, gin, grot, gw, ws
+    print(json.dumps({
+        "metric": "MobileNetV2-DK depthwise layers fwd+bwd, operator calls only (secondary workload)",
+        "config": {"workload": "mbv2_dk: 17 DeformKernel2d layers, batch %d, scope 4x4, %s" % (a.batch, a.dtype)},
+        "images_per_s": round(a.batch / (total_us * 1e-6), 1),
+        "ms_per_batch": round(total_us / 1e3, 3),
+        "algorithmic_MB": round(total_bytes / 1e6, 1),
+        "value": round(total_bytes / total_us / 1e3, 1), "unit": "GB/s",
+        "pct_of_hbm_peak": round(100.0 * total_bytes / total_us / 1e3 / HBM_PEAK_GBPS, 2),
+        "layers": per_layer, "n_gpus": 1, "dtype": a.dtype, "data": "synthetic",
+    }))
+
+
 def cpu_baseline(N, C, H, W, k, S, stride, pad, dil, groups, rot_std, esz):
     """The CPU oracle (a port of the reference's arithmetic; the reference has no CPU path),
     OpenMP over the host cores, fp32, on the first `n` images of the same seeded workload."""
@@ -344,10 +409,18 @@ def cpu_baseline(N, C, H, W, k, S, stride, pad, dil, groups, rot_std, esz):
     mean = sum(times) / len(times)
     Ho, Wo = gout.shape[2], gout.shape[3]
     _, fwd_b, bwd_b = algorithmic_bytes(n, C, H, W, Ho, Wo, k, S, groups, 4)
+    # one thread, one pass over the first 2 images (the same arithmetic, for the per-core figure)
+    orc.set_threads(1)
+    t0 = time.perf_counter()
+    orc.sample_depthwise_forward(xs[:2], rs[:2], ws_, **cfg)
+    orc.sample_depthwise_backward(gs[:2], xs[:2], rs[:2], ws_, **cfg)
+    t_one = time.perf_counter() - t0
+    orc.set_threads(threads)
     return {
         "value": round((fwd_b + bwd_b) / mean / 1e9, 3),
         "unit": "GB/s",
         "cores": threads,
+        "one_core_value": round((fwd_b + bwd_b) * 2 / n / t_one / 1e9, 4),
         "kind": "port",
         "sample": "first %d of %d images of the same seeded workload, fwd + 3 grads, fp32, mean of %d passes "
                   "(%.1f s of CPU work, %.3f s per pass, %.1f images/s)"
