@@ -39,6 +39,8 @@ DTYPES = {"fp32": "float32", "bf16": "bfloat16", "fp16": "float16"}
 OTHER_WORKLOADS = {
     # deformable variant, BASELINE config 4: N, C, H, W, k, S, stride, pad, dil, groups, rot_std, off_std
     "cfg4": ("deform", (64, 512, 28, 28, 3, (4, 4), 2, 1, 1, 1, 0.5, 2.0)),
+    # the deformable variant on the headline layer's shape (3136 output pixels per plane)
+    "deform_56": ("deform", (64, 144, 56, 56, 3, (4, 4), 1, 1, 1, 1, 0.5, 2.0)),
     # N-d sampler: data shape [C, s...], points, coordinate range
     "nd_cfg3": ("nd", ((256, 5, 5), 1152, (0.0, 4.0))),             # GlobalDeformKernel2d, config 3
     "nd_cfg5": ("nd", ((64, 32, 32, 32), 1 << 20, (-1.0, 32.0))),   # trilinear volume, config 5, full-volume coords
@@ -298,8 +300,8 @@ def other_workload(a):
             "grad_filter": (lambda: _lib.check(L.dk_deformable_sample_depthwise_backward_filter(
                 desc, P(gg), P(xg), P(og), P(rg), P(gw), P(ws2), n2, st), "gw"), by + bx + bo + br + bw),
         }
-        label = "cfg4: deform_sample_depthwise N=%d C=%d %dx%d->%dx%d k=%d scope=%dx%d stride=%d %s" % (
-            N, C, H, W, gg.shape[2], gg.shape[3], k, S[0], S[1], stride, a.dtype)
+        label = "%s: deform_sample_depthwise N=%d C=%d %dx%d->%dx%d k=%d scope=%dx%d stride=%d %s" % (
+            a.workload, N, C, H, W, gg.shape[2], gg.shape[3], k, S[0], S[1], stride, a.dtype)
     else:
         shape, B, (lo, hi) = spec
         g = torch.Generator().manual_seed(0)

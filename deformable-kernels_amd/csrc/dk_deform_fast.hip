@@ -438,6 +438,107 @@ __global__ __launch_bounds__(1024) void deform_grad_input_kernel(
 }
 
 // ---------------------------------------------------------------------------
+// grad input for output planes of more than 1024 pixels.  The same fixed-point LDS accumulation,
+// but the workgroup (1024 threads) owns only kTiledCh channels of an image and keeps one plane
+// per channel; it walks the output plane in tiles of 1024 pixels, computes a tile's tap
+// descriptors once and adds the tile's contributions for each of its channels.  The planes are
+// read back once at the end.  grid = (channel chunks of kTiledCh, image * group)
+// ---------------------------------------------------------------------------
+constexpr int kTiledCh = 4;
+
+template <typename T, int SH, int SW>
+__global__ __launch_bounds__(1024) void deform_grad_input_tiled_kernel(
+    Geo g, const T* __restrict__ gout, const T* __restrict__ off, const T* __restrict__ rot,
+    const T* __restrict__ filter, T* __restrict__ gin, const unsigned* __restrict__ gmax_bits, int shift) {
+  using Tb = WideTable<SH, SW>;
+  extern __shared__ __align__(16) float lds[];
+  const int H = g.in_h, W = g.in_w, RS = W + 2;
+  const int PS = ((H + 2) * RS + 3) & ~3;
+  unsigned long long* planes = reinterpret_cast<unsigned long long*>(lds);  // [kTiledCh][PS]
+  float* tbl = lds + 2 * kTiledCh * PS;                                     // [kTiledCh][Tb::SIZE]
+  float* wmax = tbl + kTiledCh * Tb::SIZE;                                  // [kTiledCh]
+
+  const int cpg = g.channel / g.groups;
+  const int out_plane = g.out_h * g.out_w, in_plane = H * W;
+  const BlockId b = decode_block(g, 1, ceil_div(cpg, kTiledCh));
+  if (!b.valid) return;
+  const int j0 = b.chunk * kTiledCh;
+  const int nch = min(kTiledCh, cpg - j0);
+
+  for (int e = threadIdx.x; e < kTiledCh * PS; e += blockDim.x) planes[e] = 0ull;
+  stage_wide_tables<T, SH, SW>(tbl, filter, g.channel, b.grp + g.groups * j0, g.groups, nch);
+  if (threadIdx.x < nch) {
+    const T* f = filter + (size_t)(b.grp + g.groups * (j0 + threadIdx.x)) * (SH * SW);
+    float m = 0.f;
+    for (int e = 0; e < SH * SW; ++e) m = fmaxf(m, fabsf(ld(f + e)));
+    wmax[threadIdx.x] = m;
+  }
+  __syncthreads();
+
+  const float gmax = __uint_as_float(*gmax_bits);
+  constexpr double kMagic = 6755399441055744.0;  // 1.5 * 2^52
+  const size_t chan0 = (size_t)b.n * g.channel + b.grp + (size_t)g.groups * j0;
+  const T* gp = gout + chan0 * out_plane;
+  const size_t g_step = (size_t)g.groups * out_plane, i_step = (size_t)g.groups * in_plane;
+
+  for (int tile = 0; tile * (int)blockDim.x < out_plane; ++tile) {
+    const int p = tile * (int)blockDim.x + threadIdx.x;
+    const bool live = p < out_plane;
+    ImgTap it[K9];
+    LiteTap st[K9];
+    unsigned hits = 0;
+    {
+      ScopeCoord sc[K9];
+      deform_taps<T>(g, off, rot, b.n, b.grp, p, live, RS, it, sc);
+#pragma unroll
+      for (int t = 0; t < K9; ++t) {
+        st[t] = make_lite_tap<SH, SW>(sc[t].h, sc[t].w, true);
+        const bool in = (sc[t].h > -1.f) && (sc[t].w > -1.f) && (sc[t].h < float(SH)) && (sc[t].w < float(SW));
+        hits |= in ? (1u << t) : 0u;
+      }
+    }
+    const unsigned goff = live ? (unsigned)p * (unsigned)sizeof(T) : kOutOfRange;
+    for (int j = 0; j < nch; ++j) {
+      const float gv = buf_ld(plane_rsrc(gp + (size_t)j * g_step, out_plane), goff, gout);
+      unsigned long long* pl = planes + j * PS;
+      const float* tb = tbl + j * Tb::SIZE;
+      int e;
+      (void)frexpf(gmax * wmax[j], &e);
+      const double scale = ldexp(1.0, 44 - e);
+#pragma unroll
+      for (int t = 0; t < K9; ++t) {
+        if (hits >> t & 1u) {
+          const float4 q = *reinterpret_cast<const float4*>(tb + st[t].cell);
+          const float gw = gv * lite_weight(st[t], q);
+          const float lh = it[t].lh, lw = it[t].lw, hh = 1.f - lh, hw = 1.f - lw;
+          const float term[4] = {hh * hw * gw, hh * lw * gw, lh * hw * gw, lh * lw * gw};
+          const int at[4] = {it[t].pidx, it[t].pidx + 1, it[t].pidx + RS, it[t].pidx + RS + 1};
+#pragma unroll
+          for (int k = 0; k < 4; ++k) {
+            const double d = fma((double)term[k], scale, kMagic);
+            atomicAdd(pl + at[k], (unsigned long long)__double_as_longlong(d) - 0x4338000000000000ull);
+          }
+        }
+      }
+    }
+  }
+  __syncthreads();
+
+  const int col = threadIdx.x & ((1 << shift) - 1), sub = threadIdx.x >> shift;
+  const int rpp = (int)blockDim.x >> shift;
+  T* ip = gin + chan0 * in_plane;
+  for (int j = 0; j < nch; ++j) {
+    int e;
+    (void)frexpf(gmax * wmax[j], &e);
+    const double unscale = ldexp(1.0, e - 44);
+    const unsigned long long* pl = planes + j * PS;
+    T* dst = ip + (size_t)j * i_step;
+    for (int row = sub; row < H; row += rpp)
+      if (col < W) dk::st(dst + row * W + col, (float)((double)(long long)pl[(row + 1) * RS + 1 + col] * unscale));
+  }
+}
+
+// ---------------------------------------------------------------------------
 // grad filter (K.cu:1002-1097): gW[c][i][j] = sum over (image, pixel, tap) of
 // sample_t * gout * hat(sh_t - i) * hat(sw_t - j).  As in the local operator the sum is kept
 // dense and in registers (per tap the lane holds the SH + SW hat weights, per channel it adds
@@ -654,11 +755,33 @@ template <typename T, int SH, int SW>
 bool run_deform_grad_input(const Geo& g, const T* gout, const T* off, const T* rot, const T* filter, T* gin,
                            void* ws, hipStream_t stream) {
   const DeformPlan d = grad_input_plan<SH, SW>(g);
-  if (!d.ok) return false;
+  const bool tiled = !d.ok && g.out_h * g.out_w > 1024;
+  size_t tiled_lds = 0;
+  int tiled_shift = 0;
+  if (tiled) {
+    // the basic limits of the tuned family, then room for kTiledCh 64-bit planes in LDS
+    const DeformPlan basic = deform_plan(g, WideTable<SH, SW>::SIZE, 0, 1024);
+    if (!basic.ok) return false;
+    tiled_shift = basic.shift;
+    tiled_lds = ((size_t)2 * kTiledCh * basic.PS + (size_t)kTiledCh * WideTable<SH, SW>::SIZE + kTiledCh) * sizeof(float);
+    if (tiled_lds > 150 * 1024) return false;
+  } else if (!d.ok) {
+    return false;
+  }
   unsigned* gmax = static_cast<unsigned*>(ws);
   clear_word_kernel<<<1, 1, 0, stream>>>(gmax);
   const long n = (long)g.batch * g.channel * g.out_h * g.out_w;
   absmax_kernel<T><<<(unsigned)std::min<long>(1024, (n + 255) / 256), 256, 0, stream>>>(gout, n, gmax);
+  if (tiled) {
+    auto kernel = deform_grad_input_tiled_kernel<T, SH, SW>;
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                            (int)tiled_lds) != hipSuccess)
+      return false;
+    const int cpg = g.channel / g.groups;
+    const unsigned tgrid = (unsigned)xcd_grid_size((long)ceil_div(cpg, kTiledCh) * g.batch * g.groups);
+    kernel<<<tgrid, 1024, tiled_lds, stream>>>(g, gout, off, rot, filter, gin, gmax, tiled_shift);
+    return true;
+  }
   const unsigned grid = (unsigned)xcd_grid_size((long)d.chunks * g.batch * g.groups);
   deform_grad_input_kernel<T, SH, SW><<<grid, grad_input_block(g), d.lds, stream>>>(g, gout, off, rot, filter, gin, gmax,
                                                                                    d.per, d.shift);

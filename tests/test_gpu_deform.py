@@ -28,6 +28,7 @@ CASES = [
     (1, 6, 33, 60, 3, (5, 5), 1, 1, 1, 1, 1.0, 2.5),      # wide plane (16 staging passes), scope 5, > 1024 output pixels
     (2, 80, 10, 10, 3, (3, 3), 1, 1, 1, 1, 0.8, 1.0),     # many channels: several channel chunks per image
     (1, 8, 20, 18, 3, (4, 4), 2, 1, 1, 1, 0.5, 6.0),      # large offsets: many samples outside the image
+    (2, 10, 40, 36, 3, (4, 4), 1, 1, 1, 2, 0.7, 2.0),     # 1440 output pixels: tiled grad input, 5 channels per group (partial chunk)
 ]
 NAMES = ("forward", "grad input", "grad offset", "grad rotation", "grad filter")
 
