@@ -11,7 +11,7 @@ autocast-aware cast.
 import torch
 from torch import nn
 
-from ..ops.deform_kernel.functions import nd_linear_sample
+from ..ops.deform_kernel.functions import nd_linear_sample, sample_depthwise
 from ..ops.deform_kernel.modules import (
     SampleDepthwise,
     DeformableSampleDepthwise,
@@ -62,6 +62,11 @@ class GlobalDeformKernel2d(nn.Module):
         self.fc = nn.Linear(in_planes, kernel_size * kernel_size * len(self.weight_shape))
         self.fc.zero_init = True
         self.fc_bias = _centred_tap_grid(weight_shape, kernel_size, self.weight_dilate)
+        # Depthwise layers with a 2-D scope take one call of the fused sample + depthwise operator
+        # with the image's rotation broadcast over its pixels, instead of sampling N * C kernels and
+        # running a convolution with N * C groups (the reference's route, :92-116, kept for every
+        # other configuration and when this flag is cleared).  Same function, same parameters.
+        self.fused = True
         self.reset_parameters()
 
     def reset_parameters(self):
@@ -91,7 +96,32 @@ class GlobalDeformKernel2d(nn.Module):
         return sampled.transpose(1, 2).reshape(
             n * self.out_planes, self.in_planes // self.group, self.kernel_size, self.kernel_size)
 
+    def _fusable(self, x):
+        return (self.fused and x.is_cuda and len(self.weight_shape) == 2 and self.weight_dilate == 1
+                and self.group == self.in_planes == self.out_planes)
+
+    def _forward_fused(self, x):
+        n = x.size(0)
+        taps = self.kernel_size * self.kernel_size
+        centre = torch.tensor(self.fc_bias, dtype=torch.float32, device=x.device).unsqueeze(0)
+        with torch.autocast(device_type="cuda", enabled=False):
+            pooled = x.float().mean((2, 3))
+            coord = nn.functional.linear(pooled, self.fc.weight.float(), self.fc.bias.float()) * self.weight_dilate + centre
+            coord = torch.clamp(coord, 0, self.weight_shape[0] - 1)
+            # the operator adds the tap's own position and the centring term back (K.cu:338-341)
+            rotation = (coord - centre).to(x.dtype)
+        size = lambda v: (v, v) if isinstance(v, int) else tuple(v)
+        stride, padding, dilation = size(self.stride), size(self.padding), size(self.dilation)
+        ho = (x.size(2) + 2 * padding[0] - dilation[0] * (self.kernel_size - 1) - 1) // stride[0] + 1
+        wo = (x.size(3) + 2 * padding[1] - dilation[1] * (self.kernel_size - 1) - 1) // stride[1] + 1
+        rotation = rotation.view(n, taps * 2, 1, 1).expand(n, taps * 2, ho, wo).contiguous()
+        weight = self.weight.to(x.dtype)
+        return sample_depthwise(x, rotation, weight, (self.kernel_size, self.kernel_size), stride, padding,
+                                dilation, 1)
+
     def forward(self, x):
+        if self._fusable(x):
+            return self._forward_fused(x)
         n, c, h, w = x.shape
         weight = self.dynamic_weight(x, self.weight).to(x.dtype)
         out = nn.functional.conv2d(

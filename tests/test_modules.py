@@ -169,6 +169,7 @@ def test_global_module_equals_local_operator_with_constant_rotation():
     dev = torch.device("cuda:0")
     N, C, S, k = 3, 10, 5, 3
     m = GlobalDeformKernel2d((S, S), C, C, kernel_size=k, padding=1, groups=C).to(dev)
+    m.fused = False  # the reference's route: nd_linear_sample + grouped convolution
     torch.nn.init.normal_(m.fc.weight, std=0.3)
     x = torch.randn(N, C, 9, 8, device=dev)
     out = m(x)
@@ -180,3 +181,13 @@ def test_global_module_equals_local_operator_with_constant_rotation():
     assert rel_err(out.detach().cpu(), want.cpu()) < 1e-5
     out.sum().backward()
     assert m.weight.grad is not None and m.fc.weight.grad is not None
+    # the fused route of the module (one call of the local operator): same output, same gradients
+    g_ref = [p.grad.clone() for p in (m.weight, m.fc.weight, m.fc.bias)]
+    m.zero_grad()
+    m.fused = True
+    x2 = x.clone().requires_grad_()
+    out2 = m(x2)
+    assert rel_err(out2.detach().cpu(), out.detach().cpu()) < 1e-5
+    out2.sum().backward()
+    for got, ref in zip((m.weight.grad, m.fc.weight.grad, m.fc.bias.grad), g_ref):
+        assert rel_err(got.cpu(), ref.cpu()) < 1e-4
