@@ -1,6 +1,6 @@
 // Shared device-side building blocks of the gfx950 deformable-kernel library:
 // element I/O for the four dtypes, the geometry block passed to every kernel,
-// and the per-(pixel, tap) sampling descriptors.
+// the XCD-aware block order, wave-level reductions and buffer-addressed plane access.
 //
 // Semantics follow the reference's device helpers in
 // deformable_kernels/ops/deform_kernel/csrc/filter_sample_depthwise_cuda_kernel.cu
@@ -71,82 +71,6 @@ __device__ __forceinline__ CT scope_coord(int f, CT r, double centre) {
     return t + static_cast<CT>(centre);
   else
     return static_cast<CT>(static_cast<double>(t) + centre);
-}
-
-// ---------------------------------------------------------------------------
-// Scope-tile sampling descriptor of one (pixel, tap): which 2x2 block of the
-// tile the sample falls in and the four bilinear coefficients.
-//
-// The tile is held ZERO-PADDED by one cell on every side: `cell` addresses the
-// block's top-left corner in a table of (scope_h + 2) rows of `row_stride`
-// entries, entry (i + 1, j + 1) holding tile[i][j].  With the padding, the
-// reference's four per-corner range tests (K.cu:71-78) need no branches: a
-// corner outside the tile reads a zero.  A sample outside the open box
-// (-1, scope_h) x (-1, scope_w) -- or a NaN coordinate -- contributes nothing
-// (K.cu:59, 80-82): its coefficients are forced to zero and its cell to 0.
-// ---------------------------------------------------------------------------
-template <typename CT>
-struct ScopeTap {
-  int cell;            // entry index of the top-left corner in the padded table
-  CT c00, c01, c10, c11;  // hh*hw, hh*lw, lh*hw, lh*lw
-};
-
-template <typename CT>
-__device__ __forceinline__ ScopeTap<CT> make_scope_tap(CT h, CT w, int scope_h, int scope_w,
-                                                       int row_stride, int cell_scale = 1) {
-  ScopeTap<CT> t;
-  const bool inside = (h > CT(-1)) && (w > CT(-1)) && (h < CT(scope_h)) && (w < CT(scope_w));
-  const CT hf = floor(h), wf = floor(w);
-  const CT lh = h - hf, lw = w - wf;
-  const CT hh = CT(1) - lh, hw = CT(1) - lw;
-  const int hl = inside ? static_cast<int>(hf) : -1;
-  const int wl = inside ? static_cast<int>(wf) : -1;
-  t.cell = ((hl + 1) * row_stride + (wl + 1)) * cell_scale;
-  t.c00 = inside ? hh * hw : CT(0);
-  t.c01 = inside ? hh * lw : CT(0);
-  t.c10 = inside ? lh * hw : CT(0);
-  t.c11 = inside ? lh * lw : CT(0);
-  return t;
-}
-
-// Image-plane sampling descriptor of one (pixel, tap) of the deformable
-// variant: top-left corner and four coefficients, each coefficient already
-// zero where its corner lies outside the image (K.cu:182-193), all zero when
-// the sample lies outside (-1, H) x (-1, W) (K.cu:500).  Corner k reads
-// plane[idx + {0, 1, W, W + 1}] at a clamped, always-legal index.
-template <typename CT>
-struct ImageTap {
-  int i00, i01, i10, i11;  // clamped element indices of the four corners
-  CT w00, w01, w10, w11;   // hh*hw, hh*lw, lh*hw, lh*lw, masked
-  CT lh, lw;               // fractional parts (for the coordinate gradient)
-  unsigned mask;           // bit k set when corner k is inside; 0 when the sample is outside
-};
-
-template <typename CT>
-__device__ __forceinline__ ImageTap<CT> make_image_tap(CT h, CT w, int H, int W) {
-  ImageTap<CT> t;
-  const bool inside = (h > CT(-1)) && (w > CT(-1)) && (h < CT(H)) && (w < CT(W));
-  const CT hf = floor(h), wf = floor(w);
-  const int hl = inside ? static_cast<int>(hf) : 0;
-  const int wl = inside ? static_cast<int>(wf) : 0;
-  const int hh_i = hl + 1, wh_i = wl + 1;
-  t.lh = h - hf;
-  t.lw = w - wf;
-  const CT hh = CT(1) - t.lh, hw = CT(1) - t.lw;
-  const bool top = inside && hl >= 0, bot = inside && hh_i <= H - 1;
-  const bool lef = wl >= 0, rig = wh_i <= W - 1;
-  t.mask = (top && lef ? 1u : 0u) | (top && rig ? 2u : 0u) | (bot && lef ? 4u : 0u) |
-           (bot && rig ? 8u : 0u);
-  const int hl_c = max(hl, 0), hh_c = min(hh_i, H - 1), wl_c = max(wl, 0), wh_c = min(wh_i, W - 1);
-  t.i00 = hl_c * W + wl_c;
-  t.i01 = hl_c * W + wh_c;
-  t.i10 = hh_c * W + wl_c;
-  t.i11 = hh_c * W + wh_c;
-  t.w00 = (t.mask & 1u) ? hh * hw : CT(0);
-  t.w01 = (t.mask & 2u) ? hh * t.lw : CT(0);
-  t.w10 = (t.mask & 4u) ? t.lh * hw : CT(0);
-  t.w11 = (t.mask & 8u) ? t.lh * t.lw : CT(0);
-  return t;
 }
 
 __host__ __device__ __forceinline__ int ceil_div(int a, int b) { return (a + b - 1) / b; }

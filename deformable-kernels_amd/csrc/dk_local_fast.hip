@@ -26,27 +26,6 @@ namespace {
 
 constexpr int kBlock = 256;
 
-// Zero-padded scope table of one channel: (SH + 2) rows of (SW + 2) entries.
-template <int SH, int SW>
-struct Table {
-  static constexpr int RS = SW + 2;
-  static constexpr int SIZE = (SH + 2) * RS;
-};
-
-template <typename T, int SH, int SW>
-__device__ __forceinline__ void stage_tables(float* tbl, const T* filter, int c_first, int c_step,
-                                             int nch) {
-  using Tb = Table<SH, SW>;
-  for (int e = threadIdx.x; e < nch * Tb::SIZE; e += blockDim.x) {
-    const int j = e / Tb::SIZE, r = e % Tb::SIZE;
-    const int i = r / Tb::RS - 1, k = r % Tb::RS - 1;
-    float v = 0.f;
-    if (i >= 0 && i < SH && k >= 0 && k < SW)
-      v = ld(filter + (size_t)(c_first + j * c_step) * (SH * SW) + i * SW + k);
-    tbl[e] = v;
-  }
-}
-
 // Geometry of tap (f_h, f_w) for the pixel this lane owns.
 //   forward (TRANSPOSED = false): the lane owns OUTPUT pixel (ph, pw); the tap reads input
 //     (ph*s - pad + f*d) and the rotation of the lane's own pixel (K.cu:315-336).
@@ -947,7 +926,7 @@ template void launch_reduce_partials<double, double>(const double*, int, int, do
 // ---------------------------------------------------------------------------
 namespace {
 
-constexpr int kMaxLdsTables = 96 * 1024;  // bytes of LDS a workgroup may spend on scope tables
+constexpr int kMaxLdsTables = 60 * 1024;  // bytes of LDS a workgroup may spend on scope tables (64 KB launch limit)
 
 // stride 1, unit column spacing and pad_w = 1: input and output planes share their width and a
 // pixel's taps are three runs of three consecutive elements
@@ -958,7 +937,7 @@ bool same_width_geometry(const Geo& g) {
 
 template <int SH, int SW>
 int channels_per_block(int cpg, int wanted_splits) {
-  const int fit = kMaxLdsTables / (Table<SH, SW>::SIZE * 4);
+  const int fit = kMaxLdsTables / (WideTable<SH, SW>::SIZE * 4) - 2 * kUnroll;
   int per = ceil_div(cpg, wanted_splits);
   if (per > fit) per = fit;
   if (per < 1) per = 1;

@@ -30,6 +30,7 @@ TUNED = [
     (1, 272, 12, 12, 3, (3, 3), 1, 1, 1, 1, 1.0),   # more than 256 channels: two channel splits of the matrix-core grad filter
     (2, 10, 16, 18, 3, (4, 4), 2, 0, 1, 1, 1.0),    # stride 2 without padding, even sizes (tap parity of grad input)
     (2, 8, 70, 40, 3, (4, 4), 1, 1, 1, 1, 0.7),     # 2800-pixel planes: many tiles per image, partial last tile
+    (1, 600, 40, 64, 3, (5, 5), 1, 1, 1, 1, 1.0),   # 600 channels x 36-block tables: more than one block's LDS, scope 5
 ]
 GENERIC = [
     (2, 6, 9, 8, (5, 3), (7, 4), (1, 2), (2, 0), 1, 3, 0.7),
