@@ -290,6 +290,128 @@ __global__ __launch_bounds__(kBlock, 2) void local_gather_rows_kernel(Geo g, con
 }
 
 // ---------------------------------------------------------------------------
+// forward for stride 2 (3 x 3 taps, undilated, padding 1, even input width): the three taps of a
+// row read input columns 2 ow - 1, 2 ow, 2 ow + 1.  A lane loads the PAIR (2 ow, 2 ow + 1) of each
+// tap row with one 8-byte load (4-byte for the 16-bit types) and takes column 2 ow - 1 from the
+// previous lane's pair through the DPP-fused multiply-add: 3 loads per channel instead of 9
+// strided ones.  A wave covers 63 pixels with lanes 1..63 plus the halo lane 0.  Taps in the
+// padding (row -1, column -1) get the zero scope block; their loads are redirected to element 0.
+// grid = (pixel tiles of kS2Pix, channel splits, batch * groups)
+// ---------------------------------------------------------------------------
+constexpr int kS2Lanes = 63;
+constexpr int kS2Pix = kS2Lanes * (kBlock / 64);
+
+template <typename T> struct Pair;
+template <> struct Pair<float> {
+  typedef float raw __attribute__((ext_vector_type(2), aligned(4)));
+  static __device__ __forceinline__ float get(const raw& v, int k) { return v[k]; }
+};
+template <> struct Pair<__half> {
+  typedef _Float16 raw __attribute__((ext_vector_type(2), aligned(2)));
+  static __device__ __forceinline__ float get(const raw& v, int k) { return static_cast<float>(v[k]); }
+};
+template <> struct Pair<bf16_t> {
+  typedef unsigned short raw __attribute__((ext_vector_type(2), aligned(2)));
+  static __device__ __forceinline__ float get(const raw& v, int k) { return __uint_as_float(static_cast<uint32_t>(v[k]) << 16); }
+};
+
+template <typename T, int SH, int SW>
+__global__ __launch_bounds__(kBlock, 2) void local_forward_s2_kernel(Geo g, const T* __restrict__ x,
+                                                                     const T* __restrict__ rot,
+                                                                     const T* __restrict__ filter,
+                                                                     T* __restrict__ out, int ch_per_block) {
+  using Tb = WideTable<SH, SW>;
+  constexpr int KH = 3, KW = 3, K = 9;
+  extern __shared__ __align__(16) float tbl[];
+
+  const int cpg = g.channel / g.groups;
+  const int out_plane = g.out_h * g.out_w, in_plane = g.in_h * g.in_w;
+  const int tiles = ceil_div(out_plane, kS2Pix), splits = ceil_div(cpg, ch_per_block);
+  const int total = tiles * splits * g.batch * g.groups;
+  const int lb = logical_block(total);
+  if (lb >= total) return;
+  const int bx = lb % tiles, by = lb / tiles % splits, bz = lb / tiles / splits;
+  const int n = bz / g.groups, grp = bz % g.groups;
+  const int j0 = by * ch_per_block;
+  const int nch = min(ch_per_block, cpg - j0);
+  stage_wide_tables<T, SH, SW>(tbl, filter, g.channel, grp + g.groups * j0, g.groups, nch);
+
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int p = bx * kS2Pix + wave * kS2Lanes + lane - 1;  // lane 0 is the halo: the pixel before the wave's first
+  const bool owns = lane >= 1 && p < out_plane;
+  const int pc = min(max(p, 0), out_plane - 1);  // halo and tail lanes load some valid pixel's pairs
+  const int ph = pc / g.out_w, pw = pc % g.out_w;
+
+  // first element of the pair of tap row r (element 0 when the row is in the padding)
+  int pe[KH];
+#pragma unroll
+  for (int r = 0; r < KH; ++r) {
+    const int ih = 2 * ph - 1 + r;
+    pe[r] = (ih >= 0 && ih < g.in_h) ? ih * g.in_w + 2 * pw : 0;
+  }
+
+  LiteTap tap[K];
+  const rsrc_t rr = plane_rsrc(rot + (size_t)(n * g.groups + grp) * (K * 2) * out_plane, K * 2 * out_plane);
+#pragma unroll
+  for (int t = 0; t < K; ++t) {
+    const int f_h = t / KW, f_w = t % KW;
+    int s_el, rpix;
+    const bool ok = tap_geometry<false>(g, ph, pw, f_h, f_w, s_el, rpix) && owns;
+    const unsigned ro = ok ? (unsigned)((2 * t) * out_plane + rpix) * (unsigned)sizeof(T) : kOutOfRange;
+    const float r_h = buf_ld(rr, ro, rot);
+    const float r_w = buf_ld(rr, ro + (unsigned)out_plane * (unsigned)sizeof(T), rot);
+    tap[t] = make_lite_tap<SH, SW>(scope_coord<float>(f_h, r_h, g.centre_h),
+                                   scope_coord<float>(f_w, r_w, g.centre_w), ok);
+  }
+  __syncthreads();
+
+  const size_t chan0 = (size_t)n * g.channel + grp + (size_t)g.groups * j0;
+  const T* sp = x + chan0 * in_plane;
+  T* dp = out + chan0 * out_plane;
+  const size_t s_step = (size_t)g.groups * in_plane, d_step = (size_t)g.groups * out_plane;
+  const unsigned doff = owns ? (unsigned)p * (unsigned)sizeof(T) : kOutOfRange;
+
+  typedef typename Pair<T>::raw pair_t;
+  auto load_stage = [&](pair_t (&xc)[kUnroll][KH], int jb) {
+#pragma unroll
+    for (int u = 0; u < kUnroll; ++u) {
+      const T* plane = sp + (size_t)min(jb + u, nch - 1) * s_step;  // past the last channel: reload it, the store is dropped
+#pragma unroll
+      for (int r = 0; r < KH; ++r) xc[u][r] = *reinterpret_cast<const pair_t*>(plane + pe[r]);
+    }
+  };
+  auto compute_stage = [&](const pair_t (&xc)[kUnroll][KH], int jb) {
+    const float* tb = tbl + jb * Tb::SIZE;
+#pragma unroll
+    for (int u = 0; u < kUnroll; ++u) {
+      float acc = 0.f;
+#pragma unroll
+      for (int r = 0; r < KH; ++r) {
+        const float x0 = Pair<T>::get(xc[u][r], 0), x1 = Pair<T>::get(xc[u][r], 1);
+#pragma unroll
+        for (int f_w = 0; f_w < KW; ++f_w) {
+          const int t = r * KW + f_w;
+          const float4 q = *reinterpret_cast<const float4*>(tb + tap[t].cell + u * Tb::SIZE);
+          const float wt = lite_weight(tap[t], q);
+          // column 2 ow - 1 is the previous lane's second element
+          acc = f_w == 0 ? fma_lane_below(x1, wt, acc) : f_w == 1 ? fmaf(x0, wt, acc) : fmaf(x1, wt, acc);
+        }
+      }
+      buf_st(plane_rsrc(dp + (size_t)(jb + u) * d_step, (jb + u) < nch ? out_plane : 0), doff, acc, out);
+    }
+  };
+
+  pair_t xa[kUnroll][KH], xb[kUnroll][KH];
+  load_stage(xa, 0);
+  for (int j = 0; j < nch; j += 2 * kUnroll) {
+    load_stage(xb, j + kUnroll);
+    compute_stage(xa, j);
+    load_stage(xa, j + 2 * kUnroll);
+    compute_stage(xb, j + kUnroll);
+  }
+}
+
+// ---------------------------------------------------------------------------
 // grad rotation: the lane owns output pixel p of (n, group) and sums over channels.
 // With the block in difference form {a, b, c, d} the derivatives of the bilinear read are
 // d/dh = c + lw * d and d/dw = b + lh * d (K.cu:137-158 in corner form), with channel-independent
@@ -969,6 +1091,13 @@ bool run_gather(const Geo& g, bool transposed, const T* src, const T* rot, const
     return true;
   }
   const int per = channels_per_block<SH, SW>(cpg, pick_splits(g, pixels));
+  if (!transposed && g.stride_h == 2 && g.stride_w == 2 && g.dil_h == 1 && g.dil_w == 1 && g.pad_h == 1 &&
+      g.pad_w == 1 && g.in_w % 2 == 0 && !path_disabled("DK_NO_ROWS")) {
+    const unsigned grid2 = (unsigned)xcd_grid_size((long)ceil_div(pixels, kS2Pix) * ceil_div(cpg, per) * g.batch * g.groups);
+    const size_t lds2 = (size_t)(per + 2 * kUnroll) * WideTable<SH, SW>::SIZE * sizeof(float);
+    local_forward_s2_kernel<T, SH, SW><<<grid2, kBlock, lds2, stream>>>(g, src, rot, filter, dst, per);
+    return true;
+  }
   const unsigned grid = (unsigned)xcd_grid_size((long)ceil_div(pixels, kBlock) * ceil_div(cpg, per) * g.batch * g.groups);
   // stages past the last channel still read (and discard) table entries: pad to whole stages
   const size_t lds = (size_t)(per + 2 * kUnroll) * WideTable<SH, SW>::SIZE * sizeof(float);

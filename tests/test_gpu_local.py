@@ -31,6 +31,8 @@ TUNED = [
     (2, 10, 16, 18, 3, (4, 4), 2, 0, 1, 1, 1.0),    # stride 2 without padding, even sizes (tap parity of grad input)
     (2, 8, 70, 40, 3, (4, 4), 1, 1, 1, 1, 0.7),     # 2800-pixel planes: many tiles per image, partial last tile
     (1, 600, 40, 64, 3, (5, 5), 1, 1, 1, 1, 1.0),   # 600 channels x 36-block tables: more than one block's LDS, scope 5
+    (2, 12, 15, 16, 3, (4, 4), 2, 1, 1, 2, 1.0),    # stride 2, padding 1, even width: pair-load kernels; odd height, 2 groups
+    (1, 20, 40, 44, 3, (3, 3), 2, 1, 1, 1, 0.8),    # the same on 440-pixel output planes (two tiles), scope 3
 ]
 GENERIC = [
     (2, 6, 9, 8, (5, 3), (7, 4), (1, 2), (2, 0), 1, 3, 0.7),
