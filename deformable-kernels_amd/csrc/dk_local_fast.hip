@@ -430,20 +430,22 @@ __global__ __launch_bounds__(kBlock, 2) void local_forward_s2_kernel(Geo g, cons
 // result directly.
 // grid = (pixel tiles, splits, batch * groups)
 // ---------------------------------------------------------------------------
-template <typename T, int KH, int KW, int SH, int SW, bool ROWS>
+template <typename T, int KH, int KW, int SH, int SW, int MODE>
 __global__ __launch_bounds__(kBlock, 2) void local_grad_rotation_kernel(
     Geo g, const T* __restrict__ gout, const T* __restrict__ x, const T* __restrict__ rot,
     const T* __restrict__ filter, T* __restrict__ grot, float* __restrict__ partial, int splits,
     int ch_per_pass) {
   using Tb = WideTable<SH, SW>;
   constexpr int K = KH * KW;
-  constexpr int NLOAD = ROWS ? KH : K;  // input loads per channel
+  constexpr bool ROWS = MODE == 1, S2 = MODE == 2;  // MODE 0: one load per tap
+  constexpr int NLOAD = MODE == 0 ? K : KH;          // input loads per channel
+  constexpr int PIX = ROWS ? kRowPix : S2 ? kS2Pix : kBlock;  // pixels per workgroup
   extern __shared__ __align__(16) float tbl[];
 
   const int cpg = g.channel / g.groups;
   const int out_plane = g.out_h * g.out_w, in_plane = g.in_h * g.in_w;
   // logical block = (tile, channel split, image * group), tile fastest
-  const int tiles = ceil_div(out_plane, ROWS ? kRowPix : kBlock);
+  const int tiles = ceil_div(out_plane, PIX);
   const int total = tiles * splits * g.batch * g.groups;
   const int lb = logical_block(total);
   if (lb >= total) return;
@@ -452,8 +454,9 @@ __global__ __launch_bounds__(kBlock, 2) void local_grad_rotation_kernel(
   const int per_split = ceil_div(cpg, splits);
   const int c_begin = split * per_split, c_end = min(cpg, c_begin + per_split);
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int p = ROWS ? bx * kRowPix + wave * kRowLanes + lane - 1 : bx * kBlock + threadIdx.x;
-  const bool owns = (ROWS ? (lane >= 1 && lane <= kRowLanes) : true) && p < out_plane;
+  const int p = ROWS ? bx * kRowPix + wave * kRowLanes + lane - 1
+                : S2 ? bx * kS2Pix + wave * kS2Lanes + lane - 1 : bx * kBlock + threadIdx.x;
+  const bool owns = (ROWS ? (lane >= 1 && lane <= kRowLanes) : S2 ? lane >= 1 : true) && p < out_plane;
   const int pc = owns ? p : 0;
   const int ph = pc / g.out_w, pw = pc % g.out_w;
 
@@ -467,7 +470,7 @@ __global__ __launch_bounds__(kBlock, 2) void local_grad_rotation_kernel(
     const int f_h = t / KW, f_w = t % KW;
     int s_el, rpix;
     const bool ok = tap_geometry<false>(g, ph, pw, f_h, f_w, s_el, rpix) && owns;
-    if (!ROWS) soff[t] = ok ? (unsigned)s_el * (unsigned)sizeof(T) : kOutOfRange;
+    if (MODE == 0) soff[t] = ok ? (unsigned)s_el * (unsigned)sizeof(T) : kOutOfRange;
     const unsigned ro = owns ? (unsigned)((2 * t) * out_plane + pc) * (unsigned)sizeof(T) : kOutOfRange;
     const float h = scope_coord<float>(f_h, buf_ld(rr, ro, rot), g.centre_h);
     const float w = scope_coord<float>(f_w, buf_ld(rr, ro + (unsigned)out_plane * (unsigned)sizeof(T), rot),
@@ -482,6 +485,18 @@ __global__ __launch_bounds__(kBlock, 2) void local_grad_rotation_kernel(
     for (int r = 0; r < KH; ++r) {
       const long e = (long)p + (long)(r * g.dil_h - g.pad_h) * g.in_w;
       soff[r] = (e >= 0 && e < in_plane) ? (unsigned)e * (unsigned)sizeof(T) : kOutOfRange;
+    }
+  }
+  // S2: first element of the pair (columns 2 ow, 2 ow + 1) of tap row r, for the lane's pixel or,
+  // on halo and tail lanes, for some valid pixel (see local_forward_s2_kernel)
+  int pe[KH];
+  if (S2) {
+    const int pl = min(max(p, 0), out_plane - 1);
+    const int plh = pl / g.out_w, plw = pl % g.out_w;
+#pragma unroll
+    for (int r = 0; r < KH; ++r) {
+      const int ih = 2 * plh - 1 + r;
+      pe[r] = (ih >= 0 && ih < g.in_h) ? ih * g.in_w + 2 * plw : 0;
     }
   }
   const unsigned goff = owns ? (unsigned)p * (unsigned)sizeof(T) : kOutOfRange;
@@ -502,13 +517,21 @@ __global__ __launch_bounds__(kBlock, 2) void local_grad_rotation_kernel(
     const T* gp = gout + chan0 * out_plane;
     const size_t x_step = (size_t)g.groups * in_plane, g_step = (size_t)g.groups * out_plane;
 
+    typedef typename Pair<T>::raw pair_t;
     float xv[2][NLOAD], gv[2];
+    pair_t xq[2][KH];
     auto load = [&](int s, int j) {
-      const rsrc_t rx = plane_rsrc(xp + (size_t)j * x_step, j < nch ? in_plane : 0);
       const rsrc_t rg = plane_rsrc(gp + (size_t)j * g_step, j < nch ? out_plane : 0);
       gv[s] = buf_ld(rg, goff, gout);
+      if (S2) {
+        const T* plane = xp + (size_t)min(j, nch - 1) * x_step;  // past the last channel gv is 0
 #pragma unroll
-      for (int t = 0; t < NLOAD; ++t) xv[s][t] = buf_ld(rx, soff[t], x);
+        for (int r = 0; r < KH; ++r) xq[s][r] = *reinterpret_cast<const pair_t*>(plane + pe[r]);
+      } else {
+        const rsrc_t rx = plane_rsrc(xp + (size_t)j * x_step, j < nch ? in_plane : 0);
+#pragma unroll
+        for (int t = 0; t < NLOAD; ++t) xv[s][t] = buf_ld(rx, soff[t], x);
+      }
     };
     auto accumulate = [&](int s, int j) {
       // j == nch happens (odd nch) with zero inputs: that table is a stale or the zeroed spare one
@@ -519,6 +542,10 @@ __global__ __launch_bounds__(kBlock, 2) void local_grad_rotation_kernel(
         if (ROWS) {
           const int r = t / KW, f_w = t % KW;
           xt = f_w == 0 ? from_lane_below(xv[s][r]) : f_w == 1 ? xv[s][r] : from_lane_above(xv[s][r]);
+        } else if (S2) {
+          const int r = t / KW, f_w = t % KW;
+          const float x0 = Pair<T>::get(xq[s][r], 0), x1 = Pair<T>::get(xq[s][r], 1);
+          xt = f_w == 0 ? from_lane_below(x1) : f_w == 1 ? x0 : x1;
         } else {
           xt = xv[s][t];
         }
@@ -577,14 +604,15 @@ __global__ __launch_bounds__(kBlock, 2) void local_grad_rotation_kernel(
 // workgroup goes to the workspace; reduce_partials_kernel adds the partials in order.
 // grid = (parts, channel splits, groups)
 // ---------------------------------------------------------------------------
-template <typename T, int KH, int KW, int SH, int SW, bool ROWS>
+template <typename T, int KH, int KW, int SH, int SW, int MODE>
 __global__ __launch_bounds__(kBlock, 2) void local_grad_filter_kernel(
     Geo g, const T* __restrict__ gout, const T* __restrict__ x, const T* __restrict__ rot,
     float* __restrict__ partial, int tiles, int ch_per_block, int parts) {
   constexpr int K = KH * KW;
   constexpr int CELLS = SH * SW;
-  constexpr int NLOAD = ROWS ? KH : K;
-  constexpr int PIX = ROWS ? kRowPix : kBlock;  // pixels per (image, tile) item
+  constexpr bool ROWS = MODE == 1, S2 = MODE == 2;  // as in local_grad_rotation_kernel
+  constexpr int NLOAD = MODE == 0 ? K : KH;
+  constexpr int PIX = ROWS ? kRowPix : S2 ? kS2Pix : kBlock;  // pixels per (image, tile) item
   static_assert(CELLS <= 16, "the fold below handles up to 16 cells per 16-lane row");
   constexpr int kPitch = 20;  // floats per lane in the transpose scratch: 16-byte aligned, bank-skewed
   constexpr int kWaves = kBlock / 64;
@@ -617,8 +645,9 @@ __global__ __launch_bounds__(kBlock, 2) void local_grad_filter_kernel(
 
   for (int item = bx; item < items; item += parts) {
     const int n = item / tiles, tile = item % tiles;
-    const int p = ROWS ? tile * PIX + wave * kRowLanes + lane - 1 : tile * PIX + (int)threadIdx.x;
-    const bool owns = (ROWS ? (lane >= 1 && lane <= kRowLanes) : true) && p < out_plane;
+    const int p = ROWS ? tile * PIX + wave * kRowLanes + lane - 1
+                  : S2 ? tile * PIX + wave * kS2Lanes + lane - 1 : tile * PIX + (int)threadIdx.x;
+    const bool owns = (ROWS ? (lane >= 1 && lane <= kRowLanes) : S2 ? lane >= 1 : true) && p < out_plane;
     const int pc = owns ? p : 0;
     const int ph = pc / g.out_w, pw = pc % g.out_w;
 
@@ -630,7 +659,7 @@ __global__ __launch_bounds__(kBlock, 2) void local_grad_filter_kernel(
       const int f_h = t / KW, f_w = t % KW;
       int s_el, rpix;
       const bool ok = tap_geometry<false>(g, ph, pw, f_h, f_w, s_el, rpix) && owns;
-      if (!ROWS) soff[t] = ok ? (unsigned)s_el * (unsigned)sizeof(T) : kOutOfRange;
+      if (MODE == 0) soff[t] = ok ? (unsigned)s_el * (unsigned)sizeof(T) : kOutOfRange;
       const unsigned ro = ok ? (unsigned)((2 * t) * out_plane + rpix) * (unsigned)sizeof(T) : kOutOfRange;
       const float h = scope_coord<float>(f_h, buf_ld(rr, ro, rot), g.centre_h);
       const float w = scope_coord<float>(f_w, buf_ld(rr, ro + (unsigned)out_plane * (unsigned)sizeof(T), rot),
@@ -654,6 +683,16 @@ __global__ __launch_bounds__(kBlock, 2) void local_grad_filter_kernel(
         soff[r] = (e >= 0 && e < in_plane) ? (unsigned)e * (unsigned)sizeof(T) : kOutOfRange;
       }
     }
+    int pe[KH];  // S2: first element of the pair of tap row r (see local_forward_s2_kernel)
+    if (S2) {
+      const int pl = min(max(p, 0), out_plane - 1);
+      const int plh = pl / g.out_w, plw = pl % g.out_w;
+#pragma unroll
+      for (int r = 0; r < KH; ++r) {
+        const int ih = 2 * plh - 1 + r;
+        pe[r] = (ih >= 0 && ih < g.in_h) ? ih * g.in_w + 2 * plw : 0;
+      }
+    }
     const unsigned goff = owns ? (unsigned)p * (unsigned)sizeof(T) : kOutOfRange;
 
     const size_t chan0 = (size_t)n * g.channel + grp + (size_t)g.groups * j0;
@@ -661,13 +700,21 @@ __global__ __launch_bounds__(kBlock, 2) void local_grad_filter_kernel(
     const T* gp = gout + chan0 * out_plane;
     const size_t x_step = (size_t)g.groups * in_plane, g_step = (size_t)g.groups * out_plane;
 
+    typedef typename Pair<T>::raw pair_t;
     float xv[2][NLOAD], gv[2];
+    pair_t xq[2][KH];
     auto load = [&](int s, int j) {
-      const rsrc_t rx = plane_rsrc(xp + (size_t)j * x_step, j < nch ? in_plane : 0);
       const rsrc_t rg = plane_rsrc(gp + (size_t)j * g_step, j < nch ? out_plane : 0);
       gv[s] = buf_ld(rg, goff, gout);
+      if (S2) {
+        const T* plane = xp + (size_t)min(j, nch - 1) * x_step;  // past the last channel gv is 0
 #pragma unroll
-      for (int t = 0; t < NLOAD; ++t) xv[s][t] = buf_ld(rx, soff[t], x);
+        for (int r = 0; r < KH; ++r) xq[s][r] = *reinterpret_cast<const pair_t*>(plane + pe[r]);
+      } else {
+        const rsrc_t rx = plane_rsrc(xp + (size_t)j * x_step, j < nch ? in_plane : 0);
+#pragma unroll
+        for (int t = 0; t < NLOAD; ++t) xv[s][t] = buf_ld(rx, soff[t], x);
+      }
     };
     auto accumulate = [&](int s, int j) {
       float acc[SH][SW];
@@ -681,6 +728,10 @@ __global__ __launch_bounds__(kBlock, 2) void local_grad_filter_kernel(
         if (ROWS) {
           const int r = t / KW, f_w = t % KW;
           xt = f_w == 0 ? from_lane_below(xv[s][r]) : f_w == 1 ? xv[s][r] : from_lane_above(xv[s][r]);
+        } else if (S2) {
+          const int r = t / KW, f_w = t % KW;
+          const float x0 = Pair<T>::get(xq[s][r], 0), x1 = Pair<T>::get(xq[s][r], 1);
+          xt = f_w == 0 ? from_lane_below(x1) : f_w == 1 ? x0 : x1;
         } else {
           xt = xv[s][t];
         }
@@ -1075,6 +1126,13 @@ int pick_splits(const Geo& g, int planes_pixels) {
   return splits;
 }
 
+// stride 2 x 2, 3 x 3 undilated taps, padding 1, even input width: the pair-load kernels apply
+bool stride2_geometry(const Geo& g) {
+  return g.stride_h == 2 && g.stride_w == 2 && g.dil_h == 1 && g.dil_w == 1 && g.pad_h == 1 && g.pad_w == 1 &&
+         g.k_h == 3 && g.k_w == 3 && g.in_w % 2 == 0 && !path_disabled("DK_NO_ROWS");
+}
+int rotation_tile(const Geo& g) { return same_width_geometry(g) ? kRowPix : stride2_geometry(g) ? kS2Pix : kBlock; }
+
 template <typename T, int SH, int SW>
 bool run_gather(const Geo& g, bool transposed, const T* src, const T* rot, const T* filter, T* dst,
                 hipStream_t stream) {
@@ -1091,8 +1149,7 @@ bool run_gather(const Geo& g, bool transposed, const T* src, const T* rot, const
     return true;
   }
   const int per = channels_per_block<SH, SW>(cpg, pick_splits(g, pixels));
-  if (!transposed && g.stride_h == 2 && g.stride_w == 2 && g.dil_h == 1 && g.dil_w == 1 && g.pad_h == 1 &&
-      g.pad_w == 1 && g.in_w % 2 == 0 && !path_disabled("DK_NO_ROWS")) {
+  if (!transposed && stride2_geometry(g)) {
     const unsigned grid2 = (unsigned)xcd_grid_size((long)ceil_div(pixels, kS2Pix) * ceil_div(cpg, per) * g.batch * g.groups);
     const size_t lds2 = (size_t)(per + 2 * kUnroll) * WideTable<SH, SW>::SIZE * sizeof(float);
     local_forward_s2_kernel<T, SH, SW><<<grid2, kBlock, lds2, stream>>>(g, src, rot, filter, dst, per);
@@ -1114,7 +1171,7 @@ bool run_gather(const Geo& g, bool transposed, const T* src, const T* rot, const
 // block per CU, else enough for four per CU with at least 16 channels per split.
 int rotation_splits(const Geo& g) {
   const int cpg = g.channel / g.groups;
-  const long base = (long)ceil_div(g.out_h * g.out_w, same_width_geometry(g) ? kRowPix : kBlock) * g.batch * g.groups;
+  const long base = (long)ceil_div(g.out_h * g.out_w, rotation_tile(g)) * g.batch * g.groups;
   if (base >= 256) return 1;  // measured: at one block per CU and more, splitting does not pay
   const long want = (1024 + base - 1) / base;
   return (int)std::max<long>(1, std::min<long>(want, cpg / 16));
@@ -1128,13 +1185,13 @@ bool run_grad_rotation(const Geo& g, const T* gout, const T* x, const T* rot, co
   const int splits = rotation_splits(g);
   const int per = std::min(ceil_div(cpg, splits), 36);  // channels staged per pass
   const size_t lds = (size_t)(per + 1) * Tb::SIZE * sizeof(float);
-  if (same_width_geometry(g)) {
-    const unsigned grid = (unsigned)xcd_grid_size((long)ceil_div(g.out_h * g.out_w, kRowPix) * splits * g.batch * g.groups);
-    local_grad_rotation_kernel<T, 3, 3, SH, SW, true><<<grid, kBlock, lds, stream>>>(g, gout, x, rot, filter, grot, ws, splits, per);
-  } else {
-    const unsigned grid = (unsigned)xcd_grid_size((long)ceil_div(g.out_h * g.out_w, kBlock) * splits * g.batch * g.groups);
-    local_grad_rotation_kernel<T, 3, 3, SH, SW, false><<<grid, kBlock, lds, stream>>>(g, gout, x, rot, filter, grot, ws, splits, per);
-  }
+  const unsigned grid = (unsigned)xcd_grid_size((long)ceil_div(g.out_h * g.out_w, rotation_tile(g)) * splits * g.batch * g.groups);
+  if (same_width_geometry(g))
+    local_grad_rotation_kernel<T, 3, 3, SH, SW, 1><<<grid, kBlock, lds, stream>>>(g, gout, x, rot, filter, grot, ws, splits, per);
+  else if (stride2_geometry(g))
+    local_grad_rotation_kernel<T, 3, 3, SH, SW, 2><<<grid, kBlock, lds, stream>>>(g, gout, x, rot, filter, grot, ws, splits, per);
+  else
+    local_grad_rotation_kernel<T, 3, 3, SH, SW, 0><<<grid, kBlock, lds, stream>>>(g, gout, x, rot, filter, grot, ws, splits, per);
   if (splits > 1)
     launch_reduce_partials<float, T>(ws, splits, g.batch * g.groups * 18 * g.out_h * g.out_w, grot, stream);
   return true;
@@ -1181,7 +1238,7 @@ FilterGrid filter_grid(const Geo& g) {
   }
   f.splits = ceil_div(cpg, kFilterChPerBlock);
   f.per = ceil_div(cpg, f.splits);
-  f.tiles = ceil_div(g.out_h * g.out_w, same_width_geometry(g) ? kRowPix : kBlock);
+  f.tiles = ceil_div(g.out_h * g.out_w, rotation_tile(g));
   const int items = g.batch * f.tiles;
   // one (image, tile) item per workgroup while that keeps the partial buffer small; many more
   // workgroups than the GPU holds at once, so the dispatcher evens out the load
@@ -1205,9 +1262,11 @@ bool run_grad_filter(const Geo& g, const T* gout, const T* x, const T* rot, T* g
     }
     const size_t lds = ((size_t)(kBlock / 64) * f.per * 16 + (size_t)(kBlock / 64) * 64 * 20) * sizeof(float);
     if (same_width_geometry(g))
-      local_grad_filter_kernel<T, 3, 3, SH, SW, true><<<grid, kBlock, lds, stream>>>(g, gout, x, rot, ws, f.tiles, f.per, f.parts);
+      local_grad_filter_kernel<T, 3, 3, SH, SW, 1><<<grid, kBlock, lds, stream>>>(g, gout, x, rot, ws, f.tiles, f.per, f.parts);
+    else if (stride2_geometry(g))
+      local_grad_filter_kernel<T, 3, 3, SH, SW, 2><<<grid, kBlock, lds, stream>>>(g, gout, x, rot, ws, f.tiles, f.per, f.parts);
     else
-      local_grad_filter_kernel<T, 3, 3, SH, SW, false><<<grid, kBlock, lds, stream>>>(g, gout, x, rot, ws, f.tiles, f.per, f.parts);
+      local_grad_filter_kernel<T, 3, 3, SH, SW, 0><<<grid, kBlock, lds, stream>>>(g, gout, x, rot, ws, f.tiles, f.per, f.parts);
     launch_reduce_partials<float, T>(ws, f.parts, g.channel * SH * SW, gfilter, stream);
     return true;
   }
