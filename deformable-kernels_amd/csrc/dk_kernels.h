@@ -20,7 +20,7 @@ namespace dk {
 inline bool path_disabled(const char* name) { return std::getenv(name) != nullptr; }
 
 template <typename CT, typename T>
-void launch_reduce_partials(const CT* partial, int parts, int count, T* out, hipStream_t stream);
+void launch_reduce_partials(const CT* partial, int parts, long count, T* out, hipStream_t stream);
 
 // ---- tuned local path (dk_local_fast.hip): 3x3 taps, scope 3x3 / 4x4 / 5x5, fp32/fp16/bf16
 template <typename T>

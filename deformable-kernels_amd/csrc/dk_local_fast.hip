@@ -1085,14 +1085,29 @@ __global__ __launch_bounds__(kRedEl * kRedSlices) void reduce_partials_kernel(
   }
 }
 
+// The same sum for few parts of many elements (channel splits of a gradient image): one
+// element per thread, parts added in order, coalesced.
 template <typename CT, typename T>
-void launch_reduce_partials(const CT* partial, int parts, int count, T* out, hipStream_t stream) {
-  reduce_partials_kernel<CT, T><<<ceil_div(count, kRedEl), kRedEl * kRedSlices, 0, stream>>>(partial, parts, count, out);
+__global__ __launch_bounds__(kBlock) void reduce_few_parts_kernel(const CT* __restrict__ partial, int parts,
+                                                                  long count, T* __restrict__ out) {
+  const long e = (long)blockIdx.x * kBlock + threadIdx.x;
+  if (e >= count) return;
+  CT s = partial[e];
+  for (int q = 1; q < parts; ++q) s += partial[(size_t)q * count + e];
+  st(out + e, s);
 }
-template void launch_reduce_partials<float, float>(const float*, int, int, float*, hipStream_t);
-template void launch_reduce_partials<float, __half>(const float*, int, int, __half*, hipStream_t);
-template void launch_reduce_partials<float, bf16_t>(const float*, int, int, bf16_t*, hipStream_t);
-template void launch_reduce_partials<double, double>(const double*, int, int, double*, hipStream_t);
+
+template <typename CT, typename T>
+void launch_reduce_partials(const CT* partial, int parts, long count, T* out, hipStream_t stream) {
+  if (parts <= kRedSlices && count >= 16384)
+    reduce_few_parts_kernel<CT, T><<<(unsigned)((count + kBlock - 1) / kBlock), kBlock, 0, stream>>>(partial, parts, count, out);
+  else
+    reduce_partials_kernel<CT, T><<<(unsigned)((count + kRedEl - 1) / kRedEl), kRedEl * kRedSlices, 0, stream>>>(partial, parts, (int)count, out);
+}
+template void launch_reduce_partials<float, float>(const float*, int, long, float*, hipStream_t);
+template void launch_reduce_partials<float, __half>(const float*, int, long, __half*, hipStream_t);
+template void launch_reduce_partials<float, bf16_t>(const float*, int, long, bf16_t*, hipStream_t);
+template void launch_reduce_partials<double, double>(const double*, int, long, double*, hipStream_t);
 
 // ---------------------------------------------------------------------------
 // host-side dispatch of the tuned path
@@ -1167,13 +1182,12 @@ bool run_gather(const Geo& g, bool transposed, const T* src, const T* rot, const
   return true;
 }
 
-// Channel splits of the grad-rotation grid: 1 when the (tile, image, group) blocks alone give a
-// block per CU, else enough for four per CU with at least 16 channels per split.
+// Channel splits of the grad-rotation grid: enough for about four blocks per CU with at least
+// 16 channels per split.
 int rotation_splits(const Geo& g) {
   const int cpg = g.channel / g.groups;
   const long base = (long)ceil_div(g.out_h * g.out_w, rotation_tile(g)) * g.batch * g.groups;
-  if (base >= 256) return 1;  // measured: at one block per CU and more, splitting does not pay
-  const long want = (1024 + base - 1) / base;
+  const long want = 1024 / base;  // measured: about four blocks per CU is the best grid
   return (int)std::max<long>(1, std::min<long>(want, cpg / 16));
 }
 
@@ -1193,7 +1207,7 @@ bool run_grad_rotation(const Geo& g, const T* gout, const T* x, const T* rot, co
   else
     local_grad_rotation_kernel<T, 3, 3, SH, SW, 0><<<grid, kBlock, lds, stream>>>(g, gout, x, rot, filter, grot, ws, splits, per);
   if (splits > 1)
-    launch_reduce_partials<float, T>(ws, splits, g.batch * g.groups * 18 * g.out_h * g.out_w, grot, stream);
+    launch_reduce_partials<float, T>(ws, splits, (long)g.batch * g.groups * 18 * g.out_h * g.out_w, grot, stream);
   return true;
 }
 
