@@ -23,6 +23,9 @@ int make_geo(const dk_conv_desc* d, Geo& g) {
       d->dil_h <= 0 || d->dil_w <= 0 || d->scope_h <= 0 || d->scope_w <= 0 || d->groups <= 0)
     return DK_ERR_BAD_SHAPE;
   if (d->channel % d->groups != 0) return DK_ERR_BAD_SHAPE;
+  if (d->rotation_clip < DK_CLIP_NONE || d->rotation_clip > DK_CLIP_COORD ||
+      (d->rotation_clip != DK_CLIP_NONE && !(d->clip_min <= d->clip_max)))
+    return DK_ERR_BAD_SHAPE;
   // K.cpp:42-43
   const long oh = ((long)d->in_h + 2L * d->pad_h - ((long)d->dil_h * (d->k_h - 1) + 1)) / d->stride_h + 1;
   const long ow = ((long)d->in_w + 2L * d->pad_w - ((long)d->dil_w * (d->k_w - 1) + 1)) / d->stride_w + 1;
@@ -55,6 +58,9 @@ int make_geo(const dk_conv_desc* d, Geo& g) {
   g.groups = d->groups;
   g.centre_h = (d->scope_h - d->k_h) / 2.0;  // K.cu:338-341
   g.centre_w = (d->scope_w - d->k_w) / 2.0;
+  g.clip_mode = d->rotation_clip;
+  g.clip_lo = d->clip_min;
+  g.clip_hi = d->clip_max;
   return DK_OK;
 }
 

@@ -54,7 +54,16 @@ struct Geo {
   int out_h, out_w;
   int scope_h, scope_w, groups;
   double centre_h, centre_w;  // (scope - k) / 2.0, the double literal of K.cu:338-341
+  int clip_mode;              // kClipNone / kClipRotation / kClipCoord
+  float clip_lo, clip_hi;
 };
+
+// Clamp of the kernel-space offsets, folded into the operator.  The reference clamps the rotation
+// tensor in its module before the operator runs (modules/deform_kernel.py:185-212): a plain
+// range on the offsets (kClipRotation), or "scope", a range on the scope coordinate
+// f + r + centre (kClipCoord, with [0, scope_h - 1] for both axes as written there).  The
+// gradient with respect to a clamped offset is zero, as torch.clamp's is.
+enum { kClipNone = 0, kClipRotation = 1, kClipCoord = 2 };
 
 // Scope coordinate of tap f with kernel-space offset r.  The reference writes
 // `f + r + (scope - k) / 2.0`: int + scalar_t in scalar_t, then + double in
@@ -71,6 +80,26 @@ __device__ __forceinline__ CT scope_coord(int f, CT r, double centre) {
     return t + static_cast<CT>(centre);
   else
     return static_cast<CT>(static_cast<double>(t) + centre);
+}
+
+// The same with the descriptor's clamp applied; `open` tells whether the offset was inside the
+// range (its gradient passes) or clamped (gradient zero).
+template <typename CT>
+__device__ __forceinline__ CT scope_coord(const Geo& g, int f, CT r, double centre, bool* open = nullptr) {
+  bool inside = true;
+  if (g.clip_mode == kClipRotation) {
+    inside = r >= static_cast<CT>(g.clip_lo) && r <= static_cast<CT>(g.clip_hi);
+    r = r < static_cast<CT>(g.clip_lo) ? static_cast<CT>(g.clip_lo) : r;
+    r = r > static_cast<CT>(g.clip_hi) ? static_cast<CT>(g.clip_hi) : r;
+  }
+  CT c = scope_coord<CT>(f, r, centre);
+  if (g.clip_mode == kClipCoord) {
+    inside = c >= static_cast<CT>(g.clip_lo) && c <= static_cast<CT>(g.clip_hi);
+    c = c < static_cast<CT>(g.clip_lo) ? static_cast<CT>(g.clip_lo) : c;
+    c = c > static_cast<CT>(g.clip_hi) ? static_cast<CT>(g.clip_hi) : c;
+  }
+  if (open) *open = inside;
+  return c;
 }
 
 __host__ __device__ __forceinline__ int ceil_div(int a, int b) { return (a + b - 1) / b; }

@@ -66,8 +66,8 @@ __device__ __forceinline__ void deform_taps(const Geo& g, const T* off, const T*
     it[t].pidx = hit ? (static_cast<int>(hf) + 1) * RS + static_cast<int>(wf) + 1 : 0;
     it[t].lh = hit ? h - hf : 0.f;
     it[t].lw = hit ? w - wf : 0.f;
-    const float sh = scope_coord<float>(f_h, buf_ld(rr, o, rot), g.centre_h);
-    const float sw = scope_coord<float>(f_w, buf_ld(rr, o + step, rot), g.centre_w);
+    const float sh = scope_coord<float>(g, f_h, buf_ld(rr, o, rot), g.centre_h);
+    const float sw = scope_coord<float>(g, f_w, buf_ld(rr, o + step, rot), g.centre_w);
     sc[t].h = hit ? sh : -2.f;
     sc[t].w = hit ? sw : -2.f;
   }
@@ -299,10 +299,18 @@ __global__ __launch_bounds__(kDBlock, 2) void deform_grad_coord_kernel(
     const size_t img = ROTATION ? (size_t)(b.n * g.groups + b.grp) : (size_t)b.n;
     const size_t imgs = ROTATION ? (size_t)g.batch * g.groups : (size_t)g.batch;
     float* dst = partial + ((part * imgs + img) * (K9 * 2)) * out_plane + p;
+    const T* rp = rot + (size_t)(b.n * g.groups + b.grp) * (K9 * 2) * out_plane + p;
 #pragma unroll
     for (int t = 0; t < K9; ++t) {
-      const float dh = ROTATION ? fmaf(st[t].lw, s2[t], s1[t]) : s0[t];
-      const float dw = ROTATION ? fmaf(st[t].lh, s2[t], s0[t]) : s1[t];
+      float dh = ROTATION ? fmaf(st[t].lw, s2[t], s1[t]) : s0[t];
+      float dw = ROTATION ? fmaf(st[t].lh, s2[t], s0[t]) : s1[t];
+      if (ROTATION && g.clip_mode != kClipNone) {  // a clamped offset has no gradient
+        bool open_h, open_w;
+        scope_coord<float>(g, t / 3, ld(rp + (size_t)(2 * t) * out_plane), g.centre_h, &open_h);
+        scope_coord<float>(g, t % 3, ld(rp + (size_t)(2 * t + 1) * out_plane), g.centre_w, &open_w);
+        dh = open_h ? dh : 0.f;
+        dw = open_w ? dw : 0.f;
+      }
       dst[(size_t)(2 * t) * out_plane] = dh;
       dst[(size_t)(2 * t + 1) * out_plane] = dw;
     }

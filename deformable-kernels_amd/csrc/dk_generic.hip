@@ -173,8 +173,8 @@ __global__ __launch_bounds__(kBlock) void generic_forward_kernel(
         const CT xv = tap_input<T, CT, DEFORM>(g, xp, off, b, t, f_h, f_w, oh, ow, hit, ihf, iwf);
         if (hit) {
           const size_t ri = rot_index(g, b, grp, t, pix);
-          const CT h = scope_coord<CT>(f_h, ld(rot + ri), g.centre_h);
-          const CT w = scope_coord<CT>(f_w, ld(rot + ri + plane), g.centre_w);
+          const CT h = scope_coord<CT>(g, f_h, ld(rot + ri), g.centre_h);
+          const CT w = scope_coord<CT>(g, f_w, ld(rot + ri + plane), g.centre_w);
           sum += xv * tile_bilinear<T, CT>(tile, g.scope_h, g.scope_w, h, w);
         }
       }
@@ -210,8 +210,8 @@ __global__ __launch_bounds__(kBlock) void generic_local_grad_input_kernel(
         if (ow >= g.out_w) continue;
         const int t = f_h * g.k_w + f_w, opix = oh * g.out_w + ow;
         const size_t ri = rot_index(g, b, grp, t, opix);
-        const CT h = scope_coord<CT>(f_h, ld(rot + ri), g.centre_h);
-        const CT w = scope_coord<CT>(f_w, ld(rot + ri + oplane), g.centre_w);
+        const CT h = scope_coord<CT>(g, f_h, ld(rot + ri), g.centre_h);
+        const CT w = scope_coord<CT>(g, f_w, ld(rot + ri + oplane), g.centre_w);
         sum += ld(gp + opix) * tile_bilinear<T, CT>(tile, g.scope_h, g.scope_w, h, w);
       }
     }
@@ -239,8 +239,8 @@ __global__ __launch_bounds__(kBlock) void generic_deform_grad_input_kernel(
     if (!hit) continue;
     const int grp = c % g.groups;
     const size_t ri = rot_index(g, b, grp, t, pix);
-    const CT sh = scope_coord<CT>(f_h, ld(rot + ri), g.centre_h);
-    const CT sw = scope_coord<CT>(f_w, ld(rot + ri + oplane), g.centre_w);
+    const CT sh = scope_coord<CT>(g, f_h, ld(rot + ri), g.centre_h);
+    const CT sw = scope_coord<CT>(g, f_w, ld(rot + ri + oplane), g.centre_w);
     const CT ps = tile_bilinear<T, CT>(filter + (size_t)c * g.scope_h * g.scope_w, g.scope_h,
                                        g.scope_w, sh, sw) *
                   ld(gout + ((size_t)b * g.channel + c) * oplane + pix);
@@ -283,8 +283,9 @@ __global__ __launch_bounds__(kBlock) void generic_grad_rotation_kernel(
     const int oh = pix / g.out_w, ow = pix % g.out_w;
     const int f_h = t / g.k_w, f_w = t % g.k_w;
     const size_t ri = rot_index(g, b, grp, t, pix);
-    const CT h = scope_coord<CT>(f_h, ld(rot + ri), g.centre_h);
-    const CT w = scope_coord<CT>(f_w, ld(rot + ri + oplane), g.centre_w);
+    bool open_h, open_w;  // false: the offset was clamped, its gradient is zero
+    const CT h = scope_coord<CT>(g, f_h, ld(rot + ri), g.centre_h, &open_h);
+    const CT w = scope_coord<CT>(g, f_w, ld(rot + ri + oplane), g.centre_w, &open_w);
     CT gh = 0, gw = 0;
     bool hit;
     CT ihf, iwf;
@@ -302,8 +303,8 @@ __global__ __launch_bounds__(kBlock) void generic_grad_rotation_kernel(
         gw += ps * dw;
       }
     }
-    st(grot + ri, gh);
-    st(grot + ri + oplane, gw);
+    st(grot + ri, open_h ? gh : CT(0));
+    st(grot + ri + oplane, open_w ? gw : CT(0));
   }
 }
 
@@ -328,8 +329,8 @@ __global__ __launch_bounds__(kBlock) void generic_grad_offset_kernel(
       for (int c = 0; c < g.channel; ++c) {
         const int grp = c % g.groups;
         const size_t ri = rot_index(g, b, grp, t, pix);
-        const CT sh = scope_coord<CT>(f_h, ld(rot + ri), g.centre_h);
-        const CT sw = scope_coord<CT>(f_w, ld(rot + ri + oplane), g.centre_w);
+        const CT sh = scope_coord<CT>(g, f_h, ld(rot + ri), g.centre_h);
+        const CT sw = scope_coord<CT>(g, f_w, ld(rot + ri + oplane), g.centre_w);
         const CT ps = tile_bilinear<T, CT>(filter + (size_t)c * g.scope_h * g.scope_w, g.scope_h,
                                            g.scope_w, sh, sw) *
                       ld(gout + ((size_t)b * g.channel + c) * oplane + pix);
@@ -378,8 +379,8 @@ __global__ __launch_bounds__(kBlock) void generic_grad_filter_kernel(
           const CT xv = tap_input<T, CT, DEFORM>(g, xp, off, b, t, f_h, f_w, oh, ow, hit, ihf, iwf);
           if (!hit) continue;
           const size_t ri = rot_index(g, b, grp, t, pix);
-          const CT h = scope_coord<CT>(f_h, ld(rot + ri), g.centre_h);
-          const CT w = scope_coord<CT>(f_w, ld(rot + ri + oplane), g.centre_w);
+          const CT h = scope_coord<CT>(g, f_h, ld(rot + ri), g.centre_h);
+          const CT w = scope_coord<CT>(g, f_w, ld(rot + ri + oplane), g.centre_w);
           if (!(h > CT(-1) && w > CT(-1) && h < CT(S_h) && w < CT(S_w))) continue;
           const CT ps = xv * go;
           const CT hf = floor(h), wf = floor(w);

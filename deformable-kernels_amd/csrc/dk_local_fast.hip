@@ -121,8 +121,8 @@ __global__ __launch_bounds__(kBlock, 2) void local_gather_kernel(Geo g, const T*
     const unsigned ro = ok ? (unsigned)((2 * t) * out_plane + rpix) * (unsigned)sizeof(T) : kOutOfRange;
     const float r_h = buf_ld(rr, ro, rot);
     const float r_w = buf_ld(rr, ro + (unsigned)out_plane * (unsigned)sizeof(T), rot);
-    tap[slot] = make_lite_tap<SH, SW>(scope_coord<float>(f_h, r_h, g.centre_h),
-                                   scope_coord<float>(f_w, r_w, g.centre_w), ok);
+    tap[slot] = make_lite_tap<SH, SW>(scope_coord<float>(g, f_h, r_h, g.centre_h),
+                                   scope_coord<float>(g, f_w, r_w, g.centre_w), ok);
   }
   __syncthreads();
 
@@ -236,8 +236,8 @@ __global__ __launch_bounds__(kBlock, 2) void local_gather_rows_kernel(Geo g, con
     const unsigned ro = ok ? (unsigned)((2 * t) * out_plane + rpix) * (unsigned)sizeof(T) : kOutOfRange;
     const float r_h = buf_ld(rr, ro, rot);
     const float r_w = buf_ld(rr, ro + (unsigned)out_plane * (unsigned)sizeof(T), rot);
-    tap[t] = make_lite_tap<SH, SW>(scope_coord<float>(f_h, r_h, g.centre_h),
-                                   scope_coord<float>(f_w, r_w, g.centre_w), ok);  // !ok: tap in the padding
+    tap[t] = make_lite_tap<SH, SW>(scope_coord<float>(g, f_h, r_h, g.centre_h),
+                                   scope_coord<float>(g, f_w, r_w, g.centre_w), ok);  // !ok: tap in the padding
   }
   __syncthreads();
 
@@ -360,8 +360,8 @@ __global__ __launch_bounds__(kBlock, 2) void local_forward_s2_kernel(Geo g, cons
     const unsigned ro = ok ? (unsigned)((2 * t) * out_plane + rpix) * (unsigned)sizeof(T) : kOutOfRange;
     const float r_h = buf_ld(rr, ro, rot);
     const float r_w = buf_ld(rr, ro + (unsigned)out_plane * (unsigned)sizeof(T), rot);
-    tap[t] = make_lite_tap<SH, SW>(scope_coord<float>(f_h, r_h, g.centre_h),
-                                   scope_coord<float>(f_w, r_w, g.centre_w), ok);
+    tap[t] = make_lite_tap<SH, SW>(scope_coord<float>(g, f_h, r_h, g.centre_h),
+                                   scope_coord<float>(g, f_w, r_w, g.centre_w), ok);
   }
   __syncthreads();
 
@@ -472,8 +472,8 @@ __global__ __launch_bounds__(kBlock, 2) void local_grad_rotation_kernel(
     const bool ok = tap_geometry<false>(g, ph, pw, f_h, f_w, s_el, rpix) && owns;
     if (MODE == 0) soff[t] = ok ? (unsigned)s_el * (unsigned)sizeof(T) : kOutOfRange;
     const unsigned ro = owns ? (unsigned)((2 * t) * out_plane + pc) * (unsigned)sizeof(T) : kOutOfRange;
-    const float h = scope_coord<float>(f_h, buf_ld(rr, ro, rot), g.centre_h);
-    const float w = scope_coord<float>(f_w, buf_ld(rr, ro + (unsigned)out_plane * (unsigned)sizeof(T), rot),
+    const float h = scope_coord<float>(g, f_h, buf_ld(rr, ro, rot), g.centre_h);
+    const float w = scope_coord<float>(g, f_w, buf_ld(rr, ro + (unsigned)out_plane * (unsigned)sizeof(T), rot),
                                        g.centre_w);
     const bool in = (h > -1.f) && (w > -1.f) && (h < float(SH)) && (w < float(SW));
     cell[t] = Tb::slot(in ? (static_cast<int>(floorf(h)) + 1) * Tb::RS + static_cast<int>(floorf(w)) + 1 : 0) * 4;
@@ -571,13 +571,16 @@ __global__ __launch_bounds__(kBlock, 2) void local_grad_rotation_kernel(
   for (int t = 0; t < K; ++t) {
     const int f_h = t / KW, f_w = t % KW;
     const unsigned ro = owns ? (unsigned)((2 * t) * out_plane + pc) * (unsigned)sizeof(T) : kOutOfRange;
-    const float h = scope_coord<float>(f_h, buf_ld(rr, ro, rot), g.centre_h);
-    const float w = scope_coord<float>(f_w, buf_ld(rr, ro + (unsigned)out_plane * (unsigned)sizeof(T), rot),
-                                       g.centre_w);
+    bool open_h, open_w;  // false: the offset was clamped, its gradient is zero
+    const float h = scope_coord<float>(g, f_h, buf_ld(rr, ro, rot), g.centre_h, &open_h);
+    const float w = scope_coord<float>(g, f_w, buf_ld(rr, ro + (unsigned)out_plane * (unsigned)sizeof(T), rot),
+                                       g.centre_w, &open_w);
     const float lh = h - floorf(h), lw = w - floorf(w);
     float gh = fmaf(lw, sd[t], sc[t]);
     float gw = fmaf(lh, sd[t], sb[t]);
     if (!(inside >> t & 1u)) gh = gw = 0.f;
+    if (!open_h) gh = 0.f;
+    if (!open_w) gw = 0.f;
     if (splits == 1) {
       buf_st(ro_, ro, gh, grot);
       buf_st(ro_, ro + (unsigned)out_plane * (unsigned)sizeof(T), gw, grot);
@@ -661,8 +664,8 @@ __global__ __launch_bounds__(kBlock, 2) void local_grad_filter_kernel(
       const bool ok = tap_geometry<false>(g, ph, pw, f_h, f_w, s_el, rpix) && owns;
       if (MODE == 0) soff[t] = ok ? (unsigned)s_el * (unsigned)sizeof(T) : kOutOfRange;
       const unsigned ro = ok ? (unsigned)((2 * t) * out_plane + rpix) * (unsigned)sizeof(T) : kOutOfRange;
-      const float h = scope_coord<float>(f_h, buf_ld(rr, ro, rot), g.centre_h);
-      const float w = scope_coord<float>(f_w, buf_ld(rr, ro + (unsigned)out_plane * (unsigned)sizeof(T), rot),
+      const float h = scope_coord<float>(g, f_h, buf_ld(rr, ro, rot), g.centre_h);
+      const float w = scope_coord<float>(g, f_w, buf_ld(rr, ro + (unsigned)out_plane * (unsigned)sizeof(T), rot),
                                          g.centre_w);
       // hat(h - i) = lh at i = floor(h) + 1, 1 - lh at i = floor(h), else 0: the same products
       // (hh, lh) x (hw, lw) as K.cu:101-112, laid out densely; all zero outside (-1, S) and for
@@ -944,8 +947,8 @@ __global__ __launch_bounds__(kMfBlock, 4) void local_grad_filter_mfma_kernel(
           const int f_h = t / 3, f_w = t % 3;
           const int ih = ph + f_h * g.dil_h - g.pad_h, iw = pw + f_w - 1;
           const bool ok = live && ih >= 0 && ih < g.in_h && iw >= 0 && iw < W;
-          const float h = scope_coord<float>(f_h, r_rot[2 * k], g.centre_h);
-          const float w = scope_coord<float>(f_w, r_rot[2 * k + 1], g.centre_w);
+          const float h = scope_coord<float>(g, f_h, r_rot[2 * k], g.centre_h);
+          const float w = scope_coord<float>(g, f_w, r_rot[2 * k + 1], g.centre_w);
           const bool in = ok && (h > -1.f) && (w > -1.f) && (h < float(SH)) && (w < float(SW));
           hw[t * kMfPix + pix] = in ? make_float2(h, w) : make_float2(-2.f, -2.f);
         }

@@ -167,6 +167,9 @@ class LocalDeformKernel2d(nn.Module):
             kernel_size, stride, padding, dilation, bias=True)
         self.rotation_conv.zero_init = True
         self.rotation_clip = rotation_clip
+        # True: the operator clamps the offsets itself (same values and gradients as clamping
+        # the tensor first, without the extra passes over it); False: the reference's sequence
+        self.fused_clip = True
 
         self.inner_conv = SampleDepthwise(
             weight_shape, in_planes, out_planes, kernel_size=kernel_size, stride=stride,
@@ -192,6 +195,13 @@ class LocalDeformKernel2d(nn.Module):
 
     def forward(self, x):
         rotation = self.rotation_conv(x)
+        if self.rotation_clip is not None and self.fused_clip and self.weight_dilate == 1 \
+                and len(self.weight_shape) == 2:
+            clip = self.rotation_clip
+            if not (clip == 'scope' or isinstance(clip, dict) or
+                    (isinstance(clip, (tuple, list)) and len(clip) == 2)):
+                return self.inner_conv(x, self._clip_rotation(rotation))  # raises NotImplementedError
+            return self.inner_conv(x, rotation, clip)
         if self.rotation_clip is not None:
             rotation = self._clip_rotation(rotation)
         if self.weight_dilate != 1:

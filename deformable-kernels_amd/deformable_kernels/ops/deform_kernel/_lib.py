@@ -24,7 +24,8 @@ ND_MAX_DIMS = 8
 class ConvDesc(ctypes.Structure):
     _fields_ = [(n, ctypes.c_int32) for n in (
         "batch", "channel", "in_h", "in_w", "k_h", "k_w", "stride_h", "stride_w",
-        "pad_h", "pad_w", "dil_h", "dil_w", "scope_h", "scope_w", "groups", "dtype")]
+        "pad_h", "pad_w", "dil_h", "dil_w", "scope_h", "scope_w", "groups", "dtype", "rotation_clip")
+    ] + [("clip_min", ctypes.c_float), ("clip_max", ctypes.c_float)]
 
 
 class NdDesc(ctypes.Structure):
@@ -129,12 +130,35 @@ def workspace(nbytes, device):
     return buf, nbytes
 
 
-def conv_desc(input, weight, kernel_size, stride, padding, dilation, rotation_groups):
+CLIP_NONE, CLIP_ROTATION, CLIP_COORD = 0, 1, 2
+
+
+def clip_triple(rotation_clip, weight):
+    """(mode, min, max) of the descriptor for a module-level ``rotation_clip`` setting:
+    ``None``, a ``(min, max)`` pair / ``clamp`` kwargs dict on the offsets, or ``'scope'``
+    (scope coordinate kept inside ``[0, scope_h - 1]``, reference ``modules/deform_kernel.py:188-206``)."""
+    if rotation_clip is None:
+        return (CLIP_NONE, 0.0, 0.0)
+    if isinstance(rotation_clip, str):
+        if rotation_clip != 'scope':
+            raise NotImplementedError("rotation_clip must be a (min, max) pair or 'scope', got %r" % (rotation_clip,))
+        return (CLIP_COORD, 0.0, float(weight.size(2) - 1))
+    if isinstance(rotation_clip, dict):
+        lo, hi = rotation_clip.get('min'), rotation_clip.get('max')
+    else:
+        lo, hi = rotation_clip
+    lo = -float('inf') if lo is None else float(lo)
+    hi = float('inf') if hi is None else float(hi)
+    return (CLIP_ROTATION, lo, hi)
+
+
+def conv_desc(input, weight, kernel_size, stride, padding, dilation, rotation_groups, rotation_clip=None):
+    mode, lo, hi = clip_triple(rotation_clip, weight)
     return ConvDesc(
         input.size(0), input.size(1), input.size(2), input.size(3),
         int(kernel_size[0]), int(kernel_size[1]), int(stride[0]), int(stride[1]),
         int(padding[0]), int(padding[1]), int(dilation[0]), int(dilation[1]),
-        weight.size(2), weight.size(3), int(rotation_groups), dtype_tag(input))
+        weight.size(2), weight.size(3), int(rotation_groups), dtype_tag(input), mode, lo, hi)
 
 
 def nd_desc(data, coord):

@@ -12,6 +12,9 @@ Differences a user can observe:
   * tensors are validated (device, dtype, shape) and a failing native call
     raises instead of printing;
   * bfloat16 is accepted; fp16/bf16 accumulate in fp32;
+  * one optional trailing argument, ``rotation_clip`` (``None``, a ``(min, max)`` pair or
+    ``'scope'``): the clamp the reference's module applies to the rotation tensor before the
+    call (``modules/deform_kernel.py:185-212``), applied inside the kernels instead;
   * the ``apex.amp.float_function`` wrapper (``:209-211``) is replaced by an
     autocast-aware cast to fp32, apex not being a dependency.
 """
@@ -69,12 +72,14 @@ class SampleDepthwiseFunction(Function):
         padding=(1, 1),
         dilation=(1, 1),
         rotation_groups=1,
+        rotation_clip=None,
     ):
         ctx.kernel_size = kernel_size
         ctx.stride = stride
         ctx.padding = padding
         ctx.dilation = dilation
         ctx.rotation_groups = rotation_groups
+        ctx.rotation_clip = rotation_clip
 
         _lib.require_gpu(input, rotation, weight)
         out_size = _output_size(input, kernel_size, stride, padding, dilation)
@@ -82,7 +87,8 @@ class SampleDepthwiseFunction(Function):
         input, rotation, weight = input.contiguous(), rotation.contiguous(), weight.contiguous()
         ctx.save_for_backward(input, rotation, weight)
         output = input.new_empty(out_size)
-        desc = _lib.conv_desc(input, weight, kernel_size, stride, padding, dilation, rotation_groups)
+        desc = _lib.conv_desc(input, weight, kernel_size, stride, padding, dilation, rotation_groups,
+                              rotation_clip)
         with torch.cuda.device(input.device):
             _lib.check(_lib.lib().dk_sample_depthwise_forward(
                 desc, _lib.ptr(input), _lib.ptr(rotation), _lib.ptr(weight), _lib.ptr(output),
@@ -96,7 +102,7 @@ class SampleDepthwiseFunction(Function):
         _lib.require_gpu(grad_output, input)
         grad_output = grad_output.contiguous()
         desc = _lib.conv_desc(input, weight, ctx.kernel_size, ctx.stride, ctx.padding, ctx.dilation,
-                              ctx.rotation_groups)
+                              ctx.rotation_groups, ctx.rotation_clip)
         L = _lib.lib()
         with torch.cuda.device(input.device):
             s = _lib.stream_ptr(input)
@@ -115,7 +121,7 @@ class SampleDepthwiseFunction(Function):
                 desc, _lib.ptr(grad_output), _lib.ptr(input), _lib.ptr(rotation), _lib.ptr(weight),
                 _lib.ptr(grad_input), _lib.ptr(grad_rotation), _lib.ptr(grad_weight),
                 _lib.ptr(ws), nbytes, s), "sample_depthwise backward")
-        return (grad_input, grad_rotation, grad_weight,) + (None,) * 5
+        return (grad_input, grad_rotation, grad_weight,) + (None,) * 6
 
 
 class DeformableSampleDepthwiseFunction(Function):
@@ -131,12 +137,14 @@ class DeformableSampleDepthwiseFunction(Function):
         padding=(1, 1),
         dilation=(1, 1),
         rotation_groups=1,
+        rotation_clip=None,
     ):
         ctx.kernel_size = kernel_size
         ctx.stride = stride
         ctx.padding = padding
         ctx.dilation = dilation
         ctx.rotation_groups = rotation_groups
+        ctx.rotation_clip = rotation_clip
 
         _lib.require_gpu(input, offset, rotation, weight)
         out_size = _output_size(input, kernel_size, stride, padding, dilation)
@@ -145,7 +153,8 @@ class DeformableSampleDepthwiseFunction(Function):
         rotation, weight = rotation.contiguous(), weight.contiguous()
         ctx.save_for_backward(input, offset, rotation, weight)
         output = input.new_empty(out_size)
-        desc = _lib.conv_desc(input, weight, kernel_size, stride, padding, dilation, rotation_groups)
+        desc = _lib.conv_desc(input, weight, kernel_size, stride, padding, dilation, rotation_groups,
+                              rotation_clip)
         with torch.cuda.device(input.device):
             _lib.check(_lib.lib().dk_deformable_sample_depthwise_forward(
                 desc, _lib.ptr(input), _lib.ptr(offset), _lib.ptr(rotation), _lib.ptr(weight),
@@ -159,7 +168,7 @@ class DeformableSampleDepthwiseFunction(Function):
         _lib.require_gpu(grad_output, input)
         grad_output = grad_output.contiguous()
         desc = _lib.conv_desc(input, weight, ctx.kernel_size, ctx.stride, ctx.padding, ctx.dilation,
-                              ctx.rotation_groups)
+                              ctx.rotation_groups, ctx.rotation_clip)
         L = _lib.lib()
         p = _lib.ptr
         with torch.cuda.device(input.device):
@@ -192,7 +201,7 @@ class DeformableSampleDepthwiseFunction(Function):
                 _lib.check(L.dk_deformable_sample_depthwise_backward_filter(
                     desc, p(grad_output), p(input), p(offset), p(rotation), p(grad_weight),
                     p(ws), nbytes, s), "deform_sample_depthwise backward_filter")
-        return (grad_input, grad_offset, grad_rotation, grad_weight,) + (None,) * 5
+        return (grad_input, grad_offset, grad_rotation, grad_weight,) + (None,) * 6
 
 
 def _float_function(fn):

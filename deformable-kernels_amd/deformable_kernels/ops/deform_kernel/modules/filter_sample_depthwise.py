@@ -91,26 +91,27 @@ class _ScopeDepthwiseBase(nn.Module):
 
 
 class SampleDepthwise(_ScopeDepthwiseBase):
-    """Local deformable kernel: ``forward(input, rotation=None)``."""
+    """Local deformable kernel: ``forward(input, rotation=None)``.  ``rotation_clip`` (not in
+    the reference) has the operator clamp the offsets itself, see ``sample_depthwise``."""
 
-    def forward(self, input, rotation=None):
+    def forward(self, input, rotation=None, rotation_clip=None):
         if rotation is None:
             rotation = self._zeros_per_tap(input, self.rotation_groups)
         out = sample_depthwise(
             input, rotation, self.weight, self.kernel_size, self.stride,
-            self.padding, self.dilation, self.rotation_groups)
+            self.padding, self.dilation, self.rotation_groups, rotation_clip)
         return self._add_bias(out)
 
 
 class DeformableSampleDepthwise(_ScopeDepthwiseBase):
     """Deformable kernel with image-space offsets: ``forward(input, offset=None, rotation=None)``."""
 
-    def forward(self, input, offset=None, rotation=None):
+    def forward(self, input, offset=None, rotation=None, rotation_clip=None):
         if offset is None:
             offset = self._zeros_per_tap(input, 1)
         if rotation is None:
             rotation = self._zeros_per_tap(input, self.rotation_groups)
         out = deform_sample_depthwise(
             input, offset, rotation, self.weight, self.kernel_size,
-            self.stride, self.padding, self.dilation, self.rotation_groups)
+            self.stride, self.padding, self.dilation, self.rotation_groups, rotation_clip)
         return self._add_bias(out)

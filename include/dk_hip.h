@@ -50,6 +50,13 @@ typedef enum {
 
 typedef enum { DK_F32 = 0, DK_F16 = 1, DK_BF16 = 2, DK_F64 = 3 } dk_dtype;
 
+typedef enum dk_rotation_clip {
+  DK_CLIP_NONE = 0,
+  DK_CLIP_ROTATION = 1, /* offset r -> min(max(r, clip_min), clip_max)  (a (min, max) rotation_clip) */
+  DK_CLIP_COORD = 2     /* scope coordinate f + r + (scope - k) / 2 -> the same range, both axes
+                           (rotation_clip == 'scope': clip_min = 0, clip_max = scope_h - 1) */
+} dk_rotation_clip;
+
 /* Geometry of one depthwise deformable-kernel layer: the fields the
  * reference packs into SampleDepthwiseArgs (csrc/filter_sample_depthwise_cuda.h:1-28)
  * from the tensor sizes and the eleven ints of each pybind call; out_h/out_w
@@ -73,6 +80,13 @@ typedef struct dk_conv_desc {
   int32_t scope_h, scope_w;
   int32_t groups;           /* rotation groups ("sampling_group") */
   int32_t dtype;            /* dk_dtype of every tensor of the call */
+  /* Clamp of the kernel-space offsets applied inside the operator, so that a caller need not
+   * clamp (read, write, re-read) the rotation tensor first.  The reference's operators have no
+   * such argument: its module clamps the tensor beforehand (modules/deform_kernel.py:185-212,
+   * _clip_rotation).  DK_CLIP_NONE (0) reproduces the reference operator exactly.  The
+   * gradient with respect to a clamped offset is zero, as torch.clamp's is. */
+  int32_t rotation_clip;    /* dk_rotation_clip */
+  float clip_min, clip_max; /* the range; ignored for DK_CLIP_NONE */
 } dk_conv_desc;
 
 /* Output extent for the descriptor, or a negative dk_status. */

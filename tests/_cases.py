@@ -53,3 +53,21 @@ def rel_err(a, b):
     if scale == 0.0:
         return float((a - b).abs().max())
     return float((a - b).abs().max()) / scale
+
+
+def clipped_rotation(rot, clip, kernel_size, scope, groups):
+    """What the reference's module does to the rotation tensor before the operator
+    (modules/deform_kernel.py:185-212), restated on torch CPU tensors in the tensor's own
+    precision: returns (clamped rotation, mask of the entries that were NOT clamped)."""
+    if clip == 'scope':
+        kh, kw = kernel_size
+        bias = []
+        for h in range(kh):
+            for w in range(kw):
+                bias += [(scope[0] - (kh - 1) - 1) / 2.0 + h, (scope[1] - (kw - 1) - 1) / 2.0 + w]
+        bias = torch.tensor(bias, dtype=rot.dtype).repeat(groups)[None, :, None, None]
+        coord = rot + bias
+        open_ = (coord >= 0) & (coord <= scope[0] - 1)
+        return coord.clamp(0, scope[0] - 1) - bias, open_
+    lo, hi = clip
+    return rot.clamp(lo, hi), (rot >= lo) & (rot <= hi)

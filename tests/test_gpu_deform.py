@@ -11,7 +11,7 @@ import numpy as np
 import pytest
 import torch
 
-from _cases import make_deform, rel_err
+from _cases import clipped_rotation, make_deform, rel_err
 from oracle import dk_oracle as orc
 
 pytestmark = pytest.mark.gpu
@@ -78,6 +78,30 @@ def test_half_precisions_match_fp32_oracle(case, dtype):
     for g, w, name in zip(got, want, NAMES):
         assert g.dtype == dtype
         assert rel_err(g.float(), w) < 1e-2, name
+
+
+@pytest.mark.parametrize("clip", [(-0.5, 0.25), 'scope'])
+@pytest.mark.parametrize("case", [CASES[0], CASES[2], CASES[4], CASES[6]])
+def test_rotation_clip_inside_the_operator(case, clip):
+    # the operator clamping the kernel-space offsets itself == clamping the tensor first
+    from deformable_kernels.ops.deform_kernel.functions import deform_sample_depthwise
+    N, C, H, W, k, S, s, p, d, G, rs, os_ = case
+    x, wt, rot, off, gout, cfg = make_deform(N, C, H, W, k, S, s, p, d, G, 2.0 * rs, os_, seed=7)
+    dev = torch.device("cuda:0")
+    xg, og, rg, wg = [t.to(dev).requires_grad_() for t in (x, off, rot, wt)]
+    out = deform_sample_depthwise(xg, og, rg, wg, cfg["kernel_size"], cfg["stride"], cfg["padding"],
+                                  cfg["dilation"], cfg["groups"], clip)
+    out.backward(gout.to(dev))
+    got = [t.detach().cpu() for t in (out, xg.grad, og.grad, rg.grad, wg.grad)]
+    rot_c, open_ = clipped_rotation(rot, clip, cfg["kernel_size"], S, G)
+    assert 0.02 < 1.0 - open_.float().mean().item() < 0.9
+    inputs = (x, wt, rot_c, off, gout, cfg)
+    o32, o64 = _oracle(inputs, np.float32), _oracle(inputs, np.float64)
+    assert rel_err(got[0], o32[0]) < 1e-5, NAMES[0]
+    for i in (1, 2, 4):
+        assert rel_err(got[i], o64[i]) < 1e-4, NAMES[i]
+    assert rel_err(got[3], torch.as_tensor(o64[3]) * open_) < 1e-4, NAMES[3]
+    assert (got[3][~open_] == 0).all()
 
 
 def test_zero_image_offsets_equal_the_local_operator_on_gpu():

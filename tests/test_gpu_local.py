@@ -12,7 +12,7 @@ import numpy as np
 import pytest
 import torch
 
-from _cases import make_local, rel_err
+from _cases import clipped_rotation, make_local, rel_err
 from oracle import dk_oracle as orc
 
 pytestmark = pytest.mark.gpu
@@ -33,6 +33,7 @@ TUNED = [
     (1, 600, 40, 64, 3, (5, 5), 1, 1, 1, 1, 1.0),   # 600 channels x 36-block tables: more than one block's LDS, scope 5
     (2, 12, 15, 16, 3, (4, 4), 2, 1, 1, 2, 1.0),    # stride 2, padding 1, even width: pair-load kernels; odd height, 2 groups
     (1, 20, 40, 44, 3, (3, 3), 2, 1, 1, 1, 0.8),    # the same on 440-pixel output planes (two tiles), scope 3
+    (4, 64, 28, 28, 3, (4, 4), 1, 1, 1, 1, 1.0),    # grad rotation in 4 channel splits, summed by the few-parts reduction
 ]
 GENERIC = [
     (2, 6, 9, 8, (5, 3), (7, 4), (1, 2), (2, 0), 1, 3, 0.7),
@@ -93,6 +94,31 @@ def test_half_precisions_match_fp32_oracle(case, dtype):
     for g, w, name in zip(got, want, ("forward", "grad input", "grad rotation", "grad filter")):
         assert g.dtype == dtype
         assert rel_err(g.float(), w) < 1e-2, name
+
+
+@pytest.mark.parametrize("clip", [(-0.4, 0.3), 'scope'])
+@pytest.mark.parametrize("case", [TUNED[0], TUNED[2], TUNED[3], TUNED[5], GENERIC[0], GENERIC[1]])
+def test_rotation_clip_inside_the_operator(case, clip):
+    # the operator clamping the offsets itself == the reference's sequence (clamp the tensor,
+    # then the plain operator); the rotation gradient is zero where the clamp was active
+    from deformable_kernels.ops.deform_kernel.functions import sample_depthwise
+    N, C, H, W, k, S, s, p, d, G, rs = case
+    x, wt, rot, gout, cfg = make_local(N, C, H, W, k, S, s, p, d, G, 1.5 * rs, seed=5)
+    dev = torch.device("cuda:0")
+    xg, rg, wg = [t.to(dev).requires_grad_() for t in (x, rot, wt)]
+    out = sample_depthwise(xg, rg, wg, cfg["kernel_size"], cfg["stride"], cfg["padding"], cfg["dilation"],
+                           cfg["groups"], clip)
+    out.backward(gout.to(dev))
+    got = [t.detach().cpu() for t in (out, xg.grad, rg.grad, wg.grad)]
+    rot_c, open_ = clipped_rotation(rot, clip, cfg["kernel_size"], S, G)
+    assert 0.02 < 1.0 - open_.float().mean().item() < 0.9  # the clamp is active on a real share of the offsets
+    o32 = _oracle((x, wt, rot_c, gout, cfg), np.float32)
+    o64 = _oracle((x, wt, rot_c, gout, cfg), np.float64)
+    assert rel_err(got[0], o32[0]) < 1e-5, "forward"
+    assert rel_err(got[1], o32[1]) < 1e-5, "grad input"
+    assert rel_err(got[2], torch.as_tensor(o64[2]) * open_) < 1e-4, "grad rotation"
+    assert rel_err(got[3], o64[3]) < 1e-4, "grad filter"
+    assert (got[2][~open_] == 0).all()
 
 
 def test_taps_outside_the_scope_and_nan_free_borders():

@@ -93,6 +93,10 @@ def test_c_abi_rejects_bad_arguments_before_any_launch():
     assert L.dk_conv_out_size(ctypes.byref(too_small), None, None) == -2
     bad_dtype = _lib.ConvDesc(1, 4, 8, 8, 3, 3, 1, 1, 1, 1, 1, 1, 4, 4, 1, 9)
     assert L.dk_conv_out_size(ctypes.byref(bad_dtype), None, None) == -3
+    bad_clip = _lib.ConvDesc(1, 4, 8, 8, 3, 3, 1, 1, 1, 1, 1, 1, 4, 4, 1, _lib.DK_F32, 3, 0.0, 1.0)
+    assert L.dk_conv_out_size(ctypes.byref(bad_clip), None, None) == -2
+    empty_range = _lib.ConvDesc(1, 4, 8, 8, 3, 3, 1, 1, 1, 1, 1, 1, 4, 4, 1, _lib.DK_F32, 1, 1.0, 0.0)
+    assert L.dk_conv_out_size(ctypes.byref(empty_range), None, None) == -2
     huge = _lib.ConvDesc(4096, 4096, 512, 512, 3, 3, 1, 1, 1, 1, 1, 1, 4, 4, 1, _lib.DK_F32)
     assert L.dk_conv_out_size(ctypes.byref(huge), None, None) == -4
     # a workspace that is too small is refused
@@ -191,3 +195,31 @@ def test_global_module_equals_local_operator_with_constant_rotation():
     out2.sum().backward()
     for got, ref in zip((m.weight.grad, m.fc.weight.grad, m.fc.bias.grad), g_ref):
         assert rel_err(got.cpu(), ref.cpu()) < 1e-4
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("clip", ['scope', (-0.3, 0.2)])
+def test_local_module_clamps_inside_the_operator_as_the_reference_sequence_does(clip):
+    """LocalDeformKernel2d with rotation_clip: clamping inside the operator (fused_clip, the
+    default) against the reference's sequence of clamping the rotation tensor first
+    (modules/deform_kernel.py:185-221) -- same output, same gradients down to rotation_conv."""
+    from deformable_kernels.modules import LocalDeformKernel2d
+    torch.manual_seed(11)
+    dev = torch.device("cuda:0")
+    C = 12
+    m = LocalDeformKernel2d((4, 4), C, C, 3, 1, 1, 1, C, 2, False, clip).to(dev)
+    torch.nn.init.normal_(m.rotation_conv.weight, std=0.2)
+    x = torch.randn(2, C, 11, 10, device=dev)
+    gout = torch.randn(2, C, 11, 10, device=dev)
+    results = []
+    for fused in (False, True):
+        m.fused_clip = fused
+        m.zero_grad()
+        xi = x.clone().requires_grad_()
+        out = m(xi)
+        out.backward(gout)
+        results.append([t.detach().cpu().clone() for t in (
+            out, xi.grad, m.inner_conv.weight.grad, m.rotation_conv.weight.grad, m.rotation_conv.bias.grad)])
+    assert rel_err(results[1][0], results[0][0]) < 1e-5
+    for got, ref in zip(results[1][1:], results[0][1:]):
+        assert rel_err(got, ref) < 1e-4
