@@ -322,22 +322,34 @@ __global__ __launch_bounds__(kDBlock, 2) void deform_grad_coord_kernel(
 // the four input elements around its sample -- a scatter with data-dependent targets, done by
 // the reference with global float atomics.  LDS float atomics are slow on gfx950 (about 190 clk
 // per wave instruction) but 64-bit integer ones are not (about 15 clk), so the workgroup, which
-// owns the whole output plane of its channels, accumulates each channel's input-gradient plane
-// in LDS in 64-bit FIXED POINT: a contribution v becomes round(v * 2^s) through the
-// "add 1.5 * 2^52 in double" trick and ds_add_u64 adds it.  s is chosen per channel from
-// max|gout| (over the tensor, computed by a small kernel into the workspace) times max|Wt[c]| so
-// that a term stays below 2^44 and the plane's sum below 2^62: the grid is 2^-44 of the largest
-// possible term, far below fp32 rounding, and the sum is exact on that grid and independent of
-// the order of the additions (run-to-run reproducible, which float atomics are not).
+// owns the whole output plane of its channels, accumulates the input-gradient planes in LDS in
+// FIXED POINT, two channels per 64-bit add: each term becomes a signed 32-bit integer
+// round(v * 2^s), and the pair travels as b * 2^32 + a (decoded after the sum: a is the low
+// word read as signed, b the high word plus the borrow a negative a took).  s is chosen per
+// channel from max|gout| (over the tensor, computed by a small kernel into the workspace),
+// max|Wt[c]| and M, the largest number of samples touching one input element of this image
+// (counted by the workgroup with a 32-bit LDS histogram), so that a term stays below
+// 2^(30 - ceil(log2 M)) and no sum overflows.  This is used for M <= 64, where the grid is
+// 2^-24 of the largest possible term or finer; an image with more samples on one element falls
+// back to one channel per 64-bit sum on a 2^-44 grid.  Either sum is exact on its grid and
+// independent of the order of the additions (run-to-run reproducible, which float atomics are not).
 // Corners outside the image fall on the plane's zero padding, which is never read back.
 // One block per (image, group, channel chunk); blockDim = output pixels rounded up to a wave.
+// The kernel for planes of more than 1024 output pixels further down always uses the 2^-44 grid.
 // ---------------------------------------------------------------------------
 template <typename T>
 __global__ __launch_bounds__(256) void absmax_kernel(const T* __restrict__ p, long n, unsigned* __restrict__ out) {
   __shared__ float wave_max[4];
   float m = 0.f;
-  for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (long)gridDim.x * blockDim.x)
-    m = fmaxf(m, fabsf(ld(p + i)));
+  const long stride = (long)gridDim.x * blockDim.x;
+  constexpr int kInFlight = 8;  // independent loads per thread and trip
+  for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += kInFlight * stride) {
+    float v[kInFlight];
+#pragma unroll
+    for (int k = 0; k < kInFlight; ++k) v[k] = i + k * stride < n ? fabsf(ld(p + i + k * stride)) : 0.f;
+#pragma unroll
+    for (int k = 0; k < kInFlight; ++k) m = fmaxf(m, v[k]);
+  }
   for (int s = 32; s > 0; s >>= 1) m = fmaxf(m, __shfl_xor(m, s));
   if ((threadIdx.x & 63) == 0) wave_max[threadIdx.x >> 6] = m;
   __syncthreads();
@@ -346,6 +358,16 @@ __global__ __launch_bounds__(256) void absmax_kernel(const T* __restrict__ p, lo
     atomicMax(out, __float_as_uint(fmaxf(fmaxf(wave_max[0], wave_max[1]), fmaxf(wave_max[2], wave_max[3]))));
 }
 __global__ void clear_word_kernel(unsigned* p) { *p = 0u; }
+
+// Two channels share a 64-bit sum while at most 2^kPairHead samples touch one input element.
+constexpr int kPairHead = 6;
+
+// floor(v + 0.5) as a signed 32-bit integer, one instruction
+__device__ __forceinline__ int round_half_up(float v) {
+  int r;
+  asm("v_cvt_rpi_i32_f32 %0, %1" : "=v"(r) : "v"(v));
+  return r;
+}
 
 template <typename T, int SH, int SW>
 __global__ __launch_bounds__(1024) void deform_grad_input_kernel(
@@ -388,9 +410,39 @@ __global__ __launch_bounds__(1024) void deform_grad_input_kernel(
     for (int t = 0; t < K9; ++t) {
       st[t] = make_lite_tap<SH, SW>(sc[t].h, sc[t].w, true);
       const bool in = (sc[t].h > -1.f) && (sc[t].w > -1.f) && (sc[t].h < float(SH)) && (sc[t].w < float(SW));
-      hits |= in ? (1u << t) : 0u;
+      hits |= (live && in) ? (1u << t) : 0u;
     }
   }
+  __syncthreads();  // planes are zero
+
+  // The largest number of samples that touch one input element, M: a 32-bit histogram over the
+  // (still empty) planes.  A plane element then sums at most M terms, so terms scaled below
+  // 2^(30 - ceil(log2 M)) cannot overflow a signed 32-bit sum.
+  __shared__ unsigned wave_most[16];
+  {
+    unsigned* count = reinterpret_cast<unsigned*>(planes);
+#pragma unroll
+    for (int t = 0; t < K9; ++t) {
+      if (hits >> t & 1u) {
+        atomicAdd(count + it[t].pidx, 1u);
+        atomicAdd(count + it[t].pidx + 1, 1u);
+        atomicAdd(count + it[t].pidx + RS, 1u);
+        atomicAdd(count + it[t].pidx + RS + 1, 1u);
+      }
+    }
+    __syncthreads();
+    unsigned most = 1u;
+    for (int e = threadIdx.x; e < PS; e += blockDim.x) {
+      most = max(most, count[e]);
+      count[e] = 0u;
+    }
+    for (int sft = 32; sft > 0; sft >>= 1) most = max(most, (unsigned)__shfl_xor((int)most, sft));
+    if ((threadIdx.x & 63) == 0) wave_most[threadIdx.x >> 6] = most;
+    __syncthreads();
+  }
+  unsigned most = 1u;
+  for (int w = 0; w < (int)blockDim.x / 64; ++w) most = max(most, wave_most[w]);
+  const int head = most <= 1u ? 0 : 32 - __builtin_clz(most - 1u);  // ceil(log2(most))
 
   const size_t chan0 = (size_t)b.n * g.channel + b.grp + (size_t)g.groups * j0;
   const T* gp = gout + chan0 * out_plane;
@@ -401,45 +453,96 @@ __global__ __launch_bounds__(1024) void deform_grad_input_kernel(
   const int col = threadIdx.x & ((1 << shift) - 1), sub = threadIdx.x >> shift;
   const int rpp = (int)blockDim.x >> shift;
 
-  float gv = buf_ld(plane_rsrc(gp, out_plane), goff, gout);
-  __syncthreads();
-  for (int j = 0; j < nch; ++j) {
-    float gv_next = 0.f;
-    if (j + 1 < nch) gv_next = buf_ld(plane_rsrc(gp + (size_t)(j + 1) * g_step, out_plane), goff, gout);
-    unsigned long long* pl = planes + (j & 1) * PS;
-    const float* tb = tbl + j * Tb::SIZE;
-    // a term is at most gmax * wmax < 2^e: scale 2^(44 - e)
-    int e;
-    (void)frexpf(gmax * wmax[j], &e);
-    const double scale = ldexp(1.0, 44 - e), unscale = ldexp(1.0, e - 44);
-    constexpr double kMagic = 6755399441055744.0;  // 1.5 * 2^52: the sum's low mantissa bits are the rounded integer
+  if (head > kPairHead) {
+    // many samples on one element: one channel per 64-bit sum, on a 2^-44 grid through the
+    // "add 1.5 * 2^52 in double" trick (the low mantissa bits of the sum are the rounded integer)
+    float gv = buf_ld(plane_rsrc(gp, out_plane), goff, gout);
+    for (int j = 0; j < nch; ++j) {
+      const float gv_next = buf_ld(plane_rsrc(gp + (size_t)(j + 1) * g_step, j + 1 < nch ? out_plane : 0), goff, gout);
+      unsigned long long* pl = planes + (j & 1) * PS;
+      const float* tb = tbl + j * Tb::SIZE;
+      int e;  // a term is at most gmax * wmax < 2^e: scale 2^(44 - e), the plane's sum stays below 2^62
+      (void)frexpf(gmax * wmax[j], &e);
+      const double scale = ldexp(1.0, 44 - e), unscale = ldexp(1.0, e - 44);
+      constexpr double kMagic = 6755399441055744.0;  // 1.5 * 2^52
 #pragma unroll
-    for (int t = 0; t < K9; ++t) {
-      if (hits >> t & 1u) {
-        const float4 q = *reinterpret_cast<const float4*>(tb + st[t].cell);
-        const float gw = gv * lite_weight(st[t], q);
-        const float lh = it[t].lh, lw = it[t].lw, hh = 1.f - lh, hw = 1.f - lw;
-        const float term[4] = {hh * hw * gw, hh * lw * gw, lh * hw * gw, lh * lw * gw};  // K.cu:776-789
-        const int at[4] = {it[t].pidx, it[t].pidx + 1, it[t].pidx + RS, it[t].pidx + RS + 1};
+      for (int t = 0; t < K9; ++t) {
+        if (hits >> t & 1u) {
+          const float gw = gv * lite_weight(st[t], *reinterpret_cast<const float4*>(tb + st[t].cell));
+          const float lh = it[t].lh, lw = it[t].lw, hh = 1.f - lh, hw = 1.f - lw;
+          const float term[4] = {hh * hw * gw, hh * lw * gw, lh * hw * gw, lh * lw * gw};  // K.cu:776-789
+          const int at[4] = {it[t].pidx, it[t].pidx + 1, it[t].pidx + RS, it[t].pidx + RS + 1};
 #pragma unroll
-        for (int k = 0; k < 4; ++k) {
-          const double d = fma((double)term[k], scale, kMagic);
-          // bits(d) - bits(kMagic): the magic's low word is 0, so only the high word changes
-          const unsigned long long fixed = (unsigned long long)__double_as_longlong(d) - 0x4338000000000000ull;
-          atomicAdd(pl + at[k], fixed);
+          for (int k = 0; k < 4; ++k) {
+            const double d = fma((double)term[k], scale, kMagic);
+            // bits(d) - bits(kMagic): the magic's low word is 0, so only the high word changes
+            atomicAdd(pl + at[k], (unsigned long long)__double_as_longlong(d) - 0x4338000000000000ull);
+          }
+        }
+      }
+      gv = gv_next;
+      __syncthreads();
+      T* dst = ip + (size_t)j * i_step;
+      for (int row = sub; row < H; row += rpp) {
+        if (col < W) {
+          unsigned long long* cell = pl + (row + 1) * RS + 1 + col;
+          const long long v = (long long)*cell;
+          *cell = 0ull;
+          dk::st(dst + row * W + col, (float)((double)v * unscale));
         }
       }
     }
-    gv = gv_next;
+    return;
+  }
+
+  float gva = buf_ld(plane_rsrc(gp, out_plane), goff, gout);
+  float gvb = buf_ld(plane_rsrc(gp + g_step, 1 < nch ? out_plane : 0), goff, gout);
+  for (int j = 0; j < nch; j += 2) {
+    const bool pair = j + 1 < nch;
+    const float ga_next = buf_ld(plane_rsrc(gp + (size_t)(j + 2) * g_step, j + 2 < nch ? out_plane : 0), goff, gout);
+    const float gb_next = buf_ld(plane_rsrc(gp + (size_t)(j + 3) * g_step, j + 3 < nch ? out_plane : 0), goff, gout);
+    unsigned long long* pl = planes + ((j >> 1) & 1) * PS;
+    const float* ta = tbl + j * Tb::SIZE;
+    const float* tb = tbl + (pair ? j + 1 : j) * Tb::SIZE;
+    // a term of channel c is below gmax * wmax[c] < 2^e: scale 2^(30 - head - e)
+    int ea, eb;
+    (void)frexpf(gmax * wmax[j], &ea);
+    (void)frexpf(gmax * wmax[pair ? j + 1 : j], &eb);
+    const int sa = min(max(30 - head - ea, -100), 100), sb = min(max(30 - head - eb, -100), 100);
+    const float ga_s = gva * ldexpf(1.f, sa), gb_s = pair ? gvb * ldexpf(1.f, sb) : 0.f;
+#pragma unroll
+    for (int t = 0; t < K9; ++t) {
+      if (hits >> t & 1u) {
+        const float wa = ga_s * lite_weight(st[t], *reinterpret_cast<const float4*>(ta + st[t].cell));
+        const float wb = gb_s * lite_weight(st[t], *reinterpret_cast<const float4*>(tb + st[t].cell));
+        const float lh = it[t].lh, lw = it[t].lw, hh = 1.f - lh, hw = 1.f - lw;
+        const float cw[4] = {hh * hw, hh * lw, lh * hw, lh * lw};  // K.cu:776-789
+        const int at[4] = {it[t].pidx, it[t].pidx + 1, it[t].pidx + RS, it[t].pidx + RS + 1};
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+          // two signed 32-bit fixed-point terms in one 64-bit add: b * 2^32 + a
+          const int ia = round_half_up(cw[k] * wa), ib = round_half_up(cw[k] * wb);
+          const unsigned long long both =
+              ((unsigned long long)(unsigned)(ib + (ia >> 31)) << 32) | (unsigned long long)(unsigned)ia;
+          atomicAdd(pl + at[k], both);
+        }
+      }
+    }
+    gva = ga_next;
+    gvb = gb_next;
     __syncthreads();
-    // read the channel's plane back, clear it for the channel after next
+    // read the pair's plane back, clear it for the pair after next
+    const float ua = ldexpf(1.f, -sa), ub = ldexpf(1.f, -sb);
     T* dst = ip + (size_t)j * i_step;
     for (int row = sub; row < H; row += rpp) {
       if (col < W) {
         unsigned long long* cell = pl + (row + 1) * RS + 1 + col;
-        const long long v = (long long)*cell;
+        const unsigned long long v = *cell;
         *cell = 0ull;
-        dk::st(dst + row * W + col, (float)((double)v * unscale));
+        const int lo = (int)(unsigned)v;
+        const int hi = (int)(unsigned)(v >> 32) + (lo < 0 ? 1 : 0);
+        dk::st(dst + row * W + col, (float)lo * ua);
+        if (pair) dk::st(dst + i_step + row * W + col, (float)hi * ub);
       }
     }
   }
@@ -779,7 +882,7 @@ bool run_deform_grad_input(const Geo& g, const T* gout, const T* off, const T* r
   unsigned* gmax = static_cast<unsigned*>(ws);
   clear_word_kernel<<<1, 1, 0, stream>>>(gmax);
   const long n = (long)g.batch * g.channel * g.out_h * g.out_w;
-  absmax_kernel<T><<<(unsigned)std::min<long>(1024, (n + 255) / 256), 256, 0, stream>>>(gout, n, gmax);
+  absmax_kernel<T><<<(unsigned)std::min<long>(2048, (n + 255) / 256), 256, 0, stream>>>(gout, n, gmax);
   if (tiled) {
     auto kernel = deform_grad_input_tiled_kernel<T, SH, SW>;
     if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,

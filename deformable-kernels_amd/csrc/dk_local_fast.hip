@@ -73,6 +73,7 @@ __device__ __forceinline__ bool tap_geometry(const Geo& g, int ph, int pw, int f
 // one ds_read_b128 each at an immediate offset from one per-tap LDS address.
 // ---------------------------------------------------------------------------
 constexpr int kUnroll = 2;
+constexpr int kRowStages = 2;  // register stages of the rows kernel's load pipeline (3 and 4 measured slower)
 
 template <typename T, int KH, int KW, int SH, int SW, bool TRANSPOSED, int NT>
 __global__ __launch_bounds__(kBlock, 2) void local_gather_kernel(Geo g, const T* __restrict__ src,
@@ -279,13 +280,16 @@ __global__ __launch_bounds__(kBlock, 2) void local_gather_rows_kernel(Geo g, con
     }
   };
 
-  float xa[kUnroll][KH], xb[kUnroll][KH];
-  load_stage(xa, 0);
-  for (int j = 0; j < nch; j += 2 * kUnroll) {
-    load_stage(xb, j + kUnroll);
-    compute_stage(xa, j);
-    load_stage(xa, j + 2 * kUnroll);
-    compute_stage(xb, j + kUnroll);
+  constexpr int S = kRowStages;
+  float xs[S][kUnroll][KH];
+#pragma unroll
+  for (int s = 0; s + 1 < S; ++s) load_stage(xs[s], s * kUnroll);
+  for (int j = 0; j < nch; j += S * kUnroll) {
+#pragma unroll
+    for (int s = 0; s < S; ++s) {
+      load_stage(xs[(s + S - 1) % S], j + (s + S - 1) * kUnroll);
+      compute_stage(xs[s], j + s * kUnroll);
+    }
   }
 }
 
@@ -1128,7 +1132,7 @@ bool same_width_geometry(const Geo& g) {
 
 template <int SH, int SW>
 int channels_per_block(int cpg, int wanted_splits) {
-  const int fit = kMaxLdsTables / (WideTable<SH, SW>::SIZE * 4) - 2 * kUnroll;
+  const int fit = kMaxLdsTables / (WideTable<SH, SW>::SIZE * 4) - std::max(2, kRowStages) * kUnroll;
   int per = ceil_div(cpg, wanted_splits);
   if (per > fit) per = fit;
   if (per < 1) per = 1;
@@ -1159,7 +1163,7 @@ bool run_gather(const Geo& g, bool transposed, const T* src, const T* rot, const
   if (same_width_geometry(g)) {
     const int per = channels_per_block<SH, SW>(cpg, pick_splits(g, pixels));
     const unsigned grid = (unsigned)xcd_grid_size((long)ceil_div(pixels, kRowPix) * ceil_div(cpg, per) * g.batch * g.groups);
-    const size_t lds = (size_t)(per + 2 * kUnroll) * WideTable<SH, SW>::SIZE * sizeof(float);
+    const size_t lds = (size_t)(per + kRowStages * kUnroll) * WideTable<SH, SW>::SIZE * sizeof(float);
     if (transposed)
       local_gather_rows_kernel<T, 3, SH, SW, true><<<grid, kBlock, lds, stream>>>(g, src, rot, filter, dst, per);
     else

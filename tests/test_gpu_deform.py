@@ -104,6 +104,33 @@ def test_rotation_clip_inside_the_operator(case, clip):
     assert (got[3][~open_] == 0).all()
 
 
+def test_grad_input_when_every_sample_lands_on_one_input_element():
+    # all 9 x P samples of an image within one input cell: the grad-input kernel's fixed-point
+    # scale has to leave room for that many terms in one sum
+    from deformable_kernels.ops.deform_kernel.functions import deform_sample_depthwise
+    case = (2, 12, 14, 14, 3, (4, 4), 1, 1, 1, 1, 0.5, 0.0)
+    N, C, H, W, k, S, s, p, d, G, rs, os_ = case
+    x, wt, rot, off, gout, cfg = make_deform(N, C, H, W, k, S, s, p, d, G, rs, os_, seed=9)
+    g = torch.Generator().manual_seed(1)
+    oh, ow = torch.meshgrid(torch.arange(H), torch.arange(W), indexing="ij")
+    for t in range(9):
+        # tap position oh - 1 + t // 3, ow - 1 + t % 3; target (6.3, 7.6) plus a little jitter
+        off[:, 2 * t] = 6.3 - (oh - 1 + t // 3) + 0.2 * torch.rand(N, H, W, generator=g)
+        off[:, 2 * t + 1] = 7.6 - (ow - 1 + t % 3) + 0.2 * torch.rand(N, H, W, generator=g)
+    dev = torch.device("cuda:0")
+    xg, og, rg, wg = [t_.to(dev).requires_grad_() for t_ in (x, off, rot, wt)]
+    out = deform_sample_depthwise(xg, og, rg, wg, cfg["kernel_size"], cfg["stride"], cfg["padding"],
+                                  cfg["dilation"], cfg["groups"])
+    out.backward(gout.to(dev))
+    got = [t_.detach().cpu() for t_ in (out, xg.grad, og.grad, rg.grad, wg.grad)]
+    inputs = (x, wt, rot, off, gout, cfg)
+    o32, o64 = _oracle(inputs, np.float32), _oracle(inputs, np.float64)
+    assert rel_err(got[0], o32[0]) < 1e-5, NAMES[0]
+    assert rel_err(got[1], o64[1]) < 1e-5, NAMES[1]
+    for i in range(2, 5):
+        assert rel_err(got[i], o64[i]) < 1e-4, NAMES[i]
+
+
 def test_zero_image_offsets_equal_the_local_operator_on_gpu():
     from deformable_kernels.ops.deform_kernel.functions import deform_sample_depthwise, sample_depthwise
     x, wt, rot, off, gout, cfg = make_deform(2, 16, 12, 12, 3, (4, 4), 1, 1, 1, 1, 1.0, 0.0, seed=3)
