@@ -44,6 +44,7 @@ OTHER_WORKLOADS = {
     # N-d sampler: data shape [C, s...], points, coordinate range
     "nd_cfg3": ("nd", ((256, 5, 5), 1152, (0.0, 4.0))),             # GlobalDeformKernel2d, config 3
     "nd_cfg5": ("nd", ((64, 32, 32, 32), 1 << 20, (-1.0, 32.0))),   # trilinear volume, config 5, full-volume coords
+    "nd_cfg5_unit": ("nd", ((64, 32, 32, 32), 1 << 20, (-1.0, 1.0))),  # the same with config 5's own range [-1, 1]^3
 }
 
 

@@ -15,6 +15,10 @@
 //  * Direct path (any dimension count, small problems): one lane per (point, channel).
 // The coordinate gradient is reduced over channels inside the kernel instead of
 // materialising the reference's [B, n, C] intermediate (ND.cu:281-286 and the caller's sum).
+#include <rocprim/device/device_radix_sort.hpp>
+#include <rocprim/iterator/counting_iterator.hpp>
+
+#include "dk_kernels.h"
 #include "dk_nd.h"
 
 namespace dk {
@@ -363,6 +367,216 @@ __global__ __launch_bounds__(kBlock) void nd_grad_data_cl_kernel(NdGeo g, const 
   }
 }
 
+// ---------------------------------------------------------------------------
+// binned channel-last path: many points per cell of the volume
+//
+// With more points than cells, points that fall into the same cell read (forward, grad coord)
+// or update (grad data) the same 2^n corner rows.  The points are therefore sorted by cell
+// first -- rocPRIM's radix sort of (key, point index) pairs, the key being the cell's low corner,
+// (low[d] + 1) over extents shape[d] + 1, plus one last bin for the points outside the volume;
+// a radix sort rather than a counting sort with atomics because the points of a real workload
+// may all sit in a handful of cells -- and a wave walks 64
+// consecutive points of the sorted order, lanes over channels: the corner rows stay in
+// registers while the cell does not change (forward, grad coord), and the input gradient of a
+// cell's corners is summed in registers and leaves as one atomic per corner and channel when the
+// cell changes (grad data).  Results go to / come from each point's original row.
+// ---------------------------------------------------------------------------
+template <typename T>
+__device__ __forceinline__ int point_bin(const NdGeo& g, const T* coord_b, int nbins) {
+  const NdPoint<float> p = load_point<T, float>(g, coord_b);
+  if (!p.inside) return nbins - 1;
+  int key = 0;
+#pragma unroll
+  for (int d = 0; d < kClMaxDims; ++d)
+    if (d < g.dims) key = key * (g.shape[d] + 1) + p.low[d] + 1;
+  return key;
+}
+
+template <typename T>
+__global__ __launch_bounds__(kBlock) void nd_bin_keys_kernel(NdGeo g, const T* __restrict__ coord, int nbins,
+                                                             unsigned* __restrict__ keys) {
+  const long b = (long)blockIdx.x * kBlock + threadIdx.x;
+  if (b < g.batch) keys[b] = (unsigned)point_bin<T>(g, coord + b * g.dims, nbins);
+}
+
+// What a wave of the binned kernels knows about its 64 sorted points: lane q holds point q.
+template <typename T>
+struct BinnedWave {
+  int npts, id, key;
+  ClCorners cc;
+  __device__ __forceinline__ bool init(const NdGeo& g, const T* coord, const int* order, int nbins) {
+    const int lane = threadIdx.x & 63;
+    const long wave0 = ((long)blockIdx.x * (kBlock / 64) + (threadIdx.x >> 6)) * 64;
+    if (wave0 >= g.batch) return false;
+    npts = (int)min(64L, g.batch - wave0);
+    const bool valid = lane < npts;
+    id = valid ? order[wave0 + lane] : 0;
+    cc = cl_corners<T>(g, coord, id, valid);
+    key = valid ? point_bin<T>(g, coord + (long)id * g.dims, nbins) : -1;
+    return true;
+  }
+  __device__ __forceinline__ int key_of(int q) const { return __builtin_amdgcn_readlane(key, q); }
+  __device__ __forceinline__ long id_of(int q) const { return __builtin_amdgcn_readlane(id, q); }
+  __device__ __forceinline__ int off_of(int i, int q) const { return __builtin_amdgcn_readlane(cc.off[i], q); }
+  __device__ __forceinline__ float w_of(int i, int q) const {
+    return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, cc.w[i]), q));
+  }
+};
+
+// Makes the corner rows just loaded count as used here, so that the wait for them sits in the
+// (rare) cell-change branch.  Otherwise the compiler waits for every outstanding memory operation
+// at the first use after the branch, for every point, and that includes the point's own store.
+__device__ __forceinline__ void settle(float (&v)[kClCorners]) {
+  asm volatile("" : "+v"(v[0]), "+v"(v[1]), "+v"(v[2]), "+v"(v[3]), "+v"(v[4]), "+v"(v[5]), "+v"(v[6]), "+v"(v[7]));
+}
+
+template <typename T>
+__global__ __launch_bounds__(kBlock) void nd_forward_binned_kernel(NdGeo g, const T* __restrict__ data_cl,
+                                                                   const T* __restrict__ coord,
+                                                                   const int* __restrict__ order, int nbins,
+                                                                   T* __restrict__ out) {
+  BinnedWave<T> wv;
+  if (!wv.init(g, coord, order, nbins)) return;
+  const int lane = threadIdx.x & 63, ncorner = 1 << g.dims;
+  for (int c0 = 0; c0 < g.channel; c0 += 64) {
+    const int c = c0 + lane;
+    const bool cin = c < g.channel;
+    float v[kClCorners];
+#pragma unroll
+    for (int i = 0; i < kClCorners; ++i) v[i] = 0.f;
+    int cur = -2;
+    for (int q = 0; q < wv.npts; ++q) {
+      const int key = wv.key_of(q);
+      if (key != cur) {  // wave-uniform: a new cell, fetch its corner rows
+        cur = key;
+#pragma unroll
+        for (int i = 0; i < kClCorners; ++i)
+          v[i] = (cin && i < ncorner) ? ld(data_cl + (size_t)wv.off_of(i, q) * g.channel + c) : 0.f;
+        settle(v);
+      }
+      float acc = 0.f;
+#pragma unroll
+      for (int i = 0; i < kClCorners; ++i) acc += wv.w_of(i, q) * v[i];
+      if (cin) st(out + wv.id_of(q) * g.channel + c, acc);
+    }
+  }
+}
+
+template <typename T>
+__global__ __launch_bounds__(kBlock) void nd_grad_data_binned_kernel(NdGeo g, const T* __restrict__ gout,
+                                                                     const T* __restrict__ coord,
+                                                                     const int* __restrict__ order, int nbins,
+                                                                     float* __restrict__ gdata_cl) {
+  BinnedWave<T> wv;
+  if (!wv.init(g, coord, order, nbins)) return;
+  const int lane = threadIdx.x & 63, ncorner = 1 << g.dims;
+  constexpr int PU = 8;  // output-gradient rows in flight
+  for (int c0 = 0; c0 < g.channel; c0 += 64) {
+    const int c = c0 + lane;
+    const bool cin = c < g.channel;
+    float acc[kClCorners];
+    int at[kClCorners];
+#pragma unroll
+    for (int i = 0; i < kClCorners; ++i) acc[i] = 0.f, at[i] = 0;
+    int cur = -2;
+#define DK_FLUSH()                                                                             \
+  _Pragma("unroll") for (int i = 0; i < kClCorners; ++i) if (cin && i < ncorner && acc[i] != 0.f) \
+      atomicAdd(gdata_cl + (size_t)at[i] * g.channel + c, acc[i])
+    for (int q0 = 0; q0 < wv.npts; q0 += PU) {
+      float go[PU];
+#pragma unroll
+      for (int u = 0; u < PU; ++u)
+        go[u] = (cin && q0 + u < wv.npts) ? ld(gout + wv.id_of(min(q0 + u, wv.npts - 1)) * g.channel + c) : 0.f;
+#pragma unroll
+      for (int u = 0; u < PU; ++u) {
+        const int q = q0 + u;
+        if (q < wv.npts) {
+          const int key = wv.key_of(q);
+          if (key != cur) {  // wave-uniform: the sums of the finished cell leave
+            DK_FLUSH();
+            cur = key;
+#pragma unroll
+            for (int i = 0; i < kClCorners; ++i) acc[i] = 0.f, at[i] = wv.off_of(i, q);
+          }
+#pragma unroll
+          for (int i = 0; i < kClCorners; ++i) acc[i] += wv.w_of(i, q) * go[u];
+        }
+      }
+    }
+    DK_FLUSH();
+#undef DK_FLUSH
+  }
+}
+
+template <typename T>
+__global__ __launch_bounds__(kBlock) void nd_grad_coord_binned_kernel(NdGeo g, const T* __restrict__ gout,
+                                                                      const T* __restrict__ data_cl,
+                                                                      const T* __restrict__ coord,
+                                                                      const int* __restrict__ order, int nbins,
+                                                                      T* __restrict__ gcoord) {
+  BinnedWave<T> wv;
+  if (!wv.init(g, coord, order, nbins)) return;
+  const int lane = threadIdx.x & 63, ncorner = 1 << g.dims;
+  constexpr int PU = 4;
+  // s[i] of point q lands in lane q: sum over channels of gout * data at corner i
+  float s[kClCorners];
+#pragma unroll
+  for (int i = 0; i < kClCorners; ++i) s[i] = 0.f;
+  for (int c0 = 0; c0 < g.channel; c0 += 64) {
+    const int c = c0 + lane;
+    const bool cin = c < g.channel;
+    float v[kClCorners];
+#pragma unroll
+    for (int i = 0; i < kClCorners; ++i) v[i] = 0.f;
+    int cur = -2;
+    for (int q0 = 0; q0 < wv.npts; q0 += PU) {
+      float go[PU];
+#pragma unroll
+      for (int u = 0; u < PU; ++u)
+        go[u] = (cin && q0 + u < wv.npts) ? ld(gout + wv.id_of(min(q0 + u, wv.npts - 1)) * g.channel + c) : 0.f;
+#pragma unroll
+      for (int u = 0; u < PU; ++u) {
+        const int q = q0 + u;
+        if (q < wv.npts) {
+          const int key = wv.key_of(q);
+          if (key != cur) {
+            cur = key;
+#pragma unroll
+            for (int i = 0; i < kClCorners; ++i)
+              v[i] = (cin && i < ncorner) ? ld(data_cl + (size_t)wv.off_of(i, q) * g.channel + c) : 0.f;
+            settle(v);
+          }
+#pragma unroll
+          for (int i = 0; i < kClCorners; ++i) {
+            if (i < ncorner) {
+              const float t = wave_sum(go[u] * v[i]);
+              if (lane == q) s[i] += t;
+            }
+          }
+        }
+      }
+    }
+  }
+  if (lane >= wv.npts) return;
+  // lane <-> point again: apply the derivative weights (ND.cu:161,165) to the corner sums
+  const NdPoint<float> p = load_point<T, float>(g, coord + (long)wv.id * g.dims);
+#pragma unroll
+  for (int d = 0; d < kClMaxDims; ++d) {
+    if (d < g.dims) {
+      float gd = 0.f;
+      if (p.inside) {
+#pragma unroll
+        for (int i = 0; i < kClCorners; ++i) {
+          long o;
+          float w;
+          if (i < ncorner && corner<float>(g, p, (unsigned)i, d, o, w)) gd += s[i] * w;
+        }
+      }
+      st(gcoord + (long)wv.id * g.dims + d, gd);
+    }
+  }
+}
+
 template <typename CT>
 __global__ void nd_fill_zero_kernel(CT* p, long n) {
   for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (long)gridDim.x * blockDim.x)
@@ -421,12 +635,82 @@ bool nd_use_channel_last(const dk_nd_desc& d) {
   return d.batch * d.channel >= 65536 && d.channel >= 16;
 }
 
+// Bins of the counting sort (cells of low corners plus the bin of outside points), or 0 when
+// the binned kernels do not apply: they pay off with several points per cell.
+int nd_bins(const dk_nd_desc& d) {
+  if (!nd_use_channel_last(d) || path_disabled("DK_NO_ND_BINS")) return 0;
+  long bins = 1;
+  for (int i = 0; i < d.dims; ++i) bins *= (long)d.shape[i] + 1;
+  bins += 1;
+  if (bins > 262144 || d.batch < 2 * bins || d.batch < 65536 || d.batch >= (1L << 30)) return 0;
+  return (int)bins;
+}
+
+size_t round256(size_t n) { return (n + 255) / 256 * 256; }
+
+namespace {
+
+// Onesweep radix passes for every size: the keys have few significant bits (two or three 8-bit
+// passes), where rocPRIM's default for up to 2^20 items is a merge sort of ten passes.
+using SortConfig = rocprim::radix_sort_config<rocprim::default_config, rocprim::default_config,
+                                              rocprim::default_config, 0>;
+
+int key_bits(int bins) {
+  int bits = 1;
+  while ((1L << bits) < bins) ++bits;
+  return bits;
+}
+
+// rocPRIM's temporary storage for sorting n (key, index) pairs; 0 if the query fails
+size_t sort_temp_bytes(long n, int bins) {
+  size_t bytes = 0;
+  const hipError_t e = rocprim::radix_sort_pairs<SortConfig>(
+      nullptr, bytes, static_cast<unsigned*>(nullptr), static_cast<unsigned*>(nullptr),
+      rocprim::counting_iterator<int>(0), static_cast<int*>(nullptr), (size_t)n, 0u, (unsigned)key_bits(bins));
+  return e == hipSuccess ? bytes : 0;
+}
+
+}  // namespace
+
+// bytes for the sort: keys, sorted keys, the sorted order of the points, rocPRIM's scratch
+size_t nd_sort_workspace(const dk_nd_desc& d) {
+  const int bins = nd_bins(d);
+  if (!bins) return 0;
+  return 3 * round256((size_t)d.batch * sizeof(int)) + round256(sort_temp_bytes(d.batch, bins));
+}
+
 size_t nd_data_cl_workspace(const dk_nd_desc& d) {
   if (!nd_use_channel_last(d)) return 0;
   size_t n = (size_t)d.channel;
   for (int i = 0; i < d.dims; ++i) n *= (size_t)d.shape[i];
-  return n * elem_size(d.dtype);
+  return round256(n * elem_size(d.dtype)) + nd_sort_workspace(d);
 }
+
+namespace {
+
+// Sorts the points by cell into `order` (at `sort_ws`, laid out as nd_sort_workspace says).
+template <typename T>
+const int* sort_points(const NdGeo& g, const T* coord, int bins, void* sort_ws, hipStream_t stream) {
+  const size_t n4 = round256((size_t)g.batch * sizeof(int));
+  char* base = static_cast<char*>(sort_ws);
+  unsigned* keys = reinterpret_cast<unsigned*>(base);
+  unsigned* keys_sorted = reinterpret_cast<unsigned*>(base + n4);
+  int* order = reinterpret_cast<int*>(base + 2 * n4);
+  void* temp = base + 3 * n4;
+  nd_bin_keys_kernel<T><<<(unsigned)((g.batch + kBlock - 1) / kBlock), kBlock, 0, stream>>>(g, coord, bins, keys);
+  size_t temp_bytes = sort_temp_bytes(g.batch, bins);
+  (void)rocprim::radix_sort_pairs<SortConfig>(temp, temp_bytes, keys, keys_sorted, rocprim::counting_iterator<int>(0), order,
+                                  (size_t)g.batch, 0u, (unsigned)key_bits(bins), stream);
+  return order;
+}
+
+size_t data_bytes(const dk_nd_desc& d) {
+  size_t n = (size_t)d.channel;
+  for (int i = 0; i < d.dims; ++i) n *= (size_t)d.shape[i];
+  return n;
+}
+
+}  // namespace
 
 template <typename T>
 void nd_forward(const dk_nd_desc& d, const T* data, const T* coord, T* out, void* ws,
@@ -436,6 +720,11 @@ void nd_forward(const dk_nd_desc& d, const T* data, const T* coord, T* out, void
     if (nd_use_channel_last(d)) {
       T* data_cl = static_cast<T*>(ws);
       transpose<T, T>(data, data_cl, g.channel, g.prod_shape, stream);
+      if (const int bins = nd_bins(d)) {
+        const int* order = sort_points<T>(g, coord, bins, static_cast<char*>(ws) + round256(data_bytes(d) * sizeof(T)), stream);
+        nd_forward_binned_kernel<T><<<(unsigned)((g.batch + 255) / 256), kBlock, 0, stream>>>(g, data_cl, coord, order, bins, out);
+        return;
+      }
       const int ppw = points_per_wave(g);
       const long waves = (g.batch + ppw - 1) / ppw;
       nd_forward_cl_kernel<T><<<(unsigned)((waves + 3) / 4), kBlock, 0, stream>>>(g, data_cl, coord, out, ppw);
@@ -449,7 +738,7 @@ void nd_forward(const dk_nd_desc& d, const T* data, const T* coord, T* out, void
 size_t nd_grad_data_workspace(const dk_nd_desc& d) {
   size_t n = (size_t)d.channel;
   for (int i = 0; i < d.dims; ++i) n *= (size_t)d.shape[i];
-  if (nd_use_channel_last(d)) return n * sizeof(float);  // fp32 channel-last accumulation image
+  if (nd_use_channel_last(d)) return round256(n * sizeof(float)) + nd_sort_workspace(d);  // fp32 channel-last accumulation image
   if (d.dtype == DK_F16 || d.dtype == DK_BF16) return n * sizeof(float);
   return 0;
 }
@@ -465,9 +754,14 @@ void nd_grad_data(const dk_nd_desc& d, const T* gout, const T* coord, T* gdata, 
     if (nd_use_channel_last(d)) {
       float* acc = static_cast<float*>(ws);
       nd_fill_zero_kernel<float><<<grid_for(n_data), kBlock, 0, stream>>>(acc, n_data);
-      const int ppw = points_per_wave(g);
-      const long waves = (g.batch + ppw - 1) / ppw;
-      nd_grad_data_cl_kernel<T><<<(unsigned)((waves + 3) / 4), kBlock, 0, stream>>>(g, gout, coord, acc, ppw);
+      if (const int bins = nd_bins(d)) {
+        const int* order = sort_points<T>(g, coord, bins, static_cast<char*>(ws) + round256((size_t)n_data * sizeof(float)), stream);
+        nd_grad_data_binned_kernel<T><<<(unsigned)((g.batch + 255) / 256), kBlock, 0, stream>>>(g, gout, coord, order, bins, acc);
+      } else {
+        const int ppw = points_per_wave(g);
+        const long waves = (g.batch + ppw - 1) / ppw;
+        nd_grad_data_cl_kernel<T><<<(unsigned)((waves + 3) / 4), kBlock, 0, stream>>>(g, gout, coord, acc, ppw);
+      }
       transpose<float, T>(acc, gdata, g.prod_shape, g.channel, stream);
       return;
     }
@@ -488,6 +782,11 @@ void nd_grad_coord(const dk_nd_desc& d, const T* gout, const T* data, const T* c
     if (nd_use_channel_last(d)) {
       T* data_cl = static_cast<T*>(ws);
       transpose<T, T>(data, data_cl, g.channel, g.prod_shape, stream);
+      if (const int bins = nd_bins(d)) {
+        const int* order = sort_points<T>(g, coord, bins, static_cast<char*>(ws) + round256(data_bytes(d) * sizeof(T)), stream);
+        nd_grad_coord_binned_kernel<T><<<(unsigned)((g.batch + 255) / 256), kBlock, 0, stream>>>(g, gout, data_cl, coord, order, bins, gcoord);
+        return;
+      }
       const int ppw = points_per_wave(g);
       const long waves = (g.batch + ppw - 1) / ppw;
       nd_grad_coord_cl_kernel<T><<<(unsigned)((waves + 3) / 4), kBlock, 0, stream>>>(g, gout, data_cl, coord, gcoord, ppw);

@@ -50,6 +50,38 @@ def test_fp32_matches_oracle(shape, C, B):
     assert rel_err(got[2], o64[2]) < 1e-4
 
 
+@pytest.mark.parametrize("shape,C,B,lo,hi", [
+    ((8, 8, 8), 64, 65536 + 37, -1.5, 9.5),    # many points per cell: the sorted-by-cell kernels; ragged last wave
+    ((16, 12), 80, 70001, -1.5, 17.0),         # two channel passes (64 + 16)
+    ((40,), 16, 66000, -2.0, 42.0),            # one dimension
+    ((8, 8, 8), 32, 65536, -1.0, 1.0),         # config 5's coordinate range: every point in the 8 corner cells
+    ((6, 5, 4), 64, 65536, 2.2, 2.9),          # every point in one cell
+])
+def test_many_points_per_cell_match_oracle(shape, C, B, lo, hi):
+    g = torch.Generator().manual_seed(45)
+    data = torch.randn(C, *shape, generator=g)
+    coord = torch.rand(B, len(shape), generator=g) * (hi - lo) + lo
+    gout = torch.randn(B, C, generator=g)
+    got = _run(data, coord, gout)
+    o32, o64 = _oracle(data, coord, gout, np.float32), _oracle(data, coord, gout, np.float64)
+    assert rel_err(got[0], o32[0]) < 1e-5
+    assert rel_err(got[1], o64[1]) < 1e-4
+    assert rel_err(got[2], o64[2]) < 1e-4
+
+
+def test_sorted_and_unsorted_kernels_agree(monkeypatch):
+    g = torch.Generator().manual_seed(46)
+    data = torch.randn(64, 8, 8, 8, generator=g)
+    coord = torch.rand(70000, 3, generator=g) * 10.0 - 1.0
+    gout = torch.randn(70000, 64, generator=g)
+    a = _run(data, coord, gout)
+    monkeypatch.setenv("DK_NO_ND_BINS", "1")
+    b = _run(data, coord, gout)
+    assert torch.equal(a[0], b[0])  # same arithmetic per point
+    assert rel_err(a[1], b[1]) < 1e-5
+    assert rel_err(a[2], b[2]) < 1e-5
+
+
 def test_fp64_matches_oracle():
     data, coord, gout = _inputs((4, 5, 6), 9, 257, seed=42, dtype=torch.float64)
     got = _run(data, coord, gout)
@@ -58,7 +90,7 @@ def test_fp64_matches_oracle():
         assert rel_err(g, w) < 1e-11
 
 
-@pytest.mark.parametrize("points", [300, 4096])   # direct path / channel-last path
+@pytest.mark.parametrize("points", [300, 4096, 65536])   # direct path / channel-last path / sorted by cell
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 def test_half_precisions_match_fp32_oracle(dtype, points):
     data, coord, gout = _inputs((5, 5), 64, points, seed=43, dtype=dtype)
