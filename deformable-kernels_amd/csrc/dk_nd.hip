@@ -217,11 +217,13 @@ __global__ __launch_bounds__(256) void nd_transpose_kernel(const A* __restrict__
 struct ClCorners {
   int off[kClCorners];
   float w[kClCorners];
+  unsigned present;  // bit i: corner i lies inside the volume (its weight may still be 0)
 };
 
 template <typename T>
 __device__ __forceinline__ ClCorners cl_corners(const NdGeo& g, const T* coord, long b, bool valid) {
   ClCorners cc;
+  cc.present = 0u;
   NdPoint<float> p;
   p.inside = false;
   if (valid) p = load_point<T, float>(g, coord + b * g.dims);
@@ -232,6 +234,7 @@ __device__ __forceinline__ ClCorners cl_corners(const NdGeo& g, const T* coord, 
     const bool ok = valid && p.inside && i < (1 << g.dims) && corner<float>(g, p, (unsigned)i, -1, o, w);
     cc.off[i] = ok ? (int)o : 0;
     cc.w[i] = ok ? w : 0.f;
+    cc.present |= ok ? (1u << i) : 0u;
   }
   return cc;
 }
@@ -508,6 +511,13 @@ __global__ __launch_bounds__(kBlock) void nd_grad_data_binned_kernel(NdGeo g, co
   }
 }
 
+// grad coord on the sorted points.  Per cell the eight corner rows are turned into the
+// coefficients of the multilinear polynomial,
+//   value = c0 + c1 f0 + c2 f1 + c3 f2 + c4 f0 f1 + c5 f0 f2 + c6 f1 f2 + c7 f0 f1 f2
+// (f = fractional position; absent corners and absent dimensions enter as zeros, which is what
+// skipping them amounts to), so that a point's three partial derivatives cost nine fused
+// multiply-adds per channel instead of eight corner products, and three wave reductions
+// instead of eight.
 template <typename T>
 __global__ __launch_bounds__(kBlock) void nd_grad_coord_binned_kernel(NdGeo g, const T* __restrict__ gout,
                                                                       const T* __restrict__ data_cl,
@@ -516,18 +526,25 @@ __global__ __launch_bounds__(kBlock) void nd_grad_coord_binned_kernel(NdGeo g, c
                                                                       T* __restrict__ gcoord) {
   BinnedWave<T> wv;
   if (!wv.init(g, coord, order, nbins)) return;
-  const int lane = threadIdx.x & 63, ncorner = 1 << g.dims;
-  constexpr int PU = 4;
-  // s[i] of point q lands in lane q: sum over channels of gout * data at corner i
-  float s[kClCorners];
+  const int lane = threadIdx.x & 63;
+  const bool valid = lane < wv.npts;
+  // lane <-> point: fractional position and its pairwise products
+  NdPoint<float> p;
+  p.inside = false;
 #pragma unroll
-  for (int i = 0; i < kClCorners; ++i) s[i] = 0.f;
+  for (int d = 0; d < DK_ND_MAX_DIMS; ++d) p.frac[d] = 0.f, p.low[d] = 0;
+  if (valid) p = load_point<T, float>(g, coord + (long)wv.id * g.dims);
+  const float f0 = p.frac[0], f1 = p.frac[1], f2 = p.frac[2];
+  const float f01 = f0 * f1, f02 = f0 * f2, f12 = f1 * f2;
+  auto uni = [](float v, int q) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), q));
+  };
+  constexpr int PU = 4;
+  float gd0 = 0.f, gd1 = 0.f, gd2 = 0.f;  // of point q, in lane q
   for (int c0 = 0; c0 < g.channel; c0 += 64) {
     const int c = c0 + lane;
     const bool cin = c < g.channel;
-    float v[kClCorners];
-#pragma unroll
-    for (int i = 0; i < kClCorners; ++i) v[i] = 0.f;
+    float k1 = 0.f, k2 = 0.f, k3 = 0.f, k4 = 0.f, k5 = 0.f, k6 = 0.f, k7 = 0.f;
     int cur = -2;
     for (int q0 = 0; q0 < wv.npts; q0 += PU) {
       float go[PU];
@@ -541,40 +558,45 @@ __global__ __launch_bounds__(kBlock) void nd_grad_coord_binned_kernel(NdGeo g, c
           const int key = wv.key_of(q);
           if (key != cur) {
             cur = key;
+            float v[kClCorners];
+            const unsigned present = (unsigned)__builtin_amdgcn_readlane((int)wv.cc.present, q);
 #pragma unroll
             for (int i = 0; i < kClCorners; ++i)
-              v[i] = (cin && i < ncorner) ? ld(data_cl + (size_t)wv.off_of(i, q) * g.channel + c) : 0.f;
+              v[i] = (cin && (present >> i & 1u)) ? ld(data_cl + (size_t)wv.off_of(i, q) * g.channel + c) : 0.f;
             settle(v);
+            // corner index: bit d = high side of dimension d
+            k1 = v[1] - v[0];
+            k2 = v[2] - v[0];
+            k3 = v[4] - v[0];
+            k4 = (v[3] - v[2]) - k1;
+            k5 = (v[5] - v[4]) - k1;
+            k6 = (v[6] - v[4]) - k2;
+            k7 = ((v[7] - v[6]) - (v[5] - v[4])) - k4;
           }
-#pragma unroll
-          for (int i = 0; i < kClCorners; ++i) {
-            if (i < ncorner) {
-              const float t = wave_sum(go[u] * v[i]);
-              if (lane == q) s[i] += t;
-            }
+          const float u0 = uni(f0, q), u1 = uni(f1, q), u2 = uni(f2, q);
+          const float u01 = uni(f01, q), u02 = uni(f02, q), u12 = uni(f12, q);
+          const float d0 = fmaf(k7, u12, fmaf(k5, u2, fmaf(k4, u1, k1)));
+          const float d1 = fmaf(k7, u02, fmaf(k6, u2, fmaf(k4, u0, k2)));
+          const float d2 = fmaf(k7, u01, fmaf(k6, u1, fmaf(k5, u0, k3)));
+          const float t0 = wave_sum(go[u] * d0);
+          if (lane == q) gd0 += t0;
+          if (g.dims > 1) {
+            const float t1 = wave_sum(go[u] * d1);
+            if (lane == q) gd1 += t1;
+          }
+          if (g.dims > 2) {
+            const float t2 = wave_sum(go[u] * d2);
+            if (lane == q) gd2 += t2;
           }
         }
       }
     }
   }
-  if (lane >= wv.npts) return;
-  // lane <-> point again: apply the derivative weights (ND.cu:161,165) to the corner sums
-  const NdPoint<float> p = load_point<T, float>(g, coord + (long)wv.id * g.dims);
+  if (!valid) return;
+  const float gd[3] = {gd0, gd1, gd2};
 #pragma unroll
-  for (int d = 0; d < kClMaxDims; ++d) {
-    if (d < g.dims) {
-      float gd = 0.f;
-      if (p.inside) {
-#pragma unroll
-        for (int i = 0; i < kClCorners; ++i) {
-          long o;
-          float w;
-          if (i < ncorner && corner<float>(g, p, (unsigned)i, d, o, w)) gd += s[i] * w;
-        }
-      }
-      st(gcoord + (long)wv.id * g.dims + d, gd);
-    }
-  }
+  for (int d = 0; d < kClMaxDims; ++d)
+    if (d < g.dims) st(gcoord + (long)wv.id * g.dims + d, p.inside ? gd[d] : 0.f);
 }
 
 template <typename CT>

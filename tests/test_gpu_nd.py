@@ -69,6 +69,21 @@ def test_many_points_per_cell_match_oracle(shape, C, B, lo, hi):
     assert rel_err(got[2], o64[2]) < 1e-4
 
 
+def test_many_points_on_grid_nodes_and_half_way_between():
+    # fractional positions of exactly 0 and 0.5: a corner with interpolation weight 0 still
+    # enters the coordinate gradient
+    g = torch.Generator().manual_seed(47)
+    data = torch.randn(32, 7, 6, 5, generator=g)
+    hi = torch.tensor([7.0, 6.0, 5.0])
+    coord = torch.round((torch.rand(65536, 3, generator=g) * (hi + 2.0) - 1.0) * 2.0) / 2.0
+    gout = torch.randn(65536, 32, generator=g)
+    got = _run(data, coord, gout)
+    o32, o64 = _oracle(data, coord, gout, np.float32), _oracle(data, coord, gout, np.float64)
+    assert rel_err(got[0], o32[0]) < 1e-5
+    assert rel_err(got[1], o64[1]) < 1e-4
+    assert rel_err(got[2], o64[2]) < 1e-4
+
+
 def test_sorted_and_unsorted_kernels_agree(monkeypatch):
     g = torch.Generator().manual_seed(46)
     data = torch.randn(64, 8, 8, 8, generator=g)
