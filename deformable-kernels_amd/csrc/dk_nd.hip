@@ -407,9 +407,11 @@ template <typename T>
 struct BinnedWave {
   int npts, id, key;
   ClCorners cc;
-  __device__ __forceinline__ bool init(const NdGeo& g, const T* coord, const int* order, int nbins) {
+  // the wave's `sub`-th chunk of 64 points when a wave walks `per_wave` consecutive chunks
+  __device__ __forceinline__ bool init(const NdGeo& g, const T* coord, const int* order, int nbins,
+                                       int per_wave = 1, int sub = 0) {
     const int lane = threadIdx.x & 63;
-    const long wave0 = ((long)blockIdx.x * (kBlock / 64) + (threadIdx.x >> 6)) * 64;
+    const long wave0 = (((long)blockIdx.x * (kBlock / 64) + (threadIdx.x >> 6)) * per_wave + sub) * 64;
     if (wave0 >= g.batch) return false;
     npts = (int)min(64L, g.batch - wave0);
     const bool valid = lane < npts;
@@ -469,9 +471,7 @@ template <typename T>
 __global__ __launch_bounds__(kBlock) void nd_grad_data_binned_kernel(NdGeo g, const T* __restrict__ gout,
                                                                      const T* __restrict__ coord,
                                                                      const int* __restrict__ order, int nbins,
-                                                                     float* __restrict__ gdata_cl) {
-  BinnedWave<T> wv;
-  if (!wv.init(g, coord, order, nbins)) return;
+                                                                     float* __restrict__ gdata_cl, int per_wave) {
   const int lane = threadIdx.x & 63, ncorner = 1 << g.dims;
   constexpr int PU = 8;  // output-gradient rows in flight
   for (int c0 = 0; c0 < g.channel; c0 += 64) {
@@ -485,24 +485,30 @@ __global__ __launch_bounds__(kBlock) void nd_grad_data_binned_kernel(NdGeo g, co
 #define DK_FLUSH()                                                                             \
   _Pragma("unroll") for (int i = 0; i < kClCorners; ++i) if (cin && i < ncorner && acc[i] != 0.f) \
       atomicAdd(gdata_cl + (size_t)at[i] * g.channel + c, acc[i])
-    for (int q0 = 0; q0 < wv.npts; q0 += PU) {
-      float go[PU];
+    // the sums of a cell stay in registers across the wave's chunks: when thousands of points
+    // share a cell, fewer waves send fewer atomics to the same rows
+    for (int sub = 0; sub < per_wave; ++sub) {
+      BinnedWave<T> wv;
+      if (!wv.init(g, coord, order, nbins, per_wave, sub)) break;
+      for (int q0 = 0; q0 < wv.npts; q0 += PU) {
+        float go[PU];
 #pragma unroll
-      for (int u = 0; u < PU; ++u)
-        go[u] = (cin && q0 + u < wv.npts) ? ld(gout + wv.id_of(min(q0 + u, wv.npts - 1)) * g.channel + c) : 0.f;
+        for (int u = 0; u < PU; ++u)
+          go[u] = (cin && q0 + u < wv.npts) ? ld(gout + wv.id_of(min(q0 + u, wv.npts - 1)) * g.channel + c) : 0.f;
 #pragma unroll
-      for (int u = 0; u < PU; ++u) {
-        const int q = q0 + u;
-        if (q < wv.npts) {
-          const int key = wv.key_of(q);
-          if (key != cur) {  // wave-uniform: the sums of the finished cell leave
-            DK_FLUSH();
-            cur = key;
+        for (int u = 0; u < PU; ++u) {
+          const int q = q0 + u;
+          if (q < wv.npts) {
+            const int key = wv.key_of(q);
+            if (key != cur) {  // wave-uniform: the sums of the finished cell leave
+              DK_FLUSH();
+              cur = key;
 #pragma unroll
-            for (int i = 0; i < kClCorners; ++i) acc[i] = 0.f, at[i] = wv.off_of(i, q);
+              for (int i = 0; i < kClCorners; ++i) acc[i] = 0.f, at[i] = wv.off_of(i, q);
+            }
+#pragma unroll
+            for (int i = 0; i < kClCorners; ++i) acc[i] += wv.w_of(i, q) * go[u];
           }
-#pragma unroll
-          for (int i = 0; i < kClCorners; ++i) acc[i] += wv.w_of(i, q) * go[u];
         }
       }
     }
@@ -778,7 +784,11 @@ void nd_grad_data(const dk_nd_desc& d, const T* gout, const T* coord, T* gdata, 
       nd_fill_zero_kernel<float><<<grid_for(n_data), kBlock, 0, stream>>>(acc, n_data);
       if (const int bins = nd_bins(d)) {
         const int* order = sort_points<T>(g, coord, bins, static_cast<char*>(ws) + round256((size_t)n_data * sizeof(float)), stream);
-        nd_grad_data_binned_kernel<T><<<(unsigned)((g.batch + 255) / 256), kBlock, 0, stream>>>(g, gout, coord, order, bins, acc);
+        // chunks of 64 points per wave: as many as keep about 16 waves per CU in the grid
+        int per_wave = 1;
+        while (per_wave < 8 && g.batch / (64L * per_wave * 2) >= 4096) per_wave *= 2;
+        const long waves = (g.batch + 64L * per_wave - 1) / (64L * per_wave);
+        nd_grad_data_binned_kernel<T><<<(unsigned)((waves + 3) / 4), kBlock, 0, stream>>>(g, gout, coord, order, bins, acc, per_wave);
       } else {
         const int ppw = points_per_wave(g);
         const long waves = (g.batch + ppw - 1) / ppw;
