@@ -337,23 +337,33 @@ __global__ __launch_bounds__(kDBlock, 2) void deform_grad_coord_kernel(
 // One block per (image, group, channel chunk); blockDim = output pixels rounded up to a wave.
 // The kernel for planes of more than 1024 output pixels further down always uses the 2^-44 grid.
 // ---------------------------------------------------------------------------
+// max |p[i]| into *out (as the bits of a non-negative float, which order like unsigned integers).
+// 16-byte loads, four in flight per thread; p must be 16-byte aligned (the host checks).
 template <typename T>
 __global__ __launch_bounds__(256) void absmax_kernel(const T* __restrict__ p, long n, unsigned* __restrict__ out) {
   __shared__ float wave_max[4];
+  constexpr int V = 16 / (int)sizeof(T);
+  struct alignas(16) Vec {
+    T e[V];
+  };
+  const long nv = n / V, stride = (long)gridDim.x * blockDim.x, tid = (long)blockIdx.x * blockDim.x + threadIdx.x;
+  const Vec* pv = reinterpret_cast<const Vec*>(p);
   float m = 0.f;
-  const long stride = (long)gridDim.x * blockDim.x;
-  constexpr int kInFlight = 8;  // independent loads per thread and trip
-  for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += kInFlight * stride) {
-    float v[kInFlight];
+  constexpr int kInFlight = 4;
+  for (long i = tid; i < nv; i += kInFlight * stride) {
+    Vec q[kInFlight];
 #pragma unroll
-    for (int k = 0; k < kInFlight; ++k) v[k] = i + k * stride < n ? fabsf(ld(p + i + k * stride)) : 0.f;
+    for (int k = 0; k < kInFlight; ++k) q[k] = pv[min(i + k * stride, nv - 1)];  // a repeated element does not change a maximum
 #pragma unroll
-    for (int k = 0; k < kInFlight; ++k) m = fmaxf(m, v[k]);
+    for (int k = 0; k < kInFlight; ++k)
+#pragma unroll
+      for (int e = 0; e < V; ++e) m = fmaxf(m, fabsf(ld(&q[k].e[e])));
   }
+  for (long i = nv * V + tid; i < n; i += stride) m = fmaxf(m, fabsf(ld(p + i)));
   for (int s = 32; s > 0; s >>= 1) m = fmaxf(m, __shfl_xor(m, s));
   if ((threadIdx.x & 63) == 0) wave_max[threadIdx.x >> 6] = m;
   __syncthreads();
-  // one atomic per block (atomics on one address serialise): non-negative floats order like their bits
+  // one atomic per block (atomics on one address serialise)
   if (threadIdx.x == 0)
     atomicMax(out, __float_as_uint(fmaxf(fmaxf(wave_max[0], wave_max[1]), fmaxf(wave_max[2], wave_max[3]))));
 }
@@ -879,10 +889,11 @@ bool run_deform_grad_input(const Geo& g, const T* gout, const T* off, const T* r
   } else if (!d.ok) {
     return false;
   }
+  if (reinterpret_cast<uintptr_t>(gout) % 16 != 0) return false;  // absmax_kernel reads 16-byte vectors
   unsigned* gmax = static_cast<unsigned*>(ws);
   clear_word_kernel<<<1, 1, 0, stream>>>(gmax);
   const long n = (long)g.batch * g.channel * g.out_h * g.out_w;
-  absmax_kernel<T><<<(unsigned)std::min<long>(2048, (n + 255) / 256), 256, 0, stream>>>(gout, n, gmax);
+  absmax_kernel<T><<<(unsigned)std::min<long>(1024, (n / (16 / (long)sizeof(T)) + 1023) / 1024 + 1), 256, 0, stream>>>(gout, n, gmax);
   if (tiled) {
     auto kernel = deform_grad_input_tiled_kernel<T, SH, SW>;
     if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
