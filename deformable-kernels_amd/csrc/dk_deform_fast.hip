@@ -782,7 +782,9 @@ struct DeformPlan {
 };
 
 // table_floats: LDS floats per channel beyond the two planes; plane_floats: LDS floats per plane
-DeformPlan deform_plan(const Geo& g, int table_floats, int planes, int block) {
+// blocks_per_cu: how many workgroups per CU the channel chunking aims at (measured per kernel on
+// N=64 C=512 28x28 -> 14x14: forward and grad input 4, grad offset and grad filter 3, grad rotation 2)
+DeformPlan deform_plan(const Geo& g, int table_floats, int planes, int block, int blocks_per_cu) {
   DeformPlan d{};
   d.ok = false;
   if (path_disabled("DK_NO_DEFORM_FAST")) return d;
@@ -804,9 +806,9 @@ DeformPlan deform_plan(const Geo& g, int table_floats, int planes, int block) {
   const long room = 64 * 1024 - plane_bytes;
   if (room < (long)table_floats * 4 * 4) return d;
   const int fit = (int)std::min<long>(room / ((long)table_floats * 4), cpg);
-  // enough blocks for two per CU, chunks of at least 8 channels
+  // enough blocks for blocks_per_cu per CU, chunks of at least 8 channels
   const long base = (long)d.tiles * g.batch * g.groups;
-  int chunks = (int)std::max<long>(1, (2 * 256 + base - 1) / base);
+  int chunks = (int)std::max<long>(1, (blocks_per_cu * 256L + base - 1) / base);
   chunks = std::min(chunks, std::max(1, cpg / 8));
   chunks = std::max(chunks, ceil_div(cpg, fit));
   d.per = ceil_div(cpg, chunks);
@@ -820,7 +822,7 @@ DeformPlan deform_plan(const Geo& g, int table_floats, int planes, int block) {
 template <typename T, int SH, int SW>
 bool run_deform_forward(const Geo& g, const T* x, const T* off, const T* rot, const T* filter, T* out,
                         hipStream_t stream) {
-  const DeformPlan d = deform_plan(g, WideTable<SH, SW>::SIZE, 2, kDBlock);
+  const DeformPlan d = deform_plan(g, WideTable<SH, SW>::SIZE, 2, kDBlock, 4);
   if (!d.ok) return false;
   const unsigned grid = (unsigned)xcd_grid_size((long)d.tiles * d.chunks * g.batch * g.groups);
 #define DK_LAUNCH(NP) \
@@ -836,7 +838,7 @@ bool run_deform_forward(const Geo& g, const T* x, const T* off, const T* rot, co
 template <typename T, int SH, int SW>
 bool run_deform_grad_coord(const Geo& g, bool rotation, const T* gout, const T* x, const T* off, const T* rot,
                            const T* filter, T* result, float* ws, hipStream_t stream) {
-  const DeformPlan d = deform_plan(g, WideTable<SH, SW>::SIZE, 2, kDBlock);
+  const DeformPlan d = deform_plan(g, WideTable<SH, SW>::SIZE, 2, kDBlock, rotation ? 2 : 3);
   if (!d.ok) return false;
   const unsigned grid = (unsigned)xcd_grid_size((long)d.tiles * d.chunks * g.batch * g.groups);
 #define DK_LAUNCH(NP, ROT)                                                                          \
@@ -869,7 +871,7 @@ DeformPlan grad_input_plan(const Geo& g) {
   d.ok = false;
   if (g.out_h * g.out_w > 1024) return d;
   // 4 floats of LDS per plane element (two 64-bit planes), one more float per channel for max|Wt[c]|
-  return deform_plan(g, WideTable<SH, SW>::SIZE + 1, 4, grad_input_block(g));
+  return deform_plan(g, WideTable<SH, SW>::SIZE + 1, 4, grad_input_block(g), 4);
 }
 
 template <typename T, int SH, int SW>
@@ -881,7 +883,7 @@ bool run_deform_grad_input(const Geo& g, const T* gout, const T* off, const T* r
   int tiled_shift = 0;
   if (tiled) {
     // the basic limits of the tuned family, then room for kTiledCh 64-bit planes in LDS
-    const DeformPlan basic = deform_plan(g, WideTable<SH, SW>::SIZE, 0, 1024);
+    const DeformPlan basic = deform_plan(g, WideTable<SH, SW>::SIZE, 0, 1024, 2);
     if (!basic.ok) return false;
     tiled_shift = basic.shift;
     tiled_lds = ((size_t)2 * kTiledCh * basic.PS + (size_t)kTiledCh * WideTable<SH, SW>::SIZE + kTiledCh) * sizeof(float);
@@ -916,7 +918,7 @@ bool run_deform_grad_filter(const Geo& g, const T* gout, const T* x, const T* of
   if constexpr (SH * SW > 16) {
     return false;  // 25 dense accumulators and 90 hat weights per lane do not fit the register budget
   } else {
-    const DeformPlan d = deform_plan(g, (kDBlock / 64) * SH * SW, 2, kDBlock);
+    const DeformPlan d = deform_plan(g, (kDBlock / 64) * SH * SW, 2, kDBlock, 3);
     if (!d.ok) return false;
     const unsigned grid = (unsigned)xcd_grid_size((long)d.tiles * d.chunks * g.batch * g.groups);
 #define DK_LAUNCH(NP) \
@@ -958,9 +960,9 @@ bool fast_deform_grad_coord(const Geo& g, bool rotation, const T* gout, const T*
 
 size_t fast_deform_grad_coord_workspace(const Geo& g, bool rotation) {
   const int table = g.scope_h == 3 ? WideTable<3, 3>::SIZE : g.scope_h == 4 ? WideTable<4, 4>::SIZE : WideTable<5, 5>::SIZE;
-  const DeformPlan d = deform_plan(g, table, 2, kDBlock);
+  const DeformPlan d = deform_plan(g, table, 2, kDBlock, rotation ? 2 : 3);
   if (!d.ok) return 0;
-  (void)rotation;  // both lay out chunks * groups * batch planes of 18 * out pixels
+  // both lay out chunks * groups * batch planes of 18 * out pixels
   return (size_t)d.chunks * g.groups * g.batch * 18 * g.out_h * g.out_w * sizeof(float);
 }
 
