@@ -365,6 +365,45 @@ int dk_deformable_sample_depthwise_backward_rotation(const dk_conv_desc* desc, c
   });
 }
 
+// ---- offset branch -----------------------------------------------------------------------
+
+static int check_offset_conv(const dk_offset_conv_desc* d) {
+  if (!d) return DK_ERR_NULL_POINTER;
+  if (d->batch < 0 || d->in_channels <= 0 || d->out_channels <= 0 || d->h <= 0 || d->w <= 0) return DK_ERR_BAD_SHAPE;
+  if (d->dtype != DK_F32) return DK_ERR_UNSUPPORTED;
+  if ((long)d->batch * d->in_channels * d->h * d->w > kMaxElems) return DK_ERR_TOO_LARGE;
+  if (!offset_conv_supported(d->in_channels, d->out_channels, d->h, d->w)) return DK_ERR_UNSUPPORTED;
+  return DK_OK;
+}
+
+int dk_offset_conv_supported(const dk_offset_conv_desc* desc) { return check_offset_conv(desc) == DK_OK; }
+
+int dk_offset_conv_worthwhile(const dk_offset_conv_desc* desc) {
+  return check_offset_conv(desc) == DK_OK &&
+         offset_conv_worthwhile(desc->batch, desc->in_channels, desc->out_channels, desc->h, desc->w);
+}
+
+size_t dk_offset_conv_forward_workspace(const dk_offset_conv_desc* desc) {
+  if (check_offset_conv(desc) != DK_OK) return 0;
+  return offset_conv_workspace(desc->in_channels, desc->out_channels);
+}
+
+int dk_offset_conv_forward(const dk_offset_conv_desc* desc, const void* input, const void* weight,
+                           const void* bias, void* output, void* workspace, size_t workspace_bytes,
+                           void* stream) {
+  const int rc = check_offset_conv(desc);
+  if (rc != DK_OK) return rc;
+  if (!input || !weight || !bias || !output) return DK_ERR_NULL_POINTER;
+  const size_t need = offset_conv_workspace(desc->in_channels, desc->out_channels);
+  if (!workspace || workspace_bytes < need) return DK_ERR_WORKSPACE;
+  if (!offset_conv_forward(desc->batch, desc->in_channels, desc->out_channels, desc->h, desc->w,
+                           static_cast<const float*>(input), static_cast<const float*>(weight),
+                           static_cast<const float*>(bias), static_cast<float*>(output), workspace,
+                           static_cast<hipStream_t>(stream)))
+    return DK_ERR_UNSUPPORTED;
+  return launch_status();
+}
+
 // ---- N-d linear sample --------------------------------------------------------------------
 
 static int check_nd(const dk_nd_desc* d) {

@@ -76,4 +76,11 @@ template <typename T>
 void generic_grad_filter(const Geo& g, bool deform, const T* gout, const T* x, const T* off,
                          const T* rot, T* gfilter, void* ws, hipStream_t stream);
 
+// dk_offset_conv.hip: the 3x3 offset-branch convolution (stride 1, padding 1, fp32)
+bool offset_conv_supported(int cin, int cout, int h, int w);
+bool offset_conv_worthwhile(int batch, int cin, int cout, int h, int w);
+size_t offset_conv_workspace(int cin, int cout);
+bool offset_conv_forward(int batch, int cin, int cout, int h, int w, const float* x, const float* weight,
+                         const float* bias, float* out, void* ws, hipStream_t stream);
+
 }  // namespace dk

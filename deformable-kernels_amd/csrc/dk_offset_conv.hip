@@ -1,0 +1,303 @@
+// The offset branch of a deformable-kernel layer: the 3x3 convolution that predicts the
+// kernel-space offsets ("rotation_conv", reference modules/deform_kernel.py:165-168 and :214-216:
+// nn.Conv2d(in_planes, rotation_groups * k * k * 2, k, stride, padding, dilation, bias=True)).
+// It has many input channels and only 18 output channels per rotation group, a shape on which
+// the library convolution spends twice the time of the deformable-kernel operator itself.
+//
+// Forward as a shift-GEMM on the matrix cores, full fp32 (v_mfma_f32_16x16x4_f32):
+//   out[o][p] = bias[o] + sum over taps t, channels c of W[o][c][t] * x[c][p + shift_t].
+// A workgroup owns a tile of TH rows of one image (up to 448 pixels = 28 groups of 16 pixels,
+// seven per wave) and walks the input channels in chunks of 16, staged zero-padded in LDS.
+// Per tap and 4 channels one MFMA per pixel group multiplies the 16 x 4 block of weights
+// (outputs 0..15; A operand, one coalesced 256-byte load from the packed copy [tap][c][16]) with
+// the 4 x 16 block of shifted inputs (B operand, one LDS read per lane: lane = (channel k,
+// pixel n); the channel pitch is 16 mod 64 words so the four channels of a read hit disjoint
+// banks).  The outputs beyond the 16th (two of the 18) are summed on the vector ALU, their
+// weights staged in LDS per chunk and read as broadcasts.  Stride 1, padding 1, no dilation, fp32; other cases are left
+// to the caller's library convolution.
+#include <algorithm>
+
+#include "dk_kernels.h"
+
+namespace dk {
+
+namespace {
+
+constexpr int kCvBlock = 256;
+constexpr int kCvChunk = 16;     // input channels staged per pass
+constexpr int kCvGroups = 7;     // 16-pixel groups per wave
+constexpr int kCvTilePix = kCvGroups * 16 * (kCvBlock / 64);  // 448
+
+typedef float v4f __attribute__((ext_vector_type(4)));
+
+struct ConvGeo {
+  int batch, cin, cout, h;
+  int tiles;  // row tiles per image
+};
+
+// The plane width is a template constant, so that every LDS offset of the unrolled tap / channel
+// loops is an immediate: rows per tile, 64-column segments per staged row, floats per staged
+// row and per staged channel (rounded up to 16 mod 64).
+template <int W>
+struct ConvTile {
+  static constexpr int TH = W <= 56 ? 8 : 4;  // (4 and 2 rows at width 56 measured slower: more halo rows staged)
+  static constexpr int SEGS = (W + 63) / 64;
+  static constexpr int RS = W + 2;
+  static constexpr int PS = ((TH + 2) * RS + 47) / 64 * 64 + 16;
+  static_assert(TH * W <= kCvTilePix && PS >= (TH + 2) * RS && PS % 64 == 16, "tile does not fit the workgroup");
+};
+
+// weights [cout][cin][3][3] -> w16 [9][cin][16] (outputs 0..15, zero where cout < 16) and
+// wrest [9][cin][rest] (outputs 16..)
+__global__ void conv_pack_weights_kernel(const float* __restrict__ w, int cout, int cin, int rest,
+                                         float* __restrict__ w16, float* __restrict__ wrest) {
+  const int idx = blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx < 9 * cin * 16) {
+    const int m = idx % 16, c = idx / 16 % cin, t = idx / 16 / cin;
+    w16[idx] = m < cout ? w[((size_t)m * cin + c) * 9 + t] : 0.f;
+  }
+  if (idx < 9 * cin * rest) {
+    const int o = 16 + idx % rest, c = idx / rest % cin, t = idx / rest / cin;
+    wrest[idx] = w[((size_t)o * cin + c) * 9 + t];
+  }
+}
+
+template <int W, int REST>
+__global__ __launch_bounds__(kCvBlock, 2) void offset_conv_forward_kernel(
+    ConvGeo g, const float* __restrict__ x, const float* __restrict__ w16, const float* __restrict__ wrest,
+    const float* __restrict__ bias, float* __restrict__ out) {
+  extern __shared__ __align__(16) float xs[];  // [kCvChunk][PS], then the chunk's VALU-path weights [kCvChunk][9][REST]
+  constexpr int TH = ConvTile<W>::TH, SEGS = ConvTile<W>::SEGS, RS = ConvTile<W>::RS, PS = ConvTile<W>::PS;
+  constexpr int kStage = (kCvChunk / 4) * (TH + 2) * SEGS;  // row segments of 64 columns a wave stages per chunk
+  constexpr int kPixPerThread = (kCvTilePix + kCvBlock - 1) / kCvBlock;  // of the VALU path
+
+  const int total = g.batch * g.tiles;
+  const int lb = logical_block(total);
+  if (lb >= total) return;
+  const int n = lb / g.tiles, r0 = (lb % g.tiles) * TH;
+  // the wave index enters scalar offsets and loop bounds: tell the compiler it is uniform
+  const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  constexpr int tile_pix = TH * W, groups = (tile_pix + 15) / 16;
+  constexpr int GPW = (groups + 3) / 4;  // pixel groups per wave; a wave with fewer repeats its last pixel (not stored)
+
+  // LDS float index of the lane's pixel of each group (padded coordinates), plus the lane's
+  // channel of a 4-channel step
+  int base[GPW];
+#pragma unroll
+  for (int i = 0; i < GPW; ++i) {
+    const int q = min((wave + 4 * i) * 16 + (lane & 15), tile_pix - 1);
+    base[i] = (q / W + 1) * RS + q % W + 1 + (lane >> 4) * PS;
+  }
+  int rbase[kPixPerThread];
+#pragma unroll
+  for (int j = 0; j < kPixPerThread; ++j) {
+    const int q = min((int)threadIdx.x + kCvBlock * j, tile_pix - 1);
+    rbase[j] = (q / W + 1) * RS + q % W + 1;
+  }
+
+  for (int e = threadIdx.x; e < kCvChunk * PS; e += kCvBlock) xs[e] = 0.f;  // the padding stays zero
+
+  v4f acc[GPW];
+#pragma unroll
+  for (int i = 0; i < GPW; ++i) acc[i] = v4f{0.f, 0.f, 0.f, 0.f};
+  float racc[kPixPerThread][REST > 0 ? REST : 1];
+#pragma unroll
+  for (int j = 0; j < kPixPerThread; ++j)
+#pragma unroll
+    for (int o = 0; o < (REST > 0 ? REST : 1); ++o) racc[j][o] = 0.f;
+
+  // staging: wave w takes channels w, w + 4, w + 8, w + 12 of the chunk; its i-th row segment is
+  // (channel w + 4 * (i / rows), staged row, 64-column segment).  Buffer loads: the lane part of
+  // the address is one register per segment, the (channel, row) part a scalar offset (which
+  // the hardware's range check does not see, so it must stay inside the chunk), and rows or
+  // columns outside the image read 0 through an out-of-range lane offset.
+  const int plane = g.h * W;
+  unsigned vcol[SEGS];
+#pragma unroll
+  for (int sg = 0; sg < SEGS; ++sg)
+    vcol[sg] = sg * 64 + lane < W ? (unsigned)((sg * 64 + lane) * 4) : kOutOfRange;
+  const int lds_row0 = wave * PS + 1 + lane;  // + immediate per row segment
+  float stage[kStage];
+  // the chunk's weights of the outputs beyond the 16th go through LDS as well: read as scalars
+  // from memory they cost a round trip per (channel, tap)
+  constexpr int kRestW = kCvChunk * 9 * REST, kRestPerThread = (kRestW + kCvBlock - 1) / kCvBlock;
+  float* wl = xs + kCvChunk * PS;
+  float wstage[kRestPerThread > 0 ? kRestPerThread : 1];
+#define DK_LOAD_CHUNK(CK)                                                                                  \
+  {                                                                                                        \
+    _Pragma("unroll") for (int u = 0; u < kRestPerThread; ++u) {                                           \
+      const int e = (int)threadIdx.x + kCvBlock * u; /* = (c * 9 + t) * REST + o */                        \
+      const int o = e % (REST > 0 ? REST : 1), t = e / (REST > 0 ? REST : 1) % 9, c = e / (REST > 0 ? REST : 1) / 9; \
+      wstage[u] = e < kRestW ? wrest[((size_t)t * g.cin + (CK) * kCvChunk + c) * REST + o] : 0.f;          \
+    }                                                                                                      \
+    const rsrc_t rx = plane_rsrc(x + ((size_t)n * g.cin + (size_t)(CK) * kCvChunk) * plane, kCvChunk * plane); \
+    _Pragma("unroll") for (int i = 0; i < kStage; ++i) {                                                   \
+      const int chq = i / ((TH + 2) * SEGS), ry = i / SEGS % (TH + 2), sg = i % SEGS;                      \
+      const int row = r0 - 1 + ry;                                                                         \
+      const bool ok = row >= 0 && row < g.h;                                                               \
+      const int soff = ok ? ((wave + 4 * chq) * g.h + row) * W * 4 : 0;                                    \
+      stage[i] = __builtin_bit_cast(                                                                       \
+          float, __builtin_amdgcn_raw_buffer_load_b32(rx, (int)(ok ? vcol[sg] : kOutOfRange), soff, 0));   \
+    }                                                                                                      \
+  }
+
+  const rsrc_t rw = plane_rsrc(w16, 9 * g.cin * 16);
+  const int nchunks = g.cin / kCvChunk;
+  DK_LOAD_CHUNK(0)
+  for (int ck = 0; ck < nchunks; ++ck) {
+    __syncthreads();  // every wave is done with the previous chunk
+#pragma unroll
+    for (int i = 0; i < kStage; ++i) {
+      const int chq = i / ((TH + 2) * SEGS), ry = i / SEGS % (TH + 2), sg = i % SEGS;
+      if (sg * 64 + lane < W) xs[lds_row0 + 4 * chq * PS + ry * RS + sg * 64] = stage[i];
+    }
+#pragma unroll
+    for (int u = 0; u < kRestPerThread; ++u)
+      if ((int)threadIdx.x + kCvBlock * u < kRestW) wl[threadIdx.x + kCvBlock * u] = wstage[u];
+    __syncthreads();
+    if (ck + 1 < nchunks) DK_LOAD_CHUNK(ck + 1)
+
+    // matrix-core part: outputs 0..15
+    // A operand of (tap t, channels 4 cs .. 4 cs + 3): w16[(t * cin + c) * 16 + m], lane = 16 k + m
+    auto load_a = [&](int t, int cs) {
+      return __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(
+                                           rw, lane * 4, ((t * g.cin + ck * kCvChunk + 4 * cs) * 16) * 4, 0));
+    };
+    float a[4], a_next[4];
+#pragma unroll
+    for (int cs = 0; cs < 4; ++cs) a[cs] = load_a(0, cs);
+#pragma unroll
+    for (int t = 0; t < 9; ++t) {
+      if (t + 1 < 9) {
+#pragma unroll
+        for (int cs = 0; cs < 4; ++cs) a_next[cs] = load_a(t + 1, cs);
+      }
+      const int shift = (t / 3 - 1) * RS + (t % 3 - 1);
+#pragma unroll
+      for (int cs = 0; cs < 4; ++cs) {
+#pragma unroll
+        for (int i = 0; i < GPW; ++i) {
+          const float b = xs[base[i] + 4 * cs * PS + shift];
+          acc[i] = __builtin_amdgcn_mfma_f32_16x16x4f32(a[cs], b, acc[i], 0, 0, 0);
+        }
+      }
+#pragma unroll
+      for (int cs = 0; cs < 4; ++cs) a[cs] = a_next[cs];
+      // keep the scheduler from hoisting the LDS reads of all nine taps to the front (252 registers)
+      __builtin_amdgcn_sched_barrier(0);
+    }
+
+    // vector part: the outputs beyond the 16th; the weights are LDS broadcast reads
+    if (REST > 0) {
+#pragma unroll 4
+      for (int c = 0; c < kCvChunk; ++c) {
+        float wv[9][REST > 0 ? REST : 1];
+#pragma unroll
+        for (int t = 0; t < 9; ++t)
+#pragma unroll
+          for (int o = 0; o < REST; ++o) wv[t][o] = wl[(c * 9 + t) * REST + o];
+#pragma unroll
+        for (int t = 0; t < 9; ++t) {
+          const int shift = (t / 3 - 1) * RS + (t % 3 - 1);
+#pragma unroll
+          for (int j = 0; j < kPixPerThread; ++j) {
+            const float xv = xs[c * PS + rbase[j] + shift];
+#pragma unroll
+            for (int o = 0; o < REST; ++o) racc[j][o] = fmaf(wv[t][o], xv, racc[j][o]);
+          }
+        }
+      }
+    }
+  }
+
+#undef DK_LOAD_CHUNK
+  // results: lane holds outputs 4 * (lane / 16) + j of pixel lane % 16 of each of its groups
+  float* on = out + (size_t)n * g.cout * plane;  // plane = h * W
+#pragma unroll
+  for (int i = 0; i < GPW; ++i) {
+    const int q = (wave + 4 * i) * 16 + (lane & 15);
+    const int row = r0 + q / W;
+    if (q < tile_pix && row < g.h) {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int o = 4 * (lane >> 4) + j;
+        if (o < g.cout) on[(size_t)o * plane + row * W + q % W] = acc[i][j] + bias[o];
+      }
+    }
+  }
+  if (REST > 0) {
+#pragma unroll
+    for (int j = 0; j < kPixPerThread; ++j) {
+      const int q = (int)threadIdx.x + kCvBlock * j;
+      const int row = r0 + q / W;
+      if (q < tile_pix && row < g.h) {
+#pragma unroll
+        for (int o = 0; o < REST; ++o)
+          on[(size_t)(16 + o) * plane + row * W + q % W] = racc[j][o] + bias[16 + o];
+      }
+    }
+  }
+}
+
+size_t round256(size_t n) { return (n + 255) / 256 * 256; }
+
+}  // namespace
+
+bool offset_conv_supported(int cin, int cout, int h, int w) {
+  const bool outputs_ok = (cout >= 1 && cout <= 16) || cout == 18 || cout == 20;  // the instantiated VALU widths
+  return cin >= kCvChunk && cin % kCvChunk == 0 && outputs_ok && (w == 7 || w == 14 || w == 28 || w == 56 || w == 112) && h >= 1 &&
+         (long)cin * h * w < (1L << 31) / 4;
+}
+
+// Whether the kernel is also the faster choice (measured against the library convolution on
+// MI355X): it is on the 56- and 112-wide planes once there is about a workgroup per CU; on
+// smaller planes a workgroup's serial walk over all input channels loses.
+bool offset_conv_worthwhile(int batch, int cin, int cout, int h, int w) {
+  if (!offset_conv_supported(cin, cout, h, w) || w < 56) return false;
+  const int th = w <= 56 ? 8 : 4;
+  return (long)batch * ceil_div(h, th) >= 192;
+}
+
+// packed weights: w16 [9][cin][16] and wrest [9][cin][cout - 16]
+size_t offset_conv_workspace(int cin, int cout) {
+  return round256((size_t)9 * cin * 16 * sizeof(float)) + round256((size_t)9 * cin * std::max(0, cout - 16) * sizeof(float));
+}
+
+bool offset_conv_forward(int batch, int cin, int cout, int h, int w, const float* x, const float* weight,
+                         const float* bias, float* out, void* ws, hipStream_t stream) {
+  if (!offset_conv_supported(cin, cout, h, w)) return false;
+  if (batch == 0) return true;
+  const int rest = std::max(0, cout - 16);
+  float* w16 = static_cast<float*>(ws);
+  float* wrest = reinterpret_cast<float*>(static_cast<char*>(ws) + round256((size_t)9 * cin * 16 * sizeof(float)));
+  conv_pack_weights_kernel<<<ceil_div(9 * cin * 16, 256), 256, 0, stream>>>(weight, cout, cin, rest, w16, wrest);
+  ConvGeo g;
+  g.batch = batch, g.cin = cin, g.cout = cout, g.h = h;
+#define DK_LAUNCH(WW, REST)                                                                             \
+  {                                                                                                     \
+    g.tiles = ceil_div(h, ConvTile<WW>::TH);                                                            \
+    const size_t lds = (size_t)kCvChunk * (ConvTile<WW>::PS + 9 * REST) * sizeof(float);                \
+    const unsigned grid = (unsigned)xcd_grid_size((long)batch * g.tiles);                               \
+    offset_conv_forward_kernel<WW, REST><<<grid, kCvBlock, lds, stream>>>(g, x, w16, wrest, bias, out); \
+  }
+#define DK_WIDTH(REST)                       \
+  switch (w) {                               \
+    case 7: DK_LAUNCH(7, REST) break;        \
+    case 14: DK_LAUNCH(14, REST) break;      \
+    case 28: DK_LAUNCH(28, REST) break;      \
+    case 56: DK_LAUNCH(56, REST) break;      \
+    case 112: DK_LAUNCH(112, REST) break;    \
+    default: return false;                   \
+  }
+  switch (rest) {
+    case 0: DK_WIDTH(0) break;
+    case 2: DK_WIDTH(2) break;
+    case 4: DK_WIDTH(4) break;
+    default: return false;
+  }
+#undef DK_WIDTH
+#undef DK_LAUNCH
+  return true;
+}
+
+}  // namespace dk

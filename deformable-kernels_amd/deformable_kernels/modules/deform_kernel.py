@@ -11,7 +11,7 @@ autocast-aware cast.
 import torch
 from torch import nn
 
-from ..ops.deform_kernel.functions import nd_linear_sample, sample_depthwise
+from ..ops.deform_kernel.functions import nd_linear_sample, offset_conv, sample_depthwise
 from ..ops.deform_kernel.modules import (
     SampleDepthwise,
     DeformableSampleDepthwise,
@@ -170,6 +170,9 @@ class LocalDeformKernel2d(nn.Module):
         # True: the operator clamps the offsets itself (same values and gradients as clamping
         # the tensor first, without the extra passes over it); False: the reference's sequence
         self.fused_clip = True
+        # True: rotation_conv's forward runs on the library's own kernel where that is faster
+        # (wide planes, float32, stride 1); its parameters and gradients are unchanged
+        self.native_offset_conv = True
 
         self.inner_conv = SampleDepthwise(
             weight_shape, in_planes, out_planes, kernel_size=kernel_size, stride=stride,
@@ -194,7 +197,11 @@ class LocalDeformKernel2d(nn.Module):
             'but get {}'.format(clip))
 
     def forward(self, x):
-        rotation = self.rotation_conv(x)
+        conv = self.rotation_conv
+        if self.native_offset_conv:
+            rotation = offset_conv(x, conv.weight, conv.bias, conv.stride, conv.padding, conv.dilation)
+        else:
+            rotation = conv(x)
         if self.rotation_clip is not None and self.fused_clip and self.weight_dilate == 1 \
                 and len(self.weight_shape) == 2:
             clip = self.rotation_clip

@@ -33,12 +33,16 @@ class NdDesc(ctypes.Structure):
                 ("shape", ctypes.c_int32 * ND_MAX_DIMS), ("dtype", ctypes.c_int32)]
 
 
+class OffsetConvDesc(ctypes.Structure):
+    _fields_ = [(n, ctypes.c_int32) for n in ("batch", "in_channels", "out_channels", "h", "w", "dtype")]
+
+
 class DkError(RuntimeError):
     pass
 
 
 _P, _SZ = ctypes.c_void_p, ctypes.c_size_t
-_CD, _ND = ctypes.POINTER(ConvDesc), ctypes.POINTER(NdDesc)
+_CD, _ND, _OC = ctypes.POINTER(ConvDesc), ctypes.POINTER(NdDesc), ctypes.POINTER(OffsetConvDesc)
 
 # name -> (restype, argtypes); must list every symbol include/dk_hip.h declares
 SIGNATURES = {
@@ -68,6 +72,10 @@ SIGNATURES = {
     "dk_nd_linear_sample_backward_data": (ctypes.c_int, [_ND, _P, _P, _P, _P, _SZ, _P]),
     "dk_nd_linear_sample_backward_coord_workspace": (_SZ, [_ND]),
     "dk_nd_linear_sample_backward_coord": (ctypes.c_int, [_ND, _P, _P, _P, _P, _P, _SZ, _P]),
+    "dk_offset_conv_supported": (ctypes.c_int, [_OC]),
+    "dk_offset_conv_worthwhile": (ctypes.c_int, [_OC]),
+    "dk_offset_conv_forward_workspace": (_SZ, [_OC]),
+    "dk_offset_conv_forward": (ctypes.c_int, [_OC, _P, _P, _P, _P, _P, _SZ, _P]),
 }
 
 _lib = None

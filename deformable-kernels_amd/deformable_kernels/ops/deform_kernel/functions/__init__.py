@@ -3,9 +3,12 @@ from .filter_sample_depthwise import (
     deform_sample_depthwise,
 )
 from .nd_linear_sample import nd_linear_sample
+from .offset_conv import offset_conv, offset_conv_supported
 
 __all__ = [
     'sample_depthwise',
     'deform_sample_depthwise',
     'nd_linear_sample',
+    'offset_conv',
+    'offset_conv_supported',
 ]

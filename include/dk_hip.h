@@ -214,6 +214,30 @@ int dk_nd_linear_sample_backward_coord(const dk_nd_desc *desc, const void *out_g
                                        const void *data, const void *coord, void *coord_grad,
                                        void *workspace, size_t workspace_bytes, void *stream);
 
+/* ---- offset branch ---------------------------------------------------------- */
+
+/* The 3x3 convolution that predicts the kernel-space offsets of a LocalDeformKernel2d layer
+ * (modules/deform_kernel.py:165-168: nn.Conv2d(in_planes, rotation_groups*k*k*2, k, stride,
+ * padding, dilation, bias=True), applied at :214).  The reference calls the framework's
+ * convolution there; this entry point is a faster kernel for that one shape family: stride 1,
+ * padding 1, dilation 1, float32, in_channels a multiple of 16, out_channels <= 16 or 18 or 20,
+ * width 7, 14, 28, 56 or 112.  dk_offset_conv_supported() tells whether a shape is covered,
+ * dk_offset_conv_worthwhile() whether it is also expected to beat the library convolution
+ * (56- and 112-wide planes with enough images to fill the GPU); the caller keeps its library
+ * convolution otherwise.
+ *   input [batch, in_channels, h, w], weight [out_channels, in_channels, 3, 3],
+ *   bias [out_channels], output [batch, out_channels, h, w]; workspace: packed weights. */
+typedef struct dk_offset_conv_desc {
+  int32_t batch, in_channels, out_channels, h, w;
+  int32_t dtype; /* DK_F32 */
+} dk_offset_conv_desc;
+int dk_offset_conv_supported(const dk_offset_conv_desc *desc);
+int dk_offset_conv_worthwhile(const dk_offset_conv_desc *desc);
+size_t dk_offset_conv_forward_workspace(const dk_offset_conv_desc *desc);
+int dk_offset_conv_forward(const dk_offset_conv_desc *desc, const void *input, const void *weight,
+                           const void *bias, void *output, void *workspace, size_t workspace_bytes,
+                           void *stream);
+
 /* ---- misc ------------------------------------------------------------------- */
 
 const char *dk_status_string(int status);

@@ -1,0 +1,73 @@
+"""The offset branch's 3x3 convolution (the library's kernel for LocalDeformKernel2d's
+rotation_conv) against torch's convolution: forward within 1e-5 of the float64 result (relative to
+its largest magnitude), gradients equal to those of F.conv2d (they come from the same
+routines), and the module with the kernel switched on and off."""
+import pytest
+import torch
+import torch.nn.functional as F
+
+from _cases import rel_err
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.mark.parametrize("shape", [
+    (2, 16, 5, 7, 18),      # N, C, H, W, out channels: one partial tile
+    (3, 32, 14, 14, 18),
+    (2, 48, 28, 28, 18),    # tile rows 8: the last tile has 4 rows
+    (2, 144, 56, 56, 18),   # the headline layer's offset branch
+    (1, 32, 9, 112, 18),    # two 64-column segments per staged row, tile rows 4
+    (2, 32, 56, 56, 16),    # no outputs beyond the matrix-core tile
+    (2, 32, 20, 56, 8),     # fewer than 16 outputs
+    (1, 16, 13, 28, 20),    # four outputs on the vector path
+])
+def test_forward_matches_float64_convolution(shape):
+    from deformable_kernels.ops.deform_kernel.functions import offset_conv, offset_conv_supported
+    N, C, H, W, O = shape
+    g = torch.Generator().manual_seed(31)
+    dev = torch.device("cuda:0")
+    x = torch.randn(N, C, H, W, generator=g).to(dev)
+    w = (torch.randn(O, C, 3, 3, generator=g) * 0.05).to(dev)
+    b = torch.randn(O, generator=g).to(dev)
+    assert offset_conv_supported(x, w, b, 1, 1, 1)
+    got = offset_conv(x, w, b, force=True)
+    want = F.conv2d(x.double(), w.double(), b.double(), padding=1)
+    assert got.shape == want.shape and got.dtype == torch.float32
+    assert rel_err(got.cpu(), want.cpu()) < 1e-5
+
+
+def test_unsupported_calls_go_to_the_library_convolution():
+    from deformable_kernels.ops.deform_kernel.functions import offset_conv, offset_conv_supported
+    dev = torch.device("cuda:0")
+    x = torch.randn(2, 24, 10, 10, device=dev)   # 24 channels: not a multiple of 16; width 10
+    w = torch.randn(18, 24, 3, 3, device=dev)
+    assert not offset_conv_supported(x, w, None, 1, 1, 1)
+    assert torch.equal(offset_conv(x, w, None), F.conv2d(x, w, None, 1, 1, 1))
+    x2 = torch.randn(2, 32, 56, 56, device=dev)
+    w2 = torch.randn(18, 32, 3, 3, device=dev)
+    assert not offset_conv_supported(x2, w2, None, 2, 1, 1)          # stride 2
+    assert not offset_conv_supported(x2.half(), w2.half(), None, 1, 1, 1)
+    assert torch.equal(offset_conv(x2, w2, None, stride=2), F.conv2d(x2, w2, None, 2, 1, 1))
+
+
+def test_gradients_and_module_switch():
+    from deformable_kernels.modules import LocalDeformKernel2d
+    torch.manual_seed(32)
+    dev = torch.device("cuda:0")
+    C = 16
+    m = LocalDeformKernel2d((4, 4), C, C, 3, 1, 1, 1, C, 1, False, 'scope').to(dev)
+    torch.nn.init.normal_(m.rotation_conv.weight, std=0.1)
+    x = torch.randn(28, C, 56, 56, device=dev)    # 28 images x 7 row tiles: the native kernel is chosen
+    gout = torch.randn(28, C, 56, 56, device=dev)
+    results = []
+    for native in (False, True):
+        m.native_offset_conv = native
+        m.zero_grad()
+        xi = x.clone().requires_grad_()
+        out = m(xi)
+        out.backward(gout)
+        results.append([t.detach().cpu().clone() for t in (
+            out, xi.grad, m.inner_conv.weight.grad, m.rotation_conv.weight.grad, m.rotation_conv.bias.grad)])
+    assert rel_err(results[1][0], results[0][0]) < 1e-5
+    for got, ref in zip(results[1][1:], results[0][1:]):
+        assert rel_err(got, ref) < 1e-4
