@@ -404,6 +404,25 @@ int dk_offset_conv_forward(const dk_offset_conv_desc* desc, const void* input, c
   return launch_status();
 }
 
+size_t dk_offset_conv_backward_bias_workspace(const dk_offset_conv_desc* desc) {
+  if (!desc || desc->batch < 0 || desc->out_channels <= 0) return 0;
+  return offset_conv_bias_grad_workspace(desc->batch, desc->out_channels);
+}
+
+int dk_offset_conv_backward_bias(const dk_offset_conv_desc* desc, const void* out_grad, void* bias_grad,
+                                 void* workspace, size_t workspace_bytes, void* stream) {
+  if (!desc) return DK_ERR_NULL_POINTER;
+  if (desc->batch < 0 || desc->out_channels <= 0 || desc->h <= 0 || desc->w <= 0) return DK_ERR_BAD_SHAPE;
+  if (desc->dtype != DK_F32) return DK_ERR_UNSUPPORTED;
+  if ((long)desc->batch * desc->out_channels * desc->h * desc->w > kMaxElems) return DK_ERR_TOO_LARGE;
+  if (!out_grad || !bias_grad) return DK_ERR_NULL_POINTER;
+  const size_t need = offset_conv_bias_grad_workspace(desc->batch, desc->out_channels);
+  if (need && (!workspace || workspace_bytes < need)) return DK_ERR_WORKSPACE;
+  offset_conv_bias_grad(desc->batch, desc->out_channels, desc->h * desc->w, static_cast<const float*>(out_grad),
+                        static_cast<float*>(bias_grad), workspace, static_cast<hipStream_t>(stream));
+  return launch_status();
+}
+
 // ---- N-d linear sample --------------------------------------------------------------------
 
 static int check_nd(const dk_nd_desc* d) {

@@ -241,7 +241,33 @@ __global__ __launch_bounds__(kCvBlock, 2) void offset_conv_forward_kernel(
 
 size_t round256(size_t n) { return (n + 255) / 256 * 256; }
 
+// Bias gradient: partial[n][o] = sum over the pixels of gout[n][o]; one workgroup per plane.
+__global__ __launch_bounds__(kCvBlock) void conv_bias_grad_kernel(const float* __restrict__ gout, int plane,
+                                                                  float* __restrict__ partial) {
+  __shared__ float wave_sums[kCvBlock / 64];
+  const float* p = gout + (size_t)blockIdx.x * plane;
+  float s[4] = {0.f, 0.f, 0.f, 0.f};
+  for (int i = threadIdx.x; i < plane; i += 4 * kCvBlock) {
+#pragma unroll
+    for (int u = 0; u < 4; ++u) s[u] += i + u * kCvBlock < plane ? p[i + u * kCvBlock] : 0.f;
+  }
+  const float t = wave_sum((s[0] + s[1]) + (s[2] + s[3]));
+  if ((threadIdx.x & 63) == 0) wave_sums[threadIdx.x >> 6] = t;
+  __syncthreads();
+  if (threadIdx.x == 0) partial[blockIdx.x] = (wave_sums[0] + wave_sums[1]) + (wave_sums[2] + wave_sums[3]);
+}
+
 }  // namespace
+
+// gbias[o] = sum over images and pixels of gout[n][o][.]; workspace: batch * cout floats
+size_t offset_conv_bias_grad_workspace(int batch, int cout) { return (size_t)batch * cout * sizeof(float); }
+
+void offset_conv_bias_grad(int batch, int cout, int plane, const float* gout, float* gbias, void* ws,
+                           hipStream_t stream) {
+  float* partial = static_cast<float*>(ws);
+  if (batch > 0) conv_bias_grad_kernel<<<batch * cout, kCvBlock, 0, stream>>>(gout, plane, partial);
+  launch_reduce_partials<float, float>(partial, batch, cout, gbias, stream);  // the images, added in order
+}
 
 bool offset_conv_supported(int cin, int cout, int h, int w) {
   const bool outputs_ok = (cout >= 1 && cout <= 16) || cout == 18 || cout == 20;  // the instantiated VALU widths

@@ -4,7 +4,8 @@ shape family where it applies, and through ``torch.nn.functional.conv2d`` everyw
 
 The forward runs on the native kernel (stride 1, padding 1, dilation 1, float32, input channels
 a multiple of 16, 18 output channels or at most 16, plane width 7 / 14 / 28 / 56 / 112); the
-gradients come from the framework's convolution-backward routines.
+input and weight gradients come from the framework's convolution-backward routines, the bias
+gradient from a reduction kernel of the library.
 """
 import torch
 import torch.nn.functional as F
@@ -66,7 +67,13 @@ class OffsetConvFunction(Function):
         if ctx.needs_input_grad[1]:
             gw = torch.nn.grad.conv2d_weight(input, weight.shape, grad_output, padding=1)
         if ctx.has_bias and ctx.needs_input_grad[2]:
-            gb = grad_output.sum((0, 2, 3))
+            gb = grad_output.new_empty(weight.size(0))
+            desc = _desc(input, weight)
+            L = _lib.lib()
+            with torch.cuda.device(input.device):
+                ws, nbytes = _lib.workspace(L.dk_offset_conv_backward_bias_workspace(desc), input.device)
+                _lib.check(L.dk_offset_conv_backward_bias(desc, _lib.ptr(grad_output), _lib.ptr(gb), _lib.ptr(ws),
+                                                          nbytes, _lib.stream_ptr(input)), "offset_conv bias gradient")
         return gi, gw, gb
 
 
