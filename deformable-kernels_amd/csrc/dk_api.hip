@@ -404,6 +404,25 @@ int dk_offset_conv_forward(const dk_offset_conv_desc* desc, const void* input, c
   return launch_status();
 }
 
+size_t dk_offset_conv_backward_weight_workspace(const dk_offset_conv_desc* desc) {
+  if (check_offset_conv(desc) != DK_OK) return 0;
+  return offset_conv_wgrad_workspace(desc->batch, desc->in_channels, desc->out_channels, desc->h, desc->w);
+}
+
+int dk_offset_conv_backward_weight(const dk_offset_conv_desc* desc, const void* out_grad, const void* input,
+                                   void* weight_grad, void* workspace, size_t workspace_bytes, void* stream) {
+  const int rc = check_offset_conv(desc);
+  if (rc != DK_OK) return rc;
+  if (!out_grad || !input || !weight_grad) return DK_ERR_NULL_POINTER;
+  const size_t need = offset_conv_wgrad_workspace(desc->batch, desc->in_channels, desc->out_channels, desc->h, desc->w);
+  if (!workspace || workspace_bytes < need) return DK_ERR_WORKSPACE;
+  if (!offset_conv_wgrad(desc->batch, desc->in_channels, desc->out_channels, desc->h, desc->w,
+                         static_cast<const float*>(input), static_cast<const float*>(out_grad),
+                         static_cast<float*>(weight_grad), workspace, static_cast<hipStream_t>(stream)))
+    return DK_ERR_UNSUPPORTED;
+  return launch_status();
+}
+
 size_t dk_offset_conv_backward_bias_workspace(const dk_offset_conv_desc* desc) {
   if (!desc || desc->batch < 0 || desc->out_channels <= 0) return 0;
   return offset_conv_bias_grad_workspace(desc->batch, desc->out_channels);

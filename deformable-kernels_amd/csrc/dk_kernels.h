@@ -83,6 +83,9 @@ size_t offset_conv_workspace(int cin, int cout);
 size_t offset_conv_bias_grad_workspace(int batch, int cout);
 void offset_conv_bias_grad(int batch, int cout, int plane, const float* gout, float* gbias, void* ws,
                            hipStream_t stream);
+size_t offset_conv_wgrad_workspace(int batch, int cin, int cout, int h, int w);
+bool offset_conv_wgrad(int batch, int cin, int cout, int h, int w, const float* x, const float* gout, float* gweight,
+                       void* ws, hipStream_t stream);
 bool offset_conv_forward(int batch, int cin, int cout, int h, int w, const float* x, const float* weight,
                          const float* bias, float* out, void* ws, hipStream_t stream);
 

@@ -239,6 +239,174 @@ __global__ __launch_bounds__(kCvBlock, 2) void offset_conv_forward_kernel(
   }
 }
 
+// ---------------------------------------------------------------------------
+// Weight gradient: gW[o][c][t] = sum over images n and pixels p of gout[n][o][p] * x[n][c][p + shift_t].
+// With q = p + shift_t this is a sum over the positions q of the zero-padded input tile,
+//   gW[o][c][t] = sum_q G[o][q - shift_t] * X[c][q],
+// G being the output-gradient tile, zero outside the tile: a matrix product whose rows are the
+// cout * 9 pairs (o, t), whose columns are the channels and whose inner dimension is the padded
+// position -- the (o, t) rows of a tile of 16 read G at 16 different (plane, shift) offsets, the
+// 16 channels read X unshifted, and neither operand needs a per-tap pass.  18 outputs are 162
+// rows = 11 MFMA tiles, 92 % of them useful, with no special case for the outputs beyond 16.
+// A workgroup of 8 waves owns one chunk of 16 input channels and walks its share of the
+// (image, row tile) items: both tiles staged in LDS (X channel pitch and row count chosen
+// 4 mod 64 words, so 16 channels x 4 positions hit 64 banks), the waves split the positions in
+// steps of 4, each accumulating the 11 tiles in registers over all items; at the end the waves'
+// sums are added in a fixed order and one partial per workgroup goes to the workspace.
+// ---------------------------------------------------------------------------
+constexpr int kWgBlock = 512;
+constexpr int kWgWaves = kWgBlock / 64;
+constexpr int kWgMaxRowTiles = 12;  // (cout * 9 + 15) / 16 for cout <= 20
+
+template <int W>
+struct WgradTile {
+  static constexpr int TH = ConvTile<W>::TH, RS = W + 2, ROWS = TH + 2;
+  static constexpr int PSX = (ROWS * RS + 59) / 64 * 64 + 4;  // positions per channel, 4 mod 64
+  static constexpr int KSTEPS = PSX / 4;
+  static constexpr int MARGIN = RS + 1;                         // the largest |shift|
+  static constexpr int GP = (PSX + 2 * MARGIN + 31) / 64 * 64 + 32;  // floats per output plane of G, 32 mod 64
+  static constexpr int SEGS = ConvTile<W>::SEGS;
+  static_assert(PSX >= ROWS * RS && PSX % 64 == 4 && GP >= PSX + 2 * MARGIN, "tile layout");
+};
+
+template <int W, int NT>
+__global__ __launch_bounds__(kWgBlock, 1) void offset_conv_wgrad_kernel(
+    ConvGeo g, const float* __restrict__ x, const float* __restrict__ gout, float* __restrict__ partial, int parts) {
+  using Tl = WgradTile<W>;
+  constexpr int TH = Tl::TH, RS = Tl::RS, PSX = Tl::PSX, GP = Tl::GP, SEGS = Tl::SEGS;
+  extern __shared__ __align__(16) float lds[];
+  float* xs = lds;                      // [kCvChunk][PSX]
+  float* gs = lds + kCvChunk * PSX;     // [cout][GP], position q at gs[o * GP + MARGIN + q]
+
+  const int nchunks = g.cin / kCvChunk;
+  const int chunk = blockIdx.x % nchunks, part = blockIdx.x / nchunks;
+  const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int m = lane & 15, k = lane >> 4;
+  const int plane = g.h * W, items = g.batch * g.tiles;
+
+  for (int e = threadIdx.x; e < kCvChunk * PSX + g.cout * GP; e += kWgBlock) lds[e] = 0.f;  // padding and margins
+
+  // A operand of row tile j: row v = 16 j + m = (o, t); G[o][q - shift_t] at q = 4 ks + k
+  int offa[NT];
+#pragma unroll
+  for (int j = 0; j < NT; ++j) {
+    const int v = 16 * j + m;
+    const int o = v / 9, t = v % 9;
+    const int shift = (t / 3 - 1) * RS + (t % 3 - 1);
+    offa[j] = v < g.cout * 9 ? o * GP + Tl::MARGIN - shift + k : k;  // rows past cout * 9: any valid address
+  }
+  const bool last_rows_real = 16 * (NT - 1) + m < g.cout * 9;  // the last row tile may be partial
+  const int offb = m * PSX + k;  // B operand: X[c = m][q]
+  const float* xs_w = xs + 4 * wave;  // the wave's first step
+  const float* gs_w = gs + 4 * wave;
+
+  v4f acc[NT];
+#pragma unroll
+  for (int j = 0; j < NT; ++j) acc[j] = v4f{0.f, 0.f, 0.f, 0.f};
+
+  // staging, as in the forward kernel: wave w takes channels w and w + 8 of the chunk (TH + 2 rows
+  // each) and output planes w, w + 8, w + 16 (TH rows each)
+  constexpr int kXStage = (kCvChunk / kWgWaves) * (TH + 2) * SEGS;
+  constexpr int kGPlanes = 3;  // ceil(20 / 8)
+  constexpr int kGStage = kGPlanes * TH * SEGS;
+  unsigned vcol[SEGS];
+#pragma unroll
+  for (int sg = 0; sg < SEGS; ++sg) vcol[sg] = sg * 64 + lane < W ? (unsigned)((sg * 64 + lane) * 4) : kOutOfRange;
+  float xst[kXStage], gst[kGStage];
+#define DK_LOAD_ITEM(ITEM)                                                                                     \
+  {                                                                                                            \
+    const int n_ = (ITEM) / g.tiles, r0_ = (ITEM) % g.tiles * TH;                                              \
+    const rsrc_t rx = plane_rsrc(x + ((size_t)n_ * g.cin + (size_t)chunk * kCvChunk) * plane, kCvChunk * plane); \
+    const rsrc_t rg = plane_rsrc(gout + (size_t)n_ * g.cout * plane, g.cout * plane);                          \
+    _Pragma("unroll") for (int i = 0; i < kXStage; ++i) {                                                      \
+      const int chq = i / ((TH + 2) * SEGS), ry = i / SEGS % (TH + 2), sg = i % SEGS;                          \
+      const int row = r0_ - 1 + ry;                                                                            \
+      const bool ok = row >= 0 && row < g.h;                                                                   \
+      const int soff = ok ? ((wave + kWgWaves * chq) * g.h + row) * W * 4 : 0;                                 \
+      xst[i] = __builtin_bit_cast(                                                                             \
+          float, __builtin_amdgcn_raw_buffer_load_b32(rx, (int)(ok ? vcol[sg] : kOutOfRange), soff, 0));       \
+    }                                                                                                          \
+    _Pragma("unroll") for (int i = 0; i < kGStage; ++i) {                                                      \
+      const int pq = i / (TH * SEGS), ry = i / SEGS % TH, sg = i % SEGS;                                       \
+      const int o = wave + kWgWaves * pq, row = r0_ + ry;                                                      \
+      const bool ok = o < g.cout && row < g.h;                                                                 \
+      const int soff = ok ? (o * g.h + row) * W * 4 : 0;                                                       \
+      gst[i] = __builtin_bit_cast(                                                                             \
+          float, __builtin_amdgcn_raw_buffer_load_b32(rg, (int)(ok ? vcol[sg] : kOutOfRange), soff, 0));       \
+    }                                                                                                          \
+  }
+
+  int item = part;
+  if (item < items) DK_LOAD_ITEM(item)
+  for (; item < items; item += parts) {
+    __syncthreads();  // the previous item's products are done (and, the first time, the zero fill)
+#pragma unroll
+    for (int i = 0; i < kXStage; ++i) {
+      const int chq = i / ((TH + 2) * SEGS), ry = i / SEGS % (TH + 2), sg = i % SEGS;
+      if (sg * 64 + lane < W) xs[(wave + kWgWaves * chq) * PSX + ry * RS + 1 + sg * 64 + lane] = xst[i];
+    }
+#pragma unroll
+    for (int i = 0; i < kGStage; ++i) {
+      const int pq = i / (TH * SEGS), ry = i / SEGS % TH, sg = i % SEGS;
+      const int o = wave + kWgWaves * pq;
+      // tile row ry is row ry + 1 of the padded geometry
+      if (o < g.cout && sg * 64 + lane < W) gs[o * GP + Tl::MARGIN + (ry + 1) * RS + 1 + sg * 64 + lane] = gst[i];
+    }
+    __syncthreads();
+    if (item + parts < items) DK_LOAD_ITEM(item + parts)
+
+    // wave w takes the steps w, w + 8, ...: the wave part of the LDS address sits in the base
+    // registers, the rest is an immediate of the unrolled loop
+    constexpr int kTrips = (Tl::KSTEPS + kWgWaves - 1) / kWgWaves;
+#pragma unroll 3
+    for (int i = 0; i < kTrips; ++i) {
+      if (wave + kWgWaves * i < Tl::KSTEPS) {  // wave-uniform; false only in the last trip
+        const float b = xs_w[offb + 4 * kWgWaves * i];
+#pragma unroll
+        for (int j = 0; j < NT; ++j) {
+          float a = gs_w[offa[j] + 4 * kWgWaves * i];
+          if (j == NT - 1 && !last_rows_real) a = 0.f;
+          acc[j] = __builtin_amdgcn_mfma_f32_16x16x4f32(a, b, acc[j], 0, 0, 0);
+        }
+      }
+    }
+  }
+#undef DK_LOAD_ITEM
+
+  // add the waves' sums in wave order into red[NT][256] (entry 4 * lane + r of a tile), then out
+  __syncthreads();
+  float* red = lds;
+  for (int w = 0; w < kWgWaves; ++w) {
+    if (wave == w) {
+#pragma unroll
+      for (int j = 0; j < NT; ++j) {
+        v4f* dst = reinterpret_cast<v4f*>(red + j * 256 + lane * 4);
+        *dst = w == 0 ? acc[j] : *dst + acc[j];
+      }
+    }
+    __syncthreads();
+  }
+  // D[row 4 * (l / 16) + r][channel l % 16] sits at red[j * 256 + 4 * l + r]
+  float* dst = partial + (size_t)(part * nchunks + chunk) * (NT * 256);
+  for (int e = threadIdx.x; e < NT * 256; e += kWgBlock) dst[e] = red[e];
+}
+
+// gW[o][c][t] = sum over parts of partial[part][chunk(c)][row tile][...], parts added in order
+__global__ __launch_bounds__(256) void offset_conv_wgrad_reduce_kernel(const float* __restrict__ partial, int parts,
+                                                                       int nchunks, int nt, int cout, int cin,
+                                                                       float* __restrict__ gw) {
+  const int idx = blockIdx.x * 256 + threadIdx.x;  // = (o * cin + c) * 9 + t
+  if (idx >= cout * cin * 9) return;
+  const int t = idx % 9, c = idx / 9 % cin, o = idx / 9 / cin;
+  const int v = o * 9 + t, j = v / 16, mrow = v % 16;
+  // row mrow = 4 * (l / 16) + r, column c % 16 = l % 16
+  const int l = (mrow / 4) * 16 + c % 16, r = mrow % 4;
+  const float* p = partial + (size_t)(c / kCvChunk) * (nt * 256) + j * 256 + 4 * l + r;
+  float s = 0.f;
+  for (int q = 0; q < parts; ++q) s += p[(size_t)q * nchunks * (nt * 256)];
+  gw[idx] = s;
+}
+
 size_t round256(size_t n) { return (n + 255) / 256 * 256; }
 
 // Bias gradient: partial[n][o] = sum over the pixels of gout[n][o]; one workgroup per plane.
@@ -323,6 +491,65 @@ bool offset_conv_forward(int batch, int cin, int cout, int h, int w, const float
   }
 #undef DK_WIDTH
 #undef DK_LAUNCH
+  return true;
+}
+
+// parts of the (image, row tile) items a chunk's workgroups split: about one workgroup per CU
+int wgrad_parts(int batch, int cin, int h, int w) {
+  const int th = w <= 56 ? 8 : 4;
+  const int items = batch * ceil_div(h, th), nchunks = cin / kCvChunk;
+  return std::max(1, std::min(items, 256 / nchunks));
+}
+
+size_t offset_conv_wgrad_workspace(int batch, int cin, int cout, int h, int w) {
+  const int nt = ceil_div(cout * 9, 16);
+  return (size_t)wgrad_parts(batch, cin, h, w) * (cin / kCvChunk) * nt * 256 * sizeof(float);
+}
+
+bool offset_conv_wgrad(int batch, int cin, int cout, int h, int w, const float* x, const float* gout, float* gweight,
+                       void* ws, hipStream_t stream) {
+  if (!offset_conv_supported(cin, cout, h, w)) return false;
+  const int nt = ceil_div(cout * 9, 16), nchunks = cin / kCvChunk;
+  const int parts = wgrad_parts(batch, cin, h, w);
+  float* partial = static_cast<float*>(ws);
+  ConvGeo g;
+  g.batch = batch, g.cin = cin, g.cout = cout, g.h = h;
+  bool ok = true;
+#define DK_LAUNCH(WW, NT)                                                                                      \
+  {                                                                                                            \
+    auto kernel = offset_conv_wgrad_kernel<WW, NT>;                                                            \
+    g.tiles = ceil_div(h, WgradTile<WW>::TH);                                                                  \
+    const size_t lds = (size_t)(kCvChunk * WgradTile<WW>::PSX + cout * WgradTile<WW>::GP) * sizeof(float);     \
+    const size_t lds_red = (size_t)NT * 256 * sizeof(float);                                                   \
+    const size_t bytes = std::max(lds, lds_red);                                                               \
+    if (bytes > 160 * 1024 ||                                                                                  \
+        hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, \
+                            (int)bytes) != hipSuccess)                                                         \
+      ok = false;                                                                                              \
+    else if (batch > 0)                                                                                        \
+      kernel<<<parts * nchunks, kWgBlock, bytes, stream>>>(g, x, gout, partial, parts);                        \
+  }
+#define DK_WIDTH(NT)                       \
+  switch (w) {                             \
+    case 7: DK_LAUNCH(7, NT) break;        \
+    case 14: DK_LAUNCH(14, NT) break;      \
+    case 28: DK_LAUNCH(28, NT) break;      \
+    case 56: DK_LAUNCH(56, NT) break;      \
+    case 112: DK_LAUNCH(112, NT) break;    \
+    default: ok = false;                   \
+  }
+  switch (nt) {
+    case 9: DK_WIDTH(9) break;    // 16 outputs
+    case 11: DK_WIDTH(11) break;  // 18 outputs
+    case 12: DK_WIDTH(12) break;  // 20 outputs
+    default: ok = false;
+  }
+#undef DK_WIDTH
+#undef DK_LAUNCH
+  if (!ok) return false;
+  const int total = cout * cin * 9;
+  offset_conv_wgrad_reduce_kernel<<<ceil_div(total, 256), 256, 0, stream>>>(partial, batch > 0 ? parts : 0, nchunks, nt,
+                                                                           cout, cin, gweight);
   return true;
 }
 

@@ -76,6 +76,8 @@ SIGNATURES = {
     "dk_offset_conv_worthwhile": (ctypes.c_int, [_OC]),
     "dk_offset_conv_forward_workspace": (_SZ, [_OC]),
     "dk_offset_conv_forward": (ctypes.c_int, [_OC, _P, _P, _P, _P, _P, _SZ, _P]),
+    "dk_offset_conv_backward_weight_workspace": (_SZ, [_OC]),
+    "dk_offset_conv_backward_weight": (ctypes.c_int, [_OC, _P, _P, _P, _P, _SZ, _P]),
     "dk_offset_conv_backward_bias_workspace": (_SZ, [_OC]),
     "dk_offset_conv_backward_bias": (ctypes.c_int, [_OC, _P, _P, _P, _SZ, _P]),
 }

@@ -4,8 +4,8 @@ shape family where it applies, and through ``torch.nn.functional.conv2d`` everyw
 
 The forward runs on the native kernel (stride 1, padding 1, dilation 1, float32, input channels
 a multiple of 16, 18 output channels or at most 16, plane width 7 / 14 / 28 / 56 / 112); the
-input and weight gradients come from the framework's convolution-backward routines, the bias
-gradient from a reduction kernel of the library.
+weight and bias gradients come from kernels of the library as well, the input gradient from
+the framework's convolution-backward routine.
 """
 import torch
 import torch.nn.functional as F
@@ -65,7 +65,14 @@ class OffsetConvFunction(Function):
         if ctx.needs_input_grad[0]:
             gi = torch.nn.grad.conv2d_input(input.shape, weight, grad_output, padding=1)
         if ctx.needs_input_grad[1]:
-            gw = torch.nn.grad.conv2d_weight(input, weight.shape, grad_output, padding=1)
+            gw = torch.empty_like(weight)
+            desc = _desc(input, weight)
+            L = _lib.lib()
+            with torch.cuda.device(input.device):
+                ws, nbytes = _lib.workspace(L.dk_offset_conv_backward_weight_workspace(desc), input.device)
+                _lib.check(L.dk_offset_conv_backward_weight(desc, _lib.ptr(grad_output), _lib.ptr(input), _lib.ptr(gw),
+                                                            _lib.ptr(ws), nbytes, _lib.stream_ptr(input)),
+                           "offset_conv weight gradient")
         if ctx.has_bias and ctx.needs_input_grad[2]:
             gb = grad_output.new_empty(weight.size(0))
             desc = _desc(input, weight)

@@ -238,9 +238,17 @@ int dk_offset_conv_forward(const dk_offset_conv_desc *desc, const void *input, c
                            const void *bias, void *output, void *workspace, size_t workspace_bytes,
                            void *stream);
 
+/* Gradient of that convolution's weight, weight_grad [out_channels, in_channels, 3, 3] (fully
+ * written), for the shapes dk_offset_conv_supported() accepts; per-workgroup partial sums in the
+ * workspace are added in a fixed order. */
+size_t dk_offset_conv_backward_weight_workspace(const dk_offset_conv_desc *desc);
+int dk_offset_conv_backward_weight(const dk_offset_conv_desc *desc, const void *out_grad, const void *input,
+                                   void *weight_grad, void *workspace, size_t workspace_bytes,
+                                   void *stream);
+
 /* Gradient of that convolution's bias: bias_grad[o] = sum over images and pixels of
- * out_grad[n][o][.], float32, any shape; the images are added in a fixed order.  (The other two
- * gradients of the convolution are left to the caller's library.) */
+ * out_grad[n][o][.], float32, any shape; the images are added in a fixed order.  (The input
+ * gradient of the convolution is left to the caller's library.) */
 size_t dk_offset_conv_backward_bias_workspace(const dk_offset_conv_desc *desc);
 int dk_offset_conv_backward_bias(const dk_offset_conv_desc *desc, const void *out_grad, void *bias_grad,
                                  void *workspace, size_t workspace_bytes, void *stream);

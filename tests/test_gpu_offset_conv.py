@@ -36,6 +36,27 @@ def test_forward_matches_float64_convolution(shape):
     assert rel_err(got.cpu(), want.cpu()) < 1e-5
 
 
+@pytest.mark.parametrize("shape", [
+    (2, 16, 5, 7, 18), (3, 32, 14, 14, 18), (2, 48, 28, 28, 18), (2, 144, 56, 56, 18), (1, 32, 9, 112, 18),
+    (2, 32, 56, 56, 16), (1, 16, 13, 28, 20), (40, 32, 56, 56, 18),   # the last: several items per workgroup
+])
+def test_weight_and_bias_gradients_match_float64(shape):
+    from deformable_kernels.ops.deform_kernel.functions.offset_conv import OffsetConvFunction
+    N, C, H, W, O = shape
+    g = torch.Generator().manual_seed(33)
+    dev = torch.device("cuda:0")
+    x = torch.randn(N, C, H, W, generator=g).to(dev).requires_grad_()
+    w = (torch.randn(O, C, 3, 3, generator=g) * 0.05).to(dev).requires_grad_()
+    b = torch.randn(O, generator=g).to(dev).requires_grad_()
+    gout = torch.randn(N, O, H, W, generator=g).to(dev)
+    OffsetConvFunction.apply(x, w, b).backward(gout)
+    xd, wd, bd = [t.detach().double().requires_grad_() for t in (x, w, b)]
+    F.conv2d(xd, wd, bd, padding=1).backward(gout.double())
+    assert rel_err(w.grad.cpu(), wd.grad.cpu()) < 1e-5
+    assert rel_err(b.grad.cpu(), bd.grad.cpu()) < 1e-5
+    assert rel_err(x.grad.cpu(), xd.grad.cpu()) < 1e-5
+
+
 def test_unsupported_calls_go_to_the_library_convolution():
     from deformable_kernels.ops.deform_kernel.functions import offset_conv, offset_conv_supported
     dev = torch.device("cuda:0")
