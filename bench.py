@@ -94,7 +94,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--workload", default="cfg2", choices=sorted(WORKLOADS) + sorted(OTHER_WORKLOADS) + ["mbv2_dk"])
+    ap.add_argument("--workload", default="cfg2", choices=sorted(WORKLOADS) + sorted(OTHER_WORKLOADS) + ["mbv2_dk", "layer_cfg2"])
     ap.add_argument("--batch", type=int, default=64, help="batch size of the mbv2_dk workload")
     ap.add_argument("--dtype", default="fp32", choices=sorted(DTYPES))
     ap.add_argument("--no-cpu-baseline", action="store_true")
@@ -113,6 +113,8 @@ def main():
         sys.exit("bench.py needs a GPU")
     if a.workload == "mbv2_dk":
         return mobilenet_workload(a)
+    if a.workload == "layer_cfg2":
+        return layer_workload(a)
     if a.workload in OTHER_WORKLOADS:
         return other_workload(a)
     dev = torch.device("cuda:0")
@@ -344,6 +346,54 @@ def other_workload(a):
 MBV2_DW_LAYERS = [(32, 112, 1), (96, 112, 2), (144, 56, 1), (144, 56, 2), (192, 28, 1), (192, 28, 1), (192, 28, 2),
                   (384, 14, 1), (384, 14, 1), (384, 14, 1), (384, 14, 1), (576, 14, 1), (576, 14, 1), (576, 14, 2),
                   (960, 7, 1), (960, 7, 1), (960, 7, 1)]
+
+
+def layer_workload(a):
+    """A whole LocalDeformKernel2d layer of config 2's shape through the modules and autograd:
+    the 3x3 offset branch (rotation_conv), the 'scope' clamp and the operator, forward + backward.
+    Times the reference's sequence (library convolution, clamp as tensor ops) against the
+    library's own offset-branch kernels and the clamp inside the operator."""
+    import torch
+    from deformable_kernels.modules import LocalDeformKernel2d
+    dev = torch.device("cuda:0")
+    torch.manual_seed(0)
+    N, C, H = a.batch, 144, 56
+    m = LocalDeformKernel2d((4, 4), C, C, 3, 1, 1, 1, C, 1, False, "scope").to(dev)
+    torch.nn.init.normal_(m.rotation_conv.weight, std=0.01)
+    x = torch.randn(N, C, H, H, device=dev, requires_grad=True)
+    gout = torch.randn(N, C, H, H, device=dev)
+
+    def timed(fn):
+        for _ in range(a.warmup):
+            fn()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(a.steps):
+            fn()
+        e1.record()
+        e1.synchronize()
+        return round(e0.elapsed_time(e1) * 1e3 / a.steps, 1)
+
+    def step():
+        m(x).backward(gout)
+
+    def forward():
+        with torch.no_grad():
+            m(x)
+
+    def branch():
+        r = m.rotation_conv(x)
+        r.backward(torch.ones_like(r))
+
+    res = {}
+    for name, native, fused in (("reference_sequence", False, False), ("clamp_in_operator", False, True),
+                                ("clamp_in_operator+native_offset_branch", True, True)):
+        m.native_offset_conv, m.fused_clip = native, fused
+        res[name] = {"step_us": timed(step), "forward_us": timed(forward)}
+    res["library_offset_branch_alone"] = {"step_us": timed(branch)}
+    print(json.dumps({"metric": "LocalDeformKernel2d layer fwd+bwd through the modules (secondary workload)",
+                      "config": {"workload": "layer_cfg2: N=%d C=144 56x56 k=3 scope=4x4 rotation_clip='scope' fp32" % N},
+                      "variants": res, "n_gpus": 1, "dtype": "fp32", "data": "synthetic"}))
 
 
 def mobilenet_workload(a):
