@@ -256,7 +256,6 @@ __global__ __launch_bounds__(kCvBlock, 2) void offset_conv_forward_kernel(
 // ---------------------------------------------------------------------------
 constexpr int kWgBlock = 512;
 constexpr int kWgWaves = kWgBlock / 64;
-constexpr int kWgMaxRowTiles = 12;  // (cout * 9 + 15) / 16 for cout <= 20
 
 template <int W>
 struct WgradTile {
