@@ -170,8 +170,9 @@ class LocalDeformKernel2d(nn.Module):
         # True: the operator clamps the offsets itself (same values and gradients as clamping
         # the tensor first, without the extra passes over it); False: the reference's sequence
         self.fused_clip = True
-        # True: rotation_conv's forward runs on the library's own kernel where that is faster
-        # (wide planes, float32, stride 1); its parameters and gradients are unchanged
+        # True: rotation_conv runs through offset_conv() -- the library's own forward and weight
+        # gradient kernels where they are faster (wide planes, float32, stride 1), its bias
+        # gradient kernel everywhere; parameters and results are unchanged
         self.native_offset_conv = True
 
         self.inner_conv = SampleDepthwise(
@@ -242,13 +243,19 @@ class DeformKernelConv2d(nn.Module):
             kernel_size, stride, padding, dilation, bias=True)
         self.offset_conv.zero_init = True
         self.offset_clip = offset_clip
+        # as in LocalDeformKernel2d: the library's kernels for the offset branch where they apply
+        self.native_offset_conv = True
 
         self.inner_conv = DeformableSampleDepthwise(
             weight_shape, in_planes, out_planes, kernel_size=kernel_size, stride=stride,
             padding=padding, dilation=dilation, groups=groups, bias=bias)
 
     def forward(self, x):
-        offset = self.offset_conv(x)
+        conv = self.offset_conv
+        if self.native_offset_conv:
+            offset = offset_conv(x, conv.weight, conv.bias, conv.stride, conv.padding, conv.dilation)
+        else:
+            offset = conv(x)
         if self.offset_clip is not None:
             offset = offset.clamp(**self.offset_clip)
         if self.dilation != 1:

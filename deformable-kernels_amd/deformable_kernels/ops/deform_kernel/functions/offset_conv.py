@@ -1,11 +1,19 @@
 """The offset branch of ``LocalDeformKernel2d``: its 3x3 ``rotation_conv`` (reference
-``modules/deform_kernel.py:165-168``, applied at ``:214``) through the library's kernel for that
-shape family where it applies, and through ``torch.nn.functional.conv2d`` everywhere else.
+``modules/deform_kernel.py:165-168``, applied at ``:214``).
 
-The forward runs on the native kernel (stride 1, padding 1, dilation 1, float32, input channels
-a multiple of 16, 18 output channels or at most 16, plane width 7 / 14 / 28 / 56 / 112); the
-weight and bias gradients come from kernels of the library as well, the input gradient from
-the framework's convolution-backward routine.
+``offset_conv(input, weight, bias, stride, padding, dilation)`` returns what
+``torch.nn.functional.conv2d`` returns.  For float32 GPU tensors it runs
+
+  * the forward and the weight gradient on the library's matrix-core kernels where they apply
+    and are the faster choice (stride 1, padding 1, dilation 1, input channels a multiple of 16,
+    18 output channels or at most 16, plane width 56 or 112 with enough images to fill the GPU;
+    ``force=True``: wherever they apply, also widths 7 / 14 / 28),
+  * the bias gradient on the library's reduction kernel for every shape (the framework's
+    reduction over (N, H, W) takes 60-230 us on the large planes),
+  * everything else -- the input gradient, and forward / weight gradient of the other shapes --
+    on the framework's convolution routines.
+
+Other dtypes, CPU tensors and autocast regions go to ``F.conv2d`` unchanged.
 """
 import torch
 import torch.nn.functional as F
@@ -16,25 +24,31 @@ from .. import _lib
 __all__ = ['offset_conv', 'offset_conv_supported']
 
 
-def _desc(input, weight):
-    return _lib.OffsetConvDesc(input.size(0), input.size(1), weight.size(0), input.size(2), input.size(3),
-                               _lib.DK_F32)
+def _pair(v):
+    return tuple(int(e) for e in v) if isinstance(v, (tuple, list)) else (int(v), int(v))
+
+
+def _desc(input, weight, out=None):
+    h, w = (input.size(2), input.size(3)) if out is None else (out.size(2), out.size(3))
+    return _lib.OffsetConvDesc(input.size(0), input.size(1), weight.size(0), h, w, _lib.DK_F32)
+
+
+def _float32_gpu(input, weight, bias):
+    if not (input.is_cuda and weight.is_cuda and input.dtype == torch.float32 and weight.dtype == torch.float32):
+        return False
+    if bias is not None and not (bias.is_cuda and bias.dtype == torch.float32):
+        return False
+    return input.dim() == 4 and weight.dim() == 4 and not torch.is_autocast_enabled()
 
 
 def offset_conv_supported(input, weight, bias, stride, padding, dilation, worthwhile=False):
-    """Whether the native kernel covers this call; with ``worthwhile`` also whether it is
-    expected to be faster than the library convolution."""
-    def pair(v):
-        return tuple(v) if isinstance(v, (tuple, list)) else (v, v)
-    if not (input.is_cuda and input.dtype == torch.float32 and weight.dtype == torch.float32):
+    """Whether the native forward / weight-gradient kernels cover this call; with ``worthwhile``
+    also whether they are expected to be faster than the library convolution."""
+    if not _float32_gpu(input, weight, bias):
         return False
-    if input.dim() != 4 or weight.dim() != 4 or tuple(weight.shape[2:]) != (3, 3) or weight.size(1) != input.size(1):
+    if tuple(weight.shape[2:]) != (3, 3) or weight.size(1) != input.size(1):
         return False
-    if pair(stride) != (1, 1) or pair(padding) != (1, 1) or pair(dilation) != (1, 1):
-        return False
-    if bias is not None and bias.dtype != torch.float32:
-        return False
-    if torch.is_autocast_enabled():
+    if _pair(stride) != (1, 1) or _pair(padding) != (1, 1) or _pair(dilation) != (1, 1):
         return False
     L = _lib.lib()
     return bool((L.dk_offset_conv_worthwhile if worthwhile else L.dk_offset_conv_supported)(_desc(input, weight)))
@@ -42,10 +56,14 @@ def offset_conv_supported(input, weight, bias, stride, padding, dilation, worthw
 
 class OffsetConvFunction(Function):
     @staticmethod
-    def forward(ctx, input, weight, bias):
+    def forward(ctx, input, weight, bias, stride, padding, dilation, native):
         input, weight = input.contiguous(), weight.contiguous()
         ctx.save_for_backward(input, weight)
+        ctx.conv = (stride, padding, dilation)
+        ctx.native = native
         ctx.has_bias = bias is not None
+        if not native:
+            return F.conv2d(input, weight, bias, stride, padding, dilation)
         b = bias.contiguous() if bias is not None else input.new_zeros(weight.size(0))
         out = input.new_empty(input.size(0), weight.size(0), input.size(2), input.size(3))
         desc = _desc(input, weight)
@@ -60,33 +78,40 @@ class OffsetConvFunction(Function):
     @staticmethod
     def backward(ctx, grad_output):
         input, weight = ctx.saved_tensors
+        stride, padding, dilation = ctx.conv
         grad_output = grad_output.contiguous()
+        need_input, need_weight = ctx.needs_input_grad[0], ctx.needs_input_grad[1]
         gi = gw = gb = None
-        if ctx.needs_input_grad[0]:
-            gi = torch.nn.grad.conv2d_input(input.shape, weight, grad_output, padding=1)
-        if ctx.needs_input_grad[1]:
-            gw = torch.empty_like(weight)
-            desc = _desc(input, weight)
-            L = _lib.lib()
-            with torch.cuda.device(input.device):
+        L = _lib.lib()
+        library_weight = need_weight and not ctx.native
+        if need_input or library_weight:
+            # the framework's routine, without its bias gradient
+            gi, gw_lib, _ = torch.ops.aten.convolution_backward(
+                grad_output, input, weight, None, list(stride), list(padding), list(dilation), False, [0, 0], 1,
+                [need_input, library_weight, False])
+            if library_weight:
+                gw = gw_lib
+        with torch.cuda.device(input.device):
+            if need_weight and ctx.native:
+                gw = torch.empty_like(weight)
+                desc = _desc(input, weight)
                 ws, nbytes = _lib.workspace(L.dk_offset_conv_backward_weight_workspace(desc), input.device)
                 _lib.check(L.dk_offset_conv_backward_weight(desc, _lib.ptr(grad_output), _lib.ptr(input), _lib.ptr(gw),
                                                             _lib.ptr(ws), nbytes, _lib.stream_ptr(input)),
                            "offset_conv weight gradient")
-        if ctx.has_bias and ctx.needs_input_grad[2]:
-            gb = grad_output.new_empty(weight.size(0))
-            desc = _desc(input, weight)
-            L = _lib.lib()
-            with torch.cuda.device(input.device):
+            if ctx.has_bias and ctx.needs_input_grad[2]:
+                gb = grad_output.new_empty(weight.size(0))
+                desc = _desc(input, weight, grad_output)
                 ws, nbytes = _lib.workspace(L.dk_offset_conv_backward_bias_workspace(desc), input.device)
                 _lib.check(L.dk_offset_conv_backward_bias(desc, _lib.ptr(grad_output), _lib.ptr(gb), _lib.ptr(ws),
                                                           nbytes, _lib.stream_ptr(input)), "offset_conv bias gradient")
-        return gi, gw, gb
+        return gi, gw, gb, None, None, None, None
 
 
 def offset_conv(input, weight, bias=None, stride=1, padding=1, dilation=1, force=False):
-    """``F.conv2d(input, weight, bias, stride, padding, dilation)`` for the offset branch: the
-    native kernel where it is the faster choice (``force``: wherever it applies)."""
-    if offset_conv_supported(input, weight, bias, stride, padding, dilation, worthwhile=not force):
-        return OffsetConvFunction.apply(input, weight, bias)
-    return F.conv2d(input, weight, bias, stride, padding, dilation)
+    """``F.conv2d(input, weight, bias, stride, padding, dilation)`` for the offset branch (see the
+    module docstring for what runs where)."""
+    if not _float32_gpu(input, weight, bias):
+        return F.conv2d(input, weight, bias, stride, padding, dilation)
+    native = offset_conv_supported(input, weight, bias, stride, padding, dilation, worthwhile=not force)
+    return OffsetConvFunction.apply(input, weight, bias, _pair(stride), _pair(padding), _pair(dilation), native)

@@ -41,7 +41,7 @@ def test_forward_matches_float64_convolution(shape):
     (2, 32, 56, 56, 16), (1, 16, 13, 28, 20), (40, 32, 56, 56, 18),   # the last: several items per workgroup
 ])
 def test_weight_and_bias_gradients_match_float64(shape):
-    from deformable_kernels.ops.deform_kernel.functions.offset_conv import OffsetConvFunction
+    from deformable_kernels.ops.deform_kernel.functions import offset_conv
     N, C, H, W, O = shape
     g = torch.Generator().manual_seed(33)
     dev = torch.device("cuda:0")
@@ -49,7 +49,7 @@ def test_weight_and_bias_gradients_match_float64(shape):
     w = (torch.randn(O, C, 3, 3, generator=g) * 0.05).to(dev).requires_grad_()
     b = torch.randn(O, generator=g).to(dev).requires_grad_()
     gout = torch.randn(N, O, H, W, generator=g).to(dev)
-    OffsetConvFunction.apply(x, w, b).backward(gout)
+    offset_conv(x, w, b, force=True).backward(gout)
     xd, wd, bd = [t.detach().double().requires_grad_() for t in (x, w, b)]
     F.conv2d(xd, wd, bd, padding=1).backward(gout.double())
     assert rel_err(w.grad.cpu(), wd.grad.cpu()) < 1e-5
@@ -69,6 +69,30 @@ def test_unsupported_calls_go_to_the_library_convolution():
     assert not offset_conv_supported(x2, w2, None, 2, 1, 1)          # stride 2
     assert not offset_conv_supported(x2.half(), w2.half(), None, 1, 1, 1)
     assert torch.equal(offset_conv(x2, w2, None, stride=2), F.conv2d(x2, w2, None, 2, 1, 1))
+    assert torch.equal(offset_conv(x2.half(), w2.half(), None), F.conv2d(x2.half(), w2.half(), None, 1, 1, 1))
+
+
+@pytest.mark.parametrize("conv", [(2, 1, 1), (1, 0, 1), (1, 2, 2), (2, 1, 1, 24)])
+def test_other_convolutions_keep_the_library_kernels_but_not_its_bias_gradient(conv):
+    # stride 2 / no padding / dilation 2 / 24 channels: the forward is F.conv2d's, the gradients match autograd's
+    from deformable_kernels.ops.deform_kernel.functions import offset_conv
+    stride, padding, dilation = conv[:3]
+    C = conv[3] if len(conv) > 3 else 32
+    g = torch.Generator().manual_seed(34)
+    dev = torch.device("cuda:0")
+    x = torch.randn(3, C, 20, 22, generator=g).to(dev).requires_grad_()
+    w = (torch.randn(18, C, 3, 3, generator=g) * 0.05).to(dev).requires_grad_()
+    b = torch.randn(18, generator=g).to(dev).requires_grad_()
+    out = offset_conv(x, w, b, stride, padding, dilation)
+    x2, w2, b2 = [t.detach().clone().requires_grad_() for t in (x, w, b)]
+    ref = F.conv2d(x2, w2, b2, stride, padding, dilation)
+    assert torch.equal(out, ref)
+    gout = torch.randn(ref.shape, generator=g).to(dev)
+    out.backward(gout)
+    ref.backward(gout)
+    assert rel_err(x.grad.cpu(), x2.grad.cpu()) < 1e-6
+    assert rel_err(w.grad.cpu(), w2.grad.cpu()) < 1e-6
+    assert rel_err(b.grad.cpu(), gout.double().sum((0, 2, 3)).float().cpu()) < 1e-5
 
 
 def test_gradients_and_module_switch():
