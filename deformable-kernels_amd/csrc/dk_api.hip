@@ -385,7 +385,7 @@ int dk_offset_conv_worthwhile(const dk_offset_conv_desc* desc) {
 
 size_t dk_offset_conv_forward_workspace(const dk_offset_conv_desc* desc) {
   if (check_offset_conv(desc) != DK_OK) return 0;
-  return offset_conv_workspace(desc->in_channels, desc->out_channels);
+  return offset_conv_workspace(desc->batch, desc->in_channels, desc->out_channels, desc->h, desc->w);
 }
 
 int dk_offset_conv_forward(const dk_offset_conv_desc* desc, const void* input, const void* weight,
@@ -394,7 +394,7 @@ int dk_offset_conv_forward(const dk_offset_conv_desc* desc, const void* input, c
   const int rc = check_offset_conv(desc);
   if (rc != DK_OK) return rc;
   if (!input || !weight || !bias || !output) return DK_ERR_NULL_POINTER;
-  const size_t need = offset_conv_workspace(desc->in_channels, desc->out_channels);
+  const size_t need = offset_conv_workspace(desc->batch, desc->in_channels, desc->out_channels, desc->h, desc->w);
   if (!workspace || workspace_bytes < need) return DK_ERR_WORKSPACE;
   if (!offset_conv_forward(desc->batch, desc->in_channels, desc->out_channels, desc->h, desc->w,
                            static_cast<const float*>(input), static_cast<const float*>(weight),

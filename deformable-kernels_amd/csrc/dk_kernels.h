@@ -79,7 +79,7 @@ void generic_grad_filter(const Geo& g, bool deform, const T* gout, const T* x, c
 // dk_offset_conv.hip: the 3x3 offset-branch convolution (stride 1, padding 1, fp32)
 bool offset_conv_supported(int cin, int cout, int h, int w);
 bool offset_conv_worthwhile(int batch, int cin, int cout, int h, int w);
-size_t offset_conv_workspace(int cin, int cout);
+size_t offset_conv_workspace(int batch, int cin, int cout, int h, int w);
 size_t offset_conv_bias_grad_workspace(int batch, int cout);
 void offset_conv_bias_grad(int batch, int cout, int plane, const float* gout, float* gbias, void* ws,
                            hipStream_t stream);

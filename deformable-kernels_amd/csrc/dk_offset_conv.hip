@@ -65,16 +65,19 @@ __global__ void conv_pack_weights_kernel(const float* __restrict__ w, int cout, 
 template <int W, int REST>
 __global__ __launch_bounds__(kCvBlock, 2) void offset_conv_forward_kernel(
     ConvGeo g, const float* __restrict__ x, const float* __restrict__ w16, const float* __restrict__ wrest,
-    const float* __restrict__ bias, float* __restrict__ out) {
+    const float* __restrict__ bias, float* __restrict__ out, float* __restrict__ partial, int ksplit) {
   extern __shared__ __align__(16) float xs[];  // [kCvChunk][PS], then the chunk's VALU-path weights [kCvChunk][9][REST]
   constexpr int TH = ConvTile<W>::TH, SEGS = ConvTile<W>::SEGS, RS = ConvTile<W>::RS, PS = ConvTile<W>::PS;
   constexpr int kStage = (kCvChunk / 4) * (TH + 2) * SEGS;  // row segments of 64 columns a wave stages per chunk
   constexpr int kPixPerThread = (kCvTilePix + kCvBlock - 1) / kCvBlock;  // of the VALU path
 
-  const int total = g.batch * g.tiles;
+  // logical block = (input-channel split, row tile, image), split fastest.  With ksplit > 1 (small
+  // planes, where (image, tile) alone gives too few workgroups) a workgroup sums a share of the
+  // channel chunks and writes partial[split][...]; the splits are added afterwards, in order.
+  const int total = g.batch * g.tiles * ksplit;
   const int lb = logical_block(total);
   if (lb >= total) return;
-  const int n = lb / g.tiles, r0 = (lb % g.tiles) * TH;
+  const int split = lb % ksplit, n = lb / ksplit / g.tiles, r0 = (lb / ksplit % g.tiles) * TH;
   // the wave index enters scalar offsets and loop bounds: tell the compiler it is uniform
   const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   constexpr int tile_pix = TH * W, groups = (tile_pix + 15) / 16;
@@ -142,9 +145,10 @@ __global__ __launch_bounds__(kCvBlock, 2) void offset_conv_forward_kernel(
   }
 
   const rsrc_t rw = plane_rsrc(w16, 9 * g.cin * 16);
-  const int nchunks = g.cin / kCvChunk;
-  DK_LOAD_CHUNK(0)
-  for (int ck = 0; ck < nchunks; ++ck) {
+  const int per_split = ceil_div(g.cin / kCvChunk, ksplit);
+  const int ck_begin = split * per_split, nchunks = min(g.cin / kCvChunk, ck_begin + per_split);
+  if (ck_begin < nchunks) DK_LOAD_CHUNK(ck_begin)
+  for (int ck = ck_begin; ck < nchunks; ++ck) {
     __syncthreads();  // every wave is done with the previous chunk
 #pragma unroll
     for (int i = 0; i < kStage; ++i) {
@@ -212,7 +216,8 @@ __global__ __launch_bounds__(kCvBlock, 2) void offset_conv_forward_kernel(
 
 #undef DK_LOAD_CHUNK
   // results: lane holds outputs 4 * (lane / 16) + j of pixel lane % 16 of each of its groups
-  float* on = out + (size_t)n * g.cout * plane;  // plane = h * W
+  float* on = (ksplit > 1 ? partial + (size_t)split * g.batch * g.cout * plane : out) + (size_t)n * g.cout * plane;
+  const bool add_bias = split == 0;
 #pragma unroll
   for (int i = 0; i < GPW; ++i) {
     const int q = (wave + 4 * i) * 16 + (lane & 15);
@@ -221,7 +226,7 @@ __global__ __launch_bounds__(kCvBlock, 2) void offset_conv_forward_kernel(
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
         const int o = 4 * (lane >> 4) + j;
-        if (o < g.cout) on[(size_t)o * plane + row * W + q % W] = acc[i][j] + bias[o];
+        if (o < g.cout) on[(size_t)o * plane + row * W + q % W] = acc[i][j] + (add_bias ? bias[o] : 0.f);
       }
     }
   }
@@ -233,7 +238,7 @@ __global__ __launch_bounds__(kCvBlock, 2) void offset_conv_forward_kernel(
       if (q < tile_pix && row < g.h) {
 #pragma unroll
         for (int o = 0; o < REST; ++o)
-          on[(size_t)(16 + o) * plane + row * W + q % W] = racc[j][o] + bias[16 + o];
+          on[(size_t)(16 + o) * plane + row * W + q % W] = racc[j][o] + (add_bias ? bias[16 + o] : 0.f);
       }
     }
   }
@@ -439,21 +444,33 @@ void offset_conv_bias_grad(int batch, int cout, int plane, const float* gout, fl
 bool offset_conv_supported(int cin, int cout, int h, int w) {
   const bool outputs_ok = (cout >= 1 && cout <= 16) || cout == 18 || cout == 20;  // the instantiated VALU widths
   return cin >= kCvChunk && cin % kCvChunk == 0 && outputs_ok && (w == 7 || w == 14 || w == 28 || w == 56 || w == 112) && h >= 1 &&
-         (long)cin * h * w < (1L << 31) / 4;
+         (long)cin * h * w < (1L << 31) / 4 && (long)cout * h * w < (1L << 31) / 4;  // 32-bit byte offsets per image
 }
 
-// Whether the kernel is also the faster choice (measured against the library convolution on
-// MI355X): it is on the 56- and 112-wide planes once there is about a workgroup per CU; on
-// smaller planes a workgroup's serial walk over all input channels loses.
-bool offset_conv_worthwhile(int batch, int cin, int cout, int h, int w) {
-  if (!offset_conv_supported(cin, cout, h, w) || w < 56) return false;
+// Input-channel splits of the forward: enough for about two workgroups per CU, at least two
+// chunks of 16 channels per split
+int forward_splits(int batch, int cin, int h, int w) {
   const int th = w <= 56 ? 8 : 4;
-  return (long)batch * ceil_div(h, th) >= 192;
+  const long base = (long)batch * ceil_div(h, th);
+  if (base >= 384) return 1;
+  return (int)std::max<long>(1, std::min<long>((512 + base - 1) / base, cin / kCvChunk / 2));
 }
 
-// packed weights: w16 [9][cin][16] and wrest [9][cin][cout - 16]
-size_t offset_conv_workspace(int cin, int cout) {
-  return round256((size_t)9 * cin * 16 * sizeof(float)) + round256((size_t)9 * cin * std::max(0, cout - 16) * sizeof(float));
+// Whether the kernels are also the faster choice (measured against the library convolution on
+// MI355X, batch 64, forward + backward): on planes 28 wide and wider (56 and 112: by 30-40 %)
+// once the grid -- (image, row tile) items times the input-channel splits -- gives about a
+// workgroup per CU; on the 14- and 7-wide planes the two are within 10 % of each other either way.
+bool offset_conv_worthwhile(int batch, int cin, int cout, int h, int w) {
+  if (!offset_conv_supported(cin, cout, h, w) || w < 28) return false;
+  const int th = w <= 56 ? 8 : 4;
+  return (long)batch * ceil_div(h, th) * forward_splits(batch, cin, h, w) >= 192;
+}
+
+// packed weights: w16 [9][cin][16] and wrest [9][cin][cout - 16]; then the splits' partial outputs
+size_t offset_conv_workspace(int batch, int cin, int cout, int h, int w) {
+  const int ks = forward_splits(batch, cin, h, w);
+  return round256((size_t)9 * cin * 16 * sizeof(float)) + round256((size_t)9 * cin * std::max(0, cout - 16) * sizeof(float)) +
+         (ks > 1 ? (size_t)ks * batch * cout * h * w * sizeof(float) : 0);
 }
 
 bool offset_conv_forward(int batch, int cin, int cout, int h, int w, const float* x, const float* weight,
@@ -462,7 +479,10 @@ bool offset_conv_forward(int batch, int cin, int cout, int h, int w, const float
   if (batch == 0) return true;
   const int rest = std::max(0, cout - 16);
   float* w16 = static_cast<float*>(ws);
-  float* wrest = reinterpret_cast<float*>(static_cast<char*>(ws) + round256((size_t)9 * cin * 16 * sizeof(float)));
+  char* after16 = static_cast<char*>(ws) + round256((size_t)9 * cin * 16 * sizeof(float));
+  float* wrest = reinterpret_cast<float*>(after16);
+  float* partial = reinterpret_cast<float*>(after16 + round256((size_t)9 * cin * rest * sizeof(float)));
+  const int ksplit = forward_splits(batch, cin, h, w);
   conv_pack_weights_kernel<<<ceil_div(9 * cin * 16, 256), 256, 0, stream>>>(weight, cout, cin, rest, w16, wrest);
   ConvGeo g;
   g.batch = batch, g.cin = cin, g.cout = cout, g.h = h;
@@ -470,8 +490,9 @@ bool offset_conv_forward(int batch, int cin, int cout, int h, int w, const float
   {                                                                                                     \
     g.tiles = ceil_div(h, ConvTile<WW>::TH);                                                            \
     const size_t lds = (size_t)kCvChunk * (ConvTile<WW>::PS + 9 * REST) * sizeof(float);                \
-    const unsigned grid = (unsigned)xcd_grid_size((long)batch * g.tiles);                               \
-    offset_conv_forward_kernel<WW, REST><<<grid, kCvBlock, lds, stream>>>(g, x, w16, wrest, bias, out); \
+    const unsigned grid = (unsigned)xcd_grid_size((long)batch * g.tiles * ksplit);                      \
+    offset_conv_forward_kernel<WW, REST><<<grid, kCvBlock, lds, stream>>>(g, x, w16, wrest, bias, out,  \
+                                                                         partial, ksplit);              \
   }
 #define DK_WIDTH(REST)                       \
   switch (w) {                               \
@@ -490,6 +511,7 @@ bool offset_conv_forward(int batch, int cin, int cout, int h, int w, const float
   }
 #undef DK_WIDTH
 #undef DK_LAUNCH
+  if (ksplit > 1) launch_reduce_partials<float, float>(partial, ksplit, (long)batch * cout * h * w, out, stream);
   return true;
 }
 
