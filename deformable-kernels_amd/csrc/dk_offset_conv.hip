@@ -9,7 +9,7 @@
 // A workgroup owns a tile of TH rows of one image (up to 448 pixels = 28 groups of 16 pixels,
 // seven per wave) and walks the input channels in chunks of 16, staged zero-padded in LDS.
 // Per tap and 4 channels one MFMA per pixel group multiplies the 16 x 4 block of weights
-// (outputs 0..15; A operand, one coalesced 256-byte load from the packed copy [tap][c][16]) with
+// (outputs 0..15; A operand, from the chunk's slice of the packed copy [tap][c][16] in LDS) with
 // the 4 x 16 block of shifted inputs (B operand, one LDS read per lane: lane = (channel k,
 // pixel n); the channel pitch is 16 mod 64 words so the four channels of a read hit disjoint
 // banks).  The outputs beyond the 16th (two of the 18) are summed on the vector ALU, their
@@ -66,7 +66,7 @@ template <int W, int REST>
 __global__ __launch_bounds__(kCvBlock, 2) void offset_conv_forward_kernel(
     ConvGeo g, const float* __restrict__ x, const float* __restrict__ w16, const float* __restrict__ wrest,
     const float* __restrict__ bias, float* __restrict__ out, float* __restrict__ partial, int ksplit) {
-  extern __shared__ __align__(16) float xs[];  // [kCvChunk][PS], then the chunk's VALU-path weights [kCvChunk][9][REST]
+  extern __shared__ __align__(16) float xs[];  // [kCvChunk][PS], the chunk's VALU-path weights [kCvChunk][9][REST], its MFMA weights [9][256]
   constexpr int TH = ConvTile<W>::TH, SEGS = ConvTile<W>::SEGS, RS = ConvTile<W>::RS, PS = ConvTile<W>::PS;
   constexpr int kStage = (kCvChunk / 4) * (TH + 2) * SEGS;  // row segments of 64 columns a wave stages per chunk
   constexpr int kPixPerThread = (kCvTilePix + kCvBlock - 1) / kCvBlock;  // of the VALU path
@@ -126,8 +126,14 @@ __global__ __launch_bounds__(kCvBlock, 2) void offset_conv_forward_kernel(
   constexpr int kRestW = kCvChunk * 9 * REST, kRestPerThread = (kRestW + kCvBlock - 1) / kCvBlock;
   float* wl = xs + kCvChunk * PS;
   float wstage[kRestPerThread > 0 ? kRestPerThread : 1];
+  // The chunk's matrix-core weights [9][16 channels][16 outputs] travel through LDS too, loaded
+  // with the next chunk's inputs, so that the multiply loop holds LDS reads and MFMAs only.
+  float* wa = wl + kCvChunk * 9 * REST;
+  float astage[9];
 #define DK_LOAD_CHUNK(CK)                                                                                  \
   {                                                                                                        \
+    _Pragma("unroll") for (int t = 0; t < 9; ++t)                                                          \
+      astage[t] = w16[((size_t)t * g.cin + (size_t)(CK) * kCvChunk) * 16 + threadIdx.x];                   \
     _Pragma("unroll") for (int u = 0; u < kRestPerThread; ++u) {                                           \
       const int e = (int)threadIdx.x + kCvBlock * u; /* = (c * 9 + t) * REST + o */                        \
       const int o = e % (REST > 0 ? REST : 1), t = e / (REST > 0 ? REST : 1) % 9, c = e / (REST > 0 ? REST : 1) / 9; \
@@ -144,7 +150,6 @@ __global__ __launch_bounds__(kCvBlock, 2) void offset_conv_forward_kernel(
     }                                                                                                      \
   }
 
-  const rsrc_t rw = plane_rsrc(w16, 9 * g.cin * 16);
   const int per_split = ceil_div(g.cin / kCvChunk, ksplit);
   const int ck_begin = split * per_split, nchunks = min(g.cin / kCvChunk, ck_begin + per_split);
   if (ck_begin < nchunks) DK_LOAD_CHUNK(ck_begin)
@@ -158,36 +163,34 @@ __global__ __launch_bounds__(kCvBlock, 2) void offset_conv_forward_kernel(
 #pragma unroll
     for (int u = 0; u < kRestPerThread; ++u)
       if ((int)threadIdx.x + kCvBlock * u < kRestW) wl[threadIdx.x + kCvBlock * u] = wstage[u];
+#pragma unroll
+    for (int t = 0; t < 9; ++t) wa[t * 256 + threadIdx.x] = astage[t];
     __syncthreads();
     if (ck + 1 < nchunks) DK_LOAD_CHUNK(ck + 1)
 
     // matrix-core part: outputs 0..15
-    // A operand of (tap t, channels 4 cs .. 4 cs + 3): w16[(t * cin + c) * 16 + m], lane = 16 k + m
-    auto load_a = [&](int t, int cs) {
-      return __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(
-                                           rw, lane * 4, ((t * g.cin + ck * kCvChunk + 4 * cs) * 16) * 4, 0));
-    };
-    float a[4], a_next[4];
+    // A operand of (tap t, channels 4 cs .. 4 cs + 3): wa[t][4 cs + k][m], lane = 16 k + m
+    // 36 steps (tap, 4 channels); the B operands of the next step are read from LDS before the
+    // MFMAs of the current one are issued, and a scheduling barrier per step keeps the compiler
+    // from hoisting the reads of all steps to the front (252 registers)
+    float bcur[GPW], bnext[GPW];
 #pragma unroll
-    for (int cs = 0; cs < 4; ++cs) a[cs] = load_a(0, cs);
+    for (int i = 0; i < GPW; ++i) bcur[i] = xs[base[i] - RS - 1];
+    float acur = wa[lane], anext = 0.f;
 #pragma unroll
-    for (int t = 0; t < 9; ++t) {
-      if (t + 1 < 9) {
+    for (int st = 0; st < 36; ++st) {
+      if (st + 1 < 36) {
+        const int t2 = (st + 1) / 4, cs2 = (st + 1) % 4;
+        const int off2 = 4 * cs2 * PS + (t2 / 3 - 1) * RS + (t2 % 3 - 1);
+        anext = wa[t2 * 256 + cs2 * 64 + lane];
 #pragma unroll
-        for (int cs = 0; cs < 4; ++cs) a_next[cs] = load_a(t + 1, cs);
-      }
-      const int shift = (t / 3 - 1) * RS + (t % 3 - 1);
-#pragma unroll
-      for (int cs = 0; cs < 4; ++cs) {
-#pragma unroll
-        for (int i = 0; i < GPW; ++i) {
-          const float b = xs[base[i] + 4 * cs * PS + shift];
-          acc[i] = __builtin_amdgcn_mfma_f32_16x16x4f32(a[cs], b, acc[i], 0, 0, 0);
-        }
+        for (int i = 0; i < GPW; ++i) bnext[i] = xs[base[i] + off2];
       }
 #pragma unroll
-      for (int cs = 0; cs < 4; ++cs) a[cs] = a_next[cs];
-      // keep the scheduler from hoisting the LDS reads of all nine taps to the front (252 registers)
+      for (int i = 0; i < GPW; ++i) acc[i] = __builtin_amdgcn_mfma_f32_16x16x4f32(acur, bcur[i], acc[i], 0, 0, 0);
+#pragma unroll
+      for (int i = 0; i < GPW; ++i) bcur[i] = bnext[i];
+      acur = anext;
       __builtin_amdgcn_sched_barrier(0);
     }
 
@@ -489,7 +492,7 @@ bool offset_conv_forward(int batch, int cin, int cout, int h, int w, const float
 #define DK_LAUNCH(WW, REST)                                                                             \
   {                                                                                                     \
     g.tiles = ceil_div(h, ConvTile<WW>::TH);                                                            \
-    const size_t lds = (size_t)kCvChunk * (ConvTile<WW>::PS + 9 * REST) * sizeof(float);                \
+    const size_t lds = (size_t)(kCvChunk * (ConvTile<WW>::PS + 9 * REST) + 9 * 256) * sizeof(float);    \
     const unsigned grid = (unsigned)xcd_grid_size((long)batch * g.tiles * ksplit);                      \
     offset_conv_forward_kernel<WW, REST><<<grid, kCvBlock, lds, stream>>>(g, x, w16, wrest, bias, out,  \
                                                                          partial, ksplit);              \
