@@ -512,7 +512,7 @@ __global__ __launch_bounds__(kBlock, 2) void local_grad_rotation_kernel(
   for (int t = 0; t < K; ++t) sb[t] = sc[t] = sd[t] = 0.f;
 
   // ch_per_pass + 1 tables: the spare one is read, times zero, by the odd channel out of a pair
-  for (int e = threadIdx.x; e < (ch_per_pass + 1) * Tb::SIZE; e += kBlock) tbl[e] = 0.f;
+  for (int e = threadIdx.x; e < (ch_per_pass + 1) * Tb::SIZE; e += blockDim.x) tbl[e] = 0.f;
   for (int j0 = c_begin; j0 < c_end; j0 += ch_per_pass) {
     const int nch = min(ch_per_pass, c_end - j0);
     __syncthreads();
@@ -639,7 +639,7 @@ __global__ __launch_bounds__(kBlock, 2) void local_grad_filter_kernel(
   const int by = lb % splits, bx = lb / splits % parts, grp = lb / splits / parts;
 
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  for (int e = threadIdx.x; e < kWaves * ch_per_block * 16; e += kBlock) wacc[e] = 0.f;
+  for (int e = threadIdx.x; e < kWaves * ch_per_block * 16; e += blockDim.x) wacc[e] = 0.f;
   __syncthreads();
 
   const int j0 = by * ch_per_block;
@@ -782,7 +782,7 @@ __global__ __launch_bounds__(kBlock, 2) void local_grad_filter_kernel(
   }
   __syncthreads();
 
-  for (int e = threadIdx.x; e < nch * CELLS; e += kBlock) {
+  for (int e = threadIdx.x; e < nch * CELLS; e += blockDim.x) {
     const int j = e / CELLS, r = e % CELLS;
     float s_ = 0.f;
 #pragma unroll
@@ -1157,6 +1157,12 @@ bool stride2_geometry(const Geo& g) {
 }
 int rotation_tile(const Geo& g) { return same_width_geometry(g) ? kRowPix : stride2_geometry(g) ? kS2Pix : kBlock; }
 
+// Threads of a workgroup of the row kernels: whole waves, no more than the plane needs (a 7 x 7
+// plane fits the 62 pixels of one wave; three more waves would only walk the channels idle).
+unsigned row_block(int pixels, int lanes_per_wave) {
+  return 64u * (unsigned)std::min(kBlock / 64, ceil_div(pixels, lanes_per_wave));
+}
+
 template <typename T, int SH, int SW>
 bool run_gather(const Geo& g, bool transposed, const T* src, const T* rot, const T* filter, T* dst,
                 hipStream_t stream) {
@@ -1167,16 +1173,16 @@ bool run_gather(const Geo& g, bool transposed, const T* src, const T* rot, const
     const unsigned grid = (unsigned)xcd_grid_size((long)ceil_div(pixels, kRowPix) * ceil_div(cpg, per) * g.batch * g.groups);
     const size_t lds = (size_t)(per + kRowStages * kUnroll) * WideTable<SH, SW>::SIZE * sizeof(float);
     if (transposed)
-      local_gather_rows_kernel<T, 3, SH, SW, true><<<grid, kBlock, lds, stream>>>(g, src, rot, filter, dst, per);
+      local_gather_rows_kernel<T, 3, SH, SW, true><<<grid, row_block(pixels, kRowLanes), lds, stream>>>(g, src, rot, filter, dst, per);
     else
-      local_gather_rows_kernel<T, 3, SH, SW, false><<<grid, kBlock, lds, stream>>>(g, src, rot, filter, dst, per);
+      local_gather_rows_kernel<T, 3, SH, SW, false><<<grid, row_block(pixels, kRowLanes), lds, stream>>>(g, src, rot, filter, dst, per);
     return true;
   }
   const int per = channels_per_block<SH, SW>(cpg, pick_splits(g, pixels));
   if (!transposed && stride2_geometry(g)) {
     const unsigned grid2 = (unsigned)xcd_grid_size((long)ceil_div(pixels, kS2Pix) * ceil_div(cpg, per) * g.batch * g.groups);
     const size_t lds2 = (size_t)(per + 2 * kUnroll) * WideTable<SH, SW>::SIZE * sizeof(float);
-    local_forward_s2_kernel<T, SH, SW><<<grid2, kBlock, lds2, stream>>>(g, src, rot, filter, dst, per);
+    local_forward_s2_kernel<T, SH, SW><<<grid2, row_block(pixels, kS2Lanes), lds2, stream>>>(g, src, rot, filter, dst, per);
     return true;
   }
   const unsigned grid = (unsigned)xcd_grid_size((long)ceil_div(pixels, kBlock) * ceil_div(cpg, per) * g.batch * g.groups);
@@ -1210,9 +1216,9 @@ bool run_grad_rotation(const Geo& g, const T* gout, const T* x, const T* rot, co
   const size_t lds = (size_t)(per + 1) * Tb::SIZE * sizeof(float);
   const unsigned grid = (unsigned)xcd_grid_size((long)ceil_div(g.out_h * g.out_w, rotation_tile(g)) * splits * g.batch * g.groups);
   if (same_width_geometry(g))
-    local_grad_rotation_kernel<T, 3, 3, SH, SW, 1><<<grid, kBlock, lds, stream>>>(g, gout, x, rot, filter, grot, ws, splits, per);
+    local_grad_rotation_kernel<T, 3, 3, SH, SW, 1><<<grid, row_block(g.out_h * g.out_w, kRowLanes), lds, stream>>>(g, gout, x, rot, filter, grot, ws, splits, per);
   else if (stride2_geometry(g))
-    local_grad_rotation_kernel<T, 3, 3, SH, SW, 2><<<grid, kBlock, lds, stream>>>(g, gout, x, rot, filter, grot, ws, splits, per);
+    local_grad_rotation_kernel<T, 3, 3, SH, SW, 2><<<grid, row_block(g.out_h * g.out_w, kS2Lanes), lds, stream>>>(g, gout, x, rot, filter, grot, ws, splits, per);
   else
     local_grad_rotation_kernel<T, 3, 3, SH, SW, 0><<<grid, kBlock, lds, stream>>>(g, gout, x, rot, filter, grot, ws, splits, per);
   if (splits > 1)
@@ -1285,9 +1291,9 @@ bool run_grad_filter(const Geo& g, const T* gout, const T* x, const T* rot, T* g
     }
     const size_t lds = ((size_t)(kBlock / 64) * f.per * 16 + (size_t)(kBlock / 64) * 64 * 20) * sizeof(float);
     if (same_width_geometry(g))
-      local_grad_filter_kernel<T, 3, 3, SH, SW, 1><<<grid, kBlock, lds, stream>>>(g, gout, x, rot, ws, f.tiles, f.per, f.parts);
+      local_grad_filter_kernel<T, 3, 3, SH, SW, 1><<<grid, row_block(g.out_h * g.out_w, kRowLanes), lds, stream>>>(g, gout, x, rot, ws, f.tiles, f.per, f.parts);
     else if (stride2_geometry(g))
-      local_grad_filter_kernel<T, 3, 3, SH, SW, 2><<<grid, kBlock, lds, stream>>>(g, gout, x, rot, ws, f.tiles, f.per, f.parts);
+      local_grad_filter_kernel<T, 3, 3, SH, SW, 2><<<grid, row_block(g.out_h * g.out_w, kS2Lanes), lds, stream>>>(g, gout, x, rot, ws, f.tiles, f.per, f.parts);
     else
       local_grad_filter_kernel<T, 3, 3, SH, SW, 0><<<grid, kBlock, lds, stream>>>(g, gout, x, rot, ws, f.tiles, f.per, f.parts);
     launch_reduce_partials<float, T>(ws, f.parts, g.channel * SH * SW, gfilter, stream);
