@@ -318,19 +318,35 @@ def other_workload(a):
         st = _lib.stream_ptr(data)
         e = data.element_size()
         bd, bc, bo = data.numel() * e, coord.numel() * e, go.numel() * e
+        # each entry point alone (order = NULL: it sorts the points itself when it works on sorted
+        # points), then the autograd Function's sequence: order once, the three calls with it
+        order, wo, no_ = None, None, 0
+        if L.dk_nd_linear_sample_order_bytes(desc):
+            order = torch.empty(L.dk_nd_linear_sample_order_bytes(desc), dtype=torch.uint8, device=dev)
+            wo, no_ = _lib.workspace(L.dk_nd_linear_sample_order_workspace(desc), dev)
+
+        def whole_step():
+            if order is not None:
+                _lib.check(L.dk_nd_linear_sample_order(desc, P(coord), P(order), P(wo), no_, st), "order")
+            _lib.check(L.dk_nd_linear_sample_forward(desc, P(data), P(coord), P(order), P(out), P(wf), nf, st), "fwd")
+            _lib.check(L.dk_nd_linear_sample_backward_data(desc, P(go), P(coord), P(order), P(gd), P(ws), nb, st), "gd")
+            _lib.check(L.dk_nd_linear_sample_backward_coord(desc, P(go), P(data), P(coord), P(order), P(gc), P(wf), nf, st),
+                       "gc")
+
         calls = {
-            "forward": (lambda: _lib.check(L.dk_nd_linear_sample_forward(desc, P(data), P(coord), P(out), P(wf), nf, st), "fwd"),
-                        bd + bc + bo),
+            "forward": (lambda: _lib.check(L.dk_nd_linear_sample_forward(
+                desc, P(data), P(coord), P(None), P(out), P(wf), nf, st), "fwd"), bd + bc + bo),
             "grad_data": (lambda: _lib.check(L.dk_nd_linear_sample_backward_data(
-                desc, P(go), P(coord), P(gd), P(ws), nb, st), "gd"), bo + bc + bd),
+                desc, P(go), P(coord), P(None), P(gd), P(ws), nb, st), "gd"), bo + bc + bd),
             "grad_coord": (lambda: _lib.check(L.dk_nd_linear_sample_backward_coord(
-                desc, P(go), P(data), P(coord), P(gc), P(wf), nf, st), "gc"), bo + bd + bc + bc),
+                desc, P(go), P(data), P(coord), P(None), P(gc), P(wf), nf, st), "gc"), bo + bd + bc + bc),
+            "forward+backward, one sort": (whole_step, 2 * (bd + bc + bo) + bo + bd + 2 * bc),
         }
         label = "%s: nd_linear_sample data=%s points=%d %s" % (a.workload, list(shape), B, a.dtype)
     for name, (fn, nb_) in calls.items():
         us[name] = _time_us(fn, reps)
         nbytes[name] = nb_
-    total_us = sum(us.values())
+    total_us = sum(v for k_, v in us.items() if "+" not in k_)
     print(json.dumps({
         "metric": "per-entry-point time (secondary workload, not the BASELINE headline)",
         "config": {"workload": label},

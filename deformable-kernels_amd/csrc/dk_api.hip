@@ -464,7 +464,31 @@ size_t dk_nd_linear_sample_forward_workspace(const dk_nd_desc* desc) {
   return nd_data_cl_workspace(*desc);
 }
 
-int dk_nd_linear_sample_forward(const dk_nd_desc* desc, const void* data, const void* coord,
+size_t dk_nd_linear_sample_order_bytes(const dk_nd_desc* desc) {
+  if (check_nd(desc) != DK_OK) return 0;
+  return nd_order_bytes(*desc);
+}
+
+size_t dk_nd_linear_sample_order_workspace(const dk_nd_desc* desc) {
+  if (check_nd(desc) != DK_OK) return 0;
+  return nd_sort_workspace(*desc);
+}
+
+int dk_nd_linear_sample_order(const dk_nd_desc* desc, const void* coord, void* order, void* workspace,
+                              size_t workspace_bytes, void* stream) {
+  const int rc = check_nd(desc);
+  if (rc != DK_OK) return rc;
+  if (nd_order_bytes(*desc) == 0) return DK_ERR_UNSUPPORTED;
+  if (!coord || !order) return DK_ERR_NULL_POINTER;
+  const size_t need = nd_sort_workspace(*desc);
+  if (!workspace || workspace_bytes < need) return DK_ERR_WORKSPACE;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  return by_dtype(desc->dtype, [&]<typename T>() {
+    nd_order<T>(*desc, in<T>(coord), static_cast<int*>(order), workspace, s);
+  });
+}
+
+int dk_nd_linear_sample_forward(const dk_nd_desc* desc, const void* data, const void* coord, const void* order,
                                 void* output, void* workspace, size_t workspace_bytes,
                                 void* stream) {
   const int rc = check_nd(desc);
@@ -475,7 +499,7 @@ int dk_nd_linear_sample_forward(const dk_nd_desc* desc, const void* data, const 
   if (desc->batch == 0) return DK_OK;
   hipStream_t s = static_cast<hipStream_t>(stream);
   return by_dtype(desc->dtype, [&]<typename T>() {
-    nd_forward<T>(*desc, in<T>(data), in<T>(coord), out<T>(output), workspace, s);
+    nd_forward<T>(*desc, in<T>(data), in<T>(coord), out<T>(output), workspace, static_cast<const int*>(order), s);
   });
 }
 
@@ -485,7 +509,7 @@ size_t dk_nd_linear_sample_backward_data_workspace(const dk_nd_desc* desc) {
 }
 
 int dk_nd_linear_sample_backward_data(const dk_nd_desc* desc, const void* out_grad,
-                                      const void* coord, void* in_grad, void* workspace,
+                                      const void* coord, const void* order, void* in_grad, void* workspace,
                                       size_t workspace_bytes, void* stream) {
   const int rc = check_nd(desc);
   if (rc != DK_OK) return rc;
@@ -494,7 +518,7 @@ int dk_nd_linear_sample_backward_data(const dk_nd_desc* desc, const void* out_gr
   if (need && (!workspace || workspace_bytes < need)) return DK_ERR_WORKSPACE;
   hipStream_t s = static_cast<hipStream_t>(stream);
   return by_dtype(desc->dtype, [&]<typename T>() {
-    nd_grad_data<T>(*desc, in<T>(out_grad), in<T>(coord), out<T>(in_grad), workspace, s);
+    nd_grad_data<T>(*desc, in<T>(out_grad), in<T>(coord), out<T>(in_grad), workspace, static_cast<const int*>(order), s);
   });
 }
 
@@ -504,7 +528,7 @@ size_t dk_nd_linear_sample_backward_coord_workspace(const dk_nd_desc* desc) {
 }
 
 int dk_nd_linear_sample_backward_coord(const dk_nd_desc* desc, const void* out_grad,
-                                       const void* data, const void* coord, void* coord_grad,
+                                       const void* data, const void* coord, const void* order, void* coord_grad,
                                        void* workspace, size_t workspace_bytes, void* stream) {
   const int rc = check_nd(desc);
   if (rc != DK_OK) return rc;
@@ -514,7 +538,8 @@ int dk_nd_linear_sample_backward_coord(const dk_nd_desc* desc, const void* out_g
   if (need && (!workspace || workspace_bytes < need)) return DK_ERR_WORKSPACE;
   hipStream_t s = static_cast<hipStream_t>(stream);
   return by_dtype(desc->dtype, [&]<typename T>() {
-    nd_grad_coord<T>(*desc, in<T>(out_grad), in<T>(data), in<T>(coord), out<T>(coord_grad), workspace, s);
+    nd_grad_coord<T>(*desc, in<T>(out_grad), in<T>(data), in<T>(coord), out<T>(coord_grad), workspace,
+                     static_cast<const int*>(order), s);
   });
 }
 

@@ -741,7 +741,7 @@ size_t data_bytes(const dk_nd_desc& d) {
 }  // namespace
 
 template <typename T>
-void nd_forward(const dk_nd_desc& d, const T* data, const T* coord, T* out, void* ws,
+void nd_forward(const dk_nd_desc& d, const T* data, const T* coord, T* out, void* ws, const int* order,
                 hipStream_t stream) {
   const NdGeo g = make_geo(d);
   if constexpr (!std::is_same<T, double>::value) {
@@ -749,7 +749,7 @@ void nd_forward(const dk_nd_desc& d, const T* data, const T* coord, T* out, void
       T* data_cl = static_cast<T*>(ws);
       transpose<T, T>(data, data_cl, g.channel, g.prod_shape, stream);
       if (const int bins = nd_bins(d)) {
-        const int* order = sort_points<T>(g, coord, bins, static_cast<char*>(ws) + round256(data_bytes(d) * sizeof(T)), stream);
+        if (!order) order = sort_points<T>(g, coord, bins, static_cast<char*>(ws) + round256(data_bytes(d) * sizeof(T)), stream);
         nd_forward_binned_kernel<T><<<(unsigned)((g.batch + 255) / 256), kBlock, 0, stream>>>(g, data_cl, coord, order, bins, out);
         return;
       }
@@ -772,7 +772,7 @@ size_t nd_grad_data_workspace(const dk_nd_desc& d) {
 }
 
 template <typename T>
-void nd_grad_data(const dk_nd_desc& d, const T* gout, const T* coord, T* gdata, void* ws,
+void nd_grad_data(const dk_nd_desc& d, const T* gout, const T* coord, T* gdata, void* ws, const int* order,
                   hipStream_t stream) {
   using CT = compute_t<T>;
   const NdGeo g = make_geo(d);
@@ -783,7 +783,7 @@ void nd_grad_data(const dk_nd_desc& d, const T* gout, const T* coord, T* gdata, 
       float* acc = static_cast<float*>(ws);
       nd_fill_zero_kernel<float><<<grid_for(n_data), kBlock, 0, stream>>>(acc, n_data);
       if (const int bins = nd_bins(d)) {
-        const int* order = sort_points<T>(g, coord, bins, static_cast<char*>(ws) + round256((size_t)n_data * sizeof(float)), stream);
+        if (!order) order = sort_points<T>(g, coord, bins, static_cast<char*>(ws) + round256((size_t)n_data * sizeof(float)), stream);
         // chunks of 64 points per wave: as many as keep about 16 waves per CU in the grid
         int per_wave = 1;
         while (per_wave < 8 && g.batch / (64L * per_wave * 2) >= 4096) per_wave *= 2;
@@ -808,14 +808,14 @@ void nd_grad_data(const dk_nd_desc& d, const T* gout, const T* coord, T* gdata, 
 
 template <typename T>
 void nd_grad_coord(const dk_nd_desc& d, const T* gout, const T* data, const T* coord, T* gcoord,
-                   void* ws, hipStream_t stream) {
+                   void* ws, const int* order, hipStream_t stream) {
   const NdGeo g = make_geo(d);
   if constexpr (!std::is_same<T, double>::value) {
     if (nd_use_channel_last(d)) {
       T* data_cl = static_cast<T*>(ws);
       transpose<T, T>(data, data_cl, g.channel, g.prod_shape, stream);
       if (const int bins = nd_bins(d)) {
-        const int* order = sort_points<T>(g, coord, bins, static_cast<char*>(ws) + round256(data_bytes(d) * sizeof(T)), stream);
+        if (!order) order = sort_points<T>(g, coord, bins, static_cast<char*>(ws) + round256(data_bytes(d) * sizeof(T)), stream);
         nd_grad_coord_binned_kernel<T><<<(unsigned)((g.batch + 255) / 256), kBlock, 0, stream>>>(g, gout, data_cl, coord, order, bins, gcoord);
         return;
       }
@@ -830,10 +830,27 @@ void nd_grad_coord(const dk_nd_desc& d, const T* gout, const T* data, const T* c
   nd_grad_coord_kernel<T><<<(int)blocks, kBlock, 0, stream>>>(g, gout, data, coord, gcoord);
 }
 
+// The sorted order of the points alone, for a caller that issues several of the three calls on
+// the same coordinates: `order` receives batch ints; ws as nd_sort_workspace() sizes it.
+size_t nd_order_bytes(const dk_nd_desc& d) { return nd_bins(d) ? (size_t)d.batch * sizeof(int) : 0; }
+
+template <typename T>
+void nd_order(const dk_nd_desc& d, const T* coord, int* order, void* ws, hipStream_t stream) {
+  const NdGeo g = make_geo(d);
+  if constexpr (!std::is_same<T, double>::value) {
+    if (const int bins = nd_bins(d)) {
+      const int* sorted = sort_points<T>(g, coord, bins, ws, stream);
+      (void)hipMemcpyAsync(order, sorted, (size_t)d.batch * sizeof(int), hipMemcpyDeviceToDevice, stream);
+    }
+  }
+}
+
 #define DK_INSTANTIATE(T)                                                                             \
-  template void nd_forward<T>(const dk_nd_desc&, const T*, const T*, T*, void*, hipStream_t);          \
-  template void nd_grad_data<T>(const dk_nd_desc&, const T*, const T*, T*, void*, hipStream_t);        \
-  template void nd_grad_coord<T>(const dk_nd_desc&, const T*, const T*, const T*, T*, void*, hipStream_t);
+  template void nd_forward<T>(const dk_nd_desc&, const T*, const T*, T*, void*, const int*, hipStream_t);   \
+  template void nd_grad_data<T>(const dk_nd_desc&, const T*, const T*, T*, void*, const int*, hipStream_t); \
+  template void nd_grad_coord<T>(const dk_nd_desc&, const T*, const T*, const T*, T*, void*, const int*,    \
+                                 hipStream_t);                                                         \
+  template void nd_order<T>(const dk_nd_desc&, const T*, int*, void*, hipStream_t);
 DK_INSTANTIATE(float)
 DK_INSTANTIATE(double)
 DK_INSTANTIATE(__half)

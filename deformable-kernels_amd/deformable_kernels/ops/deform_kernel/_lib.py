@@ -67,11 +67,14 @@ SIGNATURES = {
     "dk_deformable_sample_depthwise_backward_rotation_workspace": (_SZ, [_CD]),
     "dk_deformable_sample_depthwise_backward_rotation": (ctypes.c_int, [_CD, _P, _P, _P, _P, _P, _P, _P, _SZ, _P]),
     "dk_nd_linear_sample_forward_workspace": (_SZ, [_ND]),
-    "dk_nd_linear_sample_forward": (ctypes.c_int, [_ND, _P, _P, _P, _P, _SZ, _P]),
+    "dk_nd_linear_sample_forward": (ctypes.c_int, [_ND, _P, _P, _P, _P, _P, _SZ, _P]),
+    "dk_nd_linear_sample_order_bytes": (_SZ, [_ND]),
+    "dk_nd_linear_sample_order_workspace": (_SZ, [_ND]),
+    "dk_nd_linear_sample_order": (ctypes.c_int, [_ND, _P, _P, _P, _SZ, _P]),
     "dk_nd_linear_sample_backward_data_workspace": (_SZ, [_ND]),
-    "dk_nd_linear_sample_backward_data": (ctypes.c_int, [_ND, _P, _P, _P, _P, _SZ, _P]),
+    "dk_nd_linear_sample_backward_data": (ctypes.c_int, [_ND, _P, _P, _P, _P, _P, _SZ, _P]),
     "dk_nd_linear_sample_backward_coord_workspace": (_SZ, [_ND]),
-    "dk_nd_linear_sample_backward_coord": (ctypes.c_int, [_ND, _P, _P, _P, _P, _P, _SZ, _P]),
+    "dk_nd_linear_sample_backward_coord": (ctypes.c_int, [_ND, _P, _P, _P, _P, _P, _P, _SZ, _P]),
     "dk_offset_conv_supported": (ctypes.c_int, [_OC]),
     "dk_offset_conv_worthwhile": (ctypes.c_int, [_OC]),
     "dk_offset_conv_forward_workspace": (_SZ, [_OC]),

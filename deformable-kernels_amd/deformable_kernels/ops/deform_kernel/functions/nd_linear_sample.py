@@ -29,9 +29,19 @@ class NdLinearSampleFunction(Function):
         desc = _lib.nd_desc(input, coord)
         L = _lib.lib()
         with torch.cuda.device(input.device):
+            # many points per cell: the kernels work on the points sorted by cell; sort once,
+            # here, and keep the order for the backward pass
+            order = None
+            order_bytes = L.dk_nd_linear_sample_order_bytes(desc)
+            if order_bytes:
+                order = torch.empty(order_bytes, dtype=torch.uint8, device=input.device)
+                ws, nbytes = _lib.workspace(L.dk_nd_linear_sample_order_workspace(desc), input.device)
+                _lib.check(L.dk_nd_linear_sample_order(desc, _lib.ptr(coord), _lib.ptr(order), _lib.ptr(ws), nbytes,
+                                                       _lib.stream_ptr(input)), "nd_linear_sample order")
+            ctx.order = order
             ws, nbytes = _lib.workspace(L.dk_nd_linear_sample_forward_workspace(desc), input.device)
             _lib.check(L.dk_nd_linear_sample_forward(
-                desc, _lib.ptr(input), _lib.ptr(coord), _lib.ptr(output), _lib.ptr(ws), nbytes,
+                desc, _lib.ptr(input), _lib.ptr(coord), _lib.ptr(order), _lib.ptr(output), _lib.ptr(ws), nbytes,
                 _lib.stream_ptr(input)), "nd_linear_sample forward")
         return output
 
@@ -49,13 +59,13 @@ class NdLinearSampleFunction(Function):
                 grad_input = torch.empty_like(input)
                 ws, nbytes = _lib.workspace(L.dk_nd_linear_sample_backward_data_workspace(desc), input.device)
                 _lib.check(L.dk_nd_linear_sample_backward_data(
-                    desc, _lib.ptr(grad_output), _lib.ptr(coord), _lib.ptr(grad_input),
+                    desc, _lib.ptr(grad_output), _lib.ptr(coord), _lib.ptr(ctx.order), _lib.ptr(grad_input),
                     _lib.ptr(ws), nbytes, s), "nd_linear_sample backward_data")
             if ctx.needs_input_grad[1]:
                 grad_coord = torch.zeros_like(coord)
                 ws, nbytes = _lib.workspace(L.dk_nd_linear_sample_backward_coord_workspace(desc), input.device)
                 _lib.check(L.dk_nd_linear_sample_backward_coord(
-                    desc, _lib.ptr(grad_output), _lib.ptr(input), _lib.ptr(coord),
+                    desc, _lib.ptr(grad_output), _lib.ptr(input), _lib.ptr(coord), _lib.ptr(ctx.order),
                     _lib.ptr(grad_coord), _lib.ptr(ws), nbytes, s), "nd_linear_sample backward_coord")
         return (grad_input, grad_coord)
 

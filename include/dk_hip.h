@@ -194,8 +194,19 @@ typedef struct dk_nd_desc {
  * path is used. */
 size_t dk_nd_linear_sample_forward_workspace(const dk_nd_desc *desc);
 int dk_nd_linear_sample_forward(const dk_nd_desc *desc, const void *data, const void *coord,
-                                void *output, void *workspace, size_t workspace_bytes,
-                                void *stream);
+                                const void *order, void *output, void *workspace,
+                                size_t workspace_bytes, void *stream);
+
+/* With many points per cell of the volume the three functions sort the points by cell first.
+ * A caller that issues more than one of them on the same coordinates (a forward and its
+ * backward) can have the order computed once: dk_nd_linear_sample_order_bytes() is the size of
+ * the order array (0 when the configuration does not sort: pass order = NULL then),
+ * dk_nd_linear_sample_order() fills it, and the three functions take it as `order`; with
+ * order = NULL they sort for themselves.  No counterpart in the reference. */
+size_t dk_nd_linear_sample_order_bytes(const dk_nd_desc *desc);
+size_t dk_nd_linear_sample_order_workspace(const dk_nd_desc *desc);
+int dk_nd_linear_sample_order(const dk_nd_desc *desc, const void *coord, void *order,
+                              void *workspace, size_t workspace_bytes, void *stream);
 
 /* nd_linear_sample_backward_data_cuda (nd_linear_sample_cuda.cpp:29-45); in_grad is
  * fully written (the reference zero-fills it in C++ and scatters atomically).  The workspace
@@ -203,16 +214,17 @@ int dk_nd_linear_sample_forward(const dk_nd_desc *desc, const void *data, const 
  * gradients, and the channel-last path for large problems). */
 size_t dk_nd_linear_sample_backward_data_workspace(const dk_nd_desc *desc);
 int dk_nd_linear_sample_backward_data(const dk_nd_desc *desc, const void *out_grad,
-                                      const void *coord, void *in_grad, void *workspace,
-                                      size_t workspace_bytes, void *stream);
+                                      const void *coord, const void *order, void *in_grad,
+                                      void *workspace, size_t workspace_bytes, void *stream);
 
 /* nd_linear_sample_backward_coord_cuda (nd_linear_sample_cuda.cpp:47-64) fused with the
  * `.sum(2)` its Python caller applies (functions/nd_linear_sample.py:48-55):
  * coord_grad is [batch, dims], already summed over channels. */
 size_t dk_nd_linear_sample_backward_coord_workspace(const dk_nd_desc *desc);
 int dk_nd_linear_sample_backward_coord(const dk_nd_desc *desc, const void *out_grad,
-                                       const void *data, const void *coord, void *coord_grad,
-                                       void *workspace, size_t workspace_bytes, void *stream);
+                                       const void *data, const void *coord, const void *order,
+                                       void *coord_grad, void *workspace, size_t workspace_bytes,
+                                       void *stream);
 
 /* ---- offset branch ---------------------------------------------------------- */
 

@@ -105,7 +105,7 @@ def test_c_abi_rejects_bad_arguments_before_any_launch():
     assert need > 0
     assert L.dk_sample_depthwise_backward_filter(ctypes.byref(ok), one, one, one, one, one, need - 1, null) == -5
     nd = _lib.NdDesc(4, 2, 9, (ctypes.c_int32 * 8)(*([2] * 8)), _lib.DK_F32)
-    assert L.dk_nd_linear_sample_forward(ctypes.byref(nd), one, one, one, null, 0, null) == -7
+    assert L.dk_nd_linear_sample_forward(ctypes.byref(nd), one, one, null, one, null, 0, null) == -7
     assert b"workspace" in L.dk_status_string(-5)
 
 
