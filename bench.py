@@ -32,6 +32,9 @@ WORKLOADS = {
     # name: (N, C, H, W, k, S, stride, pad, dil, groups, rot_std)
     "cfg2": (64, 144, 56, 56, 3, (4, 4), 1, 1, 1, 1, 1.0),
     "cfg1": (2, 32, 28, 28, 3, (4, 4), 1, 1, 1, 1, 0.5),
+    # config 3 (GlobalDeformKernel2d, run with --dtype fp16) as the module's fused route issues it:
+    # the local operator on the layer's shape, scope 5 x 5 (the rotation is one value per image there)
+    "cfg3": (128, 256, 28, 28, 3, (5, 5), 1, 1, 1, 1, 0.5),
 }
 DTYPES = {"fp32": "float32", "bf16": "bfloat16", "fp16": "float16"}
 

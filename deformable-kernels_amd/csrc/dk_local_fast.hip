@@ -613,8 +613,13 @@ __global__ __launch_bounds__(kBlock, 2) void local_grad_rotation_kernel(
 // workgroup goes to the workspace; reduce_partials_kernel adds the partials in order.
 // grid = (parts, channel splits, groups)
 // ---------------------------------------------------------------------------
+// accumulator slots per channel and floats per lane of the fold's transpose scratch (16-byte
+// aligned, bank-skewed) for a scope of `cells` cells
+constexpr int filter_slots(int cells) { return cells <= 16 ? 16 : 32; }
+constexpr int filter_pitch(int cells) { return cells <= 16 ? 20 : 36; }
+
 template <typename T, int KH, int KW, int SH, int SW, int MODE>
-__global__ __launch_bounds__(kBlock, 2) void local_grad_filter_kernel(
+__global__ __launch_bounds__(kBlock, (SH * SW <= 16 ? 2 : 1)) void local_grad_filter_kernel(
     Geo g, const T* __restrict__ gout, const T* __restrict__ x, const T* __restrict__ rot,
     float* __restrict__ partial, int tiles, int ch_per_block, int parts) {
   constexpr int K = KH * KW;
@@ -622,12 +627,12 @@ __global__ __launch_bounds__(kBlock, 2) void local_grad_filter_kernel(
   constexpr bool ROWS = MODE == 1, S2 = MODE == 2;  // as in local_grad_rotation_kernel
   constexpr int NLOAD = MODE == 0 ? K : KH;
   constexpr int PIX = ROWS ? kRowPix : S2 ? kS2Pix : kBlock;  // pixels per (image, tile) item
-  static_assert(CELLS <= 16, "the fold below handles up to 16 cells per 16-lane row");
-  constexpr int kPitch = 20;  // floats per lane in the transpose scratch: 16-byte aligned, bank-skewed
+  static_assert(CELLS <= 32, "the fold below handles up to two cells per lane of a 16-lane row");
+  constexpr int CP = filter_slots(CELLS), kPitch = filter_pitch(CELLS);
   constexpr int kWaves = kBlock / 64;
   extern __shared__ __align__(16) float lds[];
-  float* wacc = lds;                                  // [kWaves][ch_per_block][16]
-  float* scratch = lds + kWaves * ch_per_block * 16;  // [kWaves][64][kPitch]
+  float* wacc = lds;                                  // [kWaves][ch_per_block][CP]
+  float* scratch = lds + kWaves * ch_per_block * CP;  // [kWaves][64][kPitch]
 
   // logical block = (channel split, part, group), split fastest: the splits of one
   // (image, tile) item and the items of one image share an XCD
@@ -639,14 +644,14 @@ __global__ __launch_bounds__(kBlock, 2) void local_grad_filter_kernel(
   const int by = lb % splits, bx = lb / splits % parts, grp = lb / splits / parts;
 
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  for (int e = threadIdx.x; e < kWaves * ch_per_block * 16; e += blockDim.x) wacc[e] = 0.f;
+  for (int e = threadIdx.x; e < kWaves * ch_per_block * CP; e += blockDim.x) wacc[e] = 0.f;
   __syncthreads();
 
   const int j0 = by * ch_per_block;
   const int nch = min(ch_per_block, cpg - j0);
   const int out_plane = g.out_h * g.out_w, in_plane = g.in_h * g.in_w;
   const int items = g.batch * tiles;
-  float* my_acc = wacc + wave * ch_per_block * 16;
+  float* my_acc = wacc + wave * ch_per_block * CP;
   float* my_scr = scratch + wave * 64 * kPitch;
   // read-back pattern of the fold: lane (row = lane / 16, m = lane % 16) sums cell m over the
   // 16 lanes of its row, starting 4 * row lanes in so the four rows hit disjoint banks
@@ -761,15 +766,21 @@ __global__ __launch_bounds__(kBlock, 2) void local_grad_filter_kernel(
         for (int k = 0; k < SW; ++k) mine[i * SW + k] = acc[i][k];
       __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
       __builtin_amdgcn_wave_barrier();
-      float sum = 0.f;
-      if (m < CELLS) {
+      float sum[CP / 16];
 #pragma unroll
-        for (int q = 0; q < 16; ++q) sum += my_scr[(row * 16 + ((q + 4 * row) & 15)) * kPitch + m];
+      for (int h = 0; h < CP / 16; ++h) {  // cells m and (scopes of more than 16 cells) m + 16
+        sum[h] = 0.f;
+        if (m + 16 * h < CELLS) {
+#pragma unroll
+          for (int q = 0; q < 16; ++q) sum[h] += my_scr[(row * 16 + ((q + 4 * row) & 15)) * kPitch + m + 16 * h];
+        }
+        sum[h] += __shfl_xor(sum[h], 16, 64);
+        sum[h] += __shfl_xor(sum[h], 32, 64);
       }
-      sum += __shfl_xor(sum, 16, 64);
-      sum += __shfl_xor(sum, 32, 64);
       __builtin_amdgcn_wave_barrier();
-      if (lane < CELLS && j < nch) my_acc[j * 16 + lane] += sum;
+#pragma unroll
+      for (int h = 0; h < CP / 16; ++h)
+        if (lane < 16 && lane + 16 * h < CELLS && j < nch) my_acc[j * CP + lane + 16 * h] += sum[h];
     };
 
     load(0, 0);
@@ -786,7 +797,7 @@ __global__ __launch_bounds__(kBlock, 2) void local_grad_filter_kernel(
     const int j = e / CELLS, r = e % CELLS;
     float s_ = 0.f;
 #pragma unroll
-    for (int wv = 0; wv < kWaves; ++wv) s_ += wacc[(wv * ch_per_block + j) * 16 + r];
+    for (int wv = 0; wv < kWaves; ++wv) s_ += wacc[(wv * ch_per_block + j) * CP + r];
     const int c = grp + g.groups * (j0 + j);
     partial[((size_t)bx * g.channel + c) * CELLS + r] = s_;
   }
@@ -837,13 +848,15 @@ __device__ __forceinline__ int mf_row(int j, int pitch_x) { return j * pitch_x +
 
 __device__ __forceinline__ float hat(float d) { return __builtin_amdgcn_fmed3f(1.f - fabsf(d), 0.f, 1.f); }
 
-template <typename T, int SH, int SW>
+// CELL0: the kernel sums the scope cells CELL0 .. CELL0 + 15 (the 16 rows of one MFMA block); a
+// scope of more than 16 cells (5 x 5) takes a second launch with CELL0 = 16.
+template <typename T, int SH, int SW, int CELL0>
 __global__ __launch_bounds__(kMfBlock, 4) void local_grad_filter_mfma_kernel(
     Geo g, const T* __restrict__ gout, const T* __restrict__ x, const T* __restrict__ rot,
     float* __restrict__ partial, int tiles, int nwg, int csplits, int pitch_x) {
   constexpr int K = 9, CELLS = SH * SW;
   constexpr int kWaves = kMfBlock / 64;
-  static_assert(CELLS <= 16, "one 16-row MFMA block holds the cells");
+  static_assert(CELL0 % 16 == 0 && CELL0 < CELLS && CELLS <= 32, "one or two 16-row MFMA blocks hold the cells");
   static_assert(kMfPix == 16 * kWaves, "one 16-pixel group per wave");
   extern __shared__ __align__(16) float lds[];
   float* xs = lds;                                                  // [kMfCh][pitch_x]
@@ -869,7 +882,8 @@ __global__ __launch_bounds__(kMfBlock, 4) void local_grad_filter_mfma_kernel(
   const int row_step = g.dil_h * W;               // elements between two tap rows
   const int lo = -g.pad_h * W - 1;                // first staged input element, relative to the tile
   const int xt = kMfPix + 2 + 2 * row_step;       // staged input elements per channel
-  const float ci = q < CELLS ? float(q / SW) : 64.f, cj = float(q % SW);  // rows 9..15 of a 3x3 scope stay 0
+  // rows past the last cell (9..15 of a 3 x 3 scope, 25..31 of a 5 x 5 one) stay 0
+  const float ci = CELL0 + q < CELLS ? float((CELL0 + q) / SW) : 64.f, cj = float((CELL0 + q) % SW);
 
   for (int e = threadIdx.x; e < nblk * 256; e += kMfBlock) accs[e] = 0.f;
 
@@ -1063,7 +1077,7 @@ __global__ __launch_bounds__(kMfBlock, 4) void local_grad_filter_mfma_kernel(
   __syncthreads();
   for (int e = threadIdx.x; e < nblk * 256; e += kMfBlock) {
     const int b = e / 256, l = (e % 256) / 4, r = e % 4;
-    const int cell = 4 * (l / 16) + r, cj_ = (cb_lo + b) * kMfCh + l % 16;
+    const int cell = CELL0 + 4 * (l / 16) + r, cj_ = (cb_lo + b) * kMfCh + l % 16;
     if (cell < CELLS && cj_ < cpg)
       partial[((size_t)wg * g.channel + grp + (size_t)g.groups * cj_) * CELLS + cell] = accs[e];
   }
@@ -1243,7 +1257,7 @@ FilterGrid filter_grid(const Geo& g) {
   f.mfma = false;
   f.pitch_x = 0;
   f.lds = 0;
-  if (same_width_geometry(g) && g.scope_h * g.scope_w <= 16 && !path_disabled("DK_NO_MFMA")) {
+  if (same_width_geometry(g) && !path_disabled("DK_NO_MFMA")) {
     const long xt = kMfPix + 2 + 2L * g.dil_h * g.in_w;
     const long pitch = (xt + 51 + 63) / 64 * 64;  // rows 64 floats apart plus the skew of mf_row() (at most 51)
     const int nblk = ceil_div(cpg, kMfCh);
@@ -1279,17 +1293,18 @@ FilterGrid filter_grid(const Geo& g) {
 template <typename T, int SH, int SW>
 bool run_grad_filter(const Geo& g, const T* gout, const T* x, const T* rot, T* gfilter, float* ws,
                      hipStream_t stream) {
-  if constexpr (SH * SW > 16) {
-    return false;
-  } else {
+  {
     const FilterGrid f = filter_grid(g);
     const unsigned grid = (unsigned)xcd_grid_size((long)f.parts * f.splits * g.groups);
     if (f.mfma) {
-      local_grad_filter_mfma_kernel<T, SH, SW><<<grid, kMfBlock, f.lds, stream>>>(g, gout, x, rot, ws, f.tiles, f.parts, f.splits, f.pitch_x);
+      local_grad_filter_mfma_kernel<T, SH, SW, 0><<<grid, kMfBlock, f.lds, stream>>>(g, gout, x, rot, ws, f.tiles, f.parts, f.splits, f.pitch_x);
+      if constexpr (SH * SW > 16)  // cells 16 .. 24 of a 5 x 5 scope: the other slice of the same partials
+        local_grad_filter_mfma_kernel<T, SH, SW, 16><<<grid, kMfBlock, f.lds, stream>>>(g, gout, x, rot, ws, f.tiles, f.parts, f.splits, f.pitch_x);
       launch_reduce_partials<float, T>(ws, f.parts, g.channel * SH * SW, gfilter, stream);
       return true;
     }
-    const size_t lds = ((size_t)(kBlock / 64) * f.per * 16 + (size_t)(kBlock / 64) * 64 * 20) * sizeof(float);
+    const size_t lds = ((size_t)(kBlock / 64) * f.per * filter_slots(SH * SW) +
+                        (size_t)(kBlock / 64) * 64 * filter_pitch(SH * SW)) * sizeof(float);
     if (same_width_geometry(g))
       local_grad_filter_kernel<T, 3, 3, SH, SW, 1><<<grid, row_block(g.out_h * g.out_w, kRowLanes), lds, stream>>>(g, gout, x, rot, ws, f.tiles, f.per, f.parts);
     else if (stride2_geometry(g))
@@ -1344,14 +1359,14 @@ size_t fast_local_grad_rotation_workspace(const Geo& g) {
 }
 
 size_t fast_local_grad_filter_workspace(const Geo& g) {
-  if (!fast_shape(g) || g.scope_h * g.scope_w > 16) return 0;
+  if (!fast_shape(g)) return 0;
   return (size_t)filter_grid(g).parts * g.channel * g.scope_h * g.scope_w * sizeof(float);
 }
 
 template <typename T>
 bool fast_local_grad_filter(const Geo& g, const T* gout, const T* x, const T* rot, T* gfilter,
                             void* ws, hipStream_t stream) {
-  if (!fast_shape(g) || g.scope_h * g.scope_w > 16) return false;
+  if (!fast_shape(g)) return false;
 #define CALL(SH, SW) run_grad_filter<T, SH, SW>(g, gout, x, rot, gfilter, static_cast<float*>(ws), stream)
   DK_DISPATCH_SCOPE(g, CALL)
 #undef CALL
