@@ -849,14 +849,14 @@ __device__ __forceinline__ int mf_row(int j, int pitch_x) { return j * pitch_x +
 __device__ __forceinline__ float hat(float d) { return __builtin_amdgcn_fmed3f(1.f - fabsf(d), 0.f, 1.f); }
 
 // CELL0: the kernel sums the scope cells CELL0 .. CELL0 + 15 (the 16 rows of one MFMA block); a
-// scope of more than 16 cells (5 x 5) takes a second launch with CELL0 = 16.
+// scope of more than 16 cells takes further launches (5 x 5: CELL0 = 16; 7 x 7: 16, 32, 48).
 template <typename T, int SH, int SW, int CELL0>
 __global__ __launch_bounds__(kMfBlock, 4) void local_grad_filter_mfma_kernel(
     Geo g, const T* __restrict__ gout, const T* __restrict__ x, const T* __restrict__ rot,
     float* __restrict__ partial, int tiles, int nwg, int csplits, int pitch_x) {
   constexpr int K = 9, CELLS = SH * SW;
   constexpr int kWaves = kMfBlock / 64;
-  static_assert(CELL0 % 16 == 0 && CELL0 < CELLS && CELLS <= 32, "one or two 16-row MFMA blocks hold the cells");
+  static_assert(CELL0 % 16 == 0 && CELL0 < CELLS, "the cells come in slices of 16, the rows of one MFMA block");
   static_assert(kMfPix == 16 * kWaves, "one 16-pixel group per wave");
   extern __shared__ __align__(16) float lds[];
   float* xs = lds;                                                  // [kMfCh][pitch_x]
@@ -1298,11 +1298,19 @@ bool run_grad_filter(const Geo& g, const T* gout, const T* x, const T* rot, T* g
     const unsigned grid = (unsigned)xcd_grid_size((long)f.parts * f.splits * g.groups);
     if (f.mfma) {
       local_grad_filter_mfma_kernel<T, SH, SW, 0><<<grid, kMfBlock, f.lds, stream>>>(g, gout, x, rot, ws, f.tiles, f.parts, f.splits, f.pitch_x);
-      if constexpr (SH * SW > 16)  // cells 16 .. 24 of a 5 x 5 scope: the other slice of the same partials
+      // the further 16-cell slices of a larger scope, into the same partials
+      if constexpr (SH * SW > 16)
         local_grad_filter_mfma_kernel<T, SH, SW, 16><<<grid, kMfBlock, f.lds, stream>>>(g, gout, x, rot, ws, f.tiles, f.parts, f.splits, f.pitch_x);
+      if constexpr (SH * SW > 32)
+        local_grad_filter_mfma_kernel<T, SH, SW, 32><<<grid, kMfBlock, f.lds, stream>>>(g, gout, x, rot, ws, f.tiles, f.parts, f.splits, f.pitch_x);
+      if constexpr (SH * SW > 48)
+        local_grad_filter_mfma_kernel<T, SH, SW, 48><<<grid, kMfBlock, f.lds, stream>>>(g, gout, x, rot, ws, f.tiles, f.parts, f.splits, f.pitch_x);
       launch_reduce_partials<float, T>(ws, f.parts, g.channel * SH * SW, gfilter, stream);
       return true;
     }
+    if constexpr (SH * SW > 32) {
+      return false;  // the dense kernel's fold holds two cells per lane: a 7 x 7 scope goes to the generic kernel
+    } else {
     const size_t lds = ((size_t)(kBlock / 64) * f.per * filter_slots(SH * SW) +
                         (size_t)(kBlock / 64) * 64 * filter_pitch(SH * SW)) * sizeof(float);
     if (same_width_geometry(g))
@@ -1313,6 +1321,7 @@ bool run_grad_filter(const Geo& g, const T* gout, const T* x, const T* rot, T* g
       local_grad_filter_kernel<T, 3, 3, SH, SW, 0><<<grid, kBlock, lds, stream>>>(g, gout, x, rot, ws, f.tiles, f.per, f.parts);
     launch_reduce_partials<float, T>(ws, f.parts, g.channel * SH * SW, gfilter, stream);
     return true;
+    }
   }
 }
 
@@ -1324,7 +1333,7 @@ bool fast_shape(const Geo& g) {
   return g.k_h == 3 && g.k_w == 3 && max_blocks < (1L << 31) - 8 &&
          (long)g.in_h * g.in_w < plane_limit && (long)g.out_h * g.out_w < plane_limit &&
          ((g.scope_h == 4 && g.scope_w == 4) || (g.scope_h == 3 && g.scope_w == 3) ||
-          (g.scope_h == 5 && g.scope_w == 5));
+          (g.scope_h == 5 && g.scope_w == 5) || (g.scope_h == 7 && g.scope_w == 7));
 }
 
 }  // namespace
@@ -1332,7 +1341,8 @@ bool fast_shape(const Geo& g) {
 #define DK_DISPATCH_SCOPE(g, CALL)                                   \
   if ((g).scope_h == 4) return CALL(4, 4);                           \
   if ((g).scope_h == 3) return CALL(3, 3);                           \
-  return CALL(5, 5);
+  if ((g).scope_h == 5) return CALL(5, 5);                           \
+  return CALL(7, 7);
 
 template <typename T>
 bool fast_local_gather(const Geo& g, bool transposed, const T* src, const T* rot, const T* filter,
@@ -1360,7 +1370,11 @@ size_t fast_local_grad_rotation_workspace(const Geo& g) {
 
 size_t fast_local_grad_filter_workspace(const Geo& g) {
   if (!fast_shape(g)) return 0;
-  return (size_t)filter_grid(g).parts * g.channel * g.scope_h * g.scope_w * sizeof(float);
+  const FilterGrid f = filter_grid(g);
+  // more than 32 cells outside the matrix-core kernel's geometry: run_grad_filter() declines, and
+  // the caller sizes the workspace for the generic kernel
+  if (!f.mfma && g.scope_h * g.scope_w > 32) return 0;
+  return (size_t)f.parts * g.channel * g.scope_h * g.scope_w * sizeof(float);
 }
 
 template <typename T>
