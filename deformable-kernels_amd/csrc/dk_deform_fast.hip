@@ -19,6 +19,9 @@
 // corner).  Planes are double buffered: the next channel's plane is loaded into registers before
 // the current channel is computed and written to the other buffer afterwards (one barrier per
 // channel).  The scope tiles of the chunk sit in LDS in the corner-expanded difference form.
+// Where LDS has room (planes up to about 28 x 28) forward, grad offset and grad rotation interleave
+// four channel planes, element e of channel c at [e][c]: the corner gathers at per-lane addresses
+// bound these kernels, and one 16-byte read per corner then serves four channels.
 #include <algorithm>
 #include <cstdlib>
 
@@ -203,6 +206,141 @@ __global__ __launch_bounds__(kDBlock, 2) void deform_forward_kernel(
   }
 }
 
+// The same with CH channel planes interleaved in LDS, element e of channel c at [e][c]: a corner
+// of a sample is one 16-byte read for CH = 4 channels instead of four 4-byte reads, and the
+// gathers at per-lane addresses are what bounds these kernels.
+template <typename T, int NPASS, int CH>
+struct PlaneStageN {
+  float v[CH][NPASS];
+  __device__ __forceinline__ void load(const T* plane0, size_t step, int live_channels, int H, int W, int shift) {
+    const int col = threadIdx.x & ((1 << shift) - 1), sub = threadIdx.x >> shift;
+    const int rpp = (int)blockDim.x >> shift;
+#pragma unroll
+    for (int c = 0; c < CH; ++c) {
+      const bool on = c < live_channels;
+      const rsrc_t r = plane_rsrc(plane0 + (on ? (size_t)c * step : 0), on ? H * W : 0);
+#pragma unroll
+      for (int k = 0; k < NPASS; ++k) {
+        const int row = k * rpp + sub;
+        v[c][k] = buf_ld(r, (col < W && row < H) ? (unsigned)(row * W + col) * (unsigned)sizeof(T) : kOutOfRange, plane0);
+      }
+    }
+  }
+  __device__ __forceinline__ void store(float* lds_planes, int H, int W, int shift) const {
+    const int col = threadIdx.x & ((1 << shift) - 1), sub = threadIdx.x >> shift;
+    const int rpp = (int)blockDim.x >> shift;
+    const int RS = W + 2;
+#pragma unroll
+    for (int k = 0; k < NPASS; ++k) {
+      const int row = k * rpp + sub;
+      if (col < W && row < H) {
+        float* dst = lds_planes + ((row + 1) * RS + 1 + col) * CH;
+        if constexpr (CH == 4) {
+          *reinterpret_cast<float4*>(dst) = make_float4(v[0][k], v[1][k], v[2][k], v[3][k]);
+        } else {
+#pragma unroll
+          for (int c = 0; c < CH; ++c) dst[c] = v[c][k];
+        }
+      }
+    }
+  }
+};
+
+template <int CH>
+struct CornersN {
+  float a[CH], b[CH], c[CH], d[CH];
+};
+template <int CH>
+__device__ __forceinline__ CornersN<CH> read_corners_n(const float* planes, int pidx_ch, int RS) {
+  CornersN<CH> q;
+  const float* p0 = planes + pidx_ch;
+  const float* p1 = p0 + RS * CH;
+  static_assert(CH == 4 || CH == 2, "16-byte or 8-byte corner reads");
+  if constexpr (CH == 4) {
+    const float4 a = *reinterpret_cast<const float4*>(p0), b = *reinterpret_cast<const float4*>(p0 + 4);
+    const float4 c = *reinterpret_cast<const float4*>(p1), d = *reinterpret_cast<const float4*>(p1 + 4);
+    q.a[0] = a.x; q.a[1] = a.y; q.a[2] = a.z; q.a[3] = a.w;
+    q.b[0] = b.x; q.b[1] = b.y; q.b[2] = b.z; q.b[3] = b.w;
+    q.c[0] = c.x; q.c[1] = c.y; q.c[2] = c.z; q.c[3] = c.w;
+    q.d[0] = d.x; q.d[1] = d.y; q.d[2] = d.z; q.d[3] = d.w;
+  } else {
+    const float2 a = *reinterpret_cast<const float2*>(p0), b = *reinterpret_cast<const float2*>(p0 + 2);
+    const float2 c = *reinterpret_cast<const float2*>(p1), d = *reinterpret_cast<const float2*>(p1 + 2);
+    q.a[0] = a.x; q.a[1] = a.y; q.b[0] = b.x; q.b[1] = b.y;
+    q.c[0] = c.x; q.c[1] = c.y; q.d[0] = d.x; q.d[1] = d.y;
+  }
+  return q;
+}
+
+template <typename T, int SH, int SW, int NPASS, int CH>
+__global__ __launch_bounds__(kDBlock, 2) void deform_forward_ch_kernel(
+    Geo g, const T* __restrict__ x, const T* __restrict__ off, const T* __restrict__ rot,
+    const T* __restrict__ filter, T* __restrict__ out, int ch_per_block, int shift) {
+  using Tb = WideTable<SH, SW>;
+  extern __shared__ __align__(16) float lds[];
+  const int H = g.in_h, W = g.in_w, RS = W + 2;
+  const int PS = ((H + 2) * RS + 3) & ~3;
+  float* planes = lds;                // [2][PS][CH]
+  float* tbl = lds + 2 * PS * CH;     // [ch_per_block rounded up to CH][Tb::SIZE]
+
+  const int cpg = g.channel / g.groups;
+  const int out_plane = g.out_h * g.out_w, in_plane = H * W;
+  const BlockId b = decode_block(g, ceil_div(out_plane, kDBlock), ceil_div(cpg, ch_per_block));
+  if (!b.valid) return;
+  const int j0 = b.chunk * ch_per_block;
+  const int nch = min(ch_per_block, cpg - j0);
+  const int nq = ceil_div(nch, CH);
+
+  for (int e = threadIdx.x; e < 2 * PS * CH; e += kDBlock) planes[e] = 0.f;
+  // the tables of the channels that pad the last CH-tuple are read (their products discarded)
+  for (int e = nch * Tb::SIZE + threadIdx.x; e < nq * CH * Tb::SIZE; e += kDBlock) tbl[e] = 0.f;
+  stage_wide_tables<T, SH, SW>(tbl, filter, g.channel, b.grp + g.groups * j0, g.groups, nch);
+
+  const int p = b.tile * kDBlock + threadIdx.x;
+  const bool live = p < out_plane;
+  ImgTap it[K9];
+  LiteTap st[K9];
+  deform_taps<T, SH, SW>(g, off, rot, b.n, b.grp, p, live, RS, it, st);
+#pragma unroll
+  for (int t = 0; t < K9; ++t) it[t].pidx *= CH;
+
+  const size_t chan0 = (size_t)b.n * g.channel + b.grp + (size_t)g.groups * j0;
+  const T* xp = x + chan0 * in_plane;
+  T* op = out + chan0 * out_plane;
+  const size_t x_step = (size_t)g.groups * in_plane, o_step = (size_t)g.groups * out_plane;
+  const unsigned ooff = live ? (unsigned)p * (unsigned)sizeof(T) : kOutOfRange;
+
+  PlaneStageN<T, NPASS, CH> stage;
+  stage.load(xp, x_step, nch, H, W, shift);
+  __syncthreads();  // the zero fill is done
+  stage.store(planes, H, W, shift);
+  __syncthreads();
+  for (int jq = 0; jq < nq; ++jq) {
+    if (jq + 1 < nq) stage.load(xp + (size_t)(jq + 1) * CH * x_step, x_step, nch - (jq + 1) * CH, H, W, shift);
+    const float* pl = planes + (jq & 1) * PS * CH;
+    const float* tb = tbl + jq * CH * Tb::SIZE;
+    float acc[CH];
+#pragma unroll
+    for (int c = 0; c < CH; ++c) acc[c] = 0.f;
+#pragma unroll
+    for (int t = 0; t < K9; ++t) {
+      const CornersN<CH> q = read_corners_n<CH>(pl, it[t].pidx, RS);
+#pragma unroll
+      for (int c = 0; c < CH; ++c) {
+        const float top = fmaf(it[t].lw, q.b[c] - q.a[c], q.a[c]), bot = fmaf(it[t].lw, q.d[c] - q.c[c], q.c[c]);
+        const float v = fmaf(it[t].lh, bot - top, top);
+        const float4 w = *reinterpret_cast<const float4*>(tb + c * Tb::SIZE + st[t].cell);
+        acc[c] = fmaf(v, lite_weight(st[t], w), acc[c]);
+      }
+    }
+#pragma unroll
+    for (int c = 0; c < CH; ++c)
+      buf_st(plane_rsrc(op + (size_t)(jq * CH + c) * o_step, jq * CH + c < nch ? out_plane : 0), ooff, acc[c], out);
+    if (jq + 1 < nq) stage.store(planes + ((jq + 1) & 1) * PS * CH, H, W, shift);
+    __syncthreads();
+  }
+}
+
 
 // ---------------------------------------------------------------------------
 // grad offset / grad rotation: the lane owns output pixel p and sums over the channels of its
@@ -291,6 +429,131 @@ __global__ __launch_bounds__(kDBlock, 2) void deform_grad_coord_kernel(
     }
     gv = gv_next;
     if (j + 1 < nch) stage.store(planes + ((j + 1) & 1) * PS, H, W, shift);
+    __syncthreads();
+  }
+
+  if (live) {
+    const size_t part = ROTATION ? (size_t)b.chunk : (size_t)b.grp * chunks + b.chunk;
+    const size_t img = ROTATION ? (size_t)(b.n * g.groups + b.grp) : (size_t)b.n;
+    const size_t imgs = ROTATION ? (size_t)g.batch * g.groups : (size_t)g.batch;
+    float* dst = partial + ((part * imgs + img) * (K9 * 2)) * out_plane + p;
+    const T* rp = rot + (size_t)(b.n * g.groups + b.grp) * (K9 * 2) * out_plane + p;
+#pragma unroll
+    for (int t = 0; t < K9; ++t) {
+      float dh = ROTATION ? fmaf(st[t].lw, s2[t], s1[t]) : s0[t];
+      float dw = ROTATION ? fmaf(st[t].lh, s2[t], s0[t]) : s1[t];
+      if (ROTATION && g.clip_mode != kClipNone) {  // a clamped offset has no gradient
+        bool open_h, open_w;
+        scope_coord<float>(g, t / 3, ld(rp + (size_t)(2 * t) * out_plane), g.centre_h, &open_h);
+        scope_coord<float>(g, t % 3, ld(rp + (size_t)(2 * t + 1) * out_plane), g.centre_w, &open_w);
+        dh = open_h ? dh : 0.f;
+        dw = open_w ? dw : 0.f;
+      }
+      dst[(size_t)(2 * t) * out_plane] = dh;
+      dst[(size_t)(2 * t + 1) * out_plane] = dw;
+    }
+  }
+}
+
+// The same with CH channel planes interleaved in LDS (see deform_forward_ch_kernel).
+template <typename T, int SH, int SW, int NPASS, bool ROTATION, int CH>
+__global__ __launch_bounds__(kDBlock, 2) void deform_grad_coord_ch_kernel(
+    Geo g, const T* __restrict__ gout, const T* __restrict__ x, const T* __restrict__ off,
+    const T* __restrict__ rot, const T* __restrict__ filter, float* __restrict__ partial,
+    int ch_per_block, int shift) {
+  using Tb = WideTable<SH, SW>;
+  extern __shared__ __align__(16) float lds[];
+  const int H = g.in_h, W = g.in_w, RS = W + 2;
+  const int PS = ((H + 2) * RS + 3) & ~3;
+  float* planes = lds;               // [2][PS][CH]
+  float* tbl = lds + 2 * PS * CH;    // [ch_per_block rounded up to CH][Tb::SIZE]
+
+  const int cpg = g.channel / g.groups;
+  const int out_plane = g.out_h * g.out_w, in_plane = H * W;
+  const int chunks = ceil_div(cpg, ch_per_block);
+  const BlockId b = decode_block(g, ceil_div(out_plane, kDBlock), chunks);
+  if (!b.valid) return;
+  const int j0 = b.chunk * ch_per_block;
+  const int nch = min(ch_per_block, cpg - j0);
+  const int nq = ceil_div(nch, CH);
+
+  for (int e = threadIdx.x; e < 2 * PS * CH; e += kDBlock) planes[e] = 0.f;
+  // the padding channels of the last CH-tuple have gout = 0; their tables must be finite
+  for (int e = nch * Tb::SIZE + threadIdx.x; e < nq * CH * Tb::SIZE; e += kDBlock) tbl[e] = 0.f;
+  stage_wide_tables<T, SH, SW>(tbl, filter, g.channel, b.grp + g.groups * j0, g.groups, nch);
+
+  const int p = b.tile * kDBlock + threadIdx.x;
+  const bool live = p < out_plane;
+  ImgTap it[K9];
+  LiteTap st[K9];
+  deform_taps<T, SH, SW>(g, off, rot, b.n, b.grp, p, live, RS, it, st);
+#pragma unroll
+  for (int t = 0; t < K9; ++t) it[t].pidx *= CH;
+
+  const size_t chan0 = (size_t)b.n * g.channel + b.grp + (size_t)g.groups * j0;
+  const T* xp = x + chan0 * in_plane;
+  const T* gp = gout + chan0 * out_plane;
+  const size_t x_step = (size_t)g.groups * in_plane, g_step = (size_t)g.groups * out_plane;
+  const unsigned goff = live ? (unsigned)p * (unsigned)sizeof(T) : kOutOfRange;
+
+  float s0[K9], s1[K9], s2[K9];
+#pragma unroll
+  for (int t = 0; t < K9; ++t) s0[t] = s1[t] = s2[t] = 0.f;
+
+  PlaneStageN<T, NPASS, CH> stage;
+  float gv[CH], gv_next[CH];
+  stage.load(xp, x_step, nch, H, W, shift);
+#pragma unroll
+  for (int c = 0; c < CH; ++c) gv[c] = buf_ld(plane_rsrc(gp + (size_t)c * g_step, c < nch ? out_plane : 0), goff, gout);
+  __syncthreads();
+  stage.store(planes, H, W, shift);
+  __syncthreads();
+  for (int jq = 0; jq < nq; ++jq) {
+#pragma unroll
+    for (int c = 0; c < CH; ++c) gv_next[c] = 0.f;
+    if (jq + 1 < nq) {
+      const int jn = (jq + 1) * CH;
+      stage.load(xp + (size_t)jn * x_step, x_step, nch - jn, H, W, shift);
+#pragma unroll
+      for (int c = 0; c < CH; ++c)
+        gv_next[c] = buf_ld(plane_rsrc(gp + (size_t)(jn + c) * g_step, jn + c < nch ? out_plane : 0), goff, gout);
+    }
+    const float* pl = planes + (jq & 1) * PS * CH;
+    const float* tb = tbl + jq * CH * Tb::SIZE;
+#pragma unroll
+    for (int t = 0; t < K9; ++t) {
+      const CornersN<CH> cq = read_corners_n<CH>(pl, it[t].pidx, RS);
+#pragma unroll
+      for (int c = 0; c < CH; ++c) {
+        if (ROTATION) {
+          const float top = fmaf(it[t].lw, cq.b[c] - cq.a[c], cq.a[c]), bot = fmaf(it[t].lw, cq.d[c] - cq.c[c], cq.c[c]);
+          const float ps = fmaf(it[t].lh, bot - top, top) * gv[c];
+          const float4 q = lds_read4(tb + c * Tb::SIZE + st[t].cell);
+          s0[t] = fmaf(ps, q.y, s0[t]);
+          s1[t] = fmaf(ps, q.z, s1[t]);
+          s2[t] = fmaf(ps, q.w, s2[t]);
+        } else {
+          const float4 q = *reinterpret_cast<const float4*>(tb + c * Tb::SIZE + st[t].cell);
+          const float gw = gv[c] * lite_weight(st[t], q);
+          const float ca = cq.c[c] - cq.a[c], ba = cq.b[c] - cq.a[c];
+          const float dh = fmaf(it[t].lw, (cq.d[c] - cq.b[c]) - ca, ca);
+          const float dw = fmaf(it[t].lh, (cq.d[c] - cq.c[c]) - ba, ba);
+          s0[t] = fmaf(dh, gw, s0[t]);
+          s1[t] = fmaf(dw, gw, s1[t]);
+        }
+      }
+      // keeps the compiler from issuing every tap's reads first (8 x 16 bytes per tap: registers)
+      // the tap's sums are complete here: without this the compiler sinks the arithmetic of all nine
+      // taps below the plane store and keeps their 9 x 32 loaded values in registers meanwhile
+      if (ROTATION)
+        asm volatile("" : "+v"(s0[t]), "+v"(s1[t]), "+v"(s2[t])::"memory");
+      else
+        asm volatile("" : "+v"(s0[t]), "+v"(s1[t])::"memory");
+      __builtin_amdgcn_sched_barrier(0);
+    }
+#pragma unroll
+    for (int c = 0; c < CH; ++c) gv[c] = gv_next[c];
+    if (jq + 1 < nq) stage.store(planes + ((jq + 1) & 1) * PS * CH, H, W, shift);
     __syncthreads();
   }
 
@@ -783,7 +1046,8 @@ struct DeformPlan {
 
 // table_floats: LDS floats per channel beyond the two planes; plane_floats: LDS floats per plane
 // blocks_per_cu: how many workgroups per CU the channel chunking aims at (measured per kernel on
-// N=64 C=512 28x28 -> 14x14: forward and grad input 4, grad offset and grad filter 3, grad rotation 2)
+// N=64 C=512 28x28 -> 14x14: grad input 4, grad filter 3, the channel-interleaved kernels 3; the
+// one-plane forward 4, grad offset 3, grad rotation 2)
 DeformPlan deform_plan(const Geo& g, int table_floats, int planes, int block, int blocks_per_cu) {
   DeformPlan d{};
   d.ok = false;
@@ -819,9 +1083,31 @@ DeformPlan deform_plan(const Geo& g, int table_floats, int planes, int block, in
   return d;
 }
 
+// Plan of the kernels that interleave kDeformCh channel planes in LDS; ok only when the two
+// interleaved buffers, the tables and a four-pass register stage fit.
+constexpr int kDeformCh = 4;
+
+DeformPlan deform_plan_ch(const Geo& g, int table_floats, int blocks_per_cu) {
+  DeformPlan d{};
+  d.ok = false;
+  if (path_disabled("DK_NO_DEFORM_CH")) return d;
+  d = deform_plan(g, table_floats, 2 * kDeformCh, kDBlock, blocks_per_cu);
+  if (!d.ok) return d;
+  d.lds += (size_t)(kDeformCh - 1) * table_floats * 4;  // tables of the channels that pad the last tuple
+  d.ok = d.npass == 4 && d.lds <= 64 * 1024;
+  return d;
+}
+
 template <typename T, int SH, int SW>
 bool run_deform_forward(const Geo& g, const T* x, const T* off, const T* rot, const T* filter, T* out,
                         hipStream_t stream) {
+  // four channel planes interleaved in LDS while a double buffer of them leaves room for the tables
+  const DeformPlan d4 = deform_plan_ch(g, WideTable<SH, SW>::SIZE, 3);
+  if (d4.ok) {
+    const unsigned grid = (unsigned)xcd_grid_size((long)d4.tiles * d4.chunks * g.batch * g.groups);
+    deform_forward_ch_kernel<T, SH, SW, 4, kDeformCh><<<grid, kDBlock, d4.lds, stream>>>(g, x, off, rot, filter, out, d4.per, d4.shift);
+    return true;
+  }
   const DeformPlan d = deform_plan(g, WideTable<SH, SW>::SIZE, 2, kDBlock, 4);
   if (!d.ok) return false;
   const unsigned grid = (unsigned)xcd_grid_size((long)d.tiles * d.chunks * g.batch * g.groups);
@@ -838,9 +1124,16 @@ bool run_deform_forward(const Geo& g, const T* x, const T* off, const T* rot, co
 template <typename T, int SH, int SW>
 bool run_deform_grad_coord(const Geo& g, bool rotation, const T* gout, const T* x, const T* off, const T* rot,
                            const T* filter, T* result, float* ws, hipStream_t stream) {
-  const DeformPlan d = deform_plan(g, WideTable<SH, SW>::SIZE, 2, kDBlock, rotation ? 2 : 3);
+  const DeformPlan d4 = deform_plan_ch(g, WideTable<SH, SW>::SIZE, 3);
+  const DeformPlan d = d4.ok ? d4 : deform_plan(g, WideTable<SH, SW>::SIZE, 2, kDBlock, rotation ? 2 : 3);
   if (!d.ok) return false;
   const unsigned grid = (unsigned)xcd_grid_size((long)d.tiles * d.chunks * g.batch * g.groups);
+  if (d4.ok) {
+    if (rotation)
+      deform_grad_coord_ch_kernel<T, SH, SW, 4, true, kDeformCh><<<grid, kDBlock, d.lds, stream>>>(g, gout, x, off, rot, filter, ws, d.per, d.shift);
+    else
+      deform_grad_coord_ch_kernel<T, SH, SW, 4, false, kDeformCh><<<grid, kDBlock, d.lds, stream>>>(g, gout, x, off, rot, filter, ws, d.per, d.shift);
+  } else {
 #define DK_LAUNCH(NP, ROT)                                                                          \
   deform_grad_coord_kernel<T, SH, SW, NP, ROT><<<grid, kDBlock, d.lds, stream>>>(g, gout, x, off, rot, filter, ws, \
                                                                                  d.per, d.shift)
@@ -854,6 +1147,7 @@ bool run_deform_grad_coord(const Geo& g, bool rotation, const T* gout, const T* 
     else DK_LAUNCH(16, false);
   }
 #undef DK_LAUNCH
+  }
   const int plane18 = 18 * g.out_h * g.out_w;
   if (rotation)
     launch_reduce_partials<float, T>(ws, d.chunks, g.batch * g.groups * plane18, result, stream);
@@ -960,7 +1254,8 @@ bool fast_deform_grad_coord(const Geo& g, bool rotation, const T* gout, const T*
 
 size_t fast_deform_grad_coord_workspace(const Geo& g, bool rotation) {
   const int table = g.scope_h == 3 ? WideTable<3, 3>::SIZE : g.scope_h == 4 ? WideTable<4, 4>::SIZE : WideTable<5, 5>::SIZE;
-  const DeformPlan d = deform_plan(g, table, 2, kDBlock, rotation ? 2 : 3);
+  const DeformPlan d4 = deform_plan_ch(g, table, 3);
+  const DeformPlan d = d4.ok ? d4 : deform_plan(g, table, 2, kDBlock, rotation ? 2 : 3);
   if (!d.ok) return 0;
   // both lay out chunks * groups * batch planes of 18 * out pixels
   return (size_t)d.chunks * g.groups * g.batch * 18 * g.out_h * g.out_w * sizeof(float);

@@ -29,6 +29,8 @@ CASES = [
     (2, 80, 10, 10, 3, (3, 3), 1, 1, 1, 1, 0.8, 1.0),     # many channels: several channel chunks per image
     (1, 8, 20, 18, 3, (4, 4), 2, 1, 1, 1, 0.5, 6.0),      # large offsets: many samples outside the image
     (2, 10, 40, 36, 3, (4, 4), 1, 1, 1, 2, 0.7, 2.0),     # 1440 output pixels: tiled grad input, 5 channels per group (partial chunk)
+    (2, 27, 14, 14, 3, (4, 4), 2, 1, 1, 1, 0.5, 2.0),     # three chunks of 9 channels: the four-channel tuples end in a single channel
+    (1, 9, 16, 17, 3, (5, 5), 1, 1, 1, 1, 1.0, 2.0),      # scope 5 on the channel-interleaved kernels
 ]
 NAMES = ("forward", "grad input", "grad offset", "grad rotation", "grad filter")
 
