@@ -1031,6 +1031,214 @@ __global__ __launch_bounds__(kDBlock, 2) void deform_grad_filter_kernel(
 }
 
 // ---------------------------------------------------------------------------
+// grad filter on the matrix cores, for input planes small enough that 16 of them fit LDS.
+//
+// With k = (pixel, tap) the sum is a matrix product per block of 16 channels,
+//   gW[cell][c] = sum_k A[cell][k] * P[k][c],
+//   A[cell = (i, j)][k] = hat(sh_k - i) * hat(sw_k - j)          (channel independent),
+//   P[k][c] = sample(x[c], h_k, w_k) * gout[c][pixel_k],
+// and v_mfma_f32_16x16x4_f32 adds a 16 (cells) x 16 (channels) block over four k per issue in
+// full fp32: lane l supplies A[l % 16][l / 16] and P[l / 16][l % 16].  A workgroup of 16 waves owns
+// (image, tile of 256 output pixels) and walks a range of channel blocks; wave w owns pixels
+// 16 w .. 16 w + 15, lane l the four pixels 16 w + 4 (l / 16) .. + 3 on the A side (its 36 hat
+// products stay in registers for all channel blocks) and channel l % 16 on the P side.
+//   * set-up: per (pixel, tap) where the tap samples the padded plane (byte offset, lh, lw) goes to
+//     LDS, read back as one 16-byte broadcast per (lane, pixel, tap);
+//   * per channel block: the 16 input planes are staged zero-padded and channel-interleaved,
+//     position e of channel c at [e][c] with 20 floats per position (a thread owns a position and
+//     writes its 16 channels as four 16-byte stores; with the pitch of 20 the 16 positions of one
+//     store pass hit distinct banks), so the corner reads of the 16 lanes of a pixel quad are 64
+//     contiguous bytes; the gout tile is staged channel-major.  The next block's loads are issued
+//     before the MFMAs and land in registers while they run;
+//   * the waves' 16 x 16 results are added in wave order by 256 owner threads and go out as the
+//     partial of (image, tile): reduce_partials_kernel adds those in order.
+// CELL0: the launch covers the scope cells CELL0 .. CELL0 + 15 (a 5 x 5 scope takes two).
+// ---------------------------------------------------------------------------
+constexpr int kGfBlock = 1024;            // threads per workgroup
+constexpr int kGfPix = 256;               // output pixels per tile
+constexpr int kGfCh = 16;                 // channels per block
+constexpr int kGfPitch = 20;              // floats per position of the interleaved planes
+constexpr int kGfPitchG = kGfPix + 4;     // floats per channel of the gout tile
+
+typedef float gf4 __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ float hat1(float d) { return __builtin_amdgcn_fmed3f(1.f - fabsf(d), 0.f, 1.f); }
+
+template <typename T, int SH, int SW, int CELL0>
+__global__ __launch_bounds__(kGfBlock, 1) void deform_grad_filter_mfma_kernel(
+    Geo g, const T* __restrict__ gout, const T* __restrict__ x, const T* __restrict__ off,
+    const T* __restrict__ rot, float* __restrict__ partial, int tiles, int csplits, int shift) {
+  constexpr int CELLS = SH * SW;
+  constexpr int kWaves = kGfBlock / 64;
+  static_assert(CELL0 % 16 == 0 && CELL0 < CELLS, "the cells come in slices of 16, the rows of one MFMA block");
+  static_assert(kGfPix == 16 * kWaves, "one 16-pixel group per wave");
+  extern __shared__ __align__(16) float lds[];
+  const int H = g.in_h, W = g.in_w, RS = W + 2;
+  const int PS = (H + 2) * RS;
+  float* planes = lds;                                               // [PS][kGfPitch]
+  float* gs = planes + PS * kGfPitch;                                // [kGfCh][kGfPitchG]
+  float4* hwd = reinterpret_cast<float4*>(gs + kGfCh * kGfPitchG);   // [K9][kGfPix] {byte offset, lh, lw, -}
+  float* red = reinterpret_cast<float*>(hwd + K9 * kGfPix);          // [kWaves][256]; set-up: scope coordinates [K9][kGfPix][2]
+  float2* sc = reinterpret_cast<float2*>(red);
+
+  const int cpg = g.channel / g.groups;
+  const int out_plane = g.out_h * g.out_w, in_plane = H * W;
+  const int nblk_all = ceil_div(cpg, kGfCh);
+  const int total = tiles * csplits * g.batch * g.groups;
+  const int lb = logical_block(total);
+  if (lb >= total) return;
+  const int tile = lb % tiles, cs = lb / tiles % csplits;
+  const int n = lb / tiles / csplits / g.groups, grp = lb / tiles / csplits % g.groups;
+  const int blk_per = ceil_div(nblk_all, csplits);
+  const int cb_lo = cs * blk_per, nblk = min(blk_per, nblk_all - cb_lo);
+  if (nblk <= 0) return;
+
+  const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int q = lane & 15, kg = lane >> 4;
+  const int p0 = tile * kGfPix;
+  const int live_pixels = min(kGfPix, out_plane - p0);
+  const int live_waves = ceil_div(live_pixels, 16);
+  const bool wave_live = wave < live_waves;
+
+  // register stage of a channel block: the 16 channels of this thread's plane position, and four
+  // channels of gout at its pixel
+  const int s_col = threadIdx.x & ((1 << shift) - 1), s_row = threadIdx.x >> shift;
+  const bool s_on = s_col < W && s_row < H;
+  const unsigned s_off = s_on ? (unsigned)(s_row * W + s_col) * (unsigned)sizeof(T) : kOutOfRange;
+  const int g_pix = threadIdx.x % kGfPix, g_cq = __builtin_amdgcn_readfirstlane(threadIdx.x / kGfPix);
+  const unsigned g_off = p0 + g_pix < out_plane ? (unsigned)(p0 + g_pix) * (unsigned)sizeof(T) : kOutOfRange;
+  float r_x[kGfCh], r_g[4];
+#define DK_GF_ISSUE(cb)                                                                              \
+  {                                                                                                  \
+    _Pragma("unroll") for (int c = 0; c < kGfCh; ++c) {                                              \
+      const int cj_ = (cb) * kGfCh + c;                                                              \
+      const bool chan = cj_ < cpg;                                                                   \
+      const size_t ci_ = (size_t)n * g.channel + grp + (size_t)g.groups * (chan ? cj_ : 0);          \
+      r_x[c] = buf_ld(plane_rsrc(x + ci_ * in_plane, chan ? in_plane : 0), s_off, x);                \
+    }                                                                                                \
+    _Pragma("unroll") for (int c = 0; c < 4; ++c) {                                                  \
+      const int cj_ = (cb) * kGfCh + g_cq * 4 + c;                                                   \
+      const bool chan = cj_ < cpg;                                                                   \
+      const size_t ci_ = (size_t)n * g.channel + grp + (size_t)g.groups * (chan ? cj_ : 0);          \
+      r_g[c] = buf_ld(plane_rsrc(gout + ci_ * out_plane, chan ? out_plane : 0), g_off, gout);        \
+    }                                                                                                \
+  }
+#define DK_GF_STORE()                                                                                \
+  {                                                                                                  \
+    if (s_on) {                                                                                      \
+      float* dst = planes + ((s_row + 1) * RS + 1 + s_col) * kGfPitch;                               \
+      _Pragma("unroll") for (int c = 0; c < kGfCh; c += 4)                                           \
+        *reinterpret_cast<float4*>(dst + c) = make_float4(r_x[c], r_x[c + 1], r_x[c + 2], r_x[c + 3]); \
+    }                                                                                                \
+    _Pragma("unroll") for (int c = 0; c < 4; ++c) gs[(g_cq * 4 + c) * kGfPitchG + g_pix] = r_g[c];   \
+  }
+
+  DK_GF_ISSUE(cb_lo)
+
+  for (int e = threadIdx.x; e < PS * kGfPitch; e += kGfBlock) planes[e] = 0.f;
+
+  // set-up: this thread's pixel, taps g_cq, g_cq + 4, g_cq + 8 (K.cu:486-500 and 338-341)
+  {
+    const int p = p0 + g_pix;
+    const bool live = p < out_plane;
+    const int pc = live ? p : 0;
+    const int oh = pc / g.out_w, ow = pc % g.out_w;
+    const rsrc_t ro = plane_rsrc(off + (size_t)n * (K9 * 2) * out_plane, K9 * 2 * out_plane);
+    const rsrc_t rr = plane_rsrc(rot + (size_t)(n * g.groups + grp) * (K9 * 2) * out_plane, K9 * 2 * out_plane);
+    const unsigned step = (unsigned)out_plane * (unsigned)sizeof(T);
+#pragma unroll
+    for (int k = 0; k < 3; ++k) {
+      const int t = g_cq + 4 * k;
+      if (t < K9) {
+        const int f_h = t / 3, f_w = t % 3;
+        const unsigned o = live ? (unsigned)((2 * t) * out_plane + pc) * (unsigned)sizeof(T) : kOutOfRange;
+        const float h = float(oh * g.stride_h - g.pad_h + f_h * g.dil_h) + buf_ld(ro, o, off);
+        const float w = float(ow * g.stride_w - g.pad_w + f_w * g.dil_w) + buf_ld(ro, o + step, off);
+        const bool hit = live && (h > -1.f) && (w > -1.f) && (h < float(H)) && (w < float(W));
+        const float hf = floorf(h), wf = floorf(w);
+        const int pidx = hit ? (static_cast<int>(hf) + 1) * RS + static_cast<int>(wf) + 1 : 0;
+        const float sh = scope_coord<float>(g, f_h, buf_ld(rr, o, rot), g.centre_h);
+        const float sw = scope_coord<float>(g, f_w, buf_ld(rr, o + step, rot), g.centre_w);
+        const bool in = hit && (sh > -1.f) && (sw > -1.f) && (sh < float(SH)) && (sw < float(SW));
+        hwd[t * kGfPix + g_pix] =
+            make_float4(__int_as_float(pidx * kGfPitch * 4), hit ? h - hf : 0.f, hit ? w - wf : 0.f, 0.f);
+        sc[t * kGfPix + g_pix] = in ? make_float2(sh, sw) : make_float2(-2.f, -2.f);
+      }
+    }
+  }
+  __syncthreads();
+
+  const int px = wave * 16 + 4 * kg;  // first of this lane's four pixels in the tile
+  // rows past the last cell stay 0
+  const float ci = CELL0 + q < CELLS ? float((CELL0 + q) / SW) : 64.f, cj = float((CELL0 + q) % SW);
+  float A[4][K9];
+#pragma unroll
+  for (int t = 0; t < K9; ++t) {
+    const float4 s01 = *reinterpret_cast<const float4*>(sc + t * kGfPix + px);
+    const float4 s23 = *reinterpret_cast<const float4*>(sc + t * kGfPix + px + 2);
+    A[0][t] = hat1(s01.x - ci) * hat1(s01.y - cj);
+    A[1][t] = hat1(s01.z - ci) * hat1(s01.w - cj);
+    A[2][t] = hat1(s23.x - ci) * hat1(s23.y - cj);
+    A[3][t] = hat1(s23.z - ci) * hat1(s23.w - cj);
+  }
+
+  const size_t part = (size_t)n * tiles + tile;
+  // owner threads: entry e of a block's result is D[cell = CELL0 + 4 * (l / 16) + r][channel l % 16]
+  // with l = e / 4, r = e % 4 (register r of lane l)
+#define DK_GF_FLUSH(cb)                                                                              \
+  if (threadIdx.x < 256) {                                                                           \
+    float s_ = 0.f;                                                                                  \
+    for (int w_ = 0; w_ < live_waves; ++w_) s_ += red[w_ * 256 + threadIdx.x];                       \
+    const int l_ = threadIdx.x / 4, r_ = threadIdx.x % 4;                                            \
+    const int cell_ = CELL0 + 4 * (l_ / 16) + r_, cj_ = (cb) * kGfCh + l_ % 16;                      \
+    if (cell_ < CELLS && cj_ < cpg)                                                                  \
+      partial[(part * g.channel + grp + (size_t)g.groups * cj_) * CELLS + cell_] = s_;               \
+  }
+
+  gf4 acc = {0.f, 0.f, 0.f, 0.f};
+  const unsigned row_bytes = (unsigned)RS * kGfPitch * 4;
+  const char* plane_q = reinterpret_cast<const char*>(planes) + q * 4;
+  for (int i = 0; i < nblk; ++i) {
+    __syncthreads();  // the previous block's reads of the planes, the gout tile and `red` are done
+    DK_GF_STORE()
+    if (i > 0 && wave_live) *reinterpret_cast<gf4*>(red + (wave * 64 + lane) * 4) = acc;
+    __syncthreads();
+    if (i + 1 < nblk) DK_GF_ISSUE(cb_lo + i + 1)
+    if (i > 0) DK_GF_FLUSH(cb_lo + i - 1)
+    if (wave_live) {
+      gf4 acc0 = {0.f, 0.f, 0.f, 0.f}, acc1 = {0.f, 0.f, 0.f, 0.f};
+      const float4 gv = *reinterpret_cast<const float4*>(gs + q * kGfPitchG + px);
+      const float gq[4] = {gv.x, gv.y, gv.z, gv.w};
+#pragma unroll
+      for (int t = 0; t < K9; ++t) {
+#pragma unroll
+        for (int ii = 0; ii < 4; ++ii) {
+          const float4 d = hwd[t * kGfPix + px + ii];
+          const char* c0 = plane_q + __float_as_uint(d.x);
+          const char* c1 = c0 + row_bytes;
+          const float ca = *reinterpret_cast<const float*>(c0), cb_ = *reinterpret_cast<const float*>(c0 + kGfPitch * 4);
+          const float cc = *reinterpret_cast<const float*>(c1), cd = *reinterpret_cast<const float*>(c1 + kGfPitch * 4);
+          const float top = fmaf(d.z, cb_ - ca, ca), bot = fmaf(d.z, cd - cc, cc);
+          const float b = fmaf(d.y, bot - top, top) * gq[ii];
+          if ((ii + t) & 1)
+            acc1 = __builtin_amdgcn_mfma_f32_16x16x4f32(A[ii][t], b, acc1, 0, 0, 0);
+          else
+            acc0 = __builtin_amdgcn_mfma_f32_16x16x4f32(A[ii][t], b, acc0, 0, 0, 0);
+        }
+      }
+      acc = acc0 + acc1;
+    }
+  }
+  __syncthreads();
+  if (wave_live) *reinterpret_cast<gf4*>(red + (wave * 64 + lane) * 4) = acc;
+  __syncthreads();
+  DK_GF_FLUSH(cb_lo + nblk - 1)
+#undef DK_GF_ISSUE
+#undef DK_GF_STORE
+#undef DK_GF_FLUSH
+}
+
+// ---------------------------------------------------------------------------
 // host side
 // ---------------------------------------------------------------------------
 struct DeformPlan {
@@ -1206,9 +1414,57 @@ bool run_deform_grad_input(const Geo& g, const T* gout, const T* off, const T* r
   return true;
 }
 
+// Launch shape of the matrix-core grad filter, ok when the geometry fits it.
+struct GradFilterMfma {
+  bool ok;
+  int tiles, csplits, shift;
+  size_t lds;
+};
+GradFilterMfma grad_filter_mfma_plan(const Geo& g) {
+  GradFilterMfma m{};
+  m.ok = false;
+  if (path_disabled("DK_NO_DEFORM_MFMA")) return m;
+  const DeformPlan basic = deform_plan(g, 64, 0, kGfBlock, 1);  // the family's limits and the row mapping only
+  if (!basic.ok) return m;
+  m.shift = basic.shift;
+  if (g.in_h > (kGfBlock >> m.shift)) return m;  // a thread per plane position
+  const long PS = (long)(g.in_h + 2) * (g.in_w + 2);
+  const long floats = PS * kGfPitch + (long)kGfCh * kGfPitchG + 4L * K9 * kGfPix +
+                      std::max((kGfBlock / 64) * 256, 2 * K9 * kGfPix);
+  if (floats * 4 > 150 * 1024) return m;
+  m.lds = (size_t)floats * 4;
+  m.tiles = ceil_div(g.out_h * g.out_w, kGfPix);
+  const int nblk = ceil_div(g.channel / g.groups, kGfCh);
+  const long base = (long)m.tiles * g.batch * g.groups;
+  m.csplits = (int)std::max<long>(1, std::min<long>(nblk, (512 + base - 1) / base));
+  if (base * m.csplits >= (1L << 31) - 8) return m;
+  m.ok = true;
+  return m;
+}
+
+template <typename T, int SH, int SW, int CELL0>
+bool launch_deform_grad_filter_mfma(const Geo& g, const GradFilterMfma& m, const T* gout, const T* x, const T* off,
+                                    const T* rot, float* ws, hipStream_t stream) {
+  auto kernel = deform_grad_filter_mfma_kernel<T, SH, SW, CELL0>;
+  if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                          (int)m.lds) != hipSuccess)
+    return false;
+  const unsigned grid = (unsigned)xcd_grid_size((long)m.tiles * m.csplits * g.batch * g.groups);
+  kernel<<<grid, kGfBlock, m.lds, stream>>>(g, gout, x, off, rot, ws, m.tiles, m.csplits, m.shift);
+  return true;
+}
+
 template <typename T, int SH, int SW>
 bool run_deform_grad_filter(const Geo& g, const T* gout, const T* x, const T* off, const T* rot, T* gfilter,
                             float* ws, hipStream_t stream) {
+  const GradFilterMfma m = grad_filter_mfma_plan(g);
+  if (m.ok) {
+    if (!launch_deform_grad_filter_mfma<T, SH, SW, 0>(g, m, gout, x, off, rot, ws, stream)) return false;
+    if constexpr (SH * SW > 16)
+      if (!launch_deform_grad_filter_mfma<T, SH, SW, 16>(g, m, gout, x, off, rot, ws, stream)) return false;
+    launch_reduce_partials<float, T>(ws, g.batch * m.tiles, g.channel * SH * SW, gfilter, stream);
+    return true;
+  }
   if constexpr (SH * SW > 16) {
     return false;  // 25 dense accumulators and 90 hat weights per lane do not fit the register budget
   } else {
