@@ -600,8 +600,11 @@ __global__ __launch_bounds__(kDBlock, 2) void deform_grad_coord_ch_kernel(
 // One block per (image, group, channel chunk); blockDim = output pixels rounded up to a wave.
 // The kernel for planes of more than 1024 output pixels further down always uses the 2^-44 grid.
 // ---------------------------------------------------------------------------
-// max |p[i]| into *out (as the bits of a non-negative float, which order like unsigned integers).
-// 16-byte loads, four in flight per thread; p must be 16-byte aligned (the host checks).
+// max |p[i]| over a workgroup's share into out[blockIdx.x] (as the bits of a non-negative float,
+// which order like unsigned integers); the consumer takes the maximum of the kAbsParts words
+// (one atomic maximum per workgroup on a single word cost more than the reads: the atomics on one
+// address serialise).  16-byte loads, four in flight per thread; p must be 16-byte aligned (the
+// host checks).
 template <typename T>
 __global__ __launch_bounds__(256) void absmax_kernel(const T* __restrict__ p, long n, unsigned* __restrict__ out) {
   __shared__ float wave_max[4];
@@ -626,11 +629,23 @@ __global__ __launch_bounds__(256) void absmax_kernel(const T* __restrict__ p, lo
   for (int s = 32; s > 0; s >>= 1) m = fmaxf(m, __shfl_xor(m, s));
   if ((threadIdx.x & 63) == 0) wave_max[threadIdx.x >> 6] = m;
   __syncthreads();
-  // one atomic per block (atomics on one address serialise)
   if (threadIdx.x == 0)
-    atomicMax(out, __float_as_uint(fmaxf(fmaxf(wave_max[0], wave_max[1]), fmaxf(wave_max[2], wave_max[3]))));
+    out[blockIdx.x] = __float_as_uint(fmaxf(fmaxf(wave_max[0], wave_max[1]), fmaxf(wave_max[2], wave_max[3])));
 }
-__global__ void clear_word_kernel(unsigned* p) { *p = 0u; }
+constexpr int kAbsParts = 512;  // workgroups of absmax_kernel = words the consumers reduce
+
+// The maximum of absmax_kernel's words, for every thread of the workgroup (two barriers).
+__device__ __forceinline__ float block_absmax(const unsigned* __restrict__ parts) {
+  __shared__ unsigned s_max;
+  if (threadIdx.x == 0) s_max = 0u;
+  __syncthreads();
+  unsigned m = 0u;
+  for (int i = threadIdx.x; i < kAbsParts; i += blockDim.x) m = max(m, parts[i]);
+  for (int s = 32; s > 0; s >>= 1) m = max(m, (unsigned)__shfl_xor((int)m, s));
+  if ((threadIdx.x & 63) == 0) atomicMax(&s_max, m);
+  __syncthreads();
+  return __uint_as_float(s_max);
+}
 
 // Two channels share a 64-bit sum while at most 2^kPairHead samples touch one input element.
 constexpr int kPairHead = 6;
@@ -722,7 +737,7 @@ __global__ __launch_bounds__(1024) void deform_grad_input_kernel(
   T* ip = gin + chan0 * in_plane;
   const size_t g_step = (size_t)g.groups * out_plane, i_step = (size_t)g.groups * in_plane;
   const unsigned goff = live ? (unsigned)p * (unsigned)sizeof(T) : kOutOfRange;
-  const float gmax = __uint_as_float(*gmax_bits);
+  const float gmax = block_absmax(gmax_bits);
   const int col = threadIdx.x & ((1 << shift) - 1), sub = threadIdx.x >> shift;
   const int rpp = (int)blockDim.x >> shift;
 
@@ -859,7 +874,7 @@ __global__ __launch_bounds__(1024) void deform_grad_input_tiled_kernel(
   }
   __syncthreads();
 
-  const float gmax = __uint_as_float(*gmax_bits);
+  const float gmax = block_absmax(gmax_bits);
   constexpr double kMagic = 6755399441055744.0;  // 1.5 * 2^52
   const size_t chan0 = (size_t)b.n * g.channel + b.grp + (size_t)g.groups * j0;
   const T* gp = gout + chan0 * out_plane;
@@ -1395,9 +1410,8 @@ bool run_deform_grad_input(const Geo& g, const T* gout, const T* off, const T* r
   }
   if (reinterpret_cast<uintptr_t>(gout) % 16 != 0) return false;  // absmax_kernel reads 16-byte vectors
   unsigned* gmax = static_cast<unsigned*>(ws);
-  clear_word_kernel<<<1, 1, 0, stream>>>(gmax);
   const long n = (long)g.batch * g.channel * g.out_h * g.out_w;
-  absmax_kernel<T><<<(unsigned)std::min<long>(1024, (n / (16 / (long)sizeof(T)) + 1023) / 1024 + 1), 256, 0, stream>>>(gout, n, gmax);
+  absmax_kernel<T><<<kAbsParts, 256, 0, stream>>>(gout, n, gmax);
   if (tiled) {
     auto kernel = deform_grad_input_tiled_kernel<T, SH, SW>;
     if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -1529,7 +1543,7 @@ bool fast_deform_grad_input(const Geo& g, const T* gout, const T* off, const T* 
 
 size_t fast_deform_grad_input_workspace(const Geo& g) {
   (void)g;
-  return 256;  // one word: max |gout|
+  return (size_t)kAbsParts * sizeof(unsigned);  // absmax_kernel's per-workgroup maxima of |gout|
 }
 
 template <typename T>
