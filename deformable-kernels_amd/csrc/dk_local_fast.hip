@@ -887,27 +887,20 @@ __global__ __launch_bounds__(kMfBlock, 4) void local_grad_filter_mfma_kernel(
 
   for (int e = threadIdx.x; e < nblk * 256; e += kMfBlock) accs[e] = 0.f;
 
-  // This workgroup's share of the (tile, channel block) units of its group and channel split, as
-  // segments (tile, first block, end block).  Whole tiles are dealt out round-robin, tile t to
-  // workgroup t % nwg, so that neighbouring workgroups (same XCD, same pace) hold neighbouring
-  // tiles of the same channel block at the same time and the halo rows they share are fetched
-  // from memory once; the channel blocks of the last items % nwg tiles are dealt out singly to
-  // keep the load even.
+  // This workgroup's share of the (tile, channel block) units of its group and channel split: a
+  // contiguous range of the units in (tile, block) order, cut into segments (tile, first block,
+  // end block) at the tile boundaries.  Its tiles are neighbours, so the halo rows two tiles share
+  // are fetched from memory once, and a tile's set-up (scope coordinates, hat products) is paid
+  // once per segment -- with fewer tiles than workgroups, once per workgroup.
   const int items = g.batch * tiles;
-  const int whole = items / nwg;                      // whole tiles per workgroup
-  const int rest_units = (items - whole * nwg) * nblk;
-  const int nseg = whole + (rest_units > wg ? (rest_units - wg + nwg - 1) / nwg : 0);
+  const long units = (long)items * nblk;
+  const long u_lo = units * wg / nwg, u_hi = units * (wg + 1) / nwg;
+  const int item_lo = (int)(u_lo / nblk), item_hi = u_hi > u_lo ? (int)((u_hi - 1) / nblk) : item_lo - 1;
+  const int nseg = item_hi - item_lo + 1;
   auto segment = [&](int k, int& item, int& cb_begin, int& cb_end) {
-    if (k < whole) {
-      item = wg + k * nwg;
-      cb_begin = 0;
-      cb_end = nblk;
-    } else {
-      const int r = wg + (k - whole) * nwg;
-      item = whole * nwg + r / nblk;
-      cb_begin = r % nblk;
-      cb_end = cb_begin + 1;
-    }
+    item = item_lo + k;
+    cb_begin = k == 0 ? (int)(u_lo % nblk) : 0;
+    cb_end = item == item_hi ? (int)((u_hi - 1) % nblk) + 1 : nblk;
   };
 
   // Register stage of one unit: what this thread loads (the rotation values of its pixel for
