@@ -836,7 +836,7 @@ constexpr int kMfPix = 128;            // output pixels per tile
 constexpr int kMfCh = 16;              // channels per unit
 constexpr int kMfBlock = 512;          // threads per workgroup
 constexpr int kMfPitchG = kMfPix + 4;  // floats per channel of the gout tile (16-byte reads, bank skew)
-constexpr int kMfX = 6;                // input elements per lane and channel: tile + halo rows <= 64 * kMfX
+constexpr int kMfX = 6;                // at most this many input elements per lane and channel: tile + halo rows <= 64 * kMfX
 constexpr int kMfMaxBlk = 16;          // channel blocks accumulated by one workgroup
 
 typedef float mf4 __attribute__((ext_vector_type(4)));
@@ -850,7 +850,7 @@ __device__ __forceinline__ float hat(float d) { return __builtin_amdgcn_fmed3f(1
 
 // CELL0: the kernel sums the scope cells CELL0 .. CELL0 + 15 (the 16 rows of one MFMA block); a
 // scope of more than 16 cells takes further launches (5 x 5: CELL0 = 16; 7 x 7: 16, 32, 48).
-template <typename T, int SH, int SW, int CELL0>
+template <typename T, int SH, int SW, int CELL0, int NX>
 __global__ __launch_bounds__(kMfBlock, 4) void local_grad_filter_mfma_kernel(
     Geo g, const T* __restrict__ gout, const T* __restrict__ x, const T* __restrict__ rot,
     float* __restrict__ partial, int tiles, int nwg, int csplits, int pitch_x) {
@@ -881,7 +881,6 @@ __global__ __launch_bounds__(kMfBlock, 4) void local_grad_filter_mfma_kernel(
   const int q = lane & 15, kg = lane >> 4;
   const int row_step = g.dil_h * W;               // elements between two tap rows
   const int lo = -g.pad_h * W - 1;                // first staged input element, relative to the tile
-  const int xt = kMfPix + 2 + 2 * row_step;       // staged input elements per channel
   // rows past the last cell (9..15 of a 3 x 3 scope, 25..31 of a 5 x 5 one) stay 0
   const float ci = CELL0 + q < CELLS ? float((CELL0 + q) / SW) : 64.f, cj = float((CELL0 + q) % SW);
 
@@ -910,7 +909,7 @@ __global__ __launch_bounds__(kMfBlock, 4) void local_grad_filter_mfma_kernel(
   constexpr int kTapsT = (K + kMfBlock / kMfPix - 1) / (kMfBlock / kMfPix);  // taps staged per thread
   const int pix = threadIdx.x % kMfPix;                                 // pixel whose coordinates this thread stages
   const int tapq = __builtin_amdgcn_readfirstlane(threadIdx.x / kMfPix);  // ... for taps tapq + 4 k
-  float r_rot[2 * kTapsT], r_x[kChW][kMfX], r_g[kChW][kMfPix / 64];
+  float r_rot[2 * kTapsT], r_x[kChW][NX], r_g[kChW][kMfPix / 64];
   auto issue_loads = [&](int item, int cbi, bool with_rot) {
     const int cb = cb_lo + cbi;
     const int n = item / tiles, p0 = (item % tiles) * kMfPix;
@@ -933,17 +932,14 @@ __global__ __launch_bounds__(kMfBlock, 4) void local_grad_filter_mfma_kernel(
       const size_t c = (size_t)n * g.channel + grp + (size_t)g.groups * (chan ? cj_ : 0);
       const rsrc_t rx = plane_rsrc(x + c * in_plane, chan ? in_plane : 0);
       const rsrc_t rg = plane_rsrc(gout + c * out_plane, chan ? out_plane : 0);
+      // elements before the plane (negative, so huge as unsigned) or past its end fail the buffer's
+      // range check and read 0; the 64 * NX staged elements may run past xt (never read)
 #pragma unroll
-      for (int k = 0; k < kMfX; ++k) {
-        const int i = lane + 64 * k;
-        const long e = (long)p0 + lo + i;
-        r_x[jj][k] = buf_ld(rx, (i < xt && e >= 0 && e < in_plane) ? (unsigned)e * (unsigned)sizeof(T) : kOutOfRange, x);
-      }
+      for (int k = 0; k < NX; ++k)
+        r_x[jj][k] = buf_ld(rx, (unsigned)(p0 + lo + lane + 64 * k) * (unsigned)sizeof(T), x);
 #pragma unroll
-      for (int k = 0; k < kMfPix / 64; ++k) {
-        const int e = p0 + lane + 64 * k;
-        r_g[jj][k] = buf_ld(rg, e < out_plane ? (unsigned)e * (unsigned)sizeof(T) : kOutOfRange, gout);
-      }
+      for (int k = 0; k < kMfPix / 64; ++k)
+        r_g[jj][k] = buf_ld(rg, (unsigned)(p0 + lane + 64 * k) * (unsigned)sizeof(T), gout);
     }
   };
   // Register stage -> LDS.  Scope coordinates: K.cu:338-341 and the band test of K.cu:59.
@@ -971,8 +967,7 @@ __global__ __launch_bounds__(kMfBlock, 4) void local_grad_filter_mfma_kernel(
     for (int jj = 0; jj < kChW; ++jj) {
       const int j = wave + jj * kWaves;
 #pragma unroll
-      for (int k = 0; k < kMfX; ++k)
-        if (lane + 64 * k < xt) xs[mf_row(j, pitch_x) + lane + 64 * k] = r_x[jj][k];
+      for (int k = 0; k < NX; ++k) xs[mf_row(j, pitch_x) + lane + 64 * k] = r_x[jj][k];
 #pragma unroll
       for (int k = 0; k < kMfPix / 64; ++k) gs[j * kMfPitchG + lane + 64 * k] = r_g[jj][k];
     }
@@ -1241,6 +1236,7 @@ struct FilterGrid {
   int per, splits, parts, tiles;
   bool mfma;       // matrix-core kernel: 16 channels per workgroup, 256-pixel tiles
   int pitch_x;     // its floats per channel of the staged input tile
+  int nx;          // its staged input elements per lane and channel (4 or 6)
   size_t lds;      // its LDS bytes
 };
 
@@ -1249,10 +1245,12 @@ FilterGrid filter_grid(const Geo& g) {
   const int cpg = g.channel / g.groups;
   f.mfma = false;
   f.pitch_x = 0;
+  f.nx = 0;
   f.lds = 0;
   if (same_width_geometry(g) && !path_disabled("DK_NO_MFMA")) {
     const long xt = kMfPix + 2 + 2L * g.dil_h * g.in_w;
-    const long pitch = (xt + 51 + 63) / 64 * 64;  // rows 64 floats apart plus the skew of mf_row() (at most 51)
+    // a row holds 64 * nx staged elements (nx = 4 or 6 per lane) plus the skew of mf_row() (at most 51)
+    const long pitch = (xt <= 256 ? 256 : 64 * kMfX) + 64;
     const int nblk = ceil_div(cpg, kMfCh);
     const int csplits = ceil_div(nblk, kMfMaxBlk);
     const long lds = ((long)kMfCh * pitch + (long)kMfCh * kMfPitchG) * 4 + 9L * kMfPix * 8 +
@@ -1260,6 +1258,7 @@ FilterGrid filter_grid(const Geo& g) {
     if (lds <= 64 * 1024 && xt <= 64 * kMfX) {
       f.mfma = true;
       f.pitch_x = (int)pitch;
+      f.nx = xt <= 256 ? 4 : kMfX;
       f.lds = (size_t)lds;
       f.per = kMfCh;
       f.splits = csplits;
@@ -1290,14 +1289,17 @@ bool run_grad_filter(const Geo& g, const T* gout, const T* x, const T* rot, T* g
     const FilterGrid f = filter_grid(g);
     const unsigned grid = (unsigned)xcd_grid_size((long)f.parts * f.splits * g.groups);
     if (f.mfma) {
-      local_grad_filter_mfma_kernel<T, SH, SW, 0><<<grid, kMfBlock, f.lds, stream>>>(g, gout, x, rot, ws, f.tiles, f.parts, f.splits, f.pitch_x);
+#define DK_LAUNCH(CELL0)                                                                                         \
+  if (f.nx == 4)                                                                                                 \
+    local_grad_filter_mfma_kernel<T, SH, SW, CELL0, 4><<<grid, kMfBlock, f.lds, stream>>>(g, gout, x, rot, ws, f.tiles, f.parts, f.splits, f.pitch_x); \
+  else                                                                                                           \
+    local_grad_filter_mfma_kernel<T, SH, SW, CELL0, kMfX><<<grid, kMfBlock, f.lds, stream>>>(g, gout, x, rot, ws, f.tiles, f.parts, f.splits, f.pitch_x);
+      DK_LAUNCH(0)
       // the further 16-cell slices of a larger scope, into the same partials
-      if constexpr (SH * SW > 16)
-        local_grad_filter_mfma_kernel<T, SH, SW, 16><<<grid, kMfBlock, f.lds, stream>>>(g, gout, x, rot, ws, f.tiles, f.parts, f.splits, f.pitch_x);
-      if constexpr (SH * SW > 32)
-        local_grad_filter_mfma_kernel<T, SH, SW, 32><<<grid, kMfBlock, f.lds, stream>>>(g, gout, x, rot, ws, f.tiles, f.parts, f.splits, f.pitch_x);
-      if constexpr (SH * SW > 48)
-        local_grad_filter_mfma_kernel<T, SH, SW, 48><<<grid, kMfBlock, f.lds, stream>>>(g, gout, x, rot, ws, f.tiles, f.parts, f.splits, f.pitch_x);
+      if constexpr (SH * SW > 16) DK_LAUNCH(16)
+      if constexpr (SH * SW > 32) DK_LAUNCH(32)
+      if constexpr (SH * SW > 48) DK_LAUNCH(48)
+#undef DK_LAUNCH
       launch_reduce_partials<float, T>(ws, f.parts, g.channel * SH * SW, gfilter, stream);
       return true;
     }
