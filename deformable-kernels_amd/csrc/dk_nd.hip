@@ -605,6 +605,152 @@ __global__ __launch_bounds__(kBlock) void nd_grad_coord_binned_kernel(NdGeo g, c
     if (d < g.dims) st(gcoord + (long)wv.id * g.dims + d, p.inside ? gd[d] : 0.f);
 }
 
+// Orders LDS writes of a wave before the reads of its other lanes (a wave owns its LDS slice).
+__device__ __forceinline__ void wave_lds_sync() {
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
+typedef float nd4 __attribute__((ext_vector_type(4)));
+
+// grad coord on the sorted points with the sums over the channels on the matrix cores (fp32,
+// channel count a multiple of 64).  With the polynomial coefficients k1 .. k7 of a cell (see
+// nd_grad_coord_binned_kernel) a point's derivatives are
+//   d0 = S1 + f1 S4 + f2 S5 + f1 f2 S7,  d1 = S2 + f0 S4 + f2 S6 + f0 f2 S7,
+//   d2 = S3 + f0 S5 + f1 S6 + f0 f1 S7,       S_m = sum_c gout[c] * k_m[c],
+// and the S_m of 16 points of one cell are a 16 x 64 by 64 x 16 product: v_mfma_f32_16x16x4_f32 with
+// lane l supplying gout[point l % 16][channel 16 (l / 16) + step] and k_{l % 16}[the same channel]
+// over 16 steps (a lane's 16 channels are contiguous: four 16-byte loads of its point's row; the
+// coefficients go through the wave's LDS slice).  The three wave reductions per point and channel
+// block of the VALU kernel (75 VALU instructions per point) become one MFMA per point.
+template <typename T>
+__global__ __launch_bounds__(kBlock) void nd_grad_coord_mfma_kernel(NdGeo g, const float* __restrict__ gout,
+                                                                    const float* __restrict__ data_cl,
+                                                                    const float* __restrict__ coord,
+                                                                    const int* __restrict__ order, int nbins,
+                                                                    float* __restrict__ gcoord) {
+  __shared__ __align__(16) float s_coef[kBlock / 64][8][64];  // [wave][m][channel of the block]
+  __shared__ __align__(16) float s_sum[kBlock / 64][16][16];  // [wave][point of the batch][m]
+  BinnedWave<float> wv;
+  if (!wv.init(g, coord, order, nbins)) return;
+  const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  float(*coef)[64] = s_coef[wave];
+  float(*sums)[16] = s_sum[wave];
+  const bool valid = lane < wv.npts;
+  NdPoint<float> p;
+  p.inside = false;
+#pragma unroll
+  for (int d = 0; d < DK_ND_MAX_DIMS; ++d) p.frac[d] = 0.f, p.low[d] = 0;
+  if (valid) p = load_point<float, float>(g, coord + (long)wv.id * g.dims);
+  const float f0 = p.frac[0], f1 = p.frac[1], f2 = p.frac[2];
+  const float f01 = f0 * f1, f02 = f0 * f2, f12 = f1 * f2;
+  const int pr = lane & 15, kg = lane >> 4;  // MFMA row (point of the batch / coefficient index), K group
+  float gd0 = 0.f, gd1 = 0.f, gd2 = 0.f;     // of point q, in lane q
+
+  int qs = 0;
+  while (qs < wv.npts) {
+    // the run of points in the cell of point qs: the keys are sorted
+    const int key = wv.key_of(qs);
+    const int qe = qs + (int)__popcll(__ballot(wv.key == key));
+    const unsigned present = (unsigned)__builtin_amdgcn_readlane((int)wv.cc.present, qs);
+    nd4 acc[4];
+#pragma unroll
+    for (int b = 0; b < 4; ++b) acc[b] = nd4{0.f, 0.f, 0.f, 0.f};
+    for (int c0 = 0; c0 < g.channel; c0 += 64) {
+      // this lane's 16 channels of its point in batch b: issued two batches ahead of their MFMAs,
+      // the first two before the cell's corner rows, so that the two latencies overlap
+      float av[4][16];
+#define DK_ND_LOAD_A(b)                                                                          \
+  if (qs + 16 * (b) < qe) {                                                                      \
+    const int q_ = qs + 16 * (b) + pr;                                                           \
+    const bool on_ = q_ < qe;                                                                    \
+    const long id_ = __shfl(wv.id, on_ ? q_ : qs);                                               \
+    const float4* rowp_ = reinterpret_cast<const float4*>(gout + id_ * g.channel + c0 + 16 * kg); \
+    _Pragma("unroll") for (int j = 0; j < 4; ++j) {                                              \
+      const float4 t_ = rowp_[j];                                                                \
+      av[b][4 * j] = on_ ? t_.x : 0.f;                                                           \
+      av[b][4 * j + 1] = on_ ? t_.y : 0.f;                                                       \
+      av[b][4 * j + 2] = on_ ? t_.z : 0.f;                                                       \
+      av[b][4 * j + 3] = on_ ? t_.w : 0.f;                                                       \
+    }                                                                                            \
+  }
+#define DK_ND_MFMA(b)                                                                            \
+  if (qs + 16 * (b) < qe) {                                                                      \
+    _Pragma("unroll") for (int s_ = 0; s_ < 16; ++s_)                                            \
+      acc[b] = __builtin_amdgcn_mfma_f32_16x16x4f32(av[b][s_], bv[s_], acc[b], 0, 0, 0);         \
+  }
+      DK_ND_LOAD_A(0)
+      DK_ND_LOAD_A(1)
+      {
+        float v[kClCorners];
+#pragma unroll
+        for (int i = 0; i < kClCorners; ++i)
+          v[i] = (present >> i & 1u) ? data_cl[(size_t)wv.off_of(i, qs) * g.channel + c0 + lane] : 0.f;
+        // corner index: bit d = high side of dimension d
+        const float k1 = v[1] - v[0], k2 = v[2] - v[0], k3 = v[4] - v[0];
+        const float k4 = (v[3] - v[2]) - k1, k5 = (v[5] - v[4]) - k1, k6 = (v[6] - v[4]) - k2;
+        const float k7 = ((v[7] - v[6]) - (v[5] - v[4])) - k4;
+        wave_lds_sync();  // the previous block's coefficient reads are done
+        coef[1][lane] = k1;
+        coef[2][lane] = k2;
+        coef[3][lane] = k3;
+        coef[4][lane] = k4;
+        coef[5][lane] = k5;
+        coef[6][lane] = k6;
+        coef[7][lane] = k7;
+        wave_lds_sync();
+      }
+      float bv[16];
+      {
+        const bool row = pr >= 1 && pr < 8;  // rows 0 and 8 .. 15 of the coefficient matrix are zero
+        const float4* src = reinterpret_cast<const float4*>(&coef[row ? pr : 1][16 * kg]);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const float4 t = src[j];
+          bv[4 * j] = row ? t.x : 0.f;
+          bv[4 * j + 1] = row ? t.y : 0.f;
+          bv[4 * j + 2] = row ? t.z : 0.f;
+          bv[4 * j + 3] = row ? t.w : 0.f;
+        }
+      }
+      DK_ND_MFMA(0)
+      DK_ND_LOAD_A(2)
+      DK_ND_MFMA(1)
+      DK_ND_LOAD_A(3)
+      DK_ND_MFMA(2)
+      DK_ND_MFMA(3)
+#undef DK_ND_LOAD_A
+#undef DK_ND_MFMA
+    }
+    // D[point 4 (l / 16) + r][m = l % 16] in register r of lane l: through LDS to the points' lanes
+#pragma unroll
+    for (int b = 0; b < 4; ++b) {
+      if (qs + 16 * b < qe) {
+        wave_lds_sync();
+#pragma unroll
+        for (int r = 0; r < 4; ++r) sums[4 * kg + r][pr] = acc[b][r];
+        wave_lds_sync();
+        const int mine = lane - (qs + 16 * b);
+        if (mine >= 0 && mine < 16 && lane < qe) {
+          const float4 lo4 = *reinterpret_cast<const float4*>(&sums[mine][0]);
+          const float4 hi4 = *reinterpret_cast<const float4*>(&sums[mine][4]);
+          const float S1 = lo4.y, S2 = lo4.z, S3 = lo4.w, S4 = hi4.x, S5 = hi4.y, S6 = hi4.z, S7 = hi4.w;
+          gd0 += fmaf(f12, S7, fmaf(f2, S5, fmaf(f1, S4, S1)));
+          gd1 += fmaf(f02, S7, fmaf(f2, S6, fmaf(f0, S4, S2)));
+          gd2 += fmaf(f01, S7, fmaf(f1, S6, fmaf(f0, S5, S3)));
+        }
+      }
+    }
+    qs = qe;
+  }
+  if (!valid) return;
+  const float gd[3] = {gd0, gd1, gd2};
+#pragma unroll
+  for (int d = 0; d < kClMaxDims; ++d)
+    if (d < g.dims) gcoord[(long)wv.id * g.dims + d] = p.inside ? gd[d] : 0.f;
+}
+
 template <typename CT>
 __global__ void nd_fill_zero_kernel(CT* p, long n) {
   for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (long)gridDim.x * blockDim.x)
@@ -787,6 +933,7 @@ void nd_grad_data(const dk_nd_desc& d, const T* gout, const T* coord, T* gdata, 
         // chunks of 64 points per wave: as many as keep about 16 waves per CU in the grid
         int per_wave = 1;
         while (per_wave < 8 && g.batch / (64L * per_wave * 2) >= 4096) per_wave *= 2;
+        if (std::getenv("DK_ND_PW")) per_wave = std::atoi(std::getenv("DK_ND_PW"));  // TUNING
         const long waves = (g.batch + 64L * per_wave - 1) / (64L * per_wave);
         nd_grad_data_binned_kernel<T><<<(unsigned)((waves + 3) / 4), kBlock, 0, stream>>>(g, gout, coord, order, bins, acc, per_wave);
       } else {
@@ -816,6 +963,13 @@ void nd_grad_coord(const dk_nd_desc& d, const T* gout, const T* data, const T* c
       transpose<T, T>(data, data_cl, g.channel, g.prod_shape, stream);
       if (const int bins = nd_bins(d)) {
         if (!order) order = sort_points<T>(g, coord, bins, static_cast<char*>(ws) + round256(data_bytes(d) * sizeof(T)), stream);
+        if constexpr (std::is_same<T, float>::value) {
+          // rows of gout are read as 16-byte vectors at multiples of 16 channels
+          if (g.channel % 64 == 0 && reinterpret_cast<uintptr_t>(gout) % 16 == 0 && !path_disabled("DK_NO_ND_MFMA")) {
+            nd_grad_coord_mfma_kernel<T><<<(unsigned)((g.batch + 255) / 256), kBlock, 0, stream>>>(g, gout, data_cl, coord, order, bins, gcoord);
+            return;
+          }
+        }
         nd_grad_coord_binned_kernel<T><<<(unsigned)((g.batch + 255) / 256), kBlock, 0, stream>>>(g, gout, data_cl, coord, order, bins, gcoord);
         return;
       }
