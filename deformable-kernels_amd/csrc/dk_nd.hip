@@ -501,10 +501,35 @@ __global__ __launch_bounds__(kBlock) void nd_grad_data_binned_kernel(NdGeo g, co
           if (q < wv.npts) {
             const int key = wv.key_of(q);
             if (key != cur) {  // wave-uniform: the sums of the finished cell leave
-              DK_FLUSH();
               cur = key;
+              int nat[kClCorners];
+              float nacc[kClCorners];
 #pragma unroll
-              for (int i = 0; i < kClCorners; ++i) acc[i] = 0.f, at[i] = wv.off_of(i, q);
+              for (int i = 0; i < kClCorners; ++i) nacc[i] = 0.f, nat[i] = wv.off_of(i, q);
+              // The next cell in key order is mostly the neighbour along the last dimension, whose
+              // low-side rows are this cell's high-side rows: those sums stay in registers (rows are
+              // matched by their offsets, so any other successor just flushes everything).  Atomics
+              // on the volume are what bounds this kernel; this halves them.
+#define DK_CARRY(HB)                                                                            \
+  _Pragma("unroll") for (int i = 0; i < kClCorners; ++i) {                                      \
+    if ((i & (HB)) && i < 2 * (HB)) {                                                           \
+      if (at[i] == nat[i - (HB)]) {                                                             \
+        nacc[i - (HB)] = acc[i];                                                                \
+        acc[i] = 0.f;                                                                           \
+      }                                                                                         \
+    }                                                                                           \
+  }
+              if (g.dims == 3) {
+                DK_CARRY(4)
+              } else if (g.dims == 2) {
+                DK_CARRY(2)
+              } else {
+                DK_CARRY(1)
+              }
+#undef DK_CARRY
+              DK_FLUSH();
+#pragma unroll
+              for (int i = 0; i < kClCorners; ++i) acc[i] = nacc[i], at[i] = nat[i];
             }
 #pragma unroll
             for (int i = 0; i < kClCorners; ++i) acc[i] += wv.w_of(i, q) * go[u];
@@ -751,6 +776,97 @@ __global__ __launch_bounds__(kBlock) void nd_grad_coord_mfma_kernel(NdGeo g, con
     if (d < g.dims) gcoord[(long)wv.id * g.dims + d] = p.inside ? gd[d] : 0.f;
 }
 
+// grad data on the sorted points on the matrix cores (fp32, channel count a multiple of 64): the
+// sums of a cell's corner rows over the points of a run are a product
+//   D[corner][channel] = sum_p w_corner(p) * gout[p][channel],
+// done 16 points at a time by v_mfma_f32_16x16x4_f32: lane l supplies w_{l % 16}(point 4 step + l / 16)
+// (from the wave's LDS copy of its points' corner weights; rows 8 .. 15 are zero) and the four
+// channels 4 (l % 16) .. + 3 of that point's gout row (one 16-byte load; the 16 lanes of a point read
+// its 256-byte row), one MFMA per channel of the quad.  The VALU kernel spends its time on the
+// per-point broadcasts (v_readlane of eight weights, key and row index per point).
+template <typename T>
+__global__ __launch_bounds__(kBlock) void nd_grad_data_mfma_kernel(NdGeo g, const float* __restrict__ gout,
+                                                                   const float* __restrict__ coord,
+                                                                   const int* __restrict__ order, int nbins,
+                                                                   float* __restrict__ gdata_cl, int per_wave) {
+  __shared__ __align__(16) float s_w[kBlock / 64][64][kClCorners];  // [wave][point][corner]
+  __shared__ __align__(16) float s_d[kBlock / 64][kClCorners][64];  // [wave][corner][channel]
+  const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int pr = lane & 15, kg = lane >> 4, ncorner = 1 << g.dims;
+  float(*wl)[kClCorners] = s_w[wave];
+  float(*dl)[64] = s_d[wave];
+  for (int c0 = 0; c0 < g.channel; c0 += 64) {
+    nd4 acc[4];
+#pragma unroll
+    for (int cb = 0; cb < 4; ++cb) acc[cb] = nd4{0.f, 0.f, 0.f, 0.f};
+    int at[kClCorners];
+#pragma unroll
+    for (int i = 0; i < kClCorners; ++i) at[i] = 0;
+    int cur = -2;
+    // D[corner 4 (l / 16) + r][channel 4 (l % 16) + cb] sits in acc[cb][r] of lane l: through LDS to
+    // one lane per channel, which sends the corner rows' sums
+#define DK_FLUSH()                                                                                   \
+  if (cur != -2) {                                                                                   \
+    wave_lds_sync();                                                                                 \
+    if (kg < 2) {                                                                                    \
+      _Pragma("unroll") for (int r = 0; r < 4; ++r)                                                  \
+        *reinterpret_cast<float4*>(&dl[4 * kg + r][4 * pr]) = make_float4(acc[0][r], acc[1][r], acc[2][r], acc[3][r]); \
+    }                                                                                                \
+    wave_lds_sync();                                                                                 \
+    _Pragma("unroll") for (int i = 0; i < kClCorners; ++i) {                                         \
+      if (i < ncorner) {                                                                             \
+        const float v_ = dl[i][lane];                                                                \
+        if (v_ != 0.f) atomicAdd(gdata_cl + (size_t)at[i] * g.channel + c0 + lane, v_);              \
+      }                                                                                              \
+    }                                                                                                \
+  }
+    // the sums of a cell stay in registers across the wave's chunks: when thousands of points
+    // share a cell, fewer waves send fewer atomics to the same rows
+    for (int sub = 0; sub < per_wave; ++sub) {
+      BinnedWave<float> wv;
+      if (!wv.init(g, coord, order, nbins, per_wave, sub)) break;
+      wave_lds_sync();  // the previous chunk's weight reads are done
+      *reinterpret_cast<float4*>(&wl[lane][0]) = make_float4(wv.cc.w[0], wv.cc.w[1], wv.cc.w[2], wv.cc.w[3]);
+      *reinterpret_cast<float4*>(&wl[lane][4]) = make_float4(wv.cc.w[4], wv.cc.w[5], wv.cc.w[6], wv.cc.w[7]);
+      wave_lds_sync();
+      int qs = 0;
+      while (qs < wv.npts) {
+        const int key = wv.key_of(qs);
+        const int qe = qs + (int)__popcll(__ballot(wv.key == key));  // the keys are sorted
+        if (key != cur) {
+          DK_FLUSH();
+          cur = key;
+#pragma unroll
+          for (int i = 0; i < kClCorners; ++i) at[i] = wv.off_of(i, qs);
+#pragma unroll
+          for (int cb = 0; cb < 4; ++cb) acc[cb] = nd4{0.f, 0.f, 0.f, 0.f};
+        }
+#pragma unroll
+        for (int b = 0; b < 4; ++b) {
+          if (qs + 16 * b < qe) {  // wave-uniform
+#pragma unroll
+            for (int s = 0; s < 4; ++s) {
+              const int q = qs + 16 * b + 4 * s + kg;
+              const bool on = q < qe;
+              const int qc = on ? q : qs;
+              const long id = __shfl(wv.id, qc);
+              const float4 t = *reinterpret_cast<const float4*>(gout + id * g.channel + c0 + 4 * pr);
+              const float a = (on && pr < kClCorners) ? wl[qc][pr & (kClCorners - 1)] : 0.f;
+              acc[0] = __builtin_amdgcn_mfma_f32_16x16x4f32(a, t.x, acc[0], 0, 0, 0);
+              acc[1] = __builtin_amdgcn_mfma_f32_16x16x4f32(a, t.y, acc[1], 0, 0, 0);
+              acc[2] = __builtin_amdgcn_mfma_f32_16x16x4f32(a, t.z, acc[2], 0, 0, 0);
+              acc[3] = __builtin_amdgcn_mfma_f32_16x16x4f32(a, t.w, acc[3], 0, 0, 0);
+            }
+          }
+        }
+        qs = qe;
+      }
+    }
+    DK_FLUSH();
+#undef DK_FLUSH
+  }
+}
+
 template <typename CT>
 __global__ void nd_fill_zero_kernel(CT* p, long n) {
   for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (long)gridDim.x * blockDim.x)
@@ -933,9 +1049,17 @@ void nd_grad_data(const dk_nd_desc& d, const T* gout, const T* coord, T* gdata, 
         // chunks of 64 points per wave: as many as keep about 16 waves per CU in the grid
         int per_wave = 1;
         while (per_wave < 8 && g.batch / (64L * per_wave * 2) >= 4096) per_wave *= 2;
-        if (std::getenv("DK_ND_PW")) per_wave = std::atoi(std::getenv("DK_ND_PW"));  // TUNING
         const long waves = (g.batch + 64L * per_wave - 1) / (64L * per_wave);
-        nd_grad_data_binned_kernel<T><<<(unsigned)((waves + 3) / 4), kBlock, 0, stream>>>(g, gout, coord, order, bins, acc, per_wave);
+        bool on_matrix_cores = false;
+        if constexpr (std::is_same<T, float>::value)
+          // rows of gout are read as 16-byte vectors at multiples of 4 channels
+          on_matrix_cores = g.channel % 64 == 0 && reinterpret_cast<uintptr_t>(gout) % 16 == 0 && !path_disabled("DK_NO_ND_MFMA");
+        if (on_matrix_cores) {
+          if constexpr (std::is_same<T, float>::value)
+            nd_grad_data_mfma_kernel<T><<<(unsigned)((waves + 3) / 4), kBlock, 0, stream>>>(g, gout, coord, order, bins, acc, per_wave);
+        } else {
+          nd_grad_data_binned_kernel<T><<<(unsigned)((waves + 3) / 4), kBlock, 0, stream>>>(g, gout, coord, order, bins, acc, per_wave);
+        }
       } else {
         const int ppw = points_per_wave(g);
         const long waves = (g.batch + ppw - 1) / ppw;
