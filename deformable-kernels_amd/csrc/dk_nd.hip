@@ -867,6 +867,76 @@ __global__ __launch_bounds__(kBlock) void nd_grad_data_mfma_kernel(NdGeo g, cons
   }
 }
 
+// forward on the sorted points on the matrix cores (fp32, channel count a multiple of 64): for the
+// points of a cell run,
+//   out[p][channel] = sum_corner w_corner(p) * row_corner[channel],
+// 16 points at a time: lane l supplies w_{4 step + l / 16}(point l % 16) (from the wave's LDS copy of
+// its points' corner weights) and the channels 4 (l % 16) .. + 3 of corner row 4 step + l / 16 (one
+// 16-byte load per run), two steps of v_mfma_f32_16x16x4_f32 per channel of the quad; the results
+// leave as 16-byte stores, the 16 lanes of a point writing its 256-byte row.
+template <typename T>
+__global__ __launch_bounds__(kBlock) void nd_forward_mfma_kernel(NdGeo g, const float* __restrict__ data_cl,
+                                                                 const float* __restrict__ coord,
+                                                                 const int* __restrict__ order, int nbins,
+                                                                 float* __restrict__ out) {
+  __shared__ __align__(16) float s_w[kBlock / 64][64][kClCorners];  // [wave][point][corner]
+  BinnedWave<float> wv;
+  if (!wv.init(g, coord, order, nbins)) return;
+  const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int pr = lane & 15, kg = lane >> 4;
+  float(*wl)[kClCorners] = s_w[wave];
+  *reinterpret_cast<float4*>(&wl[lane][0]) = make_float4(wv.cc.w[0], wv.cc.w[1], wv.cc.w[2], wv.cc.w[3]);
+  *reinterpret_cast<float4*>(&wl[lane][4]) = make_float4(wv.cc.w[4], wv.cc.w[5], wv.cc.w[6], wv.cc.w[7]);
+  wave_lds_sync();
+  for (int c0 = 0; c0 < g.channel; c0 += 64) {
+    int qs = 0;
+    while (qs < wv.npts) {
+      const int key = wv.key_of(qs);
+      const int qe = qs + (int)__popcll(__ballot(wv.key == key));  // the keys are sorted
+      const unsigned present = (unsigned)__builtin_amdgcn_readlane((int)wv.cc.present, qs);
+      float4 bq[2];
+#pragma unroll
+      for (int s = 0; s < 2; ++s) {
+        const int o0 = wv.off_of(4 * s, qs), o1 = wv.off_of(4 * s + 1, qs), o2 = wv.off_of(4 * s + 2, qs),
+                  o3 = wv.off_of(4 * s + 3, qs);
+        const int o = kg == 0 ? o0 : kg == 1 ? o1 : kg == 2 ? o2 : o3;
+        const bool on = present >> (4 * s + kg) & 1u;
+        const float4 t = *reinterpret_cast<const float4*>(data_cl + (size_t)(on ? o : 0) * g.channel + c0 + 4 * pr);
+        bq[s] = on ? t : make_float4(0.f, 0.f, 0.f, 0.f);
+      }
+#pragma unroll
+      for (int b = 0; b < 4; ++b) {
+        if (qs + 16 * b < qe) {  // wave-uniform
+          const int q = qs + 16 * b + pr;
+          const bool onp = q < qe;
+          const int qc = onp ? q : qs;
+          nd4 acc[4];
+#pragma unroll
+          for (int cb = 0; cb < 4; ++cb) acc[cb] = nd4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+          for (int s = 0; s < 2; ++s) {
+            const float a = onp ? wl[qc][4 * s + kg] : 0.f;
+            acc[0] = __builtin_amdgcn_mfma_f32_16x16x4f32(a, bq[s].x, acc[0], 0, 0, 0);
+            acc[1] = __builtin_amdgcn_mfma_f32_16x16x4f32(a, bq[s].y, acc[1], 0, 0, 0);
+            acc[2] = __builtin_amdgcn_mfma_f32_16x16x4f32(a, bq[s].z, acc[2], 0, 0, 0);
+            acc[3] = __builtin_amdgcn_mfma_f32_16x16x4f32(a, bq[s].w, acc[3], 0, 0, 0);
+          }
+          // D[point 4 (l / 16) + r][channel 4 (l % 16) + cb] in acc[cb][r] of lane l
+#pragma unroll
+          for (int r = 0; r < 4; ++r) {
+            const int qo = qs + 16 * b + 4 * kg + r;
+            const long id = __shfl(wv.id, qo < qe ? qo : qs);
+            if (qo < qe)
+              *reinterpret_cast<float4*>(out + id * g.channel + c0 + 4 * pr) =
+                  make_float4(acc[0][r], acc[1][r], acc[2][r], acc[3][r]);
+          }
+        }
+      }
+      qs = qe;
+    }
+  }
+}
+
 template <typename CT>
 __global__ void nd_fill_zero_kernel(CT* p, long n) {
   for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (long)gridDim.x * blockDim.x)
@@ -1012,6 +1082,13 @@ void nd_forward(const dk_nd_desc& d, const T* data, const T* coord, T* out, void
       transpose<T, T>(data, data_cl, g.channel, g.prod_shape, stream);
       if (const int bins = nd_bins(d)) {
         if (!order) order = sort_points<T>(g, coord, bins, static_cast<char*>(ws) + round256(data_bytes(d) * sizeof(T)), stream);
+        if constexpr (std::is_same<T, float>::value) {
+          // rows of out are written as 16-byte vectors at multiples of 4 channels
+          if (g.channel % 64 == 0 && reinterpret_cast<uintptr_t>(out) % 16 == 0 && !path_disabled("DK_NO_ND_MFMA")) {
+            nd_forward_mfma_kernel<T><<<(unsigned)((g.batch + 255) / 256), kBlock, 0, stream>>>(g, data_cl, coord, order, bins, out);
+            return;
+          }
+        }
         nd_forward_binned_kernel<T><<<(unsigned)((g.batch + 255) / 256), kBlock, 0, stream>>>(g, data_cl, coord, order, bins, out);
         return;
       }
