@@ -58,10 +58,10 @@ OTHER_WORKLOADS = {
 FETCH_SCALE, WRITE_SCALE = 112896.0 / 56469.2, 1.0
 MEASURED_KIB = {
     ("cfg2", "fp32"): {
-        "forward": (64467.1, 134834.0),
-        "grad_input": (64497.7, 134602.0),
-        "grad_rotation": (127217.0, 16623.6),
-        "grad_filter": (122038.0 + 9226.5, 4608.0 + 9.0),  # accumulate kernel + ordered reduce of partials
+        "forward": (64484.9, 135004.0),
+        "grad_input": (64510.5, 134518.0),
+        "grad_rotation": (127256.0, 16606.6),
+        "grad_filter": (122407.0 + 9232.5, 4608.0 + 9.0),  # accumulate kernel + ordered reduce of partials
     },
 }
 

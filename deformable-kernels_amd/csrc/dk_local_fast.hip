@@ -886,20 +886,32 @@ __global__ __launch_bounds__(kMfBlock, 4) void local_grad_filter_mfma_kernel(
 
   for (int e = threadIdx.x; e < nblk * 256; e += kMfBlock) accs[e] = 0.f;
 
-  // This workgroup's share of the (tile, channel block) units of its group and channel split: a
-  // contiguous range of the units in (tile, block) order, cut into segments (tile, first block,
-  // end block) at the tile boundaries.  Its tiles are neighbours, so the halo rows two tiles share
-  // are fetched from memory once, and a tile's set-up (scope coordinates, hat products) is paid
-  // once per segment -- with fewer tiles than workgroups, once per workgroup.
+  // This workgroup's share of the (tile, channel block) units of its group and channel split, as
+  // segments (tile, first block, end block).  Whole tiles are dealt out round-robin, tile t to
+  // workgroup t % nwg, so that neighbouring workgroups (same XCD, same pace) hold neighbouring
+  // tiles of the same channel block at the same time and the halo rows they share are fetched
+  // from memory once (a contiguous range of tiles per workgroup re-fetches them: 1.5 x the reads).
+  // The units of the last items % nwg tiles -- all of them when the tiles are fewer than the
+  // workgroups -- are dealt out as contiguous ranges in (tile, block) order, cut at the tile
+  // boundaries, so that a tile's set-up (scope coordinates, hat products) is paid once per
+  // workgroup and not once per unit.
   const int items = g.batch * tiles;
-  const long units = (long)items * nblk;
-  const long u_lo = units * wg / nwg, u_hi = units * (wg + 1) / nwg;
-  const int item_lo = (int)(u_lo / nblk), item_hi = u_hi > u_lo ? (int)((u_hi - 1) / nblk) : item_lo - 1;
-  const int nseg = item_hi - item_lo + 1;
+  const int whole = items / nwg;                      // whole tiles per workgroup
+  const long rest_units = (long)(items - whole * nwg) * nblk;
+  const long r_lo = rest_units * wg / nwg, r_hi = rest_units * (wg + 1) / nwg;
+  const int rest_lo = (int)(r_lo / nblk), rest_hi = r_hi > r_lo ? (int)((r_hi - 1) / nblk) : rest_lo - 1;
+  const int nseg = whole + (rest_hi - rest_lo + 1);
   auto segment = [&](int k, int& item, int& cb_begin, int& cb_end) {
-    item = item_lo + k;
-    cb_begin = k == 0 ? (int)(u_lo % nblk) : 0;
-    cb_end = item == item_hi ? (int)((u_hi - 1) % nblk) + 1 : nblk;
+    if (k < whole) {
+      item = wg + k * nwg;
+      cb_begin = 0;
+      cb_end = nblk;
+    } else {
+      const int t = rest_lo + (k - whole);
+      item = whole * nwg + t;
+      cb_begin = t == rest_lo ? (int)(r_lo % nblk) : 0;
+      cb_end = t == rest_hi ? (int)((r_hi - 1) % nblk) + 1 : nblk;
+    }
   };
 
   // Register stage of one unit: what this thread loads (the rotation values of its pixel for
