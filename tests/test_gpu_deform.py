@@ -198,6 +198,17 @@ def test_config4_properties_at_full_size():
     assert torch.equal(part.cpu(), out[sl])
 
 
+@pytest.mark.parametrize("switch", ["DK_NO_DEFORM_CH", "DK_NO_DEFORM_MFMA"])
+def test_one_plane_kernels_on_a_shape_the_newer_ones_cover(monkeypatch, switch):
+    """Without the channel-interleaved kernels / the matrix-core grad filter the one-plane kernels serve the shape."""
+    monkeypatch.setenv(switch, "1")
+    inputs, got = _run(CASES[0], torch.float32)
+    o32, o64 = _oracle(inputs, np.float32), _oracle(inputs, np.float64)
+    assert rel_err(got[0], o32[0]) < 1e-5
+    for i in range(1, 5):
+        assert rel_err(got[i], o64[i]) < 1e-4, NAMES[i]
+
+
 def test_generic_kernels_on_a_shape_the_tuned_ones_cover(monkeypatch):
     """With the tuned deformable kernels switched off the generic ones serve the same shape."""
     monkeypatch.setenv("DK_NO_DEFORM_FAST", "1")
