@@ -6,10 +6,10 @@ A "step" is one forward + backward of a DeformKernel2d layer's operator
 batch of synthetic input resident in HBM, issued through the C ABI of
 libdk_hip.so on torch's current stream with preallocated outputs.
 
-Default workload: BASELINE config 2 -- N=64, C=144, 56x56, 3x3 taps, scope 4x4,
+Default workload: benchmark configuration 2 -- N=64, C=144, 56x56, 3x3 taps, scope 4x4,
 stride 1, pad 1, fp32, rotation ~ N(0, 1).
 
-Prints ONE JSON line: the BASELINE metric (achieved HBM GB/s on the
+Prints ONE JSON line: the headline metric (achieved HBM GB/s on the
 algorithmic bytes of the step), a `roofline` object for the dominant kernel
 (timed with events on the launch stream) and a `cpu_baseline` object (the CPU
 oracle, OpenMP, on a bounded slice of the same workload).
@@ -40,7 +40,7 @@ DTYPES = {"fp32": "float32", "bf16": "bfloat16", "fp16": "float16"}
 
 # Other rows of the operator path, timed per entry point with --workload (not the headline metric).
 OTHER_WORKLOADS = {
-    # deformable variant, BASELINE config 4: N, C, H, W, k, S, stride, pad, dil, groups, rot_std, off_std
+    # deformable variant, benchmark configuration 4: N, C, H, W, k, S, stride, pad, dil, groups, rot_std, off_std
     "cfg4": ("deform", (64, 512, 28, 28, 3, (4, 4), 2, 1, 1, 1, 0.5, 2.0)),
     # the deformable variant on the headline layer's shape (3136 output pixels per plane)
     "deform_56": ("deform", (64, 144, 56, 56, 3, (4, 4), 1, 1, 1, 1, 0.5, 2.0)),
@@ -269,7 +269,7 @@ def _time_us(fn, reps):
 
 def other_workload(a):
     """Per-entry-point timing of the deformable variant or the N-d sampler (one JSON line,
-    `metric` says which; these are not the BASELINE headline)."""
+    `metric` says which; these are not the headline)."""
     import torch
     from _cases import make_deform
     from deformable_kernels.ops.deform_kernel import _lib
@@ -351,7 +351,7 @@ def other_workload(a):
         nbytes[name] = nb_
     total_us = sum(v for k_, v in us.items() if "+" not in k_)
     print(json.dumps({
-        "metric": "per-entry-point time (secondary workload, not the BASELINE headline)",
+        "metric": "per-entry-point time (secondary workload, not the headline)",
         "config": {"workload": label},
         "kernel_us": {k_: round(v, 2) for k_, v in us.items()},
         "algorithmic_GBps": {k_: round(nbytes[k_] / (us[k_] * 1e-6) / 1e9, 1) for k_ in us},
@@ -361,7 +361,7 @@ def other_workload(a):
 
 
 # The 17 depthwise 3x3 layers of MobileNetV2 at 224 x 224 (channels, input size, stride), each
-# replaced by DeformKernel2d with a 4 x 4 scope (BASELINE config 5, operator calls only).
+# replaced by DeformKernel2d with a 4 x 4 scope (benchmark configuration 5, operator calls only).
 MBV2_DW_LAYERS = [(32, 112, 1), (96, 112, 2), (144, 56, 1), (144, 56, 2), (192, 28, 1), (192, 28, 1), (192, 28, 2),
                   (384, 14, 1), (384, 14, 1), (384, 14, 1), (384, 14, 1), (576, 14, 1), (576, 14, 1), (576, 14, 2),
                   (960, 7, 1), (960, 7, 1), (960, 7, 1)]
@@ -417,7 +417,7 @@ def layer_workload(a):
 
 def mobilenet_workload(a):
     """Forward + backward of the 17 deformable-kernel depthwise layers of MobileNetV2-DK, operator
-    calls only (one JSON line; secondary to the BASELINE headline)."""
+    calls only (one JSON line; secondary to the headline)."""
     import collections
     import torch
     from _cases import make_local

@@ -18,7 +18,7 @@ pytestmark = pytest.mark.gpu
 
 # N, C, H, W, k, S, stride, pad, dil, groups, rot_std, off_std
 CASES = [
-    (2, 16, 14, 14, 3, (4, 4), 2, 1, 1, 1, 0.5, 2.0),     # BASELINE config 4 geometry, small
+    (2, 16, 14, 14, 3, (4, 4), 2, 1, 1, 1, 0.5, 2.0),     # benchmark configuration 4 geometry, small
     (2, 12, 13, 11, 3, (4, 4), 1, 1, 1, 1, 1.0, 2.0),
     (2, 12, 9, 10, 3, (4, 4), 1, 2, 2, 3, 0.7, 3.0),      # dilation, rotation groups
     (1, 8, 12, 12, 3, (3, 3), 1, 1, 1, 1, 0.0, 1.5),      # DeformConv2d: scope == kernel, zero rotation
@@ -156,7 +156,7 @@ def test_samples_outside_the_image_give_exact_zeros():
 
 
 def test_config4_shape_on_a_batch_slice():
-    """BASELINE config 4 geometry at full channel count (C=512, 28x28 -> 14x14, stride 2) on 4
+    """benchmark configuration 4 geometry at full channel count (C=512, 28x28 -> 14x14, stride 2) on 4
     images: forward and all four gradients against the oracle."""
     case = (4, 512, 28, 28, 3, (4, 4), 2, 1, 1, 1, 0.5, 2.0)
     inputs, got = _run(case, torch.float32)
@@ -167,7 +167,7 @@ def test_config4_shape_on_a_batch_slice():
 
 
 def test_config4_properties_at_full_size():
-    """BASELINE config 4 (N=64, C=512, 28x28 -> 14x14, stride 2, fp32) at full size: the oracle on
+    """benchmark configuration 4 (N=64, C=512, 28x28 -> 14x14, stride 2, fp32) at full size: the oracle on
     two images; the whole batch through properties that need no oracle -- the operator is linear
     in the input and in the filter, so <gout, F> = <grad_input, x> = <grad_filter, Wt>, and it is
     independent per image."""

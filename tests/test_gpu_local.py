@@ -19,7 +19,7 @@ pytestmark = pytest.mark.gpu
 
 # N, C, H, W, k, S, stride, pad, dil, groups, rot_std
 TUNED = [
-    (2, 32, 28, 28, 3, (4, 4), 1, 1, 1, 1, 0.5),    # BASELINE config 1
+    (2, 32, 28, 28, 3, (4, 4), 1, 1, 1, 1, 0.5),    # benchmark configuration 1
     (3, 20, 17, 23, 3, (4, 4), 1, 1, 1, 1, 1.0),    # ragged sizes, partial tiles
     (2, 24, 19, 19, 3, (4, 4), 2, 1, 1, 1, 1.0),    # stride 2
     (2, 12, 15, 14, 3, (4, 4), 1, 2, 2, 3, 1.0),    # dilation 2, rotation groups 3
@@ -172,7 +172,7 @@ def test_runs_on_a_side_stream_and_empty_batch():
 
 
 def test_headline_shape_properties_at_full_size():
-    """BASELINE config 2 (N=64, C=144, 56x56, k=3, scope 4x4, fp32) at full size: the oracle is
+    """benchmark configuration 2 (N=64, C=144, 56x56, k=3, scope 4x4, fp32) at full size: the oracle is
     run on a slice of images; the rest is covered by size-independent properties -- batch
     independence, linearity in the input, and <gout, F(x)> = <grad_input, x>."""
     from deformable_kernels.ops.deform_kernel.functions import sample_depthwise
