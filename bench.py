@@ -95,8 +95,8 @@ def algorithmic_bytes(N, C, H, W, Ho, Wo, k, S, groups, esz):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=50)
-    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=50)
     ap.add_argument("--workload", default="cfg2", choices=sorted(WORKLOADS) + sorted(OTHER_WORKLOADS) + ["mbv2_dk", "layer_cfg2"])
     ap.add_argument("--batch", type=int, default=64, help="batch size of the mbv2_dk workload")
     ap.add_argument("--dtype", default="fp32", choices=sorted(DTYPES))
