@@ -56,7 +56,9 @@ def test_fp32_matches_oracle(shape, C, B):
     ((40,), 16, 66000, -2.0, 42.0),            # one dimension
     ((8, 8, 8), 32, 65536, -1.0, 1.0),         # config 5's coordinate range: every point in the 8 corner cells
     ((6, 5, 4), 64, 65536, 2.2, 2.9),          # every point in one cell
-    ((10, 9), 128, 66000, -1.5, 10.5),         # two dimensions, two 64-channel blocks of the matrix-core grad coord
+    ((10, 9), 128, 66000, -1.5, 10.5),         # two dimensions, two 64-channel blocks of the matrix-core kernels
+    ((50,), 64, 66000, -2.0, 52.0),            # one dimension on the matrix-core kernels
+    ((5, 6, 7), 192, 65536, -1.5, 7.5),        # three 64-channel blocks
 ])
 def test_many_points_per_cell_match_oracle(shape, C, B, lo, hi):
     g = torch.Generator().manual_seed(45)
