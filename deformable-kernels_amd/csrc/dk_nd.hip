@@ -15,8 +15,6 @@
 //  * Direct path (any dimension count, small problems): one lane per (point, channel).
 // The coordinate gradient is reduced over channels inside the kernel instead of
 // materialising the reference's [B, n, C] intermediate (ND.cu:281-286 and the caller's sum).
-#include <rocprim/device/device_radix_sort.hpp>
-#include <rocprim/iterator/counting_iterator.hpp>
 
 #include "dk_kernels.h"
 #include "dk_nd.h"
@@ -375,7 +373,7 @@ __global__ __launch_bounds__(kBlock) void nd_grad_data_cl_kernel(NdGeo g, const 
 //
 // With more points than cells, points that fall into the same cell read (forward, grad coord)
 // or update (grad data) the same 2^n corner rows.  The points are therefore sorted by cell
-// first -- rocPRIM's radix sort of (key, point index) pairs, the key being the cell's low corner,
+// first -- a radix sort of (key, point index) pairs (radix_*_kernel below), the key being the cell's low corner,
 // (low[d] + 1) over extents shape[d] + 1, plus one last bin for the points outside the volume;
 // a radix sort rather than a counting sort with atomics because the points of a real workload
 // may all sit in a handful of cells -- and a wave walks 64
@@ -948,6 +946,155 @@ __global__ void nd_convert_kernel(const CT* __restrict__ a, T* __restrict__ out,
     st(out + i, a[i]);
 }
 
+// ---------------------------------------------------------------------------
+// Sort of the (cell key, point) pairs: a least-significant-digit radix sort in two passes of at
+// most 9 bits (the keys have at most 18), each pass three kernels that launch nothing but
+// themselves (so the sorted path can be captured into a graph):
+//   radix_count_kernel    a workgroup counts the digits of its tile of 4096 keys (LDS atomics) into
+//                         table[digit][workgroup];
+//   radix_scan_*_kernel   exclusive prefix sum of the table in (digit, workgroup) order (per tile of
+//                         4096 entries, then over the tile sums): where each workgroup's keys of each
+//                         digit start in the output;
+//   radix_scatter_kernel  stable scatter.  A wave owns 1024 consecutive keys of the tile, 16 rounds
+//                         of 64; the four waves' starts per digit follow from their counts; within
+//                         a round a lane's rank among the lanes with its digit comes from nine
+//                         ballots, and the first of them advances the wave's LDS counter.
+// ---------------------------------------------------------------------------
+constexpr int kSortTile = 4096, kSortWaveKeys = kSortTile / (kBlock / 64), kSortRounds = kSortWaveKeys / 64;
+constexpr int kSortMaxDigits = 512;
+
+__global__ __launch_bounds__(kBlock) void radix_count_kernel(const unsigned* __restrict__ keys, long n, int shift,
+                                                             int digits, int nblocks, unsigned* __restrict__ table) {
+  __shared__ unsigned h[kSortMaxDigits];
+  for (int d = threadIdx.x; d < digits; d += kBlock) h[d] = 0u;
+  __syncthreads();
+  const long base = (long)blockIdx.x * kSortTile;
+#pragma unroll 4
+  for (int r = 0; r < kSortTile / kBlock; ++r) {
+    const long i = base + r * kBlock + threadIdx.x;
+    if (i < n) atomicAdd(&h[(keys[i] >> shift) & (unsigned)(digits - 1)], 1u);
+  }
+  __syncthreads();
+  for (int d = threadIdx.x; d < digits; d += kBlock) table[(size_t)d * nblocks + blockIdx.x] = h[d];
+}
+
+// Exclusive prefix sum of 1024 values, one per thread of the workgroup; `total` receives their sum.
+__device__ __forceinline__ unsigned block_exclusive_scan(unsigned v, unsigned* wave_sum /* [16] LDS */, unsigned& total) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  unsigned incl = v;
+#pragma unroll
+  for (int step = 1; step < 64; step <<= 1) {
+    const unsigned up = (unsigned)__shfl_up((int)incl, step);
+    if (lane >= step) incl += up;
+  }
+  __syncthreads();  // the previous use of wave_sum is over
+  if (lane == 63) wave_sum[wave] = incl;
+  __syncthreads();
+  unsigned before = 0u, all = 0u;
+#pragma unroll
+  for (int w = 0; w < 16; ++w) {
+    const unsigned t = wave_sum[w];
+    before += w < wave ? t : 0u;
+    all += t;
+  }
+  total = all;
+  return before + incl - v;
+}
+
+// in place, per tile of 4096 entries (a thread owns four consecutive ones); sums[tile] = the tile's sum
+constexpr int kScanTile = 4096;
+__global__ __launch_bounds__(1024) void radix_scan_tiles_kernel(unsigned* __restrict__ table, int total,
+                                                               unsigned* __restrict__ sums) {
+  __shared__ unsigned wave_sum[16];
+  const int i0 = blockIdx.x * kScanTile + 4 * (int)threadIdx.x;
+  unsigned v[4];
+#pragma unroll
+  for (int k = 0; k < 4; ++k) v[k] = i0 + k < total ? table[i0 + k] : 0u;
+  unsigned all;
+  unsigned run = block_exclusive_scan(v[0] + v[1] + v[2] + v[3], wave_sum, all);
+#pragma unroll
+  for (int k = 0; k < 4; ++k) {
+    if (i0 + k < total) table[i0 + k] = run;
+    run += v[k];
+  }
+  if (threadIdx.x == 0) sums[blockIdx.x] = all;
+}
+// exclusive prefix sum of the tile sums, in place: one workgroup walks them 1024 at a time
+__global__ __launch_bounds__(1024) void radix_scan_sums_kernel(unsigned* __restrict__ sums, int count) {
+  __shared__ unsigned wave_sum[16];
+  unsigned carry = 0u;
+  for (int base = 0; base < count; base += 1024) {
+    const int i = base + (int)threadIdx.x;
+    const unsigned v = i < count ? sums[i] : 0u;
+    unsigned all;
+    const unsigned excl = block_exclusive_scan(v, wave_sum, all);
+    if (i < count) sums[i] = carry + excl;
+    carry += all;
+  }
+}
+
+// idx_in == nullptr: the points are still in their own order (index = position);
+// keys_out == nullptr: the keys are not needed after this pass
+__global__ __launch_bounds__(kBlock) void radix_scatter_kernel(const unsigned* __restrict__ keys,
+                                                               const int* __restrict__ idx_in, long n, int shift,
+                                                               int digits, int nblocks,
+                                                               const unsigned* __restrict__ table,
+                                                               const unsigned* __restrict__ tile_start,
+                                                               unsigned* __restrict__ keys_out,
+                                                               int* __restrict__ idx_out) {
+  constexpr int kWaves = kBlock / 64;
+  __shared__ unsigned h[kWaves][kSortMaxDigits];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  for (int e = threadIdx.x; e < kWaves * kSortMaxDigits; e += kBlock) (&h[0][0])[e] = 0u;
+  __syncthreads();
+  const long base = (long)blockIdx.x * kSortTile + (long)wave * kSortWaveKeys;
+  const unsigned mask = (unsigned)(digits - 1);
+  unsigned key[kSortRounds];
+  int idx[kSortRounds];
+#pragma unroll
+  for (int r = 0; r < kSortRounds; ++r) {
+    const long i = base + r * 64 + lane;
+    key[r] = i < n ? keys[i] : 0u;
+    idx[r] = i < n ? (idx_in ? idx_in[i] : (int)i) : 0;
+  }
+#pragma unroll
+  for (int r = 0; r < kSortRounds; ++r)
+    if (base + r * 64 + lane < n) atomicAdd(&h[wave][(key[r] >> shift) & mask], 1u);
+  __syncthreads();
+  // counts -> where each wave's keys of each digit start
+  for (int d = threadIdx.x; d < digits; d += kBlock) {
+    const size_t j = (size_t)d * nblocks + blockIdx.x;
+    unsigned run = table[j] + tile_start[j / kScanTile];
+#pragma unroll
+    for (int w = 0; w < kWaves; ++w) {
+      const unsigned c = h[w][d];
+      h[w][d] = run;
+      run += c;
+    }
+  }
+  __syncthreads();
+#pragma unroll
+  for (int r = 0; r < kSortRounds; ++r) {
+    const bool valid = base + r * 64 + lane < n;
+    const unsigned d = (key[r] >> shift) & mask;
+    // the lanes of this round with the same digit
+    unsigned long long same = __ballot(valid);
+    for (int b = 0; (1 << b) < digits; ++b) {
+      const bool bit = (d >> b) & 1u;
+      const unsigned long long set = __ballot(bit);
+      same &= bit ? set : ~set;
+    }
+    if (valid) {
+      const unsigned rank = (unsigned)__popcll(same & ((1ull << lane) - 1ull));
+      const unsigned pos = h[wave][d] + rank;
+      if (rank == 0u) h[wave][d] += (unsigned)__popcll(same);  // after every lane of the wave has read
+      if (keys_out) keys_out[pos] = key[r];
+      idx_out[pos] = idx[r];
+    }
+    wave_lds_sync();  // the next round reads the counters this round advanced
+  }
+}
+
 inline int grid_for(long total) {
   long b = (total + kBlock - 1) / kBlock;
   if (b > 1048576) b = 1048576;
@@ -1010,33 +1157,22 @@ size_t round256(size_t n) { return (n + 255) / 256 * 256; }
 
 namespace {
 
-// Onesweep radix passes for every size: the keys have few significant bits (two or three 8-bit
-// passes), where rocPRIM's default for up to 2^20 items is a merge sort of ten passes.
-using SortConfig = rocprim::radix_sort_config<rocprim::default_config, rocprim::default_config,
-                                              rocprim::default_config, 0>;
-
 int key_bits(int bins) {
   int bits = 1;
   while ((1L << bits) < bins) ++bits;
   return bits;
 }
 
-// rocPRIM's temporary storage for sorting n (key, index) pairs; 0 if the query fails
-size_t sort_temp_bytes(long n, int bins) {
-  size_t bytes = 0;
-  const hipError_t e = rocprim::radix_sort_pairs<SortConfig>(
-      nullptr, bytes, static_cast<unsigned*>(nullptr), static_cast<unsigned*>(nullptr),
-      rocprim::counting_iterator<int>(0), static_cast<int*>(nullptr), (size_t)n, 0u, (unsigned)key_bits(bins));
-  return e == hipSuccess ? bytes : 0;
-}
-
 }  // namespace
 
-// bytes for the sort: keys, sorted keys, the sorted order of the points, rocPRIM's scratch
+// bytes for the sort: keys, half-sorted keys, the sorted order of the points, the half-sorted order,
+// and the (digit, workgroup) table of the radix passes with its tile sums
 size_t nd_sort_workspace(const dk_nd_desc& d) {
   const int bins = nd_bins(d);
   if (!bins) return 0;
-  return 3 * round256((size_t)d.batch * sizeof(int)) + round256(sort_temp_bytes(d.batch, bins));
+  const size_t n4 = round256((size_t)d.batch * sizeof(int));
+  const size_t table = (size_t)kSortMaxDigits * ((d.batch + kSortTile - 1) / kSortTile);  // entries
+  return 4 * n4 + round256((table + table / kScanTile + 1) * sizeof(unsigned));
 }
 
 size_t nd_data_cl_workspace(const dk_nd_desc& d) {
@@ -1056,11 +1192,29 @@ const int* sort_points(const NdGeo& g, const T* coord, int bins, void* sort_ws, 
   unsigned* keys = reinterpret_cast<unsigned*>(base);
   unsigned* keys_sorted = reinterpret_cast<unsigned*>(base + n4);
   int* order = reinterpret_cast<int*>(base + 2 * n4);
-  void* temp = base + 3 * n4;
   nd_bin_keys_kernel<T><<<(unsigned)((g.batch + kBlock - 1) / kBlock), kBlock, 0, stream>>>(g, coord, bins, keys);
-  size_t temp_bytes = sort_temp_bytes(g.batch, bins);
-  (void)rocprim::radix_sort_pairs<SortConfig>(temp, temp_bytes, keys, keys_sorted, rocprim::counting_iterator<int>(0), order,
-                                  (size_t)g.batch, 0u, (unsigned)key_bits(bins), stream);
+  {
+    // two radix passes of half the key bits each (one pass for keys of up to 9 bits)
+    const int bits = key_bits(bins);
+    const int lo_bits = bits <= 9 ? bits : (bits + 1) / 2, hi_bits = bits - lo_bits;
+    const int nblocks = (int)((g.batch + kSortTile - 1) / kSortTile);
+    int* half_order = reinterpret_cast<int*>(base + 3 * n4);
+    unsigned* table = reinterpret_cast<unsigned*>(base + 4 * n4);
+    unsigned* sums = table + (size_t)kSortMaxDigits * nblocks;
+    auto pass = [&](const unsigned* k_in, const int* i_in, int shift, int nbits, unsigned* k_out, int* i_out) {
+      const int digits = 1 << nbits, total = digits * nblocks, tiles = (total + kScanTile - 1) / kScanTile;
+      radix_count_kernel<<<nblocks, kBlock, 0, stream>>>(k_in, g.batch, shift, digits, nblocks, table);
+      radix_scan_tiles_kernel<<<tiles, 1024, 0, stream>>>(table, total, sums);
+      radix_scan_sums_kernel<<<1, 1024, 0, stream>>>(sums, tiles);
+      radix_scatter_kernel<<<nblocks, kBlock, 0, stream>>>(k_in, i_in, g.batch, shift, digits, nblocks, table, sums, k_out, i_out);
+    };
+    if (hi_bits == 0) {
+      pass(keys, nullptr, 0, lo_bits, nullptr, order);
+    } else {
+      pass(keys, nullptr, 0, lo_bits, keys_sorted, half_order);
+      pass(keys_sorted, half_order, lo_bits, hi_bits, nullptr, order);
+    }
+  }
   return order;
 }
 
