@@ -311,14 +311,22 @@ template <typename T> struct Pair;
 template <> struct Pair<float> {
   typedef float raw __attribute__((ext_vector_type(2), aligned(4)));
   static __device__ __forceinline__ float get(const raw& v, int k) { return v[k]; }
+  static __device__ __forceinline__ raw make(float a, float b) { return raw{a, b}; }
 };
 template <> struct Pair<__half> {
   typedef _Float16 raw __attribute__((ext_vector_type(2), aligned(2)));
   static __device__ __forceinline__ float get(const raw& v, int k) { return static_cast<float>(v[k]); }
+  static __device__ __forceinline__ raw make(float a, float b) { return raw{static_cast<_Float16>(a), static_cast<_Float16>(b)}; }
 };
 template <> struct Pair<bf16_t> {
   typedef unsigned short raw __attribute__((ext_vector_type(2), aligned(2)));
   static __device__ __forceinline__ float get(const raw& v, int k) { return __uint_as_float(static_cast<uint32_t>(v[k]) << 16); }
+  static __device__ __forceinline__ raw make(float a, float b) {
+    bf16_t x, y;
+    st(&x, a);
+    st(&y, b);
+    return raw{x.bits, y.bits};
+  }
 };
 
 template <typename T, int SH, int SW>
@@ -414,6 +422,120 @@ __global__ __launch_bounds__(kBlock, 2) void local_forward_s2_kernel(Geo g, cons
     compute_stage(xa, j);
     load_stage(xa, j + 2 * kUnroll);
     compute_stage(xb, j + kUnroll);
+  }
+}
+
+// ---------------------------------------------------------------------------
+// grad input for the same stride-2 geometry.  The 2 x 2 input quad (2 qh .. + 1, 2 qw .. + 1) is fed
+// by exactly nine (output pixel, tap) pairs of the four output pixels P00 = (qh, qw), P01 = (qh, qw + 1),
+// P10 = (qh + 1, qw), P11 = (qh + 1, qw + 1):
+//   (even, even)  P00 (1,1)
+//   (even, odd)   P00 (1,2)  P01 (1,0)
+//   (odd, even)   P00 (2,1)  P10 (0,1)
+//   (odd, odd)    P00 (2,2)  P01 (2,0)  P10 (0,2)  P11 (0,0)
+// so a lane that owns the quad of output pixel P00 does the forward kernel's nine weights per
+// channel, from two gout loads (its own pixel and the one a row below; the right-hand neighbours
+// come from the next lane through the DPP-fused multiply-add), and every lane has the same work.
+// A gather over input pixels has 1, 2 or 4 taps per lane depending on the pixel's parities
+// (local_gather_kernel<.., true, 4>: 16 tap slots per quad instead of 9).  A wave covers 63 quads
+// with lanes 0 .. 62 plus the halo lane 63.
+// grid = (quad tiles of kS2Pix, channel splits, batch * groups)
+// ---------------------------------------------------------------------------
+template <typename T, int SH, int SW>
+__global__ __launch_bounds__(kBlock, 2) void local_grad_input_s2_kernel(Geo g, const T* __restrict__ gout,
+                                                                        const T* __restrict__ rot,
+                                                                        const T* __restrict__ filter,
+                                                                        T* __restrict__ gin, int ch_per_block) {
+  using Tb = WideTable<SH, SW>;
+  constexpr int K = 9;
+  extern __shared__ __align__(16) float tbl[];
+
+  const int cpg = g.channel / g.groups;
+  const int out_plane = g.out_h * g.out_w, in_plane = g.in_h * g.in_w;
+  const int tiles = ceil_div(out_plane, kS2Pix), splits = ceil_div(cpg, ch_per_block);
+  const int total = tiles * splits * g.batch * g.groups;
+  const int lb = logical_block(total);
+  if (lb >= total) return;
+  const int bx = lb % tiles, by = lb / tiles % splits, bz = lb / tiles / splits;
+  const int n = bz / g.groups, grp = bz % g.groups;
+  const int j0 = by * ch_per_block;
+  const int nch = min(ch_per_block, cpg - j0);
+  stage_wide_tables<T, SH, SW>(tbl, filter, g.channel, grp + g.groups * j0, g.groups, nch);
+
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int p = bx * kS2Pix + wave * kS2Lanes + lane;  // lane 63 is the halo: the quad after the wave's last
+  const bool exists = p < out_plane;
+  const bool owns = lane < kS2Lanes && exists;
+  const int pc = exists ? p : 0;
+  const int qh = pc / g.out_w, qw = pc % g.out_w;
+  const bool right = qw + 1 < g.out_w, below = qh + 1 < g.out_h;
+
+  // the nine (output pixel, tap) pairs in the order of the table above
+  constexpr int kDh[K] = {0, 0, 0, 0, 1, 0, 0, 1, 1}, kDw[K] = {0, 0, 1, 0, 0, 0, 1, 0, 1};
+  constexpr int kTap[K] = {4, 5, 3, 7, 1, 8, 6, 2, 0};
+  LiteTap tap[K];
+  const rsrc_t rr = plane_rsrc(rot + (size_t)(n * g.groups + grp) * (K * 2) * out_plane, K * 2 * out_plane);
+#pragma unroll
+  for (int k = 0; k < K; ++k) {
+    const bool ok = exists && (kDh[k] == 0 || below) && (kDw[k] == 0 || right);
+    const int rp = pc + kDh[k] * g.out_w + kDw[k];
+    const unsigned ro = ok ? (unsigned)((2 * kTap[k]) * out_plane + rp) * (unsigned)sizeof(T) : kOutOfRange;
+    const float r_h = buf_ld(rr, ro, rot);
+    const float r_w = buf_ld(rr, ro + (unsigned)out_plane * (unsigned)sizeof(T), rot);
+    tap[k] = make_lite_tap<SH, SW>(scope_coord<float>(g, kTap[k] / 3, r_h, g.centre_h),
+                                   scope_coord<float>(g, kTap[k] % 3, r_w, g.centre_w), ok);
+  }
+  __syncthreads();
+
+  const size_t chan0 = (size_t)n * g.channel + grp + (size_t)g.groups * j0;
+  const T* sp = gout + chan0 * out_plane;
+  T* dp = gin + chan0 * in_plane;
+  const size_t s_step = (size_t)g.groups * out_plane, d_step = (size_t)g.groups * in_plane;
+  // gout of the lane's pixel (halo lane included: its pixel is the next wave's first) and of the one below
+  const unsigned g0off = exists ? (unsigned)p * (unsigned)sizeof(T) : kOutOfRange;
+  const unsigned g1off = (exists && below) ? (unsigned)(p + g.out_w) * (unsigned)sizeof(T) : kOutOfRange;
+  // the quad's elements: the pairs of rows 2 qh and 2 qh + 1 (the latter may lie past an odd-height plane)
+  typedef typename Pair<T>::raw pair_t;
+  const int d0 = 2 * qh * g.in_w + 2 * qw;
+  const bool row1 = 2 * qh + 1 < g.in_h;
+
+  auto load_stage = [&](float (&gc)[kUnroll][2], int jb) {
+#pragma unroll
+    for (int u = 0; u < kUnroll; ++u) {
+      const rsrc_t rs = plane_rsrc(sp + (size_t)(jb + u) * s_step, (jb + u) < nch ? out_plane : 0);
+      gc[u][0] = buf_ld(rs, g0off, gout);
+      gc[u][1] = buf_ld(rs, g1off, gout);
+    }
+  };
+  auto compute_stage = [&](const float (&gc)[kUnroll][2], int jb) {
+    const float* tb = tbl + jb * Tb::SIZE;
+#pragma unroll
+    for (int u = 0; u < kUnroll; ++u) {
+      float w[K];
+#pragma unroll
+      for (int k = 0; k < K; ++k)
+        w[k] = lite_weight(tap[k], *reinterpret_cast<const float4*>(tb + tap[k].cell + u * Tb::SIZE));
+      const float g0 = gc[u][0], g1 = gc[u][1];
+      const float v00 = g0 * w[0];
+      const float v01 = fma_lane_above(g0, w[2], g0 * w[1]);
+      const float v10 = fmaf(g1, w[4], g0 * w[3]);
+      const float v11 = fma_lane_above(g1, w[8], fmaf(g1, w[7], fma_lane_above(g0, w[6], g0 * w[5])));
+      // one store per row pair (the wave writes 63 contiguous pairs); non-temporal like the other results
+      if (owns && jb + u < nch) {
+        T* plane = dp + (size_t)(jb + u) * d_step + d0;
+        __builtin_nontemporal_store(Pair<T>::make(v00, v01), reinterpret_cast<pair_t*>(plane));
+        if (row1) __builtin_nontemporal_store(Pair<T>::make(v10, v11), reinterpret_cast<pair_t*>(plane + g.in_w));
+      }
+    }
+  };
+
+  float ga[kUnroll][2], gb[kUnroll][2];
+  load_stage(ga, 0);
+  for (int j = 0; j < nch; j += 2 * kUnroll) {
+    load_stage(gb, j + kUnroll);
+    compute_stage(ga, j);
+    load_stage(ga, j + 2 * kUnroll);
+    compute_stage(gb, j + kUnroll);
   }
 }
 
@@ -1190,6 +1312,15 @@ bool run_gather(const Geo& g, bool transposed, const T* src, const T* rot, const
       local_gather_rows_kernel<T, 3, SH, SW, true><<<grid, row_block(pixels, kRowLanes), lds, stream>>>(g, src, rot, filter, dst, per);
     else
       local_gather_rows_kernel<T, 3, SH, SW, false><<<grid, row_block(pixels, kRowLanes), lds, stream>>>(g, src, rot, filter, dst, per);
+    return true;
+  }
+  if (transposed && stride2_geometry(g) && !path_disabled("DK_NO_S2_QUADS")) {
+    // lanes own 2 x 2 input quads, one per output pixel
+    const int quads = g.out_h * g.out_w;
+    const int perq = channels_per_block<SH, SW>(cpg, pick_splits(g, quads));
+    const unsigned gridq = (unsigned)xcd_grid_size((long)ceil_div(quads, kS2Pix) * ceil_div(cpg, perq) * g.batch * g.groups);
+    const size_t ldsq = (size_t)(perq + 2 * kUnroll) * WideTable<SH, SW>::SIZE * sizeof(float);
+    local_grad_input_s2_kernel<T, SH, SW><<<gridq, row_block(quads, kS2Lanes), ldsq, stream>>>(g, src, rot, filter, dst, perq);
     return true;
   }
   const int per = channels_per_block<SH, SW>(cpg, pick_splits(g, pixels));
