@@ -960,6 +960,8 @@ constexpr int kMfBlock = 512;          // threads per workgroup
 constexpr int kMfPitchG = kMfPix + 4;  // floats per channel of the gout tile (16-byte reads, bank skew)
 constexpr int kMfX = 6;                // at most this many input elements per lane and channel: tile + halo rows <= 64 * kMfX
 constexpr int kMfMaxBlk = 16;          // channel blocks accumulated by one workgroup
+constexpr int kMfXS2 = 9;              // stride 2: staged input elements per lane and channel
+constexpr int kMfMaxBlkS2 = 12;        // stride 2: channel blocks per workgroup (two workgroups' LDS fit a CU)
 
 typedef float mf4 __attribute__((ext_vector_type(4)));
 
@@ -972,10 +974,14 @@ __device__ __forceinline__ float hat(float d) { return __builtin_amdgcn_fmed3f(1
 
 // CELL0: the kernel sums the scope cells CELL0 .. CELL0 + 15 (the 16 rows of one MFMA block); a
 // scope of more than 16 cells takes further launches (5 x 5: CELL0 = 16; 7 x 7: 16, 32, 48).
-template <typename T, int SH, int SW, int CELL0, int NX>
+// S2: the stride-2 geometry of local_forward_s2_kernel.  A tile is then `th` whole output rows (at
+// most 128 pixels), so that the input rows its taps read, 2 oh0 - 1 .. 2 (oh0 + th - 1) + 1, are
+// one contiguous range of the plane like the stride-1 tile with its halo rows; a lane's four
+// pixels may sit in different rows, so each reads its own 3 x 3 inputs.
+template <typename T, int SH, int SW, int CELL0, int NX, bool S2>
 __global__ __launch_bounds__(kMfBlock, 4) void local_grad_filter_mfma_kernel(
     Geo g, const T* __restrict__ gout, const T* __restrict__ x, const T* __restrict__ rot,
-    float* __restrict__ partial, int tiles, int nwg, int csplits, int pitch_x) {
+    float* __restrict__ partial, int tiles, int nwg, int csplits, int pitch_x, int th) {
   constexpr int K = 9, CELLS = SH * SW;
   constexpr int kWaves = kMfBlock / 64;
   static_assert(CELL0 % 16 == 0 && CELL0 < CELLS, "the cells come in slices of 16, the rows of one MFMA block");
@@ -996,8 +1002,10 @@ __global__ __launch_bounds__(kMfBlock, 4) void local_grad_filter_mfma_kernel(
   const int blk_per = ceil_div(nblk_all, csplits);
   const int cb_lo = cs * blk_per, nblk = min(blk_per, nblk_all - cb_lo);
 
-  const int W = g.in_w;  // == out_w
-  const int out_plane = g.out_h * W, in_plane = g.in_h * W;
+  const int W = g.in_w;  // == out_w unless S2
+  const int OW = g.out_w;
+  const int out_plane = g.out_h * OW, in_plane = g.in_h * W;
+  const int tile_pix = S2 ? th * OW : kMfPix;  // pixels of a tile (pixel slots past them carry zero weights)
   // the wave index picks channel planes (buffer resources): tell the compiler it is uniform
   const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int q = lane & 15, kg = lane >> 4;
@@ -1046,7 +1054,10 @@ __global__ __launch_bounds__(kMfBlock, 4) void local_grad_filter_mfma_kernel(
   float r_rot[2 * kTapsT], r_x[kChW][NX], r_g[kChW][kMfPix / 64];
   auto issue_loads = [&](int item, int cbi, bool with_rot) {
     const int cb = cb_lo + cbi;
-    const int n = item / tiles, p0 = (item % tiles) * kMfPix;
+    const int n = item / tiles, p0 = (item % tiles) * tile_pix;
+    // first staged input element: the tile's first pixel minus the halo; S2: one element before
+    // input row 2 oh0 - 1 (so that column -1 of a row's first pixel is a valid, unused slot)
+    const int x0 = S2 ? (2 * (item % tiles) * th - 1) * W - 1 : p0 + lo;
     if (with_rot) {
       const int p = p0 + pix;
       const rsrc_t rr = plane_rsrc(rot + (size_t)(n * g.groups + grp) * (K * 2) * out_plane, K * 2 * out_plane);
@@ -1070,7 +1081,7 @@ __global__ __launch_bounds__(kMfBlock, 4) void local_grad_filter_mfma_kernel(
       // range check and read 0; the 64 * NX staged elements may run past xt (never read)
 #pragma unroll
       for (int k = 0; k < NX; ++k)
-        r_x[jj][k] = buf_ld(rx, (unsigned)(p0 + lo + lane + 64 * k) * (unsigned)sizeof(T), x);
+        r_x[jj][k] = buf_ld(rx, (unsigned)(x0 + lane + 64 * k) * (unsigned)sizeof(T), x);
 #pragma unroll
       for (int k = 0; k < kMfPix / 64; ++k)
         r_g[jj][k] = buf_ld(rg, (unsigned)(p0 + lane + 64 * k) * (unsigned)sizeof(T), gout);
@@ -1079,16 +1090,16 @@ __global__ __launch_bounds__(kMfBlock, 4) void local_grad_filter_mfma_kernel(
   // Register stage -> LDS.  Scope coordinates: K.cu:338-341 and the band test of K.cu:59.
   auto store_unit = [&](int item, bool with_rot) {
     if (with_rot) {
-      const int p = (item % tiles) * kMfPix + pix;
-      const bool live = p < out_plane;
+      const int p = (item % tiles) * tile_pix + pix;
+      const bool live = pix < tile_pix && p < out_plane;
       const int pc = live ? p : 0;
-      const int ph = pc / W, pw = pc % W;
+      const int ph = pc / OW, pw = pc % OW;
 #pragma unroll
       for (int k = 0; k < kTapsT; ++k) {
         const int t = tapq + (kMfBlock / kMfPix) * k;
         if (t < K) {
           const int f_h = t / 3, f_w = t % 3;
-          const int ih = ph + f_h * g.dil_h - g.pad_h, iw = pw + f_w - 1;
+          const int ih = S2 ? 2 * ph - 1 + f_h : ph + f_h * g.dil_h - g.pad_h, iw = S2 ? 2 * pw - 1 + f_w : pw + f_w - 1;
           const bool ok = live && ih >= 0 && ih < g.in_h && iw >= 0 && iw < W;
           const float h = scope_coord<float>(g, f_h, r_rot[2 * k], g.centre_h);
           const float w = scope_coord<float>(g, f_w, r_rot[2 * k + 1], g.centre_w);
@@ -1108,6 +1119,16 @@ __global__ __launch_bounds__(kMfBlock, 4) void local_grad_filter_mfma_kernel(
   };
 
   const int px = wave * 16 + 4 * kg;  // first of this lane's four pixels in the tile
+  // S2: pixel (dh, pw) of the tile reads the staged elements (2 dh + r) W + 2 pw + f_w (pixel slots
+  // past the tile read the last pixel's: their weights are zero)
+  int xb[4] = {0, 0, 0, 0};
+  if constexpr (S2) {
+#pragma unroll
+    for (int ii = 0; ii < 4; ++ii) {
+      const int pi = min(px + ii, tile_pix - 1), dh = pi / OW, pw = pi - dh * OW;
+      xb[ii] = 2 * dh * W + 2 * pw;
+    }
+  }
   float A[4][K];
   mf4 acc = {0.f, 0.f, 0.f, 0.f};
   int done_cb = -1;  // channel block (within the split) whose result `acc` holds
@@ -1133,17 +1154,31 @@ __global__ __launch_bounds__(kMfBlock, 4) void local_grad_filter_mfma_kernel(
     const float gq[4] = {gv.x, gv.y, gv.z, gv.w};
 #pragma unroll
     for (int r = 0; r < 3; ++r) {
-      // columns -1 .. +4 of tap row r around the four pixels
-      const float* xr = xs + mf_row(q, pitch_x) + px + r * row_step;
-      float x6[6];
+      float xv[4][3];  // the inputs of tap row r: pixel ii, column f_w
+      if constexpr (S2) {
 #pragma unroll
-      for (int k = 0; k < 6; ++k) x6[k] = xr[k];
+        for (int ii = 0; ii < 4; ++ii) {
+          const float* xr = xs + mf_row(q, pitch_x) + xb[ii] + r * W;
+#pragma unroll
+          for (int f_w = 0; f_w < 3; ++f_w) xv[ii][f_w] = xr[f_w];
+        }
+      } else {
+        // columns -1 .. +4 of tap row r around the four pixels
+        const float* xr = xs + mf_row(q, pitch_x) + px + r * row_step;
+        float x6[6];
+#pragma unroll
+        for (int k = 0; k < 6; ++k) x6[k] = xr[k];
+#pragma unroll
+        for (int ii = 0; ii < 4; ++ii)
+#pragma unroll
+          for (int f_w = 0; f_w < 3; ++f_w) xv[ii][f_w] = x6[ii + f_w];
+      }
 #pragma unroll
       for (int f_w = 0; f_w < 3; ++f_w) {
         const int t = r * 3 + f_w;
 #pragma unroll
         for (int ii = 0; ii < 4; ++ii) {
-          const float b = x6[ii + f_w] * gq[ii];
+          const float b = xv[ii][f_w] * gq[ii];
           if ((ii + t) & 1)
             acc1 = __builtin_amdgcn_mfma_f32_16x16x4f32(A[ii][t], b, acc1, 0, 0, 0);
           else
@@ -1379,7 +1414,8 @@ struct FilterGrid {
   int per, splits, parts, tiles;
   bool mfma;       // matrix-core kernel: 16 channels per workgroup, 256-pixel tiles
   int pitch_x;     // its floats per channel of the staged input tile
-  int nx;          // its staged input elements per lane and channel (4 or 6)
+  int nx;          // its staged input elements per lane and channel (4 or 6; 9 for stride 2)
+  int th;          // stride 2: output rows per tile
   size_t lds;      // its LDS bytes
 };
 
@@ -1389,6 +1425,7 @@ FilterGrid filter_grid(const Geo& g) {
   f.mfma = false;
   f.pitch_x = 0;
   f.nx = 0;
+  f.th = 0;
   f.lds = 0;
   if (same_width_geometry(g) && !path_disabled("DK_NO_MFMA")) {
     const long xt = kMfPix + 2 + 2L * g.dil_h * g.in_w;
@@ -1414,6 +1451,33 @@ FilterGrid filter_grid(const Geo& g) {
       return f;
     }
   }
+  if (stride2_geometry(g) && !path_disabled("DK_NO_MFMA") && !path_disabled("DK_NO_MFMA_S2") && g.out_w <= kMfPix) {
+    // tiles of whole output rows whose input rows (2 th + 1 of them, plus one element) fit the stage
+    int th = std::min(kMfPix / g.out_w, g.out_h);
+    while (th > 1 && (2L * th + 1) * g.in_w + 1 > 64 * kMfXS2) --th;
+    const long xt = (2L * th + 1) * g.in_w + 1;
+    const long pitch = 64 * kMfXS2 + 64;
+    const int nblk = ceil_div(cpg, kMfCh);
+    const int csplits = ceil_div(nblk, kMfMaxBlkS2);
+    const long lds = ((long)kMfCh * pitch + (long)kMfCh * kMfPitchG) * 4 + 9L * kMfPix * 8 +
+                     (long)(kMfBlock / 64) * 256 * 4 + (long)ceil_div(nblk, csplits) * 256 * 4;
+    const int tiles = ceil_div(g.out_h, th);
+    const bool countable = (long)g.batch * tiles * ceil_div(nblk, csplits) < (1L << 30);
+    if (xt <= 64 * kMfXS2 && lds <= 80 * 1024 && countable) {
+      f.mfma = true;
+      f.pitch_x = (int)pitch;
+      f.nx = kMfXS2;
+      f.th = th;
+      f.lds = (size_t)lds;
+      f.per = kMfCh;
+      f.splits = csplits;
+      f.tiles = tiles;
+      const long units = (long)g.batch * f.tiles * ceil_div(nblk, csplits);
+      const long slots = std::max(1, 2 * 256 / (csplits * g.groups));
+      f.parts = (int)std::max(1L, std::min(units, slots));
+      return f;
+    }
+  }
   f.splits = ceil_div(cpg, kFilterChPerBlock);
   f.per = ceil_div(cpg, f.splits);
   f.tiles = ceil_div(g.out_h * g.out_w, rotation_tile(g));
@@ -1433,10 +1497,16 @@ bool run_grad_filter(const Geo& g, const T* gout, const T* x, const T* rot, T* g
     const unsigned grid = (unsigned)xcd_grid_size((long)f.parts * f.splits * g.groups);
     if (f.mfma) {
 #define DK_LAUNCH(CELL0)                                                                                         \
-  if (f.nx == 4)                                                                                                 \
-    local_grad_filter_mfma_kernel<T, SH, SW, CELL0, 4><<<grid, kMfBlock, f.lds, stream>>>(g, gout, x, rot, ws, f.tiles, f.parts, f.splits, f.pitch_x); \
+  if (f.th > 0) {                                                                                                \
+    auto kernel = local_grad_filter_mfma_kernel<T, SH, SW, CELL0, kMfXS2, true>;                                 \
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,  \
+                            (int)f.lds) != hipSuccess)                                                           \
+      return false;                                                                                              \
+    kernel<<<grid, kMfBlock, f.lds, stream>>>(g, gout, x, rot, ws, f.tiles, f.parts, f.splits, f.pitch_x, f.th); \
+  } else if (f.nx == 4)                                                                                          \
+    local_grad_filter_mfma_kernel<T, SH, SW, CELL0, 4, false><<<grid, kMfBlock, f.lds, stream>>>(g, gout, x, rot, ws, f.tiles, f.parts, f.splits, f.pitch_x, 0); \
   else                                                                                                           \
-    local_grad_filter_mfma_kernel<T, SH, SW, CELL0, kMfX><<<grid, kMfBlock, f.lds, stream>>>(g, gout, x, rot, ws, f.tiles, f.parts, f.splits, f.pitch_x);
+    local_grad_filter_mfma_kernel<T, SH, SW, CELL0, kMfX, false><<<grid, kMfBlock, f.lds, stream>>>(g, gout, x, rot, ws, f.tiles, f.parts, f.splits, f.pitch_x, 0);
       DK_LAUNCH(0)
       // the further 16-cell slices of a larger scope, into the same partials
       if constexpr (SH * SW > 16) DK_LAUNCH(16)
