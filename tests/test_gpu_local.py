@@ -36,7 +36,8 @@ TUNED = [
     (4, 64, 28, 28, 3, (4, 4), 1, 1, 1, 1, 1.0),    # grad rotation in 4 channel splits, summed by the few-parts reduction
     (2, 20, 14, 14, 3, (7, 7), 1, 1, 1, 1, 2.0),    # scope 7: four 16-cell slices of the matrix-core grad filter
     (2, 12, 15, 16, 3, (7, 7), 2, 1, 1, 2, 2.0),    # scope 7, stride 2: grad filter on the generic kernel
-    (1, 24, 40, 44, 3, (5, 5), 2, 1, 1, 1, 1.5),    # scope 5, stride 2: dense grad filter with two cells per lane
+    (1, 24, 40, 44, 3, (5, 5), 2, 1, 1, 1, 1.5),    # scope 5, stride 2: two slices of the stride-2 matrix-core grad filter
+    (1, 24, 41, 43, 3, (5, 5), 2, 1, 1, 1, 1.5),    # the same with an odd width: dense grad filter with two cells per lane
 ]
 GENERIC = [
     (2, 6, 9, 8, (5, 3), (7, 4), (1, 2), (2, 0), 1, 3, 0.7),
@@ -216,6 +217,20 @@ def test_more_general_kernels_on_a_same_width_shape(switch, monkeypatch):
     matrix-core one; per-tap loads instead of the row kernels), which must give the same results."""
     monkeypatch.setenv(switch, "1")
     case = (2, 40, 20, 24, 3, (4, 4), 1, 1, 1, 2, 1.0)
+    inputs, got = _run(case, torch.float32)
+    o32, o64 = _oracle(inputs, np.float32), _oracle(inputs, np.float64)
+    assert rel_err(got[0], o32[0]) < 1e-5
+    assert rel_err(got[1], o32[1]) < 1e-5
+    assert rel_err(got[2], o64[2]) < 1e-4
+    assert rel_err(got[3], o64[3]) < 1e-4
+
+
+@pytest.mark.parametrize("switch", ["DK_NO_MFMA_S2", "DK_NO_S2_QUADS"])
+def test_more_general_kernels_on_a_stride_2_shape(switch, monkeypatch):
+    """Stride 2, padding 1, even width: the dense pair-load grad filter instead of the matrix-core one,
+    the gather over input pixels instead of the one over 2 x 2 input quads."""
+    monkeypatch.setenv(switch, "1")
+    case = (2, 24, 22, 20, 3, (4, 4), 2, 1, 1, 2, 1.0)
     inputs, got = _run(case, torch.float32)
     o32, o64 = _oracle(inputs, np.float32), _oracle(inputs, np.float64)
     assert rel_err(got[0], o32[0]) < 1e-5
