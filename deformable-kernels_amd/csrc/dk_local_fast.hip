@@ -558,8 +558,11 @@ __global__ __launch_bounds__(kBlock, 2) void local_grad_input_s2_kernel(Geo g, c
 // result directly.
 // grid = (pixel tiles, splits, batch * groups)
 // ---------------------------------------------------------------------------
-template <typename T, int KH, int KW, int SH, int SW, int MODE>
-__global__ __launch_bounds__(kBlock, 2) void local_grad_rotation_kernel(
+// OCC: waves per SIMD the register allocation leaves room for.  The 27 sums make this the
+// register-heaviest gather kernel; with 96 registers (five waves) it is slower per wave but faster
+// where the grid has more than four workgroups per CU to offer (112 x 112 C=32: 125 -> 96 us).
+template <typename T, int KH, int KW, int SH, int SW, int MODE, int OCC = 2>
+__global__ __launch_bounds__(kBlock, OCC) void local_grad_rotation_kernel(
     Geo g, const T* __restrict__ gout, const T* __restrict__ x, const T* __restrict__ rot,
     const T* __restrict__ filter, T* __restrict__ grot, float* __restrict__ partial, int splits,
     int ch_per_pass) {
@@ -1396,7 +1399,10 @@ bool run_grad_rotation(const Geo& g, const T* gout, const T* x, const T* rot, co
   const size_t lds = (size_t)(per + 1) * Tb::SIZE * sizeof(float);
   const unsigned grid = (unsigned)xcd_grid_size((long)ceil_div(g.out_h * g.out_w, rotation_tile(g)) * splits * g.batch * g.groups);
   if (same_width_geometry(g))
-    local_grad_rotation_kernel<T, 3, 3, SH, SW, 1><<<grid, row_block(g.out_h * g.out_w, kRowLanes), lds, stream>>>(g, gout, x, rot, filter, grot, ws, splits, per);
+    if (grid > 5 * 256)
+      local_grad_rotation_kernel<T, 3, 3, SH, SW, 1, 5><<<grid, row_block(g.out_h * g.out_w, kRowLanes), lds, stream>>>(g, gout, x, rot, filter, grot, ws, splits, per);
+    else
+      local_grad_rotation_kernel<T, 3, 3, SH, SW, 1><<<grid, row_block(g.out_h * g.out_w, kRowLanes), lds, stream>>>(g, gout, x, rot, filter, grot, ws, splits, per);
   else if (stride2_geometry(g))
     local_grad_rotation_kernel<T, 3, 3, SH, SW, 2><<<grid, row_block(g.out_h * g.out_w, kS2Lanes), lds, stream>>>(g, gout, x, rot, filter, grot, ws, splits, per);
   else
