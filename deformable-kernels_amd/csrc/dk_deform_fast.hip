@@ -4,11 +4,11 @@
 //
 // Reference kernels covered (K.cu =
 // deformable_kernels/ops/deform_kernel/csrc/filter_sample_depthwise_cuda_kernel.cu):
-//   forward        K.cu:433-528   -> deform_forward_kernel
-//   grad input     K.cu:704-795   -> deform_grad_input_kernel
-//   grad offset    K.cu:1147-1243 -> deform_grad_coord_kernel<.., OFFSET>
-//   grad rotation  K.cu:1410-1508 -> deform_grad_coord_kernel<.., ROTATION>
-//   grad filter    K.cu:1002-1097 -> deform_grad_filter_kernel
+//   forward        K.cu:433-528   -> deform_forward_ch_kernel | deform_forward_kernel
+//   grad input     K.cu:704-795   -> deform_grad_input_kernel | deform_grad_input_tiled_kernel
+//   grad offset    K.cu:1147-1243 -> deform_grad_coord_ch_kernel | deform_grad_coord_kernel <.., OFFSET>
+//   grad rotation  K.cu:1410-1508 -> deform_grad_coord_ch_kernel | deform_grad_coord_kernel <.., ROTATION>
+//   grad filter    K.cu:1002-1097 -> deform_grad_filter_mfma_kernel | deform_grad_filter_kernel
 //
 // Common structure: a lane owns an output pixel and walks the channels of a chunk.  What depends
 // only on (pixel, tap) -- where the tap samples the image and the scope tile -- is computed once
@@ -19,7 +19,7 @@
 // corner).  Planes are double buffered: the next channel's plane is loaded into registers before
 // the current channel is computed and written to the other buffer afterwards (one barrier per
 // channel).  The scope tiles of the chunk sit in LDS in the corner-expanded difference form.
-// Where LDS has room (planes up to about 28 x 28) forward, grad offset and grad rotation interleave
+// Where LDS has room (planes up to about 36 x 36) forward, grad offset and grad rotation interleave
 // four channel planes, element e of channel c at [e][c]: the corner gathers at per-lane addresses
 // bound these kernels, and one 16-byte read per corner then serves four channels.
 #include <algorithm>

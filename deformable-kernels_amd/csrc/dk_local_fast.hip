@@ -1,5 +1,5 @@
 // Local deformable kernel (kernel-space offsets only), tuned path for gfx950: 3x3 taps, scope
-// 3x3 / 4x4 / 5x5, fp32 / fp16 / bf16.  Everything else runs on dk_generic.hip.
+// 3x3 / 4x4 / 5x5 / 7x7, fp32 / fp16 / bf16.  Everything else runs on dk_generic.hip.
 //
 // One lane owns one pixel and walks the channels of its rotation group.  What depends only on
 // (pixel, tap) -- the scope cell and the fractional position inside it -- is computed once and
@@ -11,9 +11,10 @@
 // deformable_kernels/ops/deform_kernel/csrc/filter_sample_depthwise_cuda_kernel.cu):
 //   forward        K.cu:270-386   -> local_gather_rows_kernel<.., false> (stride 1, same width),
 //                                    local_forward_s2_kernel (stride 2), local_gather_kernel<.., false, 9>
-//   grad input     K.cu:577-669   -> local_gather_rows_kernel<.., true>, local_gather_kernel<.., true, 9 | 4>
+//   grad input     K.cu:577-669   -> local_gather_rows_kernel<.., true>, local_grad_input_s2_kernel (stride 2),
+//                                    local_gather_kernel<.., true, 9 | 4>
 //   grad rotation  K.cu:1285-1370 -> local_grad_rotation_kernel<.., MODE> (+ reduce_few_parts_kernel)
-//   grad filter    K.cu:836-955   -> local_grad_filter_mfma_kernel | local_grad_filter_kernel<.., MODE>
+//   grad filter    K.cu:836-955   -> local_grad_filter_mfma_kernel<.., S2> | local_grad_filter_kernel<.., MODE>
 //                                    + reduce_partials_kernel
 #include <cstdlib>
 
