@@ -1415,7 +1415,7 @@ bool run_deform_grad_input(const Geo& g, const T* gout, const T* off, const T* r
   if (tiled) {
     auto kernel = deform_grad_input_tiled_kernel<T, SH, SW>;
     if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
-                            (int)tiled_lds) != hipSuccess)
+                            kMaxDynamicLds) != hipSuccess)
       return false;
     const int cpg = g.channel / g.groups;
     const unsigned tgrid = (unsigned)xcd_grid_size((long)ceil_div(cpg, kTiledCh) * g.batch * g.groups);
@@ -1463,7 +1463,7 @@ bool launch_deform_grad_filter_mfma(const Geo& g, const GradFilterMfma& m, const
                                     const T* rot, float* ws, hipStream_t stream) {
   auto kernel = deform_grad_filter_mfma_kernel<T, SH, SW, CELL0>;
   if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
-                          (int)m.lds) != hipSuccess)
+                          kMaxDynamicLds) != hipSuccess)
     return false;
   const unsigned grid = (unsigned)xcd_grid_size((long)m.tiles * m.csplits * g.batch * g.groups);
   kernel<<<grid, kGfBlock, m.lds, stream>>>(g, gout, x, off, rot, ws, m.tiles, m.csplits, m.shift);

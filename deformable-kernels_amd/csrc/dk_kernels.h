@@ -19,6 +19,12 @@ namespace dk {
 // Read at every call, so a test can toggle them inside one process.
 inline bool path_disabled(const char* name) { return std::getenv(name) != nullptr; }
 
+// Upper bound handed to hipFuncAttributeMaxDynamicSharedMemorySize for the kernels that need more
+// than 64 KB of LDS: the attribute is per kernel, not per launch, so a launch must not lower what a
+// concurrent one (another host thread, another shape) relies on.  A gfx950 CU has 160 KB of LDS;
+// the kernels' small static arrays come out of the same budget, so the bound stays 8 KB below.
+constexpr int kMaxDynamicLds = 152 * 1024;
+
 template <typename CT, typename T>
 void launch_reduce_partials(const CT* partial, int parts, long count, T* out, hipStream_t stream);
 

@@ -1507,7 +1507,7 @@ bool run_grad_filter(const Geo& g, const T* gout, const T* x, const T* rot, T* g
   if (f.th > 0) {                                                                                                \
     auto kernel = local_grad_filter_mfma_kernel<T, SH, SW, CELL0, kMfXS2, true>;                                 \
     if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,  \
-                            (int)f.lds) != hipSuccess)                                                           \
+                            kMaxDynamicLds) != hipSuccess)                                                           \
       return false;                                                                                              \
     kernel<<<grid, kMfBlock, f.lds, stream>>>(g, gout, x, rot, ws, f.tiles, f.parts, f.splits, f.pitch_x, f.th); \
   } else if (f.nx == 4)                                                                                          \

@@ -546,9 +546,9 @@ bool offset_conv_wgrad(int batch, int cin, int cout, int h, int w, const float* 
     const size_t lds = (size_t)(kCvChunk * WgradTile<WW>::PSX + cout * WgradTile<WW>::GP) * sizeof(float);     \
     const size_t lds_red = (size_t)NT * 256 * sizeof(float);                                                   \
     const size_t bytes = std::max(lds, lds_red);                                                               \
-    if (bytes > 160 * 1024 ||                                                                                  \
+    if (bytes > (size_t)kMaxDynamicLds ||                                                                                  \
         hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, \
-                            (int)bytes) != hipSuccess)                                                         \
+                            kMaxDynamicLds) != hipSuccess)                                                         \
       ok = false;                                                                                              \
     else if (batch > 0)                                                                                        \
       kernel<<<parts * nchunks, kWgBlock, bytes, stream>>>(g, x, gout, partial, parts);                        \
