@@ -1081,11 +1081,17 @@ __global__ __launch_bounds__(kMfBlock, 4) void local_grad_filter_mfma_kernel(
       const size_t c = (size_t)n * g.channel + grp + (size_t)g.groups * (chan ? cj_ : 0);
       const rsrc_t rx = plane_rsrc(x + c * in_plane, chan ? in_plane : 0);
       const rsrc_t rg = plane_rsrc(gout + c * out_plane, chan ? out_plane : 0);
-      // elements before the plane (negative, so huge as unsigned) or past its end fail the buffer's
-      // range check and read 0; the 64 * NX staged elements may run past xt (never read)
+      // Elements past the plane's end fail the buffer's range check and read 0; the 64 * NX staged
+      // elements may run past the tile's halo (never read).  Elements BEFORE the plane (the first
+      // tile's top halo row) get the out-of-range offset explicitly: left as negative offsets they
+      // are huge unsigned numbers and also fail the check, but the compiler then addresses the
+      // loads of one lane as one base register plus immediates, and with a negative base the
+      // first three elements of the plane came back as 0 on planes 64 and 112 columns wide.
 #pragma unroll
-      for (int k = 0; k < NX; ++k)
-        r_x[jj][k] = buf_ld(rx, (unsigned)(x0 + lane + 64 * k) * (unsigned)sizeof(T), x);
+      for (int k = 0; k < NX; ++k) {
+        const int e = x0 + lane + 64 * k;
+        r_x[jj][k] = buf_ld(rx, e < 0 ? kOutOfRange : (unsigned)e * (unsigned)sizeof(T), x);
+      }
 #pragma unroll
       for (int k = 0; k < kMfPix / 64; ++k)
         r_g[jj][k] = buf_ld(rg, (unsigned)(p0 + lane + 64 * k) * (unsigned)sizeof(T), gout);

@@ -34,6 +34,11 @@ TUNED = [
     (2, 12, 15, 16, 3, (4, 4), 2, 1, 1, 2, 1.0),    # stride 2, padding 1, even width: pair-load kernels; odd height, 2 groups
     (1, 20, 40, 44, 3, (3, 3), 2, 1, 1, 1, 0.8),    # the same on 440-pixel output planes (two tiles), scope 3
     (4, 64, 28, 28, 3, (4, 4), 1, 1, 1, 1, 1.0),    # grad rotation in 4 channel splits, summed by the few-parts reduction
+    (1, 5, 5, 64, 3, (4, 4), 1, 1, 1, 1, 1.0),      # planes 64 / 112 / 130 columns wide: the first element of the plane
+    (1, 3, 4, 112, 3, (3, 3), 1, 1, 1, 1, 1.0),     # sits in the second or third 64-element chunk of the first tile's
+    (1, 3, 3, 130, 3, (4, 4), 1, 1, 1, 1, 1.0),     # staged range, behind the (out-of-range) top halo row
+    (1, 4, 6, 64, 3, (4, 4), 2, 1, 1, 1, 1.0),      # the same for the stride-2 geometry
+    (1, 3, 5, 130, 3, (5, 5), 2, 1, 1, 1, 1.0),
     (2, 20, 14, 14, 3, (7, 7), 1, 1, 1, 1, 2.0),    # scope 7: four 16-cell slices of the matrix-core grad filter
     (2, 12, 15, 16, 3, (7, 7), 2, 1, 1, 2, 2.0),    # scope 7, stride 2: grad filter on the generic kernel
     (1, 24, 40, 44, 3, (5, 5), 2, 1, 1, 1, 1.5),    # scope 5, stride 2: two slices of the stride-2 matrix-core grad filter
