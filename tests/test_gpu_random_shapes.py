@@ -1,0 +1,70 @@
+"""Seeded random geometries through the tuned kernels against the CPU oracle: plane sizes from one
+pixel to 260 columns, channel counts that fill no tile, every scope and stride of the tuned
+families, rotation groups.  The fixed cases of test_gpu_local.py / test_gpu_deform.py name the
+situations they cover; this sweep is for the ones nobody thought of (it found planes 64 and 112
+columns wide losing their first three elements in the matrix-core grad filter)."""
+import random
+
+import numpy as np
+import pytest
+import torch
+
+import test_gpu_deform as td
+import test_gpu_local as tl
+from _cases import rel_err
+
+pytestmark = pytest.mark.gpu
+
+
+def _local_cases():
+    rnd = random.Random(5)
+    cases = []
+    for _ in range(24):   # stride 2, padding 1: pair-load forward, quad grad input, matrix-core or dense grad filter
+        cases.append((rnd.choice([1, 2, 3]), rnd.choice([1, 2, 3, 5, 16, 17, 33, 48]),
+                      rnd.choice([2, 3, 4, 5, 6, 7, 9, 12, 14, 17, 28, 33]),
+                      rnd.choice([2, 4, 6, 8, 10, 14, 18, 26, 30, 56, 64, 112, 130, 260]), 3,
+                      rnd.choice([(3, 3), (4, 4), (5, 5), (7, 7)]), 2, 1, 1, 1, 1.0))
+    for _ in range(12):   # stride 1, padding 1: row kernels, matrix-core grad filter
+        cases.append((rnd.choice([1, 2]), rnd.choice([1, 3, 16, 20, 40]), rnd.choice([1, 2, 3, 5, 8, 13]),
+                      rnd.choice([1, 2, 3, 5, 9, 31, 63, 64, 112, 130]), 3,
+                      rnd.choice([(3, 3), (4, 4), (5, 5), (7, 7)]), 1, 1, 1, 1, 1.0))
+    out = []
+    for c in cases:   # rotation groups that divide the channel count
+        groups = [g for g in (1, 2, 3) if c[1] % g == 0]
+        out.append(c[:9] + (rnd.choice(groups), c[10]))
+    return out
+
+
+def _deform_cases():
+    rnd = random.Random(11)
+    cases = []
+    while len(cases) < 20:
+        H = rnd.choice([1, 2, 3, 5, 7, 8, 14, 16, 17, 28, 31, 32, 33, 36])
+        W = rnd.choice([1, 2, 3, 7, 8, 14, 16, 28, 31, 32, 33, 36, 40, 64])
+        C = rnd.choice([1, 2, 3, 4, 5, 8, 9, 16, 17, 33, 48])
+        G = rnd.choice([g for g in (1, 2, 3) if C % g == 0])
+        s, p, d = rnd.choice([1, 2]), rnd.choice([0, 1]), rnd.choice([1, 1, 2])
+        if (H + 2 * p - 2 * d - 1) // s + 1 < 1 or (W + 2 * p - 2 * d - 1) // s + 1 < 1:
+            continue
+        cases.append((rnd.choice([1, 2]), C, H, W, 3, rnd.choice([(3, 3), (4, 4), (5, 5)]), s, p, d, G, 0.7,
+                      rnd.choice([0.5, 2.0, 6.0])))
+    return cases
+
+
+@pytest.mark.parametrize("case", _local_cases())
+def test_local_operator_on_random_geometries(case):
+    inputs, got = tl._run(case, torch.float32)
+    o32, o64 = tl._oracle(inputs, np.float32), tl._oracle(inputs, np.float64)
+    assert rel_err(got[0], o32[0]) < 1e-5
+    assert rel_err(got[1], o32[1]) < 1e-5
+    assert rel_err(got[2], o64[2]) < 1e-4
+    assert rel_err(got[3], o64[3]) < 1e-4
+
+
+@pytest.mark.parametrize("case", _deform_cases())
+def test_deformable_operator_on_random_geometries(case):
+    inputs, got = td._run(case, torch.float32)
+    o32, o64 = td._oracle(inputs, np.float32), td._oracle(inputs, np.float64)
+    assert rel_err(got[0], o32[0]) < 1e-5
+    for i in range(1, 5):
+        assert rel_err(got[i], o64[i]) < 1e-4, td.NAMES[i]
