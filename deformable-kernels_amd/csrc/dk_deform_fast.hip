@@ -19,9 +19,11 @@
 // corner).  Planes are double buffered: the next channel's plane is loaded into registers before
 // the current channel is computed and written to the other buffer afterwards (one barrier per
 // channel).  The scope tiles of the chunk sit in LDS in the corner-expanded difference form.
-// Where LDS has room (planes up to about 36 x 36) forward, grad offset and grad rotation interleave
-// four channel planes, element e of channel c at [e][c]: the corner gathers at per-lane addresses
-// bound these kernels, and one 16-byte read per corner then serves four channels.
+// Forward, grad offset and grad rotation interleave four channel planes, element e of channel c at
+// [e][c]: the corner gathers at per-lane addresses bound these kernels, and one 16-byte read per
+// corner then serves four channels.  Planes up to about 30 x 30 run that form in workgroups of 256
+// threads, several per CU; larger ones (up to 64 x 64) in one workgroup of 1024 threads per CU that
+// takes most of the CU's LDS for the two interleaved buffers.
 #include <algorithm>
 #include <cstdlib>
 
@@ -272,10 +274,10 @@ __device__ __forceinline__ CornersN<CH> read_corners_n(const float* planes, int 
   return q;
 }
 
-template <typename T, int SH, int SW, int NPASS, int CH>
-__global__ __launch_bounds__(kDBlock, 2) void deform_forward_ch_kernel(
+template <typename T, int SH, int SW, int NPASS, int CH, int BLOCK = kDBlock>
+__global__ __launch_bounds__(BLOCK, BLOCK == kDBlock ? 2 : 1) void deform_forward_ch_kernel(
     Geo g, const T* __restrict__ x, const T* __restrict__ off, const T* __restrict__ rot,
-    const T* __restrict__ filter, T* __restrict__ out, int ch_per_block, int shift) {
+    const T* __restrict__ filter, T* __restrict__ out, int ch_per_block, int shift, int tile_pix) {
   using Tb = WideTable<SH, SW>;
   extern __shared__ __align__(16) float lds[];
   const int H = g.in_h, W = g.in_w, RS = W + 2;
@@ -285,19 +287,19 @@ __global__ __launch_bounds__(kDBlock, 2) void deform_forward_ch_kernel(
 
   const int cpg = g.channel / g.groups;
   const int out_plane = g.out_h * g.out_w, in_plane = H * W;
-  const BlockId b = decode_block(g, ceil_div(out_plane, kDBlock), ceil_div(cpg, ch_per_block));
+  const BlockId b = decode_block(g, ceil_div(out_plane, tile_pix), ceil_div(cpg, ch_per_block));
   if (!b.valid) return;
   const int j0 = b.chunk * ch_per_block;
   const int nch = min(ch_per_block, cpg - j0);
   const int nq = ceil_div(nch, CH);
 
-  for (int e = threadIdx.x; e < 2 * PS * CH; e += kDBlock) planes[e] = 0.f;
+  for (int e = threadIdx.x; e < 2 * PS * CH; e += BLOCK) planes[e] = 0.f;
   // the tables of the channels that pad the last CH-tuple are read (their products discarded)
-  for (int e = nch * Tb::SIZE + threadIdx.x; e < nq * CH * Tb::SIZE; e += kDBlock) tbl[e] = 0.f;
+  for (int e = nch * Tb::SIZE + threadIdx.x; e < nq * CH * Tb::SIZE; e += BLOCK) tbl[e] = 0.f;
   stage_wide_tables<T, SH, SW>(tbl, filter, g.channel, b.grp + g.groups * j0, g.groups, nch);
 
-  const int p = b.tile * kDBlock + threadIdx.x;
-  const bool live = p < out_plane;
+  const int p = b.tile * tile_pix + threadIdx.x;
+  const bool live = (int)threadIdx.x < tile_pix && p < out_plane;
   ImgTap it[K9];
   LiteTap st[K9];
   deform_taps<T, SH, SW>(g, off, rot, b.n, b.grp, p, live, RS, it, st);
@@ -456,11 +458,11 @@ __global__ __launch_bounds__(kDBlock, 2) void deform_grad_coord_kernel(
 }
 
 // The same with CH channel planes interleaved in LDS (see deform_forward_ch_kernel).
-template <typename T, int SH, int SW, int NPASS, bool ROTATION, int CH>
-__global__ __launch_bounds__(kDBlock, 2) void deform_grad_coord_ch_kernel(
+template <typename T, int SH, int SW, int NPASS, bool ROTATION, int CH, int BLOCK = kDBlock>
+__global__ __launch_bounds__(BLOCK, BLOCK == kDBlock ? 2 : 1) void deform_grad_coord_ch_kernel(
     Geo g, const T* __restrict__ gout, const T* __restrict__ x, const T* __restrict__ off,
     const T* __restrict__ rot, const T* __restrict__ filter, float* __restrict__ partial,
-    int ch_per_block, int shift) {
+    int ch_per_block, int shift, int tile_pix) {
   using Tb = WideTable<SH, SW>;
   extern __shared__ __align__(16) float lds[];
   const int H = g.in_h, W = g.in_w, RS = W + 2;
@@ -471,19 +473,19 @@ __global__ __launch_bounds__(kDBlock, 2) void deform_grad_coord_ch_kernel(
   const int cpg = g.channel / g.groups;
   const int out_plane = g.out_h * g.out_w, in_plane = H * W;
   const int chunks = ceil_div(cpg, ch_per_block);
-  const BlockId b = decode_block(g, ceil_div(out_plane, kDBlock), chunks);
+  const BlockId b = decode_block(g, ceil_div(out_plane, tile_pix), chunks);
   if (!b.valid) return;
   const int j0 = b.chunk * ch_per_block;
   const int nch = min(ch_per_block, cpg - j0);
   const int nq = ceil_div(nch, CH);
 
-  for (int e = threadIdx.x; e < 2 * PS * CH; e += kDBlock) planes[e] = 0.f;
+  for (int e = threadIdx.x; e < 2 * PS * CH; e += BLOCK) planes[e] = 0.f;
   // the padding channels of the last CH-tuple have gout = 0; their tables must be finite
-  for (int e = nch * Tb::SIZE + threadIdx.x; e < nq * CH * Tb::SIZE; e += kDBlock) tbl[e] = 0.f;
+  for (int e = nch * Tb::SIZE + threadIdx.x; e < nq * CH * Tb::SIZE; e += BLOCK) tbl[e] = 0.f;
   stage_wide_tables<T, SH, SW>(tbl, filter, g.channel, b.grp + g.groups * j0, g.groups, nch);
 
-  const int p = b.tile * kDBlock + threadIdx.x;
-  const bool live = p < out_plane;
+  const int p = b.tile * tile_pix + threadIdx.x;
+  const bool live = (int)threadIdx.x < tile_pix && p < out_plane;
   ImgTap it[K9];
   LiteTap st[K9];
   deform_taps<T, SH, SW>(g, off, rot, b.n, b.grp, p, live, RS, it, st);
@@ -1264,6 +1266,8 @@ struct DeformPlan {
   int per;     // channels per block
   int chunks;  // channel chunks per group
   int tiles;   // pixel tiles
+  int block;   // threads of a workgroup
+  int tile_pix;  // output pixels of a tile (<= block)
   size_t lds;
 };
 
@@ -1271,7 +1275,8 @@ struct DeformPlan {
 // blocks_per_cu: how many workgroups per CU the channel chunking aims at (measured per kernel on
 // N=64 C=512 28x28 -> 14x14: grad input 4, grad filter 3, the channel-interleaved kernels 3; the
 // one-plane forward 4, grad offset 3, grad rotation 2)
-DeformPlan deform_plan(const Geo& g, int table_floats, int planes, int block, int blocks_per_cu) {
+DeformPlan deform_plan(const Geo& g, int table_floats, int planes, int block, int blocks_per_cu,
+                       long lds_budget = 64 * 1024) {
   DeformPlan d{};
   d.ok = false;
   if (path_disabled("DK_NO_DEFORM_FAST")) return d;
@@ -1289,8 +1294,9 @@ DeformPlan deform_plan(const Geo& g, int table_floats, int planes, int block, in
   d.PS = ((g.in_h + 2) * (g.in_w + 2) + 3) & ~3;
   const int cpg = g.channel / g.groups;
   d.tiles = ceil_div(g.out_h * g.out_w, block);
+  d.block = d.tile_pix = block;
   const long plane_bytes = (long)planes * d.PS * 4;
-  const long room = 64 * 1024 - plane_bytes;
+  const long room = lds_budget - plane_bytes;
   if (room < (long)table_floats * 4 * 4) return d;
   const int fit = (int)std::min<long>(room / ((long)table_floats * 4), cpg);
   // enough blocks for blocks_per_cu per CU, chunks of at least 8 channels
@@ -1309,15 +1315,30 @@ DeformPlan deform_plan(const Geo& g, int table_floats, int planes, int block, in
 // Plan of the kernels that interleave kDeformCh channel planes in LDS; ok only when the two
 // interleaved buffers, the tables and a four-pass register stage fit.
 constexpr int kDeformCh = 4;
+constexpr int kDBigBlock = 1024;
+constexpr int kDBigBlocksPerCu = 1;
+constexpr long kDBigLds = 150 * 1024;
 
 DeformPlan deform_plan_ch(const Geo& g, int table_floats, int blocks_per_cu) {
   DeformPlan d{};
   d.ok = false;
   if (path_disabled("DK_NO_DEFORM_CH")) return d;
   d = deform_plan(g, table_floats, 2 * kDeformCh, kDBlock, blocks_per_cu);
+  if (d.ok) {
+    d.lds += (size_t)(kDeformCh - 1) * table_floats * 4;  // tables of the channels that pad the last tuple
+    d.ok = d.npass == 4 && d.lds <= 64 * 1024;
+    if (d.ok) return d;
+  }
+  // Larger planes (up to 64 x 64): one workgroup of kDBigBlock threads per CU with most of the CU's LDS (its
+  // sixteen waves hide the gathers' latency: 512 threads were 25 % slower, more than one channel chunk per
+  // CU's worth of workgroups no faster), and tiles of equal size (a plane of 56 x 56 is 4 tiles of 13 waves).
+  if (path_disabled("DK_NO_DEFORM_CH_BIG")) { d.ok = false; return d; }
+  d = deform_plan(g, table_floats, 2 * kDeformCh, kDBigBlock, kDBigBlocksPerCu,
+                  kDBigLds - (long)(kDeformCh - 1) * table_floats * 4);
   if (!d.ok) return d;
-  d.lds += (size_t)(kDeformCh - 1) * table_floats * 4;  // tables of the channels that pad the last tuple
-  d.ok = d.npass == 4 && d.lds <= 64 * 1024;
+  d.lds += (size_t)(kDeformCh - 1) * table_floats * 4;
+  d.tile_pix = ceil_div(ceil_div(g.out_h * g.out_w, d.tiles), 64) * 64;
+  d.ok = d.npass == 4 && d.lds <= (size_t)kDBigLds;
   return d;
 }
 
@@ -1328,7 +1349,15 @@ bool run_deform_forward(const Geo& g, const T* x, const T* off, const T* rot, co
   const DeformPlan d4 = deform_plan_ch(g, WideTable<SH, SW>::SIZE, 3);
   if (d4.ok) {
     const unsigned grid = (unsigned)xcd_grid_size((long)d4.tiles * d4.chunks * g.batch * g.groups);
-    deform_forward_ch_kernel<T, SH, SW, 4, kDeformCh><<<grid, kDBlock, d4.lds, stream>>>(g, x, off, rot, filter, out, d4.per, d4.shift);
+    if (d4.block == kDBlock) {
+      deform_forward_ch_kernel<T, SH, SW, 4, kDeformCh><<<grid, kDBlock, d4.lds, stream>>>(g, x, off, rot, filter, out, d4.per, d4.shift, d4.tile_pix);
+      return true;
+    }
+    auto kernel = deform_forward_ch_kernel<T, SH, SW, 4, kDeformCh, kDBigBlock>;
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                            kMaxDynamicLds) != hipSuccess)
+      return false;
+    kernel<<<grid, kDBigBlock, d4.lds, stream>>>(g, x, off, rot, filter, out, d4.per, d4.shift, d4.tile_pix);
     return true;
   }
   const DeformPlan d = deform_plan(g, WideTable<SH, SW>::SIZE, 2, kDBlock, 4);
@@ -1351,11 +1380,18 @@ bool run_deform_grad_coord(const Geo& g, bool rotation, const T* gout, const T* 
   const DeformPlan d = d4.ok ? d4 : deform_plan(g, WideTable<SH, SW>::SIZE, 2, kDBlock, rotation ? 2 : 3);
   if (!d.ok) return false;
   const unsigned grid = (unsigned)xcd_grid_size((long)d.tiles * d.chunks * g.batch * g.groups);
-  if (d4.ok) {
+  if (d4.ok && d.block == kDBigBlock) {
+    auto kernel = rotation ? deform_grad_coord_ch_kernel<T, SH, SW, 4, true, kDeformCh, kDBigBlock>
+                           : deform_grad_coord_ch_kernel<T, SH, SW, 4, false, kDeformCh, kDBigBlock>;
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                            kMaxDynamicLds) != hipSuccess)
+      return false;
+    kernel<<<grid, kDBigBlock, d.lds, stream>>>(g, gout, x, off, rot, filter, ws, d.per, d.shift, d.tile_pix);
+  } else if (d4.ok) {
     if (rotation)
-      deform_grad_coord_ch_kernel<T, SH, SW, 4, true, kDeformCh><<<grid, kDBlock, d.lds, stream>>>(g, gout, x, off, rot, filter, ws, d.per, d.shift);
+      deform_grad_coord_ch_kernel<T, SH, SW, 4, true, kDeformCh><<<grid, kDBlock, d.lds, stream>>>(g, gout, x, off, rot, filter, ws, d.per, d.shift, d.tile_pix);
     else
-      deform_grad_coord_ch_kernel<T, SH, SW, 4, false, kDeformCh><<<grid, kDBlock, d.lds, stream>>>(g, gout, x, off, rot, filter, ws, d.per, d.shift);
+      deform_grad_coord_ch_kernel<T, SH, SW, 4, false, kDeformCh><<<grid, kDBlock, d.lds, stream>>>(g, gout, x, off, rot, filter, ws, d.per, d.shift, d.tile_pix);
   } else {
 #define DK_LAUNCH(NP, ROT)                                                                          \
   deform_grad_coord_kernel<T, SH, SW, NP, ROT><<<grid, kDBlock, d.lds, stream>>>(g, gout, x, off, rot, filter, ws, \
