@@ -951,8 +951,9 @@ __global__ __launch_bounds__(kBlock, (SH * SW <= 16 ? 2 : 1)) void local_grad_fi
 //     channel blocks of the tile;
 //   * per unit: the 16 channels' tiles of gout and of x with its halo rows are staged
 //     channel-major in LDS from loads coalesced along pixels; a lane reads its channel's
-//     4 gout and 3 x 6 input values and issues 36 MFMAs.  The loads of the next unit are
-//     issued before the MFMAs and land in registers while they run.
+//     4 gout and 3 x 6 input values and issues 36 MFMAs (fp32 inputs: v_mfma_f32_16x16x4_f32;
+//     16-bit inputs: 9 v_mfma_f32_16x16x16_bf16 on operands rounded to bfloat16, fp32 sums).
+//     The loads of the next unit are issued before the MFMAs and land in registers while they run.
 //   * the 8 waves' 16 x 16 results of a unit are added into a per-channel-block accumulator in
 //     LDS (by a fixed owner thread, in wave order), piggybacked on the next unit's barriers.
 // One partial per workgroup goes to the workspace; reduce_partials_kernel adds them in order.
@@ -968,6 +969,7 @@ constexpr int kMfXS2 = 9;              // stride 2: staged input elements per la
 constexpr int kMfMaxBlkS2 = 12;        // stride 2: channel blocks per workgroup (two workgroups' LDS fit a CU)
 
 typedef float mf4 __attribute__((ext_vector_type(4)));
+typedef __bf16 mfb4 __attribute__((ext_vector_type(4)));
 
 // First float of channel j's row in the staged input tile.  The rows are a multiple of 64 floats
 // apart plus a skew: in the MFMA phase lane (channel q, pixel quad kg) reads row q at
@@ -1139,7 +1141,13 @@ __global__ __launch_bounds__(kMfBlock, 4) void local_grad_filter_mfma_kernel(
       xb[ii] = 2 * dh * W + 2 * pw;
     }
   }
-  float A[4][K];
+  // 16-bit inputs: the four pixels a lane holds per tap become the four k of one
+  // v_mfma_f32_16x16x16_bf16 (k = 4 kg + ii), hat products and x * gout products rounded to
+  // bfloat16 (for fp16 inputs too: the products can leave fp16's range), fp32 accumulation --
+  // 9 matrix instructions of 16 clk per unit instead of 36 of 32 clk.
+  constexpr bool kHalfIn = sizeof(T) == 2;
+  float A[kHalfIn ? 1 : 4][K];
+  mfb4 Ab[kHalfIn ? K : 1];
   mf4 acc = {0.f, 0.f, 0.f, 0.f};
   int done_cb = -1;  // channel block (within the split) whose result `acc` holds
 
@@ -1186,13 +1194,23 @@ __global__ __launch_bounds__(kMfBlock, 4) void local_grad_filter_mfma_kernel(
 #pragma unroll
       for (int f_w = 0; f_w < 3; ++f_w) {
         const int t = r * 3 + f_w;
+        if constexpr (kHalfIn) {
+          mfb4 b;
 #pragma unroll
-        for (int ii = 0; ii < 4; ++ii) {
-          const float b = xv[ii][f_w] * gq[ii];
-          if ((ii + t) & 1)
-            acc1 = __builtin_amdgcn_mfma_f32_16x16x4f32(A[ii][t], b, acc1, 0, 0, 0);
+          for (int ii = 0; ii < 4; ++ii) b[ii] = static_cast<__bf16>(xv[ii][f_w] * gq[ii]);
+          if (t & 1)
+            acc1 = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(Ab[t], b, acc1, 0, 0, 0);
           else
-            acc0 = __builtin_amdgcn_mfma_f32_16x16x4f32(A[ii][t], b, acc0, 0, 0, 0);
+            acc0 = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(Ab[t], b, acc0, 0, 0, 0);
+        } else {
+#pragma unroll
+          for (int ii = 0; ii < 4; ++ii) {
+            const float b = xv[ii][f_w] * gq[ii];
+            if ((ii + t) & 1)
+              acc1 = __builtin_amdgcn_mfma_f32_16x16x4f32(A[ii][t], b, acc1, 0, 0, 0);
+            else
+              acc0 = __builtin_amdgcn_mfma_f32_16x16x4f32(A[ii][t], b, acc0, 0, 0, 0);
+          }
         }
       }
     }
@@ -1214,10 +1232,16 @@ __global__ __launch_bounds__(kMfBlock, 4) void local_grad_filter_mfma_kernel(
     for (int t = 0; t < K; ++t) {
       const float4 hw01 = *reinterpret_cast<const float4*>(hw + t * kMfPix + px);
       const float4 hw23 = *reinterpret_cast<const float4*>(hw + t * kMfPix + px + 2);
-      A[0][t] = hat(hw01.x - ci) * hat(hw01.y - cj);
-      A[1][t] = hat(hw01.z - ci) * hat(hw01.w - cj);
-      A[2][t] = hat(hw23.x - ci) * hat(hw23.y - cj);
-      A[3][t] = hat(hw23.z - ci) * hat(hw23.w - cj);
+      const float a0 = hat(hw01.x - ci) * hat(hw01.y - cj), a1 = hat(hw01.z - ci) * hat(hw01.w - cj);
+      const float a2 = hat(hw23.x - ci) * hat(hw23.y - cj), a3 = hat(hw23.z - ci) * hat(hw23.w - cj);
+      if constexpr (kHalfIn) {
+        Ab[t] = mfb4{static_cast<__bf16>(a0), static_cast<__bf16>(a1), static_cast<__bf16>(a2), static_cast<__bf16>(a3)};
+      } else {
+        A[0][t] = a0;
+        A[1][t] = a1;
+        A[2][t] = a2;
+        A[3][t] = a3;
+      }
     }
     multiply_unit(cb_begin);
     for (int cbi = cb_begin + 1; cbi < cb_end; ++cbi) {

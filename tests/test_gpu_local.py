@@ -96,7 +96,9 @@ def test_fp64_matches_oracle(case):
 
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
-@pytest.mark.parametrize("case", TUNED[:5] + GENERIC[:2])
+# the matrix-core grad filter multiplies 16-bit inputs with bfloat16 matrix instructions (hat products and
+# x * gout products rounded to bfloat16, fp32 sums): same-width, wide-plane, stride-2, 5 x 5 and 7 x 7 geometries
+@pytest.mark.parametrize("case", TUNED[:5] + [TUNED[7], TUNED[10], TUNED[15], TUNED[18], TUNED[20], TUNED[22]] + GENERIC[:2])
 def test_half_precisions_match_fp32_oracle(case, dtype):
     inputs, got = _run(case, dtype)
     want = _oracle(inputs, np.float32)  # the inputs are already rounded to `dtype`
