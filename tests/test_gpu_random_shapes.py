@@ -61,10 +61,30 @@ def test_local_operator_on_random_geometries(case):
     assert rel_err(got[3], o64[3]) < 1e-4
 
 
-@pytest.mark.parametrize("case", _deform_cases())
+def _deform_large_cases():
+    """Planes of 30 to 64 rows and columns: the 1024-thread channel-interleaved kernels, tiled grad input."""
+    rnd = random.Random(13)
+    cases = []
+    for _ in range(10):
+        C = rnd.choice([1, 3, 4, 6, 9, 13])
+        cases.append((rnd.choice([1, 2]), C, rnd.randint(30, 64), rnd.randint(30, 64), 3,
+                      rnd.choice([(3, 3), (4, 4), (5, 5)]), rnd.choice([1, 2]), rnd.choice([0, 1]), rnd.choice([1, 1, 2]),
+                      rnd.choice([g for g in (1, 3) if C % g == 0]), 0.7, rnd.choice([0.5, 2.0, 6.0])))
+    return cases
+
+
+@pytest.mark.parametrize("case", _deform_cases() + _deform_large_cases())
 def test_deformable_operator_on_random_geometries(case):
     inputs, got = td._run(case, torch.float32)
-    o32, o64 = td._oracle(inputs, np.float32), td._oracle(inputs, np.float64)
-    assert rel_err(got[0], o32[0]) < 1e-5
-    for i in range(1, 5):
-        assert rel_err(got[i], o64[i]) < 1e-4, td.NAMES[i]
+    td.assert_fp32_parity(got, td._oracle(inputs, np.float32), td._oracle(inputs, np.float64))
+
+
+@pytest.mark.parametrize("k,case", list(enumerate(_local_cases()))[::2])
+def test_local_operator_on_random_geometries_in_16_bits(k, case):
+    """bf16 and fp16 in turn; the matrix-core grad filter multiplies them with bfloat16 instructions."""
+    dtype = torch.bfloat16 if k % 4 == 0 else torch.float16
+    inputs, got = tl._run(case, dtype)
+    want = tl._oracle(inputs, np.float32)   # on the inputs as rounded to dtype
+    for g, w, name in zip(got, want, ("forward", "grad input", "grad rotation", "grad filter")):
+        assert g.dtype == dtype
+        assert rel_err(g.float(), w) < 1e-2, name
