@@ -984,7 +984,7 @@ __device__ __forceinline__ float hat(float d) { return __builtin_amdgcn_fmed3f(1
 // most 128 pixels), so that the input rows its taps read, 2 oh0 - 1 .. 2 (oh0 + th - 1) + 1, are
 // one contiguous range of the plane like the stride-1 tile with its halo rows; a lane's four
 // pixels may sit in different rows, so each reads its own 3 x 3 inputs.
-template <typename T, int SH, int SW, int CELL0, int NX, bool S2>
+template <typename T, int SH, int SW, int CELL0, int NX, bool S2, bool BF = false>
 __global__ __launch_bounds__(kMfBlock, 4) void local_grad_filter_mfma_kernel(
     Geo g, const T* __restrict__ gout, const T* __restrict__ x, const T* __restrict__ rot,
     float* __restrict__ partial, int tiles, int nwg, int csplits, int pitch_x, int th) {
@@ -1145,7 +1145,12 @@ __global__ __launch_bounds__(kMfBlock, 4) void local_grad_filter_mfma_kernel(
   // v_mfma_f32_16x16x16_bf16 (k = 4 kg + ii), hat products and x * gout products rounded to
   // bfloat16 (for fp16 inputs too: the products can leave fp16's range), fp32 accumulation --
   // 9 matrix instructions of 16 clk per unit instead of 36 of 32 clk.
-  constexpr bool kHalfIn = sizeof(T) == 2;
+  // Against the result's largest element the rounding noise is about 3e-3 when a group has many
+  // (channel, cell) results, but with a handful of results that largest element can itself be
+  // small (one channel, 3 x 3 scope: 1.1e-2 seen), so groups of fewer than 16 channels keep the
+  // fp32 instructions (template parameter BF, chosen by the host).
+  static_assert(!BF || sizeof(T) == 2, "bfloat16 matrix instructions are for 16-bit inputs");
+  constexpr bool kHalfIn = BF;
   float A[kHalfIn ? 1 : 4][K];
   mfb4 Ab[kHalfIn ? K : 1];
   mf4 acc = {0.f, 0.f, 0.f, 0.f};
@@ -1533,23 +1538,30 @@ bool run_grad_filter(const Geo& g, const T* gout, const T* x, const T* rot, T* g
     const FilterGrid f = filter_grid(g);
     const unsigned grid = (unsigned)xcd_grid_size((long)f.parts * f.splits * g.groups);
     if (f.mfma) {
-#define DK_LAUNCH(CELL0)                                                                                         \
+#define DK_LAUNCH_BF(CELL0, BF)                                                                                  \
   if (f.th > 0) {                                                                                                \
-    auto kernel = local_grad_filter_mfma_kernel<T, SH, SW, CELL0, kMfXS2, true>;                                 \
+    auto kernel = local_grad_filter_mfma_kernel<T, SH, SW, CELL0, kMfXS2, true, BF>;                             \
     if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,  \
                             kMaxDynamicLds) != hipSuccess)                                                           \
       return false;                                                                                              \
     kernel<<<grid, kMfBlock, f.lds, stream>>>(g, gout, x, rot, ws, f.tiles, f.parts, f.splits, f.pitch_x, f.th); \
   } else if (f.nx == 4)                                                                                          \
-    local_grad_filter_mfma_kernel<T, SH, SW, CELL0, 4, false><<<grid, kMfBlock, f.lds, stream>>>(g, gout, x, rot, ws, f.tiles, f.parts, f.splits, f.pitch_x, 0); \
+    local_grad_filter_mfma_kernel<T, SH, SW, CELL0, 4, false, BF><<<grid, kMfBlock, f.lds, stream>>>(g, gout, x, rot, ws, f.tiles, f.parts, f.splits, f.pitch_x, 0); \
   else                                                                                                           \
-    local_grad_filter_mfma_kernel<T, SH, SW, CELL0, kMfX, false><<<grid, kMfBlock, f.lds, stream>>>(g, gout, x, rot, ws, f.tiles, f.parts, f.splits, f.pitch_x, 0);
+    local_grad_filter_mfma_kernel<T, SH, SW, CELL0, kMfX, false, BF><<<grid, kMfBlock, f.lds, stream>>>(g, gout, x, rot, ws, f.tiles, f.parts, f.splits, f.pitch_x, 0);
+      // 16-bit inputs with at least one full block of 16 channels per group: bfloat16 matrix instructions
+#define DK_LAUNCH(CELL0)                                          \
+  if constexpr (sizeof(T) == 2) {                                 \
+    if (g.channel / g.groups >= kMfCh) { DK_LAUNCH_BF(CELL0, true) } \
+    else { DK_LAUNCH_BF(CELL0, false) }                           \
+  } else { DK_LAUNCH_BF(CELL0, false) }
       DK_LAUNCH(0)
       // the further 16-cell slices of a larger scope, into the same partials
       if constexpr (SH * SW > 16) DK_LAUNCH(16)
       if constexpr (SH * SW > 32) DK_LAUNCH(32)
       if constexpr (SH * SW > 48) DK_LAUNCH(48)
 #undef DK_LAUNCH
+#undef DK_LAUNCH_BF
       launch_reduce_partials<float, T>(ws, f.parts, g.channel * SH * SW, gfilter, stream);
       return true;
     }
