@@ -1318,7 +1318,8 @@ __global__ __launch_bounds__(kBlock) void reduce_few_parts_kernel(const CT* __re
 
 template <typename CT, typename T>
 void launch_reduce_partials(const CT* partial, int parts, long count, T* out, hipStream_t stream) {
-  if (parts <= kRedSlices && count >= 16384)
+  // parts == 0 (an empty batch) takes the second kernel, which then writes zeros and reads nothing
+  if (parts > 0 && parts <= kRedSlices && count >= 16384)
     reduce_few_parts_kernel<CT, T><<<(unsigned)((count + kBlock - 1) / kBlock), kBlock, 0, stream>>>(partial, parts, count, out);
   else
     reduce_partials_kernel<CT, T><<<(unsigned)((count + kRedEl - 1) / kRedEl), kRedEl * kRedSlices, 0, stream>>>(partial, parts, (int)count, out);
