@@ -85,6 +85,16 @@ template <typename T> constexpr bool kHasFast = !std::is_same<T, double>::value;
 template <typename T> const T* in(const void* p) { return static_cast<const T*>(p); }
 template <typename T> T* out(void* p) { return static_cast<T*>(p); }
 
+// The filter gradient of an empty batch is all zeros: the ordered reduction over zero partial
+// buffers writes them (a kernel, not a memset, so the call can be captured into a graph).
+int zero_filter_grad(const Geo& g, int dtype, void* filter_grad, hipStream_t s) {
+  const long count = (long)g.channel * g.scope_h * g.scope_w;
+  return by_dtype(dtype, [&]<typename T>() {
+    using CT = compute_t<T>;
+    launch_reduce_partials<CT, T>(static_cast<const CT*>(nullptr), 0, count, out<T>(filter_grad), s);
+  });
+}
+
 size_t local_filter_ws(const Geo& g, int dtype) {
   const size_t a = dtype == DK_F64 ? 0 : fast_local_grad_filter_workspace(g);
   return a ? a : generic_grad_filter_workspace(g, dtype);
@@ -168,6 +178,7 @@ int dk_sample_depthwise_backward_filter(const dk_conv_desc* desc, const void* ou
   const size_t need = local_filter_ws(g, desc->dtype);
   if (need && (!workspace || workspace_bytes < need)) return DK_ERR_WORKSPACE;
   hipStream_t s = static_cast<hipStream_t>(stream);
+  if (g.batch == 0) return zero_filter_grad(g, desc->dtype, filter_grad, s);
   return by_dtype(desc->dtype, [&]<typename T>() {
     if constexpr (kHasFast<T>)
       if (fast_local_grad_filter<T>(g, in<T>(out_grad), in<T>(input), in<T>(rotation), out<T>(filter_grad), workspace, s)) return;
@@ -299,7 +310,7 @@ int dk_deformable_sample_depthwise_backward_filter(const dk_conv_desc* desc, con
   const size_t need = dk_deformable_sample_depthwise_backward_filter_workspace(desc);
   if (need && (!workspace || workspace_bytes < need)) return DK_ERR_WORKSPACE;
   hipStream_t s = static_cast<hipStream_t>(stream);
-  if (g.batch == 0) return DK_OK;
+  if (g.batch == 0) return zero_filter_grad(g, desc->dtype, filter_grad, s);
   return by_dtype(desc->dtype, [&]<typename T>() {
     if constexpr (kHasFast<T>)
       if (fast_deform_grad_filter<T>(g, in<T>(out_grad), in<T>(input), in<T>(offset), in<T>(rotation),
