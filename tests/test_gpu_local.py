@@ -252,3 +252,31 @@ def test_more_general_kernels_on_a_stride_2_shape(switch, monkeypatch):
     assert rel_err(got[1], o32[1]) < 1e-5
     assert rel_err(got[2], o64[2]) < 1e-4
     assert rel_err(got[3], o64[3]) < 1e-4
+
+
+@pytest.mark.parametrize("deform", [False, True])
+@pytest.mark.parametrize("shape", [(8, 4), (1200, 4)])  # channels, scope: both reduction kernels
+def test_c_abi_filter_gradient_of_an_empty_batch_is_written_as_zeros(deform, shape):
+    """batch == 0 through the raw C ABI (the Python Functions refuse empty batches as the reference's
+    output-size rule does): the filter gradient is the one result that is not empty, and it is zeros."""
+    from deformable_kernels.ops.deform_kernel import _lib
+    L, P = _lib.lib(), _lib.ptr
+    dev = torch.device("cuda:0")
+    C, S = shape
+    x = torch.empty(0, C, 12, 12, device=dev)
+    wt = torch.empty(C, 1, S, S, device=dev)
+    desc = _lib.conv_desc(x, wt, (3, 3), (1, 1), (1, 1), (1, 1), 1)
+    gw = torch.full_like(wt, float("nan"))
+    s = torch.cuda.current_stream().cuda_stream
+    one = P(gw)  # never read: the batch is empty
+    if deform:
+        need = L.dk_deformable_sample_depthwise_backward_filter_workspace(desc)
+        ws, nbytes = _lib.workspace(max(need, 16), dev)
+        rc = L.dk_deformable_sample_depthwise_backward_filter(desc, one, one, one, one, P(gw), P(ws), nbytes, s)
+    else:
+        need = L.dk_sample_depthwise_backward_filter_workspace(desc)
+        ws, nbytes = _lib.workspace(max(need, 16), dev)
+        rc = L.dk_sample_depthwise_backward_filter(desc, one, one, one, P(gw), P(ws), nbytes, s)
+    torch.cuda.synchronize()
+    assert rc == 0
+    assert torch.count_nonzero(gw).item() == 0 and torch.isfinite(gw).all()
