@@ -4,6 +4,7 @@
 // (K.cpp = deformable_kernels/ops/deform_kernel/csrc/filter_sample_depthwise_cuda.cpp,
 //  ND.cpp = .../csrc/nd_linear_sample_cuda.cpp).
 #include <algorithm>
+#include <atomic>
 #include <cstdlib>
 
 #include "dk_kernels.h"
@@ -102,6 +103,33 @@ size_t local_filter_ws(const Geo& g, int dtype) {
 
 }  // namespace
 
+// ---- the filter gradient for callers that cannot allocate ---------------------------------
+//
+// The per-workgroup partial sums live in a file-scope device array instead of a caller's
+// workspace.  Each GPU holds its own copy of the array at its own address; the address is looked
+// up once per device (first call with that device current) and kept.  Host code never uses the
+// array's name as a pointer: kernels, and anything else that needs the memory, get `ptr`.
+static __device__ __align__(256) unsigned char dk_static_scratch[DK_STATIC_SCRATCH_BYTES];
+
+namespace {
+constexpr int kMaxDevices = 64;
+std::atomic<void*> g_static_scratch[kMaxDevices];
+
+int static_scratch_of_current_device(void** ptr) {
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess) return DK_ERR_LAUNCH;
+  if (dev < 0 || dev >= kMaxDevices) return DK_ERR_UNSUPPORTED;
+  void* p = g_static_scratch[dev].load(std::memory_order_acquire);
+  if (!p) {
+    // two threads racing here both get the same address
+    if (hipGetSymbolAddress(&p, HIP_SYMBOL(dk_static_scratch)) != hipSuccess || !p) return DK_ERR_LAUNCH;
+    g_static_scratch[dev].store(p, std::memory_order_release);
+  }
+  *ptr = p;
+  return DK_OK;
+}
+}  // namespace
+
 extern "C" {
 
 int dk_version(void) { return (0 << 16) | 1; }
@@ -116,6 +144,7 @@ const char* dk_status_string(int status) {
     case DK_ERR_WORKSPACE: return "workspace missing or too small";
     case DK_ERR_LAUNCH: return "HIP kernel launch failed";
     case DK_ERR_UNSUPPORTED: return "unsupported configuration";
+    case DK_ERR_SCRATCH_LIMIT: return "problem needs more scratch memory than the library's static buffer holds";
     default: return "unknown status";
   }
 }
@@ -212,6 +241,25 @@ int dk_sample_depthwise_backward_rotation(const dk_conv_desc* desc, const void* 
     generic_grad_rotation<T>(g, false, in<T>(out_grad), in<T>(input), (const T*)nullptr, in<T>(rotation),
                              in<T>(filter), out<T>(rotation_grad), s);
   });
+}
+
+// ---- the filter gradient for callers that cannot allocate ---------------------------------
+
+int dk_sample_depthwise_backward_filter_static(const dk_conv_desc* desc, const void* out_grad,
+                                               const void* input, const void* rotation,
+                                               void* filter_grad, void* stream) {
+  Geo g;
+  const int rc = make_geo(desc, g);
+  if (rc != DK_OK) return rc;
+  if (!out_grad || !input || !rotation || !filter_grad) return DK_ERR_NULL_POINTER;
+  if (local_filter_ws(g, desc->dtype) > (size_t)DK_STATIC_SCRATCH_BYTES) return DK_ERR_SCRATCH_LIMIT;
+  void* ptr = nullptr;
+  const int st = static_scratch_of_current_device(&ptr);
+  if (st != DK_OK) return st;
+  // Every partial sum the reduction reads is written by this call's kernels first, so nothing
+  // of an earlier call's contents has to be cleared.
+  return dk_sample_depthwise_backward_filter(desc, out_grad, input, rotation, filter_grad, ptr,
+                                             DK_STATIC_SCRATCH_BYTES, stream);
 }
 
 // The rotation and the filter gradient run one after the other on the stream and share the buffer.

@@ -53,6 +53,7 @@ SIGNATURES = {
     "dk_sample_depthwise_backward_data": (ctypes.c_int, [_CD, _P, _P, _P, _P, _P]),
     "dk_sample_depthwise_backward_filter_workspace": (_SZ, [_CD]),
     "dk_sample_depthwise_backward_filter": (ctypes.c_int, [_CD, _P, _P, _P, _P, _P, _SZ, _P]),
+    "dk_sample_depthwise_backward_filter_static": (ctypes.c_int, [_CD, _P, _P, _P, _P, _P]),
     "dk_sample_depthwise_backward_rotation_workspace": (_SZ, [_CD]),
     "dk_sample_depthwise_backward_rotation": (ctypes.c_int, [_CD, _P, _P, _P, _P, _P, _P, _SZ, _P]),
     "dk_sample_depthwise_backward_workspace": (_SZ, [_CD]),

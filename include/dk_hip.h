@@ -45,7 +45,9 @@ typedef enum {
   DK_ERR_TOO_LARGE = -4,      /* a tensor has >= 2^31 elements (32-bit plane indexing)  */
   DK_ERR_WORKSPACE = -5,      /* workspace NULL or smaller than the *_workspace() query */
   DK_ERR_LAUNCH = -6,         /* the HIP runtime refused the launch                     */
-  DK_ERR_UNSUPPORTED = -7     /* e.g. more than DK_ND_MAX_DIMS sampling dimensions      */
+  DK_ERR_UNSUPPORTED = -7,    /* e.g. more than DK_ND_MAX_DIMS sampling dimensions      */
+  DK_ERR_SCRATCH_LIMIT = -8   /* *_static entry point: the problem needs more scratch   */
+                              /* memory than DK_STATIC_SCRATCH_BYTES                    */
 } dk_status;
 
 typedef enum { DK_F32 = 0, DK_F16 = 1, DK_BF16 = 2, DK_F64 = 3 } dk_dtype;
@@ -111,6 +113,21 @@ int dk_sample_depthwise_backward_filter(const dk_conv_desc *desc, const void *ou
                                         const void *input, const void *rotation,
                                         void *filter_grad, void *workspace,
                                         size_t workspace_bytes, void *stream);
+
+/* The same filter gradient for callers that cannot allocate device memory or hand over a
+ * workspace: code under HIP graph capture, tight serving loops, harnesses that forbid
+ * hipMalloc.  No counterpart in the reference.  The per-workgroup partial sums go to a buffer of
+ * DK_STATIC_SCRATCH_BYTES that is part of the library's device image (every GPU the library runs
+ * on holds it until the process ends); the call allocates nothing and runs the same kernels as
+ * dk_sample_depthwise_backward_filter, so the result is bit-identical to that function's.
+ * Returns DK_ERR_SCRATCH_LIMIT, launching nothing, when
+ * dk_sample_depthwise_backward_filter_workspace(desc) exceeds DK_STATIC_SCRATCH_BYTES.
+ * All calls on one GPU share the one buffer: calls that may overlap on a GPU (different streams,
+ * different host threads) race on it and must be ordered by the caller. */
+#define DK_STATIC_SCRATCH_BYTES (8u << 20)
+int dk_sample_depthwise_backward_filter_static(const dk_conv_desc *desc, const void *out_grad,
+                                               const void *input, const void *rotation,
+                                               void *filter_grad, void *stream);
 
 /* sample_depthwise_backward_rotation_cuda (filter_sample_depthwise_cuda.cpp:178-235).
  * Small planes split the channel sum over several workgroups whose partial sums go through the
