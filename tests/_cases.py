@@ -55,6 +55,20 @@ def rel_err(a, b):
     return float((a - b).abs().max()) / scale
 
 
+def mixed_err(a, b):
+    """max over the elements of |a - b| / (max|b| + |b|): `mixed_err(a, b) < tol` says that every
+    element is within tol * max|b| + tol * |b| of the expected one -- the absolute part bounds the
+    elements that are small by cancellation, the relative part scales with the element itself."""
+    a = torch.as_tensor(a).detach().to(torch.float64)
+    b = torch.as_tensor(b).detach().to(torch.float64)
+    if b.numel() == 0:
+        return 0.0
+    scale = float(b.abs().max())
+    if scale == 0.0:
+        return float((a - b).abs().max())
+    return float(((a - b).abs() / (scale + b.abs())).max())
+
+
 def clipped_rotation(rot, clip, kernel_size, scope, groups):
     """What the reference's module does to the rotation tensor before the operator
     (modules/deform_kernel.py:185-212), restated on torch CPU tensors in the tensor's own
