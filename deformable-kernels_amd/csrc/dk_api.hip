@@ -6,11 +6,60 @@
 #include <algorithm>
 #include <atomic>
 #include <cstdlib>
+#include <mutex>
+#include <utility>
+#include <vector>
 
 #include "dk_kernels.h"
 #include "dk_nd.h"
 
 using namespace dk;
+
+namespace dk {
+
+namespace {
+constexpr unsigned kSwitchesUnread = 0x80000000u;
+std::atomic<unsigned> g_switches{kSwitchesUnread};
+
+unsigned switches_from_environment() {
+  static const struct { const char* name; unsigned bit; } vars[] = {
+      {"DK_NO_ROWS", kNoRows}, {"DK_NO_MFMA", kNoMfma}, {"DK_NO_MFMA_S2", kNoMfmaS2},
+      {"DK_NO_S2_QUADS", kNoS2Quads}, {"DK_NO_DEFORM_FAST", kNoDeformFast}, {"DK_NO_DEFORM_CH", kNoDeformCh},
+      {"DK_NO_DEFORM_CH_BIG", kNoDeformChBig}, {"DK_NO_DEFORM_MFMA", kNoDeformMfma},
+      {"DK_NO_ND_BINS", kNoNdBins}, {"DK_NO_ND_MFMA", kNoNdMfma}};
+  unsigned m = 0;
+  for (const auto& v : vars)
+    if (std::getenv(v.name)) m |= v.bit;
+  return m;
+}
+
+std::mutex g_lds_mutex;
+std::vector<std::pair<const void*, int>> g_lds_allowed;  // (kernel, device) pairs already set
+}  // namespace
+
+unsigned test_switches() {
+  unsigned m = g_switches.load(std::memory_order_relaxed);
+  if (m == kSwitchesUnread) {
+    m = switches_from_environment();
+    unsigned expected = kSwitchesUnread;
+    if (!g_switches.compare_exchange_strong(expected, m)) m = expected;  // a dk_test_switches() call came first
+  }
+  return m;
+}
+
+bool allow_max_dynamic_lds(const void* kernel) {
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess) return false;
+  std::lock_guard<std::mutex> lock(g_lds_mutex);
+  for (const auto& e : g_lds_allowed)
+    if (e.first == kernel && e.second == dev) return true;
+  if (hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, kMaxDynamicLds) != hipSuccess)
+    return false;
+  g_lds_allowed.emplace_back(kernel, dev);
+  return true;
+}
+
+}  // namespace dk
 
 namespace {
 
@@ -132,7 +181,13 @@ int static_scratch_of_current_device(void** ptr) {
 
 extern "C" {
 
-int dk_version(void) { return (0 << 16) | 1; }
+int dk_version(void) { return (0 << 16) | 2; }
+
+unsigned dk_test_switches(unsigned mask) {
+  const unsigned before = test_switches();
+  g_switches.store(mask & ~kSwitchesUnread, std::memory_order_relaxed);
+  return before;
+}
 
 const char* dk_status_string(int status) {
   switch (status) {

@@ -602,21 +602,24 @@ __global__ __launch_bounds__(BLOCK, BLOCK == kDBlock ? 2 : 1) void deform_grad_c
 // One block per (image, group, channel chunk); blockDim = output pixels rounded up to a wave.
 // The kernel for planes of more than 1024 output pixels further down always uses the 2^-44 grid.
 // ---------------------------------------------------------------------------
-// max |p[i]| over a workgroup's share into out[blockIdx.x] (as the bits of a non-negative float,
-// which order like unsigned integers); the consumer takes the maximum of the kAbsParts words
+// max |p[i]| over a workgroup's share into out[blockIdx.x], as the bits of a non-negative float,
+// which order like unsigned integers -- and the maximum is taken on those bits, so that an
+// infinity (0x7f800000) or a NaN (anything above) in p wins and reaches the consumer, where a
+// float maximum would drop a NaN; the consumer takes the maximum of the kAbsParts words
 // (one atomic maximum per workgroup on a single word cost more than the reads: the atomics on one
 // address serialise).  16-byte loads, four in flight per thread; p must be 16-byte aligned (the
 // host checks).
 template <typename T>
 __global__ __launch_bounds__(256) void absmax_kernel(const T* __restrict__ p, long n, unsigned* __restrict__ out) {
-  __shared__ float wave_max[4];
+  __shared__ unsigned wave_max[4];
   constexpr int V = 16 / (int)sizeof(T);
   struct alignas(16) Vec {
     T e[V];
   };
   const long nv = n / V, stride = (long)gridDim.x * blockDim.x, tid = (long)blockIdx.x * blockDim.x + threadIdx.x;
   const Vec* pv = reinterpret_cast<const Vec*>(p);
-  float m = 0.f;
+  unsigned m = 0u;
+  auto absbits = [](float v) { return __float_as_uint(v) & 0x7fffffffu; };
   constexpr int kInFlight = 4;
   for (long i = tid; i < nv; i += kInFlight * stride) {
     Vec q[kInFlight];
@@ -625,14 +628,13 @@ __global__ __launch_bounds__(256) void absmax_kernel(const T* __restrict__ p, lo
 #pragma unroll
     for (int k = 0; k < kInFlight; ++k)
 #pragma unroll
-      for (int e = 0; e < V; ++e) m = fmaxf(m, fabsf(ld(&q[k].e[e])));
+      for (int e = 0; e < V; ++e) m = max(m, absbits(ld(&q[k].e[e])));
   }
-  for (long i = nv * V + tid; i < n; i += stride) m = fmaxf(m, fabsf(ld(p + i)));
-  for (int s = 32; s > 0; s >>= 1) m = fmaxf(m, __shfl_xor(m, s));
+  for (long i = nv * V + tid; i < n; i += stride) m = max(m, absbits(ld(p + i)));
+  for (int s = 32; s > 0; s >>= 1) m = max(m, (unsigned)__shfl_xor((int)m, s));
   if ((threadIdx.x & 63) == 0) wave_max[threadIdx.x >> 6] = m;
   __syncthreads();
-  if (threadIdx.x == 0)
-    out[blockIdx.x] = __float_as_uint(fmaxf(fmaxf(wave_max[0], wave_max[1]), fmaxf(wave_max[2], wave_max[3])));
+  if (threadIdx.x == 0) out[blockIdx.x] = max(max(wave_max[0], wave_max[1]), max(wave_max[2], wave_max[3]));
 }
 constexpr int kAbsParts = 512;  // workgroups of absmax_kernel = words the consumers reduce
 
@@ -647,6 +649,24 @@ __device__ __forceinline__ float block_absmax(const unsigned* __restrict__ parts
   if ((threadIdx.x & 63) == 0) atomicMax(&s_max, m);
   __syncthreads();
   return __uint_as_float(s_max);
+}
+
+// The fixed-point sums need a finite bound gmax * wmax[c] on a term.  With an infinity or a NaN in
+// out_grad (gmax is then that value: the maximum is taken on bit patterns) or in a channel's filter
+// there is none, and the conversions to integers would turn such terms into zeros or wrapped numbers:
+// the workgroup then writes NaN to the planes it owns instead (all of grad_input for a non-finite
+// out_grad).  The reference's float atomics carry a non-finite term to the elements it touches;
+// what a caller tests -- any non-finite value in the gradient, as loss scaling does -- gives the
+// same answer.  Uniform over the workgroup; must be called by all its threads after wmax is visible.
+template <typename T>
+__device__ __forceinline__ bool write_nan_if_unbounded(float gmax, const float* wmax, int nch, T* planes0, size_t step,
+                                                       int plane) {
+  bool bounded = true;
+  for (int j = 0; j < nch; ++j) bounded = bounded && (fabsf(gmax * wmax[j]) < __builtin_inff());  // false for NaN
+  if (bounded) return false;
+  for (int j = 0; j < nch; ++j)
+    for (int e = threadIdx.x; e < plane; e += blockDim.x) dk::st(planes0 + (size_t)j * step + e, __builtin_nanf(""));
+  return true;
 }
 
 // Two channels share a 64-bit sum while at most 2^kPairHead samples touch one input element.
@@ -683,9 +703,9 @@ __global__ __launch_bounds__(1024) void deform_grad_input_kernel(
   stage_wide_tables<T, SH, SW>(tbl, filter, g.channel, b.grp + g.groups * j0, g.groups, nch);
   for (int j = threadIdx.x; j < nch; j += blockDim.x) {
     const T* f = filter + (size_t)(b.grp + g.groups * (j0 + j)) * (SH * SW);
-    float m = 0.f;
-    for (int e = 0; e < SH * SW; ++e) m = fmaxf(m, fabsf(ld(f + e)));
-    wmax[j] = m;
+    unsigned m = 0u;  // on bit patterns, so that a NaN is not dropped
+    for (int e = 0; e < SH * SW; ++e) m = max(m, __float_as_uint(ld(f + e)) & 0x7fffffffu);
+    wmax[j] = __uint_as_float(m);
   }
 
   const int p = threadIdx.x;
@@ -740,6 +760,7 @@ __global__ __launch_bounds__(1024) void deform_grad_input_kernel(
   const size_t g_step = (size_t)g.groups * out_plane, i_step = (size_t)g.groups * in_plane;
   const unsigned goff = live ? (unsigned)p * (unsigned)sizeof(T) : kOutOfRange;
   const float gmax = block_absmax(gmax_bits);
+  if (write_nan_if_unbounded(gmax, wmax, nch, ip, i_step, in_plane)) return;
   const int col = threadIdx.x & ((1 << shift) - 1), sub = threadIdx.x >> shift;
   const int rpp = (int)blockDim.x >> shift;
 
@@ -870,9 +891,9 @@ __global__ __launch_bounds__(1024) void deform_grad_input_tiled_kernel(
   stage_wide_tables<T, SH, SW>(tbl, filter, g.channel, b.grp + g.groups * j0, g.groups, nch);
   if (threadIdx.x < nch) {
     const T* f = filter + (size_t)(b.grp + g.groups * (j0 + threadIdx.x)) * (SH * SW);
-    float m = 0.f;
-    for (int e = 0; e < SH * SW; ++e) m = fmaxf(m, fabsf(ld(f + e)));
-    wmax[threadIdx.x] = m;
+    unsigned m = 0u;  // on bit patterns, so that a NaN is not dropped
+    for (int e = 0; e < SH * SW; ++e) m = max(m, __float_as_uint(ld(f + e)) & 0x7fffffffu);
+    wmax[threadIdx.x] = __uint_as_float(m);
   }
   __syncthreads();
 
@@ -881,6 +902,7 @@ __global__ __launch_bounds__(1024) void deform_grad_input_tiled_kernel(
   const size_t chan0 = (size_t)b.n * g.channel + b.grp + (size_t)g.groups * j0;
   const T* gp = gout + chan0 * out_plane;
   const size_t g_step = (size_t)g.groups * out_plane, i_step = (size_t)g.groups * in_plane;
+  if (write_nan_if_unbounded(gmax, wmax, nch, gin + chan0 * in_plane, i_step, in_plane)) return;
 
   for (int tile = 0; tile * (int)blockDim.x < out_plane; ++tile) {
     const int p = tile * (int)blockDim.x + threadIdx.x;
@@ -1279,7 +1301,7 @@ DeformPlan deform_plan(const Geo& g, int table_floats, int planes, int block, in
                        long lds_budget = 64 * 1024) {
   DeformPlan d{};
   d.ok = false;
-  if (path_disabled("DK_NO_DEFORM_FAST")) return d;
+  if (path_disabled(kNoDeformFast)) return d;
   if (g.k_h != 3 || g.k_w != 3 || g.in_w > 64) return d;
   if (!((g.scope_h == 3 && g.scope_w == 3) || (g.scope_h == 4 && g.scope_w == 4) ||
         (g.scope_h == 5 && g.scope_w == 5)))
@@ -1322,7 +1344,7 @@ constexpr long kDBigLds = 150 * 1024;
 DeformPlan deform_plan_ch(const Geo& g, int table_floats, int blocks_per_cu) {
   DeformPlan d{};
   d.ok = false;
-  if (path_disabled("DK_NO_DEFORM_CH")) return d;
+  if (path_disabled(kNoDeformCh)) return d;
   d = deform_plan(g, table_floats, 2 * kDeformCh, kDBlock, blocks_per_cu);
   if (d.ok) {
     d.lds += (size_t)(kDeformCh - 1) * table_floats * 4;  // tables of the channels that pad the last tuple
@@ -1332,7 +1354,7 @@ DeformPlan deform_plan_ch(const Geo& g, int table_floats, int blocks_per_cu) {
   // Larger planes (up to 64 x 64): one workgroup of kDBigBlock threads per CU with most of the CU's LDS (its
   // sixteen waves hide the gathers' latency: 512 threads were 25 % slower, more than one channel chunk per
   // CU's worth of workgroups no faster), and tiles of equal size (a plane of 56 x 56 is 4 tiles of 13 waves).
-  if (path_disabled("DK_NO_DEFORM_CH_BIG")) { d.ok = false; return d; }
+  if (path_disabled(kNoDeformChBig)) { d.ok = false; return d; }
   d = deform_plan(g, table_floats, 2 * kDeformCh, kDBigBlock, kDBigBlocksPerCu,
                   kDBigLds - (long)(kDeformCh - 1) * table_floats * 4);
   if (!d.ok) return d;
@@ -1354,8 +1376,7 @@ bool run_deform_forward(const Geo& g, const T* x, const T* off, const T* rot, co
       return true;
     }
     auto kernel = deform_forward_ch_kernel<T, SH, SW, 4, kDeformCh, kDBigBlock>;
-    if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
-                            kMaxDynamicLds) != hipSuccess)
+    if (!allow_max_dynamic_lds(reinterpret_cast<const void*>(kernel)))
       return false;
     kernel<<<grid, kDBigBlock, d4.lds, stream>>>(g, x, off, rot, filter, out, d4.per, d4.shift, d4.tile_pix);
     return true;
@@ -1383,8 +1404,7 @@ bool run_deform_grad_coord(const Geo& g, bool rotation, const T* gout, const T* 
   if (d4.ok && d.block == kDBigBlock) {
     auto kernel = rotation ? deform_grad_coord_ch_kernel<T, SH, SW, 4, true, kDeformCh, kDBigBlock>
                            : deform_grad_coord_ch_kernel<T, SH, SW, 4, false, kDeformCh, kDBigBlock>;
-    if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
-                            kMaxDynamicLds) != hipSuccess)
+    if (!allow_max_dynamic_lds(reinterpret_cast<const void*>(kernel)))
       return false;
     kernel<<<grid, kDBigBlock, d.lds, stream>>>(g, gout, x, off, rot, filter, ws, d.per, d.shift, d.tile_pix);
   } else if (d4.ok) {
@@ -1450,8 +1470,7 @@ bool run_deform_grad_input(const Geo& g, const T* gout, const T* off, const T* r
   absmax_kernel<T><<<kAbsParts, 256, 0, stream>>>(gout, n, gmax);
   if (tiled) {
     auto kernel = deform_grad_input_tiled_kernel<T, SH, SW>;
-    if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
-                            kMaxDynamicLds) != hipSuccess)
+    if (!allow_max_dynamic_lds(reinterpret_cast<const void*>(kernel)))
       return false;
     const int cpg = g.channel / g.groups;
     const unsigned tgrid = (unsigned)xcd_grid_size((long)ceil_div(cpg, kTiledCh) * g.batch * g.groups);
@@ -1473,7 +1492,7 @@ struct GradFilterMfma {
 GradFilterMfma grad_filter_mfma_plan(const Geo& g) {
   GradFilterMfma m{};
   m.ok = false;
-  if (path_disabled("DK_NO_DEFORM_MFMA")) return m;
+  if (path_disabled(kNoDeformMfma)) return m;
   const DeformPlan basic = deform_plan(g, 64, 0, kGfBlock, 1);  // the family's limits and the row mapping only
   if (!basic.ok) return m;
   m.shift = basic.shift;
@@ -1498,8 +1517,7 @@ template <typename T, int SH, int SW, int CELL0>
 bool launch_deform_grad_filter_mfma(const Geo& g, const GradFilterMfma& m, const T* gout, const T* x, const T* off,
                                     const T* rot, float* ws, hipStream_t stream) {
   auto kernel = deform_grad_filter_mfma_kernel<T, SH, SW, CELL0>;
-  if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
-                          kMaxDynamicLds) != hipSuccess)
+  if (!allow_max_dynamic_lds(reinterpret_cast<const void*>(kernel)))
     return false;
   const unsigned grid = (unsigned)xcd_grid_size((long)m.tiles * m.csplits * g.batch * g.groups);
   kernel<<<grid, kGfBlock, m.lds, stream>>>(g, gout, x, off, rot, ws, m.tiles, m.csplits, m.shift);

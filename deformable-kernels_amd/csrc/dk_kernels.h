@@ -10,14 +10,29 @@
 
 namespace dk {
 
-// Test switches.  Setting one of these environment variables (to anything) makes the dispatch
-// skip a specialised kernel family and take the next more general one, so that every kernel can
-// be reached for the same shape:
-//   DK_NO_ROWS         the "same-width" row kernels (and with them the matrix-core grad filter)
-//   DK_NO_MFMA         the matrix-core grad filter (the dense register form runs instead)
-//   DK_NO_DEFORM_FAST  the tuned deformable kernels (the generic ones run instead)
-// Read at every call, so a test can toggle them inside one process.
-inline bool path_disabled(const char* name) { return std::getenv(name) != nullptr; }
+// Test switches: each bit makes the dispatch skip a specialised kernel family and take the next
+// more general one, so that every kernel can be reached for the same shape.  The mask is read from
+// the environment once, at the first call that looks at it (a variable DK_NO_ROWS, DK_NO_MFMA, ...
+// set to anything sets its bit), and can be replaced at run time with dk_test_switches(); the
+// dispatch only loads one word per call.
+enum TestSwitch : unsigned {
+  kNoRows = 1u << 0,        // DK_NO_ROWS         the "same-width" and stride-2 row kernels (and with them the matrix-core grad filter)
+  kNoMfma = 1u << 1,        // DK_NO_MFMA         the matrix-core grad filter (the dense register form runs instead)
+  kNoMfmaS2 = 1u << 2,      // DK_NO_MFMA_S2      its stride-2 form
+  kNoS2Quads = 1u << 3,     // DK_NO_S2_QUADS     the stride-2 grad input over 2 x 2 input quads
+  kNoDeformFast = 1u << 4,  // DK_NO_DEFORM_FAST  the tuned deformable kernels (the generic ones run instead)
+  kNoDeformCh = 1u << 5,    // DK_NO_DEFORM_CH    their channel-interleaved forms
+  kNoDeformChBig = 1u << 6, // DK_NO_DEFORM_CH_BIG  only the 1024-thread channel-interleaved form
+  kNoDeformMfma = 1u << 7,  // DK_NO_DEFORM_MFMA  the matrix-core deformable grad filter
+  kNoNdBins = 1u << 8,      // DK_NO_ND_BINS      the N-d kernels that sort the points by cell
+  kNoNdMfma = 1u << 9,      // DK_NO_ND_MFMA      the matrix-core N-d kernels
+};
+unsigned test_switches();  // dk_api.hip
+inline bool path_disabled(unsigned sw) { return (test_switches() & sw) != 0; }
+
+// hipFuncAttributeMaxDynamicSharedMemorySize belongs to (kernel, device) and does not change once
+// set: the first launch of a kernel on a device sets it, later launches only look it up.
+bool allow_max_dynamic_lds(const void* kernel);  // dk_api.hip
 
 // Upper bound handed to hipFuncAttributeMaxDynamicSharedMemorySize for the kernels that need more
 // than 64 KB of LDS: the attribute is per kernel, not per launch, so a launch must not lower what a

@@ -1340,7 +1340,7 @@ constexpr int kMaxLdsTables = 60 * 1024;  // bytes of LDS a workgroup may spend 
 // pixel's taps are three runs of three consecutive elements
 bool same_width_geometry(const Geo& g) {
   return g.stride_h == 1 && g.stride_w == 1 && g.dil_w == 1 && g.pad_w == 1 && g.k_w == 3 &&
-         g.in_w == g.out_w && !path_disabled("DK_NO_ROWS");
+         g.in_w == g.out_w && !path_disabled(kNoRows);
 }
 
 template <int SH, int SW>
@@ -1364,7 +1364,7 @@ int pick_splits(const Geo& g, int planes_pixels) {
 // stride 2 x 2, 3 x 3 undilated taps, padding 1, even input width: the pair-load kernels apply
 bool stride2_geometry(const Geo& g) {
   return g.stride_h == 2 && g.stride_w == 2 && g.dil_h == 1 && g.dil_w == 1 && g.pad_h == 1 && g.pad_w == 1 &&
-         g.k_h == 3 && g.k_w == 3 && g.in_w % 2 == 0 && !path_disabled("DK_NO_ROWS");
+         g.k_h == 3 && g.k_w == 3 && g.in_w % 2 == 0 && !path_disabled(kNoRows);
 }
 int rotation_tile(const Geo& g) { return same_width_geometry(g) ? kRowPix : stride2_geometry(g) ? kS2Pix : kBlock; }
 
@@ -1389,7 +1389,7 @@ bool run_gather(const Geo& g, bool transposed, const T* src, const T* rot, const
       local_gather_rows_kernel<T, 3, SH, SW, false><<<grid, row_block(pixels, kRowLanes), lds, stream>>>(g, src, rot, filter, dst, per);
     return true;
   }
-  if (transposed && stride2_geometry(g) && !path_disabled("DK_NO_S2_QUADS")) {
+  if (transposed && stride2_geometry(g) && !path_disabled(kNoS2Quads)) {
     // lanes own 2 x 2 input quads, one per output pixel
     const int quads = g.out_h * g.out_w;
     const int perq = channels_per_block<SH, SW>(cpg, pick_splits(g, quads));
@@ -1470,7 +1470,7 @@ FilterGrid filter_grid(const Geo& g) {
   f.nx = 0;
   f.th = 0;
   f.lds = 0;
-  if (same_width_geometry(g) && !path_disabled("DK_NO_MFMA")) {
+  if (same_width_geometry(g) && !path_disabled(kNoMfma)) {
     const long xt = kMfPix + 2 + 2L * g.dil_h * g.in_w;
     // a row holds 64 * nx staged elements (nx = 4 or 6 per lane) plus the skew of mf_row() (at most 51)
     const long pitch = (xt <= 256 ? 256 : 64 * kMfX) + 64;
@@ -1494,7 +1494,7 @@ FilterGrid filter_grid(const Geo& g) {
       return f;
     }
   }
-  if (stride2_geometry(g) && !path_disabled("DK_NO_MFMA") && !path_disabled("DK_NO_MFMA_S2") && g.out_w <= kMfPix) {
+  if (stride2_geometry(g) && !path_disabled(kNoMfma) && !path_disabled(kNoMfmaS2) && g.out_w <= kMfPix) {
     // tiles of whole output rows whose input rows (2 th + 1 of them, plus one element) fit the stage
     int th = std::min(kMfPix / g.out_w, g.out_h);
     while (th > 1 && (2L * th + 1) * g.in_w + 1 > 64 * kMfXS2) --th;
@@ -1542,8 +1542,7 @@ bool run_grad_filter(const Geo& g, const T* gout, const T* x, const T* rot, T* g
 #define DK_LAUNCH_BF(CELL0, BF)                                                                                  \
   if (f.th > 0) {                                                                                                \
     auto kernel = local_grad_filter_mfma_kernel<T, SH, SW, CELL0, kMfXS2, true, BF>;                             \
-    if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,  \
-                            kMaxDynamicLds) != hipSuccess)                                                           \
+    if (!allow_max_dynamic_lds(reinterpret_cast<const void*>(kernel)))                                                           \
       return false;                                                                                              \
     kernel<<<grid, kMfBlock, f.lds, stream>>>(g, gout, x, rot, ws, f.tiles, f.parts, f.splits, f.pitch_x, f.th); \
   } else if (f.nx == 4)                                                                                          \

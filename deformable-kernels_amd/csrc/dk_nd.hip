@@ -1145,7 +1145,7 @@ bool nd_use_channel_last(const dk_nd_desc& d) {
 // Bins of the counting sort (cells of low corners plus the bin of outside points), or 0 when
 // the binned kernels do not apply: they pay off with several points per cell.
 int nd_bins(const dk_nd_desc& d) {
-  if (!nd_use_channel_last(d) || path_disabled("DK_NO_ND_BINS")) return 0;
+  if (!nd_use_channel_last(d) || path_disabled(kNoNdBins)) return 0;
   long bins = 1;
   for (int i = 0; i < d.dims; ++i) bins *= (long)d.shape[i] + 1;
   bins += 1;
@@ -1238,7 +1238,7 @@ void nd_forward(const dk_nd_desc& d, const T* data, const T* coord, T* out, void
         if (!order) order = sort_points<T>(g, coord, bins, static_cast<char*>(ws) + round256(data_bytes(d) * sizeof(T)), stream);
         if constexpr (std::is_same<T, float>::value) {
           // rows of out are written as 16-byte vectors at multiples of 4 channels
-          if (g.channel % 64 == 0 && reinterpret_cast<uintptr_t>(out) % 16 == 0 && !path_disabled("DK_NO_ND_MFMA")) {
+          if (g.channel % 64 == 0 && reinterpret_cast<uintptr_t>(out) % 16 == 0 && !path_disabled(kNoNdMfma)) {
             nd_forward_mfma_kernel<T><<<(unsigned)((g.batch + 255) / 256), kBlock, 0, stream>>>(g, data_cl, coord, order, bins, out);
             return;
           }
@@ -1284,7 +1284,7 @@ void nd_grad_data(const dk_nd_desc& d, const T* gout, const T* coord, T* gdata, 
         bool on_matrix_cores = false;
         if constexpr (std::is_same<T, float>::value)
           // rows of gout are read as 16-byte vectors at multiples of 4 channels
-          on_matrix_cores = g.channel % 64 == 0 && reinterpret_cast<uintptr_t>(gout) % 16 == 0 && !path_disabled("DK_NO_ND_MFMA");
+          on_matrix_cores = g.channel % 64 == 0 && reinterpret_cast<uintptr_t>(gout) % 16 == 0 && !path_disabled(kNoNdMfma);
         if (on_matrix_cores) {
           if constexpr (std::is_same<T, float>::value)
             nd_grad_data_mfma_kernel<T><<<(unsigned)((waves + 3) / 4), kBlock, 0, stream>>>(g, gout, coord, order, bins, acc, per_wave);
@@ -1320,7 +1320,7 @@ void nd_grad_coord(const dk_nd_desc& d, const T* gout, const T* data, const T* c
         if (!order) order = sort_points<T>(g, coord, bins, static_cast<char*>(ws) + round256(data_bytes(d) * sizeof(T)), stream);
         if constexpr (std::is_same<T, float>::value) {
           // rows of gout are read as 16-byte vectors at multiples of 16 channels
-          if (g.channel % 64 == 0 && reinterpret_cast<uintptr_t>(gout) % 16 == 0 && !path_disabled("DK_NO_ND_MFMA")) {
+          if (g.channel % 64 == 0 && reinterpret_cast<uintptr_t>(gout) % 16 == 0 && !path_disabled(kNoNdMfma)) {
             nd_grad_coord_mfma_kernel<T><<<(unsigned)((g.batch + 255) / 256), kBlock, 0, stream>>>(g, gout, data_cl, coord, order, bins, gcoord);
             return;
           }

@@ -547,8 +547,7 @@ bool offset_conv_wgrad(int batch, int cin, int cout, int h, int w, const float* 
     const size_t lds_red = (size_t)NT * 256 * sizeof(float);                                                   \
     const size_t bytes = std::max(lds, lds_red);                                                               \
     if (bytes > (size_t)kMaxDynamicLds ||                                                                                  \
-        hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, \
-                            kMaxDynamicLds) != hipSuccess)                                                         \
+        !allow_max_dynamic_lds(reinterpret_cast<const void*>(kernel)))                                                         \
       ok = false;                                                                                              \
     else if (batch > 0)                                                                                        \
       kernel<<<parts * nchunks, kWgBlock, bytes, stream>>>(g, x, gout, partial, parts);                        \

@@ -47,6 +47,7 @@ _CD, _ND, _OC = ctypes.POINTER(ConvDesc), ctypes.POINTER(NdDesc), ctypes.POINTER
 # name -> (restype, argtypes); must list every symbol include/dk_hip.h declares
 SIGNATURES = {
     "dk_version": (ctypes.c_int, []),
+    "dk_test_switches": (ctypes.c_uint, [ctypes.c_uint]),
     "dk_status_string": (ctypes.c_char_p, [ctypes.c_int]),
     "dk_conv_out_size": (ctypes.c_int, [_CD, ctypes.POINTER(ctypes.c_int32), ctypes.POINTER(ctypes.c_int32)]),
     "dk_sample_depthwise_forward": (ctypes.c_int, [_CD, _P, _P, _P, _P, _P]),
@@ -144,6 +145,28 @@ def workspace(nbytes, device):
         return None, 0
     buf = torch.empty(nbytes, dtype=torch.uint8, device=device)
     return buf, nbytes
+
+
+TEST_SWITCHES = ("DK_NO_ROWS", "DK_NO_MFMA", "DK_NO_MFMA_S2", "DK_NO_S2_QUADS", "DK_NO_DEFORM_FAST",
+                 "DK_NO_DEFORM_CH", "DK_NO_DEFORM_CH_BIG", "DK_NO_DEFORM_MFMA", "DK_NO_ND_BINS", "DK_NO_ND_MFMA")
+
+
+class test_switches:
+    """Context manager for tests: run the enclosed calls with the named kernel families switched off
+    (``dk_test_switches`` in ``include/dk_hip.h``), then restore the previous mask."""
+
+    def __init__(self, *names):
+        self.mask = 0
+        for n in names:
+            self.mask |= 1 << TEST_SWITCHES.index(n)
+
+    def __enter__(self):
+        self.before = lib().dk_test_switches(self.mask)
+        return self
+
+    def __exit__(self, *exc):
+        lib().dk_test_switches(self.before)
+        return False
 
 
 CLIP_NONE, CLIP_ROTATION, CLIP_COORD = 0, 1, 2

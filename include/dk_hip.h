@@ -20,7 +20,7 @@
  *     reference's filter/data gradients accumulate atomically into buffers
  *     its Python caller zero-fills -- functions/filter_sample_depthwise.py:64-80);
  *   - calls are asynchronous on `stream`, thread-safe and hold no global
- *     mutable state;
+ *     mutable state (apart from the test hook dk_test_switches());
  *   - the return value is DK_OK (0) or a negative dk_status; nothing is
  *     launched when an argument is rejected.  (The reference validates
  *     nothing and always returns 1 -- filter_sample_depthwise_cuda.cpp:61.)
@@ -285,6 +285,16 @@ int dk_offset_conv_backward_bias(const dk_offset_conv_desc *desc, const void *ou
 /* ---- misc ------------------------------------------------------------------- */
 
 const char *dk_status_string(int status);
+
+/* Test hook, not for production use: a bit mask that makes the dispatch skip a specialised kernel
+ * family and run the next more general one for the same shape, so that tests can reach every
+ * kernel.  Bit i belongs to the i-th of DK_NO_ROWS, DK_NO_MFMA, DK_NO_MFMA_S2, DK_NO_S2_QUADS,
+ * DK_NO_DEFORM_FAST, DK_NO_DEFORM_CH, DK_NO_DEFORM_CH_BIG, DK_NO_DEFORM_MFMA, DK_NO_ND_BINS,
+ * DK_NO_ND_MFMA.  The mask starts from the environment variables of those names, read once
+ * (at the first call that consults it); this call replaces it and returns the previous mask.
+ * Workspace queries consult it too: query and call must see the same mask.  The one piece of
+ * process-wide state in the library. */
+unsigned dk_test_switches(unsigned mask);
 
 /* Library version, (major << 16) | minor. */
 int dk_version(void);

@@ -30,3 +30,21 @@ def pytest_collection_modifyitems(config, items):
     for item in items:
         if "gpu" in item.keywords:
             item.add_marker(skip)
+
+
+@pytest.fixture
+def switch_off():
+    """`switch_off("DK_NO_MFMA", ...)` switches the named kernel families of the library off (its test
+    hook dk_test_switches) until the test ends, so that the next more general kernels serve the call."""
+    from deformable_kernels.ops.deform_kernel import _lib
+    before = _lib.lib().dk_test_switches(0)
+    _lib.lib().dk_test_switches(before)
+    active = [before]
+
+    def off(*names):
+        for n in names:
+            active[0] |= 1 << _lib.TEST_SWITCHES.index(n)
+        _lib.lib().dk_test_switches(active[0])
+
+    yield off
+    _lib.lib().dk_test_switches(before)

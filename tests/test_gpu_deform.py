@@ -11,7 +11,7 @@ import numpy as np
 import pytest
 import torch
 
-from _cases import clipped_rotation, make_deform, rel_err
+from _cases import mixed_err, clipped_rotation, make_deform, rel_err
 from oracle import dk_oracle as orc
 
 pytestmark = pytest.mark.gpu
@@ -60,7 +60,9 @@ def _oracle(inputs, np_dtype):
 
 def assert_fp32_parity(got, o32, o64):
     assert rel_err(got[0], o32[0]) < 1e-5, NAMES[0]
-    for i in (1, 3, 4):
+    # grad input: fixed-point sums, exact on a grid of 2^-24 of the largest term or finer
+    assert mixed_err(got[1], o64[1]) < 1e-5, NAMES[1]
+    for i in (3, 4):
         assert rel_err(got[i], o64[i]) < 1e-4, NAMES[i]
     # The offset gradient is the slope of the bilinear patch a sample falls in, so it jumps where a
     # sampling position crosses a grid line; a position that fp32 rounds onto the line (36 + 0.9999987
@@ -214,10 +216,10 @@ def test_config4_properties_at_full_size():
 
 @pytest.mark.parametrize("switch,case", [("DK_NO_DEFORM_CH", CASES[0]), ("DK_NO_DEFORM_MFMA", CASES[0]),
                                          ("DK_NO_DEFORM_CH_BIG", CASES[7])])
-def test_one_plane_kernels_on_a_shape_the_newer_ones_cover(monkeypatch, switch, case):
+def test_one_plane_kernels_on_a_shape_the_newer_ones_cover(switch_off, switch, case):
     """Without the channel-interleaved kernels (those for small planes and those for large ones) / the
     matrix-core grad filter the one-plane kernels serve the shape."""
-    monkeypatch.setenv(switch, "1")
+    switch_off(switch)
     inputs, got = _run(case, torch.float32)
     o32, o64 = _oracle(inputs, np.float32), _oracle(inputs, np.float64)
     assert rel_err(got[0], o32[0]) < 1e-5
@@ -225,11 +227,44 @@ def test_one_plane_kernels_on_a_shape_the_newer_ones_cover(monkeypatch, switch, 
         assert rel_err(got[i], o64[i]) < 1e-4, NAMES[i]
 
 
-def test_generic_kernels_on_a_shape_the_tuned_ones_cover(monkeypatch):
+def test_generic_kernels_on_a_shape_the_tuned_ones_cover(switch_off):
     """With the tuned deformable kernels switched off the generic ones serve the same shape."""
-    monkeypatch.setenv("DK_NO_DEFORM_FAST", "1")
+    switch_off("DK_NO_DEFORM_FAST")
     inputs, got = _run(CASES[0], torch.float32)
     o32, o64 = _oracle(inputs, np.float32), _oracle(inputs, np.float64)
     assert rel_err(got[0], o32[0]) < 1e-5
     for i in range(1, 5):
         assert rel_err(got[i], o64[i]) < 1e-4, NAMES[i]
+
+
+@pytest.mark.parametrize("case", [CASES[0], CASES[10]])  # one plane per workgroup; tiled planes above 1024 pixels
+@pytest.mark.parametrize("poison", [float("inf"), float("nan")])
+@pytest.mark.parametrize("where", ["out_grad", "filter"])
+def test_non_finite_values_reach_the_input_gradient(case, poison, where):
+    """The tuned grad-input kernels add fixed-point integers whose scale comes from max|out_grad| and
+    max|filter[c]|; an infinity or a NaN there must not come back as finite numbers (the reference's
+    float atomics carry it to the elements it touches; loss scaling only asks whether any gradient
+    is non-finite).  out_grad: the whole input gradient is NaN; filter: at least the poisoned
+    channel's planes are, and the planes of other channel chunks stay finite."""
+    from deformable_kernels.ops.deform_kernel import _lib
+    L, P = _lib.lib(), _lib.ptr
+    N, C, H, W, k, S, s, p, d, G, rs, os_ = case
+    x, wt, rot, off, gout, cfg = make_deform(N, C, H, W, k, S, s, p, d, G, rs, os_, seed=9)
+    if where == "out_grad":
+        gout[N - 1, C // 2, 3, 4] = poison
+    else:
+        wt[1, 0, 2, 1] = poison
+    dev = torch.device("cuda:0")
+    wg, rg, og, gg = [t.to(dev) for t in (wt, rot, off, gout)]
+    xs = torch.empty(N, C, H, W, device=dev)
+    desc = _lib.conv_desc(xs, wg, cfg["kernel_size"], cfg["stride"], cfg["padding"], cfg["dilation"], G)
+    ws, nbytes = _lib.workspace(L.dk_deformable_sample_depthwise_backward_data_workspace(desc), dev)
+    gin = torch.zeros_like(xs)
+    _lib.check(L.dk_deformable_sample_depthwise_backward_data(
+        desc, P(gg), P(og), P(rg), P(wg), P(gin), P(ws), nbytes, torch.cuda.current_stream().cuda_stream), "data")
+    torch.cuda.synchronize()
+    bad = ~torch.isfinite(gin)
+    if where == "out_grad":
+        assert bool(bad[N - 1, C // 2].any())   # where the reference's atomics would have put it
+    else:
+        assert bool(bad[:, 1].any())

@@ -226,11 +226,11 @@ def test_headline_shape_properties_at_full_size():
 
 
 @pytest.mark.parametrize("switch", ["DK_NO_MFMA", "DK_NO_ROWS"])
-def test_more_general_kernels_on_a_same_width_shape(switch, monkeypatch):
+def test_more_general_kernels_on_a_same_width_shape(switch, switch_off):
     """The dispatch prefers the most specialised kernel; the library's test switches make it take
     the next more general family for the same shape (dense grad filter instead of the
     matrix-core one; per-tap loads instead of the row kernels), which must give the same results."""
-    monkeypatch.setenv(switch, "1")
+    switch_off(switch)
     case = (2, 40, 20, 24, 3, (4, 4), 1, 1, 1, 2, 1.0)
     inputs, got = _run(case, torch.float32)
     o32, o64 = _oracle(inputs, np.float32), _oracle(inputs, np.float64)
@@ -241,10 +241,10 @@ def test_more_general_kernels_on_a_same_width_shape(switch, monkeypatch):
 
 
 @pytest.mark.parametrize("switch", ["DK_NO_MFMA_S2", "DK_NO_S2_QUADS"])
-def test_more_general_kernels_on_a_stride_2_shape(switch, monkeypatch):
+def test_more_general_kernels_on_a_stride_2_shape(switch, switch_off):
     """Stride 2, padding 1, even width: the dense pair-load grad filter instead of the matrix-core one,
     the gather over input pixels instead of the one over 2 x 2 input quads."""
-    monkeypatch.setenv(switch, "1")
+    switch_off(switch)
     case = (2, 24, 22, 20, 3, (4, 4), 2, 1, 1, 2, 1.0)
     inputs, got = _run(case, torch.float32)
     o32, o64 = _oracle(inputs, np.float32), _oracle(inputs, np.float64)

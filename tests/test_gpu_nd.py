@@ -87,27 +87,27 @@ def test_many_points_on_grid_nodes_and_half_way_between():
     assert rel_err(got[2], o64[2]) < 1e-4
 
 
-def test_sorted_and_unsorted_kernels_agree(monkeypatch):
+def test_sorted_and_unsorted_kernels_agree(switch_off):
     g = torch.Generator().manual_seed(46)
     data = torch.randn(64, 8, 8, 8, generator=g)
     coord = torch.rand(70000, 3, generator=g) * 10.0 - 1.0
     gout = torch.randn(70000, 64, generator=g)
     a = _run(data, coord, gout)
-    monkeypatch.setenv("DK_NO_ND_BINS", "1")
+    switch_off("DK_NO_ND_BINS")
     b = _run(data, coord, gout)
     assert rel_err(a[0], b[0]) < 1e-6  # the same eight products per point and channel, summed in another order
     assert rel_err(a[1], b[1]) < 1e-5
     assert rel_err(a[2], b[2]) < 1e-5
 
 
-def test_sorted_kernels_with_and_without_the_matrix_cores_agree(monkeypatch):
+def test_sorted_kernels_with_and_without_the_matrix_cores_agree(switch_off):
     """64 channels in fp32 take the matrix-core kernels; switched off, the VALU kernels serve the same call."""
     g = torch.Generator().manual_seed(47)
     data = torch.randn(64, 7, 9, 8, generator=g)
     coord = torch.rand(66000, 3, generator=g) * 11.0 - 1.5
     gout = torch.randn(66000, 64, generator=g)
     a = _run(data, coord, gout)
-    monkeypatch.setenv("DK_NO_ND_MFMA", "1")
+    switch_off("DK_NO_ND_MFMA")
     b = _run(data, coord, gout)
     want = _oracle(data, coord, gout, np.float64)
     for x, y, w in zip(a, b, want):
