@@ -6,6 +6,7 @@
 #include <algorithm>
 #include <atomic>
 #include <cstdlib>
+#include <initializer_list>
 #include <mutex>
 #include <utility>
 #include <vector>
@@ -82,12 +83,19 @@ int make_geo(const dk_conv_desc* d, Geo& g) {
   if ((long)d->in_h + 2L * d->pad_h < (long)d->dil_h * (d->k_h - 1) + 1 ||
       (long)d->in_w + 2L * d->pad_w < (long)d->dil_w * (d->k_w - 1) + 1 || oh <= 0 || ow <= 0)
     return DK_ERR_BAD_SHAPE;
-  const long taps2 = 2L * d->k_h * d->k_w;
-  if ((long)d->batch * d->channel * d->in_h * d->in_w > kMaxElems ||
-      (long)d->batch * d->channel * oh * ow > kMaxElems ||
-      (long)d->batch * d->groups * taps2 * oh * ow > kMaxElems ||
-      (long)d->batch * d->channel * taps2 / 2 * oh * ow > 4 * kMaxElems ||
-      (long)d->channel * d->scope_h * d->scope_w > kMaxElems)
+  // element counts as saturating products: the factors are only known to be positive 32-bit
+  // numbers here, and four of them can exceed 64 bits
+  auto count = [](std::initializer_list<long> f) {
+    long p = 1;
+    for (long v : f) p = (v != 0 && p > (1L << 62) / v) ? (1L << 62) : p * v;
+    return p;
+  };
+  const long taps = count({d->k_h, d->k_w});
+  if (count({d->batch, d->channel, d->in_h, d->in_w}) > kMaxElems ||
+      count({d->batch, d->channel, oh, ow}) > kMaxElems ||
+      count({d->batch, d->groups, 2, taps, oh, ow}) > kMaxElems ||
+      count({d->batch, d->channel, taps, oh, ow}) > 4 * kMaxElems ||
+      count({d->channel, d->scope_h, d->scope_w}) > kMaxElems)
     return DK_ERR_TOO_LARGE;
   g.batch = d->batch;
   g.channel = d->channel;

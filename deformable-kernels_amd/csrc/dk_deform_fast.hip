@@ -1322,7 +1322,7 @@ DeformPlan deform_plan(const Geo& g, int table_floats, int planes, int block, in
   if (room < (long)table_floats * 4 * 4) return d;
   const int fit = (int)std::min<long>(room / ((long)table_floats * 4), cpg);
   // enough blocks for blocks_per_cu per CU, chunks of at least 8 channels
-  const long base = (long)d.tiles * g.batch * g.groups;
+  const long base = std::max(1L, (long)d.tiles * g.batch * g.groups);  // batch may be 0
   int chunks = (int)std::max<long>(1, (blocks_per_cu * 256L + base - 1) / base);
   chunks = std::min(chunks, std::max(1, cpg / 8));
   chunks = std::max(chunks, ceil_div(cpg, fit));
@@ -1504,7 +1504,7 @@ GradFilterMfma grad_filter_mfma_plan(const Geo& g) {
   m.lds = (size_t)floats * 4;
   m.tiles = ceil_div(g.out_h * g.out_w, kGfPix);
   const int nblk = ceil_div(g.channel / g.groups, kGfCh);
-  const long base = (long)m.tiles * g.batch * g.groups;
+  const long base = std::max(1L, (long)m.tiles * g.batch * g.groups);  // batch may be 0
   // one workgroup per CU, all resident at once: the set-up of a workgroup (descriptors, hat products,
   // zero fill) costs about as much as two channel blocks (measured: 256 workgroups 73 us, 512: 79, 1024: 93)
   m.csplits = (int)std::max<long>(1, std::min<long>(nblk, (256 + base - 1) / base));

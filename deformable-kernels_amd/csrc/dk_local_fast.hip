@@ -1421,7 +1421,7 @@ bool run_gather(const Geo& g, bool transposed, const T* src, const T* rot, const
 // 16 channels per split.
 int rotation_splits(const Geo& g) {
   const int cpg = g.channel / g.groups;
-  const long base = (long)ceil_div(g.out_h * g.out_w, rotation_tile(g)) * g.batch * g.groups;
+  const long base = std::max(1L, (long)ceil_div(g.out_h * g.out_w, rotation_tile(g)) * g.batch * g.groups);  // batch may be 0
   const long want = 1024 / base;  // measured: about four blocks per CU is the best grid
   return (int)std::max<long>(1, std::min<long>(want, cpg / 16));
 }

@@ -454,7 +454,7 @@ bool offset_conv_supported(int cin, int cout, int h, int w) {
 // chunks of 16 channels per split
 int forward_splits(int batch, int cin, int h, int w) {
   const int th = w <= 56 ? 8 : 4;
-  const long base = (long)batch * ceil_div(h, th);
+  const long base = std::max(1L, (long)batch * ceil_div(h, th));  // batch may be 0
   if (base >= 384) return 1;
   return (int)std::max<long>(1, std::min<long>((512 + base - 1) / base, cin / kCvChunk / 2));
 }

@@ -109,6 +109,22 @@ def test_c_abi_rejects_bad_arguments_before_any_launch():
     assert b"workspace" in L.dk_status_string(-5)
 
 
+def test_native_self_tests_of_the_c_abi_and_the_oracle():
+    """The C driver of the C ABI's argument handling (every rejection path and the workspace arithmetic
+    over a sweep of geometries; all answered on the host) against the library as built, and the oracle's
+    own driver under AddressSanitizer + UndefinedBehaviorSanitizer.  (`make -C deformable-kernels_amd/csrc
+    sanitize` runs the first one with the library's host code under the sanitizers as well: a build of
+    minutes, not part of this suite.)"""
+    import os
+    import subprocess
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    r = subprocess.run(["make", "-s", "-C", os.path.join(root, "deformable-kernels_amd", "csrc"), "selftest"],
+                       capture_output=True, text=True)
+    assert r.returncode == 0 and "abi selftest ok" in r.stdout, r.stdout[-2000:] + r.stderr[-2000:]
+    r = subprocess.run(["make", "-s", "-C", os.path.join(root, "oracle"), "sanitize"], capture_output=True, text=True)
+    assert r.returncode == 0 and "oracle selftest ok" in r.stdout, r.stdout[-2000:] + r.stderr[-2000:]
+
+
 @pytest.mark.gpu
 def test_local_module_matches_composite_and_backpropagates():
     from deformable_kernels.modules import DeformKernel2d
