@@ -38,6 +38,15 @@ def _centred_tap_grid(weight_shape, kernel_size, weight_dilate):
     return grid
 
 
+def _plain_conv(conv):
+    """Whether calling ``offset_conv`` on the convolution's parameters is the same as calling the
+    module: no forward / pre-forward / backward hooks on it (hook-based weight or spectral
+    norm, profilers and quantisation observers rely on the module call) and ordinary zero padding."""
+    hooks = (conv._forward_hooks, conv._forward_pre_hooks, conv._backward_hooks,
+             getattr(conv, "_backward_pre_hooks", {}))
+    return not any(len(h) for h in hooks) and conv.padding_mode == 'zeros' and conv.groups == 1
+
+
 class GlobalDeformKernel2d(nn.Module):
     """One set of kernel-space offsets per image, predicted from the pooled
     input; the per-image kernels are sampled with ``nd_linear_sample`` and
@@ -199,7 +208,7 @@ class LocalDeformKernel2d(nn.Module):
 
     def forward(self, x):
         conv = self.rotation_conv
-        if self.native_offset_conv:
+        if self.native_offset_conv and _plain_conv(conv):
             rotation = offset_conv(x, conv.weight, conv.bias, conv.stride, conv.padding, conv.dilation)
         else:
             rotation = conv(x)
@@ -252,7 +261,7 @@ class DeformKernelConv2d(nn.Module):
 
     def forward(self, x):
         conv = self.offset_conv
-        if self.native_offset_conv:
+        if self.native_offset_conv and _plain_conv(conv):
             offset = offset_conv(x, conv.weight, conv.bias, conv.stride, conv.padding, conv.dilation)
         else:
             offset = conv(x)

@@ -20,6 +20,7 @@ Differences a user can observe:
 """
 import torch
 from torch.autograd import Function
+from torch.autograd.function import once_differentiable
 
 from .. import _lib
 
@@ -96,6 +97,7 @@ class SampleDepthwiseFunction(Function):
         return output
 
     @staticmethod
+    @once_differentiable  # the kernels are not differentiable a second time: asking for it raises
     def backward(ctx, grad_output):
         input, rotation, weight = ctx.saved_tensors
         grad_input = grad_rotation = grad_weight = None
@@ -162,6 +164,7 @@ class DeformableSampleDepthwiseFunction(Function):
         return output
 
     @staticmethod
+    @once_differentiable  # the kernels are not differentiable a second time: asking for it raises
     def backward(ctx, grad_output):
         input, offset, rotation, weight = ctx.saved_tensors
         grad_input = grad_offset = grad_rotation = grad_weight = None

@@ -10,6 +10,7 @@ summed over channels (the reference sums a ``[B, n, C]`` buffer in Python,
 """
 import torch
 from torch.autograd import Function
+from torch.autograd.function import once_differentiable
 
 from .. import _lib
 
@@ -46,6 +47,7 @@ class NdLinearSampleFunction(Function):
         return output
 
     @staticmethod
+    @once_differentiable  # the kernels are not differentiable a second time: asking for it raises
     def backward(ctx, grad_output):
         input, coord = ctx.saved_tensors
         grad_input = grad_coord = None

@@ -18,6 +18,7 @@ Other dtypes, CPU tensors and autocast regions go to ``F.conv2d`` unchanged.
 import torch
 import torch.nn.functional as F
 from torch.autograd import Function
+from torch.autograd.function import once_differentiable
 
 from .. import _lib
 
@@ -76,6 +77,7 @@ class OffsetConvFunction(Function):
         return out
 
     @staticmethod
+    @once_differentiable  # the kernels are not differentiable a second time: asking for it raises
     def backward(ctx, grad_output):
         input, weight = ctx.saved_tensors
         stride, padding, dilation = ctx.conv

@@ -61,6 +61,20 @@ def test_cpu_tensors_are_rejected_like_the_reference():
         m(torch.randn(1, 4, 6, 6))
 
 
+def test_hooks_on_the_offset_branch_convolution_fire():
+    """A forward hook on rotation_conv / offset_conv (weight norm, profilers, quantisation observers)
+    relies on the convolution being called as a module: the library's own offset-branch kernels,
+    which take the parameters directly, are only used on a convolution without hooks."""
+    from deformable_kernels.modules import DeformKernel2d, DeformKernelConv2d
+    for m, conv in ((lambda m: (m, m.rotation_conv))(DeformKernel2d((4, 4), 4, 4, 3, 1, 1, groups=4)),
+                    (lambda m: (m, m.offset_conv))(DeformKernelConv2d((4, 4), 4, 4, 3, 1, 1, groups=4))):
+        seen = []
+        conv.register_forward_hook(lambda mod, i, o: seen.append(tuple(o.shape)))
+        with pytest.raises(NotImplementedError):   # the operator itself exists on the GPU only
+            m(torch.randn(1, 4, 6, 6))
+        assert seen == [(1, 18, 6, 6)]
+
+
 def test_c_abi_exports_every_declared_symbol():
     import ctypes
     import os
