@@ -27,7 +27,7 @@ unsigned switches_from_environment() {
       {"DK_NO_ROWS", kNoRows}, {"DK_NO_MFMA", kNoMfma}, {"DK_NO_MFMA_S2", kNoMfmaS2},
       {"DK_NO_S2_QUADS", kNoS2Quads}, {"DK_NO_DEFORM_FAST", kNoDeformFast}, {"DK_NO_DEFORM_CH", kNoDeformCh},
       {"DK_NO_DEFORM_CH_BIG", kNoDeformChBig}, {"DK_NO_DEFORM_MFMA", kNoDeformMfma},
-      {"DK_NO_ND_BINS", kNoNdBins}, {"DK_NO_ND_MFMA", kNoNdMfma}};
+      {"DK_NO_ND_BINS", kNoNdBins}, {"DK_NO_ND_MFMA", kNoNdMfma}, {"DK_NO_GATHER_MFMA", kNoGatherMfma}};
   unsigned m = 0;
   for (const auto& v : vars)
     if (std::getenv(v.name)) m |= v.bit;
@@ -35,7 +35,8 @@ unsigned switches_from_environment() {
 }
 
 std::mutex g_lds_mutex;
-std::vector<std::pair<const void*, int>> g_lds_allowed;  // (kernel, device) pairs already set
+struct LdsAllowed { const void* kernel; int device, bytes; };
+std::vector<LdsAllowed> g_lds_allowed;  // what has been set so far
 }  // namespace
 
 unsigned test_switches() {
@@ -48,17 +49,23 @@ unsigned test_switches() {
   return m;
 }
 
-bool allow_max_dynamic_lds(const void* kernel) {
+bool allow_dynamic_lds(const void* kernel, int bytes) {
   int dev = -1;
   if (hipGetDevice(&dev) != hipSuccess) return false;
   std::lock_guard<std::mutex> lock(g_lds_mutex);
-  for (const auto& e : g_lds_allowed)
-    if (e.first == kernel && e.second == dev) return true;
-  if (hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, kMaxDynamicLds) != hipSuccess)
-    return false;
-  g_lds_allowed.emplace_back(kernel, dev);
+  for (auto& e : g_lds_allowed)
+    if (e.kernel == kernel && e.device == dev) {
+      if (e.bytes >= bytes) return true;
+      if (hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes) != hipSuccess) return false;
+      e.bytes = bytes;  // only ever raised: a concurrent launch may rely on the old value
+      return true;
+    }
+  if (hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes) != hipSuccess) return false;
+  g_lds_allowed.push_back({kernel, dev, bytes});
   return true;
 }
+
+bool allow_max_dynamic_lds(const void* kernel) { return allow_dynamic_lds(kernel, kMaxDynamicLds); }
 
 }  // namespace dk
 

@@ -26,6 +26,7 @@ enum TestSwitch : unsigned {
   kNoDeformMfma = 1u << 7,  // DK_NO_DEFORM_MFMA  the matrix-core deformable grad filter
   kNoNdBins = 1u << 8,      // DK_NO_ND_BINS      the N-d kernels that sort the points by cell
   kNoNdMfma = 1u << 9,      // DK_NO_ND_MFMA      the matrix-core N-d kernels
+  kNoGatherMfma = 1u << 10, // DK_NO_GATHER_MFMA  the matrix-core forward / grad input (the row kernels run instead)
 };
 unsigned test_switches();  // dk_api.hip
 inline bool path_disabled(unsigned sw) { return (test_switches() & sw) != 0; }
@@ -33,6 +34,9 @@ inline bool path_disabled(unsigned sw) { return (test_switches() & sw) != 0; }
 // hipFuncAttributeMaxDynamicSharedMemorySize belongs to (kernel, device) and does not change once
 // set: the first launch of a kernel on a device sets it, later launches only look it up.
 bool allow_max_dynamic_lds(const void* kernel);  // dk_api.hip
+// The same with a given bound, for kernels whose static LDS arrays leave less room (the bound is only
+// ever raised).
+bool allow_dynamic_lds(const void* kernel, int bytes);
 
 // Upper bound handed to hipFuncAttributeMaxDynamicSharedMemorySize for the kernels that need more
 // than 64 KB of LDS: the attribute is per kernel, not per launch, so a launch must not lower what a
@@ -42,6 +46,11 @@ constexpr int kMaxDynamicLds = 152 * 1024;
 
 template <typename CT, typename T>
 void launch_reduce_partials(const CT* partial, int parts, long count, T* out, hipStream_t stream);
+
+// ---- forward / grad input on the matrix cores (dk_local_mfma.hip): same-width geometries, scope <= 16 cells
+template <typename T>
+bool mfma_local_gather(const Geo& g, bool transposed, const T* src, const T* rot, const T* filter, T* dst,
+                       hipStream_t stream);
 
 // ---- tuned local path (dk_local_fast.hip): 3x3 taps, scope 3x3 / 4x4 / 5x5, fp32/fp16/bf16
 template <typename T>

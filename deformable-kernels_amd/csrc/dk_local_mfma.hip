@@ -1,0 +1,538 @@
+// Local deformable kernel on the matrix cores, for "same-width" geometries (3 x 3 taps, stride 1,
+// unit column spacing, pad_w = 1: input and output planes share their width) and scopes of at
+// most 16 cells: forward and grad input (K.cu:270-386, 577-669; K.cu =
+// deformable_kernels/ops/deform_kernel/csrc/filter_sample_depthwise_cuda_kernel.cu).
+//
+// The bilinear read of a channel's scope tile is a dense contraction over the tile's cells,
+//   w_eff[(pixel, tap)][c] = sum_cell A[(pixel, tap)][cell] * Wt[cell][c],
+//   A[(p, t)][cell = (i, j)] = hat(h_pt - i) * hat(w_pt - j)          (channel independent),
+// with at most four non-zero A per row (K.cu:51-83 writes the same sum corner by corner).  On
+// the vector ALU the sparse form wins (three FMAs per weight from a 16-byte LDS table gather), but
+// those gathers and FMAs are what bounds the gather kernels of dk_local_fast.hip -- LDS pipe and
+// VALU issue both sit at the HBM time -- while the matrix pipe idles.  16-bit matrix instructions
+// run beside VALU work of other waves (measured: a v_mfma_f32_16x16x32_f16 adds about 6 clk to a
+// SIMD that is busy with FMAs; the fp32 instruction takes its 32 clk from the same issue slots), so
+// the dense product goes there, in split precision:
+//   fp32 tensors   A = Ah + Al, Wt * s = Wh + Wl in fp16 (s a power of two per channel, so that the
+//                  tile's largest entry lies in [0.5, 1)), three products Ah Wh + Al Wh + Ah Wl with
+//                  fp32 sums -- the dropped terms are below 2^-21 of the channel's largest weight;
+//   fp16 / bf16    A = Ah + Al in the tensor's type, Wt as it is: two products.
+// Ah Wh + Al Wh is one K = 32 instruction ([Ah | Al] against [Wh ; Wh]), Ah Wl another ([Wl ; 0]).
+//
+// A unit of work is (image, 128-pixel tile, block of 16 channels); a workgroup of 8 waves walks
+// units, channel block fastest; wave w owns pixels 16 w .. 16 w + 15 of the tile.
+//   * per workgroup: every channel block's split filter operands go to LDS once;
+//   * per tile: the scope coordinates (h, w) of the (pixel, tap) pairs go to LDS and every lane
+//     derives the A operands of its pixel (l % 16) and its four cells (4 (l / 16) ..), 36 registers,
+//     kept for all channel blocks of the tile;
+//   * per unit: the 16 channels' source tiles with their halo rows are staged channel-major in LDS
+//     from loads coalesced along pixels (issued one unit ahead, into registers); per tap two or
+//     three matrix instructions leave w_eff[pixels 4 kg .. 4 kg + 3][channel q] in lane (kg, q),
+//     which holds the same channel's inputs for those pixels: four FMAs per tap.
+// grad input is the same kernel on the transposed geometry: the lane owns input pixels, tap t is fed
+// by output pixel o = q + pad - f * dil and uses o's rotation (K.cu:611-651), so the coordinate
+// table covers the staged range of output pixels instead of the tile.
+#include <algorithm>
+
+#include "dk_kernels.h"
+
+namespace dk {
+
+namespace {
+
+constexpr int kPix = 128;     // pixels per tile
+constexpr int kCh = 16;       // channels per unit
+constexpr int kThreads = 512;
+constexpr int kWaves = kThreads / 64;
+constexpr int kMaxX = 6;      // staged source elements per lane and channel: tile + halo rows <= 64 * kMaxX
+
+typedef float f4 __attribute__((ext_vector_type(4)));
+
+// The matrix element type of a tensor type and its two instruction shapes.
+// Both run as one K = 32 matrix instruction per product pair.  They are issued from inline
+// assembly, three taps at a time, because the result registers must not overlap the operands: the
+// compiler lets the result of a 4-register MFMA share registers with an operand at the operand's
+// last use (`v_mfma_f32_16x16x32_f16 v[156:159], v[32:35], v[154:157], 0` is what the builtin
+// produced), and on gfx950 rows 0 and 1 of such a result came out as garbage.  "=&v" (early
+// clobber) rules the overlap out.  What the compiler's hazard recogniser would otherwise insert is
+// written out: the second instruction on a result follows two independent ones (its SrcC is
+// complete by then), and s_nop 7 after the last one covers the 4-pass instruction's 7 wait states
+// before a vector ALU instruction may read the result.
+template <typename E> struct Mx;
+template <> struct Mx<_Float16> {
+  typedef _Float16 v4 __attribute__((ext_vector_type(4)));
+  typedef _Float16 v8 __attribute__((ext_vector_type(8)));
+  // d_i = a_i * b0 (+ a_i * b1): rows = the 16 pixels, columns = the 16 channels
+  template <bool SECOND>
+  static __device__ __forceinline__ void row(f4& d0, f4& d1, f4& d2, v8 a0, v8 a1, v8 a2, v8 b0, v8 b1) {
+    if constexpr (SECOND)
+      asm volatile(
+          "s_nop 1\n\t"
+          "v_mfma_f32_16x16x32_f16 %0, %3, %6, 0\n\t"
+          "v_mfma_f32_16x16x32_f16 %1, %4, %6, 0\n\t"
+          "v_mfma_f32_16x16x32_f16 %2, %5, %6, 0\n\t"
+          "v_mfma_f32_16x16x32_f16 %0, %3, %7, %0\n\t"
+          "v_mfma_f32_16x16x32_f16 %1, %4, %7, %1\n\t"
+          "v_mfma_f32_16x16x32_f16 %2, %5, %7, %2\n\t"
+          "s_nop 7"
+          : "=&v"(d0), "=&v"(d1), "=&v"(d2)
+          : "v"(a0), "v"(a1), "v"(a2), "v"(b0), "v"(b1));
+    else
+      asm volatile(
+          "s_nop 1\n\t"
+          "v_mfma_f32_16x16x32_f16 %0, %3, %6, 0\n\t"
+          "v_mfma_f32_16x16x32_f16 %1, %4, %6, 0\n\t"
+          "v_mfma_f32_16x16x32_f16 %2, %5, %6, 0\n\t"
+          "s_nop 7"
+          : "=&v"(d0), "=&v"(d1), "=&v"(d2)
+          : "v"(a0), "v"(a1), "v"(a2), "v"(b0));
+  }
+};
+template <> struct Mx<__bf16> {
+  typedef __bf16 v4 __attribute__((ext_vector_type(4)));
+  typedef __bf16 v8 __attribute__((ext_vector_type(8)));
+  template <bool SECOND>
+  static __device__ __forceinline__ void row(f4& d0, f4& d1, f4& d2, v8 a0, v8 a1, v8 a2, v8 b0, v8 b1) {
+    static_assert(!SECOND, "bfloat16 tensors need no second product");
+    asm volatile(
+        "s_nop 1\n\t"
+        "v_mfma_f32_16x16x32_bf16 %0, %3, %6, 0\n\t"
+        "v_mfma_f32_16x16x32_bf16 %1, %4, %6, 0\n\t"
+        "v_mfma_f32_16x16x32_bf16 %2, %5, %6, 0\n\t"
+        "s_nop 7"
+        : "=&v"(d0), "=&v"(d1), "=&v"(d2)
+        : "v"(a0), "v"(a1), "v"(a2), "v"(b0));
+  }
+};
+template <typename T> struct MxOf { using type = _Float16; };  // float, __half
+template <> struct MxOf<bf16_t> { using type = __bf16; };
+
+// v = hi + lo + (an error below 2^-2p |v| for a p-bit type), both parts in the matrix type.
+// The empty asm pins v as one fp32 value: where v is a product the compiler otherwise contracts
+// it into the conversions -- hi packed from the fp32-rounded product, lo taken against the once-rounded
+// exact product (v_fma_mixlo_f16) -- and the two roundings of hi differ by one unit in the last
+// place about once in 4096 values, which leaves a hi + lo that is off by that unit.
+template <typename E>
+__device__ __forceinline__ void split2(float v, E& hi, E& lo) {
+  asm volatile("" : "+v"(v));
+  hi = static_cast<E>(v);
+  lo = static_cast<E>(v - static_cast<float>(hi));
+}
+
+__device__ __forceinline__ float hat(float d) { return __builtin_amdgcn_fmed3f(1.f - fabsf(d), 0.f, 1.f); }
+
+// First slot of channel j's row in the staged source tile.  Rows are a multiple of 64 slots
+// apart plus a skew: lane (channel q, pixel quad kg) reads row q at 4 kg + const, and
+// (q % 4) + 16 (q / 4) + 4 kg covers the 64 banks exactly once.
+__device__ __forceinline__ constexpr int tile_row(int j, int pitch) { return j * pitch + (j & 3) + 16 * (j >> 2); }
+
+// A staged element: the tile holds one 32-bit slot per element, written by the buffer load itself
+// (a 2-byte load leaves the element zero-extended in its slot).
+__device__ __forceinline__ float slot_value(unsigned bits, const float*) { return __uint_as_float(bits); }
+__device__ __forceinline__ float slot_value(unsigned bits, const bf16_t*) { return __uint_as_float(bits << 16); }
+__device__ __forceinline__ float slot_value(unsigned bits, const __half*) {
+  return static_cast<float>(__builtin_bit_cast(_Float16, static_cast<unsigned short>(bits)));
+}
+
+typedef __attribute__((address_space(3))) void* lds_void_ptr;
+
+// Wait until at most N of this wave's vector-memory operations are outstanding and its LDS
+// operations are done, then the workgroup barrier.  __syncthreads() would do, but it waits for
+// ALL outstanding vector-memory operations, and the point of the staging scheme below is that the
+// loads of the unit after next stay in flight across the barrier.
+template <int N>
+__device__ __forceinline__ void wait_barrier() {
+  asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(N) : "memory");
+}
+
+// One unit of work, and whether it is the first of its tile that this workgroup handles.
+struct Unit {
+  int item, cb, seg;
+  bool first, valid;
+};
+
+// Source tiles are staged by buffer loads that write LDS directly (no register stage), two units
+// ahead, into three buffers used in rotation; the buffers are separate static arrays so that the
+// compiler's wait-count insertion can tell which loads a read of a tile depends on (with one
+// dynamic array it waits for all of them, which would take the look-ahead away).
+template <typename T, int SH, int SW, bool TRANSPOSED, int NX>
+__global__ __launch_bounds__(kThreads, 4) void local_gather_mfma_kernel(
+    Geo g, const T* __restrict__ src, const T* __restrict__ rot, const T* __restrict__ filter,
+    T* __restrict__ dst, int tiles, int nwg) {
+  using E = typename MxOf<T>::type;
+  using M = Mx<E>;
+  constexpr bool kThird = sizeof(T) == 4;  // fp32 tensors: the filter has a low part
+  constexpr int K = 9, CELLS = SH * SW;
+  static_assert(CELLS <= 16, "one K = 16 block of cells");
+  constexpr int PITCH = 64 * NX + 64;
+  constexpr int kEntries = (K * kPix + kThreads - 1) / kThreads;  // coordinate entries staged per thread
+  constexpr int kChW = kCh / kWaves;                              // channels staged per wave
+  constexpr int kDma = kChW * NX;                                 // staging loads per wave and unit
+  __shared__ unsigned xs0[kCh * PITCH], xs1[kCh * PITCH], xs2[kCh * PITCH];
+  __shared__ float2 hw[K * kPix];  // scope coordinates (h, w) of (tap, pixel of the tile)
+  extern __shared__ __align__(16) unsigned dyn[];
+
+  const int cpg = g.channel / g.groups;
+  const int nblk = ceil_div(cpg, kCh);
+  uint4* wsp = reinterpret_cast<uint4*>(dyn);                  // [nblk][64]: Wh (2 words), Wl (2 words)
+  float* unscale = reinterpret_cast<float*>(wsp + nblk * 64);  // [nblk][kCh]: 1 / s of the channel
+
+  const int total = nwg * g.groups;
+  const int lb = logical_block(total);
+  if (lb >= total) return;
+  const int wg = lb % nwg, grp = lb / nwg;
+
+  const int W = g.in_w;  // == out_w
+  const int out_plane = g.out_h * W, in_plane = g.in_h * W;
+  const int dst_plane = TRANSPOSED ? in_plane : out_plane, src_plane = TRANSPOSED ? out_plane : in_plane;
+  const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int q = lane & 15, kg = lane >> 4;
+  const int row_step = g.dil_h * W;  // elements between two tap rows
+  // first staged source element relative to the tile's first pixel: the lowest tap offset.
+  // forward: tap (f_h, f_w) reads p + (f_h dil - pad) W + f_w - 1; grad input: output pixel
+  // q + (pad - f_h dil) W + 1 - f_w.  Either way the taps read staged index
+  // px + rr * row_step + cc with (rr, cc) = (f_h, f_w), or (2 - f_h, 2 - f_w) for grad input.
+  const int lo = TRANSPOSED ? (g.pad_h - 2 * g.dil_h) * W - 1 : -g.pad_h * W - 1;
+
+  // ---- per workgroup: the split filter operands of every channel block.  Lane (q, kg) of the
+  // B side stands for channel q and cells 4 kg .. 4 kg + 3.
+  for (int e = threadIdx.x; e < nblk * 64; e += kThreads) {
+    const int b = e >> 6, l = e & 63, cj = b * kCh + (l & 15), c0 = 4 * (l >> 4);
+    float v[4] = {0.f, 0.f, 0.f, 0.f}, s = 1.f;
+    if (cj < cpg) {
+      const T* f = filter + (size_t)(grp + g.groups * cj) * CELLS;
+      if constexpr (kThird) {
+        float m = 0.f;
+#pragma unroll
+        for (int k = 0; k < CELLS; ++k) m = fmaxf(m, fabsf(ld(f + k)));
+        int ex = 0;
+        if (m > 0.f && m < __builtin_inff()) (void)frexpf(m, &ex);  // m = fraction * 2^ex, fraction in [0.5, 1)
+        ex = min(max(ex, -100), 100);
+        s = ldexpf(1.f, -ex);
+        if ((l >> 4) == 0) unscale[b * kCh + (l & 15)] = ldexpf(1.f, ex);
+      }
+#pragma unroll
+      for (int k = 0; k < 4; ++k)
+        if (c0 + k < CELLS) v[k] = ld(f + c0 + k) * s;
+    } else if constexpr (kThird) {
+      if ((l >> 4) == 0) unscale[b * kCh + (l & 15)] = 0.f;
+    }
+    typename M::v4 h, lw;
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      E a, bb;
+      split2<E>(v[k], a, bb);
+      h[k] = a;
+      lw[k] = bb;
+    }
+    uint2 hb = __builtin_bit_cast(uint2, h), lb2 = __builtin_bit_cast(uint2, lw);
+    wsp[e] = make_uint4(hb.x, hb.y, lb2.x, lb2.y);
+  }
+
+  // ---- this workgroup's share of the (tile, channel block) units: whole tiles round-robin (tile t
+  // to workgroup t % nwg: neighbouring workgroups stage neighbouring tiles at the same time and
+  // the halo rows they share come from L2), the units of the last items % nwg tiles as contiguous
+  // ranges in (tile, block) order cut at the tile boundaries.
+  const int items = g.batch * tiles;
+  const int whole = items / nwg;
+  const long rest_units = (long)(items - whole * nwg) * nblk;
+  const long r_lo = rest_units * wg / nwg, r_hi = rest_units * (wg + 1) / nwg;
+  const int rest_lo = (int)(r_lo / nblk), rest_hi = r_hi > r_lo ? (int)((r_hi - 1) / nblk) : rest_lo - 1;
+  const int nseg = whole + (rest_hi - rest_lo + 1);
+  auto segment = [&](int k, int& item, int& cb_begin, int& cb_end) {
+    if (k < whole) {
+      item = wg + k * nwg;
+      cb_begin = 0;
+      cb_end = nblk;
+    } else {
+      const int t = rest_lo + (k - whole);
+      item = whole * nwg + t;
+      cb_begin = t == rest_lo ? (int)(r_lo % nblk) : 0;
+      cb_end = t == rest_hi ? (int)((r_hi - 1) % nblk) + 1 : nblk;
+    }
+  };
+  auto first_unit = [&]() {
+    Unit u{0, 0, 0, true, nseg > 0};
+    if (u.valid) {
+      int e;
+      segment(0, u.item, u.cb, e);
+    }
+    return u;
+  };
+  auto next_unit = [&](Unit u) {
+    if (!u.valid) return u;
+    int item, b, e;
+    segment(u.seg, item, b, e);
+    if (u.cb + 1 < e) {
+      ++u.cb;
+      u.first = false;
+      return u;
+    }
+    ++u.seg;
+    u.first = true;
+    u.valid = u.seg < nseg;
+    if (u.valid) segment(u.seg, u.item, u.cb, e);
+    return u;
+  };
+
+  // ---- staging
+  auto stage_tile = [&](const Unit& u, unsigned* buf) {
+    const int n = u.item / tiles, x0 = (u.item % tiles) * kPix + lo;
+#pragma unroll
+    for (int jj = 0; jj < kChW; ++jj) {
+      const int j = wave + jj * kWaves, cj = u.cb * kCh + j;
+      const bool chan = cj < cpg;
+      const size_t c = (size_t)n * g.channel + grp + (size_t)g.groups * (chan ? cj : 0);
+      const rsrc_t rx = plane_rsrc(src + c * src_plane, chan ? src_plane : 0);
+      // elements past the plane fail the buffer's range check and arrive as 0; elements before it
+      // get the out-of-range offset explicitly (a negative index must not reach the address arithmetic)
+#pragma unroll
+      for (int k = 0; k < NX; ++k) {
+        const int e = x0 + lane + 64 * k;
+        const lds_void_ptr to = (lds_void_ptr)(buf + tile_row(j, PITCH) + 64 * k);
+        const int off = e < 0 ? (int)kOutOfRange : e * (int)sizeof(T);
+        if constexpr (sizeof(T) == 4)
+          __builtin_amdgcn_raw_ptr_buffer_load_lds(rx, to, 4, off, 0, 0, 0);
+        else
+          __builtin_amdgcn_raw_ptr_buffer_load_lds(rx, to, 2, off, 0, 0, 0);
+      }
+    }
+  };
+  // The rotation pixel of (tap t, pixel idx of the tile), and whether the tap contributes at all.
+  // forward: the pixel itself, if the tap's input element lies in the image; grad input: the
+  // output pixel q + pad - f dil that feeds input pixel q through tap t, if it exists.
+  auto rotation_pixel = [&](int p0, int t, int idx, int& o) {
+    const int p = p0 + idx, f_h = t / 3, f_w = t % 3;
+    const bool live = p < dst_plane;
+    const int pc = live ? p : 0;
+    const int ph = pc / W, pw = pc - ph * W;
+    const int rh = TRANSPOSED ? ph + g.pad_h - f_h * g.dil_h : ph + f_h * g.dil_h - g.pad_h;
+    const int rw = TRANSPOSED ? pw + 1 - f_w : pw + f_w - 1;
+    const bool ok = live && rw >= 0 && rw < W && rh >= 0 && rh < (TRANSPOSED ? g.out_h : g.in_h);
+    o = TRANSPOSED ? rh * W + rw : pc;
+    return ok;
+  };
+  float r_rot[2 * kEntries];
+  auto load_rotation = [&](const Unit& u) {
+    const int n = u.item / tiles, p0 = (u.item % tiles) * kPix;
+    const rsrc_t rr = plane_rsrc(rot + (size_t)(n * g.groups + grp) * (K * 2) * out_plane, K * 2 * out_plane);
+#pragma unroll
+    for (int k = 0; k < kEntries; ++k) {
+      const int e = threadIdx.x + k * kThreads;
+      const int t = e / kPix, idx = e - t * kPix;
+      int o = 0;
+      const bool ok = t < K && rotation_pixel(p0, t, idx, o);
+      const unsigned off = ok ? (unsigned)(2 * t * out_plane + o) * (unsigned)sizeof(T) : kOutOfRange;
+      r_rot[2 * k] = buf_ld(rr, off, rot);
+      r_rot[2 * k + 1] = buf_ld(rr, off + (unsigned)out_plane * (unsigned)sizeof(T), rot);
+    }
+  };
+  // Scope coordinates: K.cu:338-341 and the band test of K.cu:59; a tap that contributes nothing
+  // gets (-2, -2), where every hat is 0.
+  auto store_coordinates = [&](const Unit& u) {
+    const int p0 = (u.item % tiles) * kPix;
+#pragma unroll
+    for (int k = 0; k < kEntries; ++k) {
+      const int e = threadIdx.x + k * kThreads;
+      const int t = e / kPix, idx = e - t * kPix;
+      if (t < K) {
+        int o = 0;
+        const bool ok = rotation_pixel(p0, t, idx, o);
+        const float h = scope_coord<float>(g, t / 3, r_rot[2 * k], g.centre_h);
+        const float w = scope_coord<float>(g, t % 3, r_rot[2 * k + 1], g.centre_w);
+        const bool in = ok && (h > -1.f) && (w > -1.f) && (h < float(SH)) && (w < float(SW));
+        hw[e] = in ? make_float2(h, w) : make_float2(-2.f, -2.f);
+      }
+    }
+  };
+
+  // A side: lane (pixel q of the wave's 16, cells 4 kg .. 4 kg + 3)
+  float ci[4], cj4[4];
+#pragma unroll
+  for (int k = 0; k < 4; ++k) {
+    const int cell = 4 * kg + k;
+    ci[k] = cell < CELLS ? float(cell / SW) : 64.f;  // rows past the last cell stay 0
+    cj4[k] = float(cell % SW);
+  }
+  typename M::v8 A[K];
+  const int px = wave * 16 + 4 * kg;  // D side: first of this lane's four pixels in the tile
+
+  auto derive_operands = [&]() {
+#pragma unroll
+    for (int t = 0; t < K; ++t) {
+      const float2 c = hw[t * kPix + wave * 16 + q];
+      typename M::v8 a;
+#pragma unroll
+      for (int k = 0; k < 4; ++k) {
+        E hi, lo2;
+        split2<E>(hat(c.x - ci[k]) * hat(c.y - cj4[k]), hi, lo2);
+        a[k] = hi;
+        a[4 + k] = lo2;
+      }
+      A[t] = a;
+    }
+  };
+
+  auto multiply_unit = [&](const Unit& u, const unsigned* buf) {
+    const uint4 wv = wsp[u.cb * 64 + lane];
+    const typename M::v4 wh = __builtin_bit_cast(typename M::v4, make_uint2(wv.x, wv.y));
+    const typename M::v4 wl = __builtin_bit_cast(typename M::v4, make_uint2(wv.z, wv.w));
+    // [Wh ; Wh] pairs with [Ah | Al]; [Wl ; 0] adds Ah Wl
+    const typename M::v8 whh = __builtin_shufflevector(wh, wh, 0, 1, 2, 3, 0, 1, 2, 3);
+    const typename M::v4 zero4 = {E(0), E(0), E(0), E(0)};
+    const typename M::v8 wl0 = __builtin_shufflevector(wl, zero4, 0, 1, 2, 3, 4, 5, 6, 7);
+    float acc[4] = {0.f, 0.f, 0.f, 0.f};
+    const unsigned* xr0 = buf + tile_row(q, PITCH) + px;
+#pragma unroll
+    for (int rr = 0; rr < 3; ++rr) {
+      float x6[6];  // columns -1 .. +4 of staged tap row rr around the four pixels
+#pragma unroll
+      for (int k = 0; k < 6; ++k) x6[k] = slot_value(xr0[rr * row_step + k], src);
+      const int t0 = TRANSPOSED ? (2 - rr) * 3 + 2 : rr * 3, dt = TRANSPOSED ? -1 : 1;  // the taps of columns 0, 1, 2
+      f4 d[3];
+      M::template row<kThird>(d[0], d[1], d[2], A[t0], A[t0 + dt], A[t0 + 2 * dt], whh, wl0);
+#pragma unroll
+      for (int cc = 0; cc < 3; ++cc)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) acc[i] = fmaf(x6[i + cc], d[cc][i], acc[i]);
+    }
+    // lane (kg, q): channel q of the block, pixels px .. px + 3 of the tile
+    const int cj = u.cb * kCh + q;
+    const int n = u.item / tiles, p = (u.item % tiles) * kPix + px;
+    if (cj < cpg && p < dst_plane) {
+      if constexpr (kThird) {
+        const float us = unscale[u.cb * kCh + q];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) acc[i] *= us;
+      }
+      T* out = dst + ((size_t)n * g.channel + grp + (size_t)g.groups * cj) * dst_plane + p;
+      if ((dst_plane & 3) == 0) {
+        // p is a multiple of 4, so the four pixels are inside the plane and 16-byte aligned
+        if constexpr (sizeof(T) == 4) {
+          f4 v = {acc[0], acc[1], acc[2], acc[3]};
+          __builtin_nontemporal_store(v, reinterpret_cast<f4*>(out));
+        } else {
+          struct { T e[4]; } pk;
+#pragma unroll
+          for (int i = 0; i < 4; ++i) st(pk.e + i, acc[i]);
+          const uint2 bits = __builtin_bit_cast(uint2, pk);
+          typedef unsigned u2 __attribute__((ext_vector_type(2)));
+          __builtin_nontemporal_store(u2{bits.x, bits.y}, reinterpret_cast<u2*>(out));
+        }
+      } else {
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+          if (p + i < dst_plane) st(out + i, acc[i]);
+      }
+    }
+  };
+
+  // ---- the walk.  In flight when unit u starts: the tiles of u (issued two units ago) and of
+  // u + 1.  Per unit: wait for the own loads of u's tile and for everybody to have left the
+  // previous unit; [first unit of a tile: coordinates -> LDS, barrier, operands]; multiply and
+  // store; start the rotation loads of the next unit if it begins a tile; start the tile loads
+  // of unit u + 2 into the buffer the previous unit used.
+  Unit u0 = first_unit(), u1 = next_unit(u0), u2 = next_unit(u1);
+  if (u0.valid) {
+    load_rotation(u0);
+    stage_tile(u0, xs0);
+  }
+  if (u1.valid) stage_tile(u1, xs1);
+  auto step = [&](unsigned* cur, unsigned* free_buf) {
+    // everything older than the kDma loads of u1's tile must have landed -- if those were issued
+    if (u1.valid)
+      wait_barrier<kDma>();
+    else
+      wait_barrier<0>();
+    if (u0.first) {
+      store_coordinates(u0);
+      wait_barrier<63>();  // LDS only: the tile loads stay in flight
+      derive_operands();
+    }
+    multiply_unit(u0, cur);
+    if (u1.valid && u1.first) load_rotation(u1);
+    if (u2.valid) stage_tile(u2, free_buf);
+    u0 = u1;
+    u1 = u2;
+    u2 = next_unit(u2);
+  };
+  while (u0.valid) {
+    step(xs0, xs2);
+    if (!u0.valid) break;
+    step(xs1, xs0);
+    if (!u0.valid) break;
+    step(xs2, xs1);
+  }
+}
+
+struct GatherPlan {
+  bool ok;
+  int nx, pitch, tiles, nwg;
+  size_t lds;
+};
+
+template <int SH, int SW>
+GatherPlan gather_plan(const Geo& g, bool transposed) {
+  GatherPlan p{};
+  p.ok = false;
+  const bool same_width = g.stride_h == 1 && g.stride_w == 1 && g.dil_w == 1 && g.pad_w == 1 && g.k_h == 3 &&
+                          g.k_w == 3 && g.in_w == g.out_w;
+  if (!same_width || SH * SW > 16 || path_disabled(kNoRows) || path_disabled(kNoGatherMfma)) return p;
+  const long xt = kPix + 2 + 2L * g.dil_h * g.in_w;  // tile + halo rows
+  if (xt > 64 * kMaxX) return p;
+  p.nx = xt <= 256 ? 4 : kMaxX;
+  p.pitch = 64 * p.nx + 64;
+  const int cpg = g.channel / g.groups, nblk = ceil_div(cpg, kCh);
+  const long plane = transposed ? (long)g.in_h * g.in_w : (long)g.out_h * g.out_w;
+  p.tiles = (int)ceil_div((int)plane, kPix);
+  // dynamic part: the split filter operands; static: three tiles and the coordinate table
+  const long lds = (long)nblk * 64 * 16 + (long)nblk * kCh * 4;
+  if (lds + 3L * kCh * p.pitch * 4 + 9L * kPix * 8 > 160 * 1024) return p;
+  p.lds = (size_t)lds;
+  const long units = (long)g.batch * p.tiles * nblk;
+  if (units >= (1L << 30)) return p;
+  // at most two workgroups per CU, all resident at once, each walking an equal share of the units
+  p.nwg = (int)std::max(1L, std::min((long)g.batch * p.tiles, (long)std::max(1, 2 * 256 / g.groups)));
+  p.ok = true;
+  return p;
+}
+
+template <typename T, int SH, int SW>
+bool run_gather_mfma(const Geo& g, bool transposed, const T* src, const T* rot, const T* filter, T* dst,
+                     hipStream_t stream) {
+  const GatherPlan p = gather_plan<SH, SW>(g, transposed);
+  if (!p.ok) return false;
+  const unsigned grid = (unsigned)xcd_grid_size((long)p.nwg * g.groups);
+#define DK_LAUNCH(TR, NXV)                                                                        \
+  {                                                                                               \
+    auto kernel = local_gather_mfma_kernel<T, SH, SW, TR, NXV>;                                   \
+    const int room = 160 * 1024 - (3 * kCh * (64 * NXV + 64) * 4 + 9 * kPix * 8);                 \
+    if (!allow_dynamic_lds(reinterpret_cast<const void*>(kernel), room)) return false;            \
+    kernel<<<grid, kThreads, p.lds, stream>>>(g, src, rot, filter, dst, p.tiles, p.nwg);          \
+  }
+  if (transposed) {
+    if (p.nx == 4) DK_LAUNCH(true, 4) else DK_LAUNCH(true, kMaxX)
+  } else {
+    if (p.nx == 4) DK_LAUNCH(false, 4) else DK_LAUNCH(false, kMaxX)
+  }
+#undef DK_LAUNCH
+  return true;
+}
+
+}  // namespace
+
+template <typename T>
+bool mfma_local_gather(const Geo& g, bool transposed, const T* src, const T* rot, const T* filter, T* dst,
+                       hipStream_t stream) {
+  if (g.k_h != 3 || g.k_w != 3) return false;
+  if ((long)g.in_h * g.in_w >= (1L << 24) || (long)g.out_h * g.out_w >= (1L << 24)) return false;  // byte offsets of 18 rotation planes in 31 bits
+  if (g.scope_h == 4 && g.scope_w == 4) return run_gather_mfma<T, 4, 4>(g, transposed, src, rot, filter, dst, stream);
+  if (g.scope_h == 3 && g.scope_w == 3) return run_gather_mfma<T, 3, 3>(g, transposed, src, rot, filter, dst, stream);
+  return false;
+}
+
+template bool mfma_local_gather<float>(const Geo&, bool, const float*, const float*, const float*, float*, hipStream_t);
+template bool mfma_local_gather<__half>(const Geo&, bool, const __half*, const __half*, const __half*, __half*, hipStream_t);
+template bool mfma_local_gather<bf16_t>(const Geo&, bool, const bf16_t*, const bf16_t*, const bf16_t*, bf16_t*, hipStream_t);
+
+}  // namespace dk
