@@ -135,6 +135,29 @@ __device__ __forceinline__ float slot_value(unsigned bits, const __half*) {
 }
 
 typedef __attribute__((address_space(3))) void* lds_void_ptr;
+typedef unsigned u4 __attribute__((ext_vector_type(4)));
+
+// One buffer load that writes LDS: lane l's element (SIZE bytes at byte offset `off` of the buffer,
+// zero if out of range) goes to the 32-bit slot `to + l`.  Issued from inline assembly so that the
+// compiler does not see it: it guards every LDS read that might alias an outstanding load of this
+// kind with a wait for ALL outstanding loads (it cannot tell the buffers of the rotation below apart
+// once the pointers pass through the unit loop), which would take the look-ahead away.  The waits are
+// written out instead (wait_barrier): a tile is read only after the wave's own loads of it have
+// landed and the workgroup has passed a barrier.
+// (The buffer resource as its four words: base address, 48 bits; stride 0; size in bytes; flags.)
+template <typename T>
+__device__ __forceinline__ u4 resource_words(const T* base, int elems) {
+  const unsigned long a = reinterpret_cast<unsigned long>(base);
+  return u4{(unsigned)a, (unsigned)(a >> 32) & 0xffffu, (unsigned)elems * (unsigned)sizeof(T), (unsigned)kRsrcFlags};
+}
+template <int SIZE>
+__device__ __forceinline__ void load_to_lds(u4 r, unsigned* to, int off) {
+  const unsigned addr = (unsigned)(unsigned long)(lds_void_ptr)to;
+  if constexpr (SIZE == 4)
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dword %1, %2, 0 offen lds" ::"s"(addr), "v"(off), "s"(r) : "memory", "m0");
+  else
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_ushort %1, %2, 0 offen lds" ::"s"(addr), "v"(off), "s"(r) : "memory", "m0");
+}
 
 // Wait until at most N of this wave's vector-memory operations are outstanding and its LDS
 // operations are done, then the workgroup barrier.  __syncthreads() would do, but it waits for
@@ -145,16 +168,43 @@ __device__ __forceinline__ void wait_barrier() {
   asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(N) : "memory");
 }
 
+// NX consecutive 64-element runs with one per-lane offset: the steps are the instruction's
+// immediate offset, which the hardware adds to the memory address AND to the LDS address, so M0 is
+// set once.
+template <int SIZE, int NX>
+__device__ __forceinline__ void load_run_to_lds(u4 r, unsigned* to, int off) {
+  const unsigned addr = (unsigned)(unsigned long)(lds_void_ptr)to;
+  static_assert(SIZE == 4, "the LDS side steps by 4 bytes per element, the memory side by SIZE: equal only for 4");
+  static_assert(NX == 4 || NX == 6, "four or six runs");
+  if constexpr (NX == 4)
+    asm volatile(
+        "s_mov_b32 m0, %0\n\ts_nop 0\n\t"
+        "buffer_load_dword %1, %2, 0 offen lds\n\t"
+        "buffer_load_dword %1, %2, 0 offen offset:256 lds\n\t"
+        "buffer_load_dword %1, %2, 0 offen offset:512 lds\n\t"
+        "buffer_load_dword %1, %2, 0 offen offset:768 lds" ::"s"(addr), "v"(off), "s"(r)
+        : "memory", "m0");
+  else
+    asm volatile(
+        "s_mov_b32 m0, %0\n\ts_nop 0\n\t"
+        "buffer_load_dword %1, %2, 0 offen lds\n\t"
+        "buffer_load_dword %1, %2, 0 offen offset:256 lds\n\t"
+        "buffer_load_dword %1, %2, 0 offen offset:512 lds\n\t"
+        "buffer_load_dword %1, %2, 0 offen offset:768 lds\n\t"
+        "buffer_load_dword %1, %2, 0 offen offset:1024 lds\n\t"
+        "buffer_load_dword %1, %2, 0 offen offset:1280 lds" ::"s"(addr), "v"(off), "s"(r)
+        : "memory", "m0");
+}
+
 // One unit of work, and whether it is the first of its tile that this workgroup handles.
 struct Unit {
-  int item, cb, seg;
+  int n, p0;            // image and first pixel of the tile (set once per segment: a division by the tile count)
+  int cb, seg, cb_end;  // channel block; segment and the end of its channel blocks
   bool first, valid;
 };
 
 // Source tiles are staged by buffer loads that write LDS directly (no register stage), two units
-// ahead, into three buffers used in rotation; the buffers are separate static arrays so that the
-// compiler's wait-count insertion can tell which loads a read of a tile depends on (with one
-// dynamic array it waits for all of them, which would take the look-ahead away).
+// ahead, into three buffers used in rotation.
 template <typename T, int SH, int SW, bool TRANSPOSED, int NX>
 __global__ __launch_bounds__(kThreads, 4) void local_gather_mfma_kernel(
     Geo g, const T* __restrict__ src, const T* __restrict__ rot, const T* __restrict__ filter,
@@ -193,6 +243,7 @@ __global__ __launch_bounds__(kThreads, 4) void local_gather_mfma_kernel(
   // q + (pad - f_h dil) W + 1 - f_w.  Either way the taps read staged index
   // px + rr * row_step + cc with (rr, cc) = (f_h, f_w), or (2 - f_h, 2 - f_w) for grad input.
   const int lo = TRANSPOSED ? (g.pad_h - 2 * g.dil_h) * W - 1 : -g.pad_h * W - 1;
+  const unsigned w_magic = (unsigned)(0x100000000ull / (unsigned)W) + 1u;  // floor(p / W) = (p * magic) >> 32 for p < 2^24
 
   // ---- per workgroup: the split filter operands of every channel block.  Lane (q, kg) of the
   // B side stands for channel q and cells 4 kg .. 4 kg + 3.
@@ -251,50 +302,52 @@ __global__ __launch_bounds__(kThreads, 4) void local_gather_mfma_kernel(
       cb_end = t == rest_hi ? (int)((r_hi - 1) % nblk) + 1 : nblk;
     }
   };
-  auto first_unit = [&]() {
-    Unit u{0, 0, 0, true, nseg > 0};
+  auto first_of_segment = [&](int seg) {
+    Unit u{0, 0, 0, seg, 0, true, seg < nseg};
     if (u.valid) {
-      int e;
-      segment(0, u.item, u.cb, e);
+      int item;
+      segment(seg, item, u.cb, u.cb_end);
+      u.n = item / tiles;
+      u.p0 = (item - u.n * tiles) * kPix;
     }
     return u;
   };
-  auto next_unit = [&](Unit u) {
+  auto first_unit = [&]() { return first_of_segment(0); };
+  auto next_unit = [&](Unit u) {  // one scalar add and compare except at the end of a segment
     if (!u.valid) return u;
-    int item, b, e;
-    segment(u.seg, item, b, e);
-    if (u.cb + 1 < e) {
+    if (u.cb + 1 < u.cb_end) {
       ++u.cb;
       u.first = false;
       return u;
     }
-    ++u.seg;
-    u.first = true;
-    u.valid = u.seg < nseg;
-    if (u.valid) segment(u.seg, u.item, u.cb, e);
-    return u;
+    return first_of_segment(u.seg + 1);
   };
 
   // ---- staging
   auto stage_tile = [&](const Unit& u, unsigned* buf) {
-    const int n = u.item / tiles, x0 = (u.item % tiles) * kPix + lo;
+    const int n = u.n, x0 = u.p0 + lo;
 #pragma unroll
     for (int jj = 0; jj < kChW; ++jj) {
       const int j = wave + jj * kWaves, cj = u.cb * kCh + j;
       const bool chan = cj < cpg;
       const size_t c = (size_t)n * g.channel + grp + (size_t)g.groups * (chan ? cj : 0);
-      const rsrc_t rx = plane_rsrc(src + c * src_plane, chan ? src_plane : 0);
-      // elements past the plane fail the buffer's range check and arrive as 0; elements before it
-      // get the out-of-range offset explicitly (a negative index must not reach the address arithmetic)
+      const T* plane = src + c * src_plane;
+      if (sizeof(T) == 4 && x0 >= 0) {
+        // the buffer starts at the first staged element: every lane's offset is its lane number,
+        // the 64-element steps are immediates, and what lies past the plane fails the range check
+        if constexpr (sizeof(T) == 4) {
+          const u4 rx = resource_words(plane + x0, chan ? max(src_plane - x0, 0) : 0);
+          load_run_to_lds<4, NX>(rx, buf + tile_row(j, PITCH), lane * 4);
+        }
+      } else {
+        // the first tile of a plane: the elements before the plane must read as zeros (16-bit
+        // tensors always come this way: their memory and LDS steps differ)
+        const u4 rx = resource_words(plane, chan ? src_plane : 0);
 #pragma unroll
-      for (int k = 0; k < NX; ++k) {
-        const int e = x0 + lane + 64 * k;
-        const lds_void_ptr to = (lds_void_ptr)(buf + tile_row(j, PITCH) + 64 * k);
-        const int off = e < 0 ? (int)kOutOfRange : e * (int)sizeof(T);
-        if constexpr (sizeof(T) == 4)
-          __builtin_amdgcn_raw_ptr_buffer_load_lds(rx, to, 4, off, 0, 0, 0);
-        else
-          __builtin_amdgcn_raw_ptr_buffer_load_lds(rx, to, 2, off, 0, 0, 0);
+        for (int k = 0; k < NX; ++k) {
+          const int e = x0 + lane + 64 * k;
+          load_to_lds<sizeof(T)>(rx, buf + tile_row(j, PITCH) + 64 * k, e < 0 ? (int)kOutOfRange : e * (int)sizeof(T));
+        }
       }
     }
   };
@@ -305,41 +358,57 @@ __global__ __launch_bounds__(kThreads, 4) void local_gather_mfma_kernel(
     const int p = p0 + idx, f_h = t / 3, f_w = t % 3;
     const bool live = p < dst_plane;
     const int pc = live ? p : 0;
-    const int ph = pc / W, pw = pc - ph * W;
+    const int ph = (int)__umulhi((unsigned)pc, w_magic), pw = pc - ph * W;  // pc / W, exact below 2^32 / W
     const int rh = TRANSPOSED ? ph + g.pad_h - f_h * g.dil_h : ph + f_h * g.dil_h - g.pad_h;
     const int rw = TRANSPOSED ? pw + 1 - f_w : pw + f_w - 1;
     const bool ok = live && rw >= 0 && rw < W && rh >= 0 && rh < (TRANSPOSED ? g.out_h : g.in_h);
     o = TRANSPOSED ? rh * W + rw : pc;
     return ok;
   };
-  float r_rot[2 * kEntries];
+  // The rotation values of a tile go straight into the coordinate table, again by loads that write
+  // LDS (no registers held while they are in flight): entry e = (tap, pixel) is two slots, so a
+  // wave-load fills 32 entries, lane l the component l % 2 of entry l / 2; the gather of the
+  // rotation pixel is the load's own per-lane offset.  store_coordinates() then turns the
+  // values into scope coordinates in place.
+  constexpr int kRotLoads = K * kPix / 32;                         // wave-loads per tile
+  constexpr int kRotPerWave = (kRotLoads + kWaves - 1) / kWaves;   // ... per wave
+  // (The empty asm in these two once-per-tile functions makes the thread's index opaque, so that
+  // the per-thread constants derived from it -- tap, pixel, plane offsets of each entry -- are
+  // recomputed when needed instead of living in registers through the unit loop, which has none to spare.)
   auto load_rotation = [&](const Unit& u) {
-    const int n = u.item / tiles, p0 = (u.item % tiles) * kPix;
-    const rsrc_t rr = plane_rsrc(rot + (size_t)(n * g.groups + grp) * (K * 2) * out_plane, K * 2 * out_plane);
+    int lane_ = lane;
+    asm volatile("" : "+v"(lane_));
+    const int n = u.n, p0 = u.p0;
+    const u4 rr = resource_words(rot + (size_t)(n * g.groups + grp) * (K * 2) * out_plane, K * 2 * out_plane);
 #pragma unroll
-    for (int k = 0; k < kEntries; ++k) {
-      const int e = threadIdx.x + k * kThreads;
-      const int t = e / kPix, idx = e - t * kPix;
-      int o = 0;
-      const bool ok = t < K && rotation_pixel(p0, t, idx, o);
-      const unsigned off = ok ? (unsigned)(2 * t * out_plane + o) * (unsigned)sizeof(T) : kOutOfRange;
-      r_rot[2 * k] = buf_ld(rr, off, rot);
-      r_rot[2 * k + 1] = buf_ld(rr, off + (unsigned)out_plane * (unsigned)sizeof(T), rot);
+    for (int k = 0; k < kRotPerWave; ++k) {
+      const int ld_ = wave + k * kWaves;  // wave-uniform
+      if (ld_ < kRotLoads) {
+        const int e = ld_ * 32 + (lane_ >> 1);
+        const int t = e / kPix, idx = e - t * kPix;
+        int o = 0;
+        const bool ok = rotation_pixel(p0, t, idx, o);
+        const int off = ok ? (int)((unsigned)((2 * t + (lane_ & 1)) * out_plane + o) * (unsigned)sizeof(T)) : (int)kOutOfRange;
+        load_to_lds<sizeof(T)>(rr, reinterpret_cast<unsigned*>(hw) + ld_ * 64, off);
+      }
     }
   };
   // Scope coordinates: K.cu:338-341 and the band test of K.cu:59; a tap that contributes nothing
   // gets (-2, -2), where every hat is 0.
   auto store_coordinates = [&](const Unit& u) {
-    const int p0 = (u.item % tiles) * kPix;
+    int tid_ = threadIdx.x;
+    asm volatile("" : "+v"(tid_));
+    const int p0 = u.p0;
 #pragma unroll
     for (int k = 0; k < kEntries; ++k) {
-      const int e = threadIdx.x + k * kThreads;
+      const int e = tid_ + k * kThreads;
       const int t = e / kPix, idx = e - t * kPix;
       if (t < K) {
         int o = 0;
         const bool ok = rotation_pixel(p0, t, idx, o);
-        const float h = scope_coord<float>(g, t / 3, r_rot[2 * k], g.centre_h);
-        const float w = scope_coord<float>(g, t % 3, r_rot[2 * k + 1], g.centre_w);
+        const uint2 raw = *reinterpret_cast<const uint2*>(hw + e);
+        const float h = scope_coord<float>(g, t / 3, slot_value(raw.x, rot), g.centre_h);
+        const float w = scope_coord<float>(g, t % 3, slot_value(raw.y, rot), g.centre_w);
         const bool in = ok && (h > -1.f) && (w > -1.f) && (h < float(SH)) && (w < float(SW));
         hw[e] = in ? make_float2(h, w) : make_float2(-2.f, -2.f);
       }
@@ -347,13 +416,10 @@ __global__ __launch_bounds__(kThreads, 4) void local_gather_mfma_kernel(
   };
 
   // A side: lane (pixel q of the wave's 16, cells 4 kg .. 4 kg + 3)
-  float ci[4], cj4[4];
-#pragma unroll
-  for (int k = 0; k < 4; ++k) {
-    const int cell = 4 * kg + k;
-    ci[k] = cell < CELLS ? float(cell / SW) : 64.f;  // rows past the last cell stay 0
-    cj4[k] = float(cell % SW);
-  }
+  // cell 4 kg + k = (row, column); rows past the last cell stay 0.  With four columns the row is kg
+  // and the column k, which costs one register instead of eight.
+  auto cell_row = [&](int k) { return SW == 4 ? float(kg) : (4 * kg + k < CELLS ? float((4 * kg + k) / SW) : 64.f); };
+  auto cell_col = [&](int k) { return SW == 4 ? float(k) : float((4 * kg + k) % SW); };
   typename M::v8 A[K];
   const int px = wave * 16 + 4 * kg;  // D side: first of this lane's four pixels in the tile
 
@@ -365,7 +431,7 @@ __global__ __launch_bounds__(kThreads, 4) void local_gather_mfma_kernel(
 #pragma unroll
       for (int k = 0; k < 4; ++k) {
         E hi, lo2;
-        split2<E>(hat(c.x - ci[k]) * hat(c.y - cj4[k]), hi, lo2);
+        split2<E>(hat(c.x - cell_row(k)) * hat(c.y - cell_col(k)), hi, lo2);
         a[k] = hi;
         a[4 + k] = lo2;
       }
@@ -398,7 +464,7 @@ __global__ __launch_bounds__(kThreads, 4) void local_gather_mfma_kernel(
     }
     // lane (kg, q): channel q of the block, pixels px .. px + 3 of the tile
     const int cj = u.cb * kCh + q;
-    const int n = u.item / tiles, p = (u.item % tiles) * kPix + px;
+    const int n = u.n, p = u.p0 + px;
     if (cj < cpg && p < dst_plane) {
       if constexpr (kThird) {
         const float us = unscale[u.cb * kCh + q];
@@ -429,28 +495,47 @@ __global__ __launch_bounds__(kThreads, 4) void local_gather_mfma_kernel(
 
   // ---- the walk.  In flight when unit u starts: the tiles of u (issued two units ago) and of
   // u + 1.  Per unit: wait for the own loads of u's tile and for everybody to have left the
-  // previous unit; [first unit of a tile: coordinates -> LDS, barrier, operands]; multiply and
-  // store; start the rotation loads of the next unit if it begins a tile; start the tile loads
-  // of unit u + 2 into the buffer the previous unit used.
+  // previous unit; [first unit of a tile: rotation values -> coordinates in place, barrier, operands];
+  // multiply and store; start the rotation loads of the next tile where the table is free for them,
+  // then the tile loads of unit u + 2 into the buffer the previous unit used (always last, so that
+  // "all but the newest kDma operations" is the right thing to wait for).
+  // The rotation loads of tile T + 1 go out in the second unit of tile T (the table is read in the
+  // first); a tile with a single unit here is followed by a stall on them.
   Unit u0 = first_unit(), u1 = next_unit(u0), u2 = next_unit(u1);
+  bool rot_in_flight = false;
   if (u0.valid) {
     load_rotation(u0);
     stage_tile(u0, xs0);
   }
   if (u1.valid) stage_tile(u1, xs1);
   auto step = [&](unsigned* cur, unsigned* free_buf) {
-    // everything older than the kDma loads of u1's tile must have landed -- if those were issued
-    if (u1.valid)
-      wait_barrier<kDma>();
-    else
+    if (u0.first && !rot_in_flight && u0.seg > 0) {
+      // single-unit tile before this one: its loads could not be issued ahead
+      wait_barrier<63>();  // everybody is past the previous tile's operands
+      load_rotation(u0);
       wait_barrier<0>();
+    } else if (u1.valid) {
+      wait_barrier<kDma>();  // everything older than the loads of u1's tile has landed
+    } else {
+      wait_barrier<0>();
+    }
     if (u0.first) {
+      rot_in_flight = false;
       store_coordinates(u0);
       wait_barrier<63>();  // LDS only: the tile loads stay in flight
       derive_operands();
     }
+    const bool table_free = !u0.first;  // read in the first unit of this tile, at least a barrier ago
     multiply_unit(u0, cur);
-    if (u1.valid && u1.first) load_rotation(u1);
+    // vector-memory operations of this step, oldest first: the result stores, the rotation loads,
+    // the tile loads -- so that "all but the newest kDma" at the next step means "all but u2's tile"
+    if (table_free && !rot_in_flight) {
+      const Unit nx = first_of_segment(u0.seg + 1);
+      if (nx.valid) {
+        load_rotation(nx);
+        rot_in_flight = true;
+      }
+    }
     if (u2.valid) stage_tile(u2, free_buf);
     u0 = u1;
     u1 = u2;
@@ -477,7 +562,7 @@ GatherPlan gather_plan(const Geo& g, bool transposed) {
   p.ok = false;
   const bool same_width = g.stride_h == 1 && g.stride_w == 1 && g.dil_w == 1 && g.pad_w == 1 && g.k_h == 3 &&
                           g.k_w == 3 && g.in_w == g.out_w;
-  if (!same_width || SH * SW > 16 || path_disabled(kNoRows) || path_disabled(kNoGatherMfma)) return p;
+  if (!same_width || SH * SW > 16 || g.in_w < 2 || path_disabled(kNoRows) || path_disabled(kNoGatherMfma)) return p;  // in_w >= 2: the division by the width is a multiplication
   const long xt = kPix + 2 + 2L * g.dil_h * g.in_w;  // tile + halo rows
   if (xt > 64 * kMaxX) return p;
   p.nx = xt <= 256 ? 4 : kMaxX;
@@ -525,6 +610,9 @@ template <typename T>
 bool mfma_local_gather(const Geo& g, bool transposed, const T* src, const T* rot, const T* filter, T* dst,
                        hipStream_t stream) {
   if (g.k_h != 3 || g.k_w != 3) return false;
+  // 16-bit tensors: measured slower than the row kernels so far (60 against 66 us on N=64 C=144 56 x 56:
+  // their tiles are staged element by element, 2-byte loads into 4-byte slots), so those keep the row kernels
+  if (sizeof(T) != 4) return false;
   if ((long)g.in_h * g.in_w >= (1L << 24) || (long)g.out_h * g.out_w >= (1L << 24)) return false;  // byte offsets of 18 rotation planes in 31 bits
   if (g.scope_h == 4 && g.scope_w == 4) return run_gather_mfma<T, 4, 4>(g, transposed, src, rot, filter, dst, stream);
   if (g.scope_h == 3 && g.scope_w == 3) return run_gather_mfma<T, 3, 3>(g, transposed, src, rot, filter, dst, stream);
