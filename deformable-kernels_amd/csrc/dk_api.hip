@@ -27,7 +27,8 @@ unsigned switches_from_environment() {
       {"DK_NO_ROWS", kNoRows}, {"DK_NO_MFMA", kNoMfma}, {"DK_NO_MFMA_S2", kNoMfmaS2},
       {"DK_NO_S2_QUADS", kNoS2Quads}, {"DK_NO_DEFORM_FAST", kNoDeformFast}, {"DK_NO_DEFORM_CH", kNoDeformCh},
       {"DK_NO_DEFORM_CH_BIG", kNoDeformChBig}, {"DK_NO_DEFORM_MFMA", kNoDeformMfma},
-      {"DK_NO_ND_BINS", kNoNdBins}, {"DK_NO_ND_MFMA", kNoNdMfma}, {"DK_NO_GATHER_MFMA", kNoGatherMfma}};
+      {"DK_NO_ND_BINS", kNoNdBins}, {"DK_NO_ND_MFMA", kNoNdMfma}, {"DK_NO_GATHER_MFMA", kNoGatherMfma},
+      {"DK_NO_FILTER_SPLIT", kNoFilterSplit}};
   unsigned m = 0;
   for (const auto& v : vars)
     if (std::getenv(v.name)) m |= v.bit;

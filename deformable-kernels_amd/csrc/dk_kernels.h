@@ -27,6 +27,7 @@ enum TestSwitch : unsigned {
   kNoNdBins = 1u << 8,      // DK_NO_ND_BINS      the N-d kernels that sort the points by cell
   kNoNdMfma = 1u << 9,      // DK_NO_ND_MFMA      the matrix-core N-d kernels
   kNoGatherMfma = 1u << 10, // DK_NO_GATHER_MFMA  the matrix-core forward / grad input (the row kernels run instead)
+  kNoFilterSplit = 1u << 11, // DK_NO_FILTER_SPLIT the bfloat16-pair form of the float32 matrix-core grad filter (fp32 matrix instructions instead)
 };
 unsigned test_switches();  // dk_api.hip
 inline bool path_disabled(unsigned sw) { return (test_switches() & sw) != 0; }

@@ -984,7 +984,17 @@ __device__ __forceinline__ float hat(float d) { return __builtin_amdgcn_fmed3f(1
 // most 128 pixels), so that the input rows its taps read, 2 oh0 - 1 .. 2 (oh0 + th - 1) + 1, are
 // one contiguous range of the plane like the stride-1 tile with its halo rows; a lane's four
 // pixels may sit in different rows, so each reads its own 3 x 3 inputs.
-template <typename T, int SH, int SW, int CELL0, int NX, bool S2, bool BF = false>
+// SPLIT (float32 tensors): both operands as bfloat16 pairs, A = Ah + Al and P = Ph + Pl (hi = the
+// value rounded to bfloat16, lo = the rounded remainder: together 16 significand bits), and three
+// products Ah Ph + Ah Pl + Al Ph on v_mfma_f32_16x16x16_bf16 with fp32 sums instead of one on
+// v_mfma_f32_16x16x4_f32.  The fp32 instruction takes 32 clk of the SIMD's issue slots for 4 k and
+// does not overlap with vector ALU work, not even of other waves; a bfloat16 one covers 16 k in
+// 16 clk of the matrix pipe and runs beside other waves' vector ALU work (measured: it adds about
+// 6 clk to a SIMD busy with FMAs).  A unit is then 27 matrix instructions instead of 36 and pays
+// 12 more vector ALU instructions per tap for the split of P.  The dropped Al Pl and the rounding
+// of the lo parts leave a relative error of about 2^-16 per product -- the filter gradient is held
+// to 1e-4 of its largest element and sums thousands of products of either sign.
+template <typename T, int SH, int SW, int CELL0, int NX, bool S2, bool BF = false, bool SPLIT = false>
 __global__ __launch_bounds__(kMfBlock, 4) void local_grad_filter_mfma_kernel(
     Geo g, const T* __restrict__ gout, const T* __restrict__ x, const T* __restrict__ rot,
     float* __restrict__ partial, int tiles, int nwg, int csplits, int pitch_x, int th) {
@@ -1150,9 +1160,11 @@ __global__ __launch_bounds__(kMfBlock, 4) void local_grad_filter_mfma_kernel(
   // small (one channel, 3 x 3 scope: 1.1e-2 seen), so groups of fewer than 16 channels keep the
   // fp32 instructions (template parameter BF, chosen by the host).
   static_assert(!BF || sizeof(T) == 2, "bfloat16 matrix instructions are for 16-bit inputs");
+  static_assert(!SPLIT || (sizeof(T) == 4 && !BF), "the split is for float32 inputs");
   constexpr bool kHalfIn = BF;
-  float A[kHalfIn ? 1 : 4][K];
-  mfb4 Ab[kHalfIn ? K : 1];
+  float A[(kHalfIn || SPLIT) ? 1 : 4][K];
+  mfb4 Ab[(kHalfIn || SPLIT) ? K : 1];  // SPLIT: the hi parts
+  mfb4 Al[SPLIT ? K : 1];               // ... and the lo parts
   mf4 acc = {0.f, 0.f, 0.f, 0.f};
   int done_cb = -1;  // channel block (within the split) whose result `acc` holds
 
@@ -1199,7 +1211,27 @@ __global__ __launch_bounds__(kMfBlock, 4) void local_grad_filter_mfma_kernel(
 #pragma unroll
       for (int f_w = 0; f_w < 3; ++f_w) {
         const int t = r * 3 + f_w;
-        if constexpr (kHalfIn) {
+        if constexpr (SPLIT) {
+          // every instruction adds into a live accumulator, so its result registers cannot be
+          // given to one of its operands (see dk_local_mfma.hip for what happens when they can)
+          mfb4 bh, bl;
+#pragma unroll
+          for (int ii = 0; ii < 4; ++ii) {
+            float pr = xv[ii][f_w] * gq[ii];
+            asm volatile("" : "+v"(pr));  // one fp32 value for both parts: no contraction into the conversions
+            bh[ii] = static_cast<__bf16>(pr);
+            bl[ii] = static_cast<__bf16>(pr - static_cast<float>(bh[ii]));
+          }
+          if (t & 1) {
+            acc1 = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(Ab[t], bh, acc1, 0, 0, 0);
+            acc1 = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(Ab[t], bl, acc1, 0, 0, 0);
+            acc1 = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(Al[t], bh, acc1, 0, 0, 0);
+          } else {
+            acc0 = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(Ab[t], bh, acc0, 0, 0, 0);
+            acc0 = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(Ab[t], bl, acc0, 0, 0, 0);
+            acc0 = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(Al[t], bh, acc0, 0, 0, 0);
+          }
+        } else if constexpr (kHalfIn) {
           mfb4 b;
 #pragma unroll
           for (int ii = 0; ii < 4; ++ii) b[ii] = static_cast<__bf16>(xv[ii][f_w] * gq[ii]);
@@ -1239,7 +1271,15 @@ __global__ __launch_bounds__(kMfBlock, 4) void local_grad_filter_mfma_kernel(
       const float4 hw23 = *reinterpret_cast<const float4*>(hw + t * kMfPix + px + 2);
       const float a0 = hat(hw01.x - ci) * hat(hw01.y - cj), a1 = hat(hw01.z - ci) * hat(hw01.w - cj);
       const float a2 = hat(hw23.x - ci) * hat(hw23.y - cj), a3 = hat(hw23.z - ci) * hat(hw23.w - cj);
-      if constexpr (kHalfIn) {
+      if constexpr (SPLIT) {
+        float av[4] = {a0, a1, a2, a3};
+#pragma unroll
+        for (int ii = 0; ii < 4; ++ii) {
+          asm volatile("" : "+v"(av[ii]));
+          Ab[t][ii] = static_cast<__bf16>(av[ii]);
+          Al[t][ii] = static_cast<__bf16>(av[ii] - static_cast<float>(Ab[t][ii]));
+        }
+      } else if constexpr (kHalfIn) {
         Ab[t] = mfb4{static_cast<__bf16>(a0), static_cast<__bf16>(a1), static_cast<__bf16>(a2), static_cast<__bf16>(a3)};
       } else {
         A[0][t] = a0;
@@ -1539,22 +1579,25 @@ bool run_grad_filter(const Geo& g, const T* gout, const T* x, const T* rot, T* g
     const FilterGrid f = filter_grid(g);
     const unsigned grid = (unsigned)xcd_grid_size((long)f.parts * f.splits * g.groups);
     if (f.mfma) {
-#define DK_LAUNCH_BF(CELL0, BF)                                                                                  \
+#define DK_LAUNCH_BF(CELL0, BF, SP)                                                                                 \
   if (f.th > 0) {                                                                                                \
-    auto kernel = local_grad_filter_mfma_kernel<T, SH, SW, CELL0, kMfXS2, true, BF>;                             \
+    auto kernel = local_grad_filter_mfma_kernel<T, SH, SW, CELL0, kMfXS2, true, BF, false>; /* stride 2: no split form yet */                      \
     if (!allow_max_dynamic_lds(reinterpret_cast<const void*>(kernel)))                                                           \
       return false;                                                                                              \
     kernel<<<grid, kMfBlock, f.lds, stream>>>(g, gout, x, rot, ws, f.tiles, f.parts, f.splits, f.pitch_x, f.th); \
   } else if (f.nx == 4)                                                                                          \
-    local_grad_filter_mfma_kernel<T, SH, SW, CELL0, 4, false, BF><<<grid, kMfBlock, f.lds, stream>>>(g, gout, x, rot, ws, f.tiles, f.parts, f.splits, f.pitch_x, 0); \
+    local_grad_filter_mfma_kernel<T, SH, SW, CELL0, 4, false, BF, SP><<<grid, kMfBlock, f.lds, stream>>>(g, gout, x, rot, ws, f.tiles, f.parts, f.splits, f.pitch_x, 0); \
   else                                                                                                           \
-    local_grad_filter_mfma_kernel<T, SH, SW, CELL0, kMfX, false, BF><<<grid, kMfBlock, f.lds, stream>>>(g, gout, x, rot, ws, f.tiles, f.parts, f.splits, f.pitch_x, 0);
+    local_grad_filter_mfma_kernel<T, SH, SW, CELL0, kMfX, false, BF, SP><<<grid, kMfBlock, f.lds, stream>>>(g, gout, x, rot, ws, f.tiles, f.parts, f.splits, f.pitch_x, 0);
       // 16-bit inputs with at least one full block of 16 channels per group: bfloat16 matrix instructions
-#define DK_LAUNCH(CELL0)                                          \
-  if constexpr (sizeof(T) == 2) {                                 \
-    if (g.channel / g.groups >= kMfCh) { DK_LAUNCH_BF(CELL0, true) } \
-    else { DK_LAUNCH_BF(CELL0, false) }                           \
-  } else { DK_LAUNCH_BF(CELL0, false) }
+      // float32 inputs: bfloat16 pairs (three products) unless switched off
+      const bool split = !path_disabled(kNoFilterSplit);
+#define DK_LAUNCH(CELL0)                                                    \
+  if constexpr (sizeof(T) == 2) {                                           \
+    if (g.channel / g.groups >= kMfCh) { DK_LAUNCH_BF(CELL0, true, false) } \
+    else { DK_LAUNCH_BF(CELL0, false, false) }                              \
+  } else if (split) { DK_LAUNCH_BF(CELL0, false, true) }                    \
+  else { DK_LAUNCH_BF(CELL0, false, false) }
       DK_LAUNCH(0)
       // the further 16-cell slices of a larger scope, into the same partials
       if constexpr (SH * SW > 16) DK_LAUNCH(16)
