@@ -51,27 +51,113 @@ OTHER_WORKLOADS = {
 }
 
 
-# HBM traffic per launch measured with the L2 counters (KiB per dispatch as rocprofv3 reports
-# them: FETCH_SIZE, WRITE_SIZE), one --pmc run each, for the workloads that were profiled.  The
-# same runs hold a plain elementwise kernel reading and writing |x| = 112896 KiB: WRITE_SIZE reads
-# 112896 for it, FETCH_SIZE reads 56469, so fetches are scaled by 2.0 and writes by 1.0.
-FETCH_SCALE, WRITE_SCALE = 112896.0 / 56469.2, 1.0
-MEASURED_KIB = {
-    ("cfg2", "fp32"): {
-        "forward": (64484.9, 135004.0),
-        "grad_input": (64510.5, 134518.0),
-        "grad_rotation": (127256.0, 16606.6),
-        "grad_filter": (122407.0 + 9232.5, 4608.0 + 9.0),  # accumulate kernel + ordered reduce of partials
-    },
+# HBM traffic per launch comes from two counter runs (rocprofv3 --pmc FETCH_SIZE, then WRITE_SIZE,
+# KiB per dispatch) of this script, summarised by `--traffic-from` into profiles/hbm_traffic_<workload>_
+# <dtype>.json together with a hash of the kernel sources they were measured on.  Each counter is
+# scaled by what it reads for plain elementwise kernels of known size in the same run (the
+# calibration multiply below and the 1 GiB streaming passes).
+TRAFFIC_RULES = {  # entry point -> regular expressions; a dispatch belongs to the first entry it matches
+    "forward": [r"dk::.*local_gather\w*_kernel<[^>]*\bfalse\b", r"dk::.*local_forward"],
+    "grad_input": [r"dk::.*local_gather\w*_kernel<[^>]*\btrue\b", r"dk::.*local_grad_input"],
+    "grad_rotation": [r"dk::.*local_grad_rotation"],
+    "grad_filter": [r"dk::.*local_grad_filter", r"dk::.*reduce_partials"],
 }
 
 
+def kernel_source_hash():
+    """sha256 over the kernel sources and the C header: the identity the traffic tables are tied to."""
+    import glob
+    import hashlib
+    h = hashlib.sha256()
+    csrc = os.path.join(ROOT, "deformable-kernels_amd", "csrc")
+    files = sorted(glob.glob(os.path.join(csrc, "*.hip")) + glob.glob(os.path.join(csrc, "*.h"))
+                   + glob.glob(os.path.join(ROOT, "include", "*.h")))
+    for f in files:
+        h.update(os.path.basename(f).encode() + b"\0")
+        with open(f, "rb") as fh:
+            h.update(fh.read())
+    return h.hexdigest()
+
+
+def traffic_file(workload, dtype):
+    return os.path.join(ROOT, "profiles", "hbm_traffic_%s_%s.json" % (workload, dtype))
+
+
 def measured_traffic(workload, dtype, kernel):
-    """HBM bytes per launch from the counters above (None where no counter run exists)."""
-    kib = MEASURED_KIB.get((workload, dtype), {}).get(kernel)
-    if kib is None:
-        return None
-    return int((kib[0] * FETCH_SCALE + kib[1] * WRITE_SCALE) * 1024)
+    """(HBM bytes per launch, stale) from the tracked counter table of this workload: bytes are None
+    where no table exists, the entry point was not matched, or the kernel sources have changed since
+    the counters were read (stale = True)."""
+    try:
+        with open(traffic_file(workload, dtype)) as fh:
+            table = json.load(fh)
+    except (OSError, ValueError):
+        return None, False
+    if table.get("kernel_source_sha256") != kernel_source_hash():
+        return None, True
+    e = table.get("entries", {}).get(kernel)
+    if not e:
+        return None, False
+    return int((e["fetch_kib"] * table["fetch_scale"] + e["write_kib"] * table["write_scale"]) * 1024), False
+
+
+def summarise_traffic(a):
+    """--traffic-from FETCH.db WRITE.db: reduce two rocprofv3 counter databases of `bench.py
+    --workload W --dtype D` (one run with --pmc FETCH_SIZE, one with --pmc WRITE_SIZE) to the tracked
+    table.  Runs on the CPU; needs no GPU."""
+    import re
+    import sqlite3
+    import subprocess
+    N, C, H, W = WORKLOADS[a.workload][:4]
+    esz = {"fp32": 4, "bf16": 2, "fp16": 2}[a.dtype]
+    x_kib = N * C * H * W * esz / 1024.0
+    out = {"workload": a.workload, "dtype": a.dtype, "kernel_source_sha256": kernel_source_hash(),
+           "unit": "KiB per call of the entry point, as rocprofv3 reports the counter",
+           "commands": ["rocprofv3 --pmc %s -d <dir> -o pmc -- python3 bench.py --workload %s --dtype %s --steps 3 "
+                        "--warmup 1 --no-cpu-baseline" % (c, a.workload, a.dtype) for c in ("FETCH_SIZE", "WRITE_SIZE")],
+           "entries": {}, "kernels": {}}
+    try:
+        head = subprocess.run(["git", "-C", ROOT, "rev-parse", "HEAD"], capture_output=True, text=True).stdout.strip()
+        dirty = subprocess.run(["git", "-C", ROOT, "status", "--porcelain", "--", "deformable-kernels_amd/csrc", "include"],
+                               capture_output=True, text=True).stdout.strip()
+        out["git_head"] = head + (" + uncommitted changes to the kernel sources" if dirty else "")
+    except OSError:
+        out["git_head"] = None
+    for counter, path, key in (("FETCH_SIZE", a.traffic_from[0], "fetch"), ("WRITE_SIZE", a.traffic_from[1], "write")):
+        rows = sqlite3.connect(path).execute(
+            "select kernel_name, value from counters_collection where counter_name = ? order by start", (counter,)).fetchall()
+        if not rows:
+            sys.exit("%s holds no %s values" % (path, counter))
+        # calibration: the elementwise multiplies, in launch order: |x| first, then 1 GiB each
+        mul = [v for n, v in rows if "MulFunctor" in n]
+        known = [x_kib] + [float(1 << 20)] * (len(mul) - 1)
+        out[key + "_scale"] = round(sum(known) / sum(mul), 4)
+        out[key + "_calibration"] = {"dispatches": len(mul), "known_kib": round(sum(known), 1), "counter_kib": round(sum(mul), 1),
+                                     "first_known_kib": x_kib, "first_counter_kib": mul[0]}
+        per_name = {}
+        for n, v in rows:
+            if "dk::" in n:
+                per_name.setdefault(n, []).append(v)
+        for n, vs in per_name.items():
+            short = re.sub(r"\(.*$", "", n.replace("(anonymous namespace)::", "")).replace("void ", "")
+            out["kernels"].setdefault(short, {})[key + "_kib"] = round(sum(vs) / len(vs), 1)
+            out["kernels"][short]["dispatches"] = len(vs)
+    # entry point = its kernels; a kernel launched k times per call counts k times
+    calls = {}
+    for short, k in out["kernels"].items():
+        for entry, rules in TRAFFIC_RULES.items():
+            if any(re.search(r, short) for r in rules):
+                calls.setdefault(entry, []).append(k)
+                break
+    for entry, ks in calls.items():
+        base = max(k["dispatches"] for k in ks)
+        out["entries"][entry] = {
+            "fetch_kib": round(sum(k.get("fetch_kib", 0.0) * k["dispatches"] / base for k in ks), 1),
+            "write_kib": round(sum(k.get("write_kib", 0.0) * k["dispatches"] / base for k in ks), 1)}
+    dest = a.traffic_out or traffic_file(a.workload, a.dtype)
+    with open(dest, "w") as fh:
+        json.dump(out, fh, indent=1, sort_keys=True)
+        fh.write("\n")
+    print("wrote", dest)
 
 
 def algorithmic_bytes(N, C, H, W, Ho, Wo, k, S, groups, esz):
@@ -102,7 +188,12 @@ def main():
     ap.add_argument("--dtype", default="fp32", choices=sorted(DTYPES))
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--kernels", default="", help="comma list restricting the per-kernel timing (tuning aid)")
+    ap.add_argument("--traffic-from", nargs=2, metavar=("FETCH_DB", "WRITE_DB"),
+                    help="summarise two rocprofv3 counter databases into the tracked traffic table and exit")
+    ap.add_argument("--traffic-out", default="", help="where --traffic-from writes (default: profiles/)")
     a = ap.parse_args()
+    if a.traffic_from:
+        return summarise_traffic(a)
     if a.gpus != 1:
         sys.exit("bench.py measures one GPU only: every box of this build has one GPU and no "
                  "multi-GPU path exists (the operator shards over the batch with no exchange); "
@@ -173,15 +264,23 @@ def main():
     # elementwise multiply rather than copy_(), which the runtime turns into its own blit.)
     calib = torch.empty_like(xg)
     torch.mul(xg, 1.0, out=calib)
-    # The same kernel for 0.2 s more: a GPU that has sat idle through the CPU-side input generation
-    # runs its first hundred steps below its steady clocks (50 steps from a cold start read 8 % low),
-    # however few warm-up steps the caller asks for.
-    t_wake = time.perf_counter()
-    while time.perf_counter() - t_wake < 0.2:
-        for _ in range(20):
-            torch.mul(xg, 1.0, out=calib)
-        torch.cuda.synchronize()
     del calib
+    # Wake-up, untimed and before the warm-up steps: a GPU that has sat idle through the CPU-side
+    # input generation runs its first steps below its steady clocks (20 timed steps straight after 5
+    # warm-up steps read 13 % low), so the step itself is run in windows of 10 until two consecutive
+    # windows agree within 2 % (or 1 s has passed); `wake_ms` says how long that took.
+    t_wake = time.perf_counter()
+    prev = None
+    while time.perf_counter() - t_wake < 1.0:
+        t_win = time.perf_counter()
+        for _ in range(10):
+            step()
+        torch.cuda.synchronize()
+        win = time.perf_counter() - t_win
+        if prev is not None and abs(win - prev) <= 0.02 * prev:
+            break
+        prev = win
+    wake_ms = (time.perf_counter() - t_wake) * 1e3
     for _ in range(a.warmup):
         step()
     torch.cuda.synchronize()
@@ -224,6 +323,7 @@ def main():
     dominant = max((n for n in per_kernel_us if n != "backward"), key=per_kernel_us.get, default="backward")
     achieved = per_kernel_bytes[dominant] / (per_kernel_us[dominant] * 1e-6) / 1e9
 
+    traffic, traffic_stale = measured_traffic(a.workload, a.dtype, dominant)
     result = {
         "metric": "DK fwd+bwd achieved HBM GB/s",
         "value": round(gbps, 2),
@@ -231,6 +331,7 @@ def main():
         "n_gpus": 1,
         "steps": a.steps,
         "warmup": a.warmup,
+        "wake_ms": round(wake_ms, 1),
         "ms_per_step": round(ms_per_step, 4),
         "higher_is_better": True,
         "scaling": "weak",
@@ -254,9 +355,11 @@ def main():
             "unit": "GB/s",
             "frac": round(achieved / HBM_PEAK_GBPS, 4),
             "algorithmic_bytes": per_kernel_bytes[dominant],
-            "traffic": measured_traffic(a.workload, a.dtype, dominant),
+            "traffic": traffic,
         },
     }
+    if traffic_stale:
+        result["roofline"]["traffic_stale"] = True  # kernel sources changed since the counters were read
 
     if not a.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(N, C, H, W, k, S, stride, pad, dil, groups, rot_std, esz)
@@ -476,8 +579,20 @@ def cpu_baseline(N, C, H, W, k, S, stride, pad, dil, groups, rot_std, esz):
     n = min(N, 16)
     x, wt, rot, gout, cfg = make_local(n, C, H, W, k, S, stride, pad, dil, groups, rot_std, seed=0)
     xs, ws_, rs, gs = [t.numpy() for t in (x, wt, rot, gout)]
-    threads = min(orc.max_threads(), 16)
+    # The threads this job may use: the OpenMP default (OMP_NUM_THREADS where the host sets a CPU share
+    # for the job) bounded by the CPUs this process may run on; `host_cpus` is the whole machine.
+    try:
+        allowed = len(os.sched_getaffinity(0))
+    except AttributeError:
+        allowed = os.cpu_count() or 1
+    threads = max(1, min(orc.max_threads(), allowed))
     orc.set_threads(threads)
+    model = ""
+    try:
+        with open("/proc/cpuinfo") as fh:
+            model = next((ln.split(":", 1)[1].strip() for ln in fh if ln.startswith("model name")), "")
+    except OSError:
+        pass
     # passes over the sample until about 12 s of CPU work are done (at least 3 passes)
     times = []
     t_all = time.perf_counter()
@@ -500,6 +615,9 @@ def cpu_baseline(N, C, H, W, k, S, stride, pad, dil, groups, rot_std, esz):
         "value": round((fwd_b + bwd_b) / mean / 1e9, 3),
         "unit": "GB/s",
         "cores": threads,
+        "host_cpus": os.cpu_count(),
+        "cpus_allowed": allowed,
+        "cpu_model": model,
         "one_core_value": round((fwd_b + bwd_b) * 2 / n / t_one / 1e9, 4),
         "kind": "port",
         "sample": "first %d of %d images of the same seeded workload, fwd + 3 grads, fp32, mean of %d passes "

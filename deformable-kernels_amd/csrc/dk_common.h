@@ -175,6 +175,10 @@ using rsrc_t = __amdgpu_buffer_rsrc_t;
 // they push the operands of the next kernel out of the 256 MB memory-side cache
 // (measured: 6 % of a forward + backward step on a 245 MB layer).
 constexpr int kStreamingStore = 2;  // "nt" bit of the buffer instruction's cache-policy field
+// 2-byte stores keep the default policy: a wave's 2-byte stores cover half a cache line or less, and
+// written non-temporally they reached memory as partial lines (WRITE_SIZE 47 % above the tensor's
+// size on a 58 MB bfloat16 result; forward and grad input 4-6 % slower than with this policy).
+constexpr int kMergedStore = 0;
 
 template <typename T>
 __device__ __forceinline__ rsrc_t plane_rsrc(const T* base, int elems) {
@@ -197,12 +201,12 @@ __device__ __forceinline__ void buf_st(rsrc_t r, unsigned byte_off, float v, flo
 }
 __device__ __forceinline__ void buf_st(rsrc_t r, unsigned byte_off, float v, __half*) {
   const _Float16 h = static_cast<_Float16>(v);
-  __builtin_amdgcn_raw_buffer_store_b16(__builtin_bit_cast(unsigned short, h), r, (int)byte_off, 0, kStreamingStore);
+  __builtin_amdgcn_raw_buffer_store_b16(__builtin_bit_cast(unsigned short, h), r, (int)byte_off, 0, kMergedStore);
 }
 __device__ __forceinline__ void buf_st(rsrc_t r, unsigned byte_off, float v, bf16_t*) {
   bf16_t t;
   st(&t, v);
-  __builtin_amdgcn_raw_buffer_store_b16(t.bits, r, (int)byte_off, 0, kStreamingStore);
+  __builtin_amdgcn_raw_buffer_store_b16(t.bits, r, (int)byte_off, 0, kMergedStore);
 }
 
 }  // namespace dk

@@ -476,7 +476,7 @@ __global__ __launch_bounds__(kThreads, 4) void local_gather_mfma_kernel(
         // p is a multiple of 4, so the four pixels are inside the plane and 16-byte aligned
         if constexpr (sizeof(T) == 4) {
           f4 v = {acc[0], acc[1], acc[2], acc[3]};
-          __builtin_nontemporal_store(v, reinterpret_cast<f4*>(out));
+          *reinterpret_cast<f4*>(out) = v;  // default policy: the wave's 64-byte runs merge to whole lines in L2
         } else {
           struct { T e[4]; } pk;
 #pragma unroll

@@ -225,11 +225,13 @@ def test_headline_shape_properties_at_full_size():
         assert abs(a - b) < 1e-6 * max(abs(a), 1.0)
 
 
-@pytest.mark.parametrize("switch", ["DK_NO_MFMA", "DK_NO_ROWS"])
+@pytest.mark.parametrize("switch", ["DK_NO_MFMA", "DK_NO_ROWS", "DK_NO_GATHER_MFMA", "DK_NO_FILTER_SPLIT"])
 def test_more_general_kernels_on_a_same_width_shape(switch, switch_off):
     """The dispatch prefers the most specialised kernel; the library's test switches make it take
     the next more general family for the same shape (dense grad filter instead of the
-    matrix-core one; per-tap loads instead of the row kernels), which must give the same results."""
+    matrix-core one; per-tap loads instead of the row kernels; the row kernels instead of the
+    matrix-core forward / grad input; float32 matrix instructions instead of bfloat16 pairs in the
+    grad filter), which must give the same results."""
     switch_off(switch)
     case = (2, 40, 20, 24, 3, (4, 4), 1, 1, 1, 2, 1.0)
     inputs, got = _run(case, torch.float32)
