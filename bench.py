@@ -32,10 +32,13 @@ WORKLOADS = {
     # name: (N, C, H, W, k, S, stride, pad, dil, groups, rot_std)
     "cfg2": (64, 144, 56, 56, 3, (4, 4), 1, 1, 1, 1, 1.0),
     "cfg1": (2, 32, 28, 28, 3, (4, 4), 1, 1, 1, 1, 0.5),
-    # config 3 (GlobalDeformKernel2d, run with --dtype fp16) as the module's fused route issues it:
-    # the local operator on the layer's shape, scope 5 x 5 (the rotation is one value per image there)
-    "cfg3": (128, 256, 28, 28, 3, (5, 5), 1, 1, 1, 1, 0.5),
+    # the per-pixel operator on config 3's layer shape, scope 5 x 5 (what GlobalDeformKernel2d's
+    # `fused` route issues, with one rotation per image repeated over the pixels)
+    "cfg3_local": (128, 256, 28, 28, 3, (5, 5), 1, 1, 1, 1, 0.5),
 }
+# config 3 (GlobalDeformKernel2d, run with --dtype fp16): N, C, H, W, k, S, stride, pad -- the layer's
+# operator sequence: kernels sampled per image (N-d sampler), per-image depthwise convolution, and back
+GLOBAL_WORKLOADS = {"cfg3": (128, 256, 28, 28, 3, (5, 5), 1, 1)}
 DTYPES = {"fp32": "float32", "bf16": "bfloat16", "fp16": "float16"}
 
 # Other rows of the operator path, timed per entry point with --workload (not the headline metric).
@@ -183,7 +186,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=50)
-    ap.add_argument("--workload", default="cfg2", choices=sorted(WORKLOADS) + sorted(OTHER_WORKLOADS) + ["mbv2_dk", "layer_cfg2"])
+    ap.add_argument("--workload", default="cfg2", choices=sorted(WORKLOADS) + sorted(OTHER_WORKLOADS) + sorted(GLOBAL_WORKLOADS) + ["mbv2_dk", "layer_cfg2"])
     ap.add_argument("--batch", type=int, default=64, help="batch size of the mbv2_dk workload")
     ap.add_argument("--dtype", default="fp32", choices=sorted(DTYPES))
     ap.add_argument("--no-cpu-baseline", action="store_true")
@@ -211,6 +214,8 @@ def main():
         return layer_workload(a)
     if a.workload in OTHER_WORKLOADS:
         return other_workload(a)
+    if a.workload in GLOBAL_WORKLOADS:
+        return global_workload(a)
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
     tdtype = getattr(torch, DTYPES[a.dtype])
@@ -376,6 +381,120 @@ def _time_us(fn, reps):
     e1.record()
     e1.synchronize()
     return e0.elapsed_time(e1) * 1e3 / reps
+
+
+def global_workload(a):
+    """Forward + backward of GlobalDeformKernel2d's operator sequence (config 3) through the C ABI:
+    nd_linear_sample of the N * 9 per-image taps from the [C, 5, 5] scope weights, the per-image
+    depthwise convolution, its two gradients, and the sampler's two gradients.  The pooled branch
+    (mean, fc, clamp) that predicts the coordinates is framework code in the reference and is not
+    part of the step; the coordinates are synthetic, uniform over the scope."""
+    import torch
+    from deformable_kernels.ops.deform_kernel import _lib
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    tdtype = getattr(torch, DTYPES[a.dtype])
+    N, C, H, W, k, S, stride, pad = GLOBAL_WORKLOADS[a.workload]
+    taps = k * k
+    g = torch.Generator().manual_seed(0)
+    x = torch.randn(N, C, H, W, generator=g).to(tdtype).to(dev)
+    scope = torch.randn(C, S[0], S[1], generator=g).to(tdtype).to(dev)
+    coord = (torch.rand(N * taps, 2, generator=g) * (S[0] - 1)).to(tdtype).to(dev)
+    L, P = _lib.lib(), _lib.ptr
+    cdesc = _lib.ConvDesc(N, C, H, W, k, k, stride, stride, pad, pad, 1, 1, 1, 1, 1, _lib.dtype_tag(x), 0, 0.0, 0.0)
+    oh, ow = ctypes.c_int32(0), ctypes.c_int32(0)
+    _lib.check(L.dk_conv_out_size(cdesc, ctypes.byref(oh), ctypes.byref(ow)), "shape")
+    gout = torch.randn(N, C, oh.value, ow.value, generator=g).to(tdtype).to(dev)
+    ndesc = _lib.nd_desc(scope, coord)
+    # the sampled kernels stay as the sampler writes them, [N * 9, C]: the convolution takes them
+    # through element strides (image, channel, tap row, tap column), its kernel gradient likewise
+    sampled = torch.empty(N * taps, C, dtype=tdtype, device=dev)
+    w_img, wstr = sampled, (ctypes.c_int64 * 4)(taps * C, 1, k * C, C)
+    out, gin = torch.empty_like(gout), torch.empty_like(x)
+    g_sampled, g_scope, g_coord = torch.empty_like(sampled), torch.empty_like(scope), torch.empty_like(coord)
+    gw_img = g_sampled
+    wf, nf = _lib.workspace(L.dk_nd_linear_sample_forward_workspace(ndesc), dev)
+    wd, nd_ = _lib.workspace(L.dk_nd_linear_sample_backward_data_workspace(ndesc), dev)
+    order, wo, no_ = None, None, 0
+    if L.dk_nd_linear_sample_order_bytes(ndesc):
+        order = torch.empty(L.dk_nd_linear_sample_order_bytes(ndesc), dtype=torch.uint8, device=dev)
+        wo, no_ = _lib.workspace(L.dk_nd_linear_sample_order_workspace(ndesc), dev)
+    st = _lib.stream_ptr(x)
+
+    def k_sample():
+        if order is not None:
+            _lib.check(L.dk_nd_linear_sample_order(ndesc, P(coord), P(order), P(wo), no_, st), "order")
+        _lib.check(L.dk_nd_linear_sample_forward(ndesc, P(scope), P(coord), P(order), P(sampled), P(wf), nf, st), "sample")
+
+    def k_forward():
+        _lib.check(L.dk_image_depthwise_forward(cdesc, P(x), P(w_img), wstr, P(out), st), "conv forward")
+
+    def k_grad_input():
+        _lib.check(L.dk_image_depthwise_backward_data(cdesc, P(gout), P(w_img), wstr, P(gin), st), "conv grad input")
+
+    def k_grad_kernels():
+        _lib.check(L.dk_image_depthwise_backward_weight(cdesc, P(gout), P(x), P(gw_img), wstr, st), "conv grad kernels")
+
+    def k_sample_backward():
+        _lib.check(L.dk_nd_linear_sample_backward_data(ndesc, P(g_sampled), P(coord), P(order), P(g_scope), P(wd), nd_, st),
+                   "sample grad data")
+        _lib.check(L.dk_nd_linear_sample_backward_coord(ndesc, P(g_sampled), P(scope), P(coord), P(order), P(g_coord),
+                                                        P(wf), nf, st), "sample grad coord")
+
+    kernels = {"sample_kernels": k_sample, "forward": k_forward, "grad_input": k_grad_input,
+               "grad_kernels": k_grad_kernels, "sample_backward": k_sample_backward}
+
+    def step():
+        for fn in kernels.values():
+            fn()
+
+    calib = torch.empty_like(x)
+    torch.mul(x, 1.0, out=calib)
+    del calib
+    t_wake, prev = time.perf_counter(), None
+    while time.perf_counter() - t_wake < 1.0:
+        t_win = time.perf_counter()
+        for _ in range(10):
+            step()
+        torch.cuda.synchronize()
+        win = time.perf_counter() - t_win
+        if prev is not None and abs(win - prev) <= 0.02 * prev:
+            break
+        prev = win
+    wake_ms = (time.perf_counter() - t_wake) * 1e3
+    for _ in range(a.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(a.steps):
+        step()
+    torch.cuda.synchronize()
+    ms_per_step = (time.perf_counter() - t0) * 1e3 / a.steps
+    us = {name: _time_us(fn, max(a.steps, 20)) for name, fn in kernels.items()}
+    e = x.element_size()
+    bx, by, bw = x.numel() * e, gout.numel() * e, w_img.numel() * e
+    small = (sampled.numel() + scope.numel() + coord.numel()) * e
+    nbytes = {"sample_kernels": small + 2 * bw, "forward": bx + bw + by, "grad_input": by + bw + bx,
+              "grad_kernels": by + bx + bw, "sample_backward": 2 * small + 2 * bw}
+    step_bytes = sum(nbytes.values())
+    dominant = max(us, key=us.get)
+    achieved = nbytes[dominant] / (us[dominant] * 1e-6) / 1e9
+    gbps = step_bytes / (ms_per_step * 1e-3) / 1e9
+    print(json.dumps({
+        "metric": "GlobalDK fwd+bwd achieved HBM GB/s", "value": round(gbps, 2), "unit": "GB/s", "n_gpus": 1,
+        "steps": a.steps, "warmup": a.warmup, "wake_ms": round(wake_ms, 1), "ms_per_step": round(ms_per_step, 4),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": {"fp32": "f32", "bf16": "bf16", "fp16": "f16"}[a.dtype], "data": "synthetic",
+        "config": {"workload": "%s: GlobalDeformKernel2d operator sequence fwd+bwd N=%d C=%d %dx%d k=%d scope=%dx%d "
+                               "stride=%d pad=%d %s" % (a.workload, N, C, H, W, k, S[0], S[1], stride, pad, a.dtype),
+                   "algorithmic_MB_per_step": round(step_bytes / 1e6, 2)},
+        "pct_of_hbm_peak": round(100.0 * gbps / HBM_PEAK_GBPS, 2),
+        "images_per_s": round(N / (ms_per_step * 1e-3), 1),
+        "kernel_us": {n: round(v, 2) for n, v in us.items()},
+        "roofline": {"kernel": dominant, "bound": "hbm", "achieved": round(achieved, 2), "peak": HBM_PEAK_GBPS,
+                     "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4), "algorithmic_bytes": nbytes[dominant],
+                     "traffic": None},
+    }))
 
 
 def other_workload(a):

@@ -28,7 +28,8 @@ unsigned switches_from_environment() {
       {"DK_NO_S2_QUADS", kNoS2Quads}, {"DK_NO_DEFORM_FAST", kNoDeformFast}, {"DK_NO_DEFORM_CH", kNoDeformCh},
       {"DK_NO_DEFORM_CH_BIG", kNoDeformChBig}, {"DK_NO_DEFORM_MFMA", kNoDeformMfma},
       {"DK_NO_ND_BINS", kNoNdBins}, {"DK_NO_ND_MFMA", kNoNdMfma}, {"DK_NO_GATHER_MFMA", kNoGatherMfma},
-      {"DK_NO_FILTER_SPLIT", kNoFilterSplit}};
+      {"DK_NO_FILTER_SPLIT", kNoFilterSplit}, {"DK_NO_IMAGE_FLAT", kNoImageFlat},
+      {"DK_NO_ND_SMALL", kNoNdSmall}};
   unsigned m = 0;
   for (const auto& v : vars)
     if (std::getenv(v.name)) m |= v.bit;
@@ -496,6 +497,87 @@ int dk_deformable_sample_depthwise_backward_rotation(const dk_conv_desc* desc, c
 }
 
 // ---- offset branch -----------------------------------------------------------------------
+
+// ---- depthwise convolution with one kernel per image and channel ---------------------------
+
+// The kernel tensor's strides as the kernels take them; false for a layout whose offsets do not fit
+// (negative strides, or a span of 2^31 elements or more).
+static bool kernel_strides(const Geo& g, const int64_t* given, long (&ws)[4], const long** out) {
+  *out = nullptr;
+  if (!given) return true;
+  const long ext[4] = {g.batch, g.channel, g.k_h, g.k_w};
+  long span = 0;
+  for (int i = 0; i < 4; ++i) {
+    if (given[i] < 0 || given[i] >= kMaxElems) return false;
+    ws[i] = (long)given[i];
+    span += (ext[i] - 1) * ws[i];
+  }
+  if (span >= kMaxElems) return false;
+  *out = ws;
+  return true;
+}
+
+int dk_image_depthwise_supported(const dk_conv_desc* desc) {
+  Geo g;
+  return make_geo(desc, g) == DK_OK && image_conv_supported(g, desc->dtype);
+}
+
+int dk_image_depthwise_forward(const dk_conv_desc* desc, const void* input, const void* weight,
+                               const int64_t* weight_strides, void* output, void* stream) {
+  Geo g;
+  const int rc = make_geo(desc, g);
+  if (rc != DK_OK) return rc;
+  if (!input || !weight || !output) return DK_ERR_NULL_POINTER;
+  if (!image_conv_supported(g, desc->dtype)) return DK_ERR_UNSUPPORTED;
+  long ws_buf[4];
+  const long* ws;
+  if (!kernel_strides(g, weight_strides, ws_buf, &ws)) return DK_ERR_BAD_SHAPE;
+  if (g.batch == 0) return DK_OK;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  bool ok = true;
+  const int st = by_dtype(desc->dtype, [&]<typename T>() {
+    ok = image_conv_forward<T>(g, ws, in<T>(input), in<T>(weight), out<T>(output), s);
+  });
+  return ok ? st : DK_ERR_UNSUPPORTED;
+}
+
+int dk_image_depthwise_backward_data(const dk_conv_desc* desc, const void* out_grad, const void* weight,
+                                     const int64_t* weight_strides, void* in_grad, void* stream) {
+  Geo g;
+  const int rc = make_geo(desc, g);
+  if (rc != DK_OK) return rc;
+  if (!out_grad || !weight || !in_grad) return DK_ERR_NULL_POINTER;
+  if (!image_conv_supported(g, desc->dtype)) return DK_ERR_UNSUPPORTED;
+  long ws_buf[4];
+  const long* ws;
+  if (!kernel_strides(g, weight_strides, ws_buf, &ws)) return DK_ERR_BAD_SHAPE;
+  if (g.batch == 0) return DK_OK;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  bool ok = true;
+  const int st = by_dtype(desc->dtype, [&]<typename T>() {
+    ok = image_conv_grad_input<T>(g, ws, in<T>(out_grad), in<T>(weight), out<T>(in_grad), s);
+  });
+  return ok ? st : DK_ERR_UNSUPPORTED;
+}
+
+int dk_image_depthwise_backward_weight(const dk_conv_desc* desc, const void* out_grad, const void* input,
+                                       void* weight_grad, const int64_t* weight_strides, void* stream) {
+  Geo g;
+  const int rc = make_geo(desc, g);
+  if (rc != DK_OK) return rc;
+  if (!out_grad || !input || !weight_grad) return DK_ERR_NULL_POINTER;
+  if (!image_conv_supported(g, desc->dtype)) return DK_ERR_UNSUPPORTED;
+  long ws_buf[4];
+  const long* ws;
+  if (!kernel_strides(g, weight_strides, ws_buf, &ws)) return DK_ERR_BAD_SHAPE;
+  if (g.batch == 0) return DK_OK;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  bool ok = true;
+  const int st = by_dtype(desc->dtype, [&]<typename T>() {
+    ok = image_conv_grad_weight<T>(g, ws, in<T>(out_grad), in<T>(input), out<T>(weight_grad), s);
+  });
+  return ok ? st : DK_ERR_UNSUPPORTED;
+}
 
 static int check_offset_conv(const dk_offset_conv_desc* d) {
   if (!d) return DK_ERR_NULL_POINTER;

@@ -28,6 +28,8 @@ enum TestSwitch : unsigned {
   kNoNdMfma = 1u << 9,      // DK_NO_ND_MFMA      the matrix-core N-d kernels
   kNoGatherMfma = 1u << 10, // DK_NO_GATHER_MFMA  the matrix-core forward / grad input (the row kernels run instead)
   kNoFilterSplit = 1u << 11, // DK_NO_FILTER_SPLIT the bfloat16-pair form of the float32 matrix-core grad filter (fp32 matrix instructions instead)
+  kNoNdSmall = 1u << 13,    // DK_NO_ND_SMALL     the few-points-on-a-tiny-volume path of the N-d sampler
+  kNoImageFlat = 1u << 12,  // DK_NO_IMAGE_FLAT   the flat-copy kernels of the per-image depthwise convolution (the band kernels run instead)
 };
 unsigned test_switches();  // dk_api.hip
 inline bool path_disabled(unsigned sw) { return (test_switches() & sw) != 0; }
@@ -119,5 +121,18 @@ bool offset_conv_wgrad(int batch, int cin, int cout, int h, int w, const float* 
                        void* ws, hipStream_t stream);
 bool offset_conv_forward(int batch, int cin, int cout, int h, int w, const float* x, const float* weight,
                          const float* bias, float* out, void* ws, hipStream_t stream);
+
+// dk_image_conv.hip: depthwise convolution with one kernel per (image, channel) plane, all dtypes
+bool image_conv_supported(const Geo& g, int dtype);
+// wstrides: element strides of the kernel tensor's (image, channel, tap row, tap column) axes, or null
+// for a contiguous [N, C, k_h, k_w] tensor
+template <typename T>
+bool image_conv_forward(const Geo& g, const long* wstrides, const T* x, const T* weight, T* out, hipStream_t stream);
+template <typename T>
+bool image_conv_grad_input(const Geo& g, const long* wstrides, const T* gout, const T* weight, T* gin,
+                           hipStream_t stream);
+template <typename T>
+bool image_conv_grad_weight(const Geo& g, const long* wstrides, const T* gout, const T* x, T* gweight,
+                            hipStream_t stream);
 
 }  // namespace dk

@@ -369,6 +369,198 @@ __global__ __launch_bounds__(kBlock) void nd_grad_data_cl_kernel(NdGeo g, const 
 }
 
 // ---------------------------------------------------------------------------
+// few points on a tiny volume (GlobalDeformKernel2d: 9 points per image on a 5 x 5 scope, hundreds of
+// channels).  The forward takes the direct kernel above (one launch, the volume stays in cache);
+// grad data and grad coord are one launch each here instead of fill + atomics + transpose /
+// transpose + kernel.  These calls are bound by the latency of their few dependent loads, so both
+// kernels know the number of dimensions at compile time (no branches between the loads) and issue
+// every load of a stage before the first use.
+//
+// grad data: a small dense product on the matrix cores (below; scattering into sums instead --
+// LDS or global float atomics on 25 x 256 sums that each receive 184 additions -- took 75-100 us).
+// grad coord: one wave per point, lanes over channels; the volume is read where it lies.
+// ---------------------------------------------------------------------------
+constexpr int kSmallMaxCells = 64;
+
+// The point's low corner and fractions for NDIM dimensions (load_point above, without its loop over
+// DK_ND_MAX_DIMS); b is clamped by the caller.
+template <typename T, int NDIM>
+__device__ __forceinline__ NdPoint<float> small_point(const NdGeo& g, const T* coord_b) {
+  float x[NDIM];
+#pragma unroll
+  for (int d = 0; d < NDIM; ++d) x[d] = ld(coord_b + d);
+  NdPoint<float> p;
+  p.inside = true;
+#pragma unroll
+  for (int d = 0; d < DK_ND_MAX_DIMS; ++d) {
+    p.low[d] = 0;
+    p.frac[d] = 0.f;
+  }
+#pragma unroll
+  for (int d = 0; d < NDIM; ++d) {
+    const float xf = floorf(x[d]);
+    const bool in = x[d] > -1.f && x[d] < (float)g.shape[d];
+    if (!in) p.inside = false;
+    p.low[d] = in ? (int)xf : 0;
+    p.frac[d] = x[d] - xf;
+  }
+  return p;
+}
+
+// grad data as a small dense product on the matrix cores: gdata[c][cell] = sum_b gout[b][c] * W[b][cell],
+// W[b][.] being the point's 2^n corner weights spread over a row of zeros.  A workgroup of 16 waves owns
+// 16 channels.  Per chunk of points it writes W into LDS (row = point, 16 cells per column tile), then
+// each wave multiplies its share of the chunk's points, four at a time, with
+// v_mfma_f32_16x16x4_f32 (M = channels, N = cells, K = points; fp32 products and sums).  The waves'
+// 16 x 16 tiles are added in wave order at the end: no atomics, a fixed order of additions.
+typedef float nd_f4 __attribute__((ext_vector_type(4)));
+constexpr int kSmallTileMax = 4;                 // column tiles of 16 cells: volumes of up to 64 cells
+constexpr int kSmallWBytes = 144 * 1024;         // LDS for W
+
+template <typename T, int NDIM, int NT>
+__global__ __launch_bounds__(1024) void nd_small_grad_data_kernel(NdGeo g, const T* __restrict__ gout,
+                                                                   const T* __restrict__ coord,
+                                                                   T* __restrict__ gdata, int chunk_points) {
+  constexpr int NC = 1 << NDIM;
+  constexpr int ROW = NT * 16;  // floats of a row of W
+  extern __shared__ __align__(16) unsigned char small_lds[];
+  float* W = reinterpret_cast<float*>(small_lds);
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int c = min(blockIdx.x * 16 + (lane & 15), g.channel - 1);  // lanes past the last channel repeat it; not stored
+  nd_f4 acc[NT];
+#pragma unroll
+  for (int t = 0; t < NT; ++t) acc[t] = nd_f4{0.f, 0.f, 0.f, 0.f};
+
+  for (long chunk0 = 0; chunk0 < g.batch; chunk0 += chunk_points) {
+    const int npts = (int)min((long)chunk_points, g.batch - chunk0);
+    const int rows = (npts + 63) & ~63;  // whole 4-point steps for every wave; the extra rows stay zero
+    // this thread's points of the chunk (loads first), then W = 0, then the corners' weights
+    NdPoint<float> p[2];
+    bool has[2];
+#pragma unroll
+    for (int r = 0; r < 2; ++r) {
+      const int q = threadIdx.x + 1024 * r;
+      has[r] = q < npts;
+      p[r] = small_point<T, NDIM>(g, coord + min(chunk0 + q, g.batch - 1) * NDIM);
+    }
+    __syncthreads();  // the previous chunk's products have read W
+    for (int i = threadIdx.x; i < rows * ROW / 4; i += 1024) reinterpret_cast<nd_f4*>(W)[i] = nd_f4{0.f, 0.f, 0.f, 0.f};
+    __syncthreads();
+#pragma unroll
+    for (int r = 0; r < 2; ++r) {
+      if (has[r] && p[r].inside) {
+#pragma unroll
+        for (int i = 0; i < NC; ++i) {
+          long o;
+          float w;
+          if (corner<float>(g, p[r], (unsigned)i, -1, o, w)) W[(threadIdx.x + 1024 * r) * ROW + (int)o] = w;
+        }
+      }
+    }
+    __syncthreads();
+    // wave w: rows [w * share, (w + 1) * share), share a multiple of 4
+    const int share = rows / 16;
+    const int r0 = wave * share;
+    for (int s0 = 0; s0 < share; s0 += 32) {  // eight 4-point steps at a time, their out_grad loads first
+      T raw[8];
+#pragma unroll
+      for (int k = 0; k < 8; ++k) {
+        const int row = r0 + s0 + 4 * k + (lane >> 4);
+        raw[k] = gout[min(chunk0 + row, g.batch - 1) * g.channel + c];
+      }
+#pragma unroll
+      for (int k = 0; k < 8; ++k) {
+        if (s0 + 4 * k < share) {  // uniform over the wave
+          const int row = r0 + s0 + 4 * k + (lane >> 4);
+          const float a = ld(&raw[k]);  // rows past the chunk's points multiply a zero row of W
+#pragma unroll
+          for (int t = 0; t < NT; ++t)
+            acc[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(a, W[row * ROW + t * 16 + (lane & 15)], acc[t], 0, 0, 0);
+        }
+      }
+    }
+  }
+  __syncthreads();
+  // the waves' tiles through LDS (W's space), added in wave order
+  float* red = W;  // [16 waves][NT][16 channels][16 cells]
+#pragma unroll
+  for (int t = 0; t < NT; ++t)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) red[((wave * NT + t) * 16 + 4 * (lane >> 4) + i) * 16 + (lane & 15)] = acc[t][i];
+  __syncthreads();
+  const int cells = (int)g.prod_shape;
+  for (int i = threadIdx.x; i < NT * 256; i += 1024) {
+    const int t = i >> 8, m = (i >> 4) & 15, n = i & 15;
+    float v = 0.f;
+    for (int w = 0; w < 16; ++w) v += red[((w * NT + t) * 16 + m) * 16 + n];
+    const int co = blockIdx.x * 16 + m, cell = t * 16 + n;
+    if (co < g.channel && cell < cells) st(gdata + (size_t)co * g.prod_shape + cell, v);
+  }
+}
+
+template <typename T, int NDIM>
+__global__ __launch_bounds__(kBlock) void nd_small_grad_coord_kernel(NdGeo g, const T* __restrict__ gout,
+                                                                     const T* __restrict__ data,
+                                                                     const T* __restrict__ coord,
+                                                                     T* __restrict__ gcoord) {
+  constexpr int NC = 1 << NDIM;
+  const int lane = threadIdx.x & 63;
+  const long b = (long)blockIdx.x * (kBlock / 64) + (threadIdx.x >> 6);
+  if (b >= g.batch) return;
+  const NdPoint<float> p = small_point<T, NDIM>(g, coord + b * NDIM);
+  int off[NC];
+  float dw[NDIM][NC];  // derivative weights (ND.cu:161,165); 0 for a corner outside the volume
+#pragma unroll
+  for (int i = 0; i < NC; ++i) {
+    long o = 0;
+    float w = 0.f;
+    const bool ok = p.inside && corner<float>(g, p, (unsigned)i, -1, o, w);
+    off[i] = ok ? (int)o : 0;
+#pragma unroll
+    for (int d = 0; d < NDIM; ++d) {
+      long o2;
+      float w2 = 0.f;
+      const bool ok2 = ok && corner<float>(g, p, (unsigned)i, d, o2, w2);
+      dw[d][i] = ok2 ? w2 : 0.f;
+    }
+  }
+  float part[NC];
+#pragma unroll
+  for (int i = 0; i < NC; ++i) part[i] = 0.f;
+  const T* grow = gout + b * g.channel;
+  for (int c0 = 0; c0 < g.channel; c0 += 256) {
+    // four 64-channel tiles at a time, loads first (channels past the end repeat the last one with a zero out_grad)
+    T graw[4], draw[4][NC];
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+      const int c = min(c0 + 64 * t + lane, g.channel - 1);
+      graw[t] = grow[c];
+#pragma unroll
+      for (int i = 0; i < NC; ++i) draw[t][i] = data[(size_t)c * g.prod_shape + off[i]];
+    }
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+      const float go = c0 + 64 * t + lane < g.channel ? ld(&graw[t]) : 0.f;
+#pragma unroll
+      for (int i = 0; i < NC; ++i) part[i] += go * ld(&draw[t][i]);
+    }
+  }
+  float gd[NDIM];
+#pragma unroll
+  for (int d = 0; d < NDIM; ++d) gd[d] = 0.f;
+#pragma unroll
+  for (int i = 0; i < NC; ++i) {
+    const float v = wave_sum(part[i]);
+#pragma unroll
+    for (int d = 0; d < NDIM; ++d) gd[d] += v * dw[d][i];
+  }
+  if (lane == 0) {
+#pragma unroll
+    for (int d = 0; d < NDIM; ++d) st(gcoord + b * NDIM + d, gd[d]);
+  }
+}
+
+// ---------------------------------------------------------------------------
 // binned channel-last path: many points per cell of the volume
 //
 // With more points than cells, points that fall into the same cell read (forward, grad coord)
@@ -1134,8 +1326,16 @@ void transpose(const A* in, B* out, long rows, long cols, hipStream_t stream) {
 
 // The channel-last path pays for a transpose of `data`; it is taken for 1..3 dimensions in
 // fp32 / fp16 / bf16 when there are enough (point, channel) pairs to amortise it.
+// Few points on a tiny volume: the direct kernels and the one-launch grad data (nd_small_grad_data_kernel).
+bool nd_small(const dk_nd_desc& d) {
+  if (d.dtype == DK_F64 || d.dims > kClMaxDims || path_disabled(kNoNdSmall)) return false;
+  long prod = 1;
+  for (int i = 0; i < d.dims; ++i) prod *= d.shape[i];
+  return prod <= kSmallMaxCells && d.batch > 0 && d.batch * d.channel <= (1L << 20);
+}
+
 bool nd_use_channel_last(const dk_nd_desc& d) {
-  if (d.dtype == DK_F64 || d.dims > kClMaxDims) return false;
+  if (d.dtype == DK_F64 || d.dims > kClMaxDims || nd_small(d)) return false;
   long prod = 1;
   for (int i = 0; i < d.dims; ++i) prod *= d.shape[i];
   if (prod > 2147483647L / 4) return false;  // corner offsets are kept as 32-bit element counts
@@ -1257,6 +1457,7 @@ void nd_forward(const dk_nd_desc& d, const T* data, const T* coord, T* out, void
 }
 
 size_t nd_grad_data_workspace(const dk_nd_desc& d) {
+  if (nd_small(d)) return 0;
   size_t n = (size_t)d.channel;
   for (int i = 0; i < d.dims; ++i) n *= (size_t)d.shape[i];
   if (nd_use_channel_last(d)) return round256(n * sizeof(float)) + nd_sort_workspace(d);  // fp32 channel-last accumulation image
@@ -1272,6 +1473,29 @@ void nd_grad_data(const dk_nd_desc& d, const T* gout, const T* coord, T* gdata, 
   const long n_data = (long)g.channel * g.prod_shape;
   const long total = g.batch * g.channel;
   if constexpr (!std::is_same<T, double>::value) {
+    if (nd_small(d)) {
+      const int nt = ((int)g.prod_shape + 15) / 16;
+      // points per chunk: rows of W that fit its LDS, a multiple of 64, at most two points per thread
+      int chunk = kSmallWBytes / (nt * 16 * (int)sizeof(float)) / 64 * 64;
+      if (chunk > 2048) chunk = 2048;
+      const size_t lds = std::max<size_t>((size_t)std::min<long>(chunk, (g.batch + 63) / 64 * 64) * nt * 16 * sizeof(float),
+                                          (size_t)16 * nt * 256 * sizeof(float));
+      const unsigned grid = (unsigned)((g.channel + 15) / 16);
+#define DK_ND_SMALL_GD(ND, NT)                                                                                                    \
+  if (lds <= 64 * 1024 || allow_dynamic_lds(reinterpret_cast<const void*>(&nd_small_grad_data_kernel<T, ND, NT>), kSmallWBytes)) \
+  nd_small_grad_data_kernel<T, ND, NT><<<grid, 1024, lds, stream>>>(g, gout, coord, gdata, chunk)
+#define DK_ND_SMALL_GD_NT(ND)          \
+  if (nt == 1) { DK_ND_SMALL_GD(ND, 1); } \
+  else if (nt == 2) { DK_ND_SMALL_GD(ND, 2); } \
+  else if (nt == 3) { DK_ND_SMALL_GD(ND, 3); } \
+  else { DK_ND_SMALL_GD(ND, 4); }
+      if (g.dims == 1) { DK_ND_SMALL_GD_NT(1) }
+      else if (g.dims == 2) { DK_ND_SMALL_GD_NT(2) }
+      else { DK_ND_SMALL_GD_NT(3) }
+#undef DK_ND_SMALL_GD_NT
+#undef DK_ND_SMALL_GD
+      return;
+    }
     if (nd_use_channel_last(d)) {
       float* acc = static_cast<float*>(ws);
       nd_fill_zero_kernel<float><<<grid_for(n_data), kBlock, 0, stream>>>(acc, n_data);
@@ -1313,6 +1537,13 @@ void nd_grad_coord(const dk_nd_desc& d, const T* gout, const T* data, const T* c
                    void* ws, const int* order, hipStream_t stream) {
   const NdGeo g = make_geo(d);
   if constexpr (!std::is_same<T, double>::value) {
+    if (nd_small(d)) {
+      const unsigned grid = (unsigned)((g.batch + kBlock / 64 - 1) / (kBlock / 64));
+      if (g.dims == 1) nd_small_grad_coord_kernel<T, 1><<<grid, kBlock, 0, stream>>>(g, gout, data, coord, gcoord);
+      else if (g.dims == 2) nd_small_grad_coord_kernel<T, 2><<<grid, kBlock, 0, stream>>>(g, gout, data, coord, gcoord);
+      else nd_small_grad_coord_kernel<T, 3><<<grid, kBlock, 0, stream>>>(g, gout, data, coord, gcoord);
+      return;
+    }
     if (nd_use_channel_last(d)) {
       T* data_cl = static_cast<T*>(ws);
       transpose<T, T>(data, data_cl, g.channel, g.prod_shape, stream);

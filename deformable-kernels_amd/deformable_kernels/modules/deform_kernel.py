@@ -11,7 +11,8 @@ autocast-aware cast.
 import torch
 from torch import nn
 
-from ..ops.deform_kernel.functions import nd_linear_sample, offset_conv, sample_depthwise
+from ..ops.deform_kernel.functions import (
+    image_depthwise_conv, image_depthwise_conv_supported, nd_linear_sample, offset_conv, sample_depthwise)
 from ..ops.deform_kernel.modules import (
     SampleDepthwise,
     DeformableSampleDepthwise,
@@ -71,11 +72,17 @@ class GlobalDeformKernel2d(nn.Module):
         self.fc = nn.Linear(in_planes, kernel_size * kernel_size * len(self.weight_shape))
         self.fc.zero_init = True
         self.fc_bias = _centred_tap_grid(weight_shape, kernel_size, self.weight_dilate)
-        # Depthwise layers with a 2-D scope take one call of the fused sample + depthwise operator
-        # with the image's rotation broadcast over its pixels, instead of sampling N * C kernels and
-        # running a convolution with N * C groups (the reference's route, :92-116, kept for every
-        # other configuration and when this flag is cleared).  Same function, same parameters.
-        self.fused = True
+        # Depthwise layers on the GPU apply the sampled kernels with the library's per-image depthwise
+        # convolution (forward, input gradient, kernel gradient as streaming kernels) instead of the
+        # framework's convolution with N * C groups (:103-111); same values, same gradients.  Every
+        # other configuration, and this one when the flag is cleared, takes the framework's.
+        self.native_conv = True
+        # Alternative for depthwise layers with a 2-D scope: one call of the fused sample + depthwise
+        # operator with the image's rotation broadcast over its pixels, no sampled kernels at all.
+        # Off by default: it is the slower route, and it rounds the coordinates (not the sampled
+        # kernels) to the input's dtype, so in 16-bit types its results differ from the reference's
+        # sequence by more than rounding of the output where a coordinate sits on a cell border.
+        self.fused = False
         self.reset_parameters()
 
     def reset_parameters(self):
@@ -83,13 +90,16 @@ class GlobalDeformKernel2d(nn.Module):
         # initialiser; give it a definite default so a fresh module is usable.
         nn.init.kaiming_normal_(self.weight.view(self.weight.size(0), self.weight.size(1), -1))
 
-    def dynamic_weight(self, x, weight):
+    def dynamic_weight(self, x, weight, per_image=False):
+        """The kernels sampled for every image: ``[N * out_planes, in_planes / groups, k, k]`` as in
+        the reference (:68-101); with ``per_image`` (depthwise layers) the same values as a
+        ``[N, C, k, k]`` view of the sampler's output, without the transposing copy of :97-101."""
         if torch.is_autocast_enabled():
             with torch.autocast(device_type="cuda", enabled=False):
-                return self._dynamic_weight(x.float(), weight.float())
-        return self._dynamic_weight(x, weight)
+                return self._dynamic_weight(x.float(), weight.float(), per_image)
+        return self._dynamic_weight(x, weight, per_image)
 
-    def _dynamic_weight(self, x, weight):
+    def _dynamic_weight(self, x, weight, per_image):
         n, c, h, w = x.shape
         taps = self.kernel_size * self.kernel_size
         kernels = self.out_planes * self.in_planes // self.group
@@ -101,8 +111,10 @@ class GlobalDeformKernel2d(nn.Module):
         sampled = nd_linear_sample(
             weight.reshape(kernels, *self.weight_shape),
             coord.reshape(n * taps, len(self.weight_shape)),
-        ).view(n, taps, kernels)
-        return sampled.transpose(1, 2).reshape(
+        )
+        if per_image:
+            return sampled.view(n, self.kernel_size, self.kernel_size, kernels).permute(0, 3, 1, 2)
+        return sampled.view(n, taps, kernels).transpose(1, 2).reshape(
             n * self.out_planes, self.in_planes // self.group, self.kernel_size, self.kernel_size)
 
     def _fusable(self, x):
@@ -132,7 +144,13 @@ class GlobalDeformKernel2d(nn.Module):
         if self._fusable(x):
             return self._forward_fused(x)
         n, c, h, w = x.shape
-        weight = self.dynamic_weight(x, self.weight).to(x.dtype)
+        if self.native_conv and x.is_cuda and self.group == self.in_planes == self.out_planes:
+            kernels = self.dynamic_weight(x, self.weight, per_image=True).to(x.dtype)
+            if image_depthwise_conv_supported(x, kernels, self.stride, self.padding, self.dilation):
+                return image_depthwise_conv(x, kernels, self.stride, self.padding, self.dilation)
+            weight = kernels.reshape(n * c, 1, self.kernel_size, self.kernel_size)
+        else:
+            weight = self.dynamic_weight(x, self.weight).to(x.dtype)
         out = nn.functional.conv2d(
             x.reshape(1, n * c, h, w), weight, stride=self.stride, padding=self.padding,
             dilation=self.dilation, groups=n * self.group)

@@ -42,6 +42,7 @@ class DkError(RuntimeError):
 
 
 _P, _SZ = ctypes.c_void_p, ctypes.c_size_t
+_I64P = ctypes.POINTER(ctypes.c_int64)
 _CD, _ND, _OC = ctypes.POINTER(ConvDesc), ctypes.POINTER(NdDesc), ctypes.POINTER(OffsetConvDesc)
 
 # name -> (restype, argtypes); must list every symbol include/dk_hip.h declares
@@ -77,6 +78,10 @@ SIGNATURES = {
     "dk_nd_linear_sample_backward_data": (ctypes.c_int, [_ND, _P, _P, _P, _P, _P, _SZ, _P]),
     "dk_nd_linear_sample_backward_coord_workspace": (_SZ, [_ND]),
     "dk_nd_linear_sample_backward_coord": (ctypes.c_int, [_ND, _P, _P, _P, _P, _P, _P, _SZ, _P]),
+    "dk_image_depthwise_supported": (ctypes.c_int, [_CD]),
+    "dk_image_depthwise_forward": (ctypes.c_int, [_CD, _P, _P, _I64P, _P, _P]),
+    "dk_image_depthwise_backward_data": (ctypes.c_int, [_CD, _P, _P, _I64P, _P, _P]),
+    "dk_image_depthwise_backward_weight": (ctypes.c_int, [_CD, _P, _P, _P, _I64P, _P]),
     "dk_offset_conv_supported": (ctypes.c_int, [_OC]),
     "dk_offset_conv_worthwhile": (ctypes.c_int, [_OC]),
     "dk_offset_conv_forward_workspace": (_SZ, [_OC]),
@@ -149,7 +154,7 @@ def workspace(nbytes, device):
 
 TEST_SWITCHES = ("DK_NO_ROWS", "DK_NO_MFMA", "DK_NO_MFMA_S2", "DK_NO_S2_QUADS", "DK_NO_DEFORM_FAST",
                  "DK_NO_DEFORM_CH", "DK_NO_DEFORM_CH_BIG", "DK_NO_DEFORM_MFMA", "DK_NO_ND_BINS", "DK_NO_ND_MFMA",
-                 "DK_NO_GATHER_MFMA", "DK_NO_FILTER_SPLIT")
+                 "DK_NO_GATHER_MFMA", "DK_NO_FILTER_SPLIT", "DK_NO_IMAGE_FLAT", "DK_NO_ND_SMALL")
 
 
 class test_switches:

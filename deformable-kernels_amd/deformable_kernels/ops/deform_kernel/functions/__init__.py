@@ -4,6 +4,7 @@ from .filter_sample_depthwise import (
 )
 from .nd_linear_sample import nd_linear_sample
 from .offset_conv import offset_conv, offset_conv_supported
+from .image_depthwise_conv import image_depthwise_conv, image_depthwise_conv_supported
 
 __all__ = [
     'sample_depthwise',
@@ -11,4 +12,6 @@ __all__ = [
     'nd_linear_sample',
     'offset_conv',
     'offset_conv_supported',
+    'image_depthwise_conv',
+    'image_depthwise_conv_supported',
 ]

@@ -282,6 +282,33 @@ size_t dk_offset_conv_backward_bias_workspace(const dk_offset_conv_desc *desc);
 int dk_offset_conv_backward_bias(const dk_offset_conv_desc *desc, const void *out_grad, void *bias_grad,
                                  void *workspace, size_t workspace_bytes, void *stream);
 
+/* ---- depthwise convolution with one kernel per image and channel ------------- */
+
+/* The convolution GlobalDeformKernel2d applies with the kernels it has sampled for every image:
+ * nn.functional.conv2d(x.view(1, n * c, h, w), weight, stride, padding, dilation, groups = n * c)
+ * for a depthwise layer (modules/deform_kernel.py:103-111, weight [n * c, 1, k, k] from
+ * dynamic_weight, :68-101), and the two gradients the framework derives for that call.  The
+ * reference uses the framework's grouped convolution there; a convolution with n * c groups of
+ * one channel each is a streaming operation, and these entry points run it as one.
+ *   input [batch, channel, in_h, in_w], weight [batch, channel, k_h, k_w] (= [n * c, 1, k_h, k_w]),
+ *   output [batch, channel, out_h, out_w]; weight_strides: NULL for a contiguous weight (and
+ *   weight_grad), or the four non-negative element strides of its (batch, channel, k_h, k_w) axes --
+ *   the sampler leaves the kernels as [n * k_h * k_w, c] (nd_linear_sample's output, :92-96), which is
+ *   strides {k_h * k_w * c, 1, k_w * c, c}, and the module's transpose + reshape (:97-101) is then
+ *   not needed; desc: scope_h, scope_w, groups, rotation_clip are not
+ *   used (scope >= 1 and groups = 1 keep the descriptor valid); any dk_dtype.
+ * dk_image_depthwise_supported() tells whether the geometry is covered (a band of one output
+ * row's taps must fit a wave's share of LDS, at most 128 taps); the calls return
+ * DK_ERR_UNSUPPORTED otherwise and the caller keeps its library convolution.  No workspace;
+ * every result is fully written; each kernel gradient is one wave's sum in a fixed order. */
+int dk_image_depthwise_supported(const dk_conv_desc *desc);
+int dk_image_depthwise_forward(const dk_conv_desc *desc, const void *input, const void *weight,
+                               const int64_t *weight_strides, void *output, void *stream);
+int dk_image_depthwise_backward_data(const dk_conv_desc *desc, const void *out_grad, const void *weight,
+                                     const int64_t *weight_strides, void *in_grad, void *stream);
+int dk_image_depthwise_backward_weight(const dk_conv_desc *desc, const void *out_grad, const void *input,
+                                       void *weight_grad, const int64_t *weight_strides, void *stream);
+
 /* ---- misc ------------------------------------------------------------------- */
 
 const char *dk_status_string(int status);
@@ -290,7 +317,7 @@ const char *dk_status_string(int status);
  * family and run the next more general one for the same shape, so that tests can reach every
  * kernel.  Bit i belongs to the i-th of DK_NO_ROWS, DK_NO_MFMA, DK_NO_MFMA_S2, DK_NO_S2_QUADS,
  * DK_NO_DEFORM_FAST, DK_NO_DEFORM_CH, DK_NO_DEFORM_CH_BIG, DK_NO_DEFORM_MFMA, DK_NO_ND_BINS,
- * DK_NO_ND_MFMA, DK_NO_GATHER_MFMA, DK_NO_FILTER_SPLIT.  The mask starts from the environment variables of those names, read once
+ * DK_NO_ND_MFMA, DK_NO_GATHER_MFMA, DK_NO_FILTER_SPLIT, DK_NO_IMAGE_FLAT, DK_NO_ND_SMALL.  The mask starts from the environment variables of those names, read once
  * (at the first call that consults it); this call replaces it and returns the previous mask.
  * Workspace queries consult it too: query and call must see the same mask.  The one piece of
  * process-wide state in the library. */

@@ -202,3 +202,53 @@ def nd_linear_sample_backward(gout, data, coord):
     getattr(L, "dko_nd_linear_sample_backward_coord" + _suffix(dt))(
         B, C, n, ctypes.c_long(P), _p(gout), _p(data), _p(shape), _p(coord), _p(gcoord_c))
     return gdata, gcoord_c.sum(2)
+
+
+# ---- the convolution GlobalDeformKernel2d applies with its sampled kernels ------------------
+#
+# Reference: modules/deform_kernel.py:103-111, F.conv2d(x.view(1, n * c, h, w), weight, stride,
+# padding, dilation, groups = n * c) with weight [n * c, 1, k, k] for a depthwise layer -- the
+# framework's grouped cross-correlation; its gradients are the framework's.  Restated in numpy as
+# the textbook sums (one shifted, strided slice of the zero-padded plane per tap), in the dtype of
+# the arrays handed in.  Pinned in tests/test_oracle_image_conv.py against torch's conv2d and its autograd
+# gradients on the CPU in float64 (a library routine), over strides, paddings and dilations.
+
+def _padded(x, k, stride, pad, dil, out):
+    """x zero-padded so that every tap of every output position is inside the array."""
+    need = [(out[d] - 1) * stride[d] + (k[d] - 1) * dil[d] + 1 for d in (0, 1)]
+    hi = [max(need[d] - pad[d] - x.shape[2 + d], 0) for d in (0, 1)]
+    return np.pad(x, ((0, 0), (0, 0), (pad[0], hi[0]), (pad[1], hi[1])))
+
+
+def image_depthwise_forward(x, w, stride=(1, 1), padding=(0, 0), dilation=(1, 1)):
+    """x [N, C, H, W], w [N, C, k_h, k_w] (one kernel per image and channel) -> [N, C, Ho, Wo]."""
+    stride, padding, dilation = _pair(stride), _pair(padding), _pair(dilation)
+    k = w.shape[2:]
+    out = [output_size(x.shape[2 + d], k[d], stride[d], padding[d], dilation[d]) for d in (0, 1)]
+    xp = _padded(x, k, stride, padding, dilation, out)
+    y = np.zeros(x.shape[:2] + tuple(out), dtype=x.dtype)
+    for i in range(k[0]):
+        for j in range(k[1]):
+            r0, c0 = i * dilation[0], j * dilation[1]
+            y += w[:, :, i, j, None, None] * xp[:, :, r0:r0 + (out[0] - 1) * stride[0] + 1:stride[0],
+                                                c0:c0 + (out[1] - 1) * stride[1] + 1:stride[1]]
+    return y
+
+
+def image_depthwise_backward(gout, x, w, stride=(1, 1), padding=(0, 0), dilation=(1, 1)):
+    """Gradients of image_depthwise_forward w.r.t. x and w for the output gradient gout."""
+    stride, padding, dilation = _pair(stride), _pair(padding), _pair(dilation)
+    k = w.shape[2:]
+    out = gout.shape[2:]
+    xp = _padded(x, k, stride, padding, dilation, out)
+    gxp = np.zeros_like(xp)
+    gw = np.zeros_like(w)
+    for i in range(k[0]):
+        for j in range(k[1]):
+            r0, c0 = i * dilation[0], j * dilation[1]
+            rows = slice(r0, r0 + (out[0] - 1) * stride[0] + 1, stride[0])
+            cols = slice(c0, c0 + (out[1] - 1) * stride[1] + 1, stride[1])
+            gw[:, :, i, j] = (gout * xp[:, :, rows, cols]).sum((2, 3))
+            gxp[:, :, rows, cols] += w[:, :, i, j, None, None] * gout
+    gx = gxp[:, :, padding[0]:padding[0] + x.shape[2], padding[1]:padding[1] + x.shape[3]]
+    return np.ascontiguousarray(gx), gw

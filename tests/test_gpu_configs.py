@@ -70,6 +70,7 @@ def test_config3_global_deform_kernel_float16_at_full_size():
     x = torch.randn(N, C, H, H, generator=g).half()
     gout = torch.randn(N, C, H, H, generator=g).half()
     m = _global_module(torch.float16, seed=30)
+    m.fused = True  # first the route that hands each image's offsets to the local operator
     xg = x.to(DEV).requires_grad_()
     out = m(xg)
     out.backward(gout.to(DEV))
@@ -120,6 +121,21 @@ def test_config3_global_deform_kernel_float16_at_full_size():
     _within(rel_err(centred(x2.grad), centred(xg.grad)), 1e-2, "unfused grad input")
     _within(rel_err(m.weight.grad.float().cpu(), gw), 2e-2, "unfused grad scope weight")
 
+    # That run applied the sampled kernels with the library's per-image depthwise convolution (the
+    # default); the framework's convolution with N * C groups on the same sampled kernels must agree
+    # with it in every result, the gradients that pass through the coordinates included.
+    native = [out2.detach().float().cpu(), x2.grad.float().cpu()] + [p.grad.float().cpu() for p in m.parameters()]
+    m.native_conv = False
+    for p in m.parameters():
+        p.grad = None
+    x3 = x.to(DEV).requires_grad_()
+    out3 = m(x3)
+    out3.backward(gout.to(DEV))
+    torch.cuda.synchronize()
+    library = [out3.detach().float().cpu(), x3.grad.float().cpu()] + [p.grad.float().cpu() for p in m.parameters()]
+    for name, a, b in zip(("forward", "grad input", "grad scope weight", "grad fc weight", "grad fc bias"), native, library):
+        _within(rel_err(a, b), 1e-2, "per-image convolution against the framework's: " + name)
+
 
 def test_config3_kernel_synthesis_float16():
     """The sampler call of configuration 3: 1152 = 128 x 9 points on 256 kernels of 5 x 5, float16."""
@@ -164,10 +180,12 @@ def test_config5_trilinear_sampler_at_2_to_the_20_points(lo, hi):
     _within(mixed_err(out.detach().cpu()[pick], want), 1e-5, "forward")
     _, gc = orc.nd_linear_sample_backward(gout[pick].double().numpy(), data.double().numpy(), sub.double().numpy())
     _within(rel_err(cg.grad.cpu()[pick], gc), 1e-4, "grad coord")
-    # adjoint identity, sums in float64
+    # adjoint identity, sums in float64.  Both sides are sums of 2^26 signed terms of order 1 built from
+    # float32 results (a spread of about 2^13 with a rounding error of about 2^13 * 2^-24 of it), and the
+    # data gradient's float32 atomics add in an order that changes from run to run: 1e-5 of the larger side.
     a = (gout.to(DEV).double() * out.detach().double()).sum().item()
     b = (dg.grad.double() * dg.detach().double()).sum().item()
-    assert abs(a - b) < 1e-6 * max(abs(a), abs(b), 1.0), (a, b)
+    assert abs(a - b) < 1e-5 * max(abs(a), abs(b), 1.0), (a, b)
     # one channel of the data gradient against the float64 oracle over all 2^20 points
     gd, _ = orc.nd_linear_sample_backward(gout[:, 5:6].double().numpy(), data[5:6].double().numpy(),
                                           coord.double().numpy())

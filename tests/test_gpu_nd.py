@@ -115,6 +115,21 @@ def test_sorted_kernels_with_and_without_the_matrix_cores_agree(switch_off):
         assert rel_err(y, w) < 1e-4
 
 
+@pytest.mark.parametrize("dtype,C,B", [(torch.float32, 256, 1152), (torch.float16, 64, 4096), (torch.bfloat16, 100, 700)])
+def test_channel_last_kernels_on_few_points_over_a_tiny_volume(dtype, C, B, switch_off):
+    """Few points on a volume of at most 64 cells take the direct kernels and the one-launch grad
+    data; with that path switched off the channel-last kernels serve the same call."""
+    data, coord, gout = _inputs((5, 5), C, B, seed=44, dtype=dtype)
+    small = _run(data, coord, gout)
+    switch_off("DK_NO_ND_SMALL")
+    general = _run(data, coord, gout)
+    want = _oracle(data, coord, gout, np.float64)
+    tol = (1e-5, 1e-4, 1e-4) if dtype == torch.float32 else (1e-2, 1e-2, 1e-2)
+    for a, b, w, t in zip(small, general, want, tol):
+        assert rel_err(a.float(), w) < t
+        assert rel_err(b.float(), w) < t
+
+
 def test_fp64_matches_oracle():
     data, coord, gout = _inputs((4, 5, 6), 9, 257, seed=42, dtype=torch.float64)
     got = _run(data, coord, gout)
