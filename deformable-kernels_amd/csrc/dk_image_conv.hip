@@ -453,14 +453,14 @@ struct FlatLoads {
   __device__ __forceinline__ void issue(const T* __restrict__ src, long total, const FlatUnit& u, int lane) {
 #pragma unroll
     for (int j = 0; j < NCH; ++j) {
-      const int chunk = lane + kWave * j;
-      // (a chunk outside the range is not loaded; its slot in LDS is not read either)
-      if (chunk < u.chunks) {
-        long e = (long)u.first + chunk * kPer<T>;
-        e = e < 0 ? 0 : e;
-        e = e > total - kPer<T> ? total - kPer<T> : e;
-        v[j] = *reinterpret_cast<const u4*>(src + e);
-      }
+      // Every lane loads every time (a lane past the range repeats the range's last chunk, which
+      // commit() then leaves out): with a fixed number of loads per unit the waits on them can be
+      // counted, and the next unit's loads stay in flight behind this unit's arithmetic.
+      const int chunk = min(lane + kWave * j, u.chunks - 1);
+      long e = (long)u.first + chunk * kPer<T>;
+      e = e < 0 ? 0 : e;
+      e = e > total - kPer<T> ? total - kPer<T> : e;
+      v[j] = *reinterpret_cast<const u4*>(src + e);
     }
   }
   __device__ __forceinline__ void commit(float* tile, const FlatUnit& u, int lane) const {
@@ -492,16 +492,17 @@ __device__ __forceinline__ void zero_row(float* row, int w, int lane) {
 }
 
 // Columns oc - 1 .. oc + 4 of three consecutive staged rows, zero where the column is outside the plane.
-template <bool W4>
-__device__ __forceinline__ void load_rows(const float* top, int w, int oc, float (&x)[3][kStrip + 2]) {
+// (PR + 2 rows for a patch of PR output rows)
+template <bool W4, int PR>
+__device__ __forceinline__ void load_rows(const float* top, int w, int oc, float (&x)[PR + 2][kStrip + 2]) {
 #pragma unroll
-  for (int i = 0; i < 3; ++i)
+  for (int i = 0; i < PR + 2; ++i)
 #pragma unroll
     for (int c = 0; c < kStrip + 2; ++c) x[i][c] = top[i * w + c];
   if constexpr (W4) {  // only the strip's outer columns can be outside
     const bool left = oc == 0, right = oc + kStrip == w;
 #pragma unroll
-    for (int i = 0; i < 3; ++i) {
+    for (int i = 0; i < PR + 2; ++i) {
       x[i][0] = left ? 0.f : x[i][0];
       x[i][kStrip + 1] = right ? 0.f : x[i][kStrip + 1];
     }
@@ -510,14 +511,16 @@ __device__ __forceinline__ void load_rows(const float* top, int w, int oc, float
     for (int c = 0; c < kStrip + 2; ++c) {
       const bool outside = (unsigned)(oc - 1 + c) >= (unsigned)w;
 #pragma unroll
-      for (int i = 0; i < 3; ++i) x[i][c] = outside ? 0.f : x[i][c];
+      for (int i = 0; i < PR + 2; ++i) x[i][c] = outside ? 0.f : x[i][c];
     }
   }
 }
 
 __device__ __forceinline__ long tap_offset(const WLayout& wl, int t) { return (t / 3) * wl.i + (t % 3) * wl.j; }
 
-template <typename T, int NCH, bool W4>
+// PR: output rows of a lane's patch (1, or 4 when the band's rows are a multiple of 4: the six staged
+// rows a patch reads serve four output rows instead of three rows serving one)
+template <typename T, int NCH, bool W4, int PR>
 __global__ __launch_bounds__(kWave* kWaves) void image_conv3_flat_kernel(FlatConv a, const T* __restrict__ src,
                                                                          const T* __restrict__ weight,
                                                                          T* __restrict__ dst) {
@@ -543,7 +546,8 @@ __global__ __launch_bounds__(kWave* kWaves) void image_conv3_flat_kernel(FlatCon
   T taps_next = taps_of(first_plane);
   for (;;) {
     loads.commit(tile, cur, lane);
-    const float taps_cur = ld(&taps_next);
+    float taps_cur = ld(&taps_next);
+    asm volatile("" : "+v"(taps_cur));  // converted here, before the next loads are issued, not next to its use
     if (cur.r0 == 0) zero_row(tile + kFront + cur.shift, a.w, lane);
     if (cur.r1 == a.h) zero_row(tile + kFront + cur.shift + (cur.r1 - cur.r0 + 1) * a.w, a.w, lane);
     // the next band's loads fly while this one is computed
@@ -561,20 +565,23 @@ __global__ __launch_bounds__(kWave* kWaves) void image_conv3_flat_kernel(FlatCon
     for (int t = 0; t < 9; ++t) w9[t] = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, taps_cur), t));
     T* dp = dst + (size_t)cur.plane * a.hw;
     const float* band = tile + kFront + cur.shift - 1;  // column -1 of the halo row above the band's first row
-    const int items = (cur.r1 - cur.r0) * strips;
-    int orow = lane / strips, os = lane - orow * strips;
+    const int items = (cur.r1 - cur.r0) / PR * strips;
+    int orow = lane / strips, os = lane - orow * strips;  // orow counts patches
     for (int item = lane; item < items; item += kWave) {
       const int oc = os * kStrip;
-      float x[3][kStrip + 2];
-      load_rows<W4>(band + orow * a.w + oc, a.w, oc, x);
-      float acc[kStrip] = {0.f, 0.f, 0.f, 0.f};
+      float x[PR + 2][kStrip + 2];
+      load_rows<W4, PR>(band + orow * PR * a.w + oc, a.w, oc, x);
 #pragma unroll
-      for (int i = 0; i < 3; ++i)
+      for (int pr = 0; pr < PR; ++pr) {
+        float acc[kStrip] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-        for (int j = 0; j < 3; ++j)
+        for (int i = 0; i < 3; ++i)
 #pragma unroll
-          for (int p = 0; p < kStrip; ++p) acc[p] = fmaf(w9[i * 3 + j], x[i][p + j], acc[p]);
-      store_strip<T, float>(dp + (size_t)(cur.r0 + orow) * a.w, oc, a.w, acc, W4);
+          for (int j = 0; j < 3; ++j)
+#pragma unroll
+            for (int p = 0; p < kStrip; ++p) acc[p] = fmaf(w9[i * 3 + j], x[pr + i][p + j], acc[p]);
+        store_strip<T, float>(dp + (size_t)(cur.r0 + orow * PR + pr) * a.w, oc, a.w, acc, W4);
+      }
       orow += dro;
       os += dso;
       if (os >= strips) {
@@ -590,7 +597,7 @@ __global__ __launch_bounds__(kWave* kWaves) void image_conv3_flat_kernel(FlatCon
 
 // Kernel gradient of that shape: input band (with halo) and out_grad band staged the same way, nine
 // running sums per lane over the plane's bands, added up over the wave when the plane is done.
-template <typename T, int NCH, bool W4>
+template <typename T, int NCH, bool W4, int PR>
 __global__ __launch_bounds__(kWave* kWaves) void image_conv3_flat_grad_weight_kernel(FlatConv a,
                                                                                      const T* __restrict__ gout,
                                                                                      const T* __restrict__ x,
@@ -630,24 +637,28 @@ __global__ __launch_bounds__(kWave* kWaves) void image_conv3_flat_grad_weight_ke
     lds_sync();
     const float* band = xtile + kFront + cur.shift - 1;
     const float* gband = gtile + kFront + gcur.shift;
-    const int items = (cur.r1 - cur.r0) * strips;
-    int orow = lane / strips, os = lane - orow * strips;
+    const int items = (cur.r1 - cur.r0) / PR * strips;
+    int orow = lane / strips, os = lane - orow * strips;  // orow counts patches
     for (int item = lane; item < items; item += kWave) {
       const int oc = os * kStrip;
-      float xv[3][kStrip + 2];
-      load_rows<W4>(band + orow * a.w + oc, a.w, oc, xv);
-      float gv[kStrip];
+      float xv[PR + 2][kStrip + 2];
+      load_rows<W4, PR>(band + orow * PR * a.w + oc, a.w, oc, xv);
+      float gv[PR][kStrip];
 #pragma unroll
-      for (int p = 0; p < kStrip; ++p) {
-        gv[p] = gband[orow * a.w + oc + p];
-        if constexpr (!W4) gv[p] = oc + p < a.w ? gv[p] : 0.f;
-      }
+      for (int pr = 0; pr < PR; ++pr)
 #pragma unroll
-      for (int i = 0; i < 3; ++i)
+        for (int p = 0; p < kStrip; ++p) {
+          gv[pr][p] = gband[(orow * PR + pr) * a.w + oc + p];
+          if constexpr (!W4) gv[pr][p] = oc + p < a.w ? gv[pr][p] : 0.f;
+        }
 #pragma unroll
-        for (int j = 0; j < 3; ++j)
+      for (int pr = 0; pr < PR; ++pr)
 #pragma unroll
-          for (int p = 0; p < kStrip; ++p) sum[i * 3 + j] = fmaf(gv[p], xv[i][p + j], sum[i * 3 + j]);
+        for (int i = 0; i < 3; ++i)
+#pragma unroll
+          for (int j = 0; j < 3; ++j)
+#pragma unroll
+            for (int p = 0; p < kStrip; ++p) sum[i * 3 + j] = fmaf(gv[pr][p], xv[pr + i][p + j], sum[i * 3 + j]);
       orow += dro;
       os += dso;
       if (os >= strips) {
@@ -695,6 +706,8 @@ bool flat_plan(FlatConv& a, const Geo& g, const long* ws, int budget, const void
   a.h = g.in_h, a.w = g.in_w, a.hw = g.in_h * g.in_w;
   a.bands = (g.in_h + max_rows - 1) / max_rows;
   a.band_rows = (g.in_h + a.bands - 1) / a.bands;
+  // bands of a multiple of four rows where the plane allows it: the kernels then work on 4 x 4 patches
+  if (g.in_h % 4 == 0 && (a.band_rows + 3) / 4 * 4 <= max_rows) a.band_rows = (a.band_rows + 3) / 4 * 4;
   a.bands = (g.in_h + a.band_rows - 1) / a.band_rows;
   a.flip = 0;
   return true;
@@ -731,9 +744,11 @@ bool launch_flat_conv(const Geo& g, const long* ws, bool flip, const T* src, con
     const size_t lds = (size_t)kWaves * a.tile_elems * sizeof(float);
     const dim3 grid(flat_grid(a)), block(kWave * kWaves);
     const bool w4 = a.vec_ok != 0;  // whole, aligned strips: one vector store each
-#define DK_FLAT(NN)                                                                                           \
-  if (w4) hipLaunchKernelGGL((image_conv3_flat_kernel<T, NN, true>), grid, block, lds, stream, a, src, weight, dst); \
-  else hipLaunchKernelGGL((image_conv3_flat_kernel<T, NN, false>), grid, block, lds, stream, a, src, weight, dst)
+    const bool patches = w4 && a.h % 4 == 0 && a.band_rows % 4 == 0;
+#define DK_FLAT(NN)                                                                                                        \
+  if (patches) hipLaunchKernelGGL((image_conv3_flat_kernel<T, NN, true, 4>), grid, block, lds, stream, a, src, weight, dst);  \
+  else if (w4) hipLaunchKernelGGL((image_conv3_flat_kernel<T, NN, true, 1>), grid, block, lds, stream, a, src, weight, dst);  \
+  else hipLaunchKernelGGL((image_conv3_flat_kernel<T, NN, false, 1>), grid, block, lds, stream, a, src, weight, dst)
     if (nch == 1) { DK_FLAT(1); }
     else if (nch == 2) { DK_FLAT(2); }
     else if (nch == 4) { DK_FLAT(4); }
@@ -756,9 +771,11 @@ bool launch_flat_grad_weight(const Geo& g, const long* ws, const T* gout, const 
     const size_t lds = (size_t)kWaves * 2 * a.tile_elems * sizeof(float);
     const dim3 grid(flat_grid(a)), block(kWave * kWaves);
     const bool w4 = a.w % kStrip == 0;
-#define DK_FLAT(NN)                                                                                                  \
-  if (w4) hipLaunchKernelGGL((image_conv3_flat_grad_weight_kernel<T, NN, true>), grid, block, lds, stream, a, gout, x, gweight); \
-  else hipLaunchKernelGGL((image_conv3_flat_grad_weight_kernel<T, NN, false>), grid, block, lds, stream, a, gout, x, gweight)
+    const bool patches = w4 && a.h % 4 == 0 && a.band_rows % 4 == 0;
+#define DK_FLAT(NN)                                                                                                                    \
+  if (patches) hipLaunchKernelGGL((image_conv3_flat_grad_weight_kernel<T, NN, true, 4>), grid, block, lds, stream, a, gout, x, gweight); \
+  else if (w4) hipLaunchKernelGGL((image_conv3_flat_grad_weight_kernel<T, NN, true, 1>), grid, block, lds, stream, a, gout, x, gweight); \
+  else hipLaunchKernelGGL((image_conv3_flat_grad_weight_kernel<T, NN, false, 1>), grid, block, lds, stream, a, gout, x, gweight)
     if (nch == 1) { DK_FLAT(1); }
     else if (nch == 2) { DK_FLAT(2); }
     else { DK_FLAT(4); }
