@@ -47,6 +47,8 @@ OTHER_WORKLOADS = {
     "cfg4": ("deform", (64, 512, 28, 28, 3, (4, 4), 2, 1, 1, 1, 0.5, 2.0)),
     # the deformable variant on the headline layer's shape (3136 output pixels per plane)
     "deform_56": ("deform", (64, 144, 56, 56, 3, (4, 4), 1, 1, 1, 1, 0.5, 2.0)),
+    # DeformConv2d (scope = kernel, no rotation tensor: rot_std None) on configuration 4's geometry
+    "deform_conv_28": ("deform", (64, 512, 28, 28, 3, (3, 3), 2, 1, 1, 1, None, 2.0)),
     # N-d sampler: data shape [C, s...], points, coordinate range
     "nd_cfg3": ("nd", ((256, 5, 5), 1152, (0.0, 4.0))),             # GlobalDeformKernel2d, config 3
     "nd_cfg5": ("nd", ((64, 32, 32, 32), 1 << 20, (-1.0, 32.0))),   # trilinear volume, config 5, full-volume coords
@@ -512,10 +514,12 @@ def other_workload(a):
     us, nbytes = {}, {}
     if kind == "deform":
         N, C, H, W, k, S, stride, pad, dil, groups, rot_std, off_std = spec
-        x, wt, rot, off, gout, cfg = make_deform(N, C, H, W, k, S, stride, pad, dil, groups, rot_std, off_std,
+        x, wt, rot, off, gout, cfg = make_deform(N, C, H, W, k, S, stride, pad, dil, groups, rot_std or 0.0, off_std,
                                                  seed=0, dtype=tdtype)
         xg, wg, rg, og, gg = [t.to(dev) for t in (x, wt, rot, off, gout)]
         out, gin, grot, goff, gw = [torch.empty_like(t) for t in (gg, xg, rg, og, wg)]
+        if rot_std is None:
+            rg = None  # NULL at the C ABI: no kernel-space offsets, no rotation tensor read
         desc = _lib.conv_desc(xg, wg, cfg["kernel_size"], cfg["stride"], cfg["padding"], cfg["dilation"], groups)
         ws1, n1 = _lib.workspace(L.dk_deformable_sample_depthwise_backward_data_workspace(desc), dev)
         ws2, n2 = _lib.workspace(L.dk_deformable_sample_depthwise_backward_filter_workspace(desc), dev)
@@ -523,7 +527,7 @@ def other_workload(a):
         ws4, n4 = _lib.workspace(L.dk_deformable_sample_depthwise_backward_rotation_workspace(desc), dev)
         st = _lib.stream_ptr(xg)
         e = xg.element_size()
-        bx, by, br, bo, bw = [t.numel() * e for t in (xg, gg, rg, og, wg)]
+        bx, by, br, bo, bw = [(t.numel() * e if t is not None else 0) for t in (xg, gg, rg, og, wg)]
         calls = {
             "forward": (lambda: _lib.check(L.dk_deformable_sample_depthwise_forward(
                 desc, P(xg), P(og), P(rg), P(wg), P(out), st), "fwd"), bx + bo + br + bw + by),
@@ -536,8 +540,11 @@ def other_workload(a):
             "grad_filter": (lambda: _lib.check(L.dk_deformable_sample_depthwise_backward_filter(
                 desc, P(gg), P(xg), P(og), P(rg), P(gw), P(ws2), n2, st), "gw"), by + bx + bo + br + bw),
         }
-        label = "%s: deform_sample_depthwise N=%d C=%d %dx%d->%dx%d k=%d scope=%dx%d stride=%d %s" % (
-            a.workload, N, C, H, W, gg.shape[2], gg.shape[3], k, S[0], S[1], stride, a.dtype)
+        if rg is None:
+            del calls["grad_rotation"]
+        label = "%s: deform_sample_depthwise N=%d C=%d %dx%d->%dx%d k=%d scope=%dx%d stride=%d %s%s" % (
+            a.workload, N, C, H, W, gg.shape[2], gg.shape[3], k, S[0], S[1], stride, a.dtype,
+            "" if rg is not None else ", no rotation tensor")
     else:
         shape, B, (lo, hi) = spec
         g = torch.Generator().manual_seed(0)

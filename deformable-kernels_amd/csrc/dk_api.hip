@@ -375,7 +375,7 @@ int dk_deformable_sample_depthwise_forward(const dk_conv_desc* desc, const void*
   Geo g;
   const int rc = make_geo(desc, g);
   if (rc != DK_OK) return rc;
-  if (!input || !offset || !rotation || !filter || !output) return DK_ERR_NULL_POINTER;
+  if (!input || !offset || !filter || !output) return DK_ERR_NULL_POINTER;  // rotation may be NULL: all zeros
   if (g.batch == 0) return DK_OK;
   hipStream_t s = static_cast<hipStream_t>(stream);
   return by_dtype(desc->dtype, [&]<typename T>() {
@@ -398,7 +398,7 @@ int dk_deformable_sample_depthwise_backward_data(const dk_conv_desc* desc, const
   Geo g;
   const int rc = make_geo(desc, g);
   if (rc != DK_OK) return rc;
-  if (!out_grad || !offset || !rotation || !filter || !in_grad) return DK_ERR_NULL_POINTER;
+  if (!out_grad || !offset || !filter || !in_grad) return DK_ERR_NULL_POINTER;  // rotation may be NULL: all zeros
   const size_t need = dk_deformable_sample_depthwise_backward_data_workspace(desc);
   if (need && (!workspace || workspace_bytes < need)) return DK_ERR_WORKSPACE;
   if (g.batch == 0) return DK_OK;
@@ -426,7 +426,7 @@ int dk_deformable_sample_depthwise_backward_filter(const dk_conv_desc* desc, con
   Geo g;
   const int rc = make_geo(desc, g);
   if (rc != DK_OK) return rc;
-  if (!out_grad || !input || !offset || !rotation || !filter_grad) return DK_ERR_NULL_POINTER;
+  if (!out_grad || !input || !offset || !filter_grad) return DK_ERR_NULL_POINTER;  // rotation may be NULL: all zeros
   const size_t need = dk_deformable_sample_depthwise_backward_filter_workspace(desc);
   if (need && (!workspace || workspace_bytes < need)) return DK_ERR_WORKSPACE;
   hipStream_t s = static_cast<hipStream_t>(stream);
@@ -454,7 +454,7 @@ int dk_deformable_sample_depthwise_backward_offset(const dk_conv_desc* desc, con
   Geo g;
   const int rc = make_geo(desc, g);
   if (rc != DK_OK) return rc;
-  if (!out_grad || !input || !offset || !rotation || !filter || !offset_grad) return DK_ERR_NULL_POINTER;
+  if (!out_grad || !input || !offset || !filter || !offset_grad) return DK_ERR_NULL_POINTER;  // rotation may be NULL: all zeros
   const size_t need = fast_deform_grad_coord_workspace(g, false);
   if (need && (!workspace || workspace_bytes < need)) return DK_ERR_WORKSPACE;
   if (g.batch == 0) return DK_OK;

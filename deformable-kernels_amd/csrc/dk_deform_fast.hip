@@ -57,7 +57,9 @@ __device__ __forceinline__ void deform_taps(const Geo& g, const T* off, const T*
   const int pc = live ? p : 0;
   const int oh = pc / g.out_w, ow = pc % g.out_w;
   const rsrc_t ro = plane_rsrc(off + (size_t)n * (K9 * 2) * out_plane, K9 * 2 * out_plane);
-  const rsrc_t rr = plane_rsrc(rot + (size_t)(n * g.groups + grp) * (K9 * 2) * out_plane, K9 * 2 * out_plane);
+  // no rotation tensor (the caller's offsets in kernel space are all zero): a resource of no bytes reads as zeros
+  const rsrc_t rr = rot ? plane_rsrc(rot + (size_t)(n * g.groups + grp) * (K9 * 2) * out_plane, K9 * 2 * out_plane)
+                        : plane_rsrc(rot, 0);
   const unsigned step = (unsigned)out_plane * (unsigned)sizeof(T);
 #pragma unroll
   for (int t = 0; t < K9; ++t) {
@@ -1183,7 +1185,8 @@ __global__ __launch_bounds__(kGfBlock, 1) void deform_grad_filter_mfma_kernel(
     const int pc = live ? p : 0;
     const int oh = pc / g.out_w, ow = pc % g.out_w;
     const rsrc_t ro = plane_rsrc(off + (size_t)n * (K9 * 2) * out_plane, K9 * 2 * out_plane);
-    const rsrc_t rr = plane_rsrc(rot + (size_t)(n * g.groups + grp) * (K9 * 2) * out_plane, K9 * 2 * out_plane);
+    const rsrc_t rr = rot ? plane_rsrc(rot + (size_t)(n * g.groups + grp) * (K9 * 2) * out_plane, K9 * 2 * out_plane)
+                          : plane_rsrc(rot, 0);  // no rotation tensor: reads as zeros
     const unsigned step = (unsigned)out_plane * (unsigned)sizeof(T);
 #pragma unroll
     for (int k = 0; k < 3; ++k) {

@@ -22,6 +22,13 @@ inline int grid_for(long total) {
   return (int)b;
 }
 
+// Kernel-space offset at element `i` of the rotation tensor; a null tensor stands for all zeros
+// (the deformable operator without kernel-space offsets).
+template <typename T>
+__device__ __forceinline__ compute_t<T> rot_at(const T* rot, size_t i) {
+  return rot ? static_cast<compute_t<T>>(ld(rot + i)) : compute_t<T>(0);
+}
+
 // planar_bilinear, K.cu:51-83, on a tile in global memory.
 template <typename T, typename CT>
 __device__ __forceinline__ CT tile_bilinear(const T* tile, int S_h, int S_w, CT h, CT w) {
@@ -173,8 +180,8 @@ __global__ __launch_bounds__(kBlock) void generic_forward_kernel(
         const CT xv = tap_input<T, CT, DEFORM>(g, xp, off, b, t, f_h, f_w, oh, ow, hit, ihf, iwf);
         if (hit) {
           const size_t ri = rot_index(g, b, grp, t, pix);
-          const CT h = scope_coord<CT>(g, f_h, ld(rot + ri), g.centre_h);
-          const CT w = scope_coord<CT>(g, f_w, ld(rot + ri + plane), g.centre_w);
+          const CT h = scope_coord<CT>(g, f_h, rot_at(rot, ri), g.centre_h);
+          const CT w = scope_coord<CT>(g, f_w, rot_at(rot, ri + plane), g.centre_w);
           sum += xv * tile_bilinear<T, CT>(tile, g.scope_h, g.scope_w, h, w);
         }
       }
@@ -210,8 +217,8 @@ __global__ __launch_bounds__(kBlock) void generic_local_grad_input_kernel(
         if (ow >= g.out_w) continue;
         const int t = f_h * g.k_w + f_w, opix = oh * g.out_w + ow;
         const size_t ri = rot_index(g, b, grp, t, opix);
-        const CT h = scope_coord<CT>(g, f_h, ld(rot + ri), g.centre_h);
-        const CT w = scope_coord<CT>(g, f_w, ld(rot + ri + oplane), g.centre_w);
+        const CT h = scope_coord<CT>(g, f_h, rot_at(rot, ri), g.centre_h);
+        const CT w = scope_coord<CT>(g, f_w, rot_at(rot, ri + oplane), g.centre_w);
         sum += ld(gp + opix) * tile_bilinear<T, CT>(tile, g.scope_h, g.scope_w, h, w);
       }
     }
@@ -239,8 +246,8 @@ __global__ __launch_bounds__(kBlock) void generic_deform_grad_input_kernel(
     if (!hit) continue;
     const int grp = c % g.groups;
     const size_t ri = rot_index(g, b, grp, t, pix);
-    const CT sh = scope_coord<CT>(g, f_h, ld(rot + ri), g.centre_h);
-    const CT sw = scope_coord<CT>(g, f_w, ld(rot + ri + oplane), g.centre_w);
+    const CT sh = scope_coord<CT>(g, f_h, rot_at(rot, ri), g.centre_h);
+    const CT sw = scope_coord<CT>(g, f_w, rot_at(rot, ri + oplane), g.centre_w);
     const CT ps = tile_bilinear<T, CT>(filter + (size_t)c * g.scope_h * g.scope_w, g.scope_h,
                                        g.scope_w, sh, sw) *
                   ld(gout + ((size_t)b * g.channel + c) * oplane + pix);
@@ -284,8 +291,8 @@ __global__ __launch_bounds__(kBlock) void generic_grad_rotation_kernel(
     const int f_h = t / g.k_w, f_w = t % g.k_w;
     const size_t ri = rot_index(g, b, grp, t, pix);
     bool open_h, open_w;  // false: the offset was clamped, its gradient is zero
-    const CT h = scope_coord<CT>(g, f_h, ld(rot + ri), g.centre_h, &open_h);
-    const CT w = scope_coord<CT>(g, f_w, ld(rot + ri + oplane), g.centre_w, &open_w);
+    const CT h = scope_coord<CT>(g, f_h, rot_at(rot, ri), g.centre_h, &open_h);
+    const CT w = scope_coord<CT>(g, f_w, rot_at(rot, ri + oplane), g.centre_w, &open_w);
     CT gh = 0, gw = 0;
     bool hit;
     CT ihf, iwf;
@@ -329,8 +336,8 @@ __global__ __launch_bounds__(kBlock) void generic_grad_offset_kernel(
       for (int c = 0; c < g.channel; ++c) {
         const int grp = c % g.groups;
         const size_t ri = rot_index(g, b, grp, t, pix);
-        const CT sh = scope_coord<CT>(g, f_h, ld(rot + ri), g.centre_h);
-        const CT sw = scope_coord<CT>(g, f_w, ld(rot + ri + oplane), g.centre_w);
+        const CT sh = scope_coord<CT>(g, f_h, rot_at(rot, ri), g.centre_h);
+        const CT sw = scope_coord<CT>(g, f_w, rot_at(rot, ri + oplane), g.centre_w);
         const CT ps = tile_bilinear<T, CT>(filter + (size_t)c * g.scope_h * g.scope_w, g.scope_h,
                                            g.scope_w, sh, sw) *
                       ld(gout + ((size_t)b * g.channel + c) * oplane + pix);
@@ -379,8 +386,8 @@ __global__ __launch_bounds__(kBlock) void generic_grad_filter_kernel(
           const CT xv = tap_input<T, CT, DEFORM>(g, xp, off, b, t, f_h, f_w, oh, ow, hit, ihf, iwf);
           if (!hit) continue;
           const size_t ri = rot_index(g, b, grp, t, pix);
-          const CT h = scope_coord<CT>(g, f_h, ld(rot + ri), g.centre_h);
-          const CT w = scope_coord<CT>(g, f_w, ld(rot + ri + oplane), g.centre_w);
+          const CT h = scope_coord<CT>(g, f_h, rot_at(rot, ri), g.centre_h);
+          const CT w = scope_coord<CT>(g, f_w, rot_at(rot, ri + oplane), g.centre_w);
           if (!(h > CT(-1) && w > CT(-1) && h < CT(S_h) && w < CT(S_w))) continue;
           const CT ps = xv * go;
           const CT hf = floor(h), wf = floor(w);

@@ -53,7 +53,7 @@ def _check_shapes(input, rotation, weight, out_size, kernel_size, rotation_group
         raise ValueError("channels (%d) must be divisible by rotation_groups (%d)" % (c, rotation_groups))
     taps2 = kernel_size[0] * kernel_size[1] * 2
     want = (input.size(0), rotation_groups * taps2, out_size[2], out_size[3])
-    if tuple(rotation.shape) != want:
+    if rotation is not None and tuple(rotation.shape) != want:
         raise ValueError("rotation must be %s, got %s" % (want, tuple(rotation.shape)))
     if offset is not None:
         want = (input.size(0), taps2, out_size[2], out_size[3])
@@ -148,11 +148,13 @@ class DeformableSampleDepthwiseFunction(Function):
         ctx.rotation_groups = rotation_groups
         ctx.rotation_clip = rotation_clip
 
-        _lib.require_gpu(input, offset, rotation, weight)
+        # rotation = None: no kernel-space offsets (DeformKernelConv2d / DeformConv2d); the library
+        # then reads no rotation tensor, where the reference's module hands over a tensor of zeros
+        _lib.require_gpu(*(t for t in (input, offset, rotation, weight) if t is not None))
         out_size = _output_size(input, kernel_size, stride, padding, dilation)
         _check_shapes(input, rotation, weight, out_size, kernel_size, rotation_groups, offset)
-        input, offset = input.contiguous(), offset.contiguous()
-        rotation, weight = rotation.contiguous(), weight.contiguous()
+        input, offset, weight = input.contiguous(), offset.contiguous(), weight.contiguous()
+        rotation = rotation.contiguous() if rotation is not None else None
         ctx.save_for_backward(input, offset, rotation, weight)
         output = input.new_empty(out_size)
         desc = _lib.conv_desc(input, weight, kernel_size, stride, padding, dilation, rotation_groups,
@@ -190,7 +192,7 @@ class DeformableSampleDepthwiseFunction(Function):
                 _lib.check(L.dk_deformable_sample_depthwise_backward_offset(
                     desc, p(grad_output), p(input), p(offset), p(rotation), p(weight),
                     p(grad_offset), p(ws), nbytes, s), "deform_sample_depthwise backward_offset")
-            if ctx.needs_input_grad[2]:
+            if ctx.needs_input_grad[2] and rotation is not None:
                 grad_rotation = torch.empty_like(rotation)
                 ws, nbytes = _lib.workspace(
                     L.dk_deformable_sample_depthwise_backward_rotation_workspace(desc), input.device)

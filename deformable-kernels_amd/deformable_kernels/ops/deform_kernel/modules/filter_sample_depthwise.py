@@ -109,8 +109,8 @@ class DeformableSampleDepthwise(_ScopeDepthwiseBase):
     def forward(self, input, offset=None, rotation=None, rotation_clip=None):
         if offset is None:
             offset = self._zeros_per_tap(input, 1)
-        if rotation is None:
-            rotation = self._zeros_per_tap(input, self.rotation_groups)
+        # rotation = None goes to the operator as it is: the library reads no rotation tensor then,
+        # where the reference fills one with zeros (:163-168); same values
         out = deform_sample_depthwise(
             input, offset, rotation, self.weight, self.kernel_size,
             self.stride, self.padding, self.dilation, self.rotation_groups, rotation_clip)

@@ -151,6 +151,15 @@ int dk_sample_depthwise_backward(const dk_conv_desc *desc, const void *out_grad,
 
 /* ---- deformable kernel with image-space offsets ---------------------------- */
 
+/* In the forward and in the data / filter / offset gradients below, `rotation` may be NULL: the
+ * kernel-space offsets are then all zero and no rotation tensor is read.  This is the call of
+ * DeformKernelConv2d / DeformConv2d (modules/deform_kernel.py:276-279 passes rotation = None,
+ * modules/deform_conv.py:31-42 sets scope = kernel), for which the reference allocates, fills
+ * and reads a zero tensor of batch x groups*k*k*2 x out_h x out_w elements
+ * (ops/deform_kernel/modules/filter_sample_depthwise.py:163-168); with scope = kernel the taps
+ * then sit on the scope's own cells and the result is the depthwise deformable convolution.
+ * Same values as with a tensor of zeros. */
+
 /* deformable_sample_depthwise_forward_cuda (filter_sample_depthwise_cuda.cpp:237-294). */
 int dk_deformable_sample_depthwise_forward(const dk_conv_desc *desc, const void *input,
                                            const void *offset, const void *rotation,

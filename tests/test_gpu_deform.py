@@ -268,3 +268,60 @@ def test_non_finite_values_reach_the_input_gradient(case, poison, where):
         assert bool(bad[N - 1, C // 2].any())   # where the reference's atomics would have put it
     else:
         assert bool(bad[:, 1].any())
+
+
+# ---- no rotation tensor (DeformKernelConv2d / DeformConv2d: rotation = None) ----------------------
+
+NO_ROTATION_CASES = [
+    (2, 16, 14, 14, 3, (3, 3), 2, 1, 1, 1, 0.0, 2.0),    # DeformConv2d: scope == kernel, stride 2
+    (1, 9, 56, 56, 3, (3, 3), 1, 1, 1, 1, 0.0, 2.0),     # 56 x 56 planes, the 1024-thread kernels
+    (2, 12, 13, 11, 3, (4, 4), 1, 1, 1, 1, 0.0, 2.0),    # DeformKernelConv2d with a scope larger than the kernel
+    (2, 6, 8, 8, (2, 3), (4, 5), (1, 2), (0, 1), 1, 3, 0.0, 1.0),  # the general kernels
+    (1, 3, 5, 70, 3, (3, 3), 1, 1, 1, 1, 0.0, 1.5),      # wider than the tuned kernels take
+]
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float64, torch.bfloat16])
+@pytest.mark.parametrize("case", NO_ROTATION_CASES)
+def test_without_a_rotation_tensor_equals_the_oracle_with_zero_rotation(case, dtype):
+    """rotation = None (a NULL pointer at the C ABI) is the reference's call with a tensor of zeros
+    (ops/deform_kernel/modules/filter_sample_depthwise.py:163-168), without that tensor."""
+    from deformable_kernels.ops.deform_kernel.functions import deform_sample_depthwise
+    N, C, H, W, k, S, s, p, d, G, rs, os_ = case
+    x, wt, rot, off, gout, cfg = make_deform(N, C, H, W, k, S, s, p, d, G, 0.0, os_, seed=7, dtype=dtype)
+    assert float(rot.abs().max()) == 0.0
+    dev = torch.device("cuda:0")
+    xg, og, wg = [t.to(dev).requires_grad_() for t in (x, off, wt)]
+    out = deform_sample_depthwise(xg, og, None, wg, cfg["kernel_size"], cfg["stride"], cfg["padding"],
+                                  cfg["dilation"], cfg["groups"])
+    out.backward(gout.to(dev))
+    torch.cuda.synchronize()
+    got = [t.detach().cpu() for t in (out, xg.grad, og.grad, wg.grad)]
+    o64 = _oracle((x, wt, rot, off, gout, cfg), np.float64)
+    want = [o64[i] for i in (0, 1, 2, 4)]
+    tol = {torch.float32: (1e-5, 1e-5, 1e-4, 1e-4), torch.float64: (1e-11,) * 4, torch.bfloat16: (1e-2,) * 4}[dtype]
+    for name, a, b, t in zip(("forward", "grad input", "grad offset", "grad filter"), got, want, tol):
+        if name == "grad offset" and dtype == torch.float32:
+            o32 = _oracle((x, wt, rot, off, gout, cfg), np.float32)[2].astype(np.float64)
+            err = np.minimum(np.abs(a.double().numpy() - b), np.abs(a.double().numpy() - o32))
+            assert err.max() / np.abs(b).max() < t, name
+        else:
+            assert rel_err(a.float() if dtype == torch.bfloat16 else a, b) < t, name
+
+
+def test_deform_conv_module_runs_without_a_rotation_tensor_and_is_a_depthwise_deformable_convolution():
+    """DeformConv2d (scope = kernel, rotation = None, reference modules/deform_conv.py:15-42): with
+    zero image-space offsets it is the plain depthwise convolution with its own weights."""
+    from deformable_kernels.modules import DeformConv2d
+    dev = torch.device("cuda:0")
+    torch.manual_seed(11)
+    m = DeformConv2d(12, 12, kernel_size=3, stride=1, padding=1, groups=12).to(dev)
+    with torch.no_grad():                                # the module marks offset_conv for zero initialisation (:262)
+        m.offset_conv.weight.zero_()
+        m.offset_conv.bias.zero_()
+    x = torch.randn(2, 12, 10, 9, device=dev, requires_grad=True)
+    out = m(x)
+    want = torch.nn.functional.conv2d(x.detach().double(), m.inner_conv.weight.detach().double(), padding=1, groups=12)
+    assert rel_err(out.detach().cpu(), want.cpu()) < 1e-5
+    out.sum().backward()
+    assert x.grad is not None and m.inner_conv.weight.grad is not None and m.offset_conv.weight.grad is not None
