@@ -191,6 +191,8 @@ def main():
     ap.add_argument("--workload", default="cfg2", choices=sorted(WORKLOADS) + sorted(OTHER_WORKLOADS) + sorted(GLOBAL_WORKLOADS) + ["mbv2_dk", "layer_cfg2"])
     ap.add_argument("--batch", type=int, default=64, help="batch size of the mbv2_dk workload")
     ap.add_argument("--dtype", default="fp32", choices=sorted(DTYPES))
+    ap.add_argument("--layout", default="nchw", choices=["nchw", "nhwc"],
+                    help="memory layout of the tensors of the local-operator workloads (nhwc: the channels-last kernels)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--kernels", default="", help="comma list restricting the per-kernel timing (tuning aid)")
     ap.add_argument("--traffic-from", nargs=2, metavar=("FETCH_DB", "WRITE_DB"),
@@ -225,12 +227,15 @@ def main():
     x, wt, rot, gout, cfg = make_local(N, C, H, W, k, S, stride, pad, dil, groups, rot_std, seed=0, dtype=tdtype)
     Ho, Wo = gout.shape[2], gout.shape[3]
     xg, wg, rg, gg = [t.to(dev) for t in (x, wt, rot, gout)]
+    if a.layout == "nhwc":
+        xg, rg, gg = [t.contiguous(memory_format=torch.channels_last) for t in (xg, rg, gg)]
     out = torch.empty_like(gg)
     gin = torch.empty_like(xg)
     grot = torch.empty_like(rg)
     gw = torch.empty_like(wg)
     L = _lib.lib()
-    desc = _lib.conv_desc(xg, wg, cfg["kernel_size"], cfg["stride"], cfg["padding"], cfg["dilation"], groups)
+    desc = _lib.conv_desc(xg, wg, cfg["kernel_size"], cfg["stride"], cfg["padding"], cfg["dilation"], groups,
+                          layout=_lib.LAYOUT_NHWC if a.layout == "nhwc" else _lib.LAYOUT_NCHW)
     ws, ws_bytes = _lib.workspace(L.dk_sample_depthwise_backward_workspace(desc), dev)
     P = _lib.ptr
 
@@ -330,7 +335,7 @@ def main():
     dominant = max((n for n in per_kernel_us if n != "backward"), key=per_kernel_us.get, default="backward")
     achieved = per_kernel_bytes[dominant] / (per_kernel_us[dominant] * 1e-6) / 1e9
 
-    traffic, traffic_stale = measured_traffic(a.workload, a.dtype, dominant)
+    traffic, traffic_stale = measured_traffic(a.workload, a.dtype, dominant) if a.layout == "nchw" else (None, False)
     result = {
         "metric": "DK fwd+bwd achieved HBM GB/s",
         "value": round(gbps, 2),
@@ -345,8 +350,9 @@ def main():
         "vs_baseline": None,
         "dtype": {"fp32": "f32", "bf16": "bf16", "fp16": "f16"}[a.dtype],
         "data": "synthetic",
-        "config": {"workload": "%s: DeformKernel2d op fwd+bwd N=%d C=%d %dx%d k=%d scope=%dx%d stride=%d pad=%d %s"
-                               % (a.workload, N, C, H, W, k, S[0], S[1], stride, pad, a.dtype),
+        "config": {"workload": "%s: DeformKernel2d op fwd+bwd N=%d C=%d %dx%d k=%d scope=%dx%d stride=%d pad=%d %s%s"
+                               % (a.workload, N, C, H, W, k, S[0], S[1], stride, pad, a.dtype,
+                                  ", channels-last tensors" if a.layout == "nhwc" else ""),
                    "algorithmic_MB_per_step": round(step_bytes / 1e6, 2)},
         "pct_of_hbm_peak": round(100.0 * gbps / HBM_PEAK_GBPS, 2),
         "device_copy_GBps": round(copy_gbps, 1),

@@ -83,6 +83,7 @@ int make_geo(const dk_conv_desc* d, Geo& g) {
       d->dil_h <= 0 || d->dil_w <= 0 || d->scope_h <= 0 || d->scope_w <= 0 || d->groups <= 0)
     return DK_ERR_BAD_SHAPE;
   if (d->channel % d->groups != 0) return DK_ERR_BAD_SHAPE;
+  if (d->layout != DK_LAYOUT_NCHW && d->layout != DK_LAYOUT_NHWC) return DK_ERR_BAD_SHAPE;
   if (d->rotation_clip < DK_CLIP_NONE || d->rotation_clip > DK_CLIP_COORD ||
       (d->rotation_clip != DK_CLIP_NONE && !(d->clip_min <= d->clip_max)))
     return DK_ERR_BAD_SHAPE;
@@ -162,7 +163,8 @@ int zero_filter_grad(const Geo& g, int dtype, void* filter_grad, hipStream_t s) 
   });
 }
 
-size_t local_filter_ws(const Geo& g, int dtype) {
+size_t local_filter_ws(const Geo& g, int dtype, int layout = DK_LAYOUT_NCHW) {
+  if (layout == DK_LAYOUT_NHWC) return nhwc_supported(g, dtype) ? nhwc_grad_filter_workspace(g, dtype) : 0;
   const size_t a = dtype == DK_F64 ? 0 : fast_local_grad_filter_workspace(g);
   return a ? a : generic_grad_filter_workspace(g, dtype);
 }
@@ -238,8 +240,13 @@ int dk_sample_depthwise_forward(const dk_conv_desc* desc, const void* input, con
   const int rc = make_geo(desc, g);
   if (rc != DK_OK) return rc;
   if (!input || !rotation || !filter || !output) return DK_ERR_NULL_POINTER;
+  if (desc->layout == DK_LAYOUT_NHWC && !nhwc_supported(g, desc->dtype)) return DK_ERR_UNSUPPORTED;
   if (g.batch == 0) return DK_OK;
   hipStream_t s = static_cast<hipStream_t>(stream);
+  if (desc->layout == DK_LAYOUT_NHWC)
+    return by_dtype(desc->dtype, [&]<typename T>() {
+      nhwc_gather<T>(g, false, in<T>(input), in<T>(rotation), in<T>(filter), out<T>(output), s);
+    });
   return by_dtype(desc->dtype, [&]<typename T>() {
     if constexpr (kHasFast<T>)
       if (fast_local_gather<T>(g, false, in<T>(input), in<T>(rotation), in<T>(filter), out<T>(output), s)) return;
@@ -254,8 +261,13 @@ int dk_sample_depthwise_backward_data(const dk_conv_desc* desc, const void* out_
   const int rc = make_geo(desc, g);
   if (rc != DK_OK) return rc;
   if (!out_grad || !rotation || !filter || !in_grad) return DK_ERR_NULL_POINTER;
+  if (desc->layout == DK_LAYOUT_NHWC && !nhwc_supported(g, desc->dtype)) return DK_ERR_UNSUPPORTED;
   if (g.batch == 0) return DK_OK;
   hipStream_t s = static_cast<hipStream_t>(stream);
+  if (desc->layout == DK_LAYOUT_NHWC)
+    return by_dtype(desc->dtype, [&]<typename T>() {
+      nhwc_gather<T>(g, true, in<T>(out_grad), in<T>(rotation), in<T>(filter), out<T>(in_grad), s);
+    });
   return by_dtype(desc->dtype, [&]<typename T>() {
     if constexpr (kHasFast<T>)
       if (fast_local_gather<T>(g, true, in<T>(out_grad), in<T>(rotation), in<T>(filter), out<T>(in_grad), s)) return;
@@ -266,7 +278,7 @@ int dk_sample_depthwise_backward_data(const dk_conv_desc* desc, const void* out_
 size_t dk_sample_depthwise_backward_filter_workspace(const dk_conv_desc* desc) {
   Geo g;
   if (make_geo(desc, g) != DK_OK) return 0;
-  return local_filter_ws(g, desc->dtype);
+  return local_filter_ws(g, desc->dtype, desc->layout);
 }
 
 int dk_sample_depthwise_backward_filter(const dk_conv_desc* desc, const void* out_grad,
@@ -276,10 +288,15 @@ int dk_sample_depthwise_backward_filter(const dk_conv_desc* desc, const void* ou
   const int rc = make_geo(desc, g);
   if (rc != DK_OK) return rc;
   if (!out_grad || !input || !rotation || !filter_grad) return DK_ERR_NULL_POINTER;
-  const size_t need = local_filter_ws(g, desc->dtype);
+  if (desc->layout == DK_LAYOUT_NHWC && !nhwc_supported(g, desc->dtype)) return DK_ERR_UNSUPPORTED;
+  const size_t need = local_filter_ws(g, desc->dtype, desc->layout);
   if (need && (!workspace || workspace_bytes < need)) return DK_ERR_WORKSPACE;
   hipStream_t s = static_cast<hipStream_t>(stream);
   if (g.batch == 0) return zero_filter_grad(g, desc->dtype, filter_grad, s);
+  if (desc->layout == DK_LAYOUT_NHWC)
+    return by_dtype(desc->dtype, [&]<typename T>() {
+      nhwc_grad_filter<T>(g, in<T>(out_grad), in<T>(input), in<T>(rotation), out<T>(filter_grad), workspace, s);
+    });
   return by_dtype(desc->dtype, [&]<typename T>() {
     if constexpr (kHasFast<T>)
       if (fast_local_grad_filter<T>(g, in<T>(out_grad), in<T>(input), in<T>(rotation), out<T>(filter_grad), workspace, s)) return;
@@ -291,6 +308,7 @@ int dk_sample_depthwise_backward_filter(const dk_conv_desc* desc, const void* ou
 size_t dk_sample_depthwise_backward_rotation_workspace(const dk_conv_desc* desc) {
   Geo g;
   if (make_geo(desc, g) != DK_OK) return 0;
+  if (desc->layout == DK_LAYOUT_NHWC) return 0;
   return desc->dtype == DK_F64 ? 0 : fast_local_grad_rotation_workspace(g);
 }
 
@@ -302,10 +320,15 @@ int dk_sample_depthwise_backward_rotation(const dk_conv_desc* desc, const void* 
   const int rc = make_geo(desc, g);
   if (rc != DK_OK) return rc;
   if (!out_grad || !input || !rotation || !filter || !rotation_grad) return DK_ERR_NULL_POINTER;
+  if (desc->layout == DK_LAYOUT_NHWC && !nhwc_supported(g, desc->dtype)) return DK_ERR_UNSUPPORTED;
   const size_t need = dk_sample_depthwise_backward_rotation_workspace(desc);
   if (need && (!workspace || workspace_bytes < need)) return DK_ERR_WORKSPACE;
   if (g.batch == 0) return DK_OK;
   hipStream_t s = static_cast<hipStream_t>(stream);
+  if (desc->layout == DK_LAYOUT_NHWC)
+    return by_dtype(desc->dtype, [&]<typename T>() {
+      nhwc_grad_rotation<T>(g, in<T>(out_grad), in<T>(input), in<T>(rotation), in<T>(filter), out<T>(rotation_grad), s);
+    });
   return by_dtype(desc->dtype, [&]<typename T>() {
     if constexpr (kHasFast<T>)
       if (fast_local_grad_rotation<T>(g, in<T>(out_grad), in<T>(input), in<T>(rotation), in<T>(filter),
@@ -324,7 +347,7 @@ int dk_sample_depthwise_backward_filter_static(const dk_conv_desc* desc, const v
   const int rc = make_geo(desc, g);
   if (rc != DK_OK) return rc;
   if (!out_grad || !input || !rotation || !filter_grad) return DK_ERR_NULL_POINTER;
-  if (local_filter_ws(g, desc->dtype) > (size_t)DK_STATIC_SCRATCH_BYTES) return DK_ERR_SCRATCH_LIMIT;
+  if (local_filter_ws(g, desc->dtype, desc->layout) > (size_t)DK_STATIC_SCRATCH_BYTES) return DK_ERR_SCRATCH_LIMIT;
   void* ptr = nullptr;
   const int st = static_scratch_of_current_device(&ptr);
   if (st != DK_OK) return st;
@@ -375,6 +398,7 @@ int dk_deformable_sample_depthwise_forward(const dk_conv_desc* desc, const void*
   Geo g;
   const int rc = make_geo(desc, g);
   if (rc != DK_OK) return rc;
+  if (desc->layout != DK_LAYOUT_NCHW) return DK_ERR_UNSUPPORTED;
   if (!input || !offset || !filter || !output) return DK_ERR_NULL_POINTER;  // rotation may be NULL: all zeros
   if (g.batch == 0) return DK_OK;
   hipStream_t s = static_cast<hipStream_t>(stream);
@@ -398,6 +422,7 @@ int dk_deformable_sample_depthwise_backward_data(const dk_conv_desc* desc, const
   Geo g;
   const int rc = make_geo(desc, g);
   if (rc != DK_OK) return rc;
+  if (desc->layout != DK_LAYOUT_NCHW) return DK_ERR_UNSUPPORTED;
   if (!out_grad || !offset || !filter || !in_grad) return DK_ERR_NULL_POINTER;  // rotation may be NULL: all zeros
   const size_t need = dk_deformable_sample_depthwise_backward_data_workspace(desc);
   if (need && (!workspace || workspace_bytes < need)) return DK_ERR_WORKSPACE;
@@ -426,6 +451,7 @@ int dk_deformable_sample_depthwise_backward_filter(const dk_conv_desc* desc, con
   Geo g;
   const int rc = make_geo(desc, g);
   if (rc != DK_OK) return rc;
+  if (desc->layout != DK_LAYOUT_NCHW) return DK_ERR_UNSUPPORTED;
   if (!out_grad || !input || !offset || !filter_grad) return DK_ERR_NULL_POINTER;  // rotation may be NULL: all zeros
   const size_t need = dk_deformable_sample_depthwise_backward_filter_workspace(desc);
   if (need && (!workspace || workspace_bytes < need)) return DK_ERR_WORKSPACE;
@@ -454,6 +480,7 @@ int dk_deformable_sample_depthwise_backward_offset(const dk_conv_desc* desc, con
   Geo g;
   const int rc = make_geo(desc, g);
   if (rc != DK_OK) return rc;
+  if (desc->layout != DK_LAYOUT_NCHW) return DK_ERR_UNSUPPORTED;
   if (!out_grad || !input || !offset || !filter || !offset_grad) return DK_ERR_NULL_POINTER;  // rotation may be NULL: all zeros
   const size_t need = fast_deform_grad_coord_workspace(g, false);
   if (need && (!workspace || workspace_bytes < need)) return DK_ERR_WORKSPACE;
@@ -482,6 +509,7 @@ int dk_deformable_sample_depthwise_backward_rotation(const dk_conv_desc* desc, c
   Geo g;
   const int rc = make_geo(desc, g);
   if (rc != DK_OK) return rc;
+  if (desc->layout != DK_LAYOUT_NCHW) return DK_ERR_UNSUPPORTED;
   if (!out_grad || !input || !offset || !rotation || !filter || !rotation_grad) return DK_ERR_NULL_POINTER;
   const size_t need = fast_deform_grad_coord_workspace(g, true);
   if (need && (!workspace || workspace_bytes < need)) return DK_ERR_WORKSPACE;
@@ -519,7 +547,7 @@ static bool kernel_strides(const Geo& g, const int64_t* given, long (&ws)[4], co
 
 int dk_image_depthwise_supported(const dk_conv_desc* desc) {
   Geo g;
-  return make_geo(desc, g) == DK_OK && image_conv_supported(g, desc->dtype);
+  return make_geo(desc, g) == DK_OK && desc->layout == DK_LAYOUT_NCHW && image_conv_supported(g, desc->dtype);
 }
 
 int dk_image_depthwise_forward(const dk_conv_desc* desc, const void* input, const void* weight,
@@ -527,6 +555,7 @@ int dk_image_depthwise_forward(const dk_conv_desc* desc, const void* input, cons
   Geo g;
   const int rc = make_geo(desc, g);
   if (rc != DK_OK) return rc;
+  if (desc->layout != DK_LAYOUT_NCHW) return DK_ERR_UNSUPPORTED;
   if (!input || !weight || !output) return DK_ERR_NULL_POINTER;
   if (!image_conv_supported(g, desc->dtype)) return DK_ERR_UNSUPPORTED;
   long ws_buf[4];
@@ -546,6 +575,7 @@ int dk_image_depthwise_backward_data(const dk_conv_desc* desc, const void* out_g
   Geo g;
   const int rc = make_geo(desc, g);
   if (rc != DK_OK) return rc;
+  if (desc->layout != DK_LAYOUT_NCHW) return DK_ERR_UNSUPPORTED;
   if (!out_grad || !weight || !in_grad) return DK_ERR_NULL_POINTER;
   if (!image_conv_supported(g, desc->dtype)) return DK_ERR_UNSUPPORTED;
   long ws_buf[4];
@@ -565,6 +595,7 @@ int dk_image_depthwise_backward_weight(const dk_conv_desc* desc, const void* out
   Geo g;
   const int rc = make_geo(desc, g);
   if (rc != DK_OK) return rc;
+  if (desc->layout != DK_LAYOUT_NCHW) return DK_ERR_UNSUPPORTED;
   if (!out_grad || !input || !weight_grad) return DK_ERR_NULL_POINTER;
   if (!image_conv_supported(g, desc->dtype)) return DK_ERR_UNSUPPORTED;
   long ws_buf[4];

@@ -122,6 +122,19 @@ bool offset_conv_wgrad(int batch, int cin, int cout, int h, int w, const float* 
 bool offset_conv_forward(int batch, int cin, int cout, int h, int w, const float* x, const float* weight,
                          const float* bias, float* out, void* ws, hipStream_t stream);
 
+// dk_local_nhwc.hip: the local operator on channels-last tensors, all dtypes, any geometry whose tables fit LDS
+bool nhwc_supported(const Geo& g, int dtype);
+template <typename T>
+void nhwc_gather(const Geo& g, bool transposed, const T* src, const T* rot, const T* filter, T* dst,
+                 hipStream_t stream);
+template <typename T>
+void nhwc_grad_rotation(const Geo& g, const T* gout, const T* x, const T* rot, const T* filter, T* grot,
+                        hipStream_t stream);
+size_t nhwc_grad_filter_workspace(const Geo& g, int dtype);
+template <typename T>
+void nhwc_grad_filter(const Geo& g, const T* gout, const T* x, const T* rot, T* gfilter, void* ws,
+                      hipStream_t stream);
+
 // dk_image_conv.hip: depthwise convolution with one kernel per (image, channel) plane, all dtypes
 bool image_conv_supported(const Geo& g, int dtype);
 // wstrides: element strides of the kernel tensor's (image, channel, tap row, tap column) axes, or null

@@ -25,7 +25,7 @@ class ConvDesc(ctypes.Structure):
     _fields_ = [(n, ctypes.c_int32) for n in (
         "batch", "channel", "in_h", "in_w", "k_h", "k_w", "stride_h", "stride_w",
         "pad_h", "pad_w", "dil_h", "dil_w", "scope_h", "scope_w", "groups", "dtype", "rotation_clip")
-    ] + [("clip_min", ctypes.c_float), ("clip_max", ctypes.c_float)]
+    ] + [("clip_min", ctypes.c_float), ("clip_max", ctypes.c_float), ("layout", ctypes.c_int32)]
 
 
 class NdDesc(ctypes.Structure):
@@ -197,13 +197,22 @@ def clip_triple(rotation_clip, weight):
     return (CLIP_ROTATION, lo, hi)
 
 
-def conv_desc(input, weight, kernel_size, stride, padding, dilation, rotation_groups, rotation_clip=None):
+LAYOUT_NCHW, LAYOUT_NHWC = 0, 1
+
+
+def channels_last(t):
+    """Whether a 4-d tensor is stored channels-last and not also in the default order."""
+    return t.dim() == 4 and not t.is_contiguous() and t.is_contiguous(memory_format=torch.channels_last)
+
+
+def conv_desc(input, weight, kernel_size, stride, padding, dilation, rotation_groups, rotation_clip=None,
+              layout=LAYOUT_NCHW):
     mode, lo, hi = clip_triple(rotation_clip, weight)
     return ConvDesc(
         input.size(0), input.size(1), input.size(2), input.size(3),
         int(kernel_size[0]), int(kernel_size[1]), int(stride[0]), int(stride[1]),
         int(padding[0]), int(padding[1]), int(dilation[0]), int(dilation[1]),
-        weight.size(2), weight.size(3), int(rotation_groups), dtype_tag(input), mode, lo, hi)
+        weight.size(2), weight.size(3), int(rotation_groups), dtype_tag(input), mode, lo, hi, layout)
 
 
 def nd_desc(data, coord):

@@ -85,11 +85,18 @@ class SampleDepthwiseFunction(Function):
         _lib.require_gpu(input, rotation, weight)
         out_size = _output_size(input, kernel_size, stride, padding, dilation)
         _check_shapes(input, rotation, weight, out_size, kernel_size, rotation_groups)
-        input, rotation, weight = input.contiguous(), rotation.contiguous(), weight.contiguous()
+        # A channels-last input runs the library's channels-last kernels and gets a channels-last
+        # output (and gradients): no layout change around the operator.  The reference's kernels
+        # take planar tensors only.
+        nhwc = _lib.channels_last(input)
+        fmt = torch.channels_last if nhwc else torch.contiguous_format
+        ctx.layout = _lib.LAYOUT_NHWC if nhwc else _lib.LAYOUT_NCHW
+        input, rotation = input.contiguous(memory_format=fmt), rotation.contiguous(memory_format=fmt)
+        weight = weight.contiguous()
         ctx.save_for_backward(input, rotation, weight)
-        output = input.new_empty(out_size)
+        output = torch.empty(out_size, dtype=input.dtype, device=input.device, memory_format=fmt)
         desc = _lib.conv_desc(input, weight, kernel_size, stride, padding, dilation, rotation_groups,
-                              rotation_clip)
+                              rotation_clip, ctx.layout)
         with torch.cuda.device(input.device):
             _lib.check(_lib.lib().dk_sample_depthwise_forward(
                 desc, _lib.ptr(input), _lib.ptr(rotation), _lib.ptr(weight), _lib.ptr(output),
@@ -102,9 +109,10 @@ class SampleDepthwiseFunction(Function):
         input, rotation, weight = ctx.saved_tensors
         grad_input = grad_rotation = grad_weight = None
         _lib.require_gpu(grad_output, input)
-        grad_output = grad_output.contiguous()
+        nhwc = ctx.layout == _lib.LAYOUT_NHWC
+        grad_output = grad_output.contiguous(memory_format=torch.channels_last if nhwc else torch.contiguous_format)
         desc = _lib.conv_desc(input, weight, ctx.kernel_size, ctx.stride, ctx.padding, ctx.dilation,
-                              ctx.rotation_groups, ctx.rotation_clip)
+                              ctx.rotation_groups, ctx.rotation_clip, ctx.layout)
         L = _lib.lib()
         with torch.cuda.device(input.device):
             s = _lib.stream_ptr(input)

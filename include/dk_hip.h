@@ -59,6 +59,8 @@ typedef enum dk_rotation_clip {
                            (rotation_clip == 'scope': clip_min = 0, clip_max = scope_h - 1) */
 } dk_rotation_clip;
 
+typedef enum dk_layout { DK_LAYOUT_NCHW = 0, DK_LAYOUT_NHWC = 1 } dk_layout;
+
 /* Geometry of one depthwise deformable-kernel layer: the fields the
  * reference packs into SampleDepthwiseArgs (csrc/filter_sample_depthwise_cuda.h:1-28)
  * from the tensor sizes and the eleven ints of each pybind call; out_h/out_w
@@ -89,6 +91,14 @@ typedef struct dk_conv_desc {
    * gradient with respect to a clamped offset is zero, as torch.clamp's is. */
   int32_t rotation_clip;    /* dk_rotation_clip */
   float clip_min, clip_max; /* the range; ignored for DK_CLIP_NONE */
+  /* Memory layout of the 4-d tensors of the call (input, rotation, output and their gradients;
+   * the filter is always [channel][scope_h][scope_w]).  DK_LAYOUT_NCHW (0) is the reference's.
+   * DK_LAYOUT_NHWC: the same logical tensors stored channels-last ([batch][h][w][channel];
+   * rotation [batch][out_h][out_w][groups*k_h*k_w*2]), for networks whose other layers run
+   * channels-last.  Taken by the local operator's entry points (dk_sample_depthwise_*); the
+   * deformable and per-image entry points return DK_ERR_UNSUPPORTED for it.  The reference has
+   * no such argument. */
+  int32_t layout;           /* dk_layout */
 } dk_conv_desc;
 
 /* Output extent for the descriptor, or a negative dk_status. */

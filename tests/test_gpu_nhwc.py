@@ -1,0 +1,127 @@
+"""The local deformable-kernel operator on channels-last tensors against the CPU oracle (which works on
+the logical NCHW tensors: the layout changes where an element is stored, not its value), through the
+Python Function and the C ABI's layout field.  Tolerances as for the planar operator: fp32 forward and
+grad input 1e-5 (fp32 oracle), grad rotation and grad filter 1e-4 (fp64 oracle); fp64 1e-11; fp16 /
+bf16 1e-2 against the fp32 oracle on the rounded inputs."""
+import numpy as np
+import pytest
+import torch
+
+from _cases import clipped_rotation, make_local, rel_err
+from oracle import dk_oracle as orc
+
+pytestmark = pytest.mark.gpu
+DEV = torch.device("cuda:0")
+
+# N, C, H, W, k, S, stride, pad, dil, groups, rot_std
+CASES = [
+    (2, 32, 28, 28, 3, (4, 4), 1, 1, 1, 1, 0.5),    # benchmark configuration 1: four channels per lane
+    (3, 20, 17, 23, 3, (4, 4), 1, 1, 1, 1, 1.0),    # ragged sizes
+    (2, 24, 19, 19, 3, (4, 4), 2, 1, 1, 1, 1.0),    # stride 2: grad input skips the taps off the stride's grid
+    (2, 12, 15, 14, 3, (4, 4), 1, 2, 2, 3, 1.0),    # dilation 2, rotation groups 3: one channel per lane
+    (2, 18, 13, 13, 3, (3, 3), 1, 1, 1, 1, 1.0),    # scope == kernel, channels not a multiple of 4
+    (1, 16, 13, 12, 3, (5, 5), 1, 0, 1, 2, 1.5),    # scope 5, no padding, two groups
+    (1, 300, 9, 9, 3, (4, 4), 1, 1, 1, 1, 2.0),     # more channels than a chunk (256): two channel chunks
+    (2, 6, 9, 8, (5, 3), (7, 4), (1, 2), (2, 0), 1, 3, 0.7),   # general taps and scope: sums in LDS columns
+    (1, 4, 8, 8, 2, (4, 4), 2, 0, 1, 2, 0.5),
+    (2, 8, 40, 36, 3, (4, 4), 1, 1, 1, 1, 0.7),     # 2880 pixels: several partial sums of the grad filter
+]
+
+
+def _run(case, dtype, seed=0, clip=None):
+    from deformable_kernels.ops.deform_kernel.functions import sample_depthwise
+    N, C, H, W, k, S, s, p, d, G, rs = case
+    x, wt, rot, gout, cfg = make_local(N, C, H, W, k, S, s, p, d, G, rs, seed=seed, dtype=dtype)
+    cl = torch.channels_last
+    xg = x.to(DEV).contiguous(memory_format=cl).requires_grad_()
+    rg = rot.to(DEV).contiguous(memory_format=cl).requires_grad_()
+    wg = wt.to(DEV).requires_grad_()
+    out = sample_depthwise(xg, rg, wg, cfg["kernel_size"], cfg["stride"], cfg["padding"], cfg["dilation"],
+                           cfg["groups"], clip)
+    assert out.is_contiguous(memory_format=cl)
+    out.backward(gout.to(DEV).contiguous(memory_format=cl))
+    torch.cuda.synchronize()
+    if C > 1 and H * W > 1:
+        assert xg.grad.is_contiguous(memory_format=cl) and rg.grad.is_contiguous(memory_format=cl)
+    return (x, wt, rot, gout, cfg), [t.detach().cpu().contiguous() for t in (out, xg.grad, rg.grad, wg.grad)]
+
+
+def _oracle(inputs, np_dtype):
+    x, wt, rot, gout, cfg = inputs
+    a = [t.to(torch.float64).numpy().astype(np_dtype) for t in (x, rot, wt, gout)]
+    out = orc.sample_depthwise_forward(a[0], a[1], a[2], **cfg)
+    return (out,) + tuple(orc.sample_depthwise_backward(a[3], a[0], a[1], a[2], **cfg))
+
+
+@pytest.mark.parametrize("case", CASES)
+def test_fp32_matches_oracle(case):
+    inputs, got = _run(case, torch.float32)
+    o32, o64 = _oracle(inputs, np.float32), _oracle(inputs, np.float64)
+    assert rel_err(got[0], o32[0]) < 1e-5
+    assert rel_err(got[1], o32[1]) < 1e-5
+    assert rel_err(got[2], o64[2]) < 1e-4
+    assert rel_err(got[3], o64[3]) < 1e-4
+
+
+@pytest.mark.parametrize("case", CASES[:4] + CASES[7:8])
+def test_fp64_matches_oracle(case):
+    inputs, got = _run(case, torch.float64)
+    want = _oracle(inputs, np.float64)
+    for g, w in zip(got, want):
+        assert rel_err(g, w) < 1e-11
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("case", CASES[:3] + CASES[5:7])
+def test_half_precisions_match_fp32_oracle(case, dtype):
+    inputs, got = _run(case, dtype, seed=3)
+    want = _oracle(inputs, np.float32)
+    for g, w in zip(got, want):
+        assert g.dtype == dtype
+        assert rel_err(g.float(), w) < 1e-2
+
+
+def test_equals_the_planar_operator_on_the_same_tensors():
+    """Same logical input, two layouts: the results agree to rounding (the sums run in another order)."""
+    from deformable_kernels.ops.deform_kernel.functions import sample_depthwise
+    case = (2, 48, 30, 26, 3, (4, 4), 1, 1, 1, 1, 1.0)
+    N, C, H, W, k, S, s, p, d, G, rs = case
+    x, wt, rot, gout, cfg = make_local(N, C, H, W, k, S, s, p, d, G, rs, seed=9)
+    res = []
+    for fmt in (torch.contiguous_format, torch.channels_last):
+        xg = x.to(DEV).contiguous(memory_format=fmt).requires_grad_()
+        rg = rot.to(DEV).contiguous(memory_format=fmt).requires_grad_()
+        wg = wt.to(DEV).requires_grad_()
+        out = sample_depthwise(xg, rg, wg, cfg["kernel_size"], cfg["stride"], cfg["padding"], cfg["dilation"], G)
+        out.backward(gout.to(DEV))  # a planar out_grad for both: the Function brings it into its layout
+        res.append([t.detach().cpu().contiguous() for t in (out, xg.grad, rg.grad, wg.grad)])
+    for a, b, tol in zip(res[1], res[0], (1e-5, 1e-5, 1e-4, 1e-4)):
+        assert rel_err(a, b) < tol
+
+
+@pytest.mark.parametrize("clip", ['scope', (-0.3, 0.2)])
+def test_rotation_clip_inside_the_channels_last_operator(clip):
+    case = (2, 12, 11, 10, 3, (4, 4), 1, 1, 1, 2, 1.5)
+    inputs, got = _run(case, torch.float32, seed=5, clip=clip)
+    x, wt, rot, gout, cfg = inputs
+    clamped, open_ = clipped_rotation(rot, clip, cfg["kernel_size"], (4, 4), 2)
+    o64 = _oracle((x, wt, clamped, gout, cfg), np.float64)
+    assert rel_err(got[0], o64[0]) < 1e-5
+    assert rel_err(got[1], o64[1]) < 1e-5
+    assert rel_err(got[2], torch.as_tensor(o64[2]) * open_.double()) < 1e-4
+    assert rel_err(got[3], o64[3]) < 1e-4
+
+
+def test_c_abi_layout_field():
+    from deformable_kernels.ops.deform_kernel import _lib
+    L = _lib.lib()
+    x = torch.zeros(1, 4, 6, 6, device=DEV)
+    d = _lib.ConvDesc(1, 4, 6, 6, 3, 3, 1, 1, 1, 1, 1, 1, 4, 4, 1, _lib.DK_F32, 0, 0.0, 0.0, 7)
+    assert L.dk_sample_depthwise_forward(d, _lib.ptr(x), _lib.ptr(x), _lib.ptr(x), _lib.ptr(x), None) == -2  # bad layout
+    d.layout = _lib.LAYOUT_NHWC
+    off = torch.zeros(1, 18, 6, 6, device=DEV)
+    assert L.dk_deformable_sample_depthwise_forward(d, _lib.ptr(x), _lib.ptr(off), _lib.ptr(off), _lib.ptr(x),
+                                                    _lib.ptr(x), None) == -7  # DK_ERR_UNSUPPORTED
+    assert L.dk_image_depthwise_supported(d) == 0
+    assert L.dk_sample_depthwise_backward_filter_workspace(d) > 0
+    assert L.dk_sample_depthwise_backward_rotation_workspace(d) == 0
