@@ -107,7 +107,9 @@ struct NhwcLaunch {
 
 // forward (TRANSPOSED = false) and grad input (true); VEC channels per lane (4 needs one rotation
 // group, channels a multiple of 4 and 16-byte aligned tensors)
-template <typename T, int VEC, bool TRANSPOSED>
+// TAPS: the tap count when it is known at compile time (9: a lane's nine source loads are issued
+// before the first is used), 0: any.
+template <typename T, int VEC, bool TRANSPOSED, int TAPS>
 __global__ __launch_bounds__(kNBlock) void nhwc_gather_kernel(Geo g, NhwcLaunch L, const T* __restrict__ src,
                                                               const T* __restrict__ rot,
                                                               const T* __restrict__ filter, T* __restrict__ dst) {
@@ -139,35 +141,58 @@ __global__ __launch_bounds__(kNBlock) void nhwc_gather_kernel(Geo g, NhwcLaunch 
 #pragma unroll
     for (int v = 0; v < VEC; ++v) acc[v] = CT(0);
     const NhwcTap<CT>* row = table + (size_t)(pl * g.groups + (VEC == 1 ? c % g.groups : 0)) * taps;
-    for (int t = 0; t < taps; ++t) {
-      const NhwcTap<CT> e = row[t];
-      if (e.src < 0) continue;
-      CT xv[VEC];
-      if constexpr (VEC == 4) {
-        struct alignas(sizeof(T) * 4) Pack { T v[4]; };
-        const Pack pk = *reinterpret_cast<const Pack*>(src + e.src + c);
+    struct alignas(sizeof(T) * VEC) Pack { T v[VEC]; };
+    struct alignas(sizeof(CT) * VEC) WVec { CT v[VEC]; };
+    if constexpr (TAPS > 0) {
+      Pack pk[TAPS];
+      bool on[TAPS];
 #pragma unroll
-        for (int v = 0; v < 4; ++v) xv[v] = (CT)ld(pk.v + v);
-      } else {
-        xv[0] = (CT)ld(src + e.src + c);
+      for (int t = 0; t < TAPS; ++t) {
+        const long so = row[t].src;
+        on[t] = so >= 0;
+        pk[t] = *reinterpret_cast<const Pack*>(src + (on[t] ? so : 0) + c);  // a dead tap reads element c of the tensor: valid, unused
       }
 #pragma unroll
-      for (int v = 0; v < VEC; ++v) {
-        CT wv = CT(0);
+      for (int t = 0; t < TAPS; ++t) {
+        int cell[4];
+        CT w[4];
 #pragma unroll
-        for (int k = 0; k < 4; ++k) wv += e.w[k] * wt[e.cell[k] * L.cc + cl + v];
-        acc[v] += xv[v] * wv;
+        for (int k = 0; k < 4; ++k) cell[k] = row[t].cell[k], w[k] = row[t].w[k];
+        // the lane's VEC channels of a cell in one LDS read (a read per channel has the lanes VEC banks apart)
+        WVec f[4];
+#pragma unroll
+        for (int k = 0; k < 4; ++k) f[k] = *reinterpret_cast<const WVec*>(wt + cell[k] * L.cc + cl);
+#pragma unroll
+        for (int v = 0; v < VEC; ++v) {
+          CT wv = CT(0);
+#pragma unroll
+          for (int k = 0; k < 4; ++k) wv += w[k] * f[k].v[v];
+          const CT xv = on[t] ? (CT)ld(pk[t].v + v) : CT(0);
+          acc[v] += xv * wv;
+        }
+      }
+    } else {
+      for (int t = 0; t < taps; ++t) {
+        const NhwcTap<CT> e = row[t];
+        if (e.src < 0) continue;
+        const Pack pk = *reinterpret_cast<const Pack*>(src + e.src + c);
+        WVec f[4];
+#pragma unroll
+        for (int k = 0; k < 4; ++k) f[k] = *reinterpret_cast<const WVec*>(wt + e.cell[k] * L.cc + cl);
+#pragma unroll
+        for (int v = 0; v < VEC; ++v) {
+          CT wv = CT(0);
+#pragma unroll
+          for (int k = 0; k < 4; ++k) wv += e.w[k] * f[k].v[v];
+          acc[v] += (CT)ld(pk.v + v) * wv;
+        }
       }
     }
     T* out = dst + ((size_t)b * L.dst_pixels + p0 + pl) * g.channel + c;
-    if constexpr (VEC == 4) {
-      struct alignas(sizeof(T) * 4) Pack { T v[4]; } pk;
+    Pack res;
 #pragma unroll
-      for (int v = 0; v < 4; ++v) st(pk.v + v, acc[v]);
-      *reinterpret_cast<Pack*>(out) = pk;
-    } else {
-      st(out, acc[0]);
-    }
+    for (int v = 0; v < VEC; ++v) st(res.v + v, acc[v]);
+    *reinterpret_cast<Pack*>(out) = res;
   }
 }
 
@@ -247,9 +272,122 @@ __global__ __launch_bounds__(kNBlock) void nhwc_grad_rotation_kernel(Geo g, cons
   }
 }
 
+// grad rotation for 3 x 3 taps with the filter in LDS: the derivative weights of each (pixel, group,
+// tap) are computed once into a table (one thread per entry); a wave then takes a (pixel, group),
+// walks the group's channels with lanes over channels -- out_grad and the nine tap inputs loaded
+// first -- and keeps 18 running sums, added up over the wave at the end and written as one
+// contiguous run of 18 values.
+template <typename CT>
+struct NhwcRotTap {
+  int cell[4];
+  CT dh[4], dw[4];
+  long src;
+  int open;  // bit 0 / 1: the h / w offset was not clamped (its gradient passes)
+};
+
+template <typename T>
+__global__ __launch_bounds__(kNBlock) void nhwc_grad_rotation9_kernel(Geo g, const T* __restrict__ gout,
+                                                                      const T* __restrict__ x,
+                                                                      const T* __restrict__ rot,
+                                                                      const T* __restrict__ filter,
+                                                                      T* __restrict__ grot, int pb) {
+  using CT = compute_t<T>;
+  constexpr int TAPS = 9;
+  extern __shared__ __align__(16) unsigned char nhwc_lds[];
+  const int cells = g.scope_h * g.scope_w;
+  CT* wt = reinterpret_cast<CT*>(nhwc_lds);  // [cells][channel]
+  NhwcRotTap<CT>* table =
+      reinterpret_cast<NhwcRotTap<CT>*>(nhwc_lds + (((size_t)cells * g.channel * sizeof(CT) + 15) & ~(size_t)15));
+  const int oplane = g.out_h * g.out_w;
+  const long total_pix = (long)g.batch * oplane;
+  const long q0 = (long)blockIdx.x * pb;
+  const int npix = (int)min((long)pb, total_pix - q0);
+  for (int i = threadIdx.x; i < cells * g.channel; i += kNBlock) {
+    const int ch = i / cells, cell = i - ch * cells;
+    wt[(size_t)cell * g.channel + ch] = (CT)ld(filter + i);
+  }
+  for (int i = threadIdx.x; i < npix * g.groups * TAPS; i += kNBlock) {
+    const int t = i % TAPS, grp = i / TAPS % g.groups, pl = i / TAPS / g.groups;
+    const long q = q0 + pl;
+    const int b = (int)(q / oplane), pix = (int)(q % oplane);
+    NhwcRotTap<CT> e;
+#pragma unroll
+    for (int k = 0; k < 4; ++k) e.cell[k] = 0, e.dh[k] = CT(0), e.dw[k] = CT(0);
+    e.src = -1;
+    int opix;
+    long src_pix;
+    const bool hit = tap_pixels<false>(g, pix, t, opix, src_pix);
+    const size_t ri = rot_index_nhwc(g, b, pix, grp, t, 0);
+    bool open_h = true, open_w = true;
+    const CT sh = scope_coord<CT>(g, t / 3, (CT)ld(rot + ri), g.centre_h, &open_h);
+    const CT sw = scope_coord<CT>(g, t % 3, (CT)ld(rot + ri + 1), g.centre_w, &open_w);
+    e.open = (open_h ? 1 : 0) | (open_w ? 2 : 0);
+    if (hit && sh > CT(-1) && sw > CT(-1) && sh < CT(g.scope_h) && sw < CT(g.scope_w)) {
+      const CT hf = floor(sh), wf = floor(sw);
+      const int hl = (int)hf, wl = (int)wf, hi = hl + 1, wi = wl + 1;
+      const CT lh = sh - hf, lw = sw - wf, hh = CT(1) - lh, hw = CT(1) - lw;
+      const bool c00 = hl >= 0 && wl >= 0, c01 = hl >= 0 && wi <= g.scope_w - 1;
+      const bool c10 = hi <= g.scope_h - 1 && wl >= 0, c11 = hi <= g.scope_h - 1 && wi <= g.scope_w - 1;
+      e.cell[0] = c00 ? hl * g.scope_w + wl : 0, e.cell[1] = c01 ? hl * g.scope_w + wi : 0;
+      e.cell[2] = c10 ? hi * g.scope_w + wl : 0, e.cell[3] = c11 ? hi * g.scope_w + wi : 0;
+      e.dh[0] = c00 ? -hw : CT(0), e.dh[1] = c01 ? -lw : CT(0), e.dh[2] = c10 ? hw : CT(0), e.dh[3] = c11 ? lw : CT(0);
+      e.dw[0] = c00 ? -hh : CT(0), e.dw[1] = c01 ? hh : CT(0), e.dw[2] = c10 ? -lh : CT(0), e.dw[3] = c11 ? lh : CT(0);
+      e.src = ((long)b * g.in_h * g.in_w + src_pix) * g.channel;
+    }
+    table[i] = e;
+  }
+  __syncthreads();
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int cpg = g.channel / g.groups;
+  for (int item = wave; item < npix * g.groups; item += kNBlock / 64) {
+    const int grp = item % g.groups, pl = item / g.groups;
+    const long q = q0 + pl;
+    const NhwcRotTap<CT>* row = table + (size_t)item * TAPS;
+    CT ph[TAPS], pw[TAPS];
+#pragma unroll
+    for (int t = 0; t < TAPS; ++t) ph[t] = CT(0), pw[t] = CT(0);
+    for (int j = lane; j < cpg; j += 64) {
+      const int c = grp + g.groups * j;
+      const T graw = gout[(size_t)q * g.channel + c];
+      T xraw[TAPS];
+      bool on[TAPS];
+#pragma unroll
+      for (int t = 0; t < TAPS; ++t) {
+        const long so = row[t].src;
+        on[t] = so >= 0;
+        xraw[t] = x[(on[t] ? so : 0) + c];
+      }
+      const CT gv = (CT)ld(&graw);
+#pragma unroll
+      for (int t = 0; t < TAPS; ++t) {
+        const CT pv = on[t] ? gv * (CT)ld(&xraw[t]) : CT(0);
+        CT fh = CT(0), fw = CT(0);
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+          const CT f = wt[(size_t)row[t].cell[k] * g.channel + c];
+          fh += row[t].dh[k] * f;
+          fw += row[t].dw[k] * f;
+        }
+        ph[t] += pv * fh;
+        pw[t] += pv * fw;
+      }
+    }
+    CT mine = CT(0);
+#pragma unroll
+    for (int t = 0; t < TAPS; ++t) {
+      const CT sh_ = group_sum(ph[t]), sw_ = group_sum(pw[t]);
+      const int open = row[t].open;
+      mine = lane == 2 * t ? ((open & 1) ? sh_ : CT(0)) : mine;
+      mine = lane == 2 * t + 1 ? ((open & 2) ? sw_ : CT(0)) : mine;
+    }
+    if (lane < 2 * TAPS)
+      st(grot + rot_index_nhwc(g, (int)(q / oplane), (int)(q % oplane), grp, 0, 0) + lane, mine);
+  }
+}
+
 // grad filter.  CELLS > 0: the scope's cell count, sums in registers; CELLS == 0: any scope, sums in
 // the thread's own column of LDS.
-template <typename T, int CELLS>
+template <typename T, int CELLS, int TAPS>
 __global__ __launch_bounds__(kNBlock) void nhwc_grad_filter_kernel(Geo g, const T* __restrict__ gout,
                                                                    const T* __restrict__ x,
                                                                    const T* __restrict__ rot,
@@ -289,18 +427,39 @@ __global__ __launch_bounds__(kNBlock) void nhwc_grad_filter_kernel(Geo g, const 
     __syncthreads();
     if (live) {
       for (int pl = 0; pl < npix; ++pl) {
-        const CT gv = (CT)ld(gout + (size_t)(qb + pl) * g.channel + c);
         const int base = (pl * g.groups + grp) * taps;
-        for (int t = 0; t < taps; ++t) {
-          const long s = srcs[base + t];
-          if (s < 0) continue;
-          const CT pv = gv * (CT)ld(x + s + c);
-          const CT* h = hats + (size_t)(base + t) * cells;
-          if constexpr (CELLS > 0) {
+        if constexpr (TAPS > 0 && CELLS > 0) {
+          // the pixel's ten loads first
+          const T graw = gout[(size_t)(qb + pl) * g.channel + c];
+          T xraw[TAPS];
+          bool on[TAPS];
+#pragma unroll
+          for (int t = 0; t < TAPS; ++t) {
+            const long so = srcs[base + t];
+            on[t] = so >= 0;
+            xraw[t] = x[(on[t] ? so : 0) + c];
+          }
+          const CT gv = (CT)ld(&graw);
+#pragma unroll
+          for (int t = 0; t < TAPS; ++t) {
+            const CT pv = on[t] ? gv * (CT)ld(&xraw[t]) : CT(0);
+            const CT* h = hats + (size_t)(base + t) * cells;
 #pragma unroll
             for (int k = 0; k < CELLS; ++k) acc[k] += h[k] * pv;
-          } else {
-            for (int k = 0; k < cells; ++k) col[k * kNBlock + threadIdx.x] += h[k] * pv;
+          }
+        } else {
+          const CT gv = (CT)ld(gout + (size_t)(qb + pl) * g.channel + c);
+          for (int t = 0; t < taps; ++t) {
+            const long so = srcs[base + t];
+            if (so < 0) continue;
+            const CT pv = gv * (CT)ld(x + so + c);
+            const CT* h = hats + (size_t)(base + t) * cells;
+            if constexpr (CELLS > 0) {
+#pragma unroll
+              for (int k = 0; k < CELLS; ++k) acc[k] += h[k] * pv;
+            } else {
+              for (int k = 0; k < cells; ++k) col[k * kNBlock + threadIdx.x] += h[k] * pv;
+            }
           }
         }
       }
@@ -317,9 +476,292 @@ __global__ __launch_bounds__(kNBlock) void nhwc_grad_filter_kernel(Geo g, const 
   }
 }
 
+// ---------------------------------------------------------------------------
+// grad filter and grad rotation on the matrix cores (one rotation group, scopes of up to 32 cells,
+// 16- and 32-bit types).  With k = (pixel, tap) and P[k][c] = out_grad[pixel][c] * input(tap)[c]:
+//   grad filter    gW[cell][c]  = sum_k A[k][cell] * P[k][c]       A: the hat products of (pixel, tap)
+//   grad rotation  R[k][cell]   = sum_c P[k][c] * W[c][cell]       then  grot[k][dir] = sum_cell dA_dir[k][cell] * R[k][cell]
+// Channels-last is the natural layout for both: P's rows are contiguous over c.  Both use
+// v_mfma_f32_16x16x4_f32 (fp32 products and sums): lane l supplies A[l % 16][l / 16] and
+// B[l / 16][l % 16] and holds D[4 * (l / 16) + i][l % 16].  The tables of a batch of pixels (dense
+// rows of A or dA over the cells, source offsets) are written by one thread per row.
+// ---------------------------------------------------------------------------
+typedef float nhwc_f4 __attribute__((ext_vector_type(4)));
+constexpr int kMfRows = 144;  // table rows ((pixel, tap) pairs) per batch; a multiple of 16
+
+struct NhwcRow {
+  unsigned src;   // byte offset of the tap's input pixel (channel 0) in the input tensor
+  unsigned gsrc;  // byte offset of the pixel's out_grad (channel 0)
+};                // a row that contributes nothing has both at kOutOfRange: its buffer loads return zeros
+
+// One element / four consecutive elements at a byte offset of a buffer resource, as stored (converted when used:
+// a conversion next to the load would wait for it).
+template <typename T> struct RawOf { using type = unsigned; };
+template <> struct RawOf<__half> { using type = unsigned short; };
+template <> struct RawOf<bf16_t> { using type = unsigned short; };
+__device__ __forceinline__ unsigned raw_ld(rsrc_t r, unsigned off, const float*) { return __builtin_amdgcn_raw_buffer_load_b32(r, (int)off, 0, 0); }
+__device__ __forceinline__ unsigned short raw_ld(rsrc_t r, unsigned off, const __half*) { return __builtin_amdgcn_raw_buffer_load_b16(r, (int)off, 0, 0); }
+__device__ __forceinline__ unsigned short raw_ld(rsrc_t r, unsigned off, const bf16_t*) { return __builtin_amdgcn_raw_buffer_load_b16(r, (int)off, 0, 0); }
+__device__ __forceinline__ float raw_cvt(unsigned v, const float*) { return __uint_as_float(v); }
+__device__ __forceinline__ float raw_cvt(unsigned short v, const __half*) { return static_cast<float>(__builtin_bit_cast(_Float16, v)); }
+__device__ __forceinline__ float raw_cvt(unsigned short v, const bf16_t*) { return __uint_as_float((unsigned)v << 16); }
+
+typedef unsigned nhwc_u4 __attribute__((ext_vector_type(4)));
+typedef unsigned nhwc_u2 __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ nhwc_u4 raw_ld4(rsrc_t r, unsigned off, const float*) { return __builtin_amdgcn_raw_buffer_load_b128(r, (int)off, 0, 0); }
+__device__ __forceinline__ nhwc_u2 raw_ld4(rsrc_t r, unsigned off, const __half*) { return __builtin_amdgcn_raw_buffer_load_b64(r, (int)off, 0, 0); }
+__device__ __forceinline__ nhwc_u2 raw_ld4(rsrc_t r, unsigned off, const bf16_t*) { return __builtin_amdgcn_raw_buffer_load_b64(r, (int)off, 0, 0); }
+__device__ __forceinline__ void raw_cvt4(nhwc_u4 v, float (&f)[4], const float*) {
+  const unsigned u[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+  for (int i = 0; i < 4; ++i) f[i] = __uint_as_float(u[i]);
+}
+__device__ __forceinline__ void raw_cvt4(nhwc_u2 v, float (&f)[4], const __half*) {
+  const unsigned u[2] = {v.x, v.y};
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    f[2 * i] = static_cast<float>(__builtin_bit_cast(_Float16, (unsigned short)(u[i] & 0xffffu)));
+    f[2 * i + 1] = static_cast<float>(__builtin_bit_cast(_Float16, (unsigned short)(u[i] >> 16)));
+  }
+}
+__device__ __forceinline__ void raw_cvt4(nhwc_u2 v, float (&f)[4], const bf16_t*) {
+  const unsigned u[2] = {v.x, v.y};
+#pragma unroll
+  for (int i = 0; i < 2; ++i) f[2 * i] = __uint_as_float(u[i] << 16), f[2 * i + 1] = __uint_as_float(u[i] & 0xffff0000u);
+}
+
+// Sum over the 16 lanes of a DPP row, in every lane of the row.
+__device__ __forceinline__ float row16_sum(float v) {
+#define DK_DPP_ADD(ctrl) \
+  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), ctrl, 0xf, 0xf, true))
+  DK_DPP_ADD(0xB1);   // quad_perm [1,0,3,2]
+  DK_DPP_ADD(0x4E);   // quad_perm [2,3,0,1]
+  DK_DPP_ADD(0x141);  // row_half_mirror
+  DK_DPP_ADD(0x140);  // row_mirror
+#undef DK_DPP_ADD
+  return v;
+}
+
+// Rows of a batch: row r = (pixel q0 + r / taps, tap r % taps).  Writes the row's offsets and its dense
+// cell rows: MODE 0: hat products (grad filter); MODE 1: d/dh and d/dw of them, zero where the offset is
+// clamped (grad rotation; planar_bilinear_backward_coord, K.cu:116-163).
+template <typename T, int MODE, int NCT>
+__device__ __forceinline__ void nhwc_build_rows(const Geo& g, const T* __restrict__ rot, long q0, int nrows, int rows_padded,
+                                                NhwcRow* rows, float* dense_a, float* dense_b) {
+  constexpr int ROW = 16 * NCT;
+  const int taps = g.k_h * g.k_w, oplane = g.out_h * g.out_w;
+  for (int r = threadIdx.x; r < rows_padded; r += blockDim.x) {
+    // the dense rows start as zeros; the (at most four) corners are then stored over them by the same thread
+#pragma unroll
+    for (int k = 0; k < ROW; k += 4) {
+      *reinterpret_cast<nhwc_f4*>(dense_a + (size_t)r * ROW + k) = nhwc_f4{0.f, 0.f, 0.f, 0.f};
+      if (MODE == 1) *reinterpret_cast<nhwc_f4*>(dense_b + (size_t)r * ROW + k) = nhwc_f4{0.f, 0.f, 0.f, 0.f};
+    }
+    NhwcRow row{kOutOfRange, kOutOfRange};
+    if (r < nrows) {
+      const long q = q0 + r / taps;
+      const int t = r % taps, b = (int)(q / oplane), pix = (int)(q % oplane);
+      int opix;
+      long src_pix;
+      const bool hit = tap_pixels<false>(g, pix, t, opix, src_pix);
+      const size_t ri = rot_index_nhwc(g, b, pix, 0, t, 0);
+      bool open_h = true, open_w = true;
+      const float sh = scope_coord<float>(g, t / g.k_w, (float)ld(rot + ri), g.centre_h, &open_h);
+      const float sw = scope_coord<float>(g, t % g.k_w, (float)ld(rot + ri + 1), g.centre_w, &open_w);
+      if (hit && sh > -1.f && sw > -1.f && sh < (float)g.scope_h && sw < (float)g.scope_w) {
+        row.src = (unsigned)((((long)b * g.in_h * g.in_w + src_pix) * g.channel) * (long)sizeof(T));
+        row.gsrc = (unsigned)(q * g.channel * (long)sizeof(T));
+        const float hf = floorf(sh), wf = floorf(sw);
+        const int hl = (int)hf, wl = (int)wf, hi = hl + 1, wi = wl + 1;
+        const float lh = sh - hf, lw = sw - wf, hh = 1.f - lh, hw = 1.f - lw;
+        const bool cok[4] = {hl >= 0 && wl >= 0, hl >= 0 && wi <= g.scope_w - 1, hi <= g.scope_h - 1 && wl >= 0,
+                             hi <= g.scope_h - 1 && wi <= g.scope_w - 1};
+        const int ci[4] = {hl * g.scope_w + wl, hl * g.scope_w + wi, hi * g.scope_w + wl, hi * g.scope_w + wi};
+        const float w0[4] = {hh * hw, hh * lw, lh * hw, lh * lw};
+        const float dh[4] = {-hw, -lw, hw, lw}, dw[4] = {-hh, hh, -lh, lh};
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront", "local");  // the zeros above go first
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+          if (!cok[k]) continue;
+          if (MODE == 0) dense_a[(size_t)r * ROW + ci[k]] = w0[k];
+          if (MODE == 1) {
+            dense_a[(size_t)r * ROW + ci[k]] = open_h ? dh[k] : 0.f;
+            dense_b[(size_t)r * ROW + ci[k]] = open_w ? dw[k] : 0.f;
+          }
+        }
+      }
+    }
+    rows[r] = row;
+  }
+}
+
+// grad filter: a workgroup owns a range of pixels and up to 16 tiles of 16 channels, one per wave, so the
+// table of a batch is built once for all of them and every tile's loads are in flight together
+constexpr int kMfTiles = 1;
+template <typename T, int NCT>
+__global__ __launch_bounds__(1024) void nhwc_grad_filter_mfma_kernel(Geo g, const T* __restrict__ gout,
+                                                                        const T* __restrict__ x,
+                                                                        const T* __restrict__ rot,
+                                                                        float* __restrict__ partial, int pix_per_block) {
+  constexpr int ROW = 16 * NCT;
+  __shared__ NhwcRow rows[kMfRows];
+  __shared__ __align__(16) float hats[kMfRows * ROW];
+  const int taps = g.k_h * g.k_w, cells = g.scope_h * g.scope_w;
+  const int oplane = g.out_h * g.out_w;
+  const long total_pix = (long)g.batch * oplane;
+  const long q_lo = (long)blockIdx.x * pix_per_block, q_hi = min(total_pix, q_lo + pix_per_block);
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int kg = lane >> 4, n = lane & 15;
+  const int tile0 = blockIdx.y * (blockDim.x >> 6) + wave;  // this wave's tile
+  const rsrc_t rg = plane_rsrc(gout, (int)(total_pix * g.channel)), rx = plane_rsrc(x, g.batch * g.in_h * g.in_w * g.channel);
+  const int pb = kMfRows / taps;                      // pixels per batch (taps <= kMfRows, checked by the host)
+  nhwc_f4 acc[kMfTiles][NCT];
+#pragma unroll
+  for (int j = 0; j < kMfTiles; ++j)
+#pragma unroll
+    for (int t = 0; t < NCT; ++t) acc[j][t] = nhwc_f4{0.f, 0.f, 0.f, 0.f};
+  for (long qb = q_lo; qb < q_hi; qb += pb) {
+    const int nrows = (int)min((long)pb, q_hi - qb) * taps;
+    __syncthreads();
+    nhwc_build_rows<T, 0, NCT>(g, rot, qb, nrows, kMfRows, rows, hats, nullptr);  // rows past nrows: dead, zero hats
+    __syncthreads();
+#pragma unroll
+    for (int j = 0; j < kMfTiles; ++j) {
+      const int c0 = (tile0 + 4 * j) * 16;
+      if (c0 >= g.channel) continue;              // uniform over the wave
+      const int c = min(c0 + n, g.channel - 1);   // columns past the last channel repeat it; they are not stored
+      // half a batch's loads first, then its products (a dead row loads zeros: no select anywhere)
+      constexpr int STEPS = kMfRows / 8;
+      const unsigned cb_ = (unsigned)c * (unsigned)sizeof(T);
+      for (int k0 = 0; 4 * k0 < nrows; k0 += STEPS) {
+        typename RawOf<T>::type graw[STEPS], xraw[STEPS];
+#pragma unroll
+        for (int k = 0; k < STEPS; ++k) {
+          const NhwcRow rw = rows[4 * (k0 + k) + kg];
+          graw[k] = raw_ld(rg, rw.gsrc + cb_, gout);
+          xraw[k] = raw_ld(rx, rw.src + cb_, x);
+        }
+#pragma unroll
+        for (int k = 0; k < STEPS; ++k) {
+          if (4 * (k0 + k) < nrows) {  // uniform over the wave
+            const float pv = raw_cvt(graw[k], gout) * raw_cvt(xraw[k], x);
+#pragma unroll
+            for (int t = 0; t < NCT; ++t)
+              acc[j][t] = __builtin_amdgcn_mfma_f32_16x16x4f32(hats[(size_t)(4 * (k0 + k) + kg) * ROW + t * 16 + n], pv,
+                                                               acc[j][t], 0, 0, 0);
+          }
+        }
+      }
+    }
+  }
+#pragma unroll
+  for (int j = 0; j < kMfTiles; ++j) {
+    const int c0 = (tile0 + 4 * j) * 16;
+    if (c0 + n < g.channel) {
+      float* out = partial + ((size_t)blockIdx.x * g.channel + c0 + n) * cells;
+#pragma unroll
+      for (int t = 0; t < NCT; ++t)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const int cell = t * 16 + 4 * kg + i;
+          if (cell < cells) out[cell] = acc[j][t][i];
+        }
+    }
+  }
+}
+
+// grad rotation: a workgroup takes batches of pixels; a wave takes 16 rows ((pixel, tap) pairs) at a time and
+// walks the channels 16 at a time, each lane loading four consecutive channels of its row.  The filter
+// sits in LDS as [channel][16 * NCT] (zero rows up to a multiple of 16 channels).
+template <typename T, int NCT>
+__global__ __launch_bounds__(kNBlock) void nhwc_grad_rotation_mfma_kernel(Geo g, const T* __restrict__ gout,
+                                                                          const T* __restrict__ x,
+                                                                          const T* __restrict__ rot,
+                                                                          const T* __restrict__ filter,
+                                                                          T* __restrict__ grot, int batches_per_block) {
+  constexpr int ROW = 16 * NCT;
+  extern __shared__ __align__(16) unsigned char nhwc_lds[];
+  __shared__ NhwcRow rows[kMfRows];
+  __shared__ __align__(16) float dah[kMfRows * ROW];
+  __shared__ __align__(16) float daw[kMfRows * ROW];
+  float* wl = reinterpret_cast<float*>(nhwc_lds);  // [channels rounded up to 16][ROW]
+  const int taps = g.k_h * g.k_w, cells = g.scope_h * g.scope_w;
+  const int oplane = g.out_h * g.out_w;
+  const long total_pix = (long)g.batch * oplane;
+  const int cpad = (g.channel + 15) & ~15;
+  for (int i = threadIdx.x; i < cpad * ROW; i += kNBlock) {
+    const int ch = i / ROW, cell = i - ch * ROW;
+    wl[i] = ch < g.channel && cell < cells ? (float)ld(filter + (size_t)ch * cells + cell) : 0.f;
+  }
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int kg = lane >> 4, m = lane & 15;
+  const int pb = kMfRows / taps;
+  const rsrc_t rg = plane_rsrc(gout, (int)(total_pix * g.channel)), rx = plane_rsrc(x, g.batch * g.in_h * g.in_w * g.channel);
+  for (int bi = 0; bi < batches_per_block; ++bi) {
+    const long qb = ((long)blockIdx.x * batches_per_block + bi) * pb;
+    if (qb >= total_pix) break;  // uniform over the workgroup
+    const int nrows = (int)min((long)pb, total_pix - qb) * taps;
+    __syncthreads();
+    nhwc_build_rows<T, 1, NCT>(g, rot, qb, nrows, (nrows + 15) & ~15, rows, dah, daw);
+    __syncthreads();
+    for (int rt = wave * 16; rt < nrows; rt += 64) {
+      const NhwcRow rw = rows[rt + m];  // rows past nrows were written as dead rows
+      nhwc_f4 acc[NCT];
+#pragma unroll
+      for (int t = 0; t < NCT; ++t) acc[t] = nhwc_f4{0.f, 0.f, 0.f, 0.f};
+      for (int cb = 0; cb < cpad; cb += 64) {  // four 16-channel blocks at a time, their loads first
+        decltype(raw_ld4(rg, 0u, gout)) gp[4], xp[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+          // channels past the last one: out of the resource's range for the last row, a neighbour's values for
+          // the others -- multiplied by the filter's zero rows either way
+          const unsigned cc = (unsigned)min(cb + 16 * u + 4 * kg, g.channel - 4) * (unsigned)sizeof(T);
+          gp[u] = raw_ld4(rg, rw.gsrc + cc, gout);
+          xp[u] = raw_ld4(rx, rw.src + cc, x);
+        }
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+          if (cb + 16 * u < cpad) {  // uniform
+            const bool inside = cb + 16 * u + 4 * kg < g.channel;
+            float gv[4], xv[4];
+            raw_cvt4(gp[u], gv, gout);
+            raw_cvt4(xp[u], xv, x);
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+              const float pv = inside ? gv[j] * xv[j] : 0.f;
+              const float* wrow = wl + (size_t)(cb + 16 * u + 4 * kg + j) * ROW + m;
+#pragma unroll
+              for (int t = 0; t < NCT; ++t) acc[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(pv, wrow[t * 16], acc[t], 0, 0, 0);
+            }
+          }
+        }
+      }
+      // lane (kg, m) holds R[row rt + 4 kg + i][cell t * 16 + m]
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int r = rt + 4 * kg + i;
+        float sh_ = 0.f, sw_ = 0.f;
+#pragma unroll
+        for (int t = 0; t < NCT; ++t) {
+          sh_ += dah[(size_t)r * ROW + t * 16 + m] * acc[t][i];
+          sw_ += daw[(size_t)r * ROW + t * 16 + m] * acc[t][i];
+        }
+        sh_ = row16_sum(sh_);
+        sw_ = row16_sum(sw_);
+        if (m == 0 && r < nrows) {
+          const long q = qb + r / taps;
+          const size_t ri = rot_index_nhwc(g, (int)(q / oplane), (int)(q % oplane), 0, r % taps, 0);
+          st(grot + ri, sh_);
+          st(grot + ri + 1, sw_);
+        }
+      }
+    }
+  }
+}
+
 // ---- host side --------------------------------------------------------------------------
 
-constexpr int kFilterPixPerBlock = 512;
+constexpr int kFilterPixPerBlock = 128;
 constexpr int kFilterBatch = 16;  // pixels per table batch of the grad filter
 
 template <typename T>
@@ -362,14 +804,16 @@ void nhwc_gather(const Geo& g, bool transposed, const T* src, const T* rot, cons
   const NhwcLaunch L = gather_launch<T>(g, transposed, lds);
   const dim3 grid((unsigned)(g.batch * L.pblocks), (unsigned)ceil_div(g.channel, L.cc));
   const bool v4 = vec4_ok<T>(g, src, dst) && L.cc % 4 == 0;
-#define DK_NHWC_GATHER(VV, TT) \
-  hipLaunchKernelGGL((nhwc_gather_kernel<T, VV, TT>), grid, dim3(kNBlock), lds, stream, g, L, src, rot, filter, dst)
+  const bool nine = g.k_h * g.k_w == 9;
+#define DK_NHWC_GATHER(VV, TT)                                                                                             \
+  if (nine) hipLaunchKernelGGL((nhwc_gather_kernel<T, VV, TT, 9>), grid, dim3(kNBlock), lds, stream, g, L, src, rot, filter, dst); \
+  else hipLaunchKernelGGL((nhwc_gather_kernel<T, VV, TT, 0>), grid, dim3(kNBlock), lds, stream, g, L, src, rot, filter, dst)
   if (transposed) {
-    if (v4) DK_NHWC_GATHER(4, true);
-    else DK_NHWC_GATHER(1, true);
+    if (v4) { DK_NHWC_GATHER(4, true); }
+    else { DK_NHWC_GATHER(1, true); }
   } else {
-    if (v4) DK_NHWC_GATHER(4, false);
-    else DK_NHWC_GATHER(1, false);
+    if (v4) { DK_NHWC_GATHER(4, false); }
+    else { DK_NHWC_GATHER(1, false); }
   }
 #undef DK_NHWC_GATHER
 }
@@ -378,8 +822,41 @@ template <typename T>
 void nhwc_grad_rotation(const Geo& g, const T* gout, const T* x, const T* rot, const T* filter, T* grot,
                         hipStream_t stream) {
   using CT = compute_t<T>;
+  const int cells_ = g.scope_h * g.scope_w, taps_ = g.k_h * g.k_w;
+  if constexpr (!std::is_same<T, double>::value) {
+    const int nct = (cells_ + 15) / 16;
+    const size_t wl_bytes = (size_t)((g.channel + 15) & ~15) * 16 * nct * sizeof(float);
+    const bool aligned = g.channel % 4 == 0 && reinterpret_cast<uintptr_t>(gout) % (4 * sizeof(T)) == 0 &&
+                         reinterpret_cast<uintptr_t>(x) % (4 * sizeof(T)) == 0;
+    const bool small = (long)g.batch * g.channel * std::max((long)g.in_h * g.in_w, (long)g.out_h * g.out_w) * (long)sizeof(T) < (1L << 31);
+    if (g.groups == 1 && nct <= 2 && taps_ <= kMfRows && aligned && small && wl_bytes <= 96 * 1024 && !path_disabled(kNoNhwcMfma)) {
+      const int pb = kMfRows / taps_;
+      const long batches = ceil_div((long)g.batch * g.out_h * g.out_w, (long)pb);
+      const int per_block = 4;
+      const dim3 grid((unsigned)ceil_div(batches, (long)per_block));
+      if (nct == 1) {
+        if (wl_bytes <= 40 * 1024 || allow_dynamic_lds(reinterpret_cast<const void*>(&nhwc_grad_rotation_mfma_kernel<T, 1>), 96 * 1024))
+          hipLaunchKernelGGL((nhwc_grad_rotation_mfma_kernel<T, 1>), grid, dim3(kNBlock), wl_bytes, stream, g, gout, x, rot,
+                             filter, grot, per_block);
+      } else {
+        if (wl_bytes <= 24 * 1024 || allow_dynamic_lds(reinterpret_cast<const void*>(&nhwc_grad_rotation_mfma_kernel<T, 2>), 96 * 1024))
+          hipLaunchKernelGGL((nhwc_grad_rotation_mfma_kernel<T, 2>), grid, dim3(kNBlock), wl_bytes, stream, g, gout, x, rot,
+                             filter, grot, per_block);
+      }
+      return;
+    }
+  }
   const size_t wt_bytes = (size_t)g.scope_h * g.scope_w * g.channel * sizeof(CT);
   const int in_lds = wt_bytes <= 48 * 1024;
+  if (in_lds && g.k_h == 3 && g.k_w == 3) {
+    const size_t entry = sizeof(NhwcRotTap<CT>) * g.groups * 9;
+    const int pb = (int)std::max<size_t>(1, std::min<size_t>(16, 12 * 1024 / entry));
+    const long total_pix = (long)g.batch * g.out_h * g.out_w;
+    const size_t lds = ((wt_bytes + 15) & ~(size_t)15) + pb * entry;
+    hipLaunchKernelGGL((nhwc_grad_rotation9_kernel<T>), dim3((unsigned)ceil_div(total_pix, (long)pb)), dim3(kNBlock), lds,
+                       stream, g, gout, x, rot, filter, grot, pb);
+    return;
+  }
   const long items = (long)g.batch * g.out_h * g.out_w * g.groups * g.k_h * g.k_w;
   const long blocks = std::min<long>((items + 3) / 4, 256L * 32);
   hipLaunchKernelGGL((nhwc_grad_rotation_kernel<T>), dim3((unsigned)blocks), dim3(kNBlock), in_lds ? wt_bytes : 0, stream,
@@ -404,15 +881,35 @@ void nhwc_grad_filter(const Geo& g, const T* gout, const T* x, const T* rot, T* 
   const int pb = (int)std::max<size_t>(1, std::min<size_t>(kFilterBatch, 40 * 1024 / per_pixel));
   const size_t lds = pb * per_pixel + colb;  // at most 40 KB of table and 100 KB of sums
   CT* partial = static_cast<CT*>(ws);
+  if constexpr (!std::is_same<T, double>::value) {
+    const int nct = (cells + 15) / 16;
+    const bool small = (long)g.batch * g.channel * std::max((long)g.in_h * g.in_w, (long)g.out_h * g.out_w) * (long)sizeof(T) < (1L << 31);
+    if (g.groups == 1 && nct <= 2 && taps <= kMfRows && small && !path_disabled(kNoNhwcMfma)) {
+      const int ntiles = ceil_div(g.channel, 16), wpb = std::min(ntiles, 16);
+      const dim3 mgrid((unsigned)parts, (unsigned)ceil_div(ntiles, wpb));
+      if (nct == 1)
+        hipLaunchKernelGGL((nhwc_grad_filter_mfma_kernel<T, 1>), mgrid, dim3(64 * wpb), 0, stream, g, gout, x, rot, partial,
+                           kFilterPixPerBlock);
+      else
+        hipLaunchKernelGGL((nhwc_grad_filter_mfma_kernel<T, 2>), mgrid, dim3(64 * wpb), 0, stream, g, gout, x, rot, partial,
+                           kFilterPixPerBlock);
+      launch_reduce_partials<CT, T>(partial, parts, (long)g.channel * cells, gfilter, stream);
+      return;
+    }
+  }
   const dim3 grid((unsigned)parts, (unsigned)ceil_div(g.channel, kNBlock));
-#define DK_NHWC_GF(CC)                                                                                                        \
-  if (lds <= 64 * 1024 || allow_dynamic_lds(reinterpret_cast<const void*>(&nhwc_grad_filter_kernel<T, CC>), 144 * 1024))   \
-  hipLaunchKernelGGL((nhwc_grad_filter_kernel<T, CC>), grid, dim3(kNBlock), lds, stream, g, gout, x, rot, partial, kFilterPixPerBlock, pb)
+  const bool nine = taps == 9;
+#define DK_NHWC_GF1(CC, TT)                                                                                                    \
+  if (lds <= 64 * 1024 || allow_dynamic_lds(reinterpret_cast<const void*>(&nhwc_grad_filter_kernel<T, CC, TT>), 144 * 1024))   \
+  hipLaunchKernelGGL((nhwc_grad_filter_kernel<T, CC, TT>), grid, dim3(kNBlock), lds, stream, g, gout, x, rot, partial, kFilterPixPerBlock, pb)
+#define DK_NHWC_GF(CC) \
+  if (nine) { DK_NHWC_GF1(CC, 9); } else { DK_NHWC_GF1(CC, 0); }
   if (cells == 9) { DK_NHWC_GF(9); }
   else if (cells == 16) { DK_NHWC_GF(16); }
   else if (cells == 25) { DK_NHWC_GF(25); }
   else { DK_NHWC_GF(0); }
 #undef DK_NHWC_GF
+#undef DK_NHWC_GF1
   launch_reduce_partials<CT, T>(partial, parts, (long)g.channel * cells, gfilter, stream);
 }
 

@@ -63,6 +63,19 @@ def test_fp32_matches_oracle(case):
     assert rel_err(got[3], o64[3]) < 1e-4
 
 
+@pytest.mark.parametrize("case", CASES[:3] + CASES[4:7] + CASES[9:])
+def test_fp32_without_the_matrix_core_kernels(case, switch_off):
+    """Grad filter and grad rotation of one-group layers run on the matrix cores; with that family
+    switched off the channel-per-thread and wave-per-pixel kernels serve the same shapes."""
+    switch_off("DK_NO_NHWC_MFMA")
+    inputs, got = _run(case, torch.float32, seed=2)
+    o32, o64 = _oracle(inputs, np.float32), _oracle(inputs, np.float64)
+    assert rel_err(got[0], o32[0]) < 1e-5
+    assert rel_err(got[1], o32[1]) < 1e-5
+    assert rel_err(got[2], o64[2]) < 1e-4
+    assert rel_err(got[3], o64[3]) < 1e-4
+
+
 @pytest.mark.parametrize("case", CASES[:4] + CASES[7:8])
 def test_fp64_matches_oracle(case):
     inputs, got = _run(case, torch.float64)
