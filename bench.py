@@ -191,6 +191,8 @@ def main():
     ap.add_argument("--workload", default="cfg2", choices=sorted(WORKLOADS) + sorted(OTHER_WORKLOADS) + sorted(GLOBAL_WORKLOADS) + ["mbv2_dk", "layer_cfg2"])
     ap.add_argument("--batch", type=int, default=64, help="batch size of the mbv2_dk workload")
     ap.add_argument("--dtype", default="fp32", choices=sorted(DTYPES))
+    ap.add_argument("--shape", default="", help="N,C,H,W,stride: a local-operator layer of that shape (3x3 taps, scope 4x4, "
+                    "padding 1) instead of the workload's; for looking at single layers of a network")
     ap.add_argument("--layout", default="nchw", choices=["nchw", "nhwc"],
                     help="memory layout of the tensors of the local-operator workloads (nhwc: the channels-last kernels)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
@@ -224,6 +226,9 @@ def main():
     torch.cuda.set_device(dev)
     tdtype = getattr(torch, DTYPES[a.dtype])
     N, C, H, W, k, S, stride, pad, dil, groups, rot_std = WORKLOADS[a.workload]
+    if a.shape:
+        N, C, H, W, stride = [int(v) for v in a.shape.split(",")]
+        a.workload = "shape %s" % a.shape
     x, wt, rot, gout, cfg = make_local(N, C, H, W, k, S, stride, pad, dil, groups, rot_std, seed=0, dtype=tdtype)
     Ho, Wo = gout.shape[2], gout.shape[3]
     xg, wg, rg, gg = [t.to(dev) for t in (x, wt, rot, gout)]

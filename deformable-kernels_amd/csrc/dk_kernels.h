@@ -30,6 +30,7 @@ enum TestSwitch : unsigned {
   kNoFilterSplit = 1u << 11, // DK_NO_FILTER_SPLIT the bfloat16-pair form of the float32 matrix-core grad filter (fp32 matrix instructions instead)
   kNoNdSmall = 1u << 13,    // DK_NO_ND_SMALL     the few-points-on-a-tiny-volume path of the N-d sampler
   kNoNhwcMfma = 1u << 14,   // DK_NO_NHWC_MFMA    the matrix-core grad filter / grad rotation of the channels-last operator
+  kForceGatherMfma = 1u << 15,  // DK_FORCE_GATHER_MFMA  the matrix-core forward / grad input wherever it applies, not only where it is the faster kernel
   kNoImageFlat = 1u << 12,  // DK_NO_IMAGE_FLAT   the flat-copy kernels of the per-image depthwise convolution (the band kernels run instead)
 };
 unsigned test_switches();  // dk_api.hip

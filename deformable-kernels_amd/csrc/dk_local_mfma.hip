@@ -614,6 +614,11 @@ bool mfma_local_gather(const Geo& g, bool transposed, const T* src, const T* rot
   // their tiles are staged element by element, 2-byte loads into 4-byte slots), so those keep the row kernels
   if (sizeof(T) != 4) return false;
   if ((long)g.in_h * g.in_w >= (1L << 24) || (long)g.out_h * g.out_w >= (1L << 24)) return false;  // byte offsets of 18 rotation planes in 31 bits
+  // A tile's set-up (coordinates, operands) is paid once per tile and its 128 pixels must be filled: the kernel
+  // wins where a plane has many tiles and a group at least six 16-channel blocks (N=64 C=144 56 x 56: 64 against
+  // 68 us), and loses to the row kernels on small planes or few channels (C=960 7 x 7: 73 against 18 us;
+  // C=384 14 x 14: 37 / 21; C=192 28 x 28: 39 / 35; C=32 112 x 112: 121 / 62).
+  if (!path_disabled(kForceGatherMfma) && ((long)g.out_h * g.out_w < 2048 || g.channel / g.groups < 96)) return false;
   if (g.scope_h == 4 && g.scope_w == 4) return run_gather_mfma<T, 4, 4>(g, transposed, src, rot, filter, dst, stream);
   if (g.scope_h == 3 && g.scope_w == 3) return run_gather_mfma<T, 3, 3>(g, transposed, src, rot, filter, dst, stream);
   return false;

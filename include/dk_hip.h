@@ -336,7 +336,7 @@ const char *dk_status_string(int status);
  * family and run the next more general one for the same shape, so that tests can reach every
  * kernel.  Bit i belongs to the i-th of DK_NO_ROWS, DK_NO_MFMA, DK_NO_MFMA_S2, DK_NO_S2_QUADS,
  * DK_NO_DEFORM_FAST, DK_NO_DEFORM_CH, DK_NO_DEFORM_CH_BIG, DK_NO_DEFORM_MFMA, DK_NO_ND_BINS,
- * DK_NO_ND_MFMA, DK_NO_GATHER_MFMA, DK_NO_FILTER_SPLIT, DK_NO_IMAGE_FLAT, DK_NO_ND_SMALL, DK_NO_NHWC_MFMA.  The mask starts from the environment variables of those names, read once
+ * DK_NO_ND_MFMA, DK_NO_GATHER_MFMA, DK_NO_FILTER_SPLIT, DK_NO_IMAGE_FLAT, DK_NO_ND_SMALL, DK_NO_NHWC_MFMA, DK_FORCE_GATHER_MFMA.  The mask starts from the environment variables of those names, read once
  * (at the first call that consults it); this call replaces it and returns the previous mask.
  * Workspace queries consult it too: query and call must see the same mask.  The one piece of
  * process-wide state in the library. */

@@ -86,6 +86,18 @@ def test_fp32_matches_oracle(case):
     assert rel_err(got[3], o64[3]) < 1e-4, "grad filter"
 
 
+@pytest.mark.parametrize("case", [c for c in TUNED if c[6] == 1 and c[7] == 1 and c[8] == 1 and c[5] in ((4, 4), (3, 3))])
+def test_matrix_core_forward_and_grad_input_on_every_same_width_shape(case, switch_off):
+    """The dispatch takes the matrix-core forward / grad input only on large planes with many channels,
+    where it is the faster kernel (the full-size configuration 2 test runs it); forced, it must serve
+    every same-width shape: ragged tiles, few channels, planes smaller than a tile, several groups."""
+    switch_off("DK_FORCE_GATHER_MFMA")
+    inputs, got = _run(case, torch.float32, seed=6)
+    o32 = _oracle(inputs, np.float32)
+    assert rel_err(got[0], o32[0]) < 1e-5, "forward"
+    assert rel_err(got[1], o32[1]) < 1e-5, "grad input"
+
+
 @pytest.mark.parametrize("case", TUNED[:4] + GENERIC[:2])
 def test_fp64_matches_oracle(case):
     inputs, got = _run(case, torch.float64)
