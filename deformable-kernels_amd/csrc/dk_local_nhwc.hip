@@ -78,8 +78,11 @@ __device__ __forceinline__ bool tap_pixels(const Geo& g, int pix, int t, int& op
   }
 }
 
+// cell_pitch: what a cell index is multiplied with in the entry (the gather kernels store the cell's
+// offset in their [cell][channel chunk] copy of the filter, so that no lane multiplies)
 template <typename T, typename CT, bool TRANSPOSED>
-__device__ __forceinline__ NhwcTap<CT> make_tap(const Geo& g, const T* __restrict__ rot, int b, int pix, int grp, int t) {
+__device__ __forceinline__ NhwcTap<CT> make_tap(const Geo& g, const T* __restrict__ rot, int b, int pix, int grp, int t,
+                                                int cell_pitch = 1) {
   NhwcTap<CT> e;
   int opix = 0;
   long src_pix = 0;
@@ -92,6 +95,8 @@ __device__ __forceinline__ NhwcTap<CT> make_tap(const Geo& g, const T* __restric
     const CT sh = scope_coord<CT>(g, t / g.k_w, (CT)ld(rot + ri), g.centre_h);
     const CT sw = scope_coord<CT>(g, t % g.k_w, (CT)ld(rot + ri + 1), g.centre_w);
     scope_corners<CT>(g, sh, sw, e.cell, e.w);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) e.cell[i] *= cell_pitch;
     const long plane = TRANSPOSED ? (long)g.out_h * g.out_w : (long)g.in_h * g.in_w;
     e.src = ((long)b * plane + src_pix) * g.channel;
   }
@@ -130,12 +135,13 @@ __global__ __launch_bounds__(kNBlock) void nhwc_gather_kernel(Geo g, NhwcLaunch 
   const int entries = npix * g.groups * taps;
   for (int i = threadIdx.x; i < entries; i += kNBlock) {
     const int t = i % taps, grp = i / taps % g.groups, pl = i / taps / g.groups;
-    table[i] = make_tap<T, CT, TRANSPOSED>(g, rot, b, p0 + pl, grp, t);
+    table[i] = make_tap<T, CT, TRANSPOSED>(g, rot, b, p0 + pl, grp, t, L.cc);
   }
   __syncthreads();
   const int ccv = (cc + VEC - 1) / VEC;
+  const unsigned ccv_magic = 0xffffffffu / (unsigned)ccv + 1u;  // i / ccv for i < 2^16 (a workgroup has at most 32 * 256 items)
   for (int i = threadIdx.x; i < npix * ccv; i += kNBlock) {
-    const int pl = i / ccv, cl = (i - pl * ccv) * VEC;
+    const int pl = (int)__umulhi((unsigned)i, ccv_magic), cl = (i - pl * ccv) * VEC;
     const int c = c0 + cl;
     CT acc[VEC];
 #pragma unroll
@@ -161,7 +167,7 @@ __global__ __launch_bounds__(kNBlock) void nhwc_gather_kernel(Geo g, NhwcLaunch 
         // the lane's VEC channels of a cell in one LDS read (a read per channel has the lanes VEC banks apart)
         WVec f[4];
 #pragma unroll
-        for (int k = 0; k < 4; ++k) f[k] = *reinterpret_cast<const WVec*>(wt + cell[k] * L.cc + cl);
+        for (int k = 0; k < 4; ++k) f[k] = *reinterpret_cast<const WVec*>(wt + cell[k] + cl);
 #pragma unroll
         for (int v = 0; v < VEC; ++v) {
           CT wv = CT(0);
@@ -178,7 +184,7 @@ __global__ __launch_bounds__(kNBlock) void nhwc_gather_kernel(Geo g, NhwcLaunch 
         const Pack pk = *reinterpret_cast<const Pack*>(src + e.src + c);
         WVec f[4];
 #pragma unroll
-        for (int k = 0; k < 4; ++k) f[k] = *reinterpret_cast<const WVec*>(wt + e.cell[k] * L.cc + cl);
+        for (int k = 0; k < 4; ++k) f[k] = *reinterpret_cast<const WVec*>(wt + e.cell[k] + cl);
 #pragma unroll
         for (int v = 0; v < VEC; ++v) {
           CT wv = CT(0);
@@ -492,6 +498,8 @@ constexpr int kMfRows = 144;  // table rows ((pixel, tap) pairs) per batch; a mu
 struct NhwcRow {
   unsigned src;   // byte offset of the tap's input pixel (channel 0) in the input tensor
   unsigned gsrc;  // byte offset of the pixel's out_grad (channel 0)
+  unsigned rix;   // element index of the row's h entry in the rotation tensor (the w entry follows)
+  unsigned pad_;
 };                // a row that contributes nothing has both at kOutOfRange: its buffer loads return zeros
 
 // One element / four consecutive elements at a byte offset of a buffer resource, as stored (converted when used:
@@ -557,7 +565,7 @@ __device__ __forceinline__ void nhwc_build_rows(const Geo& g, const T* __restric
       *reinterpret_cast<nhwc_f4*>(dense_a + (size_t)r * ROW + k) = nhwc_f4{0.f, 0.f, 0.f, 0.f};
       if (MODE == 1) *reinterpret_cast<nhwc_f4*>(dense_b + (size_t)r * ROW + k) = nhwc_f4{0.f, 0.f, 0.f, 0.f};
     }
-    NhwcRow row{kOutOfRange, kOutOfRange};
+    NhwcRow row{kOutOfRange, kOutOfRange, 0u, 0u};
     if (r < nrows) {
       const long q = q0 + r / taps;
       const int t = r % taps, b = (int)(q / oplane), pix = (int)(q % oplane);
@@ -565,6 +573,7 @@ __device__ __forceinline__ void nhwc_build_rows(const Geo& g, const T* __restric
       long src_pix;
       const bool hit = tap_pixels<false>(g, pix, t, opix, src_pix);
       const size_t ri = rot_index_nhwc(g, b, pix, 0, t, 0);
+      row.rix = (unsigned)ri;
       bool open_h = true, open_w = true;
       const float sh = scope_coord<float>(g, t / g.k_w, (float)ld(rot + ri), g.centre_h, &open_h);
       const float sw = scope_coord<float>(g, t % g.k_w, (float)ld(rot + ri + 1), g.centre_w, &open_w);
@@ -631,7 +640,7 @@ __global__ __launch_bounds__(1024) void nhwc_grad_filter_mfma_kernel(Geo g, cons
       if (c0 >= g.channel) continue;              // uniform over the wave
       const int c = min(c0 + n, g.channel - 1);   // columns past the last channel repeat it; they are not stored
       // half a batch's loads first, then its products (a dead row loads zeros: no select anywhere)
-      constexpr int STEPS = kMfRows / 8;
+      constexpr int STEPS = kMfRows / 8;  // (the whole batch at once needs 126 registers and is slower: 268 against 189 us)
       const unsigned cb_ = (unsigned)c * (unsigned)sizeof(T);
       for (int k0 = 0; 4 * k0 < nrows; k0 += STEPS) {
         typename RawOf<T>::type graw[STEPS], xraw[STEPS];
@@ -684,13 +693,16 @@ __global__ __launch_bounds__(kNBlock) void nhwc_grad_rotation_mfma_kernel(Geo g,
   __shared__ NhwcRow rows[kMfRows];
   __shared__ __align__(16) float dah[kMfRows * ROW];
   __shared__ __align__(16) float daw[kMfRows * ROW];
-  float* wl = reinterpret_cast<float*>(nhwc_lds);  // [channels rounded up to 16][ROW]
+  // filter rows 4 floats apart from a multiple of 16: lane (kg, m) reads row 4 kg + j at column m, and
+  // 4 * WROW = 16 mod 64 puts the four kg groups on four different sets of 16 banks
+  constexpr int WROW = ROW + 4;
+  float* wl = reinterpret_cast<float*>(nhwc_lds);  // [channels rounded up to 16][WROW]
   const int taps = g.k_h * g.k_w, cells = g.scope_h * g.scope_w;
   const int oplane = g.out_h * g.out_w;
   const long total_pix = (long)g.batch * oplane;
   const int cpad = (g.channel + 15) & ~15;
-  for (int i = threadIdx.x; i < cpad * ROW; i += kNBlock) {
-    const int ch = i / ROW, cell = i - ch * ROW;
+  for (int i = threadIdx.x; i < cpad * WROW; i += kNBlock) {
+    const int ch = i / WROW, cell = i - ch * WROW;
     wl[i] = ch < g.channel && cell < cells ? (float)ld(filter + (size_t)ch * cells + cell) : 0.f;
   }
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -709,7 +721,9 @@ __global__ __launch_bounds__(kNBlock) void nhwc_grad_rotation_mfma_kernel(Geo g,
       nhwc_f4 acc[NCT];
 #pragma unroll
       for (int t = 0; t < NCT; ++t) acc[t] = nhwc_f4{0.f, 0.f, 0.f, 0.f};
+      const float* wlane = wl + 4 * kg * WROW + m;
       for (int cb = 0; cb < cpad; cb += 64) {  // four 16-channel blocks at a time, their loads first
+        const float* wcb = wlane + cb * WROW;
         decltype(raw_ld4(rg, 0u, gout)) gp[4], xp[4];
 #pragma unroll
         for (int u = 0; u < 4; ++u) {
@@ -722,16 +736,16 @@ __global__ __launch_bounds__(kNBlock) void nhwc_grad_rotation_mfma_kernel(Geo g,
 #pragma unroll
         for (int u = 0; u < 4; ++u) {
           if (cb + 16 * u < cpad) {  // uniform
-            const bool inside = cb + 16 * u + 4 * kg < g.channel;
+            const bool inside = cpad == g.channel || cb + 16 * u + 4 * kg < g.channel;
             float gv[4], xv[4];
             raw_cvt4(gp[u], gv, gout);
             raw_cvt4(xp[u], xv, x);
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
               const float pv = inside ? gv[j] * xv[j] : 0.f;
-              const float* wrow = wl + (size_t)(cb + 16 * u + 4 * kg + j) * ROW + m;
 #pragma unroll
-              for (int t = 0; t < NCT; ++t) acc[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(pv, wrow[t * 16], acc[t], 0, 0, 0);
+              for (int t = 0; t < NCT; ++t)
+                acc[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(pv, wcb[(16 * u + j) * WROW + t * 16], acc[t], 0, 0, 0);
             }
           }
         }
@@ -749,8 +763,7 @@ __global__ __launch_bounds__(kNBlock) void nhwc_grad_rotation_mfma_kernel(Geo g,
         sh_ = row16_sum(sh_);
         sw_ = row16_sum(sw_);
         if (m == 0 && r < nrows) {
-          const long q = qb + r / taps;
-          const size_t ri = rot_index_nhwc(g, (int)(q / oplane), (int)(q % oplane), 0, r % taps, 0);
+          const unsigned ri = rows[r].rix;
           st(grot + ri, sh_);
           st(grot + ri + 1, sw_);
         }
@@ -825,7 +838,7 @@ void nhwc_grad_rotation(const Geo& g, const T* gout, const T* x, const T* rot, c
   const int cells_ = g.scope_h * g.scope_w, taps_ = g.k_h * g.k_w;
   if constexpr (!std::is_same<T, double>::value) {
     const int nct = (cells_ + 15) / 16;
-    const size_t wl_bytes = (size_t)((g.channel + 15) & ~15) * 16 * nct * sizeof(float);
+    const size_t wl_bytes = (size_t)((g.channel + 15) & ~15) * (16 * nct + 4) * sizeof(float);
     const bool aligned = g.channel % 4 == 0 && reinterpret_cast<uintptr_t>(gout) % (4 * sizeof(T)) == 0 &&
                          reinterpret_cast<uintptr_t>(x) % (4 * sizeof(T)) == 0;
     const bool small = (long)g.batch * g.channel * std::max((long)g.in_h * g.in_w, (long)g.out_h * g.out_w) * (long)sizeof(T) < (1L << 31);
