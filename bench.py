@@ -47,6 +47,8 @@ OTHER_WORKLOADS = {
     "cfg4": ("deform", (64, 512, 28, 28, 3, (4, 4), 2, 1, 1, 1, 0.5, 2.0)),
     # the deformable variant on the headline layer's shape (3136 output pixels per plane)
     "deform_56": ("deform", (64, 144, 56, 56, 3, (4, 4), 1, 1, 1, 1, 0.5, 2.0)),
+    # the deformable variant on MobileNetV2's first depthwise stage (112 x 112 planes: wider than 64 columns)
+    "deform_112": ("deform", (64, 32, 112, 112, 3, (4, 4), 1, 1, 1, 1, 0.5, 2.0)),
     # DeformConv2d (scope = kernel, no rotation tensor: rot_std None) on configuration 4's geometry
     "deform_conv_28": ("deform", (64, 512, 28, 28, 3, (3, 3), 2, 1, 1, 1, None, 2.0)),
     # N-d sampler: data shape [C, s...], points, coordinate range

@@ -52,7 +52,8 @@ struct ScopeCoord {
 
 template <typename T>
 __device__ __forceinline__ void deform_taps(const Geo& g, const T* off, const T* rot, int n, int grp, int p,
-                                            bool live, int RS, ImgTap (&it)[K9], ScopeCoord (&sc)[K9]) {
+                                            bool live, int RS, ImgTap (&it)[K9], ScopeCoord (&sc)[K9],
+                                            unsigned* hits = nullptr) {
   const int out_plane = g.out_h * g.out_w;
   const int pc = live ? p : 0;
   const int oh = pc / g.out_w, ow = pc % g.out_w;
@@ -77,14 +78,16 @@ __device__ __forceinline__ void deform_taps(const Geo& g, const T* off, const T*
     const float sw = scope_coord<float>(g, f_w, buf_ld(rr, o + step, rot), g.centre_w);
     sc[t].h = hit ? sh : -2.f;
     sc[t].w = hit ? sw : -2.f;
+    if (hits) *hits |= hit ? (1u << t) : 0u;  // bit t: tap t samples the image
   }
 }
 
 template <typename T, int SH, int SW>
 __device__ __forceinline__ void deform_taps(const Geo& g, const T* off, const T* rot, int n, int grp, int p,
-                                            bool live, int RS, ImgTap (&it)[K9], LiteTap (&st)[K9]) {
+                                            bool live, int RS, ImgTap (&it)[K9], LiteTap (&st)[K9],
+                                            unsigned* hits = nullptr) {
   ScopeCoord sc[K9];
-  deform_taps<T>(g, off, rot, n, grp, p, live, RS, it, sc);
+  deform_taps<T>(g, off, rot, n, grp, p, live, RS, it, sc, hits);
 #pragma unroll
   for (int t = 0; t < K9; ++t) st[t] = make_lite_tap<SH, SW>(sc[t].h, sc[t].w, true);
 }
@@ -109,30 +112,79 @@ __device__ __forceinline__ float lerp2(const Corners& q, float lh, float lw) {
 // Cooperative load of one H x W plane into the padded LDS layout.  A row takes 2^shift lanes
 // (the smallest power of two >= W), so a thread's (row, column) needs no division; NPASS passes
 // of blockDim / 2^shift rows cover the plane.  load() fills the register stage, store() writes it.
+// WINDOW: only the plane rows row0 .. row0 + nrows - 1 are staged, in as many passes as they take
+// (the LDS layout stays that of the whole plane: rows outside the window keep what they held).
+struct RowWindow {
+  int row0, nrows;
+};
 template <typename T, int NPASS>
 struct PlaneStage {
   float v[NPASS];
-  __device__ __forceinline__ void load(const T* plane, bool on, int H, int W, int shift) {
+  template <bool WINDOW = false>
+  __device__ __forceinline__ void load(const T* plane, bool on, int H, int W, int shift, RowWindow rw = RowWindow{0, 0}) {
     const int col = threadIdx.x & ((1 << shift) - 1), sub = threadIdx.x >> shift;
     const int rpp = (int)blockDim.x >> shift;
     const rsrc_t r = plane_rsrc(plane, on ? H * W : 0);
 #pragma unroll
     for (int k = 0; k < NPASS; ++k) {
       const int row = k * rpp + sub;
-      v[k] = buf_ld(r, (col < W && row < H) ? (unsigned)(row * W + col) * (unsigned)sizeof(T) : kOutOfRange, plane);
+      if constexpr (WINDOW) {
+        if (k * rpp < rw.nrows)  // uniform
+          v[k] = buf_ld(r, (col < W && row < rw.nrows) ? (unsigned)((rw.row0 + row) * W + col) * (unsigned)sizeof(T) : kOutOfRange, plane);
+      } else {
+        v[k] = buf_ld(r, (col < W && row < H) ? (unsigned)(row * W + col) * (unsigned)sizeof(T) : kOutOfRange, plane);
+      }
     }
   }
-  __device__ __forceinline__ void store(float* lds_plane, int H, int W, int shift) const {
+  template <bool WINDOW = false>
+  __device__ __forceinline__ void store(float* lds_plane, int H, int W, int shift, RowWindow rw = RowWindow{0, 0}) const {
     const int col = threadIdx.x & ((1 << shift) - 1), sub = threadIdx.x >> shift;
     const int rpp = (int)blockDim.x >> shift;
     const int RS = W + 2;
 #pragma unroll
     for (int k = 0; k < NPASS; ++k) {
       const int row = k * rpp + sub;
-      if (col < W && row < H) lds_plane[(row + 1) * RS + 1 + col] = v[k];
+      if constexpr (WINDOW) {
+        if (k * rpp < rw.nrows)
+          if (col < W && row < rw.nrows) lds_plane[(rw.row0 + row + 1) * RS + 1 + col] = v[k];
+      } else {
+        if (col < W && row < H) lds_plane[(row + 1) * RS + 1 + col] = v[k];
+      }
     }
   }
 };
+
+// The rows of the input plane that the workgroup's samples read: the taps' descriptors point at
+// the top-left corner in the padded plane (row r of the plane is padded row r + 1), a sample reads
+// that padded row and the next.  Two barriers; every thread of the workgroup must call it.
+__device__ __forceinline__ RowWindow sample_rows(const ImgTap (&it)[K9], unsigned hits, int RS, int H) {
+  __shared__ int s_lo[16], s_hi[16];
+  int lo = H + 2, hi = -1;  // padded rows
+#pragma unroll
+  for (int t = 0; t < K9; ++t) {
+    if (hits >> t & 1u) {
+      const int pr = it[t].pidx / RS;
+      lo = min(lo, pr);
+      hi = max(hi, pr + 1);
+    }
+  }
+  for (int s = 32; s > 0; s >>= 1) {
+    lo = min(lo, __shfl_xor(lo, s));
+    hi = max(hi, __shfl_xor(hi, s));
+  }
+  if ((threadIdx.x & 63) == 0) {
+    s_lo[threadIdx.x >> 6] = lo;
+    s_hi[threadIdx.x >> 6] = hi;
+  }
+  __syncthreads();
+  for (int w = 0; w < (int)blockDim.x / 64; ++w) {
+    lo = min(lo, s_lo[w]);
+    hi = max(hi, s_hi[w]);
+  }
+  __syncthreads();
+  const int first = max(lo - 1, 0), last = min(hi - 1, H - 1);
+  return RowWindow{first, max(last - first + 1, 0)};
+}
 
 // logical block = (pixel tile, channel chunk, image * group), tile fastest (see logical_block())
 struct BlockId {
@@ -155,8 +207,10 @@ __device__ __forceinline__ BlockId decode_block(const Geo& g, int tiles, int chu
 // ---------------------------------------------------------------------------
 // forward: out[n, c, p] = sum_t sample(x[n, c], h_t, w_t) * B(Wt[c], sh_t, sw_t)
 // ---------------------------------------------------------------------------
-template <typename T, int SH, int SW, int NPASS>
-__global__ __launch_bounds__(kDBlock, 2) void deform_forward_kernel(
+// BLOCK > kDBlock: the form for planes that the others do not take (wider than 64 columns, or taller than their
+// staging passes cover): one workgroup per CU, and only the plane rows that the tile's samples touch are staged.
+template <typename T, int SH, int SW, int NPASS, int BLOCK = kDBlock>
+__global__ __launch_bounds__(BLOCK, 2) void deform_forward_kernel(
     Geo g, const T* __restrict__ x, const T* __restrict__ off, const T* __restrict__ rot,
     const T* __restrict__ filter, T* __restrict__ out, int ch_per_block, int shift) {
   using Tb = WideTable<SH, SW>;
@@ -168,19 +222,23 @@ __global__ __launch_bounds__(kDBlock, 2) void deform_forward_kernel(
 
   const int cpg = g.channel / g.groups;
   const int out_plane = g.out_h * g.out_w, in_plane = H * W;
-  const BlockId b = decode_block(g, ceil_div(out_plane, kDBlock), ceil_div(cpg, ch_per_block));
+  const BlockId b = decode_block(g, ceil_div(out_plane, BLOCK), ceil_div(cpg, ch_per_block));
   if (!b.valid) return;
   const int j0 = b.chunk * ch_per_block;
   const int nch = min(ch_per_block, cpg - j0);
 
-  for (int e = threadIdx.x; e < 2 * PS; e += kDBlock) planes[e] = 0.f;
+  for (int e = threadIdx.x; e < 2 * PS; e += BLOCK) planes[e] = 0.f;
   stage_wide_tables<T, SH, SW>(tbl, filter, g.channel, b.grp + g.groups * j0, g.groups, nch);
 
-  const int p = b.tile * kDBlock + threadIdx.x;
+  const int p = b.tile * BLOCK + threadIdx.x;
   const bool live = p < out_plane;
   ImgTap it[K9];
   LiteTap st[K9];
-  deform_taps<T, SH, SW>(g, off, rot, b.n, b.grp, p, live, RS, it, st);
+  constexpr bool WINDOW = BLOCK != kDBlock;
+  unsigned hits = 0;
+  deform_taps<T, SH, SW>(g, off, rot, b.n, b.grp, p, live, RS, it, st, &hits);
+  RowWindow rw{0, H};
+  if constexpr (WINDOW) rw = sample_rows(it, hits, RS, H);
 
   const size_t chan0 = (size_t)b.n * g.channel + b.grp + (size_t)g.groups * j0;
   const T* xp = x + chan0 * in_plane;
@@ -189,12 +247,12 @@ __global__ __launch_bounds__(kDBlock, 2) void deform_forward_kernel(
   const unsigned ooff = live ? (unsigned)p * (unsigned)sizeof(T) : kOutOfRange;
 
   PlaneStage<T, NPASS> stage;
-  stage.load(xp, true, H, W, shift);
+  stage.template load<WINDOW>(xp, true, H, W, shift, rw);
   __syncthreads();  // the zero fill is done
-  stage.store(planes, H, W, shift);
+  stage.template store<WINDOW>(planes, H, W, shift, rw);
   __syncthreads();
   for (int j = 0; j < nch; ++j) {
-    if (j + 1 < nch) stage.load(xp + (size_t)(j + 1) * x_step, true, H, W, shift);
+    if (j + 1 < nch) stage.template load<WINDOW>(xp + (size_t)(j + 1) * x_step, true, H, W, shift, rw);
     const float* pl = planes + (j & 1) * PS;
     const float* tb = tbl + j * Tb::SIZE;
     float acc = 0.f;
@@ -205,7 +263,7 @@ __global__ __launch_bounds__(kDBlock, 2) void deform_forward_kernel(
       acc = fmaf(v, lite_weight(st[t], q), acc);
     }
     buf_st(plane_rsrc(op + (size_t)j * o_step, out_plane), ooff, acc, out);
-    if (j + 1 < nch) stage.store(planes + ((j + 1) & 1) * PS, H, W, shift);
+    if (j + 1 < nch) stage.template store<WINDOW>(planes + ((j + 1) & 1) * PS, H, W, shift, rw);
     __syncthreads();
   }
 }
@@ -359,8 +417,8 @@ __global__ __launch_bounds__(BLOCK, BLOCK == kDBlock ? 2 : 1) void deform_forwar
 // partial layout: [part][image (* group for rotation)][2 t + dir][pixel], part = chunk for
 // rotation and group * chunks + chunk for offset (which sums over the groups as well).
 // ---------------------------------------------------------------------------
-template <typename T, int SH, int SW, int NPASS, bool ROTATION>
-__global__ __launch_bounds__(kDBlock, 2) void deform_grad_coord_kernel(
+template <typename T, int SH, int SW, int NPASS, bool ROTATION, int BLOCK = kDBlock>
+__global__ __launch_bounds__(BLOCK, 2) void deform_grad_coord_kernel(
     Geo g, const T* __restrict__ gout, const T* __restrict__ x, const T* __restrict__ off,
     const T* __restrict__ rot, const T* __restrict__ filter, float* __restrict__ partial,
     int ch_per_block, int shift) {
@@ -374,19 +432,23 @@ __global__ __launch_bounds__(kDBlock, 2) void deform_grad_coord_kernel(
   const int cpg = g.channel / g.groups;
   const int out_plane = g.out_h * g.out_w, in_plane = H * W;
   const int chunks = ceil_div(cpg, ch_per_block);
-  const BlockId b = decode_block(g, ceil_div(out_plane, kDBlock), chunks);
+  const BlockId b = decode_block(g, ceil_div(out_plane, BLOCK), chunks);
   if (!b.valid) return;
   const int j0 = b.chunk * ch_per_block;
   const int nch = min(ch_per_block, cpg - j0);
 
-  for (int e = threadIdx.x; e < 2 * PS; e += kDBlock) planes[e] = 0.f;
+  for (int e = threadIdx.x; e < 2 * PS; e += BLOCK) planes[e] = 0.f;
   stage_wide_tables<T, SH, SW>(tbl, filter, g.channel, b.grp + g.groups * j0, g.groups, nch);
 
-  const int p = b.tile * kDBlock + threadIdx.x;
+  const int p = b.tile * BLOCK + threadIdx.x;
   const bool live = p < out_plane;
   ImgTap it[K9];
   LiteTap st[K9];
-  deform_taps<T, SH, SW>(g, off, rot, b.n, b.grp, p, live, RS, it, st);
+  constexpr bool WINDOW = BLOCK != kDBlock;
+  unsigned hits = 0;
+  deform_taps<T, SH, SW>(g, off, rot, b.n, b.grp, p, live, RS, it, st, &hits);
+  RowWindow rw{0, H};
+  if constexpr (WINDOW) rw = sample_rows(it, hits, RS, H);
 
   const size_t chan0 = (size_t)b.n * g.channel + b.grp + (size_t)g.groups * j0;
   const T* xp = x + chan0 * in_plane;
@@ -399,15 +461,15 @@ __global__ __launch_bounds__(kDBlock, 2) void deform_grad_coord_kernel(
   for (int t = 0; t < K9; ++t) s0[t] = s1[t] = s2[t] = 0.f;
 
   PlaneStage<T, NPASS> stage;
-  stage.load(xp, true, H, W, shift);
+  stage.template load<WINDOW>(xp, true, H, W, shift, rw);
   float gv = buf_ld(plane_rsrc(gp, out_plane), goff, gout);
   __syncthreads();
-  stage.store(planes, H, W, shift);
+  stage.template store<WINDOW>(planes, H, W, shift, rw);
   __syncthreads();
   for (int j = 0; j < nch; ++j) {
     float gv_next = 0.f;
     if (j + 1 < nch) {
-      stage.load(xp + (size_t)(j + 1) * x_step, true, H, W, shift);
+      stage.template load<WINDOW>(xp + (size_t)(j + 1) * x_step, true, H, W, shift, rw);
       gv_next = buf_ld(plane_rsrc(gp + (size_t)(j + 1) * g_step, out_plane), goff, gout);
     }
     const float* pl = planes + (j & 1) * PS;
@@ -432,7 +494,7 @@ __global__ __launch_bounds__(kDBlock, 2) void deform_grad_coord_kernel(
       }
     }
     gv = gv_next;
-    if (j + 1 < nch) stage.store(planes + ((j + 1) & 1) * PS, H, W, shift);
+    if (j + 1 < nch) stage.template store<WINDOW>(planes + ((j + 1) & 1) * PS, H, W, shift, rw);
     __syncthreads();
   }
 
@@ -868,9 +930,7 @@ __global__ __launch_bounds__(1024) void deform_grad_input_kernel(
 // descriptors once and adds the tile's contributions for each of its channels.  The planes are
 // read back once at the end.  grid = (channel chunks of kTiledCh, image * group)
 // ---------------------------------------------------------------------------
-constexpr int kTiledCh = 4;
-
-template <typename T, int SH, int SW>
+template <typename T, int SH, int SW, int kTiledCh>
 __global__ __launch_bounds__(1024) void deform_grad_input_tiled_kernel(
     Geo g, const T* __restrict__ gout, const T* __restrict__ off, const T* __restrict__ rot,
     const T* __restrict__ filter, T* __restrict__ gin, const unsigned* __restrict__ gmax_bits, int shift) {
@@ -971,12 +1031,13 @@ __global__ __launch_bounds__(1024) void deform_grad_input_tiled_kernel(
 // wave reductions and lane `cell` adds the wave's total to a per-wave LDS accumulator.  One
 // partial per (image, tile) workgroup; reduce_partials_kernel adds them in order.
 // ---------------------------------------------------------------------------
-template <typename T, int SH, int SW, int NPASS>
-__global__ __launch_bounds__(kDBlock, 2) void deform_grad_filter_kernel(
+template <typename T, int SH, int SW, int NPASS, int BLOCK = kDBlock>
+__global__ __launch_bounds__(BLOCK, 2) void deform_grad_filter_kernel(
     Geo g, const T* __restrict__ gout, const T* __restrict__ x, const T* __restrict__ off,
     const T* __restrict__ rot, float* __restrict__ partial, int ch_per_block, int shift) {
   constexpr int CELLS = SH * SW;
-  constexpr int kWaves = kDBlock / 64;
+  constexpr int kWaves = BLOCK / 64;
+  constexpr bool WINDOW = BLOCK != kDBlock;
   extern __shared__ __align__(16) float lds[];
   const int H = g.in_h, W = g.in_w, RS = W + 2;
   const int PS = ((H + 2) * RS + 3) & ~3;
@@ -985,23 +1046,24 @@ __global__ __launch_bounds__(kDBlock, 2) void deform_grad_filter_kernel(
 
   const int cpg = g.channel / g.groups;
   const int out_plane = g.out_h * g.out_w, in_plane = H * W;
-  const int tiles = ceil_div(out_plane, kDBlock);
+  const int tiles = ceil_div(out_plane, BLOCK);
   const BlockId b = decode_block(g, tiles, ceil_div(cpg, ch_per_block));
   if (!b.valid) return;
   const int j0 = b.chunk * ch_per_block;
   const int nch = min(ch_per_block, cpg - j0);
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
 
-  for (int e = threadIdx.x; e < 2 * PS; e += kDBlock) planes[e] = 0.f;
-  for (int e = threadIdx.x; e < kWaves * ch_per_block * CELLS; e += kDBlock) wacc[e] = 0.f;
+  for (int e = threadIdx.x; e < 2 * PS; e += BLOCK) planes[e] = 0.f;
+  for (int e = threadIdx.x; e < kWaves * ch_per_block * CELLS; e += BLOCK) wacc[e] = 0.f;
 
-  const int p = b.tile * kDBlock + threadIdx.x;
+  const int p = b.tile * BLOCK + threadIdx.x;
   const bool live = p < out_plane;
   ImgTap it[K9];
   float ah[K9][SH], bw[K9][SW];
+  unsigned hits = 0;
   {
     ScopeCoord sc[K9];
-    deform_taps<T>(g, off, rot, b.n, b.grp, p, live, RS, it, sc);
+    deform_taps<T>(g, off, rot, b.n, b.grp, p, live, RS, it, sc, &hits);
 #pragma unroll
     for (int t = 0; t < K9; ++t) {
       // outside the open box (-1, S) every hat below is 0 by itself, NaN coordinates excepted
@@ -1019,16 +1081,18 @@ __global__ __launch_bounds__(kDBlock, 2) void deform_grad_filter_kernel(
   const size_t x_step = (size_t)g.groups * in_plane, g_step = (size_t)g.groups * out_plane;
   const unsigned goff = live ? (unsigned)p * (unsigned)sizeof(T) : kOutOfRange;
 
+  RowWindow rw{0, H};
+  if constexpr (WINDOW) rw = sample_rows(it, hits, RS, H);
   PlaneStage<T, NPASS> stage;
-  stage.load(xp, true, H, W, shift);
+  stage.template load<WINDOW>(xp, true, H, W, shift, rw);
   float gv = buf_ld(plane_rsrc(gp, out_plane), goff, gout);
   __syncthreads();
-  stage.store(planes, H, W, shift);
+  stage.template store<WINDOW>(planes, H, W, shift, rw);
   __syncthreads();
   for (int j = 0; j < nch; ++j) {
     float gv_next = 0.f;
     if (j + 1 < nch) {
-      stage.load(xp + (size_t)(j + 1) * x_step, true, H, W, shift);
+      stage.template load<WINDOW>(xp + (size_t)(j + 1) * x_step, true, H, W, shift, rw);
       gv_next = buf_ld(plane_rsrc(gp + (size_t)(j + 1) * g_step, out_plane), goff, gout);
     }
     const float* pl = planes + (j & 1) * PS;
@@ -1057,12 +1121,12 @@ __global__ __launch_bounds__(kDBlock, 2) void deform_grad_filter_kernel(
       }
     if (lane < CELLS) wacc[(wave * ch_per_block + j) * CELLS + lane] += mine;
     gv = gv_next;
-    if (j + 1 < nch) stage.store(planes + ((j + 1) & 1) * PS, H, W, shift);
+    if (j + 1 < nch) stage.template store<WINDOW>(planes + ((j + 1) & 1) * PS, H, W, shift, rw);
     __syncthreads();
   }
 
   const size_t part = (size_t)b.n * tiles + b.tile;
-  for (int e = threadIdx.x; e < nch * CELLS; e += kDBlock) {
+  for (int e = threadIdx.x; e < nch * CELLS; e += BLOCK) {
     float s = 0.f;
 #pragma unroll
     for (int w = 0; w < kWaves; ++w) s += wacc[w * ch_per_block * CELLS + e];
@@ -1301,11 +1365,11 @@ struct DeformPlan {
 // N=64 C=512 28x28 -> 14x14: grad input 4, grad filter 3, the channel-interleaved kernels 3; the
 // one-plane forward 4, grad offset 3, grad rotation 2)
 DeformPlan deform_plan(const Geo& g, int table_floats, int planes, int block, int blocks_per_cu,
-                       long lds_budget = 64 * 1024) {
+                       long lds_budget = 64 * 1024, int max_w = 64, int max_passes = 16) {
   DeformPlan d{};
   d.ok = false;
   if (path_disabled(kNoDeformFast)) return d;
-  if (g.k_h != 3 || g.k_w != 3 || g.in_w > 64) return d;
+  if (g.k_h != 3 || g.k_w != 3 || g.in_w > max_w) return d;
   if (!((g.scope_h == 3 && g.scope_w == 3) || (g.scope_h == 4 && g.scope_w == 4) ||
         (g.scope_h == 5 && g.scope_w == 5)))
     return d;
@@ -1313,9 +1377,10 @@ DeformPlan deform_plan(const Geo& g, int table_floats, int planes, int block, in
   d.shift = 0;
   while ((1 << d.shift) < g.in_w) ++d.shift;
   const int rpp = block >> d.shift;
+  if (rpp < 1) return d;
   const int np = ceil_div(g.in_h, rpp);
-  if (np > 16) return d;
-  d.npass = np <= 4 ? 4 : np <= 8 ? 8 : 16;
+  if (np > max_passes) return d;
+  d.npass = np <= 4 ? 4 : np <= 8 ? 8 : np <= 16 ? 16 : 32;
   d.PS = ((g.in_h + 2) * (g.in_w + 2) + 3) & ~3;
   const int cpg = g.channel / g.groups;
   d.tiles = ceil_div(g.out_h * g.out_w, block);
@@ -1367,6 +1432,16 @@ DeformPlan deform_plan_ch(const Geo& g, int table_floats, int blocks_per_cu) {
   return d;
 }
 
+// Planes that neither form above takes -- wider than 64 columns, or taller than sixteen staging passes of a
+// 256-thread workgroup -- while two padded copies fit a CU's LDS (112 x 112, 130 x 130 in fp32): the one-plane
+// kernels in workgroups of kDWideBlock threads, one per CU, staging only the rows a tile's samples touch.
+constexpr int kDWideBlock = 512;
+constexpr int kDWidePasses = 32;
+
+DeformPlan deform_plan_wide(const Geo& g, int table_floats) {
+  return deform_plan(g, table_floats, 2, kDWideBlock, 1, kDBigLds, 1 << 30, kDWidePasses);
+}
+
 template <typename T, int SH, int SW>
 bool run_deform_forward(const Geo& g, const T* x, const T* off, const T* rot, const T* filter, T* out,
                         hipStream_t stream) {
@@ -1385,7 +1460,15 @@ bool run_deform_forward(const Geo& g, const T* x, const T* off, const T* rot, co
     return true;
   }
   const DeformPlan d = deform_plan(g, WideTable<SH, SW>::SIZE, 2, kDBlock, 4);
-  if (!d.ok) return false;
+  if (!d.ok) {
+    const DeformPlan w = deform_plan_wide(g, WideTable<SH, SW>::SIZE);
+    if (!w.ok) return false;
+    auto kernel = deform_forward_kernel<T, SH, SW, kDWidePasses, kDWideBlock>;
+    if (!allow_max_dynamic_lds(reinterpret_cast<const void*>(kernel))) return false;
+    const unsigned wgrid = (unsigned)xcd_grid_size((long)w.tiles * w.chunks * g.batch * g.groups);
+    kernel<<<wgrid, kDWideBlock, w.lds, stream>>>(g, x, off, rot, filter, out, w.per, w.shift);
+    return true;
+  }
   const unsigned grid = (unsigned)xcd_grid_size((long)d.tiles * d.chunks * g.batch * g.groups);
 #define DK_LAUNCH(NP) \
   deform_forward_kernel<T, SH, SW, NP><<<grid, kDBlock, d.lds, stream>>>(g, x, off, rot, filter, out, d.per, d.shift)
@@ -1401,10 +1484,17 @@ template <typename T, int SH, int SW>
 bool run_deform_grad_coord(const Geo& g, bool rotation, const T* gout, const T* x, const T* off, const T* rot,
                            const T* filter, T* result, float* ws, hipStream_t stream) {
   const DeformPlan d4 = deform_plan_ch(g, WideTable<SH, SW>::SIZE, 3);
-  const DeformPlan d = d4.ok ? d4 : deform_plan(g, WideTable<SH, SW>::SIZE, 2, kDBlock, rotation ? 2 : 3);
+  DeformPlan d = d4.ok ? d4 : deform_plan(g, WideTable<SH, SW>::SIZE, 2, kDBlock, rotation ? 2 : 3);
+  const bool wide = !d.ok;
+  if (wide) d = deform_plan_wide(g, WideTable<SH, SW>::SIZE);
   if (!d.ok) return false;
   const unsigned grid = (unsigned)xcd_grid_size((long)d.tiles * d.chunks * g.batch * g.groups);
-  if (d4.ok && d.block == kDBigBlock) {
+  if (wide) {
+    auto kernel = rotation ? deform_grad_coord_kernel<T, SH, SW, kDWidePasses, true, kDWideBlock>
+                           : deform_grad_coord_kernel<T, SH, SW, kDWidePasses, false, kDWideBlock>;
+    if (!allow_max_dynamic_lds(reinterpret_cast<const void*>(kernel))) return false;
+    kernel<<<grid, kDWideBlock, d.lds, stream>>>(g, gout, x, off, rot, filter, ws, d.per, d.shift);
+  } else if (d4.ok && d.block == kDBigBlock) {
     auto kernel = rotation ? deform_grad_coord_ch_kernel<T, SH, SW, 4, true, kDeformCh, kDBigBlock>
                            : deform_grad_coord_ch_kernel<T, SH, SW, 4, false, kDeformCh, kDBigBlock>;
     if (!allow_max_dynamic_lds(reinterpret_cast<const void*>(kernel)))
@@ -1450,36 +1540,49 @@ DeformPlan grad_input_plan(const Geo& g) {
   return deform_plan(g, WideTable<SH, SW>::SIZE + 1, 4, grad_input_block(g), 4);
 }
 
+// Channels per workgroup of the tiled grad input: as many 64-bit planes (4, 2 or 1) as fit LDS; 0 if not even one.
+template <int SH, int SW>
+int tiled_channels(const DeformPlan& basic, size_t* lds) {
+  for (int ch = 4; ch >= 1; ch >>= 1) {
+    *lds = ((size_t)2 * ch * basic.PS + (size_t)ch * WideTable<SH, SW>::SIZE + ch) * sizeof(float);
+    if (*lds <= 150 * 1024) return ch;
+  }
+  return 0;
+}
+
 template <typename T, int SH, int SW>
 bool run_deform_grad_input(const Geo& g, const T* gout, const T* off, const T* rot, const T* filter, T* gin,
                            void* ws, hipStream_t stream) {
   const DeformPlan d = grad_input_plan<SH, SW>(g);
-  const bool tiled = !d.ok && g.out_h * g.out_w > 1024;
+  const bool tiled = !d.ok;  // output planes of more than 1024 pixels, input planes wider than 64 columns
   size_t tiled_lds = 0;
-  int tiled_shift = 0;
+  int tiled_shift = 0, tiled_ch = 0;
   if (tiled) {
-    // the basic limits of the tuned family, then room for kTiledCh 64-bit planes in LDS
-    const DeformPlan basic = deform_plan(g, WideTable<SH, SW>::SIZE, 0, 1024, 2);
+    // the basic limits of the tuned family (any width: the read-back loop walks the rows), then room for the 64-bit planes
+    const DeformPlan basic = deform_plan(g, WideTable<SH, SW>::SIZE, 0, 1024, 2, 64 * 1024, 1 << 30, 1 << 30);
     if (!basic.ok) return false;
     tiled_shift = basic.shift;
-    tiled_lds = ((size_t)2 * kTiledCh * basic.PS + (size_t)kTiledCh * WideTable<SH, SW>::SIZE + kTiledCh) * sizeof(float);
-    if (tiled_lds > 150 * 1024) return false;
-  } else if (!d.ok) {
-    return false;
+    tiled_ch = tiled_channels<SH, SW>(basic, &tiled_lds);
+    if (tiled_ch == 0) return false;
   }
   if (reinterpret_cast<uintptr_t>(gout) % 16 != 0) return false;  // absmax_kernel reads 16-byte vectors
   unsigned* gmax = static_cast<unsigned*>(ws);
   const long n = (long)g.batch * g.channel * g.out_h * g.out_w;
-  absmax_kernel<T><<<kAbsParts, 256, 0, stream>>>(gout, n, gmax);
   if (tiled) {
-    auto kernel = deform_grad_input_tiled_kernel<T, SH, SW>;
-    if (!allow_max_dynamic_lds(reinterpret_cast<const void*>(kernel)))
-      return false;
     const int cpg = g.channel / g.groups;
-    const unsigned tgrid = (unsigned)xcd_grid_size((long)ceil_div(cpg, kTiledCh) * g.batch * g.groups);
-    kernel<<<tgrid, 1024, tiled_lds, stream>>>(g, gout, off, rot, filter, gin, gmax, tiled_shift);
+    const unsigned tgrid = (unsigned)xcd_grid_size((long)ceil_div(cpg, tiled_ch) * g.batch * g.groups);
+#define DK_LAUNCH(CH)                                                                                   \
+  {                                                                                                     \
+    auto kernel = deform_grad_input_tiled_kernel<T, SH, SW, CH>;                                        \
+    if (!allow_max_dynamic_lds(reinterpret_cast<const void*>(kernel))) return false;                    \
+    absmax_kernel<T><<<kAbsParts, 256, 0, stream>>>(gout, n, gmax);                                     \
+    kernel<<<tgrid, 1024, tiled_lds, stream>>>(g, gout, off, rot, filter, gin, gmax, tiled_shift);      \
+  }
+    if (tiled_ch == 4) DK_LAUNCH(4) else if (tiled_ch == 2) DK_LAUNCH(2) else DK_LAUNCH(1)
+#undef DK_LAUNCH
     return true;
   }
+  absmax_kernel<T><<<kAbsParts, 256, 0, stream>>>(gout, n, gmax);
   const unsigned grid = (unsigned)xcd_grid_size((long)d.chunks * g.batch * g.groups);
   deform_grad_input_kernel<T, SH, SW><<<grid, grad_input_block(g), d.lds, stream>>>(g, gout, off, rot, filter, gin, gmax,
                                                                                    d.per, d.shift);
@@ -1542,7 +1645,16 @@ bool run_deform_grad_filter(const Geo& g, const T* gout, const T* x, const T* of
     return false;  // 25 dense accumulators and 90 hat weights per lane do not fit the register budget
   } else {
     const DeformPlan d = deform_plan(g, (kDBlock / 64) * SH * SW, 2, kDBlock, 3);
-    if (!d.ok) return false;
+    if (!d.ok) {
+      const DeformPlan w = deform_plan_wide(g, (kDWideBlock / 64) * SH * SW);
+      if (!w.ok) return false;
+      auto kernel = deform_grad_filter_kernel<T, SH, SW, kDWidePasses, kDWideBlock>;
+      if (!allow_max_dynamic_lds(reinterpret_cast<const void*>(kernel))) return false;
+      const unsigned wgrid = (unsigned)xcd_grid_size((long)w.tiles * w.chunks * g.batch * g.groups);
+      kernel<<<wgrid, kDWideBlock, w.lds, stream>>>(g, gout, x, off, rot, ws, w.per, w.shift);
+      launch_reduce_partials<float, T>(ws, g.batch * w.tiles, g.channel * SH * SW, gfilter, stream);
+      return true;
+    }
     const unsigned grid = (unsigned)xcd_grid_size((long)d.tiles * d.chunks * g.batch * g.groups);
 #define DK_LAUNCH(NP) \
   deform_grad_filter_kernel<T, SH, SW, NP><<<grid, kDBlock, d.lds, stream>>>(g, gout, x, off, rot, ws, d.per, d.shift)
@@ -1584,7 +1696,8 @@ bool fast_deform_grad_coord(const Geo& g, bool rotation, const T* gout, const T*
 size_t fast_deform_grad_coord_workspace(const Geo& g, bool rotation) {
   const int table = g.scope_h == 3 ? WideTable<3, 3>::SIZE : g.scope_h == 4 ? WideTable<4, 4>::SIZE : WideTable<5, 5>::SIZE;
   const DeformPlan d4 = deform_plan_ch(g, table, 3);
-  const DeformPlan d = d4.ok ? d4 : deform_plan(g, table, 2, kDBlock, rotation ? 2 : 3);
+  DeformPlan d = d4.ok ? d4 : deform_plan(g, table, 2, kDBlock, rotation ? 2 : 3);
+  if (!d.ok) d = deform_plan_wide(g, table);
   if (!d.ok) return 0;
   // both lay out chunks * groups * batch planes of 18 * out pixels
   return (size_t)d.chunks * g.groups * g.batch * 18 * g.out_h * g.out_w * sizeof(float);

@@ -34,6 +34,10 @@ CASES = [
     (1, 9, 56, 56, 3, (4, 4), 1, 1, 1, 1, 0.7, 2.0),      # 56 x 56: 512-thread channel-interleaved kernels, 7 tiles of 7 waves
     (1, 6, 64, 64, 3, (5, 5), 2, 1, 1, 1, 1.0, 2.5),      # the largest plane they take, stride 2
     (2, 10, 45, 50, 3, (3, 3), 1, 1, 1, 2, 0.6, 3.0),     # 5 tiles of 512, the last one ragged; two groups, scope 3; one sample on a grid line in fp32
+    (1, 5, 112, 112, 3, (4, 4), 1, 1, 1, 1, 0.7, 2.0),    # 112 x 112: wider than 64 columns, row-window staging, one 64-bit plane per workgroup in grad input
+    (1, 4, 40, 130, 3, (3, 3), 1, 1, 1, 2, 0.6, 3.0),     # 130 columns: 256 lanes per staged row, two groups
+    (2, 6, 112, 112, 3, (4, 4), 2, 1, 1, 1, 0.5, 8.0),    # 112 x 112 stride 2 with offsets that spread a tile's samples over most of the plane
+    (1, 3, 100, 30, 3, (5, 5), 1, 1, 1, 1, 1.0, 2.5),     # narrow but taller than the 256-thread staging covers; scope 5
 ]
 NAMES = ("forward", "grad input", "grad offset", "grad rotation", "grad filter")
 
@@ -89,7 +93,7 @@ def test_fp64_matches_oracle(case):
 
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
-@pytest.mark.parametrize("case", CASES[:3] + [CASES[10], CASES[13], CASES[14]])   # the last three: planes above 30 x 30
+@pytest.mark.parametrize("case", CASES[:3] + [CASES[10], CASES[13], CASES[14], CASES[16], CASES[17]])   # planes above 30 x 30; the last two wider than 64 columns
 def test_half_precisions_match_fp32_oracle(case, dtype):
     inputs, got = _run(case, dtype)
     want = _oracle(inputs, np.float32)
