@@ -36,13 +36,8 @@ __device__ __forceinline__ void st(float* p, float v) { *p = v; }
 __device__ __forceinline__ void st(double* p, double v) { *p = v; }
 __device__ __forceinline__ void st(__half* p, float v) { *p = __float2half_rn(v); }
 __device__ __forceinline__ void st(bf16_t* p, float v) {
-  uint32_t u = __float_as_uint(v);
-  if ((u & 0x7fffffffu) > 0x7f800000u) {  // NaN: keep it a NaN
-    p->bits = static_cast<uint16_t>((u >> 16) | 0x40u);
-  } else {
-    u += 0x7fffu + ((u >> 16) & 1u);  // round to nearest even
-    p->bits = static_cast<uint16_t>(u >> 16);
-  }
+  // the hardware conversion (v_cvt_pk_bf16_f32): round to nearest even, a NaN stays a NaN
+  p->bits = __builtin_bit_cast(uint16_t, static_cast<__bf16>(v));
 }
 
 // ---------------------------------------------------------------------------

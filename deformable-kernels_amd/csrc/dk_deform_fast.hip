@@ -1,6 +1,7 @@
 // Tuned gfx950 kernels of the DEFORMABLE variant (the input taps are themselves sampled
 // bilinearly at image-space offsets) for 3x3 taps, scope 3x3 / 4x4 / 5x5, fp32 / fp16 / bf16,
-// input planes up to 64 columns wide that fit LDS.  Everything else runs on dk_generic.hip.
+// input planes whose zero-padded copy fits LDS twice (up to about 130 x 130 in a workgroup of its own).
+// Everything else runs on dk_generic.hip.
 //
 // Reference kernels covered (K.cu =
 // deformable_kernels/ops/deform_kernel/csrc/filter_sample_depthwise_cuda_kernel.cu):
@@ -23,7 +24,9 @@
 // [e][c]: the corner gathers at per-lane addresses bound these kernels, and one 16-byte read per
 // corner then serves four channels.  Planes up to about 30 x 30 run that form in workgroups of 256
 // threads, several per CU; larger ones (up to 64 x 64) in one workgroup of 1024 threads per CU that
-// takes most of the CU's LDS for the two interleaved buffers.
+// takes most of the CU's LDS for the two interleaved buffers.  Wider or taller planes (112 x 112) run the
+// one-plane forms of forward, the coordinate gradients and grad filter in workgroups of 512 threads that
+// stage only the plane rows the tile's samples touch, and grad input with fewer planes per workgroup.
 #include <algorithm>
 #include <cstdlib>
 

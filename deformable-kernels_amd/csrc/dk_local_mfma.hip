@@ -41,7 +41,7 @@ namespace dk {
 namespace {
 
 constexpr int kPix = 128;     // pixels per tile
-constexpr int kCh = 16;       // channels per unit
+constexpr int kCh = 16;       // channels per matrix block; a unit is one block of fp32 channels or two of 16-bit ones
 constexpr int kThreads = 512;
 constexpr int kWaves = kThreads / 64;
 constexpr int kMaxX = 6;      // staged source elements per lane and channel: tile + halo rows <= 64 * kMaxX
@@ -125,6 +125,10 @@ __device__ __forceinline__ float hat(float d) { return __builtin_amdgcn_fmed3f(1
 // apart plus a skew: lane (channel q, pixel quad kg) reads row q at 4 kg + const, and
 // (q % 4) + 16 (q / 4) + 4 kg covers the 64 banks exactly once.
 __device__ __forceinline__ constexpr int tile_row(int j, int pitch) { return j * pitch + (j & 3) + 16 * (j >> 2); }
+// The same for 16-bit tensors, whose tile holds two elements per slot: lane (q, kg) reads rows q and
+// q + 16 at 2 kg + const; with a pitch of 8 mod 64 the rows q % 8 start 8 banks apart, and the one
+// slot of skew for q / 8 odd fills the gaps between the even 2 kg.
+__device__ __forceinline__ constexpr int tile_row16(int j, int pitch) { return j * pitch + ((j >> 3) & 1); }
 
 // A staged element: the tile holds one 32-bit slot per element, written by the buffer load itself
 // (a 2-byte load leaves the element zero-extended in its slot).
@@ -132,6 +136,18 @@ __device__ __forceinline__ float slot_value(unsigned bits, const float*) { retur
 __device__ __forceinline__ float slot_value(unsigned bits, const bf16_t*) { return __uint_as_float(bits << 16); }
 __device__ __forceinline__ float slot_value(unsigned bits, const __half*) {
   return static_cast<float>(__builtin_bit_cast(_Float16, static_cast<unsigned short>(bits)));
+}
+
+// The two elements of a slot of a 16-bit tile (the lower address in the lower half).
+__device__ __forceinline__ float pair_lo(unsigned bits, const float*) { return 0.f; }
+__device__ __forceinline__ float pair_hi(unsigned bits, const float*) { return 0.f; }
+__device__ __forceinline__ float pair_lo(unsigned bits, const bf16_t*) { return __uint_as_float(bits << 16); }
+__device__ __forceinline__ float pair_hi(unsigned bits, const bf16_t*) { return __uint_as_float(bits & 0xffff0000u); }
+__device__ __forceinline__ float pair_lo(unsigned bits, const __half*) {
+  return static_cast<float>(__builtin_bit_cast(_Float16, static_cast<unsigned short>(bits)));
+}
+__device__ __forceinline__ float pair_hi(unsigned bits, const __half*) {
+  return static_cast<float>(__builtin_bit_cast(_Float16, static_cast<unsigned short>(bits >> 16)));
 }
 
 typedef __attribute__((address_space(3))) void* lds_void_ptr;
@@ -175,8 +191,21 @@ template <int SIZE, int NX>
 __device__ __forceinline__ void load_run_to_lds(u4 r, unsigned* to, int off) {
   const unsigned addr = (unsigned)(unsigned long)(lds_void_ptr)to;
   static_assert(SIZE == 4, "the LDS side steps by 4 bytes per element, the memory side by SIZE: equal only for 4");
-  static_assert(NX == 4 || NX == 6, "four or six runs");
-  if constexpr (NX == 4)
+  static_assert(NX == 2 || NX == 3 || NX == 4 || NX == 6, "two, three, four or six runs");
+  if constexpr (NX == 2)
+    asm volatile(
+        "s_mov_b32 m0, %0\n\ts_nop 0\n\t"
+        "buffer_load_dword %1, %2, 0 offen lds\n\t"
+        "buffer_load_dword %1, %2, 0 offen offset:256 lds" ::"s"(addr), "v"(off), "s"(r)
+        : "memory", "m0");
+  else if constexpr (NX == 3)
+    asm volatile(
+        "s_mov_b32 m0, %0\n\ts_nop 0\n\t"
+        "buffer_load_dword %1, %2, 0 offen lds\n\t"
+        "buffer_load_dword %1, %2, 0 offen offset:256 lds\n\t"
+        "buffer_load_dword %1, %2, 0 offen offset:512 lds" ::"s"(addr), "v"(off), "s"(r)
+        : "memory", "m0");
+  else if constexpr (NX == 4)
     asm volatile(
         "s_mov_b32 m0, %0\n\ts_nop 0\n\t"
         "buffer_load_dword %1, %2, 0 offen lds\n\t"
@@ -212,20 +241,23 @@ __global__ __launch_bounds__(kThreads, 4) void local_gather_mfma_kernel(
   using E = typename MxOf<T>::type;
   using M = Mx<E>;
   constexpr bool kThird = sizeof(T) == 4;  // fp32 tensors: the filter has a low part
+  constexpr bool kPacked = sizeof(T) == 2; // 16-bit tensors: two elements per slot of the tile, two channel blocks per unit
+  constexpr int CHU = kPacked ? 2 * kCh : kCh;  // channels per unit
+  constexpr int NRUN = kPacked ? NX / 2 : NX;   // 64-slot runs of a staged row
   constexpr int K = 9, CELLS = SH * SW;
   static_assert(CELLS <= 16, "one K = 16 block of cells");
-  constexpr int PITCH = 64 * NX + 64;
+  constexpr int PITCH = kPacked ? 64 * NRUN + 8 : 64 * NX + 64;
   constexpr int kEntries = (K * kPix + kThreads - 1) / kThreads;  // coordinate entries staged per thread
-  constexpr int kChW = kCh / kWaves;                              // channels staged per wave
-  constexpr int kDma = kChW * NX;                                 // staging loads per wave and unit
-  __shared__ unsigned xs0[kCh * PITCH], xs1[kCh * PITCH], xs2[kCh * PITCH];
+  constexpr int kChW = CHU / kWaves;                              // channels staged per wave
+  constexpr int kDma = kChW * NRUN;                               // staging loads per wave and unit
+  __shared__ unsigned xs0[CHU * PITCH], xs1[CHU * PITCH], xs2[CHU * PITCH];
   __shared__ float2 hw[K * kPix];  // scope coordinates (h, w) of (tap, pixel of the tile)
   extern __shared__ __align__(16) unsigned dyn[];
 
   const int cpg = g.channel / g.groups;
-  const int nblk = ceil_div(cpg, kCh);
-  uint4* wsp = reinterpret_cast<uint4*>(dyn);                  // [nblk][64]: Wh (2 words), Wl (2 words)
-  float* unscale = reinterpret_cast<float*>(wsp + nblk * 64);  // [nblk][kCh]: 1 / s of the channel
+  const int nblk = ceil_div(cpg, CHU);
+  uint4* wsp = reinterpret_cast<uint4*>(dyn);                  // [nblk][64]: Wh (2 words), Wl (2 words); 16-bit: W of channel q, W of channel q + 16
+  float* unscale = reinterpret_cast<float*>(wsp + nblk * 64);  // [nblk][kCh]: 1 / s of the channel (fp32 tensors)
 
   const int total = nwg * g.groups;
   const int lb = logical_block(total);
@@ -248,7 +280,21 @@ __global__ __launch_bounds__(kThreads, 4) void local_gather_mfma_kernel(
   // ---- per workgroup: the split filter operands of every channel block.  Lane (q, kg) of the
   // B side stands for channel q and cells 4 kg .. 4 kg + 3.
   for (int e = threadIdx.x; e < nblk * 64; e += kThreads) {
-    const int b = e >> 6, l = e & 63, cj = b * kCh + (l & 15), c0 = 4 * (l >> 4);
+    const int b = e >> 6, l = e & 63, cj = b * CHU + (l & 15), c0 = 4 * (l >> 4);
+    if constexpr (kPacked) {
+      // the filter is exact in the matrix type: the cells 4 kg .. 4 kg + 3 of channel q and of channel q + 16
+      typename M::v4 w2[2];
+#pragma unroll
+      for (int h = 0; h < 2; ++h) {
+        const int ch = cj + h * kCh;
+        const T* f = filter + (size_t)(grp + g.groups * (ch < cpg ? ch : 0)) * CELLS;
+#pragma unroll
+        for (int k = 0; k < 4; ++k) w2[h][k] = static_cast<E>((ch < cpg && c0 + k < CELLS) ? ld(f + c0 + k) : 0.f);
+      }
+      const uint2 b0 = __builtin_bit_cast(uint2, w2[0]), b1 = __builtin_bit_cast(uint2, w2[1]);
+      wsp[e] = make_uint4(b0.x, b0.y, b1.x, b1.y);
+      continue;
+    }
     float v[4] = {0.f, 0.f, 0.f, 0.f}, s = 1.f;
     if (cj < cpg) {
       const T* f = filter + (size_t)(grp + g.groups * cj) * CELLS;
@@ -324,29 +370,47 @@ __global__ __launch_bounds__(kThreads, 4) void local_gather_mfma_kernel(
   };
 
   // ---- staging
+  // bytes between two channels of the group, and this wave's first staged channel of a unit in those terms
+  const size_t ch_bytes = (size_t)g.groups * src_plane * sizeof(T);
+  const size_t wave_first = (size_t)wave * ch_bytes;
   auto stage_tile = [&](const Unit& u, unsigned* buf) {
     const int n = u.n, x0 = u.p0 + lo;
+    // channel u.cb * CHU + wave of the unit: one 64-bit scalar product per unit, an addition per channel
+    const char* unit_first = reinterpret_cast<const char*>(src) + (size_t)(n * g.channel + grp) * src_plane * sizeof(T) +
+                             (size_t)(u.cb * CHU) * ch_bytes + wave_first;
 #pragma unroll
     for (int jj = 0; jj < kChW; ++jj) {
-      const int j = wave + jj * kWaves, cj = u.cb * kCh + j;
+      const int j = wave + jj * kWaves, cj = u.cb * CHU + j;
       const bool chan = cj < cpg;
-      const size_t c = (size_t)n * g.channel + grp + (size_t)g.groups * (chan ? cj : 0);
-      const T* plane = src + c * src_plane;
-      if (sizeof(T) == 4 && x0 >= 0) {
+      const T* plane = reinterpret_cast<const T*>(unit_first + (chan ? (size_t)jj * kWaves * ch_bytes : 0));
+      if constexpr (kPacked) {
+        // pairs of elements from the even element below x0 (the width is even, so x0 is odd and every
+        // plane starts on a 4-byte boundary): slot i of the row holds elements x0 - 1 + 2 i, + 1
+        const int x0e = x0 - 1;
+        unsigned* row = buf + tile_row16(j, PITCH);
+        if (x0e >= 0) {
+          const u4 rx = resource_words(plane + x0e, chan ? max(src_plane - x0e, 0) : 0);
+          load_run_to_lds<4, NRUN>(rx, row, lane * 4);
+        } else {
+          const u4 rx = resource_words(plane, chan ? src_plane : 0);
+#pragma unroll
+          for (int k = 0; k < NRUN; ++k) {
+            const int e = x0e + 2 * (lane + 64 * k);  // even: both elements of the pair lie before the plane, or neither
+            load_to_lds<4>(rx, row + 64 * k, e < 0 ? (int)kOutOfRange : e * 2);
+          }
+        }
+      } else if (x0 >= 0) {
         // the buffer starts at the first staged element: every lane's offset is its lane number,
         // the 64-element steps are immediates, and what lies past the plane fails the range check
-        if constexpr (sizeof(T) == 4) {
-          const u4 rx = resource_words(plane + x0, chan ? max(src_plane - x0, 0) : 0);
-          load_run_to_lds<4, NX>(rx, buf + tile_row(j, PITCH), lane * 4);
-        }
+        const u4 rx = resource_words(plane + x0, chan ? max(src_plane - x0, 0) : 0);
+        load_run_to_lds<4, NX>(rx, buf + tile_row(j, PITCH), lane * 4);
       } else {
-        // the first tile of a plane: the elements before the plane must read as zeros (16-bit
-        // tensors always come this way: their memory and LDS steps differ)
+        // the first tile of a plane: the elements before the plane must read as zeros
         const u4 rx = resource_words(plane, chan ? src_plane : 0);
 #pragma unroll
         for (int k = 0; k < NX; ++k) {
           const int e = x0 + lane + 64 * k;
-          load_to_lds<sizeof(T)>(rx, buf + tile_row(j, PITCH) + 64 * k, e < 0 ? (int)kOutOfRange : e * (int)sizeof(T));
+          load_to_lds<4>(rx, buf + tile_row(j, PITCH) + 64 * k, e < 0 ? (int)kOutOfRange : e * 4);
         }
       }
     }
@@ -439,7 +503,53 @@ __global__ __launch_bounds__(kThreads, 4) void local_gather_mfma_kernel(
     }
   };
 
+  // Where a lane's four results go: a scalar 64-bit part per unit (image, first channel of the unit, tile) and a
+  // 32-bit part per lane (its channel within the unit, its pixels within the tile) that never changes.
+  const unsigned lane_out = (unsigned)(g.groups * q) * (unsigned)dst_plane + (unsigned)px;
+  auto unit_out = [&](const Unit& u) {
+    return dst + ((size_t)(u.n * g.channel + grp) + (size_t)g.groups * (u.cb * CHU)) * dst_plane + u.p0;
+  };
   auto multiply_unit = [&](const Unit& u, const unsigned* buf) {
+    if constexpr (kPacked) {
+      // one channel block after the other (block h: channel q + 16 h), each with its own store, so that only
+      // one block's sums and filter operand are live
+      const int p = u.p0 + px;
+#pragma unroll
+      for (int h = 0; h < 2; ++h) {
+        // [W ; W] pairs with [Ah | Al]
+        const uint2 wbits = reinterpret_cast<const uint2*>(wsp + u.cb * 64 + lane)[h];
+        const typename M::v4 w4 = __builtin_bit_cast(typename M::v4, wbits);
+        const typename M::v8 wb = __builtin_shufflevector(w4, w4, 0, 1, 2, 3, 0, 1, 2, 3);
+        float acc[4] = {0.f, 0.f, 0.f, 0.f};
+        const unsigned* xr0 = buf + tile_row16(q + h * kCh, PITCH) + (px >> 1);
+#pragma unroll
+        for (int rr = 0; rr < 3; ++rr) {
+          // columns -1 .. +4 around the four pixels: element px + rr * row_step + k of the range that starts at
+          // x0 = slot-aligned start + 1, so k = 0 is the upper half of the first slot
+          const unsigned* xr = xr0 + ((rr * row_step) >> 1);
+          const unsigned u0 = xr[0], u1 = xr[1], u2 = xr[2], u3 = xr[3];
+          const float x6[6] = {pair_hi(u0, src), pair_lo(u1, src), pair_hi(u1, src),
+                               pair_lo(u2, src), pair_hi(u2, src), pair_lo(u3, src)};
+          const int t0 = TRANSPOSED ? (2 - rr) * 3 + 2 : rr * 3, dt = TRANSPOSED ? -1 : 1;
+          f4 d[3];
+          M::template row<false>(d[0], d[1], d[2], A[t0], A[t0 + dt], A[t0 + 2 * dt], wb, wb);
+#pragma unroll
+          for (int cc = 0; cc < 3; ++cc)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) acc[i] = fmaf(x6[i + cc], d[cc][i], acc[i]);
+        }
+        const int cj = u.cb * CHU + h * kCh + q;
+        if (cj < cpg && p < dst_plane) {
+          // the plane is a multiple of 4 pixels (the host checks), so the four pixels are inside it and 8-byte aligned
+          T* out = unit_out(u) + (lane_out + (unsigned)h * (unsigned)(kCh * g.groups * dst_plane));
+          struct { T e[4]; } pk;
+#pragma unroll
+          for (int i = 0; i < 4; ++i) st(pk.e + i, acc[i]);
+          *reinterpret_cast<uint2*>(out) = __builtin_bit_cast(uint2, pk);  // default policy: 2-byte runs merge to whole lines in L2
+        }
+      }
+      return;
+    }
     const uint4 wv = wsp[u.cb * 64 + lane];
     const typename M::v4 wh = __builtin_bit_cast(typename M::v4, make_uint2(wv.x, wv.y));
     const typename M::v4 wl = __builtin_bit_cast(typename M::v4, make_uint2(wv.z, wv.w));
@@ -453,7 +563,7 @@ __global__ __launch_bounds__(kThreads, 4) void local_gather_mfma_kernel(
     for (int rr = 0; rr < 3; ++rr) {
       float x6[6];  // columns -1 .. +4 of staged tap row rr around the four pixels
 #pragma unroll
-      for (int k = 0; k < 6; ++k) x6[k] = slot_value(xr0[rr * row_step + k], src);
+      for (int k = 0; k < 6; ++k) x6[k] = __uint_as_float(xr0[rr * row_step + k]);
       const int t0 = TRANSPOSED ? (2 - rr) * 3 + 2 : rr * 3, dt = TRANSPOSED ? -1 : 1;  // the taps of columns 0, 1, 2
       f4 d[3];
       M::template row<kThird>(d[0], d[1], d[2], A[t0], A[t0 + dt], A[t0 + 2 * dt], whh, wl0);
@@ -464,27 +574,16 @@ __global__ __launch_bounds__(kThreads, 4) void local_gather_mfma_kernel(
     }
     // lane (kg, q): channel q of the block, pixels px .. px + 3 of the tile
     const int cj = u.cb * kCh + q;
-    const int n = u.n, p = u.p0 + px;
+    const int p = u.p0 + px;
     if (cj < cpg && p < dst_plane) {
-      if constexpr (kThird) {
-        const float us = unscale[u.cb * kCh + q];
+      const float us = unscale[u.cb * kCh + q];
 #pragma unroll
-        for (int i = 0; i < 4; ++i) acc[i] *= us;
-      }
-      T* out = dst + ((size_t)n * g.channel + grp + (size_t)g.groups * cj) * dst_plane + p;
+      for (int i = 0; i < 4; ++i) acc[i] *= us;
+      T* out = unit_out(u) + lane_out;
       if ((dst_plane & 3) == 0) {
         // p is a multiple of 4, so the four pixels are inside the plane and 16-byte aligned
-        if constexpr (sizeof(T) == 4) {
-          f4 v = {acc[0], acc[1], acc[2], acc[3]};
-          *reinterpret_cast<f4*>(out) = v;  // default policy: the wave's 64-byte runs merge to whole lines in L2
-        } else {
-          struct { T e[4]; } pk;
-#pragma unroll
-          for (int i = 0; i < 4; ++i) st(pk.e + i, acc[i]);
-          const uint2 bits = __builtin_bit_cast(uint2, pk);
-          typedef unsigned u2 __attribute__((ext_vector_type(2)));
-          __builtin_nontemporal_store(u2{bits.x, bits.y}, reinterpret_cast<u2*>(out));
-        }
+        f4 v = {acc[0], acc[1], acc[2], acc[3]};
+        *reinterpret_cast<f4*>(out) = v;  // default policy: the wave's 64-byte runs merge to whole lines in L2
       } else {
 #pragma unroll
         for (int i = 0; i < 4; ++i)
@@ -556,23 +655,33 @@ struct GatherPlan {
   size_t lds;
 };
 
+// Static LDS of the kernel: three tiles and the coordinate table.
+constexpr long gather_static_lds(bool packed, int nx) {
+  return 3L * (packed ? 2 * kCh * (64 * (nx / 2) + 8) : kCh * (64 * nx + 64)) * 4 + 9L * kPix * 8;
+}
+
 template <int SH, int SW>
-GatherPlan gather_plan(const Geo& g, bool transposed) {
+GatherPlan gather_plan(const Geo& g, bool transposed, bool packed) {
   GatherPlan p{};
   p.ok = false;
   const bool same_width = g.stride_h == 1 && g.stride_w == 1 && g.dil_w == 1 && g.pad_w == 1 && g.k_h == 3 &&
                           g.k_w == 3 && g.in_w == g.out_w;
   if (!same_width || SH * SW > 16 || g.in_w < 2 || path_disabled(kNoRows) || path_disabled(kNoGatherMfma)) return p;  // in_w >= 2: the division by the width is a multiplication
-  const long xt = kPix + 2 + 2L * g.dil_h * g.in_w;  // tile + halo rows
+  // 16-bit tiles are staged as pairs of elements: rows of an even number of elements keep every plane, every
+  // tap row and every lane's four pixels on pair boundaries
+  if (packed && (g.in_w & 1)) return p;
+  const long xt = kPix + 2 + 2L * g.dil_h * g.in_w + (packed ? 1 : 0);  // tile + halo rows (+ the element below an odd start)
   if (xt > 64 * kMaxX) return p;
   p.nx = xt <= 256 ? 4 : kMaxX;
-  p.pitch = 64 * p.nx + 64;
-  const int cpg = g.channel / g.groups, nblk = ceil_div(cpg, kCh);
+  const int chu = packed ? 2 * kCh : kCh;
+  const int cpg = g.channel / g.groups, nblk = ceil_div(cpg, chu);
   const long plane = transposed ? (long)g.in_h * g.in_w : (long)g.out_h * g.out_w;
+  if (packed && (plane & 3)) return p;  // four pixels per 8-byte store
+  if ((long)g.groups * 2 * kCh * plane >= (1L << 31)) return p;  // a lane's channel offset within a unit in 32 bits
   p.tiles = (int)ceil_div((int)plane, kPix);
-  // dynamic part: the split filter operands; static: three tiles and the coordinate table
+  // dynamic part: the split filter operands
   const long lds = (long)nblk * 64 * 16 + (long)nblk * kCh * 4;
-  if (lds + 3L * kCh * p.pitch * 4 + 9L * kPix * 8 > 160 * 1024) return p;
+  if (lds + gather_static_lds(packed, p.nx) > 160 * 1024) return p;
   p.lds = (size_t)lds;
   const long units = (long)g.batch * p.tiles * nblk;
   if (units >= (1L << 30)) return p;
@@ -585,13 +694,15 @@ GatherPlan gather_plan(const Geo& g, bool transposed) {
 template <typename T, int SH, int SW>
 bool run_gather_mfma(const Geo& g, bool transposed, const T* src, const T* rot, const T* filter, T* dst,
                      hipStream_t stream) {
-  const GatherPlan p = gather_plan<SH, SW>(g, transposed);
+  constexpr bool packed = sizeof(T) == 2;
+  const GatherPlan p = gather_plan<SH, SW>(g, transposed, packed);
   if (!p.ok) return false;
+  if (packed && (reinterpret_cast<uintptr_t>(src) % 4 != 0 || reinterpret_cast<uintptr_t>(dst) % 8 != 0)) return false;
   const unsigned grid = (unsigned)xcd_grid_size((long)p.nwg * g.groups);
 #define DK_LAUNCH(TR, NXV)                                                                        \
   {                                                                                               \
     auto kernel = local_gather_mfma_kernel<T, SH, SW, TR, NXV>;                                   \
-    const int room = 160 * 1024 - (3 * kCh * (64 * NXV + 64) * 4 + 9 * kPix * 8);                 \
+    const int room = 160 * 1024 - (int)gather_static_lds(packed, NXV);                            \
     if (!allow_dynamic_lds(reinterpret_cast<const void*>(kernel), room)) return false;            \
     kernel<<<grid, kThreads, p.lds, stream>>>(g, src, rot, filter, dst, p.tiles, p.nwg);          \
   }
@@ -610,9 +721,6 @@ template <typename T>
 bool mfma_local_gather(const Geo& g, bool transposed, const T* src, const T* rot, const T* filter, T* dst,
                        hipStream_t stream) {
   if (g.k_h != 3 || g.k_w != 3) return false;
-  // 16-bit tensors: measured slower than the row kernels so far (60 against 66 us on N=64 C=144 56 x 56:
-  // their tiles are staged element by element, 2-byte loads into 4-byte slots), so those keep the row kernels
-  if (sizeof(T) != 4) return false;
   if ((long)g.in_h * g.in_w >= (1L << 24) || (long)g.out_h * g.out_w >= (1L << 24)) return false;  // byte offsets of 18 rotation planes in 31 bits
   // A tile's set-up (coordinates, operands) is paid once per tile and its 128 pixels must be filled: the kernel
   // wins where a plane has many tiles and a group at least six 16-channel blocks (N=64 C=144 56 x 56: 64 against

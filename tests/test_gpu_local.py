@@ -43,6 +43,7 @@ TUNED = [
     (2, 12, 15, 16, 3, (7, 7), 2, 1, 1, 2, 2.0),    # scope 7, stride 2: grad filter on the generic kernel
     (1, 24, 40, 44, 3, (5, 5), 2, 1, 1, 1, 1.5),    # scope 5, stride 2: two slices of the stride-2 matrix-core grad filter
     (1, 24, 41, 43, 3, (5, 5), 2, 1, 1, 1, 1.5),    # the same with an odd width: dense grad filter with two cells per lane
+    (2, 80, 12, 18, 3, (4, 4), 1, 1, 1, 2, 1.0),    # same width, even: 40 channels per group (1.25 units of the 16-bit matrix-core forward), 2 groups
 ]
 GENERIC = [
     (2, 6, 9, 8, (5, 3), (7, 4), (1, 2), (2, 0), 1, 3, 0.7),
@@ -96,6 +97,19 @@ def test_matrix_core_forward_and_grad_input_on_every_same_width_shape(case, swit
     o32 = _oracle(inputs, np.float32)
     assert rel_err(got[0], o32[0]) < 1e-5, "forward"
     assert rel_err(got[1], o32[1]) < 1e-5, "grad input"
+
+
+@pytest.mark.parametrize("dtype,tol", [(torch.float16, 1e-3), (torch.bfloat16, 5e-3)])
+@pytest.mark.parametrize("case", [c for c in TUNED if c[6] == 1 and c[7] == 1 and c[8] == 1 and c[5] in ((4, 4), (3, 3))])
+def test_matrix_core_forward_and_grad_input_on_16_bit_tensors(case, dtype, tol, switch_off):
+    """16-bit tensors take the same kernel with two elements per slot of its staged tiles and two channel
+    blocks per unit (rows of an even number of elements; other widths stay on the row kernels, which this
+    test then runs).  The products carry fp32 sums, so the error is the result's own rounding to the type."""
+    switch_off("DK_FORCE_GATHER_MFMA")
+    inputs, got = _run(case, dtype, seed=7)
+    want = _oracle(inputs, np.float32)  # the inputs are already rounded to `dtype`
+    assert rel_err(got[0].float(), want[0]) < tol, "forward"
+    assert rel_err(got[1].float(), want[1]) < tol, "grad input"
 
 
 @pytest.mark.parametrize("case", TUNED[:4] + GENERIC[:2])
