@@ -1392,12 +1392,15 @@ int channels_per_block(int cpg, int wanted_splits) {
   return per;
 }
 
-// How many channel splits give the forward / grad-input grid enough waves to fill 256 CUs.
+// How many channel splits give the forward / grad-input grid enough waves to fill 256 CUs.  A plane of up to
+// 62 pixels is one wave per workgroup (row_block), so it takes four times the splits of a four-wave plane.
 int pick_splits(const Geo& g, int planes_pixels) {
-  const long waves = (long)ceil_div(planes_pixels, kBlock) * (kBlock / 64) * g.batch * g.groups;
+  const int waves_per_block = std::min(kBlock / 64, ceil_div(planes_pixels, 62));
+  const long waves = (long)ceil_div(planes_pixels, kBlock) * waves_per_block * g.batch * g.groups;
   const int cpg = g.channel / g.groups;
+  const int least = waves_per_block == 1 ? 8 : 16;  // channels per split
   int splits = 1;
-  while (waves * splits < 8192 && cpg / (splits * 2) >= 16) splits *= 2;
+  while (waves * splits < 8192 && cpg / (splits * 2) >= least) splits *= 2;
   return splits;
 }
 
@@ -1458,7 +1461,8 @@ bool run_gather(const Geo& g, bool transposed, const T* src, const T* rot, const
 }
 
 // Channel splits of the grad-rotation grid: enough for about four blocks per CU with at least
-// 16 channels per split.
+// 16 channels per split.  (One-wave blocks -- planes of up to 62 pixels -- were tried with four times
+// the splits: N=128 C=960 7 x 7 59 -> 66 us, the partial sums cost more than the fuller grid gains.)
 int rotation_splits(const Geo& g) {
   const int cpg = g.channel / g.groups;
   const long base = std::max(1L, (long)ceil_div(g.out_h * g.out_w, rotation_tile(g)) * g.batch * g.groups);  // batch may be 0
