@@ -686,7 +686,9 @@ GatherPlan gather_plan(const Geo& g, bool transposed, bool packed) {
   const long units = (long)g.batch * p.tiles * nblk;
   if (units >= (1L << 30)) return p;
   // at most two workgroups per CU, all resident at once, each walking an equal share of the units
-  p.nwg = (int)std::max(1L, std::min((long)g.batch * p.tiles, (long)std::max(1, 2 * 256 / g.groups)));
+  // (with fewer tiles than that, the workgroups share tiles: contiguous ranges of a tile's channel blocks, at least
+  // four units each, every range paying the tile's set-up)
+  p.nwg = (int)std::max(1L, std::min(std::max((long)g.batch * p.tiles, units / 4), (long)std::max(1, 2 * 256 / g.groups)));
   p.ok = true;
   return p;
 }
@@ -724,9 +726,17 @@ bool mfma_local_gather(const Geo& g, bool transposed, const T* src, const T* rot
   if ((long)g.in_h * g.in_w >= (1L << 24) || (long)g.out_h * g.out_w >= (1L << 24)) return false;  // byte offsets of 18 rotation planes in 31 bits
   // A tile's set-up (coordinates, operands) is paid once per tile and its 128 pixels must be filled: the kernel
   // wins where a plane has many tiles and a group at least six 16-channel blocks (N=64 C=144 56 x 56: 64 against
-  // 68 us), and loses to the row kernels on small planes or few channels (C=960 7 x 7: 73 against 18 us;
-  // C=384 14 x 14: 37 / 21; C=192 28 x 28: 39 / 35; C=32 112 x 112: 121 / 62).
-  if (!path_disabled(kForceGatherMfma) && ((long)g.out_h * g.out_w < 2048 || g.channel / g.groups < 96)) return false;
+  // 68 us), and loses to the row kernels on small planes or few channels (fp32, N=64: C=960 7 x 7: 73 against 18 us;
+  // C=384 14 x 14: 31 / 19; C=192 28 x 28: 41 / 34; C=32 112 x 112: 122 / 58).  16-bit tensors, whose units hold 32
+  // channels, also win on smaller planes once there are enough units to share out (bf16, N=128: C=384 14 x 14
+  // 29 against 33 us, C=576 14 x 14 38 / 44, C=192 28 x 28 45 / 54; N=64: 22.8 / 19.1, 29.4 / 27.4, 29.9 / 33.7).
+  if (!path_disabled(kForceGatherMfma)) {
+    const long plane = (long)g.out_h * g.out_w;
+    const int cpg = g.channel / g.groups;
+    const long units = (long)g.batch * ceil_div((int)plane, kPix) * ceil_div(cpg, 2 * kCh);
+    const bool large = plane >= 2048 || (sizeof(T) == 2 && units >= 2560);
+    if (!large || cpg < 96) return false;
+  }
   if (g.scope_h == 4 && g.scope_w == 4) return run_gather_mfma<T, 4, 4>(g, transposed, src, rot, filter, dst, stream);
   if (g.scope_h == 3 && g.scope_w == 3) return run_gather_mfma<T, 3, 3>(g, transposed, src, rot, filter, dst, stream);
   return false;
