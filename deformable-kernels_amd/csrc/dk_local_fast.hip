@@ -971,6 +971,16 @@ constexpr int kMfMaxBlkS2 = 12;        // stride 2: channel blocks per workgroup
 typedef float mf4 __attribute__((ext_vector_type(4)));
 typedef __bf16 mfb4 __attribute__((ext_vector_type(4)));
 
+// Two floats rounded to bfloat16 by one instruction (v_cvt_pk_bf16_f32), a in the lower half; and the two halves
+// of such a pair back as floats.
+__device__ __forceinline__ unsigned pack_bf16(float a, float b) {
+  typedef float f2 __attribute__((ext_vector_type(2)));
+  typedef __bf16 b2 __attribute__((ext_vector_type(2)));
+  return __builtin_bit_cast(unsigned, __builtin_convertvector(f2{a, b}, b2));
+}
+__device__ __forceinline__ float bf16_lo(unsigned pair) { return __uint_as_float(pair << 16); }
+__device__ __forceinline__ float bf16_hi(unsigned pair) { return __uint_as_float(pair & 0xffff0000u); }
+
 // First float of channel j's row in the staged input tile.  The rows are a multiple of 64 floats
 // apart plus a skew: in the MFMA phase lane (channel q, pixel quad kg) reads row q at
 // 4 * kg + const, and (q % 4) + 16 * (q / 4) + 4 * kg covers the 64 banks exactly once.
@@ -1214,14 +1224,20 @@ __global__ __launch_bounds__(kMfBlock, 4) void local_grad_filter_mfma_kernel(
         if constexpr (SPLIT) {
           // every instruction adds into a live accumulator, so its result registers cannot be
           // given to one of its operands (see dk_local_mfma.hip for what happens when they can)
-          mfb4 bh, bl;
+          // two values per conversion instruction (v_cvt_pk_bf16_f32 leaves them packed as the matrix operand wants
+          // them; converted one by one they cost a conversion and half a byte permute each, six vector
+          // instructions per product instead of four)
+          float pr[4];
 #pragma unroll
           for (int ii = 0; ii < 4; ++ii) {
-            float pr = xv[ii][f_w] * gq[ii];
-            asm volatile("" : "+v"(pr));  // one fp32 value for both parts: no contraction into the conversions
-            bh[ii] = static_cast<__bf16>(pr);
-            bl[ii] = static_cast<__bf16>(pr - static_cast<float>(bh[ii]));
+            pr[ii] = xv[ii][f_w] * gq[ii];
+            asm volatile("" : "+v"(pr[ii]));  // one fp32 value for both parts: no contraction into the conversions
           }
+          const unsigned h01 = pack_bf16(pr[0], pr[1]), h23 = pack_bf16(pr[2], pr[3]);
+          const unsigned l01 = pack_bf16(pr[0] - bf16_lo(h01), pr[1] - bf16_hi(h01));
+          const unsigned l23 = pack_bf16(pr[2] - bf16_lo(h23), pr[3] - bf16_hi(h23));
+          const mfb4 bh = __builtin_bit_cast(mfb4, make_uint2(h01, h23));
+          const mfb4 bl = __builtin_bit_cast(mfb4, make_uint2(l01, l23));
           if (t & 1) {
             acc1 = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(Ab[t], bh, acc1, 0, 0, 0);
             acc1 = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(Ab[t], bl, acc1, 0, 0, 0);
@@ -1232,9 +1248,8 @@ __global__ __launch_bounds__(kMfBlock, 4) void local_grad_filter_mfma_kernel(
             acc0 = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(Al[t], bh, acc0, 0, 0, 0);
           }
         } else if constexpr (kHalfIn) {
-          mfb4 b;
-#pragma unroll
-          for (int ii = 0; ii < 4; ++ii) b[ii] = static_cast<__bf16>(xv[ii][f_w] * gq[ii]);
+          const mfb4 b = __builtin_bit_cast(mfb4, make_uint2(pack_bf16(xv[0][f_w] * gq[0], xv[1][f_w] * gq[1]),
+                                                             pack_bf16(xv[2][f_w] * gq[2], xv[3][f_w] * gq[3])));
           if (t & 1)
             acc1 = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(Ab[t], b, acc1, 0, 0, 0);
           else
@@ -1274,13 +1289,13 @@ __global__ __launch_bounds__(kMfBlock, 4) void local_grad_filter_mfma_kernel(
       if constexpr (SPLIT) {
         float av[4] = {a0, a1, a2, a3};
 #pragma unroll
-        for (int ii = 0; ii < 4; ++ii) {
-          asm volatile("" : "+v"(av[ii]));
-          Ab[t][ii] = static_cast<__bf16>(av[ii]);
-          Al[t][ii] = static_cast<__bf16>(av[ii] - static_cast<float>(Ab[t][ii]));
-        }
+        for (int ii = 0; ii < 4; ++ii) asm volatile("" : "+v"(av[ii]));
+        const unsigned h01 = pack_bf16(av[0], av[1]), h23 = pack_bf16(av[2], av[3]);
+        Ab[t] = __builtin_bit_cast(mfb4, make_uint2(h01, h23));
+        Al[t] = __builtin_bit_cast(mfb4, make_uint2(pack_bf16(av[0] - bf16_lo(h01), av[1] - bf16_hi(h01)),
+                                                    pack_bf16(av[2] - bf16_lo(h23), av[3] - bf16_hi(h23))));
       } else if constexpr (kHalfIn) {
-        Ab[t] = mfb4{static_cast<__bf16>(a0), static_cast<__bf16>(a1), static_cast<__bf16>(a2), static_cast<__bf16>(a3)};
+        Ab[t] = __builtin_bit_cast(mfb4, make_uint2(pack_bf16(a0, a1), pack_bf16(a2, a3)));
       } else {
         A[0][t] = a0;
         A[1][t] = a1;
