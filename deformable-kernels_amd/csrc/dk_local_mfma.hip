@@ -491,15 +491,21 @@ __global__ __launch_bounds__(kThreads, 4) void local_gather_mfma_kernel(
 #pragma unroll
     for (int t = 0; t < K; ++t) {
       const float2 c = hw[t * kPix + wave * 16 + q];
-      typename M::v8 a;
+      // hi and lo parts, two values per conversion instruction (vector conversions: they also leave the values
+      // packed; one at a time a value costs two conversions and two packing moves more)
+      typedef float f2v __attribute__((ext_vector_type(2)));
+      typedef E e2v __attribute__((ext_vector_type(2)));
+      float v[4];
 #pragma unroll
       for (int k = 0; k < 4; ++k) {
-        E hi, lo2;
-        split2<E>(hat(c.x - cell_row(k)) * hat(c.y - cell_col(k)), hi, lo2);
-        a[k] = hi;
-        a[4 + k] = lo2;
+        v[k] = hat(c.x - cell_row(k)) * hat(c.y - cell_col(k));
+        asm volatile("" : "+v"(v[k]));  // as in split2: one fp32 value for both parts
       }
-      A[t] = a;
+      const e2v h01 = __builtin_convertvector(f2v{v[0], v[1]}, e2v), h23 = __builtin_convertvector(f2v{v[2], v[3]}, e2v);
+      const f2v b01 = __builtin_convertvector(h01, f2v), b23 = __builtin_convertvector(h23, f2v);
+      const e2v l01 = __builtin_convertvector(f2v{v[0] - b01[0], v[1] - b01[1]}, e2v);
+      const e2v l23 = __builtin_convertvector(f2v{v[2] - b23[0], v[3] - b23[1]}, e2v);
+      A[t] = typename M::v8{h01[0], h01[1], h23[0], h23[1], l01[0], l01[1], l23[0], l23[1]};
     }
   };
 
