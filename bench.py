@@ -555,6 +555,12 @@ def other_workload(a):
         }
         if rg is None:
             del calls["grad_rotation"]
+        else:
+            ws5, n5 = _lib.workspace(L.dk_deformable_sample_depthwise_backward_offset_rotation_workspace(desc), dev)
+            calls["grad_offset+rotation, one call"] = (
+                lambda: _lib.check(L.dk_deformable_sample_depthwise_backward_offset_rotation(
+                    desc, P(gg), P(xg), P(og), P(rg), P(wg), P(goff), P(grot), P(ws5), n5, st), "gcoords"),
+                by + bx + 2 * bo + 2 * br + bw)
         label = "%s: deform_sample_depthwise N=%d C=%d %dx%d->%dx%d k=%d scope=%dx%d stride=%d %s%s" % (
             a.workload, N, C, H, W, gg.shape[2], gg.shape[3], k, S[0], S[1], stride, a.dtype,
             "" if rg is not None else ", no rotation tensor")
@@ -600,12 +606,16 @@ def other_workload(a):
         us[name] = _time_us(fn, reps)
         nbytes[name] = nb_
     total_us = sum(v for k_, v in us.items() if "+" not in k_)
+    extra = {}
+    if "grad_offset+rotation, one call" in us:  # the Function's backward: both coordinate gradients from one call
+        extra["sum_with_one_call_us"] = round(total_us - us["grad_offset"] - us["grad_rotation"]
+                                              + us["grad_offset+rotation, one call"], 2)
     print(json.dumps({
         "metric": "per-entry-point time (secondary workload, not the headline)",
         "config": {"workload": label},
         "kernel_us": {k_: round(v, 2) for k_, v in us.items()},
         "algorithmic_GBps": {k_: round(nbytes[k_] / (us[k_] * 1e-6) / 1e9, 1) for k_ in us},
-        "sum_us": round(total_us, 2),
+        "sum_us": round(total_us, 2), **extra,
         "n_gpus": 1, "dtype": a.dtype, "data": "synthetic",
     }))
 

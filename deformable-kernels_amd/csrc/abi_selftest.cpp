@@ -45,6 +45,8 @@ int main() {
   EXPECT(dk_deformable_sample_depthwise_backward_filter(&ok, one, one, one, one, nullptr, one, 1 << 20, nullptr) == DK_ERR_NULL_POINTER);
   EXPECT(dk_deformable_sample_depthwise_backward_offset(&ok, one, one, one, one, one, nullptr, one, 1 << 20, nullptr) == DK_ERR_NULL_POINTER);
   EXPECT(dk_deformable_sample_depthwise_backward_rotation(&ok, one, one, one, one, one, nullptr, one, 1 << 20, nullptr) == DK_ERR_NULL_POINTER);
+  EXPECT(dk_deformable_sample_depthwise_backward_offset_rotation(&ok, one, one, one, nullptr, one, one, one, one, 1 << 20, nullptr) == DK_ERR_NULL_POINTER);
+  EXPECT(dk_deformable_sample_depthwise_backward_offset_rotation(&ok, one, one, one, one, one, one, nullptr, one, 1 << 20, nullptr) == DK_ERR_NULL_POINTER);
 
   // shapes
   dk_conv_desc bad = ok;
@@ -93,7 +95,8 @@ int main() {
                        dk_sample_depthwise_backward_workspace(&d) + dk_deformable_sample_depthwise_backward_data_workspace(&d) +
                        dk_deformable_sample_depthwise_backward_filter_workspace(&d) +
                        dk_deformable_sample_depthwise_backward_offset_workspace(&d) +
-                       dk_deformable_sample_depthwise_backward_rotation_workspace(&d);
+                       dk_deformable_sample_depthwise_backward_rotation_workspace(&d) +
+                       dk_deformable_sample_depthwise_backward_offset_rotation_workspace(&d);
             }
   EXPECT(total > 0);
 

@@ -525,6 +525,43 @@ int dk_deformable_sample_depthwise_backward_rotation(const dk_conv_desc* desc, c
   });
 }
 
+size_t dk_deformable_sample_depthwise_backward_offset_rotation_workspace(const dk_conv_desc* desc) {
+  Geo g;
+  if (make_geo(desc, g) != DK_OK) return 0;
+  return std::max(fast_deform_grad_coords_workspace(g),
+                  std::max(fast_deform_grad_coord_workspace(g, false), fast_deform_grad_coord_workspace(g, true)));
+}
+
+int dk_deformable_sample_depthwise_backward_offset_rotation(const dk_conv_desc* desc, const void* out_grad,
+                                                            const void* input, const void* offset,
+                                                            const void* rotation, const void* filter,
+                                                            void* offset_grad, void* rotation_grad,
+                                                            void* workspace, size_t workspace_bytes, void* stream) {
+  Geo g;
+  const int rc = make_geo(desc, g);
+  if (rc != DK_OK) return rc;
+  if (desc->layout != DK_LAYOUT_NCHW) return DK_ERR_UNSUPPORTED;
+  if (!out_grad || !input || !offset || !rotation || !filter || !offset_grad || !rotation_grad) return DK_ERR_NULL_POINTER;
+  const size_t need = dk_deformable_sample_depthwise_backward_offset_rotation_workspace(desc);
+  if (need && (!workspace || workspace_bytes < need)) return DK_ERR_WORKSPACE;
+  if (g.batch == 0) return DK_OK;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  bool fused = false;
+  const int st = by_dtype(desc->dtype, [&]<typename T>() {
+    if constexpr (kHasFast<T>)
+      fused = fast_deform_grad_coords_workspace(g) != 0 &&
+              fast_deform_grad_coords<T>(g, in<T>(out_grad), in<T>(input), in<T>(offset), in<T>(rotation), in<T>(filter),
+                                         out<T>(offset_grad), out<T>(rotation_grad), workspace, s);
+  });
+  if (st != DK_OK || fused) return st;
+  // one after the other, sharing the workspace (stream order)
+  const int so = dk_deformable_sample_depthwise_backward_offset(desc, out_grad, input, offset, rotation, filter,
+                                                                offset_grad, workspace, workspace_bytes, stream);
+  if (so != DK_OK) return so;
+  return dk_deformable_sample_depthwise_backward_rotation(desc, out_grad, input, offset, rotation, filter,
+                                                          rotation_grad, workspace, workspace_bytes, stream);
+}
+
 // ---- offset branch -----------------------------------------------------------------------
 
 // ---- depthwise convolution with one kernel per image and channel ---------------------------

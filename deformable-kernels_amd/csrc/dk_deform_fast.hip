@@ -525,11 +525,15 @@ __global__ __launch_bounds__(BLOCK, 2) void deform_grad_coord_kernel(
 }
 
 // The same with CH channel planes interleaved in LDS (see deform_forward_ch_kernel).
-template <typename T, int SH, int SW, int NPASS, bool ROTATION, int CH, int BLOCK = kDBlock>
+// MODE 0: grad offset, 1: grad rotation, 2: both from one pass over the staged planes (the corner gathers and
+// the table reads, which bound these kernels, are shared; the rotation partials go to `partial`, the offset
+// partials to `partial_off`).
+template <typename T, int SH, int SW, int NPASS, int MODE, int CH, int BLOCK = kDBlock>
 __global__ __launch_bounds__(BLOCK, BLOCK == kDBlock ? 2 : 1) void deform_grad_coord_ch_kernel(
     Geo g, const T* __restrict__ gout, const T* __restrict__ x, const T* __restrict__ off,
     const T* __restrict__ rot, const T* __restrict__ filter, float* __restrict__ partial,
-    int ch_per_block, int shift, int tile_pix) {
+    int ch_per_block, int shift, int tile_pix, float* __restrict__ partial_off) {
+  constexpr bool ROTATION = MODE != 0, OFFSET = MODE != 1;
   using Tb = WideTable<SH, SW>;
   extern __shared__ __align__(16) float lds[];
   const int H = g.in_h, W = g.in_w, RS = W + 2;
@@ -565,9 +569,12 @@ __global__ __launch_bounds__(BLOCK, BLOCK == kDBlock ? 2 : 1) void deform_grad_c
   const size_t x_step = (size_t)g.groups * in_plane, g_step = (size_t)g.groups * out_plane;
   const unsigned goff = live ? (unsigned)p * (unsigned)sizeof(T) : kOutOfRange;
 
-  float s0[K9], s1[K9], s2[K9];
+  float s0[K9], s1[K9], s2[K9];                    // rotation: sums of sample * gout * {b, c, d}
+  float o0[OFFSET ? K9 : 1], o1[OFFSET ? K9 : 1];  // offset: sums of d sample / d{h, w} * gout * B
 #pragma unroll
   for (int t = 0; t < K9; ++t) s0[t] = s1[t] = s2[t] = 0.f;
+#pragma unroll
+  for (int t = 0; t < (OFFSET ? K9 : 1); ++t) o0[t] = o1[t] = 0.f;
 
   PlaneStageN<T, NPASS, CH> stage;
   float gv[CH], gv_next[CH];
@@ -594,30 +601,29 @@ __global__ __launch_bounds__(BLOCK, BLOCK == kDBlock ? 2 : 1) void deform_grad_c
       const CornersN<CH> cq = read_corners_n<CH>(pl, it[t].pidx, RS);
 #pragma unroll
       for (int c = 0; c < CH; ++c) {
-        if (ROTATION) {
+        const float4 q = MODE == 1 ? lds_read4(tb + c * Tb::SIZE + st[t].cell)
+                                   : *reinterpret_cast<const float4*>(tb + c * Tb::SIZE + st[t].cell);
+        if constexpr (ROTATION) {
           const float top = fmaf(it[t].lw, cq.b[c] - cq.a[c], cq.a[c]), bot = fmaf(it[t].lw, cq.d[c] - cq.c[c], cq.c[c]);
           const float ps = fmaf(it[t].lh, bot - top, top) * gv[c];
-          const float4 q = lds_read4(tb + c * Tb::SIZE + st[t].cell);
           s0[t] = fmaf(ps, q.y, s0[t]);
           s1[t] = fmaf(ps, q.z, s1[t]);
           s2[t] = fmaf(ps, q.w, s2[t]);
-        } else {
-          const float4 q = *reinterpret_cast<const float4*>(tb + c * Tb::SIZE + st[t].cell);
+        }
+        if constexpr (OFFSET) {
           const float gw = gv[c] * lite_weight(st[t], q);
           const float ca = cq.c[c] - cq.a[c], ba = cq.b[c] - cq.a[c];
           const float dh = fmaf(it[t].lw, (cq.d[c] - cq.b[c]) - ca, ca);
           const float dw = fmaf(it[t].lh, (cq.d[c] - cq.c[c]) - ba, ba);
-          s0[t] = fmaf(dh, gw, s0[t]);
-          s1[t] = fmaf(dw, gw, s1[t]);
+          o0[t] = fmaf(dh, gw, o0[t]);
+          o1[t] = fmaf(dw, gw, o1[t]);
         }
       }
       // keeps the compiler from issuing every tap's reads first (8 x 16 bytes per tap: registers)
       // the tap's sums are complete here: without this the compiler sinks the arithmetic of all nine
       // taps below the plane store and keeps their 9 x 32 loaded values in registers meanwhile
-      if (ROTATION)
-        asm volatile("" : "+v"(s0[t]), "+v"(s1[t]), "+v"(s2[t])::"memory");
-      else
-        asm volatile("" : "+v"(s0[t]), "+v"(s1[t])::"memory");
+      if constexpr (ROTATION) asm volatile("" : "+v"(s0[t]), "+v"(s1[t]), "+v"(s2[t])::"memory");
+      if constexpr (OFFSET) asm volatile("" : "+v"(o0[t]), "+v"(o1[t])::"memory");
       __builtin_amdgcn_sched_barrier(0);
     }
 #pragma unroll
@@ -627,24 +633,32 @@ __global__ __launch_bounds__(BLOCK, BLOCK == kDBlock ? 2 : 1) void deform_grad_c
   }
 
   if (live) {
-    const size_t part = ROTATION ? (size_t)b.chunk : (size_t)b.grp * chunks + b.chunk;
-    const size_t img = ROTATION ? (size_t)(b.n * g.groups + b.grp) : (size_t)b.n;
-    const size_t imgs = ROTATION ? (size_t)g.batch * g.groups : (size_t)g.batch;
-    float* dst = partial + ((part * imgs + img) * (K9 * 2)) * out_plane + p;
-    const T* rp = rot + (size_t)(b.n * g.groups + b.grp) * (K9 * 2) * out_plane + p;
+    if constexpr (ROTATION) {
+      float* dst = partial + (((size_t)b.chunk * g.batch * g.groups + (size_t)(b.n * g.groups + b.grp)) * (K9 * 2)) * out_plane + p;
+      const T* rp = rot + (size_t)(b.n * g.groups + b.grp) * (K9 * 2) * out_plane + p;
 #pragma unroll
-    for (int t = 0; t < K9; ++t) {
-      float dh = ROTATION ? fmaf(st[t].lw, s2[t], s1[t]) : s0[t];
-      float dw = ROTATION ? fmaf(st[t].lh, s2[t], s0[t]) : s1[t];
-      if (ROTATION && g.clip_mode != kClipNone) {  // a clamped offset has no gradient
-        bool open_h, open_w;
-        scope_coord<float>(g, t / 3, ld(rp + (size_t)(2 * t) * out_plane), g.centre_h, &open_h);
-        scope_coord<float>(g, t % 3, ld(rp + (size_t)(2 * t + 1) * out_plane), g.centre_w, &open_w);
-        dh = open_h ? dh : 0.f;
-        dw = open_w ? dw : 0.f;
+      for (int t = 0; t < K9; ++t) {
+        float dh = fmaf(st[t].lw, s2[t], s1[t]);
+        float dw = fmaf(st[t].lh, s2[t], s0[t]);
+        if (g.clip_mode != kClipNone) {  // a clamped offset has no gradient
+          bool open_h, open_w;
+          scope_coord<float>(g, t / 3, ld(rp + (size_t)(2 * t) * out_plane), g.centre_h, &open_h);
+          scope_coord<float>(g, t % 3, ld(rp + (size_t)(2 * t + 1) * out_plane), g.centre_w, &open_w);
+          dh = open_h ? dh : 0.f;
+          dw = open_w ? dw : 0.f;
+        }
+        dst[(size_t)(2 * t) * out_plane] = dh;
+        dst[(size_t)(2 * t + 1) * out_plane] = dw;
       }
-      dst[(size_t)(2 * t) * out_plane] = dh;
-      dst[(size_t)(2 * t + 1) * out_plane] = dw;
+    }
+    if constexpr (OFFSET) {
+      float* base = MODE == 2 ? partial_off : partial;
+      float* dst = base + ((((size_t)b.grp * chunks + b.chunk) * g.batch + (size_t)b.n) * (K9 * 2)) * out_plane + p;
+#pragma unroll
+      for (int t = 0; t < K9; ++t) {
+        dst[(size_t)(2 * t) * out_plane] = o0[t];
+        dst[(size_t)(2 * t + 1) * out_plane] = o1[t];
+      }
     }
   }
 }
@@ -1498,16 +1512,16 @@ bool run_deform_grad_coord(const Geo& g, bool rotation, const T* gout, const T* 
     if (!allow_max_dynamic_lds(reinterpret_cast<const void*>(kernel))) return false;
     kernel<<<grid, kDWideBlock, d.lds, stream>>>(g, gout, x, off, rot, filter, ws, d.per, d.shift);
   } else if (d4.ok && d.block == kDBigBlock) {
-    auto kernel = rotation ? deform_grad_coord_ch_kernel<T, SH, SW, 4, true, kDeformCh, kDBigBlock>
-                           : deform_grad_coord_ch_kernel<T, SH, SW, 4, false, kDeformCh, kDBigBlock>;
+    auto kernel = rotation ? deform_grad_coord_ch_kernel<T, SH, SW, 4, 1, kDeformCh, kDBigBlock>
+                           : deform_grad_coord_ch_kernel<T, SH, SW, 4, 0, kDeformCh, kDBigBlock>;
     if (!allow_max_dynamic_lds(reinterpret_cast<const void*>(kernel)))
       return false;
-    kernel<<<grid, kDBigBlock, d.lds, stream>>>(g, gout, x, off, rot, filter, ws, d.per, d.shift, d.tile_pix);
+    kernel<<<grid, kDBigBlock, d.lds, stream>>>(g, gout, x, off, rot, filter, ws, d.per, d.shift, d.tile_pix, nullptr);
   } else if (d4.ok) {
     if (rotation)
-      deform_grad_coord_ch_kernel<T, SH, SW, 4, true, kDeformCh><<<grid, kDBlock, d.lds, stream>>>(g, gout, x, off, rot, filter, ws, d.per, d.shift, d.tile_pix);
+      deform_grad_coord_ch_kernel<T, SH, SW, 4, 1, kDeformCh><<<grid, kDBlock, d.lds, stream>>>(g, gout, x, off, rot, filter, ws, d.per, d.shift, d.tile_pix, nullptr);
     else
-      deform_grad_coord_ch_kernel<T, SH, SW, 4, false, kDeformCh><<<grid, kDBlock, d.lds, stream>>>(g, gout, x, off, rot, filter, ws, d.per, d.shift, d.tile_pix);
+      deform_grad_coord_ch_kernel<T, SH, SW, 4, 0, kDeformCh><<<grid, kDBlock, d.lds, stream>>>(g, gout, x, off, rot, filter, ws, d.per, d.shift, d.tile_pix, nullptr);
   } else {
 #define DK_LAUNCH(NP, ROT)                                                                          \
   deform_grad_coord_kernel<T, SH, SW, NP, ROT><<<grid, kDBlock, d.lds, stream>>>(g, gout, x, off, rot, filter, ws, \
@@ -1528,6 +1542,45 @@ bool run_deform_grad_coord(const Geo& g, bool rotation, const T* gout, const T* 
     launch_reduce_partials<float, T>(ws, d.chunks, g.batch * g.groups * plane18, result, stream);
   else
     launch_reduce_partials<float, T>(ws, d.chunks * g.groups, g.batch * plane18, result, stream);
+  return true;
+}
+
+// Plan of the one-pass offset + rotation gradient: the 256-thread channel-interleaved form, or, for planes up to
+// 64 x 64, workgroups of 512 threads (the 45 sums do not fit the 128 registers of the 1024-thread form).
+constexpr int kDCoordsBlock = 512;
+DeformPlan coords_plan(const Geo& g, int table_floats) {
+  DeformPlan d = deform_plan_ch(g, table_floats, 3);
+  if (d.ok && d.block == kDBlock) return d;
+  if (!d.ok) return d;
+  d = deform_plan(g, table_floats, 2 * kDeformCh, kDCoordsBlock, kDBigBlocksPerCu,
+                  kDBigLds - (long)(kDeformCh - 1) * table_floats * 4);
+  if (!d.ok) return d;
+  d.lds += (size_t)(kDeformCh - 1) * table_floats * 4;
+  d.tile_pix = ceil_div(ceil_div(g.out_h * g.out_w, d.tiles), 64) * 64;
+  d.ok = d.npass <= 8 && d.lds <= (size_t)kDBigLds;
+  return d;
+}
+
+// Offset and rotation gradient from one pass (MODE 2 of the channel-interleaved kernel in 256-thread workgroups: its
+// 45 sums fit their register budget, not that of the 1024-thread form); false where that form does not apply.
+// Workspace: the rotation partials, then the offset partials (the same number of floats).
+template <typename T, int SH, int SW>
+bool run_deform_grad_coords(const Geo& g, const T* gout, const T* x, const T* off, const T* rot, const T* filter,
+                            T* goff, T* grot, float* ws, hipStream_t stream) {
+  const DeformPlan d = coords_plan(g, WideTable<SH, SW>::SIZE);
+  if (!d.ok) return false;
+  const int plane18 = 18 * g.out_h * g.out_w;
+  float* ws_off = ws + (size_t)d.chunks * g.groups * g.batch * plane18;
+  const unsigned grid = (unsigned)xcd_grid_size((long)d.tiles * d.chunks * g.batch * g.groups);
+  if (d.block == kDBlock) {
+    deform_grad_coord_ch_kernel<T, SH, SW, 4, 2, kDeformCh><<<grid, kDBlock, d.lds, stream>>>(g, gout, x, off, rot, filter, ws, d.per, d.shift, d.tile_pix, ws_off);
+  } else {
+    auto kernel = deform_grad_coord_ch_kernel<T, SH, SW, 8, 2, kDeformCh, kDCoordsBlock>;
+    if (!allow_max_dynamic_lds(reinterpret_cast<const void*>(kernel))) return false;
+    kernel<<<grid, kDCoordsBlock, d.lds, stream>>>(g, gout, x, off, rot, filter, ws, d.per, d.shift, d.tile_pix, ws_off);
+  }
+  launch_reduce_partials<float, T>(ws, d.chunks, g.batch * g.groups * plane18, grot, stream);
+  launch_reduce_partials<float, T>(ws_off, d.chunks * g.groups, g.batch * plane18, goff, stream);
   return true;
 }
 
@@ -1706,6 +1759,22 @@ size_t fast_deform_grad_coord_workspace(const Geo& g, bool rotation) {
   return (size_t)d.chunks * g.groups * g.batch * 18 * g.out_h * g.out_w * sizeof(float);
 }
 
+size_t fast_deform_grad_coords_workspace(const Geo& g) {
+  const int table = g.scope_h == 3 ? WideTable<3, 3>::SIZE : g.scope_h == 4 ? WideTable<4, 4>::SIZE : WideTable<5, 5>::SIZE;
+  const DeformPlan d = coords_plan(g, table);
+  if (!d.ok) return 0;
+  return 2 * (size_t)d.chunks * g.groups * g.batch * 18 * g.out_h * g.out_w * sizeof(float);
+}
+
+template <typename T>
+bool fast_deform_grad_coords(const Geo& g, const T* gout, const T* x, const T* off, const T* rot, const T* filter,
+                             T* goff, T* grot, void* ws, hipStream_t stream) {
+#define CALL(SH, SW) \
+  run_deform_grad_coords<T, SH, SW>(g, gout, x, off, rot, filter, goff, grot, static_cast<float*>(ws), stream)
+  DK_DISPATCH_SCOPE(g, CALL)
+#undef CALL
+}
+
 template <typename T>
 bool fast_deform_grad_input(const Geo& g, const T* gout, const T* off, const T* rot, const T* filter, T* gin,
                             void* ws, hipStream_t stream) {
@@ -1735,6 +1804,8 @@ size_t fast_deform_grad_filter_workspace(const Geo& g) {
   template bool fast_deform_forward<T>(const Geo&, const T*, const T*, const T*, const T*, T*, hipStream_t);      \
   template bool fast_deform_grad_coord<T>(const Geo&, bool, const T*, const T*, const T*, const T*, const T*, T*,  \
                                           void*, hipStream_t);                                                     \
+  template bool fast_deform_grad_coords<T>(const Geo&, const T*, const T*, const T*, const T*, const T*, T*, T*,    \
+                                           void*, hipStream_t);                                                    \
   template bool fast_deform_grad_input<T>(const Geo&, const T*, const T*, const T*, const T*, T*, void*,           \
                                           hipStream_t);                                                            \
   template bool fast_deform_grad_filter<T>(const Geo&, const T*, const T*, const T*, const T*, T*, void*,          \

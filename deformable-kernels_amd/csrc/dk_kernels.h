@@ -84,6 +84,11 @@ size_t fast_deform_grad_coord_workspace(const Geo& g, bool rotation);
 template <typename T>
 bool fast_deform_grad_coord(const Geo& g, bool rotation, const T* gout, const T* x, const T* off, const T* rot,
                             const T* filter, T* result, void* ws, hipStream_t stream);
+// both coordinate gradients from one pass over the input; 0 / false where only the separate kernels apply
+size_t fast_deform_grad_coords_workspace(const Geo& g);
+template <typename T>
+bool fast_deform_grad_coords(const Geo& g, const T* gout, const T* x, const T* off, const T* rot, const T* filter,
+                             T* goff, T* grot, void* ws, hipStream_t stream);
 size_t fast_deform_grad_filter_workspace(const Geo& g);
 template <typename T>
 bool fast_deform_grad_filter(const Geo& g, const T* gout, const T* x, const T* off, const T* rot, T* gfilter,

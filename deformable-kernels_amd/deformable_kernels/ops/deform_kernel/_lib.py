@@ -69,6 +69,8 @@ SIGNATURES = {
     "dk_deformable_sample_depthwise_backward_offset": (ctypes.c_int, [_CD, _P, _P, _P, _P, _P, _P, _P, _SZ, _P]),
     "dk_deformable_sample_depthwise_backward_rotation_workspace": (_SZ, [_CD]),
     "dk_deformable_sample_depthwise_backward_rotation": (ctypes.c_int, [_CD, _P, _P, _P, _P, _P, _P, _P, _SZ, _P]),
+    "dk_deformable_sample_depthwise_backward_offset_rotation_workspace": (_SZ, [_CD]),
+    "dk_deformable_sample_depthwise_backward_offset_rotation": (ctypes.c_int, [_CD, _P, _P, _P, _P, _P, _P, _P, _P, _SZ, _P]),
     "dk_nd_linear_sample_forward_workspace": (_SZ, [_ND]),
     "dk_nd_linear_sample_forward": (ctypes.c_int, [_ND, _P, _P, _P, _P, _P, _SZ, _P]),
     "dk_nd_linear_sample_order_bytes": (_SZ, [_ND]),

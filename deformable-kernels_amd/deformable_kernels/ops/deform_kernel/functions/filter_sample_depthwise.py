@@ -193,14 +193,24 @@ class DeformableSampleDepthwiseFunction(Function):
                 _lib.check(L.dk_deformable_sample_depthwise_backward_data(
                     desc, p(grad_output), p(offset), p(rotation), p(weight), p(grad_input),
                     p(ws), nbytes, s), "deform_sample_depthwise backward_data")
-            if ctx.needs_input_grad[1]:
+            both = ctx.needs_input_grad[1] and ctx.needs_input_grad[2] and rotation is not None
+            if both:
+                # one call for both coordinate gradients (one pass over the input where the library has that kernel)
+                grad_offset, grad_rotation = torch.empty_like(offset), torch.empty_like(rotation)
+                ws, nbytes = _lib.workspace(
+                    L.dk_deformable_sample_depthwise_backward_offset_rotation_workspace(desc), input.device)
+                _lib.check(L.dk_deformable_sample_depthwise_backward_offset_rotation(
+                    desc, p(grad_output), p(input), p(offset), p(rotation), p(weight),
+                    p(grad_offset), p(grad_rotation), p(ws), nbytes, s),
+                    "deform_sample_depthwise backward_offset_rotation")
+            if ctx.needs_input_grad[1] and not both:
                 grad_offset = torch.empty_like(offset)
                 ws, nbytes = _lib.workspace(
                     L.dk_deformable_sample_depthwise_backward_offset_workspace(desc), input.device)
                 _lib.check(L.dk_deformable_sample_depthwise_backward_offset(
                     desc, p(grad_output), p(input), p(offset), p(rotation), p(weight),
                     p(grad_offset), p(ws), nbytes, s), "deform_sample_depthwise backward_offset")
-            if ctx.needs_input_grad[2] and rotation is not None:
+            if ctx.needs_input_grad[2] and rotation is not None and not both:
                 grad_rotation = torch.empty_like(rotation)
                 ws, nbytes = _lib.workspace(
                     L.dk_deformable_sample_depthwise_backward_rotation_workspace(desc), input.device)

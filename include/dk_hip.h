@@ -210,6 +210,19 @@ int dk_deformable_sample_depthwise_backward_rotation(const dk_conv_desc *desc,
                                                      void *workspace, size_t workspace_bytes,
                                                      void *stream);
 
+/* Both coordinate gradients of the deformable operator in one call -- what the reference's backward
+ * (functions/filter_sample_depthwise.py:163-197) asks for with its two calls
+ * deformable_sample_depthwise_backward_offset_cuda and ..._backward_rotation_cuda.  Where one pass over the
+ * input can produce both (planes of up to 64 x 64 pixels) they come from one kernel; otherwise the two
+ * entry points above run one after the other on the stream.  `rotation` must not be NULL here. */
+size_t dk_deformable_sample_depthwise_backward_offset_rotation_workspace(const dk_conv_desc *desc);
+int dk_deformable_sample_depthwise_backward_offset_rotation(const dk_conv_desc *desc, const void *out_grad,
+                                                            const void *input, const void *offset,
+                                                            const void *rotation, const void *filter,
+                                                            void *offset_grad, void *rotation_grad,
+                                                            void *workspace, size_t workspace_bytes,
+                                                            void *stream);
+
 /* ---- N-d linear sample -------------------------------------------------------
  * data [channel, shape[0..dims-1]], coord [batch, dims] in absolute index units,
  * output [batch, channel].  The reference passes `shape` as a device tensor of the

@@ -329,3 +329,29 @@ def test_deform_conv_module_runs_without_a_rotation_tensor_and_is_a_depthwise_de
     assert rel_err(out.detach().cpu(), want.cpu()) < 1e-5
     out.sum().backward()
     assert x.grad is not None and m.inner_conv.weight.grad is not None and m.offset_conv.weight.grad is not None
+
+
+@pytest.mark.parametrize("case", [CASES[0], CASES[8], CASES[13]])  # one kernel (small planes, several chunks); 56 x 56: the two kernels in turn
+def test_both_coordinate_gradients_from_one_call_equal_the_separate_entry_points(case):
+    """dk_deformable_sample_depthwise_backward_offset_rotation forms the same sums in the same order as
+    the two separate entry points, whether it runs as one kernel or as the two in turn: equal bits."""
+    from deformable_kernels.ops.deform_kernel import _lib
+    N, C, H, W, k, S, s, p, d, G, rs, os_ = case
+    x, wt, rot, off, gout, cfg = make_deform(N, C, H, W, k, S, s, p, d, G, rs, os_, seed=3, dtype=torch.float32)
+    dev = torch.device("cuda:0")
+    xg, wg, rg, og, gg = [t.to(dev) for t in (x, wt, rot, off, gout)]
+    L, P = _lib.lib(), _lib.ptr
+    desc = _lib.conv_desc(xg, wg, cfg["kernel_size"], cfg["stride"], cfg["padding"], cfg["dilation"], G)
+    st = _lib.stream_ptr(xg)
+    goff, grot, goff2, grot2 = [torch.empty_like(t) for t in (og, rg, og, rg)]
+    ws, n = _lib.workspace(L.dk_deformable_sample_depthwise_backward_offset_workspace(desc), dev)
+    _lib.check(L.dk_deformable_sample_depthwise_backward_offset(desc, P(gg), P(xg), P(og), P(rg), P(wg), P(goff), P(ws), n, st), "offset")
+    ws, n = _lib.workspace(L.dk_deformable_sample_depthwise_backward_rotation_workspace(desc), dev)
+    _lib.check(L.dk_deformable_sample_depthwise_backward_rotation(desc, P(gg), P(xg), P(og), P(rg), P(wg), P(grot), P(ws), n, st), "rotation")
+    ws, n = _lib.workspace(L.dk_deformable_sample_depthwise_backward_offset_rotation_workspace(desc), dev)
+    _lib.check(L.dk_deformable_sample_depthwise_backward_offset_rotation(
+        desc, P(gg), P(xg), P(og), P(rg), P(wg), P(goff2), P(grot2), P(ws), n, st), "both")
+    assert L.dk_deformable_sample_depthwise_backward_offset_rotation(
+        desc, P(gg), P(xg), P(og), P(rg), P(wg), P(goff2), P(grot2), P(ws), max(n - 1, 0), st) == (-5 if n else 0)  # DK_ERR_WORKSPACE
+    torch.cuda.synchronize()
+    assert torch.equal(goff, goff2) and torch.equal(grot, grot2)
