@@ -941,32 +941,37 @@ __global__ __launch_bounds__(1024) void deform_grad_input_kernel(
 }
 
 // ---------------------------------------------------------------------------
-// grad input for output planes of more than 1024 pixels.  The same fixed-point LDS accumulation,
-// but the workgroup (1024 threads) owns only kTiledCh channels of an image and keeps one plane
-// per channel; it walks the output plane in tiles of 1024 pixels, computes a tile's tap
-// descriptors once and adds the tile's contributions for each of its channels.  The planes are
-// read back once at the end.  grid = (channel chunks of kTiledCh, image * group)
+// grad input for output planes of more than 1024 pixels, or input planes the kernel above has no room for.  The
+// same fixed-point LDS accumulation, but the workgroup (1024 threads) owns 2 NP channels of an image and NP 64-bit
+// planes; it walks the output plane in tiles of 1024 pixels, computes a tile's tap descriptors once and adds the
+// tile's contributions for each of its channels.  A first walk over the tiles counts the samples per input element
+// (M, as above): while M <= 2^kPairHead two channels share a plane, each as a signed 32-bit term in its half
+// of the 64-bit sum, and one walk serves all 2 NP channels; otherwise every channel gets a plane of its own on the
+// 2^-44 grid and the channels take two walks.  The planes are read back at the end of a walk.
+// grid = (channel chunks of 2 NP, image * group)
 // ---------------------------------------------------------------------------
-template <typename T, int SH, int SW, int kTiledCh>
+template <typename T, int SH, int SW, int NP>
 __global__ __launch_bounds__(1024) void deform_grad_input_tiled_kernel(
     Geo g, const T* __restrict__ gout, const T* __restrict__ off, const T* __restrict__ rot,
     const T* __restrict__ filter, T* __restrict__ gin, const unsigned* __restrict__ gmax_bits, int shift) {
   using Tb = WideTable<SH, SW>;
+  constexpr int NC = 2 * NP;  // channels per workgroup
   extern __shared__ __align__(16) float lds[];
   const int H = g.in_h, W = g.in_w, RS = W + 2;
   const int PS = ((H + 2) * RS + 3) & ~3;
-  unsigned long long* planes = reinterpret_cast<unsigned long long*>(lds);  // [kTiledCh][PS]
-  float* tbl = lds + 2 * kTiledCh * PS;                                     // [kTiledCh][Tb::SIZE]
-  float* wmax = tbl + kTiledCh * Tb::SIZE;                                  // [kTiledCh]
+  unsigned long long* planes = reinterpret_cast<unsigned long long*>(lds);  // [NP][PS]
+  float* tbl = lds + 2 * NP * PS;                                           // [NC][Tb::SIZE]
+  float* wmax = tbl + NC * Tb::SIZE;                                        // [NC]
+  __shared__ unsigned wave_most[16];
 
   const int cpg = g.channel / g.groups;
   const int out_plane = g.out_h * g.out_w, in_plane = H * W;
-  const BlockId b = decode_block(g, 1, ceil_div(cpg, kTiledCh));
+  const BlockId b = decode_block(g, 1, ceil_div(cpg, NC));
   if (!b.valid) return;
-  const int j0 = b.chunk * kTiledCh;
-  const int nch = min(kTiledCh, cpg - j0);
+  const int j0 = b.chunk * NC;
+  const int nch = min(NC, cpg - j0);
 
-  for (int e = threadIdx.x; e < kTiledCh * PS; e += blockDim.x) planes[e] = 0ull;
+  for (int e = threadIdx.x; e < NP * PS; e += blockDim.x) planes[e] = 0ull;
   stage_wide_tables<T, SH, SW>(tbl, filter, g.channel, b.grp + g.groups * j0, g.groups, nch);
   if (threadIdx.x < nch) {
     const T* f = filter + (size_t)(b.grp + g.groups * (j0 + threadIdx.x)) * (SH * SW);
@@ -980,63 +985,173 @@ __global__ __launch_bounds__(1024) void deform_grad_input_tiled_kernel(
   constexpr double kMagic = 6755399441055744.0;  // 1.5 * 2^52
   const size_t chan0 = (size_t)b.n * g.channel + b.grp + (size_t)g.groups * j0;
   const T* gp = gout + chan0 * out_plane;
+  T* ip = gin + chan0 * in_plane;
   const size_t g_step = (size_t)g.groups * out_plane, i_step = (size_t)g.groups * in_plane;
-  if (write_nan_if_unbounded(gmax, wmax, nch, gin + chan0 * in_plane, i_step, in_plane)) return;
+  if (write_nan_if_unbounded(gmax, wmax, nch, ip, i_step, in_plane)) return;
 
-  for (int tile = 0; tile * (int)blockDim.x < out_plane; ++tile) {
+  // a tile's descriptors; bit t of the result: tap t samples the image inside the scope band
+  auto tile_taps = [&](int tile, ImgTap (&it)[K9], LiteTap (&st)[K9], unsigned& goff) {
     const int p = tile * (int)blockDim.x + threadIdx.x;
     const bool live = p < out_plane;
-    ImgTap it[K9];
-    LiteTap st[K9];
+    ScopeCoord sc[K9];
+    deform_taps<T>(g, off, rot, b.n, b.grp, p, live, RS, it, sc);
     unsigned hits = 0;
-    {
-      ScopeCoord sc[K9];
-      deform_taps<T>(g, off, rot, b.n, b.grp, p, live, RS, it, sc);
 #pragma unroll
-      for (int t = 0; t < K9; ++t) {
-        st[t] = make_lite_tap<SH, SW>(sc[t].h, sc[t].w, true);
-        const bool in = (sc[t].h > -1.f) && (sc[t].w > -1.f) && (sc[t].h < float(SH)) && (sc[t].w < float(SW));
-        hits |= in ? (1u << t) : 0u;
-      }
+    for (int t = 0; t < K9; ++t) {
+      st[t] = make_lite_tap<SH, SW>(sc[t].h, sc[t].w, true);
+      const bool in = (sc[t].h > -1.f) && (sc[t].w > -1.f) && (sc[t].h < float(SH)) && (sc[t].w < float(SW));
+      hits |= in ? (1u << t) : 0u;
     }
-    const unsigned goff = live ? (unsigned)p * (unsigned)sizeof(T) : kOutOfRange;
-    for (int j = 0; j < nch; ++j) {
-      const float gv = buf_ld(plane_rsrc(gp + (size_t)j * g_step, out_plane), goff, gout);
-      unsigned long long* pl = planes + j * PS;
-      const float* tb = tbl + j * Tb::SIZE;
-      int e;
-      (void)frexpf(gmax * wmax[j], &e);
-      const double scale = ldexp(1.0, 44 - e);
+    goff = live ? (unsigned)p * (unsigned)sizeof(T) : kOutOfRange;
+    return hits;
+  };
+  const int ntiles = ceil_div(out_plane, (int)blockDim.x);
+
+  // M: the largest number of samples on one input element, over the whole output plane
+  {
+    unsigned* count = reinterpret_cast<unsigned*>(planes);
+    for (int tile = 0; tile < ntiles; ++tile) {
+      ImgTap it[K9];
+      LiteTap st[K9];
+      unsigned goff;
+      const unsigned hits = tile_taps(tile, it, st, goff);
 #pragma unroll
       for (int t = 0; t < K9; ++t) {
         if (hits >> t & 1u) {
-          const float4 q = *reinterpret_cast<const float4*>(tb + st[t].cell);
-          const float gw = gv * lite_weight(st[t], q);
-          const float lh = it[t].lh, lw = it[t].lw, hh = 1.f - lh, hw = 1.f - lw;
-          const float term[4] = {hh * hw * gw, hh * lw * gw, lh * hw * gw, lh * lw * gw};
-          const int at[4] = {it[t].pidx, it[t].pidx + 1, it[t].pidx + RS, it[t].pidx + RS + 1};
+          atomicAdd(count + it[t].pidx, 1u);
+          atomicAdd(count + it[t].pidx + 1, 1u);
+          atomicAdd(count + it[t].pidx + RS, 1u);
+          atomicAdd(count + it[t].pidx + RS + 1, 1u);
+        }
+      }
+    }
+    __syncthreads();
+    unsigned most = 1u;
+    for (int e = threadIdx.x; e < PS; e += blockDim.x) {
+      most = max(most, count[e]);
+      count[e] = 0u;
+    }
+    for (int sft = 32; sft > 0; sft >>= 1) most = max(most, (unsigned)__shfl_xor((int)most, sft));
+    if ((threadIdx.x & 63) == 0) wave_most[threadIdx.x >> 6] = most;
+    __syncthreads();
+  }
+  unsigned most = 1u;
+  for (int w = 0; w < (int)blockDim.x / 64; ++w) most = max(most, wave_most[w]);
+  const int head = most <= 1u ? 0 : 32 - __builtin_clz(most - 1u);  // ceil(log2(most))
+  const int col = threadIdx.x & ((1 << shift) - 1), sub = threadIdx.x >> shift;
+  const int rpp = (int)blockDim.x >> shift;
+
+  if (head <= kPairHead) {
+    // two channels per plane: channel 2 q in the low half, 2 q + 1 in the high half (see deform_grad_input_kernel)
+    for (int tile = 0; tile < ntiles; ++tile) {
+      ImgTap it[K9];
+      LiteTap st[K9];
+      unsigned goff;
+      const unsigned hits = tile_taps(tile, it, st, goff);
+      for (int j = 0; j < nch; j += 2) {
+        const bool pair = j + 1 < nch;
+        const float gva = buf_ld(plane_rsrc(gp + (size_t)j * g_step, out_plane), goff, gout);
+        const float gvb = buf_ld(plane_rsrc(gp + (size_t)(j + 1) * g_step, pair ? out_plane : 0), goff, gout);
+        unsigned long long* pl = planes + (j >> 1) * PS;
+        const float* ta = tbl + j * Tb::SIZE;
+        const float* tb = tbl + (pair ? j + 1 : j) * Tb::SIZE;
+        int ea, eb;  // a term of channel c is below gmax * wmax[c] < 2^e: scale 2^(30 - head - e)
+        (void)frexpf(gmax * wmax[j], &ea);
+        (void)frexpf(gmax * wmax[pair ? j + 1 : j], &eb);
+        const int sa = min(max(30 - head - ea, -100), 100), sb = min(max(30 - head - eb, -100), 100);
+        const float ga_s = gva * ldexpf(1.f, sa), gb_s = pair ? gvb * ldexpf(1.f, sb) : 0.f;
 #pragma unroll
-          for (int k = 0; k < 4; ++k) {
-            const double d = fma((double)term[k], scale, kMagic);
-            atomicAdd(pl + at[k], (unsigned long long)__double_as_longlong(d) - 0x4338000000000000ull);
+        for (int t = 0; t < K9; ++t) {
+          if (hits >> t & 1u) {
+            const float wa = ga_s * lite_weight(st[t], *reinterpret_cast<const float4*>(ta + st[t].cell));
+            const float wb = gb_s * lite_weight(st[t], *reinterpret_cast<const float4*>(tb + st[t].cell));
+            const float lh = it[t].lh, lw = it[t].lw, hh = 1.f - lh, hw = 1.f - lw;
+            const float cw[4] = {hh * hw, hh * lw, lh * hw, lh * lw};  // K.cu:776-789
+            const int at[4] = {it[t].pidx, it[t].pidx + 1, it[t].pidx + RS, it[t].pidx + RS + 1};
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+              const int ia = round_half_up(cw[k] * wa), ib = round_half_up(cw[k] * wb);
+              const unsigned long long both =
+                  ((unsigned long long)(unsigned)(ib + (ia >> 31)) << 32) | (unsigned long long)(unsigned)ia;
+              atomicAdd(pl + at[k], both);
+            }
           }
         }
       }
     }
+    __syncthreads();
+    for (int j = 0; j < nch; j += 2) {
+      const bool pair = j + 1 < nch;
+      int ea, eb;
+      (void)frexpf(gmax * wmax[j], &ea);
+      (void)frexpf(gmax * wmax[pair ? j + 1 : j], &eb);
+      const int sa = min(max(30 - head - ea, -100), 100), sb = min(max(30 - head - eb, -100), 100);
+      const float ua = ldexpf(1.f, -sa), ub = ldexpf(1.f, -sb);
+      const unsigned long long* pl = planes + (j >> 1) * PS;
+      T* dst = ip + (size_t)j * i_step;
+      for (int row = sub; row < H; row += rpp) {
+        if (col < W) {
+          const unsigned long long v = pl[(row + 1) * RS + 1 + col];
+          const int lo = (int)(unsigned)v;
+          const int hi = (int)(unsigned)(v >> 32) + (lo < 0 ? 1 : 0);
+          dk::st(dst + row * W + col, (float)lo * ua);
+          if (pair) dk::st(dst + i_step + row * W + col, (float)hi * ub);
+        }
+      }
+    }
+    return;
   }
-  __syncthreads();
 
-  const int col = threadIdx.x & ((1 << shift) - 1), sub = threadIdx.x >> shift;
-  const int rpp = (int)blockDim.x >> shift;
-  T* ip = gin + chan0 * in_plane;
-  for (int j = 0; j < nch; ++j) {
-    int e;
-    (void)frexpf(gmax * wmax[j], &e);
-    const double unscale = ldexp(1.0, e - 44);
-    const unsigned long long* pl = planes + j * PS;
-    T* dst = ip + (size_t)j * i_step;
-    for (int row = sub; row < H; row += rpp)
-      if (col < W) dk::st(dst + row * W + col, (float)((double)(long long)pl[(row + 1) * RS + 1 + col] * unscale));
+  // many samples on one element: a plane per channel on the 2^-44 grid, NP channels per walk over the tiles
+  for (int c0 = 0; c0 < nch; c0 += NP) {
+    const int nc = min(NP, nch - c0);
+    for (int tile = 0; tile < ntiles; ++tile) {
+      ImgTap it[K9];
+      LiteTap st[K9];
+      unsigned goff;
+      const unsigned hits = tile_taps(tile, it, st, goff);
+      for (int jj = 0; jj < nc; ++jj) {
+        const int j = c0 + jj;
+        const float gv = buf_ld(plane_rsrc(gp + (size_t)j * g_step, out_plane), goff, gout);
+        unsigned long long* pl = planes + jj * PS;
+        const float* tb = tbl + j * Tb::SIZE;
+        int e;
+        (void)frexpf(gmax * wmax[j], &e);
+        const double scale = ldexp(1.0, 44 - e);
+#pragma unroll
+        for (int t = 0; t < K9; ++t) {
+          if (hits >> t & 1u) {
+            const float4 q = *reinterpret_cast<const float4*>(tb + st[t].cell);
+            const float gw = gv * lite_weight(st[t], q);
+            const float lh = it[t].lh, lw = it[t].lw, hh = 1.f - lh, hw = 1.f - lw;
+            const float term[4] = {hh * hw * gw, hh * lw * gw, lh * hw * gw, lh * lw * gw};
+            const int at[4] = {it[t].pidx, it[t].pidx + 1, it[t].pidx + RS, it[t].pidx + RS + 1};
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+              const double d = fma((double)term[k], scale, kMagic);
+              atomicAdd(pl + at[k], (unsigned long long)__double_as_longlong(d) - 0x4338000000000000ull);
+            }
+          }
+        }
+      }
+    }
+    __syncthreads();
+    for (int jj = 0; jj < nc; ++jj) {
+      const int j = c0 + jj;
+      int e;
+      (void)frexpf(gmax * wmax[j], &e);
+      const double unscale = ldexp(1.0, e - 44);
+      unsigned long long* pl = planes + jj * PS;
+      T* dst = ip + (size_t)j * i_step;
+      for (int row = sub; row < H; row += rpp) {
+        if (col < W) {
+          unsigned long long* cell = pl + (row + 1) * RS + 1 + col;
+          dk::st(dst + row * W + col, (float)((double)(long long)*cell * unscale));
+          *cell = 0ull;  // for the next walk
+        }
+      }
+    }
+    __syncthreads();
   }
 }
 
@@ -1596,12 +1711,13 @@ DeformPlan grad_input_plan(const Geo& g) {
   return deform_plan(g, WideTable<SH, SW>::SIZE + 1, 4, grad_input_block(g), 4);
 }
 
-// Channels per workgroup of the tiled grad input: as many 64-bit planes (4, 2 or 1) as fit LDS; 0 if not even one.
+// 64-bit planes per workgroup of the tiled grad input (it owns twice as many channels): 4, 2 or 1, as many as fit
+// LDS; 0 if not even one.
 template <int SH, int SW>
-int tiled_channels(const DeformPlan& basic, size_t* lds) {
-  for (int ch = 4; ch >= 1; ch >>= 1) {
-    *lds = ((size_t)2 * ch * basic.PS + (size_t)ch * WideTable<SH, SW>::SIZE + ch) * sizeof(float);
-    if (*lds <= 150 * 1024) return ch;
+int tiled_planes(const DeformPlan& basic, size_t* lds) {
+  for (int np = 4; np >= 1; np >>= 1) {
+    *lds = ((size_t)2 * np * basic.PS + (size_t)2 * np * WideTable<SH, SW>::SIZE + 2 * np) * sizeof(float);
+    if (*lds <= 150 * 1024) return np;
   }
   return 0;
 }
@@ -1618,7 +1734,7 @@ bool run_deform_grad_input(const Geo& g, const T* gout, const T* off, const T* r
     const DeformPlan basic = deform_plan(g, WideTable<SH, SW>::SIZE, 0, 1024, 2, 64 * 1024, 1 << 30, 1 << 30);
     if (!basic.ok) return false;
     tiled_shift = basic.shift;
-    tiled_ch = tiled_channels<SH, SW>(basic, &tiled_lds);
+    tiled_ch = tiled_planes<SH, SW>(basic, &tiled_lds);
     if (tiled_ch == 0) return false;
   }
   if (reinterpret_cast<uintptr_t>(gout) % 16 != 0) return false;  // absmax_kernel reads 16-byte vectors
@@ -1626,7 +1742,7 @@ bool run_deform_grad_input(const Geo& g, const T* gout, const T* off, const T* r
   const long n = (long)g.batch * g.channel * g.out_h * g.out_w;
   if (tiled) {
     const int cpg = g.channel / g.groups;
-    const unsigned tgrid = (unsigned)xcd_grid_size((long)ceil_div(cpg, tiled_ch) * g.batch * g.groups);
+    const unsigned tgrid = (unsigned)xcd_grid_size((long)ceil_div(cpg, 2 * tiled_ch) * g.batch * g.groups);
 #define DK_LAUNCH(CH)                                                                                   \
   {                                                                                                     \
     auto kernel = deform_grad_input_tiled_kernel<T, SH, SW, CH>;                                        \

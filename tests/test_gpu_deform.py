@@ -126,11 +126,14 @@ def test_rotation_clip_inside_the_operator(case, clip):
     assert (got[3][~open_] == 0).all()
 
 
-def test_grad_input_when_every_sample_lands_on_one_input_element():
+# 14 x 14: one workgroup per output plane; 40 x 36 with 11 channels: the tiled kernel (planes above 1024 pixels:
+# a plane per channel and two walks over the tiles when an element collects more than 64 samples, last chunk ragged)
+@pytest.mark.parametrize("case", [(2, 12, 14, 14, 3, (4, 4), 1, 1, 1, 1, 0.5, 0.0),
+                                  (1, 11, 40, 36, 3, (4, 4), 1, 1, 1, 1, 0.5, 0.0)])
+def test_grad_input_when_every_sample_lands_on_one_input_element(case):
     # all 9 x P samples of an image within one input cell: the grad-input kernel's fixed-point
     # scale has to leave room for that many terms in one sum
     from deformable_kernels.ops.deform_kernel.functions import deform_sample_depthwise
-    case = (2, 12, 14, 14, 3, (4, 4), 1, 1, 1, 1, 0.5, 0.0)
     N, C, H, W, k, S, s, p, d, G, rs, os_ = case
     x, wt, rot, off, gout, cfg = make_deform(N, C, H, W, k, S, s, p, d, G, rs, os_, seed=9)
     g = torch.Generator().manual_seed(1)
