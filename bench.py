@@ -190,7 +190,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=50)
-    ap.add_argument("--workload", default="cfg2", choices=sorted(WORKLOADS) + sorted(OTHER_WORKLOADS) + sorted(GLOBAL_WORKLOADS) + ["mbv2_dk", "layer_cfg2"])
+    ap.add_argument("--workload", default="cfg2", choices=sorted(WORKLOADS) + sorted(OTHER_WORKLOADS) + sorted(GLOBAL_WORKLOADS) + ["mbv2_dk", "mbv2_net", "layer_cfg2"])
     ap.add_argument("--batch", type=int, default=64, help="batch size of the mbv2_dk workload")
     ap.add_argument("--dtype", default="fp32", choices=sorted(DTYPES))
     ap.add_argument("--shape", default="", help="N,C,H,W,stride: a local-operator layer of that shape (3x3 taps, scope 4x4, "
@@ -218,6 +218,8 @@ def main():
         sys.exit("bench.py needs a GPU")
     if a.workload == "mbv2_dk":
         return mobilenet_workload(a)
+    if a.workload == "mbv2_net":
+        return network_workload(a)
     if a.workload == "layer_cfg2":
         return layer_workload(a)
     if a.workload in OTHER_WORKLOADS:
@@ -717,6 +719,54 @@ def mobilenet_workload(a):
         "value": round(total_bytes / total_us / 1e3, 1), "unit": "GB/s",
         "pct_of_hbm_peak": round(100.0 * total_bytes / total_us / 1e3 / HBM_PEAK_GBPS, 2),
         "layers": per_layer, "n_gpus": 1, "dtype": a.dtype, "data": "synthetic",
+    }))
+
+
+def network_workload(a):
+    """The whole MobileNetV2-DK network of tests/_mbv2_dk.py (benchmark configuration 5: every depthwise 3 x 3
+    convolution a DeformKernel2d with a 4 x 4 scope): forward, cross-entropy, backward and an SGD step on
+    synthetic images.  The 1 x 1 convolutions, batch norms and the classifier are the framework's; the
+    deformable-kernel layers (operator and, where the library has kernels for the shape, their offset
+    branch) are this library's.  One JSON line; secondary to the headline."""
+    import torch
+    from _mbv2_dk import MobileNetV2DK
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    tdtype = getattr(torch, DTYPES[a.dtype])
+    torch.manual_seed(0)
+    net = MobileNetV2DK().to(dev).to(tdtype)
+    # random labels, nothing to learn, and an untrained network's gradients are large (3e3 on the first offset
+    # branch): a step size that leaves the parameters where they are keeps every step's work the same
+    opt = torch.optim.SGD(net.parameters(), lr=1e-7, momentum=0.9)
+    g = torch.Generator().manual_seed(0)
+    x = torch.randn(a.batch, 3, 224, 224, generator=g).to(dev).to(tdtype)
+    labels = torch.randint(0, 1000, (a.batch,), generator=g).to(dev)
+
+    def step():
+        opt.zero_grad(set_to_none=True)
+        loss = torch.nn.functional.cross_entropy(net(x).float(), labels)
+        loss.backward()
+        opt.step()
+        return loss
+
+    for _ in range(max(a.warmup, 3)):
+        loss = step()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(a.steps):
+        loss = step()
+    e1.record()
+    e1.synchronize()
+    ms = e0.elapsed_time(e1) / a.steps
+    if not bool(torch.isfinite(loss)):
+        sys.exit("the loss is not finite: %r" % float(loss))
+    print(json.dumps({
+        "metric": "MobileNetV2-DK training step, images/s (secondary workload: the whole network)",
+        "config": {"workload": "mbv2_net: MobileNetV2 with 17 DeformKernel2d layers (scope 4x4), 224x224, batch %d, %s, "
+                               "forward + loss + backward + SGD step" % (a.batch, a.dtype)},
+        "images_per_s": round(a.batch / (ms * 1e-3), 1), "ms_per_step": round(ms, 3), "steps": a.steps,
+        "n_gpus": 1, "dtype": a.dtype, "data": "synthetic",
     }))
 
 

@@ -651,7 +651,7 @@ int dk_image_depthwise_backward_weight(const dk_conv_desc* desc, const void* out
 static int check_offset_conv(const dk_offset_conv_desc* d) {
   if (!d) return DK_ERR_NULL_POINTER;
   if (d->batch < 0 || d->in_channels <= 0 || d->out_channels <= 0 || d->h <= 0 || d->w <= 0) return DK_ERR_BAD_SHAPE;
-  if (d->dtype != DK_F32) return DK_ERR_UNSUPPORTED;
+  if (d->dtype != DK_F32 && d->dtype != DK_F16 && d->dtype != DK_BF16) return d->dtype == DK_F64 ? DK_ERR_UNSUPPORTED : DK_ERR_BAD_DTYPE;
   if ((long)d->batch * d->in_channels * d->h * d->w > kMaxElems) return DK_ERR_TOO_LARGE;
   if (!offset_conv_supported(d->in_channels, d->out_channels, d->h, d->w)) return DK_ERR_UNSUPPORTED;
   return DK_OK;
@@ -661,7 +661,7 @@ int dk_offset_conv_supported(const dk_offset_conv_desc* desc) { return check_off
 
 int dk_offset_conv_worthwhile(const dk_offset_conv_desc* desc) {
   return check_offset_conv(desc) == DK_OK &&
-         offset_conv_worthwhile(desc->batch, desc->in_channels, desc->out_channels, desc->h, desc->w);
+         offset_conv_worthwhile(desc->batch, desc->in_channels, desc->out_channels, desc->h, desc->w, desc->dtype != DK_F32);
 }
 
 size_t dk_offset_conv_forward_workspace(const dk_offset_conv_desc* desc) {
@@ -677,12 +677,13 @@ int dk_offset_conv_forward(const dk_offset_conv_desc* desc, const void* input, c
   if (!input || !weight || !bias || !output) return DK_ERR_NULL_POINTER;
   const size_t need = offset_conv_workspace(desc->batch, desc->in_channels, desc->out_channels, desc->h, desc->w);
   if (!workspace || workspace_bytes < need) return DK_ERR_WORKSPACE;
-  if (!offset_conv_forward(desc->batch, desc->in_channels, desc->out_channels, desc->h, desc->w,
-                           static_cast<const float*>(input), static_cast<const float*>(weight),
-                           static_cast<const float*>(bias), static_cast<float*>(output), workspace,
-                           static_cast<hipStream_t>(stream)))
-    return DK_ERR_UNSUPPORTED;
-  return launch_status();
+  bool ok = false;
+  const int st = by_dtype(desc->dtype, [&]<typename T>() {
+    if constexpr (kHasFast<T>)
+      ok = offset_conv_forward<T>(desc->batch, desc->in_channels, desc->out_channels, desc->h, desc->w, in<T>(input),
+                                  in<T>(weight), in<T>(bias), out<T>(output), workspace, static_cast<hipStream_t>(stream));
+  });
+  return ok ? st : DK_ERR_UNSUPPORTED;
 }
 
 size_t dk_offset_conv_backward_weight_workspace(const dk_offset_conv_desc* desc) {
@@ -697,11 +698,13 @@ int dk_offset_conv_backward_weight(const dk_offset_conv_desc* desc, const void* 
   if (!out_grad || !input || !weight_grad) return DK_ERR_NULL_POINTER;
   const size_t need = offset_conv_wgrad_workspace(desc->batch, desc->in_channels, desc->out_channels, desc->h, desc->w);
   if (!workspace || workspace_bytes < need) return DK_ERR_WORKSPACE;
-  if (!offset_conv_wgrad(desc->batch, desc->in_channels, desc->out_channels, desc->h, desc->w,
-                         static_cast<const float*>(input), static_cast<const float*>(out_grad),
-                         static_cast<float*>(weight_grad), workspace, static_cast<hipStream_t>(stream)))
-    return DK_ERR_UNSUPPORTED;
-  return launch_status();
+  bool ok = false;
+  const int st = by_dtype(desc->dtype, [&]<typename T>() {
+    if constexpr (kHasFast<T>)
+      ok = offset_conv_wgrad<T>(desc->batch, desc->in_channels, desc->out_channels, desc->h, desc->w, in<T>(input),
+                                in<T>(out_grad), out<T>(weight_grad), workspace, static_cast<hipStream_t>(stream));
+  });
+  return ok ? st : DK_ERR_UNSUPPORTED;
 }
 
 size_t dk_offset_conv_backward_bias_workspace(const dk_offset_conv_desc* desc) {
@@ -713,14 +716,17 @@ int dk_offset_conv_backward_bias(const dk_offset_conv_desc* desc, const void* ou
                                  void* workspace, size_t workspace_bytes, void* stream) {
   if (!desc) return DK_ERR_NULL_POINTER;
   if (desc->batch < 0 || desc->out_channels <= 0 || desc->h <= 0 || desc->w <= 0) return DK_ERR_BAD_SHAPE;
-  if (desc->dtype != DK_F32) return DK_ERR_UNSUPPORTED;
+  if (desc->dtype != DK_F32 && desc->dtype != DK_F16 && desc->dtype != DK_BF16)
+    return desc->dtype == DK_F64 ? DK_ERR_UNSUPPORTED : DK_ERR_BAD_DTYPE;
   if ((long)desc->batch * desc->out_channels * desc->h * desc->w > kMaxElems) return DK_ERR_TOO_LARGE;
   if (!out_grad || !bias_grad) return DK_ERR_NULL_POINTER;
   const size_t need = offset_conv_bias_grad_workspace(desc->batch, desc->out_channels);
   if (need && (!workspace || workspace_bytes < need)) return DK_ERR_WORKSPACE;
-  offset_conv_bias_grad(desc->batch, desc->out_channels, desc->h * desc->w, static_cast<const float*>(out_grad),
-                        static_cast<float*>(bias_grad), workspace, static_cast<hipStream_t>(stream));
-  return launch_status();
+  return by_dtype(desc->dtype, [&]<typename T>() {
+    if constexpr (kHasFast<T>)
+      offset_conv_bias_grad<T>(desc->batch, desc->out_channels, desc->h * desc->w, in<T>(out_grad), out<T>(bias_grad),
+                               workspace, static_cast<hipStream_t>(stream));
+  });
 }
 
 // ---- N-d linear sample --------------------------------------------------------------------

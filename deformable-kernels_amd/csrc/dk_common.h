@@ -191,6 +191,18 @@ __device__ __forceinline__ float buf_ld(rsrc_t r, unsigned byte_off, const bf16_
   const unsigned short b = __builtin_amdgcn_raw_buffer_load_b16(r, (int)byte_off, 0, 0);
   return __uint_as_float(static_cast<uint32_t>(b) << 16);
 }
+// The same with a scalar part of the address (which the range check does not see: it must stay inside the buffer).
+__device__ __forceinline__ float buf_ld2(rsrc_t r, unsigned lane_off, int scalar_off, const float*) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(r, (int)lane_off, scalar_off, 0));
+}
+__device__ __forceinline__ float buf_ld2(rsrc_t r, unsigned lane_off, int scalar_off, const __half*) {
+  const unsigned short b = __builtin_amdgcn_raw_buffer_load_b16(r, (int)lane_off, scalar_off, 0);
+  return static_cast<float>(__builtin_bit_cast(_Float16, b));
+}
+__device__ __forceinline__ float buf_ld2(rsrc_t r, unsigned lane_off, int scalar_off, const bf16_t*) {
+  const unsigned short b = __builtin_amdgcn_raw_buffer_load_b16(r, (int)lane_off, scalar_off, 0);
+  return __uint_as_float(static_cast<uint32_t>(b) << 16);
+}
 __device__ __forceinline__ void buf_st(rsrc_t r, unsigned byte_off, float v, float*) {
   __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, v), r, (int)byte_off, 0, kStreamingStore);
 }

@@ -116,18 +116,20 @@ template <typename T>
 void generic_grad_filter(const Geo& g, bool deform, const T* gout, const T* x, const T* off,
                          const T* rot, T* gfilter, void* ws, hipStream_t stream);
 
-// dk_offset_conv.hip: the 3x3 offset-branch convolution (stride 1, padding 1, fp32)
+// dk_offset_conv.hip: the 3x3 offset-branch convolution (stride 1, padding 1; fp32 / fp16 / bf16 tensors, fp32 arithmetic)
 bool offset_conv_supported(int cin, int cout, int h, int w);
-bool offset_conv_worthwhile(int batch, int cin, int cout, int h, int w);
+bool offset_conv_worthwhile(int batch, int cin, int cout, int h, int w, bool sixteen_bit);
 size_t offset_conv_workspace(int batch, int cin, int cout, int h, int w);
 size_t offset_conv_bias_grad_workspace(int batch, int cout);
-void offset_conv_bias_grad(int batch, int cout, int plane, const float* gout, float* gbias, void* ws,
-                           hipStream_t stream);
+template <typename T>
+void offset_conv_bias_grad(int batch, int cout, int plane, const T* gout, T* gbias, void* ws, hipStream_t stream);
 size_t offset_conv_wgrad_workspace(int batch, int cin, int cout, int h, int w);
-bool offset_conv_wgrad(int batch, int cin, int cout, int h, int w, const float* x, const float* gout, float* gweight,
-                       void* ws, hipStream_t stream);
-bool offset_conv_forward(int batch, int cin, int cout, int h, int w, const float* x, const float* weight,
-                         const float* bias, float* out, void* ws, hipStream_t stream);
+template <typename T>
+bool offset_conv_wgrad(int batch, int cin, int cout, int h, int w, const T* x, const T* gout, T* gweight, void* ws,
+                       hipStream_t stream);
+template <typename T>
+bool offset_conv_forward(int batch, int cin, int cout, int h, int w, const T* x, const T* weight, const T* bias, T* out,
+                         void* ws, hipStream_t stream);
 
 // dk_local_nhwc.hip: the local operator on channels-last tensors, all dtypes, any geometry whose tables fit LDS
 bool nhwc_supported(const Geo& g, int dtype);

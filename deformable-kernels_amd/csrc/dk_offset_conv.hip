@@ -13,8 +13,9 @@
 // the 4 x 16 block of shifted inputs (B operand, one LDS read per lane: lane = (channel k,
 // pixel n); the channel pitch is 16 mod 64 words so the four channels of a read hit disjoint
 // banks).  The outputs beyond the 16th (two of the 18) are summed on the vector ALU, their
-// weights staged in LDS per chunk and read as broadcasts.  Stride 1, padding 1, no dilation, fp32; other cases are left
-// to the caller's library convolution.
+// weights staged in LDS per chunk and read as broadcasts.  Stride 1, padding 1, no dilation; other cases are left
+// to the caller's library convolution.  16-bit tensors (fp16 / bf16) take the same kernels: their elements are
+// converted to fp32 on the way into LDS, the products and sums are fp32, the results are rounded once.
 #include <algorithm>
 
 #include "dk_kernels.h"
@@ -49,23 +50,24 @@ struct ConvTile {
 
 // weights [cout][cin][3][3] -> w16 [9][cin][16] (outputs 0..15, zero where cout < 16) and
 // wrest [9][cin][rest] (outputs 16..)
-__global__ void conv_pack_weights_kernel(const float* __restrict__ w, int cout, int cin, int rest,
+template <typename T>
+__global__ void conv_pack_weights_kernel(const T* __restrict__ w, int cout, int cin, int rest,
                                          float* __restrict__ w16, float* __restrict__ wrest) {
   const int idx = blockIdx.x * blockDim.x + threadIdx.x;
   if (idx < 9 * cin * 16) {
     const int m = idx % 16, c = idx / 16 % cin, t = idx / 16 / cin;
-    w16[idx] = m < cout ? w[((size_t)m * cin + c) * 9 + t] : 0.f;
+    w16[idx] = m < cout ? ld(w + ((size_t)m * cin + c) * 9 + t) : 0.f;
   }
   if (idx < 9 * cin * rest) {
     const int o = 16 + idx % rest, c = idx / rest % cin, t = idx / rest / cin;
-    wrest[idx] = w[((size_t)o * cin + c) * 9 + t];
+    wrest[idx] = ld(w + ((size_t)o * cin + c) * 9 + t);
   }
 }
 
-template <int W, int REST>
+template <typename T, int W, int REST>
 __global__ __launch_bounds__(kCvBlock, 2) void offset_conv_forward_kernel(
-    ConvGeo g, const float* __restrict__ x, const float* __restrict__ w16, const float* __restrict__ wrest,
-    const float* __restrict__ bias, float* __restrict__ out, float* __restrict__ partial, int ksplit) {
+    ConvGeo g, const T* __restrict__ x, const float* __restrict__ w16, const float* __restrict__ wrest,
+    const T* __restrict__ bias, T* __restrict__ out, float* __restrict__ partial, int ksplit) {
   extern __shared__ __align__(16) float xs[];  // [kCvChunk][PS], the chunk's VALU-path weights [kCvChunk][9][REST], its MFMA weights [9][256]
   constexpr int TH = ConvTile<W>::TH, SEGS = ConvTile<W>::SEGS, RS = ConvTile<W>::RS, PS = ConvTile<W>::PS;
   constexpr int kStage = (kCvChunk / 4) * (TH + 2) * SEGS;  // row segments of 64 columns a wave stages per chunk
@@ -118,7 +120,7 @@ __global__ __launch_bounds__(kCvBlock, 2) void offset_conv_forward_kernel(
   unsigned vcol[SEGS];
 #pragma unroll
   for (int sg = 0; sg < SEGS; ++sg)
-    vcol[sg] = sg * 64 + lane < W ? (unsigned)((sg * 64 + lane) * 4) : kOutOfRange;
+    vcol[sg] = sg * 64 + lane < W ? (unsigned)((sg * 64 + lane) * sizeof(T)) : kOutOfRange;
   const int lds_row0 = wave * PS + 1 + lane;  // + immediate per row segment
   float stage[kStage];
   // the chunk's weights of the outputs beyond the 16th go through LDS as well: read as scalars
@@ -144,9 +146,8 @@ __global__ __launch_bounds__(kCvBlock, 2) void offset_conv_forward_kernel(
       const int chq = i / ((TH + 2) * SEGS), ry = i / SEGS % (TH + 2), sg = i % SEGS;                      \
       const int row = r0 - 1 + ry;                                                                         \
       const bool ok = row >= 0 && row < g.h;                                                               \
-      const int soff = ok ? ((wave + 4 * chq) * g.h + row) * W * 4 : 0;                                    \
-      stage[i] = __builtin_bit_cast(                                                                       \
-          float, __builtin_amdgcn_raw_buffer_load_b32(rx, (int)(ok ? vcol[sg] : kOutOfRange), soff, 0));   \
+      const int soff = ok ? ((wave + 4 * chq) * g.h + row) * W * (int)sizeof(T) : 0;                       \
+      stage[i] = buf_ld2(rx, ok ? vcol[sg] : kOutOfRange, soff, x);                                        \
     }                                                                                                      \
   }
 
@@ -218,9 +219,18 @@ __global__ __launch_bounds__(kCvBlock, 2) void offset_conv_forward_kernel(
   }
 
 #undef DK_LOAD_CHUNK
-  // results: lane holds outputs 4 * (lane / 16) + j of pixel lane % 16 of each of its groups
-  float* on = (ksplit > 1 ? partial + (size_t)split * g.batch * g.cout * plane : out) + (size_t)n * g.cout * plane;
+  // results: lane holds outputs 4 * (lane / 16) + j of pixel lane % 16 of each of its groups.  One split: the
+  // result with its bias, in the tensor's type; several: fp32 partial sums (the bias with split 0), added afterwards.
+  float* pn = partial + ((size_t)split * g.batch + n) * g.cout * plane;
+  T* on = out + (size_t)n * g.cout * plane;
   const bool add_bias = split == 0;
+  auto put = [&](int o, int at, float v) {
+    v += add_bias ? ld(bias + o) : 0.f;
+    if (ksplit > 1)
+      pn[(size_t)o * plane + at] = v;
+    else
+      st(on + (size_t)o * plane + at, v);
+  };
 #pragma unroll
   for (int i = 0; i < GPW; ++i) {
     const int q = (wave + 4 * i) * 16 + (lane & 15);
@@ -229,7 +239,7 @@ __global__ __launch_bounds__(kCvBlock, 2) void offset_conv_forward_kernel(
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
         const int o = 4 * (lane >> 4) + j;
-        if (o < g.cout) on[(size_t)o * plane + row * W + q % W] = acc[i][j] + (add_bias ? bias[o] : 0.f);
+        if (o < g.cout) put(o, row * W + q % W, acc[i][j]);
       }
     }
   }
@@ -240,8 +250,7 @@ __global__ __launch_bounds__(kCvBlock, 2) void offset_conv_forward_kernel(
       const int row = r0 + q / W;
       if (q < tile_pix && row < g.h) {
 #pragma unroll
-        for (int o = 0; o < REST; ++o)
-          on[(size_t)(16 + o) * plane + row * W + q % W] = racc[j][o] + (add_bias ? bias[16 + o] : 0.f);
+        for (int o = 0; o < REST; ++o) put(16 + o, row * W + q % W, racc[j][o]);
       }
     }
   }
@@ -276,9 +285,9 @@ struct WgradTile {
   static_assert(PSX >= ROWS * RS && PSX % 64 == 4 && GP >= PSX + 2 * MARGIN, "tile layout");
 };
 
-template <int W, int NT>
+template <typename T, int W, int NT>
 __global__ __launch_bounds__(kWgBlock, 1) void offset_conv_wgrad_kernel(
-    ConvGeo g, const float* __restrict__ x, const float* __restrict__ gout, float* __restrict__ partial, int parts) {
+    ConvGeo g, const T* __restrict__ x, const T* __restrict__ gout, float* __restrict__ partial, int parts) {
   using Tl = WgradTile<W>;
   constexpr int TH = Tl::TH, RS = Tl::RS, PSX = Tl::PSX, GP = Tl::GP, SEGS = Tl::SEGS;
   extern __shared__ __align__(16) float lds[];
@@ -318,7 +327,7 @@ __global__ __launch_bounds__(kWgBlock, 1) void offset_conv_wgrad_kernel(
   constexpr int kGStage = kGPlanes * TH * SEGS;
   unsigned vcol[SEGS];
 #pragma unroll
-  for (int sg = 0; sg < SEGS; ++sg) vcol[sg] = sg * 64 + lane < W ? (unsigned)((sg * 64 + lane) * 4) : kOutOfRange;
+  for (int sg = 0; sg < SEGS; ++sg) vcol[sg] = sg * 64 + lane < W ? (unsigned)((sg * 64 + lane) * sizeof(T)) : kOutOfRange;
   float xst[kXStage], gst[kGStage];
 #define DK_LOAD_ITEM(ITEM)                                                                                     \
   {                                                                                                            \
@@ -329,17 +338,15 @@ __global__ __launch_bounds__(kWgBlock, 1) void offset_conv_wgrad_kernel(
       const int chq = i / ((TH + 2) * SEGS), ry = i / SEGS % (TH + 2), sg = i % SEGS;                          \
       const int row = r0_ - 1 + ry;                                                                            \
       const bool ok = row >= 0 && row < g.h;                                                                   \
-      const int soff = ok ? ((wave + kWgWaves * chq) * g.h + row) * W * 4 : 0;                                 \
-      xst[i] = __builtin_bit_cast(                                                                             \
-          float, __builtin_amdgcn_raw_buffer_load_b32(rx, (int)(ok ? vcol[sg] : kOutOfRange), soff, 0));       \
+      const int soff = ok ? ((wave + kWgWaves * chq) * g.h + row) * W * (int)sizeof(T) : 0;                    \
+      xst[i] = buf_ld2(rx, ok ? vcol[sg] : kOutOfRange, soff, x);                                              \
     }                                                                                                          \
     _Pragma("unroll") for (int i = 0; i < kGStage; ++i) {                                                      \
       const int pq = i / (TH * SEGS), ry = i / SEGS % TH, sg = i % SEGS;                                       \
       const int o = wave + kWgWaves * pq, row = r0_ + ry;                                                      \
       const bool ok = o < g.cout && row < g.h;                                                                 \
-      const int soff = ok ? (o * g.h + row) * W * 4 : 0;                                                       \
-      gst[i] = __builtin_bit_cast(                                                                             \
-          float, __builtin_amdgcn_raw_buffer_load_b32(rg, (int)(ok ? vcol[sg] : kOutOfRange), soff, 0));       \
+      const int soff = ok ? (o * g.h + row) * W * (int)sizeof(T) : 0;                                          \
+      gst[i] = buf_ld2(rg, ok ? vcol[sg] : kOutOfRange, soff, gout);                                           \
     }                                                                                                          \
   }
 
@@ -399,9 +406,10 @@ __global__ __launch_bounds__(kWgBlock, 1) void offset_conv_wgrad_kernel(
 }
 
 // gW[o][c][t] = sum over parts of partial[part][chunk(c)][row tile][...], parts added in order
+template <typename T>
 __global__ __launch_bounds__(256) void offset_conv_wgrad_reduce_kernel(const float* __restrict__ partial, int parts,
                                                                        int nchunks, int nt, int cout, int cin,
-                                                                       float* __restrict__ gw) {
+                                                                       T* __restrict__ gw) {
   const int idx = blockIdx.x * 256 + threadIdx.x;  // = (o * cin + c) * 9 + t
   if (idx >= cout * cin * 9) return;
   const int t = idx % 9, c = idx / 9 % cin, o = idx / 9 / cin;
@@ -411,20 +419,21 @@ __global__ __launch_bounds__(256) void offset_conv_wgrad_reduce_kernel(const flo
   const float* p = partial + (size_t)(c / kCvChunk) * (nt * 256) + j * 256 + 4 * l + r;
   float s = 0.f;
   for (int q = 0; q < parts; ++q) s += p[(size_t)q * nchunks * (nt * 256)];
-  gw[idx] = s;
+  st(gw + idx, s);
 }
 
 size_t round256(size_t n) { return (n + 255) / 256 * 256; }
 
 // Bias gradient: partial[n][o] = sum over the pixels of gout[n][o]; one workgroup per plane.
-__global__ __launch_bounds__(kCvBlock) void conv_bias_grad_kernel(const float* __restrict__ gout, int plane,
+template <typename T>
+__global__ __launch_bounds__(kCvBlock) void conv_bias_grad_kernel(const T* __restrict__ gout, int plane,
                                                                   float* __restrict__ partial) {
   __shared__ float wave_sums[kCvBlock / 64];
-  const float* p = gout + (size_t)blockIdx.x * plane;
+  const T* p = gout + (size_t)blockIdx.x * plane;
   float s[4] = {0.f, 0.f, 0.f, 0.f};
   for (int i = threadIdx.x; i < plane; i += 4 * kCvBlock) {
 #pragma unroll
-    for (int u = 0; u < 4; ++u) s[u] += i + u * kCvBlock < plane ? p[i + u * kCvBlock] : 0.f;
+    for (int u = 0; u < 4; ++u) s[u] += i + u * kCvBlock < plane ? ld(p + i + u * kCvBlock) : 0.f;
   }
   const float t = wave_sum((s[0] + s[1]) + (s[2] + s[3]));
   if ((threadIdx.x & 63) == 0) wave_sums[threadIdx.x >> 6] = t;
@@ -437,11 +446,11 @@ __global__ __launch_bounds__(kCvBlock) void conv_bias_grad_kernel(const float* _
 // gbias[o] = sum over images and pixels of gout[n][o][.]; workspace: batch * cout floats
 size_t offset_conv_bias_grad_workspace(int batch, int cout) { return (size_t)batch * cout * sizeof(float); }
 
-void offset_conv_bias_grad(int batch, int cout, int plane, const float* gout, float* gbias, void* ws,
-                           hipStream_t stream) {
+template <typename T>
+void offset_conv_bias_grad(int batch, int cout, int plane, const T* gout, T* gbias, void* ws, hipStream_t stream) {
   float* partial = static_cast<float*>(ws);
-  if (batch > 0) conv_bias_grad_kernel<<<batch * cout, kCvBlock, 0, stream>>>(gout, plane, partial);
-  launch_reduce_partials<float, float>(partial, batch, cout, gbias, stream);  // the images, added in order
+  if (batch > 0) conv_bias_grad_kernel<T><<<batch * cout, kCvBlock, 0, stream>>>(gout, plane, partial);
+  launch_reduce_partials<float, T>(partial, batch, cout, gbias, stream);  // the images, added in order
 }
 
 bool offset_conv_supported(int cin, int cout, int h, int w) {
@@ -460,11 +469,13 @@ int forward_splits(int batch, int cin, int h, int w) {
 }
 
 // Whether the kernels are also the faster choice (measured against the library convolution on
-// MI355X, batch 64, forward + backward): on planes 28 wide and wider (56 and 112: by 30-40 %)
+// MI355X, forward + backward): float32, batch 64: on planes 28 wide and wider (56 and 112: by 30-40 %)
 // once the grid -- (image, row tile) items times the input-channel splits -- gives about a
 // workgroup per CU; on the 14- and 7-wide planes the two are within 10 % of each other either way.
-bool offset_conv_worthwhile(int batch, int cin, int cout, int h, int w) {
-  if (!offset_conv_supported(cin, cout, h, w) || w < 28) return false;
+// 16-bit tensors, batch 128 (the library multiplies them on 16-bit matrix instructions, these kernels in fp32):
+// 112 wide 955 against 1399 us, 56 wide 930 / 1274, 28 wide 394 / 370, 14 wide 298 / 224: from 56 columns on.
+bool offset_conv_worthwhile(int batch, int cin, int cout, int h, int w, bool sixteen_bit) {
+  if (!offset_conv_supported(cin, cout, h, w) || w < (sixteen_bit ? 56 : 28)) return false;
   const int th = w <= 56 ? 8 : 4;
   return (long)batch * ceil_div(h, th) * forward_splits(batch, cin, h, w) >= 192;
 }
@@ -476,8 +487,9 @@ size_t offset_conv_workspace(int batch, int cin, int cout, int h, int w) {
          (ks > 1 ? (size_t)ks * batch * cout * h * w * sizeof(float) : 0);
 }
 
-bool offset_conv_forward(int batch, int cin, int cout, int h, int w, const float* x, const float* weight,
-                         const float* bias, float* out, void* ws, hipStream_t stream) {
+template <typename T>
+bool offset_conv_forward(int batch, int cin, int cout, int h, int w, const T* x, const T* weight, const T* bias, T* out,
+                         void* ws, hipStream_t stream) {
   if (!offset_conv_supported(cin, cout, h, w)) return false;
   if (batch == 0) return true;
   const int rest = std::max(0, cout - 16);
@@ -486,7 +498,7 @@ bool offset_conv_forward(int batch, int cin, int cout, int h, int w, const float
   float* wrest = reinterpret_cast<float*>(after16);
   float* partial = reinterpret_cast<float*>(after16 + round256((size_t)9 * cin * rest * sizeof(float)));
   const int ksplit = forward_splits(batch, cin, h, w);
-  conv_pack_weights_kernel<<<ceil_div(9 * cin * 16, 256), 256, 0, stream>>>(weight, cout, cin, rest, w16, wrest);
+  conv_pack_weights_kernel<T><<<ceil_div(9 * cin * 16, 256), 256, 0, stream>>>(weight, cout, cin, rest, w16, wrest);
   ConvGeo g;
   g.batch = batch, g.cin = cin, g.cout = cout, g.h = h;
 #define DK_LAUNCH(WW, REST)                                                                             \
@@ -494,8 +506,8 @@ bool offset_conv_forward(int batch, int cin, int cout, int h, int w, const float
     g.tiles = ceil_div(h, ConvTile<WW>::TH);                                                            \
     const size_t lds = (size_t)(kCvChunk * (ConvTile<WW>::PS + 9 * REST) + 9 * 256) * sizeof(float);    \
     const unsigned grid = (unsigned)xcd_grid_size((long)batch * g.tiles * ksplit);                      \
-    offset_conv_forward_kernel<WW, REST><<<grid, kCvBlock, lds, stream>>>(g, x, w16, wrest, bias, out,  \
-                                                                         partial, ksplit);              \
+    offset_conv_forward_kernel<T, WW, REST><<<grid, kCvBlock, lds, stream>>>(g, x, w16, wrest, bias, out, \
+                                                                            partial, ksplit);            \
   }
 #define DK_WIDTH(REST)                       \
   switch (w) {                               \
@@ -514,7 +526,7 @@ bool offset_conv_forward(int batch, int cin, int cout, int h, int w, const float
   }
 #undef DK_WIDTH
 #undef DK_LAUNCH
-  if (ksplit > 1) launch_reduce_partials<float, float>(partial, ksplit, (long)batch * cout * h * w, out, stream);
+  if (ksplit > 1) launch_reduce_partials<float, T>(partial, ksplit, (long)batch * cout * h * w, out, stream);
   return true;
 }
 
@@ -530,8 +542,9 @@ size_t offset_conv_wgrad_workspace(int batch, int cin, int cout, int h, int w) {
   return (size_t)wgrad_parts(batch, cin, h, w) * (cin / kCvChunk) * nt * 256 * sizeof(float);
 }
 
-bool offset_conv_wgrad(int batch, int cin, int cout, int h, int w, const float* x, const float* gout, float* gweight,
-                       void* ws, hipStream_t stream) {
+template <typename T>
+bool offset_conv_wgrad(int batch, int cin, int cout, int h, int w, const T* x, const T* gout, T* gweight, void* ws,
+                       hipStream_t stream) {
   if (!offset_conv_supported(cin, cout, h, w)) return false;
   const int nt = ceil_div(cout * 9, 16), nchunks = cin / kCvChunk;
   const int parts = wgrad_parts(batch, cin, h, w);
@@ -541,7 +554,7 @@ bool offset_conv_wgrad(int batch, int cin, int cout, int h, int w, const float* 
   bool ok = true;
 #define DK_LAUNCH(WW, NT)                                                                                      \
   {                                                                                                            \
-    auto kernel = offset_conv_wgrad_kernel<WW, NT>;                                                            \
+    auto kernel = offset_conv_wgrad_kernel<T, WW, NT>;                                                            \
     g.tiles = ceil_div(h, WgradTile<WW>::TH);                                                                  \
     const size_t lds = (size_t)(kCvChunk * WgradTile<WW>::PSX + cout * WgradTile<WW>::GP) * sizeof(float);     \
     const size_t lds_red = (size_t)NT * 256 * sizeof(float);                                                   \
@@ -571,9 +584,18 @@ bool offset_conv_wgrad(int batch, int cin, int cout, int h, int w, const float* 
 #undef DK_LAUNCH
   if (!ok) return false;
   const int total = cout * cin * 9;
-  offset_conv_wgrad_reduce_kernel<<<ceil_div(total, 256), 256, 0, stream>>>(partial, batch > 0 ? parts : 0, nchunks, nt,
-                                                                           cout, cin, gweight);
+  offset_conv_wgrad_reduce_kernel<T><<<ceil_div(total, 256), 256, 0, stream>>>(partial, batch > 0 ? parts : 0, nchunks,
+                                                                              nt, cout, cin, gweight);
   return true;
 }
+
+#define DK_INSTANTIATE(T)                                                                                          \
+  template void offset_conv_bias_grad<T>(int, int, int, const T*, T*, void*, hipStream_t);                         \
+  template bool offset_conv_forward<T>(int, int, int, int, int, const T*, const T*, const T*, T*, void*, hipStream_t); \
+  template bool offset_conv_wgrad<T>(int, int, int, int, int, const T*, const T*, T*, void*, hipStream_t);
+DK_INSTANTIATE(float)
+DK_INSTANTIATE(__half)
+DK_INSTANTIATE(bf16_t)
+#undef DK_INSTANTIATE
 
 }  // namespace dk

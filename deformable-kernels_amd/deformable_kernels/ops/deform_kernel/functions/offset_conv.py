@@ -2,7 +2,8 @@
 ``modules/deform_kernel.py:165-168``, applied at ``:214``).
 
 ``offset_conv(input, weight, bias, stride, padding, dilation)`` returns what
-``torch.nn.functional.conv2d`` returns.  For float32 GPU tensors it runs
+``torch.nn.functional.conv2d`` returns.  For float32, float16 and bfloat16 GPU tensors (all of one dtype; the
+kernels multiply and add in float32 and round the results once) it runs
 
   * the forward and the weight gradient on the library's matrix-core kernels where they apply
     and are the faster choice (stride 1, padding 1, dilation 1, input channels a multiple of 16,
@@ -13,7 +14,7 @@
   * everything else -- the input gradient, and forward / weight gradient of the other shapes --
     on the framework's convolution routines.
 
-Other dtypes, CPU tensors and autocast regions go to ``F.conv2d`` unchanged.
+float64, CPU tensors, mixed dtypes and autocast regions go to ``F.conv2d`` unchanged.
 """
 import torch
 import torch.nn.functional as F
@@ -31,13 +32,17 @@ def _pair(v):
 
 def _desc(input, weight, out=None):
     h, w = (input.size(2), input.size(3)) if out is None else (out.size(2), out.size(3))
-    return _lib.OffsetConvDesc(input.size(0), input.size(1), weight.size(0), h, w, _lib.DK_F32)
+    return _lib.OffsetConvDesc(input.size(0), input.size(1), weight.size(0), h, w, _lib.dtype_tag(input))
+
+
+_NATIVE_DTYPES = (torch.float32, torch.float16, torch.bfloat16)
 
 
 def _float32_gpu(input, weight, bias):
-    if not (input.is_cuda and weight.is_cuda and input.dtype == torch.float32 and weight.dtype == torch.float32):
+    """Tensors the library's kernels take: on the GPU, all float32 or all float16 or all bfloat16."""
+    if not (input.is_cuda and weight.is_cuda and input.dtype in _NATIVE_DTYPES and weight.dtype == input.dtype):
         return False
-    if bias is not None and not (bias.is_cuda and bias.dtype == torch.float32):
+    if bias is not None and not (bias.is_cuda and bias.dtype == input.dtype):
         return False
     return input.dim() == 4 and weight.dim() == 4 and not torch.is_autocast_enabled()
 

@@ -281,7 +281,8 @@ int dk_nd_linear_sample_backward_coord(const dk_nd_desc *desc, const void *out_g
  * (modules/deform_kernel.py:165-168: nn.Conv2d(in_planes, rotation_groups*k*k*2, k, stride,
  * padding, dilation, bias=True), applied at :214).  The reference calls the framework's
  * convolution there; this entry point is a faster kernel for that one shape family: stride 1,
- * padding 1, dilation 1, float32, in_channels a multiple of 16, out_channels <= 16 or 18 or 20,
+ * padding 1, dilation 1, float32 / float16 / bfloat16 tensors (fp32 products and sums, results rounded
+ * once), in_channels a multiple of 16, out_channels <= 16 or 18 or 20,
  * width 7, 14, 28, 56 or 112.  dk_offset_conv_supported() tells whether a shape is covered,
  * dk_offset_conv_worthwhile() whether it is also expected to beat the library convolution
  * (56- and 112-wide planes with enough images to fill the GPU); the caller keeps its library
@@ -290,7 +291,7 @@ int dk_nd_linear_sample_backward_coord(const dk_nd_desc *desc, const void *out_g
  *   bias [out_channels], output [batch, out_channels, h, w]; workspace: packed weights. */
 typedef struct dk_offset_conv_desc {
   int32_t batch, in_channels, out_channels, h, w;
-  int32_t dtype; /* DK_F32 */
+  int32_t dtype; /* DK_F32, DK_F16 or DK_BF16 */
 } dk_offset_conv_desc;
 int dk_offset_conv_supported(const dk_offset_conv_desc *desc);
 int dk_offset_conv_worthwhile(const dk_offset_conv_desc *desc);
@@ -308,7 +309,7 @@ int dk_offset_conv_backward_weight(const dk_offset_conv_desc *desc, const void *
                                    void *stream);
 
 /* Gradient of that convolution's bias: bias_grad[o] = sum over images and pixels of
- * out_grad[n][o][.], float32, any shape; the images are added in a fixed order.  (The input
+ * out_grad[n][o][.], any shape; fp32 sums, the images are added in a fixed order.  (The input
  * gradient of the convolution is left to the caller's library.) */
 size_t dk_offset_conv_backward_bias_workspace(const dk_offset_conv_desc *desc);
 int dk_offset_conv_backward_bias(const dk_offset_conv_desc *desc, const void *out_grad, void *bias_grad,

@@ -57,6 +57,35 @@ def test_weight_and_bias_gradients_match_float64(shape):
     assert rel_err(x.grad.cpu(), xd.grad.cpu()) < 1e-5
 
 
+@pytest.mark.parametrize("dtype,tol", [(torch.float16, 2e-3), (torch.bfloat16, 1e-2)])
+@pytest.mark.parametrize("shape", [(2, 16, 5, 7, 18), (3, 32, 14, 14, 18), (2, 144, 56, 56, 18), (1, 32, 9, 112, 18),
+                                   (2, 32, 56, 56, 16), (40, 32, 56, 56, 18), (64, 960, 7, 7, 18)])
+def test_sixteen_bit_tensors_match_float64_on_the_rounded_inputs(shape, dtype, tol):
+    """float16 / bfloat16 tensors through the same kernels: fp32 products and sums, so the error against the
+    float64 convolution of the rounded inputs is the results' own rounding (forward; weight and bias gradient,
+    whose partial sums are fp32)."""
+    from deformable_kernels.ops.deform_kernel.functions import offset_conv, offset_conv_supported
+    N, C, H, W, O = shape
+    g = torch.Generator().manual_seed(37)
+    dev = torch.device("cuda:0")
+    x = torch.randn(N, C, H, W, generator=g).to(dtype).to(dev).requires_grad_()
+    w = (torch.randn(O, C, 3, 3, generator=g) * 0.05).to(dtype).to(dev).requires_grad_()
+    b = torch.randn(O, generator=g).to(dtype).to(dev).requires_grad_()
+    gout = torch.randn(N, O, H, W, generator=g).to(dtype).to(dev)
+    assert offset_conv_supported(x, w, b, 1, 1, 1)
+    out = offset_conv(x, w, b, force=True)
+    assert out.dtype == dtype
+    out.backward(gout)
+    xd, wd, bd = [t.detach().double().requires_grad_() for t in (x, w, b)]
+    want = F.conv2d(xd, wd, bd, padding=1)
+    want.backward(gout.double())
+    assert rel_err(out.detach().double().cpu(), want.detach().cpu()) < tol
+    assert w.grad.dtype == dtype and b.grad.dtype == dtype
+    assert rel_err(w.grad.double().cpu(), wd.grad.cpu()) < tol
+    assert rel_err(b.grad.double().cpu(), bd.grad.cpu()) < tol
+    assert rel_err(x.grad.double().cpu(), xd.grad.cpu()) < tol   # the library's routine
+
+
 def test_unsupported_calls_go_to_the_library_convolution():
     from deformable_kernels.ops.deform_kernel.functions import offset_conv, offset_conv_supported
     dev = torch.device("cuda:0")
@@ -67,9 +96,10 @@ def test_unsupported_calls_go_to_the_library_convolution():
     x2 = torch.randn(2, 32, 56, 56, device=dev)
     w2 = torch.randn(18, 32, 3, 3, device=dev)
     assert not offset_conv_supported(x2, w2, None, 2, 1, 1)          # stride 2
-    assert not offset_conv_supported(x2.half(), w2.half(), None, 1, 1, 1)
+    assert not offset_conv_supported(x2.double(), w2.double(), None, 1, 1, 1)   # float64
+    assert not offset_conv_supported(x2.half(), w2, None, 1, 1, 1)              # mixed dtypes
     assert torch.equal(offset_conv(x2, w2, None, stride=2), F.conv2d(x2, w2, None, 2, 1, 1))
-    assert torch.equal(offset_conv(x2.half(), w2.half(), None), F.conv2d(x2.half(), w2.half(), None, 1, 1, 1))
+    assert torch.equal(offset_conv(x2.double(), w2.double(), None), F.conv2d(x2.double(), w2.double(), None, 1, 1, 1))
 
 
 @pytest.mark.parametrize("conv", [(2, 1, 1), (1, 0, 1), (1, 2, 2), (2, 1, 1, 24)])
