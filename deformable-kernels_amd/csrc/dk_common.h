@@ -191,7 +191,8 @@ __device__ __forceinline__ float buf_ld(rsrc_t r, unsigned byte_off, const bf16_
   const unsigned short b = __builtin_amdgcn_raw_buffer_load_b16(r, (int)byte_off, 0, 0);
   return __uint_as_float(static_cast<uint32_t>(b) << 16);
 }
-// The same with a scalar part of the address (which the range check does not see: it must stay inside the buffer).
+// The same with a scalar part of the address.  The range check compares the lane's offset with the buffer's
+// size less the scalar part, so the descriptor must cover every position the scalar part selects.
 __device__ __forceinline__ float buf_ld2(rsrc_t r, unsigned lane_off, int scalar_off, const float*) {
   return __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(r, (int)lane_off, scalar_off, 0));
 }

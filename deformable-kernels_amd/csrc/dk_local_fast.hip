@@ -637,8 +637,6 @@ __global__ __launch_bounds__(kBlock, OCC) void local_grad_rotation_kernel(
 #pragma unroll
   for (int t = 0; t < K; ++t) sb[t] = sc[t] = sd[t] = 0.f;
 
-  // ch_per_pass + 1 tables: the spare one is read, times zero, by the odd channel out of a pair
-  for (int e = threadIdx.x; e < (ch_per_pass + 1) * Tb::SIZE; e += blockDim.x) tbl[e] = 0.f;
   for (int j0 = c_begin; j0 < c_end; j0 += ch_per_pass) {
     const int nch = min(ch_per_pass, c_end - j0);
     __syncthreads();
@@ -650,23 +648,30 @@ __global__ __launch_bounds__(kBlock, OCC) void local_grad_rotation_kernel(
     const size_t x_step = (size_t)g.groups * in_plane, g_step = (size_t)g.groups * out_plane;
 
     typedef typename Pair<T>::raw pair_t;
-    float xv[2][NLOAD], gv[2];
-    pair_t xq[2][KH];
+    // loads run DEPTH - 1 channels ahead of the arithmetic: with one channel ahead the bytes a CU has
+    // in flight (about 1.5 KB per wave) cover the memory latency only up to 3 TB/s
+    constexpr int DEPTH = (ROWS && OCC < 5) ? 4 : 2;
+    float xv[DEPTH][NLOAD], gv[DEPTH];
+    pair_t xq[DEPTH][KH];
+    // one descriptor per tensor for the whole pass, up to the end of its last channel's plane: a lane's
+    // offset is either inside a plane or kOutOfRange, the channel is a scalar offset kept to the pass's
+    // channels (what a load past the last channel returns is never accumulated)
+    const rsrc_t rg = plane_rsrc(gp, (int)((nch - 1) * g_step) + out_plane);
+    const rsrc_t rx = plane_rsrc(xp, (int)((nch - 1) * x_step) + in_plane);
+    const int g_bytes = (int)(g_step * sizeof(T)), x_bytes = (int)(x_step * sizeof(T));
     auto load = [&](int s, int j) {
-      const rsrc_t rg = plane_rsrc(gp + (size_t)j * g_step, j < nch ? out_plane : 0);
-      gv[s] = buf_ld(rg, goff, gout);
+      const int jc = min(j, nch - 1);
+      gv[s] = buf_ld2(rg, goff, jc * g_bytes, gout);
       if (S2) {
-        const T* plane = xp + (size_t)min(j, nch - 1) * x_step;  // past the last channel gv is 0
+        const T* plane = xp + (size_t)jc * x_step;
 #pragma unroll
         for (int r = 0; r < KH; ++r) xq[s][r] = *reinterpret_cast<const pair_t*>(plane + pe[r]);
       } else {
-        const rsrc_t rx = plane_rsrc(xp + (size_t)j * x_step, j < nch ? in_plane : 0);
 #pragma unroll
-        for (int t = 0; t < NLOAD; ++t) xv[s][t] = buf_ld(rx, soff[t], x);
+        for (int t = 0; t < NLOAD; ++t) xv[s][t] = buf_ld2(rx, soff[t], jc * x_bytes, x);
       }
     };
     auto accumulate = [&](int s, int j) {
-      // j == nch happens (odd nch) with zero inputs: that table is a stale or the zeroed spare one
       const float* tb = tbl + j * Tb::SIZE;
 #pragma unroll
       for (int t = 0; t < K; ++t) {
@@ -689,12 +694,14 @@ __global__ __launch_bounds__(kBlock, OCC) void local_grad_rotation_kernel(
         sd[t] = fmaf(ps, q.w, sd[t]);
       }
     };
-    load(0, 0);
-    for (int j = 0; j < nch; j += 2) {
-      load(1, j + 1);
-      accumulate(0, j);
-      load(0, j + 2);
-      accumulate(1, j + 1);
+#pragma unroll
+    for (int u = 0; u < DEPTH - 1; ++u) load(u, u);
+    for (int j = 0; j < nch; j += DEPTH) {
+#pragma unroll
+      for (int u = 0; u < DEPTH; ++u) {
+        load((u + DEPTH - 1) % DEPTH, j + u + DEPTH - 1);
+        if (j + u < nch) accumulate(u, j + u);
+      }
     }
   }
 
@@ -1491,8 +1498,10 @@ bool run_grad_rotation(const Geo& g, const T* gout, const T* x, const T* rot, co
   using Tb = WideTable<SH, SW>;
   const int cpg = g.channel / g.groups;
   const int splits = rotation_splits(g);
-  const int per = std::min(ceil_div(cpg, splits), 36);  // channels staged per pass
-  const size_t lds = (size_t)(per + 1) * Tb::SIZE * sizeof(float);
+  // channels staged per pass; their planes stay within the 2 GiB a scalar byte offset reaches
+  const long step_bytes = (long)g.groups * std::max(g.in_h * g.in_w, g.out_h * g.out_w) * (long)sizeof(T);
+  const int per = (int)std::max(1L, std::min<long>(std::min(ceil_div(cpg, splits), 36), ((1L << 31) - 1) / step_bytes));
+  const size_t lds = (size_t)per * Tb::SIZE * sizeof(float);
   const unsigned grid = (unsigned)xcd_grid_size((long)ceil_div(g.out_h * g.out_w, rotation_tile(g)) * splits * g.batch * g.groups);
   if (same_width_geometry(g))
     if (grid > 5 * 256)
