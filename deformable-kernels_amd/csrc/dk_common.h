@@ -217,4 +217,14 @@ __device__ __forceinline__ void buf_st(rsrc_t r, unsigned byte_off, float v, bf1
   __builtin_amdgcn_raw_buffer_store_b16(t.bits, r, (int)byte_off, 0, kMergedStore);
 }
 
+// Two floats rounded to bfloat16 by one instruction (v_cvt_pk_bf16_f32), a in the lower half; and the two halves
+// of such a pair back as floats.
+__device__ __forceinline__ unsigned pack_bf16(float a, float b) {
+  typedef float f2 __attribute__((ext_vector_type(2)));
+  typedef __bf16 b2 __attribute__((ext_vector_type(2)));
+  return __builtin_bit_cast(unsigned, __builtin_convertvector(f2{a, b}, b2));
+}
+__device__ __forceinline__ float bf16_lo(unsigned pair) { return __uint_as_float(pair << 16); }
+__device__ __forceinline__ float bf16_hi(unsigned pair) { return __uint_as_float(pair & 0xffff0000u); }
+
 }  // namespace dk

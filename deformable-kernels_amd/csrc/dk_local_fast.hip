@@ -572,6 +572,7 @@ __global__ __launch_bounds__(kBlock, OCC) void local_grad_rotation_kernel(
   constexpr bool ROWS = MODE == 1, S2 = MODE == 2;  // MODE 0: one load per tap
   constexpr int NLOAD = MODE == 0 ? K : KH;          // input loads per channel
   constexpr int PIX = ROWS ? kRowPix : S2 ? kS2Pix : kBlock;  // pixels per workgroup
+  constexpr bool PAIRS = ROWS && sizeof(T) == 2;  // 16-bit tensors: two channels per step, bfloat16 products
   extern __shared__ __align__(16) float tbl[];
 
   const int cpg = g.channel / g.groups;
@@ -640,7 +641,10 @@ __global__ __launch_bounds__(kBlock, OCC) void local_grad_rotation_kernel(
   for (int j0 = c_begin; j0 < c_end; j0 += ch_per_pass) {
     const int nch = min(ch_per_pass, c_end - j0);
     __syncthreads();
-    stage_wide_tables<T, SH, SW>(tbl, filter, g.channel, grp + g.groups * j0, g.groups, nch);
+    if constexpr (PAIRS)
+      stage_pair_tables<T, SH, SW>(tbl, filter, g.channel, grp + g.groups * j0, g.groups, nch);
+    else
+      stage_wide_tables<T, SH, SW>(tbl, filter, g.channel, grp + g.groups * j0, g.groups, nch);
     __syncthreads();
     const size_t chan0 = (size_t)n * g.channel + grp + (size_t)g.groups * j0;
     const T* xp = x + chan0 * in_plane;
@@ -694,13 +698,57 @@ __global__ __launch_bounds__(kBlock, OCC) void local_grad_rotation_kernel(
         sd[t] = fmaf(ps, q.w, sd[t]);
       }
     };
+    if constexpr (PAIRS) {
+      // two channels per step: their products, rounded to bfloat16, are one operand of three
+      // v_dot2c_f32_bf16 against the pair table's {b, c, d} (fp32 sums) -- six vector instructions and one
+      // table read per tap and channel pair where the fp32 form takes eight and two.  The second channel
+      // of an odd count's last pair is the last channel again, against a table of zeros.
+      float xw[2][2][KH], gw[2][2];
+      auto load_pair = [&](int s, int jp) {
 #pragma unroll
-    for (int u = 0; u < DEPTH - 1; ++u) load(u, u);
-    for (int j = 0; j < nch; j += DEPTH) {
+        for (int h = 0; h < 2; ++h) {
+          const int jc = min(2 * jp + h, nch - 1);
+          gw[s][h] = buf_ld2(rg, goff, jc * g_bytes, gout);
 #pragma unroll
-      for (int u = 0; u < DEPTH; ++u) {
-        load((u + DEPTH - 1) % DEPTH, j + u + DEPTH - 1);
-        if (j + u < nch) accumulate(u, j + u);
+          for (int r_ = 0; r_ < KH; ++r_) xw[s][h][r_] = buf_ld2(rx, soff[r_], jc * x_bytes, x);
+        }
+      };
+      auto accumulate_pair = [&](int s, int jp) {
+        const float* tb = tbl + jp * Tb::SIZE;
+#pragma unroll
+        for (int t = 0; t < K; ++t) {
+          const int r_ = t / KW, f_w = t % KW;
+          float ps[2];
+#pragma unroll
+          for (int h = 0; h < 2; ++h) {
+            const float xt = f_w == 0 ? from_lane_below(xw[s][h][r_]) : f_w == 1 ? xw[s][h][r_] : from_lane_above(xw[s][h][r_]);
+            ps[h] = xt * gw[s][h];
+          }
+          typedef __bf16 b2 __attribute__((ext_vector_type(2)));
+          const b2 pk = __builtin_bit_cast(b2, pack_bf16(ps[0], ps[1]));
+          const float4 q = lds_read4(tb + cell[t]);
+          sb[t] = __builtin_amdgcn_fdot2_f32_bf16(pk, __builtin_bit_cast(b2, q.x), sb[t], false);
+          sc[t] = __builtin_amdgcn_fdot2_f32_bf16(pk, __builtin_bit_cast(b2, q.y), sc[t], false);
+          sd[t] = __builtin_amdgcn_fdot2_f32_bf16(pk, __builtin_bit_cast(b2, q.z), sd[t], false);
+        }
+      };
+      const int npair = (nch + 1) / 2;
+      load_pair(0, 0);
+      for (int jp = 0; jp < npair; jp += 2) {
+        load_pair(1, jp + 1);
+        accumulate_pair(0, jp);
+        load_pair(0, jp + 2);
+        if (jp + 1 < npair) accumulate_pair(1, jp + 1);
+      }
+    } else {
+#pragma unroll
+      for (int u = 0; u < DEPTH - 1; ++u) load(u, u);
+      for (int j = 0; j < nch; j += DEPTH) {
+#pragma unroll
+        for (int u = 0; u < DEPTH; ++u) {
+          load((u + DEPTH - 1) % DEPTH, j + u + DEPTH - 1);
+          if (j + u < nch) accumulate(u, j + u);
+        }
       }
     }
   }
@@ -977,16 +1025,6 @@ constexpr int kMfMaxBlkS2 = 12;        // stride 2: channel blocks per workgroup
 
 typedef float mf4 __attribute__((ext_vector_type(4)));
 typedef __bf16 mfb4 __attribute__((ext_vector_type(4)));
-
-// Two floats rounded to bfloat16 by one instruction (v_cvt_pk_bf16_f32), a in the lower half; and the two halves
-// of such a pair back as floats.
-__device__ __forceinline__ unsigned pack_bf16(float a, float b) {
-  typedef float f2 __attribute__((ext_vector_type(2)));
-  typedef __bf16 b2 __attribute__((ext_vector_type(2)));
-  return __builtin_bit_cast(unsigned, __builtin_convertvector(f2{a, b}, b2));
-}
-__device__ __forceinline__ float bf16_lo(unsigned pair) { return __uint_as_float(pair << 16); }
-__device__ __forceinline__ float bf16_hi(unsigned pair) { return __uint_as_float(pair & 0xffff0000u); }
 
 // First float of channel j's row in the staged input tile.  The rows are a multiple of 64 floats
 // apart plus a skew: in the MFMA phase lane (channel q, pixel quad kg) reads row q at

@@ -88,6 +88,45 @@ __device__ __forceinline__ void stage_wide_tables(float* tbl, const T* filter, i
   }
 }
 
+// Pair tables for kernels that need the derivatives only and take two channels per step: block m of
+// channels (2 jp, 2 jp + 1) is {b, c, d} as three bfloat16 pairs (the even channel in the lower half)
+// and an unused word, in the slot order of the wide table; table jp starts at tbl + jp * SIZE.  A
+// channel past the last one leaves zeros.
+template <typename T, int SH, int SW>
+__device__ __forceinline__ void stage_pair_tables(float* tbl, const T* filter, int channels, int c_first,
+                                                  int c_step, int nch) {
+  using Tb = WideTable<SH, SW>;
+  constexpr int CB = Tb::BLOCKS <= 32 ? 32 : 64;  // threads per table
+  const int m = threadIdx.x % CB;
+  if (m >= Tb::BLOCKS) return;
+  const int i = m / Tb::RS - 1, k = m % Tb::RS - 1;
+  unsigned off[4];
+#pragma unroll
+  for (int q = 0; q < 4; ++q) {
+    const int ii = i + (q >> 1), kk = k + (q & 1);
+    off[q] = (ii >= 0 && ii < SH && kk >= 0 && kk < SW) ? (unsigned)(ii * SW + kk) * (unsigned)sizeof(T) : kOutOfRange;
+  }
+  const rsrc_t rf = plane_rsrc(filter, channels * SH * SW);
+  float* dst = tbl + Tb::slot(m) * 4;
+  const int npair = (nch + 1) / 2;
+  for (int jp = threadIdx.x / CB; jp < npair; jp += (int)blockDim.x / CB) {
+    float d[2][3];
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      const int j = 2 * jp + h;
+      const unsigned cb = (unsigned)(c_first + min(j, nch - 1) * c_step) * (unsigned)(SH * SW * sizeof(T));
+      const float tl = buf_ld(rf, off[0] + cb, filter), tr = buf_ld(rf, off[1] + cb, filter);
+      const float bl = buf_ld(rf, off[2] + cb, filter), br = buf_ld(rf, off[3] + cb, filter);
+      // (two out-of-range parts of an offset add up to an offset in range: the zeros are written out)
+      d[h][0] = j < nch ? tr - tl : 0.f;
+      d[h][1] = j < nch ? bl - tl : 0.f;
+      d[h][2] = j < nch ? (br - tr) - (bl - tl) : 0.f;
+    }
+    *reinterpret_cast<uint4*>(dst + jp * Tb::SIZE) =
+        make_uint4(pack_bf16(d[0][0], d[1][0]), pack_bf16(d[0][1], d[1][1]), pack_bf16(d[0][2], d[1][2]), 0u);
+  }
+}
+
 // One 16-byte LDS read for a caller that uses only some components: the empty asm counts as
 // a use of all four, so the compiler keeps the single wide read instead of two narrower ones
 // (two LDS issues).
