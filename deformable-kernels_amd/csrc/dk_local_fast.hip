@@ -19,6 +19,7 @@
 #include <cstdlib>
 
 #include <algorithm>
+#include <type_traits>
 
 #include "dk_kernels.h"
 #include "dk_scope_table.h"
@@ -562,7 +563,7 @@ __global__ __launch_bounds__(kBlock, 2) void local_grad_input_s2_kernel(Geo g, c
 // OCC: waves per SIMD the register allocation leaves room for.  The 27 sums make this the
 // register-heaviest gather kernel; with 96 registers (five waves) it is slower per wave but faster
 // where the grid has more than four workgroups per CU to offer (112 x 112 C=32: 125 -> 96 us).
-template <typename T, int KH, int KW, int SH, int SW, int MODE, int OCC = 2>
+template <typename T, int KH, int KW, int SH, int SW, int MODE, int OCC = 2, bool PAIR = false>
 __global__ __launch_bounds__(kBlock, OCC) void local_grad_rotation_kernel(
     Geo g, const T* __restrict__ gout, const T* __restrict__ x, const T* __restrict__ rot,
     const T* __restrict__ filter, T* __restrict__ grot, float* __restrict__ partial, int splits,
@@ -572,7 +573,10 @@ __global__ __launch_bounds__(kBlock, OCC) void local_grad_rotation_kernel(
   constexpr bool ROWS = MODE == 1, S2 = MODE == 2;  // MODE 0: one load per tap
   constexpr int NLOAD = MODE == 0 ? K : KH;          // input loads per channel
   constexpr int PIX = ROWS ? kRowPix : S2 ? kS2Pix : kBlock;  // pixels per workgroup
-  constexpr bool PAIRS = ROWS && sizeof(T) == 2;  // 16-bit tensors: two channels per step, bfloat16 products
+  // 16-bit tensors: two channels per step, bfloat16 products (PAIR: the host asks for it when a group has
+  // at least 16 channels; with a few channels the products' rounding shows in the result: 1.2e-2 of the
+  // largest element was seen with one channel per group)
+  constexpr bool PAIRS = PAIR && ROWS && sizeof(T) == 2;
   extern __shared__ __align__(16) float tbl[];
 
   const int cpg = g.channel / g.groups;
@@ -1541,12 +1545,24 @@ bool run_grad_rotation(const Geo& g, const T* gout, const T* x, const T* rot, co
   const int per = (int)std::max(1L, std::min<long>(std::min(ceil_div(cpg, splits), 36), ((1L << 31) - 1) / step_bytes));
   const size_t lds = (size_t)per * Tb::SIZE * sizeof(float);
   const unsigned grid = (unsigned)xcd_grid_size((long)ceil_div(g.out_h * g.out_w, rotation_tile(g)) * splits * g.batch * g.groups);
-  if (same_width_geometry(g))
-    if (grid > 5 * 256)
-      local_grad_rotation_kernel<T, 3, 3, SH, SW, 1, 5><<<grid, row_block(g.out_h * g.out_w, kRowLanes), lds, stream>>>(g, gout, x, rot, filter, grot, ws, splits, per);
-    else
-      local_grad_rotation_kernel<T, 3, 3, SH, SW, 1><<<grid, row_block(g.out_h * g.out_w, kRowLanes), lds, stream>>>(g, gout, x, rot, filter, grot, ws, splits, per);
-  else if (stride2_geometry(g))
+  if (same_width_geometry(g)) {
+    // Channel pairs on bfloat16 dot products, for bfloat16 tensors: the products' and the table's rounding
+    // (2^-9 each) comes to about what the result's own rounding to bfloat16 is, 6.5e-3 of the largest
+    // element at worst over random shapes against 4e-3 without.  float16 tensors would lose three of
+    // their eleven bits (5e-4 -> 6e-3) and keep the fp32 multiply-adds.
+    constexpr bool k16 = std::is_same<T, bf16_t>::value;
+    const unsigned block = row_block(g.out_h * g.out_w, kRowLanes);
+    if (k16 && cpg >= 16) {
+      if (grid > 5 * 256)
+        local_grad_rotation_kernel<T, 3, 3, SH, SW, 1, 5, k16><<<grid, block, lds, stream>>>(g, gout, x, rot, filter, grot, ws, splits, per);
+      else
+        local_grad_rotation_kernel<T, 3, 3, SH, SW, 1, 2, k16><<<grid, block, lds, stream>>>(g, gout, x, rot, filter, grot, ws, splits, per);
+    } else if (grid > 5 * 256) {
+      local_grad_rotation_kernel<T, 3, 3, SH, SW, 1, 5><<<grid, block, lds, stream>>>(g, gout, x, rot, filter, grot, ws, splits, per);
+    } else {
+      local_grad_rotation_kernel<T, 3, 3, SH, SW, 1><<<grid, block, lds, stream>>>(g, gout, x, rot, filter, grot, ws, splits, per);
+    }
+  } else if (stride2_geometry(g))
     local_grad_rotation_kernel<T, 3, 3, SH, SW, 2><<<grid, row_block(g.out_h * g.out_w, kS2Lanes), lds, stream>>>(g, gout, x, rot, filter, grot, ws, splits, per);
   else
     local_grad_rotation_kernel<T, 3, 3, SH, SW, 0><<<grid, kBlock, lds, stream>>>(g, gout, x, rot, filter, grot, ws, splits, per);

@@ -112,6 +112,23 @@ def test_matrix_core_forward_and_grad_input_on_16_bit_tensors(case, dtype, tol, 
     assert rel_err(got[1].float(), want[1]) < tol, "grad input"
 
 
+@pytest.mark.parametrize("case", [
+    (2, 37, 28, 28, 3, (4, 4), 1, 1, 1, 1, 1.0),   # odd channel count: the last pair's second channel is a dummy
+    (1, 74, 12, 18, 3, (5, 5), 1, 1, 1, 2, 1.5),   # 37 channels per group, two groups, scope 5
+    (1, 73, 20, 22, 3, (3, 3), 1, 1, 1, 1, 1.0),   # passes of 36, 36 and 1 channels
+    (4, 64, 28, 28, 3, (4, 4), 1, 1, 1, 1, 1.0),   # four channel splits of 16 channels, partial sums
+])
+def test_grad_rotation_by_channel_pairs_on_bfloat16_tensors(case):
+    """bfloat16 tensors with at least 16 channels per group take grad rotation two channels per step, the
+    products rounded to bfloat16 and summed in fp32 by dot-product instructions: the result stays within the
+    1e-2 the 16-bit types are held to (about 6e-3 of the largest element at worst, of which 4e-3 is the
+    result's own rounding)."""
+    inputs, got = _run(case, torch.bfloat16, seed=11)
+    want = _oracle(inputs, np.float32)  # the inputs are already rounded to bfloat16
+    assert got[2].dtype == torch.bfloat16
+    assert rel_err(got[2].float(), want[2]) < 1e-2, "grad rotation"
+
+
 @pytest.mark.parametrize("case", TUNED[:4] + GENERIC[:2])
 def test_fp64_matches_oracle(case):
     inputs, got = _run(case, torch.float64)
