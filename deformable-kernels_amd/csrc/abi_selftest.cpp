@@ -128,6 +128,17 @@ int main() {
   EXPECT(dk_offset_conv_supported(&oc) == 0);
   EXPECT(dk_offset_conv_forward(&oc, one, one, one, one, one, 1 << 30, nullptr) == DK_ERR_UNSUPPORTED);
   EXPECT(dk_offset_conv_backward_bias(nullptr, one, one, one, 0, nullptr) == DK_ERR_NULL_POINTER);
+  // the input gradient: 16-bit tensors on planes 28 / 56 / 112 wide only
+  oc.w = 56;
+  EXPECT(dk_offset_conv_backward_input_workspace(&oc) == 0);
+  EXPECT(dk_offset_conv_backward_input(&oc, one, one, one, one, 1 << 30, nullptr) == DK_ERR_UNSUPPORTED);
+  oc.dtype = DK_BF16;
+  EXPECT(dk_offset_conv_backward_input_workspace(&oc) > 0);
+  EXPECT(dk_offset_conv_forward_workspace(&oc) > 0);
+  EXPECT(dk_offset_conv_backward_input(&oc, nullptr, one, one, one, 1 << 30, nullptr) == DK_ERR_NULL_POINTER);
+  EXPECT(dk_offset_conv_backward_input(&oc, one, one, one, one, 0, nullptr) == DK_ERR_WORKSPACE);
+  oc.w = oc.h = 14;
+  EXPECT(dk_offset_conv_backward_input(&oc, one, one, one, one, 1 << 30, nullptr) == DK_ERR_UNSUPPORTED);
 
   EXPECT(std::strstr(dk_status_string(DK_ERR_WORKSPACE), "workspace") != nullptr);
   EXPECT(dk_status_string(-99) != nullptr);

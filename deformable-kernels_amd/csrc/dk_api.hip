@@ -661,12 +661,22 @@ int dk_offset_conv_supported(const dk_offset_conv_desc* desc) { return check_off
 
 int dk_offset_conv_worthwhile(const dk_offset_conv_desc* desc) {
   return check_offset_conv(desc) == DK_OK &&
-         offset_conv_worthwhile(desc->batch, desc->in_channels, desc->out_channels, desc->h, desc->w, desc->dtype != DK_F32);
+         offset_conv_worthwhile(desc->batch, desc->in_channels, desc->out_channels, desc->h, desc->w);
+}
+
+// 16-bit tensors on planes the 16-bit matrix-instruction kernels cover
+static bool offset_conv_on_16_bit_matrix(const dk_offset_conv_desc* d) {
+  return d->dtype != DK_F32 && offset_conv16_supported(d->in_channels, d->out_channels, d->h, d->w);
+}
+
+static size_t offset_conv_forward_need(const dk_offset_conv_desc* d) {
+  return offset_conv_on_16_bit_matrix(d) ? offset_conv16_workspace(d->in_channels, d->out_channels)
+                                         : offset_conv_workspace(d->batch, d->in_channels, d->out_channels, d->h, d->w);
 }
 
 size_t dk_offset_conv_forward_workspace(const dk_offset_conv_desc* desc) {
   if (check_offset_conv(desc) != DK_OK) return 0;
-  return offset_conv_workspace(desc->batch, desc->in_channels, desc->out_channels, desc->h, desc->w);
+  return offset_conv_forward_need(desc);
 }
 
 int dk_offset_conv_forward(const dk_offset_conv_desc* desc, const void* input, const void* weight,
@@ -675,13 +685,49 @@ int dk_offset_conv_forward(const dk_offset_conv_desc* desc, const void* input, c
   const int rc = check_offset_conv(desc);
   if (rc != DK_OK) return rc;
   if (!input || !weight || !bias || !output) return DK_ERR_NULL_POINTER;
-  const size_t need = offset_conv_workspace(desc->batch, desc->in_channels, desc->out_channels, desc->h, desc->w);
+  const size_t need = offset_conv_forward_need(desc);
   if (!workspace || workspace_bytes < need) return DK_ERR_WORKSPACE;
   bool ok = false;
+  const bool matrix16 = offset_conv_on_16_bit_matrix(desc);
   const int st = by_dtype(desc->dtype, [&]<typename T>() {
+    if constexpr (sizeof(T) == 2) {
+      if (matrix16) {
+        ok = offset_conv16_forward<T>(desc->batch, desc->in_channels, desc->out_channels, desc->h, desc->w, in<T>(input),
+                                      in<T>(weight), in<T>(bias), out<T>(output), workspace, static_cast<hipStream_t>(stream));
+        return;
+      }
+    }
     if constexpr (kHasFast<T>)
       ok = offset_conv_forward<T>(desc->batch, desc->in_channels, desc->out_channels, desc->h, desc->w, in<T>(input),
                                   in<T>(weight), in<T>(bias), out<T>(output), workspace, static_cast<hipStream_t>(stream));
+  });
+  return ok ? st : DK_ERR_UNSUPPORTED;
+}
+
+static int check_offset_conv_backward_input(const dk_offset_conv_desc* d) {
+  const int rc = check_offset_conv(d);
+  if (rc != DK_OK) return rc;
+  if ((long)d->batch * d->out_channels * d->h * d->w > kMaxElems) return DK_ERR_TOO_LARGE;
+  return offset_conv_on_16_bit_matrix(d) ? DK_OK : DK_ERR_UNSUPPORTED;
+}
+
+size_t dk_offset_conv_backward_input_workspace(const dk_offset_conv_desc* desc) {
+  if (check_offset_conv_backward_input(desc) != DK_OK) return 0;
+  return offset_conv16_workspace(desc->in_channels, desc->out_channels);
+}
+
+int dk_offset_conv_backward_input(const dk_offset_conv_desc* desc, const void* out_grad, const void* weight,
+                                  void* input_grad, void* workspace, size_t workspace_bytes, void* stream) {
+  const int rc = check_offset_conv_backward_input(desc);
+  if (rc != DK_OK) return rc;
+  if (!out_grad || !weight || !input_grad) return DK_ERR_NULL_POINTER;
+  if (!workspace || workspace_bytes < offset_conv16_workspace(desc->in_channels, desc->out_channels)) return DK_ERR_WORKSPACE;
+  bool ok = false;
+  const int st = by_dtype(desc->dtype, [&]<typename T>() {
+    if constexpr (sizeof(T) == 2)
+      ok = offset_conv16_backward_input<T>(desc->batch, desc->in_channels, desc->out_channels, desc->h, desc->w,
+                                           in<T>(out_grad), in<T>(weight), out<T>(input_grad), workspace,
+                                           static_cast<hipStream_t>(stream));
   });
   return ok ? st : DK_ERR_UNSUPPORTED;
 }

@@ -118,7 +118,7 @@ void generic_grad_filter(const Geo& g, bool deform, const T* gout, const T* x, c
 
 // dk_offset_conv.hip: the 3x3 offset-branch convolution (stride 1, padding 1; fp32 / fp16 / bf16 tensors, fp32 arithmetic)
 bool offset_conv_supported(int cin, int cout, int h, int w);
-bool offset_conv_worthwhile(int batch, int cin, int cout, int h, int w, bool sixteen_bit);
+bool offset_conv_worthwhile(int batch, int cin, int cout, int h, int w);
 size_t offset_conv_workspace(int batch, int cin, int cout, int h, int w);
 size_t offset_conv_bias_grad_workspace(int batch, int cout);
 template <typename T>
@@ -130,6 +130,17 @@ bool offset_conv_wgrad(int batch, int cin, int cout, int h, int w, const T* x, c
 template <typename T>
 bool offset_conv_forward(int batch, int cin, int cout, int h, int w, const T* x, const T* weight, const T* bias, T* out,
                          void* ws, hipStream_t stream);
+
+// dk_offset_conv16.hip: forward and input gradient of the same convolution on 16-bit matrix instructions
+// (fp16 / bf16 tensors, planes 28 / 56 / 112 wide, at most 32 output channels)
+bool offset_conv16_supported(int cin, int cout, int h, int w);
+size_t offset_conv16_workspace(int cin, int cout);
+template <typename T>
+bool offset_conv16_forward(int batch, int cin, int cout, int h, int w, const T* x, const T* weight, const T* bias,
+                           T* out, void* ws, hipStream_t stream);
+template <typename T>
+bool offset_conv16_backward_input(int batch, int cin, int cout, int h, int w, const T* gout, const T* weight, T* gin,
+                                  void* ws, hipStream_t stream);
 
 // dk_local_nhwc.hip: the local operator on channels-last tensors, all dtypes, any geometry whose tables fit LDS
 bool nhwc_supported(const Geo& g, int dtype);

@@ -1,0 +1,232 @@
+// The offset branch's 3x3 convolution (reference modules/deform_kernel.py:165-168, applied at :214)
+// on 16-bit tensors: forward and input gradient on the 16-bit matrix instructions
+// (v_mfma_f32_16x16x32_bf16 / _f16: the tensors' elements are the operands as they are, the products
+// exact, the sums fp32, one rounding of the result).  Stride 1, padding 1, no dilation, planes 28, 56 or
+// 112 wide.
+//
+// Both passes are the same shift-GEMM, out[m][p] = sum over taps t, channels k of A_t[m][k] * in[k][p + shift_t]:
+//   forward          in = x (Cin channels),   m = output channel,  A_t[m][k] = W[m][k][t], + bias;
+//   input gradient   in = gout (Cout channels), m = input channel, A_t[m][k] = W[k][m][8 - t]  (the taps flipped).
+// A workgroup of four waves owns 448 pixels (whole rows) of one image and walks the `in` channels in chunks
+// of 32, staged zero-padded and channel-interleaved in LDS: position e holds the chunk's 32 elements in 64
+// bytes of an 80-byte slot, so that the B operand of a lane -- pixel l % 16, channels 8 (l / 16) .. + 7 -- is
+// one 16-byte read, and the 16 lanes of a pass (20 words apart) hit disjoint banks.  The A operands come
+// packed per (tap, chunk, 16-row block) as the instruction wants them, one coalesced 16-byte load per lane.
+// A wave holds seven pixel groups x MTB row blocks of accumulators; row blocks beyond MTB take another walk
+// over the staged chunk (the input gradient: 18 channels in, one chunk, three walks of three blocks for 144 out).
+#include <algorithm>
+#include <type_traits>
+
+#include "dk_kernels.h"
+
+namespace dk {
+
+namespace {
+
+constexpr int kC16Block = 256;
+constexpr int kC16Chunk = 32;     // channels per matrix instruction
+constexpr int kC16Pitch = 20;     // 32-bit words per staged position: 16 of data, 4 of bank skew
+constexpr int kC16Pix = 448;      // pixels per workgroup: 28 groups of 16, seven per wave
+constexpr int kC16Gpw = kC16Pix / 16 / (kC16Block / 64);
+
+template <int W>
+struct Tile16 {
+  static constexpr int TH = kC16Pix / W;
+  static constexpr int RS = W + 2;
+  static constexpr int POS = (TH + 2) * RS;
+  static_assert(TH * W == kC16Pix, "whole rows");
+};
+
+typedef float c16f4 __attribute__((ext_vector_type(4)));
+typedef __bf16 c16b8 __attribute__((ext_vector_type(8)));
+typedef _Float16 c16h8 __attribute__((ext_vector_type(8)));
+
+template <typename T>
+__device__ __forceinline__ c16f4 mma16(const uint4& a, const uint4& b, c16f4 acc) {
+  if constexpr (std::is_same<T, bf16_t>::value)
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(c16b8, a), __builtin_bit_cast(c16b8, b), acc, 0, 0, 0);
+  else
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(c16h8, a), __builtin_bit_cast(c16h8, b), acc, 0, 0, 0);
+}
+
+// wp[t][chunk][block][lane] = the eight elements A_t[16 block + lane % 16][32 chunk + 8 (lane / 16) .. + 7], zeros
+// past the tensor.  weight is [O][C][3][3]; forward: rows = O, k = C; transposed: rows = C, k = O, taps flipped.
+template <typename T>
+__global__ void conv16_pack_kernel(const T* __restrict__ weight, int O, int C, int transposed, int chunks, int blocks,
+                                   uint4* __restrict__ wp) {
+  const int idx = blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= 9 * chunks * blocks * 64) return;
+  const int lane = idx % 64, mb = idx / 64 % blocks, ch = idx / 64 / blocks % chunks, t = idx / 64 / blocks / chunks;
+  const int m = 16 * mb + (lane & 15), k0 = kC16Chunk * ch + 8 * (lane >> 4);
+  const unsigned short* w = reinterpret_cast<const unsigned short*>(weight);
+  unsigned v[8];
+#pragma unroll
+  for (int j = 0; j < 8; ++j) {
+    const int k = k0 + j;
+    const int o = transposed ? k : m, c = transposed ? m : k;
+    v[j] = (o < O && c < C) ? w[((size_t)o * C + c) * 9 + (transposed ? 8 - t : t)] : 0u;
+  }
+  wp[idx] = make_uint4(v[0] | v[1] << 16, v[2] | v[3] << 16, v[4] | v[5] << 16, v[6] | v[7] << 16);
+}
+
+// in [batch][kin][h][W] -> out [batch][mout][h][W]; wp as packed above with `chunks` = ceil(kin / 32) and
+// `blocks` = ceil(mout / 16); bias [mout] or null.
+// grid = (image, row tile)
+template <typename T, int W, int MTB>
+__global__ __launch_bounds__(kC16Block, 2) void conv16_kernel(int batch, int kin, int mout, int h, int tiles, int chunks,
+                                                              int blocks, const T* __restrict__ in,
+                                                              const uint4* __restrict__ wp, const T* __restrict__ bias,
+                                                              T* __restrict__ out) {
+  using Tl = Tile16<W>;
+  constexpr int TH = Tl::TH, RS = Tl::RS, POS = Tl::POS;
+  extern __shared__ __align__(16) unsigned tile[];  // [POS][kC16Pitch]
+
+  const int total = batch * tiles;
+  const int lb = logical_block(total);
+  if (lb >= total) return;
+  const int n = lb / tiles, r0 = (lb % tiles) * TH;
+  const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int plane = h * W;
+
+  for (int e = threadIdx.x; e < POS * kC16Pitch; e += kC16Block) tile[e] = 0u;  // the padding stays zero
+
+  // word index of the lane's B operand for each of its pixel groups (tap shifts are immediates)
+  int bword[kC16Gpw];
+#pragma unroll
+  for (int i = 0; i < kC16Gpw; ++i) {
+    const int q = (wave + 4 * i) * 16 + (lane & 15);
+    bword[i] = ((q / W + 1) * RS + q % W + 1) * kC16Pitch + (lane >> 4) * 4;
+  }
+
+  for (int mb0 = 0; mb0 < blocks; mb0 += MTB) {
+    c16f4 acc[kC16Gpw][MTB];
+#pragma unroll
+    for (int i = 0; i < kC16Gpw; ++i)
+#pragma unroll
+      for (int m = 0; m < MTB; ++m) acc[i][m] = c16f4{0.f, 0.f, 0.f, 0.f};
+
+    for (int ch = 0; ch < chunks; ++ch) {
+      if (chunks > 1 || mb0 == 0) {  // a single chunk stays staged for every walk
+        __syncthreads();             // the previous chunk's reads are done
+        // one buffer over the chunk's planes: channels past the tensor and rows outside the image fail
+        // the range check and read zero
+        const int kc = min(kC16Chunk, kin - ch * kC16Chunk);
+        const rsrc_t rs = plane_rsrc(in + ((size_t)n * kin + (size_t)ch * kC16Chunk) * plane, kc * plane);
+        for (int e = threadIdx.x; e < (TH + 2) * 4 * W; e += kC16Block) {
+          const int col = e % W, ry = e / W % (TH + 2), oct = e / W / (TH + 2);
+          const int row = r0 - 1 + ry;
+          const bool live = row >= 0 && row < h;
+          unsigned v[8];
+#pragma unroll
+          for (int j = 0; j < 8; ++j) {
+            const unsigned o = live ? (unsigned)((oct * 8 + j) * plane + row * W + col) * 2u : kOutOfRange;
+            v[j] = __builtin_amdgcn_raw_buffer_load_b16(rs, (int)o, 0, 0);
+          }
+          *reinterpret_cast<uint4*>(tile + (ry * RS + col + 1) * kC16Pitch + oct * 4) =
+              make_uint4(v[0] | v[1] << 16, v[2] | v[3] << 16, v[4] | v[5] << 16, v[6] | v[7] << 16);
+        }
+        __syncthreads();
+      }
+#pragma unroll
+      for (int t = 0; t < 9; ++t) {
+        const int shift = ((t / 3 - 1) * RS + (t % 3 - 1)) * kC16Pitch;
+        uint4 a[MTB];
+#pragma unroll
+        for (int m = 0; m < MTB; ++m) {
+          const int mb = min(mb0 + m, blocks - 1);  // a block past the last repeats it; its results are not stored
+          a[m] = wp[((size_t)(t * chunks + ch) * blocks + mb) * 64 + lane];
+        }
+#pragma unroll
+        for (int i = 0; i < kC16Gpw; ++i) {
+          const uint4 b = *reinterpret_cast<const uint4*>(tile + bword[i] + shift);
+#pragma unroll
+          for (int m = 0; m < MTB; ++m) acc[i][m] = mma16<T>(a[m], b, acc[i][m]);
+        }
+      }
+    }
+
+    // lane (pixel l % 16, rows 4 (l / 16) .. + 3 of each block)
+#pragma unroll
+    for (int m = 0; m < MTB; ++m) {
+      if (mb0 + m >= blocks) break;
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const int o = 16 * (mb0 + m) + 4 * (lane >> 4) + r;
+        if (o >= mout) continue;
+        const float bv = bias ? ld(bias + o) : 0.f;
+        T* dst = out + ((size_t)n * mout + o) * plane + (size_t)r0 * W;
+#pragma unroll
+        for (int i = 0; i < kC16Gpw; ++i) {
+          const int q = (wave + 4 * i) * 16 + (lane & 15);
+          if (r0 * W + q < plane) st(dst + q, acc[i][m][r] + bv);
+        }
+      }
+    }
+  }
+}
+
+size_t pack_bytes(int kin, int mout) {
+  return (size_t)9 * ceil_div(kin, kC16Chunk) * ceil_div(mout, 16) * 64 * sizeof(uint4);
+}
+
+template <typename T, int MTB>
+bool launch_conv16(int batch, int kin, int mout, int h, int w, const T* in, const uint4* wp, const T* bias, T* out,
+                   hipStream_t stream) {
+  const int chunks = ceil_div(kin, kC16Chunk), blocks = ceil_div(mout, 16);
+#define DK_C16(WW)                                                                                                     \
+  {                                                                                                                    \
+    const int tiles = ceil_div(h, Tile16<WW>::TH);                                                                     \
+    const size_t lds = (size_t)Tile16<WW>::POS * kC16Pitch * sizeof(unsigned);                                         \
+    conv16_kernel<T, WW, MTB><<<(unsigned)xcd_grid_size((long)batch * tiles), kC16Block, lds, stream>>>(               \
+        batch, kin, mout, h, tiles, chunks, blocks, in, wp, bias, out);                                                \
+  }
+  switch (w) {
+    case 28: DK_C16(28) break;
+    case 56: DK_C16(56) break;
+    case 112: DK_C16(112) break;
+    default: return false;
+  }
+#undef DK_C16
+  return true;
+}
+
+}  // namespace
+
+bool offset_conv16_supported(int cin, int cout, int h, int w) {
+  return cin >= 1 && cout >= 1 && cout <= 32 && h >= 1 && (w == 28 || w == 56 || w == 112) &&
+         (long)kC16Chunk * h * w * 2 < (1L << 31) && (long)cin * h * w < (1L << 31) && (long)cout * h * w < (1L << 31);
+}
+
+size_t offset_conv16_workspace(int cin, int cout) { return std::max(pack_bytes(cin, cout), pack_bytes(cout, cin)); }
+
+template <typename T>
+bool offset_conv16_forward(int batch, int cin, int cout, int h, int w, const T* x, const T* weight, const T* bias,
+                           T* out, void* ws, hipStream_t stream) {
+  if (!offset_conv16_supported(cin, cout, h, w)) return false;
+  if (batch == 0) return true;
+  uint4* wp = static_cast<uint4*>(ws);
+  const int chunks = ceil_div(cin, kC16Chunk), blocks = ceil_div(cout, 16);
+  conv16_pack_kernel<T><<<ceil_div(9 * chunks * blocks * 64, 256), 256, 0, stream>>>(weight, cout, cin, 0, chunks, blocks, wp);
+  return blocks == 1 ? launch_conv16<T, 1>(batch, cin, cout, h, w, x, wp, bias, out, stream)
+                     : launch_conv16<T, 2>(batch, cin, cout, h, w, x, wp, bias, out, stream);
+}
+
+template <typename T>
+bool offset_conv16_backward_input(int batch, int cin, int cout, int h, int w, const T* gout, const T* weight, T* gin,
+                                  void* ws, hipStream_t stream) {
+  if (!offset_conv16_supported(cin, cout, h, w)) return false;
+  if (batch == 0) return true;
+  uint4* wp = static_cast<uint4*>(ws);
+  const int chunks = ceil_div(cout, kC16Chunk), blocks = ceil_div(cin, 16);
+  conv16_pack_kernel<T><<<ceil_div(9 * chunks * blocks * 64, 256), 256, 0, stream>>>(weight, cout, cin, 1, chunks, blocks, wp);
+  return launch_conv16<T, 3>(batch, cout, cin, h, w, gout, wp, static_cast<const T*>(nullptr), gin, stream);
+}
+
+#define DK_INST(T)                                                                                                      \
+  template bool offset_conv16_forward<T>(int, int, int, int, int, const T*, const T*, const T*, T*, void*, hipStream_t); \
+  template bool offset_conv16_backward_input<T>(int, int, int, int, int, const T*, const T*, T*, void*, hipStream_t);
+DK_INST(__half)
+DK_INST(bf16_t)
+#undef DK_INST
+
+}  // namespace dk

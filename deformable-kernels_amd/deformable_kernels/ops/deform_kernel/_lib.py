@@ -92,6 +92,8 @@ SIGNATURES = {
     "dk_offset_conv_backward_weight": (ctypes.c_int, [_OC, _P, _P, _P, _P, _SZ, _P]),
     "dk_offset_conv_backward_bias_workspace": (_SZ, [_OC]),
     "dk_offset_conv_backward_bias": (ctypes.c_int, [_OC, _P, _P, _P, _SZ, _P]),
+    "dk_offset_conv_backward_input_workspace": (_SZ, [_OC]),
+    "dk_offset_conv_backward_input": (ctypes.c_int, [_OC, _P, _P, _P, _P, _SZ, _P]),
 }
 
 _lib = None

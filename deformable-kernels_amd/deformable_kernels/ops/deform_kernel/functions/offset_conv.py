@@ -7,12 +7,14 @@ kernels multiply and add in float32 and round the results once) it runs
 
   * the forward and the weight gradient on the library's matrix-core kernels where they apply
     and are the faster choice (stride 1, padding 1, dilation 1, input channels a multiple of 16,
-    18 output channels or at most 16, plane width 56 or 112 with enough images to fill the GPU;
+    18 output channels or at most 16, plane width 28, 56 or 112 with enough images to fill the GPU;
     ``force=True``: wherever they apply, also widths 7 / 14 / 28),
   * the bias gradient on the library's reduction kernel for every shape (the framework's
     reduction over (N, H, W) takes 60-230 us on the large planes),
-  * everything else -- the input gradient, and forward / weight gradient of the other shapes --
-    on the framework's convolution routines.
+  * for float16 / bfloat16 tensors on planes 28, 56 or 112 wide, the forward and the input gradient on
+    the library's 16-bit matrix-instruction kernel (the elements are the operands as they are),
+  * everything else -- the input gradient of float32 tensors and of the other planes, and forward /
+    weight gradient of the other shapes -- on the framework's convolution routines.
 
 float64, CPU tensors, mixed dtypes and autocast regions go to ``F.conv2d`` unchanged.
 """
@@ -91,14 +93,23 @@ class OffsetConvFunction(Function):
         gi = gw = gb = None
         L = _lib.lib()
         library_weight = need_weight and not ctx.native
-        if need_input or library_weight:
+        # the input gradient has a kernel of its own for 16-bit tensors on the wider planes
+        desc = _desc(input, weight)
+        native_input = need_input and ctx.native and L.dk_offset_conv_backward_input_workspace(desc) > 0
+        if (need_input and not native_input) or library_weight:
             # the framework's routine, without its bias gradient
             gi, gw_lib, _ = torch.ops.aten.convolution_backward(
                 grad_output, input, weight, None, list(stride), list(padding), list(dilation), False, [0, 0], 1,
-                [need_input, library_weight, False])
+                [need_input and not native_input, library_weight, False])
             if library_weight:
                 gw = gw_lib
         with torch.cuda.device(input.device):
+            if native_input:
+                gi = torch.empty_like(input)
+                ws, nbytes = _lib.workspace(L.dk_offset_conv_backward_input_workspace(desc), input.device)
+                _lib.check(L.dk_offset_conv_backward_input(desc, _lib.ptr(grad_output), _lib.ptr(weight), _lib.ptr(gi),
+                                                           _lib.ptr(ws), nbytes, _lib.stream_ptr(input)),
+                           "offset_conv input gradient")
             if need_weight and ctx.native:
                 gw = torch.empty_like(weight)
                 desc = _desc(input, weight)

@@ -281,12 +281,12 @@ int dk_nd_linear_sample_backward_coord(const dk_nd_desc *desc, const void *out_g
  * (modules/deform_kernel.py:165-168: nn.Conv2d(in_planes, rotation_groups*k*k*2, k, stride,
  * padding, dilation, bias=True), applied at :214).  The reference calls the framework's
  * convolution there; this entry point is a faster kernel for that one shape family: stride 1,
- * padding 1, dilation 1, float32 / float16 / bfloat16 tensors (fp32 products and sums, results rounded
- * once), in_channels a multiple of 16, out_channels <= 16 or 18 or 20,
- * width 7, 14, 28, 56 or 112.  dk_offset_conv_supported() tells whether a shape is covered,
- * dk_offset_conv_worthwhile() whether it is also expected to beat the library convolution
- * (56- and 112-wide planes with enough images to fill the GPU); the caller keeps its library
- * convolution otherwise.
+ * padding 1, dilation 1, float32 / float16 / bfloat16 tensors (fp32 sums of fp32 products, or of the
+ * exact products of the 16-bit elements; results rounded once), in_channels a multiple of 16,
+ * out_channels <= 16 or 18 or 20, width 7, 14, 28, 56 or 112.  dk_offset_conv_supported() tells
+ * whether a shape is covered, dk_offset_conv_worthwhile() whether it is also expected to beat the
+ * library convolution (planes 28 wide and wider with enough images to fill the GPU); the caller
+ * keeps its library convolution otherwise.
  *   input [batch, in_channels, h, w], weight [out_channels, in_channels, 3, 3],
  *   bias [out_channels], output [batch, out_channels, h, w]; workspace: packed weights. */
 typedef struct dk_offset_conv_desc {
@@ -309,11 +309,20 @@ int dk_offset_conv_backward_weight(const dk_offset_conv_desc *desc, const void *
                                    void *stream);
 
 /* Gradient of that convolution's bias: bias_grad[o] = sum over images and pixels of
- * out_grad[n][o][.], any shape; fp32 sums, the images are added in a fixed order.  (The input
- * gradient of the convolution is left to the caller's library.) */
+ * out_grad[n][o][.], any shape; fp32 sums, the images are added in a fixed order. */
 size_t dk_offset_conv_backward_bias_workspace(const dk_offset_conv_desc *desc);
 int dk_offset_conv_backward_bias(const dk_offset_conv_desc *desc, const void *out_grad, void *bias_grad,
                                  void *workspace, size_t workspace_bytes, void *stream);
+
+/* Gradient of that convolution's input (what autograd derives for the rotation_conv call at
+ * modules/deform_kernel.py:214), input_grad [batch, in_channels, h, w] (fully written), for float16 /
+ * bfloat16 tensors on planes 28, 56 or 112 wide: the 16-bit matrix instructions multiply the tensors'
+ * elements as they are (exact products, fp32 sums, one rounding of the result).  The forward of such
+ * tensors and planes runs on the same kernel.  Other shapes and float32 return DK_ERR_UNSUPPORTED (the
+ * workspace query 0): the caller keeps its library's routine there. */
+size_t dk_offset_conv_backward_input_workspace(const dk_offset_conv_desc *desc);
+int dk_offset_conv_backward_input(const dk_offset_conv_desc *desc, const void *out_grad, const void *weight,
+                                  void *input_grad, void *workspace, size_t workspace_bytes, void *stream);
 
 /* ---- depthwise convolution with one kernel per image and channel ------------- */
 
