@@ -139,6 +139,12 @@ int main() {
   EXPECT(dk_offset_conv_backward_input(&oc, one, one, one, one, 0, nullptr) == DK_ERR_WORKSPACE);
   oc.w = oc.h = 14;
   EXPECT(dk_offset_conv_backward_input(&oc, one, one, one, one, 1 << 30, nullptr) == DK_ERR_UNSUPPORTED);
+  // the weight gradient: 15 and more outputs
+  EXPECT(dk_offset_conv_backward_weight_workspace(&oc) > 0);
+  oc.out_channels = 7;
+  EXPECT(dk_offset_conv_supported(&oc) == 1);
+  EXPECT(dk_offset_conv_backward_weight_workspace(&oc) == 0);
+  EXPECT(dk_offset_conv_backward_weight(&oc, one, one, one, one, 1 << 30, nullptr) == DK_ERR_UNSUPPORTED);
 
   EXPECT(std::strstr(dk_status_string(DK_ERR_WORKSPACE), "workspace") != nullptr);
   EXPECT(dk_status_string(-99) != nullptr);

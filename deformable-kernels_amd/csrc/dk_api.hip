@@ -743,6 +743,7 @@ int dk_offset_conv_backward_weight(const dk_offset_conv_desc* desc, const void* 
   if (rc != DK_OK) return rc;
   if (!out_grad || !input || !weight_grad) return DK_ERR_NULL_POINTER;
   const size_t need = offset_conv_wgrad_workspace(desc->batch, desc->in_channels, desc->out_channels, desc->h, desc->w);
+  if (need == 0) return DK_ERR_UNSUPPORTED;  // fewer than 15 outputs
   if (!workspace || workspace_bytes < need) return DK_ERR_WORKSPACE;
   bool ok = false;
   const int st = by_dtype(desc->dtype, [&]<typename T>() {

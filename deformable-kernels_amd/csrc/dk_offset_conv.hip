@@ -539,8 +539,11 @@ int wgrad_parts(int batch, int cin, int h, int w) {
   return std::max(1, std::min(items, 256 / nchunks));
 }
 
+// The weight gradient's 16-row blocks of (output, tap) pairs are instantiated for 9, 11 and 12 blocks:
+// 15 or 16, 18 and 20 outputs.  0 bytes: not covered.
 size_t offset_conv_wgrad_workspace(int batch, int cin, int cout, int h, int w) {
   const int nt = ceil_div(cout * 9, 16);
+  if (nt != 9 && nt != 11 && nt != 12) return 0;
   return (size_t)wgrad_parts(batch, cin, h, w) * (cin / kCvChunk) * nt * 256 * sizeof(float);
 }
 

@@ -92,9 +92,11 @@ class OffsetConvFunction(Function):
         need_input, need_weight = ctx.needs_input_grad[0], ctx.needs_input_grad[1]
         gi = gw = gb = None
         L = _lib.lib()
-        library_weight = need_weight and not ctx.native
-        # the input gradient has a kernel of its own for 16-bit tensors on the wider planes
+        # the input gradient has a kernel of its own for 16-bit tensors on the wider planes, the weight
+        # gradient for 15 and more outputs: a workspace query of 0 says "not covered"
         desc = _desc(input, weight)
+        native_weight = need_weight and ctx.native and L.dk_offset_conv_backward_weight_workspace(desc) > 0
+        library_weight = need_weight and not native_weight
         native_input = need_input and ctx.native and L.dk_offset_conv_backward_input_workspace(desc) > 0
         if (need_input and not native_input) or library_weight:
             # the framework's routine, without its bias gradient
@@ -110,9 +112,8 @@ class OffsetConvFunction(Function):
                 _lib.check(L.dk_offset_conv_backward_input(desc, _lib.ptr(grad_output), _lib.ptr(weight), _lib.ptr(gi),
                                                            _lib.ptr(ws), nbytes, _lib.stream_ptr(input)),
                            "offset_conv input gradient")
-            if need_weight and ctx.native:
+            if native_weight:
                 gw = torch.empty_like(weight)
-                desc = _desc(input, weight)
                 ws, nbytes = _lib.workspace(L.dk_offset_conv_backward_weight_workspace(desc), input.device)
                 _lib.check(L.dk_offset_conv_backward_weight(desc, _lib.ptr(grad_output), _lib.ptr(input), _lib.ptr(gw),
                                                             _lib.ptr(ws), nbytes, _lib.stream_ptr(input)),

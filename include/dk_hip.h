@@ -301,8 +301,9 @@ int dk_offset_conv_forward(const dk_offset_conv_desc *desc, const void *input, c
                            void *stream);
 
 /* Gradient of that convolution's weight, weight_grad [out_channels, in_channels, 3, 3] (fully
- * written), for the shapes dk_offset_conv_supported() accepts; per-workgroup partial sums in the
- * workspace are added in a fixed order. */
+ * written), for the shapes dk_offset_conv_supported() accepts with 15, 16, 18 or 20 output channels
+ * (fewer: the workspace query returns 0, the call DK_ERR_UNSUPPORTED, and the caller keeps its
+ * library's routine); per-workgroup partial sums in the workspace are added in a fixed order. */
 size_t dk_offset_conv_backward_weight_workspace(const dk_offset_conv_desc *desc);
 int dk_offset_conv_backward_weight(const dk_offset_conv_desc *desc, const void *out_grad, const void *input,
                                    void *weight_grad, void *workspace, size_t workspace_bytes,

@@ -90,6 +90,27 @@ def test_sixteen_bit_tensors_match_float64_on_the_rounded_inputs(shape, dtype, t
     assert rel_err(x.grad.double().cpu(), xd.grad.cpu()) < tol
 
 
+@pytest.mark.parametrize("dtype,tol", [(torch.float32, 1e-5), (torch.bfloat16, 1e-2)])
+def test_fewer_than_15_outputs_take_the_library_weight_gradient(dtype, tol):
+    """The forward covers 1 to 16 outputs, the weight gradient 15 and more: with 7 outputs its workspace query
+    says 0 and the weight gradient comes from the framework's routine, everything else from the library."""
+    from deformable_kernels.ops.deform_kernel.functions import offset_conv, offset_conv_supported
+    g = torch.Generator().manual_seed(41)
+    dev = torch.device("cuda:0")
+    x = torch.randn(2, 32, 9, 56, generator=g).to(dtype).to(dev).requires_grad_()
+    w = (torch.randn(7, 32, 3, 3, generator=g) * 0.05).to(dtype).to(dev).requires_grad_()
+    b = torch.randn(7, generator=g).to(dtype).to(dev).requires_grad_()
+    gout = torch.randn(2, 7, 9, 56, generator=g).to(dtype).to(dev)
+    assert offset_conv_supported(x, w, b, 1, 1, 1)
+    out = offset_conv(x, w, b, force=True)
+    out.backward(gout)
+    xd, wd, bd = [t.detach().double().requires_grad_() for t in (x, w, b)]
+    want = F.conv2d(xd, wd, bd, padding=1)
+    want.backward(gout.double())
+    for got, ref in ((out.detach(), want.detach()), (x.grad, xd.grad), (w.grad, wd.grad), (b.grad, bd.grad)):
+        assert got.dtype == dtype and rel_err(got.double().cpu(), ref.cpu()) < tol
+
+
 def test_unsupported_calls_go_to_the_library_convolution():
     from deformable_kernels.ops.deform_kernel.functions import offset_conv, offset_conv_supported
     dev = torch.device("cuda:0")
