@@ -5,10 +5,10 @@
 ``torch.nn.functional.conv2d`` returns.  For float32, float16 and bfloat16 GPU tensors (all of one dtype; the
 kernels multiply and add in float32 and round the results once) it runs
 
-  * the forward and the weight gradient on the library's matrix-core kernels where they apply
-    and are the faster choice (stride 1, padding 1, dilation 1, input channels a multiple of 16,
+  * the forward and -- for float32 tensors, or with ``force=True`` -- the weight gradient on the library's
+    matrix-core kernels where they apply and are the faster choice (stride 1, padding 1, dilation 1, input channels a multiple of 16,
     18 output channels or at most 16, plane width 28, 56 or 112 with enough images to fill the GPU;
-    ``force=True``: wherever they apply, also widths 7 / 14 / 28),
+    ``force=True``: wherever they apply, also widths 7 / 14),
   * the bias gradient on the library's reduction kernel for every shape (the framework's
     reduction over (N, H, W) takes 60-230 us on the large planes),
   * for float16 / bfloat16 tensors on planes 28, 56 or 112 wide, the forward and the input gradient on
@@ -64,11 +64,12 @@ def offset_conv_supported(input, weight, bias, stride, padding, dilation, worthw
 
 class OffsetConvFunction(Function):
     @staticmethod
-    def forward(ctx, input, weight, bias, stride, padding, dilation, native):
+    def forward(ctx, input, weight, bias, stride, padding, dilation, native, forced=False):
         input, weight = input.contiguous(), weight.contiguous()
         ctx.save_for_backward(input, weight)
         ctx.conv = (stride, padding, dilation)
         ctx.native = native
+        ctx.forced = forced
         ctx.has_bias = bias is not None
         if not native:
             return F.conv2d(input, weight, bias, stride, padding, dilation)
@@ -96,6 +97,11 @@ class OffsetConvFunction(Function):
         # gradient for 15 and more outputs: a workspace query of 0 says "not covered"
         desc = _desc(input, weight)
         native_weight = need_weight and ctx.native and L.dk_offset_conv_backward_weight_workspace(desc) > 0
+        # 16-bit tensors: the weight-gradient kernel multiplies in fp32 and the framework's on 16-bit matrix
+        # instructions, which is ahead on every plane (bf16, batch 128: 317 / 264 / 95 us against 330 / 290 / 150
+        # on planes 112 / 56 / 28 wide), so it keeps that pass unless the kernels were asked for
+        if native_weight and input.dtype != torch.float32 and not ctx.forced:
+            native_weight = False
         library_weight = need_weight and not native_weight
         native_input = need_input and ctx.native and L.dk_offset_conv_backward_input_workspace(desc) > 0
         if (need_input and not native_input) or library_weight:
@@ -124,7 +130,7 @@ class OffsetConvFunction(Function):
                 ws, nbytes = _lib.workspace(L.dk_offset_conv_backward_bias_workspace(desc), input.device)
                 _lib.check(L.dk_offset_conv_backward_bias(desc, _lib.ptr(grad_output), _lib.ptr(gb), _lib.ptr(ws),
                                                           nbytes, _lib.stream_ptr(input)), "offset_conv bias gradient")
-        return gi, gw, gb, None, None, None, None
+        return gi, gw, gb, None, None, None, None, None
 
 
 def offset_conv(input, weight, bias=None, stride=1, padding=1, dilation=1, force=False):
@@ -133,4 +139,5 @@ def offset_conv(input, weight, bias=None, stride=1, padding=1, dilation=1, force
     if not _float32_gpu(input, weight, bias):
         return F.conv2d(input, weight, bias, stride, padding, dilation)
     native = offset_conv_supported(input, weight, bias, stride, padding, dilation, worthwhile=not force)
-    return OffsetConvFunction.apply(input, weight, bias, _pair(stride), _pair(padding), _pair(dilation), native)
+    return OffsetConvFunction.apply(input, weight, bias, _pair(stride), _pair(padding), _pair(dilation), native,
+                                    bool(force))
