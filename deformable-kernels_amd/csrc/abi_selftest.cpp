@@ -138,7 +138,10 @@ int main() {
   EXPECT(dk_offset_conv_backward_input(&oc, nullptr, one, one, one, 1 << 30, nullptr) == DK_ERR_NULL_POINTER);
   EXPECT(dk_offset_conv_backward_input(&oc, one, one, one, one, 0, nullptr) == DK_ERR_WORKSPACE);
   oc.w = oc.h = 14;
+  EXPECT(dk_offset_conv_backward_input_workspace(&oc) > 0);
+  oc.w = 21;
   EXPECT(dk_offset_conv_backward_input(&oc, one, one, one, one, 1 << 30, nullptr) == DK_ERR_UNSUPPORTED);
+  oc.w = 14;
   // the weight gradient: 15 and more outputs
   EXPECT(dk_offset_conv_backward_weight_workspace(&oc) > 0);
   oc.out_channels = 7;

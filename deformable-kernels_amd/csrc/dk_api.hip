@@ -660,8 +660,12 @@ static int check_offset_conv(const dk_offset_conv_desc* d) {
 int dk_offset_conv_supported(const dk_offset_conv_desc* desc) { return check_offset_conv(desc) == DK_OK; }
 
 int dk_offset_conv_worthwhile(const dk_offset_conv_desc* desc) {
-  return check_offset_conv(desc) == DK_OK &&
-         offset_conv_worthwhile(desc->batch, desc->in_channels, desc->out_channels, desc->h, desc->w);
+  if (check_offset_conv(desc) != DK_OK) return 0;
+  // 16-bit tensors: forward and input gradient on 16-bit matrix instructions are ahead of the library's on every
+  // plane they cover once there are workgroups ((image, 448-pixel tile) items) for a quarter of the CUs
+  if (desc->dtype != DK_F32 && offset_conv16_supported(desc->in_channels, desc->out_channels, desc->h, desc->w))
+    return (long)desc->batch * ((desc->h * desc->w + 447) / 448) >= 64;
+  return offset_conv_worthwhile(desc->batch, desc->in_channels, desc->out_channels, desc->h, desc->w);
 }
 
 // 16-bit tensors on planes the 16-bit matrix-instruction kernels cover
@@ -670,7 +674,7 @@ static bool offset_conv_on_16_bit_matrix(const dk_offset_conv_desc* d) {
 }
 
 static size_t offset_conv_forward_need(const dk_offset_conv_desc* d) {
-  return offset_conv_on_16_bit_matrix(d) ? offset_conv16_workspace(d->in_channels, d->out_channels)
+  return offset_conv_on_16_bit_matrix(d) ? offset_conv16_workspace(d->batch, d->in_channels, d->out_channels, d->h, d->w)
                                          : offset_conv_workspace(d->batch, d->in_channels, d->out_channels, d->h, d->w);
 }
 
@@ -713,7 +717,7 @@ static int check_offset_conv_backward_input(const dk_offset_conv_desc* d) {
 
 size_t dk_offset_conv_backward_input_workspace(const dk_offset_conv_desc* desc) {
   if (check_offset_conv_backward_input(desc) != DK_OK) return 0;
-  return offset_conv16_workspace(desc->in_channels, desc->out_channels);
+  return offset_conv16_workspace(desc->batch, desc->in_channels, desc->out_channels, desc->h, desc->w);
 }
 
 int dk_offset_conv_backward_input(const dk_offset_conv_desc* desc, const void* out_grad, const void* weight,
@@ -721,7 +725,7 @@ int dk_offset_conv_backward_input(const dk_offset_conv_desc* desc, const void* o
   const int rc = check_offset_conv_backward_input(desc);
   if (rc != DK_OK) return rc;
   if (!out_grad || !weight || !input_grad) return DK_ERR_NULL_POINTER;
-  if (!workspace || workspace_bytes < offset_conv16_workspace(desc->in_channels, desc->out_channels)) return DK_ERR_WORKSPACE;
+  if (!workspace || workspace_bytes < offset_conv16_workspace(desc->batch, desc->in_channels, desc->out_channels, desc->h, desc->w)) return DK_ERR_WORKSPACE;
   bool ok = false;
   const int st = by_dtype(desc->dtype, [&]<typename T>() {
     if constexpr (sizeof(T) == 2)

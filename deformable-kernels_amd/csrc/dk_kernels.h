@@ -132,9 +132,9 @@ bool offset_conv_forward(int batch, int cin, int cout, int h, int w, const T* x,
                          void* ws, hipStream_t stream);
 
 // dk_offset_conv16.hip: forward and input gradient of the same convolution on 16-bit matrix instructions
-// (fp16 / bf16 tensors, planes 28 / 56 / 112 wide, at most 32 output channels)
+// (fp16 / bf16 tensors, planes 7 / 14 / 28 / 56 / 112 wide, at most 32 output channels)
 bool offset_conv16_supported(int cin, int cout, int h, int w);
-size_t offset_conv16_workspace(int cin, int cout);
+size_t offset_conv16_workspace(int batch, int cin, int cout, int h, int w);
 template <typename T>
 bool offset_conv16_forward(int batch, int cin, int cout, int h, int w, const T* x, const T* weight, const T* bias,
                            T* out, void* ws, hipStream_t stream);

@@ -1,8 +1,8 @@
 // The offset branch's 3x3 convolution (reference modules/deform_kernel.py:165-168, applied at :214)
 // on 16-bit tensors: forward and input gradient on the 16-bit matrix instructions
 // (v_mfma_f32_16x16x32_bf16 / _f16: the tensors' elements are the operands as they are, the products
-// exact, the sums fp32, one rounding of the result).  Stride 1, padding 1, no dilation, planes 28, 56 or
-// 112 wide.
+// exact, the sums fp32, one rounding of the result).  Stride 1, padding 1, no dilation, planes 7, 14, 28, 56
+// or 112 wide.
 //
 // Both passes are the same shift-GEMM, out[m][p] = sum over taps t, channels k of A_t[m][k] * in[k][p + shift_t]:
 //   forward          in = x (Cin channels),   m = output channel,  A_t[m][k] = W[m][k][t], + bias;
@@ -12,8 +12,9 @@
 // bytes of an 80-byte slot, so that the B operand of a lane -- pixel l % 16, channels 8 (l / 16) .. + 7 -- is
 // one 16-byte read, and the 16 lanes of a pass (20 words apart) hit disjoint banks.  The A operands come
 // packed per (tap, chunk, 16-row block) as the instruction wants them, one coalesced 16-byte load per lane.
-// A wave holds seven pixel groups x MTB row blocks of accumulators; row blocks beyond MTB take another walk
-// over the staged chunk (the input gradient: 18 channels in, one chunk, three walks of three blocks for 144 out).
+// A wave holds seven pixel groups x MTB row blocks of accumulators; row blocks beyond MTB go to further
+// workgroups that stage the same tile (the input gradient: 18 channels in, one chunk, three workgroups of
+// three blocks for 144 channels out).
 #include <algorithm>
 #include <type_traits>
 
@@ -71,49 +72,62 @@ __global__ void conv16_pack_kernel(const T* __restrict__ weight, int O, int C, i
 
 // in [batch][kin][h][W] -> out [batch][mout][h][W]; wp as packed above with `chunks` = ceil(kin / 32) and
 // `blocks` = ceil(mout / 16); bias [mout] or null.
-// grid = (image, row tile)
+// grid = (image, row tile, walk of MTB row blocks)
 template <typename T, int W, int MTB>
 __global__ __launch_bounds__(kC16Block, 2) void conv16_kernel(int batch, int kin, int mout, int h, int tiles, int chunks,
                                                               int blocks, const T* __restrict__ in,
                                                               const uint4* __restrict__ wp, const T* __restrict__ bias,
-                                                              T* __restrict__ out) {
+                                                              T* __restrict__ out, float* __restrict__ partial,
+                                                              int ksplit) {
   using Tl = Tile16<W>;
   constexpr int TH = Tl::TH, RS = Tl::RS, POS = Tl::POS;
   extern __shared__ __align__(16) unsigned tile[];  // [POS][kC16Pitch]
 
-  const int total = batch * tiles;
+  // logical block = (walk over MTB row blocks, row tile, image), walk fastest: the workgroups that share an
+  // input tile run side by side
+  // With ksplit > 1 (small planes with many channels, where (image, tile) gives too few workgroups) a workgroup
+  // sums a share of the chunks and writes partial[split][...] in fp32; the splits are added afterwards, in order.
+  const int walks = (blocks + MTB - 1) / MTB;
+  const int total = batch * tiles * walks * ksplit;
   const int lb = logical_block(total);
   if (lb >= total) return;
-  const int n = lb / tiles, r0 = (lb % tiles) * TH;
+  const int split = lb % ksplit, lw = lb / ksplit;
+  const int mb0 = (lw % walks) * MTB, n = lw / walks / tiles, r0 = (lw / walks % tiles) * TH;
+  const int per_split = (chunks + ksplit - 1) / ksplit;
+  const int ch_lo = split * per_split, ch_hi = min(chunks, ch_lo + per_split);
   const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int plane = h * W;
 
-  for (int e = threadIdx.x; e < POS * kC16Pitch; e += kC16Block) tile[e] = 0u;  // the padding stays zero
+  // rows of the tile that lie in the image (a plane lower than the tile: 14 x 14 and 7 x 7 planes are one tile
+  // of 32 / 64 rows), and the pixel groups that hold any of their pixels
+  const int rows = min(TH, h - r0);
+  const int live_groups = (rows * W + 15) / 16;
+  for (int e = threadIdx.x; e < (rows + 2) * RS * kC16Pitch; e += kC16Block) tile[e] = 0u;  // the padding stays zero
 
   // word index of the lane's B operand for each of its pixel groups (tap shifts are immediates)
   int bword[kC16Gpw];
 #pragma unroll
   for (int i = 0; i < kC16Gpw; ++i) {
-    const int q = (wave + 4 * i) * 16 + (lane & 15);
+    const int q = min((wave + 4 * i) * 16 + (lane & 15), rows * W - 1);  // (a pixel below the image: not stored)
     bword[i] = ((q / W + 1) * RS + q % W + 1) * kC16Pitch + (lane >> 4) * 4;
   }
 
-  for (int mb0 = 0; mb0 < blocks; mb0 += MTB) {
+  {
     c16f4 acc[kC16Gpw][MTB];
 #pragma unroll
     for (int i = 0; i < kC16Gpw; ++i)
 #pragma unroll
       for (int m = 0; m < MTB; ++m) acc[i][m] = c16f4{0.f, 0.f, 0.f, 0.f};
 
-    for (int ch = 0; ch < chunks; ++ch) {
-      if (chunks > 1 || mb0 == 0) {  // a single chunk stays staged for every walk
-        __syncthreads();             // the previous chunk's reads are done
+    for (int ch = ch_lo; ch < ch_hi; ++ch) {
+      {
+        __syncthreads();  // the previous chunk's reads are done
         // one buffer over the chunk's planes: channels past the tensor and rows outside the image fail
         // the range check and read zero
         const int kc = min(kC16Chunk, kin - ch * kC16Chunk);
         const rsrc_t rs = plane_rsrc(in + ((size_t)n * kin + (size_t)ch * kC16Chunk) * plane, kc * plane);
-        for (int e = threadIdx.x; e < (TH + 2) * 4 * W; e += kC16Block) {
-          const int col = e % W, ry = e / W % (TH + 2), oct = e / W / (TH + 2);
+        for (int e = threadIdx.x; e < (rows + 2) * 4 * W; e += kC16Block) {
+          const int col = e % W, ry = e / W % (rows + 2), oct = e / W / (rows + 2);
           const int row = r0 - 1 + ry;
           const bool live = row >= 0 && row < h;
           unsigned v[8];
@@ -138,6 +152,9 @@ __global__ __launch_bounds__(kC16Block, 2) void conv16_kernel(int batch, int kin
         }
 #pragma unroll
         for (int i = 0; i < kC16Gpw; ++i) {
+          // planes lower than the tile (uniform: the wave's remaining groups lie below the image)
+          if constexpr (W <= 14)
+            if (wave + 4 * i >= live_groups) break;
           const uint4 b = *reinterpret_cast<const uint4*>(tile + bword[i] + shift);
 #pragma unroll
           for (int m = 0; m < MTB; ++m) acc[i][m] = mma16<T>(a[m], b, acc[i][m]);
@@ -153,51 +170,75 @@ __global__ __launch_bounds__(kC16Block, 2) void conv16_kernel(int batch, int kin
       for (int r = 0; r < 4; ++r) {
         const int o = 16 * (mb0 + m) + 4 * (lane >> 4) + r;
         if (o >= mout) continue;
-        const float bv = bias ? ld(bias + o) : 0.f;
-        T* dst = out + ((size_t)n * mout + o) * plane + (size_t)r0 * W;
+        const float bv = bias && split == 0 ? ld(bias + o) : 0.f;
+        const size_t at = ((size_t)n * mout + o) * plane + (size_t)r0 * W;
 #pragma unroll
         for (int i = 0; i < kC16Gpw; ++i) {
           const int q = (wave + 4 * i) * 16 + (lane & 15);
-          if (r0 * W + q < plane) st(dst + q, acc[i][m][r] + bv);
+          if (r0 * W + q < plane) {
+            if (ksplit > 1)
+              partial[(size_t)split * batch * mout * plane + at + q] = acc[i][m][r] + bv;
+            else
+              st(out + at + q, acc[i][m][r] + bv);
+          }
         }
       }
     }
   }
 }
 
+size_t round_up_256(size_t n) { return (n + 255) / 256 * 256; }
 size_t pack_bytes(int kin, int mout) {
   return (size_t)9 * ceil_div(kin, kC16Chunk) * ceil_div(mout, 16) * 64 * sizeof(uint4);
 }
 
+// Chunk splits of a pass: enough for about two workgroups per CU, at least four chunks per split
+int conv16_splits(int batch, int kin, int mout, int h, int w, int mtb) {
+  const long base = std::max(1L, (long)batch * ceil_div(h, kC16Pix / w) * ceil_div(ceil_div(mout, 16), mtb));
+  if (base >= 256) return 1;
+  return (int)std::max<long>(1, std::min<long>((512 + base - 1) / base, ceil_div(kin, kC16Chunk) / 4));
+}
+
 template <typename T, int MTB>
 bool launch_conv16(int batch, int kin, int mout, int h, int w, const T* in, const uint4* wp, const T* bias, T* out,
-                   hipStream_t stream) {
+                   float* partial, hipStream_t stream) {
   const int chunks = ceil_div(kin, kC16Chunk), blocks = ceil_div(mout, 16);
+  const int ksplit = conv16_splits(batch, kin, mout, h, w, MTB);
 #define DK_C16(WW)                                                                                                     \
   {                                                                                                                    \
     const int tiles = ceil_div(h, Tile16<WW>::TH);                                                                     \
     const size_t lds = (size_t)Tile16<WW>::POS * kC16Pitch * sizeof(unsigned);                                         \
-    conv16_kernel<T, WW, MTB><<<(unsigned)xcd_grid_size((long)batch * tiles), kC16Block, lds, stream>>>(               \
-        batch, kin, mout, h, tiles, chunks, blocks, in, wp, bias, out);                                                \
+    const long wgs = (long)batch * tiles * ceil_div(blocks, MTB) * ksplit;                                             \
+    conv16_kernel<T, WW, MTB><<<(unsigned)xcd_grid_size(wgs), kC16Block, lds, stream>>>(                               \
+        batch, kin, mout, h, tiles, chunks, blocks, in, wp, bias, out, partial, ksplit);                               \
   }
   switch (w) {
+    case 7: DK_C16(7) break;
+    case 14: DK_C16(14) break;
     case 28: DK_C16(28) break;
     case 56: DK_C16(56) break;
     case 112: DK_C16(112) break;
     default: return false;
   }
 #undef DK_C16
+  if (ksplit > 1) launch_reduce_partials<float, T>(partial, ksplit, (long)batch * mout * h * w, out, stream);
   return true;
 }
 
 }  // namespace
 
 bool offset_conv16_supported(int cin, int cout, int h, int w) {
-  return cin >= 1 && cout >= 1 && cout <= 32 && h >= 1 && (w == 28 || w == 56 || w == 112) &&
+  return cin >= 1 && cout >= 1 && cout <= 32 && h >= 1 && (w == 7 || w == 14 || w == 28 || w == 56 || w == 112) &&
          (long)kC16Chunk * h * w * 2 < (1L << 31) && (long)cin * h * w < (1L << 31) && (long)cout * h * w < (1L << 31);
 }
 
-size_t offset_conv16_workspace(int cin, int cout) { return std::max(pack_bytes(cin, cout), pack_bytes(cout, cin)); }
+// packed weights of either pass, then the forward's partial outputs (the input gradient has one chunk: no splits)
+size_t offset_conv16_workspace(int batch, int cin, int cout, int h, int w) {
+  const int mtb = ceil_div(cout, 16) == 1 ? 1 : 2;
+  const int ks = conv16_splits(batch, cin, cout, h, w, mtb);
+  return round_up_256(std::max(pack_bytes(cin, cout), pack_bytes(cout, cin))) +
+         (ks > 1 ? (size_t)ks * batch * cout * h * w * sizeof(float) : 0);
+}
 
 template <typename T>
 bool offset_conv16_forward(int batch, int cin, int cout, int h, int w, const T* x, const T* weight, const T* bias,
@@ -205,10 +246,12 @@ bool offset_conv16_forward(int batch, int cin, int cout, int h, int w, const T* 
   if (!offset_conv16_supported(cin, cout, h, w)) return false;
   if (batch == 0) return true;
   uint4* wp = static_cast<uint4*>(ws);
+  float* partial = reinterpret_cast<float*>(static_cast<char*>(ws) +
+                                            round_up_256(std::max(pack_bytes(cin, cout), pack_bytes(cout, cin))));
   const int chunks = ceil_div(cin, kC16Chunk), blocks = ceil_div(cout, 16);
   conv16_pack_kernel<T><<<ceil_div(9 * chunks * blocks * 64, 256), 256, 0, stream>>>(weight, cout, cin, 0, chunks, blocks, wp);
-  return blocks == 1 ? launch_conv16<T, 1>(batch, cin, cout, h, w, x, wp, bias, out, stream)
-                     : launch_conv16<T, 2>(batch, cin, cout, h, w, x, wp, bias, out, stream);
+  return blocks == 1 ? launch_conv16<T, 1>(batch, cin, cout, h, w, x, wp, bias, out, partial, stream)
+                     : launch_conv16<T, 2>(batch, cin, cout, h, w, x, wp, bias, out, partial, stream);
 }
 
 template <typename T>
@@ -219,7 +262,8 @@ bool offset_conv16_backward_input(int batch, int cin, int cout, int h, int w, co
   uint4* wp = static_cast<uint4*>(ws);
   const int chunks = ceil_div(cout, kC16Chunk), blocks = ceil_div(cin, 16);
   conv16_pack_kernel<T><<<ceil_div(9 * chunks * blocks * 64, 256), 256, 0, stream>>>(weight, cout, cin, 1, chunks, blocks, wp);
-  return launch_conv16<T, 3>(batch, cout, cin, h, w, gout, wp, static_cast<const T*>(nullptr), gin, stream);
+  return launch_conv16<T, 3>(batch, cout, cin, h, w, gout, wp, static_cast<const T*>(nullptr), gin,
+                             static_cast<float*>(nullptr), stream);
 }
 
 #define DK_INST(T)                                                                                                      \

@@ -11,7 +11,7 @@ kernels multiply and add in float32 and round the results once) it runs
     ``force=True``: wherever they apply, also widths 7 / 14),
   * the bias gradient on the library's reduction kernel for every shape (the framework's
     reduction over (N, H, W) takes 60-230 us on the large planes),
-  * for float16 / bfloat16 tensors on planes 28, 56 or 112 wide, the forward and the input gradient on
+  * for float16 / bfloat16 tensors on planes 7, 14, 28, 56 or 112 wide, the forward and the input gradient on
     the library's 16-bit matrix-instruction kernel (the elements are the operands as they are),
   * everything else -- the input gradient of float32 tensors and of the other planes, and forward /
     weight gradient of the other shapes -- on the framework's convolution routines.

@@ -285,8 +285,9 @@ int dk_nd_linear_sample_backward_coord(const dk_nd_desc *desc, const void *out_g
  * exact products of the 16-bit elements; results rounded once), in_channels a multiple of 16,
  * out_channels <= 16 or 18 or 20, width 7, 14, 28, 56 or 112.  dk_offset_conv_supported() tells
  * whether a shape is covered, dk_offset_conv_worthwhile() whether it is also expected to beat the
- * library convolution (planes 28 wide and wider with enough images to fill the GPU); the caller
- * keeps its library convolution otherwise.
+ * library convolution (float32: planes 28 wide and wider with enough images to fill the GPU;
+ * float16 / bfloat16: every covered plane with at least 64 (image, 448-pixel tile) items); the
+ * caller keeps its library convolution otherwise.
  *   input [batch, in_channels, h, w], weight [out_channels, in_channels, 3, 3],
  *   bias [out_channels], output [batch, out_channels, h, w]; workspace: packed weights. */
 typedef struct dk_offset_conv_desc {
@@ -317,7 +318,7 @@ int dk_offset_conv_backward_bias(const dk_offset_conv_desc *desc, const void *ou
 
 /* Gradient of that convolution's input (what autograd derives for the rotation_conv call at
  * modules/deform_kernel.py:214), input_grad [batch, in_channels, h, w] (fully written), for float16 /
- * bfloat16 tensors on planes 28, 56 or 112 wide: the 16-bit matrix instructions multiply the tensors'
+ * bfloat16 tensors on planes 7, 14, 28, 56 or 112 wide: the 16-bit matrix instructions multiply the tensors'
  * elements as they are (exact products, fp32 sums, one rounding of the result).  The forward of such
  * tensors and planes runs on the same kernel.  Other shapes and float32 return DK_ERR_UNSUPPORTED (the
  * workspace query 0): the caller keeps its library's routine there. */
