@@ -639,10 +639,12 @@ def layer_workload(a):
     dev = torch.device("cuda:0")
     torch.manual_seed(0)
     N, C, H = a.batch, 144, 56
+    tdtype = getattr(torch, DTYPES[a.dtype])
     m = LocalDeformKernel2d((4, 4), C, C, 3, 1, 1, 1, C, 1, False, "scope").to(dev)
     torch.nn.init.normal_(m.rotation_conv.weight, std=0.01)
-    x = torch.randn(N, C, H, H, device=dev, requires_grad=True)
-    gout = torch.randn(N, C, H, H, device=dev)
+    m = m.to(tdtype)
+    x = torch.randn(N, C, H, H, device=dev).to(tdtype).requires_grad_()
+    gout = torch.randn(N, C, H, H, device=dev).to(tdtype)
 
     def timed(fn):
         for _ in range(a.warmup):
@@ -673,8 +675,8 @@ def layer_workload(a):
         res[name] = {"step_us": timed(step), "forward_us": timed(forward)}
     res["library_offset_branch_alone"] = {"step_us": timed(branch)}
     print(json.dumps({"metric": "LocalDeformKernel2d layer fwd+bwd through the modules (secondary workload)",
-                      "config": {"workload": "layer_cfg2: N=%d C=144 56x56 k=3 scope=4x4 rotation_clip='scope' fp32" % N},
-                      "variants": res, "n_gpus": 1, "dtype": "fp32", "data": "synthetic"}))
+                      "config": {"workload": "layer_cfg2: N=%d C=144 56x56 k=3 scope=4x4 rotation_clip='scope' %s" % (N, a.dtype)},
+                      "variants": res, "n_gpus": 1, "dtype": a.dtype, "data": "synthetic"}))
 
 
 def mobilenet_workload(a):
