@@ -648,19 +648,28 @@ int dk_image_depthwise_backward_weight(const dk_conv_desc* desc, const void* out
   return ok ? st : DK_ERR_UNSUPPORTED;
 }
 
-static int check_offset_conv(const dk_offset_conv_desc* d) {
+// forward: the call is (or asks about) the forward, the one pass that has a stride-2 kernel
+static int check_offset_conv(const dk_offset_conv_desc* d, bool forward = false) {
   if (!d) return DK_ERR_NULL_POINTER;
   if (d->batch < 0 || d->in_channels <= 0 || d->out_channels <= 0 || d->h <= 0 || d->w <= 0) return DK_ERR_BAD_SHAPE;
+  if (d->stride < 0 || d->stride > 2) return DK_ERR_BAD_SHAPE;
   if (d->dtype != DK_F32 && d->dtype != DK_F16 && d->dtype != DK_BF16) return d->dtype == DK_F64 ? DK_ERR_UNSUPPORTED : DK_ERR_BAD_DTYPE;
   if ((long)d->batch * d->in_channels * d->h * d->w > kMaxElems) return DK_ERR_TOO_LARGE;
+  if (d->stride == 2)
+    return forward && d->dtype != DK_F32 && d->in_channels % 16 == 0 &&
+                   offset_conv16_s2_supported(d->in_channels, d->out_channels, d->h, d->w)
+               ? DK_OK
+               : DK_ERR_UNSUPPORTED;
   if (!offset_conv_supported(d->in_channels, d->out_channels, d->h, d->w)) return DK_ERR_UNSUPPORTED;
   return DK_OK;
 }
 
-int dk_offset_conv_supported(const dk_offset_conv_desc* desc) { return check_offset_conv(desc) == DK_OK; }
+int dk_offset_conv_supported(const dk_offset_conv_desc* desc) { return check_offset_conv(desc, true) == DK_OK; }
 
 int dk_offset_conv_worthwhile(const dk_offset_conv_desc* desc) {
-  if (check_offset_conv(desc) != DK_OK) return 0;
+  if (check_offset_conv(desc, true) != DK_OK) return 0;
+  if (desc->stride == 2)  // as below, on the output plane
+    return (long)desc->batch * ((((desc->h - 1) / 2 + 1) * (desc->w / 2) + 447) / 448) >= 64;
   // 16-bit tensors: forward and input gradient on 16-bit matrix instructions are ahead of the library's on every
   // plane they cover once there are workgroups ((image, 448-pixel tile) items) for a quarter of the CUs
   if (desc->dtype != DK_F32 && offset_conv16_supported(desc->in_channels, desc->out_channels, desc->h, desc->w))
@@ -674,19 +683,20 @@ static bool offset_conv_on_16_bit_matrix(const dk_offset_conv_desc* d) {
 }
 
 static size_t offset_conv_forward_need(const dk_offset_conv_desc* d) {
+  if (d->stride == 2) return offset_conv16_s2_workspace(d->batch, d->in_channels, d->out_channels, d->h, d->w);
   return offset_conv_on_16_bit_matrix(d) ? offset_conv16_workspace(d->batch, d->in_channels, d->out_channels, d->h, d->w)
                                          : offset_conv_workspace(d->batch, d->in_channels, d->out_channels, d->h, d->w);
 }
 
 size_t dk_offset_conv_forward_workspace(const dk_offset_conv_desc* desc) {
-  if (check_offset_conv(desc) != DK_OK) return 0;
+  if (check_offset_conv(desc, true) != DK_OK) return 0;
   return offset_conv_forward_need(desc);
 }
 
 int dk_offset_conv_forward(const dk_offset_conv_desc* desc, const void* input, const void* weight,
                            const void* bias, void* output, void* workspace, size_t workspace_bytes,
                            void* stream) {
-  const int rc = check_offset_conv(desc);
+  const int rc = check_offset_conv(desc, true);
   if (rc != DK_OK) return rc;
   if (!input || !weight || !bias || !output) return DK_ERR_NULL_POINTER;
   const size_t need = offset_conv_forward_need(desc);
@@ -695,6 +705,12 @@ int dk_offset_conv_forward(const dk_offset_conv_desc* desc, const void* input, c
   const bool matrix16 = offset_conv_on_16_bit_matrix(desc);
   const int st = by_dtype(desc->dtype, [&]<typename T>() {
     if constexpr (sizeof(T) == 2) {
+      if (desc->stride == 2) {
+        ok = offset_conv16_s2_forward<T>(desc->batch, desc->in_channels, desc->out_channels, desc->h, desc->w,
+                                         in<T>(input), in<T>(weight), in<T>(bias), out<T>(output), workspace,
+                                         static_cast<hipStream_t>(stream));
+        return;
+      }
       if (matrix16) {
         ok = offset_conv16_forward<T>(desc->batch, desc->in_channels, desc->out_channels, desc->h, desc->w, in<T>(input),
                                       in<T>(weight), in<T>(bias), out<T>(output), workspace, static_cast<hipStream_t>(stream));

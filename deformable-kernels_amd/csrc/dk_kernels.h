@@ -142,6 +142,13 @@ template <typename T>
 bool offset_conv16_backward_input(int batch, int cin, int cout, int h, int w, const T* gout, const T* weight, T* gin,
                                   void* ws, hipStream_t stream);
 
+// ... and its forward with stride 2 (input planes 14 / 28 / 56 / 112 wide; h, w: the input plane)
+bool offset_conv16_s2_supported(int cin, int cout, int h, int w);
+size_t offset_conv16_s2_workspace(int batch, int cin, int cout, int h, int w);
+template <typename T>
+bool offset_conv16_s2_forward(int batch, int cin, int cout, int h, int w, const T* x, const T* weight, const T* bias,
+                              T* out, void* ws, hipStream_t stream);
+
 // dk_local_nhwc.hip: the local operator on channels-last tensors, all dtypes, any geometry whose tables fit LDS
 bool nhwc_supported(const Geo& g, int dtype);
 template <typename T>

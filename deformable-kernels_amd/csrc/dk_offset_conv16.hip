@@ -187,6 +187,141 @@ __global__ __launch_bounds__(kC16Block, 2) void conv16_kernel(int batch, int kin
   }
 }
 
+
+// ---- stride 2 (forward only) -------------------------------------------------------------------------------
+// out[m][(oy, ox)] = sum over taps, channels of A_t[m][k] * in[k][(2 oy + dy - 1, 2 ox + dx - 1)].  A tile of 448
+// output pixels needs 2 TH + 1 input rows of the full width, so the chunk is 16 channels (v_mfma_f32_16x16x16):
+// a position's 16 elements in 32 bytes of a 40-byte slot (17 rows of a 112-wide plane: 77 KB, two workgroups per
+// CU); a lane's B operand -- output pixel l % 16, channels 4 (l / 16) .. + 3 -- is one 8-byte read at the input
+// position (2 r, 2 c) + (dy, dx) of the zero-padded tile, and the 16 lanes of a pass, 20 words apart, hit
+// disjoint banks.
+constexpr int kS2Chunk = 16;
+constexpr int kS2Pitch = 10;  // 32-bit words per staged position: 8 of data, 2 of bank skew
+
+typedef __bf16 c16b4 __attribute__((ext_vector_type(4)));
+typedef _Float16 c16h4 __attribute__((ext_vector_type(4)));
+
+template <typename T>
+__device__ __forceinline__ c16f4 mma16k16(const uint2& a, const uint2& b, c16f4 acc) {
+  if constexpr (std::is_same<T, bf16_t>::value)
+    return __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(__builtin_bit_cast(c16b4, a), __builtin_bit_cast(c16b4, b), acc, 0, 0, 0);
+  else
+    return __builtin_amdgcn_mfma_f32_16x16x16f16(__builtin_bit_cast(c16h4, a), __builtin_bit_cast(c16h4, b), acc, 0, 0, 0);
+}
+
+// wp[t][chunk][block][lane] = the four elements W[16 block + lane % 16][16 chunk + 4 (lane / 16) .. + 3][t]
+template <typename T>
+__global__ void conv16_s2_pack_kernel(const T* __restrict__ weight, int O, int C, int chunks, int blocks,
+                                      uint2* __restrict__ wp) {
+  const int idx = blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= 9 * chunks * blocks * 64) return;
+  const int lane = idx % 64, mb = idx / 64 % blocks, ch = idx / 64 / blocks % chunks, t = idx / 64 / blocks / chunks;
+  const int o = 16 * mb + (lane & 15), c0 = kS2Chunk * ch + 4 * (lane >> 4);
+  const unsigned short* w = reinterpret_cast<const unsigned short*>(weight);
+  unsigned v[4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) v[j] = (o < O && c0 + j < C) ? w[((size_t)o * C + c0 + j) * 9 + t] : 0u;
+  wp[idx] = make_uint2(v[0] | v[1] << 16, v[2] | v[3] << 16);
+}
+
+// in [batch][kin][h][WIN] -> out [batch][mout][ho][WIN / 2], ho = (h - 1) / 2 + 1 (padding 1, 3 x 3 taps)
+// grid = (image, tile of output rows, chunk split)
+template <typename T, int WIN, int MTB>
+__global__ __launch_bounds__(kC16Block, 2) void conv16_s2_kernel(int batch, int kin, int mout, int h, int ho, int tiles,
+                                                                 int chunks, int blocks, const T* __restrict__ in,
+                                                                 const uint2* __restrict__ wp,
+                                                                 const T* __restrict__ bias, T* __restrict__ out,
+                                                                 float* __restrict__ partial, int ksplit) {
+  constexpr int W = WIN / 2, TH = kC16Pix / W, RS = WIN + 2;
+  static_assert(WIN % 2 == 0 && TH * W == kC16Pix, "whole output rows");
+  extern __shared__ __align__(16) unsigned tile[];  // [2 rows + 1][RS][kS2Pitch]
+
+  const int total = batch * tiles * ksplit;
+  const int lb = logical_block(total);
+  if (lb >= total) return;
+  const int split = lb % ksplit, n = lb / ksplit / tiles, r0 = (lb / ksplit % tiles) * TH;
+  const int per_split = (chunks + ksplit - 1) / ksplit;
+  const int ch_lo = split * per_split, ch_hi = min(chunks, ch_lo + per_split);
+  const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int plane_in = h * WIN, plane = ho * W;
+
+  const int rows = min(TH, ho - r0);  // output rows of the tile inside the image
+  const int rows_in = 2 * rows + 1;   // input rows 2 r0 - 1 .. 2 (r0 + rows - 1) + 1
+  const int live_groups = (rows * W + 15) / 16;
+  for (int e = threadIdx.x; e < rows_in * RS * kS2Pitch; e += kC16Block) tile[e] = 0u;  // the padding stays zero
+
+  int bword[kC16Gpw];
+#pragma unroll
+  for (int i = 0; i < kC16Gpw; ++i) {
+    const int q = min((wave + 4 * i) * 16 + (lane & 15), rows * W - 1);  // (a pixel below the image: not stored)
+    bword[i] = (2 * (q / W) * RS + 2 * (q % W)) * kS2Pitch + (lane >> 4) * 2;
+  }
+
+  c16f4 acc[kC16Gpw][MTB];
+#pragma unroll
+  for (int i = 0; i < kC16Gpw; ++i)
+#pragma unroll
+    for (int m = 0; m < MTB; ++m) acc[i][m] = c16f4{0.f, 0.f, 0.f, 0.f};
+
+  for (int ch = ch_lo; ch < ch_hi; ++ch) {
+    __syncthreads();  // the previous chunk's reads are done
+    const int kc = min(kS2Chunk, kin - ch * kS2Chunk);
+    const rsrc_t rs = plane_rsrc(in + ((size_t)n * kin + (size_t)ch * kS2Chunk) * plane_in, kc * plane_in);
+    for (int e = threadIdx.x; e < rows_in * 2 * WIN; e += kC16Block) {
+      const int col = e % WIN, ry = e / WIN % rows_in, oct = e / WIN / rows_in;
+      const int row = 2 * r0 - 1 + ry;
+      const bool live = row >= 0 && row < h;
+      unsigned v[8];
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const unsigned o = live ? (unsigned)((oct * 8 + j) * plane_in + row * WIN + col) * 2u : kOutOfRange;
+        v[j] = __builtin_amdgcn_raw_buffer_load_b16(rs, (int)o, 0, 0);
+      }
+      uint2* dst = reinterpret_cast<uint2*>(tile + (ry * RS + col + 1) * kS2Pitch + oct * 4);
+      dst[0] = make_uint2(v[0] | v[1] << 16, v[2] | v[3] << 16);
+      dst[1] = make_uint2(v[4] | v[5] << 16, v[6] | v[7] << 16);
+    }
+    __syncthreads();
+#pragma unroll
+    for (int t = 0; t < 9; ++t) {
+      const int shift = ((t / 3) * RS + t % 3) * kS2Pitch;
+      uint2 a[MTB];
+#pragma unroll
+      for (int m = 0; m < MTB; ++m) a[m] = wp[((size_t)(t * chunks + ch) * blocks + min(m, blocks - 1)) * 64 + lane];
+#pragma unroll
+      for (int i = 0; i < kC16Gpw; ++i) {
+        if constexpr (W <= 14)
+          if (wave + 4 * i >= live_groups) break;
+        const uint2 b = *reinterpret_cast<const uint2*>(tile + bword[i] + shift);
+#pragma unroll
+        for (int m = 0; m < MTB; ++m) acc[i][m] = mma16k16<T>(a[m], b, acc[i][m]);
+      }
+    }
+  }
+
+#pragma unroll
+  for (int m = 0; m < MTB; ++m) {
+    if (m >= blocks) break;
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      const int o = 16 * m + 4 * (lane >> 4) + r;
+      if (o >= mout) continue;
+      const float bv = bias && split == 0 ? ld(bias + o) : 0.f;
+      const size_t at = ((size_t)n * mout + o) * plane + (size_t)r0 * W;
+#pragma unroll
+      for (int i = 0; i < kC16Gpw; ++i) {
+        const int q = (wave + 4 * i) * 16 + (lane & 15);
+        if (r0 * W + q < plane) {
+          if (ksplit > 1)
+            partial[(size_t)split * batch * mout * plane + at + q] = acc[i][m][r] + bv;
+          else
+            st(out + at + q, acc[i][m][r] + bv);
+        }
+      }
+    }
+  }
+}
+
 size_t round_up_256(size_t n) { return (n + 255) / 256 * 256; }
 size_t pack_bytes(int kin, int mout) {
   return (size_t)9 * ceil_div(kin, kC16Chunk) * ceil_div(mout, 16) * 64 * sizeof(uint4);
@@ -266,9 +401,77 @@ bool offset_conv16_backward_input(int batch, int cin, int cout, int h, int w, co
                              static_cast<float*>(nullptr), stream);
 }
 
+
+// stride 2: input planes 14, 28, 56 or 112 wide (even), at most 32 outputs
+bool offset_conv16_s2_supported(int cin, int cout, int h, int w) {
+  return cin >= 1 && cout >= 1 && cout <= 32 && h >= 1 && (w == 14 || w == 28 || w == 56 || w == 112) &&
+         (long)kS2Chunk * h * w * 2 < (1L << 31) && (long)cin * h * w < (1L << 31) && (long)cout * h * w < (1L << 31);
+}
+
+static int s2_splits(int batch, int cin, int ho, int wo) {
+  const long base = std::max(1L, (long)batch * ceil_div(ho, kC16Pix / wo));
+  if (base >= 256) return 1;
+  return (int)std::max<long>(1, std::min<long>((512 + base - 1) / base, ceil_div(cin, kS2Chunk) / 4));
+}
+
+static size_t s2_pack_bytes(int cin, int cout) {
+  return (size_t)9 * ceil_div(cin, kS2Chunk) * ceil_div(cout, 16) * 64 * sizeof(uint2);
+}
+
+size_t offset_conv16_s2_workspace(int batch, int cin, int cout, int h, int w) {
+  const int ho = (h - 1) / 2 + 1, wo = w / 2;
+  const int ks = s2_splits(batch, cin, ho, wo);
+  return (s2_pack_bytes(cin, cout) + 255) / 256 * 256 + (ks > 1 ? (size_t)ks * batch * cout * ho * wo * sizeof(float) : 0);
+}
+
+template <typename T, int MTB>
+static bool launch_conv16_s2(int batch, int cin, int cout, int h, int w, const T* x, const uint2* wp, const T* bias,
+                             T* out, float* partial, hipStream_t stream) {
+  const int ho = (h - 1) / 2 + 1, wo = w / 2;
+  const int chunks = ceil_div(cin, kS2Chunk), blocks = ceil_div(cout, 16);
+  const int ksplit = s2_splits(batch, cin, ho, wo);
+  bool ok = true;
+#define DK_S2(WW)                                                                                                      \
+  {                                                                                                                    \
+    auto kernel = conv16_s2_kernel<T, WW, MTB>;                                                                        \
+    constexpr int TH = kC16Pix / (WW / 2);                                                                             \
+    const int tiles = ceil_div(ho, TH);                                                                                \
+    const size_t lds = (size_t)(2 * std::min(TH, ho) + 1) * (WW + 2) * kS2Pitch * sizeof(unsigned);                    \
+    if (lds > (size_t)kMaxDynamicLds || !allow_max_dynamic_lds(reinterpret_cast<const void*>(kernel)))                 \
+      ok = false;                                                                                                      \
+    else                                                                                                               \
+      kernel<<<(unsigned)xcd_grid_size((long)batch * tiles * ksplit), kC16Block, lds, stream>>>(                       \
+          batch, cin, cout, h, ho, tiles, chunks, blocks, x, wp, bias, out, partial, ksplit);                          \
+  }
+  switch (w) {
+    case 14: DK_S2(14) break;
+    case 28: DK_S2(28) break;
+    case 56: DK_S2(56) break;
+    case 112: DK_S2(112) break;
+    default: ok = false;
+  }
+#undef DK_S2
+  if (ok && ksplit > 1) launch_reduce_partials<float, T>(partial, ksplit, (long)batch * cout * ho * wo, out, stream);
+  return ok;
+}
+
+template <typename T>
+bool offset_conv16_s2_forward(int batch, int cin, int cout, int h, int w, const T* x, const T* weight, const T* bias,
+                              T* out, void* ws, hipStream_t stream) {
+  if (!offset_conv16_s2_supported(cin, cout, h, w)) return false;
+  if (batch == 0) return true;
+  uint2* wp = static_cast<uint2*>(ws);
+  float* partial = reinterpret_cast<float*>(static_cast<char*>(ws) + (s2_pack_bytes(cin, cout) + 255) / 256 * 256);
+  const int chunks = ceil_div(cin, kS2Chunk), blocks = ceil_div(cout, 16);
+  conv16_s2_pack_kernel<T><<<ceil_div(9 * chunks * blocks * 64, 256), 256, 0, stream>>>(weight, cout, cin, chunks, blocks, wp);
+  return blocks == 1 ? launch_conv16_s2<T, 1>(batch, cin, cout, h, w, x, wp, bias, out, partial, stream)
+                     : launch_conv16_s2<T, 2>(batch, cin, cout, h, w, x, wp, bias, out, partial, stream);
+}
+
 #define DK_INST(T)                                                                                                      \
   template bool offset_conv16_forward<T>(int, int, int, int, int, const T*, const T*, const T*, T*, void*, hipStream_t); \
-  template bool offset_conv16_backward_input<T>(int, int, int, int, int, const T*, const T*, T*, void*, hipStream_t);
+  template bool offset_conv16_backward_input<T>(int, int, int, int, int, const T*, const T*, T*, void*, hipStream_t);  \
+  template bool offset_conv16_s2_forward<T>(int, int, int, int, int, const T*, const T*, const T*, T*, void*, hipStream_t);
 DK_INST(__half)
 DK_INST(bf16_t)
 #undef DK_INST

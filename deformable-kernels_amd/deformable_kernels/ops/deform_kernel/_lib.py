@@ -34,7 +34,8 @@ class NdDesc(ctypes.Structure):
 
 
 class OffsetConvDesc(ctypes.Structure):
-    _fields_ = [(n, ctypes.c_int32) for n in ("batch", "in_channels", "out_channels", "h", "w", "dtype")]
+    # stride: 0 or 1 for stride 1, 2 for the down-sampling layers (forward of 16-bit tensors only)
+    _fields_ = [(n, ctypes.c_int32) for n in ("batch", "in_channels", "out_channels", "h", "w", "dtype", "stride")]
 
 
 class DkError(RuntimeError):

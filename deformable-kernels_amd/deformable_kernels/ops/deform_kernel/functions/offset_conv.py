@@ -12,7 +12,8 @@ kernels multiply and add in float32 and round the results once) it runs
   * the bias gradient on the library's reduction kernel for every shape (the framework's
     reduction over (N, H, W) takes 60-230 us on the large planes),
   * for float16 / bfloat16 tensors on planes 7, 14, 28, 56 or 112 wide, the forward and the input gradient on
-    the library's 16-bit matrix-instruction kernel (the elements are the operands as they are),
+    the library's 16-bit matrix-instruction kernel (the elements are the operands as they are); with stride 2
+    (input planes 14, 28, 56 or 112 wide) the forward alone,
   * everything else -- the input gradient of float32 tensors and of the other planes, and forward /
     weight gradient of the other shapes -- on the framework's convolution routines.
 
@@ -32,9 +33,9 @@ def _pair(v):
     return tuple(int(e) for e in v) if isinstance(v, (tuple, list)) else (int(v), int(v))
 
 
-def _desc(input, weight, out=None):
+def _desc(input, weight, out=None, stride=1):
     h, w = (input.size(2), input.size(3)) if out is None else (out.size(2), out.size(3))
-    return _lib.OffsetConvDesc(input.size(0), input.size(1), weight.size(0), h, w, _lib.dtype_tag(input))
+    return _lib.OffsetConvDesc(input.size(0), input.size(1), weight.size(0), h, w, _lib.dtype_tag(input), stride)
 
 
 _NATIVE_DTYPES = (torch.float32, torch.float16, torch.bfloat16)
@@ -56,10 +57,11 @@ def offset_conv_supported(input, weight, bias, stride, padding, dilation, worthw
         return False
     if tuple(weight.shape[2:]) != (3, 3) or weight.size(1) != input.size(1):
         return False
-    if _pair(stride) != (1, 1) or _pair(padding) != (1, 1) or _pair(dilation) != (1, 1):
+    if _pair(stride) not in ((1, 1), (2, 2)) or _pair(padding) != (1, 1) or _pair(dilation) != (1, 1):
         return False
     L = _lib.lib()
-    return bool((L.dk_offset_conv_worthwhile if worthwhile else L.dk_offset_conv_supported)(_desc(input, weight)))
+    desc = _desc(input, weight, stride=_pair(stride)[0])   # stride 2: the library answers for the forward alone
+    return bool((L.dk_offset_conv_worthwhile if worthwhile else L.dk_offset_conv_supported)(desc))
 
 
 class OffsetConvFunction(Function):
@@ -74,8 +76,9 @@ class OffsetConvFunction(Function):
         if not native:
             return F.conv2d(input, weight, bias, stride, padding, dilation)
         b = bias.contiguous() if bias is not None else input.new_zeros(weight.size(0))
-        out = input.new_empty(input.size(0), weight.size(0), input.size(2), input.size(3))
-        desc = _desc(input, weight)
+        s = stride[0]
+        out = input.new_empty(input.size(0), weight.size(0), (input.size(2) - 1) // s + 1, (input.size(3) - 1) // s + 1)
+        desc = _desc(input, weight, stride=s)
         L = _lib.lib()
         with torch.cuda.device(input.device):
             ws, nbytes = _lib.workspace(L.dk_offset_conv_forward_workspace(desc), input.device)
@@ -95,7 +98,7 @@ class OffsetConvFunction(Function):
         L = _lib.lib()
         # the input gradient has a kernel of its own for 16-bit tensors on the wider planes, the weight
         # gradient for 15 and more outputs: a workspace query of 0 says "not covered"
-        desc = _desc(input, weight)
+        desc = _desc(input, weight, stride=stride[0])
         native_weight = need_weight and ctx.native and L.dk_offset_conv_backward_weight_workspace(desc) > 0
         # 16-bit tensors: the weight-gradient kernel multiplies in fp32 and the framework's on 16-bit matrix
         # instructions, which is ahead on every plane (bf16, batch 128: 317 / 264 / 95 us against 330 / 290 / 150

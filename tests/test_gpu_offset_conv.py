@@ -90,6 +90,35 @@ def test_sixteen_bit_tensors_match_float64_on_the_rounded_inputs(shape, dtype, t
     assert rel_err(x.grad.double().cpu(), xd.grad.cpu()) < tol
 
 
+@pytest.mark.parametrize("dtype,tol", [(torch.float16, 2e-3), (torch.bfloat16, 1e-2)])
+@pytest.mark.parametrize("shape", [(2, 96, 112, 112, 18), (3, 144, 56, 56, 18), (2, 192, 28, 28, 18), (5, 576, 14, 14, 18),
+                                   (2, 32, 9, 56, 18), (1, 16, 1, 14, 16), (2, 48, 30, 28, 20), (2, 32, 17, 112, 7)])
+def test_stride_2_forward_of_sixteen_bit_tensors(shape, dtype, tol):
+    """The down-sampling layers' convolution (stride 2, padding 1): the forward of float16 / bfloat16 tensors on
+    the 16-bit matrix instructions (whole, partial and single-row tiles, half chunks of 16 channels, planes lower
+    than a tile, chunk splits), its gradients on the framework's routines, the bias gradient on the library's."""
+    from deformable_kernels.ops.deform_kernel.functions import offset_conv, offset_conv_supported
+    N, C, H, W, O = shape
+    g = torch.Generator().manual_seed(43)
+    dev = torch.device("cuda:0")
+    x = torch.randn(N, C, H, W, generator=g).to(dtype).to(dev).requires_grad_()
+    w = (torch.randn(O, C, 3, 3, generator=g) * 0.05).to(dtype).to(dev).requires_grad_()
+    b = torch.randn(O, generator=g).to(dtype).to(dev).requires_grad_()
+    assert offset_conv_supported(x, w, b, 2, 1, 1)
+    assert not offset_conv_supported(x.float(), w.float(), b.float(), 2, 1, 1)
+    out = offset_conv(x, w, b, stride=2, force=True)
+    xd, wd, bd = [t.detach().double().requires_grad_() for t in (x, w, b)]
+    want = F.conv2d(xd, wd, bd, stride=2, padding=1)
+    assert out.shape == want.shape and out.dtype == dtype
+    assert rel_err(out.detach().double().cpu(), want.detach().cpu()) < tol
+    gout = torch.randn(want.shape, generator=g).to(dtype).to(dev)
+    out.backward(gout)
+    want.backward(gout.double())
+    assert rel_err(x.grad.double().cpu(), xd.grad.cpu()) < tol
+    assert rel_err(w.grad.double().cpu(), wd.grad.cpu()) < 2 * tol   # the framework's 16-bit weight gradient
+    assert rel_err(b.grad.double().cpu(), bd.grad.cpu()) < tol
+
+
 @pytest.mark.parametrize("dtype,tol", [(torch.float32, 1e-5), (torch.bfloat16, 1e-2)])
 def test_fewer_than_15_outputs_take_the_library_weight_gradient(dtype, tol):
     """The forward covers 1 to 16 outputs, the weight gradient 15 and more: with 7 outputs its workspace query
