@@ -142,16 +142,18 @@ int main() {
   oc.w = 21;
   EXPECT(dk_offset_conv_backward_input(&oc, one, one, one, one, 1 << 30, nullptr) == DK_ERR_UNSUPPORTED);
   oc.w = 14;
-  // stride 2: the forward of 16-bit tensors only
+  // stride 2: forward and input gradient of 16-bit tensors only
   oc.w = oc.h = 56, oc.stride = 2;
   EXPECT(dk_offset_conv_supported(&oc) == 1);
   EXPECT(dk_offset_conv_forward_workspace(&oc) > 0);
   EXPECT(dk_offset_conv_forward(&oc, one, one, one, one, one, 0, nullptr) == DK_ERR_WORKSPACE);
-  EXPECT(dk_offset_conv_backward_input_workspace(&oc) == 0);
+  EXPECT(dk_offset_conv_backward_input_workspace(&oc) > 0);
+  EXPECT(dk_offset_conv_backward_input(&oc, one, one, one, one, 0, nullptr) == DK_ERR_WORKSPACE);
   EXPECT(dk_offset_conv_backward_weight_workspace(&oc) == 0);
-  EXPECT(dk_offset_conv_backward_input(&oc, one, one, one, one, 1 << 30, nullptr) == DK_ERR_UNSUPPORTED);
+  EXPECT(dk_offset_conv_backward_weight(&oc, one, one, one, one, 1 << 30, nullptr) == DK_ERR_UNSUPPORTED);
   oc.dtype = DK_F32;
   EXPECT(dk_offset_conv_supported(&oc) == 0);
+  EXPECT(dk_offset_conv_backward_input_workspace(&oc) == 0);
   oc.dtype = DK_BF16, oc.stride = 3;
   EXPECT(dk_offset_conv_forward(&oc, one, one, one, one, one, 1 << 30, nullptr) == DK_ERR_BAD_SHAPE);
   oc.stride = 0, oc.w = oc.h = 14;

@@ -725,15 +725,21 @@ int dk_offset_conv_forward(const dk_offset_conv_desc* desc, const void* input, c
 }
 
 static int check_offset_conv_backward_input(const dk_offset_conv_desc* d) {
-  const int rc = check_offset_conv(d);
+  const int rc = check_offset_conv(d, true);  // (stride 2: what holds for its forward holds for this pass)
   if (rc != DK_OK) return rc;
   if ((long)d->batch * d->out_channels * d->h * d->w > kMaxElems) return DK_ERR_TOO_LARGE;
+  if (d->stride == 2) return DK_OK;
   return offset_conv_on_16_bit_matrix(d) ? DK_OK : DK_ERR_UNSUPPORTED;
+}
+
+static size_t offset_conv_backward_input_need(const dk_offset_conv_desc* d) {
+  return d->stride == 2 ? offset_conv16_s2_backward_input_workspace(d->in_channels, d->out_channels)
+                        : offset_conv16_workspace(d->batch, d->in_channels, d->out_channels, d->h, d->w);
 }
 
 size_t dk_offset_conv_backward_input_workspace(const dk_offset_conv_desc* desc) {
   if (check_offset_conv_backward_input(desc) != DK_OK) return 0;
-  return offset_conv16_workspace(desc->batch, desc->in_channels, desc->out_channels, desc->h, desc->w);
+  return offset_conv_backward_input_need(desc);
 }
 
 int dk_offset_conv_backward_input(const dk_offset_conv_desc* desc, const void* out_grad, const void* weight,
@@ -741,9 +747,17 @@ int dk_offset_conv_backward_input(const dk_offset_conv_desc* desc, const void* o
   const int rc = check_offset_conv_backward_input(desc);
   if (rc != DK_OK) return rc;
   if (!out_grad || !weight || !input_grad) return DK_ERR_NULL_POINTER;
-  if (!workspace || workspace_bytes < offset_conv16_workspace(desc->batch, desc->in_channels, desc->out_channels, desc->h, desc->w)) return DK_ERR_WORKSPACE;
+  if (!workspace || workspace_bytes < offset_conv_backward_input_need(desc)) return DK_ERR_WORKSPACE;
   bool ok = false;
   const int st = by_dtype(desc->dtype, [&]<typename T>() {
+    if constexpr (sizeof(T) == 2) {
+      if (desc->stride == 2) {
+        ok = offset_conv16_s2_backward_input<T>(desc->batch, desc->in_channels, desc->out_channels, desc->h, desc->w,
+                                                in<T>(out_grad), in<T>(weight), out<T>(input_grad), workspace,
+                                                static_cast<hipStream_t>(stream));
+        return;
+      }
+    }
     if constexpr (sizeof(T) == 2)
       ok = offset_conv16_backward_input<T>(desc->batch, desc->in_channels, desc->out_channels, desc->h, desc->w,
                                            in<T>(out_grad), in<T>(weight), out<T>(input_grad), workspace,

@@ -148,6 +148,10 @@ size_t offset_conv16_s2_workspace(int batch, int cin, int cout, int h, int w);
 template <typename T>
 bool offset_conv16_s2_forward(int batch, int cin, int cout, int h, int w, const T* x, const T* weight, const T* bias,
                               T* out, void* ws, hipStream_t stream);
+size_t offset_conv16_s2_backward_input_workspace(int cin, int cout);
+template <typename T>
+bool offset_conv16_s2_backward_input(int batch, int cin, int cout, int h, int w, const T* gout, const T* weight,
+                                     T* gin, void* ws, hipStream_t stream);
 
 // dk_local_nhwc.hip: the local operator on channels-last tensors, all dtypes, any geometry whose tables fit LDS
 bool nhwc_supported(const Geo& g, int dtype);

@@ -188,7 +188,7 @@ __global__ __launch_bounds__(kC16Block, 2) void conv16_kernel(int batch, int kin
 }
 
 
-// ---- stride 2 (forward only) -------------------------------------------------------------------------------
+// ---- stride 2, forward --------------------------------------------------------------------------------------
 // out[m][(oy, ox)] = sum over taps, channels of A_t[m][k] * in[k][(2 oy + dy - 1, 2 ox + dx - 1)].  A tile of 448
 // output pixels needs 2 TH + 1 input rows of the full width, so the chunk is 16 channels (v_mfma_f32_16x16x16):
 // a position's 16 elements in 32 bytes of a 40-byte slot (17 rows of a 112-wide plane: 77 KB, two workgroups per
@@ -316,6 +316,119 @@ __global__ __launch_bounds__(kC16Block, 2) void conv16_s2_kernel(int batch, int 
             partial[(size_t)split * batch * mout * plane + at + q] = acc[i][m][r] + bv;
           else
             st(out + at + q, acc[i][m][r] + bv);
+        }
+      }
+    }
+  }
+}
+
+
+// ---- stride 2, input gradient ---------------------------------------------------------------------------------
+// gin[c][y][x] = sum over outputs o and the taps (th, tw) with y + 1 - th and x + 1 - tw even of
+//                W[o][c][th][tw] * gout[o][(y + 1 - th) / 2][(x + 1 - tw) / 2].
+// The input pixels fall into four parity classes: y = 2 j + py takes th = 1 (gout row j) when py = 0 and
+// th = 0, 2 (rows j + 1, j) when py = 1, and x = 2 i + px likewise -- 1, 2, 2 and 4 taps, nine matrix
+// instructions per 2 x 2 quad of input pixels, each against the gout tile at a fixed offset (dj, di) from the
+// quad's (j, i).  The gout tile (at most 32 channels: one chunk) is staged channel-interleaved as in the stride-1
+// kernel, with a zero row below and a zero column to the right; a lane holds the sums of both px of its quads
+// and writes them as one 4-byte pair.  A workgroup owns 448 quads (whole j rows) of an image and MTB blocks of
+// 16 channels; further blocks go to further workgroups on the same tile.
+// grid = (image, tile of j rows, walk of MTB row blocks)
+template <typename T, int WIN, int MTB>
+__global__ __launch_bounds__(kC16Block, 2) void conv16_s2_bwd_kernel(int batch, int kin, int mout, int h, int ho,
+                                                                     int tiles, int blocks,
+                                                                     const T* __restrict__ gout,
+                                                                     const uint4* __restrict__ wp, T* __restrict__ gin) {
+  constexpr int WO = WIN / 2, TJ = kC16Pix / WO, RS = WO + 1;
+  static_assert(WIN % 2 == 0 && TJ * WO == kC16Pix, "whole rows of quads");
+  extern __shared__ __align__(16) unsigned tile[];  // [rows + 1][RS][kC16Pitch]
+
+  const int walks = (blocks + MTB - 1) / MTB;
+  const int total = batch * tiles * walks;
+  const int lb = logical_block(total);
+  if (lb >= total) return;
+  const int mb0 = (lb % walks) * MTB, n = lb / walks / tiles, j0 = (lb / walks % tiles) * TJ;
+  const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int plane_o = ho * WO;
+
+  const int rows = min(TJ, ho - j0);  // j rows of the tile; gout rows j0 .. j0 + rows are staged (the last may be zero)
+  const int live_groups = (rows * WO + 15) / 16;
+  for (int e = threadIdx.x; e < (rows + 1) * RS * kC16Pitch; e += kC16Block) tile[e] = 0u;
+  __syncthreads();
+  {
+    const rsrc_t rs = plane_rsrc(gout + (size_t)n * kin * plane_o, kin * plane_o);
+    for (int e = threadIdx.x; e < (rows + 1) * 4 * WO; e += kC16Block) {
+      const int col = e % WO, jr = e / WO % (rows + 1), oct = e / WO / (rows + 1);
+      const int row = j0 + jr;
+      unsigned v[8];
+#pragma unroll
+      for (int k = 0; k < 8; ++k) {
+        const unsigned o = row < ho ? (unsigned)((oct * 8 + k) * plane_o + row * WO + col) * 2u : kOutOfRange;
+        v[k] = __builtin_amdgcn_raw_buffer_load_b16(rs, (int)o, 0, 0);
+      }
+      *reinterpret_cast<uint4*>(tile + (jr * RS + col) * kC16Pitch + oct * 4) =
+          make_uint4(v[0] | v[1] << 16, v[2] | v[3] << 16, v[4] | v[5] << 16, v[6] | v[7] << 16);
+    }
+  }
+  __syncthreads();
+
+  int bword[kC16Gpw];
+#pragma unroll
+  for (int i = 0; i < kC16Gpw; ++i) {
+    const int q = min((wave + 4 * i) * 16 + (lane & 15), rows * WO - 1);
+    bword[i] = ((q / WO) * RS + q % WO) * kC16Pitch + (lane >> 4) * 4;
+  }
+
+#pragma unroll
+  for (int py = 0; py < 2; ++py) {
+    c16f4 acc[2][kC16Gpw][MTB];
+#pragma unroll
+    for (int px = 0; px < 2; ++px)
+#pragma unroll
+      for (int i = 0; i < kC16Gpw; ++i)
+#pragma unroll
+        for (int m = 0; m < MTB; ++m) acc[px][i][m] = c16f4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int th = 0; th < 3; ++th) {
+      if ((th == 1) != (py == 0)) continue;  // py = 0: th = 1; py = 1: th = 0, 2
+      const int dj = th == 0 ? 1 : 0;
+#pragma unroll
+      for (int tw = 0; tw < 3; ++tw) {
+        const int px = tw == 1 ? 0 : 1, di = tw == 0 ? 1 : 0;
+        const int shift = (dj * RS + di) * kC16Pitch;
+        uint4 a[MTB];
+#pragma unroll
+        for (int m = 0; m < MTB; ++m)  // the packed copy holds tap 8 - t at index t
+          a[m] = wp[((size_t)(8 - (th * 3 + tw)) * blocks + min(mb0 + m, blocks - 1)) * 64 + lane];
+#pragma unroll
+        for (int i = 0; i < kC16Gpw; ++i) {
+          if constexpr (WO <= 14)
+            if (wave + 4 * i >= live_groups) break;
+          const uint4 b = *reinterpret_cast<const uint4*>(tile + bword[i] + shift);
+#pragma unroll
+          for (int m = 0; m < MTB; ++m) acc[px][i][m] = mma16<T>(a[m], b, acc[px][i][m]);
+        }
+      }
+    }
+    // lane (quad l % 16 of each group, channels 4 (l / 16) .. + 3 of each block): the pair (x = 2 i, 2 i + 1)
+#pragma unroll
+    for (int m = 0; m < MTB; ++m) {
+      if (mb0 + m >= blocks) break;
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const int c = 16 * (mb0 + m) + 4 * (lane >> 4) + r;
+        if (c >= mout) continue;
+        T* plane = gin + ((size_t)n * mout + c) * h * WIN;
+#pragma unroll
+        for (int i = 0; i < kC16Gpw; ++i) {
+          const int q = (wave + 4 * i) * 16 + (lane & 15);
+          const int y = 2 * (j0 + q / WO) + py;
+          if (q < rows * WO && y < h) {
+            T pair[2];
+            st(&pair[0], acc[0][i][m][r]);
+            st(&pair[1], acc[1][i][m][r]);
+            *reinterpret_cast<unsigned*>(plane + (size_t)y * WIN + 2 * (q % WO)) = *reinterpret_cast<const unsigned*>(pair);
+          }
         }
       }
     }
@@ -468,10 +581,47 @@ bool offset_conv16_s2_forward(int batch, int cin, int cout, int h, int w, const 
                      : launch_conv16_s2<T, 2>(batch, cin, cout, h, w, x, wp, bias, out, partial, stream);
 }
 
+
+size_t offset_conv16_s2_backward_input_workspace(int cin, int cout) { return pack_bytes(cout, cin); }
+
+template <typename T>
+bool offset_conv16_s2_backward_input(int batch, int cin, int cout, int h, int w, const T* gout, const T* weight,
+                                     T* gin, void* ws, hipStream_t stream) {
+  if (!offset_conv16_s2_supported(cin, cout, h, w) || cout > kC16Chunk) return false;
+  if (batch == 0) return true;
+  uint4* wp = static_cast<uint4*>(ws);
+  const int ho = (h - 1) / 2 + 1, blocks = ceil_div(cin, 16);
+  conv16_pack_kernel<T><<<ceil_div(9 * blocks * 64, 256), 256, 0, stream>>>(weight, cout, cin, 1, 1, blocks, wp);
+  constexpr int MTB = 2;
+  bool ok = true;
+#define DK_S2B(WW)                                                                                                     \
+  {                                                                                                                    \
+    auto kernel = conv16_s2_bwd_kernel<T, WW, MTB>;                                                                    \
+    constexpr int TJ = kC16Pix / (WW / 2);                                                                             \
+    const int tiles = ceil_div(ho, TJ);                                                                                \
+    const size_t lds = (size_t)(std::min(TJ, ho) + 1) * (WW / 2 + 1) * kC16Pitch * sizeof(unsigned);                   \
+    if (lds > (size_t)kMaxDynamicLds || !allow_max_dynamic_lds(reinterpret_cast<const void*>(kernel)))                 \
+      ok = false;                                                                                                      \
+    else                                                                                                               \
+      kernel<<<(unsigned)xcd_grid_size((long)batch * tiles * ceil_div(blocks, MTB)), kC16Block, lds, stream>>>(        \
+          batch, cout, cin, h, ho, tiles, blocks, gout, wp, gin);                                                      \
+  }
+  switch (w) {
+    case 14: DK_S2B(14) break;
+    case 28: DK_S2B(28) break;
+    case 56: DK_S2B(56) break;
+    case 112: DK_S2B(112) break;
+    default: ok = false;
+  }
+#undef DK_S2B
+  return ok;
+}
+
 #define DK_INST(T)                                                                                                      \
   template bool offset_conv16_forward<T>(int, int, int, int, int, const T*, const T*, const T*, T*, void*, hipStream_t); \
   template bool offset_conv16_backward_input<T>(int, int, int, int, int, const T*, const T*, T*, void*, hipStream_t);  \
-  template bool offset_conv16_s2_forward<T>(int, int, int, int, int, const T*, const T*, const T*, T*, void*, hipStream_t);
+  template bool offset_conv16_s2_forward<T>(int, int, int, int, int, const T*, const T*, const T*, T*, void*, hipStream_t); \
+  template bool offset_conv16_s2_backward_input<T>(int, int, int, int, int, const T*, const T*, T*, void*, hipStream_t);
 DK_INST(__half)
 DK_INST(bf16_t)
 #undef DK_INST

@@ -12,8 +12,8 @@ kernels multiply and add in float32 and round the results once) it runs
   * the bias gradient on the library's reduction kernel for every shape (the framework's
     reduction over (N, H, W) takes 60-230 us on the large planes),
   * for float16 / bfloat16 tensors on planes 7, 14, 28, 56 or 112 wide, the forward and the input gradient on
-    the library's 16-bit matrix-instruction kernel (the elements are the operands as they are); with stride 2
-    (input planes 14, 28, 56 or 112 wide) the forward alone,
+    the library's 16-bit matrix-instruction kernels (the elements are the operands as they are); the same two
+    passes with stride 2 on input planes 14, 28, 56 or 112 wide,
   * everything else -- the input gradient of float32 tensors and of the other planes, and forward /
     weight gradient of the other shapes -- on the framework's convolution routines.
 

@@ -294,9 +294,9 @@ typedef struct dk_offset_conv_desc {
   int32_t batch, in_channels, out_channels, h, w; /* h, w: the input plane (= the output plane at stride 1) */
   int32_t dtype;  /* DK_F32, DK_F16 or DK_BF16 */
   int32_t stride; /* 0 or 1: stride 1.  2: the down-sampling layers' convolution (output ((h - 1) / 2 + 1) x (w / 2));
-                     only the forward of float16 / bfloat16 tensors on input planes 14, 28, 56 or 112 wide has a
-                     kernel: dk_offset_conv_supported() / _worthwhile() then speak for the forward alone, and the
-                     gradient entry points return DK_ERR_UNSUPPORTED (workspace queries 0) */
+                     only the forward and the input gradient of float16 / bfloat16 tensors on input planes 14, 28,
+                     56 or 112 wide have kernels: dk_offset_conv_supported() / _worthwhile() then speak for those
+                     two, and the weight gradient returns DK_ERR_UNSUPPORTED (workspace query 0) */
 } dk_offset_conv_desc;
 int dk_offset_conv_supported(const dk_offset_conv_desc *desc);
 int dk_offset_conv_worthwhile(const dk_offset_conv_desc *desc);

@@ -93,10 +93,11 @@ def test_sixteen_bit_tensors_match_float64_on_the_rounded_inputs(shape, dtype, t
 @pytest.mark.parametrize("dtype,tol", [(torch.float16, 2e-3), (torch.bfloat16, 1e-2)])
 @pytest.mark.parametrize("shape", [(2, 96, 112, 112, 18), (3, 144, 56, 56, 18), (2, 192, 28, 28, 18), (5, 576, 14, 14, 18),
                                    (2, 32, 9, 56, 18), (1, 16, 1, 14, 16), (2, 48, 30, 28, 20), (2, 32, 17, 112, 7)])
-def test_stride_2_forward_of_sixteen_bit_tensors(shape, dtype, tol):
-    """The down-sampling layers' convolution (stride 2, padding 1): the forward of float16 / bfloat16 tensors on
-    the 16-bit matrix instructions (whole, partial and single-row tiles, half chunks of 16 channels, planes lower
-    than a tile, chunk splits), its gradients on the framework's routines, the bias gradient on the library's."""
+def test_stride_2_forward_and_input_gradient_of_sixteen_bit_tensors(shape, dtype, tol):
+    """The down-sampling layers' convolution (stride 2, padding 1): forward and input gradient of float16 /
+    bfloat16 tensors on the 16-bit matrix instructions (whole, partial and single-row tiles, odd heights, half
+    chunks of 16 channels, planes lower than a tile, chunk splits, one to three blocks of 16 channels), the weight
+    gradient on the framework's routine, the bias gradient on the library's."""
     from deformable_kernels.ops.deform_kernel.functions import offset_conv, offset_conv_supported
     N, C, H, W, O = shape
     g = torch.Generator().manual_seed(43)
