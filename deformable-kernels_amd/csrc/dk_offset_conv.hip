@@ -472,10 +472,8 @@ int forward_splits(int batch, int cin, int h, int w) {
 // MI355X, forward + backward): float32, batch 64: on planes 28 wide and wider (56 and 112: by 30-40 %)
 // once the grid -- (image, row tile) items times the input-channel splits -- gives about a
 // workgroup per CU; on the 14- and 7-wide planes the two are within 10 % of each other either way.
-// 16-bit tensors, batch 128: planes 28, 56 and 112 wide have the forward and the input gradient on 16-bit matrix
-// instructions (dk_offset_conv16.hip; forward 61 / 103 / 107 us against the library's 147 / 520 / 387, input
-// gradient 49 / 74 / 118 against 107 / 384 / 322); on the 14-wide planes, where forward and weight gradient
-// multiply in fp32 and the library on 16-bit matrix instructions, the library is ahead (224 against 298 us).
+// (16-bit tensors have forward and input gradient on 16-bit matrix instructions, dk_offset_conv16.hip, and a
+// rule of their own in dk_offset_conv_worthwhile(); these kernels serve them where those do not apply.)
 bool offset_conv_worthwhile(int batch, int cin, int cout, int h, int w) {
   if (!offset_conv_supported(cin, cout, h, w) || w < 28) return false;
   const int th = w <= 56 ? 8 : 4;

@@ -1,10 +1,10 @@
 // The offset branch's 3x3 convolution (reference modules/deform_kernel.py:165-168, applied at :214)
 // on 16-bit tensors: forward and input gradient on the 16-bit matrix instructions
 // (v_mfma_f32_16x16x32_bf16 / _f16: the tensors' elements are the operands as they are, the products
-// exact, the sums fp32, one rounding of the result).  Stride 1, padding 1, no dilation, planes 7, 14, 28, 56
-// or 112 wide.
+// exact, the sums fp32, one rounding of the result).  Padding 1, no dilation; stride 1 on planes 7, 14, 28, 56
+// or 112 wide, stride 2 (kernels of their own, further down) on input planes 14, 28, 56 or 112 wide.
 //
-// Both passes are the same shift-GEMM, out[m][p] = sum over taps t, channels k of A_t[m][k] * in[k][p + shift_t]:
+// At stride 1 both passes are the same shift-GEMM, out[m][p] = sum over taps t, channels k of A_t[m][k] * in[k][p + shift_t]:
 //   forward          in = x (Cin channels),   m = output channel,  A_t[m][k] = W[m][k][t], + bias;
 //   input gradient   in = gout (Cout channels), m = input channel, A_t[m][k] = W[k][m][8 - t]  (the taps flipped).
 // A workgroup of four waves owns 448 pixels (whole rows) of one image and walks the `in` channels in chunks
