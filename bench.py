@@ -198,6 +198,8 @@ def main():
     ap.add_argument("--layout", default="nchw", choices=["nchw", "nhwc"],
                     help="memory layout of the tensors of the local-operator workloads (nhwc: the channels-last kernels)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--framework-offset-branch", action="store_true",
+                    help="mbv2_net: the layers' offset branch on the framework's convolution (the reference's sequence)")
     ap.add_argument("--kernels", default="", help="comma list restricting the per-kernel timing (tuning aid)")
     ap.add_argument("--traffic-from", nargs=2, metavar=("FETCH_DB", "WRITE_DB"),
                     help="summarise two rocprofv3 counter databases into the tracked traffic table and exit")
@@ -737,6 +739,10 @@ def network_workload(a):
     tdtype = getattr(torch, DTYPES[a.dtype])
     torch.manual_seed(0)
     net = MobileNetV2DK().to(dev).to(tdtype)
+    if a.framework_offset_branch:
+        for m in net.modules():
+            if hasattr(m, "native_offset_conv"):
+                m.native_offset_conv = False
     # random labels, nothing to learn, and an untrained network's gradients are large (3e3 on the first offset
     # branch): a step size that leaves the parameters where they are keeps every step's work the same
     opt = torch.optim.SGD(net.parameters(), lr=1e-7, momentum=0.9)
@@ -766,7 +772,8 @@ def network_workload(a):
     print(json.dumps({
         "metric": "MobileNetV2-DK training step, images/s (secondary workload: the whole network)",
         "config": {"workload": "mbv2_net: MobileNetV2 with 17 DeformKernel2d layers (scope 4x4), 224x224, batch %d, %s, "
-                               "forward + loss + backward + SGD step" % (a.batch, a.dtype)},
+                               "forward + loss + backward + SGD step%s" % (
+                                   a.batch, a.dtype, ", offset branch on the framework's convolution" if a.framework_offset_branch else "")},
         "images_per_s": round(a.batch / (ms * 1e-3), 1), "ms_per_step": round(ms, 3), "steps": a.steps,
         "n_gpus": 1, "dtype": a.dtype, "data": "synthetic",
     }))
