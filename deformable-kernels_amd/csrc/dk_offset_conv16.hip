@@ -42,6 +42,16 @@ typedef float c16f4 __attribute__((ext_vector_type(4)));
 typedef __bf16 c16b8 __attribute__((ext_vector_type(8)));
 typedef _Float16 c16h8 __attribute__((ext_vector_type(8)));
 
+// v rounded to T, as the 16 bits of the element
+template <typename T>
+__device__ __forceinline__ unsigned bits16(float v) {
+  T t;
+  st(&t, v);
+  unsigned short b;
+  __builtin_memcpy(&b, &t, sizeof(b));
+  return b;
+}
+
 template <typename T>
 __device__ __forceinline__ c16f4 mma16(const uint4& a, const uint4& b, c16f4 acc) {
   if constexpr (std::is_same<T, bf16_t>::value)
@@ -424,10 +434,8 @@ __global__ __launch_bounds__(kC16Block, 2) void conv16_s2_bwd_kernel(int batch, 
           const int q = (wave + 4 * i) * 16 + (lane & 15);
           const int y = 2 * (j0 + q / WO) + py;
           if (q < rows * WO && y < h) {
-            T pair[2];
-            st(&pair[0], acc[0][i][m][r]);
-            st(&pair[1], acc[1][i][m][r]);
-            *reinterpret_cast<unsigned*>(plane + (size_t)y * WIN + 2 * (q % WO)) = *reinterpret_cast<const unsigned*>(pair);
+            const unsigned pair = bits16<T>(acc[0][i][m][r]) | bits16<T>(acc[1][i][m][r]) << 16;
+            *reinterpret_cast<unsigned*>(plane + (size_t)y * WIN + 2 * (q % WO)) = pair;  // (x even, rows of even length)
           }
         }
       }
