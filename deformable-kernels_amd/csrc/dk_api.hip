@@ -30,7 +30,8 @@ unsigned switches_from_environment() {
       {"DK_NO_ND_BINS", kNoNdBins}, {"DK_NO_ND_MFMA", kNoNdMfma}, {"DK_NO_GATHER_MFMA", kNoGatherMfma},
       {"DK_NO_FILTER_SPLIT", kNoFilterSplit}, {"DK_NO_IMAGE_FLAT", kNoImageFlat},
       {"DK_NO_ND_SMALL", kNoNdSmall}, {"DK_NO_NHWC_MFMA", kNoNhwcMfma},
-      {"DK_FORCE_GATHER_MFMA", kForceGatherMfma}};
+      {"DK_FORCE_GATHER_MFMA", kForceGatherMfma}, {"DK_NO_PIXEL_LANES", kNoPixelLanes},
+      {"DK_FORCE_PIXEL_LANES", kForcePixelLanes}};
   unsigned m = 0;
   for (const auto& v : vars)
     if (std::getenv(v.name)) m |= v.bit;

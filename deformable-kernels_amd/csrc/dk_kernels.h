@@ -32,6 +32,8 @@ enum TestSwitch : unsigned {
   kNoNhwcMfma = 1u << 14,   // DK_NO_NHWC_MFMA    the matrix-core grad filter / grad rotation of the channels-last operator
   kForceGatherMfma = 1u << 15,  // DK_FORCE_GATHER_MFMA  the matrix-core forward / grad input wherever it applies, not only where it is the faster kernel
   kNoImageFlat = 1u << 12,  // DK_NO_IMAGE_FLAT   the flat-copy kernels of the per-image depthwise convolution (the band kernels run instead)
+  kNoPixelLanes = 1u << 16,     // DK_NO_PIXEL_LANES     the forward / grad input with the pixels on the matrix instruction's lanes
+  kForcePixelLanes = 1u << 17,  // DK_FORCE_PIXEL_LANES  ... wherever it applies, not only where it is the faster kernel
 };
 unsigned test_switches();  // dk_api.hip
 inline bool path_disabled(unsigned sw) { return (test_switches() & sw) != 0; }
@@ -56,6 +58,12 @@ void launch_reduce_partials(const CT* partial, int parts, long count, T* out, hi
 template <typename T>
 bool mfma_local_gather(const Geo& g, bool transposed, const T* src, const T* rot, const T* filter, T* dst,
                        hipStream_t stream);
+
+// ---- forward / grad input with the pixels on the lanes of the matrix instruction (dk_local_lanes.hip): same-width
+//      geometries, scope <= 16 cells; no LDS staging of the source tensor
+template <typename T>
+bool lanes_local_gather(const Geo& g, bool transposed, const T* src, const T* rot, const T* filter, T* dst,
+                        hipStream_t stream);
 
 // ---- tuned local path (dk_local_fast.hip): 3x3 taps, scope 3x3 / 4x4 / 5x5, fp32/fp16/bf16
 template <typename T>

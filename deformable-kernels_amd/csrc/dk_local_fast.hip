@@ -1730,6 +1730,7 @@ template <typename T>
 bool fast_local_gather(const Geo& g, bool transposed, const T* src, const T* rot, const T* filter,
                        T* dst, hipStream_t stream) {
   if (!fast_shape(g)) return false;
+  if (lanes_local_gather<T>(g, transposed, src, rot, filter, dst, stream)) return true;
   if (mfma_local_gather<T>(g, transposed, src, rot, filter, dst, stream)) return true;
 #define CALL(SH, SW) run_gather<T, SH, SW>(g, transposed, src, rot, filter, dst, stream)
   DK_DISPATCH_SCOPE(g, CALL)
