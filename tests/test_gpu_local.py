@@ -112,6 +112,28 @@ def test_matrix_core_forward_and_grad_input_on_16_bit_tensors(case, dtype, tol, 
     assert rel_err(got[1].float(), want[1]) < tol, "grad input"
 
 
+SAME_WIDTH = [c for c in TUNED if c[6] == 1 and c[7] == 1 and c[8] == 1 and c[5] in ((4, 4), (3, 3))] + [
+    (2, 144, 56, 56, 3, (4, 4), 1, 1, 1, 1, 1.0),  # the headline layer's geometry: three whole rounds of tiles per wave and a shared remainder
+    (1, 272, 12, 12, 3, (3, 3), 1, 1, 1, 1, 1.0),  # 8.5 blocks of 32 channels; waves that change tile after a single block
+    (2, 70, 9, 31, 3, (4, 4), 1, (2, 1), (2, 1), 2, 1.0),  # dilated rows (pad_h = dil_h = 2), 35 channels per group, a tile spans a row's end
+]
+
+
+@pytest.mark.parametrize("dtype,tol", [(torch.float32, 1e-5), (torch.float16, 1e-3), (torch.bfloat16, 5e-3)])
+@pytest.mark.parametrize("case", SAME_WIDTH)
+def test_forward_and_grad_input_with_the_pixels_on_the_matrix_lanes(case, dtype, tol, switch_off):
+    """dk_local_lanes.hip: channels on the rows of the 32 x 32 matrix instruction, pixels on its columns, source
+    rows loaded straight into the registers the multiply-adds read, with hand-counted waits.  The dispatch takes
+    it on large planes with many channels (the full-size configuration 2 test runs it there); forced, it must
+    serve every same-width shape: partial tiles, channel blocks that end beyond the group's last channel, several
+    groups, tiles that wrap around a row's end, one block per tile."""
+    switch_off("DK_FORCE_PIXEL_LANES")
+    inputs, got = _run(case, dtype, seed=5)
+    want = _oracle(inputs, np.float32)  # 16-bit inputs are already rounded to the type
+    assert rel_err(got[0].float(), want[0]) < tol, "forward"
+    assert rel_err(got[1].float(), want[1]) < tol, "grad input"
+
+
 @pytest.mark.parametrize("case", [
     (2, 37, 28, 28, 3, (4, 4), 1, 1, 1, 1, 1.0),   # odd channel count: the last pair's second channel is a dummy
     (1, 74, 12, 18, 3, (5, 5), 1, 1, 1, 2, 1.5),   # 37 channels per group, two groups, scope 5
@@ -268,7 +290,7 @@ def test_headline_shape_properties_at_full_size():
         assert abs(a - b) < 1e-6 * max(abs(a), 1.0)
 
 
-@pytest.mark.parametrize("switch", ["DK_NO_MFMA", "DK_NO_ROWS", "DK_NO_GATHER_MFMA", "DK_NO_FILTER_SPLIT"])
+@pytest.mark.parametrize("switch", ["DK_NO_MFMA", "DK_NO_ROWS", "DK_NO_GATHER_MFMA", "DK_NO_FILTER_SPLIT", "DK_NO_PIXEL_LANES"])
 def test_more_general_kernels_on_a_same_width_shape(switch, switch_off):
     """The dispatch prefers the most specialised kernel; the library's test switches make it take
     the next more general family for the same shape (dense grad filter instead of the
