@@ -32,6 +32,9 @@ unsigned switches_from_environment() {
       {"DK_NO_ND_SMALL", kNoNdSmall}, {"DK_NO_NHWC_MFMA", kNoNhwcMfma},
       {"DK_FORCE_GATHER_MFMA", kForceGatherMfma}, {"DK_NO_PIXEL_LANES", kNoPixelLanes},
       {"DK_FORCE_PIXEL_LANES", kForcePixelLanes}};
+  // a production process ignores these variables: they count only next to DK_ENABLE_TEST_SWITCHES=1
+  const char* on = std::getenv("DK_ENABLE_TEST_SWITCHES");
+  if (!on || on[0] != '1') return 0;
   unsigned m = 0;
   for (const auto& v : vars)
     if (std::getenv(v.name)) m |= v.bit;
@@ -202,7 +205,11 @@ int static_scratch_of_current_device(void** ptr) {
 
 extern "C" {
 
-int dk_version(void) { return (0 << 16) | 2; }
+int dk_version(void) { return (0 << 16) | 3; }
+
+size_t dk_conv_desc_size(void) { return sizeof(dk_conv_desc); }
+size_t dk_nd_desc_size(void) { return sizeof(dk_nd_desc); }
+size_t dk_offset_conv_desc_size(void) { return sizeof(dk_offset_conv_desc); }
 
 unsigned dk_test_switches(unsigned mask) {
   const unsigned before = test_switches();
@@ -232,6 +239,13 @@ int dk_conv_out_size(const dk_conv_desc* desc, int32_t* out_h, int32_t* out_w) {
   if (out_h) *out_h = g.out_h;
   if (out_w) *out_w = g.out_w;
   return DK_OK;
+}
+
+int dk_sample_depthwise_layout_supported(const dk_conv_desc* desc) {
+  Geo g;
+  const int rc = make_geo(desc, g);
+  if (rc != DK_OK) return rc;
+  return desc->layout == DK_LAYOUT_NHWC ? (nhwc_supported(g, desc->dtype) ? 1 : 0) : 1;
 }
 
 // ---- local ------------------------------------------------------------------------------

@@ -472,7 +472,9 @@ __global__ __launch_bounds__(1024) void nd_small_grad_data_kernel(NdGeo g, const
       for (int k = 0; k < 8; ++k) {
         if (s0 + 4 * k < share) {  // uniform over the wave
           const int row = r0 + s0 + 4 * k + (lane >> 4);
-          const float a = ld(&raw[k]);  // rows past the chunk's points multiply a zero row of W
+          // rows past the chunk's points re-read the last point's out_grad: they are zeroed by a select, not by
+          // their zero row of W (0 * Inf would put a NaN into every cell of the channel)
+          const float a = row < npts ? ld(&raw[k]) : 0.f;
 #pragma unroll
           for (int t = 0; t < NT; ++t)
             acc[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(a, W[row * ROW + t * 16 + (lane & 15)], acc[t], 0, 0, 0);

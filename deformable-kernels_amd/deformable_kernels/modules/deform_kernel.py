@@ -144,7 +144,10 @@ class GlobalDeformKernel2d(nn.Module):
         if self._fusable(x):
             return self._forward_fused(x)
         n, c, h, w = x.shape
-        if self.native_conv and x.is_cuda and self.group == self.in_planes == self.out_planes:
+        # (inside an autocast region the framework's convolution runs, and returns, the autocast dtype; the
+        # library's convolution computes in the tensors' own type, so it is only taken outside such regions)
+        if (self.native_conv and x.is_cuda and self.group == self.in_planes == self.out_planes
+                and not torch.is_autocast_enabled()):
             kernels = self.dynamic_weight(x, self.weight, per_image=True).to(x.dtype)
             if image_depthwise_conv_supported(x, kernels, self.stride, self.padding, self.dilation):
                 return image_depthwise_conv(x, kernels, self.stride, self.padding, self.dilation)

@@ -49,9 +49,13 @@ _CD, _ND, _OC = ctypes.POINTER(ConvDesc), ctypes.POINTER(NdDesc), ctypes.POINTER
 # name -> (restype, argtypes); must list every symbol include/dk_hip.h declares
 SIGNATURES = {
     "dk_version": (ctypes.c_int, []),
+    "dk_conv_desc_size": (_SZ, []),
+    "dk_nd_desc_size": (_SZ, []),
+    "dk_offset_conv_desc_size": (_SZ, []),
     "dk_test_switches": (ctypes.c_uint, [ctypes.c_uint]),
     "dk_status_string": (ctypes.c_char_p, [ctypes.c_int]),
     "dk_conv_out_size": (ctypes.c_int, [_CD, ctypes.POINTER(ctypes.c_int32), ctypes.POINTER(ctypes.c_int32)]),
+    "dk_sample_depthwise_layout_supported": (ctypes.c_int, [_CD]),
     "dk_sample_depthwise_forward": (ctypes.c_int, [_CD, _P, _P, _P, _P, _P]),
     "dk_sample_depthwise_backward_data": (ctypes.c_int, [_CD, _P, _P, _P, _P, _P]),
     "dk_sample_depthwise_backward_filter_workspace": (_SZ, [_CD]),
@@ -112,6 +116,14 @@ def lib():
         for name, (res, args) in SIGNATURES.items():
             fn = getattr(handle, name)
             fn.restype, fn.argtypes = res, args
+        # the descriptors are declared twice, here and in include/dk_hip.h: a struct shorter than the
+        # library's would be read past its end
+        for struct, size_of in ((ConvDesc, handle.dk_conv_desc_size), (NdDesc, handle.dk_nd_desc_size),
+                                (OffsetConvDesc, handle.dk_offset_conv_desc_size)):
+            if ctypes.sizeof(struct) != size_of():
+                raise DkError("%s is %d bytes here and %d in %s (library version %#x): the binding and the "
+                              "library are out of step" % (struct.__name__, ctypes.sizeof(struct), size_of(),
+                                                           LIB_PATH, handle.dk_version()))
         _lib = handle
     return _lib
 

@@ -88,7 +88,14 @@ class SampleDepthwiseFunction(Function):
         # A channels-last input runs the library's channels-last kernels and gets a channels-last
         # output (and gradients): no layout change around the operator.  The reference's kernels
         # take planar tensors only.
-        nhwc = _lib.channels_last(input)
+        # Geometries whose channels-last tables do not fit LDS (e.g. 64 rotation groups) take the planar
+        # kernels on a planar copy, and the output goes back to channels-last.
+        wants_nhwc = _lib.channels_last(input)
+        nhwc = wants_nhwc
+        if nhwc:
+            probe = _lib.conv_desc(input, weight, kernel_size, stride, padding, dilation, rotation_groups,
+                                   rotation_clip, _lib.LAYOUT_NHWC)
+            nhwc = _lib.lib().dk_sample_depthwise_layout_supported(probe) == 1
         fmt = torch.channels_last if nhwc else torch.contiguous_format
         ctx.layout = _lib.LAYOUT_NHWC if nhwc else _lib.LAYOUT_NCHW
         input, rotation = input.contiguous(memory_format=fmt), rotation.contiguous(memory_format=fmt)
@@ -101,6 +108,8 @@ class SampleDepthwiseFunction(Function):
             _lib.check(_lib.lib().dk_sample_depthwise_forward(
                 desc, _lib.ptr(input), _lib.ptr(rotation), _lib.ptr(weight), _lib.ptr(output),
                 _lib.stream_ptr(input)), "sample_depthwise forward")
+        if wants_nhwc and not nhwc:
+            output = output.contiguous(memory_format=torch.channels_last)
         return output
 
     @staticmethod

@@ -104,6 +104,13 @@ typedef struct dk_conv_desc {
 /* Output extent for the descriptor, or a negative dk_status. */
 int dk_conv_out_size(const dk_conv_desc *desc, int32_t *out_h, int32_t *out_w);
 
+/* 1 if the local operator's entry points (dk_sample_depthwise_*) serve the descriptor's `layout`, 0 if
+ * they would return DK_ERR_UNSUPPORTED (a channels-last geometry whose tables do not fit LDS: e.g. 64
+ * rotation groups with 3 x 3 taps and a 4 x 4 scope), a negative dk_status for an invalid descriptor.
+ * DK_LAYOUT_NCHW is always served.  A caller with channels-last tensors asks first and converts to NCHW
+ * when the answer is 0.  No counterpart in the reference, whose kernels take planar tensors only. */
+int dk_sample_depthwise_layout_supported(const dk_conv_desc *desc);
+
 /* ---- local deformable kernel: kernel-space offsets only ------------------- */
 
 /* sample_depthwise_forward_cuda (filter_sample_depthwise_cuda.cpp:8-62). */
@@ -125,15 +132,20 @@ int dk_sample_depthwise_backward_filter(const dk_conv_desc *desc, const void *ou
                                         size_t workspace_bytes, void *stream);
 
 /* The same filter gradient for callers that cannot allocate device memory or hand over a
- * workspace: code under HIP graph capture, tight serving loops, harnesses that forbid
- * hipMalloc.  No counterpart in the reference.  The per-workgroup partial sums go to a buffer of
+ * workspace: tight serving loops, harnesses that forbid hipMalloc, code that is later captured
+ * into a HIP graph.  No counterpart in the reference.  The per-workgroup partial sums go to a buffer of
  * DK_STATIC_SCRATCH_BYTES that is part of the library's device image (every GPU the library runs
  * on holds it until the process ends); the call allocates nothing and runs the same kernels as
  * dk_sample_depthwise_backward_filter, so the result is bit-identical to that function's.
  * Returns DK_ERR_SCRATCH_LIMIT, launching nothing, when
  * dk_sample_depthwise_backward_filter_workspace(desc) exceeds DK_STATIC_SCRATCH_BYTES.
  * All calls on one GPU share the one buffer: calls that may overlap on a GPU (different streams,
- * different host threads) race on it and must be ordered by the caller. */
+ * different host threads) race on it and must be ordered by the caller.
+ * The first call for a (device, descriptor shape) pair looks the buffer's address up and sets a
+ * kernel attribute -- host-side runtime calls that a stream in capture mode may refuse (the call
+ * then returns DK_ERR_LAUNCH).  A caller that captures the call into a HIP graph therefore makes
+ * one ordinary (warm-up) call with the same descriptor on that device first; every later call is
+ * kernel launches only. */
 #define DK_STATIC_SCRATCH_BYTES (8u << 20)
 int dk_sample_depthwise_backward_filter_static(const dk_conv_desc *desc, const void *out_grad,
                                                const void *input, const void *rotation,
@@ -365,14 +377,27 @@ const char *dk_status_string(int status);
  * family and run the next more general one for the same shape, so that tests can reach every
  * kernel.  Bit i belongs to the i-th of DK_NO_ROWS, DK_NO_MFMA, DK_NO_MFMA_S2, DK_NO_S2_QUADS,
  * DK_NO_DEFORM_FAST, DK_NO_DEFORM_CH, DK_NO_DEFORM_CH_BIG, DK_NO_DEFORM_MFMA, DK_NO_ND_BINS,
- * DK_NO_ND_MFMA, DK_NO_GATHER_MFMA, DK_NO_FILTER_SPLIT, DK_NO_IMAGE_FLAT, DK_NO_ND_SMALL, DK_NO_NHWC_MFMA, DK_FORCE_GATHER_MFMA.  The mask starts from the environment variables of those names, read once
- * (at the first call that consults it); this call replaces it and returns the previous mask.
+ * DK_NO_ND_MFMA, DK_NO_GATHER_MFMA, DK_NO_FILTER_SPLIT, DK_NO_IMAGE_FLAT, DK_NO_ND_SMALL, DK_NO_NHWC_MFMA,
+ * DK_FORCE_GATHER_MFMA, DK_NO_PIXEL_LANES, DK_FORCE_PIXEL_LANES.  The mask starts at 0; only a process
+ * started with DK_ENABLE_TEST_SWITCHES=1 in its environment also reads the environment variables of
+ * those names, once, at the first call that consults the mask (a stray variable in a production
+ * environment changes nothing).  This call replaces the mask and returns the previous one.
  * Workspace queries consult it too: query and call must see the same mask.  The one piece of
  * process-wide state in the library. */
 unsigned dk_test_switches(unsigned mask);
 
-/* Library version, (major << 16) | minor. */
+/* Library version, (major << 16) | minor.  The minor number goes up whenever a descriptor struct
+ * changes (0.3: dk_conv_desc has `layout`, the *_desc_size() queries exist). */
 int dk_version(void);
+
+/* sizeof() of the descriptor structs as the library was compiled.  A binding that declares the
+ * structs on its own (ctypes, cgo, JNI) compares these with its own declaration once, at load time:
+ * a descriptor that is shorter than the library's is read past its end.  No counterpart in the
+ * reference, whose pybind functions take the eleven ints one by one
+ * (csrc/filter_sample_depthwise_cuda.cpp:540-569). */
+size_t dk_conv_desc_size(void);
+size_t dk_nd_desc_size(void);
+size_t dk_offset_conv_desc_size(void);
 
 #ifdef __cplusplus
 }

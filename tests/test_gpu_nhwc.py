@@ -138,3 +138,36 @@ def test_c_abi_layout_field():
     assert L.dk_image_depthwise_supported(d) == 0
     assert L.dk_sample_depthwise_backward_filter_workspace(d) > 0
     assert L.dk_sample_depthwise_backward_rotation_workspace(d) == 0
+
+
+def test_channels_last_input_of_a_geometry_the_channels_last_kernels_do_not_cover():
+    """64 rotation groups with 3 x 3 taps and a 4 x 4 scope need 41472 bytes of tap tables, more than the
+    channels-last kernels have (dk_sample_depthwise_layout_supported says 0, the C entry point DK_ERR_UNSUPPORTED).
+    The Function then runs the planar kernels on a planar copy and hands the result back channels-last:
+    same values as the planar call."""
+    from deformable_kernels.ops.deform_kernel import _lib
+    from deformable_kernels.ops.deform_kernel.functions import sample_depthwise
+    case = (2, 64, 9, 10, 3, (4, 4), 1, 1, 1, 64, 1.0)
+    N, C, H, W, k, S, s, p, d, G, rs = case
+    x, wt, rot, gout, cfg = make_local(N, C, H, W, k, S, s, p, d, G, rs, seed=13)
+    cl = torch.channels_last
+    xg = x.to(DEV).contiguous(memory_format=cl)
+    desc = _lib.conv_desc(xg, wt.to(DEV), cfg["kernel_size"], cfg["stride"], cfg["padding"], cfg["dilation"], G,
+                          None, _lib.LAYOUT_NHWC)
+    assert _lib.lib().dk_sample_depthwise_layout_supported(desc) == 0
+    desc.layout = _lib.LAYOUT_NCHW
+    assert _lib.lib().dk_sample_depthwise_layout_supported(desc) == 1
+    res = []
+    for fmt in (torch.contiguous_format, cl):
+        xg = x.to(DEV).contiguous(memory_format=fmt).requires_grad_()
+        rg = rot.to(DEV).contiguous(memory_format=fmt).requires_grad_()
+        wg = wt.to(DEV).requires_grad_()
+        out = sample_depthwise(xg, rg, wg, cfg["kernel_size"], cfg["stride"], cfg["padding"], cfg["dilation"], G)
+        if fmt is cl:
+            assert out.is_contiguous(memory_format=cl)
+        out.backward(gout.to(DEV).contiguous(memory_format=fmt))
+        res.append([t.detach().cpu().contiguous() for t in (out, xg.grad, rg.grad, wg.grad)])
+    for a, b in zip(res[1], res[0]):
+        assert torch.equal(a, b)  # the same kernels ran on the same values
+    o64 = _oracle((x, wt, rot, gout, cfg), np.float64)
+    assert rel_err(res[1][0], o64[0]) < 1e-5 and rel_err(res[1][3], o64[3]) < 1e-4

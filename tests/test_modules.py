@@ -75,6 +75,32 @@ def test_hooks_on_the_offset_branch_convolution_fire():
         assert seen == [(1, 18, 6, 6)]
 
 
+def test_descriptor_structs_have_the_library_s_size():
+    """The descriptor structs are declared three times: in include/dk_hip.h (what the library is compiled
+    from), in the ctypes loader, and in the binding INTEGRATION.md shows a maintainer of the reference.  The
+    library reports its sizeof() for each; the loader's and the documented declaration must agree with it
+    (a struct that is shorter than the library's is read past its end)."""
+    import ctypes
+    import os
+    import re
+    from deformable_kernels.ops.deform_kernel import _lib
+    L = _lib.lib()  # the loader itself compares the three sizes and raises on a mismatch
+    assert L.dk_version() >= 3  # 0.3: dk_conv_desc has `layout`, the size queries exist
+    assert ctypes.sizeof(_lib.ConvDesc) == L.dk_conv_desc_size() == 19 * 4 + 4
+    assert ctypes.sizeof(_lib.NdDesc) == L.dk_nd_desc_size()
+    assert ctypes.sizeof(_lib.OffsetConvDesc) == L.dk_offset_conv_desc_size()
+    # the struct as INTEGRATION.md declares it: take the class statement out of the document and build it
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    doc = open(os.path.join(root, "INTEGRATION.md")).read()
+    m = re.search(r"^class ConvDesc\(ctypes\.Structure\):.*?\n(?=\nlib = )", doc, re.S | re.M)
+    assert m, "INTEGRATION.md no longer shows the ConvDesc declaration"
+    scope = {"ctypes": ctypes}
+    exec(m.group(0), scope)
+    documented = scope["ConvDesc"]
+    assert ctypes.sizeof(documented) == L.dk_conv_desc_size()
+    assert [f[0] for f in documented._fields_] == [f[0] for f in _lib.ConvDesc._fields_]
+
+
 def test_c_abi_exports_every_declared_symbol():
     import ctypes
     import os
@@ -225,6 +251,27 @@ def test_global_module_equals_local_operator_with_constant_rotation():
     out2.sum().backward()
     for got, ref in zip((m.weight.grad, m.fc.weight.grad, m.fc.bias.grad), g_ref):
         assert rel_err(got.cpu(), ref.cpu()) < 1e-4
+
+
+@pytest.mark.gpu
+def test_global_module_under_autocast_returns_what_the_framework_convolution_returns():
+    """Inside an autocast region the reference's F.conv2d (modules/deform_kernel.py:103-111) returns the autocast
+    dtype.  The library's per-image convolution computes in the tensors' own type, so the module only takes it
+    outside such regions: with and without `native_conv` the output dtype is the same."""
+    from deformable_kernels.modules import GlobalDeformKernel2d
+    dev = torch.device("cuda:0")
+    torch.manual_seed(3)
+    m = GlobalDeformKernel2d((5, 5), 16, 16, kernel_size=3, padding=1, groups=16).to(dev)
+    x = torch.randn(2, 16, 12, 12, device=dev)
+    outs = []
+    for native in (True, False):
+        m.native_conv = native
+        with torch.autocast(device_type="cuda", dtype=torch.float16):
+            outs.append(m(x))
+    assert outs[0].dtype == outs[1].dtype == torch.float16
+    assert rel_err(outs[0].float().cpu(), outs[1].float().cpu()) < 1e-6
+    m.native_conv = True
+    assert m(x).dtype == torch.float32  # outside the region: the library's convolution, in the tensors' type
 
 
 @pytest.mark.gpu

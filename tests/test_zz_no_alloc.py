@@ -72,3 +72,40 @@ def test_static_scratch_entry_point_refuses_what_does_not_fit():
     torch.cuda.synchronize()
     assert rc == -8 and b"static" in L.dk_status_string(rc)
     assert bool((gw == 7.0).all())  # nothing was launched
+
+
+def test_static_scratch_entry_point_in_a_graph_after_a_warm_up_call():
+    """The first call for a (device, shape) looks the buffer's address up and sets a kernel attribute, which a
+    capturing stream may refuse; after one ordinary call the entry point is launches only and can be captured.
+    The graph is replayed three times with eager work of the library in between (another shape through the same
+    buffer), and every replay must give the workspace entry point's bits."""
+    from deformable_kernels.ops.deform_kernel import _lib
+    L, P = _lib.lib(), _lib.ptr
+    dev = torch.device("cuda:0")
+    N, C, H, W, S, stride, dtype = CASES[1]
+    x, wt, rot, gout, cfg = make_local(N, C, H, W, 3, S, stride, 1, 1, 1, 1.0, seed=77, dtype=dtype)
+    xg, wg, rg, gg = [t.to(dev) for t in (x, wt, rot, gout)]
+    desc = _lib.conv_desc(xg, wg, cfg["kernel_size"], cfg["stride"], cfg["padding"], cfg["dilation"], 1)
+    need = L.dk_sample_depthwise_backward_filter_workspace(desc)
+    ws, nbytes = _lib.workspace(need, dev)
+    want = torch.empty_like(wg)
+    s0 = torch.cuda.current_stream().cuda_stream
+    _lib.check(L.dk_sample_depthwise_backward_filter(desc, P(gg), P(xg), P(rg), P(want), P(ws), nbytes, s0), "filter")
+    got = torch.zeros_like(wg)
+    _lib.check(L.dk_sample_depthwise_backward_filter_static(desc, P(gg), P(xg), P(rg), P(got), s0), "warm-up")
+    torch.cuda.synchronize()
+    assert torch.equal(got, want)
+    side = torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(graph, stream=side):
+            rc = L.dk_sample_depthwise_backward_filter_static(desc, P(gg), P(xg), P(rg), P(got), side.cuda_stream)
+    assert rc == 0
+    for i in range(3):
+        got.fill_(float("nan"))
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(got, want), "replay %d" % i
+        other, other_want, _ = _both(L, _lib, CASES[2], seed=500 + i)  # eager use of the same buffer in between
+        assert torch.equal(other, other_want)
