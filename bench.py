@@ -64,8 +64,11 @@ OTHER_WORKLOADS = {
 # scaled by what it reads for plain elementwise kernels of known size in the same run (the
 # calibration multiply below and the 1 GiB streaming passes).
 TRAFFIC_RULES = {  # entry point -> regular expressions; a dispatch belongs to the first entry it matches
-    "forward": [r"dk::.*local_gather\w*_kernel<[^>]*\bfalse\b", r"dk::.*local_forward"],
-    "grad_input": [r"dk::.*local_gather\w*_kernel<[^>]*\btrue\b", r"dk::.*local_grad_input"],
+    # (the pixel-lanes kernel's fourth template argument says whether it runs the transposed geometry)
+    "forward": [r"dk::.*local_pixel_lanes_kernel<[^,]*, \d+, \d+, false", r"dk::.*local_gather\w*_kernel<[^>]*\bfalse\b",
+                r"dk::.*local_forward"],
+    "grad_input": [r"dk::.*local_pixel_lanes_kernel<[^,]*, \d+, \d+, true", r"dk::.*local_gather\w*_kernel<[^>]*\btrue\b",
+                   r"dk::.*local_grad_input"],
     "grad_rotation": [r"dk::.*local_grad_rotation"],
     "grad_filter": [r"dk::.*local_grad_filter", r"dk::.*reduce_partials"],
 }
@@ -198,6 +201,8 @@ def main():
     ap.add_argument("--layout", default="nchw", choices=["nchw", "nhwc"],
                     help="memory layout of the tensors of the local-operator workloads (nhwc: the channels-last kernels)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-network-pass", action="store_true",
+                    help="skip the MobileNetV2-DK operator pass (the mbv2_dk_* keys of the default run)")
     ap.add_argument("--framework-offset-branch", action="store_true",
                     help="mbv2_net: the layers' offset branch on the framework's convolution (the reference's sequence)")
     ap.add_argument("--kernels", default="", help="comma list restricting the per-kernel timing (tuning aid)")
@@ -384,6 +389,26 @@ def main():
     }
     if traffic_stale:
         result["roofline"]["traffic_stale"] = True  # kernel sources changed since the counters were read
+    # what the arithmetic type means on this path: the tensors and all sums are `dtype`; where a kernel multiplies on
+    # the matrix cores, float32 operands go in as pairs of 16-bit numbers (the measured errors are pinned in tests/)
+    if a.dtype == "fp32" and a.layout == "nchw":
+        result["arithmetic"] = {
+            "tensors_and_sums": "f32",
+            "forward, grad_input": "weights formed on v_mfma_f32_32x32x16_f16 from fp16 (hi, lo) pairs of both operands, "
+                                   "three products, f32 sums: 2e-7 of the result's scale; the 9 multiply-adds per output in f32",
+            "grad_filter": "v_mfma_f32_16x16x16_bf16 on bfloat16 (hi, lo) pairs of both operands, three products, f32 sums: "
+                           "5e-6 of the largest element (f32 matrix instructions: 2.4e-7)",
+            "grad_rotation": "f32 vector arithmetic throughout",
+        }
+    # BASELINE's second metric: images/s of the MobileNetV2-DK operator pass (its 17 depthwise DeformKernel2d
+    # layers, forward + backward, batch 64, operator calls only) in the same run and dtype
+    if a.workload == "cfg2" and a.layout == "nchw" and not a.kernels and not a.no_network_pass:
+        del xg, rg, gg, out, gin, grot, ws
+        torch.cuda.empty_cache()
+        _, net_us, net_bytes = mobilenet_layers(64, a.dtype, 10)
+        result["mbv2_dk_ms"] = round(net_us / 1e3, 3)
+        result["mbv2_dk_images_per_s"] = round(64 / (net_us * 1e-6), 1)
+        result["mbv2_dk_GBps"] = round(net_bytes / net_us / 1e3, 1)
 
     if not a.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(N, C, H, W, k, S, stride, pad, dil, groups, rot_std, esz)
@@ -681,21 +706,20 @@ def layer_workload(a):
                       "variants": res, "n_gpus": 1, "dtype": a.dtype, "data": "synthetic"}))
 
 
-def mobilenet_workload(a):
-    """Forward + backward of the 17 deformable-kernel depthwise layers of MobileNetV2-DK, operator
-    calls only (one JSON line; secondary to the headline)."""
+def mobilenet_layers(batch, dtype_name, reps):
+    """Forward + backward of the 17 deformable-kernel depthwise layers of MobileNetV2-DK, operator calls
+    only, each distinct layer shape timed `reps` times: (per-layer rows, microseconds per batch, algorithmic bytes)."""
     import collections
     import torch
     from _cases import make_local
     from deformable_kernels.ops.deform_kernel import _lib
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
-    tdtype = getattr(torch, DTYPES[a.dtype])
+    tdtype = getattr(torch, DTYPES[dtype_name])
     L, P = _lib.lib(), _lib.ptr
-    reps = max(a.steps // 10, 10)
     per_layer, total_us, total_bytes = [], 0.0, 0
     for (C, H, stride), count in collections.Counter(MBV2_DW_LAYERS).items():
-        x, wt, rot, gout, cfg = make_local(a.batch, C, H, H, 3, (4, 4), stride, 1, 1, 1, 0.5, seed=0, dtype=tdtype)
+        x, wt, rot, gout, cfg = make_local(batch, C, H, H, 3, (4, 4), stride, 1, 1, 1, 0.5, seed=0, dtype=tdtype)
         xg, wg, rg, gg = [t.to(dev) for t in (x, wt, rot, gout)]
         out, gin, grot, gw = [torch.empty_like(t) for t in (gg, xg, rg, wg)]
         desc = _lib.conv_desc(xg, wg, cfg["kernel_size"], cfg["stride"], cfg["padding"], cfg["dilation"], 1)
@@ -708,12 +732,18 @@ def mobilenet_workload(a):
                                                       P(ws), nb, st), "backward")
         us = _time_us(step, reps)
         e = xg.element_size()
-        _, fwd_b, bwd_b = algorithmic_bytes(a.batch, C, H, H, gg.shape[2], gg.shape[3], 3, (4, 4), 1, e)
+        _, fwd_b, bwd_b = algorithmic_bytes(batch, C, H, H, gg.shape[2], gg.shape[3], 3, (4, 4), 1, e)
         per_layer.append({"C": C, "HW": H, "stride": stride, "count": count, "us": round(us, 1),
                           "GBps": round((fwd_b + bwd_b) / us / 1e3, 1)})
         total_us += us * count
         total_bytes += (fwd_b + bwd_b) * count
         del xg, wg, rg, gg, out, gin, grot, gw, ws
+    return per_layer, total_us, total_bytes
+
+
+def mobilenet_workload(a):
+    """The MobileNetV2-DK operator pass as a workload of its own (one JSON line; secondary to the headline)."""
+    per_layer, total_us, total_bytes = mobilenet_layers(a.batch, a.dtype, max(a.steps // 10, 10))
     print(json.dumps({
         "metric": "MobileNetV2-DK depthwise layers fwd+bwd, operator calls only (secondary workload)",
         "config": {"workload": "mbv2_dk: 17 DeformKernel2d layers, batch %d, scope 4x4, %s" % (a.batch, a.dtype)},

@@ -695,11 +695,16 @@ bool lanes_local_gather(const Geo& g, bool transposed, const T* src, const T* ro
   if ((long)g.in_h * g.in_w >= (1L << 24) || (long)g.out_h * g.out_w >= (1L << 24)) return false;  // byte offsets of 18 rotation planes in 31 bits
   if (!path_disabled(kForcePixelLanes)) {
     // A tile's set-up (18 rotation loads, 72 operand registers) is paid once per tile and wave and a block is 32
-    // channels: the kernel wins on large planes with many channels (N=64 C=144 56 x 56: 60 against 65 us for the
-    // kernel that stages the tiles in LDS; bfloat16 55 against 57), float16 is level (54.7 against 53.8) and stays there.
+    // channels: the kernel is for large planes with many channels.  Measured on N=64 C=144 56 x 56, against the
+    // kernel that stages its tiles in LDS (dk_local_mfma.hip): called in a loop of its own, where the 256 MB
+    // memory-side cache holds most of the 245 MB it touches, it is the faster one for float32 (60 against 63.4 us)
+    // and bfloat16 (55 / 57) and level for float16 (54.7 / 53.8); inside a forward + backward step, where the
+    // operands come from HBM, its two waves per SIMD with one block of loads in flight hide less of the latency
+    // than four waves with two staged tiles do -- float32 step 0.3165 against 0.3005 ms, bfloat16 0.2476
+    // against 0.2529 ms.  So the dispatch takes it for bfloat16 tensors only.
     const long plane = (long)g.out_h * g.out_w;
     const int cpg = g.channel / g.groups;
-    if (plane < 2048 || cpg < 96 || std::is_same<T, __half>::value) return false;
+    if (plane < 2048 || cpg < 96 || !std::is_same<T, bf16_t>::value) return false;
   }
   if (g.scope_h == 4 && g.scope_w == 4) return run_pixel_lanes<T, 4, 4>(g, transposed, src, rot, filter, dst, stream);
   if (g.scope_h == 3 && g.scope_w == 3) return run_pixel_lanes<T, 3, 3>(g, transposed, src, rot, filter, dst, stream);

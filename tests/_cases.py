@@ -69,6 +69,21 @@ def mixed_err(a, b):
     return float(((a - b).abs() / (scale + b.abs())).max())
 
 
+def elem_err(a, b, eps):
+    """max over the elements of |a - b| / (|b| + eps * max|b|): `elem_err(a, b, eps) < tol` says that EVERY element
+    is within tol of its own magnitude, with an absolute floor of tol * eps * max|b| for the elements that are small
+    by cancellation (their error is set by the terms that cancelled, not by their own size).  With eps << 1 this is
+    much tighter than rel_err() on the small elements and the same on the large ones."""
+    a = torch.as_tensor(a).detach().to(torch.float64)
+    b = torch.as_tensor(b).detach().to(torch.float64)
+    if b.numel() == 0:
+        return 0.0
+    scale = float(b.abs().max())
+    if scale == 0.0:
+        return float((a - b).abs().max())
+    return float(((a - b).abs() / (b.abs() + eps * scale)).max())
+
+
 def clipped_rotation(rot, clip, kernel_size, scope, groups):
     """What the reference's module does to the rotation tensor before the operator
     (modules/deform_kernel.py:185-212), restated on torch CPU tensors in the tensor's own
