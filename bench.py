@@ -170,6 +170,78 @@ def summarise_traffic(a):
     print("wrote", dest)
 
 
+def summarise_profile(a):
+    """--profile-from DB: a text summary of a rocprofv3 database (rocpd sqlite, `-d <dir> -o <name>`) of a
+    bench.py run: per-kernel durations, per-kernel counter averages when the run was a --pmc run, and for a
+    --kernel-trace run of the default workload the timeline of a step -- each dispatch's duration inside
+    the step and the idle gap in front of it.  Runs on the CPU; needs no GPU."""
+    import re
+    import sqlite3
+    cur = sqlite3.connect(a.profile_from).cursor()
+
+    def short(n):
+        n = n.replace("(anonymous namespace)::", "").replace("void ", "")
+        n = re.sub(r"at::native::", "", n)
+        return re.sub(r"\(.*$", "", n)[:100]
+    lines = []
+    rows = cur.execute("select name, start, end from kernels order by start").fetchall()
+    if rows:
+        stat = {}
+        for n, s0, e0 in rows:
+            stat.setdefault(short(n), []).append((e0 - s0) / 1e3)
+        total = sum(sum(v) for v in stat.values())
+        lines.append("%-100s %6s %9s %9s %9s %6s" % ("kernel", "calls", "avg_us", "min_us", "max_us", "pct"))
+        for n, v in sorted(stat.items(), key=lambda kv: -sum(kv[1])):
+            lines.append("%-100s %6d %9.2f %9.2f %9.2f %6.2f" % (n, len(v), sum(v) / len(v), min(v), max(v), 100 * sum(v) / total))
+        # the step's timeline: the longest run of consecutive library dispatches that repeats forward ... grad input
+        dk = [(short(n), s0, e0) for n, s0, e0 in rows if "dk::" in n]
+        names = [d[0] for d in dk]
+        fwd = [i for i, n in enumerate(names) if re.search(TRAFFIC_RULES["forward"][0], n) or re.search(TRAFFIC_RULES["forward"][1], n)]
+        period = None
+        for i in range(len(fwd) - 1):
+            if 2 <= fwd[i + 1] - fwd[i] <= 8:
+                period = fwd[i + 1] - fwd[i]
+                pattern = names[fwd[i]:fwd[i + 1]]
+                break
+        has_counters = bool(cur.execute("select count(*) from sqlite_master where name = 'counters_collection'").fetchone()[0]) and \
+            bool(cur.execute("select count(*) from counters_collection").fetchone()[0])
+        if period and not has_counters:  # (a counter run serialises the dispatches: its gaps say nothing)
+            steps = [i for i in fwd if names[i:i + period] == pattern and i + period < len(dk) and names[i + period] == pattern[0]]
+            if steps:
+                lines.append("")
+                lines.append("timeline of a step (%d consecutive steps of the timed loop): duration of each dispatch inside the step, and the" % len(steps))
+                lines.append("idle time between the end of the previous dispatch and its start (kernel-trace timestamps)")
+                lines.append("%-100s %9s %9s" % ("dispatch", "avg_us", "gap_us"))
+                tot_k = tot_g = 0.0
+                for j in range(period):
+                    dur = sum(dk[i + j][2] - dk[i + j][1] for i in steps) / len(steps) / 1e3
+                    gap = sum(dk[i + j][1] - dk[i + j - 1][2] for i in steps if i + j > 0) / len(steps) / 1e3
+                    tot_k += dur
+                    tot_g += gap
+                    lines.append("%-100s %9.2f %9.2f" % (pattern[j], dur, gap))
+                span = sum(dk[i + period][1] - dk[i][1] for i in steps) / len(steps) / 1e3
+                lines.append("%-100s %9.2f %9.2f   (step to step: %.2f us)" % ("sum", tot_k, tot_g, span))
+    try:
+        crow = cur.execute("select kernel_name, counter_name, count(*), avg(value) from counters_collection "
+                           "group by kernel_name, counter_name order by 1, 2").fetchall()
+    except sqlite3.Error:
+        crow = []
+    last = None
+    for k, c, n, v in crow:
+        if "dk::" not in k:
+            continue
+        if short(k) != last:
+            last = short(k)
+            lines.append("")
+            lines.append(last)
+        lines.append("   %-30s dispatches %-5d average per dispatch %.6g" % (c, n, v))
+    text = "\n".join(lines) + "\n"
+    if a.profile_out:
+        with open(a.profile_out, "a") as fh:
+            fh.write(text)
+    sys.stdout.write(text)
+
+
 def algorithmic_bytes(N, C, H, W, Ho, Wo, k, S, groups, esz):
     """Compulsory traffic, every tensor touched once (bytes), per kernel and per step."""
     x = N * C * H * W * esz
@@ -209,9 +281,14 @@ def main():
     ap.add_argument("--traffic-from", nargs=2, metavar=("FETCH_DB", "WRITE_DB"),
                     help="summarise two rocprofv3 counter databases into the tracked traffic table and exit")
     ap.add_argument("--traffic-out", default="", help="where --traffic-from writes (default: profiles/)")
+    ap.add_argument("--profile-from", default="", metavar="DB",
+                    help="summarise a rocprofv3 database of a bench.py run (kernel durations, the step's timeline, counters) and exit")
+    ap.add_argument("--profile-out", default="", help="append the --profile-from summary to this file as well")
     a = ap.parse_args()
     if a.traffic_from:
         return summarise_traffic(a)
+    if a.profile_from:
+        return summarise_profile(a)
     if a.gpus != 1:
         sys.exit("bench.py measures one GPU only: every box of this build has one GPU and no "
                  "multi-GPU path exists (the operator shards over the batch with no exchange); "
