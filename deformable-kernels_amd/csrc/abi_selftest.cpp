@@ -128,10 +128,23 @@ int main() {
   EXPECT(dk_offset_conv_supported(&oc) == 0);
   EXPECT(dk_offset_conv_forward(&oc, one, one, one, one, one, 1 << 30, nullptr) == DK_ERR_UNSUPPORTED);
   EXPECT(dk_offset_conv_backward_bias(nullptr, one, one, one, 0, nullptr) == DK_ERR_NULL_POINTER);
-  // the input gradient: 16-bit tensors on planes 28 / 56 / 112 wide only
+  // the input gradient: planes 7 .. 112 wide; float32 tensors as bfloat16 pairs unless that is switched off
   oc.w = 56;
-  EXPECT(dk_offset_conv_backward_input_workspace(&oc) == 0);
-  EXPECT(dk_offset_conv_backward_input(&oc, one, one, one, one, 1 << 30, nullptr) == DK_ERR_UNSUPPORTED);
+  EXPECT(dk_offset_conv_backward_input_workspace(&oc) > 0);
+  EXPECT(dk_offset_conv_backward_input_worthwhile(&oc) == 1);
+  EXPECT(dk_offset_conv_backward_input(&oc, one, one, one, one, 0, nullptr) == DK_ERR_WORKSPACE);
+  oc.in_channels = 32;
+  EXPECT(dk_offset_conv_backward_input_workspace(&oc) > 0);
+  EXPECT(dk_offset_conv_backward_input_worthwhile(&oc) == 0);  // covered, but not the faster choice
+  oc.in_channels = 144;
+  {
+    const unsigned pairs_off = 1u << 18;  // DK_NO_OFFSET_PAIRS
+    const unsigned before = dk_test_switches(pairs_off);
+    EXPECT(dk_offset_conv_supported(&oc) == 1);  // the fp32 matrix-instruction forward
+    EXPECT(dk_offset_conv_backward_input_workspace(&oc) == 0);
+    EXPECT(dk_offset_conv_backward_input(&oc, one, one, one, one, 1 << 30, nullptr) == DK_ERR_UNSUPPORTED);
+    dk_test_switches(before);
+  }
   oc.dtype = DK_BF16;
   EXPECT(dk_offset_conv_backward_input_workspace(&oc) > 0);
   EXPECT(dk_offset_conv_forward_workspace(&oc) > 0);
@@ -142,7 +155,7 @@ int main() {
   oc.w = 21;
   EXPECT(dk_offset_conv_backward_input(&oc, one, one, one, one, 1 << 30, nullptr) == DK_ERR_UNSUPPORTED);
   oc.w = 14;
-  // stride 2: forward and input gradient of 16-bit tensors only
+  // stride 2: forward and input gradient only
   oc.w = oc.h = 56, oc.stride = 2;
   EXPECT(dk_offset_conv_supported(&oc) == 1);
   EXPECT(dk_offset_conv_forward_workspace(&oc) > 0);
@@ -152,8 +165,9 @@ int main() {
   EXPECT(dk_offset_conv_backward_weight_workspace(&oc) == 0);
   EXPECT(dk_offset_conv_backward_weight(&oc, one, one, one, one, 1 << 30, nullptr) == DK_ERR_UNSUPPORTED);
   oc.dtype = DK_F32;
-  EXPECT(dk_offset_conv_supported(&oc) == 0);
-  EXPECT(dk_offset_conv_backward_input_workspace(&oc) == 0);
+  EXPECT(dk_offset_conv_supported(&oc) == 1);
+  EXPECT(dk_offset_conv_backward_input_workspace(&oc) > 0);
+  EXPECT(dk_offset_conv_backward_weight_workspace(&oc) == 0);
   oc.dtype = DK_BF16, oc.stride = 3;
   EXPECT(dk_offset_conv_forward(&oc, one, one, one, one, one, 1 << 30, nullptr) == DK_ERR_BAD_SHAPE);
   oc.stride = 0, oc.w = oc.h = 14;

@@ -31,7 +31,7 @@ unsigned switches_from_environment() {
       {"DK_NO_FILTER_SPLIT", kNoFilterSplit}, {"DK_NO_IMAGE_FLAT", kNoImageFlat},
       {"DK_NO_ND_SMALL", kNoNdSmall}, {"DK_NO_NHWC_MFMA", kNoNhwcMfma},
       {"DK_FORCE_GATHER_MFMA", kForceGatherMfma}, {"DK_NO_PIXEL_LANES", kNoPixelLanes},
-      {"DK_FORCE_PIXEL_LANES", kForcePixelLanes}};
+      {"DK_FORCE_PIXEL_LANES", kForcePixelLanes}, {"DK_NO_OFFSET_PAIRS", kNoOffsetPairs}};
   // a production process ignores these variables: they count only next to DK_ENABLE_TEST_SWITCHES=1
   const char* on = std::getenv("DK_ENABLE_TEST_SWITCHES");
   if (!on || on[0] != '1') return 0;
@@ -671,7 +671,7 @@ static int check_offset_conv(const dk_offset_conv_desc* d, bool forward = false)
   if (d->dtype != DK_F32 && d->dtype != DK_F16 && d->dtype != DK_BF16) return d->dtype == DK_F64 ? DK_ERR_UNSUPPORTED : DK_ERR_BAD_DTYPE;
   if ((long)d->batch * d->in_channels * d->h * d->w > kMaxElems) return DK_ERR_TOO_LARGE;
   if (d->stride == 2)
-    return forward && d->dtype != DK_F32 && d->in_channels % 16 == 0 &&
+    return forward && (d->dtype != DK_F32 || !path_disabled(kNoOffsetPairs)) && d->in_channels % 16 == 0 &&
                    offset_conv16_s2_supported(d->in_channels, d->out_channels, d->h, d->w)
                ? DK_OK
                : DK_ERR_UNSUPPORTED;
@@ -681,26 +681,30 @@ static int check_offset_conv(const dk_offset_conv_desc* d, bool forward = false)
 
 int dk_offset_conv_supported(const dk_offset_conv_desc* desc) { return check_offset_conv(desc, true) == DK_OK; }
 
+// Tensors on planes the 16-bit matrix-instruction kernels cover: 16-bit elements as they are, float32 ones as
+// bfloat16 (hi, lo) pairs
+static bool offset_conv_on_16_bit_matrix(const dk_offset_conv_desc* d) {
+  if (d->dtype == DK_F32 && path_disabled(kNoOffsetPairs)) return false;
+  return offset_conv16_supported(d->in_channels, d->out_channels, d->h, d->w);
+}
+
 int dk_offset_conv_worthwhile(const dk_offset_conv_desc* desc) {
   if (check_offset_conv(desc, true) != DK_OK) return 0;
   if (desc->stride == 2)  // as below, on the output plane
     return (long)desc->batch * ((((desc->h - 1) / 2 + 1) * (desc->w / 2) + 447) / 448) >= 64;
-  // 16-bit tensors: forward and input gradient on 16-bit matrix instructions are ahead of the library's on every
-  // plane they cover once there are workgroups ((image, 448-pixel tile) items) for a quarter of the CUs
-  if (desc->dtype != DK_F32 && offset_conv16_supported(desc->in_channels, desc->out_channels, desc->h, desc->w))
+  // forward and input gradient on 16-bit matrix instructions are ahead of the library's on every plane they cover
+  // once there are workgroups ((image, 448-pixel tile) items) for a quarter of the CUs
+  if (offset_conv_on_16_bit_matrix(desc))
     return (long)desc->batch * ((desc->h * desc->w + 447) / 448) >= 64;
   return offset_conv_worthwhile(desc->batch, desc->in_channels, desc->out_channels, desc->h, desc->w);
 }
 
-// 16-bit tensors on planes the 16-bit matrix-instruction kernels cover
-static bool offset_conv_on_16_bit_matrix(const dk_offset_conv_desc* d) {
-  return d->dtype != DK_F32 && offset_conv16_supported(d->in_channels, d->out_channels, d->h, d->w);
-}
-
 static size_t offset_conv_forward_need(const dk_offset_conv_desc* d) {
-  if (d->stride == 2) return offset_conv16_s2_workspace(d->batch, d->in_channels, d->out_channels, d->h, d->w);
-  return offset_conv_on_16_bit_matrix(d) ? offset_conv16_workspace(d->batch, d->in_channels, d->out_channels, d->h, d->w)
-                                         : offset_conv_workspace(d->batch, d->in_channels, d->out_channels, d->h, d->w);
+  const bool pairs = d->dtype == DK_F32;
+  if (d->stride == 2) return offset_conv16_s2_workspace(d->batch, d->in_channels, d->out_channels, d->h, d->w, pairs);
+  return offset_conv_on_16_bit_matrix(d)
+             ? offset_conv16_workspace(d->batch, d->in_channels, d->out_channels, d->h, d->w, pairs)
+             : offset_conv_workspace(d->batch, d->in_channels, d->out_channels, d->h, d->w);
 }
 
 size_t dk_offset_conv_forward_workspace(const dk_offset_conv_desc* desc) {
@@ -719,7 +723,7 @@ int dk_offset_conv_forward(const dk_offset_conv_desc* desc, const void* input, c
   bool ok = false;
   const bool matrix16 = offset_conv_on_16_bit_matrix(desc);
   const int st = by_dtype(desc->dtype, [&]<typename T>() {
-    if constexpr (sizeof(T) == 2) {
+    if constexpr (kHasFast<T>) {
       if (desc->stride == 2) {
         ok = offset_conv16_s2_forward<T>(desc->batch, desc->in_channels, desc->out_channels, desc->h, desc->w,
                                          in<T>(input), in<T>(weight), in<T>(bias), out<T>(output), workspace,
@@ -731,10 +735,9 @@ int dk_offset_conv_forward(const dk_offset_conv_desc* desc, const void* input, c
                                       in<T>(weight), in<T>(bias), out<T>(output), workspace, static_cast<hipStream_t>(stream));
         return;
       }
-    }
-    if constexpr (kHasFast<T>)
       ok = offset_conv_forward<T>(desc->batch, desc->in_channels, desc->out_channels, desc->h, desc->w, in<T>(input),
                                   in<T>(weight), in<T>(bias), out<T>(output), workspace, static_cast<hipStream_t>(stream));
+    }
   });
   return ok ? st : DK_ERR_UNSUPPORTED;
 }
@@ -748,8 +751,15 @@ static int check_offset_conv_backward_input(const dk_offset_conv_desc* d) {
 }
 
 static size_t offset_conv_backward_input_need(const dk_offset_conv_desc* d) {
-  return d->stride == 2 ? offset_conv16_s2_backward_input_workspace(d->in_channels, d->out_channels)
-                        : offset_conv16_workspace(d->batch, d->in_channels, d->out_channels, d->h, d->w);
+  const bool pairs = d->dtype == DK_F32;
+  return d->stride == 2 ? offset_conv16_s2_backward_input_workspace(d->in_channels, d->out_channels, pairs)
+                        : offset_conv16_workspace(d->batch, d->in_channels, d->out_channels, d->h, d->w, pairs);
+}
+
+int dk_offset_conv_backward_input_worthwhile(const dk_offset_conv_desc* desc) {
+  if (check_offset_conv_backward_input(desc) != DK_OK || !dk_offset_conv_worthwhile(desc)) return 0;
+  if (desc->dtype == DK_F32 && desc->stride != 2) return desc->in_channels >= 64 && desc->w >= 14;
+  return 1;
 }
 
 size_t dk_offset_conv_backward_input_workspace(const dk_offset_conv_desc* desc) {
@@ -765,18 +775,16 @@ int dk_offset_conv_backward_input(const dk_offset_conv_desc* desc, const void* o
   if (!workspace || workspace_bytes < offset_conv_backward_input_need(desc)) return DK_ERR_WORKSPACE;
   bool ok = false;
   const int st = by_dtype(desc->dtype, [&]<typename T>() {
-    if constexpr (sizeof(T) == 2) {
-      if (desc->stride == 2) {
+    if constexpr (kHasFast<T>) {
+      if (desc->stride == 2)
         ok = offset_conv16_s2_backward_input<T>(desc->batch, desc->in_channels, desc->out_channels, desc->h, desc->w,
                                                 in<T>(out_grad), in<T>(weight), out<T>(input_grad), workspace,
                                                 static_cast<hipStream_t>(stream));
-        return;
-      }
+      else
+        ok = offset_conv16_backward_input<T>(desc->batch, desc->in_channels, desc->out_channels, desc->h, desc->w,
+                                             in<T>(out_grad), in<T>(weight), out<T>(input_grad), workspace,
+                                             static_cast<hipStream_t>(stream));
     }
-    if constexpr (sizeof(T) == 2)
-      ok = offset_conv16_backward_input<T>(desc->batch, desc->in_channels, desc->out_channels, desc->h, desc->w,
-                                           in<T>(out_grad), in<T>(weight), out<T>(input_grad), workspace,
-                                           static_cast<hipStream_t>(stream));
   });
   return ok ? st : DK_ERR_UNSUPPORTED;
 }

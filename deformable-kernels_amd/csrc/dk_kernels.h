@@ -34,6 +34,7 @@ enum TestSwitch : unsigned {
   kNoImageFlat = 1u << 12,  // DK_NO_IMAGE_FLAT   the flat-copy kernels of the per-image depthwise convolution (the band kernels run instead)
   kNoPixelLanes = 1u << 16,     // DK_NO_PIXEL_LANES     the forward / grad input with the pixels on the matrix instruction's lanes
   kForcePixelLanes = 1u << 17,  // DK_FORCE_PIXEL_LANES  ... wherever it applies, not only where it is the faster kernel
+  kNoOffsetPairs = 1u << 18,    // DK_NO_OFFSET_PAIRS    the offset branch's convolution on float32 tensors as bfloat16 pairs (the fp32 matrix-instruction forward runs instead, the other passes are not offered)
 };
 unsigned test_switches();  // dk_api.hip
 inline bool path_disabled(unsigned sw) { return (test_switches() & sw) != 0; }
@@ -142,7 +143,7 @@ bool offset_conv_forward(int batch, int cin, int cout, int h, int w, const T* x,
 // dk_offset_conv16.hip: forward and input gradient of the same convolution on 16-bit matrix instructions
 // (fp16 / bf16 tensors, planes 7 / 14 / 28 / 56 / 112 wide, at most 32 output channels)
 bool offset_conv16_supported(int cin, int cout, int h, int w);
-size_t offset_conv16_workspace(int batch, int cin, int cout, int h, int w);
+size_t offset_conv16_workspace(int batch, int cin, int cout, int h, int w, bool pairs = false);  // pairs: float32 tensors
 template <typename T>
 bool offset_conv16_forward(int batch, int cin, int cout, int h, int w, const T* x, const T* weight, const T* bias,
                            T* out, void* ws, hipStream_t stream);
@@ -152,11 +153,11 @@ bool offset_conv16_backward_input(int batch, int cin, int cout, int h, int w, co
 
 // ... and its forward with stride 2 (input planes 14 / 28 / 56 / 112 wide; h, w: the input plane)
 bool offset_conv16_s2_supported(int cin, int cout, int h, int w);
-size_t offset_conv16_s2_workspace(int batch, int cin, int cout, int h, int w);
+size_t offset_conv16_s2_workspace(int batch, int cin, int cout, int h, int w, bool pairs = false);
 template <typename T>
 bool offset_conv16_s2_forward(int batch, int cin, int cout, int h, int w, const T* x, const T* weight, const T* bias,
                               T* out, void* ws, hipStream_t stream);
-size_t offset_conv16_s2_backward_input_workspace(int cin, int cout);
+size_t offset_conv16_s2_backward_input_workspace(int cin, int cout, bool pairs = false);
 template <typename T>
 bool offset_conv16_s2_backward_input(int batch, int cin, int cout, int h, int w, const T* gout, const T* weight,
                                      T* gin, void* ws, hipStream_t stream);

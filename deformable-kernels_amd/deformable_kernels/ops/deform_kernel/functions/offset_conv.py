@@ -2,20 +2,20 @@
 ``modules/deform_kernel.py:165-168``, applied at ``:214``).
 
 ``offset_conv(input, weight, bias, stride, padding, dilation)`` returns what
-``torch.nn.functional.conv2d`` returns.  For float32, float16 and bfloat16 GPU tensors (all of one dtype; the
-kernels multiply and add in float32 and round the results once) it runs
+``torch.nn.functional.conv2d`` returns.  For float32, float16 and bfloat16 GPU tensors (all of one dtype; fp32
+sums, results rounded once) with padding 1, dilation 1, input channels a multiple of 16, 18 output channels or
+at most 16, on planes 7, 14, 28, 56 or 112 wide (stride 2: input planes 14 to 112 wide) it runs
 
-  * the forward and -- for float32 tensors, or with ``force=True`` -- the weight gradient on the library's
-    matrix-core kernels where they apply and are the faster choice (stride 1, padding 1, dilation 1, input channels a multiple of 16,
-    18 output channels or at most 16, plane width 28, 56 or 112 with enough images to fill the GPU;
-    ``force=True``: wherever they apply, also widths 7 / 14),
+  * the forward and the input gradient on the library's shift-GEMM kernels on the 16-bit matrix instructions:
+    float16 / bfloat16 elements as they are (exact products), float32 elements as bfloat16 (hi, lo) pairs
+    (about 3.5e-6 of the result's scale against the float64 convolution),
+  * for float32 tensors at stride 1 -- or with ``force=True`` -- the weight gradient on the library's fp32
+    matrix-instruction kernel (the framework's 16-bit kernels are ahead for 16-bit tensors),
   * the bias gradient on the library's reduction kernel for every shape (the framework's
     reduction over (N, H, W) takes 60-230 us on the large planes),
-  * for float16 / bfloat16 tensors on planes 7, 14, 28, 56 or 112 wide, the forward and the input gradient on
-    the library's 16-bit matrix-instruction kernels (the elements are the operands as they are); the same two
-    passes with stride 2 on input planes 14, 28, 56 or 112 wide,
-  * everything else -- the input gradient of float32 tensors and of the other planes, and forward /
-    weight gradient of the other shapes -- on the framework's convolution routines.
+  * everything else -- other shapes, the weight gradient at stride 2, and passes the library reports as covered
+    but not worthwhile (too few images to fill the GPU; the float32 input gradient with fewer than 64 channels or
+    on 7 x 7 planes) unless ``force=True`` -- on the framework's convolution routines.
 
 float64, CPU tensors, mixed dtypes and autocast regions go to ``F.conv2d`` unchanged.
 """
@@ -107,6 +107,8 @@ class OffsetConvFunction(Function):
             native_weight = False
         library_weight = need_weight and not native_weight
         native_input = need_input and ctx.native and L.dk_offset_conv_backward_input_workspace(desc) > 0
+        if native_input and not ctx.forced and not L.dk_offset_conv_backward_input_worthwhile(desc):
+            native_input = False   # covered, but the framework's kernel is the faster one on this shape
         if (need_input and not native_input) or library_weight:
             # the framework's routine, without its bias gradient
             gi, gw_lib, _ = torch.ops.aten.convolution_backward(

@@ -292,13 +292,17 @@ int dk_nd_linear_sample_backward_coord(const dk_nd_desc *desc, const void *out_g
 /* The 3x3 convolution that predicts the kernel-space offsets of a LocalDeformKernel2d layer
  * (modules/deform_kernel.py:165-168: nn.Conv2d(in_planes, rotation_groups*k*k*2, k, stride,
  * padding, dilation, bias=True), applied at :214).  The reference calls the framework's
- * convolution there; this entry point is a faster kernel for that one shape family: stride 1,
- * padding 1, dilation 1, float32 / float16 / bfloat16 tensors (fp32 sums of fp32 products, or of the
- * exact products of the 16-bit elements; results rounded once), in_channels a multiple of 16,
- * out_channels <= 16 or 18 or 20, width 7, 14, 28, 56 or 112.  dk_offset_conv_supported() tells
+ * convolution there; this entry point is a faster kernel for that one shape family: padding 1,
+ * dilation 1, float32 / float16 / bfloat16 tensors, in_channels a multiple of 16, out_channels <= 16
+ * or 18 or 20, width 7, 14, 28, 56 or 112.  Arithmetic: fp32 sums throughout, results rounded once;
+ * float16 / bfloat16 elements are multiplied as they are (exact products) on the 16-bit matrix
+ * instructions; float32 elements go to the same instructions as bfloat16 (hi, lo) pairs, hi = bf16(v),
+ * lo = bf16(v - hi), all four products added: about 3.5e-6 of the result's scale against the float64
+ * convolution (the framework's float32 kernels: 5e-7), an infinite element gives NaN.  The test switch
+ * DK_NO_OFFSET_PAIRS restores the fp32 matrix-instruction forward (stride 1, 1e-6) and leaves the other
+ * float32 passes to the caller.  dk_offset_conv_supported() tells
  * whether a shape is covered, dk_offset_conv_worthwhile() whether it is also expected to beat the
- * library convolution (float32: planes 28 wide and wider with enough images to fill the GPU;
- * float16 / bfloat16: every covered plane with at least 64 (image, 448-pixel tile) items); the
+ * library convolution (every covered plane with at least 64 (image, 448-pixel tile) items); the
  * caller keeps its library convolution otherwise.
  *   input [batch, in_channels, h, w], weight [out_channels, in_channels, 3, 3],
  *   bias [out_channels], output [batch, out_channels, h, w]; workspace: packed weights. */
@@ -306,9 +310,9 @@ typedef struct dk_offset_conv_desc {
   int32_t batch, in_channels, out_channels, h, w; /* h, w: the input plane (= the output plane at stride 1) */
   int32_t dtype;  /* DK_F32, DK_F16 or DK_BF16 */
   int32_t stride; /* 0 or 1: stride 1.  2: the down-sampling layers' convolution (output ((h - 1) / 2 + 1) x (w / 2));
-                     only the forward and the input gradient of float16 / bfloat16 tensors on input planes 14, 28,
-                     56 or 112 wide have kernels: dk_offset_conv_supported() / _worthwhile() then speak for those
-                     two, and the weight gradient returns DK_ERR_UNSUPPORTED (workspace query 0) */
+                     only the forward and the input gradient on input planes 14, 28, 56 or 112 wide have kernels:
+                     dk_offset_conv_supported() / _worthwhile() then speak for those two, and the weight gradient
+                     returns DK_ERR_UNSUPPORTED (workspace query 0) */
 } dk_offset_conv_desc;
 int dk_offset_conv_supported(const dk_offset_conv_desc *desc);
 int dk_offset_conv_worthwhile(const dk_offset_conv_desc *desc);
@@ -333,11 +337,14 @@ int dk_offset_conv_backward_bias(const dk_offset_conv_desc *desc, const void *ou
                                  void *workspace, size_t workspace_bytes, void *stream);
 
 /* Gradient of that convolution's input (what autograd derives for the rotation_conv call at
- * modules/deform_kernel.py:214), input_grad [batch, in_channels, h, w] (fully written), for float16 /
- * bfloat16 tensors on planes 7, 14, 28, 56 or 112 wide: the 16-bit matrix instructions multiply the tensors'
- * elements as they are (exact products, fp32 sums, one rounding of the result).  The forward of such
- * tensors and planes runs on the same kernel.  Other shapes and float32 return DK_ERR_UNSUPPORTED (the
- * workspace query 0): the caller keeps its library's routine there. */
+ * modules/deform_kernel.py:214), input_grad [batch, in_channels, h, w] (fully written; float32 at stride 2:
+ * 8-byte aligned), on planes 7, 14, 28, 56 or 112 wide (stride 2: input planes 14 .. 112 wide): the same
+ * shift-GEMM kernel as the forward of such planes, arithmetic as described above.  Other shapes return
+ * DK_ERR_UNSUPPORTED (the workspace query 0): the caller keeps its library's routine there.
+ * dk_offset_conv_backward_input_worthwhile(): 1 where the kernel is also expected to be the faster choice
+ * (float32 at stride 1: from 64 input channels on planes 14 wide and wider -- with fewer channels the second,
+ * nearly empty chunk of the 18 output-gradient channels' pairs costs more than the library's kernel takes). */
+int dk_offset_conv_backward_input_worthwhile(const dk_offset_conv_desc *desc);
 size_t dk_offset_conv_backward_input_workspace(const dk_offset_conv_desc *desc);
 int dk_offset_conv_backward_input(const dk_offset_conv_desc *desc, const void *out_grad, const void *weight,
                                   void *input_grad, void *workspace, size_t workspace_bytes, void *stream);
@@ -378,7 +385,7 @@ const char *dk_status_string(int status);
  * kernel.  Bit i belongs to the i-th of DK_NO_ROWS, DK_NO_MFMA, DK_NO_MFMA_S2, DK_NO_S2_QUADS,
  * DK_NO_DEFORM_FAST, DK_NO_DEFORM_CH, DK_NO_DEFORM_CH_BIG, DK_NO_DEFORM_MFMA, DK_NO_ND_BINS,
  * DK_NO_ND_MFMA, DK_NO_GATHER_MFMA, DK_NO_FILTER_SPLIT, DK_NO_IMAGE_FLAT, DK_NO_ND_SMALL, DK_NO_NHWC_MFMA,
- * DK_FORCE_GATHER_MFMA, DK_NO_PIXEL_LANES, DK_FORCE_PIXEL_LANES.  The mask starts at 0; only a process
+ * DK_FORCE_GATHER_MFMA, DK_NO_PIXEL_LANES, DK_FORCE_PIXEL_LANES, DK_NO_OFFSET_PAIRS.  The mask starts at 0; only a process
  * started with DK_ENABLE_TEST_SWITCHES=1 in its environment also reads the environment variables of
  * those names, once, at the first call that consults the mask (a stray variable in a production
  * environment changes nothing).  This call replaces the mask and returns the previous one.
