@@ -155,28 +155,39 @@ int main() {
   oc.w = 21;
   EXPECT(dk_offset_conv_backward_input(&oc, one, one, one, one, 1 << 30, nullptr) == DK_ERR_UNSUPPORTED);
   oc.w = 14;
-  // stride 2: forward and input gradient only
+  // stride 2: every pass on the 16-bit matrix instructions
   oc.w = oc.h = 56, oc.stride = 2;
   EXPECT(dk_offset_conv_supported(&oc) == 1);
   EXPECT(dk_offset_conv_forward_workspace(&oc) > 0);
   EXPECT(dk_offset_conv_forward(&oc, one, one, one, one, one, 0, nullptr) == DK_ERR_WORKSPACE);
   EXPECT(dk_offset_conv_backward_input_workspace(&oc) > 0);
   EXPECT(dk_offset_conv_backward_input(&oc, one, one, one, one, 0, nullptr) == DK_ERR_WORKSPACE);
-  EXPECT(dk_offset_conv_backward_weight_workspace(&oc) == 0);
-  EXPECT(dk_offset_conv_backward_weight(&oc, one, one, one, one, 1 << 30, nullptr) == DK_ERR_UNSUPPORTED);
+  EXPECT(dk_offset_conv_backward_weight_workspace(&oc) > 0);
+  EXPECT(dk_offset_conv_backward_weight(&oc, one, one, one, one, 0, nullptr) == DK_ERR_WORKSPACE);
+  {
+    const unsigned before = dk_test_switches(1u << 19);  // DK_NO_OFFSET_WGRAD16
+    EXPECT(dk_offset_conv_backward_weight_workspace(&oc) == 0);
+    EXPECT(dk_offset_conv_backward_weight(&oc, one, one, one, one, 1 << 30, nullptr) == DK_ERR_UNSUPPORTED);
+    dk_test_switches(before);
+  }
   oc.dtype = DK_F32;
   EXPECT(dk_offset_conv_supported(&oc) == 1);
   EXPECT(dk_offset_conv_backward_input_workspace(&oc) > 0);
-  EXPECT(dk_offset_conv_backward_weight_workspace(&oc) == 0);
+  EXPECT(dk_offset_conv_backward_weight_workspace(&oc) > 0);
   oc.dtype = DK_BF16, oc.stride = 3;
   EXPECT(dk_offset_conv_forward(&oc, one, one, one, one, one, 1 << 30, nullptr) == DK_ERR_BAD_SHAPE);
   oc.stride = 0, oc.w = oc.h = 14;
-  // the weight gradient: 15 and more outputs
+  // the weight gradient: up to 20 outputs on the 16-bit matrix instructions, 15 and more on the fp32 ones
   EXPECT(dk_offset_conv_backward_weight_workspace(&oc) > 0);
   oc.out_channels = 7;
   EXPECT(dk_offset_conv_supported(&oc) == 1);
-  EXPECT(dk_offset_conv_backward_weight_workspace(&oc) == 0);
-  EXPECT(dk_offset_conv_backward_weight(&oc, one, one, one, one, 1 << 30, nullptr) == DK_ERR_UNSUPPORTED);
+  EXPECT(dk_offset_conv_backward_weight_workspace(&oc) > 0);
+  {
+    const unsigned before = dk_test_switches(1u << 19);
+    EXPECT(dk_offset_conv_backward_weight_workspace(&oc) == 0);
+    EXPECT(dk_offset_conv_backward_weight(&oc, one, one, one, one, 1 << 30, nullptr) == DK_ERR_UNSUPPORTED);
+    dk_test_switches(before);
+  }
 
   EXPECT(std::strstr(dk_status_string(DK_ERR_WORKSPACE), "workspace") != nullptr);
   EXPECT(dk_status_string(-99) != nullptr);

@@ -31,7 +31,7 @@ unsigned switches_from_environment() {
       {"DK_NO_FILTER_SPLIT", kNoFilterSplit}, {"DK_NO_IMAGE_FLAT", kNoImageFlat},
       {"DK_NO_ND_SMALL", kNoNdSmall}, {"DK_NO_NHWC_MFMA", kNoNhwcMfma},
       {"DK_FORCE_GATHER_MFMA", kForceGatherMfma}, {"DK_NO_PIXEL_LANES", kNoPixelLanes},
-      {"DK_FORCE_PIXEL_LANES", kForcePixelLanes}, {"DK_NO_OFFSET_PAIRS", kNoOffsetPairs}};
+      {"DK_FORCE_PIXEL_LANES", kForcePixelLanes}, {"DK_NO_OFFSET_PAIRS", kNoOffsetPairs}, {"DK_NO_OFFSET_WGRAD16", kNoOffsetWgrad16}};
   // a production process ignores these variables: they count only next to DK_ENABLE_TEST_SWITCHES=1
   const char* on = std::getenv("DK_ENABLE_TEST_SWITCHES");
   if (!on || on[0] != '1') return 0;
@@ -789,24 +789,54 @@ int dk_offset_conv_backward_input(const dk_offset_conv_desc* desc, const void* o
   return ok ? st : DK_ERR_UNSUPPORTED;
 }
 
+// The weight gradient on the 16-bit matrix instructions: 16-bit tensors, and float32 ones as bfloat16 pairs
+static bool offset_wgrad_on_16_bit_matrix(const dk_offset_conv_desc* d) {
+  if (path_disabled(kNoOffsetWgrad16) || (d->dtype == DK_F32 && path_disabled(kNoOffsetPairs))) return false;
+  return offset_wgrad16_supported(d->in_channels, d->out_channels, d->h, d->w, d->stride == 2 ? 2 : 1);
+}
+
+static int check_offset_conv_backward_weight(const dk_offset_conv_desc* d) {
+  if (!d) return DK_ERR_NULL_POINTER;
+  if (d->stride == 2) {
+    const int rc = check_offset_conv(d, true);  // shapes and dtypes as for the stride-2 forward
+    if (rc != DK_OK) return rc;
+    return offset_wgrad_on_16_bit_matrix(d) ? DK_OK : DK_ERR_UNSUPPORTED;
+  }
+  return check_offset_conv(d);
+}
+
+static size_t offset_conv_backward_weight_need(const dk_offset_conv_desc* d) {
+  if (offset_wgrad_on_16_bit_matrix(d))
+    return offset_wgrad16_workspace(d->batch, d->in_channels, d->out_channels, d->h, d->w, d->stride == 2 ? 2 : 1,
+                                    d->dtype == DK_F32);
+  return offset_conv_wgrad_workspace(d->batch, d->in_channels, d->out_channels, d->h, d->w);
+}
+
 size_t dk_offset_conv_backward_weight_workspace(const dk_offset_conv_desc* desc) {
-  if (check_offset_conv(desc) != DK_OK) return 0;
-  return offset_conv_wgrad_workspace(desc->batch, desc->in_channels, desc->out_channels, desc->h, desc->w);
+  if (check_offset_conv_backward_weight(desc) != DK_OK) return 0;
+  return offset_conv_backward_weight_need(desc);
 }
 
 int dk_offset_conv_backward_weight(const dk_offset_conv_desc* desc, const void* out_grad, const void* input,
                                    void* weight_grad, void* workspace, size_t workspace_bytes, void* stream) {
-  const int rc = check_offset_conv(desc);
+  const int rc = check_offset_conv_backward_weight(desc);
   if (rc != DK_OK) return rc;
   if (!out_grad || !input || !weight_grad) return DK_ERR_NULL_POINTER;
-  const size_t need = offset_conv_wgrad_workspace(desc->batch, desc->in_channels, desc->out_channels, desc->h, desc->w);
-  if (need == 0) return DK_ERR_UNSUPPORTED;  // fewer than 15 outputs
+  const size_t need = offset_conv_backward_weight_need(desc);
+  if (need == 0) return DK_ERR_UNSUPPORTED;  // fewer than 15 outputs on the fp32 matrix-instruction kernel
   if (!workspace || workspace_bytes < need) return DK_ERR_WORKSPACE;
+  const bool matrix16 = offset_wgrad_on_16_bit_matrix(desc);
   bool ok = false;
   const int st = by_dtype(desc->dtype, [&]<typename T>() {
-    if constexpr (kHasFast<T>)
-      ok = offset_conv_wgrad<T>(desc->batch, desc->in_channels, desc->out_channels, desc->h, desc->w, in<T>(input),
-                                in<T>(out_grad), out<T>(weight_grad), workspace, static_cast<hipStream_t>(stream));
+    if constexpr (kHasFast<T>) {
+      if (matrix16)
+        ok = offset_wgrad16<T>(desc->batch, desc->in_channels, desc->out_channels, desc->h, desc->w,
+                               desc->stride == 2 ? 2 : 1, in<T>(input), in<T>(out_grad), out<T>(weight_grad), workspace,
+                               static_cast<hipStream_t>(stream));
+      else
+        ok = offset_conv_wgrad<T>(desc->batch, desc->in_channels, desc->out_channels, desc->h, desc->w, in<T>(input),
+                                  in<T>(out_grad), out<T>(weight_grad), workspace, static_cast<hipStream_t>(stream));
+    }
   });
   return ok ? st : DK_ERR_UNSUPPORTED;
 }

@@ -34,6 +34,7 @@ enum TestSwitch : unsigned {
   kNoImageFlat = 1u << 12,  // DK_NO_IMAGE_FLAT   the flat-copy kernels of the per-image depthwise convolution (the band kernels run instead)
   kNoPixelLanes = 1u << 16,     // DK_NO_PIXEL_LANES     the forward / grad input with the pixels on the matrix instruction's lanes
   kForcePixelLanes = 1u << 17,  // DK_FORCE_PIXEL_LANES  ... wherever it applies, not only where it is the faster kernel
+  kNoOffsetWgrad16 = 1u << 19,  // DK_NO_OFFSET_WGRAD16  the offset branch's weight gradient on 16-bit matrix instructions (the fp32 matrix-instruction kernel at stride 1, nothing at stride 2)
   kNoOffsetPairs = 1u << 18,    // DK_NO_OFFSET_PAIRS    the offset branch's convolution on float32 tensors as bfloat16 pairs (the fp32 matrix-instruction forward runs instead, the other passes are not offered)
 };
 unsigned test_switches();  // dk_api.hip
@@ -161,6 +162,15 @@ size_t offset_conv16_s2_backward_input_workspace(int cin, int cout, bool pairs =
 template <typename T>
 bool offset_conv16_s2_backward_input(int batch, int cin, int cout, int h, int w, const T* gout, const T* weight,
                                      T* gin, void* ws, hipStream_t stream);
+
+// dk_offset_wgrad16.hip: the weight gradient of that convolution on 16-bit matrix instructions, stride 1 (planes
+// 7 .. 112 wide) and 2 (input planes 14 .. 112 wide), up to 20 outputs, input channels a multiple of 16; float32
+// tensors as bfloat16 pairs.  h, w: the input plane.  Workspace 0: not covered.
+bool offset_wgrad16_supported(int cin, int cout, int h, int w, int stride);
+size_t offset_wgrad16_workspace(int batch, int cin, int cout, int h, int w, int stride, bool pairs);
+template <typename T>
+bool offset_wgrad16(int batch, int cin, int cout, int h, int w, int stride, const T* x, const T* gout, T* gweight,
+                    void* ws, hipStream_t stream);
 
 // dk_local_nhwc.hip: the local operator on channels-last tensors, all dtypes, any geometry whose tables fit LDS
 bool nhwc_supported(const Geo& g, int dtype);

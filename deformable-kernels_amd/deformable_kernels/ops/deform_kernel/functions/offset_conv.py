@@ -9,11 +9,11 @@ at most 16, on planes 7, 14, 28, 56 or 112 wide (stride 2: input planes 14 to 11
   * the forward and the input gradient on the library's shift-GEMM kernels on the 16-bit matrix instructions:
     float16 / bfloat16 elements as they are (exact products), float32 elements as bfloat16 (hi, lo) pairs
     (about 3.5e-6 of the result's scale against the float64 convolution),
-  * for float32 tensors at stride 1 -- or with ``force=True`` -- the weight gradient on the library's fp32
-    matrix-instruction kernel (the framework's 16-bit kernels are ahead for 16-bit tensors),
+  * the weight gradient on the library's kernel for the 16-bit matrix instructions (stride 1 and 2, up to 20
+    outputs; float32 tensors again as bfloat16 pairs), per-workgroup partial sums added in a fixed order,
   * the bias gradient on the library's reduction kernel for every shape (the framework's
     reduction over (N, H, W) takes 60-230 us on the large planes),
-  * everything else -- other shapes, the weight gradient at stride 2, and passes the library reports as covered
+  * everything else -- other shapes, and passes the library reports as covered
     but not worthwhile (too few images to fill the GPU; the float32 input gradient with fewer than 64 channels or
     on 7 x 7 planes) unless ``force=True`` -- on the framework's convolution routines.
 
@@ -96,15 +96,9 @@ class OffsetConvFunction(Function):
         need_input, need_weight = ctx.needs_input_grad[0], ctx.needs_input_grad[1]
         gi = gw = gb = None
         L = _lib.lib()
-        # the input gradient has a kernel of its own for 16-bit tensors on the wider planes, the weight
-        # gradient for 15 and more outputs: a workspace query of 0 says "not covered"
+        # a workspace query of 0 says "this pass is not covered"
         desc = _desc(input, weight, stride=stride[0])
         native_weight = need_weight and ctx.native and L.dk_offset_conv_backward_weight_workspace(desc) > 0
-        # 16-bit tensors: the weight-gradient kernel multiplies in fp32 and the framework's on 16-bit matrix
-        # instructions, which is ahead on every plane (bf16, batch 128: 317 / 264 / 95 us against 330 / 290 / 150
-        # on planes 112 / 56 / 28 wide), so it keeps that pass unless the kernels were asked for
-        if native_weight and input.dtype != torch.float32 and not ctx.forced:
-            native_weight = False
         library_weight = need_weight and not native_weight
         native_input = need_input and ctx.native and L.dk_offset_conv_backward_input_workspace(desc) > 0
         if native_input and not ctx.forced and not L.dk_offset_conv_backward_input_worthwhile(desc):

@@ -311,8 +311,7 @@ typedef struct dk_offset_conv_desc {
   int32_t dtype;  /* DK_F32, DK_F16 or DK_BF16 */
   int32_t stride; /* 0 or 1: stride 1.  2: the down-sampling layers' convolution (output ((h - 1) / 2 + 1) x (w / 2));
                      only the forward and the input gradient on input planes 14, 28, 56 or 112 wide have kernels:
-                     dk_offset_conv_supported() / _worthwhile() then speak for those two, and the weight gradient
-                     returns DK_ERR_UNSUPPORTED (workspace query 0) */
+                     dk_offset_conv_supported() / _worthwhile() then speak for those two */
 } dk_offset_conv_desc;
 int dk_offset_conv_supported(const dk_offset_conv_desc *desc);
 int dk_offset_conv_worthwhile(const dk_offset_conv_desc *desc);
@@ -321,10 +320,13 @@ int dk_offset_conv_forward(const dk_offset_conv_desc *desc, const void *input, c
                            const void *bias, void *output, void *workspace, size_t workspace_bytes,
                            void *stream);
 
-/* Gradient of that convolution's weight, weight_grad [out_channels, in_channels, 3, 3] (fully
- * written), for the shapes dk_offset_conv_supported() accepts with 15, 16, 18 or 20 output channels
- * (fewer: the workspace query returns 0, the call DK_ERR_UNSUPPORTED, and the caller keeps its
- * library's routine); per-workgroup partial sums in the workspace are added in a fixed order. */
+/* Gradient of that convolution's weight, weight_grad [out_channels, in_channels, 3, 3] (fully written),
+ * stride 1 and 2, up to 20 output channels: on the 16-bit matrix instructions with the pixels as the inner
+ * dimension (16-bit elements as they are, float32 ones as bfloat16 pairs: about 4e-6 of the result's scale);
+ * per-workgroup partial sums in the workspace are added in a fixed order.  With the test switch
+ * DK_NO_OFFSET_WGRAD16 (or DK_NO_OFFSET_PAIRS for float32) the fp32 matrix-instruction kernel serves stride 1
+ * with 15, 16, 18 or 20 outputs.  A workspace query of 0 / DK_ERR_UNSUPPORTED: not covered, the caller keeps
+ * its library's routine. */
 size_t dk_offset_conv_backward_weight_workspace(const dk_offset_conv_desc *desc);
 int dk_offset_conv_backward_weight(const dk_offset_conv_desc *desc, const void *out_grad, const void *input,
                                    void *weight_grad, void *workspace, size_t workspace_bytes,
@@ -385,7 +387,7 @@ const char *dk_status_string(int status);
  * kernel.  Bit i belongs to the i-th of DK_NO_ROWS, DK_NO_MFMA, DK_NO_MFMA_S2, DK_NO_S2_QUADS,
  * DK_NO_DEFORM_FAST, DK_NO_DEFORM_CH, DK_NO_DEFORM_CH_BIG, DK_NO_DEFORM_MFMA, DK_NO_ND_BINS,
  * DK_NO_ND_MFMA, DK_NO_GATHER_MFMA, DK_NO_FILTER_SPLIT, DK_NO_IMAGE_FLAT, DK_NO_ND_SMALL, DK_NO_NHWC_MFMA,
- * DK_FORCE_GATHER_MFMA, DK_NO_PIXEL_LANES, DK_FORCE_PIXEL_LANES, DK_NO_OFFSET_PAIRS.  The mask starts at 0; only a process
+ * DK_FORCE_GATHER_MFMA, DK_NO_PIXEL_LANES, DK_FORCE_PIXEL_LANES, DK_NO_OFFSET_PAIRS, DK_NO_OFFSET_WGRAD16.  The mask starts at 0; only a process
  * started with DK_ENABLE_TEST_SWITCHES=1 in its environment also reads the environment variables of
  * those names, once, at the first call that consults the mask (a stray variable in a production
  * environment changes nothing).  This call replaces the mask and returns the previous one.
