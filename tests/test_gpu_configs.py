@@ -204,8 +204,8 @@ def test_config5_mobilenetv2_dk_network_bfloat16():
     """MobileNetV2 with its 17 depthwise 3 x 3 convolutions replaced by DeformKernel2d (scope 4 x 4),
     bfloat16 activations and parameters; the operator keeps float32 sums for the filter gradient.
     Batch 128: one forward + backward, every gradient finite and every deformable layer trained.
-    Batch 2: the operator calls of three layers as the network issues them (captured inputs, rotations
-    and upstream gradients) against the float32 oracle on the same rounded tensors."""
+    Batch 2: the operator calls of all 17 layers as the network issues them (captured inputs, rotations
+    and upstream gradients) against the float32 oracle on the same rounded tensors: forward and filter gradient."""
     from _mbv2_dk import MobileNetV2DK
     torch.manual_seed(5)
     net = MobileNetV2DK().to(DEV).to(torch.bfloat16)
@@ -226,9 +226,9 @@ def test_config5_mobilenetv2_dk_network_bfloat16():
         assert float(l.inner_conv.weight.grad.float().abs().max()) > 0, i
         assert float(l.rotation_conv.weight.grad.float().abs().max()) > 0, i
 
-    # batch 2: three layers' operator calls against the oracle (112 x 112 C=32; 56 x 56 C=144 stride 2; 7 x 7 C=960)
+    # batch 2: every layer's operator calls against the oracle (112 x 112 C=32 down to 7 x 7 C=960, four of them stride 2)
     net.zero_grad(set_to_none=True)
-    picked = {0: {}, 3: {}, 16: {}}
+    picked = {i: {} for i in range(17)}
     handles = [_capture(layers[i], st) for i, st in picked.items()]
     loss = torch.nn.functional.cross_entropy(net(x[:2]).float(), labels[:2])
     loss.backward()
