@@ -221,6 +221,9 @@ def summarise_profile(a):
                     lines.append("%-100s %9.2f %9.2f" % (pattern[j], dur, gap))
                 span = sum(dk[i + period][1] - dk[i][1] for i in steps) / len(steps) / 1e3
                 lines.append("%-100s %9.2f %9.2f   (step to step: %.2f us)" % ("sum", tot_k, tot_g, span))
+                lines.append("(Dispatches of one native call follow each other on the device; the gap in front of a call's first")
+                lines.append(" dispatch is the host's time between two calls, which the tracer lengthens: without it the host stays")
+                lines.append(" ahead of the device and the step takes what bench.py reports.)")
     try:
         crow = cur.execute("select kernel_name, counter_name, count(*), avg(value) from counters_collection "
                            "group by kernel_name, counter_name order by 1, 2").fetchall()

@@ -267,8 +267,18 @@ __global__ __launch_bounds__(256) void offset_wgrad16_reduce_kernel(const float*
   const int t = idx % 9, c = idx / 9 % cin, o = idx / 9 / cin;
   const int row = o % 16, l = (row / 4) * 16 + c % 16, r = row % 4;
   const float* p = partial + ((size_t)(c / kW16Chunk) * kW16Tiles + t * kW16Blocks + o / 16) * 256 + 4 * l + r;
+  const size_t step = (size_t)nchunks * (kW16Tiles * 256);
+  // eight loads in flight, added in part order
   float s = 0.f;
-  for (int q = 0; q < parts; ++q) s += p[(size_t)q * nchunks * (kW16Tiles * 256)];
+  int q = 0;
+  for (; q + 8 <= parts; q += 8) {
+    float v[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) v[j] = p[(size_t)(q + j) * step];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) s += v[j];
+  }
+  for (; q < parts; ++q) s += p[(size_t)q * step];
   st(gw + idx, s);
 }
 
