@@ -701,10 +701,16 @@ bool lanes_local_gather(const Geo& g, bool transposed, const T* src, const T* ro
     // and bfloat16 (55 / 57) and level for float16 (54.7 / 53.8); inside a forward + backward step, where the
     // operands come from HBM, its two waves per SIMD with one block of loads in flight hide less of the latency
     // than four waves with two staged tiles do -- float32 step 0.3165 against 0.3005 ms, bfloat16 0.2476
-    // against 0.2529 ms.  So the dispatch takes it for bfloat16 tensors only.
+    // against 0.2529 ms.  So on large planes the dispatch takes it for bfloat16 tensors only.  On planes of fewer
+    // than 2048 pixels (the 28 x 28, 14 x 14 and 7 x 7 stages of MobileNetV2-DK, 128 to 960 channels) its small
+    // per-tile set-up makes it the faster kernel for both 16-bit types -- forward, batch 64 / 128: 28 x 28 C=192
+    // 22.8 against 29.4 us / 38.2 against 44.5, 14 x 14 C=576 20.7 against 26.1, 7 x 7 C=960 14.2 against 16.2 /
+    // 19.7 against 29.5, the layer's forward + backward step 4 to 16 % shorter -- while float32 gains on two of
+    // those shapes (1.6 and 4 % of the step) and loses on the others, and stays where it was.
     const long plane = (long)g.out_h * g.out_w;
     const int cpg = g.channel / g.groups;
-    if (plane < 2048 || cpg < 96 || !std::is_same<T, bf16_t>::value) return false;
+    const bool large = plane >= 2048;
+    if (cpg < 96 || sizeof(T) == 4 || (large && !std::is_same<T, bf16_t>::value)) return false;
   }
   if (g.scope_h == 4 && g.scope_w == 4) return run_pixel_lanes<T, 4, 4>(g, transposed, src, rot, filter, dst, stream);
   if (g.scope_h == 3 && g.scope_w == 3) return run_pixel_lanes<T, 3, 3>(g, transposed, src, rot, filter, dst, stream);
