@@ -88,3 +88,41 @@ def test_local_operator_on_random_geometries_in_16_bits(k, case):
     for g, w, name in zip(got, want, ("forward", "grad input", "grad rotation", "grad filter")):
         assert g.dtype == dtype
         assert rel_err(g.float(), w) < 1e-2, name
+
+
+def _offset_conv_cases():
+    rnd = random.Random(23)
+    cases = []
+    for _ in range(36):
+        stride = rnd.choice([1, 1, 2])
+        W = rnd.choice([7, 14, 28, 56, 112] if stride == 1 else [14, 28, 56, 112])
+        cases.append((rnd.choice([1, 2, 3, 5]), rnd.choice([16, 32, 48, 80, 144]), rnd.choice([1, 2, 3, 5, 7, 8, 9, 14, 17, 23, 33]),
+                      W, rnd.choice([1, 2, 7, 15, 16, 18, 20]), stride, rnd.choice(["float32", "float16", "bfloat16"])))
+    return cases
+
+
+@pytest.mark.parametrize("case", _offset_conv_cases())
+def test_offset_branch_convolution_on_random_shapes(case):
+    """Every pass of the layers' 3 x 3 offset convolution (forward, input, weight and bias gradient; stride 1 and
+    2; 1 to 20 outputs; tiles of one row, partial last tiles, planes lower than a tile) against the float64
+    convolution on the CPU."""
+    import test_gpu_offset_conv as toc
+    from deformable_kernels.ops.deform_kernel.functions import offset_conv, offset_conv_supported
+    N, C, H, W, O, stride, dtype_name = case
+    dtype = getattr(torch, dtype_name)
+    tol = {"float32": 1e-5, "float16": 2e-3, "bfloat16": 1e-2}[dtype_name]
+    g = torch.Generator().manual_seed(hash(case[:6]) % 1000)
+    dev = torch.device("cuda:0")
+    x = torch.randn(N, C, H, W, generator=g).to(dtype).to(dev).requires_grad_()
+    w = (torch.randn(O, C, 3, 3, generator=g) * 0.05).to(dtype).to(dev).requires_grad_()
+    b = torch.randn(O, generator=g).to(dtype).to(dev).requires_grad_()
+    assert offset_conv_supported(x, w, b, stride, 1, 1)
+    out = offset_conv(x, w, b, stride=stride, force=True)
+    gout = torch.randn(out.shape, generator=g).to(dtype).to(dev)
+    want, gx, gw, gb = toc.reference(x, w, b, gout, stride=stride)
+    assert out.shape == want.shape and out.dtype == dtype
+    out.backward(gout)
+    assert rel_err(out.detach().double().cpu(), want) < tol, "forward"
+    assert rel_err(x.grad.double().cpu(), gx) < tol, "input gradient"
+    assert rel_err(w.grad.double().cpu(), gw) < tol, "weight gradient"
+    assert rel_err(b.grad.double().cpu(), gb) < tol, "bias gradient"
