@@ -38,6 +38,8 @@ CASES = [
     (1, 4, 40, 130, 3, (3, 3), 1, 1, 1, 2, 0.6, 3.0),     # 130 columns: 256 lanes per staged row, two groups
     (2, 6, 112, 112, 3, (4, 4), 2, 1, 1, 1, 0.5, 8.0),    # 112 x 112 stride 2 with offsets that spread a tile's samples over most of the plane
     (1, 3, 100, 30, 3, (5, 5), 1, 1, 1, 1, 1.0, 2.5),     # narrow but taller than the 256-thread staging covers; scope 5
+    (1, 20, 60, 40, 3, (4, 4), 1, 1, 1, 2, 0.7, 10.0),    # row-window grad filter: offsets of ten rows spread a tile's samples over three windows of 24 rows; two channel blocks, the second partial
+    (2, 33, 56, 56, 3, (5, 5), 1, 1, 1, 1, 1.0, 2.0),     # row-window grad filter, scope 5 (two launches of 16 cells), three channel blocks
 ]
 NAMES = ("forward", "grad input", "grad offset", "grad rotation", "grad filter")
 
@@ -222,7 +224,8 @@ def test_config4_properties_at_full_size():
 
 
 @pytest.mark.parametrize("switch,case", [("DK_NO_DEFORM_CH", CASES[0]), ("DK_NO_DEFORM_MFMA", CASES[0]),
-                                         ("DK_NO_DEFORM_CH_BIG", CASES[7])])
+                                         ("DK_NO_DEFORM_CH_BIG", CASES[7]), ("DK_NO_DEFORM_WINDOW", CASES[13]),
+                                         ("DK_NO_DEFORM_WINDOW", CASES[20])])
 def test_one_plane_kernels_on_a_shape_the_newer_ones_cover(switch_off, switch, case):
     """Without the channel-interleaved kernels (those for small planes and those for large ones) / the
     matrix-core grad filter the one-plane kernels serve the shape."""
