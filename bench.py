@@ -170,6 +170,49 @@ def summarise_traffic(a):
     print("wrote", dest)
 
 
+def traffic_table(a):
+    """--traffic-table: the tracked HBM counter tables profiles/hbm_traffic_*.json as one text
+    (profiles/local_dk_hbm_counters.txt).  Runs on the CPU; needs no GPU."""
+    import glob
+    lines = ["HBM traffic counters of the local deformable-kernel operator, MI355X, one GPU: FETCH_SIZE and WRITE_SIZE per call of each",
+             "entry point, from the tables profiles/hbm_traffic_<workload>_<dtype>.json (which bench.py reads for roofline.traffic).", "",
+             "Commands (from the repository root, on the GPU box; one counter per run, then the summaries, which need no GPU):",
+             "  rocprofv3 --pmc FETCH_SIZE -d /tmp/dk_prof/F -o pmc -- python3 bench.py --workload W --dtype D --steps 3 --warmup 1 --no-cpu-baseline --no-network-pass",
+             "  rocprofv3 --pmc WRITE_SIZE -d /tmp/dk_prof/W -o pmc -- python3 bench.py --workload W --dtype D --steps 3 --warmup 1 --no-cpu-baseline --no-network-pass",
+             "  python3 bench.py --workload W --dtype D --traffic-from /tmp/dk_prof/F/*/pmc_results.db /tmp/dk_prof/W/*/pmc_results.db",
+             "  python3 bench.py --traffic-table", "",
+             "Calibration: the same runs hold plain elementwise kernels of known size (one pass over |x|, eleven over 1 GiB, each",
+             "reading and writing that much).  WRITE_SIZE reads their size (scale 1.0); FETCH_SIZE reads half of it (scale 2.0).", ""]
+    for path in sorted(glob.glob(os.path.join(ROOT, "profiles", "hbm_traffic_*.json"))):
+        with open(path) as fh:
+            d = json.load(fh)
+        N, C, H, W, k, S, stride, pad, dil, groups = WORKLOADS[d["workload"]][:10]
+        Ho, Wo = (H + 2 * pad - dil * (k - 1) - 1) // stride + 1, (W + 2 * pad - dil * (k - 1) - 1) // stride + 1
+        esz = {"fp32": 4, "bf16": 2, "fp16": 2}[d["dtype"]]
+        per, _, _ = algorithmic_bytes(N, C, H, W, Ho, Wo, k, S, groups, esz)
+        lines.append("%s, %s (N=%d C=%d %dx%d k=%d scope %dx%d)   [kernel sources at %s]" % (
+            d["workload"], d["dtype"], N, C, H, W, k, S[0], S[1], str(d.get("git_head", ""))[:12]))
+        lines.append("  %-14s %12s %10s %12s %10s %10s %14s" % ("entry point", "FETCH KiB", "x%.1f MB" % d["fetch_scale"], "WRITE KiB", "MB", "total MB", "algorithmic MB"))
+        for key in ("forward", "grad_input", "grad_rotation", "grad_filter"):
+            e = d["entries"].get(key)
+            if not e:
+                continue
+            fm, wm = e["fetch_kib"] * d["fetch_scale"] * 1024 / 1e6, e["write_kib"] * d.get("write_scale", 1.0) * 1024 / 1e6
+            lines.append("  %-14s %12.1f %10.1f %12.1f %10.1f %10.1f %14.1f" % (key, e["fetch_kib"], fm, e["write_kib"], wm, fm + wm, per[key] / 1e6))
+        lines.append("  kernels: " + "; ".join(d["kernels"]))
+        lines.append("")
+    lines += ["(MB = 1e6 bytes; algorithmic = every operand touched once.)  The per-pixel operator with a 5 x 5 scope runs its",
+              "grad filter as two launches of 16 scope cells each, so it reads its operands twice; forward / grad input of the 16-bit",
+              "types write with the default cache policy since the non-temporal 2-byte stores reached memory as partial lines (WRITE_SIZE",
+              "47 % above the tensor's size).  Reads are within a few per cent of the compulsory amount everywhere else: the XCD-aware",
+              "block order keeps halo rows and rotation planes in one L2, and the matrix-core grad filter deals its tiles round-robin",
+              "to the resident workgroups so that neighbours stage neighbouring tiles together."]
+    text = "\n".join(lines) + "\n"
+    with open(os.path.join(ROOT, "profiles", "local_dk_hbm_counters.txt"), "w") as fh:
+        fh.write(text)
+    sys.stdout.write(text)
+
+
 def summarise_profile(a):
     """--profile-from DB: a text summary of a rocprofv3 database (rocpd sqlite, `-d <dir> -o <name>`) of a
     bench.py run: per-kernel durations, per-kernel counter averages when the run was a --pmc run, and for a
@@ -284,12 +327,16 @@ def main():
     ap.add_argument("--traffic-from", nargs=2, metavar=("FETCH_DB", "WRITE_DB"),
                     help="summarise two rocprofv3 counter databases into the tracked traffic table and exit")
     ap.add_argument("--traffic-out", default="", help="where --traffic-from writes (default: profiles/)")
+    ap.add_argument("--traffic-table", action="store_true", help="rewrite profiles/local_dk_hbm_counters.txt from the tracked tables")
     ap.add_argument("--profile-from", default="", metavar="DB",
                     help="summarise a rocprofv3 database of a bench.py run (kernel durations, the step's timeline, counters) and exit")
     ap.add_argument("--profile-out", default="", help="append the --profile-from summary to this file as well")
     a = ap.parse_args()
     if a.traffic_from:
         return summarise_traffic(a)
+    if a.traffic_table:
+        traffic_table(a)
+        return
     if a.profile_from:
         return summarise_profile(a)
     if a.gpus != 1:
