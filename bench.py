@@ -190,8 +190,8 @@ def traffic_table(a):
         Ho, Wo = (H + 2 * pad - dil * (k - 1) - 1) // stride + 1, (W + 2 * pad - dil * (k - 1) - 1) // stride + 1
         esz = {"fp32": 4, "bf16": 2, "fp16": 2}[d["dtype"]]
         per, _, _ = algorithmic_bytes(N, C, H, W, Ho, Wo, k, S, groups, esz)
-        lines.append("%s, %s (N=%d C=%d %dx%d k=%d scope %dx%d)   [kernel sources at %s]" % (
-            d["workload"], d["dtype"], N, C, H, W, k, S[0], S[1], str(d.get("git_head", ""))[:12]))
+        lines.append("%s, %s (N=%d C=%d %dx%d k=%d scope %dx%d)   [kernel sources: sha256 %s]" % (
+            d["workload"], d["dtype"], N, C, H, W, k, S[0], S[1], str(d.get("kernel_source_sha256", ""))[:12]))
         lines.append("  %-14s %12s %10s %12s %10s %10s %14s" % ("entry point", "FETCH KiB", "x%.1f MB" % d["fetch_scale"], "WRITE KiB", "MB", "total MB", "algorithmic MB"))
         for key in ("forward", "grad_input", "grad_rotation", "grad_filter"):
             e = d["entries"].get(key)
