@@ -664,6 +664,317 @@ __global__ __launch_bounds__(BLOCK, BLOCK == kDBlock ? 2 : 1) void deform_grad_c
 }
 
 // ---------------------------------------------------------------------------
+// The channel-interleaved kernels for planes whose padded copy does not fit LDS twice four at a time (wider than
+// 64 columns, or larger than 64 x 64): LDS holds a WINDOW of `wr` rows of the padded planes -- the rows the
+// tile's samples touch, from a block-wide minimum / maximum over the taps that hit the image -- followed by
+// RS + 2 zero positions, where the taps that contribute nothing point.  When the samples span more rows than the
+// window holds, the tile takes several passes over consecutive windows, each sample counted in the pass that holds
+// its two rows: any offsets are served, at one staging per pass and channel tuple.
+// ---------------------------------------------------------------------------
+constexpr int kDWinCh = 4;                                 // interleaved planes (kDeformCh of the host side)
+constexpr int kDWinFwdBlock = 1024, kDWinFwdPass = 4;      // forward: 128 registers per lane suffice
+constexpr int kDWinCoordBlock = 512, kDWinCoordPass = 8;   // coordinate gradients: up to 45 sums per lane
+
+// Block-wide range [lo, hi] of the padded rows that hold the top-left corners of the workgroup's samples
+// (hi < lo: no tap samples the image).  Two barriers; every thread of the workgroup must call it.
+__device__ __forceinline__ void sample_top_rows(const ImgTap (&it)[K9], unsigned hits, int RS, int& lo, int& hi) {
+  __shared__ int s_lo[16], s_hi[16];
+  lo = 1 << 30, hi = -1;
+#pragma unroll
+  for (int t = 0; t < K9; ++t) {
+    if (hits >> t & 1u) {
+      const int pr = it[t].pidx / RS;
+      lo = min(lo, pr);
+      hi = max(hi, pr);
+    }
+  }
+  for (int s = 32; s > 0; s >>= 1) {
+    lo = min(lo, __shfl_xor(lo, s));
+    hi = max(hi, __shfl_xor(hi, s));
+  }
+  if ((threadIdx.x & 63) == 0) {
+    s_lo[threadIdx.x >> 6] = lo;
+    s_hi[threadIdx.x >> 6] = hi;
+  }
+  __syncthreads();
+  for (int w = 0; w < (int)blockDim.x / 64; ++w) {
+    lo = min(lo, s_lo[w]);
+    hi = max(hi, s_hi[w]);
+  }
+  __syncthreads();
+}
+
+// Cooperative load of window rows of CH planes: window row w (w < wr) is padded plane row wlo + w, i.e. plane row
+// wlo + w - 1; rows outside the plane and the columns beside it load zeros, and every position of the window is
+// written, so that a later pass leaves nothing of an earlier one.
+template <typename T, int NPASS, int CH>
+struct WindowStageN {
+  float v[CH][NPASS];
+  __device__ __forceinline__ void load(const T* plane0, size_t step, int live_channels, int H, int W, int shift,
+                                       int wlo, int wr) {
+    const int col = threadIdx.x & ((1 << shift) - 1), sub = threadIdx.x >> shift;
+    const int rpp = (int)blockDim.x >> shift;
+    unsigned so[NPASS];
+#pragma unroll
+    for (int k = 0; k < NPASS; ++k) {
+      const int w = k * rpp + sub, row = wlo + w - 1;
+      so[k] = (col < W && w < wr && row >= 0 && row < H) ? (unsigned)(row * W + col) * (unsigned)sizeof(T) : kOutOfRange;
+    }
+#pragma unroll
+    for (int c = 0; c < CH; ++c) {
+      const bool on = c < live_channels;
+      const rsrc_t r = plane_rsrc(plane0 + (on ? (size_t)c * step : 0), on ? H * W : 0);
+#pragma unroll
+      for (int k = 0; k < NPASS; ++k) v[c][k] = buf_ld(r, so[k], plane0);
+    }
+  }
+  __device__ __forceinline__ void store(float* lds_planes, int W, int shift, int wr) const {
+    static_assert(CH == 4, "16-byte stores");
+    const int col = threadIdx.x & ((1 << shift) - 1), sub = threadIdx.x >> shift;
+    const int rpp = (int)blockDim.x >> shift;
+    const int RS = W + 2;
+#pragma unroll
+    for (int k = 0; k < NPASS; ++k) {
+      const int w = k * rpp + sub;
+      if (w < wr && col + 1 < RS)
+        *reinterpret_cast<float4*>(lds_planes + (w * RS + 1 + col) * CH) = make_float4(v[0][k], v[1][k], v[2][k], v[3][k]);
+    }
+  }
+};
+
+// Descriptors of a pass: element offset (times CH) of each tap's top-left corner inside the window that starts at
+// padded row wlo, or the zero area behind the window for a tap that is not in this pass.
+template <int CH>
+__device__ __forceinline__ void window_taps(const ImgTap (&it)[K9], unsigned hits, int RS, int wlo, int wr, int (&rel)[K9]) {
+#pragma unroll
+  for (int t = 0; t < K9; ++t) {
+    const bool in = (hits >> t & 1u) && it[t].pidx >= wlo * RS && it[t].pidx < (wlo + wr - 1) * RS;
+    rel[t] = (in ? it[t].pidx - wlo * RS : wr * RS) * CH;
+  }
+}
+
+template <typename T, int SH, int SW>
+__global__ __launch_bounds__(kDWinFwdBlock, 1) void deform_forward_chw_kernel(
+    Geo g, const T* __restrict__ x, const T* __restrict__ off, const T* __restrict__ rot,
+    const T* __restrict__ filter, T* __restrict__ out, int ch_per_block, int shift, int wr) {
+  constexpr int CH = kDWinCh, BLOCK = kDWinFwdBlock;
+  using Tb = WideTable<SH, SW>;
+  extern __shared__ __align__(16) float lds[];
+  const int H = g.in_h, W = g.in_w, RS = W + 2;
+  const int WP = wr * RS + RS + 2;    // positions of a buffer: the window, then the zero area
+  float* planes = lds;                // [2][WP][CH]
+  float* tbl = lds + 2 * WP * CH;     // [ch_per_block rounded up to CH][Tb::SIZE]
+
+  const int cpg = g.channel / g.groups;
+  const int out_plane = g.out_h * g.out_w, in_plane = H * W;
+  const BlockId b = decode_block(g, ceil_div(out_plane, BLOCK), ceil_div(cpg, ch_per_block));
+  if (!b.valid) return;
+  const int j0 = b.chunk * ch_per_block;
+  const int nch = min(ch_per_block, cpg - j0);
+  const int nq = ceil_div(nch, CH);
+
+  for (int e = threadIdx.x; e < 2 * WP * CH; e += BLOCK) planes[e] = 0.f;
+  for (int e = nch * Tb::SIZE + threadIdx.x; e < nq * CH * Tb::SIZE; e += BLOCK) tbl[e] = 0.f;
+  stage_wide_tables<T, SH, SW>(tbl, filter, g.channel, b.grp + g.groups * j0, g.groups, nch);
+
+  const int p = b.tile * BLOCK + threadIdx.x;
+  const bool live = p < out_plane;
+  ImgTap it[K9];
+  LiteTap st[K9];
+  unsigned hits = 0;
+  deform_taps<T, SH, SW>(g, off, rot, b.n, b.grp, p, live, RS, it, st, &hits);
+  int lo, hi;
+  sample_top_rows(it, hits, RS, lo, hi);  // (its barriers also end the zero fill)
+  const int npass = hi < lo ? 1 : ceil_div(hi - lo + 1, wr - 1);
+  if (hi < lo) lo = 0;
+
+  const size_t chan0 = (size_t)b.n * g.channel + b.grp + (size_t)g.groups * j0;
+  const T* xp = x + chan0 * in_plane;
+  T* op = out + chan0 * out_plane;
+  const size_t x_step = (size_t)g.groups * in_plane, o_step = (size_t)g.groups * out_plane;
+  const unsigned ooff = live ? (unsigned)p * (unsigned)sizeof(T) : kOutOfRange;
+
+  WindowStageN<T, kDWinFwdPass, CH> stage;
+  for (int k = 0; k < npass; ++k) {
+    const int wlo = lo + k * (wr - 1);
+    int rel[K9];
+    window_taps<CH>(it, hits, RS, wlo, wr, rel);
+    stage.load(xp, x_step, nch, H, W, shift, wlo, wr);
+    __syncthreads();  // the previous pass's reads are done
+    stage.store(planes, W, shift, wr);
+    __syncthreads();
+    for (int jq = 0; jq < nq; ++jq) {
+      if (jq + 1 < nq) stage.load(xp + (size_t)(jq + 1) * CH * x_step, x_step, nch - (jq + 1) * CH, H, W, shift, wlo, wr);
+      const float* pl = planes + (jq & 1) * WP * CH;
+      const float* tb = tbl + jq * CH * Tb::SIZE;
+      float acc[CH];
+#pragma unroll
+      for (int c = 0; c < CH; ++c) acc[c] = 0.f;
+#pragma unroll
+      for (int t = 0; t < K9; ++t) {
+        const CornersN<CH> q = read_corners_n<CH>(pl, rel[t], RS);
+#pragma unroll
+        for (int c = 0; c < CH; ++c) {
+          const float top = fmaf(it[t].lw, q.b[c] - q.a[c], q.a[c]), bot = fmaf(it[t].lw, q.d[c] - q.c[c], q.c[c]);
+          const float v = fmaf(it[t].lh, bot - top, top);
+          const float4 w = *reinterpret_cast<const float4*>(tb + c * Tb::SIZE + st[t].cell);
+          acc[c] = fmaf(v, lite_weight(st[t], w), acc[c]);
+        }
+      }
+#pragma unroll
+      for (int c = 0; c < CH; ++c) {
+        const rsrc_t ro = plane_rsrc(op + (size_t)(jq * CH + c) * o_step, jq * CH + c < nch ? out_plane : 0);
+        if (k > 0) acc[c] += buf_ld(ro, ooff, out);  // the taps of the earlier passes
+        buf_st(ro, ooff, acc[c], out);
+      }
+      if (jq + 1 < nq) stage.store(planes + ((jq + 1) & 1) * WP * CH, W, shift, wr);
+      __syncthreads();
+    }
+  }
+}
+
+// MODE as in deform_grad_coord_ch_kernel.  A tap's sums collect in the one pass that holds its sample.
+template <typename T, int SH, int SW, int MODE>
+__global__ __launch_bounds__(kDWinCoordBlock, 1) void deform_grad_coord_chw_kernel(
+    Geo g, const T* __restrict__ gout, const T* __restrict__ x, const T* __restrict__ off,
+    const T* __restrict__ rot, const T* __restrict__ filter, float* __restrict__ partial,
+    int ch_per_block, int shift, int wr, float* __restrict__ partial_off) {
+  constexpr bool ROTATION = MODE != 0, OFFSET = MODE != 1;
+  constexpr int CH = kDWinCh, BLOCK = kDWinCoordBlock;
+  using Tb = WideTable<SH, SW>;
+  extern __shared__ __align__(16) float lds[];
+  const int H = g.in_h, W = g.in_w, RS = W + 2;
+  const int WP = wr * RS + RS + 2;
+  float* planes = lds;               // [2][WP][CH]
+  float* tbl = lds + 2 * WP * CH;    // [ch_per_block rounded up to CH][Tb::SIZE]
+
+  const int cpg = g.channel / g.groups;
+  const int out_plane = g.out_h * g.out_w, in_plane = H * W;
+  const int chunks = ceil_div(cpg, ch_per_block);
+  const BlockId b = decode_block(g, ceil_div(out_plane, BLOCK), chunks);
+  if (!b.valid) return;
+  const int j0 = b.chunk * ch_per_block;
+  const int nch = min(ch_per_block, cpg - j0);
+  const int nq = ceil_div(nch, CH);
+
+  for (int e = threadIdx.x; e < 2 * WP * CH; e += BLOCK) planes[e] = 0.f;
+  for (int e = nch * Tb::SIZE + threadIdx.x; e < nq * CH * Tb::SIZE; e += BLOCK) tbl[e] = 0.f;
+  stage_wide_tables<T, SH, SW>(tbl, filter, g.channel, b.grp + g.groups * j0, g.groups, nch);
+
+  const int p = b.tile * BLOCK + threadIdx.x;
+  const bool live = p < out_plane;
+  ImgTap it[K9];
+  LiteTap st[K9];
+  unsigned hits = 0;
+  deform_taps<T, SH, SW>(g, off, rot, b.n, b.grp, p, live, RS, it, st, &hits);
+  int lo, hi;
+  sample_top_rows(it, hits, RS, lo, hi);
+  const int npass = hi < lo ? 1 : ceil_div(hi - lo + 1, wr - 1);
+  if (hi < lo) lo = 0;
+
+  const size_t chan0 = (size_t)b.n * g.channel + b.grp + (size_t)g.groups * j0;
+  const T* xp = x + chan0 * in_plane;
+  const T* gp = gout + chan0 * out_plane;
+  const size_t x_step = (size_t)g.groups * in_plane, g_step = (size_t)g.groups * out_plane;
+  const unsigned goff = live ? (unsigned)p * (unsigned)sizeof(T) : kOutOfRange;
+
+  float s0[K9], s1[K9], s2[K9];                    // rotation: sums of sample * gout * {b, c, d}
+  float o0[OFFSET ? K9 : 1], o1[OFFSET ? K9 : 1];  // offset: sums of d sample / d{h, w} * gout * B
+#pragma unroll
+  for (int t = 0; t < K9; ++t) s0[t] = s1[t] = s2[t] = 0.f;
+#pragma unroll
+  for (int t = 0; t < (OFFSET ? K9 : 1); ++t) o0[t] = o1[t] = 0.f;
+
+  WindowStageN<T, kDWinCoordPass, CH> stage;
+  for (int k = 0; k < npass; ++k) {
+    const int wlo = lo + k * (wr - 1);
+    int rel[K9];
+    window_taps<CH>(it, hits, RS, wlo, wr, rel);
+    float gv[CH], gv_next[CH];
+    stage.load(xp, x_step, nch, H, W, shift, wlo, wr);
+#pragma unroll
+    for (int c = 0; c < CH; ++c) gv[c] = buf_ld(plane_rsrc(gp + (size_t)c * g_step, c < nch ? out_plane : 0), goff, gout);
+    __syncthreads();
+    stage.store(planes, W, shift, wr);
+    __syncthreads();
+    for (int jq = 0; jq < nq; ++jq) {
+#pragma unroll
+      for (int c = 0; c < CH; ++c) gv_next[c] = 0.f;
+      if (jq + 1 < nq) {
+        const int jn = (jq + 1) * CH;
+        stage.load(xp + (size_t)jn * x_step, x_step, nch - jn, H, W, shift, wlo, wr);
+#pragma unroll
+        for (int c = 0; c < CH; ++c)
+          gv_next[c] = buf_ld(plane_rsrc(gp + (size_t)(jn + c) * g_step, jn + c < nch ? out_plane : 0), goff, gout);
+      }
+      const float* pl = planes + (jq & 1) * WP * CH;
+      const float* tb = tbl + jq * CH * Tb::SIZE;
+#pragma unroll
+      for (int t = 0; t < K9; ++t) {
+        const CornersN<CH> cq = read_corners_n<CH>(pl, rel[t], RS);
+#pragma unroll
+        for (int c = 0; c < CH; ++c) {
+          const float4 q = *reinterpret_cast<const float4*>(tb + c * Tb::SIZE + st[t].cell);
+          if constexpr (ROTATION) {
+            const float top = fmaf(it[t].lw, cq.b[c] - cq.a[c], cq.a[c]), bot = fmaf(it[t].lw, cq.d[c] - cq.c[c], cq.c[c]);
+            const float ps = fmaf(it[t].lh, bot - top, top) * gv[c];
+            s0[t] = fmaf(ps, q.y, s0[t]);
+            s1[t] = fmaf(ps, q.z, s1[t]);
+            s2[t] = fmaf(ps, q.w, s2[t]);
+          }
+          if constexpr (OFFSET) {
+            const float gw = gv[c] * lite_weight(st[t], q);
+            const float ca = cq.c[c] - cq.a[c], ba = cq.b[c] - cq.a[c];
+            const float dh = fmaf(it[t].lw, (cq.d[c] - cq.b[c]) - ca, ca);
+            const float dw = fmaf(it[t].lh, (cq.d[c] - cq.c[c]) - ba, ba);
+            o0[t] = fmaf(dh, gw, o0[t]);
+            o1[t] = fmaf(dw, gw, o1[t]);
+          }
+        }
+        // the tap's sums are complete here: keeps the arithmetic of all nine taps from sinking below the plane store
+        if constexpr (ROTATION) asm volatile("" : "+v"(s0[t]), "+v"(s1[t]), "+v"(s2[t])::"memory");
+        if constexpr (OFFSET) asm volatile("" : "+v"(o0[t]), "+v"(o1[t])::"memory");
+        __builtin_amdgcn_sched_barrier(0);
+      }
+#pragma unroll
+      for (int c = 0; c < CH; ++c) gv[c] = gv_next[c];
+      if (jq + 1 < nq) stage.store(planes + ((jq + 1) & 1) * WP * CH, W, shift, wr);
+      __syncthreads();
+    }
+  }
+
+  if (live) {
+    if constexpr (ROTATION) {
+      float* dst = partial + (((size_t)b.chunk * g.batch * g.groups + (size_t)(b.n * g.groups + b.grp)) * (K9 * 2)) * out_plane + p;
+      const T* rp = rot + (size_t)(b.n * g.groups + b.grp) * (K9 * 2) * out_plane + p;
+#pragma unroll
+      for (int t = 0; t < K9; ++t) {
+        float dh = fmaf(st[t].lw, s2[t], s1[t]);
+        float dw = fmaf(st[t].lh, s2[t], s0[t]);
+        if (g.clip_mode != kClipNone) {  // a clamped offset has no gradient
+          bool open_h, open_w;
+          scope_coord<float>(g, t / 3, ld(rp + (size_t)(2 * t) * out_plane), g.centre_h, &open_h);
+          scope_coord<float>(g, t % 3, ld(rp + (size_t)(2 * t + 1) * out_plane), g.centre_w, &open_w);
+          dh = open_h ? dh : 0.f;
+          dw = open_w ? dw : 0.f;
+        }
+        dst[(size_t)(2 * t) * out_plane] = dh;
+        dst[(size_t)(2 * t + 1) * out_plane] = dw;
+      }
+    }
+    if constexpr (OFFSET) {
+      float* base = MODE == 2 ? partial_off : partial;
+      float* dst = base + ((((size_t)b.grp * chunks + b.chunk) * g.batch + (size_t)b.n) * (K9 * 2)) * out_plane + p;
+#pragma unroll
+      for (int t = 0; t < K9; ++t) {
+        dst[(size_t)(2 * t) * out_plane] = o0[t];
+        dst[(size_t)(2 * t + 1) * out_plane] = o1[t];
+      }
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------
 // grad input (K.cu:704-795): every (pixel, tap, channel) adds gout * B(Wt[c]) * corner weight to
 // the four input elements around its sample -- a scatter with data-dependent targets, done by
 // the reference with global float atomics.  LDS float atomics are slow on gfx950 (about 190 clk
@@ -1728,6 +2039,7 @@ struct DeformPlan {
   int tiles;   // pixel tiles
   int block;   // threads of a workgroup
   int tile_pix;  // output pixels of a tile (<= block)
+  int wr;        // rows of the LDS window (the row-window forms)
   size_t lds;
 };
 
@@ -1776,6 +2088,7 @@ DeformPlan deform_plan(const Geo& g, int table_floats, int planes, int block, in
 // Plan of the kernels that interleave kDeformCh channel planes in LDS; ok only when the two
 // interleaved buffers, the tables and a four-pass register stage fit.
 constexpr int kDeformCh = 4;
+static_assert(kDeformCh == kDWinCh, "the row-window kernels interleave as many planes");
 constexpr int kDBigBlock = 1024;
 constexpr int kDBigBlocksPerCu = 1;
 constexpr long kDBigLds = 150 * 1024;
@@ -1813,6 +2126,30 @@ DeformPlan deform_plan_wide(const Geo& g, int table_floats) {
   return deform_plan(g, table_floats, 2, kDWideBlock, 1, kDBigLds, 1 << 30, kDWidePasses);
 }
 
+// The same planes on the channel-interleaved kernels with a row window in LDS: two buffers of `wr` rows of four
+// interleaved planes beside the tables of at most 64 channels.  ok only when the window holds the rows a tile's own
+// taps span plus a margin for the offsets (otherwise every tile would take several passes and the one-plane
+// kernels above are the better choice).
+DeformPlan deform_plan_chw(const Geo& g, int table_floats, int block, int npass) {
+  DeformPlan d{};
+  d.ok = false;
+  if (path_disabled(kNoDeformCh) || path_disabled(kNoDeformWindow)) return d;
+  // the family's limits, the row mapping and the channel chunks (tables in at most 26 KB)
+  d = deform_plan(g, table_floats, 0, block, 1, 26 * 1024, 1 << 30, 1 << 30);
+  if (!d.ok) return d;
+  d.ok = false;
+  const int RS = g.in_w + 2, rpp = block >> d.shift;
+  const long table_bytes = (long)(d.per + kDeformCh - 1) * table_floats * 4;
+  const long positions = (kDBigLds - table_bytes) / 2 / (kDeformCh * 4) - (RS + 2);
+  const long wr = std::min<long>({(long)g.in_h + 2, positions / RS, (long)npass * rpp});
+  const long own = (long)(ceil_div(block, g.out_w) + 1) * g.stride_h + 2L * g.dil_h + 2;  // rows without offsets
+  if (wr < std::min<long>(g.in_h + 2, own + 8)) return d;
+  d.wr = (int)wr;
+  d.lds = (size_t)(2 * (wr * RS + RS + 2) * kDeformCh * 4 + table_bytes);
+  d.ok = true;
+  return d;
+}
+
 template <typename T, int SH, int SW>
 bool run_deform_forward(const Geo& g, const T* x, const T* off, const T* rot, const T* filter, T* out,
                         hipStream_t stream) {
@@ -1832,6 +2169,14 @@ bool run_deform_forward(const Geo& g, const T* x, const T* off, const T* rot, co
   }
   const DeformPlan d = deform_plan(g, WideTable<SH, SW>::SIZE, 2, kDBlock, 4);
   if (!d.ok) {
+    const DeformPlan cw = deform_plan_chw(g, WideTable<SH, SW>::SIZE, kDWinFwdBlock, kDWinFwdPass);
+    if (cw.ok) {
+      auto kernel = deform_forward_chw_kernel<T, SH, SW>;
+      if (!allow_max_dynamic_lds(reinterpret_cast<const void*>(kernel))) return false;
+      const unsigned cgrid = (unsigned)xcd_grid_size((long)cw.tiles * cw.chunks * g.batch * g.groups);
+      kernel<<<cgrid, kDWinFwdBlock, cw.lds, stream>>>(g, x, off, rot, filter, out, cw.per, cw.shift, cw.wr);
+      return true;
+    }
     const DeformPlan w = deform_plan_wide(g, WideTable<SH, SW>::SIZE);
     if (!w.ok) return false;
     auto kernel = deform_forward_kernel<T, SH, SW, kDWidePasses, kDWideBlock>;
@@ -1857,10 +2202,19 @@ bool run_deform_grad_coord(const Geo& g, bool rotation, const T* gout, const T* 
   const DeformPlan d4 = deform_plan_ch(g, WideTable<SH, SW>::SIZE, 3);
   DeformPlan d = d4.ok ? d4 : deform_plan(g, WideTable<SH, SW>::SIZE, 2, kDBlock, rotation ? 2 : 3);
   const bool wide = !d.ok;
-  if (wide) d = deform_plan_wide(g, WideTable<SH, SW>::SIZE);
+  bool window = false;
+  if (wide) {
+    d = deform_plan_chw(g, WideTable<SH, SW>::SIZE, kDWinCoordBlock, kDWinCoordPass);
+    window = d.ok;
+    if (!window) d = deform_plan_wide(g, WideTable<SH, SW>::SIZE);
+  }
   if (!d.ok) return false;
   const unsigned grid = (unsigned)xcd_grid_size((long)d.tiles * d.chunks * g.batch * g.groups);
-  if (wide) {
+  if (window) {
+    auto kernel = rotation ? deform_grad_coord_chw_kernel<T, SH, SW, 1> : deform_grad_coord_chw_kernel<T, SH, SW, 0>;
+    if (!allow_max_dynamic_lds(reinterpret_cast<const void*>(kernel))) return false;
+    kernel<<<grid, kDWinCoordBlock, d.lds, stream>>>(g, gout, x, off, rot, filter, ws, d.per, d.shift, d.wr, nullptr);
+  } else if (wide) {
     auto kernel = rotation ? deform_grad_coord_kernel<T, SH, SW, kDWidePasses, true, kDWideBlock>
                            : deform_grad_coord_kernel<T, SH, SW, kDWidePasses, false, kDWideBlock>;
     if (!allow_max_dynamic_lds(reinterpret_cast<const void*>(kernel))) return false;
@@ -1915,18 +2269,32 @@ DeformPlan coords_plan(const Geo& g, int table_floats) {
   return d;
 }
 
+// ... and its row-window form for the planes that neither of those takes: *d is that plan when it applies
+bool coords_window(const Geo& g, int table_floats, DeformPlan* d) {
+  // only where no other channel-interleaved or one-plane 256-thread form serves the shape (as in run_deform_grad_coord)
+  if (deform_plan_ch(g, table_floats, 3).ok || deform_plan(g, table_floats, 2, kDBlock, 2).ok) return false;
+  const DeformPlan w = deform_plan_chw(g, table_floats, kDWinCoordBlock, kDWinCoordPass);
+  if (w.ok) *d = w;
+  return w.ok;
+}
+
 // Offset and rotation gradient from one pass (MODE 2 of the channel-interleaved kernel in 256-thread workgroups: its
 // 45 sums fit their register budget, not that of the 1024-thread form); false where that form does not apply.
 // Workspace: the rotation partials, then the offset partials (the same number of floats).
 template <typename T, int SH, int SW>
 bool run_deform_grad_coords(const Geo& g, const T* gout, const T* x, const T* off, const T* rot, const T* filter,
                             T* goff, T* grot, float* ws, hipStream_t stream) {
-  const DeformPlan d = coords_plan(g, WideTable<SH, SW>::SIZE);
+  DeformPlan d = coords_plan(g, WideTable<SH, SW>::SIZE);
+  const bool window = !d.ok && coords_window(g, WideTable<SH, SW>::SIZE, &d);
   if (!d.ok) return false;
   const int plane18 = 18 * g.out_h * g.out_w;
   float* ws_off = ws + (size_t)d.chunks * g.groups * g.batch * plane18;
   const unsigned grid = (unsigned)xcd_grid_size((long)d.tiles * d.chunks * g.batch * g.groups);
-  if (d.block == kDBlock) {
+  if (window) {
+    auto kernel = deform_grad_coord_chw_kernel<T, SH, SW, 2>;
+    if (!allow_max_dynamic_lds(reinterpret_cast<const void*>(kernel))) return false;
+    kernel<<<grid, kDWinCoordBlock, d.lds, stream>>>(g, gout, x, off, rot, filter, ws, d.per, d.shift, d.wr, ws_off);
+  } else if (d.block == kDBlock) {
     deform_grad_coord_ch_kernel<T, SH, SW, 4, 2, kDeformCh><<<grid, kDBlock, d.lds, stream>>>(g, gout, x, off, rot, filter, ws, d.per, d.shift, d.tile_pix, ws_off);
   } else {
     auto kernel = deform_grad_coord_ch_kernel<T, SH, SW, 8, 2, kDeformCh, kDCoordsBlock>;
@@ -2155,6 +2523,7 @@ size_t fast_deform_grad_coord_workspace(const Geo& g, bool rotation) {
   const int table = g.scope_h == 3 ? WideTable<3, 3>::SIZE : g.scope_h == 4 ? WideTable<4, 4>::SIZE : WideTable<5, 5>::SIZE;
   const DeformPlan d4 = deform_plan_ch(g, table, 3);
   DeformPlan d = d4.ok ? d4 : deform_plan(g, table, 2, kDBlock, rotation ? 2 : 3);
+  if (!d.ok) d = deform_plan_chw(g, table, kDWinCoordBlock, kDWinCoordPass);
   if (!d.ok) d = deform_plan_wide(g, table);
   if (!d.ok) return 0;
   // both lay out chunks * groups * batch planes of 18 * out pixels
@@ -2163,7 +2532,8 @@ size_t fast_deform_grad_coord_workspace(const Geo& g, bool rotation) {
 
 size_t fast_deform_grad_coords_workspace(const Geo& g) {
   const int table = g.scope_h == 3 ? WideTable<3, 3>::SIZE : g.scope_h == 4 ? WideTable<4, 4>::SIZE : WideTable<5, 5>::SIZE;
-  const DeformPlan d = coords_plan(g, table);
+  DeformPlan d = coords_plan(g, table);
+  if (!d.ok) coords_window(g, table, &d);
   if (!d.ok) return 0;
   return 2 * (size_t)d.chunks * g.groups * g.batch * 18 * g.out_h * g.out_w * sizeof(float);
 }

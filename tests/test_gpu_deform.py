@@ -40,6 +40,8 @@ CASES = [
     (1, 3, 100, 30, 3, (5, 5), 1, 1, 1, 1, 1.0, 2.5),     # narrow but taller than the 256-thread staging covers; scope 5
     (1, 20, 60, 40, 3, (4, 4), 1, 1, 1, 2, 0.7, 10.0),    # row-window grad filter: offsets of ten rows spread a tile's samples over three windows of 24 rows; two channel blocks, the second partial
     (2, 33, 56, 56, 3, (5, 5), 1, 1, 1, 1, 1.0, 2.0),     # row-window grad filter, scope 5 (two launches of 16 cells), three channel blocks
+    (1, 6, 120, 100, 3, (4, 4), 1, 1, 1, 1, 0.7, 15.0),   # row-window channel-interleaved kernels (100 columns): offsets of fifteen rows, four windows of 32 rows per tile; two channel tuples
+    (2, 9, 70, 96, 3, (3, 3), 1, 1, 1, 3, 0.6, 2.0),      # the same kernels in one pass: three groups of three channels, scope 3
 ]
 NAMES = ("forward", "grad input", "grad offset", "grad rotation", "grad filter")
 
@@ -225,16 +227,14 @@ def test_config4_properties_at_full_size():
 
 @pytest.mark.parametrize("switch,case", [("DK_NO_DEFORM_CH", CASES[0]), ("DK_NO_DEFORM_MFMA", CASES[0]),
                                          ("DK_NO_DEFORM_CH_BIG", CASES[7]), ("DK_NO_DEFORM_WINDOW", CASES[13]),
-                                         ("DK_NO_DEFORM_WINDOW", CASES[20])])
+                                         ("DK_NO_DEFORM_WINDOW", CASES[20]), ("DK_NO_DEFORM_WINDOW", CASES[16]),
+                                         ("DK_NO_DEFORM_WINDOW", CASES[22])])
 def test_one_plane_kernels_on_a_shape_the_newer_ones_cover(switch_off, switch, case):
     """Without the channel-interleaved kernels (those for small planes and those for large ones) / the
     matrix-core grad filter the one-plane kernels serve the shape."""
     switch_off(switch)
     inputs, got = _run(case, torch.float32)
-    o32, o64 = _oracle(inputs, np.float32), _oracle(inputs, np.float64)
-    assert rel_err(got[0], o32[0]) < 1e-5
-    for i in range(1, 5):
-        assert rel_err(got[i], o64[i]) < 1e-4, NAMES[i]
+    assert_fp32_parity(got, _oracle(inputs, np.float32), _oracle(inputs, np.float64))
 
 
 def test_generic_kernels_on_a_shape_the_tuned_ones_cover(switch_off):
