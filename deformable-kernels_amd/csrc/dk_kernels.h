@@ -36,6 +36,7 @@ enum TestSwitch : unsigned {
   kForcePixelLanes = 1u << 17,  // DK_FORCE_PIXEL_LANES  ... wherever it applies, not only where it is the faster kernel
   kNoOffsetWgrad16 = 1u << 19,  // DK_NO_OFFSET_WGRAD16  the offset branch's weight gradient on 16-bit matrix instructions (the fp32 matrix-instruction kernel at stride 1, nothing at stride 2)
   kNoDeformWindow = 1u << 20,   // DK_NO_DEFORM_WINDOW   the row-window form of the matrix-core deformable grad filter (the dense register kernel runs instead)
+  kForceWin2 = 1u << 21,        // DK_FORCE_WIN2         the rows-and-columns window form of that grad filter also where the row-window form applies
   kNoOffsetPairs = 1u << 18,    // DK_NO_OFFSET_PAIRS    the offset branch's convolution on float32 tensors as bfloat16 pairs (the fp32 matrix-instruction forward runs instead, the other passes are not offered)
 };
 unsigned test_switches();  // dk_api.hip

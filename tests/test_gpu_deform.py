@@ -228,10 +228,13 @@ def test_config4_properties_at_full_size():
 @pytest.mark.parametrize("switch,case", [("DK_NO_DEFORM_CH", CASES[0]), ("DK_NO_DEFORM_MFMA", CASES[0]),
                                          ("DK_NO_DEFORM_CH_BIG", CASES[7]), ("DK_NO_DEFORM_WINDOW", CASES[13]),
                                          ("DK_NO_DEFORM_WINDOW", CASES[20]), ("DK_NO_DEFORM_WINDOW", CASES[16]),
-                                         ("DK_NO_DEFORM_WINDOW", CASES[22])])
+                                         ("DK_NO_DEFORM_WINDOW", CASES[22]), ("DK_FORCE_WIN2", CASES[13]),
+                                         ("DK_FORCE_WIN2", CASES[20]), ("DK_FORCE_WIN2", CASES[21]),
+                                         ("DK_FORCE_WIN2", CASES[9])])
 def test_one_plane_kernels_on_a_shape_the_newer_ones_cover(switch_off, switch, case):
     """Without the channel-interleaved kernels (those for small planes and those for large ones) / the
-    matrix-core grad filter the one-plane kernels serve the shape."""
+    matrix-core grad filter / the row-window forms, the one-plane kernels serve the shape; and the grad filter with
+    a window in rows and columns on shapes that its row-window form takes by default."""
     switch_off(switch)
     inputs, got = _run(case, torch.float32)
     assert_fp32_parity(got, _oracle(inputs, np.float32), _oracle(inputs, np.float64))
