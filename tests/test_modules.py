@@ -77,7 +77,7 @@ def test_hooks_on_the_offset_branch_convolution_fire():
 
 def test_descriptor_structs_have_the_library_s_size():
     """The descriptor structs are declared three times: in include/dk_hip.h (what the library is compiled
-    from), in the ctypes loader, and in the binding INTEGRATION.md shows a maintainer of the reference.  The
+    from), in the ctypes loader, and in the binding that the integration guide shows a maintainer of the reference.  The
     library reports its sizeof() for each; the loader's and the documented declaration must agree with it
     (a struct that is shorter than the library's is read past its end)."""
     import ctypes
@@ -89,11 +89,11 @@ def test_descriptor_structs_have_the_library_s_size():
     assert ctypes.sizeof(_lib.ConvDesc) == L.dk_conv_desc_size() == 19 * 4 + 4
     assert ctypes.sizeof(_lib.NdDesc) == L.dk_nd_desc_size()
     assert ctypes.sizeof(_lib.OffsetConvDesc) == L.dk_offset_conv_desc_size()
-    # the struct as INTEGRATION.md declares it: take the class statement out of the document and build it
+    # the struct as the integration guide declares it: take the class statement out of the document and build it
     root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
     doc = open(os.path.join(root, "INTEGRATION.md")).read()
     m = re.search(r"^class ConvDesc\(ctypes\.Structure\):.*?\n(?=\nlib = )", doc, re.S | re.M)
-    assert m, "INTEGRATION.md no longer shows the ConvDesc declaration"
+    assert m, "the integration guide no longer shows the ConvDesc declaration"
     scope = {"ctypes": ctypes}
     exec(m.group(0), scope)
     documented = scope["ConvDesc"]
