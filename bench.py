@@ -521,7 +521,7 @@ def main():
     if a.dtype == "fp32" and a.layout == "nchw":
         result["arithmetic"] = {
             "tensors_and_sums": "f32",
-            "forward, grad_input": "weights formed on v_mfma_f32_32x32x16_f16 from fp16 (hi, lo) pairs of both operands, "
+            "forward, grad_input": "weights formed on v_mfma_f32_16x16x32_f16 from fp16 (hi, lo) pairs of both operands, "
                                    "three products, f32 sums: 2e-7 of the result's scale; the 9 multiply-adds per output in f32",
             "grad_filter": "v_mfma_f32_16x16x16_bf16 on bfloat16 (hi, lo) pairs of both operands, three products, f32 sums: "
                            "5e-6 of the largest element (f32 matrix instructions: 2.4e-7)",
