@@ -191,6 +191,32 @@ __device__ __forceinline__ float buf_ld(rsrc_t r, unsigned byte_off, const bf16_
   const unsigned short b = __builtin_amdgcn_raw_buffer_load_b16(r, (int)byte_off, 0, 0);
   return __uint_as_float(static_cast<uint32_t>(b) << 16);
 }
+// Four consecutive elements at a byte offset of a buffer resource, as stored (converted when they are used: a
+// conversion next to the load would wait for it).
+typedef unsigned nhwc_u4 __attribute__((ext_vector_type(4)));
+typedef unsigned nhwc_u2 __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ nhwc_u4 raw_ld4(rsrc_t r, unsigned off, const float*) { return __builtin_amdgcn_raw_buffer_load_b128(r, (int)off, 0, 0); }
+__device__ __forceinline__ nhwc_u2 raw_ld4(rsrc_t r, unsigned off, const __half*) { return __builtin_amdgcn_raw_buffer_load_b64(r, (int)off, 0, 0); }
+__device__ __forceinline__ nhwc_u2 raw_ld4(rsrc_t r, unsigned off, const bf16_t*) { return __builtin_amdgcn_raw_buffer_load_b64(r, (int)off, 0, 0); }
+__device__ __forceinline__ void raw_cvt4(nhwc_u4 v, float (&f)[4], const float*) {
+  const unsigned u[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+  for (int i = 0; i < 4; ++i) f[i] = __uint_as_float(u[i]);
+}
+__device__ __forceinline__ void raw_cvt4(nhwc_u2 v, float (&f)[4], const __half*) {
+  const unsigned u[2] = {v.x, v.y};
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    f[2 * i] = static_cast<float>(__builtin_bit_cast(_Float16, (unsigned short)(u[i] & 0xffffu)));
+    f[2 * i + 1] = static_cast<float>(__builtin_bit_cast(_Float16, (unsigned short)(u[i] >> 16)));
+  }
+}
+__device__ __forceinline__ void raw_cvt4(nhwc_u2 v, float (&f)[4], const bf16_t*) {
+  const unsigned u[2] = {v.x, v.y};
+#pragma unroll
+  for (int i = 0; i < 2; ++i) f[2 * i] = __uint_as_float(u[i] << 16), f[2 * i + 1] = __uint_as_float(u[i] & 0xffff0000u);
+}
+
 // The same with a scalar part of the address.  The range check compares the lane's offset with the buffer's
 // size less the scalar part, so the descriptor must cover every position the scalar part selects.
 __device__ __forceinline__ float buf_ld2(rsrc_t r, unsigned lane_off, int scalar_off, const float*) {

@@ -37,6 +37,7 @@ enum TestSwitch : unsigned {
   kNoOffsetWgrad16 = 1u << 19,  // DK_NO_OFFSET_WGRAD16  the offset branch's weight gradient on 16-bit matrix instructions (the fp32 matrix-instruction kernel at stride 1, nothing at stride 2)
   kNoDeformWindow = 1u << 20,   // DK_NO_DEFORM_WINDOW   the row-window form of the matrix-core deformable grad filter (the dense register kernel runs instead)
   kForceWin2 = 1u << 21,        // DK_FORCE_WIN2         the rows-and-columns window form of that grad filter also where the row-window form applies
+  kNoNhwcStaged = 1u << 22,     // DK_NO_NHWC_STAGED     the channels-last kernels that stage planar tiles in LDS / contract 32 channels per matrix instruction (the kernels named under DK_NO_NHWC_MFMA run instead)
   kNoOffsetPairs = 1u << 18,    // DK_NO_OFFSET_PAIRS    the offset branch's convolution on float32 tensors as bfloat16 pairs (the fp32 matrix-instruction forward runs instead, the other passes are not offered)
 };
 unsigned test_switches();  // dk_api.hip
@@ -173,6 +174,12 @@ size_t offset_wgrad16_workspace(int batch, int cin, int cout, int h, int w, int 
 template <typename T>
 bool offset_wgrad16(int batch, int cin, int cout, int h, int w, int stride, const T* x, const T* gout, T* gweight,
                     void* ws, hipStream_t stream);
+
+// dk_local_fast.hip: the matrix-core grad filter on channels-last tensors (false / workspace 0: not covered)
+size_t fast_local_grad_filter_cl_workspace(const Geo& g);
+template <typename T>
+bool fast_local_grad_filter_cl(const Geo& g, const T* gout, const T* x, const T* rot, T* gfilter, void* ws,
+                               hipStream_t stream);
 
 // dk_local_nhwc.hip: the local operator on channels-last tensors, all dtypes, any geometry whose tables fit LDS
 bool nhwc_supported(const Geo& g, int dtype);

@@ -1053,7 +1053,11 @@ __device__ __forceinline__ float hat(float d) { return __builtin_amdgcn_fmed3f(1
 // 12 more vector ALU instructions per tap for the split of P.  The dropped Al Pl and the rounding
 // of the lo parts leave a relative error of about 2^-16 per product -- the filter gradient is held
 // to 1e-4 of its largest element and sums thousands of products of either sign.
-template <typename T, int SH, int SW, int CELL0, int NX, bool S2, bool BF = false, bool SPLIT = false>
+// CL: channels-last tensors (x and gout as [image][pixel][channel], rotation as [image][pixel][tap][2];
+// one group).  Only the staging differs: a thread loads four consecutive channels of a pixel (the unit's
+// sixteen channels are 64 contiguous bytes per pixel) and stores them into the same channel-major tiles
+// in LDS, so the products run as for planar tensors.
+template <typename T, int SH, int SW, int CELL0, int NX, bool S2, bool BF = false, bool SPLIT = false, bool CL = false>
 __global__ __launch_bounds__(kMfBlock, 4) void local_grad_filter_mfma_kernel(
     Geo g, const T* __restrict__ gout, const T* __restrict__ x, const T* __restrict__ rot,
     float* __restrict__ partial, int tiles, int nwg, int csplits, int pitch_x, int th) {
@@ -1127,6 +1131,10 @@ __global__ __launch_bounds__(kMfBlock, 4) void local_grad_filter_mfma_kernel(
   const int pix = threadIdx.x % kMfPix;                                 // pixel whose coordinates this thread stages
   const int tapq = __builtin_amdgcn_readfirstlane(threadIdx.x / kMfPix);  // ... for taps tapq + 4 k
   float r_rot[2 * kTapsT], r_x[kChW][NX], r_g[kChW][kMfPix / 64];
+  // CL: thread (pixel slot cl_p, channel quad cl_q) stages four channels of NX / 2 input pixels and of one gout pixel
+  static_assert(!CL || (!S2 && NX % 2 == 0 && kMfBlock == 4 * kMfPix), "channels-last staging: four threads per pixel");
+  const int cl_p = threadIdx.x >> 2, cl_q = threadIdx.x & 3;
+  typename std::conditional<sizeof(T) == 4, nhwc_u4, nhwc_u2>::type c_x[NX / 2], c_g;
   auto issue_loads = [&](int item, int cbi, bool with_rot) {
     const int cb = cb_lo + cbi;
     const int n = item / tiles, p0 = (item % tiles) * tile_pix;
@@ -1135,6 +1143,17 @@ __global__ __launch_bounds__(kMfBlock, 4) void local_grad_filter_mfma_kernel(
     const int x0 = S2 ? (2 * (item % tiles) * th - 1) * W - 1 : p0 + lo;
     if (with_rot) {
       const int p = p0 + pix;
+      if constexpr (CL) {
+        const rsrc_t rr = plane_rsrc(rot + (size_t)n * (K * 2) * out_plane, K * 2 * out_plane);
+        const unsigned ro = p < out_plane ? (unsigned)(p * (K * 2)) * (unsigned)sizeof(T) : kOutOfRange;
+#pragma unroll
+        for (int k = 0; k < kTapsT; ++k) {
+          const int t = tapq + (kMfBlock / kMfPix) * k;
+          const unsigned o = t < K ? ro + (unsigned)(2 * t) * (unsigned)sizeof(T) : kOutOfRange;
+          r_rot[2 * k] = buf_ld(rr, o, rot);
+          r_rot[2 * k + 1] = buf_ld(rr, o + (unsigned)sizeof(T), rot);
+        }
+      } else {
       const rsrc_t rr = plane_rsrc(rot + (size_t)(n * g.groups + grp) * (K * 2) * out_plane, K * 2 * out_plane);
       const unsigned ro = p < out_plane ? (unsigned)p * (unsigned)sizeof(T) : kOutOfRange;
 #pragma unroll
@@ -1144,6 +1163,23 @@ __global__ __launch_bounds__(kMfBlock, 4) void local_grad_filter_mfma_kernel(
         r_rot[2 * k] = buf_ld(rr, o, rot);
         r_rot[2 * k + 1] = buf_ld(rr, o + (unsigned)out_plane * (unsigned)sizeof(T), rot);
       }
+      }
+    }
+    if constexpr (CL) {
+      // one image's pixels; a quad past the last channel, an element before the plane: zeros (the host
+      // admits channel counts that are a multiple of 4 only, so a quad is inside or outside as a whole)
+      const int C = g.channel;
+      const rsrc_t rx = plane_rsrc(x + (size_t)n * in_plane * C, in_plane * C);
+      const rsrc_t rg = plane_rsrc(gout + (size_t)n * out_plane * C, out_plane * C);
+      const int c4 = cb * kMfCh + 4 * cl_q;
+      const unsigned co = c4 < C ? (unsigned)c4 * (unsigned)sizeof(T) : kOutOfRange;
+#pragma unroll
+      for (int k = 0; k < NX / 2; ++k) {
+        const int e = x0 + cl_p + kMfPix * k;
+        c_x[k] = raw_ld4(rx, e < 0 ? kOutOfRange : (unsigned)(e * C) * (unsigned)sizeof(T) + co, x);
+      }
+      c_g = raw_ld4(rg, (unsigned)((p0 + cl_p) * C) * (unsigned)sizeof(T) + co, gout);
+      return;
     }
 #pragma unroll
     for (int jj = 0; jj < kChW; ++jj) {
@@ -1188,6 +1224,21 @@ __global__ __launch_bounds__(kMfBlock, 4) void local_grad_filter_mfma_kernel(
           hw[t * kMfPix + pix] = in ? make_float2(h, w) : make_float2(-2.f, -2.f);
         }
       }
+    }
+    if constexpr (CL) {
+      // channel 4 cl_q + i of pixel slot cl_p: over a wave's sixteen pixels and four quads the 64 banks once
+      float gv[4];
+      raw_cvt4(c_g, gv, gout);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) gs[(4 * cl_q + i) * kMfPitchG + cl_p] = gv[i];
+#pragma unroll
+      for (int k = 0; k < NX / 2; ++k) {
+        float xv[4];
+        raw_cvt4(c_x[k], xv, x);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) xs[mf_row(4 * cl_q + i, pitch_x) + cl_p + kMfPix * k] = xv[i];
+      }
+      return;
     }
 #pragma unroll
     for (int jj = 0; jj < kChW; ++jj) {
@@ -1654,7 +1705,8 @@ FilterGrid filter_grid(const Geo& g) {
   return f;
 }
 
-template <typename T, int SH, int SW>
+// CL: channels-last tensors, matrix-core kernel at stride 1 only (false otherwise)
+template <typename T, int SH, int SW, bool CL = false>
 bool run_grad_filter(const Geo& g, const T* gout, const T* x, const T* rot, T* gfilter, float* ws,
                      hipStream_t stream) {
   {
@@ -1663,14 +1715,17 @@ bool run_grad_filter(const Geo& g, const T* gout, const T* x, const T* rot, T* g
     if (f.mfma) {
 #define DK_LAUNCH_BF(CELL0, BF, SP)                                                                                 \
   if (f.th > 0) {                                                                                                \
+    if constexpr (CL) return false;                                                                              \
+    else {                                                                                                       \
     auto kernel = local_grad_filter_mfma_kernel<T, SH, SW, CELL0, kMfXS2, true, BF, false>; /* stride 2: no split form yet */                      \
     if (!allow_max_dynamic_lds(reinterpret_cast<const void*>(kernel)))                                                           \
       return false;                                                                                              \
     kernel<<<grid, kMfBlock, f.lds, stream>>>(g, gout, x, rot, ws, f.tiles, f.parts, f.splits, f.pitch_x, f.th); \
+    }                                                                                                            \
   } else if (f.nx == 4)                                                                                          \
-    local_grad_filter_mfma_kernel<T, SH, SW, CELL0, 4, false, BF, SP><<<grid, kMfBlock, f.lds, stream>>>(g, gout, x, rot, ws, f.tiles, f.parts, f.splits, f.pitch_x, 0); \
+    local_grad_filter_mfma_kernel<T, SH, SW, CELL0, 4, false, BF, SP, CL><<<grid, kMfBlock, f.lds, stream>>>(g, gout, x, rot, ws, f.tiles, f.parts, f.splits, f.pitch_x, 0); \
   else                                                                                                           \
-    local_grad_filter_mfma_kernel<T, SH, SW, CELL0, kMfX, false, BF, SP><<<grid, kMfBlock, f.lds, stream>>>(g, gout, x, rot, ws, f.tiles, f.parts, f.splits, f.pitch_x, 0);
+    local_grad_filter_mfma_kernel<T, SH, SW, CELL0, kMfX, false, BF, SP, CL><<<grid, kMfBlock, f.lds, stream>>>(g, gout, x, rot, ws, f.tiles, f.parts, f.splits, f.pitch_x, 0);
       // 16-bit inputs with at least one full block of 16 channels per group: bfloat16 matrix instructions
       // float32 inputs: bfloat16 pairs (three products) unless switched off
       const bool split = !path_disabled(kNoFilterSplit);
@@ -1690,7 +1745,7 @@ bool run_grad_filter(const Geo& g, const T* gout, const T* x, const T* rot, T* g
       launch_reduce_partials<float, T>(ws, f.parts, g.channel * SH * SW, gfilter, stream);
       return true;
     }
-    if constexpr (SH * SW > 32) {
+    if constexpr (CL || SH * SW > 32) {
       return false;  // the dense kernel's fold holds two cells per lane: a 7 x 7 scope goes to the generic kernel
     } else {
     const size_t lds = ((size_t)(kBlock / 64) * f.per * filter_slots(SH * SW) +
@@ -1770,7 +1825,36 @@ bool fast_local_grad_filter(const Geo& g, const T* gout, const T* x, const T* ro
 #undef CALL
 }
 
+// Channels-last tensors on the matrix-core grad filter (its staging reads four consecutive channels per
+// thread): one group, a multiple of 4 channels, stride-1 same-width geometry, 16-byte (16-bit types: 8-byte)
+// aligned tensors, an image's tensor within 2 GB.
+bool fast_local_grad_filter_cl_shape(const Geo& g, size_t elem) {
+  if (!fast_shape(g) || g.groups != 1 || g.channel % 4 != 0 || path_disabled(kNoNhwcStaged)) return false;
+  if ((long)std::max(g.in_h * g.in_w, g.out_h * g.out_w) * g.channel * (long)elem >= (1L << 31)) return false;
+  const FilterGrid f = filter_grid(g);
+  return f.mfma && f.th == 0;
+}
+
+size_t fast_local_grad_filter_cl_workspace(const Geo& g) {
+  // (queried without the element size: the 4-byte bound covers the 2-byte types)
+  if (!fast_local_grad_filter_cl_shape(g, 4)) return 0;
+  return (size_t)filter_grid(g).parts * g.channel * g.scope_h * g.scope_w * sizeof(float);
+}
+
+template <typename T>
+bool fast_local_grad_filter_cl(const Geo& g, const T* gout, const T* x, const T* rot, T* gfilter, void* ws,
+                               hipStream_t stream) {
+  if (!fast_local_grad_filter_cl_shape(g, 4)) return false;
+  if (reinterpret_cast<uintptr_t>(gout) % (4 * sizeof(T)) != 0 || reinterpret_cast<uintptr_t>(x) % (4 * sizeof(T)) != 0)
+    return false;
+#define CALL(SH, SW) run_grad_filter<T, SH, SW, true>(g, gout, x, rot, gfilter, static_cast<float*>(ws), stream)
+  DK_DISPATCH_SCOPE(g, CALL)
+#undef CALL
+}
+
 #define DK_INSTANTIATE(T)                                                                           \
+  template bool fast_local_grad_filter_cl<T>(const Geo&, const T*, const T*, const T*, T*, void*,   \
+                                             hipStream_t);                                          \
   template bool fast_local_gather<T>(const Geo&, bool, const T*, const T*, const T*, T*, hipStream_t); \
   template bool fast_local_grad_rotation<T>(const Geo&, const T*, const T*, const T*, const T*, T*, void*,  \
                                             hipStream_t);                                           \

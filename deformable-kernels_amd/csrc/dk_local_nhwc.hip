@@ -514,30 +514,6 @@ __device__ __forceinline__ float raw_cvt(unsigned v, const float*) { return __ui
 __device__ __forceinline__ float raw_cvt(unsigned short v, const __half*) { return static_cast<float>(__builtin_bit_cast(_Float16, v)); }
 __device__ __forceinline__ float raw_cvt(unsigned short v, const bf16_t*) { return __uint_as_float((unsigned)v << 16); }
 
-typedef unsigned nhwc_u4 __attribute__((ext_vector_type(4)));
-typedef unsigned nhwc_u2 __attribute__((ext_vector_type(2)));
-__device__ __forceinline__ nhwc_u4 raw_ld4(rsrc_t r, unsigned off, const float*) { return __builtin_amdgcn_raw_buffer_load_b128(r, (int)off, 0, 0); }
-__device__ __forceinline__ nhwc_u2 raw_ld4(rsrc_t r, unsigned off, const __half*) { return __builtin_amdgcn_raw_buffer_load_b64(r, (int)off, 0, 0); }
-__device__ __forceinline__ nhwc_u2 raw_ld4(rsrc_t r, unsigned off, const bf16_t*) { return __builtin_amdgcn_raw_buffer_load_b64(r, (int)off, 0, 0); }
-__device__ __forceinline__ void raw_cvt4(nhwc_u4 v, float (&f)[4], const float*) {
-  const unsigned u[4] = {v.x, v.y, v.z, v.w};
-#pragma unroll
-  for (int i = 0; i < 4; ++i) f[i] = __uint_as_float(u[i]);
-}
-__device__ __forceinline__ void raw_cvt4(nhwc_u2 v, float (&f)[4], const __half*) {
-  const unsigned u[2] = {v.x, v.y};
-#pragma unroll
-  for (int i = 0; i < 2; ++i) {
-    f[2 * i] = static_cast<float>(__builtin_bit_cast(_Float16, (unsigned short)(u[i] & 0xffffu)));
-    f[2 * i + 1] = static_cast<float>(__builtin_bit_cast(_Float16, (unsigned short)(u[i] >> 16)));
-  }
-}
-__device__ __forceinline__ void raw_cvt4(nhwc_u2 v, float (&f)[4], const bf16_t*) {
-  const unsigned u[2] = {v.x, v.y};
-#pragma unroll
-  for (int i = 0; i < 2; ++i) f[2 * i] = __uint_as_float(u[i] << 16), f[2 * i + 1] = __uint_as_float(u[i] & 0xffff0000u);
-}
-
 // Sum over the 16 lanes of a DPP row, in every lane of the row.
 __device__ __forceinline__ float row16_sum(float v) {
 #define DK_DPP_ADD(ctrl) \
@@ -878,7 +854,9 @@ void nhwc_grad_rotation(const Geo& g, const T* gout, const T* x, const T* rot, c
 
 size_t nhwc_grad_filter_workspace(const Geo& g, int dtype) {
   const long parts = ceil_div((long)g.batch * g.out_h * g.out_w, (long)kFilterPixPerBlock);
-  return (size_t)parts * g.channel * g.scope_h * g.scope_w * (dtype == DK_F64 ? 8 : 4);
+  const size_t own = (size_t)parts * g.channel * g.scope_h * g.scope_w * (dtype == DK_F64 ? 8 : 4);
+  // (the kernel that stages planar tiles is chosen by the tensors' alignment as well: room for either)
+  return std::max(own, dtype == DK_F64 ? (size_t)0 : fast_local_grad_filter_cl_workspace(g));
 }
 
 template <typename T>
@@ -895,6 +873,8 @@ void nhwc_grad_filter(const Geo& g, const T* gout, const T* x, const T* rot, T* 
   const size_t lds = pb * per_pixel + colb;  // at most 40 KB of table and 100 KB of sums
   CT* partial = static_cast<CT*>(ws);
   if constexpr (!std::is_same<T, double>::value) {
+    // stride-1 layers of one group: the planar operator's matrix-core kernel, its tiles staged from channels-last rows
+    if (fast_local_grad_filter_cl<T>(g, gout, x, rot, gfilter, ws, stream)) return;
     const int nct = (cells + 15) / 16;
     const bool small = (long)g.batch * g.channel * std::max((long)g.in_h * g.in_w, (long)g.out_h * g.out_w) * (long)sizeof(T) < (1L << 31);
     if (g.groups == 1 && nct <= 2 && taps <= kMfRows && small && !path_disabled(kNoNhwcMfma)) {

@@ -25,6 +25,9 @@ CASES = [
     (2, 6, 9, 8, (5, 3), (7, 4), (1, 2), (2, 0), 1, 3, 0.7),   # general taps and scope: sums in LDS columns
     (1, 4, 8, 8, 2, (4, 4), 2, 0, 1, 2, 0.5),
     (2, 8, 40, 36, 3, (4, 4), 1, 1, 1, 1, 0.7),     # 2880 pixels: several partial sums of the grad filter
+    (1, 36, 56, 56, 3, (4, 4), 1, 1, 1, 1, 1.0),    # a plane of the headline's size: six staged elements per lane
+    (2, 20, 13, 13, 3, (3, 3), 1, 1, 1, 1, 1.0),    # scope == kernel on the staged kernels
+    (1, 40, 13, 12, 3, (5, 5), 1, 1, 1, 1, 1.5),    # scope 5: two slices of sixteen cells
 ]
 
 
@@ -76,6 +79,19 @@ def test_fp32_without_the_matrix_core_kernels(case, switch_off):
     assert rel_err(got[3], o64[3]) < 1e-4
 
 
+@pytest.mark.parametrize("case", CASES[:2] + [CASES[6]] + CASES[9:])
+def test_fp32_without_the_staged_kernels(case, switch_off):
+    """Stride-1 layers of one group with a multiple of 4 channels take the kernels that stage planar tiles
+    in LDS; switched off, the matrix-core kernels that read the channels-last rows directly serve them."""
+    switch_off("DK_NO_NHWC_STAGED")
+    inputs, got = _run(case, torch.float32, seed=4)
+    o32, o64 = _oracle(inputs, np.float32), _oracle(inputs, np.float64)
+    assert rel_err(got[0], o32[0]) < 1e-5
+    assert rel_err(got[1], o32[1]) < 1e-5
+    assert rel_err(got[2], o64[2]) < 1e-4
+    assert rel_err(got[3], o64[3]) < 1e-4
+
+
 @pytest.mark.parametrize("case", CASES[:4] + CASES[7:8])
 def test_fp64_matches_oracle(case):
     inputs, got = _run(case, torch.float64)
@@ -85,7 +101,7 @@ def test_fp64_matches_oracle(case):
 
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
-@pytest.mark.parametrize("case", CASES[:3] + CASES[5:7])
+@pytest.mark.parametrize("case", CASES[:3] + CASES[5:7] + CASES[10:])
 def test_half_precisions_match_fp32_oracle(case, dtype):
     inputs, got = _run(case, dtype, seed=3)
     want = _oracle(inputs, np.float32)
