@@ -748,6 +748,208 @@ __global__ __launch_bounds__(kNBlock) void nhwc_grad_rotation_mfma_kernel(Geo g,
   }
 }
 
+// ---------------------------------------------------------------------------
+// grad rotation with 32 channels per matrix instruction (3 x 3 taps, one group, a multiple of 8 channels).
+// A wave owns 16 consecutive output pixels and all nine taps.  Per step of 32 channels, lane
+// (pixel m = l % 16, k group kg = l / 16) loads channels 8 kg .. 8 kg + 7 of its pixel's out_grad once and of
+// each tap's input pixel -- exactly the A operand of v_mfma_f32_16x16x32_bf16 (16 rows x 32 k, eight
+// consecutive k per lane), so P = out_grad * input goes from the loads' registers into the instruction:
+//   R_t[pixel][cell] = sum_c P_t[pixel][c] * W[c][cell]          (nine accumulators of 16 x 16 per 16 cells)
+// The filter sits in LDS as [cell][channel] bfloat16, read 16 bytes per lane as the B operand.
+// float32 / float16 tensors: P = Ph + Pl and W = Wh + Wl as bfloat16 (hi, lo) pairs and three products
+// Ph Wh + Pl Wh + Ph Wl (16 significand bits; fp32 sums); bfloat16 tensors: W = Wh is exact and so is
+// P = Ph + Pl (a product of two 8-bit significands), two products.
+// Then  grot[pixel][t][dir] = sum_cell dA_dir[cell] * R_t[pixel][cell]  touches the four corner cells of the
+// tap's scope coordinate only (planar_bilinear_backward_coord, K.cu:116-163): R_t goes to a wave-private
+// LDS tile, three taps at a time, and lane (tap, pixel) reads its four corners.
+// Invalid rows (pixels past the tensor's end, taps in the padding) and channel groups past the last
+// channel get load offsets outside the buffer's range and load zeros: bit 31 for a row, bit 30 for a
+// channel group, so that their sum stays out of range (the host admits tensors below 2^30 bytes).
+// ---------------------------------------------------------------------------
+typedef __bf16 nhwc_b8 __attribute__((ext_vector_type(8)));
+constexpr int kR16Waves = 4;
+constexpr int kR16TilesPerWave = 2;
+
+// Orders a wave's LDS writes before its LDS reads and the other way round (its LDS operations execute in
+// program order: only the compiler has to be kept from moving them across this point).
+__device__ __forceinline__ void lds_fence_wave() {
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront", "local");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront", "local");
+}
+constexpr unsigned kNoChannels = 0x40000000u;
+
+template <typename T, int NCT, bool WLO>
+__global__ __launch_bounds__(64 * kR16Waves) void nhwc_grad_rotation_mfma16_kernel(
+    Geo g, const T* __restrict__ gout, const T* __restrict__ x, const T* __restrict__ rot,
+    const T* __restrict__ filter, T* __restrict__ grot, int tiles_per_wave, int wpitch, int total_blocks) {
+  constexpr int ROW = 16 * NCT, ROWP = ROW + 4, TAPS = 9;
+  constexpr int NL = 2, HALF = 4;  // two loads of four channels for a lane's eight
+  using Raw = typename std::conditional<sizeof(T) == 4, nhwc_u4, nhwc_u2>::type;
+  extern __shared__ __align__(16) unsigned char nhwc_lds[];
+  unsigned short* wh = reinterpret_cast<unsigned short*>(nhwc_lds);  // [ROW][wpitch] hi parts, then the lo parts
+  unsigned short* wlo = wh + ROW * wpitch;
+  const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  float* rl = reinterpret_cast<float*>(nhwc_lds + (size_t)ROW * wpitch * 2 * (WLO ? 2 : 1)) + wave * (3 * 16 * ROWP);
+  const int C = g.channel, cells = g.scope_h * g.scope_w;
+  const int cpad = (C + 31) & ~31;
+  const int lb = logical_block(total_blocks);
+  if (lb >= total_blocks) return;
+
+  for (int i = threadIdx.x; i < ROW * cpad; i += 64 * kR16Waves) {
+    const int ch = i / ROW, cell = i - ch * ROW;
+    const float v = ch < C && cell < cells ? (float)ld(filter + (size_t)ch * cells + cell) : 0.f;
+    const unsigned hi = pack_bf16(v, 0.f) & 0xffffu;
+    wh[cell * wpitch + ch] = (unsigned short)hi;
+    if (WLO) wlo[cell * wpitch + ch] = (unsigned short)(pack_bf16(v - bf16_lo(hi), 0.f) & 0xffffu);
+  }
+  __syncthreads();
+
+  const int m = lane & 15, kg = lane >> 4;
+  const int oplane = g.out_h * g.out_w;
+  const long total_pix = (long)g.batch * oplane;
+  const rsrc_t rg = plane_rsrc(gout, (int)(total_pix * C));
+  const rsrc_t rx = plane_rsrc(x, g.batch * g.in_h * g.in_w * C);
+  const int nsteps = cpad / 32;
+
+  for (int tk = 0; tk < tiles_per_wave; ++tk) {
+    const long q0 = (((long)lb * kR16Waves + wave) * tiles_per_wave + tk) * 16;
+    if (q0 >= total_pix) break;  // uniform over the wave
+    const long q = q0 + m;
+    const bool live = q < total_pix;
+    const long qc = live ? q : 0;
+    const int b = (int)(qc / oplane), pix = (int)(qc - (long)b * oplane);
+    const int oh = pix / g.out_w, ow = pix - oh * g.out_w;
+    const unsigned goff = live ? (unsigned)(qc * C) * (unsigned)sizeof(T) : kOutOfRange;
+    unsigned xoff[TAPS];
+#pragma unroll
+    for (int t = 0; t < TAPS; ++t) {
+      const int ih = oh * g.stride_h - g.pad_h + (t / 3) * g.dil_h, iw = ow * g.stride_w - g.pad_w + (t % 3) * g.dil_w;
+      const bool ok = live && ih >= 0 && ih < g.in_h && iw >= 0 && iw < g.in_w;
+      xoff[t] = ok ? (unsigned)((((long)b * g.in_h + ih) * g.in_w + iw) * C) * (unsigned)sizeof(T) : kOutOfRange;
+    }
+    // byte offset of the lane's eight channels in a step, or kNoChannels
+    auto chan_off = [&](int step) {
+      const int c8 = step * 32 + 8 * kg;
+      return c8 < C ? (unsigned)c8 * (unsigned)sizeof(T) : kNoChannels;
+    };
+
+    nhwc_f4 acc[TAPS][NCT];
+#pragma unroll
+    for (int t = 0; t < TAPS; ++t)
+#pragma unroll
+      for (int n = 0; n < NCT; ++n) acc[t][n] = nhwc_f4{0.f, 0.f, 0.f, 0.f};
+
+    Raw xr[3][NL], gcur[NL], gnext[NL];  // a ring of three taps' loads: two taps ahead of the arithmetic
+    auto issue_x = [&](Raw (&buf)[NL], int t, unsigned co) {
+#pragma unroll
+      for (int h = 0; h < NL; ++h) buf[h] = raw_ld4(rx, xoff[t] + co + (unsigned)(HALF * sizeof(T)) * h, x);
+    };
+    auto issue_g = [&](Raw (&buf)[NL], unsigned co) {
+#pragma unroll
+      for (int h = 0; h < NL; ++h) buf[h] = raw_ld4(rg, goff + co + (unsigned)(HALF * sizeof(T)) * h, gout);
+    };
+    unsigned co = chan_off(0);
+    issue_g(gcur, co);
+    issue_x(xr[0], 0, co);
+    issue_x(xr[1], 1, co);
+    for (int step = 0; step < nsteps; ++step) {
+      const unsigned co_next = chan_off(step + 1);  // past the last step: no channels, the loads return zeros
+      // this step's filter operands
+      uint4 bh[NCT], bl[NCT];
+#pragma unroll
+      for (int n = 0; n < NCT; ++n) {
+        bh[n] = *reinterpret_cast<const uint4*>(wh + (n * 16 + m) * wpitch + step * 32 + 8 * kg);
+        if (WLO) bl[n] = *reinterpret_cast<const uint4*>(wlo + (n * 16 + m) * wpitch + step * 32 + 8 * kg);
+      }
+      float gv[8];
+#pragma unroll
+      for (int h = 0; h < NL; ++h) {
+        float f[4];
+        raw_cvt4(gcur[h], f, gout);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) gv[HALF * h + i] = f[i];
+      }
+#pragma unroll
+      for (int t = 0; t < TAPS; ++t) {
+        if (t + 2 < TAPS) issue_x(xr[(t + 2) % 3], t + 2, co);
+        else issue_x(xr[(t + 2) % 3], t + 2 - TAPS, co_next);
+        if (t == 4) issue_g(gnext, co_next);
+        float xv[8];
+#pragma unroll
+        for (int h = 0; h < NL; ++h) {
+          float f[4];
+          raw_cvt4(xr[t % 3][h], f, x);
+#pragma unroll
+          for (int i = 0; i < 4; ++i) xv[HALF * h + i] = f[i];
+        }
+        float pr[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+          pr[i] = gv[i] * xv[i];
+          asm volatile("" : "+v"(pr[i]));  // one fp32 value for both parts: no contraction into the conversions
+        }
+        unsigned hi[4], lo[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          hi[i] = pack_bf16(pr[2 * i], pr[2 * i + 1]);
+          lo[i] = pack_bf16(pr[2 * i] - bf16_lo(hi[i]), pr[2 * i + 1] - bf16_hi(hi[i]));
+        }
+        const nhwc_b8 ph = __builtin_bit_cast(nhwc_b8, uint4{hi[0], hi[1], hi[2], hi[3]});
+        const nhwc_b8 pl = __builtin_bit_cast(nhwc_b8, uint4{lo[0], lo[1], lo[2], lo[3]});
+#pragma unroll
+        for (int n = 0; n < NCT; ++n) {
+          const nhwc_b8 wb = __builtin_bit_cast(nhwc_b8, bh[n]);
+          acc[t][n] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ph, wb, acc[t][n], 0, 0, 0);
+          acc[t][n] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pl, wb, acc[t][n], 0, 0, 0);
+          if (WLO) acc[t][n] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ph, __builtin_bit_cast(nhwc_b8, bl[n]), acc[t][n], 0, 0, 0);
+        }
+      }
+#pragma unroll
+      for (int h = 0; h < NL; ++h) gcur[h] = gnext[h];
+      co = co_next;
+    }
+
+    // lane (kg, m) holds R_t[pixel 4 kg + i][cell 16 n + m]; lane (tap tt = l / 16 < 3, pixel m) finishes a row
+#pragma unroll
+    for (int ph_ = 0; ph_ < 3; ++ph_) {
+      lds_fence_wave();
+#pragma unroll
+      for (int tt = 0; tt < 3; ++tt)
+#pragma unroll
+        for (int n = 0; n < NCT; ++n)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) rl[(tt * 16 + 4 * kg + i) * ROWP + 16 * n + m] = acc[3 * ph_ + tt][n][i];
+      lds_fence_wave();
+      if (lane < 48 && live) {
+        const int tt = kg, t = 3 * ph_ + tt;
+        const int ih = oh * g.stride_h - g.pad_h + ph_ * g.dil_h, iw = ow * g.stride_w - g.pad_w + tt * g.dil_w;
+        const bool hit = ih >= 0 && ih < g.in_h && iw >= 0 && iw < g.in_w;
+        const size_t ri = (size_t)q * (TAPS * 2) + 2 * t;
+        bool open_h = true, open_w = true;
+        const float sh = scope_coord<float>(g, ph_, (float)ld(rot + ri), g.centre_h, &open_h);
+        const float sw = scope_coord<float>(g, tt, (float)ld(rot + ri + 1), g.centre_w, &open_w);
+        float gh = 0.f, gw = 0.f;
+        if (hit && sh > -1.f && sw > -1.f && sh < (float)g.scope_h && sw < (float)g.scope_w) {
+          const float hf = floorf(sh), wf = floorf(sw);
+          const int hl = (int)hf, wl = (int)wf, hi_ = hl + 1, wi = wl + 1;
+          const float lh = sh - hf, lw = sw - wf, hh = 1.f - lh, hw = 1.f - lw;
+          const bool top = hl >= 0, bot = hi_ <= g.scope_h - 1, lft = wl >= 0, rgt = wi <= g.scope_w - 1;
+          const float* row = rl + (tt * 16 + m) * ROWP;
+          const int c00 = max(hl, 0) * g.scope_w + max(wl, 0), c01 = max(hl, 0) * g.scope_w + min(wi, g.scope_w - 1);
+          const int c10 = min(hi_, g.scope_h - 1) * g.scope_w + max(wl, 0), c11 = min(hi_, g.scope_h - 1) * g.scope_w + min(wi, g.scope_w - 1);
+          const float r00 = top && lft ? row[c00] : 0.f, r01 = top && rgt ? row[c01] : 0.f;
+          const float r10 = bot && lft ? row[c10] : 0.f, r11 = bot && rgt ? row[c11] : 0.f;
+          gh = hw * (r10 - r00) + lw * (r11 - r01);
+          gw = hh * (r01 - r00) + lh * (r11 - r10);
+        }
+        st(grot + ri, open_h ? gh : 0.f);
+        st(grot + ri + 1, open_w ? gw : 0.f);
+      }
+    }
+  }
+}
+
 // ---- host side --------------------------------------------------------------------------
 
 constexpr int kFilterPixPerBlock = 128;
@@ -818,6 +1020,22 @@ void nhwc_grad_rotation(const Geo& g, const T* gout, const T* x, const T* rot, c
     const bool aligned = g.channel % 4 == 0 && reinterpret_cast<uintptr_t>(gout) % (4 * sizeof(T)) == 0 &&
                          reinterpret_cast<uintptr_t>(x) % (4 * sizeof(T)) == 0;
     const bool small = (long)g.batch * g.channel * std::max((long)g.in_h * g.in_w, (long)g.out_h * g.out_w) * (long)sizeof(T) < (1L << 31);
+    // 3 x 3 taps, a multiple of 8 channels: 32 channels per matrix instruction
+    const long bytes = (long)g.batch * g.channel * std::max((long)g.in_h * g.in_w, (long)g.out_h * g.out_w) * (long)sizeof(T);
+    if (g.groups == 1 && nct <= 2 && g.k_h == 3 && g.k_w == 3 && g.channel % 8 == 0 && aligned && bytes < (1L << 30) &&
+        !path_disabled(kNoNhwcMfma) && !path_disabled(kNoNhwcStaged)) {
+      constexpr bool wlo = !std::is_same<T, bf16_t>::value;
+      const int wpitch = ((g.channel + 31) & ~31) + 8;
+      const size_t lds = (size_t)16 * nct * wpitch * 2 * (wlo ? 2 : 1) + (size_t)kR16Waves * 48 * (16 * nct + 4) * sizeof(float);
+      const long tiles = ceil_div((long)g.batch * g.out_h * g.out_w, 16L);
+      const int blocks = (int)ceil_div(tiles, (long)kR16Waves * kR16TilesPerWave);
+      auto kernel = nct == 1 ? nhwc_grad_rotation_mfma16_kernel<T, 1, wlo> : nhwc_grad_rotation_mfma16_kernel<T, 2, wlo>;
+      if (lds <= 64 * 1024 || (lds <= 120 * 1024 && allow_dynamic_lds(reinterpret_cast<const void*>(kernel), 120 * 1024))) {
+        hipLaunchKernelGGL(kernel, dim3((unsigned)xcd_grid_size(blocks)), dim3(64 * kR16Waves), lds, stream, g, gout, x, rot,
+                           filter, grot, kR16TilesPerWave, wpitch, blocks);
+        return;
+      }
+    }
     if (g.groups == 1 && nct <= 2 && taps_ <= kMfRows && aligned && small && wl_bytes <= 96 * 1024 && !path_disabled(kNoNhwcMfma)) {
       const int pb = kMfRows / taps_;
       const long batches = ceil_div((long)g.batch * g.out_h * g.out_w, (long)pb);
