@@ -65,12 +65,12 @@ OTHER_WORKLOADS = {
 # calibration multiply below and the 1 GiB streaming passes).
 TRAFFIC_RULES = {  # entry point -> regular expressions; a dispatch belongs to the first entry it matches
     # (the pixel-lanes kernel's fourth template argument says whether it runs the transposed geometry)
-    "forward": [r"dk::.*local_pixel_lanes_kernel<[^,]*, \d+, \d+, false", r"dk::.*local_gather\w*_kernel<[^>]*\bfalse\b",
+    "forward": [r"dk::.*local_pixel_lanes_kernel<[^,]*, \d+, \d+, false", r"dk::.*(local|nhwc)_gather\w*_kernel<[^>]*\bfalse\b",
                 r"dk::.*local_forward"],
-    "grad_input": [r"dk::.*local_pixel_lanes_kernel<[^,]*, \d+, \d+, true", r"dk::.*local_gather\w*_kernel<[^>]*\btrue\b",
+    "grad_input": [r"dk::.*local_pixel_lanes_kernel<[^,]*, \d+, \d+, true", r"dk::.*(local|nhwc)_gather\w*_kernel<[^>]*\btrue\b",
                    r"dk::.*local_grad_input"],
-    "grad_rotation": [r"dk::.*local_grad_rotation"],
-    "grad_filter": [r"dk::.*local_grad_filter", r"dk::.*reduce_partials"],
+    "grad_rotation": [r"dk::.*(local|nhwc)_grad_rotation"],
+    "grad_filter": [r"dk::.*(local|nhwc)_grad_filter", r"dk::.*reduce_partials"],
 }
 
 

@@ -17,6 +17,16 @@
 //                          up to 5 x 5; other scopes: a column of LDS); the table holds the
 //                          dense row of hat products of each (pixel, tap); per-workgroup partial sums
 //                          are added in a fixed order by reduce_partials.
+// Layers of one rotation group with 3 x 3 taps -- the shapes networks use -- take matrix-core kernels instead:
+//   forward / grad input : nhwc_gather_mfma16_kernel (scopes of up to 16 cells): the effective weights of 16 channels
+//                          x 16 pixels per matrix instruction, landing as the four consecutive channels a 16-byte
+//                          load of the source pixel delivers;
+//   grad rotation        : nhwc_grad_rotation_mfma16_kernel: out_grad * input of 32 channels from the loads'
+//                          registers as the matrix operand, nine 16 x 16 accumulators per 16 pixels;
+//   grad filter          : the planar operator's matrix-core kernel (dk_local_fast.hip) with a staging that
+//                          reads four consecutive channels per thread (stride-1 layers);
+// and, where those do not apply, nhwc_grad_filter_mfma_kernel / nhwc_grad_rotation_mfma_kernel on fp32
+// matrix instructions with dense hat-product tables.
 #include "dk_kernels.h"
 
 namespace dk {
@@ -768,7 +778,7 @@ __global__ __launch_bounds__(kNBlock) void nhwc_grad_rotation_mfma_kernel(Geo g,
 // ---------------------------------------------------------------------------
 typedef __bf16 nhwc_b8 __attribute__((ext_vector_type(8)));
 constexpr int kR16Waves = 4;
-constexpr int kR16TilesPerWave = 2;
+constexpr int kR16TilesPerWave = 1;
 
 // Orders a wave's LDS writes before its LDS reads and the other way round (its LDS operations execute in
 // program order: only the compiler has to be kept from moving them across this point).
@@ -950,6 +960,271 @@ __global__ __launch_bounds__(64 * kR16Waves) void nhwc_grad_rotation_mfma16_kern
   }
 }
 
+// ---------------------------------------------------------------------------
+// forward / grad input on the matrix cores (3 x 3 taps, one group, scopes of up to 16 cells, a multiple of 4
+// channels).  The bilinear read of a channel's scope is the dense contraction
+//   w_eff[c][(pixel, tap)] = sum_cell W[c][cell] * A[cell][(pixel, tap)],   A = hat(h - i) * hat(w - j),
+// and with the channels on the rows of v_mfma_f32_16x16x32_{f16,bf16} and 16 destination pixels on its columns
+// the result lands as lane (kg, n) <- channels 4 kg .. 4 kg + 3 of pixel n: the four consecutive channels a
+// 16-byte load of the tap's source pixel delivers, so the sources go from global memory to registers to
+// four multiply-adds per tap with no staging, and the four results leave as one 16-byte store.
+// Split precision as in the planar matrix-core kernel: A = Ah + Al in the matrix type; float32 tensors
+// W * s = Wh + Wl in fp16 (s a power of two per channel that brings the channel's largest weight into [0.5, 1)),
+// products Ah Wh + Al Wh (one K = 32 instruction: k = the lane group's four cells' hi parts, then their lo
+// parts, against [Wh ; Wh]) and Ah Wl ([Wl ; 0]); 16-bit tensors: W is exact, one instruction.
+// A wave owns 16 consecutive destination pixels: per tile the lane groups share the work on the nine taps'
+// scope coordinates and source offsets through a wave-private LDS table, every lane derives its 36 operand
+// registers, then the wave walks the channel blocks with the sources of two tap rows in flight.
+// grad input is the same kernel on the transposed geometry (tap t of input pixel q is fed by the output
+// pixel that reads q through t, with that pixel's rotation; K.cu:611-651).
+// ---------------------------------------------------------------------------
+template <typename E> struct NhwcMx;
+template <> struct NhwcMx<_Float16> {
+  typedef _Float16 v4 __attribute__((ext_vector_type(4)));
+  typedef _Float16 v8 __attribute__((ext_vector_type(8)));
+  // d_i = w0 * h_i (+ w1 * h_i): rows = 16 channels, columns = 16 pixels.  From inline assembly with
+  // early-clobber results: a result of these instructions must not share registers with an operand,
+  // which the compiler otherwise arranges at an operand's last use.  The second product on a result
+  // follows two independent instructions; s_nop 7 covers the wait states before the vector ALU may read.
+  template <bool SECOND>
+  static __device__ __forceinline__ void rows3(nhwc_f4& d0, nhwc_f4& d1, nhwc_f4& d2, v8 w0, v8 w1, v8 h0, v8 h1, v8 h2) {
+    if constexpr (SECOND)
+      asm volatile(
+          "s_nop 1\n\t"
+          "v_mfma_f32_16x16x32_f16 %0, %3, %5, 0\n\t"
+          "v_mfma_f32_16x16x32_f16 %1, %3, %6, 0\n\t"
+          "v_mfma_f32_16x16x32_f16 %2, %3, %7, 0\n\t"
+          "v_mfma_f32_16x16x32_f16 %0, %4, %5, %0\n\t"
+          "v_mfma_f32_16x16x32_f16 %1, %4, %6, %1\n\t"
+          "v_mfma_f32_16x16x32_f16 %2, %4, %7, %2\n\t"
+          "s_nop 7"
+          : "=&v"(d0), "=&v"(d1), "=&v"(d2)
+          : "v"(w0), "v"(w1), "v"(h0), "v"(h1), "v"(h2));
+    else
+      asm volatile(
+          "s_nop 1\n\t"
+          "v_mfma_f32_16x16x32_f16 %0, %3, %4, 0\n\t"
+          "v_mfma_f32_16x16x32_f16 %1, %3, %5, 0\n\t"
+          "v_mfma_f32_16x16x32_f16 %2, %3, %6, 0\n\t"
+          "s_nop 7"
+          : "=&v"(d0), "=&v"(d1), "=&v"(d2)
+          : "v"(w0), "v"(h0), "v"(h1), "v"(h2));
+  }
+};
+template <> struct NhwcMx<__bf16> {
+  typedef __bf16 v4 __attribute__((ext_vector_type(4)));
+  typedef __bf16 v8 __attribute__((ext_vector_type(8)));
+  template <bool SECOND>
+  static __device__ __forceinline__ void rows3(nhwc_f4& d0, nhwc_f4& d1, nhwc_f4& d2, v8 w0, v8 w1, v8 h0, v8 h1, v8 h2) {
+    static_assert(!SECOND, "bfloat16 tensors need no second product");
+    asm volatile(
+        "s_nop 1\n\t"
+        "v_mfma_f32_16x16x32_bf16 %0, %3, %4, 0\n\t"
+        "v_mfma_f32_16x16x32_bf16 %1, %3, %5, 0\n\t"
+        "v_mfma_f32_16x16x32_bf16 %2, %3, %6, 0\n\t"
+        "s_nop 7"
+        : "=&v"(d0), "=&v"(d1), "=&v"(d2)
+        : "v"(w0), "v"(h0), "v"(h1), "v"(h2));
+  }
+};
+template <typename T> struct NhwcMxOf { using type = _Float16; };  // float, __half
+template <> struct NhwcMxOf<bf16_t> { using type = __bf16; };
+
+__device__ __forceinline__ float nhwc_hat(float d) { return __builtin_amdgcn_fmed3f(1.f - fabsf(d), 0.f, 1.f); }
+
+template <int AUX = 0>
+__device__ __forceinline__ void raw_st4(rsrc_t r, unsigned off, const float (&v)[4], float*) {
+  __builtin_amdgcn_raw_buffer_store_b128(nhwc_u4{__float_as_uint(v[0]), __float_as_uint(v[1]), __float_as_uint(v[2]), __float_as_uint(v[3])}, r, (int)off, 0, AUX);
+}
+template <int AUX = 0, typename T>
+__device__ __forceinline__ void raw_st4(rsrc_t r, unsigned off, const float (&v)[4], T*) {
+  struct { T e[4]; } pk;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) st(pk.e + i, v[i]);
+  __builtin_amdgcn_raw_buffer_store_b64(__builtin_bit_cast(nhwc_u2, pk), r, (int)off, 0, AUX);
+}
+
+constexpr int kG16Waves = 4;
+// One tile per wave: workgroups that live as long as one tile keep the tail of the grid short (two tiles per wave
+// measured 85.8 against 81.4 us on benchmark configuration 2, four 96).
+constexpr int kG16TilesPerWave = 1;
+
+template <typename T, int SH, int SW, bool TRANSPOSED>
+__global__ __launch_bounds__(64 * kG16Waves) void nhwc_gather_mfma16_kernel(
+    Geo g, const T* __restrict__ src, const T* __restrict__ rot, const T* __restrict__ filter, T* __restrict__ dst,
+    int tiles_per_wave, int total_blocks) {
+  using E = typename NhwcMxOf<T>::type;
+  using M = NhwcMx<E>;
+  using Raw = typename std::conditional<sizeof(T) == 4, nhwc_u4, nhwc_u2>::type;
+  constexpr bool kThird = sizeof(T) == 4;  // float32 tensors: the filter has a low part
+  constexpr int TAPS = 9, CELLS = SH * SW;
+  static_assert(CELLS <= 16, "one block of sixteen cells");
+  extern __shared__ __align__(16) unsigned char nhwc_lds[];
+  const int C = g.channel, nblk = (C + 15) >> 4;
+  uint4* wsp = reinterpret_cast<uint4*>(nhwc_lds);                // [nblk][64]: Wh (2 words), Wl (2 words) of lane (channel, cells 4 kg ..)
+  float* unscale = reinterpret_cast<float*>(wsp + nblk * 64);     // [nblk][16]: 1 / s of the channel
+  const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  float2* cw = reinterpret_cast<float2*>(unscale + nblk * 16) + wave * (TAPS * 16);             // [tap][pixel]: scope coordinates
+  unsigned* xo = reinterpret_cast<unsigned*>(reinterpret_cast<float2*>(unscale + nblk * 16) + kG16Waves * TAPS * 16) +
+                 wave * (TAPS * 16);                                                             // [tap][pixel]: source offsets
+  const int lb = logical_block(total_blocks);
+  if (lb >= total_blocks) return;
+
+  // ---- per workgroup: the split filter operands of every channel block
+  for (int e = threadIdx.x; e < nblk * 64; e += 64 * kG16Waves) {
+    const int b = e >> 6, l = e & 63, cj = b * 16 + (l & 15), c0 = 4 * (l >> 4);
+    float v[4] = {0.f, 0.f, 0.f, 0.f}, s = 1.f;
+    if (cj < C) {
+      const T* f = filter + (size_t)cj * CELLS;
+      if constexpr (kThird) {
+        float mx = 0.f;
+#pragma unroll
+        for (int k = 0; k < CELLS; ++k) mx = fmaxf(mx, fabsf(ld(f + k)));
+        int ex = 0;
+        if (mx > 0.f && mx < __builtin_inff()) (void)frexpf(mx, &ex);
+        ex = min(max(ex, -100), 100);
+        s = ldexpf(1.f, -ex);
+        if ((l >> 4) == 0) unscale[b * 16 + (l & 15)] = ldexpf(1.f, ex);
+      }
+#pragma unroll
+      for (int k = 0; k < 4; ++k)
+        if (c0 + k < CELLS) v[k] = (float)ld(f + c0 + k) * s;
+    } else if ((l >> 4) == 0) {
+      unscale[b * 16 + (l & 15)] = 0.f;
+    }
+    typename M::v4 h4, l4;
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      float vv = v[k];
+      asm volatile("" : "+v"(vv));  // one fp32 value for both parts
+      const E hi = static_cast<E>(vv);
+      h4[k] = hi;
+      l4[k] = static_cast<E>(vv - static_cast<float>(hi));
+    }
+    const uint2 hb = __builtin_bit_cast(uint2, h4), lb2 = __builtin_bit_cast(uint2, l4);
+    wsp[e] = make_uint4(hb.x, hb.y, lb2.x, lb2.y);
+  }
+  __syncthreads();
+
+  const int n = lane & 15, kg = lane >> 4;
+  const int oplane = g.out_h * g.out_w, iplane = g.in_h * g.in_w;
+  const int dplane = TRANSPOSED ? iplane : oplane, splane = TRANSPOSED ? oplane : iplane;
+  const long total_pix = (long)g.batch * dplane;
+  const rsrc_t rs = plane_rsrc(src, g.batch * splane * C);
+  const rsrc_t rd = plane_rsrc(dst, g.batch * dplane * C);
+  // the lane group's four cells: rows past the last cell never match a coordinate
+  float crow[4], ccol[4];
+#pragma unroll
+  for (int k = 0; k < 4; ++k) {
+    const int c = 4 * kg + k;
+    crow[k] = c < CELLS ? (float)(c / SW) : 64.f;
+    ccol[k] = (float)(c % SW);
+  }
+
+  for (int tk = 0; tk < tiles_per_wave; ++tk) {
+    const long q0 = (((long)lb * kG16Waves + wave) * tiles_per_wave + tk) * 16;
+    if (q0 >= total_pix) break;  // uniform over the wave
+    const long q = q0 + n;
+    const bool live = q < total_pix;
+    const long qc = live ? q : 0;
+    const int b = (int)(qc / dplane), pix = (int)(qc - (long)b * dplane);
+
+    // ---- the nine taps of the sixteen pixels: lane group kg takes taps kg, kg + 4, kg + 8
+    lds_fence_wave();
+#pragma unroll
+    for (int k = 0; k < 3; ++k) {
+      const int t = kg + 4 * k;
+      if (t < TAPS) {
+        int opix = 0;
+        long src_pix = 0;
+        const bool hit = tap_pixels<TRANSPOSED>(g, pix, t, opix, src_pix) && live;
+        float2 c = make_float2(-2.f, -2.f);
+        unsigned so = kOutOfRange;
+        if (hit) {
+          const size_t ri = ((size_t)b * oplane + opix) * (TAPS * 2) + 2 * t;
+          const float h = scope_coord<float>(g, t / 3, (float)ld(rot + ri), g.centre_h);
+          const float w = scope_coord<float>(g, t % 3, (float)ld(rot + ri + 1), g.centre_w);
+          if (h > -1.f && w > -1.f && h < (float)SH && w < (float)SW) {
+            c = make_float2(h, w);
+            so = (unsigned)(((long)b * splane + src_pix) * C) * (unsigned)sizeof(T);
+          }
+        }
+        cw[t * 16 + n] = c;
+        xo[t * 16 + n] = so;
+      }
+    }
+    lds_fence_wave();
+    typename M::v8 A[TAPS];
+    unsigned xoff[TAPS];
+#pragma unroll
+    for (int t = 0; t < TAPS; ++t) {
+      const float2 c = cw[t * 16 + n];
+      xoff[t] = xo[t * 16 + n];
+      typedef float f2v __attribute__((ext_vector_type(2)));
+      typedef E e2v __attribute__((ext_vector_type(2)));
+      float v[4];
+#pragma unroll
+      for (int k = 0; k < 4; ++k) {
+        v[k] = nhwc_hat(c.x - crow[k]) * nhwc_hat(c.y - ccol[k]);
+        asm volatile("" : "+v"(v[k]));  // one fp32 value for both parts
+      }
+      const e2v h01 = __builtin_convertvector(f2v{v[0], v[1]}, e2v), h23 = __builtin_convertvector(f2v{v[2], v[3]}, e2v);
+      const f2v b01 = __builtin_convertvector(h01, f2v), b23 = __builtin_convertvector(h23, f2v);
+      const e2v l01 = __builtin_convertvector(f2v{v[0] - b01[0], v[1] - b01[1]}, e2v);
+      const e2v l23 = __builtin_convertvector(f2v{v[2] - b23[0], v[3] - b23[1]}, e2v);
+      A[t] = typename M::v8{h01[0], h01[1], h23[0], h23[1], l01[0], l01[1], l23[0], l23[1]};
+    }
+
+    // ---- the channel blocks
+    const unsigned doff = live ? (unsigned)(qc * C) * (unsigned)sizeof(T) : kOutOfRange;
+    auto chan_off = [&](int blk) {
+      const int c4 = blk * 16 + 4 * kg;
+      return c4 < C ? (unsigned)c4 * (unsigned)sizeof(T) : kNoChannels;
+    };
+    Raw xr[3][3];  // [tap row][tap]: two tap rows ahead of the arithmetic
+    auto issue_row = [&](Raw (&buf)[3], int r, unsigned co) {
+#pragma unroll
+      for (int tt = 0; tt < 3; ++tt) buf[tt] = raw_ld4(rs, xoff[3 * r + tt] + co, src);
+    };
+    unsigned co = chan_off(0);
+    issue_row(xr[0], 0, co);
+    issue_row(xr[1], 1, co);
+    for (int blk = 0; blk < nblk; ++blk) {
+      const unsigned co_next = chan_off(blk + 1);  // past the last block: no channels, zeros
+      const uint4 wv = wsp[blk * 64 + lane];
+      const typename M::v4 wh = __builtin_bit_cast(typename M::v4, make_uint2(wv.x, wv.y));
+      const typename M::v4 wl = __builtin_bit_cast(typename M::v4, make_uint2(wv.z, wv.w));
+      const typename M::v8 whh = __builtin_shufflevector(wh, wh, 0, 1, 2, 3, 0, 1, 2, 3);
+      const typename M::v4 zero4 = {E(0), E(0), E(0), E(0)};
+      const typename M::v8 wl0 = __builtin_shufflevector(wl, zero4, 0, 1, 2, 3, 4, 5, 6, 7);
+      float acc[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int r = 0; r < 3; ++r) {
+        if (r == 0) issue_row(xr[2], 2, co);
+        else issue_row(xr[r - 1], r - 1, co_next);
+        nhwc_f4 d[3];
+        M::template rows3<kThird>(d[0], d[1], d[2], whh, wl0, A[3 * r], A[3 * r + 1], A[3 * r + 2]);
+#pragma unroll
+        for (int tt = 0; tt < 3; ++tt) {
+          float xv[4];
+          raw_cvt4(xr[r][tt], xv, src);
+#pragma unroll
+          for (int i = 0; i < 4; ++i) acc[i] = fmaf(xv[i], d[tt][i], acc[i]);
+        }
+      }
+      if constexpr (kThird) {
+        const nhwc_f4 us = *reinterpret_cast<const nhwc_f4*>(unscale + blk * 16 + 4 * kg);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) acc[i] *= us[i];
+      }
+      // non-temporal: written with the default policy the result pushes the operands of the next kernel out of
+      // the memory-side cache (the step of benchmark configuration 2 took 0.425 instead of 0.363 ms)
+      raw_st4<kStreamingStore>(rd, doff + co, acc, dst);
+      co = co_next;
+    }
+  }
+}
+
 // ---- host side --------------------------------------------------------------------------
 
 constexpr int kFilterPixPerBlock = 128;
@@ -988,9 +1263,43 @@ bool nhwc_supported(const Geo& g, int dtype) {
   return true;
 }
 
+// The matrix-core forward / grad input; false where it does not apply.
+template <typename T, int SH, int SW>
+bool launch_gather_mfma16(const Geo& g, bool transposed, const T* src, const T* rot, const T* filter, T* dst,
+                          hipStream_t stream) {
+  const int nblk = ceil_div(g.channel, 16);
+  const size_t lds = (size_t)nblk * 64 * 16 + (size_t)nblk * 16 * 4 + (size_t)kG16Waves * 9 * 16 * (8 + 4);
+  const long pixels = (long)g.batch * (transposed ? g.in_h * g.in_w : g.out_h * g.out_w);
+  const long tiles = ceil_div(pixels, 16L);
+  const int blocks = (int)ceil_div(tiles, (long)kG16Waves * kG16TilesPerWave);
+  auto kernel = transposed ? nhwc_gather_mfma16_kernel<T, SH, SW, true> : nhwc_gather_mfma16_kernel<T, SH, SW, false>;
+  if (lds > 64 * 1024 && !(lds <= 120 * 1024 && allow_dynamic_lds(reinterpret_cast<const void*>(kernel), 120 * 1024))) return false;
+  hipLaunchKernelGGL(kernel, dim3((unsigned)xcd_grid_size(blocks)), dim3(64 * kG16Waves), lds, stream, g, src, rot, filter, dst,
+                     kG16TilesPerWave, blocks);
+  return true;
+}
+
+template <typename T>
+bool nhwc_gather_mfma16(const Geo& g, bool transposed, const T* src, const T* rot, const T* filter, T* dst,
+                        hipStream_t stream) {
+  if constexpr (std::is_same<T, double>::value) {
+    return false;
+  } else {
+    const long bytes = (long)g.batch * g.channel * std::max((long)g.in_h * g.in_w, (long)g.out_h * g.out_w) * (long)sizeof(T);
+    if (g.groups != 1 || g.k_h != 3 || g.k_w != 3 || g.channel % 4 != 0 || g.channel < 16 || bytes >= (1L << 30) ||
+        reinterpret_cast<uintptr_t>(src) % (4 * sizeof(T)) != 0 || reinterpret_cast<uintptr_t>(dst) % (4 * sizeof(T)) != 0 ||
+        path_disabled(kNoNhwcMfma) || path_disabled(kNoNhwcStaged))
+      return false;
+    if (g.scope_h == 4 && g.scope_w == 4) return launch_gather_mfma16<T, 4, 4>(g, transposed, src, rot, filter, dst, stream);
+    if (g.scope_h == 3 && g.scope_w == 3) return launch_gather_mfma16<T, 3, 3>(g, transposed, src, rot, filter, dst, stream);
+    return false;
+  }
+}
+
 template <typename T>
 void nhwc_gather(const Geo& g, bool transposed, const T* src, const T* rot, const T* filter, T* dst,
                  hipStream_t stream) {
+  if (nhwc_gather_mfma16<T>(g, transposed, src, rot, filter, dst, stream)) return;
   size_t lds;
   const NhwcLaunch L = gather_launch<T>(g, transposed, lds);
   const dim3 grid((unsigned)(g.batch * L.pblocks), (unsigned)ceil_div(g.channel, L.cc));

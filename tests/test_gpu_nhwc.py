@@ -28,6 +28,8 @@ CASES = [
     (1, 36, 56, 56, 3, (4, 4), 1, 1, 1, 1, 1.0),    # a plane of the headline's size: six staged elements per lane
     (2, 20, 13, 13, 3, (3, 3), 1, 1, 1, 1, 1.0),    # scope == kernel on the staged kernels
     (1, 40, 13, 12, 3, (5, 5), 1, 1, 1, 1, 1.5),    # scope 5: two slices of sixteen cells
+    (2, 16, 15, 14, 3, (4, 4), 1, 2, 2, 1, 1.0),    # dilation 2 with one group: the matrix-core kernels' general taps
+    (1, 32, 12, 11, 3, (3, 3), 2, 0, 1, 1, 1.0),    # stride 2 without padding, scope == kernel
 ]
 
 
@@ -128,12 +130,13 @@ def test_equals_the_planar_operator_on_the_same_tensors():
         assert rel_err(a, b) < tol
 
 
+@pytest.mark.parametrize("groups", [2, 1])   # one group: the matrix-core kernels
 @pytest.mark.parametrize("clip", ['scope', (-0.3, 0.2)])
-def test_rotation_clip_inside_the_channels_last_operator(clip):
-    case = (2, 12, 11, 10, 3, (4, 4), 1, 1, 1, 2, 1.5)
+def test_rotation_clip_inside_the_channels_last_operator(clip, groups):
+    case = (2, 12 if groups == 2 else 24, 11, 10, 3, (4, 4), 1, 1, 1, groups, 1.5)
     inputs, got = _run(case, torch.float32, seed=5, clip=clip)
     x, wt, rot, gout, cfg = inputs
-    clamped, open_ = clipped_rotation(rot, clip, cfg["kernel_size"], (4, 4), 2)
+    clamped, open_ = clipped_rotation(rot, clip, cfg["kernel_size"], (4, 4), groups)
     o64 = _oracle((x, wt, clamped, gout, cfg), np.float64)
     assert rel_err(got[0], o64[0]) < 1e-5
     assert rel_err(got[1], o64[1]) < 1e-5
