@@ -1290,6 +1290,16 @@ bool nhwc_gather_mfma16(const Geo& g, bool transposed, const T* src, const T* ro
         reinterpret_cast<uintptr_t>(src) % (4 * sizeof(T)) != 0 || reinterpret_cast<uintptr_t>(dst) % (4 * sizeof(T)) != 0 ||
         path_disabled(kNoNhwcMfma) || path_disabled(kNoNhwcStaged))
       return false;
+    // Where it is the faster kernel (step-level measurements on the MobileNetV2-DK layer shapes, batch 64, float32;
+    // this kernel against the table kernel): its per-tile set-up (a third of its instructions at 144 channels) and
+    // its one-tile-per-wave grid want many channels and many tiles.  Forward 144 x 56^2: 80 against 103 us, but
+    // 32 x 112^2 136 / 109, 192 x 28^2 50 / 39, 960 x 7^2 58 / 22.  Grad input at stride 2, where the table kernel
+    // tests every tap of every input pixel against the stride's grid: 96 x 112^2 166 / 262, 144 x 56^2 61 / 96,
+    // 192 x 28^2 28 / 38.  DK_FORCE_NHWC_GATHER_MFMA takes it wherever it applies (the tests).
+    const long tiles = ((long)g.batch * (transposed ? g.in_h * g.in_w : g.out_h * g.out_w) + 15) / 16;
+    const bool strided = g.stride_h > 1 || g.stride_w > 1;
+    const bool faster = (g.channel >= 128 && tiles >= 8192) || (transposed && strided && g.channel >= 64 && tiles >= 3000);
+    if (!faster && !path_disabled(kForceNhwcGatherMfma)) return false;
     if (g.scope_h == 4 && g.scope_w == 4) return launch_gather_mfma16<T, 4, 4>(g, transposed, src, rot, filter, dst, stream);
     if (g.scope_h == 3 && g.scope_w == 3) return launch_gather_mfma16<T, 3, 3>(g, transposed, src, rot, filter, dst, stream);
     return false;

@@ -94,6 +94,36 @@ def test_fp32_without_the_staged_kernels(case, switch_off):
     assert rel_err(got[3], o64[3]) < 1e-4
 
 
+# the shapes the matrix-core forward / grad input covers: one group, 3 x 3 taps, scope 3 x 3 or 4 x 4, at least 16 channels in fours
+GATHER_CASES = [CASES[0], CASES[1], CASES[2], CASES[6], CASES[10], CASES[11], CASES[13], CASES[14]]
+
+
+@pytest.mark.parametrize("case", GATHER_CASES)
+def test_fp32_matrix_core_forward_and_grad_input_on_every_shape_they_cover(case, switch_off):
+    """The library takes the matrix-core forward / grad input only on large layers with many channels, where they
+    are the faster kernels; forced, they serve every shape they cover: ragged sizes, channel counts that are
+    not a multiple of 16, stride 2 (where the transposed walk skips the taps off the stride's grid),
+    dilation, nineteen channel blocks."""
+    switch_off("DK_FORCE_NHWC_GATHER_MFMA")
+    inputs, got = _run(case, torch.float32, seed=6)
+    o32, o64 = _oracle(inputs, np.float32), _oracle(inputs, np.float64)
+    assert rel_err(got[0], o32[0]) < 1e-5
+    assert rel_err(got[1], o32[1]) < 1e-5
+    assert rel_err(got[2], o64[2]) < 1e-4
+    assert rel_err(got[3], o64[3]) < 1e-4
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("case", [CASES[0], CASES[2], CASES[11], CASES[13]])
+def test_half_precision_matrix_core_forward_and_grad_input(case, dtype, switch_off):
+    switch_off("DK_FORCE_NHWC_GATHER_MFMA")
+    inputs, got = _run(case, dtype, seed=7)
+    want = _oracle(inputs, np.float32)
+    for g, w in zip(got, want):
+        assert g.dtype == dtype
+        assert rel_err(g.float(), w) < 1e-2
+
+
 @pytest.mark.parametrize("case", CASES[:4] + CASES[7:8])
 def test_fp64_matches_oracle(case):
     inputs, got = _run(case, torch.float64)
@@ -132,7 +162,8 @@ def test_equals_the_planar_operator_on_the_same_tensors():
 
 @pytest.mark.parametrize("groups", [2, 1])   # one group: the matrix-core kernels
 @pytest.mark.parametrize("clip", ['scope', (-0.3, 0.2)])
-def test_rotation_clip_inside_the_channels_last_operator(clip, groups):
+def test_rotation_clip_inside_the_channels_last_operator(clip, groups, switch_off):
+    switch_off("DK_FORCE_NHWC_GATHER_MFMA")
     case = (2, 12 if groups == 2 else 24, 11, 10, 3, (4, 4), 1, 1, 1, groups, 1.5)
     inputs, got = _run(case, torch.float32, seed=5, clip=clip)
     x, wt, rot, gout, cfg = inputs
