@@ -49,6 +49,8 @@ OTHER_WORKLOADS = {
     "deform_56": ("deform", (64, 144, 56, 56, 3, (4, 4), 1, 1, 1, 1, 0.5, 2.0)),
     # the deformable variant on MobileNetV2's first depthwise stage (112 x 112 planes: wider than 64 columns)
     "deform_112": ("deform", (64, 32, 112, 112, 3, (4, 4), 1, 1, 1, 1, 0.5, 2.0)),
+    # ... and on 224 x 224 planes, which do not fit LDS at all (the tensors as large as deform_112's)
+    "deform_224": ("deform", (16, 32, 224, 224, 3, (4, 4), 1, 1, 1, 1, 0.5, 2.0)),
     # DeformConv2d (scope = kernel, no rotation tensor: rot_std None) on configuration 4's geometry
     "deform_conv_28": ("deform", (64, 512, 28, 28, 3, (3, 3), 2, 1, 1, 1, None, 2.0)),
     # N-d sampler: data shape [C, s...], points, coordinate range

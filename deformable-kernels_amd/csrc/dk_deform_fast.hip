@@ -1252,6 +1252,55 @@ __global__ __launch_bounds__(1024) void deform_grad_input_kernel(
 }
 
 // ---------------------------------------------------------------------------
+// The input rows a tile of 1024 output pixels samples, for the band form of the tiled grad input below:
+// table[(image * tiles + tile) * 2] = least, [.. + 1] = largest padded row (image row + 1) of the top corners of
+// the tile's samples that hit the image (K.cu:486-500); a tile without such samples gets an empty range.
+// The offsets belong to the image, not to the rotation group.  grid = image * tiles
+// ---------------------------------------------------------------------------
+template <typename T>
+__global__ __launch_bounds__(1024) void deform_tile_rows_kernel(Geo g, const T* __restrict__ off, int* __restrict__ table,
+                                                                int ntiles) {
+  __shared__ int wave_lo[16], wave_hi[16];
+  const int out_plane = g.out_h * g.out_w;
+  const int tile = blockIdx.x % ntiles, n = blockIdx.x / ntiles;
+  const int p = tile * 1024 + threadIdx.x;
+  const bool live = p < out_plane;
+  const int pc = live ? p : 0;
+  const int oh = pc / g.out_w, ow = pc % g.out_w;
+  const rsrc_t ro = plane_rsrc(off + (size_t)n * (K9 * 2) * out_plane, K9 * 2 * out_plane);
+  const unsigned step = (unsigned)out_plane * (unsigned)sizeof(T);
+  int lo = 0x7fffffff, hi = -1;
+#pragma unroll
+  for (int t = 0; t < K9; ++t) {
+    const int f_h = t / 3, f_w = t % 3;
+    const unsigned o = live ? (unsigned)((2 * t) * out_plane + pc) * (unsigned)sizeof(T) : kOutOfRange;
+    const float h = float(oh * g.stride_h - g.pad_h + f_h * g.dil_h) + buf_ld(ro, o, off);
+    const float w = float(ow * g.stride_w - g.pad_w + f_w * g.dil_w) + buf_ld(ro, o + step, off);
+    const bool hit = live && (h > -1.f) && (w > -1.f) && (h < float(g.in_h)) && (w < float(g.in_w));
+    const int pr = static_cast<int>(floorf(h)) + 1;
+    lo = hit ? min(lo, pr) : lo;
+    hi = hit ? max(hi, pr) : hi;
+  }
+  for (int sft = 32; sft > 0; sft >>= 1) {
+    lo = min(lo, __shfl_xor(lo, sft));
+    hi = max(hi, __shfl_xor(hi, sft));
+  }
+  if ((threadIdx.x & 63) == 0) {
+    wave_lo[threadIdx.x >> 6] = lo;
+    wave_hi[threadIdx.x >> 6] = hi;
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    for (int w = 1; w < 16; ++w) {
+      lo = min(lo, wave_lo[w]);
+      hi = max(hi, wave_hi[w]);
+    }
+    table[(size_t)blockIdx.x * 2] = lo;
+    table[(size_t)blockIdx.x * 2 + 1] = hi;
+  }
+}
+
+// ---------------------------------------------------------------------------
 // grad input for output planes of more than 1024 pixels, or input planes the kernel above has no room for.  The
 // same fixed-point LDS accumulation, but the workgroup (1024 threads) owns 2 NP channels of an image and NP 64-bit
 // planes; it walks the output plane in tiles of 1024 pixels, computes a tile's tap descriptors once and adds the
@@ -1259,17 +1308,23 @@ __global__ __launch_bounds__(1024) void deform_grad_input_kernel(
 // (M, as above): while M <= 2^kPairHead two channels share a plane, each as a signed 32-bit term in its half
 // of the 64-bit sum, and one walk serves all 2 NP channels; otherwise every channel gets a plane of its own on the
 // 2^-44 grid and the channels take two walks.  The planes are read back at the end of a walk.
-// grid = (channel chunks of 2 NP, image * group)
+// BAND: input planes that do not fit LDS even once (224 x 224).  A workgroup owns a band of `band_rows` image rows
+// (of all columns) instead of the whole plane: it walks the tiles whose samples touch the band -- found in a table of
+// each tile's least and largest sample row, written by deform_tile_rows_kernel -- and adds the corner pairs that lie
+// in its rows; the other pairs are added by the band that owns theirs, so every input element is still summed in
+// one workgroup's LDS, exactly, and written once.
+// grid = ([bands,] channel chunks of 2 NP, image * group)
 // ---------------------------------------------------------------------------
-template <typename T, int SH, int SW, int NP>
+template <typename T, int SH, int SW, int NP, bool BAND = false>
 __global__ __launch_bounds__(1024) void deform_grad_input_tiled_kernel(
     Geo g, const T* __restrict__ gout, const T* __restrict__ off, const T* __restrict__ rot,
-    const T* __restrict__ filter, T* __restrict__ gin, const unsigned* __restrict__ gmax_bits, int shift) {
+    const T* __restrict__ filter, T* __restrict__ gin, const unsigned* __restrict__ gmax_bits, int shift,
+    int band_rows, const int* __restrict__ tile_rows) {
   using Tb = WideTable<SH, SW>;
   constexpr int NC = 2 * NP;  // channels per workgroup
   extern __shared__ __align__(16) float lds[];
   const int H = g.in_h, W = g.in_w, RS = W + 2;
-  const int PS = ((H + 2) * RS + 3) & ~3;
+  const int PS = ((BAND ? band_rows : H + 2) * RS + 3) & ~3;
   unsigned long long* planes = reinterpret_cast<unsigned long long*>(lds);  // [NP][PS]
   float* tbl = lds + 2 * NP * PS;                                           // [NC][Tb::SIZE]
   float* wmax = tbl + NC * Tb::SIZE;                                        // [NC]
@@ -1277,10 +1332,15 @@ __global__ __launch_bounds__(1024) void deform_grad_input_tiled_kernel(
 
   const int cpg = g.channel / g.groups;
   const int out_plane = g.out_h * g.out_w, in_plane = H * W;
-  const BlockId b = decode_block(g, 1, ceil_div(cpg, NC));
+  const BlockId b = decode_block(g, BAND ? ceil_div(H, band_rows) : 1, ceil_div(cpg, NC));
   if (!b.valid) return;
   const int j0 = b.chunk * NC;
   const int nch = min(NC, cpg - j0);
+  // BAND: the image rows r_lo .. r_hi - 1 are this workgroup's; row r sits in LDS row r - r_lo (no padding rows),
+  // and an index `pidx` of the whole padded plane lies in one of its rows when lo_idx <= pidx < hi_idx
+  const int r_lo = BAND ? b.tile * band_rows : 0, r_hi = BAND ? min(H, r_lo + band_rows) : H;
+  const int lo_idx = BAND ? (r_lo + 1) * RS : 0, hi_idx = BAND ? (r_hi + 1) * RS : 0x7fffffff;
+  constexpr int ROWOFF = BAND ? 0 : 1;  // LDS row of the first image row
 
   for (int e = threadIdx.x; e < NP * PS; e += blockDim.x) planes[e] = 0ull;
   stage_wide_tables<T, SH, SW>(tbl, filter, g.channel, b.grp + g.groups * j0, g.groups, nch);
@@ -1317,11 +1377,21 @@ __global__ __launch_bounds__(1024) void deform_grad_input_tiled_kernel(
     return hits;
   };
   const int ntiles = ceil_div(out_plane, (int)blockDim.x);
+  // BAND: the tiles whose samples touch this band's rows (tile_rows: least and largest padded row of a tile's
+  // top corners, per image), and per sample whether its upper / lower corner pair lies in the band
+  auto tile_in_band = [&](int tile) {
+    if constexpr (!BAND) return true;
+    const int* tr = tile_rows + ((size_t)b.n * ntiles + tile) * 2;
+    return tr[0] - 1 < r_hi && tr[1] >= r_lo;  // image rows tr[0] - 1 .. tr[1]
+  };
+  auto top_in = [&](int pidx) { return !BAND || (pidx >= lo_idx && pidx < hi_idx); };
+  auto bot_in = [&](int pidx) { return !BAND || (pidx + RS >= lo_idx && pidx + RS < hi_idx); };
 
   // M: the largest number of samples on one input element, over the whole output plane
   {
     unsigned* count = reinterpret_cast<unsigned*>(planes);
     for (int tile = 0; tile < ntiles; ++tile) {
+      if (!tile_in_band(tile)) continue;
       ImgTap it[K9];
       LiteTap st[K9];
       unsigned goff;
@@ -1329,10 +1399,15 @@ __global__ __launch_bounds__(1024) void deform_grad_input_tiled_kernel(
 #pragma unroll
       for (int t = 0; t < K9; ++t) {
         if (hits >> t & 1u) {
-          atomicAdd(count + it[t].pidx, 1u);
-          atomicAdd(count + it[t].pidx + 1, 1u);
-          atomicAdd(count + it[t].pidx + RS, 1u);
-          atomicAdd(count + it[t].pidx + RS + 1, 1u);
+          const int at = it[t].pidx - lo_idx;
+          if (top_in(it[t].pidx)) {
+            atomicAdd(count + at, 1u);
+            atomicAdd(count + at + 1, 1u);
+          }
+          if (bot_in(it[t].pidx)) {
+            atomicAdd(count + at + RS, 1u);
+            atomicAdd(count + at + RS + 1, 1u);
+          }
         }
       }
     }
@@ -1355,6 +1430,7 @@ __global__ __launch_bounds__(1024) void deform_grad_input_tiled_kernel(
   if (head <= kPairHead) {
     // two channels per plane: channel 2 q in the low half, 2 q + 1 in the high half (see deform_grad_input_kernel)
     for (int tile = 0; tile < ntiles; ++tile) {
+      if (!tile_in_band(tile)) continue;
       ImgTap it[K9];
       LiteTap st[K9];
       unsigned goff;
@@ -1378,9 +1454,12 @@ __global__ __launch_bounds__(1024) void deform_grad_input_tiled_kernel(
             const float wb = gb_s * lite_weight(st[t], *reinterpret_cast<const float4*>(tb + st[t].cell));
             const float lh = it[t].lh, lw = it[t].lw, hh = 1.f - lh, hw = 1.f - lw;
             const float cw[4] = {hh * hw, hh * lw, lh * hw, lh * lw};  // K.cu:776-789
-            const int at[4] = {it[t].pidx, it[t].pidx + 1, it[t].pidx + RS, it[t].pidx + RS + 1};
+            const int a0 = it[t].pidx - lo_idx;
+            const int at[4] = {a0, a0 + 1, a0 + RS, a0 + RS + 1};
+            const bool in[2] = {top_in(it[t].pidx), bot_in(it[t].pidx)};
 #pragma unroll
             for (int k = 0; k < 4; ++k) {
+              if (BAND && !in[k >> 1]) continue;
               const int ia = round_half_up(cw[k] * wa), ib = round_half_up(cw[k] * wb);
               const unsigned long long both =
                   ((unsigned long long)(unsigned)(ib + (ia >> 31)) << 32) | (unsigned long long)(unsigned)ia;
@@ -1400,13 +1479,13 @@ __global__ __launch_bounds__(1024) void deform_grad_input_tiled_kernel(
       const float ua = ldexpf(1.f, -sa), ub = ldexpf(1.f, -sb);
       const unsigned long long* pl = planes + (j >> 1) * PS;
       T* dst = ip + (size_t)j * i_step;
-      for (int row = sub; row < H; row += rpp) {
+      for (int row = sub; row < r_hi - r_lo; row += rpp) {
         if (col < W) {
-          const unsigned long long v = pl[(row + 1) * RS + 1 + col];
+          const unsigned long long v = pl[(row + ROWOFF) * RS + 1 + col];
           const int lo = (int)(unsigned)v;
           const int hi = (int)(unsigned)(v >> 32) + (lo < 0 ? 1 : 0);
-          dk::st(dst + row * W + col, (float)lo * ua);
-          if (pair) dk::st(dst + i_step + row * W + col, (float)hi * ub);
+          dk::st(dst + (r_lo + row) * W + col, (float)lo * ua);
+          if (pair) dk::st(dst + i_step + (r_lo + row) * W + col, (float)hi * ub);
         }
       }
     }
@@ -1417,6 +1496,7 @@ __global__ __launch_bounds__(1024) void deform_grad_input_tiled_kernel(
   for (int c0 = 0; c0 < nch; c0 += NP) {
     const int nc = min(NP, nch - c0);
     for (int tile = 0; tile < ntiles; ++tile) {
+      if (!tile_in_band(tile)) continue;
       ImgTap it[K9];
       LiteTap st[K9];
       unsigned goff;
@@ -1436,9 +1516,12 @@ __global__ __launch_bounds__(1024) void deform_grad_input_tiled_kernel(
             const float gw = gv * lite_weight(st[t], q);
             const float lh = it[t].lh, lw = it[t].lw, hh = 1.f - lh, hw = 1.f - lw;
             const float term[4] = {hh * hw * gw, hh * lw * gw, lh * hw * gw, lh * lw * gw};
-            const int at[4] = {it[t].pidx, it[t].pidx + 1, it[t].pidx + RS, it[t].pidx + RS + 1};
+            const int a0 = it[t].pidx - lo_idx;
+            const int at[4] = {a0, a0 + 1, a0 + RS, a0 + RS + 1};
+            const bool in[2] = {top_in(it[t].pidx), bot_in(it[t].pidx)};
 #pragma unroll
             for (int k = 0; k < 4; ++k) {
+              if (BAND && !in[k >> 1]) continue;
               const double d = fma((double)term[k], scale, kMagic);
               atomicAdd(pl + at[k], (unsigned long long)__double_as_longlong(d) - 0x4338000000000000ull);
             }
@@ -1454,10 +1537,10 @@ __global__ __launch_bounds__(1024) void deform_grad_input_tiled_kernel(
       const double unscale = ldexp(1.0, e - 44);
       unsigned long long* pl = planes + jj * PS;
       T* dst = ip + (size_t)j * i_step;
-      for (int row = sub; row < H; row += rpp) {
+      for (int row = sub; row < r_hi - r_lo; row += rpp) {
         if (col < W) {
-          unsigned long long* cell = pl + (row + 1) * RS + 1 + col;
-          dk::st(dst + row * W + col, (float)((double)(long long)*cell * unscale));
+          unsigned long long* cell = pl + (row + ROWOFF) * RS + 1 + col;
+          dk::st(dst + (r_lo + row) * W + col, (float)((double)(long long)*cell * unscale));
           *cell = 0ull;  // for the next walk
         }
       }
@@ -2382,7 +2465,10 @@ DeformPlan deform_plan_chw(const Geo& g, int table_floats, int block, int npass)
   const long positions = (kDBigLds - table_bytes) / 2 / (kDeformCh * 4) - (RS + 2);
   const long wr = std::min<long>({(long)g.in_h + 2, positions / RS, (long)npass * rpp});
   const long own = (long)(ceil_div(block, g.out_w) + 1) * g.stride_h + 2L * g.dil_h + 2;  // rows without offsets
-  if (wr < std::min<long>(g.in_h + 2, own + 8)) return d;
+  // (planes the one-plane kernels cannot take either -- 224 x 224: two padded copies do not fit LDS -- settle
+  // for a smaller margin: the alternative there is the generic kernel)
+  const long margin = deform_plan_wide(g, table_floats).ok ? 8 : 2;
+  if (wr < std::min<long>(g.in_h + 2, own + margin)) return d;
   d.wr = (int)wr;
   d.lds = (size_t)(2 * (wr * RS + RS + 2) * kDeformCh * 4 + table_bytes);
   d.ok = true;
@@ -2568,6 +2654,25 @@ int tiled_planes(const DeformPlan& basic, size_t* lds) {
   return 0;
 }
 
+// Band form of the tiled grad input: 64-bit planes per workgroup (4, 2 or 1) and rows per band, the largest
+// plane count that leaves bands of at least kBandRows rows (fewer rows: every tile is walked by many bands); 0 if
+// not even one plane of 8 rows fits.
+constexpr int kBandRows = 20;
+template <int SH, int SW>
+int band_planes(const Geo& g, int* rows, size_t* lds) {
+  const long RS = g.in_w + 2;
+  for (int np = 4; np >= 1; np >>= 1) {
+    const long fixed = ((long)2 * np * WideTable<SH, SW>::SIZE + 2 * np) * 4 + 64;
+    const long r = std::min<long>(g.in_h, (150L * 1024 - fixed) / (np * RS * 8) - 1);
+    if (r >= std::min<long>(g.in_h, np == 1 ? 8 : kBandRows)) {
+      *rows = (int)r;
+      *lds = (size_t)(2 * np * (((r * RS + 3) & ~3L)) * 4 + fixed);
+      return np;
+    }
+  }
+  return 0;
+}
+
 template <typename T, int SH, int SW>
 bool run_deform_grad_input(const Geo& g, const T* gout, const T* off, const T* rot, const T* filter, T* gin,
                            void* ws, hipStream_t stream) {
@@ -2581,7 +2686,30 @@ bool run_deform_grad_input(const Geo& g, const T* gout, const T* off, const T* r
     if (!basic.ok) return false;
     tiled_shift = basic.shift;
     tiled_ch = tiled_planes<SH, SW>(basic, &tiled_lds);
-    if (tiled_ch == 0) return false;
+    if (tiled_ch == 0) {
+      // not even one plane fits: bands of rows
+      if (reinterpret_cast<uintptr_t>(gout) % 16 != 0 || path_disabled(kNoDeformWindow)) return false;
+      size_t lds = 0;
+      int rows = 0;
+      const int np = band_planes<SH, SW>(g, &rows, &lds);
+      if (np == 0) return false;
+      unsigned* gmax_ = static_cast<unsigned*>(ws);
+      int* table = reinterpret_cast<int*>(gmax_ + kAbsParts);
+      const int ntiles = ceil_div(g.out_h * g.out_w, 1024), cpg_ = g.channel / g.groups;
+      const long count = (long)g.batch * g.channel * g.out_h * g.out_w;
+      const unsigned bgrid = (unsigned)xcd_grid_size((long)ceil_div(g.in_h, rows) * ceil_div(cpg_, 2 * np) * g.batch * g.groups);
+#define DK_LAUNCH(CH)                                                                                              \
+  {                                                                                                                \
+    auto kernel = deform_grad_input_tiled_kernel<T, SH, SW, CH, true>;                                             \
+    if (!allow_max_dynamic_lds(reinterpret_cast<const void*>(kernel))) return false;                               \
+    absmax_kernel<T><<<kAbsParts, 256, 0, stream>>>(gout, count, gmax_);                                           \
+    deform_tile_rows_kernel<T><<<(unsigned)(g.batch * ntiles), 1024, 0, stream>>>(g, off, table, ntiles);          \
+    kernel<<<bgrid, 1024, lds, stream>>>(g, gout, off, rot, filter, gin, gmax_, tiled_shift, rows, table);         \
+  }
+      if (np == 4) DK_LAUNCH(4) else if (np == 2) DK_LAUNCH(2) else DK_LAUNCH(1)
+#undef DK_LAUNCH
+      return true;
+    }
   }
   if (reinterpret_cast<uintptr_t>(gout) % 16 != 0) return false;  // absmax_kernel reads 16-byte vectors
   unsigned* gmax = static_cast<unsigned*>(ws);
@@ -2594,7 +2722,7 @@ bool run_deform_grad_input(const Geo& g, const T* gout, const T* off, const T* r
     auto kernel = deform_grad_input_tiled_kernel<T, SH, SW, CH>;                                        \
     if (!allow_max_dynamic_lds(reinterpret_cast<const void*>(kernel))) return false;                    \
     absmax_kernel<T><<<kAbsParts, 256, 0, stream>>>(gout, n, gmax);                                     \
-    kernel<<<tgrid, 1024, tiled_lds, stream>>>(g, gout, off, rot, filter, gin, gmax, tiled_shift);      \
+    kernel<<<tgrid, 1024, tiled_lds, stream>>>(g, gout, off, rot, filter, gin, gmax, tiled_shift, 0, nullptr); \
   }
     if (tiled_ch == 4) DK_LAUNCH(4) else if (tiled_ch == 2) DK_LAUNCH(2) else DK_LAUNCH(1)
 #undef DK_LAUNCH
@@ -2844,8 +2972,8 @@ bool fast_deform_grad_input(const Geo& g, const T* gout, const T* off, const T* 
 }
 
 size_t fast_deform_grad_input_workspace(const Geo& g) {
-  (void)g;
-  return (size_t)kAbsParts * sizeof(unsigned);  // absmax_kernel's per-workgroup maxima of |gout|
+  // absmax_kernel's per-workgroup maxima of |gout|, then the band form's table of two rows per (image, tile)
+  return (size_t)kAbsParts * sizeof(unsigned) + (size_t)g.batch * ceil_div(g.out_h * g.out_w, 1024) * 2 * sizeof(int);
 }
 
 template <typename T>

@@ -42,6 +42,8 @@ CASES = [
     (2, 33, 56, 56, 3, (5, 5), 1, 1, 1, 1, 1.0, 2.0),     # row-window grad filter, scope 5 (two launches of 16 cells), three channel blocks
     (1, 6, 120, 100, 3, (4, 4), 1, 1, 1, 1, 0.7, 15.0),   # row-window channel-interleaved kernels (100 columns): offsets of fifteen rows, four windows of 32 rows per tile; two channel tuples
     (2, 9, 70, 96, 3, (3, 3), 1, 1, 1, 3, 0.6, 2.0),      # the same kernels in one pass: three groups of three channels, scope 3
+    (1, 10, 224, 224, 3, (4, 4), 1, 1, 1, 1, 0.7, 2.0),   # 224 x 224: no padded plane fits LDS; grad input in bands of 20 rows (a chunk of 8 channels and one of 2), row windows with the smaller margin
+    (1, 6, 150, 200, 3, (4, 4), 2, 1, 1, 2, 0.6, 12.0),   # the band form at stride 2 with offsets of twelve rows (every band walks many tiles), two groups of three channels
 ]
 NAMES = ("forward", "grad input", "grad offset", "grad rotation", "grad filter")
 
@@ -75,11 +77,11 @@ def assert_fp32_parity(got, o32, o64):
     # The offset gradient is the slope of the bilinear patch a sample falls in, so it jumps where a
     # sampling position crosses a grid line; a position that fp32 rounds onto the line (36 + 0.9999987
     # = 37.0f) lies in the next patch than in fp64.  Each element must match one of the two oracles,
-    # and all but a few the fp64 one.
+    # and all but a few the fp64 one (a few per million samples: the bound grows with the tensor).
     g = got[2].double().numpy()
     err = np.minimum(np.abs(g - o64[2]), np.abs(g - o32[2].astype(np.float64)))
     assert err.max() / np.abs(o64[2]).max() < 1e-4, NAMES[2]
-    assert np.count_nonzero(np.abs(g - o64[2]) > 1e-4 * np.abs(o64[2]).max()) <= 2, NAMES[2]
+    assert np.count_nonzero(np.abs(g - o64[2]) > 1e-4 * np.abs(o64[2]).max()) <= 2 + g.size // 250000, NAMES[2]
 
 
 @pytest.mark.parametrize("case", CASES)
@@ -97,7 +99,7 @@ def test_fp64_matches_oracle(case):
 
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
-@pytest.mark.parametrize("case", CASES[:3] + [CASES[10], CASES[13], CASES[14], CASES[16], CASES[17]])   # planes above 30 x 30; the last two wider than 64 columns
+@pytest.mark.parametrize("case", CASES[:3] + [CASES[10], CASES[13], CASES[14], CASES[16], CASES[17], CASES[24]])   # planes above 30 x 30; wider than 64 columns; 224 x 224
 def test_half_precisions_match_fp32_oracle(case, dtype):
     inputs, got = _run(case, dtype)
     want = _oracle(inputs, np.float32)
@@ -228,7 +230,8 @@ def test_config4_properties_at_full_size():
 @pytest.mark.parametrize("switch,case", [("DK_NO_DEFORM_CH", CASES[0]), ("DK_NO_DEFORM_MFMA", CASES[0]),
                                          ("DK_NO_DEFORM_CH_BIG", CASES[7]), ("DK_NO_DEFORM_WINDOW", CASES[13]),
                                          ("DK_NO_DEFORM_WINDOW", CASES[20]), ("DK_NO_DEFORM_WINDOW", CASES[16]),
-                                         ("DK_NO_DEFORM_WINDOW", CASES[22]), ("DK_FORCE_WIN2", CASES[13]),
+                                         ("DK_NO_DEFORM_WINDOW", CASES[22]), ("DK_NO_DEFORM_WINDOW", CASES[25]),
+                                         ("DK_FORCE_WIN2", CASES[13]),
                                          ("DK_FORCE_WIN2", CASES[20]), ("DK_FORCE_WIN2", CASES[21]),
                                          ("DK_FORCE_WIN2", CASES[9])])
 def test_one_plane_kernels_on_a_shape_the_newer_ones_cover(switch_off, switch, case):
@@ -250,7 +253,7 @@ def test_generic_kernels_on_a_shape_the_tuned_ones_cover(switch_off):
         assert rel_err(got[i], o64[i]) < 1e-4, NAMES[i]
 
 
-@pytest.mark.parametrize("case", [CASES[0], CASES[10]])  # one plane per workgroup; tiled planes above 1024 pixels
+@pytest.mark.parametrize("case", [CASES[0], CASES[10], CASES[24]])  # one plane per workgroup; tiled planes above 1024 pixels; bands of rows
 @pytest.mark.parametrize("poison", [float("inf"), float("nan")])
 @pytest.mark.parametrize("where", ["out_grad", "filter"])
 def test_non_finite_values_reach_the_input_gradient(case, poison, where):
