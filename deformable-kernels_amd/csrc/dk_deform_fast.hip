@@ -2686,13 +2686,14 @@ bool run_deform_grad_input(const Geo& g, const T* gout, const T* off, const T* r
     if (!basic.ok) return false;
     tiled_shift = basic.shift;
     tiled_ch = tiled_planes<SH, SW>(basic, &tiled_lds);
-    if (tiled_ch == 0) {
-      // not even one plane fits: bands of rows
+    if (tiled_ch <= 1) {
+      // not even one plane fits, or only one (two channels per workgroup and walk): bands of rows
       if (reinterpret_cast<uintptr_t>(gout) % 16 != 0 || path_disabled(kNoDeformWindow)) return false;
       size_t lds = 0;
       int rows = 0;
       const int np = band_planes<SH, SW>(g, &rows, &lds);
-      if (np == 0) return false;
+      if (np == 0 && tiled_ch == 0) return false;
+      if (np >= 2 || tiled_ch == 0) {
       unsigned* gmax_ = static_cast<unsigned*>(ws);
       int* table = reinterpret_cast<int*>(gmax_ + kAbsParts);
       const int ntiles = ceil_div(g.out_h * g.out_w, 1024), cpg_ = g.channel / g.groups;
@@ -2709,6 +2710,7 @@ bool run_deform_grad_input(const Geo& g, const T* gout, const T* off, const T* r
       if (np == 4) DK_LAUNCH(4) else if (np == 2) DK_LAUNCH(2) else DK_LAUNCH(1)
 #undef DK_LAUNCH
       return true;
+      }
     }
   }
   if (reinterpret_cast<uintptr_t>(gout) % 16 != 0) return false;  // absmax_kernel reads 16-byte vectors
