@@ -1061,8 +1061,10 @@ __device__ __forceinline__ bool write_nan_if_unbounded(float gmax, const float* 
   return true;
 }
 
-// Two channels share a 64-bit sum while at most 2^kPairHead samples touch one input element.
-constexpr int kPairHead = 6;
+// Two channels share a 64-bit sum while at most 2^kPairHead samples touch one input element: a term is then
+// rounded on a grid of 2^-(31 - kPairHead) = 2^-24 of the largest possible term or finer.  (3 x 3 taps at stride 1
+// put 36 samples on an element on average and about 65 on the fullest element of a large plane.)
+constexpr int kPairHead = 7;
 
 // floor(v + 0.5) as a signed 32-bit integer, one instruction
 __device__ __forceinline__ int round_half_up(float v) {
@@ -1259,7 +1261,7 @@ __global__ __launch_bounds__(1024) void deform_grad_input_kernel(
 // ---------------------------------------------------------------------------
 template <typename T>
 __global__ __launch_bounds__(1024) void deform_tile_rows_kernel(Geo g, const T* __restrict__ off, int* __restrict__ table,
-                                                                int ntiles) {
+                                                                int ntiles, unsigned* __restrict__ most_img) {
   __shared__ int wave_lo[16], wave_hi[16];
   const int out_plane = g.out_h * g.out_w;
   const int tile = blockIdx.x % ntiles, n = blockIdx.x / ntiles;
@@ -1297,6 +1299,73 @@ __global__ __launch_bounds__(1024) void deform_tile_rows_kernel(Geo g, const T* 
     }
     table[(size_t)blockIdx.x * 2] = lo;
     table[(size_t)blockIdx.x * 2 + 1] = hi;
+    if (tile == 0) most_img[n] = 0u;  // deform_sample_count_kernel, next on the stream, takes maxima into it
+  }
+}
+
+// ---------------------------------------------------------------------------
+// most_img[image] = an upper bound of the number of samples whose bilinear footprint covers one input element
+// (every sample that hits the image counts, also where its scope coordinate leaves the scope band and the
+// operator adds nothing).  A workgroup holds a 32-bit histogram of a band of `band_rows` image rows in LDS
+// (the whole plane where it fits), walks the tiles that touch it and sends the band's maximum.
+// grid = image * bands
+// ---------------------------------------------------------------------------
+template <typename T>
+__global__ __launch_bounds__(1024) void deform_sample_count_kernel(Geo g, const T* __restrict__ off,
+                                                                   const int* __restrict__ tile_rows,
+                                                                   unsigned* __restrict__ most_img, int ntiles,
+                                                                   int band_rows) {
+  extern __shared__ __align__(16) float lds[];
+  unsigned* count = reinterpret_cast<unsigned*>(lds);
+  __shared__ unsigned wave_most[16];
+  const int H = g.in_h, W = g.in_w, RS = W + 2;
+  const int out_plane = g.out_h * g.out_w;
+  const int nbands = ceil_div(H, band_rows);
+  const int band = blockIdx.x % nbands, n = blockIdx.x / nbands;
+  const int r_lo = band * band_rows, r_hi = min(H, r_lo + band_rows);
+  const int lo_idx = (r_lo + 1) * RS, hi_idx = (r_hi + 1) * RS;
+  const int cells = band_rows * RS;
+  for (int e = threadIdx.x; e < cells; e += 1024) count[e] = 0u;
+  __syncthreads();
+  const rsrc_t ro = plane_rsrc(off + (size_t)n * (K9 * 2) * out_plane, K9 * 2 * out_plane);
+  const unsigned step = (unsigned)out_plane * (unsigned)sizeof(T);
+  for (int tile = 0; tile < ntiles; ++tile) {
+    const int* tr = tile_rows + ((size_t)n * ntiles + tile) * 2;
+    if (!(tr[0] - 1 < r_hi && tr[1] >= r_lo)) continue;  // uniform over the workgroup
+    const int p = tile * 1024 + threadIdx.x;
+    const bool live = p < out_plane;
+    const int pc = live ? p : 0;
+    const int oh = pc / g.out_w, ow = pc % g.out_w;
+#pragma unroll
+    for (int t = 0; t < K9; ++t) {
+      const int f_h = t / 3, f_w = t % 3;
+      const unsigned o = live ? (unsigned)((2 * t) * out_plane + pc) * (unsigned)sizeof(T) : kOutOfRange;
+      const float h = float(oh * g.stride_h - g.pad_h + f_h * g.dil_h) + buf_ld(ro, o, off);
+      const float w = float(ow * g.stride_w - g.pad_w + f_w * g.dil_w) + buf_ld(ro, o + step, off);
+      const bool hit = live && (h > -1.f) && (w > -1.f) && (h < float(H)) && (w < float(W));
+      if (hit) {
+        const int pidx = (static_cast<int>(floorf(h)) + 1) * RS + static_cast<int>(floorf(w)) + 1;
+        const int at = pidx - lo_idx;
+        if (pidx >= lo_idx && pidx < hi_idx) {
+          atomicAdd(count + at, 1u);
+          atomicAdd(count + at + 1, 1u);
+        }
+        if (pidx + RS >= lo_idx && pidx + RS < hi_idx) {
+          atomicAdd(count + at + RS, 1u);
+          atomicAdd(count + at + RS + 1, 1u);
+        }
+      }
+    }
+  }
+  __syncthreads();
+  unsigned most = 0u;
+  for (int e = threadIdx.x; e < cells; e += 1024) most = max(most, count[e]);
+  for (int sft = 32; sft > 0; sft >>= 1) most = max(most, (unsigned)__shfl_xor((int)most, sft));
+  if ((threadIdx.x & 63) == 0) wave_most[threadIdx.x >> 6] = most;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    for (int w = 1; w < 16; ++w) most = max(most, wave_most[w]);
+    atomicMax(most_img + n, most);
   }
 }
 
@@ -1304,10 +1373,12 @@ __global__ __launch_bounds__(1024) void deform_tile_rows_kernel(Geo g, const T* 
 // grad input for output planes of more than 1024 pixels, or input planes the kernel above has no room for.  The
 // same fixed-point LDS accumulation, but the workgroup (1024 threads) owns 2 NP channels of an image and NP 64-bit
 // planes; it walks the output plane in tiles of 1024 pixels, computes a tile's tap descriptors once and adds the
-// tile's contributions for each of its channels.  A first walk over the tiles counts the samples per input element
-// (M, as above): while M <= 2^kPairHead two channels share a plane, each as a signed 32-bit term in its half
-// of the 64-bit sum, and one walk serves all 2 NP channels; otherwise every channel gets a plane of its own on the
-// 2^-44 grid and the channels take two walks.  The planes are read back at the end of a walk.
+// tile's contributions for each of its channels.  M, the largest number of samples on one input element (as above),
+// comes per image from deform_sample_count_kernel -- every workgroup of an image repeating that walk took 9 % of
+// this kernel on 56 x 56 planes and 28 - 38 % of its band form: while M <= 2^kPairHead two channels share a plane,
+// each as a signed 32-bit term in its half of the 64-bit sum, and one walk serves all 2 NP channels; otherwise
+// every channel gets a plane of its own on the 2^-44 grid and the channels take two walks.  The planes are read
+// back at the end of a walk.
 // BAND: input planes that do not fit LDS even once (224 x 224).  A workgroup owns a band of `band_rows` image rows
 // (of all columns) instead of the whole plane: it walks the tiles whose samples touch the band -- found in a table of
 // each tile's least and largest sample row, written by deform_tile_rows_kernel -- and adds the corner pairs that lie
@@ -1319,7 +1390,7 @@ template <typename T, int SH, int SW, int NP, bool BAND = false>
 __global__ __launch_bounds__(1024) void deform_grad_input_tiled_kernel(
     Geo g, const T* __restrict__ gout, const T* __restrict__ off, const T* __restrict__ rot,
     const T* __restrict__ filter, T* __restrict__ gin, const unsigned* __restrict__ gmax_bits, int shift,
-    int band_rows, const int* __restrict__ tile_rows) {
+    int band_rows, const int* __restrict__ tile_rows, const unsigned* __restrict__ most_img) {
   using Tb = WideTable<SH, SW>;
   constexpr int NC = 2 * NP;  // channels per workgroup
   extern __shared__ __align__(16) float lds[];
@@ -1328,7 +1399,6 @@ __global__ __launch_bounds__(1024) void deform_grad_input_tiled_kernel(
   unsigned long long* planes = reinterpret_cast<unsigned long long*>(lds);  // [NP][PS]
   float* tbl = lds + 2 * NP * PS;                                           // [NC][Tb::SIZE]
   float* wmax = tbl + NC * Tb::SIZE;                                        // [NC]
-  __shared__ unsigned wave_most[16];
 
   const int cpg = g.channel / g.groups;
   const int out_plane = g.out_h * g.out_w, in_plane = H * W;
@@ -1380,49 +1450,14 @@ __global__ __launch_bounds__(1024) void deform_grad_input_tiled_kernel(
   // BAND: the tiles whose samples touch this band's rows (tile_rows: least and largest padded row of a tile's
   // top corners, per image), and per sample whether its upper / lower corner pair lies in the band
   auto tile_in_band = [&](int tile) {
-    if constexpr (!BAND) return true;
     const int* tr = tile_rows + ((size_t)b.n * ntiles + tile) * 2;
-    return tr[0] - 1 < r_hi && tr[1] >= r_lo;  // image rows tr[0] - 1 .. tr[1]
+    return tr[0] - 1 < r_hi && tr[1] >= r_lo;  // image rows tr[0] - 1 .. tr[1] (a tile without samples: none)
   };
   auto top_in = [&](int pidx) { return !BAND || (pidx >= lo_idx && pidx < hi_idx); };
   auto bot_in = [&](int pidx) { return !BAND || (pidx + RS >= lo_idx && pidx + RS < hi_idx); };
 
-  // M: the largest number of samples on one input element, over the whole output plane
-  {
-    unsigned* count = reinterpret_cast<unsigned*>(planes);
-    for (int tile = 0; tile < ntiles; ++tile) {
-      if (!tile_in_band(tile)) continue;
-      ImgTap it[K9];
-      LiteTap st[K9];
-      unsigned goff;
-      const unsigned hits = tile_taps(tile, it, st, goff);
-#pragma unroll
-      for (int t = 0; t < K9; ++t) {
-        if (hits >> t & 1u) {
-          const int at = it[t].pidx - lo_idx;
-          if (top_in(it[t].pidx)) {
-            atomicAdd(count + at, 1u);
-            atomicAdd(count + at + 1, 1u);
-          }
-          if (bot_in(it[t].pidx)) {
-            atomicAdd(count + at + RS, 1u);
-            atomicAdd(count + at + RS + 1, 1u);
-          }
-        }
-      }
-    }
-    __syncthreads();
-    unsigned most = 1u;
-    for (int e = threadIdx.x; e < PS; e += blockDim.x) {
-      most = max(most, count[e]);
-      count[e] = 0u;
-    }
-    for (int sft = 32; sft > 0; sft >>= 1) most = max(most, (unsigned)__shfl_xor((int)most, sft));
-    if ((threadIdx.x & 63) == 0) wave_most[threadIdx.x >> 6] = most;
-    __syncthreads();
-  }
-  unsigned most = 1u;
-  for (int w = 0; w < (int)blockDim.x / 64; ++w) most = max(most, wave_most[w]);
+  // M: an upper bound of the number of samples on one input element of this image (deform_sample_count_kernel)
+  const unsigned most = max(1u, most_img[b.n]);
   const int head = most <= 1u ? 0 : 32 - __builtin_clz(most - 1u);  // ceil(log2(most))
   const int col = threadIdx.x & ((1 << shift) - 1), sub = threadIdx.x >> shift;
   const int rpp = (int)blockDim.x >> shift;
@@ -2686,47 +2721,45 @@ bool run_deform_grad_input(const Geo& g, const T* gout, const T* off, const T* r
     if (!basic.ok) return false;
     tiled_shift = basic.shift;
     tiled_ch = tiled_planes<SH, SW>(basic, &tiled_lds);
-    if (tiled_ch <= 1) {
-      // not even one plane fits, or only one (two channels per workgroup and walk): bands of rows
-      if (reinterpret_cast<uintptr_t>(gout) % 16 != 0 || path_disabled(kNoDeformWindow)) return false;
-      size_t lds = 0;
-      int rows = 0;
-      const int np = band_planes<SH, SW>(g, &rows, &lds);
-      if (np == 0 && tiled_ch == 0) return false;
-      if (np >= 2 || tiled_ch == 0) {
-      unsigned* gmax_ = static_cast<unsigned*>(ws);
-      int* table = reinterpret_cast<int*>(gmax_ + kAbsParts);
-      const int ntiles = ceil_div(g.out_h * g.out_w, 1024), cpg_ = g.channel / g.groups;
-      const long count = (long)g.batch * g.channel * g.out_h * g.out_w;
-      const unsigned bgrid = (unsigned)xcd_grid_size((long)ceil_div(g.in_h, rows) * ceil_div(cpg_, 2 * np) * g.batch * g.groups);
-#define DK_LAUNCH(CH)                                                                                              \
-  {                                                                                                                \
-    auto kernel = deform_grad_input_tiled_kernel<T, SH, SW, CH, true>;                                             \
-    if (!allow_max_dynamic_lds(reinterpret_cast<const void*>(kernel))) return false;                               \
-    absmax_kernel<T><<<kAbsParts, 256, 0, stream>>>(gout, count, gmax_);                                           \
-    deform_tile_rows_kernel<T><<<(unsigned)(g.batch * ntiles), 1024, 0, stream>>>(g, off, table, ntiles);          \
-    kernel<<<bgrid, 1024, lds, stream>>>(g, gout, off, rot, filter, gin, gmax_, tiled_shift, rows, table);         \
-  }
-      if (np == 4) DK_LAUNCH(4) else if (np == 2) DK_LAUNCH(2) else DK_LAUNCH(1)
-#undef DK_LAUNCH
-      return true;
-      }
-    }
   }
   if (reinterpret_cast<uintptr_t>(gout) % 16 != 0) return false;  // absmax_kernel reads 16-byte vectors
   unsigned* gmax = static_cast<unsigned*>(ws);
   const long n = (long)g.batch * g.channel * g.out_h * g.out_w;
   if (tiled) {
-    const int cpg = g.channel / g.groups;
-    const unsigned tgrid = (unsigned)xcd_grid_size((long)ceil_div(cpg, 2 * tiled_ch) * g.batch * g.groups);
-#define DK_LAUNCH(CH)                                                                                   \
-  {                                                                                                     \
-    auto kernel = deform_grad_input_tiled_kernel<T, SH, SW, CH>;                                        \
-    if (!allow_max_dynamic_lds(reinterpret_cast<const void*>(kernel))) return false;                    \
-    absmax_kernel<T><<<kAbsParts, 256, 0, stream>>>(gout, n, gmax);                                     \
-    kernel<<<tgrid, 1024, tiled_lds, stream>>>(g, gout, off, rot, filter, gin, gmax, tiled_shift, 0, nullptr); \
+    // workspace: the maxima of |gout|, the images' sample counts, the tiles' rows
+    unsigned* most_img = gmax + kAbsParts;
+    int* table = reinterpret_cast<int*>(most_img + g.batch);
+    const int ntiles = ceil_div(g.out_h * g.out_w, 1024), cpg = g.channel / g.groups;
+    // the counting kernel's bands: about 512 workgroups, of at least 8 rows, of at most what fits as 32-bit counters
+    const long cfit = (150L * 1024 / 4) / (g.in_w + 2) - 1;
+    const int cbands = std::max(1, std::min(g.in_h / 8, ceil_div(512, std::max(1, g.batch))));
+    const int crows = (int)std::min<long>(cfit, ceil_div(g.in_h, cbands));
+    auto count_kernel = deform_sample_count_kernel<T>;
+    if (crows < 1 || !allow_max_dynamic_lds(reinterpret_cast<const void*>(count_kernel))) return false;
+    // not even one 64-bit plane fits, or only one (two channels per workgroup and walk): bands of rows
+    size_t blds = 0;
+    int brows = 0;
+    const int bnp = tiled_ch <= 1 && !path_disabled(kNoDeformWindow) ? band_planes<SH, SW>(g, &brows, &blds) : 0;
+    const bool band = bnp >= 2 || (tiled_ch == 0 && bnp == 1);
+    if (!band && tiled_ch == 0) return false;
+    const int np = band ? bnp : tiled_ch;
+    const size_t lds = band ? blds : tiled_lds;
+    const unsigned tgrid = (unsigned)xcd_grid_size((long)(band ? ceil_div(g.in_h, brows) : 1) * ceil_div(cpg, 2 * np) * g.batch * g.groups);
+#define DK_LAUNCH(CH, BAND)                                                                                       \
+  {                                                                                                               \
+    auto kernel = deform_grad_input_tiled_kernel<T, SH, SW, CH, BAND>;                                            \
+    if (!allow_max_dynamic_lds(reinterpret_cast<const void*>(kernel))) return false;                              \
+    absmax_kernel<T><<<kAbsParts, 256, 0, stream>>>(gout, n, gmax);                                               \
+    deform_tile_rows_kernel<T><<<(unsigned)(g.batch * ntiles), 1024, 0, stream>>>(g, off, table, ntiles, most_img); \
+    count_kernel<<<(unsigned)(g.batch * ceil_div(g.in_h, crows)), 1024, (size_t)crows * (g.in_w + 2) * 4, stream>>>( \
+        g, off, table, most_img, ntiles, crows);                                                                  \
+    kernel<<<tgrid, 1024, lds, stream>>>(g, gout, off, rot, filter, gin, gmax, tiled_shift, brows, table, most_img); \
   }
-    if (tiled_ch == 4) DK_LAUNCH(4) else if (tiled_ch == 2) DK_LAUNCH(2) else DK_LAUNCH(1)
+    if (band) {
+      if (np == 4) DK_LAUNCH(4, true) else if (np == 2) DK_LAUNCH(2, true) else DK_LAUNCH(1, true)
+    } else {
+      if (np == 4) DK_LAUNCH(4, false) else if (np == 2) DK_LAUNCH(2, false) else DK_LAUNCH(1, false)
+    }
 #undef DK_LAUNCH
     return true;
   }
@@ -2974,8 +3007,10 @@ bool fast_deform_grad_input(const Geo& g, const T* gout, const T* off, const T* 
 }
 
 size_t fast_deform_grad_input_workspace(const Geo& g) {
-  // absmax_kernel's per-workgroup maxima of |gout|, then the band form's table of two rows per (image, tile)
-  return (size_t)kAbsParts * sizeof(unsigned) + (size_t)g.batch * ceil_div(g.out_h * g.out_w, 1024) * 2 * sizeof(int);
+  // absmax_kernel's per-workgroup maxima of |gout|, then the tiled form's sample count per image and its table of
+  // two rows per (image, tile)
+  return (size_t)kAbsParts * sizeof(unsigned) + (size_t)g.batch * sizeof(unsigned) +
+         (size_t)g.batch * ceil_div(g.out_h * g.out_w, 1024) * 2 * sizeof(int);
 }
 
 template <typename T>
