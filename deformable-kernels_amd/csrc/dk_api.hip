@@ -31,7 +31,7 @@ unsigned switches_from_environment() {
       {"DK_NO_FILTER_SPLIT", kNoFilterSplit}, {"DK_NO_IMAGE_FLAT", kNoImageFlat},
       {"DK_NO_ND_SMALL", kNoNdSmall}, {"DK_NO_NHWC_MFMA", kNoNhwcMfma},
       {"DK_FORCE_GATHER_MFMA", kForceGatherMfma}, {"DK_NO_PIXEL_LANES", kNoPixelLanes},
-      {"DK_FORCE_PIXEL_LANES", kForcePixelLanes}, {"DK_NO_OFFSET_PAIRS", kNoOffsetPairs}, {"DK_NO_OFFSET_WGRAD16", kNoOffsetWgrad16}, {"DK_NO_DEFORM_WINDOW", kNoDeformWindow}, {"DK_FORCE_WIN2", kForceWin2}, {"DK_NO_NHWC_STAGED", kNoNhwcStaged}, {"DK_FORCE_NHWC_GATHER_MFMA", kForceNhwcGatherMfma}};
+      {"DK_FORCE_PIXEL_LANES", kForcePixelLanes}, {"DK_NO_OFFSET_PAIRS", kNoOffsetPairs}, {"DK_NO_OFFSET_WGRAD16", kNoOffsetWgrad16}, {"DK_NO_DEFORM_WINDOW", kNoDeformWindow}, {"DK_FORCE_WIN2", kForceWin2}, {"DK_NO_NHWC_STAGED", kNoNhwcStaged}, {"DK_FORCE_NHWC_GATHER_MFMA", kForceNhwcGatherMfma}, {"DK_NO_IMAGE_PACKED", kNoImagePacked}};
   // a production process ignores these variables: they count only next to DK_ENABLE_TEST_SWITCHES=1
   const char* on = std::getenv("DK_ENABLE_TEST_SWITCHES");
   if (!on || on[0] != '1') return 0;

@@ -684,6 +684,234 @@ __global__ __launch_bounds__(kWave* kWaves) void image_conv3_flat_grad_weight_ke
   }
 }
 
+// ---------------------------------------------------------------------------
+// The flat kernels for 16-bit tensors whose rows are a multiple of 4 elements: the staged range stays packed (two
+// elements per LDS word, written as loaded: no conversion when it is staged, half the LDS traffic) and the sums
+// run on v_dot2_f32_{f16,bf16} (two products per instruction, fp32 accumulation).  With rows and planes of an even
+// number of elements the pair (x[c], x[c + 1]) of an even column c is one word.  An output of an even column takes
+// (w1, w2) . (x[c], x[c + 1]) + (0, w0) . (x[c - 2], x[c - 1]), one of an odd column (w0, w1) . (x[c - 1], x[c]) +
+// (w2, 0) . (x[c + 1], x[c + 2]): six instructions per output instead of nine multiply-adds.
+// ---------------------------------------------------------------------------
+__device__ __forceinline__ float dot2(unsigned a, unsigned b, float c, const __half*) {
+  typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+  return __builtin_amdgcn_fdot2(__builtin_bit_cast(h2, a), __builtin_bit_cast(h2, b), c, false);
+}
+__device__ __forceinline__ float dot2(unsigned a, unsigned b, float c, const bf16_t*) {
+  typedef __bf16 b2 __attribute__((ext_vector_type(2)));
+  return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(b2, a), __builtin_bit_cast(b2, b), c, false);
+}
+// (lo, hi) as two elements of the tensor's type in one word; the values are exact in that type
+__device__ __forceinline__ unsigned pack2(float lo, float hi, const __half*) {
+  typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+  return __builtin_bit_cast(unsigned, h2{static_cast<_Float16>(lo), static_cast<_Float16>(hi)});
+}
+__device__ __forceinline__ unsigned pack2(float lo, float hi, const bf16_t*) { return pack_bf16(lo, hi); }
+
+template <typename T, int NCH>
+struct FlatLoads16 : FlatLoads<T, NCH> {
+  // the chunks go to the tile as they are
+  __device__ __forceinline__ void commit16(unsigned* tile, const FlatUnit& u, int lane) const {
+#pragma unroll
+    for (int j = 0; j < NCH; ++j) {
+      const int chunk = lane + kWave * j;
+      if (chunk < u.chunks) *reinterpret_cast<u4*>(tile + (kFront + chunk * kPer<T>) / 2) = this->v[j];
+    }
+  }
+};
+
+__device__ __forceinline__ void zero_row16(unsigned* row, int w, int lane) {
+  for (int c = lane; c < w / 2; c += kWave) row[c] = 0u;
+}
+
+// The words of columns oc - 2 .. oc + 5 of PR + 2 consecutive staged rows (oc a multiple of 4); the element left
+// of column 0 and the one right of the last column read as zero (only the outer words can hold them).
+template <int PR>
+__device__ __forceinline__ void load_rows16(const unsigned* top, int w, int oc, unsigned (&x)[PR + 2][4]) {
+  const bool left = oc == 0, right = oc + kStrip == w;
+#pragma unroll
+  for (int i = 0; i < PR + 2; ++i) {
+#pragma unroll
+    for (int c = 0; c < 4; ++c) x[i][c] = top[(i * w) / 2 + c];
+    x[i][0] = left ? 0u : x[i][0];
+    x[i][3] = right ? 0u : x[i][3];
+  }
+}
+
+template <typename T, int NCH, int PR>
+__global__ __launch_bounds__(kWave* kWaves) void image_conv3_flat16_kernel(FlatConv a, const T* __restrict__ src,
+                                                                           const T* __restrict__ weight,
+                                                                           T* __restrict__ dst) {
+  extern __shared__ __align__(16) unsigned char lds_raw[];
+  const int lane = threadIdx.x & (kWave - 1);
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
+  const int first_plane = blockIdx.x * kWaves + wave, step = gridDim.x * kWaves;
+  if (first_plane >= a.planes) return;
+  unsigned* tile = reinterpret_cast<unsigned*>(lds_raw) + (size_t)wave * (a.tile_elems / 2);
+  const long total = (long)a.planes * a.hw;
+  const int strips = a.w / kStrip;
+  const int dro = kWave / strips, dso = kWave - dro * strips;
+  const long my_tap = tap_offset(a.wl, a.flip ? 8 - min(lane, 8) : min(lane, 8));
+  auto taps_of = [&](int plane) { return weight[(plane / a.channel) * a.wl.n + (plane % a.channel) * a.wl.c + my_tap]; };
+
+  FlatUnit cur = flat_unit<T>(a, first_plane, 0, true);
+  FlatLoads16<T, NCH> loads;
+  loads.issue(src, total, cur, lane);
+  T taps_next = taps_of(first_plane);
+  for (;;) {
+    loads.commit16(tile, cur, lane);
+    float taps_cur = ld(&taps_next);
+    asm volatile("" : "+v"(taps_cur));
+    // the halo rows above the first and below the last row of the plane (the range starts at an even element)
+    if (cur.r0 == 0) zero_row16(tile + (kFront + cur.shift) / 2, a.w, lane);
+    if (cur.r1 == a.h) zero_row16(tile + (kFront + cur.shift + (cur.r1 - cur.r0 + 1) * a.w) / 2, a.w, lane);
+    const bool more_bands = cur.band + 1 < a.bands;
+    const int next_plane = more_bands ? cur.plane : cur.plane + step;
+    const bool more = next_plane < a.planes;
+    const FlatUnit nxt = flat_unit<T>(a, more ? next_plane : cur.plane, more_bands ? cur.band + 1 : 0, true);
+    if (more) {
+      loads.issue(src, total, nxt, lane);
+      if (!more_bands) taps_next = taps_of(next_plane);
+    }
+    lds_sync();
+    float w9[9];
+#pragma unroll
+    for (int t = 0; t < 9; ++t) w9[t] = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, taps_cur), t));
+    unsigned wa[3], wb[3], wc[3], wd[3];  // (w1, w2), (0, w0), (w0, w1), (w2, 0) of each tap row
+#pragma unroll
+    for (int i = 0; i < 3; ++i) {
+      wa[i] = pack2(w9[3 * i + 1], w9[3 * i + 2], src);
+      wb[i] = pack2(0.f, w9[3 * i], src);
+      wc[i] = pack2(w9[3 * i], w9[3 * i + 1], src);
+      wd[i] = pack2(w9[3 * i + 2], 0.f, src);
+    }
+    T* dp = dst + (size_t)cur.plane * a.hw;
+    const unsigned* band = tile + (kFront + cur.shift - 2) / 2;  // column -2 of the halo row above the band's first row
+    const int items = (cur.r1 - cur.r0) / PR * strips;
+    int orow = lane / strips, os = lane - orow * strips;
+    for (int item = lane; item < items; item += kWave) {
+      const int oc = os * kStrip;
+      unsigned x[PR + 2][4];
+      load_rows16<PR>(band + (orow * PR * a.w + oc) / 2, a.w, oc, x);
+#pragma unroll
+      for (int pr = 0; pr < PR; ++pr) {
+        float acc[kStrip] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int i = 0; i < 3; ++i) {
+          const unsigned* r = x[pr + i];
+          acc[0] = dot2(r[1], wa[i], dot2(r[0], wb[i], acc[0], src), src);
+          acc[1] = dot2(r[1], wc[i], dot2(r[2], wd[i], acc[1], src), src);
+          acc[2] = dot2(r[2], wa[i], dot2(r[1], wb[i], acc[2], src), src);
+          acc[3] = dot2(r[2], wc[i], dot2(r[3], wd[i], acc[3], src), src);
+        }
+        store_strip<T, float>(dp + (size_t)(cur.r0 + orow * PR + pr) * a.w, oc, a.w, acc, true);
+      }
+      orow += dro;
+      os += dso;
+      if (os >= strips) {
+        os -= strips;
+        ++orow;
+      }
+    }
+    if (!more) break;
+    lds_sync();
+    cur = nxt;
+  }
+}
+
+// Kernel gradient of that shape: per staged row the three alignments of its pairs -- (x[c - 1], x[c]), (x[c], x[c + 1]),
+// (x[c + 1], x[c + 2]) for the even columns of the strip -- are formed once (v_alignbit_b32) and serve the three
+// tap rows that read the row; a pair of out_grad elements against a pair of inputs is one instruction.
+template <typename T, int NCH, int PR>
+__global__ __launch_bounds__(kWave* kWaves) void image_conv3_flat16_grad_weight_kernel(FlatConv a,
+                                                                                       const T* __restrict__ gout,
+                                                                                       const T* __restrict__ x,
+                                                                                       T* __restrict__ gweight) {
+  extern __shared__ __align__(16) unsigned char lds_raw[];
+  const int lane = threadIdx.x & (kWave - 1);
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
+  const int first_plane = blockIdx.x * kWaves + wave, step = gridDim.x * kWaves;
+  if (first_plane >= a.planes) return;
+  unsigned* xtile = reinterpret_cast<unsigned*>(lds_raw) + (size_t)wave * a.tile_elems;  // two tiles of tile_elems / 2 words
+  unsigned* gtile = xtile + a.tile_elems / 2;
+  const long total = (long)a.planes * a.hw;
+  const int strips = a.w / kStrip;
+  const int dro = kWave / strips, dso = kWave - dro * strips;
+
+  FlatUnit cur = flat_unit<T>(a, first_plane, 0, true), gcur = flat_unit<T>(a, first_plane, 0, false);
+  FlatLoads16<T, NCH> xl, gl;
+  xl.issue(x, total, cur, lane);
+  gl.issue(gout, total, gcur, lane);
+  float sum[9];
+#pragma unroll
+  for (int t = 0; t < 9; ++t) sum[t] = 0.f;
+  for (;;) {
+    xl.commit16(xtile, cur, lane);
+    gl.commit16(gtile, gcur, lane);
+    if (cur.r0 == 0) zero_row16(xtile + (kFront + cur.shift) / 2, a.w, lane);
+    if (cur.r1 == a.h) zero_row16(xtile + (kFront + cur.shift + (cur.r1 - cur.r0 + 1) * a.w) / 2, a.w, lane);
+    const bool more_bands = cur.band + 1 < a.bands;
+    const int next_plane = more_bands ? cur.plane : cur.plane + step;
+    const bool more = next_plane < a.planes;
+    const FlatUnit nxt = flat_unit<T>(a, more ? next_plane : cur.plane, more_bands ? cur.band + 1 : 0, true);
+    const FlatUnit gnxt = flat_unit<T>(a, more ? next_plane : cur.plane, more_bands ? cur.band + 1 : 0, false);
+    if (more) {
+      xl.issue(x, total, nxt, lane);
+      gl.issue(gout, total, gnxt, lane);
+    }
+    lds_sync();
+    const unsigned* band = xtile + (kFront + cur.shift - 2) / 2;
+    const unsigned* gband = gtile + (kFront + gcur.shift) / 2;
+    const int items = (cur.r1 - cur.r0) / PR * strips;
+    int orow = lane / strips, os = lane - orow * strips;
+    for (int item = lane; item < items; item += kWave) {
+      const int oc = os * kStrip;
+      unsigned xv[PR + 2][4];
+      load_rows16<PR>(band + (orow * PR * a.w + oc) / 2, a.w, oc, xv);
+      unsigned gv[PR][2];
+#pragma unroll
+      for (int pr = 0; pr < PR; ++pr)
+#pragma unroll
+        for (int p = 0; p < 2; ++p) gv[pr][p] = gband[((orow * PR + pr) * a.w + oc) / 2 + p];
+#pragma unroll
+      for (int r = 0; r < PR + 2; ++r) {
+        // pairs of the row for the taps' three columns, for the strip's columns (0, 1) and (2, 3)
+        const unsigned l0 = __builtin_amdgcn_alignbit(xv[r][1], xv[r][0], 16), l1 = __builtin_amdgcn_alignbit(xv[r][2], xv[r][1], 16);
+        const unsigned r1_ = __builtin_amdgcn_alignbit(xv[r][3], xv[r][2], 16);
+        const unsigned p0[3] = {l0, xv[r][1], l1}, p1[3] = {l1, xv[r][2], r1_};
+#pragma unroll
+        for (int i = 0; i < 3; ++i) {
+          const int pr = r - i;  // the output row that reads staged row r through tap row i
+          if (pr < 0 || pr >= PR) continue;
+#pragma unroll
+          for (int j = 0; j < 3; ++j)
+            sum[i * 3 + j] = dot2(gv[pr][1], p1[j], dot2(gv[pr][0], p0[j], sum[i * 3 + j], x), x);
+        }
+      }
+      orow += dro;
+      os += dso;
+      if (os >= strips) {
+        os -= strips;
+        ++orow;
+      }
+    }
+    if (!more_bands) {  // the plane is done
+      float mine = 0.f;
+#pragma unroll
+      for (int t = 0; t < 9; ++t) {
+        const float total_ = wave_sum(sum[t]);
+        mine = lane == t ? total_ : mine;
+        sum[t] = 0.f;
+      }
+      if (lane < 9)
+        st(gweight + (cur.plane / a.channel) * a.wl.n + (cur.plane % a.channel) * a.wl.c + tap_offset(a.wl, lane), mine);
+    }
+    if (!more) break;
+    lds_sync();
+    cur = nxt;
+    gcur = gnxt;
+  }
+}
+
 // ---- host side of the flat kernels ----------------------------------------------------------
 
 constexpr int kFlatElems = 2048;       // largest staged range of the convolution (elements, halo rows included)
@@ -745,6 +973,20 @@ bool launch_flat_conv(const Geo& g, const long* ws, bool flip, const T* src, con
     const dim3 grid(flat_grid(a)), block(kWave * kWaves);
     const bool w4 = a.vec_ok != 0;  // whole, aligned strips: one vector store each
     const bool patches = w4 && a.h % 4 == 0 && a.band_rows % 4 == 0;
+    if constexpr (sizeof(T) == 2) {
+      // 16-bit tensors with rows of a multiple of 4 elements: the packed kernels
+      if (w4 && a.w % kStrip == 0 && a.w >= kStrip && !path_disabled(kNoImagePacked)) {
+#define DK_FLAT16(NN)                                                                                                      \
+  if (patches) hipLaunchKernelGGL((image_conv3_flat16_kernel<T, NN, 4>), grid, block, lds, stream, a, src, weight, dst);      \
+  else hipLaunchKernelGGL((image_conv3_flat16_kernel<T, NN, 1>), grid, block, lds, stream, a, src, weight, dst)
+        if (nch == 1) { DK_FLAT16(1); }
+        else if (nch == 2) { DK_FLAT16(2); }
+        else if (nch == 4) { DK_FLAT16(4); }
+        else { DK_FLAT16(8); }
+#undef DK_FLAT16
+        return true;
+      }
+    }
 #define DK_FLAT(NN)                                                                                                        \
   if (patches) hipLaunchKernelGGL((image_conv3_flat_kernel<T, NN, true, 4>), grid, block, lds, stream, a, src, weight, dst);  \
   else if (w4) hipLaunchKernelGGL((image_conv3_flat_kernel<T, NN, true, 1>), grid, block, lds, stream, a, src, weight, dst);  \
@@ -772,6 +1014,18 @@ bool launch_flat_grad_weight(const Geo& g, const long* ws, const T* gout, const 
     const dim3 grid(flat_grid(a)), block(kWave * kWaves);
     const bool w4 = a.w % kStrip == 0;
     const bool patches = w4 && a.h % 4 == 0 && a.band_rows % 4 == 0;
+    if constexpr (sizeof(T) == 2) {
+      if (w4 && a.w >= kStrip && !path_disabled(kNoImagePacked)) {
+#define DK_FLAT16(NN)                                                                                                                  \
+  if (patches) hipLaunchKernelGGL((image_conv3_flat16_grad_weight_kernel<T, NN, 4>), grid, block, lds, stream, a, gout, x, gweight);   \
+  else hipLaunchKernelGGL((image_conv3_flat16_grad_weight_kernel<T, NN, 1>), grid, block, lds, stream, a, gout, x, gweight)
+        if (nch == 1) { DK_FLAT16(1); }
+        else if (nch == 2) { DK_FLAT16(2); }
+        else { DK_FLAT16(4); }
+#undef DK_FLAT16
+        return true;
+      }
+    }
 #define DK_FLAT(NN)                                                                                                                    \
   if (patches) hipLaunchKernelGGL((image_conv3_flat_grad_weight_kernel<T, NN, true, 4>), grid, block, lds, stream, a, gout, x, gweight); \
   else if (w4) hipLaunchKernelGGL((image_conv3_flat_grad_weight_kernel<T, NN, true, 1>), grid, block, lds, stream, a, gout, x, gweight); \

@@ -39,6 +39,7 @@ enum TestSwitch : unsigned {
   kForceWin2 = 1u << 21,        // DK_FORCE_WIN2         the rows-and-columns window form of that grad filter also where the row-window form applies
   kNoNhwcStaged = 1u << 22,     // DK_NO_NHWC_STAGED     the channels-last kernels that stage planar tiles in LDS / contract 32 channels per matrix instruction (the kernels named under DK_NO_NHWC_MFMA run instead)
   kForceNhwcGatherMfma = 1u << 23,  // DK_FORCE_NHWC_GATHER_MFMA  the channels-last matrix-core forward / grad input wherever it applies, not only where it is the faster kernel
+  kNoImagePacked = 1u << 24,    // DK_NO_IMAGE_PACKED    the packed flat-copy kernels of the per-image depthwise convolution on 16-bit tensors (the flat-copy kernels that unpack to fp32 run instead)
   kNoOffsetPairs = 1u << 18,    // DK_NO_OFFSET_PAIRS    the offset branch's convolution on float32 tensors as bfloat16 pairs (the fp32 matrix-instruction forward runs instead, the other passes are not offered)
 };
 unsigned test_switches();  // dk_api.hip

@@ -173,7 +173,7 @@ def workspace(nbytes, device):
 TEST_SWITCHES = ("DK_NO_ROWS", "DK_NO_MFMA", "DK_NO_MFMA_S2", "DK_NO_S2_QUADS", "DK_NO_DEFORM_FAST",
                  "DK_NO_DEFORM_CH", "DK_NO_DEFORM_CH_BIG", "DK_NO_DEFORM_MFMA", "DK_NO_ND_BINS", "DK_NO_ND_MFMA",
                  "DK_NO_GATHER_MFMA", "DK_NO_FILTER_SPLIT", "DK_NO_IMAGE_FLAT", "DK_NO_ND_SMALL", "DK_NO_NHWC_MFMA", "DK_FORCE_GATHER_MFMA",
-                 "DK_NO_PIXEL_LANES", "DK_FORCE_PIXEL_LANES", "DK_NO_OFFSET_PAIRS", "DK_NO_OFFSET_WGRAD16", "DK_NO_DEFORM_WINDOW", "DK_FORCE_WIN2", "DK_NO_NHWC_STAGED", "DK_FORCE_NHWC_GATHER_MFMA")
+                 "DK_NO_PIXEL_LANES", "DK_FORCE_PIXEL_LANES", "DK_NO_OFFSET_PAIRS", "DK_NO_OFFSET_WGRAD16", "DK_NO_DEFORM_WINDOW", "DK_FORCE_WIN2", "DK_NO_NHWC_STAGED", "DK_FORCE_NHWC_GATHER_MFMA", "DK_NO_IMAGE_PACKED")
 
 
 class test_switches:

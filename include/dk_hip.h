@@ -388,7 +388,7 @@ const char *dk_status_string(int status);
  * DK_NO_DEFORM_FAST, DK_NO_DEFORM_CH, DK_NO_DEFORM_CH_BIG, DK_NO_DEFORM_MFMA, DK_NO_ND_BINS,
  * DK_NO_ND_MFMA, DK_NO_GATHER_MFMA, DK_NO_FILTER_SPLIT, DK_NO_IMAGE_FLAT, DK_NO_ND_SMALL, DK_NO_NHWC_MFMA,
  * DK_FORCE_GATHER_MFMA, DK_NO_PIXEL_LANES, DK_FORCE_PIXEL_LANES, DK_NO_OFFSET_PAIRS, DK_NO_OFFSET_WGRAD16, DK_NO_DEFORM_WINDOW, DK_FORCE_WIN2, DK_NO_NHWC_STAGED,
- * DK_FORCE_NHWC_GATHER_MFMA.  The mask starts at 0; only a process
+ * DK_FORCE_NHWC_GATHER_MFMA, DK_NO_IMAGE_PACKED.  The mask starts at 0; only a process
  * started with DK_ENABLE_TEST_SWITCHES=1 in its environment also reads the environment variables of
  * those names, once, at the first call that consults the mask (a stray variable in a production
  * environment changes nothing).  This call replaces the mask and returns the previous one.

@@ -101,6 +101,21 @@ def test_16_bit_types_against_the_oracle_on_the_rounded_inputs(case, dtype):
         assert rel_err(a.float(), b) < 1e-2
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("case", [CASES[0], CASES[2], CASES[3], CASES[12]])
+def test_packed_16_bit_kernels_against_the_kernels_that_unpack(case, dtype, switch_off):
+    """16-bit tensors with rows of a multiple of 4 elements stay packed in LDS and are summed two products per
+    instruction (fp32 sums); switched off, the flat-copy kernels that unpack to fp32 serve the shapes.  Both
+    sum in fp32 and round once, so they differ by the result's last bit at most, and both meet the oracle."""
+    got, want = _run(case, dtype, seed=11)
+    switch_off("DK_NO_IMAGE_PACKED")
+    got2, _ = _run(case, dtype, seed=11)
+    ulp = 2.0 ** -10 if dtype == torch.float16 else 2.0 ** -7
+    for a, b, w in zip(got, got2, want):
+        assert rel_err(a.float(), w) < 1e-2 and rel_err(b.float(), w) < 1e-2
+        assert ((a.float() - b.float()).abs() <= ulp * b.float().abs() + 1e-6 * b.float().abs().max()).all()
+
+
 def test_configuration_3_shape_float16_matches_the_grouped_convolution_it_replaces():
     """N=128, C=256, 28x28, 3x3 kernels per (image, channel), float16: the oracle on three images, and
     the framework's convolution with N * C groups (the reference's call) on the whole batch."""
