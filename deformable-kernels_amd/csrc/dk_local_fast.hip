@@ -1172,13 +1172,14 @@ __global__ __launch_bounds__(kMfBlock, 4) void local_grad_filter_mfma_kernel(
       const rsrc_t rx = plane_rsrc(x + (size_t)n * in_plane * C, in_plane * C);
       const rsrc_t rg = plane_rsrc(gout + (size_t)n * out_plane * C, out_plane * C);
       const int c4 = cb * kMfCh + 4 * cl_q;
-      const unsigned co = c4 < C ? (unsigned)c4 * (unsigned)sizeof(T) : kOutOfRange;
+      const bool quad = c4 < C;
+      const unsigned co = (unsigned)c4 * (unsigned)sizeof(T);
 #pragma unroll
       for (int k = 0; k < NX / 2; ++k) {
         const int e = x0 + cl_p + kMfPix * k;
-        c_x[k] = raw_ld4(rx, e < 0 ? kOutOfRange : (unsigned)(e * C) * (unsigned)sizeof(T) + co, x);
+        c_x[k] = raw_ld4(rx, e < 0 || !quad ? kOutOfRange : (unsigned)(e * C) * (unsigned)sizeof(T) + co, x);
       }
-      c_g = raw_ld4(rg, (unsigned)((p0 + cl_p) * C) * (unsigned)sizeof(T) + co, gout);
+      c_g = raw_ld4(rg, quad ? (unsigned)((p0 + cl_p) * C) * (unsigned)sizeof(T) + co : kOutOfRange, gout);
       return;
     }
 #pragma unroll
