@@ -1718,7 +1718,7 @@ bool run_grad_filter(const Geo& g, const T* gout, const T* x, const T* rot, T* g
   if (f.th > 0) {                                                                                                \
     if constexpr (CL) return false;                                                                              \
     else {                                                                                                       \
-    auto kernel = local_grad_filter_mfma_kernel<T, SH, SW, CELL0, kMfXS2, true, BF, false>; /* stride 2: no split form yet */                      \
+    auto kernel = local_grad_filter_mfma_kernel<T, SH, SW, CELL0, kMfXS2, true, BF, SP>;                                                           \
     if (!allow_max_dynamic_lds(reinterpret_cast<const void*>(kernel)))                                                           \
       return false;                                                                                              \
     kernel<<<grid, kMfBlock, f.lds, stream>>>(g, gout, x, rot, ws, f.tiles, f.parts, f.splits, f.pitch_x, f.th); \
@@ -1728,7 +1728,8 @@ bool run_grad_filter(const Geo& g, const T* gout, const T* x, const T* rot, T* g
   else                                                                                                           \
     local_grad_filter_mfma_kernel<T, SH, SW, CELL0, kMfX, false, BF, SP, CL><<<grid, kMfBlock, f.lds, stream>>>(g, gout, x, rot, ws, f.tiles, f.parts, f.splits, f.pitch_x, 0);
       // 16-bit inputs with at least one full block of 16 channels per group: bfloat16 matrix instructions
-      // float32 inputs: bfloat16 pairs (three products) unless switched off
+      // float32 inputs: bfloat16 pairs (three products) unless switched off, at stride 2 as well (N=64: 96 x 112^2
+      // 98 -> 90 us, 144 x 56^2 46 -> 41, 192 x 28^2 25.9 -> 24.3, 576 x 14^2 32.8 -> 30.1)
       const bool split = !path_disabled(kNoFilterSplit);
 #define DK_LAUNCH(CELL0)                                                    \
   if constexpr (sizeof(T) == 2) {                                           \
