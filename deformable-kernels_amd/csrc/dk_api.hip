@@ -324,7 +324,7 @@ int dk_sample_depthwise_backward_filter(const dk_conv_desc* desc, const void* ou
 size_t dk_sample_depthwise_backward_rotation_workspace(const dk_conv_desc* desc) {
   Geo g;
   if (make_geo(desc, g) != DK_OK) return 0;
-  if (desc->layout == DK_LAYOUT_NHWC) return 0;
+  if (desc->layout == DK_LAYOUT_NHWC) return nhwc_supported(g, desc->dtype) ? nhwc_grad_rotation_workspace(g, desc->dtype) : 0;
   return desc->dtype == DK_F64 ? 0 : fast_local_grad_rotation_workspace(g);
 }
 
@@ -343,7 +343,7 @@ int dk_sample_depthwise_backward_rotation(const dk_conv_desc* desc, const void* 
   hipStream_t s = static_cast<hipStream_t>(stream);
   if (desc->layout == DK_LAYOUT_NHWC)
     return by_dtype(desc->dtype, [&]<typename T>() {
-      nhwc_grad_rotation<T>(g, in<T>(out_grad), in<T>(input), in<T>(rotation), in<T>(filter), out<T>(rotation_grad), s);
+      nhwc_grad_rotation<T>(g, in<T>(out_grad), in<T>(input), in<T>(rotation), in<T>(filter), out<T>(rotation_grad), workspace, s);
     });
   return by_dtype(desc->dtype, [&]<typename T>() {
     if constexpr (kHasFast<T>)

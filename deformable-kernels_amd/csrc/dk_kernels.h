@@ -188,8 +188,9 @@ bool nhwc_supported(const Geo& g, int dtype);
 template <typename T>
 void nhwc_gather(const Geo& g, bool transposed, const T* src, const T* rot, const T* filter, T* dst,
                  hipStream_t stream);
+size_t nhwc_grad_rotation_workspace(const Geo& g, int dtype);
 template <typename T>
-void nhwc_grad_rotation(const Geo& g, const T* gout, const T* x, const T* rot, const T* filter, T* grot,
+void nhwc_grad_rotation(const Geo& g, const T* gout, const T* x, const T* rot, const T* filter, T* grot, void* ws,
                         hipStream_t stream);
 size_t nhwc_grad_filter_workspace(const Geo& g, int dtype);
 template <typename T>

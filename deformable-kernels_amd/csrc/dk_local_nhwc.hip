@@ -792,7 +792,8 @@ constexpr unsigned kNoChannels = 0x40000000u;
 template <typename T, int NCT, bool WLO>
 __global__ __launch_bounds__(64 * kR16Waves) void nhwc_grad_rotation_mfma16_kernel(
     Geo g, const T* __restrict__ gout, const T* __restrict__ x, const T* __restrict__ rot,
-    const T* __restrict__ filter, T* __restrict__ grot, int tiles_per_wave, int wpitch, int total_blocks) {
+    const T* __restrict__ filter, T* __restrict__ grot, int tiles_per_wave, int wpitch, int tile_blocks, int csplits,
+    float* __restrict__ partial) {
   constexpr int ROW = 16 * NCT, ROWP = ROW + 4, TAPS = 9;
   constexpr int NL = 2, HALF = 4;  // two loads of four channels for a lane's eight
   using Raw = typename std::conditional<sizeof(T) == 4, nhwc_u4, nhwc_u2>::type;
@@ -803,10 +804,15 @@ __global__ __launch_bounds__(64 * kR16Waves) void nhwc_grad_rotation_mfma16_kern
   float* rl = reinterpret_cast<float*>(nhwc_lds + (size_t)ROW * wpitch * 2 * (WLO ? 2 : 1)) + wave * (3 * 16 * ROWP);
   const int C = g.channel, cells = g.scope_h * g.scope_w;
   const int cpad = (C + 31) & ~31;
-  const int lb = logical_block(total_blocks);
-  if (lb >= total_blocks) return;
+  const int lb_all = logical_block(tile_blocks * csplits);
+  if (lb_all >= tile_blocks * csplits) return;
+  // csplits > 1 (few tiles, many channels): this workgroup sums the steps s_lo .. s_hi - 1 of 32 channels into an
+  // fp32 partial result of its own; reduce_few_parts_kernel adds the splits in order
+  const int lb = lb_all % tile_blocks, split = lb_all / tile_blocks;
+  const int nsteps_all = cpad / 32, per_split = (nsteps_all + csplits - 1) / csplits;
+  const int s_lo = split * per_split, s_hi = min(nsteps_all, s_lo + per_split);
 
-  for (int i = threadIdx.x; i < ROW * cpad; i += 64 * kR16Waves) {
+  for (int i = threadIdx.x + ROW * 32 * s_lo; i < ROW * 32 * s_hi; i += 64 * kR16Waves) {
     const int ch = i / ROW, cell = i - ch * ROW;
     const float v = ch < C && cell < cells ? (float)ld(filter + (size_t)ch * cells + cell) : 0.f;
     const unsigned hi = pack_bf16(v, 0.f) & 0xffffu;
@@ -820,7 +826,6 @@ __global__ __launch_bounds__(64 * kR16Waves) void nhwc_grad_rotation_mfma16_kern
   const long total_pix = (long)g.batch * oplane;
   const rsrc_t rg = plane_rsrc(gout, (int)(total_pix * C));
   const rsrc_t rx = plane_rsrc(x, g.batch * g.in_h * g.in_w * C);
-  const int nsteps = cpad / 32;
 
   for (int tk = 0; tk < tiles_per_wave; ++tk) {
     const long q0 = (((long)lb * kR16Waves + wave) * tiles_per_wave + tk) * 16;
@@ -841,7 +846,7 @@ __global__ __launch_bounds__(64 * kR16Waves) void nhwc_grad_rotation_mfma16_kern
     // byte offset of the lane's eight channels in a step, or kNoChannels
     auto chan_off = [&](int step) {
       const int c8 = step * 32 + 8 * kg;
-      return c8 < C ? (unsigned)c8 * (unsigned)sizeof(T) : kNoChannels;
+      return c8 < C && step < s_hi ? (unsigned)c8 * (unsigned)sizeof(T) : kNoChannels;
     };
 
     nhwc_f4 acc[TAPS][NCT];
@@ -859,11 +864,11 @@ __global__ __launch_bounds__(64 * kR16Waves) void nhwc_grad_rotation_mfma16_kern
 #pragma unroll
       for (int h = 0; h < NL; ++h) buf[h] = raw_ld4(rg, goff + co + (unsigned)(HALF * sizeof(T)) * h, gout);
     };
-    unsigned co = chan_off(0);
+    unsigned co = chan_off(s_lo);
     issue_g(gcur, co);
     issue_x(xr[0], 0, co);
     issue_x(xr[1], 1, co);
-    for (int step = 0; step < nsteps; ++step) {
+    for (int step = s_lo; step < s_hi; ++step) {
       const unsigned co_next = chan_off(step + 1);  // past the last step: no channels, the loads return zeros
       // this step's filter operands
       uint4 bh[NCT], bl[NCT];
@@ -953,8 +958,14 @@ __global__ __launch_bounds__(64 * kR16Waves) void nhwc_grad_rotation_mfma16_kern
           gh = hw * (r10 - r00) + lw * (r11 - r01);
           gw = hh * (r01 - r00) + lh * (r11 - r10);
         }
-        st(grot + ri, open_h ? gh : 0.f);
-        st(grot + ri + 1, open_w ? gw : 0.f);
+        if (partial) {
+          float* dst = partial + (size_t)split * ((size_t)total_pix * (TAPS * 2)) + ri;
+          dst[0] = open_h ? gh : 0.f;
+          dst[1] = open_w ? gw : 0.f;
+        } else {
+          st(grot + ri, open_h ? gh : 0.f);
+          st(grot + ri + 1, open_w ? gw : 0.f);
+        }
       }
     }
   }
@@ -1328,8 +1339,29 @@ void nhwc_gather(const Geo& g, bool transposed, const T* src, const T* rot, cons
 #undef DK_NHWC_GATHER
 }
 
+// Shape test and channel splits of the 32-channel matrix-core grad rotation (0: it does not apply).  Few tiles of 16
+// pixels and many channels (960 x 7 x 7 at batch 64: 196 tiles, 30 steps of 32 channels) leave most of the GPU idle:
+// the steps are then split over workgroups, at least two steps each, for about four waves per SIMD.
+int nhwc_rotation16_splits(const Geo& g, size_t elem) {
+  const int nct = (g.scope_h * g.scope_w + 15) / 16;
+  const long bytes = (long)g.batch * g.channel * std::max((long)g.in_h * g.in_w, (long)g.out_h * g.out_w) * (long)elem;
+  if (g.groups != 1 || nct > 2 || g.k_h != 3 || g.k_w != 3 || g.channel % 8 != 0 || bytes >= (1L << 30) ||
+      path_disabled(kNoNhwcMfma) || path_disabled(kNoNhwcStaged))
+    return 0;
+  const long tiles = ceil_div((long)g.batch * g.out_h * g.out_w, 16L);
+  const int nsteps = (g.channel + 31) / 32;
+  const long want = ceil_div(4096L, std::max(1L, tiles));
+  return (int)std::max(1L, std::min<long>(want, nsteps / 2));
+}
+
+size_t nhwc_grad_rotation_workspace(const Geo& g, int dtype) {
+  if (dtype == DK_F64) return 0;
+  const int splits = nhwc_rotation16_splits(g, dtype == DK_F32 ? 4 : 2);
+  return splits > 1 ? (size_t)splits * g.batch * g.out_h * g.out_w * 18 * sizeof(float) : 0;
+}
+
 template <typename T>
-void nhwc_grad_rotation(const Geo& g, const T* gout, const T* x, const T* rot, const T* filter, T* grot,
+void nhwc_grad_rotation(const Geo& g, const T* gout, const T* x, const T* rot, const T* filter, T* grot, void* ws,
                         hipStream_t stream) {
   using CT = compute_t<T>;
   const int cells_ = g.scope_h * g.scope_w, taps_ = g.k_h * g.k_w;
@@ -1340,9 +1372,8 @@ void nhwc_grad_rotation(const Geo& g, const T* gout, const T* x, const T* rot, c
                          reinterpret_cast<uintptr_t>(x) % (4 * sizeof(T)) == 0;
     const bool small = (long)g.batch * g.channel * std::max((long)g.in_h * g.in_w, (long)g.out_h * g.out_w) * (long)sizeof(T) < (1L << 31);
     // 3 x 3 taps, a multiple of 8 channels: 32 channels per matrix instruction
-    const long bytes = (long)g.batch * g.channel * std::max((long)g.in_h * g.in_w, (long)g.out_h * g.out_w) * (long)sizeof(T);
-    if (g.groups == 1 && nct <= 2 && g.k_h == 3 && g.k_w == 3 && g.channel % 8 == 0 && aligned && bytes < (1L << 30) &&
-        !path_disabled(kNoNhwcMfma) && !path_disabled(kNoNhwcStaged)) {
+    const int splits = nhwc_rotation16_splits(g, sizeof(T));
+    if (splits > 0 && aligned) {
       constexpr bool wlo = !std::is_same<T, bf16_t>::value;
       const int wpitch = ((g.channel + 31) & ~31) + 8;
       const size_t lds = (size_t)16 * nct * wpitch * 2 * (wlo ? 2 : 1) + (size_t)kR16Waves * 48 * (16 * nct + 4) * sizeof(float);
@@ -1350,8 +1381,10 @@ void nhwc_grad_rotation(const Geo& g, const T* gout, const T* x, const T* rot, c
       const int blocks = (int)ceil_div(tiles, (long)kR16Waves * kR16TilesPerWave);
       auto kernel = nct == 1 ? nhwc_grad_rotation_mfma16_kernel<T, 1, wlo> : nhwc_grad_rotation_mfma16_kernel<T, 2, wlo>;
       if (lds <= 64 * 1024 || (lds <= 120 * 1024 && allow_dynamic_lds(reinterpret_cast<const void*>(kernel), 120 * 1024))) {
-        hipLaunchKernelGGL(kernel, dim3((unsigned)xcd_grid_size(blocks)), dim3(64 * kR16Waves), lds, stream, g, gout, x, rot,
-                           filter, grot, kR16TilesPerWave, wpitch, blocks);
+        float* partial = splits > 1 ? static_cast<float*>(ws) : nullptr;
+        hipLaunchKernelGGL(kernel, dim3((unsigned)xcd_grid_size((long)blocks * splits)), dim3(64 * kR16Waves), lds, stream, g, gout,
+                           x, rot, filter, grot, kR16TilesPerWave, wpitch, blocks, splits, partial);
+        if (splits > 1) launch_reduce_partials<float, T>(partial, splits, (long)g.batch * g.out_h * g.out_w * 18, grot, stream);
         return;
       }
     }
@@ -1445,7 +1478,7 @@ void nhwc_grad_filter(const Geo& g, const T* gout, const T* x, const T* rot, T* 
 
 #define DK_INSTANTIATE(T)                                                                                  \
   template void nhwc_gather<T>(const Geo&, bool, const T*, const T*, const T*, T*, hipStream_t);           \
-  template void nhwc_grad_rotation<T>(const Geo&, const T*, const T*, const T*, const T*, T*, hipStream_t); \
+  template void nhwc_grad_rotation<T>(const Geo&, const T*, const T*, const T*, const T*, T*, void*, hipStream_t); \
   template void nhwc_grad_filter<T>(const Geo&, const T*, const T*, const T*, T*, void*, hipStream_t);
 DK_INSTANTIATE(float)
 DK_INSTANTIATE(__half)

@@ -30,6 +30,8 @@ CASES = [
     (1, 40, 13, 12, 3, (5, 5), 1, 1, 1, 1, 1.5),    # scope 5: two slices of sixteen cells
     (2, 16, 15, 14, 3, (4, 4), 1, 2, 2, 1, 1.0),    # dilation 2 with one group: the matrix-core kernels' general taps
     (1, 32, 12, 11, 3, (3, 3), 2, 0, 1, 1, 1.0),    # stride 2 without padding, scope == kernel
+    (2, 128, 7, 7, 3, (4, 4), 1, 1, 1, 1, 1.0),     # few pixels, many channels: the grad rotation's channel steps split over two workgroups
+    (1, 200, 6, 5, 3, (3, 3), 1, 1, 1, 1, 1.0),     # seven steps of 32 channels over three splits (3, 3, 1), the last step partial
 ]
 
 
@@ -95,7 +97,7 @@ def test_fp32_without_the_staged_kernels(case, switch_off):
 
 
 # the shapes the matrix-core forward / grad input covers: one group, 3 x 3 taps, scope 3 x 3 or 4 x 4, at least 16 channels in fours
-GATHER_CASES = [CASES[0], CASES[1], CASES[2], CASES[6], CASES[10], CASES[11], CASES[13], CASES[14]]
+GATHER_CASES = [CASES[0], CASES[1], CASES[2], CASES[6], CASES[10], CASES[11], CASES[13], CASES[14], CASES[15], CASES[16]]
 
 
 @pytest.mark.parametrize("case", GATHER_CASES)
@@ -133,7 +135,7 @@ def test_fp64_matches_oracle(case):
 
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
-@pytest.mark.parametrize("case", CASES[:3] + CASES[5:7] + CASES[10:])
+@pytest.mark.parametrize("case", CASES[:3] + CASES[5:7] + CASES[10:])   # (the last two: grad rotation partials reduced into a 16-bit tensor)
 def test_half_precisions_match_fp32_oracle(case, dtype):
     inputs, got = _run(case, dtype, seed=3)
     want = _oracle(inputs, np.float32)
