@@ -812,12 +812,26 @@ __global__ __launch_bounds__(64 * kR16Waves) void nhwc_grad_rotation_mfma16_kern
   const int nsteps_all = cpad / 32, per_split = (nsteps_all + csplits - 1) / csplits;
   const int s_lo = split * per_split, s_hi = min(nsteps_all, s_lo + per_split);
 
-  for (int i = threadIdx.x + ROW * 32 * s_lo; i < ROW * 32 * s_hi; i += 64 * kR16Waves) {
-    const int ch = i / ROW, cell = i - ch * ROW;
-    const float v = ch < C && cell < cells ? (float)ld(filter + (size_t)ch * cells + cell) : 0.f;
-    const unsigned hi = pack_bf16(v, 0.f) & 0xffffu;
-    wh[cell * wpitch + ch] = (unsigned short)hi;
-    if (WLO) wlo[cell * wpitch + ch] = (unsigned short)(pack_bf16(v - bf16_lo(hi), 0.f) & 0xffffu);
+  // (eight loads at a time, all issued before the first is used: one at a time every workgroup began with a
+  // chain of dependent trips to L2 that took longer than its products)
+  for (int i0 = threadIdx.x + ROW * 32 * s_lo; i0 < ROW * 32 * s_hi; i0 += 8 * 64 * kR16Waves) {
+    float v[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      const int i = i0 + u * 64 * kR16Waves;
+      const int ch = i / ROW, cell = i - ch * ROW;
+      v[u] = i < ROW * 32 * s_hi && ch < C && cell < cells ? (float)ld(filter + (size_t)ch * cells + cell) : 0.f;
+    }
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      const int i = i0 + u * 64 * kR16Waves;
+      if (i < ROW * 32 * s_hi) {
+        const int ch = i / ROW, cell = i - ch * ROW;
+        const unsigned hi = pack_bf16(v[u], 0.f) & 0xffffu;
+        wh[cell * wpitch + ch] = (unsigned short)hi;
+        if (WLO) wlo[cell * wpitch + ch] = (unsigned short)(pack_bf16(v[u] - bf16_lo(hi), 0.f) & 0xffffu);
+      }
+    }
   }
   __syncthreads();
 
@@ -854,8 +868,18 @@ __global__ __launch_bounds__(64 * kR16Waves) void nhwc_grad_rotation_mfma16_kern
     for (int t = 0; t < TAPS; ++t)
 #pragma unroll
       for (int n = 0; n < NCT; ++n) acc[t][n] = nhwc_f4{0.f, 0.f, 0.f, 0.f};
+    // the rotation values of the rows this lane finishes (tap 3 phase + kg of pixel m, lanes below 48), loaded
+    // now: the epilogue would otherwise wait for them once per phase
+    float rot_h[3], rot_w[3];
+#pragma unroll
+    for (int ph_ = 0; ph_ < 3; ++ph_) {
+      const bool mine = lane < 48 && live;
+      const size_t ri = (size_t)qc * (TAPS * 2) + 2 * (3 * ph_ + min(kg, 2));
+      rot_h[ph_] = mine ? (float)ld(rot + ri) : 0.f;
+      rot_w[ph_] = mine ? (float)ld(rot + ri + 1) : 0.f;
+    }
 
-    Raw xr[3][NL], gcur[NL], gnext[NL];  // a ring of three taps' loads: two taps ahead of the arithmetic
+    Raw xr[3][NL], gcur[NL], gnext[NL];  // a ring of three taps' loads: three taps ahead of the split and the products
     auto issue_x = [&](Raw (&buf)[NL], int t, unsigned co) {
 #pragma unroll
       for (int h = 0; h < NL; ++h) buf[h] = raw_ld4(rx, xoff[t] + co + (unsigned)(HALF * sizeof(T)) * h, x);
@@ -868,6 +892,7 @@ __global__ __launch_bounds__(64 * kR16Waves) void nhwc_grad_rotation_mfma16_kern
     issue_g(gcur, co);
     issue_x(xr[0], 0, co);
     issue_x(xr[1], 1, co);
+    issue_x(xr[2], 2, co);
     for (int step = s_lo; step < s_hi; ++step) {
       const unsigned co_next = chan_off(step + 1);  // past the last step: no channels, the loads return zeros
       // this step's filter operands
@@ -887,8 +912,6 @@ __global__ __launch_bounds__(64 * kR16Waves) void nhwc_grad_rotation_mfma16_kern
       }
 #pragma unroll
       for (int t = 0; t < TAPS; ++t) {
-        if (t + 2 < TAPS) issue_x(xr[(t + 2) % 3], t + 2, co);
-        else issue_x(xr[(t + 2) % 3], t + 2 - TAPS, co_next);
         if (t == 4) issue_g(gnext, co_next);
         float xv[8];
 #pragma unroll
@@ -904,6 +927,9 @@ __global__ __launch_bounds__(64 * kR16Waves) void nhwc_grad_rotation_mfma16_kern
           pr[i] = gv[i] * xv[i];
           asm volatile("" : "+v"(pr[i]));  // one fp32 value for both parts: no contraction into the conversions
         }
+        // the tap's registers are free again: the load three taps ahead goes into them
+        if (t + 3 < TAPS) issue_x(xr[t % 3], t + 3, co);
+        else issue_x(xr[t % 3], t + 3 - TAPS, co_next);
         unsigned hi[4], lo[4];
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
@@ -942,8 +968,8 @@ __global__ __launch_bounds__(64 * kR16Waves) void nhwc_grad_rotation_mfma16_kern
         const bool hit = ih >= 0 && ih < g.in_h && iw >= 0 && iw < g.in_w;
         const size_t ri = (size_t)q * (TAPS * 2) + 2 * t;
         bool open_h = true, open_w = true;
-        const float sh = scope_coord<float>(g, ph_, (float)ld(rot + ri), g.centre_h, &open_h);
-        const float sw = scope_coord<float>(g, tt, (float)ld(rot + ri + 1), g.centre_w, &open_w);
+        const float sh = scope_coord<float>(g, ph_, rot_h[ph_], g.centre_h, &open_h);
+        const float sw = scope_coord<float>(g, tt, rot_w[ph_], g.centre_w, &open_w);
         float gh = 0.f, gw = 0.f;
         if (hit && sh > -1.f && sw > -1.f && sh < (float)g.scope_h && sw < (float)g.scope_w) {
           const float hf = floorf(sh), wf = floorf(sw);
