@@ -1081,7 +1081,7 @@ __device__ __forceinline__ void raw_st4(rsrc_t r, unsigned off, const float (&v)
   __builtin_amdgcn_raw_buffer_store_b64(__builtin_bit_cast(nhwc_u2, pk), r, (int)off, 0, AUX);
 }
 
-constexpr int kG16Waves = 4;
+constexpr int kG16Waves = 4;  // (two: 75.9 us on benchmark configuration 2, four: 74, six: 95)
 // One tile per wave: workgroups that live as long as one tile keep the tail of the grid short (two tiles per wave
 // measured 85.8 against 81.4 us on benchmark configuration 2, four 96).
 constexpr int kG16TilesPerWave = 1;
@@ -1107,27 +1107,31 @@ __global__ __launch_bounds__(64 * kG16Waves) void nhwc_gather_mfma16_kernel(
   const int lb = logical_block(total_blocks);
   if (lb >= total_blocks) return;
 
-  // ---- per workgroup: the split filter operands of every channel block
+  // ---- per workgroup: the split filter operands of every channel block.  An entry is lane l of its wave, so the
+  // channel's largest weight is the maximum over the four lanes l % 16 + 16 k of what each holds: one load per lane
+  // instead of the channel's sixteen (a workgroup lives about as long as a dozen trips to L2, and every thread
+  // waits for this table: forward 80 -> 75 us on benchmark configuration 2).  Issuing several entries' loads
+  // together measured slower (83 us).
   for (int e = threadIdx.x; e < nblk * 64; e += 64 * kG16Waves) {
     const int b = e >> 6, l = e & 63, cj = b * 16 + (l & 15), c0 = 4 * (l >> 4);
     float v[4] = {0.f, 0.f, 0.f, 0.f}, s = 1.f;
     if (cj < C) {
       const T* f = filter + (size_t)cj * CELLS;
-      if constexpr (kThird) {
-        float mx = 0.f;
-#pragma unroll
-        for (int k = 0; k < CELLS; ++k) mx = fmaxf(mx, fabsf(ld(f + k)));
-        int ex = 0;
-        if (mx > 0.f && mx < __builtin_inff()) (void)frexpf(mx, &ex);
-        ex = min(max(ex, -100), 100);
-        s = ldexpf(1.f, -ex);
-        if ((l >> 4) == 0) unscale[b * 16 + (l & 15)] = ldexpf(1.f, ex);
-      }
 #pragma unroll
       for (int k = 0; k < 4; ++k)
-        if (c0 + k < CELLS) v[k] = (float)ld(f + c0 + k) * s;
-    } else if ((l >> 4) == 0) {
-      unscale[b * 16 + (l & 15)] = 0.f;
+        if (c0 + k < CELLS) v[k] = (float)ld(f + c0 + k);
+    }
+    if constexpr (kThird) {
+      float mx = fmaxf(fmaxf(fabsf(v[0]), fabsf(v[1])), fmaxf(fabsf(v[2]), fabsf(v[3])));
+      mx = fmaxf(mx, __shfl_xor(mx, 16));
+      mx = fmaxf(mx, __shfl_xor(mx, 32));
+      int ex = 0;
+      if (mx > 0.f && mx < __builtin_inff()) (void)frexpf(mx, &ex);
+      ex = min(max(ex, -100), 100);
+      s = ldexpf(1.f, -ex);
+      if ((l >> 4) == 0) unscale[b * 16 + (l & 15)] = cj < C ? ldexpf(1.f, ex) : 0.f;
+#pragma unroll
+      for (int k = 0; k < 4; ++k) v[k] *= s;
     }
     typename M::v4 h4, l4;
 #pragma unroll
