@@ -32,6 +32,7 @@ CASES = [
     (1, 32, 12, 11, 3, (3, 3), 2, 0, 1, 1, 1.0),    # stride 2 without padding, scope == kernel
     (2, 128, 7, 7, 3, (4, 4), 1, 1, 1, 1, 1.0),     # few pixels, many channels: the grad rotation's channel steps split over two workgroups
     (1, 200, 6, 5, 3, (3, 3), 1, 1, 1, 1, 1.0),     # seven steps of 32 channels over three splits (3, 3, 1), the last step partial
+    (1, 960, 7, 7, 3, (4, 4), 1, 1, 1, 1, 1.0),     # MobileNetV2's last stage: filter tables of more than 64 KB of LDS in the matrix-core kernels
 ]
 
 
@@ -97,7 +98,7 @@ def test_fp32_without_the_staged_kernels(case, switch_off):
 
 
 # the shapes the matrix-core forward / grad input covers: one group, 3 x 3 taps, scope 3 x 3 or 4 x 4, at least 16 channels in fours
-GATHER_CASES = [CASES[0], CASES[1], CASES[2], CASES[6], CASES[10], CASES[11], CASES[13], CASES[14], CASES[15], CASES[16]]
+GATHER_CASES = [CASES[0], CASES[1], CASES[2], CASES[6], CASES[10], CASES[11], CASES[13], CASES[14], CASES[15], CASES[16], CASES[17]]
 
 
 @pytest.mark.parametrize("case", GATHER_CASES)
