@@ -790,7 +790,7 @@ __device__ __forceinline__ void lds_fence_wave() {
 constexpr unsigned kNoChannels = 0x40000000u;
 
 template <typename T, int NCT, bool WLO>
-__global__ __launch_bounds__(64 * kR16Waves) void nhwc_grad_rotation_mfma16_kernel(
+__global__ __launch_bounds__(64 * kR16Waves, NCT == 1 ? 4 : 3) void nhwc_grad_rotation_mfma16_kernel(
     Geo g, const T* __restrict__ gout, const T* __restrict__ x, const T* __restrict__ rot,
     const T* __restrict__ filter, T* __restrict__ grot, int tiles_per_wave, int wpitch, int tile_blocks, int csplits,
     float* __restrict__ partial) {
@@ -868,18 +868,7 @@ __global__ __launch_bounds__(64 * kR16Waves) void nhwc_grad_rotation_mfma16_kern
     for (int t = 0; t < TAPS; ++t)
 #pragma unroll
       for (int n = 0; n < NCT; ++n) acc[t][n] = nhwc_f4{0.f, 0.f, 0.f, 0.f};
-    // the rotation values of the rows this lane finishes (tap 3 phase + kg of pixel m, lanes below 48), loaded
-    // now: the epilogue would otherwise wait for them once per phase
-    float rot_h[3], rot_w[3];
-#pragma unroll
-    for (int ph_ = 0; ph_ < 3; ++ph_) {
-      const bool mine = lane < 48 && live;
-      const size_t ri = (size_t)qc * (TAPS * 2) + 2 * (3 * ph_ + min(kg, 2));
-      rot_h[ph_] = mine ? (float)ld(rot + ri) : 0.f;
-      rot_w[ph_] = mine ? (float)ld(rot + ri + 1) : 0.f;
-    }
-
-    Raw xr[3][NL], gcur[NL], gnext[NL];  // a ring of three taps' loads: three taps ahead of the split and the products
+    Raw xr[3][NL], gcur[NL];  // a ring of three taps' loads: three taps ahead of the split and the products
     auto issue_x = [&](Raw (&buf)[NL], int t, unsigned co) {
 #pragma unroll
       for (int h = 0; h < NL; ++h) buf[h] = raw_ld4(rx, xoff[t] + co + (unsigned)(HALF * sizeof(T)) * h, x);
@@ -912,7 +901,6 @@ __global__ __launch_bounds__(64 * kR16Waves) void nhwc_grad_rotation_mfma16_kern
       }
 #pragma unroll
       for (int t = 0; t < TAPS; ++t) {
-        if (t == 4) issue_g(gnext, co_next);
         float xv[8];
 #pragma unroll
         for (int h = 0; h < NL; ++h) {
@@ -930,6 +918,7 @@ __global__ __launch_bounds__(64 * kR16Waves) void nhwc_grad_rotation_mfma16_kern
         // the tap's registers are free again: the load three taps ahead goes into them
         if (t + 3 < TAPS) issue_x(xr[t % 3], t + 3, co);
         else issue_x(xr[t % 3], t + 3 - TAPS, co_next);
+        if (t == TAPS - 1) issue_g(gcur, co_next);  // out_grad of the next step, once this step's is used up
         unsigned hi[4], lo[4];
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
@@ -946,8 +935,6 @@ __global__ __launch_bounds__(64 * kR16Waves) void nhwc_grad_rotation_mfma16_kern
           if (WLO) acc[t][n] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ph, __builtin_bit_cast(nhwc_b8, bl[n]), acc[t][n], 0, 0, 0);
         }
       }
-#pragma unroll
-      for (int h = 0; h < NL; ++h) gcur[h] = gnext[h];
       co = co_next;
     }
 
@@ -968,8 +955,8 @@ __global__ __launch_bounds__(64 * kR16Waves) void nhwc_grad_rotation_mfma16_kern
         const bool hit = ih >= 0 && ih < g.in_h && iw >= 0 && iw < g.in_w;
         const size_t ri = (size_t)q * (TAPS * 2) + 2 * t;
         bool open_h = true, open_w = true;
-        const float sh = scope_coord<float>(g, ph_, rot_h[ph_], g.centre_h, &open_h);
-        const float sw = scope_coord<float>(g, tt, rot_w[ph_], g.centre_w, &open_w);
+        const float sh = scope_coord<float>(g, ph_, (float)ld(rot + ri), g.centre_h, &open_h);
+        const float sw = scope_coord<float>(g, tt, (float)ld(rot + ri + 1), g.centre_w, &open_w);
         float gh = 0.f, gw = 0.f;
         if (hit && sh > -1.f && sw > -1.f && sh < (float)g.scope_h && sw < (float)g.scope_w) {
           const float hf = floorf(sh), wf = floorf(sw);
