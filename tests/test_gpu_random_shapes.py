@@ -90,6 +90,44 @@ def test_local_operator_on_random_geometries_in_16_bits(k, case):
         assert rel_err(g.float(), w) < 1e-2, name
 
 
+def _nhwc_cases():
+    """One rotation group, 3 x 3 taps, channel counts in fours and eights: the shapes the channels-last
+    matrix-core kernels cover, with every stride / padding / dilation and both of their scopes."""
+    rnd = random.Random(31)
+    cases = []
+    while len(cases) < 28:
+        H, W = rnd.choice([1, 2, 3, 5, 7, 8, 13, 14, 16, 17, 28, 33]), rnd.choice([1, 2, 3, 4, 7, 9, 15, 16, 17, 31, 40])
+        C = rnd.choice([16, 20, 24, 36, 40, 64, 72, 100, 136])
+        s, p, d = rnd.choice([1, 1, 2]), rnd.choice([0, 1, 2]), rnd.choice([1, 1, 2])
+        if (H + 2 * p - 2 * d - 1) // s + 1 < 1 or (W + 2 * p - 2 * d - 1) // s + 1 < 1:
+            continue
+        cases.append((rnd.choice([1, 2, 3]), C, H, W, 3, rnd.choice([(3, 3), (4, 4), (4, 4), (5, 5)]), s, p, d, 1, 1.0))
+    return cases
+
+
+@pytest.mark.parametrize("k,case", list(enumerate(_nhwc_cases())))
+def test_channels_last_matrix_core_kernels_on_random_geometries(k, case, switch_off):
+    """float32, and every fourth case bfloat16 / float16; the matrix-core forward / grad input forced on every
+    shape it covers (scope 5 x 5 keeps the table kernel for them; grad rotation and grad filter take their
+    matrix-core kernels)."""
+    import test_gpu_nhwc as tn
+    switch_off("DK_FORCE_NHWC_GATHER_MFMA")
+    if k % 4 == 3:
+        dtype = torch.bfloat16 if k % 8 == 3 else torch.float16
+        inputs, got = tn._run(case, dtype, seed=k)
+        want = tn._oracle(inputs, np.float32)
+        for g, w, name in zip(got, want, ("forward", "grad input", "grad rotation", "grad filter")):
+            assert g.dtype == dtype
+            assert rel_err(g.float(), w) < 1e-2, name
+        return
+    inputs, got = tn._run(case, torch.float32, seed=k)
+    o32, o64 = tn._oracle(inputs, np.float32), tn._oracle(inputs, np.float64)
+    assert rel_err(got[0], o32[0]) < 1e-5
+    assert rel_err(got[1], o32[1]) < 1e-5
+    assert rel_err(got[2], o64[2]) < 1e-4
+    assert rel_err(got[3], o64[3]) < 1e-4
+
+
 def _offset_conv_cases():
     rnd = random.Random(23)
     cases = []
