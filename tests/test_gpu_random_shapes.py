@@ -73,7 +73,20 @@ def _deform_large_cases():
     return cases
 
 
-@pytest.mark.parametrize("case", _deform_cases() + _deform_large_cases())
+def _deform_huge_cases():
+    """Planes that fit LDS once or not at all (100 to 260 rows and columns): row windows, the rows-and-columns window
+    of the grad filter, the band form of the grad input."""
+    rnd = random.Random(17)
+    cases = []
+    for _ in range(6):
+        C = rnd.choice([2, 3, 6, 10])
+        cases.append((1, C, rnd.randint(100, 260), rnd.randint(100, 260), 3, rnd.choice([(3, 3), (4, 4), (5, 5)]),
+                      rnd.choice([1, 1, 2]), rnd.choice([0, 1]), rnd.choice([1, 1, 2]),
+                      rnd.choice([g for g in (1, 2, 3) if C % g == 0]), 0.7, rnd.choice([0.5, 2.0, 9.0])))
+    return cases
+
+
+@pytest.mark.parametrize("case", _deform_cases() + _deform_large_cases() + _deform_huge_cases())
 def test_deformable_operator_on_random_geometries(case):
     inputs, got = td._run(case, torch.float32)
     td.assert_fp32_parity(got, td._oracle(inputs, np.float32), td._oracle(inputs, np.float64))
