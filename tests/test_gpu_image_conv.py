@@ -116,6 +116,23 @@ def test_packed_16_bit_kernels_against_the_kernels_that_unpack(case, dtype, swit
         assert ((a.float() - b.float()).abs() <= ulp * b.float().abs() + 1e-6 * b.float().abs().max()).all()
 
 
+def _packed_cases():
+    import random
+    rnd = random.Random(41)
+    return [(rnd.choice([1, 2, 5]), rnd.choice([1, 3, 4, 9]), rnd.choice([1, 2, 3, 4, 5, 8, 12, 17, 40, 64]),
+             rnd.choice([4, 8, 12, 20, 36, 60, 100, 128]), 3, 3, (1, 1), (1, 1), (1, 1)) for _ in range(14)]
+
+
+@pytest.mark.parametrize("k,case", list(enumerate(_packed_cases())))
+def test_packed_16_bit_kernels_on_random_planes(k, case):
+    """Rows of 4 to 128 elements, planes of one row to several bands, plane counts that fill no workgroup."""
+    dtype = torch.float16 if k % 2 == 0 else torch.bfloat16
+    got, want = _run(case, dtype, seed=20 + k, sampler_layout=k % 3 == 0)
+    for a, b in zip(got, want):
+        assert a.dtype == dtype
+        assert rel_err(a.float(), b) < 1e-2
+
+
 def test_configuration_3_shape_float16_matches_the_grouped_convolution_it_replaces():
     """N=128, C=256, 28x28, 3x3 kernels per (image, channel), float16: the oracle on three images, and
     the framework's convolution with N * C groups (the reference's call) on the whole batch."""
