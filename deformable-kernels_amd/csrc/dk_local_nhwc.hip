@@ -208,7 +208,11 @@ __global__ __launch_bounds__(kNBlock) void nhwc_gather_kernel(Geo g, NhwcLaunch 
     Pack res;
 #pragma unroll
     for (int v = 0; v < VEC; ++v) st(res.v + v, acc[v]);
-    *reinterpret_cast<Pack*>(out) = res;
+    if constexpr (sizeof(Pack) == 16) {
+      __builtin_nontemporal_store(__builtin_bit_cast(nhwc_u4, res), reinterpret_cast<nhwc_u4*>(out));
+    } else {
+      *reinterpret_cast<Pack*>(out) = res;
+    }
   }
 }
 
