@@ -1061,6 +1061,12 @@ __device__ __forceinline__ bool write_nan_if_unbounded(float gmax, const float* 
   return true;
 }
 
+// A result element that is not read again by the operator: non-temporal for 4-byte elements (a wave writes whole
+// lines), the plain store for 2-byte ones (as partial lines they reach memory one by one).
+__device__ __forceinline__ void st_stream(float* p, float v) { __builtin_nontemporal_store(v, p); }
+template <typename T>
+__device__ __forceinline__ void st_stream(T* p, float v) { dk::st(p, v); }
+
 // Two channels share a 64-bit sum while at most 2^kPairHead samples touch one input element: a term is then
 // rounded on a grid of 2^-(31 - kPairHead) = 2^-24 of the largest possible term or finer.  (3 x 3 taps at stride 1
 // put 36 samples on an element on average and about 65 on the fullest element of a large plane.)
@@ -1246,8 +1252,8 @@ __global__ __launch_bounds__(1024) void deform_grad_input_kernel(
         *cell = 0ull;
         const int lo = (int)(unsigned)v;
         const int hi = (int)(unsigned)(v >> 32) + (lo < 0 ? 1 : 0);
-        dk::st(dst + row * W + col, (float)lo * ua);
-        if (pair) dk::st(dst + i_step + row * W + col, (float)hi * ub);
+        st_stream(dst + row * W + col, (float)lo * ua);
+        if (pair) st_stream(dst + i_step + row * W + col, (float)hi * ub);
       }
     }
   }
@@ -1519,8 +1525,8 @@ __global__ __launch_bounds__(1024) void deform_grad_input_tiled_kernel(
           const unsigned long long v = pl[(row + ROWOFF) * RS + 1 + col];
           const int lo = (int)(unsigned)v;
           const int hi = (int)(unsigned)(v >> 32) + (lo < 0 ? 1 : 0);
-          dk::st(dst + (r_lo + row) * W + col, (float)lo * ua);
-          if (pair) dk::st(dst + i_step + (r_lo + row) * W + col, (float)hi * ub);
+          st_stream(dst + (r_lo + row) * W + col, (float)lo * ua);
+          if (pair) st_stream(dst + i_step + (r_lo + row) * W + col, (float)hi * ub);
         }
       }
     }
