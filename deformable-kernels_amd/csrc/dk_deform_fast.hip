@@ -1726,6 +1726,23 @@ __global__ __launch_bounds__(BLOCK, 2) void deform_grad_filter_kernel(
 //     partial of (image, tile): reduce_partials_kernel adds those in order.
 // CELL0: the launch covers the scope cells CELL0 .. CELL0 + 15 (a 5 x 5 scope takes two).
 // ---------------------------------------------------------------------------
+// The planes of one block of channels of an image behind one descriptor each (input, gout): a channel of the
+// block is selected by the scalar part of the address, `channel * x_cs` bytes, so that a load costs the scalar
+// unit two instructions and not the twenty of a descriptor of its own (the 64-bit address, the size, the
+// selects).  The range check compares the lane's offset with the descriptor's size less the scalar part, so the
+// scalar part has to stay inside: channels past the block's last one (`last_`) re-read that one -- their columns
+// of the product are never written -- and the host keeps sixteen channels' span below 2^31 bytes.
+#define DK_GF_BLOCK_PLANES(cb)                                                                       \
+  const int last_ = min(kGfCh, cpg - (cb) * kGfCh) - 1;                                              \
+  const size_t c0_ = (size_t)n * g.channel + grp + (size_t)g.groups * ((cb) * kGfCh);                \
+  const rsrc_t rx_ = plane_rsrc(x + c0_ * in_plane, last_ * g.groups * in_plane + in_plane);         \
+  const rsrc_t rg_ = plane_rsrc(gout + c0_ * out_plane, last_ * g.groups * out_plane + out_plane);
+template <typename T>
+bool block_planes_fit(const Geo& g) {  // what DK_GF_BLOCK_PLANES asks of the shape
+  const long plane = std::max<long>((long)g.in_h * g.in_w, (long)g.out_h * g.out_w);
+  return 16L * g.groups * plane * (long)sizeof(T) < (1L << 31);
+}
+
 constexpr int kGfBlock = 1024;            // threads per workgroup
 constexpr int kGfPix = 256;               // output pixels per tile
 constexpr int kGfCh = 16;                 // channels per block
@@ -1755,6 +1772,7 @@ __global__ __launch_bounds__(kGfBlock, 1) void deform_grad_filter_mfma_kernel(
 
   const int cpg = g.channel / g.groups;
   const int out_plane = g.out_h * g.out_w, in_plane = H * W;
+  const int x_cs = g.groups * in_plane * (int)sizeof(T), g_cs = g.groups * out_plane * (int)sizeof(T);  // bytes from a channel of the group to the next
   const int nblk_all = ceil_div(cpg, kGfCh);
   const int total = tiles * csplits * g.batch * g.groups;
   const int lb = logical_block(total);
@@ -1782,18 +1800,11 @@ __global__ __launch_bounds__(kGfBlock, 1) void deform_grad_filter_mfma_kernel(
   float r_x[kGfCh], r_g[4];
 #define DK_GF_ISSUE(cb)                                                                              \
   {                                                                                                  \
-    _Pragma("unroll") for (int c = 0; c < kGfCh; ++c) {                                              \
-      const int cj_ = (cb) * kGfCh + c;                                                              \
-      const bool chan = cj_ < cpg;                                                                   \
-      const size_t ci_ = (size_t)n * g.channel + grp + (size_t)g.groups * (chan ? cj_ : 0);          \
-      r_x[c] = buf_ld(plane_rsrc(x + ci_ * in_plane, chan ? in_plane : 0), s_off, x);                \
-    }                                                                                                \
-    _Pragma("unroll") for (int c = 0; c < 4; ++c) {                                                  \
-      const int cj_ = (cb) * kGfCh + g_cq * 4 + c;                                                   \
-      const bool chan = cj_ < cpg;                                                                   \
-      const size_t ci_ = (size_t)n * g.channel + grp + (size_t)g.groups * (chan ? cj_ : 0);          \
-      r_g[c] = buf_ld(plane_rsrc(gout + ci_ * out_plane, chan ? out_plane : 0), g_off, gout);        \
-    }                                                                                                \
+    DK_GF_BLOCK_PLANES(cb)                                                                           \
+    _Pragma("unroll") for (int c = 0; c < kGfCh; ++c)                                                \
+      r_x[c] = buf_ld2(rx_, s_off, min(c, last_) * x_cs, x);                                         \
+    _Pragma("unroll") for (int c = 0; c < 4; ++c)                                                    \
+      r_g[c] = buf_ld2(rg_, g_off, min(g_cq * 4 + c, last_) * g_cs, gout);                           \
   }
 #define DK_GF_STORE()                                                                                \
   {                                                                                                  \
@@ -1924,11 +1935,15 @@ constexpr int kGwBlock = 512;
 constexpr int kGwPix = 128;
 constexpr int kGwPitchG = kGwPix + 4;
 constexpr int kGwStage = 3;  // plane positions a thread stages per block
+constexpr int kGwGrid = 256; // resident workgroups: one per CU (the window takes most of a CU's LDS)
 
+// Persistent workgroups: workgroup w of `nwg` walks the units [units * w / nwg, units * (w + 1) / nwg) of the
+// order (image, group, tile) x channel block, so every CU gets the same number of channel blocks and a tile's
+// set-up (descriptors, hat products) is paid once per run of blocks, not once per launched workgroup.
 template <typename T, int SH, int SW, int CELL0>
 __global__ __launch_bounds__(kGwBlock, 1) void deform_grad_filter_win_kernel(
     Geo g, const T* __restrict__ gout, const T* __restrict__ x, const T* __restrict__ off,
-    const T* __restrict__ rot, float* __restrict__ partial, int tiles, int csplits, int shift, int wr) {
+    const T* __restrict__ rot, float* __restrict__ partial, int tiles, int nwg, int shift, int wr) {
   constexpr int CELLS = SH * SW;
   constexpr int kWaves = kGwBlock / 64;
   static_assert(CELL0 % 16 == 0 && CELL0 < CELLS, "the cells come in slices of 16, the rows of one MFMA block");
@@ -1945,93 +1960,103 @@ __global__ __launch_bounds__(kGwBlock, 1) void deform_grad_filter_win_kernel(
 
   const int cpg = g.channel / g.groups;
   const int out_plane = g.out_h * g.out_w, in_plane = H * W;
+  const int x_cs = g.groups * in_plane * (int)sizeof(T), g_cs = g.groups * out_plane * (int)sizeof(T);  // bytes from a channel of the group to the next
   const int nblk_all = ceil_div(cpg, kGfCh);
-  const int total = tiles * csplits * g.batch * g.groups;
-  const int lb = logical_block(total);
-  if (lb >= total) return;
-  const int tile = lb % tiles, cs = lb / tiles % csplits;
-  const int n = lb / tiles / csplits / g.groups, grp = lb / tiles / csplits % g.groups;
-  const int blk_per = ceil_div(nblk_all, csplits);
-  const int cb_lo = cs * blk_per, nblk = min(blk_per, nblk_all - cb_lo);
-  if (nblk <= 0) return;
+  const long units = (long)tiles * g.batch * g.groups * nblk_all;
+  const int wg = logical_block(nwg);
+  if (wg >= nwg) return;
+  long u = units * wg / nwg;
+  const long u_end = units * (wg + 1) / nwg;
 
   const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int q = lane & 15, kg = lane >> 4;
-  const int p0 = tile * kGwPix;
-  const int live_pixels = min(kGwPix, out_plane - p0);
-  const int live_waves = ceil_div(live_pixels, 16);
-  const bool wave_live = wave < live_waves;
-
-  if (threadIdx.x == 0) mm[0] = 1 << 30, mm[1] = -1;
-  for (int e = threadIdx.x; e < (wpos + RS + 2) * kGfPitch; e += kGwBlock) planes[e] = 0.f;
-
-  // set-up: this thread's pixel, taps g_cq, g_cq + 4, g_cq + 8 (K.cu:486-500 and 338-341)
-  const int g_pix = threadIdx.x % kGwPix, g_cq = __builtin_amdgcn_readfirstlane(threadIdx.x / kGwPix);
-  int t_row[3], t_col[3];   // padded row / column of the sample's top-left corner; row -1: no contribution
-  float t_lh[3], t_lw[3];
-  __syncthreads();          // mm is initialised
-  {
-    const int p = p0 + g_pix;
-    const bool live = p < out_plane;
-    const int pc = live ? p : 0;
-    const int oh = pc / g.out_w, ow = pc % g.out_w;
-    const rsrc_t ro = plane_rsrc(off + (size_t)n * (K9 * 2) * out_plane, K9 * 2 * out_plane);
-    const rsrc_t rr = rot ? plane_rsrc(rot + (size_t)(n * g.groups + grp) * (K9 * 2) * out_plane, K9 * 2 * out_plane)
-                          : plane_rsrc(rot, 0);  // no rotation tensor: reads as zeros
-    const unsigned step = (unsigned)out_plane * (unsigned)sizeof(T);
-    int lo_row = 1 << 30, hi_row = -1;
-#pragma unroll
-    for (int k = 0; k < 3; ++k) {
-      const int t = g_cq + 4 * k;
-      t_row[k] = -1, t_col[k] = 0, t_lh[k] = 0.f, t_lw[k] = 0.f;
-      if (t < K9) {
-        const int f_h = t / 3, f_w = t % 3;
-        const unsigned o = live ? (unsigned)((2 * t) * out_plane + pc) * (unsigned)sizeof(T) : kOutOfRange;
-        const float h = float(oh * g.stride_h - g.pad_h + f_h * g.dil_h) + buf_ld(ro, o, off);
-        const float w = float(ow * g.stride_w - g.pad_w + f_w * g.dil_w) + buf_ld(ro, o + step, off);
-        const bool hit = live && (h > -1.f) && (w > -1.f) && (h < float(H)) && (w < float(W));
-        const float hf = floorf(h), wf = floorf(w);
-        const float sh = scope_coord<float>(g, f_h, buf_ld(rr, o, rot), g.centre_h);
-        const float sw = scope_coord<float>(g, f_w, buf_ld(rr, o + step, rot), g.centre_w);
-        const bool in = hit && (sh > -1.f) && (sw > -1.f) && (sh < float(SH)) && (sw < float(SW));
-        sc[t * kGwPix + g_pix] = in ? make_float2(sh, sw) : make_float2(-2.f, -2.f);
-        if (hit) {
-          t_row[k] = static_cast<int>(hf) + 1, t_col[k] = static_cast<int>(wf) + 1;
-          t_lh[k] = h - hf, t_lw[k] = w - wf;
-          lo_row = min(lo_row, t_row[k]), hi_row = max(hi_row, t_row[k]);
-        }
-      }
-    }
-    if (hi_row >= 0) {
-      atomicMin(&mm[0], lo_row);
-      atomicMax(&mm[1], hi_row);
-    }
-  }
-  __syncthreads();
-  const int row_hi = mm[1], row_lo = row_hi < 0 ? 0 : mm[0];
-  // a window holds the samples whose top row lies in its first wr - 1 rows
-  const int npass = row_hi < 0 ? 1 : ceil_div(row_hi - row_lo + 1, wr - 1);
-
   const int px = wave * 16 + 4 * kg;  // first of this lane's four pixels in the tile
   // rows past the last cell stay 0
   const float ci = CELL0 + q < CELLS ? float((CELL0 + q) / SW) : 64.f, cj = float((CELL0 + q) % SW);
-  float A[4][K9];
-#pragma unroll
-  for (int t = 0; t < K9; ++t) {
-    const float4 s01 = *reinterpret_cast<const float4*>(sc + t * kGwPix + px);
-    const float4 s23 = *reinterpret_cast<const float4*>(sc + t * kGwPix + px + 2);
-    A[0][t] = hat1(s01.x - ci) * hat1(s01.y - cj);
-    A[1][t] = hat1(s01.z - ci) * hat1(s01.w - cj);
-    A[2][t] = hat1(s23.x - ci) * hat1(s23.y - cj);
-    A[3][t] = hat1(s23.z - ci) * hat1(s23.w - cj);
-  }
-
-  // register stage of a (channel block, pass): the 16 channels of this thread's window positions, and four
-  // channels of gout at its pixel
+  const int g_pix = threadIdx.x % kGwPix, g_cq = __builtin_amdgcn_readfirstlane(threadIdx.x / kGwPix);
   const int rpp = kGwBlock >> shift;  // window rows one sweep of the workgroup's threads covers
   const int s_col = threadIdx.x & ((1 << shift) - 1), s_row = threadIdx.x >> shift;
-  const unsigned g_off = p0 + g_pix < out_plane ? (unsigned)(p0 + g_pix) * (unsigned)sizeof(T) : kOutOfRange;
-  float r_x[kGwStage][kGfCh], r_g[4];
+  const unsigned row_bytes = (unsigned)RS * kGfPitch * 4;
+  const unsigned zero_off = (unsigned)wpos * kGfPitch * 4;
+  const char* plane_q = reinterpret_cast<const char*>(planes) + q * 4;
+
+  // column 0 of the window's rows and the area behind it stay zero from here on: the staging writes columns 1..W + 1
+  for (int e = threadIdx.x; e < (wpos + RS + 2) * kGfPitch; e += kGwBlock) planes[e] = 0.f;
+
+  while (u < u_end) {  // a run of channel blocks of one (image, group, tile)
+    const int tg = (int)(u / nblk_all), cb_lo = (int)(u % nblk_all);
+    const int nblk = (int)(u_end - u < (long)(nblk_all - cb_lo) ? u_end - u : (long)(nblk_all - cb_lo));
+    u += nblk;
+    const int tile = tg % tiles, grp = tg / tiles % g.groups, n = tg / tiles / g.groups;
+    const int p0 = tile * kGwPix;
+    const int live_pixels = min(kGwPix, out_plane - p0);
+    const int live_waves = ceil_div(live_pixels, 16);
+    const bool wave_live = wave < live_waves;
+
+    __syncthreads();  // the previous run's last reads of `red` (which `sc` shares) are done; the zero fill
+    if (threadIdx.x == 0) mm[0] = 1 << 30, mm[1] = -1;
+
+    // set-up: this thread's pixel, taps g_cq, g_cq + 4, g_cq + 8 (K.cu:486-500 and 338-341)
+    int t_row[3], t_col[3];   // padded row / column of the sample's top-left corner; row -1: no contribution
+    float t_lh[3], t_lw[3];
+    __syncthreads();          // mm is initialised
+    {
+      const int p = p0 + g_pix;
+      const bool live = p < out_plane;
+      const int pc = live ? p : 0;
+      const int oh = pc / g.out_w, ow = pc % g.out_w;
+      const rsrc_t ro = plane_rsrc(off + (size_t)n * (K9 * 2) * out_plane, K9 * 2 * out_plane);
+      const rsrc_t rr = rot ? plane_rsrc(rot + (size_t)(n * g.groups + grp) * (K9 * 2) * out_plane, K9 * 2 * out_plane)
+                            : plane_rsrc(rot, 0);  // no rotation tensor: reads as zeros
+      const unsigned step = (unsigned)out_plane * (unsigned)sizeof(T);
+      int lo_row = 1 << 30, hi_row = -1;
+#pragma unroll
+      for (int k = 0; k < 3; ++k) {
+        const int t = g_cq + 4 * k;
+        t_row[k] = -1, t_col[k] = 0, t_lh[k] = 0.f, t_lw[k] = 0.f;
+        if (t < K9) {
+          const int f_h = t / 3, f_w = t % 3;
+          const unsigned o = live ? (unsigned)((2 * t) * out_plane + pc) * (unsigned)sizeof(T) : kOutOfRange;
+          const float h = float(oh * g.stride_h - g.pad_h + f_h * g.dil_h) + buf_ld(ro, o, off);
+          const float w = float(ow * g.stride_w - g.pad_w + f_w * g.dil_w) + buf_ld(ro, o + step, off);
+          const bool hit = live && (h > -1.f) && (w > -1.f) && (h < float(H)) && (w < float(W));
+          const float hf = floorf(h), wf = floorf(w);
+          const float sh = scope_coord<float>(g, f_h, buf_ld(rr, o, rot), g.centre_h);
+          const float sw = scope_coord<float>(g, f_w, buf_ld(rr, o + step, rot), g.centre_w);
+          const bool in = hit && (sh > -1.f) && (sw > -1.f) && (sh < float(SH)) && (sw < float(SW));
+          sc[t * kGwPix + g_pix] = in ? make_float2(sh, sw) : make_float2(-2.f, -2.f);
+          if (hit) {
+            t_row[k] = static_cast<int>(hf) + 1, t_col[k] = static_cast<int>(wf) + 1;
+            t_lh[k] = h - hf, t_lw[k] = w - wf;
+            lo_row = min(lo_row, t_row[k]), hi_row = max(hi_row, t_row[k]);
+          }
+        }
+      }
+      if (hi_row >= 0) {
+        atomicMin(&mm[0], lo_row);
+        atomicMax(&mm[1], hi_row);
+      }
+    }
+    __syncthreads();
+    const int row_hi = mm[1], row_lo = row_hi < 0 ? 0 : mm[0];
+    // a window holds the samples whose top row lies in its first wr - 1 rows
+    const int npass = row_hi < 0 ? 1 : ceil_div(row_hi - row_lo + 1, wr - 1);
+
+    float A[4][K9];
+#pragma unroll
+    for (int t = 0; t < K9; ++t) {
+      const float4 s01 = *reinterpret_cast<const float4*>(sc + t * kGwPix + px);
+      const float4 s23 = *reinterpret_cast<const float4*>(sc + t * kGwPix + px + 2);
+      A[0][t] = hat1(s01.x - ci) * hat1(s01.y - cj);
+      A[1][t] = hat1(s01.z - ci) * hat1(s01.w - cj);
+      A[2][t] = hat1(s23.x - ci) * hat1(s23.y - cj);
+      A[3][t] = hat1(s23.z - ci) * hat1(s23.w - cj);
+    }
+
+    // register stage of a (channel block, pass): the 16 channels of this thread's window positions, and four
+    // channels of gout at its pixel
+    const unsigned g_off = p0 + g_pix < out_plane ? (unsigned)(p0 + g_pix) * (unsigned)sizeof(T) : kOutOfRange;
+    float r_x[kGwStage][kGfCh], r_g[4];
 #define DK_GW_ISSUE(cb, lo_k, with_gout)                                                             \
   {                                                                                                  \
     unsigned so_[kGwStage];                                                                          \
@@ -2040,26 +2065,20 @@ __global__ __launch_bounds__(kGwBlock, 1) void deform_grad_filter_win_kernel(
       const bool ok_ = s_row + rpp * j < wr && urow_ >= 0 && urow_ < H && s_col < W;                 \
       so_[j] = ok_ ? (unsigned)(urow_ * W + s_col) * (unsigned)sizeof(T) : kOutOfRange;              \
     }                                                                                                \
+    DK_GF_BLOCK_PLANES(cb)                                                                           \
     _Pragma("unroll") for (int c = 0; c < kGfCh; ++c) {                                              \
-      const int cj_ = (cb) * kGfCh + c;                                                              \
-      const bool chan = cj_ < cpg;                                                                   \
-      const size_t ci_ = (size_t)n * g.channel + grp + (size_t)g.groups * (chan ? cj_ : 0);          \
-      const rsrc_t rs_ = plane_rsrc(x + ci_ * in_plane, chan ? in_plane : 0);                        \
-      _Pragma("unroll") for (int j = 0; j < kGwStage; ++j) r_x[j][c] = buf_ld(rs_, so_[j], x);       \
+      const int sc_ = min(c, last_) * x_cs;                                                          \
+      _Pragma("unroll") for (int j = 0; j < kGwStage; ++j) r_x[j][c] = buf_ld2(rx_, so_[j], sc_, x); \
     }                                                                                                \
     if (with_gout) {                                                                                 \
-      _Pragma("unroll") for (int c = 0; c < 4; ++c) {                                                \
-        const int cj_ = (cb) * kGfCh + g_cq * 4 + c;                                                 \
-        const bool chan = cj_ < cpg;                                                                 \
-        const size_t ci_ = (size_t)n * g.channel + grp + (size_t)g.groups * (chan ? cj_ : 0);        \
-        r_g[c] = buf_ld(plane_rsrc(gout + ci_ * out_plane, chan ? out_plane : 0), g_off, gout);      \
-      }                                                                                              \
+      _Pragma("unroll") for (int c = 0; c < 4; ++c)                                                  \
+        r_g[c] = buf_ld2(rg_, g_off, min(g_cq * 4 + c, last_) * g_cs, gout);                         \
     }                                                                                                \
   }
 
-  const size_t part = (size_t)n * tiles + tile;
-  // owner threads: entry e of a block's result is D[cell = CELL0 + 4 * (l / 16) + r][channel l % 16]
-  // with l = e / 4, r = e % 4 (register r of lane l)
+    const size_t part = (size_t)n * tiles + tile;
+    // owner threads: entry e of a block's result is D[cell = CELL0 + 4 * (l / 16) + r][channel l % 16]
+    // with l = e / 4, r = e % 4 (register r of lane l)
 #define DK_GW_FLUSH(cb)                                                                              \
   if (threadIdx.x < 256) {                                                                           \
     float s_ = 0.f;                                                                                  \
@@ -2070,84 +2089,81 @@ __global__ __launch_bounds__(kGwBlock, 1) void deform_grad_filter_win_kernel(
       partial[(part * g.channel + grp + (size_t)g.groups * cj_) * CELLS + cell_] = s_;               \
   }
 
-  DK_GW_ISSUE(cb_lo, row_lo, true)
+    DK_GW_ISSUE(cb_lo, row_lo, true)
 
-  gf4 acc = {0.f, 0.f, 0.f, 0.f};
-  const unsigned row_bytes = (unsigned)RS * kGfPitch * 4;
-  const unsigned zero_off = (unsigned)wpos * kGfPitch * 4;
-  const char* plane_q = reinterpret_cast<const char*>(planes) + q * 4;
-  const int steps = nblk * npass;
-  for (int it = 0; it < steps; ++it) {
-    const int i = it / npass, k = it % npass;
-    const int lo_k = row_lo + k * (wr - 1);
-    __syncthreads();  // the previous step's reads of the planes, the gout tile, the descriptors and `red` are done
-    if (it == 0 || npass > 1) {
+    gf4 acc = {0.f, 0.f, 0.f, 0.f};
+    const int steps = nblk * npass;
+    for (int it = 0; it < steps; ++it) {
+      const int i = it / npass, k = it % npass;
+      const int lo_k = row_lo + k * (wr - 1);
+      __syncthreads();  // the previous step's reads of the planes, the gout tile, the descriptors and `red` are done
+      if (it == 0 || npass > 1) {
 #pragma unroll
-      for (int kk = 0; kk < 3; ++kk) {
-        const int t = g_cq + 4 * kk;
-        if (t < K9) {
-          const bool in_pass = t_row[kk] >= lo_k && t_row[kk] <= lo_k + wr - 2;  // (row -1: never)
-          const unsigned o = in_pass ? (unsigned)((t_row[kk] - lo_k) * RS + t_col[kk]) * (kGfPitch * 4) : zero_off;
-          hwd[t * kGwPix + g_pix] = make_float4(__uint_as_float(o), t_lh[kk], t_lw[kk], 0.f);
+        for (int kk = 0; kk < 3; ++kk) {
+          const int t = g_cq + 4 * kk;
+          if (t < K9) {
+            const bool in_pass = t_row[kk] >= lo_k && t_row[kk] <= lo_k + wr - 2;  // (row -1: never)
+            const unsigned o = in_pass ? (unsigned)((t_row[kk] - lo_k) * RS + t_col[kk]) * (kGfPitch * 4) : zero_off;
+            hwd[t * kGwPix + g_pix] = make_float4(__uint_as_float(o), t_lh[kk], t_lw[kk], 0.f);
+          }
         }
       }
-    }
 #pragma unroll
-    for (int j = 0; j < kGwStage; ++j) {
-      const int wrow = s_row + rpp * j;
-      if (wrow < wr && s_col + 1 < RS) {  // (a row outside the image or the column right of it: zeros were loaded)
-        float* dst = planes + (wrow * RS + 1 + s_col) * kGfPitch;
+      for (int j = 0; j < kGwStage; ++j) {
+        const int wrow = s_row + rpp * j;
+        if (wrow < wr && s_col + 1 < RS) {  // (a row outside the image or the column right of it: zeros were loaded)
+          float* dst = planes + (wrow * RS + 1 + s_col) * kGfPitch;
 #pragma unroll
-        for (int c = 0; c < kGfCh; c += 4)
-          *reinterpret_cast<float4*>(dst + c) = make_float4(r_x[j][c], r_x[j][c + 1], r_x[j][c + 2], r_x[j][c + 3]);
+          for (int c = 0; c < kGfCh; c += 4)
+            *reinterpret_cast<float4*>(dst + c) = make_float4(r_x[j][c], r_x[j][c + 1], r_x[j][c + 2], r_x[j][c + 3]);
+        }
       }
-    }
-    if (k == 0) {
+      if (k == 0) {
 #pragma unroll
-      for (int c = 0; c < 4; ++c) gs[(g_cq * 4 + c) * kGwPitchG + g_pix] = r_g[c];
-      if (it > 0 && wave_live) *reinterpret_cast<gf4*>(red + (wave * 64 + lane) * 4) = acc;
+        for (int c = 0; c < 4; ++c) gs[(g_cq * 4 + c) * kGwPitchG + g_pix] = r_g[c];
+        if (it > 0 && wave_live) *reinterpret_cast<gf4*>(red + (wave * 64 + lane) * 4) = acc;
+      }
+      __syncthreads();
+      if (it + 1 < steps) {
+        const int i1 = (it + 1) / npass, k1 = (it + 1) % npass;
+        if (k1 == 0) DK_GW_ISSUE(cb_lo + i1, row_lo, true)
+        else DK_GW_ISSUE(cb_lo + i1, row_lo + k1 * (wr - 1), false)
+      }
+      if (k == 0) {
+        if (it > 0) DK_GW_FLUSH(cb_lo + i - 1)
+        acc = gf4{0.f, 0.f, 0.f, 0.f};
+      }
+      if (wave_live) {
+        gf4 acc0 = {0.f, 0.f, 0.f, 0.f}, acc1 = {0.f, 0.f, 0.f, 0.f};
+        const float4 gv = *reinterpret_cast<const float4*>(gs + q * kGwPitchG + px);
+        const float gq[4] = {gv.x, gv.y, gv.z, gv.w};
+#pragma unroll
+        for (int t = 0; t < K9; ++t) {
+#pragma unroll
+          for (int ii = 0; ii < 4; ++ii) {
+            const float4 d = hwd[t * kGwPix + px + ii];
+            const char* c0 = plane_q + __float_as_uint(d.x);
+            const char* c1 = c0 + row_bytes;
+            const float ca = *reinterpret_cast<const float*>(c0), cb_ = *reinterpret_cast<const float*>(c0 + kGfPitch * 4);
+            const float cc = *reinterpret_cast<const float*>(c1), cd = *reinterpret_cast<const float*>(c1 + kGfPitch * 4);
+            const float top = fmaf(d.z, cb_ - ca, ca), bot = fmaf(d.z, cd - cc, cc);
+            const float b = fmaf(d.y, bot - top, top) * gq[ii];
+            if ((ii + t) & 1)
+              acc1 = __builtin_amdgcn_mfma_f32_16x16x4f32(A[ii][t], b, acc1, 0, 0, 0);
+            else
+              acc0 = __builtin_amdgcn_mfma_f32_16x16x4f32(A[ii][t], b, acc0, 0, 0, 0);
+          }
+        }
+        acc += acc0 + acc1;
+      }
     }
     __syncthreads();
-    if (it + 1 < steps) {
-      const int i1 = (it + 1) / npass, k1 = (it + 1) % npass;
-      if (k1 == 0) DK_GW_ISSUE(cb_lo + i1, row_lo, true)
-      else DK_GW_ISSUE(cb_lo + i1, row_lo + k1 * (wr - 1), false)
-    }
-    if (k == 0) {
-      if (it > 0) DK_GW_FLUSH(cb_lo + i - 1)
-      acc = gf4{0.f, 0.f, 0.f, 0.f};
-    }
-    if (wave_live) {
-      gf4 acc0 = {0.f, 0.f, 0.f, 0.f}, acc1 = {0.f, 0.f, 0.f, 0.f};
-      const float4 gv = *reinterpret_cast<const float4*>(gs + q * kGwPitchG + px);
-      const float gq[4] = {gv.x, gv.y, gv.z, gv.w};
-#pragma unroll
-      for (int t = 0; t < K9; ++t) {
-#pragma unroll
-        for (int ii = 0; ii < 4; ++ii) {
-          const float4 d = hwd[t * kGwPix + px + ii];
-          const char* c0 = plane_q + __float_as_uint(d.x);
-          const char* c1 = c0 + row_bytes;
-          const float ca = *reinterpret_cast<const float*>(c0), cb_ = *reinterpret_cast<const float*>(c0 + kGfPitch * 4);
-          const float cc = *reinterpret_cast<const float*>(c1), cd = *reinterpret_cast<const float*>(c1 + kGfPitch * 4);
-          const float top = fmaf(d.z, cb_ - ca, ca), bot = fmaf(d.z, cd - cc, cc);
-          const float b = fmaf(d.y, bot - top, top) * gq[ii];
-          if ((ii + t) & 1)
-            acc1 = __builtin_amdgcn_mfma_f32_16x16x4f32(A[ii][t], b, acc1, 0, 0, 0);
-          else
-            acc0 = __builtin_amdgcn_mfma_f32_16x16x4f32(A[ii][t], b, acc0, 0, 0, 0);
-        }
-      }
-      acc += acc0 + acc1;
-    }
-  }
-  __syncthreads();
-  if (wave_live) *reinterpret_cast<gf4*>(red + (wave * 64 + lane) * 4) = acc;
-  __syncthreads();
-  DK_GW_FLUSH(cb_lo + nblk - 1)
+    if (wave_live) *reinterpret_cast<gf4*>(red + (wave * 64 + lane) * 4) = acc;
+    __syncthreads();
+    DK_GW_FLUSH(cb_lo + nblk - 1)
 #undef DK_GW_ISSUE
-#undef DK_GW_STORE
 #undef DK_GW_FLUSH
+  }
 }
 
 // ---------------------------------------------------------------------------
@@ -2180,6 +2196,7 @@ __global__ __launch_bounds__(kGwBlock, 1) void deform_grad_filter_win2_kernel(
 
   const int cpg = g.channel / g.groups;
   const int out_plane = g.out_h * g.out_w, in_plane = H * W;
+  const int x_cs = g.groups * in_plane * (int)sizeof(T), g_cs = g.groups * out_plane * (int)sizeof(T);  // bytes from a channel of the group to the next
   const int nblk_all = ceil_div(cpg, kGfCh);
   const int total = tiles * csplits * g.batch * g.groups;
   const int lb = logical_block(total);
@@ -2279,20 +2296,14 @@ __global__ __launch_bounds__(kGwBlock, 1) void deform_grad_filter_win2_kernel(
       const bool ok_ = s_row + rpp * j < wr && urow_ >= 0 && urow_ < H && ucol_ >= 0 && ucol_ < W;   \
       so_[j] = ok_ ? (unsigned)(urow_ * W + ucol_) * (unsigned)sizeof(T) : kOutOfRange;              \
     }                                                                                                \
+    DK_GF_BLOCK_PLANES(cb)                                                                           \
     _Pragma("unroll") for (int c = 0; c < kGfCh; ++c) {                                              \
-      const int cj_ = (cb) * kGfCh + c;                                                              \
-      const bool chan = cj_ < cpg;                                                                   \
-      const size_t ci_ = (size_t)n * g.channel + grp + (size_t)g.groups * (chan ? cj_ : 0);          \
-      const rsrc_t rs_ = plane_rsrc(x + ci_ * in_plane, chan ? in_plane : 0);                        \
-      _Pragma("unroll") for (int j = 0; j < kGwStage; ++j) r_x[j][c] = buf_ld(rs_, so_[j], x);       \
+      const int sc_ = min(c, last_) * x_cs;                                                          \
+      _Pragma("unroll") for (int j = 0; j < kGwStage; ++j) r_x[j][c] = buf_ld2(rx_, so_[j], sc_, x); \
     }                                                                                                \
     if (with_gout) {                                                                                 \
-      _Pragma("unroll") for (int c = 0; c < 4; ++c) {                                                \
-        const int cj_ = (cb) * kGfCh + g_cq * 4 + c;                                                 \
-        const bool chan = cj_ < cpg;                                                                 \
-        const size_t ci_ = (size_t)n * g.channel + grp + (size_t)g.groups * (chan ? cj_ : 0);        \
-        r_g[c] = buf_ld(plane_rsrc(gout + ci_ * out_plane, chan ? out_plane : 0), g_off, gout);      \
-      }                                                                                              \
+      _Pragma("unroll") for (int c = 0; c < 4; ++c)                                                  \
+        r_g[c] = buf_ld2(rg_, g_off, min(g_cq * 4 + c, last_) * g_cs, gout);                         \
     }                                                                                                \
   }
 
@@ -2809,7 +2820,7 @@ GradFilterMfma grad_filter_mfma_plan(const Geo& g) {
 // Launch shape of its row-window form (planes of up to 64 columns that the form above does not hold)
 struct GradFilterWin {
   bool ok;
-  int tiles, csplits, shift, wr;
+  int tiles, nwg, shift, wr;
   size_t lds;
 };
 GradFilterWin grad_filter_win_plan(const Geo& g) {
@@ -2829,8 +2840,8 @@ GradFilterWin grad_filter_win_plan(const Geo& g) {
   m.tiles = ceil_div(g.out_h * g.out_w, kGwPix);
   const int nblk = ceil_div(g.channel / g.groups, kGfCh);
   const long base = std::max(1L, (long)m.tiles * g.batch * g.groups);  // batch may be 0
-  m.csplits = (int)std::max<long>(1, std::min<long>(nblk, (256 + base - 1) / base));
-  if (base * m.csplits >= (1L << 31) - 8) return m;
+  if (base >= (1L << 31) - 8) return m;
+  m.nwg = (int)std::min<long>(base * nblk, kGwGrid);  // persistent workgroups, one per CU, equal shares of the channel blocks
   m.ok = true;
   return m;
 }
@@ -2879,10 +2890,10 @@ bool launch_deform_grad_filter_win2(const Geo& g, const GradFilterWin2& m, const
 template <typename T, int SH, int SW, int CELL0>
 bool launch_deform_grad_filter_win(const Geo& g, const GradFilterWin& m, const T* gout, const T* x, const T* off,
                                    const T* rot, float* ws, hipStream_t stream) {
+  const unsigned grid = (unsigned)xcd_grid_size(m.nwg);
   auto kernel = deform_grad_filter_win_kernel<T, SH, SW, CELL0>;
   if (!allow_max_dynamic_lds(reinterpret_cast<const void*>(kernel))) return false;
-  const unsigned grid = (unsigned)xcd_grid_size((long)m.tiles * m.csplits * g.batch * g.groups);
-  kernel<<<grid, kGwBlock, m.lds, stream>>>(g, gout, x, off, rot, ws, m.tiles, m.csplits, m.shift, m.wr);
+  kernel<<<grid, kGwBlock, m.lds, stream>>>(g, gout, x, off, rot, ws, m.tiles, m.nwg, m.shift, m.wr);
   return true;
 }
 
@@ -2900,8 +2911,9 @@ bool launch_deform_grad_filter_mfma(const Geo& g, const GradFilterMfma& m, const
 template <typename T, int SH, int SW>
 bool run_deform_grad_filter(const Geo& g, const T* gout, const T* x, const T* off, const T* rot, T* gfilter,
                             float* ws, hipStream_t stream) {
+  const bool fit = block_planes_fit<T>(g);  // (the matrix-core forms address a block's channels through one descriptor)
   const GradFilterMfma m = grad_filter_mfma_plan(g);
-  if (m.ok) {
+  if (m.ok && fit) {
     if (!launch_deform_grad_filter_mfma<T, SH, SW, 0>(g, m, gout, x, off, rot, ws, stream)) return false;
     if constexpr (SH * SW > 16)
       if (!launch_deform_grad_filter_mfma<T, SH, SW, 16>(g, m, gout, x, off, rot, ws, stream)) return false;
@@ -2910,14 +2922,14 @@ bool run_deform_grad_filter(const Geo& g, const T* gout, const T* x, const T* of
   }
   const GradFilterWin2 w2 = grad_filter_win2_plan(g);
   const GradFilterWin wn = grad_filter_win_plan(g);
-  if (w2.ok && (!wn.ok || path_disabled(kForceWin2))) {
+  if (fit && w2.ok && (!wn.ok || path_disabled(kForceWin2))) {
     if (!launch_deform_grad_filter_win2<T, SH, SW, 0>(g, w2, gout, x, off, rot, ws, stream)) return false;
     if constexpr (SH * SW > 16)
       if (!launch_deform_grad_filter_win2<T, SH, SW, 16>(g, w2, gout, x, off, rot, ws, stream)) return false;
     launch_reduce_partials<float, T>(ws, g.batch * w2.tiles, g.channel * SH * SW, gfilter, stream);
     return true;
   }
-  if (wn.ok) {
+  if (fit && wn.ok) {
     if (!launch_deform_grad_filter_win<T, SH, SW, 0>(g, wn, gout, x, off, rot, ws, stream)) return false;
     if constexpr (SH * SW > 16)
       if (!launch_deform_grad_filter_win<T, SH, SW, 16>(g, wn, gout, x, off, rot, ws, stream)) return false;
