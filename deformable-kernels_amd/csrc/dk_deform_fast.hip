@@ -1931,6 +1931,17 @@ __global__ __launch_bounds__(kGfBlock, 1) void deform_grad_filter_mfma_kernel(
 // many rows), the tile takes several passes over consecutive windows, each sample counted in the pass that holds
 // its two rows: any offsets are served, at the cost of one staging per pass and block.
 // ---------------------------------------------------------------------------
+// The value that lane II of the caller's quad (four consecutive lanes) holds; the compiler folds the lane
+// selection into the instruction that uses the value where that instruction has a DPP form.
+template <int II>
+__device__ __forceinline__ float quad_lane(float v) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), II * 0x55, 0xf, 0xf, true));
+}
+template <int II>
+__device__ __forceinline__ unsigned quad_lane(unsigned v) {
+  return (unsigned)__builtin_amdgcn_update_dpp(0, (int)v, II * 0x55, 0xf, 0xf, true);
+}
+
 constexpr int kGwBlock = 512;
 constexpr int kGwPix = 128;
 constexpr int kGwPitchG = kGwPix + 4;
@@ -2042,17 +2053,6 @@ __global__ __launch_bounds__(kGwBlock, 1) void deform_grad_filter_win_kernel(
     // a window holds the samples whose top row lies in its first wr - 1 rows
     const int npass = row_hi < 0 ? 1 : ceil_div(row_hi - row_lo + 1, wr - 1);
 
-    float A[4][K9];
-#pragma unroll
-    for (int t = 0; t < K9; ++t) {
-      const float4 s01 = *reinterpret_cast<const float4*>(sc + t * kGwPix + px);
-      const float4 s23 = *reinterpret_cast<const float4*>(sc + t * kGwPix + px + 2);
-      A[0][t] = hat1(s01.x - ci) * hat1(s01.y - cj);
-      A[1][t] = hat1(s01.z - ci) * hat1(s01.w - cj);
-      A[2][t] = hat1(s23.x - ci) * hat1(s23.y - cj);
-      A[3][t] = hat1(s23.z - ci) * hat1(s23.w - cj);
-    }
-
     // register stage of a (channel block, pass): the 16 channels of this thread's window positions, and four
     // channels of gout at its pixel
     const unsigned g_off = p0 + g_pix < out_plane ? (unsigned)(p0 + g_pix) * (unsigned)sizeof(T) : kOutOfRange;
@@ -2062,7 +2062,8 @@ __global__ __launch_bounds__(kGwBlock, 1) void deform_grad_filter_win_kernel(
     unsigned so_[kGwStage];                                                                          \
     _Pragma("unroll") for (int j = 0; j < kGwStage; ++j) {                                           \
       const int urow_ = (lo_k) + s_row + rpp * j - 1;  /* plane row of window row s_row + rpp j */    \
-      const bool ok_ = s_row + rpp * j < wr && urow_ >= 0 && urow_ < H && s_col < W;                 \
+      /* (plane rows past the lowest sample's bottom row are not read: row_hi is a padded row) */    \
+      const bool ok_ = s_row + rpp * j < wr && urow_ >= 0 && urow_ < H && urow_ <= row_hi && s_col < W; \
       so_[j] = ok_ ? (unsigned)(urow_ * W + s_col) * (unsigned)sizeof(T) : kOutOfRange;              \
     }                                                                                                \
     DK_GF_BLOCK_PLANES(cb)                                                                           \
@@ -2075,6 +2076,17 @@ __global__ __launch_bounds__(kGwBlock, 1) void deform_grad_filter_win_kernel(
         r_g[c] = buf_ld2(rg_, g_off, min(g_cq * 4 + c, last_) * g_cs, gout);                         \
     }                                                                                                \
   }
+
+    float A[4][K9];
+#pragma unroll
+    for (int t = 0; t < K9; ++t) {
+      const float4 s01 = *reinterpret_cast<const float4*>(sc + t * kGwPix + px);
+      const float4 s23 = *reinterpret_cast<const float4*>(sc + t * kGwPix + px + 2);
+      A[0][t] = hat1(s01.x - ci) * hat1(s01.y - cj);
+      A[1][t] = hat1(s01.z - ci) * hat1(s01.w - cj);
+      A[2][t] = hat1(s23.x - ci) * hat1(s23.y - cj);
+      A[3][t] = hat1(s23.z - ci) * hat1(s23.w - cj);
+    }
 
     const size_t part = (size_t)n * tiles + tile;
     // owner threads: entry e of a block's result is D[cell = CELL0 + 4 * (l / 16) + r][channel l % 16]
@@ -2092,6 +2104,8 @@ __global__ __launch_bounds__(kGwBlock, 1) void deform_grad_filter_win_kernel(
     DK_GW_ISSUE(cb_lo, row_lo, true)
 
     gf4 acc = {0.f, 0.f, 0.f, 0.f};
+    unsigned d_off[K9];          // per tap, of pixel px + (q & 3): byte offset of the sample's top-left corner in the window
+    float d_lh[K9], d_lw[K9];    // ... and its bilinear fractions
     const int steps = nblk * npass;
     for (int it = 0; it < steps; ++it) {
       const int i = it / npass, k = it % npass;
@@ -2111,7 +2125,7 @@ __global__ __launch_bounds__(kGwBlock, 1) void deform_grad_filter_win_kernel(
 #pragma unroll
       for (int j = 0; j < kGwStage; ++j) {
         const int wrow = s_row + rpp * j;
-        if (wrow < wr && s_col + 1 < RS) {  // (a row outside the image or the column right of it: zeros were loaded)
+        if (wrow < wr && wrow <= row_hi + 1 - lo_k && s_col + 1 < RS) {  // (a row outside the image or the column right of it: zeros were loaded; rows below every sample: not read)
           float* dst = planes + (wrow * RS + 1 + s_col) * kGfPitch;
 #pragma unroll
           for (int c = 0; c < kGfCh; c += 4)
@@ -2133,27 +2147,53 @@ __global__ __launch_bounds__(kGwBlock, 1) void deform_grad_filter_win_kernel(
         if (it > 0) DK_GW_FLUSH(cb_lo + i - 1)
         acc = gf4{0.f, 0.f, 0.f, 0.f};
       }
+      if (it == 0 || npass > 1) {  // a lane keeps the descriptors of one of its four pixels, the one of its place in its quad
+#pragma unroll
+        for (int t = 0; t < K9; ++t) {
+          const float4 d = hwd[t * kGwPix + px + (q & 3)];
+          d_off[t] = __float_as_uint(d.x), d_lh[t] = d.y, d_lw[t] = d.z;
+        }
+      }
       if (wave_live) {
         gf4 acc0 = {0.f, 0.f, 0.f, 0.f}, acc1 = {0.f, 0.f, 0.f, 0.f};
         const float4 gv = *reinterpret_cast<const float4*>(gs + q * kGwPitchG + px);
         const float gq[4] = {gv.x, gv.y, gv.z, gv.w};
+        // Two stages kept apart by hand (the reads of LDS return in order): the corner reads of tap t + 1's four
+        // samples, the arithmetic of tap t.  Left to itself the compiler waits for every sample's corners right
+        // after asking for them.  The descriptor of sample (tap, pixel ii) comes out of the quad's lane ii.
+        float cr[2][4][4];
+#define DK_GW_CORNER(t, b, ii)                                                                       \
+  {                                                                                                  \
+    const char* c0 = plane_q + quad_lane<ii>(d_off[t]);                                              \
+    const char* c1 = c0 + row_bytes;                                                                 \
+    cr[b][ii][0] = *reinterpret_cast<const float*>(c0);                                              \
+    cr[b][ii][1] = *reinterpret_cast<const float*>(c0 + kGfPitch * 4);                               \
+    cr[b][ii][2] = *reinterpret_cast<const float*>(c1);                                              \
+    cr[b][ii][3] = *reinterpret_cast<const float*>(c1 + kGfPitch * 4);                               \
+  }
+#define DK_GW_CORNERS(t, b) DK_GW_CORNER(t, b, 0) DK_GW_CORNER(t, b, 1) DK_GW_CORNER(t, b, 2) DK_GW_CORNER(t, b, 3)
+#define DK_GW_SAMPLE(t, ii)                                                                          \
+  {                                                                                                  \
+    const float lh = quad_lane<ii>(d_lh[t]), lw = quad_lane<ii>(d_lw[t]);                            \
+    const float ca = cr[(t) & 1][ii][0], cb_ = cr[(t) & 1][ii][1], cc = cr[(t) & 1][ii][2], cd = cr[(t) & 1][ii][3]; \
+    const float top = fmaf(lw, cb_ - ca, ca), bot = fmaf(lw, cd - cc, cc);                           \
+    const float b = fmaf(lh, bot - top, top) * gq[ii];                                               \
+    if (((ii) + (t)) & 1)                                                                            \
+      acc1 = __builtin_amdgcn_mfma_f32_16x16x4f32(A[ii][t], b, acc1, 0, 0, 0);                       \
+    else                                                                                             \
+      acc0 = __builtin_amdgcn_mfma_f32_16x16x4f32(A[ii][t], b, acc0, 0, 0, 0);                       \
+  }
+        DK_GW_CORNERS(0, 0)
 #pragma unroll
         for (int t = 0; t < K9; ++t) {
-#pragma unroll
-          for (int ii = 0; ii < 4; ++ii) {
-            const float4 d = hwd[t * kGwPix + px + ii];
-            const char* c0 = plane_q + __float_as_uint(d.x);
-            const char* c1 = c0 + row_bytes;
-            const float ca = *reinterpret_cast<const float*>(c0), cb_ = *reinterpret_cast<const float*>(c0 + kGfPitch * 4);
-            const float cc = *reinterpret_cast<const float*>(c1), cd = *reinterpret_cast<const float*>(c1 + kGfPitch * 4);
-            const float top = fmaf(d.z, cb_ - ca, ca), bot = fmaf(d.z, cd - cc, cc);
-            const float b = fmaf(d.y, bot - top, top) * gq[ii];
-            if ((ii + t) & 1)
-              acc1 = __builtin_amdgcn_mfma_f32_16x16x4f32(A[ii][t], b, acc1, 0, 0, 0);
-            else
-              acc0 = __builtin_amdgcn_mfma_f32_16x16x4f32(A[ii][t], b, acc0, 0, 0, 0);
-          }
+          if (t + 1 < K9) DK_GW_CORNERS(t + 1, (t + 1) & 1)
+          __builtin_amdgcn_sched_barrier(0);
+          DK_GW_SAMPLE(t, 0) DK_GW_SAMPLE(t, 1) DK_GW_SAMPLE(t, 2) DK_GW_SAMPLE(t, 3)
+          __builtin_amdgcn_sched_barrier(0);
         }
+#undef DK_GW_CORNER
+#undef DK_GW_CORNERS
+#undef DK_GW_SAMPLE
         acc += acc0 + acc1;
       }
     }
