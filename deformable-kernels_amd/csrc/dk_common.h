@@ -131,6 +131,21 @@ __device__ __forceinline__ float wave_sum(float v) {
   return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 63));
 }
 
+// Least / largest v over the 64 lanes of the wave, returned in every lane: the same six DPP steps (a lane that a
+// step's row mask leaves out, or that has no source lane, compares with its own value).
+__device__ __forceinline__ int wave_min(int v) {
+#define DK_DPP_MIN(ctrl, row_mask) v = min(v, __builtin_amdgcn_update_dpp(v, v, ctrl, row_mask, 0xf, false))
+  DK_DPP_MIN(0xB1, 0xf);
+  DK_DPP_MIN(0x4E, 0xf);
+  DK_DPP_MIN(0x141, 0xf);
+  DK_DPP_MIN(0x140, 0xf);
+  DK_DPP_MIN(0x142, 0xa);
+  DK_DPP_MIN(0x143, 0xc);
+#undef DK_DPP_MIN
+  return __builtin_amdgcn_readlane(v, 63);
+}
+__device__ __forceinline__ int wave_max(int v) { return -wave_min(-v); }
+
 // Value held by the previous / next lane of the wave (0 at the wave's ends): one DPP move.
 __device__ __forceinline__ float from_lane_below(float v) {
   return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x138 /* wave_shr:1 */, 0xf, 0xf, true));

@@ -2043,7 +2043,9 @@ __global__ __launch_bounds__(kGwBlock, 1) void deform_grad_filter_win_kernel(
           }
         }
       }
-      if (hi_row >= 0) {
+      // one atomic per wave and bound: 512 lanes on one LDS address take their turns one by one
+      lo_row = wave_min(lo_row), hi_row = wave_max(hi_row);
+      if (lane == 0 && hi_row >= 0) {
         atomicMin(&mm[0], lo_row);
         atomicMax(&mm[1], hi_row);
       }
@@ -2218,7 +2220,7 @@ constexpr int kG2Wc = 32;                         // window columns (a power of 
 template <typename T, int SH, int SW, int CELL0>
 __global__ __launch_bounds__(kGwBlock, 1) void deform_grad_filter_win2_kernel(
     Geo g, const T* __restrict__ gout, const T* __restrict__ x, const T* __restrict__ off,
-    const T* __restrict__ rot, float* __restrict__ partial, int tiles_x, int tiles, int csplits, int wr) {
+    const T* __restrict__ rot, float* __restrict__ partial, int tiles_x, int tiles, int nwg, int wr) {
   constexpr int CELLS = SH * SW;
   constexpr int kWaves = kGwBlock / 64;
   constexpr int WC = kG2Wc;
@@ -2238,102 +2240,115 @@ __global__ __launch_bounds__(kGwBlock, 1) void deform_grad_filter_win2_kernel(
   const int out_plane = g.out_h * g.out_w, in_plane = H * W;
   const int x_cs = g.groups * in_plane * (int)sizeof(T), g_cs = g.groups * out_plane * (int)sizeof(T);  // bytes from a channel of the group to the next
   const int nblk_all = ceil_div(cpg, kGfCh);
-  const int total = tiles * csplits * g.batch * g.groups;
-  const int lb = logical_block(total);
-  if (lb >= total) return;
-  const int tile = lb % tiles, cs = lb / tiles % csplits;
-  const int n = lb / tiles / csplits / g.groups, grp = lb / tiles / csplits % g.groups;
-  const int blk_per = ceil_div(nblk_all, csplits);
-  const int cb_lo = cs * blk_per, nblk = min(blk_per, nblk_all - cb_lo);
-  if (nblk <= 0) return;
-  const int oy0 = tile / tiles_x * kG2Th, ox0 = tile % tiles_x * kG2Tw;
+  // persistent workgroups with equal shares of the (image, group, tile) x channel block units, as in the
+  // row-window form
+  const long units = (long)tiles * g.batch * g.groups * nblk_all;
+  const int wg = logical_block(nwg);
+  if (wg >= nwg) return;
+  long u = units * wg / nwg;
+  const long u_end = units * (wg + 1) / nwg;
 
   const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int q = lane & 15, kg = lane >> 4;
   // every wave computes (a pixel outside the plane has gout = 0 and descriptors in the zero area)
-
-  if (threadIdx.x == 0) mm[0] = 1 << 30, mm[1] = -1, mm[2] = 1 << 30, mm[3] = -1;
-  // the zero area (every position of the window itself is written by each staging)
-  for (int e = threadIdx.x; e < (WC + 2) * kGfPitch; e += kGwBlock) planes[wpos * kGfPitch + e] = 0.f;
-
-  // set-up: this thread's pixel (index i of the tile: row i / kG2Tw, column i % kG2Tw), taps g_cq, g_cq + 4, g_cq + 8
-  const int g_pix = threadIdx.x % kGwPix, g_cq = __builtin_amdgcn_readfirstlane(threadIdx.x / kGwPix);
-  const int g_oy = oy0 + g_pix / kG2Tw, g_ox = ox0 + g_pix % kG2Tw;
-  const bool g_live = g_oy < g.out_h && g_ox < g.out_w;
-  const int g_p = g_live ? g_oy * g.out_w + g_ox : 0;
-  int t_row[3], t_col[3];   // padded row / column of the sample's top-left corner; row -1: no contribution
-  float t_lh[3], t_lw[3];
-  __syncthreads();          // mm is initialised
-  {
-    const rsrc_t ro = plane_rsrc(off + (size_t)n * (K9 * 2) * out_plane, K9 * 2 * out_plane);
-    const rsrc_t rr = rot ? plane_rsrc(rot + (size_t)(n * g.groups + grp) * (K9 * 2) * out_plane, K9 * 2 * out_plane)
-                          : plane_rsrc(rot, 0);  // no rotation tensor: reads as zeros
-    const unsigned step = (unsigned)out_plane * (unsigned)sizeof(T);
-    int lo_row = 1 << 30, hi_row = -1, lo_col = 1 << 30, hi_col = -1;
-#pragma unroll
-    for (int k = 0; k < 3; ++k) {
-      const int t = g_cq + 4 * k;
-      t_row[k] = -1, t_col[k] = 0, t_lh[k] = 0.f, t_lw[k] = 0.f;
-      if (t < K9) {
-        const int f_h = t / 3, f_w = t % 3;
-        const unsigned o = g_live ? (unsigned)((2 * t) * out_plane + g_p) * (unsigned)sizeof(T) : kOutOfRange;
-        const float h = float(g_oy * g.stride_h - g.pad_h + f_h * g.dil_h) + buf_ld(ro, o, off);
-        const float w = float(g_ox * g.stride_w - g.pad_w + f_w * g.dil_w) + buf_ld(ro, o + step, off);
-        const bool hit = g_live && (h > -1.f) && (w > -1.f) && (h < float(H)) && (w < float(W));
-        const float hf = floorf(h), wf = floorf(w);
-        const float sh = scope_coord<float>(g, f_h, buf_ld(rr, o, rot), g.centre_h);
-        const float sw = scope_coord<float>(g, f_w, buf_ld(rr, o + step, rot), g.centre_w);
-        const bool in = hit && (sh > -1.f) && (sw > -1.f) && (sh < float(SH)) && (sw < float(SW));
-        sc[t * kGwPix + g_pix] = in ? make_float2(sh, sw) : make_float2(-2.f, -2.f);
-        if (hit) {
-          t_row[k] = static_cast<int>(hf) + 1, t_col[k] = static_cast<int>(wf) + 1;
-          t_lh[k] = h - hf, t_lw[k] = w - wf;
-          lo_row = min(lo_row, t_row[k]), hi_row = max(hi_row, t_row[k]);
-          lo_col = min(lo_col, t_col[k]), hi_col = max(hi_col, t_col[k]);
-        }
-      }
-    }
-    if (hi_row >= 0) {
-      atomicMin(&mm[0], lo_row);
-      atomicMax(&mm[1], hi_row);
-      atomicMin(&mm[2], lo_col);
-      atomicMax(&mm[3], hi_col);
-    }
-  }
-  __syncthreads();
-  const bool any = mm[1] >= 0;
-  const int row_lo = any ? mm[0] : 0, col_lo = any ? mm[2] : 0;
-  // a window holds the samples whose corner lies in its first wr - 1 rows and WC - 1 columns
-  const int npr = any ? ceil_div(mm[1] - row_lo + 1, wr - 1) : 1, npc = any ? ceil_div(mm[3] - col_lo + 1, WC - 1) : 1;
-  const int npass = npr * npc;
-
   const int px = wave * 16 + 4 * kg;  // first of this lane's four pixels in the tile
   // rows past the last cell stay 0
   const float ci = CELL0 + q < CELLS ? float((CELL0 + q) / SW) : 64.f, cj = float((CELL0 + q) % SW);
-  float A[4][K9];
-#pragma unroll
-  for (int t = 0; t < K9; ++t) {
-    const float4 s01 = *reinterpret_cast<const float4*>(sc + t * kGwPix + px);
-    const float4 s23 = *reinterpret_cast<const float4*>(sc + t * kGwPix + px + 2);
-    A[0][t] = hat1(s01.x - ci) * hat1(s01.y - cj);
-    A[1][t] = hat1(s01.z - ci) * hat1(s01.w - cj);
-    A[2][t] = hat1(s23.x - ci) * hat1(s23.y - cj);
-    A[3][t] = hat1(s23.z - ci) * hat1(s23.w - cj);
-  }
-
-  // register stage of a (channel block, pass): the 16 channels of this thread's window positions, and four
-  // channels of gout at its pixel
+  const int g_pix = threadIdx.x % kGwPix, g_cq = __builtin_amdgcn_readfirstlane(threadIdx.x / kGwPix);
   constexpr int rpp = kGwBlock / WC;  // window rows one sweep of the workgroup's threads covers
   const int s_col = threadIdx.x & (WC - 1), s_row = threadIdx.x / WC;
-  const unsigned g_off = g_live ? (unsigned)g_p * (unsigned)sizeof(T) : kOutOfRange;
-  float r_x[kGwStage][kGfCh], r_g[4];
+  const unsigned row_bytes = (unsigned)WC * kGfPitch * 4;
+  const unsigned zero_off = (unsigned)wpos * kGfPitch * 4;
+  const char* plane_q = reinterpret_cast<const char*>(planes) + q * 4;
+
+  // the zero area (every position of the window that a pass reads is written by its staging)
+  for (int e = threadIdx.x; e < (WC + 2) * kGfPitch; e += kGwBlock) planes[wpos * kGfPitch + e] = 0.f;
+
+  while (u < u_end) {  // a run of channel blocks of one (image, group, tile)
+    const int tg = (int)(u / nblk_all), cb_lo = (int)(u % nblk_all);
+    const int nblk = (int)(u_end - u < (long)(nblk_all - cb_lo) ? u_end - u : (long)(nblk_all - cb_lo));
+    u += nblk;
+    const int tile = tg % tiles, grp = tg / tiles % g.groups, n = tg / tiles / g.groups;
+    const int oy0 = tile / tiles_x * kG2Th, ox0 = tile % tiles_x * kG2Tw;
+
+    __syncthreads();  // the previous run's last reads of `red` (which `sc` shares) are done; the zero fill
+    if (threadIdx.x == 0) mm[0] = 1 << 30, mm[1] = -1, mm[2] = 1 << 30, mm[3] = -1;
+
+    // set-up: this thread's pixel (index i of the tile: row i / kG2Tw, column i % kG2Tw), taps g_cq, g_cq + 4, g_cq + 8
+    const int g_oy = oy0 + g_pix / kG2Tw, g_ox = ox0 + g_pix % kG2Tw;
+    const bool g_live = g_oy < g.out_h && g_ox < g.out_w;
+    const int g_p = g_live ? g_oy * g.out_w + g_ox : 0;
+    int t_row[3], t_col[3];   // padded row / column of the sample's top-left corner; row -1: no contribution
+    float t_lh[3], t_lw[3];
+    __syncthreads();          // mm is initialised
+    {
+      const rsrc_t ro = plane_rsrc(off + (size_t)n * (K9 * 2) * out_plane, K9 * 2 * out_plane);
+      const rsrc_t rr = rot ? plane_rsrc(rot + (size_t)(n * g.groups + grp) * (K9 * 2) * out_plane, K9 * 2 * out_plane)
+                            : plane_rsrc(rot, 0);  // no rotation tensor: reads as zeros
+      const unsigned step = (unsigned)out_plane * (unsigned)sizeof(T);
+      int lo_row = 1 << 30, hi_row = -1, lo_col = 1 << 30, hi_col = -1;
+#pragma unroll
+      for (int k = 0; k < 3; ++k) {
+        const int t = g_cq + 4 * k;
+        t_row[k] = -1, t_col[k] = 0, t_lh[k] = 0.f, t_lw[k] = 0.f;
+        if (t < K9) {
+          const int f_h = t / 3, f_w = t % 3;
+          const unsigned o = g_live ? (unsigned)((2 * t) * out_plane + g_p) * (unsigned)sizeof(T) : kOutOfRange;
+          const float h = float(g_oy * g.stride_h - g.pad_h + f_h * g.dil_h) + buf_ld(ro, o, off);
+          const float w = float(g_ox * g.stride_w - g.pad_w + f_w * g.dil_w) + buf_ld(ro, o + step, off);
+          const bool hit = g_live && (h > -1.f) && (w > -1.f) && (h < float(H)) && (w < float(W));
+          const float hf = floorf(h), wf = floorf(w);
+          const float sh = scope_coord<float>(g, f_h, buf_ld(rr, o, rot), g.centre_h);
+          const float sw = scope_coord<float>(g, f_w, buf_ld(rr, o + step, rot), g.centre_w);
+          const bool in = hit && (sh > -1.f) && (sw > -1.f) && (sh < float(SH)) && (sw < float(SW));
+          sc[t * kGwPix + g_pix] = in ? make_float2(sh, sw) : make_float2(-2.f, -2.f);
+          if (hit) {
+            t_row[k] = static_cast<int>(hf) + 1, t_col[k] = static_cast<int>(wf) + 1;
+            t_lh[k] = h - hf, t_lw[k] = w - wf;
+            lo_row = min(lo_row, t_row[k]), hi_row = max(hi_row, t_row[k]);
+            lo_col = min(lo_col, t_col[k]), hi_col = max(hi_col, t_col[k]);
+          }
+        }
+      }
+      // one atomic per wave and bound: 512 lanes on one LDS address take their turns one by one
+      lo_row = wave_min(lo_row), hi_row = wave_max(hi_row), lo_col = wave_min(lo_col), hi_col = wave_max(hi_col);
+      if (lane == 0 && hi_row >= 0) {
+        atomicMin(&mm[0], lo_row);
+        atomicMax(&mm[1], hi_row);
+        atomicMin(&mm[2], lo_col);
+        atomicMax(&mm[3], hi_col);
+      }
+    }
+    __syncthreads();
+    const bool any = mm[1] >= 0;
+    const int row_lo = any ? mm[0] : 0, col_lo = any ? mm[2] : 0, row_hi = mm[1];
+    // a window holds the samples whose corner lies in its first wr - 1 rows and WC - 1 columns
+    const int npr = any ? ceil_div(mm[1] - row_lo + 1, wr - 1) : 1, npc = any ? ceil_div(mm[3] - col_lo + 1, WC - 1) : 1;
+    const int npass = npr * npc;
+
+    float A[4][K9];
+#pragma unroll
+    for (int t = 0; t < K9; ++t) {
+      const float4 s01 = *reinterpret_cast<const float4*>(sc + t * kGwPix + px);
+      const float4 s23 = *reinterpret_cast<const float4*>(sc + t * kGwPix + px + 2);
+      A[0][t] = hat1(s01.x - ci) * hat1(s01.y - cj);
+      A[1][t] = hat1(s01.z - ci) * hat1(s01.w - cj);
+      A[2][t] = hat1(s23.x - ci) * hat1(s23.y - cj);
+      A[3][t] = hat1(s23.z - ci) * hat1(s23.w - cj);
+    }
+
+    // register stage of a (channel block, pass): the 16 channels of this thread's window positions, and four
+    // channels of gout at its pixel
+    const unsigned g_off = g_live ? (unsigned)g_p * (unsigned)sizeof(T) : kOutOfRange;
+    float r_x[kGwStage][kGfCh], r_g[4];
 #define DK_GW_ISSUE(cb, lo_r, lo_c, with_gout)                                                       \
   {                                                                                                  \
     unsigned so_[kGwStage];                                                                          \
     const int ucol_ = (lo_c) + s_col - 1;  /* plane column of window column s_col */                 \
     _Pragma("unroll") for (int j = 0; j < kGwStage; ++j) {                                           \
       const int urow_ = (lo_r) + s_row + rpp * j - 1;                                                \
-      const bool ok_ = s_row + rpp * j < wr && urow_ >= 0 && urow_ < H && ucol_ >= 0 && ucol_ < W;   \
+      /* (plane rows past the lowest sample's bottom row are not read: row_hi is a padded row) */    \
+      const bool ok_ = s_row + rpp * j < wr && urow_ >= 0 && urow_ < H && urow_ <= row_hi && ucol_ >= 0 && ucol_ < W; \
       so_[j] = ok_ ? (unsigned)(urow_ * W + ucol_) * (unsigned)sizeof(T) : kOutOfRange;              \
     }                                                                                                \
     DK_GF_BLOCK_PLANES(cb)                                                                           \
@@ -2347,9 +2362,9 @@ __global__ __launch_bounds__(kGwBlock, 1) void deform_grad_filter_win2_kernel(
     }                                                                                                \
   }
 
-  const size_t part = (size_t)n * tiles + tile;
-  // owner threads: entry e of a block's result is D[cell = CELL0 + 4 * (l / 16) + r][channel l % 16]
-  // with l = e / 4, r = e % 4 (register r of lane l)
+    const size_t part = (size_t)n * tiles + tile;
+    // owner threads: entry e of a block's result is D[cell = CELL0 + 4 * (l / 16) + r][channel l % 16]
+    // with l = e / 4, r = e % 4 (register r of lane l)
 #define DK_GW_FLUSH(cb)                                                                              \
   if (threadIdx.x < 256) {                                                                           \
     float s_ = 0.f;                                                                                  \
@@ -2360,84 +2375,109 @@ __global__ __launch_bounds__(kGwBlock, 1) void deform_grad_filter_win2_kernel(
       partial[(part * g.channel + grp + (size_t)g.groups * cj_) * CELLS + cell_] = s_;               \
   }
 
-  DK_GW_ISSUE(cb_lo, row_lo, col_lo, true)
+    DK_GW_ISSUE(cb_lo, row_lo, col_lo, true)
 
-  gf4 acc = {0.f, 0.f, 0.f, 0.f};
-  const unsigned row_bytes = (unsigned)WC * kGfPitch * 4;
-  const unsigned zero_off = (unsigned)wpos * kGfPitch * 4;
-  const char* plane_q = reinterpret_cast<const char*>(planes) + q * 4;
-  const int steps = nblk * npass;
-  for (int it = 0; it < steps; ++it) {
-    const int i = it / npass, k = it % npass;
-    const int lo_r = row_lo + (k / npc) * (wr - 1), lo_c = col_lo + (k % npc) * (WC - 1);
-    __syncthreads();  // the previous step's reads of the planes, the gout tile, the descriptors and `red` are done
-    if (it == 0 || npass > 1) {
+    gf4 acc = {0.f, 0.f, 0.f, 0.f};
+    unsigned d_off[K9];          // per tap, of pixel px + (q & 3): byte offset of the sample's top-left corner in the window
+    float d_lh[K9], d_lw[K9];    // ... and its bilinear fractions
+    const int steps = nblk * npass;
+    for (int it = 0; it < steps; ++it) {
+      const int i = it / npass, k = it % npass;
+      const int lo_r = row_lo + (k / npc) * (wr - 1), lo_c = col_lo + (k % npc) * (WC - 1);
+      __syncthreads();  // the previous step's reads of the planes, the gout tile, the descriptors and `red` are done
+      if (it == 0 || npass > 1) {
 #pragma unroll
-      for (int kk = 0; kk < 3; ++kk) {
-        const int t = g_cq + 4 * kk;
-        if (t < K9) {
-          const bool in_pass = t_row[kk] >= lo_r && t_row[kk] <= lo_r + wr - 2 && t_col[kk] >= lo_c &&
-                               t_col[kk] <= lo_c + WC - 2;  // (row -1: never)
-          const unsigned o = in_pass ? (unsigned)((t_row[kk] - lo_r) * WC + t_col[kk] - lo_c) * (kGfPitch * 4) : zero_off;
-          hwd[t * kGwPix + g_pix] = make_float4(__uint_as_float(o), t_lh[kk], t_lw[kk], 0.f);
+        for (int kk = 0; kk < 3; ++kk) {
+          const int t = g_cq + 4 * kk;
+          if (t < K9) {
+            const bool in_pass = t_row[kk] >= lo_r && t_row[kk] <= lo_r + wr - 2 && t_col[kk] >= lo_c &&
+                                 t_col[kk] <= lo_c + WC - 2;  // (row -1: never)
+            const unsigned o = in_pass ? (unsigned)((t_row[kk] - lo_r) * WC + t_col[kk] - lo_c) * (kGfPitch * 4) : zero_off;
+            hwd[t * kGwPix + g_pix] = make_float4(__uint_as_float(o), t_lh[kk], t_lw[kk], 0.f);
+          }
         }
       }
-    }
 #pragma unroll
-    for (int j = 0; j < kGwStage; ++j) {
-      const int wrow = s_row + rpp * j;
-      if (wrow < wr) {  // (a position outside the image: zeros were loaded)
-        float* dst = planes + (wrow * WC + s_col) * kGfPitch;
+      for (int j = 0; j < kGwStage; ++j) {
+        const int wrow = s_row + rpp * j;
+        if (wrow < wr && wrow <= row_hi + 1 - lo_r) {  // (a position outside the image: zeros were loaded; rows below every sample: not read)
+          float* dst = planes + (wrow * WC + s_col) * kGfPitch;
 #pragma unroll
-        for (int c = 0; c < kGfCh; c += 4)
-          *reinterpret_cast<float4*>(dst + c) = make_float4(r_x[j][c], r_x[j][c + 1], r_x[j][c + 2], r_x[j][c + 3]);
+          for (int c = 0; c < kGfCh; c += 4)
+            *reinterpret_cast<float4*>(dst + c) = make_float4(r_x[j][c], r_x[j][c + 1], r_x[j][c + 2], r_x[j][c + 3]);
+        }
       }
-    }
-    if (k == 0) {
+      if (k == 0) {
 #pragma unroll
-      for (int c = 0; c < 4; ++c) gs[(g_cq * 4 + c) * kGwPitchG + g_pix] = r_g[c];
-      if (it > 0) *reinterpret_cast<gf4*>(red + (wave * 64 + lane) * 4) = acc;
+        for (int c = 0; c < 4; ++c) gs[(g_cq * 4 + c) * kGwPitchG + g_pix] = r_g[c];
+        if (it > 0) *reinterpret_cast<gf4*>(red + (wave * 64 + lane) * 4) = acc;
+      }
+      __syncthreads();
+      if (it + 1 < steps) {
+        const int i1 = (it + 1) / npass, k1 = (it + 1) % npass;
+        if (k1 == 0) DK_GW_ISSUE(cb_lo + i1, row_lo, col_lo, true)
+        else DK_GW_ISSUE(cb_lo + i1, row_lo + (k1 / npc) * (wr - 1), col_lo + (k1 % npc) * (WC - 1), false)
+      }
+      if (k == 0) {
+        if (it > 0) DK_GW_FLUSH(cb_lo + i - 1)
+        acc = gf4{0.f, 0.f, 0.f, 0.f};
+      }
+      if (it == 0 || npass > 1) {  // a lane keeps the descriptors of one of its four pixels, the one of its place in its quad
+#pragma unroll
+        for (int t = 0; t < K9; ++t) {
+          const float4 d = hwd[t * kGwPix + px + (q & 3)];
+          d_off[t] = __float_as_uint(d.x), d_lh[t] = d.y, d_lw[t] = d.z;
+        }
+      }
+      {
+        gf4 acc0 = {0.f, 0.f, 0.f, 0.f}, acc1 = {0.f, 0.f, 0.f, 0.f};
+        const float4 gv = *reinterpret_cast<const float4*>(gs + q * kGwPitchG + px);
+        const float gq[4] = {gv.x, gv.y, gv.z, gv.w};
+        // corner reads of tap t + 1 ahead of the arithmetic of tap t, descriptors out of the quad's lanes: as in
+        // the row-window form
+        float cr[2][4][4];
+#define DK_GW_CORNER(t, b, ii)                                                                       \
+  {                                                                                                  \
+    const char* c0 = plane_q + quad_lane<ii>(d_off[t]);                                              \
+    const char* c1 = c0 + row_bytes;                                                                 \
+    cr[b][ii][0] = *reinterpret_cast<const float*>(c0);                                              \
+    cr[b][ii][1] = *reinterpret_cast<const float*>(c0 + kGfPitch * 4);                               \
+    cr[b][ii][2] = *reinterpret_cast<const float*>(c1);                                              \
+    cr[b][ii][3] = *reinterpret_cast<const float*>(c1 + kGfPitch * 4);                               \
+  }
+#define DK_GW_CORNERS(t, b) DK_GW_CORNER(t, b, 0) DK_GW_CORNER(t, b, 1) DK_GW_CORNER(t, b, 2) DK_GW_CORNER(t, b, 3)
+#define DK_GW_SAMPLE(t, ii)                                                                          \
+  {                                                                                                  \
+    const float lh = quad_lane<ii>(d_lh[t]), lw = quad_lane<ii>(d_lw[t]);                            \
+    const float ca = cr[(t) & 1][ii][0], cb_ = cr[(t) & 1][ii][1], cc = cr[(t) & 1][ii][2], cd = cr[(t) & 1][ii][3]; \
+    const float top = fmaf(lw, cb_ - ca, ca), bot = fmaf(lw, cd - cc, cc);                           \
+    const float b = fmaf(lh, bot - top, top) * gq[ii];                                               \
+    if (((ii) + (t)) & 1)                                                                            \
+      acc1 = __builtin_amdgcn_mfma_f32_16x16x4f32(A[ii][t], b, acc1, 0, 0, 0);                       \
+    else                                                                                             \
+      acc0 = __builtin_amdgcn_mfma_f32_16x16x4f32(A[ii][t], b, acc0, 0, 0, 0);                       \
+  }
+        DK_GW_CORNERS(0, 0)
+#pragma unroll
+        for (int t = 0; t < K9; ++t) {
+          if (t + 1 < K9) DK_GW_CORNERS(t + 1, (t + 1) & 1)
+          __builtin_amdgcn_sched_barrier(0);
+          DK_GW_SAMPLE(t, 0) DK_GW_SAMPLE(t, 1) DK_GW_SAMPLE(t, 2) DK_GW_SAMPLE(t, 3)
+          __builtin_amdgcn_sched_barrier(0);
+        }
+#undef DK_GW_CORNER
+#undef DK_GW_CORNERS
+#undef DK_GW_SAMPLE
+        acc += acc0 + acc1;
+      }
     }
     __syncthreads();
-    if (it + 1 < steps) {
-      const int i1 = (it + 1) / npass, k1 = (it + 1) % npass;
-      if (k1 == 0) DK_GW_ISSUE(cb_lo + i1, row_lo, col_lo, true)
-      else DK_GW_ISSUE(cb_lo + i1, row_lo + (k1 / npc) * (wr - 1), col_lo + (k1 % npc) * (WC - 1), false)
-    }
-    if (k == 0) {
-      if (it > 0) DK_GW_FLUSH(cb_lo + i - 1)
-      acc = gf4{0.f, 0.f, 0.f, 0.f};
-    }
-    {
-      gf4 acc0 = {0.f, 0.f, 0.f, 0.f}, acc1 = {0.f, 0.f, 0.f, 0.f};
-      const float4 gv = *reinterpret_cast<const float4*>(gs + q * kGwPitchG + px);
-      const float gq[4] = {gv.x, gv.y, gv.z, gv.w};
-#pragma unroll
-      for (int t = 0; t < K9; ++t) {
-#pragma unroll
-        for (int ii = 0; ii < 4; ++ii) {
-          const float4 d = hwd[t * kGwPix + px + ii];
-          const char* c0 = plane_q + __float_as_uint(d.x);
-          const char* c1 = c0 + row_bytes;
-          const float ca = *reinterpret_cast<const float*>(c0), cb_ = *reinterpret_cast<const float*>(c0 + kGfPitch * 4);
-          const float cc = *reinterpret_cast<const float*>(c1), cd = *reinterpret_cast<const float*>(c1 + kGfPitch * 4);
-          const float top = fmaf(d.z, cb_ - ca, ca), bot = fmaf(d.z, cd - cc, cc);
-          const float b = fmaf(d.y, bot - top, top) * gq[ii];
-          if ((ii + t) & 1)
-            acc1 = __builtin_amdgcn_mfma_f32_16x16x4f32(A[ii][t], b, acc1, 0, 0, 0);
-          else
-            acc0 = __builtin_amdgcn_mfma_f32_16x16x4f32(A[ii][t], b, acc0, 0, 0, 0);
-        }
-      }
-      acc += acc0 + acc1;
-    }
-  }
-  __syncthreads();
-  *reinterpret_cast<gf4*>(red + (wave * 64 + lane) * 4) = acc;
-  __syncthreads();
-  DK_GW_FLUSH(cb_lo + nblk - 1)
+    *reinterpret_cast<gf4*>(red + (wave * 64 + lane) * 4) = acc;
+    __syncthreads();
+    DK_GW_FLUSH(cb_lo + nblk - 1)
 #undef DK_GW_ISSUE
 #undef DK_GW_FLUSH
+  }
 }
 
 // ---------------------------------------------------------------------------
@@ -2889,7 +2929,7 @@ GradFilterWin grad_filter_win_plan(const Geo& g) {
 // ... and of the form with a window in rows and columns (any plane of the family)
 struct GradFilterWin2 {
   bool ok;
-  int tiles_x, tiles, csplits, wr;
+  int tiles_x, tiles, nwg, wr;
   size_t lds;
 };
 GradFilterWin2 grad_filter_win2_plan(const Geo& g) {
@@ -2911,8 +2951,8 @@ GradFilterWin2 grad_filter_win2_plan(const Geo& g) {
   m.tiles = m.tiles_x * ceil_div(g.out_h, kG2Th);
   const int nblk = ceil_div(g.channel / g.groups, kGfCh);
   const long base = std::max(1L, (long)m.tiles * g.batch * g.groups);  // batch may be 0
-  m.csplits = (int)std::max<long>(1, std::min<long>(nblk, (256 + base - 1) / base));
-  if (base * m.csplits >= (1L << 31) - 8) return m;
+  if (base >= (1L << 31) - 8) return m;
+  m.nwg = (int)std::min<long>(base * nblk, kGwGrid);  // persistent workgroups, one per CU, equal shares of the channel blocks
   m.ok = true;
   return m;
 }
@@ -2922,8 +2962,8 @@ bool launch_deform_grad_filter_win2(const Geo& g, const GradFilterWin2& m, const
                                     const T* rot, float* ws, hipStream_t stream) {
   auto kernel = deform_grad_filter_win2_kernel<T, SH, SW, CELL0>;
   if (!allow_max_dynamic_lds(reinterpret_cast<const void*>(kernel))) return false;
-  const unsigned grid = (unsigned)xcd_grid_size((long)m.tiles * m.csplits * g.batch * g.groups);
-  kernel<<<grid, kGwBlock, m.lds, stream>>>(g, gout, x, off, rot, ws, m.tiles_x, m.tiles, m.csplits, m.wr);
+  const unsigned grid = (unsigned)xcd_grid_size(m.nwg);
+  kernel<<<grid, kGwBlock, m.lds, stream>>>(g, gout, x, off, rot, ws, m.tiles_x, m.tiles, m.nwg, m.wr);
   return true;
 }
 
