@@ -1726,6 +1726,17 @@ __global__ __launch_bounds__(BLOCK, 2) void deform_grad_filter_kernel(
 //     partial of (image, tile): reduce_partials_kernel adds those in order.
 // CELL0: the launch covers the scope cells CELL0 .. CELL0 + 15 (a 5 x 5 scope takes two).
 // ---------------------------------------------------------------------------
+// The value that lane II of the caller's quad (four consecutive lanes) holds; the compiler folds the lane
+// selection into the instruction that uses the value where that instruction has a DPP form.
+template <int II>
+__device__ __forceinline__ float quad_lane(float v) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), II * 0x55, 0xf, 0xf, true));
+}
+template <int II>
+__device__ __forceinline__ unsigned quad_lane(unsigned v) {
+  return (unsigned)__builtin_amdgcn_update_dpp(0, (int)v, II * 0x55, 0xf, 0xf, true);
+}
+
 // The planes of one block of channels of an image behind one descriptor each (input, gout): a channel of the
 // block is selected by the scalar part of the address, `channel * x_cs` bytes, so that a load costs the scalar
 // unit two instructions and not the twenty of a descriptor of its own (the 64-bit address, the size, the
@@ -1865,6 +1876,15 @@ __global__ __launch_bounds__(kGfBlock, 1) void deform_grad_filter_mfma_kernel(
     A[2][t] = hat1(s23.x - ci) * hat1(s23.y - cj);
     A[3][t] = hat1(s23.z - ci) * hat1(s23.w - cj);
   }
+  // a lane keeps the descriptors of one of its four pixels, the one of its place in its quad of lanes; a sample's
+  // descriptor comes out of the quad's lane of that pixel (quad_lane)
+  unsigned d_off[K9];
+  float d_lh[K9], d_lw[K9];
+#pragma unroll
+  for (int t = 0; t < K9; ++t) {
+    const float4 d = hwd[t * kGfPix + px + (q & 3)];
+    d_off[t] = __float_as_uint(d.x), d_lh[t] = d.y, d_lw[t] = d.z;
+  }
 
   const size_t part = (size_t)n * tiles + tile;
   // owner threads: entry e of a block's result is D[cell = CELL0 + 4 * (l / 16) + r][channel l % 16]
@@ -1893,23 +1913,23 @@ __global__ __launch_bounds__(kGfBlock, 1) void deform_grad_filter_mfma_kernel(
       gf4 acc0 = {0.f, 0.f, 0.f, 0.f}, acc1 = {0.f, 0.f, 0.f, 0.f};
       const float4 gv = *reinterpret_cast<const float4*>(gs + q * kGfPitchG + px);
       const float gq[4] = {gv.x, gv.y, gv.z, gv.w};
+#define DK_GF_SAMPLE(t, ii)                                                                          \
+  {                                                                                                  \
+    const char* c0 = plane_q + quad_lane<ii>(d_off[t]);                                              \
+    const char* c1 = c0 + row_bytes;                                                                 \
+    const float ca = *reinterpret_cast<const float*>(c0), cb_ = *reinterpret_cast<const float*>(c0 + kGfPitch * 4); \
+    const float cc = *reinterpret_cast<const float*>(c1), cd = *reinterpret_cast<const float*>(c1 + kGfPitch * 4);  \
+    const float lh = quad_lane<ii>(d_lh[t]), lw = quad_lane<ii>(d_lw[t]);                            \
+    const float top = fmaf(lw, cb_ - ca, ca), bot = fmaf(lw, cd - cc, cc);                           \
+    const float b = fmaf(lh, bot - top, top) * gq[ii];                                               \
+    if (((ii) + (t)) & 1)                                                                            \
+      acc1 = __builtin_amdgcn_mfma_f32_16x16x4f32(A[ii][t], b, acc1, 0, 0, 0);                       \
+    else                                                                                             \
+      acc0 = __builtin_amdgcn_mfma_f32_16x16x4f32(A[ii][t], b, acc0, 0, 0, 0);                       \
+  }
 #pragma unroll
-      for (int t = 0; t < K9; ++t) {
-#pragma unroll
-        for (int ii = 0; ii < 4; ++ii) {
-          const float4 d = hwd[t * kGfPix + px + ii];
-          const char* c0 = plane_q + __float_as_uint(d.x);
-          const char* c1 = c0 + row_bytes;
-          const float ca = *reinterpret_cast<const float*>(c0), cb_ = *reinterpret_cast<const float*>(c0 + kGfPitch * 4);
-          const float cc = *reinterpret_cast<const float*>(c1), cd = *reinterpret_cast<const float*>(c1 + kGfPitch * 4);
-          const float top = fmaf(d.z, cb_ - ca, ca), bot = fmaf(d.z, cd - cc, cc);
-          const float b = fmaf(d.y, bot - top, top) * gq[ii];
-          if ((ii + t) & 1)
-            acc1 = __builtin_amdgcn_mfma_f32_16x16x4f32(A[ii][t], b, acc1, 0, 0, 0);
-          else
-            acc0 = __builtin_amdgcn_mfma_f32_16x16x4f32(A[ii][t], b, acc0, 0, 0, 0);
-        }
-      }
+      for (int t = 0; t < K9; ++t) { DK_GF_SAMPLE(t, 0) DK_GF_SAMPLE(t, 1) DK_GF_SAMPLE(t, 2) DK_GF_SAMPLE(t, 3) }
+#undef DK_GF_SAMPLE
       acc = acc0 + acc1;
     }
   }
@@ -1931,17 +1951,6 @@ __global__ __launch_bounds__(kGfBlock, 1) void deform_grad_filter_mfma_kernel(
 // many rows), the tile takes several passes over consecutive windows, each sample counted in the pass that holds
 // its two rows: any offsets are served, at the cost of one staging per pass and block.
 // ---------------------------------------------------------------------------
-// The value that lane II of the caller's quad (four consecutive lanes) holds; the compiler folds the lane
-// selection into the instruction that uses the value where that instruction has a DPP form.
-template <int II>
-__device__ __forceinline__ float quad_lane(float v) {
-  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), II * 0x55, 0xf, 0xf, true));
-}
-template <int II>
-__device__ __forceinline__ unsigned quad_lane(unsigned v) {
-  return (unsigned)__builtin_amdgcn_update_dpp(0, (int)v, II * 0x55, 0xf, 0xf, true);
-}
-
 constexpr int kGwBlock = 512;
 constexpr int kGwPix = 128;
 constexpr int kGwPitchG = kGwPix + 4;
