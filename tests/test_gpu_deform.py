@@ -44,6 +44,8 @@ CASES = [
     (2, 9, 70, 96, 3, (3, 3), 1, 1, 1, 3, 0.6, 2.0),      # the same kernels in one pass: three groups of three channels, scope 3
     (1, 10, 224, 224, 3, (4, 4), 1, 1, 1, 1, 0.7, 2.0),   # 224 x 224: no padded plane fits LDS; grad input in bands of 20 rows (a chunk of 8 channels and one of 2), row windows with the smaller margin
     (1, 6, 150, 200, 3, (4, 4), 2, 1, 1, 2, 0.6, 12.0),   # the band form at stride 2 with offsets of twelve rows (every band walks many tiles), two groups of three channels
+    (4, 40, 56, 56, 3, (4, 4), 1, 1, 1, 1, 0.7, 2.0),     # row-window grad filter with more (tile, channel block) units than persistent workgroups: 300 units on 256, runs that start and end inside a tile
+    (1, 40, 112, 112, 3, (4, 4), 1, 1, 1, 1, 0.7, 2.0),   # the same for the rows-and-columns-window grad filter: 98 tiles x 3 channel blocks
 ]
 NAMES = ("forward", "grad input", "grad offset", "grad rotation", "grad filter")
 
@@ -99,7 +101,7 @@ def test_fp64_matches_oracle(case):
 
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
-@pytest.mark.parametrize("case", CASES[:3] + [CASES[10], CASES[13], CASES[14], CASES[16], CASES[17], CASES[24]])   # planes above 30 x 30; wider than 64 columns; 224 x 224
+@pytest.mark.parametrize("case", CASES[:3] + [CASES[10], CASES[13], CASES[14], CASES[16], CASES[17], CASES[24], CASES[26], CASES[27]])   # planes above 30 x 30; wider than 64 columns; 224 x 224; persistent grad filter
 def test_half_precisions_match_fp32_oracle(case, dtype):
     inputs, got = _run(case, dtype)
     want = _oracle(inputs, np.float32)
