@@ -2102,10 +2102,17 @@ __global__ __launch_bounds__(kGwBlock, 1) void deform_grad_filter_win_kernel(
     const size_t part = (size_t)n * tiles + tile;
     // owner threads: entry e of a block's result is D[cell = CELL0 + 4 * (l / 16) + r][channel l % 16]
     // with l = e / 4, r = e % 4 (register r of lane l)
+    // ... in two halves: the reads of the waves' partial sums are asked for in front of a block's arithmetic and
+    // added and written behind it, so that the four owner waves do not keep the other four waiting at the barrier
+#define DK_GW_FLUSH_READ()                                                                           \
+  if (threadIdx.x < 256) {                                                                           \
+    _Pragma("unroll") for (int w_ = 0; w_ < kWaves; ++w_)                                            \
+      fl[w_] = w_ < live_waves ? red[w_ * 256 + threadIdx.x] : 0.f;                                  \
+  }
 #define DK_GW_FLUSH(cb)                                                                              \
   if (threadIdx.x < 256) {                                                                           \
     float s_ = 0.f;                                                                                  \
-    for (int w_ = 0; w_ < live_waves; ++w_) s_ += red[w_ * 256 + threadIdx.x];                       \
+    _Pragma("unroll") for (int w_ = 0; w_ < kWaves; ++w_) s_ += fl[w_];                              \
     const int l_ = threadIdx.x / 4, r_ = threadIdx.x % 4;                                            \
     const int cell_ = CELL0 + 4 * (l_ / 16) + r_, cj_ = (cb) * kGfCh + l_ % 16;                      \
     if (cell_ < CELLS && cj_ < cpg)                                                                  \
@@ -2115,6 +2122,7 @@ __global__ __launch_bounds__(kGwBlock, 1) void deform_grad_filter_win_kernel(
     DK_GW_ISSUE(cb_lo, row_lo, true)
 
     gf4 acc = {0.f, 0.f, 0.f, 0.f};
+    float fl[kWaves];            // the waves' partial sums of one entry of a block's result, on their way to `partial`
     unsigned d_off[K9];          // per tap, of pixel px + (q & 3): byte offset of the sample's top-left corner in the window
     float d_lh[K9], d_lw[K9];    // ... and its bilinear fractions
     const int steps = nblk * npass;
@@ -2154,10 +2162,9 @@ __global__ __launch_bounds__(kGwBlock, 1) void deform_grad_filter_win_kernel(
         if (k1 == 0) DK_GW_ISSUE(cb_lo + i1, row_lo, true)
         else DK_GW_ISSUE(cb_lo + i1, row_lo + k1 * (wr - 1), false)
       }
-      if (k == 0) {
-        if (it > 0) DK_GW_FLUSH(cb_lo + i - 1)
-        acc = gf4{0.f, 0.f, 0.f, 0.f};
-      }
+      const bool flush = k == 0 && it > 0;
+      if (flush) DK_GW_FLUSH_READ()
+      if (k == 0) acc = gf4{0.f, 0.f, 0.f, 0.f};
       if (it == 0 || npass > 1) {  // a lane keeps the descriptors of one of its four pixels, the one of its place in its quad
 #pragma unroll
         for (int t = 0; t < K9; ++t) {
@@ -2207,12 +2214,15 @@ __global__ __launch_bounds__(kGwBlock, 1) void deform_grad_filter_win_kernel(
 #undef DK_GW_SAMPLE
         acc += acc0 + acc1;
       }
+      if (flush) DK_GW_FLUSH(cb_lo + i - 1)
     }
     __syncthreads();
     if (wave_live) *reinterpret_cast<gf4*>(red + (wave * 64 + lane) * 4) = acc;
     __syncthreads();
+    DK_GW_FLUSH_READ()
     DK_GW_FLUSH(cb_lo + nblk - 1)
 #undef DK_GW_ISSUE
+#undef DK_GW_FLUSH_READ
 #undef DK_GW_FLUSH
   }
 }
@@ -2374,10 +2384,15 @@ __global__ __launch_bounds__(kGwBlock, 1) void deform_grad_filter_win2_kernel(
     const size_t part = (size_t)n * tiles + tile;
     // owner threads: entry e of a block's result is D[cell = CELL0 + 4 * (l / 16) + r][channel l % 16]
     // with l = e / 4, r = e % 4 (register r of lane l)
+    // ... in two halves, as in the row-window form
+#define DK_GW_FLUSH_READ()                                                                           \
+  if (threadIdx.x < 256) {                                                                           \
+    _Pragma("unroll") for (int w_ = 0; w_ < kWaves; ++w_) fl[w_] = red[w_ * 256 + threadIdx.x];      \
+  }
 #define DK_GW_FLUSH(cb)                                                                              \
   if (threadIdx.x < 256) {                                                                           \
     float s_ = 0.f;                                                                                  \
-    for (int w_ = 0; w_ < kWaves; ++w_) s_ += red[w_ * 256 + threadIdx.x];                           \
+    _Pragma("unroll") for (int w_ = 0; w_ < kWaves; ++w_) s_ += fl[w_];                              \
     const int l_ = threadIdx.x / 4, r_ = threadIdx.x % 4;                                            \
     const int cell_ = CELL0 + 4 * (l_ / 16) + r_, cj_ = (cb) * kGfCh + l_ % 16;                      \
     if (cell_ < CELLS && cj_ < cpg)                                                                  \
@@ -2387,6 +2402,7 @@ __global__ __launch_bounds__(kGwBlock, 1) void deform_grad_filter_win2_kernel(
     DK_GW_ISSUE(cb_lo, row_lo, col_lo, true)
 
     gf4 acc = {0.f, 0.f, 0.f, 0.f};
+    float fl[kWaves];            // the waves' partial sums of one entry of a block's result, on their way to `partial`
     unsigned d_off[K9];          // per tap, of pixel px + (q & 3): byte offset of the sample's top-left corner in the window
     float d_lh[K9], d_lw[K9];    // ... and its bilinear fractions
     const int steps = nblk * npass;
@@ -2427,10 +2443,9 @@ __global__ __launch_bounds__(kGwBlock, 1) void deform_grad_filter_win2_kernel(
         if (k1 == 0) DK_GW_ISSUE(cb_lo + i1, row_lo, col_lo, true)
         else DK_GW_ISSUE(cb_lo + i1, row_lo + (k1 / npc) * (wr - 1), col_lo + (k1 % npc) * (WC - 1), false)
       }
-      if (k == 0) {
-        if (it > 0) DK_GW_FLUSH(cb_lo + i - 1)
-        acc = gf4{0.f, 0.f, 0.f, 0.f};
-      }
+      const bool flush = k == 0 && it > 0;
+      if (flush) DK_GW_FLUSH_READ()
+      if (k == 0) acc = gf4{0.f, 0.f, 0.f, 0.f};
       if (it == 0 || npass > 1) {  // a lane keeps the descriptors of one of its four pixels, the one of its place in its quad
 #pragma unroll
         for (int t = 0; t < K9; ++t) {
@@ -2479,12 +2494,15 @@ __global__ __launch_bounds__(kGwBlock, 1) void deform_grad_filter_win2_kernel(
 #undef DK_GW_SAMPLE
         acc += acc0 + acc1;
       }
+      if (flush) DK_GW_FLUSH(cb_lo + i - 1)
     }
     __syncthreads();
     *reinterpret_cast<gf4*>(red + (wave * 64 + lane) * 4) = acc;
     __syncthreads();
+    DK_GW_FLUSH_READ()
     DK_GW_FLUSH(cb_lo + nblk - 1)
 #undef DK_GW_ISSUE
+#undef DK_GW_FLUSH_READ
 #undef DK_GW_FLUSH
   }
 }
