@@ -838,11 +838,12 @@ typedef float nd4 __attribute__((ext_vector_type(4)));
 //   d2 = S3 + f0 S5 + f1 S6 + f0 f1 S7,       S_m = sum_c gout[c] * k_m[c],
 // and the S_m of 16 points of one cell are a 16 x 64 by 64 x 16 product: v_mfma_f32_16x16x4_f32 with
 // lane l supplying gout[point l % 16][channel 16 (l / 16) + step] and k_{l % 16}[the same channel]
-// over 16 steps (a lane's 16 channels are contiguous: four 16-byte loads of its point's row; the
+// over 16 steps (step 4 j + i takes channel 16 j + 4 (l / 16) + i of the block, the same for both operands, so that
+// the four lanes of a point read 64 contiguous bytes of its row with each of their four 16-byte loads; the
 // coefficients go through the wave's LDS slice).  The three wave reductions per point and channel
 // block of the VALU kernel (75 VALU instructions per point) become one MFMA per point.
 template <typename T>
-__global__ __launch_bounds__(kBlock) void nd_grad_coord_mfma_kernel(NdGeo g, const float* __restrict__ gout,
+__global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(4, 4))) void nd_grad_coord_mfma_kernel(NdGeo g, const float* __restrict__ gout,
                                                                     const float* __restrict__ data_cl,
                                                                     const float* __restrict__ coord,
                                                                     const int* __restrict__ order, int nbins,
@@ -876,26 +877,27 @@ __global__ __launch_bounds__(kBlock) void nd_grad_coord_mfma_kernel(NdGeo g, con
     for (int b = 0; b < 4; ++b) acc[b] = nd4{0.f, 0.f, 0.f, 0.f};
     for (int c0 = 0; c0 < g.channel; c0 += 64) {
       // this lane's 16 channels of its point in batch b: issued two batches ahead of their MFMAs,
-      // the first two before the cell's corner rows, so that the two latencies overlap
-      float av[4][16];
+      // the first two before the cell's corner rows, so that the two latencies overlap (two buffers in turn:
+      // with four the kernel takes 168 registers and a SIMD holds three waves of it; this is four)
+      float av[2][16];
 #define DK_ND_LOAD_A(b)                                                                          \
   if (qs + 16 * (b) < qe) {                                                                      \
     const int q_ = qs + 16 * (b) + pr;                                                           \
     const bool on_ = q_ < qe;                                                                    \
     const long id_ = __shfl(wv.id, on_ ? q_ : qs);                                               \
-    const float4* rowp_ = reinterpret_cast<const float4*>(gout + id_ * g.channel + c0 + 16 * kg); \
+    const float4* rowp_ = reinterpret_cast<const float4*>(gout + id_ * g.channel + c0 + 4 * kg); \
     _Pragma("unroll") for (int j = 0; j < 4; ++j) {                                              \
-      const float4 t_ = rowp_[j];                                                                \
-      av[b][4 * j] = on_ ? t_.x : 0.f;                                                           \
-      av[b][4 * j + 1] = on_ ? t_.y : 0.f;                                                       \
-      av[b][4 * j + 2] = on_ ? t_.z : 0.f;                                                       \
-      av[b][4 * j + 3] = on_ ? t_.w : 0.f;                                                       \
+      const float4 t_ = rowp_[4 * j];  /* the four lanes of a point: 64 contiguous bytes */      \
+      av[(b) & 1][4 * j] = on_ ? t_.x : 0.f;                                                     \
+      av[(b) & 1][4 * j + 1] = on_ ? t_.y : 0.f;                                                 \
+      av[(b) & 1][4 * j + 2] = on_ ? t_.z : 0.f;                                                 \
+      av[(b) & 1][4 * j + 3] = on_ ? t_.w : 0.f;                                                 \
     }                                                                                            \
   }
 #define DK_ND_MFMA(b)                                                                            \
   if (qs + 16 * (b) < qe) {                                                                      \
     _Pragma("unroll") for (int s_ = 0; s_ < 16; ++s_)                                            \
-      acc[b] = __builtin_amdgcn_mfma_f32_16x16x4f32(av[b][s_], bv[s_], acc[b], 0, 0, 0);         \
+      acc[b] = __builtin_amdgcn_mfma_f32_16x16x4f32(av[(b) & 1][s_], bv[s_], acc[b], 0, 0, 0);   \
   }
       DK_ND_LOAD_A(0)
       DK_ND_LOAD_A(1)
@@ -921,10 +923,10 @@ __global__ __launch_bounds__(kBlock) void nd_grad_coord_mfma_kernel(NdGeo g, con
       float bv[16];
       {
         const bool row = pr >= 1 && pr < 8;  // rows 0 and 8 .. 15 of the coefficient matrix are zero
-        const float4* src = reinterpret_cast<const float4*>(&coef[row ? pr : 1][16 * kg]);
+        const float4* src = reinterpret_cast<const float4*>(&coef[row ? pr : 1][4 * kg]);
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
-          const float4 t = src[j];
+          const float4 t = src[4 * j];
           bv[4 * j] = row ? t.x : 0.f;
           bv[4 * j + 1] = row ? t.y : 0.f;
           bv[4 * j + 2] = row ? t.z : 0.f;
